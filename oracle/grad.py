@@ -1,0 +1,123 @@
+"""Gradient oracle: torch-fp64 autograd through sequential restatements.
+
+TEST INFRASTRUCTURE: imported only by tests, smoke() and bench.py's cpu_baseline.
+
+Each function re-states the forward recurrence of ``oracle.memoroid`` with
+torch ops (select-style resets through ``torch.where``, as memoroid.py:79-83
+does with ``jnp.where``) so that ``torch.autograd`` yields reference gradients.
+Autograd keeps every per-step state alive, so these are for shapes up to a few
+thousand (b, h, t) triples; full-size gradients are checked against the C
+oracle, which is itself checked against these.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+F64 = torch.float64
+
+
+def _t(x, requires_grad=False, dtype=None):
+    if isinstance(x, torch.Tensor):
+        t = x.detach().clone()
+    else:
+        t = torch.from_numpy(np.ascontiguousarray(np.asarray(x)))
+    if dtype is None:
+        dtype = torch.complex128 if t.is_complex() else F64
+    t = t.to(dtype)
+    t.requires_grad_(requires_grad)
+    return t
+
+
+def _done(done):
+    return torch.from_numpy(np.ascontiguousarray(np.asarray(done) != 0))
+
+
+def diag_scan_t(a, b, done, h0, P0=None):
+    """torch restatement of oracle.memoroid.diag_scan (differentiable)."""
+    B, T, D = b.shape
+    a = a.expand(B, T, D)
+    h = h0
+    P = torch.ones_like(h0) if P0 is None else P0
+    hs = []
+    for t in range(T):
+        r = done[:, t][:, None]
+        h = torch.where(r, b[:, t], a[:, t] * h + b[:, t])
+        P = torch.where(r, a[:, t], a[:, t] * P)
+        hs.append(h)
+    return torch.stack(hs, 1), h, P
+
+
+def elu1_t(x):
+    return torch.where(x > 0, x + 1.0, torch.exp(torch.clamp(x, max=0.0)))
+
+
+def linear_attention_t(q, k, v, done, S0, feature_map="none"):
+    if feature_map in ("elu1", 1):
+        q, k = elu1_t(q), elu1_t(k)
+    B, T, H, dk = q.shape
+    S = S0
+    os_ = []
+    for t in range(T):
+        r = done[:, t][:, None, None, None]
+        S = torch.where(r, torch.zeros_like(S), S)
+        S = S + torch.einsum("bhi,bhj->bhij", v[:, t], k[:, t])
+        os_.append(torch.einsum("bhij,bhj->bhi", S, q[:, t]))
+    return torch.stack(os_, 1), S
+
+
+def delta_rule_t(q, k, v, beta, done, S0):
+    B, T, H, dk = q.shape
+    S = S0
+    os_ = []
+    for t in range(T):
+        r = done[:, t][:, None, None, None]
+        S = torch.where(r, torch.zeros_like(S), S)
+        u = beta[:, t][..., None] * (v[:, t] - torch.einsum("bhij,bhj->bhi", S, k[:, t]))
+        S = S + torch.einsum("bhi,bhj->bhij", u, k[:, t])
+        os_.append(torch.einsum("bhij,bhj->bhi", S, q[:, t]))
+    return torch.stack(os_, 1), S
+
+
+def _np(x):
+    return None if x is None else x.detach().numpy()
+
+
+def diag_scan_grads(a, b, done, h0, g, g_last=None):
+    """Returns dict(da, db, dh0) for L = sum(g*h) + sum(g_last*h_last) (real
+    part for complex inputs, torch's conjugate-cotangent convention)."""
+    a_, b_, h0_ = _t(a, True), _t(b, True), _t(h0, True)
+    h, hl, _ = diag_scan_t(a_, b_, _done(done), h0_)
+    L = (h * _t(g).conj()).sum().real if h.is_complex() else (h * _t(g)).sum()
+    if g_last is not None:
+        L = L + ((hl * _t(g_last).conj()).sum().real if hl.is_complex() else (hl * _t(g_last)).sum())
+    L.backward()
+    return dict(da=_np(a_.grad), db=_np(b_.grad), dh0=_np(h0_.grad))
+
+
+def linear_attention_grads(q, k, v, done, S0, do, dS_last=None, feature_map="none"):
+    """Returns dict(o, S_last, dq, dk, dv, dS0) for L = sum(do*o) + sum(dS_last*S_last)."""
+    q_, k_, v_ = _t(q, True), _t(k, True), _t(v, True)
+    B, T, H, dk = q_.shape
+    S0_ = _t(np.zeros((B, H, v_.shape[-1], dk)) if S0 is None else S0, True)
+    o, Sl = linear_attention_t(q_, k_, v_, _done(done), S0_, feature_map)
+    L = (o * _t(do)).sum()
+    if dS_last is not None:
+        L = L + (Sl * _t(dS_last)).sum()
+    L.backward()
+    return dict(o=_np(o), S_last=_np(Sl), dq=_np(q_.grad), dk=_np(k_.grad),
+                dv=_np(v_.grad), dS0=_np(S0_.grad))
+
+
+def delta_rule_grads(q, k, v, beta, done, S0, do, dS_last=None):
+    """Returns dict(o, S_last, dq, dk, dv, dbeta, dS0)."""
+    q_, k_, v_, b_ = _t(q, True), _t(k, True), _t(v, True), _t(beta, True)
+    B, T, H, dk = q_.shape
+    S0_ = _t(np.zeros((B, H, v_.shape[-1], dk)) if S0 is None else S0, True)
+    o, Sl = delta_rule_t(q_, k_, v_, b_, _done(done), S0_)
+    L = (o * _t(do)).sum()
+    if dS_last is not None:
+        L = L + (Sl * _t(dS_last)).sum()
+    L.backward()
+    return dict(o=_np(o), S_last=_np(Sl), dq=_np(q_.grad), dk=_np(k_.grad),
+                dv=_np(v_.grad), dbeta=_np(b_.grad), dS0=_np(S0_.grad))

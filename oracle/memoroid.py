@@ -1,0 +1,513 @@
+"""NumPy fp64 restatement of the reference's sequence-model hot path.
+
+TEST INFRASTRUCTURE: imported only by tests, smoke() and bench.py's cpu_baseline.
+
+Reference anchors (paths relative to the reference tree):
+
+* reset-aware associative scan ........ memorax/networks/sequence_models/memoroid.py:60-91
+* reset broadcasting / slicing ......... memorax/utils/axes.py:19-32,64-77
+* diagonal algebra ..................... lru.py:92-95, s5.py:133-136, mamba.py:119-122
+* MinGRU log-space algebra ............. min_gru.py:49-78
+* linear attention (phi = elu+1) ....... linear_attention.py:58-117
+* DeltaNet delta rule .................. not in the reference; specified by
+  S_t = S_{t-1}(I - beta_t k_t k_t^T) + beta_t v_t k_t^T, o_t = S_t q_t.
+
+Conventions: arrays are (B, T, ...) with time on axis 1; carries have a size-1
+time axis (B, 1, ...) like the reference's ``initialize_carry``; ``done`` is
+(B, T), nonzero meaning "step t starts a new episode: clear the carry before
+step t consumes its input".  The matrix state is d_v x d_k (``S[i, j] = v_i k_j``,
+linear_attention.py:78).
+"""
+from __future__ import annotations
+
+import numpy as np
+
+# --------------------------------------------------------------------------
+# axes helpers (memorax/utils/axes.py:19-32,64-67)
+# --------------------------------------------------------------------------
+
+
+def tail(x):
+    return x[:, 1:]
+
+
+def last(x):
+    return x[:, -1:]
+
+
+def broadcast_done(done, carry):
+    """axes.py:64-67: append feature axes to ``done`` until ranks match."""
+    while done.ndim != carry.ndim:
+        done = done[..., None] if done.ndim < carry.ndim else done[..., 0]
+    return done
+
+
+# --------------------------------------------------------------------------
+# cell algebras: binary_operator(a=left/earlier, b=right/later)
+# --------------------------------------------------------------------------
+
+
+def diag_operator(a, b):
+    """lru.py:92-95 / s5.py:133-136 / mamba.py:119-122."""
+    state_i, decay_i = a
+    state_j, decay_j = b
+    return (decay_j * state_i + state_j, decay_j * decay_i)
+
+
+def mingru_operator(a, b):
+    """min_gru.py:67-74 (log space)."""
+    ls_i, d_i = a
+    ls_j, d_j = b
+    return (np.logaddexp(d_j + ls_i, ls_j), d_i + d_j)
+
+
+def additive_operator(a, b):
+    """linear_attention.py:82-86."""
+    return tuple(x + y for x, y in zip(a, b))
+
+
+def delta_operator(a, b):
+    """Affine-map composition for the delta rule written in the reference's
+    idiom: element (Bm, Am) stands for S -> S @ Am + Bm."""
+    B_i, A_i = a
+    B_j, A_j = b
+    return (B_i @ A_j + B_j, A_i @ A_j)
+
+
+# --------------------------------------------------------------------------
+# Memoroid.scan_fn, two independent formulations
+# --------------------------------------------------------------------------
+
+
+def _augmented(op):
+    """memoroid.py:72-85: ((carry, reset) x (carry, reset)) -> (carry, reset);
+    the right element wins by *select* when its reset flag is set."""
+
+    def aug(lhs, rhs):
+        lc, lr = lhs
+        rc, rr = rhs
+        comb = op(lc, rc)
+        out = tuple(
+            np.where(broadcast_done(rr, r) != 0, r, c) for r, c in zip(rc, comb)
+        )
+        return out, np.maximum(lr, rr)
+
+    return aug
+
+
+def _prepend(z, initial_carry, done):
+    """memoroid.py:61-68: carry becomes slot 0 with reset flag 0."""
+    zz = tuple(np.concatenate([c, e], axis=1) for c, e in zip(initial_carry, z))
+    done = np.asarray(done, dtype=np.float64)
+    reset = np.concatenate([np.zeros((done.shape[0], 1)), done], axis=1)[..., None]
+    return zz, reset
+
+
+def scan_fn_sequential(z, initial_carry, done, op):
+    """Left fold with select-style reset: h_j = reset_j ? z_j : op(h_{j-1}, z_j).
+
+    Returns (h, next_carry) like memoroid.py:87-91 (h has the carry slot removed).
+    """
+    zz, reset = _prepend(z, initial_carry, done)
+    n = reset.shape[1]
+    cur = tuple(x[:, 0:1] for x in zz)
+    outs = [cur]
+    for j in range(1, n):
+        nxt = tuple(x[:, j : j + 1] for x in zz)
+        with np.errstate(all="ignore"):
+            comb = op(cur, nxt)
+        r = reset[:, j : j + 1]
+        cur = tuple(
+            np.where(broadcast_done(r, e) != 0, e, c) for e, c in zip(nxt, comb)
+        )
+        outs.append(cur)
+    h = tuple(np.concatenate([o[i] for o in outs], axis=1) for i in range(len(zz)))
+    return tuple(tail(x) for x in h), tuple(last(x) for x in h)
+
+
+def scan_fn_tree(z, initial_carry, done, op):
+    """Inclusive scan with the augmented operator applied in Hillis-Steele
+    (doubling) order: a different association order from the sequential fold,
+    as jax.lax.associative_scan's is (memoroid.py:87)."""
+    zz, reset = _prepend(z, initial_carry, done)
+    aug = _augmented(op)
+    n = reset.shape[1]
+    cur, cur_r = zz, reset
+    shift = 1
+    while shift < n:
+        left = (tuple(x[:, :-shift] for x in cur), cur_r[:, :-shift])
+        right = (tuple(x[:, shift:] for x in cur), cur_r[:, shift:])
+        with np.errstate(all="ignore"):
+            comb, comb_r = aug(left, right)
+        cur = tuple(
+            np.concatenate([x[:, :shift], c], axis=1) for x, c in zip(cur, comb)
+        )
+        cur_r = np.concatenate([cur_r[:, :shift], comb_r], axis=1)
+        shift *= 2
+    return tuple(tail(x) for x in cur), tuple(last(x) for x in cur)
+
+
+# --------------------------------------------------------------------------
+# diagonal linear recurrence  h_t = a_t * h_{t-1} + b_t   (config 1)
+# --------------------------------------------------------------------------
+
+
+def diag_scan(a, b, done, h0=None, P0=None):
+    """Direct sequential definition (formulation independent of scan_fn_*).
+
+    h_t = done_t ? b_t : a_t h_{t-1} + b_t ;  P_t = done_t ? a_t : a_t P_{t-1}.
+    ``a`` may be (B,T,D) or broadcastable ((D,) time-invariant, lru.py:86).
+    Returns (h (B,T,D), h_last (B,D), P_last (B,D)).
+    """
+    b = np.asarray(b)
+    B, T, D = b.shape
+    dt = np.result_type(np.asarray(a).dtype, b.dtype, np.float64)
+    a = np.broadcast_to(np.asarray(a, dtype=dt), (B, T, D))
+    b = b.astype(dt)
+    h = np.zeros((B, D), dt) if h0 is None else np.asarray(h0, dtype=dt).copy()
+    P = np.ones((B, D), dt) if P0 is None else np.asarray(P0, dtype=dt).copy()
+    done = np.asarray(done) != 0
+    out = np.empty((B, T, D), dt)
+    for t in range(T):
+        r = done[:, t][:, None]
+        with np.errstate(all="ignore"):
+            hn = a[:, t] * h + b[:, t]
+            Pn = a[:, t] * P
+        h = np.where(r, b[:, t], hn)
+        P = np.where(r, a[:, t], Pn)
+        out[:, t] = h
+    return out, h, P
+
+
+def diag_scan_bwd(a, h, done, g, h0=None, g_last=None):
+    """Analytic reverse scan for the real diagonal recurrence.
+
+    lam_t = g_t + abar_{t+1} lam_{t+1},  abar_t = done_t ? 0 : a_t,
+    db_t = lam_t,  da_t = done_t ? 0 : lam_t h_{t-1},  dh0 = abar_1 lam_1.
+    For complex inputs the conjugate convention of torch.autograd is used
+    (lam_t = g_t + conj(abar_{t+1}) lam_{t+1}, da_t = lam_t conj(h_{t-1})).
+    Returns (da, db, dh0).
+    """
+    g = np.asarray(g)
+    B, T, D = g.shape
+    dt = np.result_type(np.asarray(a).dtype, g.dtype, np.float64)
+    a = np.broadcast_to(np.asarray(a, dtype=dt), (B, T, D))
+    h = np.asarray(h, dtype=dt)
+    hprev0 = np.zeros((B, D), dt) if h0 is None else np.asarray(h0, dtype=dt)
+    done = np.asarray(done) != 0
+    lam = np.zeros((B, D), dt) if g_last is None else np.asarray(g_last, dtype=dt).copy()
+    da = np.empty((B, T, D), dt)
+    db = np.empty((B, T, D), dt)
+    abar_next = np.zeros((B, D), dt)
+    first = True
+    for t in range(T - 1, -1, -1):
+        if first:
+            lam = g[:, t] + lam
+            first = False
+        else:
+            lam = g[:, t] + np.conj(abar_next) * lam
+        r = done[:, t][:, None]
+        hp = h[:, t - 1] if t > 0 else hprev0
+        db[:, t] = lam
+        da[:, t] = np.where(r, 0, lam * np.conj(hp))
+        abar_next = np.where(r, 0, a[:, t])
+    dh0 = np.conj(abar_next) * lam
+    return da, db, dh0
+
+
+# --------------------------------------------------------------------------
+# MinGRU (min_gru.py:49-78)
+# --------------------------------------------------------------------------
+
+
+def softplus(x):
+    return np.logaddexp(0.0, x)
+
+
+def sigmoid(x):
+    return 1.0 / (1.0 + np.exp(-x))
+
+
+def mingru_elements(z, h_tilde):
+    """min_gru.py:52-65: per-step (log_state, decay) from the two projections."""
+    z = np.asarray(z, dtype=np.float64)
+    h_tilde = np.asarray(h_tilde, dtype=np.float64)
+    log_z = -softplus(-z)
+    with np.errstate(all="ignore"):
+        log_h = np.where(
+            h_tilde >= 0, np.log(np.maximum(h_tilde, 0) + 0.5), -softplus(-h_tilde)
+        )
+    return (log_z + log_h, -softplus(z))
+
+
+def mingru_linear_coeffs(z, h_tilde):
+    """Linear-space equivalent: h_t = sigma(-z) h_{t-1} + sigma(z) g(h~)."""
+    z = np.asarray(z, dtype=np.float64)
+    h_tilde = np.asarray(h_tilde, dtype=np.float64)
+    gfun = np.where(h_tilde >= 0, np.maximum(h_tilde, 0) + 0.5, sigmoid(h_tilde))
+    return sigmoid(-z), sigmoid(z) * gfun
+
+
+def mingru_scan(z, h_tilde, done, carry=None):
+    """MinGRU through the reference's own route: log-space elements + scan_fn
+    + read (exp).  carry = (log_state (B,1,F), decay (B,1,F)); default is the
+    reference's (-inf, 0) (min_gru.py:80-90).  Returns (next_carry, h)."""
+    el = mingru_elements(z, h_tilde)
+    B, T, F = el[0].shape
+    if carry is None:
+        carry = (np.full((B, 1, F), -np.inf), np.zeros((B, 1, F)))
+    hs, nxt = scan_fn_sequential(el, carry, done, mingru_operator)
+    return nxt, np.exp(hs[0])
+
+
+# --------------------------------------------------------------------------
+# linear attention (linear_attention.py:58-117)
+# --------------------------------------------------------------------------
+
+
+def elu1(x):
+    """linear_attention.py:58-60."""
+    x = np.asarray(x, dtype=np.float64)
+    return np.where(x > 0, x + 1.0, np.exp(np.minimum(x, 0)))
+
+
+def _fmap(x, feature_map):
+    if feature_map in (None, "none", 0):
+        return np.asarray(x, dtype=np.float64)
+    if feature_map in ("elu1", 1):
+        return elu1(x)
+    raise ValueError(feature_map)
+
+
+def linear_attention(q, k, v, done, S0=None, feature_map="none"):
+    """Recurrent form.  S_t = r_t S_{t-1} + v_t k_t^T ; o_t = S_t q_t.
+
+    q,k: (B,T,H,dk), v: (B,T,H,dv), S0: (B,H,dv,dk).  Unnormalised numerator
+    (linear_attention.py:105).  Returns (o (B,T,H,dv), S_last (B,H,dv,dk)).
+    """
+    q = _fmap(q, feature_map)
+    k = _fmap(k, feature_map)
+    v = np.asarray(v, dtype=np.float64)
+    B, T, H, dk = q.shape
+    dv = v.shape[-1]
+    S = np.zeros((B, H, dv, dk)) if S0 is None else np.asarray(S0, np.float64).copy()
+    done = np.asarray(done) != 0
+    o = np.empty((B, T, H, dv))
+    for t in range(T):
+        r = done[:, t][:, None, None, None]
+        S = np.where(r, 0.0, S)
+        S = S + np.einsum("bhi,bhj->bhij", v[:, t], k[:, t])
+        o[:, t] = np.einsum("bhij,bhj->bhi", S, q[:, t])
+    return o, S
+
+
+def linear_attention_memoroid(q, k, v, done, carry=None, feature_map="none"):
+    """The reference's own route (linear_attention.py:62-117 + memoroid.py:60-91):
+    materialise per-step outer products, scan (S, z) additively, read
+    numerator and denominator.  Returns (next_carry, numerator, denominator)."""
+    q = _fmap(q, feature_map)
+    k = _fmap(k, feature_map)
+    v = np.asarray(v, dtype=np.float64)
+    B, T, H, dk = q.shape
+    dv = v.shape[-1]
+    S = np.einsum("bthi,bthj->bthij", v, k)
+    if carry is None:
+        carry = (np.zeros((B, 1, H, dv, dk)), np.zeros((B, 1, H, dk)))
+    (Sc, zc), nxt = scan_fn_tree((S, k), carry, done, additive_operator)
+    num = np.einsum("bthij,bthj->bthi", Sc, q)
+    den = np.einsum("bthi,bthi->bth", q, zc)
+    return nxt, num, den
+
+
+def segment_ids(done):
+    """Inclusive cumsum of done along time: rows with equal id share an episode."""
+    return np.cumsum(np.asarray(done) != 0, axis=1)
+
+
+def linear_attention_quadratic(q, k, v, done, S0=None, feature_map="none"):
+    """Textbook masked-matmul form: o = ((Q K^T) * tril * M) V + m * (Q S0^T)."""
+    q = _fmap(q, feature_map)
+    k = _fmap(k, feature_map)
+    v = np.asarray(v, dtype=np.float64)
+    B, T, H, dk = q.shape
+    seg = segment_ids(done)
+    M = (seg[:, :, None] == seg[:, None, :]) & np.tril(np.ones((T, T), bool))[None]
+    A = np.einsum("bihd,bjhd->bhij", q, k) * M[:, None]
+    o = np.einsum("bhij,bjhe->bihe", A, v)
+    if S0 is not None:
+        m = (seg == 0)[:, :, None, None]
+        o = o + m * np.einsum("bihd,bhed->bihe", q, np.asarray(S0, np.float64))
+    return o
+
+
+def linear_attention_chunked(q, k, v, done, S0=None, feature_map="none", chunk=64):
+    """Chunk form with per-chunk masks M, m, l, e computed from the cumsum of
+    done *within* the chunk: O = diag(m) Q S^T + (tril(QK^T)*M) V ;
+    S <- l S + (diag(e) V)^T K."""
+    q = _fmap(q, feature_map)
+    k = _fmap(k, feature_map)
+    v = np.asarray(v, dtype=np.float64)
+    B, T, H, dk = q.shape
+    dv = v.shape[-1]
+    S = np.zeros((B, H, dv, dk)) if S0 is None else np.asarray(S0, np.float64).copy()
+    done = np.asarray(done) != 0
+    o = np.empty((B, T, H, dv))
+    for c0 in range(0, T, chunk):
+        c1 = min(T, c0 + chunk)
+        C = c1 - c0
+        seg = np.cumsum(done[:, c0:c1], axis=1)
+        M = (seg[:, :, None] == seg[:, None, :]) & np.tril(np.ones((C, C), bool))[None]
+        m = (seg == 0).astype(np.float64)
+        e = (seg == seg[:, -1:]).astype(np.float64)
+        l = (seg[:, -1] == 0).astype(np.float64)
+        Q, K, V = q[:, c0:c1], k[:, c0:c1], v[:, c0:c1]
+        A = np.einsum("bihd,bjhd->bhij", Q, K) * M[:, None]
+        O = np.einsum("bhij,bjhe->bihe", A, V)
+        O = O + m[:, :, None, None] * np.einsum("bihd,bhed->bihe", Q, S)
+        o[:, c0:c1] = O
+        S = l[:, None, None, None] * S + np.einsum(
+            "bjhe,bjhd->bhed", V * e[:, :, None, None], K
+        )
+    return o, S
+
+
+# --------------------------------------------------------------------------
+# DeltaNet delta rule (config 4)
+# --------------------------------------------------------------------------
+
+
+def delta_rule(q, k, v, beta, done, S0=None):
+    """Sequential u-form.  S' = r_t S_{t-1}; u_t = beta_t (v_t - S' k_t);
+    S_t = S' + u_t k_t^T ; o_t = S_t q_t.   beta: (B,T,H)."""
+    q = np.asarray(q, np.float64)
+    k = np.asarray(k, np.float64)
+    v = np.asarray(v, np.float64)
+    beta = np.asarray(beta, np.float64)
+    B, T, H, dk = q.shape
+    dv = v.shape[-1]
+    S = np.zeros((B, H, dv, dk)) if S0 is None else np.asarray(S0, np.float64).copy()
+    done = np.asarray(done) != 0
+    o = np.empty((B, T, H, dv))
+    for t in range(T):
+        r = done[:, t][:, None, None, None]
+        S = np.where(r, 0.0, S)
+        u = beta[:, t][..., None] * (v[:, t] - np.einsum("bhij,bhj->bhi", S, k[:, t]))
+        S = S + np.einsum("bhi,bhj->bhij", u, k[:, t])
+        o[:, t] = np.einsum("bhij,bhj->bhi", S, q[:, t])
+    return o, S
+
+
+def delta_rule_explicit(q, k, v, beta, done, S0=None):
+    """Literal S_t = S_{t-1}(I - beta k k^T) + beta v k^T with select reset."""
+    q = np.asarray(q, np.float64)
+    k = np.asarray(k, np.float64)
+    v = np.asarray(v, np.float64)
+    beta = np.asarray(beta, np.float64)
+    B, T, H, dk = q.shape
+    dv = v.shape[-1]
+    S = np.zeros((B, H, dv, dk)) if S0 is None else np.asarray(S0, np.float64).copy()
+    done = np.asarray(done) != 0
+    eye = np.eye(dk)
+    o = np.empty((B, T, H, dv))
+    for t in range(T):
+        bt = beta[:, t][..., None, None]
+        A = eye - bt * np.einsum("bhi,bhj->bhij", k[:, t], k[:, t])
+        Bm = bt * np.einsum("bhi,bhj->bhij", v[:, t], k[:, t])
+        Sn = S @ A + Bm
+        S = np.where(done[:, t][:, None, None, None], Bm, Sn)
+        o[:, t] = np.einsum("bhij,bhj->bhi", S, q[:, t])
+    return o, S
+
+
+def delta_rule_memoroid(q, k, v, beta, done, S0=None):
+    """The delta rule pushed through the reference's scan_fn with the affine
+    pair algebra (element (B_t, A_t)); O(T d^2) memory, tiny shapes only."""
+    q = np.asarray(q, np.float64)
+    k = np.asarray(k, np.float64)
+    v = np.asarray(v, np.float64)
+    beta = np.asarray(beta, np.float64)[..., None, None]
+    B, T, H, dk = q.shape
+    dv = v.shape[-1]
+    Am = np.eye(dk) - beta * np.einsum("bthi,bthj->bthij", k, k)
+    Bm = beta * np.einsum("bthi,bthj->bthij", v, k)
+    S0 = np.zeros((B, H, dv, dk)) if S0 is None else np.asarray(S0, np.float64)
+    carry = (S0[:, None], np.broadcast_to(np.eye(dk), (B, 1, H, dk, dk)).copy())
+    (Sc, _), nxt = scan_fn_tree((Bm, Am), carry, done, delta_operator)
+    o = np.einsum("bthij,bthj->bthi", Sc, q)
+    return o, nxt[0][:, 0]
+
+
+def delta_rule_chunked(q, k, v, beta, done, S0=None, chunk=64):
+    """WY / UT-transform chunk form with resets:
+    A = tril(diag(beta)(K K^T * M), -1);  Tm = (I + A)^-1 diag(beta);
+    W = Tm K; U = Tm V; U' = U - diag(m) W S^T;
+    O = diag(m) Q S^T + (tril(Q K^T) * M) U';  S <- l S + (diag(e) U')^T K."""
+    q = np.asarray(q, np.float64)
+    k = np.asarray(k, np.float64)
+    v = np.asarray(v, np.float64)
+    beta = np.asarray(beta, np.float64)
+    B, T, H, dk = q.shape
+    dv = v.shape[-1]
+    S = np.zeros((B, H, dv, dk)) if S0 is None else np.asarray(S0, np.float64).copy()
+    done = np.asarray(done) != 0
+    o = np.empty((B, T, H, dv))
+    for c0 in range(0, T, chunk):
+        c1 = min(T, c0 + chunk)
+        C = c1 - c0
+        seg = np.cumsum(done[:, c0:c1], axis=1)
+        tril = np.tril(np.ones((C, C), bool))
+        M = (seg[:, :, None] == seg[:, None, :]) & tril[None]
+        m = (seg == 0).astype(np.float64)
+        e = (seg == seg[:, -1:]).astype(np.float64)
+        l = (seg[:, -1] == 0).astype(np.float64)
+        Q, K, V, bt = q[:, c0:c1], k[:, c0:c1], v[:, c0:c1], beta[:, c0:c1]
+        KK = np.einsum("bihd,bjhd->bhij", K, K) * M[:, None]
+        A = np.tril(np.einsum("bih,bhij->bhij", bt, KK), -1)
+        Tm = np.linalg.inv(np.eye(C) + A) * np.transpose(bt, (0, 2, 1))[:, :, None, :]
+        W = np.einsum("bhij,bjhd->bihd", Tm, K)
+        U = np.einsum("bhij,bjhe->bihe", Tm, V)
+        Up = U - m[:, :, None, None] * np.einsum("bihd,bhed->bihe", W, S)
+        Aqk = np.einsum("bihd,bjhd->bhij", Q, K) * M[:, None]
+        O = m[:, :, None, None] * np.einsum("bihd,bhed->bihe", Q, S)
+        O = O + np.einsum("bhij,bjhe->bihe", Aqk, Up)
+        o[:, c0:c1] = O
+        S = l[:, None, None, None] * S + np.einsum(
+            "bjhe,bjhd->bhed", Up * e[:, :, None, None], K
+        )
+    return o, S
+
+
+# --------------------------------------------------------------------------
+# seeded synthetic inputs for the benchmark configurations
+# --------------------------------------------------------------------------
+
+
+def make_inputs(cfg, shape=None, seed=None):
+    """Seeded fp32 inputs for configuration ``cfg`` (1..4); ``shape`` overrides
+    the default sizes.  done = rng.random((B,T)) < p."""
+    rng = np.random.default_rng(1000 + cfg if seed is None else seed)
+    if cfg == 1:
+        B, T, D = shape or (32, 128, 256)
+        a = rng.uniform(0.9, 0.999, (B, T, D)).astype(np.float32)
+        b = rng.standard_normal((B, T, D)).astype(np.float32)
+        done = rng.random((B, T)) < 0.01
+        return dict(a=a, b=b, done=done)
+    if cfg in (2, 3):
+        B, T, H, d = shape or ((64, 256, 4, 64) if cfg == 2 else (256, 4096, 8, 64))
+        q, k, v = (
+            (rng.standard_normal((B, T, H, d)) / np.sqrt(64)).astype(np.float32)
+            for _ in range(3)
+        )
+        p = 0.005 if cfg == 2 else 0.0
+        done = rng.random((B, T)) < p
+        return dict(q=q, k=k, v=v, done=done)
+    if cfg == 4:
+        B, T, H, d = shape or (64, 1024, 8, 64)
+        q = rng.standard_normal((B, T, H, d)).astype(np.float32)
+        k = rng.standard_normal((B, T, H, d)).astype(np.float32)
+        k /= np.linalg.norm(k, axis=-1, keepdims=True)
+        v = rng.standard_normal((B, T, H, d)).astype(np.float32)
+        beta = (1.0 / (1.0 + np.exp(-rng.standard_normal((B, T, H))))).astype(np.float32)
+        done = rng.random((B, T)) < 0.002
+        return dict(q=q, k=k, v=v, beta=beta, done=done)
+    raise ValueError(cfg)

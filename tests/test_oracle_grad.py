@@ -1,0 +1,103 @@
+"""Pins the gradient oracle: torch-fp64 autograd vs central finite differences on
+the NumPy forward, and vs the analytic reverse-scan formulas."""
+import numpy as np
+import pytest
+
+from oracle import grad as G
+from oracle import memoroid as M
+
+RNG = np.random.default_rng(11)
+
+
+def rnd(*s):
+    return RNG.standard_normal(s)
+
+
+def fd(f, x, eps=1e-6):
+    """Central finite-difference gradient of scalar f at x."""
+    g = np.zeros_like(x)
+    it = np.nditer(x, flags=["multi_index"])
+    for _ in it:
+        i = it.multi_index
+        old = x[i]
+        x[i] = old + eps
+        fp = f()
+        x[i] = old - eps
+        fm = f()
+        x[i] = old
+        g[i] = (fp - fm) / (2 * eps)
+    return g
+
+
+def test_diag_grads_fd_and_analytic():
+    B, T, D = 2, 9, 2
+    a, b, h0 = RNG.uniform(0.5, 1, (B, T, D)), rnd(B, T, D), rnd(B, D)
+    g, gl = rnd(B, T, D), rnd(B, D)
+    d = np.zeros((B, T), bool)
+    d[0, 4] = True
+    d[1, 0] = True
+
+    def L():
+        h, hl, _ = M.diag_scan(a, b, d, h0)
+        return (h * g).sum() + (hl * gl).sum()
+
+    ag = G.diag_scan_grads(a, b, d, h0, g, gl)
+    np.testing.assert_allclose(ag["da"], fd(L, a), rtol=1e-6, atol=1e-8)
+    np.testing.assert_allclose(ag["db"], fd(L, b), rtol=1e-6, atol=1e-8)
+    np.testing.assert_allclose(ag["dh0"], fd(L, h0), rtol=1e-6, atol=1e-8)
+    h, _, _ = M.diag_scan(a, b, d, h0)
+    da, db, dh0 = M.diag_scan_bwd(a, h, d, g, h0, gl)
+    np.testing.assert_allclose(da, ag["da"], rtol=1e-12, atol=1e-13)
+    np.testing.assert_allclose(db, ag["db"], rtol=1e-12, atol=1e-13)
+    np.testing.assert_allclose(dh0, ag["dh0"], rtol=1e-12, atol=1e-13)
+
+
+def test_diag_grads_complex_analytic_matches_autograd():
+    B, T, D = 2, 8, 3
+    a = 0.9 * np.exp(1j * RNG.uniform(0, 3, (B, T, D)))
+    b, h0 = rnd(B, T, D) + 1j * rnd(B, T, D), rnd(B, D) + 1j * rnd(B, D)
+    g = rnd(B, T, D) + 1j * rnd(B, T, D)
+    d = RNG.random((B, T)) < 0.2
+    ag = G.diag_scan_grads(a, b, d, h0, g)
+    h, _, _ = M.diag_scan(a, b, d, h0)
+    da, db, dh0 = M.diag_scan_bwd(a, h, d, g, h0)
+    np.testing.assert_allclose(da, ag["da"], rtol=1e-12, atol=1e-13)
+    np.testing.assert_allclose(db, ag["db"], rtol=1e-12, atol=1e-13)
+    np.testing.assert_allclose(dh0, ag["dh0"], rtol=1e-12, atol=1e-13)
+
+
+@pytest.mark.parametrize("fmap", ["none", "elu1"])
+def test_linear_attention_grads_fd(fmap):
+    B, T, H, dk, dv = 1, 7, 1, 3, 2
+    q, k, v, S0 = rnd(B, T, H, dk), rnd(B, T, H, dk), rnd(B, T, H, dv), rnd(B, H, dv, dk)
+    do, dSl = rnd(B, T, H, dv), rnd(B, H, dv, dk)
+    d = np.zeros((B, T), bool)
+    d[0, 3] = True
+
+    def L():
+        o, Sl = M.linear_attention(q, k, v, d, S0, fmap)
+        return (o * do).sum() + (Sl * dSl).sum()
+
+    ag = G.linear_attention_grads(q, k, v, d, S0, do, dSl, fmap)
+    for name, x in (("dq", q), ("dk", k), ("dv", v), ("dS0", S0)):
+        np.testing.assert_allclose(ag[name], fd(L, x), rtol=1e-6, atol=1e-8, err_msg=name)
+    o, Sl = M.linear_attention(q, k, v, d, S0, fmap)
+    np.testing.assert_allclose(ag["o"], o, rtol=1e-12)
+    np.testing.assert_allclose(ag["S_last"], Sl, rtol=1e-12)
+
+
+def test_delta_rule_grads_fd():
+    B, T, H, dk, dv = 1, 7, 1, 3, 2
+    q, k, v, S0 = rnd(B, T, H, dk), rnd(B, T, H, dk), rnd(B, T, H, dv), rnd(B, H, dv, dk)
+    beta = M.sigmoid(rnd(B, T, H))
+    do, dSl = rnd(B, T, H, dv), rnd(B, H, dv, dk)
+    d = np.zeros((B, T), bool)
+    d[0, 4] = True
+
+    def L():
+        o, Sl = M.delta_rule(q, k, v, beta, d, S0)
+        return (o * do).sum() + (Sl * dSl).sum()
+
+    ag = G.delta_rule_grads(q, k, v, beta, d, S0, do, dSl)
+    for name, x in (("dq", q), ("dk", k), ("dv", v), ("dbeta", beta), ("dS0", S0)):
+        np.testing.assert_allclose(ag[name], fd(L, x), rtol=1e-6, atol=1e-8, err_msg=name)
