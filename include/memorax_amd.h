@@ -1,0 +1,137 @@
+/* memorax_amd.h — C ABI of the MI355X (gfx950) sequence-model kernels.
+ *
+ * The reference (memory-rl/memorax) is pure Python/JAX and has no FFI for this
+ * path; each entry point below replaces the arithmetic that the cited
+ * reference code performs through jax.lax.associative_scan, and is what an
+ * XLA-FFI / ctypes binding for that code would bind.
+ *
+ * Common rules
+ *  - Every pointer is a DEVICE pointer owned by the caller; outputs are
+ *    pre-allocated by the caller.  Nothing here allocates, frees, copies to the
+ *    host or synchronises: a call validates its arguments on the host, enqueues
+ *    kernels on `stream` (a hipStream_t passed as void*, NULL = default stream)
+ *    and returns.
+ *  - Return value: MRX_OK (0) or a negative mrx_status; never throws.
+ *    mrx_status_string() names a code.  Arguments are checked before any launch.
+ *  - Layouts are the reference's: time on axis 1, features last, row-major,
+ *    densely packed.  `done` is (B,T); nonzero at (b,t) clears the carried state
+ *    before step t consumes its input (select semantics, memoroid.py:79-83).
+ *  - Recurrent state (S, h, P) is always fp32 (or complex64 for MRX_C64 scans).
+ */
+#ifndef MEMORAX_AMD_H
+#define MEMORAX_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    MRX_OK = 0,
+    MRX_ERR_INVALID_ARG = -1, /* null pointer, non-positive size, bad enum, misalignment */
+    MRX_ERR_UNSUPPORTED = -2, /* valid request the kernels do not cover (e.g. head dim != 64) */
+    MRX_ERR_LAUNCH = -3       /* the HIP runtime rejected the launch */
+} mrx_status;
+
+typedef enum {
+    MRX_F32 = 0,  /* float32 */
+    MRX_BF16 = 1, /* bfloat16 inputs/outputs, fp32 state and accumulation */
+    MRX_C64 = 2   /* complex64 (interleaved re,im); diagonal scan only */
+} mrx_dtype;
+
+typedef enum {
+    MRX_DONE_U8 = 0, /* bool / uint8 */
+    MRX_DONE_F32 = 1 /* float32, nonzero = reset (memoroid.py:67 casts done to float) */
+} mrx_done_dtype;
+
+typedef enum {
+    MRX_FMAP_NONE = 0,
+    MRX_FMAP_ELU1 = 1 /* phi(x) = elu(x) + 1 applied to q and k (linear_attention.py:58-60) */
+} mrx_feature_map;
+
+const char *mrx_status_string(int status);
+
+/* Library version, major*10000 + minor*100 + patch. */
+int mrx_version(void);
+
+/* Time-chunk length the chunked kernels use for `dtype`; fixes the layout of the
+ * per-chunk state checkpoints S_chk: (B, H, ceil(T/chunk), dv, dk). */
+int64_t mrx_chunk_size(int dtype);
+
+/* ---- diagonal linear recurrence --------------------------------------------
+ * Replaces Memoroid.scan_fn (memoroid.py:60-91) driven by the diagonal algebra
+ * binary_operator of lru.py:92-95 / s5.py:133-136 / mamba.py:119-122:
+ *     h_t = done_t ? b_t : a_t * h_{t-1} + b_t
+ *     P_t = done_t ? a_t : a_t * P_{t-1}          (cumulative-decay leaf)
+ * a: (B,T,D), or (D,) when a_time_invariant != 0 (LRU/S5 broadcast lambda,
+ * lru.py:86, never materialised here).  b,h: (B,T,D).  h0,P0 (nullable: 0 and 1),
+ * h_last,P_last (nullable: not written): (B,D).  dtype: MRX_F32 or MRX_C64. */
+int mrx_linear_scan_fwd(void *stream, const void *a, const void *b,
+                        const void *done, const void *h0, const void *P0,
+                        void *h, void *h_last, void *P_last, int64_t B,
+                        int64_t T, int64_t D, int dtype, int done_dtype,
+                        int a_time_invariant);
+
+/* Reverse scan of the same recurrence (what JAX autodiff of memoroid.py:87 yields):
+ *     lam_t = g_t + conj(abar_{t+1}) lam_{t+1},  abar_t = done_t ? 0 : a_t
+ *     db_t = lam_t ;  da_t = done_t ? 0 : lam_t conj(h_{t-1}) ;  dh0 = conj(abar_0) lam_0
+ * (conj is the identity for MRX_F32; for MRX_C64 cotangents follow the
+ * torch.autograd convention, the complex conjugate of JAX's).
+ * h is the forward output; g = dL/dh (B,T,D); g_last = dL/dh_last (B,D, nullable).
+ * da is per step (B,T,D) even when a is time-invariant (the caller reduces). */
+int mrx_linear_scan_bwd(void *stream, const void *a, const void *h,
+                        const void *done, const void *h0, const void *g,
+                        const void *g_last, void *da, void *db, void *dh0,
+                        int64_t B, int64_t T, int64_t D, int dtype,
+                        int done_dtype, int a_time_invariant);
+
+/* ---- causal linear attention, chunked ---------------------------------------
+ * Replaces LinearAttentionCell.__call__ / binary_operator / read numerator
+ * (linear_attention.py:62-86,105) scanned by memoroid.py:60-91, without
+ * materialising the per-step state:
+ *     S_t = (done_t ? 0 : S_{t-1}) + v_t phi(k_t)^T ;   o_t = S_t phi(q_t)
+ * q,k: (B,T,H,dk); v,o: (B,T,H,dv) in `dtype` (MRX_F32 or MRX_BF16).
+ * S0 (nullable = 0), S_last (nullable): (B,H,dv,dk) fp32.
+ * S_chk (nullable): (B,H,ceil(T/chunk),dv,dk) in `dtype`, receives the state
+ * entering each chunk; required by the backward call.  dk = dv = 64. */
+int mrx_linear_attn_fwd(void *stream, const void *q, const void *k,
+                        const void *v, const void *done, const void *S0,
+                        void *o, void *S_last, void *S_chk, int64_t B,
+                        int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
+                        int done_dtype, int feature_map);
+
+/* Gradients of the above w.r.t. q,k,v (pre-feature-map) and S0, given
+ * dout = dL/do (B,T,H,dv) and dS_last = dL/dS_last (nullable).
+ * dq,dk,dv in `dtype`; dS0 (nullable) fp32. */
+int mrx_linear_attn_bwd(void *stream, const void *q, const void *k,
+                        const void *v, const void *done, const void *S_chk,
+                        const void *dout, const void *dS_last, void *dq,
+                        void *dk_out, void *dv_out, void *dS0, int64_t B,
+                        int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
+                        int done_dtype, int feature_map);
+
+/* ---- DeltaNet delta rule, chunked WY/UT form --------------------------------
+ * No counterpart in the reference; written in its cell idiom it would be a
+ * MemoroidCellBase scanned by memoroid.py:60-91 with elements
+ * (beta v k^T, I - beta k k^T):
+ *     S' = done_t ? 0 : S_{t-1} ;  S_t = S'(I - beta_t k_t k_t^T) + beta_t v_t k_t^T ;
+ *     o_t = S_t q_t
+ * beta: (B,T,H) in `dtype`; other arguments as for linear attention. */
+int mrx_delta_rule_fwd(void *stream, const void *q, const void *k,
+                       const void *v, const void *beta, const void *done,
+                       const void *S0, void *o, void *S_last, void *S_chk,
+                       int64_t B, int64_t T, int64_t H, int64_t dk, int64_t dv,
+                       int dtype, int done_dtype);
+
+int mrx_delta_rule_bwd(void *stream, const void *q, const void *k,
+                       const void *v, const void *beta, const void *done,
+                       const void *S_chk, const void *dout, const void *dS_last,
+                       void *dq, void *dk_out, void *dv_out, void *dbeta,
+                       void *dS0, int64_t B, int64_t T, int64_t H, int64_t dk,
+                       int64_t dv, int dtype, int done_dtype);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MEMORAX_AMD_H */

@@ -1,0 +1,473 @@
+// Diagonal linear-recurrence scan for gfx950:  h_t = done_t ? b_t : a_t h_{t-1} + b_t.
+//
+// The op is pure streaming (2 loads + 1 store per element forward, 3 + 2 backward),
+// so the design is about HBM: lanes lie along the contiguous feature axis
+// (one wave row = 64 lanes x 16 B), each lane walks time in registers, and when
+// the (batch x feature) extent alone cannot fill 256 CUs the time axis is split
+// over the waves of a workgroup: every wave scans its slice from the identity,
+// per-wave summaries (P, h, reset-seen) meet in LDS, each wave folds the
+// summaries to its left into a carry-in and fixes its slice up by *select*
+// (a reset inside the slice wins over the carry, so NaN/Inf never cross a reset).
+// One pass over HBM in either case.
+#include "common.h"
+
+namespace {
+
+using namespace mrx;
+
+struct c64 {
+    float re, im;
+};
+
+template <typename E> struct Ops;
+template <> struct Ops<float> {
+    static __device__ __forceinline__ float zero() { return 0.0f; }
+    static __device__ __forceinline__ float one() { return 1.0f; }
+    static __device__ __forceinline__ float conj(float a) { return a; }
+    // a * x + y
+    static __device__ __forceinline__ float madd(float a, float x, float y) { return a * x + y; }
+    static __device__ __forceinline__ float mul(float a, float x) { return a * x; }
+};
+template <> struct Ops<c64> {
+    static __device__ __forceinline__ c64 zero() { return {0.0f, 0.0f}; }
+    static __device__ __forceinline__ c64 one() { return {1.0f, 0.0f}; }
+    static __device__ __forceinline__ c64 conj(c64 a) { return {a.re, -a.im}; }
+    static __device__ __forceinline__ c64 madd(c64 a, c64 x, c64 y)
+    {
+        return {a.re * x.re - a.im * x.im + y.re, a.re * x.im + a.im * x.re + y.im};
+    }
+    static __device__ __forceinline__ c64 mul(c64 a, c64 x)
+    {
+        return {a.re * x.re - a.im * x.im, a.re * x.im + a.im * x.re};
+    }
+};
+
+template <typename E, int VEC> struct alignas(sizeof(E) * VEC) Vec {
+    E v[VEC];
+};
+
+template <typename E, int VEC> __device__ __forceinline__ Vec<E, VEC> vfill(E x)
+{
+    Vec<E, VEC> r;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) r.v[i] = x;
+    return r;
+}
+
+constexpr int TS = 8;  // time steps a wave holds in registers per super-step
+
+// Forward.  grid = B * tiles workgroups, block = 64 * NW threads.
+// smem: sH[2][NW][64] Vec, sP[2][NW][64] Vec, sF[2][NW] int.
+template <typename E, int VEC>
+__global__ void __launch_bounds__(512)
+diag_scan_fwd_kernel(const E *__restrict__ a, const E *__restrict__ b,
+                     const void *__restrict__ done, int done_f32,
+                     const E *__restrict__ h0, const E *__restrict__ P0,
+                     E *__restrict__ h, E *__restrict__ h_last,
+                     E *__restrict__ P_last, int T, int64_t D, int tiles, int NW,
+                     int a_ti)
+{
+    using V = Vec<E, VEC>;
+    using O = Ops<E>;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    V *sH = reinterpret_cast<V *>(smem_raw);
+    V *sP = sH + 2 * NW * 64;
+    int *sF = reinterpret_cast<int *>(sP + 2 * NW * 64);
+
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int tile = blockIdx.x % tiles;
+    const int64_t bi = blockIdx.x / tiles;
+    const int64_t col = ((int64_t)tile * 64 + lane) * VEC;
+    const bool act = col < D;
+    const int64_t row0 = bi * T;
+
+    V carry_h = vfill<E, VEC>(O::zero()), carry_p = vfill<E, VEC>(O::one());
+    if (act) {
+        if (h0) carry_h = *reinterpret_cast<const V *>(h0 + bi * D + col);
+        if (P0) carry_p = *reinterpret_cast<const V *>(P0 + bi * D + col);
+    }
+
+    const int span = NW * TS;
+    int buf = 0;
+    for (int t0 = 0; t0 < T; t0 += span) {
+        const int ts = t0 + w * TS;
+        V x[TS], p[TS];
+        unsigned rmask = 0;
+#pragma unroll
+        for (int s = 0; s < TS; ++s) {
+            const int t = ts + s;
+            if (t < T && act) {
+                const int64_t off = (row0 + t) * D + col;
+                p[s] = *reinterpret_cast<const V *>(a + (a_ti ? col : off));
+                x[s] = *reinterpret_cast<const V *>(b + off);
+            } else {
+                p[s] = vfill<E, VEC>(O::one());
+                x[s] = vfill<E, VEC>(O::zero());
+            }
+            if (t < T && done_at(done, done_f32, row0 + t)) rmask |= 1u << s;
+        }
+        if (NW == 1) {
+            // no time split: continue straight from the carry
+#pragma unroll
+            for (int s = 0; s < TS; ++s) {
+                const bool r = (rmask >> s) & 1u;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    const E hn = O::madd(p[s].v[i], carry_h.v[i], x[s].v[i]);
+                    const E pn = O::mul(p[s].v[i], carry_p.v[i]);
+                    carry_h.v[i] = r ? x[s].v[i] : hn;
+                    carry_p.v[i] = r ? p[s].v[i] : pn;
+                }
+                if (ts + s < T && act)
+                    *reinterpret_cast<V *>(h + (row0 + ts + s) * D + col) = carry_h;
+            }
+            continue;
+        }
+        // local inclusive scan from the identity; x <- h_local, p <- P_local
+        {
+            V hc = vfill<E, VEC>(O::zero()), pc = vfill<E, VEC>(O::one());
+#pragma unroll
+            for (int s = 0; s < TS; ++s) {
+                const bool r = (rmask >> s) & 1u;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    const E hn = O::madd(p[s].v[i], hc.v[i], x[s].v[i]);
+                    const E pn = O::mul(p[s].v[i], pc.v[i]);
+                    hc.v[i] = r ? x[s].v[i] : hn;
+                    pc.v[i] = r ? p[s].v[i] : pn;
+                }
+                x[s] = hc;
+                p[s] = pc;
+            }
+            sH[(buf * NW + w) * 64 + lane] = hc;
+            sP[(buf * NW + w) * 64 + lane] = pc;
+            if (lane == 0) sF[buf * NW + w] = rmask != 0;
+        }
+        __syncthreads();
+        // fold the summaries: carry-in of this wave, then the workgroup carry
+        V cin_h = carry_h, cin_p = carry_p, my_h = carry_h;
+        for (int j = 0; j < NW; ++j) {
+            if (j == w) my_h = cin_h;
+            const V Hj = sH[(buf * NW + j) * 64 + lane];
+            const V Pj = sP[(buf * NW + j) * 64 + lane];
+            const bool fj = sF[buf * NW + j] != 0;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                const E hn = O::madd(Pj.v[i], cin_h.v[i], Hj.v[i]);
+                const E pn = O::mul(Pj.v[i], cin_p.v[i]);
+                cin_h.v[i] = fj ? Hj.v[i] : hn;
+                cin_p.v[i] = fj ? Pj.v[i] : pn;
+            }
+        }
+        carry_h = cin_h;
+        carry_p = cin_p;
+#pragma unroll
+        for (int s = 0; s < TS; ++s) {
+            const bool seen = (rmask & ((2u << s) - 1u)) != 0;
+            V out;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                const E fx = O::madd(p[s].v[i], my_h.v[i], x[s].v[i]);
+                out.v[i] = seen ? x[s].v[i] : fx;
+            }
+            if (ts + s < T && act)
+                *reinterpret_cast<V *>(h + (row0 + ts + s) * D + col) = out;
+        }
+        buf ^= 1;
+    }
+    if (w == 0 && act) {
+        if (h_last) *reinterpret_cast<V *>(h_last + bi * D + col) = carry_h;
+        if (P_last) *reinterpret_cast<V *>(P_last + bi * D + col) = carry_p;
+    }
+}
+
+// Backward: the same scan walked from t = T-1 down with coefficient conj(a_{t+1}),
+// cut where done_{t+1}; reversed index r = T-1-t runs forward.
+template <typename E, int VEC>
+__global__ void __launch_bounds__(512)
+diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hfw,
+                     const void *__restrict__ done, int done_f32,
+                     const E *__restrict__ h0, const E *__restrict__ g,
+                     const E *__restrict__ g_last, E *__restrict__ da,
+                     E *__restrict__ db, E *__restrict__ dh0, int T, int64_t D,
+                     int tiles, int NW, int a_ti)
+{
+    using V = Vec<E, VEC>;
+    using O = Ops<E>;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    V *sH = reinterpret_cast<V *>(smem_raw);
+    V *sP = sH + 2 * NW * 64;
+    int *sF = reinterpret_cast<int *>(sP + 2 * NW * 64);
+
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int tile = blockIdx.x % tiles;
+    const int64_t bi = blockIdx.x / tiles;
+    const int64_t col = ((int64_t)tile * 64 + lane) * VEC;
+    const bool act = col < D;
+    const int64_t row0 = bi * T;
+
+    V carry = vfill<E, VEC>(O::zero());  // lam_{t+1} entering from the right
+    if (act && g_last) carry = *reinterpret_cast<const V *>(g_last + bi * D + col);
+
+    const int span = NW * TS;
+    int buf = 0;
+    for (int r0 = 0; r0 < T; r0 += span) {
+        const int rs = r0 + w * TS;
+        V x[TS], p[TS];
+        unsigned cmask = 0;  // bit s: chain cut between step t and t+1 (done_{t+1})
+        unsigned dmask = 0;  // bit s: done_t
+#pragma unroll
+        for (int s = 0; s < TS; ++s) {
+            const int t = T - 1 - (rs + s);
+            p[s] = vfill<E, VEC>(O::one());
+            x[s] = vfill<E, VEC>(O::zero());
+            if (t >= 0) {
+                if (act) {
+                    const int64_t off = (row0 + t) * D + col;
+                    x[s] = *reinterpret_cast<const V *>(g + off);
+                    if (t + 1 < T) {
+                        V av = *reinterpret_cast<const V *>(a + (a_ti ? col : off + D));
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) p[s].v[i] = O::conj(av.v[i]);
+                    }
+                }
+                if (t + 1 < T && done_at(done, done_f32, row0 + t + 1)) cmask |= 1u << s;
+                if (done_at(done, done_f32, row0 + t)) dmask |= 1u << s;
+            }
+        }
+        V my = carry;
+        if (NW == 1) {
+#pragma unroll
+            for (int s = 0; s < TS; ++s) {
+                const bool c = (cmask >> s) & 1u;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    const E ln = O::madd(p[s].v[i], carry.v[i], x[s].v[i]);
+                    carry.v[i] = c ? x[s].v[i] : ln;
+                }
+                x[s] = carry;
+            }
+        } else {
+            V lc = vfill<E, VEC>(O::zero()), pc = vfill<E, VEC>(O::one());
+#pragma unroll
+            for (int s = 0; s < TS; ++s) {
+                const bool c = (cmask >> s) & 1u;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    const E ln = O::madd(p[s].v[i], lc.v[i], x[s].v[i]);
+                    const E pn = O::mul(p[s].v[i], pc.v[i]);
+                    lc.v[i] = c ? x[s].v[i] : ln;
+                    pc.v[i] = c ? p[s].v[i] : pn;
+                }
+                x[s] = lc;
+                p[s] = pc;
+            }
+            sH[(buf * NW + w) * 64 + lane] = lc;
+            sP[(buf * NW + w) * 64 + lane] = pc;
+            if (lane == 0) sF[buf * NW + w] = cmask != 0;
+            __syncthreads();
+            V cin = carry;
+            for (int j = 0; j < NW; ++j) {
+                if (j == w) my = cin;
+                const V Hj = sH[(buf * NW + j) * 64 + lane];
+                const V Pj = sP[(buf * NW + j) * 64 + lane];
+                const bool fj = sF[buf * NW + j] != 0;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    const E ln = O::madd(Pj.v[i], cin.v[i], Hj.v[i]);
+                    cin.v[i] = fj ? Hj.v[i] : ln;
+                }
+            }
+            carry = cin;
+#pragma unroll
+            for (int s = 0; s < TS; ++s) {
+                const bool seen = (cmask & ((2u << s) - 1u)) != 0;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    const E fx = O::madd(p[s].v[i], my.v[i], x[s].v[i]);
+                    x[s].v[i] = seen ? x[s].v[i] : fx;
+                }
+            }
+            buf ^= 1;
+        }
+        // x[s] = lam_t : emit db_t and da_t = done_t ? 0 : lam_t conj(h_{t-1})
+#pragma unroll
+        for (int s = 0; s < TS; ++s) {
+            const int t = T - 1 - (rs + s);
+            if (t >= 0 && act) {
+                const int64_t off = (row0 + t) * D + col;
+                V hp = vfill<E, VEC>(O::zero());
+                if (t > 0)
+                    hp = *reinterpret_cast<const V *>(hfw + off - D);
+                else if (h0)
+                    hp = *reinterpret_cast<const V *>(h0 + bi * D + col);
+                const bool dn = (dmask >> s) & 1u;
+                V o;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    const E prod = O::mul(x[s].v[i], O::conj(hp.v[i]));
+                    o.v[i] = dn ? O::zero() : prod;
+                }
+                *reinterpret_cast<V *>(db + off) = x[s];
+                *reinterpret_cast<V *>(da + off) = o;
+            }
+        }
+    }
+    if (w == 0 && act && dh0) {
+        // carry = lam_0 ; dh0 = done_0 ? 0 : conj(a_0) lam_0
+        const bool d0 = done_at(done, done_f32, row0);
+        const V a0 = *reinterpret_cast<const V *>(a + (a_ti ? col : row0 * D + col));
+        V o;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const E prod = O::mul(O::conj(a0.v[i]), carry.v[i]);
+            o.v[i] = d0 ? O::zero() : prod;
+        }
+        *reinterpret_cast<V *>(dh0 + bi * D + col) = o;
+    }
+}
+
+struct ScanPlan {
+    int vec, nw, tiles;
+};
+
+// Widest vector the shapes/alignments allow, then the narrowest tile and the
+// smallest time split that put >= ~8 waves on each of the 256 CUs.
+ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, bool al8)
+{
+    const int maxvec = (int)(16 / esize);
+    int vec = 1;
+    for (int v = maxvec; v >= 1; v >>= 1) {
+        const size_t bytes = esize * v;
+        const bool ok_al = bytes == 16 ? al16 : (bytes == 8 ? al8 : true);
+        if (D % v == 0 && ok_al) { vec = v; break; }
+    }
+    const int64_t want = 2048;
+    auto ntiles = [&](int v) { return (D + 64 * (int64_t)v - 1) / (64 * (int64_t)v); };
+    while (vec > 1 && B * ntiles(vec) < want) vec >>= 1;
+    const int tiles = (int)ntiles(vec);
+    int nw = 1;
+    while (nw < 8 && B * tiles * nw < want && (int64_t)nw * TS < T) nw <<= 1;
+    return {vec, nw, tiles};
+}
+
+size_t scan_smem(int nw, size_t vbytes)
+{
+    return nw == 1 ? 0 : 2 * (size_t)nw * 64 * vbytes * 2 + 2 * (size_t)nw * sizeof(int);
+}
+
+template <typename E>
+int launch_fwd(hipStream_t st, const void *a, const void *b, const void *done,
+               int done_f32, const void *h0, const void *P0, void *h, void *h_last,
+               void *P_last, int64_t B, int64_t T, int64_t D, int a_ti)
+{
+    const bool al16 = aligned(a, 16) && aligned(b, 16) && aligned(h, 16) && aligned(h0, 16) &&
+                      aligned(P0, 16) && aligned(h_last, 16) && aligned(P_last, 16);
+    const bool al8 = aligned(a, 8) && aligned(b, 8) && aligned(h, 8) && aligned(h0, 8) &&
+                     aligned(P0, 8) && aligned(h_last, 8) && aligned(P_last, 8);
+    const ScanPlan pl = plan_scan(B, T, D, sizeof(E), al16, al8);
+    const dim3 grid((unsigned)(B * pl.tiles)), block(64 * pl.nw);
+    const size_t smem = scan_smem(pl.nw, sizeof(E) * pl.vec);
+#define MRX_LAUNCH(VEC)                                                                   \
+    hipLaunchKernelGGL((diag_scan_fwd_kernel<E, VEC>), grid, block, smem, st,             \
+                       (const E *)a, (const E *)b, done, done_f32, (const E *)h0,         \
+                       (const E *)P0, (E *)h, (E *)h_last, (E *)P_last, (int)T, D,        \
+                       pl.tiles, pl.nw, a_ti)
+    if constexpr (sizeof(E) == 4) {
+        if (pl.vec == 4) MRX_LAUNCH(4);
+        else if (pl.vec == 2) MRX_LAUNCH(2);
+        else MRX_LAUNCH(1);
+    } else {
+        if (pl.vec == 2) MRX_LAUNCH(2);
+        else MRX_LAUNCH(1);
+    }
+#undef MRX_LAUNCH
+    return launch_status();
+}
+
+template <typename E>
+int launch_bwd(hipStream_t st, const void *a, const void *h, const void *done,
+               int done_f32, const void *h0, const void *g, const void *g_last, void *da,
+               void *db, void *dh0, int64_t B, int64_t T, int64_t D, int a_ti)
+{
+    const bool al16 = aligned(a, 16) && aligned(h, 16) && aligned(g, 16) && aligned(h0, 16) &&
+                      aligned(g_last, 16) && aligned(da, 16) && aligned(db, 16) && aligned(dh0, 16);
+    const bool al8 = aligned(a, 8) && aligned(h, 8) && aligned(g, 8) && aligned(h0, 8) &&
+                     aligned(g_last, 8) && aligned(da, 8) && aligned(db, 8) && aligned(dh0, 8);
+    const ScanPlan pl = plan_scan(B, T, D, sizeof(E), al16, al8);
+    const dim3 grid((unsigned)(B * pl.tiles)), block(64 * pl.nw);
+    const size_t smem = scan_smem(pl.nw, sizeof(E) * pl.vec);
+#define MRX_LAUNCH(VEC)                                                                   \
+    hipLaunchKernelGGL((diag_scan_bwd_kernel<E, VEC>), grid, block, smem, st,             \
+                       (const E *)a, (const E *)h, done, done_f32, (const E *)h0,         \
+                       (const E *)g, (const E *)g_last, (E *)da, (E *)db, (E *)dh0,       \
+                       (int)T, D, pl.tiles, pl.nw, a_ti)
+    if constexpr (sizeof(E) == 4) {
+        if (pl.vec == 4) MRX_LAUNCH(4);
+        else if (pl.vec == 2) MRX_LAUNCH(2);
+        else MRX_LAUNCH(1);
+    } else {
+        if (pl.vec == 2) MRX_LAUNCH(2);
+        else MRX_LAUNCH(1);
+    }
+#undef MRX_LAUNCH
+    return launch_status();
+}
+
+bool scan_shape_ok(int64_t B, int64_t T, int64_t D)
+{
+    return B > 0 && T > 0 && D > 0 && T < (1ll << 30) && B * ((D + 63) / 64) < (1ll << 31);
+}
+
+}  // namespace
+
+extern "C" int mrx_linear_scan_fwd(void *stream, const void *a, const void *b, const void *done,
+                                   const void *h0, const void *P0, void *h, void *h_last,
+                                   void *P_last, int64_t B, int64_t T, int64_t D, int dtype,
+                                   int done_dtype, int a_time_invariant)
+{
+    if (!a || !b || !done || !h) return MRX_ERR_INVALID_ARG;
+    if (!scan_shape_ok(B, T, D)) return MRX_ERR_INVALID_ARG;
+    if (done_dtype != MRX_DONE_U8 && done_dtype != MRX_DONE_F32) return MRX_ERR_INVALID_ARG;
+    if (done_dtype == MRX_DONE_F32 && !aligned(done, 4)) return MRX_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const int ti = a_time_invariant != 0;
+    if (dtype == MRX_F32) {
+        if (!aligned(a, 4) || !aligned(b, 4) || !aligned(h, 4)) return MRX_ERR_INVALID_ARG;
+        return launch_fwd<float>(st, a, b, done, done_dtype, h0, P0, h, h_last, P_last, B, T, D, ti);
+    }
+    if (dtype == MRX_C64) {
+        if (!aligned(a, 8) || !aligned(b, 8) || !aligned(h, 8) || !aligned(h0, 8) ||
+            !aligned(P0, 8) || !aligned(h_last, 8) || !aligned(P_last, 8))
+            return MRX_ERR_INVALID_ARG;
+        return launch_fwd<c64>(st, a, b, done, done_dtype, h0, P0, h, h_last, P_last, B, T, D, ti);
+    }
+    return dtype == MRX_BF16 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
+}
+
+extern "C" int mrx_linear_scan_bwd(void *stream, const void *a, const void *h, const void *done,
+                                   const void *h0, const void *g, const void *g_last, void *da,
+                                   void *db, void *dh0, int64_t B, int64_t T, int64_t D,
+                                   int dtype, int done_dtype, int a_time_invariant)
+{
+    if (!a || !h || !done || !g || !da || !db) return MRX_ERR_INVALID_ARG;
+    if (!scan_shape_ok(B, T, D)) return MRX_ERR_INVALID_ARG;
+    if (done_dtype != MRX_DONE_U8 && done_dtype != MRX_DONE_F32) return MRX_ERR_INVALID_ARG;
+    if (done_dtype == MRX_DONE_F32 && !aligned(done, 4)) return MRX_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const int ti = a_time_invariant != 0;
+    if (dtype == MRX_F32) {
+        if (!aligned(a, 4) || !aligned(h, 4) || !aligned(g, 4) || !aligned(da, 4) || !aligned(db, 4))
+            return MRX_ERR_INVALID_ARG;
+        return launch_bwd<float>(st, a, h, done, done_dtype, h0, g, g_last, da, db, dh0, B, T, D, ti);
+    }
+    if (dtype == MRX_C64) {
+        if (!aligned(a, 8) || !aligned(h, 8) || !aligned(g, 8) || !aligned(da, 8) ||
+            !aligned(db, 8) || !aligned(h0, 8) || !aligned(g_last, 8) || !aligned(dh0, 8))
+            return MRX_ERR_INVALID_ARG;
+        return launch_bwd<c64>(st, a, h, done, done_dtype, h0, g, g_last, da, db, dh0, B, T, D, ti);
+    }
+    return dtype == MRX_BF16 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
+}

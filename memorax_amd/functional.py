@@ -1,0 +1,109 @@
+"""Differentiable entry points over the HIP kernels (torch.autograd.Function plays
+the role jax.custom_vjp would in a JAX host).
+
+    linear_scan(a, b, done, h0=None, P0=None)            -> (h, h_last, P_last)
+    linear_attention(q, k, v, done, S0=None, feature_map) -> (o, S_last)
+    delta_rule(q, k, v, beta, done, S0=None)             -> (o, S_last)
+
+Layouts follow the reference: (B,T,D) / (B,T,H,d), state (B,H,d_v,d_k), done (B,T)
+bool or float where nonzero clears the carry before step t (memoroid.py:60-91).
+"""
+from __future__ import annotations
+
+import torch
+
+from . import kernels as K
+
+_FMAP = {None: 0, "none": 0, 0: 0, "elu1": 1, 1: 1}
+
+
+class _LinearScan(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, a, b, done, h0, P0):
+        a_, b_ = a.contiguous(), b.contiguous()
+        h0_ = None if h0 is None else h0.contiguous()
+        P0_ = None if P0 is None else P0.contiguous()
+        h, h_last, P_last = K.linear_scan_fwd(a_, b_, done, h0_, P0_)
+        ctx.save_for_backward(a_, h, h0_ if h0_ is not None else torch.empty(0, device=b.device))
+        ctx.done = done
+        ctx.has_h0 = h0 is not None
+        ctx.mark_non_differentiable(P_last)
+        return h, h_last, P_last
+
+    @staticmethod
+    def backward(ctx, g, g_last, _gP):
+        a, h, h0 = ctx.saved_tensors
+        h0 = h0 if ctx.has_h0 else None
+        g = torch.zeros_like(h) if g is None else g.contiguous()
+        g_last = None if g_last is None else g_last.contiguous()
+        da, db, dh0 = K.linear_scan_bwd(a, h, ctx.done, h0, g, g_last)
+        if a.dim() == 1:
+            da = da.sum(dim=(0, 1))
+        return (da if ctx.needs_input_grad[0] else None,
+                db if ctx.needs_input_grad[1] else None,
+                None,
+                dh0 if (ctx.has_h0 and ctx.needs_input_grad[3]) else None,
+                None)
+
+
+def linear_scan(a, b, done, h0=None, P0=None):
+    """Reset-aware diagonal recurrence h_t = a_t h_{t-1} + b_t (lru.py:92-95 scanned
+    by memoroid.py:60-91).  a: (B,T,D) or (D,); b: (B,T,D); h0,P0: (B,D).
+    P_last (the cumulative-decay leaf of the carry) is not differentiable."""
+    return _LinearScan.apply(a, b, done, h0, P0)
+
+
+class _LinearAttention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, done, S0, fmap):
+        q_, k_, v_ = q.contiguous(), k.contiguous(), v.contiguous()
+        S0_ = None if S0 is None else S0.contiguous().float()
+        need = any(ctx.needs_input_grad)
+        o, S_last, S_chk = K.linear_attn_fwd(q_, k_, v_, done, S0_, fmap, save_chk=need)
+        if need:
+            ctx.save_for_backward(q_, k_, v_, S_chk)
+        ctx.done, ctx.fmap, ctx.has_S0 = done, fmap, S0 is not None
+        return o, S_last
+
+    @staticmethod
+    def backward(ctx, do, dS_last):
+        q, k, v, S_chk = ctx.saved_tensors
+        do = torch.zeros_like(v) if do is None else do.contiguous()
+        dS_last = None if dS_last is None else dS_last.contiguous().float()
+        dq, dk, dv, dS0 = K.linear_attn_bwd(q, k, v, ctx.done, S_chk, do, dS_last, ctx.fmap,
+                                            want_dS0=ctx.has_S0)
+        return dq, dk, dv, None, (dS0 if ctx.has_S0 else None), None
+
+
+def linear_attention(q, k, v, done, S0=None, feature_map="none"):
+    """Causal unnormalised linear attention, chunked: S_t = r_t S_{t-1} + v_t phi(k_t)^T,
+    o_t = S_t phi(q_t) (linear_attention.py:62-86,105).  Returns (o, S_last)."""
+    return _LinearAttention.apply(q, k, v, done, S0, _FMAP[feature_map])
+
+
+class _DeltaRule(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, beta, done, S0):
+        q_, k_, v_, b_ = q.contiguous(), k.contiguous(), v.contiguous(), beta.contiguous()
+        S0_ = None if S0 is None else S0.contiguous().float()
+        need = any(ctx.needs_input_grad)
+        o, S_last, S_chk = K.delta_rule_fwd(q_, k_, v_, b_, done, S0_, save_chk=need)
+        if need:
+            ctx.save_for_backward(q_, k_, v_, b_, S_chk)
+        ctx.done, ctx.has_S0 = done, S0 is not None
+        return o, S_last
+
+    @staticmethod
+    def backward(ctx, do, dS_last):
+        q, k, v, beta, S_chk = ctx.saved_tensors
+        do = torch.zeros_like(v) if do is None else do.contiguous()
+        dS_last = None if dS_last is None else dS_last.contiguous().float()
+        dq, dk, dv, db, dS0 = K.delta_rule_bwd(q, k, v, beta, ctx.done, S_chk, do, dS_last,
+                                               want_dS0=ctx.has_S0)
+        return dq, dk, dv, db, None, (dS0 if ctx.has_S0 else None)
+
+
+def delta_rule(q, k, v, beta, done, S0=None):
+    """DeltaNet recurrence S_t = r_t S_{t-1}(I - beta_t k_t k_t^T) + beta_t v_t k_t^T,
+    o_t = S_t q_t, in chunked WY form.  Returns (o, S_last)."""
+    return _DeltaRule.apply(q, k, v, beta, done, S0)

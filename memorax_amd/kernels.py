@@ -1,0 +1,193 @@
+"""Thin, allocation-explicit wrappers: torch device tensors in, C-ABI call, tensors out.
+
+torch is used for device memory and the current HIP stream only.  Every function
+validates device / dtype / contiguity, allocates the outputs and forwards raw
+pointers to the library; there is no alternative code path.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+_DT = {torch.float32: _lib.MRX_F32, torch.bfloat16: _lib.MRX_BF16, torch.complex64: _lib.MRX_C64}
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _chk(t, name, dtype=None, shape=None):
+    if t is None:
+        return
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (memorax_amd has no CPU path)")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise ValueError(f"{name} must be {dtype}, got {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+
+
+def _done(done, B, T):
+    """Accept bool / uint8 / float32 (B,T); returns (tensor, done_dtype enum)."""
+    if tuple(done.shape) != (B, T):
+        raise ValueError(f"done must have shape {(B, T)}, got {tuple(done.shape)}")
+    if done.dtype == torch.bool:
+        done = done.contiguous().view(torch.uint8)
+    elif done.dtype == torch.uint8:
+        done = done.contiguous()
+    elif done.dtype == torch.float32:
+        done = done.contiguous()
+        _chk(done, "done")
+        return done, _lib.MRX_DONE_F32
+    else:
+        done = (done != 0).contiguous().view(torch.uint8)
+    _chk(done, "done")
+    return done, _lib.MRX_DONE_U8
+
+
+def chunk_size(dtype) -> int:
+    return int(_lib.load().mrx_chunk_size(_DT[dtype]))
+
+
+# ----------------------------------------------------------------- diagonal scan
+def linear_scan_fwd(a, b, done, h0=None, P0=None, want_P=True):
+    """h_t = done ? b_t : a_t h_{t-1} + b_t.  a: (B,T,D) or (D,) time-invariant.
+    Returns (h, h_last, P_last)."""
+    lib = _lib.load()
+    B, T, D = b.shape
+    dt = b.dtype
+    if dt not in (torch.float32, torch.complex64):
+        raise ValueError("linear_scan supports float32 and complex64")
+    ti = a.dim() == 1
+    _chk(a, "a", dt, (D,) if ti else (B, T, D))
+    _chk(b, "b", dt)
+    _chk(h0, "h0", dt, (B, D))
+    _chk(P0, "P0", dt, (B, D))
+    done, dd = _done(done, B, T)
+    h = torch.empty_like(b)
+    h_last = torch.empty((B, D), dtype=dt, device=b.device)
+    P_last = torch.empty((B, D), dtype=dt, device=b.device) if want_P else None
+    st = lib.mrx_linear_scan_fwd(_stream(), _ptr(a), _ptr(b), _ptr(done), _ptr(h0), _ptr(P0),
+                                 _ptr(h), _ptr(h_last), _ptr(P_last), B, T, D, _DT[dt], dd, int(ti))
+    _lib.check(st, "mrx_linear_scan_fwd")
+    return h, h_last, P_last
+
+
+def linear_scan_bwd(a, h, done, h0, g, g_last=None):
+    """Returns (da (B,T,D) per step, db, dh0)."""
+    lib = _lib.load()
+    B, T, D = g.shape
+    dt = g.dtype
+    ti = a.dim() == 1
+    _chk(a, "a", dt, (D,) if ti else (B, T, D))
+    _chk(h, "h", dt, (B, T, D))
+    _chk(g, "g", dt)
+    _chk(h0, "h0", dt, (B, D))
+    _chk(g_last, "g_last", dt, (B, D))
+    done, dd = _done(done, B, T)
+    da = torch.empty_like(g)
+    db = torch.empty_like(g)
+    dh0 = torch.empty((B, D), dtype=dt, device=g.device)
+    st = lib.mrx_linear_scan_bwd(_stream(), _ptr(a), _ptr(h), _ptr(done), _ptr(h0), _ptr(g),
+                                 _ptr(g_last), _ptr(da), _ptr(db), _ptr(dh0), B, T, D, _DT[dt],
+                                 dd, int(ti))
+    _lib.check(st, "mrx_linear_scan_bwd")
+    return da, db, dh0
+
+
+# ----------------------------------------------------------------- chunked attention
+def _attn_shapes(q, k, v):
+    B, T, H, dk = q.shape
+    dv = v.shape[-1]
+    dt = q.dtype
+    if dt not in (torch.float32, torch.bfloat16):
+        raise ValueError("chunked kernels support float32 and bfloat16")
+    _chk(q, "q", dt)
+    _chk(k, "k", dt, (B, T, H, dk))
+    _chk(v, "v", dt, (B, T, H, dv))
+    return B, T, H, dk, dv, dt
+
+
+def _n_chunks(T, dt):
+    C = chunk_size(dt)
+    return (T + C - 1) // C
+
+
+def linear_attn_fwd(q, k, v, done, S0=None, feature_map=0, save_chk=True):
+    """Returns (o, S_last fp32, S_chk or None)."""
+    lib = _lib.load()
+    B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
+    _chk(S0, "S0", torch.float32, (B, H, dv, dk))
+    done, dd = _done(done, B, T)
+    o = torch.empty_like(v)
+    S_last = torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
+    S_chk = (torch.empty((B, H, _n_chunks(T, dt), dv, dk), dtype=dt, device=q.device)
+             if save_chk else None)
+    st = lib.mrx_linear_attn_fwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(done), _ptr(S0),
+                                 _ptr(o), _ptr(S_last), _ptr(S_chk), B, T, H, dk, dv, _DT[dt], dd,
+                                 int(feature_map))
+    _lib.check(st, "mrx_linear_attn_fwd")
+    return o, S_last, S_chk
+
+
+def linear_attn_bwd(q, k, v, done, S_chk, do, dS_last=None, feature_map=0, want_dS0=True):
+    """Returns (dq, dk, dv, dS0)."""
+    lib = _lib.load()
+    B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
+    _chk(do, "do", dt, (B, T, H, dv))
+    _chk(S_chk, "S_chk", dt, (B, H, _n_chunks(T, dt), dv, dk))
+    _chk(dS_last, "dS_last", torch.float32, (B, H, dv, dk))
+    done, dd = _done(done, B, T)
+    dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dS0 = (torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
+           if want_dS0 else None)
+    st = lib.mrx_linear_attn_bwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(done), _ptr(S_chk),
+                                 _ptr(do), _ptr(dS_last), _ptr(dq), _ptr(dk_), _ptr(dv_),
+                                 _ptr(dS0), B, T, H, dk, dv, _DT[dt], dd, int(feature_map))
+    _lib.check(st, "mrx_linear_attn_bwd")
+    return dq, dk_, dv_, dS0
+
+
+def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True):
+    """Returns (o, S_last fp32, S_chk or None)."""
+    lib = _lib.load()
+    B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
+    _chk(beta, "beta", dt, (B, T, H))
+    _chk(S0, "S0", torch.float32, (B, H, dv, dk))
+    done, dd = _done(done, B, T)
+    o = torch.empty_like(v)
+    S_last = torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
+    S_chk = (torch.empty((B, H, _n_chunks(T, dt), dv, dk), dtype=dt, device=q.device)
+             if save_chk else None)
+    st = lib.mrx_delta_rule_fwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done),
+                                _ptr(S0), _ptr(o), _ptr(S_last), _ptr(S_chk), B, T, H, dk, dv,
+                                _DT[dt], dd)
+    _lib.check(st, "mrx_delta_rule_fwd")
+    return o, S_last, S_chk
+
+
+def delta_rule_bwd(q, k, v, beta, done, S_chk, do, dS_last=None, want_dS0=True):
+    """Returns (dq, dk, dv, dbeta, dS0)."""
+    lib = _lib.load()
+    B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
+    _chk(beta, "beta", dt, (B, T, H))
+    _chk(do, "do", dt, (B, T, H, dv))
+    _chk(S_chk, "S_chk", dt, (B, H, _n_chunks(T, dt), dv, dk))
+    _chk(dS_last, "dS_last", torch.float32, (B, H, dv, dk))
+    done, dd = _done(done, B, T)
+    dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dbeta = torch.empty_like(beta)
+    dS0 = (torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
+           if want_dS0 else None)
+    st = lib.mrx_delta_rule_bwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done),
+                                _ptr(S_chk), _ptr(do), _ptr(dS_last), _ptr(dq), _ptr(dk_),
+                                _ptr(dv_), _ptr(dbeta), _ptr(dS0), B, T, H, dk, dv, _DT[dt], dd)
+    _lib.check(st, "mrx_delta_rule_bwd")
+    return dq, dk_, dv_, dbeta, dS0
