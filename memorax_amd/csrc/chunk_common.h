@@ -115,6 +115,21 @@ __device__ __forceinline__ void store_acc_t(const f32x4 *acc, T *dst, int ld, in
     }
 }
 
+// Store an accumulator tile set as dst[m][n] (element-wise writes; use when the
+// consumer needs the other orientation too).
+template <typename T, int M, int N>
+__device__ __forceinline__ void store_acc_n(const f32x4 *acc, T *dst, int ld, int w, int lane)
+{
+    using TM = TileMap<M, N>;
+    const int i = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int j = 0; j < TM::TPW; ++j) {
+        const int m = TM::mt(w) * 16 + 4 * g, n = TM::nt(w, j) * 16 + i;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) dst[(m + v) * ld + n] = (T)acc[j][v];
+    }
+}
+
 __device__ __forceinline__ float elu1(float x) { return x > 0.f ? x + 1.f : __expf(x); }
 __device__ __forceinline__ float delu1(float x) { return x > 0.f ? 1.f : __expf(x); }
 
@@ -178,25 +193,11 @@ template <typename T, int C> struct TileIO {
 };
 
 // ---- per-chunk reset bookkeeping ------------------------------------------------
-// seg[r] = number of resets at rows <= r inside the chunk.  m_r = (seg[r] == 0):
-// row still belongs to the episode that entered the chunk.  e_r = (seg[r] == nres):
-// row belongs to the episode that leaves the chunk.  rows i, j interact iff
-// seg[i] == seg[j].
-struct ChunkSeg {
-    int nres;    // resets in the chunk
-    int jstart;  // first row of the last episode (0 if no reset)
-};
-
-// Called by wave 0 with flag = done(row lane) (0 for rows past the end); writes sSeg[0..C).
-template <int C> __device__ __forceinline__ void compute_seg(bool flag, int *sSeg, int *sMeta, int lane)
+// dmask has bit r set when row r of the chunk starts a new episode.  episode_of(r)
+// counts the resets at rows <= r; rows interact iff they have the same count.
+__device__ __forceinline__ int episode_of(unsigned long long dmask, int r)
 {
-    const unsigned long long mask = __ballot(flag && lane < C);
-    const unsigned long long upto = lane >= 63 ? ~0ull : ((2ull << lane) - 1ull);
-    if (lane < C) sSeg[lane] = __popcll(mask & upto);
-    if (lane == 0) {
-        sMeta[0] = __popcll(mask);
-        sMeta[1] = mask ? 63 - __clzll(mask) : 0;
-    }
+    return __popcll(dmask & ((2ull << r) - 1ull));
 }
 
 // ---- inverse of a unit lower-triangular matrix, in place, fp32 -------------------

@@ -6,7 +6,7 @@
 //                      W  = T K,  U' = T V - diag(m) W S^T
 //   both:              O  = diag(m) Q S^T + (tril(Q K^T) . M) U'
 //                      S <- l S + (diag(e) U')^T K
-// M, m, e, l are the episode masks of the chunk (see ChunkSeg).  The state is
+// M, m, e, l are the episode masks of the chunk (episode_of in chunk_common.h).  The state is
 // kept transposed (S^T, d_k x d_v) in MFMA accumulators for the whole sequence and
 // re-staged to LDS as a T-typed d_v x d_k tile once per chunk.
 #include "chunk_common.h"

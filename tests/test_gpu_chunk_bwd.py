@@ -1,0 +1,139 @@
+"""GPU parity of the chunked backward kernels (through the C ABI) against the
+torch-fp64 autograd oracle (small shapes) and the C oracle (benchmark shapes)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import clib
+from oracle import grad as G
+from oracle import memoroid as M
+from gpu_util import TOL_BF16, TOL_F32, attn_inputs, bf16_round, dev, relerr
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(1, 64, 1), (2, 128, 2), (1, 1, 1), (2, 7, 1), (1, 65, 2), (2, 200, 3), (1, 33, 1)]
+
+
+def _check(got, ref, tol, names):
+    errs = {n: relerr(g, ref[n]) for n, g in zip(names, got)}
+    bad = {n: e for n, e in errs.items() if not e <= tol}
+    assert not bad, f"rel errs {errs}"
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("p", [0.0, 0.05])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("fmap", [0, 1])
+def test_linear_attention_bwd(shape, p, dtype, fmap):
+    from memorax_amd import kernels as K
+    B, T, H = shape
+    x = attn_inputs(B, T, H, p=p, seed=B * 100 + T + H + 31, scale=1.0 / 8)
+    rng = np.random.default_rng(T)
+    do = rng.standard_normal((B, T, H, 64)).astype(np.float32)
+    dSl = (rng.standard_normal((B, H, 64, 64)) * 0.1).astype(np.float32)
+    print(f"case la_bwd shape={shape} p={p} dtype={dtype} fmap={fmap}", flush=True)
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    if dtype == "bf16":
+        for n in ("q", "k", "v"):
+            x[n] = bf16_round(x[n])
+        do = bf16_round(do)
+    tq, tk, tv, tdo = (dev(a, td) for a in (x["q"], x["k"], x["v"], do))
+    o, Sl, chk = K.linear_attn_fwd(tq, tk, tv, dev(x["done"]), dev(x["S0"]), fmap)
+    got = K.linear_attn_bwd(tq, tk, tv, dev(x["done"]), chk, tdo, dev(dSl), fmap)
+    ref = G.linear_attention_grads(x["q"], x["k"], x["v"], x["done"], x["S0"], do, dSl,
+                                   "elu1" if fmap else "none")
+    _check(got, ref, TOL_BF16 if dtype == "bf16" else TOL_F32, ("dq", "dk", "dv", "dS0"))
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("p", [0.0, 0.05])
+def test_delta_rule_bwd_bf16(shape, p):
+    from memorax_amd import kernels as K
+    B, T, H = shape
+    x = attn_inputs(B, T, H, p=p, seed=B * 100 + T + H + 57, delta=True)
+    rng = np.random.default_rng(T + 1)
+    do = bf16_round(rng.standard_normal((B, T, H, 64)).astype(np.float32))
+    dSl = (rng.standard_normal((B, H, 64, 64)) * 0.1).astype(np.float32)
+    print(f"case delta_bwd shape={shape} p={p}", flush=True)
+    for n in ("q", "k", "v", "beta"):
+        x[n] = bf16_round(x[n])
+    bf = torch.bfloat16
+    tq, tk, tv, tb, tdo = (dev(a, bf) for a in (x["q"], x["k"], x["v"], x["beta"], do))
+    o, Sl, chk = K.delta_rule_fwd(tq, tk, tv, tb, dev(x["done"]), dev(x["S0"]))
+    got = K.delta_rule_bwd(tq, tk, tv, tb, dev(x["done"]), chk, tdo, dev(dSl))
+    ref = G.delta_rule_grads(x["q"], x["k"], x["v"], x["beta"], x["done"], x["S0"], do, dSl)
+    _check(got, ref, TOL_BF16, ("dq", "dk", "dv", "dbeta", "dS0"))
+
+
+def test_delta_rule_bwd_fp32_reports_unsupported():
+    from memorax_amd import kernels as K
+    x = attn_inputs(1, 32, 1, seed=1, delta=True)
+    args = [dev(x[n]) for n in ("q", "k", "v", "beta")]
+    o, Sl, chk = K.delta_rule_fwd(*args, dev(x["done"]))
+    with pytest.raises(RuntimeError, match="unsupported"):
+        K.delta_rule_bwd(*args, dev(x["done"]), chk, torch.zeros_like(o))
+
+
+def test_bwd_reset_isolation():
+    """A poisoned (NaN) gradient / value on one side of a reset stays on that side."""
+    from memorax_amd import kernels as K
+    B, T, H = 1, 192, 1
+    x = attn_inputs(B, T, H, seed=5, delta=True)
+    x["done"][:] = False
+    x["done"][0, 100] = True
+    for n in ("q", "k", "v", "beta"):
+        x[n] = bf16_round(x[n])
+    do = bf16_round(np.random.default_rng(2).standard_normal((B, T, H, 64)).astype(np.float32))
+    do[0, 150] = np.nan      # poison in the later episode
+    bf = torch.bfloat16
+    tq, tk, tv, tb, tdo = (dev(a, bf) for a in (x["q"], x["k"], x["v"], x["beta"], do))
+    o, Sl, chk = K.delta_rule_fwd(tq, tk, tv, tb, dev(x["done"]))
+    dq, dk, dv, db, dS0 = K.delta_rule_bwd(tq, tk, tv, tb, dev(x["done"]), chk, tdo)
+    for g in (dq, dk, dv):
+        assert np.isfinite(g.float().cpu().numpy()[0, :100]).all()
+    assert np.isfinite(db.float().cpu().numpy()[0, :100]).all() and np.isfinite(dS0.cpu().numpy()).all()
+    ref = G.delta_rule_grads(x["q"][:, :100], x["k"][:, :100], x["v"][:, :100], x["beta"][:, :100],
+                             x["done"][:, :100], None, do[:, :100])
+    assert relerr(dk[:, :100], ref["dk"]) <= TOL_BF16 and relerr(dq[:, :100], ref["dq"]) <= TOL_BF16
+
+
+def test_bwd_config_shapes_small_batch():
+    """Benchmark configurations 2 (fp32, elu+1) and 4 (bf16 delta rule) at reduced batch vs the C oracle."""
+    from memorax_amd import kernels as K
+    x = M.make_inputs(2, (4, 256, 4, 64))
+    do = np.random.default_rng(0).standard_normal(x["v"].shape).astype(np.float32)
+    tq, tk, tv, tdo = (dev(a) for a in (x["q"], x["k"], x["v"], do))
+    o, Sl, chk = K.linear_attn_fwd(tq, tk, tv, dev(x["done"]), None, 1)
+    got = K.linear_attn_bwd(tq, tk, tv, dev(x["done"]), chk, tdo, None, 1)
+    ref = clib.linear_attn_bwd(x["q"], x["k"], x["v"], x["done"], None, do, None, 1)
+    _check(got, dict(zip(("dq", "dk", "dv", "dS0"), ref)), TOL_F32, ("dq", "dk", "dv", "dS0"))
+
+    x = M.make_inputs(4, (4, 1024, 8, 64))
+    xb = {n: bf16_round(x[n]) for n in ("q", "k", "v", "beta")}
+    do = bf16_round(np.random.default_rng(1).standard_normal(x["v"].shape).astype(np.float32))
+    bf = torch.bfloat16
+    tq, tk, tv, tb, tdo = (dev(a, bf) for a in (xb["q"], xb["k"], xb["v"], xb["beta"], do))
+    o, Sl, chk = K.delta_rule_fwd(tq, tk, tv, tb, dev(x["done"]))
+    got = K.delta_rule_bwd(tq, tk, tv, tb, dev(x["done"]), chk, tdo)
+    ref = clib.delta_rule_bwd(xb["q"], xb["k"], xb["v"], xb["beta"], x["done"], None, do)
+    _check(got, dict(zip(("dq", "dk", "dv", "dbeta", "dS0"), ref)), TOL_BF16, ("dq", "dk", "dv", "dbeta", "dS0"))
+
+
+def test_autograd_functions():
+    import memorax_amd as mx
+    x = attn_inputs(2, 96, 2, p=0.03, seed=77, delta=True)
+    for n in ("q", "k", "v", "beta"):
+        x[n] = bf16_round(x[n])
+    do = bf16_round(np.random.default_rng(4).standard_normal(x["v"].shape).astype(np.float32))
+    bf = torch.bfloat16
+    tq, tk, tv, tb = (dev(x[n], bf).requires_grad_() for n in ("q", "k", "v", "beta"))
+    tS0 = dev(x["S0"]).requires_grad_()
+    o, Sl = mx.delta_rule(tq, tk, tv, tb, dev(x["done"]), tS0)
+    (o.float() * dev(do)).sum().backward()
+    ref = G.delta_rule_grads(x["q"], x["k"], x["v"], x["beta"], x["done"], x["S0"], do)
+    _check((tq.grad, tk.grad, tv.grad, tb.grad, tS0.grad), ref, TOL_BF16, ("dq", "dk", "dv", "dbeta", "dS0"))
+    tq2, tk2, tv2 = (dev(x[n] / 8).requires_grad_() for n in ("q", "k", "v"))
+    o2, _ = mx.linear_attention(tq2, tk2, tv2, dev(x["done"]), None, "elu1")
+    (o2 * dev(do)).sum().backward()
+    ref = G.linear_attention_grads(x["q"] / 8, x["k"] / 8, x["v"] / 8, x["done"], None, do, None, "elu1")
+    _check((tq2.grad, tk2.grad, tv2.grad), ref, TOL_F32, ("dq", "dk", "dv"))
