@@ -1,0 +1,210 @@
+#!/usr/bin/env python3
+"""Benchmark of the memorax sequence-model hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--all]
+
+One "step" = one forward + backward pass of the DeltaNet delta rule over the
+synthetic batch of BASELINE configuration 4 (B=64, H=8, T=1024, d=64, bf16 inputs,
+fp32 state, reset mask Bernoulli(0.002)); inputs are resident in HBM before the
+timed region.  Prints ONE JSON line.  Only one GPU is used: --gpus > 1 exits.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+# Algorithmic HBM bytes per (b, t, h) token-head, d = 64, bf16:
+#   forward : read q,k,v (3*128) + beta (2), write o (128)                    = 514
+#   backward: read q,k,v,do (4*128) + beta (2), write dq,dk,dv (3*128) + dbeta (2) = 900
+BYTES_FWD, BYTES_BWD = 514, 900
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--all", action="store_true", help="also time the other configurations")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU; this build has no multi-GPU path (--gpus must be 1)",
+              file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    from memorax_amd import kernels as K
+    from oracle import memoroid as M
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    bf = torch.bfloat16
+    B, T, H, d = 64, 1024, 8, 64
+    x = M.make_inputs(4, (B, T, H, d))
+    do_np = np.random.default_rng(2004).standard_normal((B, T, H, d)).astype(np.float32)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()  # noqa: E731
+    q, k, v, beta, do = (dev(a).to(bf) for a in (x["q"], x["k"], x["v"], x["beta"], do_np))
+    done = dev(x["done"])
+    torch.cuda.synchronize()
+
+    def step():
+        o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done)
+        return K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+
+    # per-kernel durations with HIP events on the stream the kernels are launched on
+    ev = lambda: torch.cuda.Event(enable_timing=True)  # noqa: E731
+    tf = tb = 0.0
+    for _ in range(args.steps):
+        e0, e1, e2 = ev(), ev(), ev()
+        e0.record()
+        o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done)
+        e1.record()
+        K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False)
+        e2.record()
+        torch.cuda.synchronize()
+        tf += e0.elapsed_time(e1)
+        tb += e1.elapsed_time(e2)
+    tf_ms, tb_ms = tf / args.steps, tb / args.steps
+    nth = B * T * H
+    bwd_gbs = BYTES_BWD * nth / (tb_ms * 1e-3) / 1e9
+    fwd_gbs = BYTES_FWD * nth / (tf_ms * 1e-3) / 1e9
+
+    out = {
+        "metric": "tokens/sec (B×T) fwd+bwd + % HBM/MFMA roofline, DeltaNet T=1024 on 1 GPU",
+        "value": B * T / dt,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": dt * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "configs[3]: DeltaNet delta rule fwd+bwd, B=64 H=8 T=1024 d=64, "
+                               "bf16 in / fp32 state, chunk 64, resets p=0.002"},
+        "roofline": {
+            "bound": "hbm", "kernel": "delta_bwd_kernel", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
+            "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": None,
+            "launch_ms": tb_ms, "algorithmic_bytes": BYTES_BWD * nth,
+        },
+        "kernels": {
+            "delta_fwd": {"ms": tf_ms, "GB/s": fwd_gbs, "frac_hbm": fwd_gbs / HBM_PEAK_GBS},
+            "delta_bwd": {"ms": tb_ms, "GB/s": bwd_gbs, "frac_hbm": bwd_gbs / HBM_PEAK_GBS},
+            "fwd+bwd": {"ms": tf_ms + tb_ms,
+                        "GB/s": (BYTES_FWD + BYTES_BWD) * nth / ((tf_ms + tb_ms) * 1e-3) / 1e9},
+        },
+    }
+
+    out["scan"] = bench_scan(torch, K, M, dev)
+    if args.all:
+        out["linear_attention"] = bench_linear_attention(torch, K, M, dev)
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(np, M, x, do_np)
+    print(json.dumps(out))
+    return 0
+
+
+def _time_ms(torch, fn, iters=20, warm=3):
+    for _ in range(warm):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def bench_scan(torch, K, M, dev):
+    """Diagonal scan forward: configuration 1 (32,128,256) and a shape that saturates HBM."""
+    res = {}
+    for name, shape in (("cfg1_32x128x256", (32, 128, 256)), ("torso_1024x128x256", (1024, 128, 256)),
+                        ("sweep_512x1024x1024", (512, 1024, 1024))):
+        Bn, Tn, Dn = shape
+        a = torch.rand(shape, device="cuda") * 0.099 + 0.9
+        b = torch.randn(shape, device="cuda")
+        dn = torch.rand((Bn, Tn), device="cuda") < 0.01
+        ms = _time_ms(torch, lambda: K.linear_scan_fwd(a, b, dn, want_P=False), iters=10)
+        h, _, _ = K.linear_scan_fwd(a, b, dn, want_P=False)
+        g = torch.randn(shape, device="cuda")
+        msb = _time_ms(torch, lambda: K.linear_scan_bwd(a, h, dn, None, g), iters=10)
+        by = 12 * Bn * Tn * Dn
+        res[name] = {"fwd_ms": ms, "fwd_GB/s": by / ms / 1e6, "fwd_frac_hbm": by / ms / 1e6 / HBM_PEAK_GBS,
+                     "fwd_tokens/s": Bn * Tn / ms * 1e3,
+                     "bwd_ms": msb, "bwd_GB/s": 20 * Bn * Tn * Dn / msb / 1e6}
+        del a, b, g, h
+    return res
+
+
+def bench_linear_attention(torch, K, M, dev):
+    """Configuration 2 (fp32, elu+1, resets) and configuration 3 at reduced batch (bf16, no resets)."""
+    res = {}
+    x = M.make_inputs(2)
+    q, k, v = (dev(x[n]) for n in ("q", "k", "v"))
+    dn = dev(x["done"])
+    do = torch.randn_like(v)
+
+    def f2():
+        o, Sl, chk = K.linear_attn_fwd(q, k, v, dn, None, 1)
+        K.linear_attn_bwd(q, k, v, dn, chk, do, None, 1, want_dS0=False)
+    ms = _time_ms(torch, f2)
+    res["cfg2_f32_64x256x4x64"] = {"ms": ms, "tokens/s": 64 * 256 / ms * 1e3,
+                                   "GB/s": 2816 * 64 * 256 * 4 / ms / 1e6}
+    Bn, Tn, Hn = 32, 4096, 8
+    q, k, v, do = (torch.randn((Bn, Tn, Hn, 64), device="cuda").div_(8).to(torch.bfloat16) for _ in range(4))
+    dn = torch.zeros((Bn, Tn), dtype=torch.bool, device="cuda")
+
+    def f3():
+        o, Sl, chk = K.linear_attn_fwd(q, k, v, dn, None, 0)
+        K.linear_attn_bwd(q, k, v, dn, chk, do, None, 0, want_dS0=False)
+    ms = _time_ms(torch, f3, iters=5)
+    res["cfg3_bf16_B32of256_4096x8x64"] = {"ms": ms, "tokens/s": Bn * Tn / ms * 1e3,
+                                           "GB/s": 1408 * Bn * Tn * Hn / ms / 1e6}
+    return res
+
+
+def cpu_baseline(np, M, x, do_np):
+    """The C restatement (oracle/c, fp32 state, OpenMP) on a bounded sample of the same
+    workload (configuration 4, forward + backward, one pass)."""
+    from oracle import clib
+    if not clib.available():
+        return {"value": None, "unit": "tokens/s", "cores": 0, "kind": "port", "sample": "oracle not built"}
+    Bs = 64  # the whole batch: about 20 core-seconds
+    sl = {n: x[n][:Bs] for n in ("q", "k", "v", "beta", "done")}
+    dos = do_np[:Bs]
+    cores = clib.num_threads()
+    clib.delta_rule_fwd(sl["q"][:1], sl["k"][:1], sl["v"][:1], sl["beta"][:1], sl["done"][:1], None, "f32")
+    t0 = time.perf_counter()
+    clib.delta_rule_fwd(sl["q"], sl["k"], sl["v"], sl["beta"], sl["done"], None, "f32")
+    clib.delta_rule_bwd(sl["q"], sl["k"], sl["v"], sl["beta"], sl["done"], None, dos, None, "f32")
+    dt = time.perf_counter() - t0
+    T = sl["q"].shape[1]
+    return {"value": Bs * T / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"all {Bs} batch rows of configs[3] (H=8, T={T}, d=64), fwd+bwd once, "
+                      f"sequential recurrence in C (fp32 state), OpenMP over (b,h); {dt:.2f} s"}
+
+
+if __name__ == "__main__":
+    sys.exit(main())
