@@ -126,7 +126,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 
     typename IO::Regs rq, rk, rv, rdo;
     typename IOS::Regs rS;
-    bool rdone = false;
+    uint32_t rdone = 0u;  // raw bits, tested when the chunk is staged
     auto prefetch = [&](int c) {
         const int t0 = c * C;
         IO::load(rq, q + base, rs, t0, Tlen, tid);
@@ -134,16 +134,14 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
         IO::load(rv, v + base, rs, t0, Tlen, tid);
         IO::load(rdo, dout + base, rs, t0, Tlen, tid);
         IOS::load(rS, S_chk + ((int64_t)bh * NC + c) * HD * HD, HD, 0, HD, tid);
-        if (lane < C) {
-            const int t = t0 + lane;
-            rdone = t < Tlen && done_at(done, done_f32, (int64_t)b * Tlen + t);
-        }
+        rdone = 0u;
+        if (lane < C && t0 + lane < Tlen) rdone = done_raw(done, done_f32, (int64_t)b * Tlen + t0 + lane);
     };
     prefetch(NC - 1);
 
     for (int c = NC - 1; c >= 0; --c) {
         const int t0 = c * C;
-        const unsigned long long dmask = __ballot(rdone && lane < C);
+        const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
         for (int pass = nres; pass >= 0; --pass) {
             auto live = [&](int r) { return nres == 0 || episode_of(dmask, r) == pass; };
@@ -182,7 +180,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             }
             if (pass != nres) zero_acc<TMS::TPW>(dSacc);  // an episode that ends inside the chunk
             stage_dS<T>(dSacc, sDS, sDSt, L::LDD, w, lane);
-            __syncthreads();
+            sync_lds();
             if (pass == 0 && c > 0) prefetch(c - 1);
 
             // ---- Aqk^T[j][i] and dAqk[i][j] (+ transpose), causal -----------------------
@@ -210,7 +208,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 store_acc_t<T, C, C>(acc, sDAqk, L::LDC, w, lane);
                 store_acc_n<T, C, C>(acc, sDAqkT, L::LDC, w, lane);
             }
-            __syncthreads();
+            sync_lds();
             auto one = [](int, int) { return f32x4{1.f, 1.f, 1.f, 1.f}; };
             // ---- dV^T[dv][j] = dO^T Aqk + dS K^T ---------------------------------------
             {
@@ -248,7 +246,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             }
             // ---- dS^T[dk][dv] += Q^T dO ---------------------------------------------------
             gemm_nt<T, HD, HD, C>(dSacc, sQt, L::LDC, sDOt, L::LDC, w, lane);
-            __syncthreads();
+            sync_lds();
         }
     }
     if (dS0) {
@@ -326,8 +324,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 
     typename IO::Regs rq, rk, rv, rdo;
     typename IOS::Regs rS;
-    bool rdone = false;
-    float rbeta = 0.f;
+    uint32_t rdone = 0u, rbeta = 0u;  // raw bits, converted when the chunk is staged
     auto prefetch = [&](int c) {
         const int t0 = c * C;
         IO::load(rq, q + base, rs, t0, Tlen, tid);
@@ -335,17 +332,20 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         IO::load(rv, v + base, rs, t0, Tlen, tid);
         IO::load(rdo, dout + base, rs, t0, Tlen, tid);
         IOS::load(rS, S_chk + ((int64_t)bh * NC + c) * HD * HD, HD, 0, HD, tid);
-        if (lane < C) {
-            const int t = t0 + lane;
-            rdone = t < Tlen && done_at(done, done_f32, (int64_t)b * Tlen + t);
-            if (w == 0) rbeta = t < Tlen ? (float)beta[((int64_t)b * Tlen + t) * H + h] : 0.f;
+        rdone = 0u;
+        rbeta = 0u;
+        if (lane < C && t0 + lane < Tlen) {
+            const int64_t bt = (int64_t)b * Tlen + t0 + lane;
+            rdone = done_raw(done, done_f32, bt);
+            if (w == 0) rbeta = load_raw<T>(beta + bt * H + h);
         }
     };
     prefetch(NC - 1);
+    MRX_PHASE_INIT();
 
     for (int c = NC - 1; c >= 0; --c) {
         const int t0 = c * C;
-        const unsigned long long dmask = __ballot(rdone && lane < C);
+        const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
         for (int pass = nres; pass >= 0; --pass) {
             auto live = [&](int r) { return nres == 0 || episode_of(dmask, r) == pass; };
@@ -382,10 +382,11 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 IOS::to_lds(fS, sS, LDD, tid);
                 IOS::to_lds_t(fS, sSt, LDD, tid);
             }
-            if (tid < C) sBeta[tid] = live(tid) ? rbeta : 0.f;
+            if (tid < C) sBeta[tid] = live(tid) ? raw_to_float<T>(rbeta) : 0.f;
             if (pass != nres) zero_acc<TMS::TPW>(dSacc);
             stage_dS<T>(dSacc, sDS, sDSt, LDD, w, lane);
-            __syncthreads();
+            sync_lds();
+            MRX_PHASE(11);
             if (pass == 0 && c > 0) prefetch(c - 1);
 
             // ---- A = beta_i (K K^T) strictly lower -> sA ---------------------------------
@@ -403,8 +404,10 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     *reinterpret_cast<f32x4 *>(sA + n * LDA + m0) = r;
                 }
             }
-            __syncthreads();
+            sync_lds();
+            MRX_PHASE(12);
             tri_inverse<C>(sA, LDA, w, lane);
+            MRX_PHASE(13);
             // ---- sT[i][j] = Tm[i][j] beta_j ; sTmt[j][i] = Tm[i][j] ----------------------
             for (int idx = tid; idx < C * C / 4; idx += NTHREADS) {
                 const int i = idx / (C / 4), j = (idx % (C / 4)) * 4;
@@ -414,7 +417,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                 for (int e = 0; e < 4; ++e) sTmt[(j + e) * LDC + i] = (T)t[e];
             }
-            __syncthreads();
+            sync_lds();
+            MRX_PHASE(14);
             // ---- Aqk^T[j][i] ; W^T[dk][c] = K^T T^T -> sW[c][dk], sWt[dk][c] ---------------
             {
                 f32x4 acc[TMA::TPW];
@@ -436,7 +440,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 store_acc_t<T, HD, C>(acc, sW, LDD, w, lane);
                 store_acc_n<T, HD, C>(acc, sWt, LDC, w, lane);
             }
-            __syncthreads();
+            sync_lds();
+            MRX_PHASE(15);
             // ---- U'^T[dv][c] = V^T T^T - S W^T -> sU[c][dv] (over sS) ------------------------
             {
                 f32x4 acc[TMR::TPW], acc2[TMR::TPW];
@@ -446,7 +451,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 gemm_nt<T, HD, C, HD>(acc2, sS, LDD, sW, LDD, w, lane);
 #pragma unroll
                 for (int j = 0; j < TMR::TPW; ++j) acc[j] -= acc2[j];
-                __syncthreads();  // every wave is done reading sS, sVt, sQ
+                sync_lds();  // every wave is done reading sS, sVt, sQ
+                MRX_PHASE(16);
                 store_acc_t<T, HD, C>(acc, sU, LDD, w, lane);
             }
             // ---- dU'^T[dv][j] = dO^T Aqk + dS K^T -> sDU[j][dv], sDUt[dv][j] -----------------
@@ -458,7 +464,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 store_acc_t<T, HD, C>(acc, sDU, LDD, w, lane);
                 store_acc_n<T, HD, C>(acc, sDUt, LDC, w, lane);
             }
-            __syncthreads();  // sU, sDU, sDUt visible; sDS, sW dead
+            sync_lds();  // sU, sDU, sDUt visible; sDS, sW dead
+            MRX_PHASE(17);
             // ---- dAqk[i][j] = tril(dO U'^T) (+ transpose) ----------------------------------
             {
                 f32x4 acc[TMA::TPW];
@@ -474,7 +481,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 store_acc_t<T, C, C>(acc, sDAqk, LDC, w, lane);
                 store_acc_n<T, C, C>(acc, sDAqkT, LDC, w, lane);
             }
-            __syncthreads();
+            sync_lds();
+            MRX_PHASE(18);
             auto one = [](int, int) { return f32x4{1.f, 1.f, 1.f, 1.f}; };
             // ---- dQ^T[dk][i] = S^T dO^T + K^T dAqk^T -> global -------------------------------
             {
@@ -498,7 +506,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                 for (int j = 0; j < TMS::TPW; ++j) dSacc[j] -= acc[j];
             }
-            __syncthreads();  // sDO, sDOt, sQt, sDAqk*, sDSt dead
+            sync_lds();  // sDO, sDOt, sQt, sDAqk*, sDSt dead
+            MRX_PHASE(19);
             // ---- dW^T[dk][c] = -S^T dU'^T -> sDW[c][dk], sDWt[dk][c] ---------------------------
             {
                 f32x4 acc[TMR::TPW];
@@ -530,7 +539,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 rowdot(acc, sV);
                 store_rows_global<T, C>(acc, dv + base, rs, t0, Tlen, w, lane, beta_of, live);
             }
-            __syncthreads();  // sDW, sDWt visible
+            sync_lds();  // sDW, sDWt visible
+            MRX_PHASE(20);
             // ---- Zw^T[dk][j] = dW^T Tm -> dK += beta_j Zw ; dbeta += K_j . Zw_j -------------------
             {
                 f32x4 acc[TMR::TPW];
@@ -558,7 +568,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 }
                 store_acc_t<T, C, C>(acc, sDTt, LDC, w, lane);
             }
-            __syncthreads();
+            sync_lds();
+            MRX_PHASE(21);
             // ---- Y1: D[m = b][n = j] = dT^T Tm -> sY1[j][b] -----------------------------------------
             {
                 f32x4 acc[TMA::TPW];
@@ -566,7 +577,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 gemm_nt<T, C, C, C>(acc, sDTt, LDC, sTmt, LDC, w, lane);
                 store_acc_t<T, C, C>(acc, sY1, LDC, w, lane);
             }
-            __syncthreads();
+            sync_lds();
+            MRX_PHASE(22);
             // ---- dA: D[m = j][n = i] = -T Y1^T, j < i -> sDA[i][j] ; sGt[j][i] = beta_i dA[i][j] -----
             {
                 f32x4 acc[TMA::TPW];
@@ -583,7 +595,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 for (int j = 0; j < TMA::TPW; ++j) acc[j] *= sBeta[TMA::nt(w, j) * 16 + li];
                 store_acc_n<T, C, C>(acc, sGt, LDC, w, lane);
             }
-            __syncthreads();
+            sync_lds();
+            MRX_PHASE(23);
             // ---- R^T[dk][i] = K^T dA^T -> dK += beta_i R ; dbeta += K_i . R_i ; dK += K^T G ---------
             {
                 f32x4 acc[TMR::TPW];
@@ -606,14 +619,16 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 x += __shfl_xor(x, 32);
                 if (lg == 0) sDb[w * C + TMR::nt(w, j) * 16 + li] = x;
             }
-            __syncthreads();
+            sync_lds();
+            MRX_PHASE(24);
             if (tid < C && t0 + tid < Tlen && live(tid)) {
                 float x = 0.f;
 #pragma unroll
                 for (int ww = 0; ww < NWAVES; ++ww) x += sDb[ww * C + tid];
                 dbeta[((int64_t)b * Tlen + t0 + tid) * H + h] = (T)x;
             }
-            __syncthreads();
+            sync_lds();
+            MRX_PHASE(25);
         }
     }
     if (dS0) {

@@ -20,6 +20,15 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains the
+// vector-memory counter, which would make every barrier wait for the next chunk's
+// global prefetch; the compiler still inserts the vmcnt wait where a prefetched
+// register is first consumed.
+__device__ __forceinline__ void sync_lds()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 constexpr int NWAVES = 4;
 constexpr int NTHREADS = 64 * NWAVES;
 constexpr int HD = 64;  // head dim (d_k = d_v)
@@ -130,6 +139,20 @@ __device__ __forceinline__ void store_acc_n(const f32x4 *acc, T *dst, int ld, in
     }
 }
 
+// Raw bits of one T-typed scalar (converted to float only when consumed).
+template <typename T> __device__ __forceinline__ uint32_t load_raw(const T *p);
+template <> __device__ __forceinline__ uint32_t load_raw<__bf16>(const __bf16 *p)
+{
+    return (uint32_t) *reinterpret_cast<const uint16_t *>(p);
+}
+template <> __device__ __forceinline__ uint32_t load_raw<float>(const float *p)
+{
+    return *reinterpret_cast<const uint32_t *>(p);
+}
+template <typename T> __device__ __forceinline__ float raw_to_float(uint32_t raw);
+template <> __device__ __forceinline__ float raw_to_float<__bf16>(uint32_t raw) { return __uint_as_float(raw << 16); }
+template <> __device__ __forceinline__ float raw_to_float<float>(uint32_t raw) { return __uint_as_float(raw); }
+
 __device__ __forceinline__ float elu1(float x) { return x > 0.f ? x + 1.f : __expf(x); }
 __device__ __forceinline__ float delu1(float x) { return x > 0.f ? 1.f : __expf(x); }
 
@@ -204,35 +227,46 @@ __device__ __forceinline__ int episode_of(unsigned long long dmask, int r)
 // sA holds A (strictly lower part used), C x C with leading dim ld; on return the
 // inverse X of (I + A) is stored as: diagonal 16x16 blocks in place; block (b, c),
 // b > c, in the unused upper position (c, b) (same orientation).  Needs all 4 waves
-// (contains __syncthreads()).
+// (contains workgroup barriers).
 template <int C> __device__ __forceinline__ void tri_inverse(float *sA, int ld, int w, int lane)
 {
     constexpr int NB = C / 16;
     const int i = lane & 15, g = lane >> 4;
-    if (w == 0 && lane < NB * 16) {
-        // forward substitution on the diagonal blocks: lane = (block g, column i)
-        float *blk = sA + (16 * g) * ld + 16 * g;
-        float x[16];
+    if (w < NB) {
+        // Diagonal block w by repeated squaring, entirely in registers.  With N = -A
+        // (nilpotent, N^16 = 0): (I + A)^-1 = (I + N)(I + N^2)(I + N^4)(I + N^8).
+        // A 16x16 product P = X Y on the fp32 MFMA takes X^T and Y both in accumulator
+        // layout (lane (i,g) holds Z[4g+v][i]), so each matrix is carried together with
+        // its transpose and no operand goes through LDS.
+        float *blk = sA + (16 * w) * ld + 16 * w;
+        auto mm = [](const f32x4 &xt, const f32x4 &y, f32x4 c) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            float row[16];
+            for (int s = 0; s < 4; ++s) c = __builtin_amdgcn_mfma_f32_16x16x4f32(xt[s], y[s], c, 0, 0, 0);
+            return c;
+        };
+        const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+        f32x4 M, Mt, R, Rt;
+        Mt = *reinterpret_cast<const f32x4 *>(blk + i * ld + 4 * g);  // A[i][4g+v] = (A^T)[4g+v][i]
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const f32x4 t = *reinterpret_cast<const f32x4 *>(blk + r * ld + 4 * q);
-                row[4 * q + 0] = t[0]; row[4 * q + 1] = t[1]; row[4 * q + 2] = t[2]; row[4 * q + 3] = t[3];
-            }
-            float s0 = (r == i) ? 1.f : 0.f, s1 = 0.f;
-#pragma unroll
-            for (int j = 0; j < r; ++j) {
-                if (j & 1) s1 -= row[j] * x[j];
-                else s0 -= row[j] * x[j];
-            }
-            x[r] = s0 + s1;
+        for (int v = 0; v < 4; ++v) {
+            const int r = 4 * g + v;
+            M[v] = (i < r) ? -blk[r * ld + i] : 0.f;   // N[r][i], strictly lower
+            Mt[v] = (r < i) ? -Mt[v] : 0.f;            // N^T[r][i] = N[i][r], strictly upper
+            R[v] = M[v] + (r == i ? 1.f : 0.f);
+            Rt[v] = Mt[v] + (r == i ? 1.f : 0.f);
         }
 #pragma unroll
-        for (int r = 0; r < 16; ++r) blk[r * ld + i] = x[r];
+        for (int k = 0; k < 3; ++k) {
+            const f32x4 M2 = mm(Mt, M, zero);    // N^2  : X = M,  Y = M
+            const f32x4 M2t = mm(M, Mt, zero);   // (N^2)^T = M^T M^T : X = M^T, Y = M^T
+            const f32x4 R2 = mm(Rt, M2, R);      // R + R M2
+            const f32x4 R2t = mm(M2, Rt, Rt);    // R^T + M2^T R^T
+            M = M2; Mt = M2t; R = R2; Rt = R2t;
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) blk[(4 * g + v) * ld + i] = R[v];
     }
-    __syncthreads();
+    sync_lds();
 #pragma unroll
     for (int d = 1; d < NB; ++d) {
         if (w < NB - d) {
@@ -255,7 +289,7 @@ template <int C> __device__ __forceinline__ void tri_inverse(float *sA, int ld, 
 #pragma unroll
             for (int v = 0; v < 4; ++v) sA[(16 * c + 4 * g + v) * ld + 16 * b + i] = -res[v];
         }
-        __syncthreads();
+        sync_lds();
     }
 }
 

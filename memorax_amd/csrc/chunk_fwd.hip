@@ -6,7 +6,9 @@
 //                      W  = T K,  U' = T V - diag(m) W S^T
 //   both:              O  = diag(m) Q S^T + (tril(Q K^T) . M) U'
 //                      S <- l S + (diag(e) U')^T K
-// M, m, e, l are the episode masks of the chunk (episode_of in chunk_common.h).  The state is
+// M, m, e, l are the episode masks of the chunk; they are realised by processing a
+// chunk that contains resets once per episode with the other episodes' rows zeroed
+// by select, so inside a pass only the causal mask remains.  The state is
 // kept transposed (S^T, d_k x d_v) in MFMA accumulators for the whole sequence and
 // re-staged to LDS as a T-typed d_v x d_k tile once per chunk.
 #include "chunk_common.h"
@@ -30,12 +32,11 @@ template <typename T, int C, bool DELTA> struct FwdSmem {
     static constexpr int szA = DELTA ? C * LDA * 4 : 0;  // sA fp32 [C][C], overlaid by sAqk afterwards
     static constexpr int szAA = szA > szAq ? szA : szAq;
     static constexpr int oQ = 0, oK = oQ + szQ, oKt = oK + szK, oVt = oKt + szKt, oS = oVt + szVt,
-                         oT = oS + szS, oA = oT + szT, oBeta = oA + szAA, oSeg = oBeta + C * 4,
-                         oMeta = oSeg + C * 4, total = oMeta + 16;
+                         oT = oS + szS, oA = oT + szT, oBeta = oA + szAA, total = oBeta + C * 4;
 };
 
 template <typename T, int C, bool DELTA, bool FMAP>
-__global__ void __launch_bounds__(NTHREADS)
+__global__ void __launch_bounds__(NTHREADS, 2)  // 2 waves per SIMD: two workgroups share a CU
 chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
                  const float *__restrict__ S0, T *__restrict__ o, float *__restrict__ S_last,
@@ -56,7 +57,6 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     float *sA = reinterpret_cast<float *>(smem + L::oA);
     T *sAqk = reinterpret_cast<T *>(smem + L::oA);
     float *sBeta = reinterpret_cast<float *>(smem + L::oBeta);
-    int *sSeg = reinterpret_cast<int *>(smem + L::oSeg);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -81,20 +81,23 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 
     // register prefetch of the next chunk
     typename IO::Regs rq, rk, rv;
-    float rbeta = 0.f;
-    bool rdone = false;
+    uint32_t rbeta = 0u, rdone = 0u;  // raw bits, converted when the chunk is staged
     auto prefetch = [&](int c) {
         const int t0 = c * C;
         IO::load(rq, qb, rs, t0, Tlen, tid);
         IO::load(rk, kb, rs, t0, Tlen, tid);
         IO::load(rv, vb, rs, t0, Tlen, tid);
-        if (lane < C) {
-            const int t = t0 + lane;
-            rdone = t < Tlen && done_at(done, done_f32, (int64_t)b * Tlen + t);
-            if (DELTA && w == 0) rbeta = t < Tlen ? (float)beta[((int64_t)b * Tlen + t) * H + h] : 0.f;
+        rdone = 0u;
+        rbeta = 0u;
+        if (lane < C && t0 + lane < Tlen) {
+            const int64_t bt = (int64_t)b * Tlen + t0 + lane;
+            rdone = done_raw(done, done_f32, bt);
+            if (DELTA && w == 0) rbeta = load_raw<T>(beta + bt * H + h);
         }
     };
+    MRX_WG_BEGIN();
     prefetch(0);
+    MRX_PHASE_INIT();
 
     for (int c = 0; c < NC; ++c) {
         const int t0 = c * C;
@@ -102,7 +105,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         // A chunk that contains resets is processed once per episode ("pass") with
         // the rows of all other episodes replaced by zeros *by select*, so that a
         // non-finite value never meets a masked-out zero inside a matrix product.
-        const unsigned long long dmask = __ballot(rdone && lane < C);
+        const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
         for (int pass = 0; pass <= nres; ++pass) {
         // ---- P0: stage the chunk -------------------------------------------------
@@ -115,7 +118,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                 for (int p = 0; p < IO::PASSES; ++p) {
                     const int r = r0 + p * IO::RPP;
-                    if (__popcll(dmask & ((2ull << r) - 1ull)) != pass) {
+                    if (episode_of(dmask, r) != pass) {
 #pragma unroll
                         for (int e = 0; e < IO::KP; ++e) {
                             fq.v[p][e] = (T)0.f; fk.v[p][e] = (T)0.f; fv.v[p][e] = (T)0.f;
@@ -129,11 +132,8 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             IO::to_lds_t(fv, sVt, L::LDC, tid);
         }
         if (tid < C) {
-            const int sg = __popcll(dmask & ((2ull << tid) - 1ull));
-            // inside a pass every live row counts as episode 0 of the pass; rows of
-            // other episodes get a different id so that the masks below drop them
-            sSeg[tid] = nres == 0 ? 0 : (sg == pass ? 0 : 1);
-            if (DELTA) sBeta[tid] = (nres == 0 || sg == pass) ? rbeta : 0.f;
+            const int sg = episode_of(dmask, tid);
+            if (DELTA) sBeta[tid] = (nres == 0 || sg == pass) ? raw_to_float<T>(rbeta) : 0.f;
         }
         if (pass != 0) zero_acc<TMS::TPW>(Sacc);  // an episode that starts in the chunk starts from 0
         store_acc_t<T, HD, HD>(Sacc, sS, L::LDD, w, lane);  // sS[dv][dk]
@@ -146,7 +146,8 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     TT<T>::pack(Sacc[j][0], Sacc[j][1], Sacc[j][2], Sacc[j][3]);
             }
         }
-        __syncthreads();
+        sync_lds();
+        MRX_PHASE(1);
         if (pass == nres && c + 1 < NC) prefetch(c + 1);
 
         // ---- P1: O^T = m . S Q^T (m over columns), A = beta_i (K K^T) strictly lower ----
@@ -154,11 +155,6 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         f32x4 Oacc[TMO::TPW];
         zero_acc<TMO::TPW>(Oacc);
         gemm_nt<T, HD, C, HD>(Oacc, sS, L::LDD, sQ, L::LDD, w, lane);
-#pragma unroll
-        for (int j = 0; j < TMO::TPW; ++j) {
-            const int cc = TMO::nt(w, j) * 16 + li;
-            if (sSeg[cc] != 0) Oacc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
         using TMA = TileMap<C, C>;
         if (DELTA) {
             f32x4 acc[TMA::TPW];
@@ -169,26 +165,27 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             for (int j = 0; j < TMA::TPW; ++j) {
                 const int m0 = TMA::mt(w) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
                 const float bi = sBeta[n];
-                const int sn = sSeg[n];
                 f32x4 r;
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    r[e] = (m0 + e < n && sSeg[m0 + e] == sn) ? bi * acc[j][e] : 0.f;
+                for (int e = 0; e < 4; ++e) r[e] = (m0 + e < n) ? bi * acc[j][e] : 0.f;
                 *reinterpret_cast<f32x4 *>(sA + n * L::LDA + m0) = r;
             }
         }
-        __syncthreads();
+        sync_lds();
+        MRX_PHASE(2);
 
         if (DELTA) {
             // ---- P2/P3: Tm = (I + A)^-1 ; sT[i][j] = Tm[i][j] beta_j -----------------
             tri_inverse<C>(sA, L::LDA, w, lane);
+            MRX_PHASE(3);
             for (int idx = tid; idx < C * C / 4; idx += NTHREADS) {
                 const int i = idx / (C / 4), j = (idx % (C / 4)) * 4;
                 const f32x4 t = tri_inverse_get4(sA, L::LDA, i, j);
                 *reinterpret_cast<P4 *>(sT + i * L::LDC + j) =
                     TT<T>::pack(t[0] * sBeta[j], t[1] * sBeta[j + 1], t[2] * sBeta[j + 2], t[3] * sBeta[j + 3]);
             }
-            __syncthreads();
+            sync_lds();
+        MRX_PHASE(4);
         }
 
         // ---- P4: Aqk[i][j] = (q_i . k_j) [j <= i, same episode] ; U = T V ------------
@@ -199,10 +196,9 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
             for (int j = 0; j < TMA::TPW; ++j) {
                 const int m0 = TMA::mt(w) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
-                const int sn = sSeg[n];
                 float r[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) r[e] = (m0 + e <= n && sSeg[m0 + e] == sn) ? acc[j][e] : 0.f;
+                for (int e = 0; e < 4; ++e) r[e] = (m0 + e <= n) ? acc[j][e] : 0.f;
                 *reinterpret_cast<P4 *>(sAqk + n * L::LDC + m0) = TT<T>::pack(r[0], r[1], r[2], r[3]);
             }
         }
@@ -211,7 +207,8 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             f32x4 Uacc[TMU::TPW];
             zero_acc<TMU::TPW>(Uacc);
             gemm_nt<T, C, HD, C>(Uacc, sT, L::LDC, sVt, L::LDC, w, lane);
-            __syncthreads();  // sQ and sVt are dead, sAqk visible
+            sync_lds();  // sQ and sVt are dead, sAqk visible
+        MRX_PHASE(5);
             // ---- P5: W^T = K^T T^T -> sW[c][dk] ---------------------------------------
             {
                 using TMW = TileMap<HD, C>;  // m = dk, n = c
@@ -220,38 +217,38 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 gemm_nt<T, HD, C, C>(acc, sKt, L::LDC, sT, L::LDC, w, lane);
                 store_acc_t<T, HD, C>(acc, sW, L::LDD, w, lane);
             }
-            __syncthreads();
+            sync_lds();
+        MRX_PHASE(6);
             // ---- P6: U' = U - m . W S^T -> sUt[dv][c] -----------------------------------
             {
                 f32x4 acc[TMU::TPW];
                 zero_acc<TMU::TPW>(acc);
                 gemm_nt<T, C, HD, HD>(acc, sW, L::LDD, sS, L::LDD, w, lane);
-                const int m0 = TMU::mt(w) * 16 + 4 * lg;
 #pragma unroll
-                for (int j = 0; j < TMU::TPW; ++j)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (sSeg[m0 + e] == 0) Uacc[j][e] -= acc[j][e];
+                for (int j = 0; j < TMU::TPW; ++j) Uacc[j] -= acc[j];
                 store_acc_t<T, C, HD>(Uacc, sUt, L::LDC, w, lane);
             }
         }
-        __syncthreads();
+        sync_lds();
+        MRX_PHASE(7);
 
         // ---- P7: O^T += U'^T Aqk^T ; store O ----------------------------------------
         gemm_nt<T, HD, C, C>(Oacc, sUt, L::LDC, sAqk, L::LDC, w, lane);
 #pragma unroll
         for (int j = 0; j < TMO::TPW; ++j) {
             const int dv0 = TMO::mt(w) * 16 + 4 * lg, cc = TMO::nt(w, j) * 16 + li;
-            if (t0 + cc < Tlen && sSeg[cc] == 0)
+            if (t0 + cc < Tlen && (nres == 0 || episode_of(dmask, cc) == pass))
                 *reinterpret_cast<P4 *>(ob + (int64_t)(t0 + cc) * rs + dv0) =
                     TT<T>::pack(Oacc[j][0], Oacc[j][1], Oacc[j][2], Oacc[j][3]);
         }
         // ---- P8: S^T <- S^T + K^T U'  (only the episode that leaves the chunk) ---------
         if (pass == nres) gemm_nt<T, HD, HD, C>(Sacc, sKt, L::LDC, sUt, L::LDC, w, lane);
-        __syncthreads();
+        sync_lds();
+        MRX_PHASE(8);
         }  // pass
     }
 
+    MRX_WG_END();
     if (S_last) {
 #pragma unroll
         for (int j = 0; j < TMS::TPW; ++j) {
