@@ -11,14 +11,20 @@
 // Per pass (rows i >= j; all rows of one episode):
 //   Aqk = tril(Q K^T)                      dU' = Aqk^T dO + K dS^T
 //   dAqk = tril(dO U'^T)                   dQ  = dO S + dAqk K
-//   dK  = dAqk^T Q + U' dS                 dS <- dS + dO^T Q - dU'^T W
+//   dK  = dAqk^T Q + U' dS                 dS <- dS + Q^T dO - W^T dU'   (stored as dS^T)
 //   linear attention: U' = V, dV = dU', W = 0.
 //   delta rule:  A = tril(diag(beta) K K^T, -1), Tm = (I+A)^-1, T = Tm diag(beta),
 //     W = T K, U' = T V - W S^T, dW = -dU' S, Zu = Tm^T dU', Zw = Tm^T dW,
 //     dV = diag(beta) Zu, dK += diag(beta) Zw, dbeta = rowdot(V, Zu) + rowdot(K, Zw),
 //     dT = tril(dW K^T + dU' V^T), dA = -tril((Tm^T dT) T^T, -1),
 //     R = dA K, dbeta += rowdot(K, R), dK += diag(beta) R + (diag(beta) dA)^T K.
+// Every tile lives in LDS once, in its natural orientation; products that contract over
+// the row index read it through transpose loads (KROW operands).
 #include "chunk_common.h"
+
+#ifndef MRX_DELTA_BWD_WAVES
+#define MRX_DELTA_BWD_WAVES 8  // waves per workgroup of the delta-rule backward kernel (4 or 8)
+#endif
 
 namespace {
 
@@ -29,7 +35,6 @@ template <typename T, int C> struct BwdDims {
     static constexpr int LDD = HD + PAD;  // leading dim of tiles with 64 columns
     static constexpr int LDC = C + PAD;   // leading dim of tiles with C columns
     static constexpr int szRD = C * LDD * sizeof(T);   // [C][64]
-    static constexpr int szDR = HD * LDC * sizeof(T);  // [64][C]
     static constexpr int szDD = HD * LDD * sizeof(T);  // [64][64]
     static constexpr int szCC = C * LDC * sizeof(T);   // [C][C]
 };
@@ -37,23 +42,13 @@ template <typename T, int C> struct BwdDims {
 // d(phi)/dx recovered from the staged phi(x): phi > 1 <=> x > 0 (derivative 1), else phi' = phi.
 template <bool FMAP> __device__ __forceinline__ float fmap_grad(float phi) { return FMAP ? (phi > 1.f ? 1.f : phi) : 1.f; }
 
-// ---- shared pieces ----------------------------------------------------------------
-
-// Stage dS (held as dS^T: m = dk, n = dv) into sdS[dv][dk] and sdSt[dk][dv].
-template <typename T>
-__device__ __forceinline__ void stage_dS(const f32x4 *dSacc, T *sdS, T *sdSt, int ld, int w, int lane)
-{
-    store_acc_t<T, HD, HD>(dSacc, sdS, ld, w, lane);
-    store_acc_n<T, HD, HD>(dSacc, sdSt, ld, w, lane);
-}
-
 // Write an accumulator set holding X^T (m = feature, n = chunk row) to a (B,T,H,64)
-// array: 4 consecutive features per lane.  scale(row) multiplies, keep(row) gates.
-template <typename T, int C, typename ScaleF, typename KeepF>
+// array: 4 consecutive features per lane.  scale(row, d0) multiplies, keep(row) gates.
+template <typename T, int C, int NW, typename ScaleF, typename KeepF>
 __device__ __forceinline__ void store_rows_global(const f32x4 *acc, T *base, int64_t rs, int t0, int Tlen,
                                                   int w, int lane, ScaleF scale, KeepF keep)
 {
-    using TM = TileMap<HD, C>;
+    using TM = TileMap<HD, C, NW>;
     using P4 = typename TT<T>::pack4;
     const int li = lane & 15, lg = lane >> 4;
 #pragma unroll
@@ -68,42 +63,37 @@ __device__ __forceinline__ void store_rows_global(const f32x4 *acc, T *base, int
 }
 
 // =====================================================================================
-// linear attention
+// linear attention: 8 tiles, two workgroups per CU
 // =====================================================================================
 template <typename T, int C> struct LaBwdSmem : BwdDims<T, C> {
     using D = BwdDims<T, C>;
     static constexpr int oQ = 0, oK = oQ + D::szRD, oV = oK + D::szRD, oDO = oV + D::szRD,
-                         oQt = oDO + D::szRD, oKt = oQt + D::szDR, oDOt = oKt + D::szDR,
-                         oSt = oDOt + D::szDR, oDS = oSt + D::szDD, oDSt = oDS + D::szDD,
-                         oAqkT = oDSt + D::szDD, oDAqk = oAqkT + D::szCC, oDAqkT = oDAqk + D::szCC,
-                         total = oDAqkT + D::szCC;
+                         oS = oDO + D::szRD, oDS = oS + D::szDD, oAqk = oDS + D::szDD,
+                         oDAqk = oAqk + D::szCC, total = oDAqk + D::szCC;
 };
 
 template <typename T, int C, bool FMAP>
-__global__ void __launch_bounds__(NTHREADS)
+__global__ void __launch_bounds__(256, 2)
 la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
               const void *__restrict__ done, int done_f32, const T *__restrict__ S_chk,
               const T *__restrict__ dout, const float *__restrict__ dS_last, T *__restrict__ dq,
               T *__restrict__ dk, T *__restrict__ dv, float *__restrict__ dS0, int Tlen, int H)
 {
+    constexpr int NW = 4, NTHR = 64 * NW;
     using L = LaBwdSmem<T, C>;
-    using IO = TileIO<T, C>;
-    using IOS = TileIO<T, HD>;
+    using IO = TileIO<T, C, NTHR>;
+    using IOS = TileIO<T, HD, NTHR>;
     using P4 = typename TT<T>::pack4;
+    constexpr int LDD = L::LDD, LDC = L::LDC;
     extern __shared__ __align__(16) unsigned char smem[];
     T *sQ = reinterpret_cast<T *>(smem + L::oQ);
     T *sK = reinterpret_cast<T *>(smem + L::oK);
     T *sV = reinterpret_cast<T *>(smem + L::oV);
     T *sDO = reinterpret_cast<T *>(smem + L::oDO);
-    T *sQt = reinterpret_cast<T *>(smem + L::oQt);
-    T *sKt = reinterpret_cast<T *>(smem + L::oKt);
-    T *sDOt = reinterpret_cast<T *>(smem + L::oDOt);
-    T *sSt = reinterpret_cast<T *>(smem + L::oSt);
+    T *sS = reinterpret_cast<T *>(smem + L::oS);
     T *sDS = reinterpret_cast<T *>(smem + L::oDS);
-    T *sDSt = reinterpret_cast<T *>(smem + L::oDSt);
-    T *sAqkT = reinterpret_cast<T *>(smem + L::oAqkT);
+    T *sAqk = reinterpret_cast<T *>(smem + L::oAqk);
     T *sDAqk = reinterpret_cast<T *>(smem + L::oDAqk);
-    T *sDAqkT = reinterpret_cast<T *>(smem + L::oDAqkT);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -113,9 +103,9 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     const int64_t base = ((int64_t)b * Tlen * H + h) * HD;
     const int NC = (Tlen + C - 1) / C;
 
-    using TMS = TileMap<HD, HD>;
-    using TMA = TileMap<C, C>;
-    using TMR = TileMap<HD, C>;
+    using TMS = TileMap<HD, HD, NW>;
+    using TMA = TileMap<C, C, NW>;
+    using TMR = TileMap<HD, C, NW>;
     f32x4 dSacc[TMS::TPW];  // dS^T: m = dk, n = dv
 #pragma unroll
     for (int j = 0; j < TMS::TPW; ++j) {
@@ -151,101 +141,72 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 IO::template fmap<FMAP>(fq);
                 IO::template fmap<FMAP>(fk);
                 if (nres != 0) {
-                    const int r0 = tid / IO::SEGS;
-#pragma unroll
-                    for (int p = 0; p < IO::PASSES; ++p) {
-                        if (!live(r0 + p * IO::RPP)) {
-#pragma unroll
-                            for (int e = 0; e < IO::KP; ++e) {
-                                fq.v[p][e] = (T)0.f; fk.v[p][e] = (T)0.f; fv.v[p][e] = (T)0.f; fdo.v[p][e] = (T)0.f;
-                            }
-                        }
-                    }
+                    IO::mask_rows(fq, tid, live);
+                    IO::mask_rows(fk, tid, live);
+                    IO::mask_rows(fv, tid, live);
+                    IO::mask_rows(fdo, tid, live);
                 }
-                IO::to_lds(fq, sQ, L::LDD, tid);
-                IO::to_lds_t(fq, sQt, L::LDC, tid);
-                IO::to_lds(fk, sK, L::LDD, tid);
-                IO::to_lds_t(fk, sKt, L::LDC, tid);
-                IO::to_lds(fv, sV, L::LDD, tid);
-                IO::to_lds(fdo, sDO, L::LDD, tid);
-                IO::to_lds_t(fdo, sDOt, L::LDC, tid);
+                IO::to_lds(fq, sQ, LDD, tid);
+                IO::to_lds(fk, sK, LDD, tid);
+                IO::to_lds(fv, sV, LDD, tid);
+                IO::to_lds(fdo, sDO, LDD, tid);
                 typename IOS::Regs fS = rS;
-                if (pass != 0) {
-#pragma unroll
-                    for (int p = 0; p < IOS::PASSES; ++p)
-#pragma unroll
-                        for (int e = 0; e < IOS::KP; ++e) fS.v[p][e] = (T)0.f;
-                }
-                IOS::to_lds_t(fS, sSt, L::LDD, tid);  // S_chk is [dv][dk]; sSt[dk][dv]
+                if (pass != 0) IOS::zero(fS);
+                IOS::to_lds(fS, sS, LDD, tid);  // S[dv][dk]
             }
             if (pass != nres) zero_acc<TMS::TPW>(dSacc);  // an episode that ends inside the chunk
-            stage_dS<T>(dSacc, sDS, sDSt, L::LDD, w, lane);
+            store_acc<T, HD, HD, NW>(dSacc, sDS, LDD, w, lane);  // dS[dv][dk]
             sync_lds();
             if (pass == 0 && c > 0) prefetch(c - 1);
 
-            // ---- Aqk^T[j][i] and dAqk[i][j] (+ transpose), causal -----------------------
+            // ---- Aqk[i][j] = q_i.k_j, dAqk[i][j] = do_i.v_j, both j <= i ------------------
             {
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
-                gemm_nt<T, C, C, HD>(acc, sQ, L::LDD, sK, L::LDD, w, lane);  // D[m = i][n = j]
-#pragma unroll
-                for (int j = 0; j < TMA::TPW; ++j) {
-                    const int m0 = TMA::mt(w) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (m0 + e < n) acc[j][e] = 0.f;
-                }
-                store_acc_t<T, C, C>(acc, sAqkT, L::LDC, w, lane);
+                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sK, LDD, sQ, LDD, w, lane);  // D[m = j][n = i]
+                store_acc_f<T, C, C, NW>(acc, sAqk, LDC, w, lane, [](int m, int n, float x) { return m <= n ? x : 0.f; });
                 zero_acc<TMA::TPW>(acc);
-                gemm_nt<T, C, C, HD>(acc, sV, L::LDD, sDO, L::LDD, w, lane);  // D[m = j][n = i]
-#pragma unroll
-                for (int j = 0; j < TMA::TPW; ++j) {
-                    const int m0 = TMA::mt(w) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (m0 + e > n) acc[j][e] = 0.f;
-                }
-                store_acc_t<T, C, C>(acc, sDAqk, L::LDC, w, lane);
-                store_acc_n<T, C, C>(acc, sDAqkT, L::LDC, w, lane);
+                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sV, LDD, sDO, LDD, w, lane);  // D[m = j][n = i]
+                store_acc_f<T, C, C, NW>(acc, sDAqk, LDC, w, lane, [](int m, int n, float x) { return m <= n ? x : 0.f; });
             }
             sync_lds();
             auto one = [](int, int) { return f32x4{1.f, 1.f, 1.f, 1.f}; };
-            // ---- dV^T[dv][j] = dO^T Aqk + dS K^T ---------------------------------------
+            // ---- dV^T[dv][j] = sum_i dO[i][dv] Aqk[i][j] + sum_dk dS[dv][dk] K[j][dk] -------
             {
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
-                gemm_nt<T, HD, C, C>(acc, sDOt, L::LDC, sAqkT, L::LDC, w, lane);
-                gemm_nt<T, HD, C, HD>(acc, sDS, L::LDD, sK, L::LDD, w, lane);
-                store_rows_global<T, C>(acc, dv + base, rs, t0, Tlen, w, lane, one, live);
+                gemm<T, HD, C, C, KROW, KROW, NW>(acc, sDO, LDD, sAqk, LDC, w, lane);
+                gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc, sDS, LDD, sK, LDD, w, lane);
+                store_rows_global<T, C, NW>(acc, dv + base, rs, t0, Tlen, w, lane, one, live);
             }
-            // ---- dQ^T[dk][i] = S^T dO^T + K^T dAqk^T -----------------------------------
+            // ---- dQ^T[dk][i] = sum_dv S[dv][dk] dO[i][dv] + sum_j K[j][dk] dAqk[i][j] ---------
             {
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
-                gemm_nt<T, HD, C, HD>(acc, sSt, L::LDD, sDO, L::LDD, w, lane);
-                gemm_nt<T, HD, C, C>(acc, sKt, L::LDC, sDAqk, L::LDC, w, lane);
+                gemm<T, HD, C, HD, KROW, ROWK, NW>(acc, sS, LDD, sDO, LDD, w, lane);
+                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sK, LDD, sDAqk, LDC, w, lane);
                 auto sc = [&](int r, int d0) {
-                    const P4 x = *reinterpret_cast<const P4 *>(sQ + r * L::LDD + d0);
+                    const P4 x = *reinterpret_cast<const P4 *>(sQ + r * LDD + d0);
                     return f32x4{fmap_grad<FMAP>((float)x[0]), fmap_grad<FMAP>((float)x[1]),
                                  fmap_grad<FMAP>((float)x[2]), fmap_grad<FMAP>((float)x[3])};
                 };
-                store_rows_global<T, C>(acc, dq + base, rs, t0, Tlen, w, lane, sc, live);
+                store_rows_global<T, C, NW>(acc, dq + base, rs, t0, Tlen, w, lane, sc, live);
             }
-            // ---- dK^T[dk][j] = Q^T dAqk + dS^T V^T --------------------------------------
+            // ---- dK^T[dk][j] = sum_i Q[i][dk] dAqk[i][j] + sum_dv dS[dv][dk] V[j][dv] -----------
             {
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
-                gemm_nt<T, HD, C, C>(acc, sQt, L::LDC, sDAqkT, L::LDC, w, lane);
-                gemm_nt<T, HD, C, HD>(acc, sDSt, L::LDD, sV, L::LDD, w, lane);
+                gemm<T, HD, C, C, KROW, KROW, NW>(acc, sQ, LDD, sDAqk, LDC, w, lane);
+                gemm<T, HD, C, HD, KROW, ROWK, NW>(acc, sDS, LDD, sV, LDD, w, lane);
                 auto sc = [&](int r, int d0) {
-                    const P4 x = *reinterpret_cast<const P4 *>(sK + r * L::LDD + d0);
+                    const P4 x = *reinterpret_cast<const P4 *>(sK + r * LDD + d0);
                     return f32x4{fmap_grad<FMAP>((float)x[0]), fmap_grad<FMAP>((float)x[1]),
                                  fmap_grad<FMAP>((float)x[2]), fmap_grad<FMAP>((float)x[3])};
                 };
-                store_rows_global<T, C>(acc, dk + base, rs, t0, Tlen, w, lane, sc, live);
+                store_rows_global<T, C, NW>(acc, dk + base, rs, t0, Tlen, w, lane, sc, live);
             }
-            // ---- dS^T[dk][dv] += Q^T dO ---------------------------------------------------
-            gemm_nt<T, HD, HD, C>(dSacc, sQt, L::LDC, sDOt, L::LDC, w, lane);
+            // ---- dS^T[dk][dv] += sum_c Q[c][dk] dO[c][dv] -----------------------------------------
+            gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, sQ, LDD, sDO, LDD, w, lane);
             sync_lds();
         }
     }
@@ -259,49 +220,45 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 }
 
 // =====================================================================================
-// delta rule (bf16, C = 64: seventeen 9 KiB regions, reused as operands die)
+// delta rule (bf16, C = 64): twelve 9 KiB regions, reused as operands die; NW waves
 // =====================================================================================
-template <typename T, int C> struct DeltaBwdSmem : BwdDims<T, C> {
+template <typename T, int C, int NW> struct DeltaBwdSmem : BwdDims<T, C> {
     using D = BwdDims<T, C>;
     static constexpr int U = D::szDD;  // every tile type has this size for bf16 / C = 64
-    static_assert(D::szRD == U && D::szDR == U && D::szCC == U, "regions assume equal tile sizes");
+    static_assert(D::szRD == U && D::szCC == U, "regions assume equal tile sizes");
     static_assert(C * (C + 4) * 4 <= 2 * U, "fp32 A must fit two regions");
-    static constexpr int NREG = 17;
-    static constexpr int oBeta = NREG * U, oDb = oBeta + C * 4, total = oDb + NWAVES * C * 4;
+    static constexpr int NREG = 12;
+    static constexpr int oBeta = NREG * U, oDb = oBeta + C * 4, total = oDb + 4 * C * 4;
 };
 
-template <typename T, int C>
-__global__ void __launch_bounds__(NTHREADS)
+template <typename T, int C, int NW>
+__global__ void __launch_bounds__(64 * NW)
 delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
                  const T *__restrict__ S_chk, const T *__restrict__ dout,
                  const float *__restrict__ dS_last, T *__restrict__ dq, T *__restrict__ dk,
                  T *__restrict__ dv, T *__restrict__ dbeta, float *__restrict__ dS0, int Tlen, int H)
 {
-    using L = DeltaBwdSmem<T, C>;
-    using IO = TileIO<T, C>;
-    using IOS = TileIO<T, HD>;
+    constexpr int NTHR = 64 * NW;
+    using L = DeltaBwdSmem<T, C, NW>;
+    using IO = TileIO<T, C, NTHR>;
+    using IOS = TileIO<T, HD, NTHR>;
     using P4 = typename TT<T>::pack4;
     constexpr int LDD = L::LDD, LDC = L::LDC, LDA = C + 4;
     extern __shared__ __align__(16) unsigned char smem[];
     auto reg = [&](int r) { return reinterpret_cast<T *>(smem + r * L::U); };
-    // region plan (-> marks reuse once the first tenant is dead)
-    T *sK = reg(0), *sKt = reg(1), *sV = reg(2);
-    T *sVt = reg(3), *sDU = reg(3);           // Vt -> dU'[c][dv]
-    T *sQ = reg(4), *sDUt = reg(4);           // Q  -> dU'^T[dv][c]
-    T *sQt = reg(5), *sDTt = reg(5);          // Qt -> dT^T[b][a]
-    T *sDO = reg(6), *sDW = reg(6);           // dO -> dW[c][dk]
-    T *sDOt = reg(7), *sDWt = reg(7);         // dOt -> dW^T[dk][c]
-    T *sS = reg(8), *sU = reg(8);             // S[dv][dk] -> U'[c][dv]
-    T *sSt = reg(9), *sY1 = reg(9);           // St[dk][dv] -> Y1[j][b]
-    T *sDS = reg(10), *sDAqk = reg(10), *sDA = reg(10);  // dS[dv][dk] -> dAqk[i][j] -> dA[i][j]
-    T *sDSt = reg(11), *sGt = reg(11);        // dSt[dk][dv] -> G^T[j][i]
-    float *sA = reinterpret_cast<float *>(smem + 12 * L::U);  // regions 12,13 (fp32)
-    T *sAqkT = reg(12);                       // after A is consumed
-    T *sW = reg(13), *sDAqkT = reg(13);       // W[c][dk] -> dAqk^T[j][i]
-    T *sT = reg(14), *sTmt = reg(15), *sWt = reg(16);
+    // region plan (-> marks reuse once the previous tenant is dead)
+    T *sK = reg(0), *sV = reg(1);
+    T *sQ = reg(2), *sDT = reg(2);                        // Q[c][dk]  -> dT[a][b]
+    T *sDO = reg(3), *sY1 = reg(3);                       // dO[c][dv] -> Y1[j][b]
+    T *sS = reg(4), *sDA = reg(4);                        // S[dv][dk] -> dA[i][j]
+    T *sDS = reg(5), *sDW = reg(5);                       // dS[dv][dk] -> dW[c][dk]
+    float *sA = reinterpret_cast<float *>(smem + 6 * L::U);  // regions 6,7 (fp32 A / Tm)
+    T *sAqk = reg(6), *sDAqk = reg(6), *sG = reg(6);      // Aqk[i][j] -> dAqk[i][j] -> G[i][j]
+    T *sW = reg(7);                                       // W[c][dk]
+    T *sT = reg(8), *sTm = reg(9), *sU = reg(10), *sDU = reg(11);
     float *sBeta = reinterpret_cast<float *>(smem + L::oBeta);
-    float *sDb = reinterpret_cast<float *>(smem + L::oDb);
+    float *sDb = reinterpret_cast<float *>(smem + L::oDb);  // [4 feature tiles][C] dbeta partials
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -311,9 +268,9 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     const int64_t base = ((int64_t)b * Tlen * H + h) * HD;
     const int NC = (Tlen + C - 1) / C;
 
-    using TMS = TileMap<HD, HD>;
-    using TMA = TileMap<C, C>;
-    using TMR = TileMap<HD, C>;
+    using TMS = TileMap<HD, HD, NW>;
+    using TMA = TileMap<C, C, NW>;
+    using TMR = TileMap<HD, C, NW>;
     f32x4 dSacc[TMS::TPW];  // dS^T: m = dk, n = dv
 #pragma unroll
     for (int j = 0; j < TMS::TPW; ++j) {
@@ -353,172 +310,121 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             {
                 typename IO::Regs fq = rq, fk = rk, fv = rv, fdo = rdo;
                 if (nres != 0) {
-                    const int r0 = tid / IO::SEGS;
-#pragma unroll
-                    for (int p = 0; p < IO::PASSES; ++p) {
-                        if (!live(r0 + p * IO::RPP)) {
-#pragma unroll
-                            for (int e = 0; e < IO::KP; ++e) {
-                                fq.v[p][e] = (T)0.f; fk.v[p][e] = (T)0.f; fv.v[p][e] = (T)0.f; fdo.v[p][e] = (T)0.f;
-                            }
-                        }
-                    }
+                    IO::mask_rows(fq, tid, live);
+                    IO::mask_rows(fk, tid, live);
+                    IO::mask_rows(fv, tid, live);
+                    IO::mask_rows(fdo, tid, live);
                 }
                 IO::to_lds(fq, sQ, LDD, tid);
-                IO::to_lds_t(fq, sQt, LDC, tid);
                 IO::to_lds(fk, sK, LDD, tid);
-                IO::to_lds_t(fk, sKt, LDC, tid);
                 IO::to_lds(fv, sV, LDD, tid);
-                IO::to_lds_t(fv, sVt, LDC, tid);
                 IO::to_lds(fdo, sDO, LDD, tid);
-                IO::to_lds_t(fdo, sDOt, LDC, tid);
                 typename IOS::Regs fS = rS;
-                if (pass != 0) {
-#pragma unroll
-                    for (int p = 0; p < IOS::PASSES; ++p)
-#pragma unroll
-                        for (int e = 0; e < IOS::KP; ++e) fS.v[p][e] = (T)0.f;
-                }
+                if (pass != 0) IOS::zero(fS);
                 IOS::to_lds(fS, sS, LDD, tid);
-                IOS::to_lds_t(fS, sSt, LDD, tid);
             }
             if (tid < C) sBeta[tid] = live(tid) ? raw_to_float<T>(rbeta) : 0.f;
             if (pass != nres) zero_acc<TMS::TPW>(dSacc);
-            stage_dS<T>(dSacc, sDS, sDSt, LDD, w, lane);
+            store_acc<T, HD, HD, NW>(dSacc, sDS, LDD, w, lane);  // dS[dv][dk]
             sync_lds();
             MRX_PHASE(11);
             if (pass == 0 && c > 0) prefetch(c - 1);
 
-            // ---- A = beta_i (K K^T) strictly lower -> sA ---------------------------------
+            // ---- A[i][j] = beta_i (k_i . k_j), j < i -> sA -------------------------------
             {
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
-                gemm_nt<T, C, C, HD>(acc, sK, LDD, sK, LDD, w, lane);
-#pragma unroll
-                for (int j = 0; j < TMA::TPW; ++j) {
-                    const int m0 = TMA::mt(w) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
-                    const float bi = sBeta[n];
-                    f32x4 r;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) r[e] = (m0 + e < n) ? bi * acc[j][e] : 0.f;
-                    *reinterpret_cast<f32x4 *>(sA + n * LDA + m0) = r;
-                }
+                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sK, LDD, sK, LDD, w, lane);  // D[m = j][n = i]
+                store_acc_f<float, C, C, NW>(acc, sA, LDA, w, lane,
+                                             [&](int m, int n, float x) { return m < n ? sBeta[n] * x : 0.f; });
             }
             sync_lds();
             MRX_PHASE(12);
             tri_inverse<C>(sA, LDA, w, lane);
             MRX_PHASE(13);
-            // ---- sT[i][j] = Tm[i][j] beta_j ; sTmt[j][i] = Tm[i][j] ----------------------
-            for (int idx = tid; idx < C * C / 4; idx += NTHREADS) {
+            // ---- sT[i][j] = Tm[i][j] beta_j ; sTm[i][j] = Tm[i][j] -------------------------
+            for (int idx = tid; idx < C * C / 4; idx += NTHR) {
                 const int i = idx / (C / 4), j = (idx % (C / 4)) * 4;
                 const f32x4 t = tri_inverse_get4(sA, LDA, i, j);
                 *reinterpret_cast<P4 *>(sT + i * LDC + j) =
                     TT<T>::pack(t[0] * sBeta[j], t[1] * sBeta[j + 1], t[2] * sBeta[j + 2], t[3] * sBeta[j + 3]);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) sTmt[(j + e) * LDC + i] = (T)t[e];
+                *reinterpret_cast<P4 *>(sTm + i * LDC + j) = TT<T>::pack(t[0], t[1], t[2], t[3]);
             }
-            sync_lds();
+            sync_lds();  // sA dead
             MRX_PHASE(14);
-            // ---- Aqk^T[j][i] ; W^T[dk][c] = K^T T^T -> sW[c][dk], sWt[dk][c] ---------------
+            // ---- Aqk[i][j] (j <= i) ; W^T[dk][c] = sum_j K[j][dk] T[c][j] -> sW[c][dk] -------
             {
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
-                gemm_nt<T, C, C, HD>(acc, sQ, LDD, sK, LDD, w, lane);  // D[m = i][n = j]
-#pragma unroll
-                for (int j = 0; j < TMA::TPW; ++j) {
-                    const int m0 = TMA::mt(w) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (m0 + e < n) acc[j][e] = 0.f;
-                }
-                store_acc_t<T, C, C>(acc, sAqkT, LDC, w, lane);
+                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sK, LDD, sQ, LDD, w, lane);  // D[m = j][n = i]
+                store_acc_f<T, C, C, NW>(acc, sAqk, LDC, w, lane, [](int m, int n, float x) { return m <= n ? x : 0.f; });
             }
             {
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
-                gemm_nt<T, HD, C, C>(acc, sKt, LDC, sT, LDC, w, lane);  // D[m = dk][n = c]
-                store_acc_t<T, HD, C>(acc, sW, LDD, w, lane);
-                store_acc_n<T, HD, C>(acc, sWt, LDC, w, lane);
+                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sK, LDD, sT, LDC, w, lane);  // D[m = dk][n = c]
+                store_acc<T, HD, C, NW>(acc, sW, LDD, w, lane);
             }
             sync_lds();
             MRX_PHASE(15);
-            // ---- U'^T[dv][c] = V^T T^T - S W^T -> sU[c][dv] (over sS) ------------------------
+            // ---- U'^T[dv][c] = sum_j V[j][dv] T[c][j] - sum_dk S[dv][dk] W[c][dk] -> sU[c][dv] ----
             {
                 f32x4 acc[TMR::TPW], acc2[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
                 zero_acc<TMR::TPW>(acc2);
-                gemm_nt<T, HD, C, C>(acc, sVt, LDC, sT, LDC, w, lane);
-                gemm_nt<T, HD, C, HD>(acc2, sS, LDD, sW, LDD, w, lane);
+                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sV, LDD, sT, LDC, w, lane);
+                gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc2, sS, LDD, sW, LDD, w, lane);
 #pragma unroll
                 for (int j = 0; j < TMR::TPW; ++j) acc[j] -= acc2[j];
-                sync_lds();  // every wave is done reading sS, sVt, sQ
-                MRX_PHASE(16);
-                store_acc_t<T, HD, C>(acc, sU, LDD, w, lane);
+                store_acc<T, HD, C, NW>(acc, sU, LDD, w, lane);
             }
-            // ---- dU'^T[dv][j] = dO^T Aqk + dS K^T -> sDU[j][dv], sDUt[dv][j] -----------------
+            // ---- dU'^T[dv][j] = sum_i dO[i][dv] Aqk[i][j] + sum_dk dS[dv][dk] K[j][dk] -> sDU[j][dv]
             {
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
-                gemm_nt<T, HD, C, C>(acc, sDOt, LDC, sAqkT, LDC, w, lane);
-                gemm_nt<T, HD, C, HD>(acc, sDS, LDD, sK, LDD, w, lane);
-                store_acc_t<T, HD, C>(acc, sDU, LDD, w, lane);
-                store_acc_n<T, HD, C>(acc, sDUt, LDC, w, lane);
+                gemm<T, HD, C, C, KROW, KROW, NW>(acc, sDO, LDD, sAqk, LDC, w, lane);
+                gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc, sDS, LDD, sK, LDD, w, lane);
+                store_acc<T, HD, C, NW>(acc, sDU, LDD, w, lane);
             }
-            sync_lds();  // sU, sDU, sDUt visible; sDS, sW dead
-            MRX_PHASE(17);
-            // ---- dAqk[i][j] = tril(dO U'^T) (+ transpose) ----------------------------------
+            sync_lds();  // sU, sDU visible; sAqk dead
+            MRX_PHASE(16);
+            // ---- dAqk[i][j] = do_i . u'_j, j <= i -> sDAqk (over sAqk) ------------------------
             {
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
-                gemm_nt<T, C, C, HD>(acc, sU, LDD, sDO, LDD, w, lane);  // D[m = j][n = i]
-#pragma unroll
-                for (int j = 0; j < TMA::TPW; ++j) {
-                    const int m0 = TMA::mt(w) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (m0 + e > n) acc[j][e] = 0.f;
-                }
-                store_acc_t<T, C, C>(acc, sDAqk, LDC, w, lane);
-                store_acc_n<T, C, C>(acc, sDAqkT, LDC, w, lane);
+                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sU, LDD, sDO, LDD, w, lane);  // D[m = j][n = i]
+                store_acc_f<T, C, C, NW>(acc, sDAqk, LDC, w, lane, [](int m, int n, float x) { return m <= n ? x : 0.f; });
             }
             sync_lds();
-            MRX_PHASE(18);
+            MRX_PHASE(17);
             auto one = [](int, int) { return f32x4{1.f, 1.f, 1.f, 1.f}; };
-            // ---- dQ^T[dk][i] = S^T dO^T + K^T dAqk^T -> global -------------------------------
+            // ---- dQ^T[dk][i] = sum_dv S[dv][dk] dO[i][dv] + sum_j K[j][dk] dAqk[i][j] -> global ----
             {
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
-                gemm_nt<T, HD, C, HD>(acc, sSt, LDD, sDO, LDD, w, lane);
-                gemm_nt<T, HD, C, C>(acc, sKt, LDC, sDAqk, LDC, w, lane);
-                store_rows_global<T, C>(acc, dq + base, rs, t0, Tlen, w, lane, one, live);
+                gemm<T, HD, C, HD, KROW, ROWK, NW>(acc, sS, LDD, sDO, LDD, w, lane);
+                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sK, LDD, sDAqk, LDC, w, lane);
+                store_rows_global<T, C, NW>(acc, dq + base, rs, t0, Tlen, w, lane, one, live);
             }
-            // ---- dK^T[dk][j] = Q^T dAqk + dS^T U'^T  (kept in registers) ----------------------
+            // ---- dK^T[dk][j] = sum_i Q[i][dk] dAqk[i][j] + sum_dv dS[dv][dk] U'[j][dv] (registers) --
             f32x4 dKacc[TMR::TPW];
             zero_acc<TMR::TPW>(dKacc);
-            gemm_nt<T, HD, C, C>(dKacc, sQt, LDC, sDAqkT, LDC, w, lane);
-            gemm_nt<T, HD, C, HD>(dKacc, sDSt, LDD, sU, LDD, w, lane);
-            // ---- dS^T[dk][dv] += Q^T dO - W^T dU' -----------------------------------------------
+            gemm<T, HD, C, C, KROW, KROW, NW>(dKacc, sQ, LDD, sDAqk, LDC, w, lane);
+            gemm<T, HD, C, HD, KROW, ROWK, NW>(dKacc, sDS, LDD, sU, LDD, w, lane);
+            // ---- dS^T[dk][dv] += sum_c Q[c][dk] dO[c][dv] - sum_c W[c][dk] dU'[c][dv] ---------------
             {
                 f32x4 acc[TMS::TPW];
                 zero_acc<TMS::TPW>(acc);
-                gemm_nt<T, HD, HD, C>(dSacc, sQt, LDC, sDOt, LDC, w, lane);
-                gemm_nt<T, HD, HD, C>(acc, sWt, LDC, sDUt, LDC, w, lane);
+                gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, sQ, LDD, sDO, LDD, w, lane);
+                gemm<T, HD, HD, C, KROW, KROW, NW>(acc, sW, LDD, sDU, LDD, w, lane);
 #pragma unroll
                 for (int j = 0; j < TMS::TPW; ++j) dSacc[j] -= acc[j];
             }
-            sync_lds();  // sDO, sDOt, sQt, sDAqk*, sDSt dead
-            MRX_PHASE(19);
-            // ---- dW^T[dk][c] = -S^T dU'^T -> sDW[c][dk], sDWt[dk][c] ---------------------------
-            {
-                f32x4 acc[TMR::TPW];
-                zero_acc<TMR::TPW>(acc);
-                gemm_nt<T, HD, C, HD>(acc, sSt, LDD, sDU, LDD, w, lane);
-#pragma unroll
-                for (int j = 0; j < TMR::TPW; ++j) acc[j] = -acc[j];
-                store_acc_t<T, HD, C>(acc, sDW, LDD, w, lane);
-                store_acc_n<T, HD, C>(acc, sDWt, LDC, w, lane);
-            }
-            float dbp[TMR::TPW];  // per-lane partial of dbeta for row 16 j + li
+            // ---- dW^T[dk][c] = -sum_dv S[dv][dk] dU'[c][dv] (stored after the barrier: over sDS) ----
+            f32x4 dWacc[TMR::TPW];
+            zero_acc<TMR::TPW>(dWacc);
+            gemm<T, HD, C, HD, KROW, ROWK, NW>(dWacc, sS, LDD, sDU, LDD, w, lane);
+            float dbp[TMR::TPW];  // per-lane partial of dbeta for row nt*16 + li
 #pragma unroll
             for (int j = 0; j < TMR::TPW; ++j) dbp[j] = 0.f;
             auto rowdot = [&](const f32x4 *acc, const T *X) {
@@ -531,104 +437,86 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 }
             };
             auto beta_of = [&](int r, int) { const float bb = sBeta[r]; return f32x4{bb, bb, bb, bb}; };
-            // ---- Zu^T[dv][j] = dU'^T Tm -> dV = beta_j Zu ; dbeta += V_j . Zu_j -------------------
+            // ---- Zu^T[dv][j] = sum_i dU'[i][dv] Tm[i][j] -> dV = beta_j Zu ; dbeta += V_j . Zu_j ------
             {
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
-                gemm_nt<T, HD, C, C>(acc, sDUt, LDC, sTmt, LDC, w, lane);
+                gemm<T, HD, C, C, KROW, KROW, NW>(acc, sDU, LDD, sTm, LDC, w, lane);
                 rowdot(acc, sV);
-                store_rows_global<T, C>(acc, dv + base, rs, t0, Tlen, w, lane, beta_of, live);
+                store_rows_global<T, C, NW>(acc, dv + base, rs, t0, Tlen, w, lane, beta_of, live);
             }
-            sync_lds();  // sDW, sDWt visible
-            MRX_PHASE(20);
-            // ---- Zw^T[dk][j] = dW^T Tm -> dK += beta_j Zw ; dbeta += K_j . Zw_j -------------------
+            sync_lds();  // sQ, sDO, sDS, sDAqk dead
+            MRX_PHASE(18);
+            store_acc_f<T, HD, C, NW>(dWacc, sDW, LDD, w, lane, [](int, int, float x) { return -x; });
+            sync_lds();
+            MRX_PHASE(19);
+            // ---- Zw^T[dk][j] = sum_i dW[i][dk] Tm[i][j] -> dK += beta_j Zw ; dbeta += K_j . Zw_j ------
             {
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
-                gemm_nt<T, HD, C, C>(acc, sDWt, LDC, sTmt, LDC, w, lane);
+                gemm<T, HD, C, C, KROW, KROW, NW>(acc, sDW, LDD, sTm, LDC, w, lane);
                 rowdot(acc, sK);
 #pragma unroll
-                for (int j = 0; j < TMR::TPW; ++j) {
-                    const float bb = sBeta[TMR::nt(w, j) * 16 + li];
-                    dKacc[j] += acc[j] * bb;
-                }
+                for (int j = 0; j < TMR::TPW; ++j) dKacc[j] += acc[j] * sBeta[TMR::nt(w, j) * 16 + li];
             }
-            // ---- dT^T: D[m = a][n = b] = dW K^T + dU' V^T, a >= b -> sDTt[b][a] --------------------
+            // ---- dT[a][b] = dw_a . k_b + du'_a . v_b, a >= b : D[m = b][n = a] -> sDT[a][b] ------------
             {
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
-                gemm_nt<T, C, C, HD>(acc, sDW, LDD, sK, LDD, w, lane);
-                gemm_nt<T, C, C, HD>(acc, sDU, LDD, sV, LDD, w, lane);
-#pragma unroll
-                for (int j = 0; j < TMA::TPW; ++j) {
-                    const int m0 = TMA::mt(w) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (m0 + e < n) acc[j][e] = 0.f;
-                }
-                store_acc_t<T, C, C>(acc, sDTt, LDC, w, lane);
+                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sK, LDD, sDW, LDD, w, lane);
+                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sV, LDD, sDU, LDD, w, lane);
+                store_acc_f<T, C, C, NW>(acc, sDT, LDC, w, lane, [](int m, int n, float x) { return m <= n ? x : 0.f; });
+            }
+            sync_lds();
+            MRX_PHASE(20);
+            // ---- Y1[j][b] = sum_a Tm[a][j] dT[a][b] : D[m = b][n = j] -> sY1[j][b] ----------------------
+            {
+                f32x4 acc[TMA::TPW];
+                zero_acc<TMA::TPW>(acc);
+                gemm<T, C, C, C, KROW, KROW, NW>(acc, sDT, LDC, sTm, LDC, w, lane);
+                store_acc<T, C, C, NW>(acc, sY1, LDC, w, lane);
             }
             sync_lds();
             MRX_PHASE(21);
-            // ---- Y1: D[m = b][n = j] = dT^T Tm -> sY1[j][b] -----------------------------------------
+            // ---- dA[i][j] = -sum_b Y1[i][b] T[j][b], j < i : D[m = j][n = i] -> sDA ; sG = beta_i dA ------
             {
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
-                gemm_nt<T, C, C, C>(acc, sDTt, LDC, sTmt, LDC, w, lane);
-                store_acc_t<T, C, C>(acc, sY1, LDC, w, lane);
+                gemm<T, C, C, C, ROWK, ROWK, NW>(acc, sT, LDC, sY1, LDC, w, lane);
+                store_acc_f<T, C, C, NW>(acc, sDA, LDC, w, lane, [](int m, int n, float x) { return m < n ? -x : 0.f; });
+                store_acc_f<T, C, C, NW>(acc, sG, LDC, w, lane,
+                                         [&](int m, int n, float x) { return m < n ? -x * sBeta[n] : 0.f; });
             }
             sync_lds();
             MRX_PHASE(22);
-            // ---- dA: D[m = j][n = i] = -T Y1^T, j < i -> sDA[i][j] ; sGt[j][i] = beta_i dA[i][j] -----
-            {
-                f32x4 acc[TMA::TPW];
-                zero_acc<TMA::TPW>(acc);
-                gemm_nt<T, C, C, C>(acc, sT, LDC, sY1, LDC, w, lane);
-#pragma unroll
-                for (int j = 0; j < TMA::TPW; ++j) {
-                    const int m0 = TMA::mt(w) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) acc[j][e] = (m0 + e < n) ? -acc[j][e] : 0.f;
-                }
-                store_acc_t<T, C, C>(acc, sDA, LDC, w, lane);
-#pragma unroll
-                for (int j = 0; j < TMA::TPW; ++j) acc[j] *= sBeta[TMA::nt(w, j) * 16 + li];
-                store_acc_n<T, C, C>(acc, sGt, LDC, w, lane);
-            }
-            sync_lds();
-            MRX_PHASE(23);
-            // ---- R^T[dk][i] = K^T dA^T -> dK += beta_i R ; dbeta += K_i . R_i ; dK += K^T G ---------
+            // ---- R^T[dk][i] = sum_j K[j][dk] dA[i][j] -> dK += beta_i R ; dbeta += K_i . R_i ;
+            //      dK^T[dk][j] += sum_i K[i][dk] G[i][j] -------------------------------------------------
             {
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
-                gemm_nt<T, HD, C, C>(acc, sKt, LDC, sDA, LDC, w, lane);
+                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sK, LDD, sDA, LDC, w, lane);
                 rowdot(acc, sK);
 #pragma unroll
-                for (int j = 0; j < TMR::TPW; ++j) {
-                    const float bb = sBeta[TMR::nt(w, j) * 16 + li];
-                    dKacc[j] += acc[j] * bb;
-                }
-                gemm_nt<T, HD, C, C>(dKacc, sKt, LDC, sGt, LDC, w, lane);
-                store_rows_global<T, C>(dKacc, dk + base, rs, t0, Tlen, w, lane, one, live);
+                for (int j = 0; j < TMR::TPW; ++j) dKacc[j] += acc[j] * sBeta[TMR::nt(w, j) * 16 + li];
+                gemm<T, HD, C, C, KROW, KROW, NW>(dKacc, sK, LDD, sG, LDC, w, lane);
+                store_rows_global<T, C, NW>(dKacc, dk + base, rs, t0, Tlen, w, lane, one, live);
             }
-            // ---- dbeta: reduce the partials over lane groups, then over waves through LDS ---------
+            // ---- dbeta: reduce the partials over lane groups, then over feature tiles through LDS ----
 #pragma unroll
             for (int j = 0; j < TMR::TPW; ++j) {
                 float x = dbp[j];
                 x += __shfl_xor(x, 16);
                 x += __shfl_xor(x, 32);
-                if (lg == 0) sDb[w * C + TMR::nt(w, j) * 16 + li] = x;
+                if (lg == 0) sDb[TMR::mt(w) * C + TMR::nt(w, j) * 16 + li] = x;
             }
             sync_lds();
-            MRX_PHASE(24);
+            MRX_PHASE(23);
             if (tid < C && t0 + tid < Tlen && live(tid)) {
-                float x = 0.f;
-#pragma unroll
-                for (int ww = 0; ww < NWAVES; ++ww) x += sDb[ww * C + tid];
+                const float x = sDb[tid] + sDb[C + tid] + sDb[2 * C + tid] + sDb[3 * C + tid];
                 dbeta[((int64_t)b * Tlen + t0 + tid) * H + h] = (T)x;
             }
             sync_lds();
-            MRX_PHASE(25);
+            MRX_PHASE(24);
         }
     }
     if (dS0) {
@@ -660,7 +548,7 @@ int launch_la(hipStream_t st, const void *q, const void *k, const void *v, const
     constexpr int smem = LaBwdSmem<T, C>::total;
     static bool attr_set = false;
     if (set_smem(kern, smem, attr_set) != MRX_OK) return MRX_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(NTHREADS), smem, st, (const T *)q,
+    hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(256), smem, st, (const T *)q,
                        (const T *)k, (const T *)v, done, done_f32, (const T *)S_chk,
                        (const T *)dout, (const float *)dS_last, (T *)dq, (T *)dk, (T *)dv,
                        (float *)dS0, (int)Tlen, (int)H);
@@ -717,11 +605,12 @@ extern "C" int mrx_delta_rule_bwd(void *stream, const void *q, const void *k, co
     if (!beta || !dbeta) return MRX_ERR_INVALID_ARG;
     if (dtype != MRX_BF16) return MRX_ERR_UNSUPPORTED;  // fp32 delta-rule backward: not built yet
     hipStream_t st = (hipStream_t)stream;
-    auto kern = delta_bwd_kernel<__bf16, 64>;
-    constexpr int smem = DeltaBwdSmem<__bf16, 64>::total;
+    constexpr int NW = MRX_DELTA_BWD_WAVES;
+    auto kern = delta_bwd_kernel<__bf16, 64, NW>;
+    constexpr int smem = DeltaBwdSmem<__bf16, 64, NW>::total;
     static bool attr_set = false;
     if (set_smem(kern, smem, attr_set) != MRX_OK) return MRX_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(NTHREADS), smem, st, (const __bf16 *)q,
+    hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(64 * NW), smem, st, (const __bf16 *)q,
                        (const __bf16 *)k, (const __bf16 *)v, (const __bf16 *)beta, done, done_dtype,
                        (const __bf16 *)S_chk, (const __bf16 *)dout, (const float *)dS_last,
                        (__bf16 *)dq, (__bf16 *)dk_out, (__bf16 *)dv_out, (__bf16 *)dbeta, (float *)dS0,

@@ -1,16 +1,18 @@
 // Building blocks of the chunked linear-attention / delta-rule kernels (gfx950).
 //
-// One workgroup = 4 waves = one (batch, head) sequence, head dim 64, walking the
-// time axis in chunks of C rows.  All matrix products are "NT" products
-//     D[m][n] = sum_k X[m][k] * Y[n][k]
-// of two LDS tiles that are both contiguous along k, executed with 16x16 MFMA
-// tiles (bf16: v_mfma_f32_16x16x32_bf16, fp32: v_mfma_f32_16x16x4_f32) and fp32
-// accumulation.  A wave lane (i = lane % 16, g = lane / 16) holds, for a 16x16
-// accumulator tile, the four elements D[4g + v][i], v = 0..3; so four
-// consecutive m-indices sit in one lane and a tile can be stored k-contiguously
-// as the [n][m] (transposed) matrix with one 8/16-byte LDS write per lane.
-// Every product below is oriented so that its result lands k-contiguous for
-// the next product that consumes it.
+// One workgroup = NW waves = one (batch, head) sequence, head dim 64, walking the
+// time axis in chunks of C rows.  Every matrix product is executed with 16x16 MFMA
+// tiles (bf16: v_mfma_f32_16x16x32_bf16, fp32: v_mfma_f32_16x16x4_f32) on two LDS
+// tiles with fp32 accumulation:
+//     D[m][n] = sum_k X(m, k) * Y(n, k)
+// Each operand tile is stored once, in its natural orientation, and read either
+//   ROWK: tile[row][k], k contiguous  -> one 16-byte read per lane, or
+//   KROW: tile[k][row], row contiguous -> gfx950 transpose reads (ds_read_b64_tr_b16)
+//         for bf16, four 4-byte reads for fp32,
+// so no transposed copy of any tile is ever written.
+// A wave lane (i = lane % 16, g = lane / 16) holds, for a 16x16 accumulator tile, the
+// four elements D[4g + v][i], v = 0..3: four consecutive m-indices per lane, hence a
+// result is stored with one 8/16-byte write per lane as the matrix dst[n][m].
 #pragma once
 #include "common.h"
 
@@ -18,6 +20,7 @@ namespace mrx {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains the
@@ -29,9 +32,9 @@ __device__ __forceinline__ void sync_lds()
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-constexpr int NWAVES = 4;
-constexpr int NTHREADS = 64 * NWAVES;
 constexpr int HD = 64;  // head dim (d_k = d_v)
+
+enum OpMode { ROWK = 0, KROW = 1 };
 
 template <typename T> struct TT;
 template <> struct TT<__bf16> {
@@ -48,6 +51,27 @@ template <> struct TT<__bf16> {
         pack4 r;
         r[0] = (__bf16)a; r[1] = (__bf16)b; r[2] = (__bf16)c; r[3] = (__bf16)d;
         return r;
+    }
+    // 16 rows r0.., k block k0..k0+31; lane (i, g) gets k = k0 + 8g + 0..7 of row r0 + i
+    template <int MODE>
+    static __device__ __forceinline__ frag load(const __bf16 *tile, int ld, int r0, int k0, int lane)
+    {
+        const int i = lane & 15, g = lane >> 4;
+        if (MODE == ROWK) return *reinterpret_cast<const frag *>(tile + (r0 + i) * ld + k0 + 8 * g);
+        // Transpose read: within a 16-lane group, source lane s addresses the 4 elements
+        // tile[kk + (s >> 2)][r0 + 4 (s & 3) ..+3]; destination lane i receives
+        // tile[kk + e][r0 + i], e = 0..3.
+        typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+        const __bf16 *p = tile + (k0 + 8 * g + (i >> 2)) * ld + r0 + 4 * (i & 3);
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)p);
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p + 4 * ld));
+        union {
+            s16x4 h[2];
+            frag f;
+        } u;
+        u.h[0] = lo;
+        u.h[1] = hi;
+        return u.f;
     }
 };
 template <> struct TT<float> {
@@ -67,38 +91,46 @@ template <> struct TT<float> {
         pack4 r = {a, b, c, d};
         return r;
     }
+    template <int MODE>
+    static __device__ __forceinline__ frag load(const float *tile, int ld, int r0, int k0, int lane)
+    {
+        const int i = lane & 15, g = lane >> 4;
+        if (MODE == ROWK) return *reinterpret_cast<const frag *>(tile + (r0 + i) * ld + k0 + 4 * g);
+        frag f;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) f[s] = tile[(k0 + 4 * g + s) * ld + r0 + i];
+        return f;
+    }
 };
 
 // 16-byte LDS row padding (in elements) keeps 16-lane fragment reads conflict free.
 template <typename T> constexpr int pad_of() { return 16 / (int)sizeof(T); }
 
 // Which 16x16 tiles of an M x N result a wave owns: slot j -> (mt, nt).
-template <int M, int N> struct TileMap {
+template <int M, int N, int NW> struct TileMap {
     static constexpr int MT = M / 16, NT = N / 16;
-    static constexpr int TPW = MT * NT / NWAVES;
-    static_assert(MT == 2 || MT == 4, "M must be 32 or 64");
-    static_assert(MT * NT % NWAVES == 0, "tiles must divide over the waves");
-    static __device__ __forceinline__ int mt(int w) { return MT == 4 ? w : (w & 1); }
-    static __device__ __forceinline__ int nt(int w, int j) { return MT == 4 ? j : (w >> 1) * TPW + j; }
+    static constexpr int TPW = MT * NT / NW;
+    static_assert(MT * NT % NW == 0 && TPW >= 1, "tiles must divide over the waves");
+    static_assert(NW % MT == 0 && NT % (NW / MT) == 0, "wave grid must tile the result");
+    static __device__ __forceinline__ int mt(int w) { return w % MT; }
+    static __device__ __forceinline__ int nt(int w, int j) { return (w / MT) * TPW + j; }
 };
 
-// acc[j] += X[mt-th 16 rows][:] . Y[nt_j-th 16 rows][:]^T over K columns.
-template <typename T, int M, int N, int K>
-__device__ __forceinline__ void gemm_nt(f32x4 *acc, const T *X, int ldx, const T *Y, int ldy,
-                                        int w, int lane)
+// acc[j] += sum_k X(mt rows, k) * Y(nt_j rows, k), k = 0..K-1.
+template <typename T, int M, int N, int K, int XM, int YM, int NW>
+__device__ __forceinline__ void gemm(f32x4 *acc, const T *X, int ldx, const T *Y, int ldy, int w, int lane)
 {
-    using TM = TileMap<M, N>;
+    using TM = TileMap<M, N, NW>;
     using F = typename TT<T>::frag;
-    constexpr int KP = TT<T>::KP, KB = TT<T>::KB;
+    constexpr int KB = TT<T>::KB;
     static_assert(K % KB == 0, "K must be a multiple of the fragment k extent");
-    const int i = lane & 15, g = lane >> 4;
-    const T *xp = X + (TM::mt(w) * 16 + i) * ldx + g * KP;
+    const int m0 = TM::mt(w) * 16;
 #pragma unroll
     for (int kb = 0; kb < K / KB; ++kb) {
-        const F a = *reinterpret_cast<const F *>(xp + kb * KB);
+        const F a = TT<T>::template load<XM>(X, ldx, m0, kb * KB, lane);
 #pragma unroll
         for (int j = 0; j < TM::TPW; ++j) {
-            const F b = *reinterpret_cast<const F *>(Y + (TM::nt(w, j) * 16 + i) * ldy + kb * KB + g * KP);
+            const F b = TT<T>::template load<YM>(Y, ldy, TM::nt(w, j) * 16, kb * KB, lane);
             acc[j] = TT<T>::mma(a, b, acc[j]);
         }
     }
@@ -110,33 +142,25 @@ template <int N> __device__ __forceinline__ void zero_acc(f32x4 *acc)
     for (int j = 0; j < N; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 }
 
-// Store an accumulator tile set as the k-contiguous matrix dst[n][m] (type T).
-template <typename T, int M, int N>
-__device__ __forceinline__ void store_acc_t(const f32x4 *acc, T *dst, int ld, int w, int lane)
+// Store an accumulator tile set as dst[n][m] (type T), f(m, n, x) applied per element.
+template <typename T, int M, int N, int NW, typename Fn>
+__device__ __forceinline__ void store_acc_f(const f32x4 *acc, T *dst, int ld, int w, int lane, Fn f)
 {
-    using TM = TileMap<M, N>;
+    using TM = TileMap<M, N, NW>;
     using P = typename TT<T>::pack4;
     const int i = lane & 15, g = lane >> 4;
 #pragma unroll
     for (int j = 0; j < TM::TPW; ++j) {
         const int m = TM::mt(w) * 16 + 4 * g, n = TM::nt(w, j) * 16 + i;
-        *reinterpret_cast<P *>(dst + n * ld + m) = TT<T>::pack(acc[j][0], acc[j][1], acc[j][2], acc[j][3]);
+        *reinterpret_cast<P *>(dst + n * ld + m) =
+            TT<T>::pack(f(m, n, acc[j][0]), f(m + 1, n, acc[j][1]), f(m + 2, n, acc[j][2]), f(m + 3, n, acc[j][3]));
     }
 }
 
-// Store an accumulator tile set as dst[m][n] (element-wise writes; use when the
-// consumer needs the other orientation too).
-template <typename T, int M, int N>
-__device__ __forceinline__ void store_acc_n(const f32x4 *acc, T *dst, int ld, int w, int lane)
+template <typename T, int M, int N, int NW>
+__device__ __forceinline__ void store_acc(const f32x4 *acc, T *dst, int ld, int w, int lane)
 {
-    using TM = TileMap<M, N>;
-    const int i = lane & 15, g = lane >> 4;
-#pragma unroll
-    for (int j = 0; j < TM::TPW; ++j) {
-        const int m = TM::mt(w) * 16 + 4 * g, n = TM::nt(w, j) * 16 + i;
-#pragma unroll
-        for (int v = 0; v < 4; ++v) dst[(m + v) * ld + n] = (T)acc[j][v];
-    }
+    store_acc_f<T, M, N, NW>(acc, dst, ld, w, lane, [](int, int, float x) { return x; });
 }
 
 // Raw bits of one T-typed scalar (converted to float only when consumed).
@@ -154,17 +178,16 @@ template <> __device__ __forceinline__ float raw_to_float<__bf16>(uint32_t raw) 
 template <> __device__ __forceinline__ float raw_to_float<float>(uint32_t raw) { return __uint_as_float(raw); }
 
 __device__ __forceinline__ float elu1(float x) { return x > 0.f ? x + 1.f : __expf(x); }
-__device__ __forceinline__ float delu1(float x) { return x > 0.f ? 1.f : __expf(x); }
 
-// ---- global <-> register <-> LDS movement of one [C][64] input tile ----------
-// A tile is C rows of 64 T = C * SEGS 16-byte segments; thread tid owns segment
+// ---- global <-> register <-> LDS movement of one [R][64] tile --------------------
+// A tile is R rows of 64 T = R * SEGS 16-byte segments; thread tid owns segment
 // (tid % SEGS) of rows (tid / SEGS) + p * RPP, p = 0..PASSES-1.
-template <typename T, int C> struct TileIO {
+template <typename T, int R, int NTHR> struct TileIO {
     static constexpr int KP = TT<T>::KP;
     static constexpr int SEGS = HD / KP;
-    static constexpr int RPP = NTHREADS / SEGS;
-    static constexpr int PASSES = C / RPP;
-    static_assert(PASSES >= 1 && C % RPP == 0, "chunk rows must be a multiple of rows per pass");
+    static constexpr int RPP = NTHR / SEGS;
+    static constexpr int PASSES = R / RPP;
+    static_assert(PASSES >= 1 && R % RPP == 0, "tile rows must be a multiple of rows per pass");
     using F = typename TT<T>::frag;
     struct Regs {
         F v[PASSES];
@@ -195,6 +218,26 @@ template <typename T, int C> struct TileIO {
         }
     }
 
+    // zero the rows for which keep(row) is false (select, not multiply)
+    template <typename KeepF> static __device__ __forceinline__ void mask_rows(Regs &r, int tid, KeepF keep)
+    {
+        const int r0 = tid / SEGS;
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p)
+            if (!keep(r0 + p * RPP)) {
+#pragma unroll
+                for (int e = 0; e < KP; ++e) r.v[p][e] = (T)0.f;
+            }
+    }
+
+    static __device__ __forceinline__ void zero(Regs &r)
+    {
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p)
+#pragma unroll
+            for (int e = 0; e < KP; ++e) r.v[p][e] = (T)0.f;
+    }
+
     // dst[row][col], row-major with leading dim ld
     static __device__ __forceinline__ void to_lds(const Regs &r, T *dst, int ld, int tid)
     {
@@ -202,16 +245,6 @@ template <typename T, int C> struct TileIO {
 #pragma unroll
         for (int p = 0; p < PASSES; ++p)
             *reinterpret_cast<F *>(dst + (r0 + p * RPP) * ld + seg * KP) = r.v[p];
-    }
-
-    // dst[col][row]
-    static __device__ __forceinline__ void to_lds_t(const Regs &r, T *dst, int ld, int tid)
-    {
-        const int seg = tid % SEGS, r0 = tid / SEGS;
-#pragma unroll
-        for (int p = 0; p < PASSES; ++p)
-#pragma unroll
-            for (int e = 0; e < KP; ++e) dst[(seg * KP + e) * ld + r0 + p * RPP] = r.v[p][e];
     }
 };
 
@@ -226,8 +259,8 @@ __device__ __forceinline__ int episode_of(unsigned long long dmask, int r)
 // ---- inverse of a unit lower-triangular matrix, in place, fp32 -------------------
 // sA holds A (strictly lower part used), C x C with leading dim ld; on return the
 // inverse X of (I + A) is stored as: diagonal 16x16 blocks in place; block (b, c),
-// b > c, in the unused upper position (c, b) (same orientation).  Needs all 4 waves
-// (contains workgroup barriers).
+// b > c, in the unused upper position (c, b) (same orientation).  Every wave of the
+// workgroup must call it (contains workgroup barriers); waves >= C/16 only wait.
 template <int C> __device__ __forceinline__ void tri_inverse(float *sA, int ld, int w, int lane)
 {
     constexpr int NB = C / 16;

@@ -1,61 +1,69 @@
 // Forward of chunked causal linear attention and of the DeltaNet delta rule (WY/UT form).
 //
-// Per chunk (rows i, j of the chunk; S = state entering the chunk, d_v x d_k, fp32):
+// Per chunk (rows i >= j of the chunk; S = state entering the chunk, d_v x d_k, fp32):
 //   linear attention:  U' = V
-//   delta rule:        A  = tril(diag(beta) (K K^T . M), -1),  Tm = (I + A)^-1,  T = Tm diag(beta)
-//                      W  = T K,  U' = T V - diag(m) W S^T
-//   both:              O  = diag(m) Q S^T + (tril(Q K^T) . M) U'
-//                      S <- l S + (diag(e) U')^T K
-// M, m, e, l are the episode masks of the chunk; they are realised by processing a
-// chunk that contains resets once per episode with the other episodes' rows zeroed
-// by select, so inside a pass only the causal mask remains.  The state is
-// kept transposed (S^T, d_k x d_v) in MFMA accumulators for the whole sequence and
-// re-staged to LDS as a T-typed d_v x d_k tile once per chunk.
+//   delta rule:        A  = tril(diag(beta) K K^T, -1),  Tm = (I + A)^-1,  T = Tm diag(beta)
+//                      W  = T K,  U' = T V - W S^T
+//   both:              O  = Q S^T + tril(Q K^T) U' ,   S <- S + U'^T K
+// Episode resets: a chunk that contains resets is processed once per episode ("pass")
+// with the rows of all other episodes replaced by zeros *by select*; the episode that
+// enters the chunk sees S, later episodes start from 0, and only the episode that
+// leaves the chunk updates S.  Inside a pass only the causal mask remains, and a
+// non-finite value can never meet a masked-out zero inside a matrix product.
+// The state is kept transposed (S^T, d_k x d_v) in MFMA accumulators for the whole
+// sequence and re-staged to LDS as a T-typed d_v x d_k tile once per chunk.
 #include "chunk_common.h"
 
 namespace {
 
 using namespace mrx;
 
+constexpr int NW = 4;             // waves per workgroup
+constexpr int NTHR = 64 * NW;
+
 template <typename T, int C, bool DELTA> struct FwdSmem {
     static constexpr int PAD = pad_of<T>();
     static constexpr int LDD = HD + PAD;  // tiles with 64 columns
     static constexpr int LDC = C + PAD;   // tiles with C columns
     static constexpr int LDA = C + 4;     // fp32 C x C
-    static constexpr int szQ = C * LDD * sizeof(T);    // sQ, later sW   [C][64]
-    static constexpr int szK = szQ;                    // sK            [C][64]
-    static constexpr int szKt = HD * LDC * sizeof(T);  // sKt           [64][C]
-    static constexpr int szVt = szKt;                  // sVt, later sUt [64][C]
-    static constexpr int szS = HD * LDD * sizeof(T);   // sS            [64][64]
-    static constexpr int szT = DELTA ? C * LDC * sizeof(T) : 0;  // sT   [C][C]
-    static constexpr int szAq = C * LDC * sizeof(T);   // sAqk          [C][C]
-    static constexpr int szA = DELTA ? C * LDA * 4 : 0;  // sA fp32 [C][C], overlaid by sAqk afterwards
-    static constexpr int szAA = szA > szAq ? szA : szAq;
-    static constexpr int oQ = 0, oK = oQ + szQ, oKt = oK + szK, oVt = oKt + szKt, oS = oVt + szVt,
-                         oT = oS + szS, oA = oT + szT, oBeta = oA + szAA, total = oBeta + C * 4;
+    static constexpr int szRD = C * LDD * sizeof(T);   // [C][64]
+    static constexpr int szDD = HD * LDD * sizeof(T);  // [64][64]
+    static constexpr int szCC = C * LDC * sizeof(T);   // [C][C]
+    static constexpr int szA = DELTA ? C * LDA * 4 : 0;
+    // region A: fp32 A / Tm during the inverse; afterwards Aqk (offset 0) and U' (offset szCC)
+    static constexpr int szAU = DELTA ? szCC + szRD : szCC;
+    static constexpr int szRA = szA > szAU ? szA : szAU;
+    static constexpr int oQ = 0;                 // Q [C][dk], later W [C][dk]
+    static constexpr int oK = oQ + szRD;         // K [C][dk]
+    static constexpr int oV = oK + szRD;         // V [C][dv]
+    static constexpr int oS = oV + szRD;         // S [dv][dk]
+    static constexpr int oT = oS + szDD;         // T [C][C]
+    static constexpr int oA = oT + (DELTA ? szCC : 0);
+    static constexpr int oBeta = oA + szRA;
+    static constexpr int total = oBeta + C * 4;
 };
 
 template <typename T, int C, bool DELTA, bool FMAP>
-__global__ void __launch_bounds__(NTHREADS, 2)  // 2 waves per SIMD: two workgroups share a CU
+__global__ void __launch_bounds__(NTHR, 2)  // 2 waves per SIMD: two workgroups share a CU
 chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
                  const float *__restrict__ S0, T *__restrict__ o, float *__restrict__ S_last,
                  T *__restrict__ S_chk, int Tlen, int H)
 {
     using L = FwdSmem<T, C, DELTA>;
-    using IO = TileIO<T, C>;
+    using IO = TileIO<T, C, NTHR>;
     using P4 = typename TT<T>::pack4;
+    constexpr int LDD = L::LDD, LDC = L::LDC, LDA = L::LDA;
     extern __shared__ __align__(16) unsigned char smem[];
     T *sQ = reinterpret_cast<T *>(smem + L::oQ);
     T *sW = sQ;
     T *sK = reinterpret_cast<T *>(smem + L::oK);
-    T *sKt = reinterpret_cast<T *>(smem + L::oKt);
-    T *sVt = reinterpret_cast<T *>(smem + L::oVt);
-    T *sUt = sVt;
+    T *sV = reinterpret_cast<T *>(smem + L::oV);
     T *sS = reinterpret_cast<T *>(smem + L::oS);
     T *sT = reinterpret_cast<T *>(smem + L::oT);
     float *sA = reinterpret_cast<float *>(smem + L::oA);
     T *sAqk = reinterpret_cast<T *>(smem + L::oA);
+    T *sU = DELTA ? reinterpret_cast<T *>(smem + L::oA + L::szCC) : sV;
     float *sBeta = reinterpret_cast<float *>(smem + L::oBeta);
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -63,14 +71,12 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     const int li = lane & 15, lg = lane >> 4;
     const int bh = blockIdx.x, b = bh / H, h = bh % H;
     const int64_t rs = (int64_t)H * HD;  // row stride of q/k/v/o
-    const T *qb = q + ((int64_t)b * Tlen * H + h) * HD;
-    const T *kb = k + ((int64_t)b * Tlen * H + h) * HD;
-    const T *vb = v + ((int64_t)b * Tlen * H + h) * HD;
-    T *ob = o + ((int64_t)b * Tlen * H + h) * HD;
+    const int64_t base = ((int64_t)b * Tlen * H + h) * HD;
     const int NC = (Tlen + C - 1) / C;
 
-    // state S^T (m = d_k, n = d_v) in accumulators
-    using TMS = TileMap<HD, HD>;
+    using TMS = TileMap<HD, HD, NW>;  // S^T : m = dk, n = dv
+    using TMO = TileMap<HD, C, NW>;   // X^T : m = feature, n = chunk row
+    using TMA = TileMap<C, C, NW>;
     f32x4 Sacc[TMS::TPW];
 #pragma unroll
     for (int j = 0; j < TMS::TPW; ++j) {
@@ -79,14 +85,15 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                      : f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    // register prefetch of the next chunk
+    MRX_WG_BEGIN();
+    // register prefetch of the next chunk (raw bits only: no arithmetic on in-flight loads)
     typename IO::Regs rq, rk, rv;
-    uint32_t rbeta = 0u, rdone = 0u;  // raw bits, converted when the chunk is staged
+    uint32_t rbeta = 0u, rdone = 0u;
     auto prefetch = [&](int c) {
         const int t0 = c * C;
-        IO::load(rq, qb, rs, t0, Tlen, tid);
-        IO::load(rk, kb, rs, t0, Tlen, tid);
-        IO::load(rv, vb, rs, t0, Tlen, tid);
+        IO::load(rq, q + base, rs, t0, Tlen, tid);
+        IO::load(rk, k + base, rs, t0, Tlen, tid);
+        IO::load(rv, v + base, rs, t0, Tlen, tid);
         rdone = 0u;
         rbeta = 0u;
         if (lane < C && t0 + lane < Tlen) {
@@ -95,160 +102,121 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             if (DELTA && w == 0) rbeta = load_raw<T>(beta + bt * H + h);
         }
     };
-    MRX_WG_BEGIN();
     prefetch(0);
     MRX_PHASE_INIT();
 
     for (int c = 0; c < NC; ++c) {
         const int t0 = c * C;
-        // Episode structure of the chunk, known to every wave from its own ballot.
-        // A chunk that contains resets is processed once per episode ("pass") with
-        // the rows of all other episodes replaced by zeros *by select*, so that a
-        // non-finite value never meets a masked-out zero inside a matrix product.
         const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
         for (int pass = 0; pass <= nres; ++pass) {
-        // ---- P0: stage the chunk -------------------------------------------------
-        {
-            typename IO::Regs fq = rq, fk = rk, fv = rv;
-            IO::template fmap<FMAP>(fq);
-            IO::template fmap<FMAP>(fk);
-            if (nres != 0) {
-                const int r0 = tid / IO::SEGS;
+            auto live = [&](int r) { return nres == 0 || episode_of(dmask, r) == pass; };
+            // ---- stage the chunk ---------------------------------------------------
+            {
+                typename IO::Regs fq = rq, fk = rk, fv = rv;
+                IO::template fmap<FMAP>(fq);
+                IO::template fmap<FMAP>(fk);
+                if (nres != 0) {
+                    IO::mask_rows(fq, tid, live);
+                    IO::mask_rows(fk, tid, live);
+                    IO::mask_rows(fv, tid, live);
+                }
+                IO::to_lds(fq, sQ, LDD, tid);
+                IO::to_lds(fk, sK, LDD, tid);
+                IO::to_lds(fv, sV, LDD, tid);
+            }
+            if (DELTA && tid < C) sBeta[tid] = live(tid) ? raw_to_float<T>(rbeta) : 0.f;
+            if (pass != 0) zero_acc<TMS::TPW>(Sacc);  // an episode that starts in the chunk starts from 0
+            store_acc<T, HD, HD, NW>(Sacc, sS, LDD, w, lane);  // sS[dv][dk]
+            if (S_chk && pass == 0) {
+                T *dst = S_chk + ((int64_t)bh * NC + c) * HD * HD;
 #pragma unroll
-                for (int p = 0; p < IO::PASSES; ++p) {
-                    const int r = r0 + p * IO::RPP;
-                    if (episode_of(dmask, r) != pass) {
-#pragma unroll
-                        for (int e = 0; e < IO::KP; ++e) {
-                            fq.v[p][e] = (T)0.f; fk.v[p][e] = (T)0.f; fv.v[p][e] = (T)0.f;
-                        }
-                    }
+                for (int j = 0; j < TMS::TPW; ++j) {
+                    const int dk0 = TMS::mt(w) * 16 + 4 * lg, dv = TMS::nt(w, j) * 16 + li;
+                    *reinterpret_cast<P4 *>(dst + dv * HD + dk0) =
+                        TT<T>::pack(Sacc[j][0], Sacc[j][1], Sacc[j][2], Sacc[j][3]);
                 }
             }
-            IO::to_lds(fq, sQ, L::LDD, tid);
-            IO::to_lds(fk, sK, L::LDD, tid);
-            IO::to_lds_t(fk, sKt, L::LDC, tid);
-            IO::to_lds_t(fv, sVt, L::LDC, tid);
-        }
-        if (tid < C) {
-            const int sg = episode_of(dmask, tid);
-            if (DELTA) sBeta[tid] = (nres == 0 || sg == pass) ? raw_to_float<T>(rbeta) : 0.f;
-        }
-        if (pass != 0) zero_acc<TMS::TPW>(Sacc);  // an episode that starts in the chunk starts from 0
-        store_acc_t<T, HD, HD>(Sacc, sS, L::LDD, w, lane);  // sS[dv][dk]
-        if (S_chk && pass == 0) {
-            T *dst = S_chk + ((int64_t)bh * NC + c) * HD * HD;
-#pragma unroll
-            for (int j = 0; j < TMS::TPW; ++j) {
-                const int dk0 = TMS::mt(w) * 16 + 4 * lg, dv = TMS::nt(w, j) * 16 + li;
-                *reinterpret_cast<P4 *>(dst + dv * HD + dk0) =
-                    TT<T>::pack(Sacc[j][0], Sacc[j][1], Sacc[j][2], Sacc[j][3]);
-            }
-        }
-        sync_lds();
-        MRX_PHASE(1);
-        if (pass == nres && c + 1 < NC) prefetch(c + 1);
+            sync_lds();
+            MRX_PHASE(1);
+            if (pass == nres && c + 1 < NC) prefetch(c + 1);
 
-        // ---- P1: O^T = m . S Q^T (m over columns), A = beta_i (K K^T) strictly lower ----
-        using TMO = TileMap<HD, C>;  // O^T: m = dv, n = c
-        f32x4 Oacc[TMO::TPW];
-        zero_acc<TMO::TPW>(Oacc);
-        gemm_nt<T, HD, C, HD>(Oacc, sS, L::LDD, sQ, L::LDD, w, lane);
-        using TMA = TileMap<C, C>;
-        if (DELTA) {
-            f32x4 acc[TMA::TPW];
-            zero_acc<TMA::TPW>(acc);
-            gemm_nt<T, C, C, HD>(acc, sK, L::LDD, sK, L::LDD, w, lane);
-            // lane holds KK[i = n][j = m..m+3]; write sA[i][j] = beta_i KK [j < i, same episode]
-#pragma unroll
-            for (int j = 0; j < TMA::TPW; ++j) {
-                const int m0 = TMA::mt(w) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
-                const float bi = sBeta[n];
-                f32x4 r;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) r[e] = (m0 + e < n) ? bi * acc[j][e] : 0.f;
-                *reinterpret_cast<f32x4 *>(sA + n * L::LDA + m0) = r;
+            // ---- O^T[dv][i] = S Q^T ; A[i][j] = beta_i (k_i . k_j), j < i ---------------
+            f32x4 Oacc[TMO::TPW];
+            zero_acc<TMO::TPW>(Oacc);
+            gemm<T, HD, C, HD, ROWK, ROWK, NW>(Oacc, sS, LDD, sQ, LDD, w, lane);
+            if (DELTA) {
+                f32x4 acc[TMA::TPW];
+                zero_acc<TMA::TPW>(acc);
+                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sK, LDD, sK, LDD, w, lane);  // D[m = j][n = i]
+                store_acc_f<float, C, C, NW>(acc, sA, LDA, w, lane,
+                                             [&](int m, int n, float x) { return m < n ? sBeta[n] * x : 0.f; });
+                sync_lds();
+                MRX_PHASE(2);
+                tri_inverse<C>(sA, LDA, w, lane);
+                MRX_PHASE(3);
+                // sT[i][j] = Tm[i][j] beta_j
+                for (int idx = tid; idx < C * C / 4; idx += NTHR) {
+                    const int i = idx / (C / 4), j = (idx % (C / 4)) * 4;
+                    const f32x4 t = tri_inverse_get4(sA, LDA, i, j);
+                    *reinterpret_cast<P4 *>(sT + i * LDC + j) =
+                        TT<T>::pack(t[0] * sBeta[j], t[1] * sBeta[j + 1], t[2] * sBeta[j + 2], t[3] * sBeta[j + 3]);
+                }
+                sync_lds();
+                MRX_PHASE(4);
             }
-        }
-        sync_lds();
-        MRX_PHASE(2);
-
-        if (DELTA) {
-            // ---- P2/P3: Tm = (I + A)^-1 ; sT[i][j] = Tm[i][j] beta_j -----------------
-            tri_inverse<C>(sA, L::LDA, w, lane);
-            MRX_PHASE(3);
-            for (int idx = tid; idx < C * C / 4; idx += NTHREADS) {
-                const int i = idx / (C / 4), j = (idx % (C / 4)) * 4;
-                const f32x4 t = tri_inverse_get4(sA, L::LDA, i, j);
-                *reinterpret_cast<P4 *>(sT + i * L::LDC + j) =
-                    TT<T>::pack(t[0] * sBeta[j], t[1] * sBeta[j + 1], t[2] * sBeta[j + 2], t[3] * sBeta[j + 3]);
+            // ---- Aqk[i][j] = (q_i . k_j), j <= i ; U^T[dv][c] = V^T T^T ---------------------
+            {
+                f32x4 acc[TMA::TPW];
+                zero_acc<TMA::TPW>(acc);
+                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sK, LDD, sQ, LDD, w, lane);  // D[m = j][n = i]
+                store_acc_f<T, C, C, NW>(acc, sAqk, LDC, w, lane,
+                                         [](int m, int n, float x) { return m <= n ? x : 0.f; });
+            }
+            if (DELTA) {
+                f32x4 Uacc[TMO::TPW];
+                zero_acc<TMO::TPW>(Uacc);
+                gemm<T, HD, C, C, KROW, ROWK, NW>(Uacc, sV, LDD, sT, LDC, w, lane);
+                sync_lds();  // every wave is done with sQ
+                MRX_PHASE(5);
+                // W^T[dk][c] = K^T T^T -> sW[c][dk]
+                {
+                    f32x4 acc[TMO::TPW];
+                    zero_acc<TMO::TPW>(acc);
+                    gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sK, LDD, sT, LDC, w, lane);
+                    store_acc<T, HD, C, NW>(acc, sW, LDD, w, lane);
+                }
+                sync_lds();
+                MRX_PHASE(6);
+                // U'^T[dv][c] = U^T - S W^T -> sU[c][dv]
+                {
+                    f32x4 acc[TMO::TPW];
+                    zero_acc<TMO::TPW>(acc);
+                    gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc, sS, LDD, sW, LDD, w, lane);
+#pragma unroll
+                    for (int j = 0; j < TMO::TPW; ++j) Uacc[j] -= acc[j];
+                    store_acc<T, HD, C, NW>(Uacc, sU, LDD, w, lane);
+                }
             }
             sync_lds();
-        MRX_PHASE(4);
-        }
-
-        // ---- P4: Aqk[i][j] = (q_i . k_j) [j <= i, same episode] ; U = T V ------------
-        {
-            f32x4 acc[TMA::TPW];
-            zero_acc<TMA::TPW>(acc);
-            gemm_nt<T, C, C, HD>(acc, sK, L::LDD, sQ, L::LDD, w, lane);  // D[m = j][n = i]
+            MRX_PHASE(7);
+            // ---- O^T[dv][i] += sum_j U'[j][dv] Aqk[i][j] ; store O ------------------------------
+            gemm<T, HD, C, C, KROW, ROWK, NW>(Oacc, sU, LDD, sAqk, LDC, w, lane);
 #pragma unroll
-            for (int j = 0; j < TMA::TPW; ++j) {
-                const int m0 = TMA::mt(w) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
-                float r[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) r[e] = (m0 + e <= n) ? acc[j][e] : 0.f;
-                *reinterpret_cast<P4 *>(sAqk + n * L::LDC + m0) = TT<T>::pack(r[0], r[1], r[2], r[3]);
+            for (int j = 0; j < TMO::TPW; ++j) {
+                const int dv0 = TMO::mt(w) * 16 + 4 * lg, cc = TMO::nt(w, j) * 16 + li;
+                if (t0 + cc < Tlen && live(cc))
+                    *reinterpret_cast<P4 *>(o + base + (int64_t)(t0 + cc) * rs + dv0) =
+                        TT<T>::pack(Oacc[j][0], Oacc[j][1], Oacc[j][2], Oacc[j][3]);
             }
-        }
-        if (DELTA) {
-            using TMU = TileMap<C, HD>;  // U: m = c, n = dv
-            f32x4 Uacc[TMU::TPW];
-            zero_acc<TMU::TPW>(Uacc);
-            gemm_nt<T, C, HD, C>(Uacc, sT, L::LDC, sVt, L::LDC, w, lane);
-            sync_lds();  // sQ and sVt are dead, sAqk visible
-        MRX_PHASE(5);
-            // ---- P5: W^T = K^T T^T -> sW[c][dk] ---------------------------------------
-            {
-                using TMW = TileMap<HD, C>;  // m = dk, n = c
-                f32x4 acc[TMW::TPW];
-                zero_acc<TMW::TPW>(acc);
-                gemm_nt<T, HD, C, C>(acc, sKt, L::LDC, sT, L::LDC, w, lane);
-                store_acc_t<T, HD, C>(acc, sW, L::LDD, w, lane);
-            }
+            // ---- S^T[dk][dv] += sum_c K[c][dk] U'[c][dv]  (only the episode that leaves the chunk)
+            if (pass == nres) gemm<T, HD, HD, C, KROW, KROW, NW>(Sacc, sK, LDD, sU, LDD, w, lane);
             sync_lds();
-        MRX_PHASE(6);
-            // ---- P6: U' = U - m . W S^T -> sUt[dv][c] -----------------------------------
-            {
-                f32x4 acc[TMU::TPW];
-                zero_acc<TMU::TPW>(acc);
-                gemm_nt<T, C, HD, HD>(acc, sW, L::LDD, sS, L::LDD, w, lane);
-#pragma unroll
-                for (int j = 0; j < TMU::TPW; ++j) Uacc[j] -= acc[j];
-                store_acc_t<T, C, HD>(Uacc, sUt, L::LDC, w, lane);
-            }
+            MRX_PHASE(8);
         }
-        sync_lds();
-        MRX_PHASE(7);
-
-        // ---- P7: O^T += U'^T Aqk^T ; store O ----------------------------------------
-        gemm_nt<T, HD, C, C>(Oacc, sUt, L::LDC, sAqk, L::LDC, w, lane);
-#pragma unroll
-        for (int j = 0; j < TMO::TPW; ++j) {
-            const int dv0 = TMO::mt(w) * 16 + 4 * lg, cc = TMO::nt(w, j) * 16 + li;
-            if (t0 + cc < Tlen && (nres == 0 || episode_of(dmask, cc) == pass))
-                *reinterpret_cast<P4 *>(ob + (int64_t)(t0 + cc) * rs + dv0) =
-                    TT<T>::pack(Oacc[j][0], Oacc[j][1], Oacc[j][2], Oacc[j][3]);
-        }
-        // ---- P8: S^T <- S^T + K^T U'  (only the episode that leaves the chunk) ---------
-        if (pass == nres) gemm_nt<T, HD, HD, C>(Sacc, sKt, L::LDC, sUt, L::LDC, w, lane);
-        sync_lds();
-        MRX_PHASE(8);
-        }  // pass
     }
-
     MRX_WG_END();
+
     if (S_last) {
 #pragma unroll
         for (int j = 0; j < TMS::TPW; ++j) {
@@ -272,7 +240,7 @@ int launch(hipStream_t st, const void *q, const void *k, const void *v, const vo
             return MRX_ERR_LAUNCH;
         attr_set = true;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(NTHREADS), smem, st, (const T *)q,
+    hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(NTHR), smem, st, (const T *)q,
                        (const T *)k, (const T *)v, (const T *)beta, done, done_f32,
                        (const float *)S0, (T *)o, (float *)S_last, (T *)S_chk, (int)Tlen, (int)H);
     return launch_status();
