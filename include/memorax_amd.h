@@ -117,19 +117,25 @@ int mrx_linear_attn_bwd(void *stream, const void *q, const void *k,
  * (beta v k^T, I - beta k k^T):
  *     S' = done_t ? 0 : S_{t-1} ;  S_t = S'(I - beta_t k_t k_t^T) + beta_t v_t k_t^T ;
  *     o_t = S_t q_t
- * beta: (B,T,H) in `dtype`; other arguments as for linear attention. */
+ * beta: (B,T,H) in `dtype`; other arguments as for linear attention.
+ * Tm_chk (nullable): (B,H,ceil(T/chunk),chunk,chunk) in `dtype`, receives each
+ * chunk's unit-lower-triangular factor (I + tril(diag(beta) K K^T, -1))^-1, block
+ * diagonal by episode; like S_chk it is a residual the backward call requires. */
 int mrx_delta_rule_fwd(void *stream, const void *q, const void *k,
                        const void *v, const void *beta, const void *done,
                        const void *S0, void *o, void *S_last, void *S_chk,
-                       int64_t B, int64_t T, int64_t H, int64_t dk, int64_t dv,
-                       int dtype, int done_dtype);
+                       void *Tm_chk, int64_t B, int64_t T, int64_t H, int64_t dk,
+                       int64_t dv, int dtype, int done_dtype);
 
+/* Gradients w.r.t. q,k,v,beta (in `dtype`) and S0 (fp32, nullable).  S_chk and
+ * Tm_chk are the residuals written by mrx_delta_rule_fwd on the same inputs.
+ * dtype: MRX_BF16 only (MRX_F32 returns MRX_ERR_UNSUPPORTED). */
 int mrx_delta_rule_bwd(void *stream, const void *q, const void *k,
                        const void *v, const void *beta, const void *done,
-                       const void *S_chk, const void *dout, const void *dS_last,
-                       void *dq, void *dk_out, void *dv_out, void *dbeta,
-                       void *dS0, int64_t B, int64_t T, int64_t H, int64_t dk,
-                       int64_t dv, int dtype, int done_dtype);
+                       const void *S_chk, const void *Tm_chk, const void *dout,
+                       const void *dS_last, void *dq, void *dk_out, void *dv_out,
+                       void *dbeta, void *dS0, int64_t B, int64_t T, int64_t H,
+                       int64_t dk, int64_t dv, int dtype, int done_dtype);
 
 #ifdef __cplusplus
 }

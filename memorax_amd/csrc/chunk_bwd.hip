@@ -2,8 +2,9 @@
 //
 // Chunks are walked from the last to the first with dS (gradient of the state
 // leaving the chunk) carried in MFMA accumulators; the state entering each chunk
-// comes from the checkpoints the forward call wrote (S_chk), everything else of the
-// forward (A, Tm, W, U', masked QK^T) is recomputed per chunk.  A chunk that
+// comes from the checkpoints the forward call wrote (S_chk), as does the delta rule's
+// triangular factor Tm (Tm_chk); everything else of the forward (W, U', masked QK^T) is
+// recomputed per chunk.  A chunk that
 // contains resets is processed once per episode, last episode first, with the rows
 // of the other episodes zeroed by select; dS only flows into the episode that
 // leaves the chunk and only out of the episode that enters it.
@@ -13,7 +14,7 @@
 //   dAqk = tril(dO U'^T)                   dQ  = dO S + dAqk K
 //   dK  = dAqk^T Q + U' dS                 dS <- dS + Q^T dO - W^T dU'   (stored as dS^T)
 //   linear attention: U' = V, dV = dU', W = 0.
-//   delta rule:  A = tril(diag(beta) K K^T, -1), Tm = (I+A)^-1, T = Tm diag(beta),
+//   delta rule:  A = tril(diag(beta) K K^T, -1), Tm = (I+A)^-1 (from the forward call), T = Tm diag(beta),
 //     W = T K, U' = T V - W S^T, dW = -dU' S, Zu = Tm^T dU', Zw = Tm^T dW,
 //     dV = diag(beta) Zu, dK += diag(beta) Zw, dbeta = rowdot(V, Zu) + rowdot(K, Zw),
 //     dT = tril(dW K^T + dU' V^T), dA = -tril((Tm^T dT) T^T, -1),
@@ -225,9 +226,8 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 template <typename T, int C, int NW> struct DeltaBwdSmem : BwdDims<T, C> {
     using D = BwdDims<T, C>;
     static constexpr int U = D::szDD;  // every tile type has this size for bf16 / C = 64
-    static_assert(D::szRD == U && D::szCC == U, "regions assume equal tile sizes");
-    static_assert(C * (C + 4) * 4 <= 2 * U, "fp32 A must fit two regions");
-    static constexpr int NREG = 12;
+    static_assert(D::szRD == U && D::szCC == U && C == HD, "regions assume equal tile sizes");
+        static constexpr int NREG = 12;
     static constexpr int oBeta = NREG * U, oDb = oBeta + C * 4, total = oDb + 4 * C * 4;
 };
 
@@ -235,16 +235,17 @@ template <typename T, int C, int NW>
 __global__ void __launch_bounds__(64 * NW)
 delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
-                 const T *__restrict__ S_chk, const T *__restrict__ dout,
-                 const float *__restrict__ dS_last, T *__restrict__ dq, T *__restrict__ dk,
-                 T *__restrict__ dv, T *__restrict__ dbeta, float *__restrict__ dS0, int Tlen, int H)
+                 const T *__restrict__ S_chk, const T *__restrict__ Tm_chk,
+                 const T *__restrict__ dout, const float *__restrict__ dS_last, T *__restrict__ dq,
+                 T *__restrict__ dk, T *__restrict__ dv, T *__restrict__ dbeta,
+                 float *__restrict__ dS0, int Tlen, int H)
 {
     constexpr int NTHR = 64 * NW;
     using L = DeltaBwdSmem<T, C, NW>;
     using IO = TileIO<T, C, NTHR>;
     using IOS = TileIO<T, HD, NTHR>;
     using P4 = typename TT<T>::pack4;
-    constexpr int LDD = L::LDD, LDC = L::LDC, LDA = C + 4;
+    constexpr int LDD = L::LDD, LDC = L::LDC;
     extern __shared__ __align__(16) unsigned char smem[];
     auto reg = [&](int r) { return reinterpret_cast<T *>(smem + r * L::U); };
     // region plan (-> marks reuse once the previous tenant is dead)
@@ -253,7 +254,6 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     T *sDO = reg(3), *sY1 = reg(3);                       // dO[c][dv] -> Y1[j][b]
     T *sS = reg(4), *sDA = reg(4);                        // S[dv][dk] -> dA[i][j]
     T *sDS = reg(5), *sDW = reg(5);                       // dS[dv][dk] -> dW[c][dk]
-    float *sA = reinterpret_cast<float *>(smem + 6 * L::U);  // regions 6,7 (fp32 A / Tm)
     T *sAqk = reg(6), *sDAqk = reg(6), *sG = reg(6);      // Aqk[i][j] -> dAqk[i][j] -> G[i][j]
     T *sW = reg(7);                                       // W[c][dk]
     T *sT = reg(8), *sTm = reg(9), *sU = reg(10), *sDU = reg(11);
@@ -280,7 +280,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     }
 
     typename IO::Regs rq, rk, rv, rdo;
-    typename IOS::Regs rS;
+    typename IOS::Regs rS, rTm;
     uint32_t rdone = 0u, rbeta = 0u;  // raw bits, converted when the chunk is staged
     auto prefetch = [&](int c) {
         const int t0 = c * C;
@@ -289,6 +289,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         IO::load(rv, v + base, rs, t0, Tlen, tid);
         IO::load(rdo, dout + base, rs, t0, Tlen, tid);
         IOS::load(rS, S_chk + ((int64_t)bh * NC + c) * HD * HD, HD, 0, HD, tid);
+        IOS::load(rTm, Tm_chk + ((int64_t)bh * NC + c) * C * C, C, 0, C, tid);
         rdone = 0u;
         rbeta = 0u;
         if (lane < C && t0 + lane < Tlen) {
@@ -322,6 +323,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 typename IOS::Regs fS = rS;
                 if (pass != 0) IOS::zero(fS);
                 IOS::to_lds(fS, sS, LDD, tid);
+                IOS::to_lds(rTm, sTm, LDC, tid);  // Tm[i][j] from the forward call (block diagonal by episode)
             }
             if (tid < C) sBeta[tid] = live(tid) ? raw_to_float<T>(rbeta) : 0.f;
             if (pass != nres) zero_acc<TMS::TPW>(dSacc);
@@ -330,27 +332,15 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             MRX_PHASE(11);
             if (pass == 0 && c > 0) prefetch(c - 1);
 
-            // ---- A[i][j] = beta_i (k_i . k_j), j < i -> sA -------------------------------
-            {
-                f32x4 acc[TMA::TPW];
-                zero_acc<TMA::TPW>(acc);
-                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sK, LDD, sK, LDD, w, lane);  // D[m = j][n = i]
-                store_acc_f<float, C, C, NW>(acc, sA, LDA, w, lane,
-                                             [&](int m, int n, float x) { return m < n ? sBeta[n] * x : 0.f; });
-            }
-            sync_lds();
-            MRX_PHASE(12);
-            tri_inverse<C>(sA, LDA, w, lane);
-            MRX_PHASE(13);
-            // ---- sT[i][j] = Tm[i][j] beta_j ; sTm[i][j] = Tm[i][j] -------------------------
+            // ---- sT[i][j] = Tm[i][j] beta_j (beta of rows outside the pass is 0) -------------
             for (int idx = tid; idx < C * C / 4; idx += NTHR) {
                 const int i = idx / (C / 4), j = (idx % (C / 4)) * 4;
-                const f32x4 t = tri_inverse_get4(sA, LDA, i, j);
+                const P4 t = *reinterpret_cast<const P4 *>(sTm + i * LDC + j);
                 *reinterpret_cast<P4 *>(sT + i * LDC + j) =
-                    TT<T>::pack(t[0] * sBeta[j], t[1] * sBeta[j + 1], t[2] * sBeta[j + 2], t[3] * sBeta[j + 3]);
-                *reinterpret_cast<P4 *>(sTm + i * LDC + j) = TT<T>::pack(t[0], t[1], t[2], t[3]);
+                    TT<T>::pack((float)t[0] * sBeta[j], (float)t[1] * sBeta[j + 1], (float)t[2] * sBeta[j + 2],
+                                (float)t[3] * sBeta[j + 3]);
             }
-            sync_lds();  // sA dead
+            sync_lds();
             MRX_PHASE(14);
             // ---- Aqk[i][j] (j <= i) ; W^T[dk][c] = sum_j K[j][dk] T[c][j] -> sW[c][dk] -------
             {
@@ -595,14 +585,15 @@ extern "C" int mrx_linear_attn_bwd(void *stream, const void *q, const void *k, c
 
 extern "C" int mrx_delta_rule_bwd(void *stream, const void *q, const void *k, const void *v,
                                   const void *beta, const void *done, const void *S_chk,
-                                  const void *dout, const void *dS_last, void *dq, void *dk_out,
-                                  void *dv_out, void *dbeta, void *dS0, int64_t B, int64_t T, int64_t H,
-                                  int64_t dk, int64_t dv, int dtype, int done_dtype)
+                                  const void *Tm_chk, const void *dout, const void *dS_last, void *dq,
+                                  void *dk_out, void *dv_out, void *dbeta, void *dS0, int64_t B,
+                                  int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
+                                  int done_dtype)
 {
     const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
                              dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
-    if (!beta || !dbeta) return MRX_ERR_INVALID_ARG;
+    if (!beta || !dbeta || !Tm_chk || !aligned(Tm_chk, 16)) return MRX_ERR_INVALID_ARG;
     if (dtype != MRX_BF16) return MRX_ERR_UNSUPPORTED;  // fp32 delta-rule backward: not built yet
     hipStream_t st = (hipStream_t)stream;
     constexpr int NW = MRX_DELTA_BWD_WAVES;
@@ -612,7 +603,7 @@ extern "C" int mrx_delta_rule_bwd(void *stream, const void *q, const void *k, co
     if (set_smem(kern, smem, attr_set) != MRX_OK) return MRX_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(64 * NW), smem, st, (const __bf16 *)q,
                        (const __bf16 *)k, (const __bf16 *)v, (const __bf16 *)beta, done, done_dtype,
-                       (const __bf16 *)S_chk, (const __bf16 *)dout, (const float *)dS_last,
+                       (const __bf16 *)S_chk, (const __bf16 *)Tm_chk, (const __bf16 *)dout, (const float *)dS_last,
                        (__bf16 *)dq, (__bf16 *)dk_out, (__bf16 *)dv_out, (__bf16 *)dbeta, (float *)dS0,
                        (int)T, (int)H);
     return launch_status();

@@ -304,16 +304,23 @@ template <int C> __device__ __forceinline__ void tri_inverse(float *sA, int ld, 
     for (int d = 1; d < NB; ++d) {
         if (w < NB - d) {
             const int b = w + d, c = w;  // block (b, c)
-            f32x4 tmp = {0.f, 0.f, 0.f, 0.f};
-            for (int k = c; k < b; ++k) {
-                // tmp += A_bk . X_kc ; X_kc lives at rows 16c.., cols 16k.. (diagonal when k == c)
+            // tmp = sum_{k=c}^{b-1} A_bk . X_kc ; X_kc lives at rows 16c.., cols 16k.. (the
+            // diagonal block when k == c).  One accumulator per k keeps the MFMA chains short.
+            f32x4 part[NB - 1];
+#pragma unroll
+            for (int kk = 0; kk < d; ++kk) {
+                const int k = c + kk;
+                part[kk] = f32x4{0.f, 0.f, 0.f, 0.f};
                 const f32x4 a4 = *reinterpret_cast<const f32x4 *>(sA + (16 * b + i) * ld + 16 * k + 4 * g);
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
                     const float bop = sA[(16 * c + 4 * g + s) * ld + 16 * k + i];
-                    tmp = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[s], bop, tmp, 0, 0, 0);
+                    part[kk] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[s], bop, part[kk], 0, 0, 0);
                 }
             }
+            f32x4 tmp = part[0];
+#pragma unroll
+            for (int kk = 1; kk < d; ++kk) tmp += part[kk];
             // X_bc = -X_bb . tmp ; the accumulator layout of tmp is already the B-operand layout
             f32x4 res = {0.f, 0.f, 0.f, 0.f};
             const f32x4 a4 = *reinterpret_cast<const f32x4 *>(sA + (16 * b + i) * ld + 16 * b + 4 * g);

@@ -48,7 +48,7 @@ __global__ void __launch_bounds__(NTHR, 2)  // 2 waves per SIMD: two workgroups 
 chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
                  const float *__restrict__ S0, T *__restrict__ o, float *__restrict__ S_last,
-                 T *__restrict__ S_chk, int Tlen, int H)
+                 T *__restrict__ S_chk, T *__restrict__ Tm_chk, int Tlen, int H)
 {
     using L = FwdSmem<T, C, DELTA>;
     using IO = TileIO<T, C, NTHR>;
@@ -161,6 +161,11 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     const f32x4 t = tri_inverse_get4(sA, LDA, i, j);
                     *reinterpret_cast<P4 *>(sT + i * LDC + j) =
                         TT<T>::pack(t[0] * sBeta[j], t[1] * sBeta[j + 1], t[2] * sBeta[j + 2], t[3] * sBeta[j + 3]);
+                    // residual for the backward call: the rows of this pass's episode
+                    // (rows past the end of the sequence count as the last episode: identity rows)
+                    if (Tm_chk && live(i))
+                        *reinterpret_cast<P4 *>(Tm_chk + (((int64_t)bh * NC + c) * C + i) * C + j) =
+                            TT<T>::pack(t[0], t[1], t[2], t[3]);
                 }
                 sync_lds();
                 MRX_PHASE(4);
@@ -229,7 +234,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 template <typename T, int C, bool DELTA, bool FMAP>
 int launch(hipStream_t st, const void *q, const void *k, const void *v, const void *beta,
            const void *done, int done_f32, const void *S0, void *o, void *S_last, void *S_chk,
-           int64_t B, int64_t Tlen, int64_t H)
+           void *Tm_chk, int64_t B, int64_t Tlen, int64_t H)
 {
     auto kern = chunk_fwd_kernel<T, C, DELTA, FMAP>;
     constexpr int smem = FwdSmem<T, C, DELTA>::total;
@@ -242,7 +247,7 @@ int launch(hipStream_t st, const void *q, const void *k, const void *v, const vo
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(NTHR), smem, st, (const T *)q,
                        (const T *)k, (const T *)v, (const T *)beta, done, done_f32,
-                       (const float *)S0, (T *)o, (float *)S_last, (T *)S_chk, (int)Tlen, (int)H);
+                       (const float *)S0, (T *)o, (float *)S_last, (T *)S_chk, (T *)Tm_chk, (int)Tlen, (int)H);
     return launch_status();
 }
 
@@ -278,22 +283,22 @@ extern "C" int mrx_linear_attn_fwd(void *stream, const void *q, const void *k, c
     hipStream_t st = (hipStream_t)stream;
     const bool fm = feature_map == MRX_FMAP_ELU1;
     if (dtype == MRX_BF16)
-        return fm ? launch<__bf16, 64, false, true>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, B, T, H)
-                  : launch<__bf16, 64, false, false>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, B, T, H);
-    return fm ? launch<float, 32, false, true>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, B, T, H)
-              : launch<float, 32, false, false>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, B, T, H);
+        return fm ? launch<__bf16, 64, false, true>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H)
+                  : launch<__bf16, 64, false, false>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H);
+    return fm ? launch<float, 32, false, true>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H)
+              : launch<float, 32, false, false>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H);
 }
 
 extern "C" int mrx_delta_rule_fwd(void *stream, const void *q, const void *k, const void *v,
                                   const void *beta, const void *done, const void *S0, void *o,
-                                  void *S_last, void *S_chk, int64_t B, int64_t T, int64_t H,
-                                  int64_t dk, int64_t dv, int dtype, int done_dtype)
+                                  void *S_last, void *S_chk, void *Tm_chk, int64_t B, int64_t T,
+                                  int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype)
 {
     const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
-    if (!beta) return MRX_ERR_INVALID_ARG;
+    if (!beta || !aligned(Tm_chk, 16)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == MRX_BF16)
-        return launch<__bf16, 64, true, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, B, T, H);
-    return launch<float, 32, true, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, B, T, H);
+        return launch<__bf16, 64, true, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H);
+    return launch<float, 32, true, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H);
 }

@@ -87,18 +87,18 @@ class _DeltaRule(torch.autograd.Function):
         q_, k_, v_, b_ = q.contiguous(), k.contiguous(), v.contiguous(), beta.contiguous()
         S0_ = None if S0 is None else S0.contiguous().float()
         need = any(ctx.needs_input_grad)
-        o, S_last, S_chk = K.delta_rule_fwd(q_, k_, v_, b_, done, S0_, save_chk=need)
+        o, S_last, chk = K.delta_rule_fwd(q_, k_, v_, b_, done, S0_, save_chk=need)
         if need:
-            ctx.save_for_backward(q_, k_, v_, b_, S_chk)
+            ctx.save_for_backward(q_, k_, v_, b_, *chk)
         ctx.done, ctx.has_S0 = done, S0 is not None
         return o, S_last
 
     @staticmethod
     def backward(ctx, do, dS_last):
-        q, k, v, beta, S_chk = ctx.saved_tensors
+        q, k, v, beta, S_chk, Tm_chk = ctx.saved_tensors
         do = torch.zeros_like(v) if do is None else do.contiguous()
         dS_last = None if dS_last is None else dS_last.contiguous().float()
-        dq, dk, dv, db, dS0 = K.delta_rule_bwd(q, k, v, beta, ctx.done, S_chk, do, dS_last,
+        dq, dk, dv, db, dS0 = K.delta_rule_bwd(q, k, v, beta, ctx.done, (S_chk, Tm_chk), do, dS_last,
                                                want_dS0=ctx.has_S0)
         return dq, dk, dv, db, None, (dS0 if ctx.has_S0 else None)
 

@@ -156,7 +156,8 @@ def linear_attn_bwd(q, k, v, done, S_chk, do, dS_last=None, feature_map=0, want_
 
 
 def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True):
-    """Returns (o, S_last fp32, S_chk or None)."""
+    """Returns (o, S_last fp32, chk) where chk = (S_chk, Tm_chk) are the residuals the
+    backward call needs, or None."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
     _chk(beta, "beta", dt, (B, T, H))
@@ -164,19 +165,25 @@ def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True):
     done, dd = _done(done, B, T)
     o = torch.empty_like(v)
     S_last = torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
-    S_chk = (torch.empty((B, H, _n_chunks(T, dt), dv, dk), dtype=dt, device=q.device)
-             if save_chk else None)
+    S_chk = Tm_chk = None
+    if save_chk:
+        C, NC = chunk_size(dt), _n_chunks(T, dt)
+        S_chk = torch.empty((B, H, NC, dv, dk), dtype=dt, device=q.device)
+        Tm_chk = torch.empty((B, H, NC, C, C), dtype=dt, device=q.device)
     st = lib.mrx_delta_rule_fwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done),
-                                _ptr(S0), _ptr(o), _ptr(S_last), _ptr(S_chk), B, T, H, dk, dv,
-                                _DT[dt], dd)
+                                _ptr(S0), _ptr(o), _ptr(S_last), _ptr(S_chk), _ptr(Tm_chk), B, T, H,
+                                dk, dv, _DT[dt], dd)
     _lib.check(st, "mrx_delta_rule_fwd")
-    return o, S_last, S_chk
+    return o, S_last, ((S_chk, Tm_chk) if save_chk else None)
 
 
-def delta_rule_bwd(q, k, v, beta, done, S_chk, do, dS_last=None, want_dS0=True):
-    """Returns (dq, dk, dv, dbeta, dS0)."""
+def delta_rule_bwd(q, k, v, beta, done, chk, do, dS_last=None, want_dS0=True):
+    """chk = (S_chk, Tm_chk) from delta_rule_fwd.  Returns (dq, dk, dv, dbeta, dS0)."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
+    S_chk, Tm_chk = chk
+    C = chunk_size(dt)
+    _chk(Tm_chk, "Tm_chk", dt, (B, H, _n_chunks(T, dt), C, C))
     _chk(beta, "beta", dt, (B, T, H))
     _chk(do, "do", dt, (B, T, H, dv))
     _chk(S_chk, "S_chk", dt, (B, H, _n_chunks(T, dt), dv, dk))
@@ -187,7 +194,7 @@ def delta_rule_bwd(q, k, v, beta, done, S_chk, do, dS_last=None, want_dS0=True):
     dS0 = (torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
            if want_dS0 else None)
     st = lib.mrx_delta_rule_bwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done),
-                                _ptr(S_chk), _ptr(do), _ptr(dS_last), _ptr(dq), _ptr(dk_),
+                                _ptr(S_chk), _ptr(Tm_chk), _ptr(do), _ptr(dS_last), _ptr(dq), _ptr(dk_),
                                 _ptr(dv_), _ptr(dbeta), _ptr(dS0), B, T, H, dk, dv, _DT[dt], dd)
     _lib.check(st, "mrx_delta_rule_bwd")
     return dq, dk_, dv_, dbeta, dS0
