@@ -1,0 +1,384 @@
+"""Host-side mirror of memorax's sequence-model interface, on top of the HIP kernels.
+
+Same contract as the reference (memorax/networks/sequence_models):
+
+    SequenceModel.__call__(inputs (B,T,F), done (B,T), initial_carry=None) -> (next_carry, y)
+    SequenceModel.initialize_carry(key, input_shape=(B,F)) -> carry          sequence_model.py:8-19
+    MemoroidCellBase: __call__(x) -> elements, binary_operator(a, b), read(h, x),
+                      initialize_carry(key, input_shape)                      memoroid.py:20-33
+    Memoroid(cell)(inputs, done, initial_carry) = read(scan(cell(inputs)))    memoroid.py:93-109
+
+Carries keep the reference's pytree shapes (leaves with a size-1 time axis, (B,1,...)),
+so Stack-style per-block carry tuples and checkpointing keep working.
+
+What differs: the reference scans *any* cell algebra with jax.lax.associative_scan
+(memoroid.py:60-91).  Here each cell also implements ``scan(elements, carry, done)``,
+which hands its algebra to the matching fused kernel (diagonal scan, chunked linear
+attention, chunked delta rule) instead of materialising per-step states;
+``binary_operator`` remains the definition of the algebra (and is what the tests fold
+to check ``scan``).  Modules are torch.nn.Modules: torch plays the role of the array
+library / autodiff host here, the arithmetic of the recurrences runs in the kernels.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .functional import delta_rule, linear_attention, linear_scan
+
+
+# ----------------------------------------------------------------------------------
+# axes helpers (memorax/utils/axes.py:19-32,46-49)
+# ----------------------------------------------------------------------------------
+def add_time_axis(x):
+    return x[:, None]
+
+
+def remove_time_axis(x):
+    return x.squeeze(1)
+
+
+def get_input_shape(inputs):
+    """(B, T, F) -> (B, F)."""
+    return inputs.shape[:1] + inputs.shape[2:]
+
+
+class SequenceModel(nn.Module):
+    """sequence_model.py:8-19."""
+
+    def forward(self, inputs, done, initial_carry=None, **kwargs):  # pragma: no cover
+        raise NotImplementedError
+
+    def initialize_carry(self, key, input_shape):  # pragma: no cover
+        raise NotImplementedError
+
+
+class MemoroidCellBase(nn.Module):
+    """memoroid.py:20-33 plus the kernel hook ``scan``."""
+
+    def forward(self, x, **kwargs):  # elements
+        raise NotImplementedError
+
+    def binary_operator(self, a, b):
+        raise NotImplementedError
+
+    def read(self, h, x, **kwargs):
+        raise NotImplementedError
+
+    def initialize_carry(self, key, input_shape):
+        raise NotImplementedError
+
+    def scan(self, z, initial_carry, done):
+        """Reset-aware inclusive scan of the cell's algebra over time, carry-in
+        prepended (memoroid.py:60-91).  Returns (h, next_carry)."""
+        raise NotImplementedError
+
+
+class Memoroid(SequenceModel):
+    """memoroid.py:57-112 (without the RTRL hooks)."""
+
+    def __init__(self, cell: MemoroidCellBase):
+        super().__init__()
+        self.cell = cell
+
+    def forward(self, inputs, done, initial_carry=None, **kwargs):
+        if initial_carry is None:
+            initial_carry = self.cell.initialize_carry(None, get_input_shape(inputs))
+        z = self.cell(inputs, **kwargs)
+        h, next_carry = self.cell.scan(z, initial_carry, done)
+        y = self.cell.read(h, inputs, **kwargs)
+        return next_carry, y
+
+    def initialize_carry(self, key, input_shape):
+        return self.cell.initialize_carry(key, input_shape)
+
+
+# ----------------------------------------------------------------------------------
+# diagonal algebra cells
+# ----------------------------------------------------------------------------------
+class _DiagonalCell(MemoroidCellBase):
+    """Cells whose elements are (state, decay) with
+    binary_operator(a, b) = (decay_b * state_a + state_b, decay_b * decay_a)
+    (lru.py:92-95, s5.py:133-136).  ``scan`` returns h = (states (B,T,N), None): the
+    per-step cumulative decay is never materialised, only its last value (the carry)."""
+
+    def binary_operator(self, a, b):
+        state_i, decay_i = a
+        state_j, decay_j = b
+        return (decay_j * state_i + state_j, decay_j * decay_i)
+
+    def scan(self, z, initial_carry, done):
+        state, decay = z            # decay: (B,T,N) or time-invariant (N,)
+        h0, P0 = initial_carry      # (B,1,N)
+        h, h_last, P_last = linear_scan(decay, state, done, h0[:, 0].contiguous(), P0[:, 0].contiguous())
+        return (h, None), (h_last[:, None], P_last[:, None])
+
+
+class LRUCell(_DiagonalCell):
+    """Linear Recurrent Unit, complex diagonal recurrence (lru.py:32-108).  The decay
+    lambda is time-invariant and is passed to the kernel as an (N,) vector instead of
+    being broadcast to (B,T,N) (lru.py:86)."""
+
+    def __init__(self, features, hidden_dim, r_min=0.0, r_max=1.0, max_phase=6.28):
+        super().__init__()
+        self.features, self.hidden_dim = features, hidden_dim
+        u1, u2 = torch.rand(hidden_dim), torch.rand(hidden_dim)
+        nu_log = torch.log(-0.5 * torch.log(u1 * (r_max**2 - r_min**2) + r_min**2))   # lru.py:12-14
+        theta_log = torch.log(max_phase * u2)                                          # lru.py:17-19
+        lam = torch.exp(-torch.exp(nu_log) + 1j * torch.exp(theta_log))
+        self.nu_log = nn.Parameter(nu_log)
+        self.theta_log = nn.Parameter(theta_log)
+        self.gamma_log = nn.Parameter(torch.log(torch.sqrt(1 - torch.abs(lam) ** 2)))  # lru.py:22-25
+        self.B_real = nn.Parameter(torch.randn(hidden_dim, features) / math.sqrt(2 * features))
+        self.B_imag = nn.Parameter(torch.randn(hidden_dim, features) / math.sqrt(2 * features))
+        self.C_real = nn.Parameter(torch.randn(features, hidden_dim) / math.sqrt(hidden_dim))
+        self.C_imag = nn.Parameter(torch.randn(features, hidden_dim) / math.sqrt(hidden_dim))
+        self.D = nn.Parameter(torch.randn(features))
+
+    def forward(self, x, **kwargs):
+        lam = torch.exp(torch.complex(-torch.exp(self.nu_log), torch.exp(self.theta_log)))
+        B_norm = torch.complex(self.B_real, self.B_imag) * torch.exp(self.gamma_log)[:, None]
+        state = x.to(torch.complex64) @ B_norm.T
+        return (state.contiguous(), lam.to(torch.complex64))
+
+    def read(self, h, x, **kwargs):
+        state, _ = h
+        C = torch.complex(self.C_real, self.C_imag)
+        return (state @ C.T).real + self.D * x
+
+    def initialize_carry(self, key, input_shape):
+        *batch, _ = input_shape
+        dev = self.nu_log.device
+        return (torch.zeros(*batch, 1, self.hidden_dim, dtype=torch.complex64, device=dev),
+                torch.ones(*batch, 1, self.hidden_dim, dtype=torch.complex64, device=dev))
+
+
+class MinGRUCell(_DiagonalCell):
+    """MinGRU (min_gru.py:14-90).  The reference scans (log_state, log_decay) with
+    logaddexp; the same recurrence in linear space is h_t = sigma(-z) h_{t-1} +
+    sigma(z) g(h~), g(x) = x + 0.5 (x >= 0) | sigma(x), which is what the kernel scans.
+    The carry keeps the reference's log-space leaves: (log h_T, sum of log decays)."""
+
+    def __init__(self, features, in_features=None):
+        super().__init__()
+        self.features = features
+        in_features = features if in_features is None else in_features
+        self.z = nn.Linear(in_features, features, bias=False)
+        self.h = nn.Linear(in_features, features, bias=False)
+        self.intermediates = {}
+
+    def forward(self, x, **kwargs):
+        z, h_tilde = self.z(x), self.h(x)
+        a = torch.sigmoid(-z)
+        g = torch.where(h_tilde >= 0, torch.relu(h_tilde) + 0.5, torch.sigmoid(h_tilde))
+        self.intermediates["gate"] = z.mean().detach()   # min_gru.py:63 sows the mean gate
+        return ((torch.sigmoid(z) * g).contiguous(), a.contiguous())
+
+    def scan(self, z, initial_carry, done):
+        log_state, log_decay = initial_carry
+        (h, _), (h_last, P_last) = super().scan(z, (torch.exp(log_state), torch.exp(log_decay)), done)
+        return (h, None), (torch.log(h_last), torch.log(P_last))
+
+    def read(self, h, x, **kwargs):
+        return h[0]
+
+    def initialize_carry(self, key, input_shape):
+        *batch, _ = input_shape
+        dev = self.z.weight.device
+        return (torch.full((*batch, 1, self.features), -math.inf, device=dev),
+                torch.zeros(*batch, 1, self.features, device=dev))
+
+
+# ----------------------------------------------------------------------------------
+# matrix-state cells
+# ----------------------------------------------------------------------------------
+class _RMSNorm(nn.Module):
+    """y = x * rsqrt(mean(x^2) + eps) * scale (flax.linen.RMSNorm defaults, eps = 1e-6)."""
+
+    def __init__(self, dim, eps=1e-6):
+        super().__init__()
+        self.scale = nn.Parameter(torch.ones(dim))
+        self.eps = eps
+
+    def forward(self, x):
+        xf = x.float()
+        return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps) * self.scale).to(x.dtype)
+
+
+class LinearAttentionCell(MemoroidCellBase):
+    """Causal linear attention with phi = elu + 1 (linear_attention.py:14-124).
+    Elements are (v phi(k)^T, phi(k)) combined by addition; the reference materialises
+    S (B,T,H,d,d), here the numerator S_t phi(q_t) comes from the chunked kernel and the
+    normaliser z_t = sum phi(k) from the diagonal scan with decay 1."""
+
+    def __init__(self, features, head_dim, num_heads, in_features=None, eps=1e-6):
+        super().__init__()
+        in_features = features if in_features is None else in_features
+        self.features, self.head_dim, self.num_heads, self.eps = features, head_dim, num_heads, eps
+        hidden = head_dim * num_heads
+        self.key = nn.Linear(in_features, hidden, bias=False)
+        self.value = nn.Linear(in_features, hidden, bias=False)
+        self.query = nn.Linear(in_features, hidden, bias=False)
+        self.norm = _RMSNorm(hidden)
+        self.output_projection = nn.Linear(hidden, features)
+
+    def _heads(self, x):
+        return x.view(*x.shape[:2], self.num_heads, self.head_dim)
+
+    def forward(self, x, **kwargs):
+        # pre-feature-map keys: phi is applied inside the kernel (and here for z)
+        return (self._heads(self.value(x)), self._heads(self.key(x)))
+
+    def binary_operator(self, a, b):
+        return tuple(x + y for x, y in zip(a, b))
+
+    def scan(self, z, initial_carry, done):
+        """Returns h = (v, k_raw, z_cum) for read(), which needs the query."""
+        v, k_raw = z
+        S0, z0 = initial_carry            # (B,1,H,dv,dk), (B,1,H,dk)
+        B, T, H, d = k_raw.shape
+        kf = (F.elu(k_raw.float()) + 1).reshape(B, T, H * d)
+        ones = torch.ones(H * d, device=kf.device)
+        zc, z_last, _ = linear_scan(ones, kf, done, z0[:, 0].reshape(B, H * d).float().contiguous())
+        return (v, k_raw, zc.view(B, T, H, d), S0[:, 0], done), z_last.view(B, 1, H, d)
+
+    def read(self, h, x, **kwargs):
+        v, k_raw, zc, S0, done = h
+        q = self._heads(self.query(x))
+        num, S_last = linear_attention(q, k_raw, v, done, S0.float(), "elu1")
+        self._S_last = S_last
+        qf = F.elu(q.float()) + 1
+        den = torch.clamp((qf * zc).sum(-1), min=self.eps)[..., None]
+        out = (num.float() / den).reshape(*x.shape[:2], -1)
+        return self.output_projection(self.norm(out).to(x.dtype))
+
+    def initialize_carry(self, key, input_shape):
+        *batch, _ = input_shape
+        dev = self.key.weight.device
+        return (torch.zeros(*batch, 1, self.num_heads, self.head_dim, self.head_dim, device=dev),
+                torch.zeros(*batch, 1, self.num_heads, self.head_dim, device=dev))
+
+
+class LinearAttention(SequenceModel):
+    """Memoroid(LinearAttentionCell) with the read-out fused around the kernel call: the
+    numerator needs q, k, v together, so the state leaf of the carry is produced by read."""
+
+    def __init__(self, cell: LinearAttentionCell):
+        super().__init__()
+        self.cell = cell
+
+    def forward(self, inputs, done, initial_carry=None, **kwargs):
+        if initial_carry is None:
+            initial_carry = self.cell.initialize_carry(None, get_input_shape(inputs))
+        z = self.cell(inputs)
+        h, z_last = self.cell.scan(z, initial_carry, done)
+        y = self.cell.read(h, inputs)
+        return (self.cell._S_last[:, None], z_last), y
+
+    def initialize_carry(self, key, input_shape):
+        return self.cell.initialize_carry(key, input_shape)
+
+
+class DeltaNetCell(MemoroidCellBase):
+    """DeltaNet: S_t = S_{t-1}(I - beta_t k_t k_t^T) + beta_t v_t k_t^T, o_t = S_t q_t with
+    L2-normalised keys and beta = sigmoid(.).  Not in the reference; written in its cell
+    idiom the elements are the affine maps (beta v k^T, I - beta k k^T) with
+    binary_operator(a, b) = (B_a A_b + B_b, A_a A_b).  The carry is (S (B,1,H,d,d),)."""
+
+    def __init__(self, features, head_dim, num_heads, in_features=None, dtype=torch.bfloat16):
+        super().__init__()
+        in_features = features if in_features is None else in_features
+        self.features, self.head_dim, self.num_heads, self.dtype = features, head_dim, num_heads, dtype
+        hidden = head_dim * num_heads
+        self.query = nn.Linear(in_features, hidden, bias=False)
+        self.key = nn.Linear(in_features, hidden, bias=False)
+        self.value = nn.Linear(in_features, hidden, bias=False)
+        self.beta = nn.Linear(in_features, num_heads, bias=False)
+        self.norm = _RMSNorm(hidden)
+        self.output_projection = nn.Linear(hidden, features)
+
+    def _heads(self, x):
+        return x.view(*x.shape[:2], self.num_heads, self.head_dim)
+
+    def forward(self, x, **kwargs):
+        q = self._heads(self.query(x))
+        k = F.normalize(self._heads(self.key(x)).float(), dim=-1)
+        v = self._heads(self.value(x))
+        beta = torch.sigmoid(self.beta(x).float())
+        dt = self.dtype
+        return (q.to(dt), k.to(dt), v.to(dt), beta.to(dt))
+
+    def binary_operator(self, a, b):
+        B_i, A_i = a
+        B_j, A_j = b
+        return (B_i @ A_j + B_j, A_i @ A_j)
+
+    def scan(self, z, initial_carry, done):
+        q, k, v, beta = z
+        (S0,) = initial_carry
+        o, S_last = delta_rule(q, k, v, beta, done, S0[:, 0].float())
+        return o, (S_last[:, None],)
+
+    def read(self, h, x, **kwargs):
+        out = h.reshape(*x.shape[:2], -1)
+        return self.output_projection(self.norm(out).to(x.dtype))
+
+    def initialize_carry(self, key, input_shape):
+        *batch, _ = input_shape
+        dev = self.key.weight.device
+        return (torch.zeros(*batch, 1, self.num_heads, self.head_dim, self.head_dim, device=dev),)
+
+
+# ----------------------------------------------------------------------------------
+# block composition used by the torso configuration (blocks/{stack,residual,normalization}.py)
+# ----------------------------------------------------------------------------------
+class PreNorm(nn.Module):
+    """normalization.py:10-35: norm, then the wrapped sequence model."""
+
+    def __init__(self, module, dim):
+        super().__init__()
+        self.module, self.norm = module, _RMSNorm(dim)
+
+    def forward(self, inputs, done=None, initial_carry=None, **kwargs):
+        return self.module(self.norm(inputs), done, initial_carry, **kwargs)
+
+    def initialize_carry(self, key, input_shape):
+        return self.module.initialize_carry(key, input_shape)
+
+
+class Residual(nn.Module):
+    """residual.py:10-30: x + module(x)."""
+
+    def __init__(self, module):
+        super().__init__()
+        self.module = module
+
+    def forward(self, inputs, done=None, initial_carry=None, **kwargs):
+        carry, y = self.module(inputs, done, initial_carry, **kwargs)
+        return carry, inputs + y
+
+    def initialize_carry(self, key, input_shape):
+        return self.module.initialize_carry(key, input_shape)
+
+
+class Stack(nn.Module):
+    """stack.py:10-60: one carry per block, threaded as a tuple."""
+
+    def __init__(self, blocks):
+        super().__init__()
+        self.blocks = nn.ModuleList(blocks)
+
+    def forward(self, inputs, done=None, initial_carry=None, **kwargs):
+        if initial_carry is None:
+            initial_carry = tuple(None for _ in self.blocks)
+        x, carries = inputs, []
+        for block, c in zip(self.blocks, initial_carry):
+            carry, x = block(x, done=done, initial_carry=c, **kwargs)
+            carries.append(carry)
+        return tuple(carries), x
+
+    def initialize_carry(self, key, input_shape):
+        return tuple(b.initialize_carry(key, input_shape) for b in self.blocks)
