@@ -24,6 +24,11 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 #   forward : read q,k,v (3*128) + beta (2), write o (128)                    = 514
 #   backward: read q,k,v,do (4*128) + beta (2), write dq,dk,dv (3*128) + dbeta (2) = 900
 BYTES_FWD, BYTES_BWD = 514, 900
+# HBM bytes one delta_bwd_kernel launch actually moves at this workload, from rocprofv3 --pmc
+# FETCH_SIZE and WRITE_SIZE runs scaled by a plain elementwise kernel of known size
+# (summary kept under profiles/).  The excess over the algorithmic bytes is the forward's
+# per-chunk residuals (state checkpoints and triangular factors) being read back.
+TRAFFIC_BWD_BYTES = 621.5e6
 
 
 def main() -> int:
@@ -33,6 +38,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--all", action="store_true", help="also time the other configurations")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch a plain elementwise kernel of known size (256 MiB read, 256 MiB "
+                         "written) so that a rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE run can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU; this build has no multi-GPU path (--gpus must be 1)",
@@ -104,7 +112,7 @@ def main() -> int:
                                "bf16 in / fp32 state, chunk 64, resets p=0.002"},
         "roofline": {
             "bound": "hbm", "kernel": "delta_bwd_kernel", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
-            "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": None,
+            "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": TRAFFIC_BWD_BYTES,
             "launch_ms": tb_ms, "algorithmic_bytes": BYTES_BWD * nth,
         },
         "kernels": {
@@ -115,6 +123,13 @@ def main() -> int:
         },
     }
 
+    if args.calibrate:
+        cx = torch.zeros(64 * 1024 * 1024, device="cuda")  # 256 MiB fp32
+        cy = torch.empty_like(cx)
+        for _ in range(3):
+            torch.add(cx, 1.0, out=cy)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del cx, cy
     out["scan"] = bench_scan(torch, K, M, dev)
     if args.all:
         out["linear_attention"] = bench_linear_attention(torch, K, M, dev)
