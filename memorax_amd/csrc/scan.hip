@@ -9,6 +9,8 @@
 // summaries to its left into a carry-in and fixes its slice up by *select*
 // (a reset inside the slice wins over the carry, so NaN/Inf never cross a reset).
 // One pass over HBM in either case.
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
@@ -329,13 +331,149 @@ diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hfw,
     }
 }
 
+
+// ---- streaming kernels: enough (batch x feature) columns to fill the chip ------------
+// No time split.  Each lane walks all of T for its VEC channels in groups of SG steps,
+// with the loads of the next group issued before the current group is consumed
+// (register double buffering), so a wave always has 2*SG (forward) / 3*SG (backward)
+// row loads in flight.  done flags are prefetched as raw bits with the data.
+template <typename E, int VEC, int SG>
+__global__ void __launch_bounds__(256)
+diag_scan_fwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ b,
+                            const void *__restrict__ done, int done_f32,
+                            const E *__restrict__ h0, const E *__restrict__ P0,
+                            E *__restrict__ h, E *__restrict__ h_last, E *__restrict__ P_last,
+                            int64_t B, int T, int64_t D, int64_t cols_per_row, int a_ti)
+{
+    using V = Vec<E, VEC>;
+    using O = Ops<E>;
+    // one thread per VEC channels of one batch row
+    const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t bi = gid / cols_per_row;
+    const int64_t col = (gid % cols_per_row) * VEC;
+    if (bi >= B) return;  // padding threads of the last workgroup (this kernel has no barriers)
+    const int64_t row0 = bi * T;
+    V ch = vfill<E, VEC>(O::zero()), cp = vfill<E, VEC>(O::one());
+    if (h0) ch = *reinterpret_cast<const V *>(h0 + bi * D + col);
+    if (P0) cp = *reinterpret_cast<const V *>(P0 + bi * D + col);
+
+    V xa[SG], xb[SG], na[SG], nb[SG];
+    uint32_t xd[SG], nd[SG];
+    auto load = [&](int t0, V *pa, V *pb, uint32_t *pd) {
+#pragma unroll
+        for (int s = 0; s < SG; ++s) {
+            const int t = t0 + s;
+            pd[s] = 0u;
+            if (t < T) {
+                const int64_t off = (row0 + t) * D + col;
+                pa[s] = *reinterpret_cast<const V *>(a + (a_ti ? col : off));
+                pb[s] = *reinterpret_cast<const V *>(b + off);
+                pd[s] = done_raw(done, done_f32, row0 + t);
+            }
+        }
+    };
+    load(0, xa, xb, xd);
+    for (int t0 = 0; t0 < T; t0 += SG) {
+        if (t0 + SG < T) load(t0 + SG, na, nb, nd);
+#pragma unroll
+        for (int s = 0; s < SG; ++s) {
+            if (t0 + s < T) {
+                const bool r = done_test(xd[s], done_f32);
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    const E hn = O::madd(xa[s].v[i], ch.v[i], xb[s].v[i]);
+                    const E pn = O::mul(xa[s].v[i], cp.v[i]);
+                    ch.v[i] = r ? xb[s].v[i] : hn;
+                    cp.v[i] = r ? xa[s].v[i] : pn;
+                }
+                *reinterpret_cast<V *>(h + (row0 + t0 + s) * D + col) = ch;
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < SG; ++s) { xa[s] = na[s]; xb[s] = nb[s]; xd[s] = nd[s]; }
+    }
+    if (h_last) *reinterpret_cast<V *>(h_last + bi * D + col) = ch;
+    if (P_last) *reinterpret_cast<V *>(P_last + bi * D + col) = cp;
+}
+
+template <typename E, int VEC, int SG>
+__global__ void __launch_bounds__(256)
+diag_scan_bwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ hfw,
+                            const void *__restrict__ done, int done_f32,
+                            const E *__restrict__ h0, const E *__restrict__ g,
+                            const E *__restrict__ g_last, E *__restrict__ da, E *__restrict__ db,
+                            E *__restrict__ dh0, int64_t B, int T, int64_t D, int64_t cols_per_row, int a_ti)
+{
+    using V = Vec<E, VEC>;
+    using O = Ops<E>;
+    const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t bi = gid / cols_per_row;
+    const int64_t col = (gid % cols_per_row) * VEC;
+    if (bi >= B) return;
+    const int64_t row0 = bi * T;
+    V lam = vfill<E, VEC>(O::zero());  // conj(abar_{t+1}) lam_{t+1} entering step t
+    if (g_last) lam = *reinterpret_cast<const V *>(g_last + bi * D + col);
+
+    // step r (reversed index), t = T-1-r: needs g_t, a_t (for the carry to t-1), h_{t-1}, done_t
+    V xg[SG], xa[SG], xh[SG], ng[SG], na[SG], nh[SG];
+    uint32_t xd[SG], nd[SG];
+    auto load = [&](int r0, V *pg, V *pa, V *ph, uint32_t *pd) {
+#pragma unroll
+        for (int s = 0; s < SG; ++s) {
+            const int t = T - 1 - (r0 + s);
+            pd[s] = 0u;
+            ph[s] = vfill<E, VEC>(O::zero());
+            if (t >= 0) {
+                const int64_t off = (row0 + t) * D + col;
+                pg[s] = *reinterpret_cast<const V *>(g + off);
+                pa[s] = *reinterpret_cast<const V *>(a + (a_ti ? col : off));
+                if (t > 0) ph[s] = *reinterpret_cast<const V *>(hfw + off - D);
+                else if (h0) ph[s] = *reinterpret_cast<const V *>(h0 + bi * D + col);
+                pd[s] = done_raw(done, done_f32, row0 + t);
+            }
+        }
+    };
+    load(0, xg, xa, xh, xd);
+    for (int r0 = 0; r0 < T; r0 += SG) {
+        if (r0 + SG < T) load(r0 + SG, ng, na, nh, nd);
+#pragma unroll
+        for (int s = 0; s < SG; ++s) {
+            const int t = T - 1 - (r0 + s);
+            if (t >= 0) {
+                const bool dn = done_test(xd[s], done_f32);
+                const int64_t off = (row0 + t) * D + col;
+                V l, o;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    l.v[i] = O::madd(O::one(), xg[s].v[i], lam.v[i]);  // lam_t = g_t + carried term
+                    const E prod = O::mul(l.v[i], O::conj(xh[s].v[i]));
+                    o.v[i] = dn ? O::zero() : prod;
+                    const E nxt = O::mul(O::conj(xa[s].v[i]), l.v[i]);
+                    lam.v[i] = dn ? O::zero() : nxt;               // conj(abar_t) lam_t for step t-1
+                }
+                *reinterpret_cast<V *>(db + off) = l;
+                *reinterpret_cast<V *>(da + off) = o;
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < SG; ++s) { xg[s] = ng[s]; xa[s] = na[s]; xh[s] = nh[s]; xd[s] = nd[s]; }
+    }
+    if (dh0) *reinterpret_cast<V *>(dh0 + bi * D + col) = lam;  // conj(abar_0) lam_0
+}
+
 struct ScanPlan {
     int vec, nw, tiles;
+    bool stream;  // streaming kernel (no time split) instead of the wave-split kernel
 };
 
-// Widest vector the shapes/alignments allow, then the narrowest tile and the
-// smallest time split that put >= ~8 waves on each of the 256 CUs.
-ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, bool al8)
+// Tuned on MI355X (fp32; 512x1024x1024, 1024x128x256, 64x512x512, 32x128x256):
+//  - widest vector the shapes/alignments allow, narrowed until there are >= 2048 wave columns;
+//  - forward: split time over up to 8 waves until ~8192 waves exist (the wave-split kernel at
+//    4 waves reached 5.7 TB/s on the 6.4 GB shape, the streaming kernel 5.1 TB/s); with no
+//    split left to do, stream;
+//  - backward (three loads per step): the streaming kernel wins whenever the columns alone
+//    give >= 2048 waves; below that, the wave-split kernel.
+ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, bool al8, bool bwd)
 {
     const int maxvec = (int)(16 / esize);
     int vec = 1;
@@ -344,18 +482,32 @@ ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, boo
         const bool ok_al = bytes == 16 ? al16 : (bytes == 8 ? al8 : true);
         if (D % v == 0 && ok_al) { vec = v; break; }
     }
-    const int64_t want = 2048;
     auto ntiles = [&](int v) { return (D + 64 * (int64_t)v - 1) / (64 * (int64_t)v); };
-    while (vec > 1 && B * ntiles(vec) < want) vec >>= 1;
+    while (vec > 1 && B * ntiles(vec) < 2048) vec >>= 1;
     const int tiles = (int)ntiles(vec);
+    const int64_t waves = B * tiles;
     int nw = 1;
-    while (nw < 8 && B * tiles * nw < want && (int64_t)nw * TS < T) nw <<= 1;
-    return {vec, nw, tiles};
+    while (nw < 8 && waves * nw < 8192 && (int64_t)nw * TS < T) nw <<= 1;
+    const bool stream = bwd ? waves >= 2048 : nw == 1;
+    return {vec, stream ? 1 : nw, tiles, stream};
 }
 
 size_t scan_smem(int nw, size_t vbytes)
 {
     return nw == 1 ? 0 : 2 * (size_t)nw * 64 * vbytes * 2 + 2 * (size_t)nw * sizeof(int);
+}
+
+// dispatch on the compile-time vector width: f(std::integral_constant<int, VEC>)
+template <typename E, typename F> void vec_switch(int vec, F f)
+{
+    if constexpr (sizeof(E) == 4) {
+        if (vec == 4) f(std::integral_constant<int, 4>{});
+        else if (vec == 2) f(std::integral_constant<int, 2>{});
+        else f(std::integral_constant<int, 1>{});
+    } else {
+        if (vec == 2) f(std::integral_constant<int, 2>{});
+        else f(std::integral_constant<int, 1>{});
+    }
 }
 
 template <typename E>
@@ -367,23 +519,26 @@ int launch_fwd(hipStream_t st, const void *a, const void *b, const void *done,
                       aligned(P0, 16) && aligned(h_last, 16) && aligned(P_last, 16);
     const bool al8 = aligned(a, 8) && aligned(b, 8) && aligned(h, 8) && aligned(h0, 8) &&
                      aligned(P0, 8) && aligned(h_last, 8) && aligned(P_last, 8);
-    const ScanPlan pl = plan_scan(B, T, D, sizeof(E), al16, al8);
-    const dim3 grid((unsigned)(B * pl.tiles)), block(64 * pl.nw);
-    const size_t smem = scan_smem(pl.nw, sizeof(E) * pl.vec);
-#define MRX_LAUNCH(VEC)                                                                   \
-    hipLaunchKernelGGL((diag_scan_fwd_kernel<E, VEC>), grid, block, smem, st,             \
-                       (const E *)a, (const E *)b, done, done_f32, (const E *)h0,         \
-                       (const E *)P0, (E *)h, (E *)h_last, (E *)P_last, (int)T, D,        \
-                       pl.tiles, pl.nw, a_ti)
-    if constexpr (sizeof(E) == 4) {
-        if (pl.vec == 4) MRX_LAUNCH(4);
-        else if (pl.vec == 2) MRX_LAUNCH(2);
-        else MRX_LAUNCH(1);
+    const ScanPlan pl = plan_scan(B, T, D, sizeof(E), al16, al8, false);
+    if (pl.stream) {
+        const int64_t cpr = D / pl.vec;
+        const dim3 grid((unsigned)((B * cpr + 255) / 256)), block(256);
+        vec_switch<E>(pl.vec, [&](auto vc) {
+            constexpr int VEC = decltype(vc)::value;
+            hipLaunchKernelGGL((diag_scan_fwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8)>), grid, block, 0, st,
+                               (const E *)a, (const E *)b, done, done_f32, (const E *)h0, (const E *)P0,
+                               (E *)h, (E *)h_last, (E *)P_last, B, (int)T, D, cpr, a_ti);
+        });
     } else {
-        if (pl.vec == 2) MRX_LAUNCH(2);
-        else MRX_LAUNCH(1);
+        const dim3 grid((unsigned)(B * pl.tiles)), block(64 * pl.nw);
+        const size_t smem = scan_smem(pl.nw, sizeof(E) * pl.vec);
+        vec_switch<E>(pl.vec, [&](auto vc) {
+            constexpr int VEC = decltype(vc)::value;
+            hipLaunchKernelGGL((diag_scan_fwd_kernel<E, VEC>), grid, block, smem, st, (const E *)a,
+                               (const E *)b, done, done_f32, (const E *)h0, (const E *)P0, (E *)h,
+                               (E *)h_last, (E *)P_last, (int)T, D, pl.tiles, pl.nw, a_ti);
+        });
     }
-#undef MRX_LAUNCH
     return launch_status();
 }
 
@@ -396,23 +551,27 @@ int launch_bwd(hipStream_t st, const void *a, const void *h, const void *done,
                       aligned(g_last, 16) && aligned(da, 16) && aligned(db, 16) && aligned(dh0, 16);
     const bool al8 = aligned(a, 8) && aligned(h, 8) && aligned(g, 8) && aligned(h0, 8) &&
                      aligned(g_last, 8) && aligned(da, 8) && aligned(db, 8) && aligned(dh0, 8);
-    const ScanPlan pl = plan_scan(B, T, D, sizeof(E), al16, al8);
-    const dim3 grid((unsigned)(B * pl.tiles)), block(64 * pl.nw);
-    const size_t smem = scan_smem(pl.nw, sizeof(E) * pl.vec);
-#define MRX_LAUNCH(VEC)                                                                   \
-    hipLaunchKernelGGL((diag_scan_bwd_kernel<E, VEC>), grid, block, smem, st,             \
-                       (const E *)a, (const E *)h, done, done_f32, (const E *)h0,         \
-                       (const E *)g, (const E *)g_last, (E *)da, (E *)db, (E *)dh0,       \
-                       (int)T, D, pl.tiles, pl.nw, a_ti)
-    if constexpr (sizeof(E) == 4) {
-        if (pl.vec == 4) MRX_LAUNCH(4);
-        else if (pl.vec == 2) MRX_LAUNCH(2);
-        else MRX_LAUNCH(1);
+    const ScanPlan pl = plan_scan(B, T, D, sizeof(E), al16, al8, true);
+    if (pl.stream) {
+        const int64_t cpr = D / pl.vec;
+        const dim3 grid((unsigned)((B * cpr + 255) / 256)), block(256);
+        vec_switch<E>(pl.vec, [&](auto vc) {
+            constexpr int VEC = decltype(vc)::value;
+            hipLaunchKernelGGL((diag_scan_bwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8)>), grid, block, 0, st,
+                               (const E *)a, (const E *)h, done, done_f32, (const E *)h0, (const E *)g,
+                               (const E *)g_last, (E *)da, (E *)db, (E *)dh0, B, (int)T, D, cpr, a_ti);
+        });
     } else {
-        if (pl.vec == 2) MRX_LAUNCH(2);
-        else MRX_LAUNCH(1);
+        const dim3 grid((unsigned)(B * pl.tiles)), block(64 * pl.nw);
+        const size_t smem = scan_smem(pl.nw, sizeof(E) * pl.vec);
+        vec_switch<E>(pl.vec, [&](auto vc) {
+            constexpr int VEC = decltype(vc)::value;
+            hipLaunchKernelGGL((diag_scan_bwd_kernel<E, VEC>), grid, block, smem, st, (const E *)a,
+                               (const E *)h, done, done_f32, (const E *)h0, (const E *)g,
+                               (const E *)g_last, (E *)da, (E *)db, (E *)dh0, (int)T, D, pl.tiles,
+                               pl.nw, a_ti);
+        });
     }
-#undef MRX_LAUNCH
     return launch_status();
 }
 
