@@ -18,7 +18,8 @@
 //     W = T K, U' = T V - W S^T, dW = -dU' S, Zu = Tm^T dU', Zw = Tm^T dW,
 //     dV = diag(beta) Zu, dK += diag(beta) Zw, dbeta = rowdot(V, Zu) + rowdot(K, Zw),
 //     dT = tril(dW K^T + dU' V^T), dA = -tril((Tm^T dT) T^T, -1),
-//     R = dA K, dbeta += rowdot(K, R), dK += diag(beta) R + (diag(beta) dA)^T K.
+//     R = dA K, dbeta += rowdot(K, R), dK += diag(beta) R + dA^T (diag(beta) K).
+// The products with T are taken as Tm times the row-scaled tiles beta_j K_j, beta_j V_j.
 // Every tile lives in LDS once, in its natural orientation; products that contract over
 // the row index read it through transpose loads (KROW operands).
 #include "chunk_common.h"
@@ -221,13 +222,13 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 }
 
 // =====================================================================================
-// delta rule (bf16, C = 64): twelve 9 KiB regions, reused as operands die; NW waves
+// delta rule (bf16, C = 64): thirteen 9 KiB regions, reused as operands die; NW waves
 // =====================================================================================
 template <typename T, int C, int NW> struct DeltaBwdSmem : BwdDims<T, C> {
     using D = BwdDims<T, C>;
     static constexpr int U = D::szDD;  // every tile type has this size for bf16 / C = 64
     static_assert(D::szRD == U && D::szCC == U && C == HD, "regions assume equal tile sizes");
-        static constexpr int NREG = 12;
+        static constexpr int NREG = 13;
     static constexpr int oBeta = NREG * U, oDb = oBeta + C * 4, total = oDb + 4 * C * 4;
 };
 
@@ -251,12 +252,13 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     // region plan (-> marks reuse once the previous tenant is dead)
     T *sK = reg(0), *sV = reg(1);
     T *sQ = reg(2), *sDT = reg(2);                        // Q[c][dk]  -> dT[a][b]
-    T *sDO = reg(3), *sY1 = reg(3);                       // dO[c][dv] -> Y1[j][b]
+    T *sDO = reg(3), *sY1 = reg(3);                       // dO[c][dv] -> Y1[j][b] beta_b
     T *sS = reg(4), *sDA = reg(4);                        // S[dv][dk] -> dA[i][j]
     T *sDS = reg(5), *sDW = reg(5);                       // dS[dv][dk] -> dW[c][dk]
-    T *sAqk = reg(6), *sDAqk = reg(6), *sG = reg(6);      // Aqk[i][j] -> dAqk[i][j] -> G[i][j]
+    T *sAqk = reg(6), *sDAqk = reg(6);                    // Aqk[i][j] -> dAqk[i][j]
     T *sW = reg(7);                                       // W[c][dk]
-    T *sT = reg(8), *sTm = reg(9), *sU = reg(10), *sDU = reg(11);
+    T *sBK = reg(8), *sBV = reg(9);                       // beta_j K_j, beta_j V_j
+    T *sTm = reg(10), *sU = reg(11), *sDU = reg(12);
     float *sBeta = reinterpret_cast<float *>(smem + L::oBeta);
     float *sDb = reinterpret_cast<float *>(smem + L::oDb);  // [4 feature tiles][C] dbeta partials
 
@@ -282,6 +284,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     typename IO::Regs rq, rk, rv, rdo;
     typename IOS::Regs rS, rTm;
     uint32_t rdone = 0u, rbeta = 0u;  // raw bits, converted when the chunk is staged
+    uint32_t rbrow[IO::PASSES];       // beta of the rows this thread stages
     auto prefetch = [&](int c) {
         const int t0 = c * C;
         IO::load(rq, q + base, rs, t0, Tlen, tid);
@@ -290,6 +293,11 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         IO::load(rdo, dout + base, rs, t0, Tlen, tid);
         IOS::load(rS, S_chk + ((int64_t)bh * NC + c) * HD * HD, HD, 0, HD, tid);
         IOS::load(rTm, Tm_chk + ((int64_t)bh * NC + c) * C * C, C, 0, C, tid);
+#pragma unroll
+        for (int p = 0; p < IO::PASSES; ++p) {
+            const int t = t0 + IO::row_of(tid, p);
+            rbrow[p] = t < Tlen ? load_raw<T>(beta + ((int64_t)b * Tlen + t) * H + h) : 0u;
+        }
         rdone = 0u;
         rbeta = 0u;
         if (lane < C && t0 + lane < Tlen) {
@@ -320,6 +328,13 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 IO::to_lds(fk, sK, LDD, tid);
                 IO::to_lds(fv, sV, LDD, tid);
                 IO::to_lds(fdo, sDO, LDD, tid);
+                float bf[IO::PASSES];
+#pragma unroll
+                for (int p = 0; p < IO::PASSES; ++p) bf[p] = raw_to_float<T>(rbrow[p]);
+                IO::scale_rows(fk, bf);
+                IO::scale_rows(fv, bf);
+                IO::to_lds(fk, sBK, LDD, tid);
+                IO::to_lds(fv, sBV, LDD, tid);
                 typename IOS::Regs fS = rS;
                 if (pass != 0) IOS::zero(fS);
                 IOS::to_lds(fS, sS, LDD, tid);
@@ -332,17 +347,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             MRX_PHASE(11);
             if (pass == 0 && c > 0) prefetch(c - 1);
 
-            // ---- sT[i][j] = Tm[i][j] beta_j (beta of rows outside the pass is 0) -------------
-            for (int idx = tid; idx < C * C / 4; idx += NTHR) {
-                const int i = idx / (C / 4), j = (idx % (C / 4)) * 4;
-                const P4 t = *reinterpret_cast<const P4 *>(sTm + i * LDC + j);
-                *reinterpret_cast<P4 *>(sT + i * LDC + j) =
-                    TT<T>::pack((float)t[0] * sBeta[j], (float)t[1] * sBeta[j + 1], (float)t[2] * sBeta[j + 2],
-                                (float)t[3] * sBeta[j + 3]);
-            }
-            sync_lds();
-            MRX_PHASE(14);
-            // ---- Aqk[i][j] (j <= i) ; W^T[dk][c] = sum_j K[j][dk] T[c][j] -> sW[c][dk] -------
+            // ---- Aqk[i][j] (j <= i) ; W^T[dk][c] = sum_j beta_j K[j][dk] Tm[c][j] -> sW[c][dk] ----
             {
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
@@ -352,17 +357,17 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             {
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
-                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sK, LDD, sT, LDC, w, lane);  // D[m = dk][n = c]
+                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sBK, LDD, sTm, LDC, w, lane);  // D[m = dk][n = c]
                 store_acc<T, HD, C, NW>(acc, sW, LDD, w, lane);
             }
             sync_lds();
             MRX_PHASE(15);
-            // ---- U'^T[dv][c] = sum_j V[j][dv] T[c][j] - sum_dk S[dv][dk] W[c][dk] -> sU[c][dv] ----
+            // ---- U'^T[dv][c] = sum_j beta_j V[j][dv] Tm[c][j] - sum_dk S[dv][dk] W[c][dk] -> sU[c][dv]
             {
                 f32x4 acc[TMR::TPW], acc2[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
                 zero_acc<TMR::TPW>(acc2);
-                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sV, LDD, sT, LDC, w, lane);
+                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sBV, LDD, sTm, LDC, w, lane);
                 gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc2, sS, LDD, sW, LDD, w, lane);
 #pragma unroll
                 for (int j = 0; j < TMR::TPW; ++j) acc[j] -= acc2[j];
@@ -459,28 +464,26 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();
             MRX_PHASE(20);
-            // ---- Y1[j][b] = sum_a Tm[a][j] dT[a][b] : D[m = b][n = j] -> sY1[j][b] ----------------------
+            // ---- Y1[j][b] = beta_b sum_a Tm[a][j] dT[a][b] : D[m = b][n = j] -> sY1[j][b] ---------------
             {
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
                 gemm<T, C, C, C, KROW, KROW, NW>(acc, sDT, LDC, sTm, LDC, w, lane);
-                store_acc<T, C, C, NW>(acc, sY1, LDC, w, lane);
+                store_acc_f<T, C, C, NW>(acc, sY1, LDC, w, lane, [&](int m, int, float x) { return x * sBeta[m]; });
             }
             sync_lds();
             MRX_PHASE(21);
-            // ---- dA[i][j] = -sum_b Y1[i][b] T[j][b], j < i : D[m = j][n = i] -> sDA ; sG = beta_i dA ------
+            // ---- dA[i][j] = -sum_b Y1[i][b] Tm[j][b], j < i : D[m = j][n = i] -> sDA[i][j] --------------
             {
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
-                gemm<T, C, C, C, ROWK, ROWK, NW>(acc, sT, LDC, sY1, LDC, w, lane);
+                gemm<T, C, C, C, ROWK, ROWK, NW>(acc, sTm, LDC, sY1, LDC, w, lane);
                 store_acc_f<T, C, C, NW>(acc, sDA, LDC, w, lane, [](int m, int n, float x) { return m < n ? -x : 0.f; });
-                store_acc_f<T, C, C, NW>(acc, sG, LDC, w, lane,
-                                         [&](int m, int n, float x) { return m < n ? -x * sBeta[n] : 0.f; });
             }
             sync_lds();
             MRX_PHASE(22);
             // ---- R^T[dk][i] = sum_j K[j][dk] dA[i][j] -> dK += beta_i R ; dbeta += K_i . R_i ;
-            //      dK^T[dk][j] += sum_i K[i][dk] G[i][j] -------------------------------------------------
+            //      dK^T[dk][j] += sum_i beta_i K[i][dk] dA[i][j] ------------------------------------------
             {
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
@@ -488,7 +491,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 rowdot(acc, sK);
 #pragma unroll
                 for (int j = 0; j < TMR::TPW; ++j) dKacc[j] += acc[j] * sBeta[TMR::nt(w, j) * 16 + li];
-                gemm<T, HD, C, C, KROW, KROW, NW>(dKacc, sK, LDD, sG, LDC, w, lane);
+                gemm<T, HD, C, C, KROW, KROW, NW>(dKacc, sBK, LDD, sDA, LDC, w, lane);
                 store_rows_global<T, C, NW>(dKacc, dk + base, rs, t0, Tlen, w, lane, one, live);
             }
             // ---- dbeta: reduce the partials over lane groups, then over feature tiles through LDS ----

@@ -230,6 +230,17 @@ template <typename T, int R, int NTHR> struct TileIO {
             }
     }
 
+    // multiply row p of the thread's tile slice by f[p]
+    static __device__ __forceinline__ void scale_rows(Regs &r, const float *f)
+    {
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p)
+#pragma unroll
+            for (int e = 0; e < KP; ++e) r.v[p][e] = (T)((float)r.v[p][e] * f[p]);
+    }
+
+    static __device__ __forceinline__ int row_of(int tid, int p) { return tid / SEGS + p * RPP; }
+
     static __device__ __forceinline__ void zero(Regs &r)
     {
 #pragma unroll
@@ -256,35 +267,43 @@ __device__ __forceinline__ int episode_of(unsigned long long dmask, int r)
     return __popcll(dmask & ((2ull << r) - 1ull));
 }
 
-// ---- inverse of a unit lower-triangular matrix, in place, fp32 -------------------
-// sA holds A (strictly lower part used), C x C with leading dim ld; on return the
-// inverse X of (I + A) is stored as: diagonal 16x16 blocks in place; block (b, c),
-// b > c, in the unused upper position (c, b) (same orientation).  Every wave of the
-// workgroup must call it (contains workgroup barriers); waves >= C/16 only wait.
-template <int C> __device__ __forceinline__ void tri_inverse(float *sA, int ld, int w, int lane)
+// ---- inverse of a unit lower-triangular matrix (fp32 arithmetic) -----------------
+// sA holds A (strictly lower part used), C x C fp32 with leading dim lda.  The inverse
+// X = (I + A)^-1 is written, rounded to T, into the lower triangle (incl. diagonal
+// blocks) of sX[C][ldx]; the blocks above the block diagonal of sX are not touched
+// (the caller zeroes them once).  Every wave of the workgroup must call it (two
+// workgroup barriers inside, none at the end); waves >= C/16 only wait.
+//
+// Stage 1: wave w inverts diagonal block w by repeated squaring, entirely in
+//   registers: with N = -A (N^16 = 0), (I+A)^-1 = (I+N)(I+N^2)(I+N^4)(I+N^8).  A 16x16
+//   product P = X Y on the fp32 MFMA takes X^T and Y both in accumulator layout (lane
+//   (i,g) holds Z[4g+v][i]), so each matrix is carried together with its transpose.
+// Stage 2: wave c computes the whole block column c by forward substitution,
+//   X_bc = -X_bb sum_{k=c}^{b-1} A_bk X_kc ; its own earlier blocks X_kc stay in
+//   registers (the accumulator layout is the B-operand layout), only A_bk and the
+//   diagonal inverses X_bb are read from LDS.
+template <int C, typename T>
+__device__ __forceinline__ void tri_inverse(float *sA, int lda, T *sX, int ldx, int w, int lane)
 {
     constexpr int NB = C / 16;
+    using P4 = typename TT<T>::pack4;
     const int i = lane & 15, g = lane >> 4;
-    if (w < NB) {
-        // Diagonal block w by repeated squaring, entirely in registers.  With N = -A
-        // (nilpotent, N^16 = 0): (I + A)^-1 = (I + N)(I + N^2)(I + N^4)(I + N^8).
-        // A 16x16 product P = X Y on the fp32 MFMA takes X^T and Y both in accumulator
-        // layout (lane (i,g) holds Z[4g+v][i]), so each matrix is carried together with
-        // its transpose and no operand goes through LDS.
-        float *blk = sA + (16 * w) * ld + 16 * w;
-        auto mm = [](const f32x4 &xt, const f32x4 &y, f32x4 c) {
+    auto mm = [](const f32x4 &xt, const f32x4 &y, f32x4 c) {
 #pragma unroll
-            for (int s = 0; s < 4; ++s) c = __builtin_amdgcn_mfma_f32_16x16x4f32(xt[s], y[s], c, 0, 0, 0);
-            return c;
-        };
-        const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < 4; ++s) c = __builtin_amdgcn_mfma_f32_16x16x4f32(xt[s], y[s], c, 0, 0, 0);
+        return c;
+    };
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    f32x4 Xc[NB];  // Xc[r] = X_{c+r, c} in accumulator layout
+    if (w < NB) {
+        float *blk = sA + (16 * w) * lda + 16 * w;
         f32x4 M, Mt, R, Rt;
-        Mt = *reinterpret_cast<const f32x4 *>(blk + i * ld + 4 * g);  // A[i][4g+v] = (A^T)[4g+v][i]
+        Mt = *reinterpret_cast<const f32x4 *>(blk + i * lda + 4 * g);  // A[i][4g+v] = (A^T)[4g+v][i]
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const int r = 4 * g + v;
-            M[v] = (i < r) ? -blk[r * ld + i] : 0.f;   // N[r][i], strictly lower
-            Mt[v] = (r < i) ? -Mt[v] : 0.f;            // N^T[r][i] = N[i][r], strictly upper
+            M[v] = (i < r) ? -blk[r * lda + i] : 0.f;   // N[r][i], strictly lower
+            Mt[v] = (r < i) ? -Mt[v] : 0.f;             // N^T[r][i] = N[i][r], strictly upper
             R[v] = M[v] + (r == i ? 1.f : 0.f);
             Rt[v] = Mt[v] + (r == i ? 1.f : 0.f);
         }
@@ -296,50 +315,37 @@ template <int C> __device__ __forceinline__ void tri_inverse(float *sA, int ld, 
             const f32x4 R2t = mm(M2, Rt, Rt);    // R^T + M2^T R^T
             M = M2; Mt = M2t; R = R2; Rt = R2t;
         }
+        Xc[0] = R;
+        // fp32 copy in place (A-operand of the other waves' products); T-typed copy to sX:
+        // Rt[v] = X[i][4g+v], four consecutive columns of row i
 #pragma unroll
-        for (int v = 0; v < 4; ++v) blk[(4 * g + v) * ld + i] = R[v];
+        for (int v = 0; v < 4; ++v) blk[(4 * g + v) * lda + i] = R[v];
+        *reinterpret_cast<P4 *>(sX + (16 * w + i) * ldx + 16 * w + 4 * g) = TT<T>::pack(Rt[0], Rt[1], Rt[2], Rt[3]);
     }
     sync_lds();
+    if (w < NB) {
+        const int c = w;
 #pragma unroll
-    for (int d = 1; d < NB; ++d) {
-        if (w < NB - d) {
-            const int b = w + d, c = w;  // block (b, c)
-            // tmp = sum_{k=c}^{b-1} A_bk . X_kc ; X_kc lives at rows 16c.., cols 16k.. (the
-            // diagonal block when k == c).  One accumulator per k keeps the MFMA chains short.
-            f32x4 part[NB - 1];
+        for (int r = 1; r < NB; ++r) {
+            const int b = c + r;
+            if (b < NB) {
+                f32x4 part[NB - 1];
 #pragma unroll
-            for (int kk = 0; kk < d; ++kk) {
-                const int k = c + kk;
-                part[kk] = f32x4{0.f, 0.f, 0.f, 0.f};
-                const f32x4 a4 = *reinterpret_cast<const f32x4 *>(sA + (16 * b + i) * ld + 16 * k + 4 * g);
-#pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    const float bop = sA[(16 * c + 4 * g + s) * ld + 16 * k + i];
-                    part[kk] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[s], bop, part[kk], 0, 0, 0);
+                for (int kk = 0; kk < r; ++kk) {  // k = c + kk
+                    const f32x4 a4 = *reinterpret_cast<const f32x4 *>(sA + (16 * b + i) * lda + 16 * (c + kk) + 4 * g);
+                    part[kk] = mm(a4, Xc[kk], zero);
                 }
+                f32x4 tmp = part[0];
+#pragma unroll
+                for (int kk = 1; kk < r; ++kk) tmp += part[kk];
+                const f32x4 d4 = *reinterpret_cast<const f32x4 *>(sA + (16 * b + i) * lda + 16 * b + 4 * g);
+                const f32x4 res = mm(d4, tmp, zero);
+                Xc[r] = -res;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) sX[(16 * b + 4 * g + v) * ldx + 16 * c + i] = (T)Xc[r][v];
             }
-            f32x4 tmp = part[0];
-#pragma unroll
-            for (int kk = 1; kk < d; ++kk) tmp += part[kk];
-            // X_bc = -X_bb . tmp ; the accumulator layout of tmp is already the B-operand layout
-            f32x4 res = {0.f, 0.f, 0.f, 0.f};
-            const f32x4 a4 = *reinterpret_cast<const f32x4 *>(sA + (16 * b + i) * ld + 16 * b + 4 * g);
-#pragma unroll
-            for (int s = 0; s < 4; ++s) res = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[s], tmp[s], res, 0, 0, 0);
-#pragma unroll
-            for (int v = 0; v < 4; ++v) sA[(16 * c + 4 * g + v) * ld + 16 * b + i] = -res[v];
         }
-        sync_lds();
     }
-}
-
-// Element (i, j..j+3) of the inverse stored by tri_inverse (j multiple of 4).
-__device__ __forceinline__ f32x4 tri_inverse_get4(const float *sA, int ld, int i, int j)
-{
-    const int bi = i >> 4, bj = j >> 4;
-    if (bi == bj) return *reinterpret_cast<const f32x4 *>(sA + i * ld + j);
-    if (bi > bj) return *reinterpret_cast<const f32x4 *>(sA + (16 * bj + (i & 15)) * ld + 16 * bi + (j & 15));
-    return f32x4{0.f, 0.f, 0.f, 0.f};
 }
 
 }  // namespace mrx

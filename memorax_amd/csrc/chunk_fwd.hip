@@ -30,15 +30,16 @@ template <typename T, int C, bool DELTA> struct FwdSmem {
     static constexpr int szDD = HD * LDD * sizeof(T);  // [64][64]
     static constexpr int szCC = C * LDC * sizeof(T);   // [C][C]
     static constexpr int szA = DELTA ? C * LDA * 4 : 0;
-    // region A: fp32 A / Tm during the inverse; afterwards Aqk (offset 0) and U' (offset szCC)
-    static constexpr int szAU = DELTA ? szCC + szRD : szCC;
-    static constexpr int szRA = szA > szAU ? szA : szAU;
-    static constexpr int oQ = 0;                 // Q [C][dk], later W [C][dk]
-    static constexpr int oK = oQ + szRD;         // K [C][dk]
-    static constexpr int oV = oK + szRD;         // V [C][dv]
-    static constexpr int oS = oV + szRD;         // S [dv][dk]
-    static constexpr int oT = oS + szDD;         // T [C][C]
-    static constexpr int oA = oT + (DELTA ? szCC : 0);
+    // region A: fp32 A during the inverse; afterwards Aqk (offset 0) and W (offset szCC)
+    static constexpr int szAW = DELTA ? szCC + szRD : szCC;
+    static constexpr int szRA = szA > szAW ? szA : szAW;
+    static constexpr int oQ = 0;                          // Q [C][dk], later U' [C][dv]
+    static constexpr int oK = oQ + szRD;                  // K [C][dk]
+    static constexpr int oV = oK + szRD;                  // V [C][dv]  (delta rule: beta_j V_j)
+    static constexpr int oBK = oV + szRD;                 // beta_j K_j [C][dk]  (delta rule only)
+    static constexpr int oS = oBK + (DELTA ? szRD : 0);   // S [dv][dk]
+    static constexpr int oTm = oS + szDD;                 // Tm [C][C]  (delta rule only)
+    static constexpr int oA = oTm + (DELTA ? szCC : 0);
     static constexpr int oBeta = oA + szRA;
     static constexpr int total = oBeta + C * 4;
 };
@@ -56,14 +57,15 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     constexpr int LDD = L::LDD, LDC = L::LDC, LDA = L::LDA;
     extern __shared__ __align__(16) unsigned char smem[];
     T *sQ = reinterpret_cast<T *>(smem + L::oQ);
-    T *sW = sQ;
     T *sK = reinterpret_cast<T *>(smem + L::oK);
-    T *sV = reinterpret_cast<T *>(smem + L::oV);
+    T *sV = reinterpret_cast<T *>(smem + L::oV);    // delta rule: holds beta_j V_j
+    T *sBK = reinterpret_cast<T *>(smem + L::oBK);
     T *sS = reinterpret_cast<T *>(smem + L::oS);
-    T *sT = reinterpret_cast<T *>(smem + L::oT);
+    T *sTm = reinterpret_cast<T *>(smem + L::oTm);
     float *sA = reinterpret_cast<float *>(smem + L::oA);
     T *sAqk = reinterpret_cast<T *>(smem + L::oA);
-    T *sU = DELTA ? reinterpret_cast<T *>(smem + L::oA + L::szCC) : sV;
+    T *sW = reinterpret_cast<T *>(smem + L::oA + L::szCC);
+    T *sU = DELTA ? sQ : sV;                         // U' [C][dv]
     float *sBeta = reinterpret_cast<float *>(smem + L::oBeta);
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -89,6 +91,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     // register prefetch of the next chunk (raw bits only: no arithmetic on in-flight loads)
     typename IO::Regs rq, rk, rv;
     uint32_t rbeta = 0u, rdone = 0u;
+    uint32_t rbrow[IO::PASSES];  // beta of the rows this thread stages
     auto prefetch = [&](int c) {
         const int t0 = c * C;
         IO::load(rq, q + base, rs, t0, Tlen, tid);
@@ -96,6 +99,13 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         IO::load(rv, v + base, rs, t0, Tlen, tid);
         rdone = 0u;
         rbeta = 0u;
+        if (DELTA) {
+#pragma unroll
+            for (int p = 0; p < IO::PASSES; ++p) {
+                const int t = t0 + IO::row_of(tid, p);
+                rbrow[p] = t < Tlen ? load_raw<T>(beta + ((int64_t)b * Tlen + t) * H + h) : 0u;
+            }
+        }
         if (lane < C && t0 + lane < Tlen) {
             const int64_t bt = (int64_t)b * Tlen + t0 + lane;
             rdone = done_raw(done, done_f32, bt);
@@ -103,6 +113,10 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         }
     };
     prefetch(0);
+    if (DELTA) {
+        // blocks above the block diagonal of Tm are never written again
+        for (int idx = tid; idx < C * LDC * (int)sizeof(T) / 4; idx += NTHR) reinterpret_cast<uint32_t *>(sTm)[idx] = 0u;
+    }
     MRX_PHASE_INIT();
 
     for (int c = 0; c < NC; ++c) {
@@ -123,6 +137,14 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 }
                 IO::to_lds(fq, sQ, LDD, tid);
                 IO::to_lds(fk, sK, LDD, tid);
+                if (DELTA) {
+                    float bf[IO::PASSES];
+#pragma unroll
+                    for (int p = 0; p < IO::PASSES; ++p) bf[p] = raw_to_float<T>(rbrow[p]);
+                    IO::scale_rows(fk, bf);
+                    IO::scale_rows(fv, bf);
+                    IO::to_lds(fk, sBK, LDD, tid);
+                }
                 IO::to_lds(fv, sV, LDD, tid);
             }
             if (DELTA && tid < C) sBeta[tid] = live(tid) ? raw_to_float<T>(rbeta) : 0.f;
@@ -153,24 +175,11 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                                              [&](int m, int n, float x) { return m < n ? sBeta[n] * x : 0.f; });
                 sync_lds();
                 MRX_PHASE(2);
-                tri_inverse<C>(sA, LDA, w, lane);
-                MRX_PHASE(3);
-                // sT[i][j] = Tm[i][j] beta_j
-                for (int idx = tid; idx < C * C / 4; idx += NTHR) {
-                    const int i = idx / (C / 4), j = (idx % (C / 4)) * 4;
-                    const f32x4 t = tri_inverse_get4(sA, LDA, i, j);
-                    *reinterpret_cast<P4 *>(sT + i * LDC + j) =
-                        TT<T>::pack(t[0] * sBeta[j], t[1] * sBeta[j + 1], t[2] * sBeta[j + 2], t[3] * sBeta[j + 3]);
-                    // residual for the backward call: the rows of this pass's episode
-                    // (rows past the end of the sequence count as the last episode: identity rows)
-                    if (Tm_chk && live(i))
-                        *reinterpret_cast<P4 *>(Tm_chk + (((int64_t)bh * NC + c) * C + i) * C + j) =
-                            TT<T>::pack(t[0], t[1], t[2], t[3]);
-                }
+                tri_inverse<C, T>(sA, LDA, sTm, LDC, w, lane);
                 sync_lds();
-                MRX_PHASE(4);
+                MRX_PHASE(3);
             }
-            // ---- Aqk[i][j] = (q_i . k_j), j <= i ; U^T[dv][c] = V^T T^T ---------------------
+            // ---- Aqk[i][j] = (q_i . k_j), j <= i ; delta rule: W = Tm (beta K), U = Tm (beta V) ----
             {
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
@@ -181,19 +190,25 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             if (DELTA) {
                 f32x4 Uacc[TMO::TPW];
                 zero_acc<TMO::TPW>(Uacc);
-                gemm<T, HD, C, C, KROW, ROWK, NW>(Uacc, sV, LDD, sT, LDC, w, lane);
-                sync_lds();  // every wave is done with sQ
-                MRX_PHASE(5);
-                // W^T[dk][c] = K^T T^T -> sW[c][dk]
+                gemm<T, HD, C, C, KROW, ROWK, NW>(Uacc, sV, LDD, sTm, LDC, w, lane);  // U^T[dv][c]
                 {
                     f32x4 acc[TMO::TPW];
                     zero_acc<TMO::TPW>(acc);
-                    gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sK, LDD, sT, LDC, w, lane);
+                    gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sBK, LDD, sTm, LDC, w, lane);  // W^T[dk][c]
                     store_acc<T, HD, C, NW>(acc, sW, LDD, w, lane);
                 }
-                sync_lds();
-                MRX_PHASE(6);
-                // U'^T[dv][c] = U^T - S W^T -> sU[c][dv]
+                if (Tm_chk) {
+                    // residual for the backward call: the rows of this pass's episode (rows past
+                    // the end of the sequence count as the last episode: identity rows)
+                    T *dst = Tm_chk + ((int64_t)bh * NC + c) * C * C;
+                    for (int idx = tid; idx < C * C / 4; idx += NTHR) {
+                        const int i = idx / (C / 4), j = (idx % (C / 4)) * 4;
+                        if (live(i)) *reinterpret_cast<P4 *>(dst + i * C + j) = *reinterpret_cast<const P4 *>(sTm + i * LDC + j);
+                    }
+                }
+                sync_lds();  // sW, sAqk visible; every wave is done with sQ
+                MRX_PHASE(5);
+                // U'^T[dv][c] = U^T - S W^T -> sU[c][dv] (over sQ)
                 {
                     f32x4 acc[TMO::TPW];
                     zero_acc<TMO::TPW>(acc);
