@@ -222,13 +222,14 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 }
 
 // =====================================================================================
-// delta rule (bf16, C = 64): thirteen 9 KiB regions, reused as operands die; NW waves
+// delta rule (bf16, C = 64): fifteen 9 KiB LDS regions (138 KB, one workgroup per CU), a few
+// reused once their first tenant is dead; NW waves
 // =====================================================================================
 template <typename T, int C, int NW> struct DeltaBwdSmem : BwdDims<T, C> {
     using D = BwdDims<T, C>;
     static constexpr int U = D::szDD;  // every tile type has this size for bf16 / C = 64
     static_assert(D::szRD == U && D::szCC == U && C == HD, "regions assume equal tile sizes");
-        static constexpr int NREG = 13;
+        static constexpr int NREG = 15;
     static constexpr int oBeta = NREG * U, oDb = oBeta + C * 4, total = oDb + 4 * C * 4;
 };
 
@@ -251,14 +252,15 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     auto reg = [&](int r) { return reinterpret_cast<T *>(smem + r * L::U); };
     // region plan (-> marks reuse once the previous tenant is dead)
     T *sK = reg(0), *sV = reg(1);
-    T *sQ = reg(2), *sDT = reg(2);                        // Q[c][dk]  -> dT[a][b]
+    T *sQ = reg(2);                                       // Q[c][dk]
     T *sDO = reg(3), *sY1 = reg(3);                       // dO[c][dv] -> Y1[j][b] beta_b
     T *sS = reg(4), *sDA = reg(4);                        // S[dv][dk] -> dA[i][j]
-    T *sDS = reg(5), *sDW = reg(5);                       // dS[dv][dk] -> dW[c][dk]
+    T *sDS = reg(5);                                      // dS[dv][dk]
     T *sAqk = reg(6), *sDAqk = reg(6);                    // Aqk[i][j] -> dAqk[i][j]
     T *sW = reg(7);                                       // W[c][dk]
     T *sBK = reg(8), *sBV = reg(9);                       // beta_j K_j, beta_j V_j
     T *sTm = reg(10), *sU = reg(11), *sDU = reg(12);
+    T *sDW = reg(13), *sDT = reg(14);                     // dW[c][dk], dT[a][b]
     float *sBeta = reinterpret_cast<float *>(smem + L::oBeta);
     float *sDb = reinterpret_cast<float *>(smem + L::oDb);  // [4 feature tiles][C] dbeta partials
 
@@ -390,6 +392,13 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sU, LDD, sDO, LDD, w, lane);  // D[m = j][n = i]
                 store_acc_f<T, C, C, NW>(acc, sDAqk, LDC, w, lane, [](int m, int n, float x) { return m <= n ? x : 0.f; });
             }
+            // ---- dW^T[dk][c] = -sum_dv S[dv][dk] dU'[c][dv] -> sDW[c][dk] -----------------------
+            {
+                f32x4 acc[TMR::TPW];
+                zero_acc<TMR::TPW>(acc);
+                gemm<T, HD, C, HD, KROW, ROWK, NW>(acc, sS, LDD, sDU, LDD, w, lane);
+                store_acc_f<T, HD, C, NW>(acc, sDW, LDD, w, lane, [](int, int, float x) { return -x; });
+            }
             sync_lds();
             MRX_PHASE(17);
             auto one = [](int, int) { return f32x4{1.f, 1.f, 1.f, 1.f}; };
@@ -415,10 +424,6 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                 for (int j = 0; j < TMS::TPW; ++j) dSacc[j] -= acc[j];
             }
-            // ---- dW^T[dk][c] = -sum_dv S[dv][dk] dU'[c][dv] (stored after the barrier: over sDS) ----
-            f32x4 dWacc[TMR::TPW];
-            zero_acc<TMR::TPW>(dWacc);
-            gemm<T, HD, C, HD, KROW, ROWK, NW>(dWacc, sS, LDD, sDU, LDD, w, lane);
             float dbp[TMR::TPW];  // per-lane partial of dbeta for row nt*16 + li
 #pragma unroll
             for (int j = 0; j < TMR::TPW; ++j) dbp[j] = 0.f;
@@ -440,11 +445,6 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 rowdot(acc, sV);
                 store_rows_global<T, C, NW>(acc, dv + base, rs, t0, Tlen, w, lane, beta_of, live);
             }
-            sync_lds();  // sQ, sDO, sDS, sDAqk dead
-            MRX_PHASE(18);
-            store_acc_f<T, HD, C, NW>(dWacc, sDW, LDD, w, lane, [](int, int, float x) { return -x; });
-            sync_lds();
-            MRX_PHASE(19);
             // ---- Zw^T[dk][j] = sum_i dW[i][dk] Tm[i][j] -> dK += beta_j Zw ; dbeta += K_j . Zw_j ------
             {
                 f32x4 acc[TMR::TPW];
@@ -462,7 +462,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sV, LDD, sDU, LDD, w, lane);
                 store_acc_f<T, C, C, NW>(acc, sDT, LDC, w, lane, [](int m, int n, float x) { return m <= n ? x : 0.f; });
             }
-            sync_lds();
+            sync_lds();  // sDT visible; sQ, sDO, sS, sDS, sDAqk dead
             MRX_PHASE(20);
             // ---- Y1[j][b] = beta_b sum_a Tm[a][j] dT[a][b] : D[m = b][n = j] -> sY1[j][b] ---------------
             {
