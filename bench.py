@@ -133,6 +133,7 @@ def main() -> int:
     out["scan"] = bench_scan(torch, K, M, dev)
     if args.all:
         out["linear_attention"] = bench_linear_attention(torch, K, M, dev)
+        out["torso"] = bench_torso(torch, K)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(np, M, x, do_np)
     print(json.dumps(out))
@@ -198,6 +199,50 @@ def bench_linear_attention(torch, K, M, dev):
     res["cfg3_bf16_B32of256_4096x8x64"] = {"ms": ms, "tokens/s": Bn * Tn / ms * 1e3,
                                            "GB/s": 1408 * Bn * Tn * Hn / ms / 1e6}
     return res
+
+
+def bench_torso(torch, K):
+    """Configuration 5: 4 blocks of [RMSNorm -> DeltaNet(H=4, d=64) -> +x ; RMSNorm -> gated
+    linear recurrence -> +x], d_model 256, B=1024 envs x T=128, weights N(0, 0.02), done p=0.01.
+    Reports the whole torso (dense projections in torch included) and the sequence kernels alone."""
+    from memorax_amd import sequence_models as sm
+    B, T, Fe, H, d = 1024, 128, 256, 4, 64
+    torch.manual_seed(5)
+    blocks = []
+    for _ in range(4):
+        blocks += [sm.Residual(sm.PreNorm(sm.Memoroid(sm.DeltaNetCell(Fe, d, H)), Fe)),
+                   sm.Residual(sm.PreNorm(sm.GatedLinearRecurrence(Fe), Fe))]
+    torso = sm.Stack(blocks).cuda()
+    for p in torso.parameters():
+        if p.dim() > 1:
+            torch.nn.init.normal_(p, 0.0, 0.02)
+    x = torch.randn(B, T, Fe, device="cuda")
+    done = torch.rand(B, T, device="cuda") < 0.01
+
+    def full():
+        for p in torso.parameters():
+            p.grad = None
+        _, y = torso(x, done)
+        y.float().pow(2).mean().backward()
+    ms_full = _time_ms(torch, full, iters=5, warm=2)
+
+    bf = torch.bfloat16
+    q, k, v = (torch.randn(B, T, H, d, device="cuda").to(bf) for _ in range(3))
+    k = torch.nn.functional.normalize(k.float(), dim=-1).to(bf)
+    beta = torch.rand(B, T, H, device="cuda").to(bf)
+    do = torch.randn_like(v)
+    a = torch.rand(B, T, Fe, device="cuda") * 0.099 + 0.9
+    bb, g = torch.randn(B, T, Fe, device="cuda"), torch.randn(B, T, Fe, device="cuda")
+
+    def kernels_only():
+        for _ in range(4):
+            o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done)
+            K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False)
+            h, _, _ = K.linear_scan_fwd(a, bb, done, want_P=False)
+            K.linear_scan_bwd(a, h, done, None, g)
+    ms_k = _time_ms(torch, kernels_only, iters=5, warm=2)
+    return {"full_torso_ms": ms_full, "full_torso_tokens/s": B * T / ms_full * 1e3,
+            "sequence_kernels_ms": ms_k, "sequence_kernels_tokens/s": B * T / ms_k * 1e3}
 
 
 def cpu_baseline(np, M, x, do_np):

@@ -192,6 +192,29 @@ class MinGRUCell(_DiagonalCell):
                 torch.zeros(*batch, 1, self.features, device=dev))
 
 
+class GatedLinearRecurrence(SequenceModel):
+    """Gated MLP whose hidden activation is a MinGRU-style diagonal recurrence:
+    y = W_o( scan(a = sigma(-W_z x), b = sigma(W_z x) g(W_h x)) * silu(W_g x) ),
+    i.e. the recurrence of min_gru.py:49-78 inside the gating pattern of the reference's GLU
+    block (blocks/ffn.py:82-123).  Carry = MinGRUCell's (log_state, log_decay)."""
+
+    def __init__(self, features, hidden=None):
+        super().__init__()
+        hidden = features if hidden is None else hidden
+        self.cell = MinGRUCell(hidden, in_features=features)
+        self.gate = nn.Linear(features, hidden, bias=False)
+        self.out = nn.Linear(hidden, features, bias=False)
+
+    def forward(self, inputs, done, initial_carry=None, **kwargs):
+        if initial_carry is None:
+            initial_carry = self.cell.initialize_carry(None, get_input_shape(inputs))
+        h, next_carry = self.cell.scan(self.cell(inputs), initial_carry, done)
+        return next_carry, self.out(h[0] * F.silu(self.gate(inputs)))
+
+    def initialize_carry(self, key, input_shape):
+        return self.cell.initialize_carry(key, input_shape)
+
+
 # ----------------------------------------------------------------------------------
 # matrix-state cells
 # ----------------------------------------------------------------------------------
