@@ -128,8 +128,7 @@ int mrx_delta_rule_fwd(void *stream, const void *q, const void *k,
                        int64_t dv, int dtype, int done_dtype);
 
 /* Gradients w.r.t. q,k,v,beta (in `dtype`) and S0 (fp32, nullable).  S_chk and
- * Tm_chk are the residuals written by mrx_delta_rule_fwd on the same inputs.
- * dtype: MRX_BF16 only (MRX_F32 returns MRX_ERR_UNSUPPORTED). */
+ * Tm_chk are the residuals written by mrx_delta_rule_fwd on the same inputs. */
 int mrx_delta_rule_bwd(void *stream, const void *q, const void *k,
                        const void *v, const void *beta, const void *done,
                        const void *S_chk, const void *Tm_chk, const void *dout,

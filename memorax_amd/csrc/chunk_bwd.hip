@@ -222,15 +222,18 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 }
 
 // =====================================================================================
-// delta rule (bf16, C = 64): fifteen 9 KiB LDS regions (138 KB, one workgroup per CU), a few
-// reused once their first tenant is dead; NW waves
+// delta rule: fifteen LDS tiles (138 KB for bf16 / C = 64, 133 KB for fp32 / C = 32; one
+// workgroup per CU), two of them reused once their first tenant is dead; NW waves
 // =====================================================================================
 template <typename T, int C, int NW> struct DeltaBwdSmem : BwdDims<T, C> {
     using D = BwdDims<T, C>;
-    static constexpr int U = D::szDD;  // every tile type has this size for bf16 / C = 64
-    static_assert(D::szRD == U && D::szCC == U && C == HD, "regions assume equal tile sizes");
-        static constexpr int NREG = 15;
-    static constexpr int oBeta = NREG * U, oDb = oBeta + C * 4, total = oDb + 4 * C * 4;
+    // ten [C][64] tiles, two [64][64], three [C][C]; Y1 and dA reuse the dO and S tiles
+    static_assert(D::szCC <= D::szRD && D::szCC <= D::szDD, "reused regions must hold a [C][C] tile");
+    static constexpr int oK = 0, oV = oK + D::szRD, oQ = oV + D::szRD, oDO = oQ + D::szRD,
+                         oW = oDO + D::szRD, oBK = oW + D::szRD, oBV = oBK + D::szRD, oU = oBV + D::szRD,
+                         oDU = oU + D::szRD, oDW = oDU + D::szRD, oS = oDW + D::szRD, oDS = oS + D::szDD,
+                         oAqk = oDS + D::szDD, oTm = oAqk + D::szCC, oDT = oTm + D::szCC,
+                         oBeta = oDT + D::szCC, oDb = oBeta + C * 4, total = oDb + 4 * C * 4;
 };
 
 template <typename T, int C, int NW>
@@ -246,21 +249,19 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     using L = DeltaBwdSmem<T, C, NW>;
     using IO = TileIO<T, C, NTHR>;
     using IOS = TileIO<T, HD, NTHR>;
+    using IOT = TileIO<T, C, NTHR, C>;  // the [C][C] triangular factor
     using P4 = typename TT<T>::pack4;
     constexpr int LDD = L::LDD, LDC = L::LDC;
     extern __shared__ __align__(16) unsigned char smem[];
-    auto reg = [&](int r) { return reinterpret_cast<T *>(smem + r * L::U); };
-    // region plan (-> marks reuse once the previous tenant is dead)
-    T *sK = reg(0), *sV = reg(1);
-    T *sQ = reg(2);                                       // Q[c][dk]
-    T *sDO = reg(3), *sY1 = reg(3);                       // dO[c][dv] -> Y1[j][b] beta_b
-    T *sS = reg(4), *sDA = reg(4);                        // S[dv][dk] -> dA[i][j]
-    T *sDS = reg(5);                                      // dS[dv][dk]
-    T *sAqk = reg(6), *sDAqk = reg(6);                    // Aqk[i][j] -> dAqk[i][j]
-    T *sW = reg(7);                                       // W[c][dk]
-    T *sBK = reg(8), *sBV = reg(9);                       // beta_j K_j, beta_j V_j
-    T *sTm = reg(10), *sU = reg(11), *sDU = reg(12);
-    T *sDW = reg(13), *sDT = reg(14);                     // dW[c][dk], dT[a][b]
+    auto at = [&](int off) { return reinterpret_cast<T *>(smem + off); };
+    T *sK = at(L::oK), *sV = at(L::oV), *sQ = at(L::oQ), *sW = at(L::oW);
+    T *sBK = at(L::oBK), *sBV = at(L::oBV);               // beta_j K_j, beta_j V_j
+    T *sU = at(L::oU), *sDU = at(L::oDU), *sDW = at(L::oDW);
+    T *sDO = at(L::oDO), *sY1 = at(L::oDO);               // dO[c][dv] -> Y1[j][b] beta_b
+    T *sS = at(L::oS), *sDA = at(L::oS);                  // S[dv][dk] -> dA[i][j]
+    T *sDS = at(L::oDS);                                  // dS[dv][dk]
+    T *sAqk = at(L::oAqk), *sDAqk = at(L::oAqk);          // Aqk[i][j] -> dAqk[i][j]
+    T *sTm = at(L::oTm), *sDT = at(L::oDT);               // Tm[i][j], dT[a][b]
     float *sBeta = reinterpret_cast<float *>(smem + L::oBeta);
     float *sDb = reinterpret_cast<float *>(smem + L::oDb);  // [4 feature tiles][C] dbeta partials
 
@@ -284,7 +285,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     }
 
     typename IO::Regs rq, rk, rv, rdo;
-    typename IOS::Regs rS, rTm;
+    typename IOS::Regs rS;
+    typename IOT::Regs rTm;
     uint32_t rdone = 0u, rbeta = 0u;  // raw bits, converted when the chunk is staged
     uint32_t rbrow[IO::PASSES];       // beta of the rows this thread stages
     auto prefetch = [&](int c) {
@@ -294,7 +296,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         IO::load(rv, v + base, rs, t0, Tlen, tid);
         IO::load(rdo, dout + base, rs, t0, Tlen, tid);
         IOS::load(rS, S_chk + ((int64_t)bh * NC + c) * HD * HD, HD, 0, HD, tid);
-        IOS::load(rTm, Tm_chk + ((int64_t)bh * NC + c) * C * C, C, 0, C, tid);
+        IOT::load(rTm, Tm_chk + ((int64_t)bh * NC + c) * C * C, C, 0, C, tid);
 #pragma unroll
         for (int p = 0; p < IO::PASSES; ++p) {
             const int t = t0 + IO::row_of(tid, p);
@@ -340,7 +342,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 typename IOS::Regs fS = rS;
                 if (pass != 0) IOS::zero(fS);
                 IOS::to_lds(fS, sS, LDD, tid);
-                IOS::to_lds(rTm, sTm, LDC, tid);  // Tm[i][j] from the forward call (block diagonal by episode)
+                IOT::to_lds(rTm, sTm, LDC, tid);  // Tm[i][j] from the forward call (block diagonal by episode)
             }
             if (tid < C) sBeta[tid] = live(tid) ? raw_to_float<T>(rbeta) : 0.f;
             if (pass != nres) zero_acc<TMS::TPW>(dSacc);
@@ -597,17 +599,29 @@ extern "C" int mrx_delta_rule_bwd(void *stream, const void *q, const void *k, co
                              dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
     if (!beta || !dbeta || !Tm_chk || !aligned(Tm_chk, 16)) return MRX_ERR_INVALID_ARG;
-    if (dtype != MRX_BF16) return MRX_ERR_UNSUPPORTED;  // fp32 delta-rule backward: not built yet
     hipStream_t st = (hipStream_t)stream;
-    constexpr int NW = MRX_DELTA_BWD_WAVES;
-    auto kern = delta_bwd_kernel<__bf16, 64, NW>;
-    constexpr int smem = DeltaBwdSmem<__bf16, 64, NW>::total;
-    static bool attr_set = false;
-    if (set_smem(kern, smem, attr_set) != MRX_OK) return MRX_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(64 * NW), smem, st, (const __bf16 *)q,
-                       (const __bf16 *)k, (const __bf16 *)v, (const __bf16 *)beta, done, done_dtype,
-                       (const __bf16 *)S_chk, (const __bf16 *)Tm_chk, (const __bf16 *)dout, (const float *)dS_last,
-                       (__bf16 *)dq, (__bf16 *)dk_out, (__bf16 *)dv_out, (__bf16 *)dbeta, (float *)dS0,
-                       (int)T, (int)H);
+    if (dtype == MRX_BF16) {
+        constexpr int NW = MRX_DELTA_BWD_WAVES;
+        auto kern = delta_bwd_kernel<__bf16, 64, NW>;
+        constexpr int smem = DeltaBwdSmem<__bf16, 64, NW>::total;
+        static bool attr_set = false;
+        if (set_smem(kern, smem, attr_set) != MRX_OK) return MRX_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(64 * NW), smem, st, (const __bf16 *)q,
+                           (const __bf16 *)k, (const __bf16 *)v, (const __bf16 *)beta, done, done_dtype,
+                           (const __bf16 *)S_chk, (const __bf16 *)Tm_chk, (const __bf16 *)dout,
+                           (const float *)dS_last, (__bf16 *)dq, (__bf16 *)dk_out, (__bf16 *)dv_out,
+                           (__bf16 *)dbeta, (float *)dS0, (int)T, (int)H);
+    } else {
+        constexpr int NW = 4;
+        auto kern = delta_bwd_kernel<float, 32, NW>;
+        constexpr int smem = DeltaBwdSmem<float, 32, NW>::total;
+        static bool attr_set = false;
+        if (set_smem(kern, smem, attr_set) != MRX_OK) return MRX_ERR_LAUNCH;
+        hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(64 * NW), smem, st, (const float *)q,
+                           (const float *)k, (const float *)v, (const float *)beta, done, done_dtype,
+                           (const float *)S_chk, (const float *)Tm_chk, (const float *)dout,
+                           (const float *)dS_last, (float *)dq, (float *)dk_out, (float *)dv_out,
+                           (float *)dbeta, (float *)dS0, (int)T, (int)H);
+    }
     return launch_status();
 }

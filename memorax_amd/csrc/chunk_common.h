@@ -179,12 +179,12 @@ template <> __device__ __forceinline__ float raw_to_float<float>(uint32_t raw) {
 
 __device__ __forceinline__ float elu1(float x) { return x > 0.f ? x + 1.f : __expf(x); }
 
-// ---- global <-> register <-> LDS movement of one [R][64] tile --------------------
-// A tile is R rows of 64 T = R * SEGS 16-byte segments; thread tid owns segment
+// ---- global <-> register <-> LDS movement of one [R][COLS] tile ------------------
+// A tile is R rows of COLS T = R * SEGS 16-byte segments; thread tid owns segment
 // (tid % SEGS) of rows (tid / SEGS) + p * RPP, p = 0..PASSES-1.
-template <typename T, int R, int NTHR> struct TileIO {
+template <typename T, int R, int NTHR, int COLS = HD> struct TileIO {
     static constexpr int KP = TT<T>::KP;
-    static constexpr int SEGS = HD / KP;
+    static constexpr int SEGS = COLS / KP;
     static constexpr int RPP = NTHR / SEGS;
     static constexpr int PASSES = R / RPP;
     static_assert(PASSES >= 1 && R % RPP == 0, "tile rows must be a multiple of rows per pass");
@@ -193,7 +193,7 @@ template <typename T, int R, int NTHR> struct TileIO {
         F v[PASSES];
     };
 
-    // rows t0.. of a (B,T,H,64) array whose (b,h) base pointer is `base`; rows >= Tlen read as 0
+    // rows t0.. of an array with COLS-wide rows `row_stride` apart starting at `base`; rows >= Tlen read as 0
     static __device__ __forceinline__ void load(Regs &r, const T *base, int64_t row_stride, int t0,
                                                 int Tlen, int tid)
     {

@@ -47,31 +47,41 @@ def test_linear_attention_bwd(shape, p, dtype, fmap):
 
 @pytest.mark.parametrize("shape", SHAPES)
 @pytest.mark.parametrize("p", [0.0, 0.05])
-def test_delta_rule_bwd_bf16(shape, p):
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_delta_rule_bwd(shape, p, dtype):
     from memorax_amd import kernels as K
     B, T, H = shape
     x = attn_inputs(B, T, H, p=p, seed=B * 100 + T + H + 57, delta=True)
     rng = np.random.default_rng(T + 1)
-    do = bf16_round(rng.standard_normal((B, T, H, 64)).astype(np.float32))
+    do = rng.standard_normal((B, T, H, 64)).astype(np.float32)
     dSl = (rng.standard_normal((B, H, 64, 64)) * 0.1).astype(np.float32)
-    print(f"case delta_bwd shape={shape} p={p}", flush=True)
-    for n in ("q", "k", "v", "beta"):
-        x[n] = bf16_round(x[n])
-    bf = torch.bfloat16
-    tq, tk, tv, tb, tdo = (dev(a, bf) for a in (x["q"], x["k"], x["v"], x["beta"], do))
+    print(f"case delta_bwd shape={shape} p={p} dtype={dtype}", flush=True)
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    if dtype == "bf16":
+        do = bf16_round(do)
+        for n in ("q", "k", "v", "beta"):
+            x[n] = bf16_round(x[n])
+    tq, tk, tv, tb, tdo = (dev(a, td) for a in (x["q"], x["k"], x["v"], x["beta"], do))
     o, Sl, chk = K.delta_rule_fwd(tq, tk, tv, tb, dev(x["done"]), dev(x["S0"]))
     got = K.delta_rule_bwd(tq, tk, tv, tb, dev(x["done"]), chk, tdo, dev(dSl))
     ref = G.delta_rule_grads(x["q"], x["k"], x["v"], x["beta"], x["done"], x["S0"], do, dSl)
-    _check(got, ref, TOL_BF16, ("dq", "dk", "dv", "dbeta", "dS0"))
+    _check(got, ref, TOL_BF16 if dtype == "bf16" else TOL_F32, ("dq", "dk", "dv", "dbeta", "dS0"))
 
 
-def test_delta_rule_bwd_fp32_reports_unsupported():
+@pytest.mark.parametrize("done_dtype", ["uint8", "float32"])
+def test_chunk_kernels_done_dtypes(done_dtype):
+    """done as uint8 or float32 (memoroid.py:67 casts it to float) gives identical results."""
     from memorax_amd import kernels as K
-    x = attn_inputs(1, 32, 1, seed=1, delta=True)
+    x = attn_inputs(2, 130, 2, p=0.04, seed=11, delta=True)
     args = [dev(x[n]) for n in ("q", "k", "v", "beta")]
-    o, Sl, chk = K.delta_rule_fwd(*args, dev(x["done"]))
-    with pytest.raises(RuntimeError, match="unsupported"):
-        K.delta_rule_bwd(*args, dev(x["done"]), chk, torch.zeros_like(o))
+    ref = K.delta_rule_fwd(*args, dev(x["done"]))
+    dd = x["done"].astype(np.uint8) if done_dtype == "uint8" else x["done"].astype(np.float32) * 3.5
+    got = K.delta_rule_fwd(*args, dev(dd))
+    assert torch.equal(got[0], ref[0]) and torch.equal(got[1], ref[1])
+    do = torch.ones_like(ref[0])
+    g1 = K.delta_rule_bwd(*args, dev(x["done"]), ref[2], do)
+    g2 = K.delta_rule_bwd(*args, dev(dd), got[2], do)
+    assert all(torch.equal(a, b) for a, b in zip(g1, g2))
 
 
 def test_bwd_reset_isolation():
