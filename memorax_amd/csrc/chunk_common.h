@@ -268,82 +268,88 @@ __device__ __forceinline__ int episode_of(unsigned long long dmask, int r)
 }
 
 // ---- inverse of a unit lower-triangular matrix (fp32 arithmetic) -----------------
-// sA holds A (strictly lower part used), C x C fp32 with leading dim lda.  The inverse
-// X = (I + A)^-1 is written, rounded to T, into the lower triangle (incl. diagonal
-// blocks) of sX[C][ldx]; the blocks above the block diagonal of sX are not touched
-// (the caller zeroes them once).  Every wave of the workgroup must call it (two
-// workgroup barriers inside, none at the end); waves >= C/16 only wait.
+// X = (I + A)^-1 for A = tril(diag(beta) K K^T, -1), C x C, in 16x16 blocks.
 //
-// Stage 1: wave w inverts diagonal block w by repeated squaring, entirely in
-//   registers: with N = -A (N^16 = 0), (I+A)^-1 = (I+N)(I+N^2)(I+N^4)(I+N^8).  A 16x16
-//   product P = X Y on the fp32 MFMA takes X^T and Y both in accumulator layout (lane
-//   (i,g) holds Z[4g+v][i]), so each matrix is carried together with its transpose.
-// Stage 2: wave c computes the whole block column c by forward substitution,
-//   X_bc = -X_bb sum_{k=c}^{b-1} A_bk X_kc ; its own earlier blocks X_kc stay in
-//   registers (the accumulator layout is the B-operand layout), only A_bk and the
-//   diagonal inverses X_bb are read from LDS.
-template <int C, typename T>
-__device__ __forceinline__ void tri_inverse(float *sA, int lda, T *sX, int ldx, int w, int lane)
+// tri_diag_block: the wave that owns the accumulator tile (b, b) of K K^T inverts
+//   diagonal block b straight from those registers by repeated squaring: with N = -A_bb
+//   (N^16 = 0), (I+A_bb)^-1 = (I+N)(I+N^2)(I+N^4)(I+N^8).  A 16x16 product P = X Y on the
+//   fp32 MFMA takes X^T and Y both in accumulator layout (lane (i,g) holds Z[4g+v][i]),
+//   so each matrix is carried together with its transpose and nothing goes through LDS.
+//   The result is written as fp32 into the diagonal block of sA (A-operand of other
+//   waves) and, rounded to T, into sX; it is also returned in accumulator layout.
+// tri_block_column: after a workgroup barrier, the same wave computes the rest of block
+//   column c by forward substitution, X_bc = -X_bb sum_{k=c}^{b-1} A_bk X_kc; its own
+//   earlier blocks stay in registers (the accumulator layout is the B-operand layout),
+//   only A_bk (strictly lower blocks of sA) and the diagonal inverses are read from LDS.
+// Blocks above the block diagonal of sX are never written (the caller zeroes them once).
+__device__ __forceinline__ f32x4 mm16(const f32x4 &xt, const f32x4 &y, f32x4 c)
 {
-    constexpr int NB = C / 16;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) c = __builtin_amdgcn_mfma_f32_16x16x4f32(xt[s], y[s], c, 0, 0, 0);
+    return c;
+}
+
+// kk[v] = (K K^T)[16b + i][16b + 4g + v] (symmetric); sBeta indexed by chunk row
+template <typename T>
+__device__ __forceinline__ f32x4 tri_diag_block(const f32x4 &kk, const float *sBeta, int b, float *sA, int lda,
+                                                T *sX, int ldx, int lane)
+{
     using P4 = typename TT<T>::pack4;
     const int i = lane & 15, g = lane >> 4;
-    auto mm = [](const f32x4 &xt, const f32x4 &y, f32x4 c) {
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    const float beta_i = sBeta[16 * b + i];
+    const f32x4 beta_r = *reinterpret_cast<const f32x4 *>(sBeta + 16 * b + 4 * g);
+    f32x4 M, Mt, R, Rt;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) c = __builtin_amdgcn_mfma_f32_16x16x4f32(xt[s], y[s], c, 0, 0, 0);
-        return c;
-    };
+    for (int v = 0; v < 4; ++v) {
+        const int r = 4 * g + v;
+        M[v] = (i < r) ? -beta_r[v] * kk[v] : 0.f;   // N[r][i] = -beta_r KK[r][i], strictly lower
+        Mt[v] = (r < i) ? -beta_i * kk[v] : 0.f;     // N^T[r][i] = N[i][r] = -beta_i KK[i][r]
+        R[v] = M[v] + (r == i ? 1.f : 0.f);
+        Rt[v] = Mt[v] + (r == i ? 1.f : 0.f);
+    }
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        const f32x4 M2 = mm16(Mt, M, zero);    // N^2  : X = M,  Y = M
+        const f32x4 M2t = mm16(M, Mt, zero);   // (N^2)^T = M^T M^T
+        const f32x4 R2 = mm16(Rt, M2, R);      // R + R M2
+        const f32x4 R2t = mm16(M2, Rt, Rt);    // R^T + M2^T R^T
+        M = M2; Mt = M2t; R = R2; Rt = R2t;
+    }
+    float *blk = sA + (16 * b) * lda + 16 * b;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) blk[(4 * g + v) * lda + i] = R[v];
+    // Rt[v] = X[i][4g+v]: four consecutive columns of row i
+    *reinterpret_cast<P4 *>(sX + (16 * b + i) * ldx + 16 * b + 4 * g) = TT<T>::pack(Rt[0], Rt[1], Rt[2], Rt[3]);
+    return R;
+}
+
+template <int C, typename T>
+__device__ __forceinline__ void tri_block_column(const float *sA, int lda, T *sX, int ldx, int c, const f32x4 &Xcc,
+                                                 int lane)
+{
+    constexpr int NB = C / 16;
+    const int i = lane & 15, g = lane >> 4;
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
     f32x4 Xc[NB];  // Xc[r] = X_{c+r, c} in accumulator layout
-    if (w < NB) {
-        float *blk = sA + (16 * w) * lda + 16 * w;
-        f32x4 M, Mt, R, Rt;
-        Mt = *reinterpret_cast<const f32x4 *>(blk + i * lda + 4 * g);  // A[i][4g+v] = (A^T)[4g+v][i]
+    Xc[0] = Xcc;
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            const int r = 4 * g + v;
-            M[v] = (i < r) ? -blk[r * lda + i] : 0.f;   // N[r][i], strictly lower
-            Mt[v] = (r < i) ? -Mt[v] : 0.f;             // N^T[r][i] = N[i][r], strictly upper
-            R[v] = M[v] + (r == i ? 1.f : 0.f);
-            Rt[v] = Mt[v] + (r == i ? 1.f : 0.f);
-        }
+    for (int r = 1; r < NB; ++r) {
+        const int b = c + r;
+        if (b < NB) {
+            f32x4 part[NB - 1];
 #pragma unroll
-        for (int k = 0; k < 3; ++k) {
-            const f32x4 M2 = mm(Mt, M, zero);    // N^2  : X = M,  Y = M
-            const f32x4 M2t = mm(M, Mt, zero);   // (N^2)^T = M^T M^T : X = M^T, Y = M^T
-            const f32x4 R2 = mm(Rt, M2, R);      // R + R M2
-            const f32x4 R2t = mm(M2, Rt, Rt);    // R^T + M2^T R^T
-            M = M2; Mt = M2t; R = R2; Rt = R2t;
-        }
-        Xc[0] = R;
-        // fp32 copy in place (A-operand of the other waves' products); T-typed copy to sX:
-        // Rt[v] = X[i][4g+v], four consecutive columns of row i
-#pragma unroll
-        for (int v = 0; v < 4; ++v) blk[(4 * g + v) * lda + i] = R[v];
-        *reinterpret_cast<P4 *>(sX + (16 * w + i) * ldx + 16 * w + 4 * g) = TT<T>::pack(Rt[0], Rt[1], Rt[2], Rt[3]);
-    }
-    sync_lds();
-    if (w < NB) {
-        const int c = w;
-#pragma unroll
-        for (int r = 1; r < NB; ++r) {
-            const int b = c + r;
-            if (b < NB) {
-                f32x4 part[NB - 1];
-#pragma unroll
-                for (int kk = 0; kk < r; ++kk) {  // k = c + kk
-                    const f32x4 a4 = *reinterpret_cast<const f32x4 *>(sA + (16 * b + i) * lda + 16 * (c + kk) + 4 * g);
-                    part[kk] = mm(a4, Xc[kk], zero);
-                }
-                f32x4 tmp = part[0];
-#pragma unroll
-                for (int kk = 1; kk < r; ++kk) tmp += part[kk];
-                const f32x4 d4 = *reinterpret_cast<const f32x4 *>(sA + (16 * b + i) * lda + 16 * b + 4 * g);
-                const f32x4 res = mm(d4, tmp, zero);
-                Xc[r] = -res;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) sX[(16 * b + 4 * g + v) * ldx + 16 * c + i] = (T)Xc[r][v];
+            for (int kk = 0; kk < r; ++kk) {  // k = c + kk
+                const f32x4 a4 = *reinterpret_cast<const f32x4 *>(sA + (16 * b + i) * lda + 16 * (c + kk) + 4 * g);
+                part[kk] = mm16(a4, Xc[kk], zero);
             }
+            f32x4 tmp = part[0];
+#pragma unroll
+            for (int kk = 1; kk < r; ++kk) tmp += part[kk];
+            const f32x4 d4 = *reinterpret_cast<const f32x4 *>(sA + (16 * b + i) * lda + 16 * b + 4 * g);
+            Xc[r] = -mm16(d4, tmp, zero);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) sX[(16 * b + 4 * g + v) * ldx + 16 * c + i] = (T)Xc[r][v];
         }
     }
 }

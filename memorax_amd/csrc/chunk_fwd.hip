@@ -173,9 +173,17 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sK, LDD, sK, LDD, w, lane);  // D[m = j][n = i]
                 store_acc_f<float, C, C, NW>(acc, sA, LDA, w, lane,
                                              [&](int m, int n, float x) { return m < n ? sBeta[n] * x : 0.f; });
+                // the wave that holds the diagonal tile (b, b) inverts that block from registers
+                int diag = -1;
+                f32x4 kk = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < TMA::TPW; ++j)
+                    if (TMA::nt(w, j) == TMA::mt(w)) { diag = TMA::mt(w); kk = acc[j]; }
+                f32x4 Xcc = {0.f, 0.f, 0.f, 0.f};
+                if (diag >= 0) Xcc = tri_diag_block<T>(kk, sBeta, diag, sA, LDA, sTm, LDC, lane);
                 sync_lds();
                 MRX_PHASE(2);
-                tri_inverse<C, T>(sA, LDA, sTm, LDC, w, lane);
+                if (diag >= 0) tri_block_column<C, T>(sA, LDA, sTm, LDC, diag, Xcc, lane);
                 sync_lds();
                 MRX_PHASE(3);
             }
