@@ -514,6 +514,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             MRX_PHASE(24);
         }
     }
+    MRX_PHASE_FLUSH();
     if (dS0) {
 #pragma unroll
         for (int j = 0; j < TMS::TPW; ++j) {

@@ -171,8 +171,16 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
                 gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sK, LDD, sK, LDD, w, lane);  // D[m = j][n = i]
-                store_acc_f<float, C, C, NW>(acc, sA, LDA, w, lane,
-                                             [&](int m, int n, float x) { return m < n ? sBeta[n] * x : 0.f; });
+                // sA[i][j] = beta_i (k_i . k_j) for j < i, else 0 (beta read once per tile, then selects)
+#pragma unroll
+                for (int j = 0; j < TMA::TPW; ++j) {
+                    const int m = TMA::mt(w) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
+                    const float bn = sBeta[n];
+                    f32x4 a;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) a[e] = (m + e < n) ? bn * acc[j][e] : 0.f;
+                    *reinterpret_cast<f32x4 *>(sA + n * LDA + m) = a;
+                }
                 // the wave that holds the diagonal tile (b, b) inverts that block from registers
                 int diag = -1;
                 f32x4 kk = {0.f, 0.f, 0.f, 0.f};
@@ -244,6 +252,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         }
     }
     MRX_WG_END();
+    MRX_PHASE_FLUSH();
 
     if (S_last) {
 #pragma unroll

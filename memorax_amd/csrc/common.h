@@ -41,7 +41,7 @@ inline bool aligned(const void *p, size_t n)
 
 // Phase timing for kernel tuning: compiled in only with -DMRX_PHASE_TIMING (never in
 // the shipped library).  Workgroup 0 / thread 0 accumulates the shader-clock ticks
-// spent between consecutive MRX_PHASE marks into mrx_phase_ticks[].
+// spent between consecutive MRX_PHASE marks; MRX_PHASE_FLUSH adds them to mrx_phase_ticks[].
 #ifdef MRX_PHASE_TIMING
 extern __device__ unsigned long long mrx_phase_ticks[64];
 extern __device__ unsigned long long mrx_wg_trace[4096 * 3];
@@ -57,18 +57,28 @@ extern __device__ unsigned long long mrx_wg_trace[4096 * 3];
     do {                                                                                  \
         if (threadIdx.x == 0 && blockIdx.x < 4096) mrx_wg_trace[blockIdx.x * 3 + 1] = wall_clock64(); \
     } while (0)
-#define MRX_PHASE_INIT() unsigned long long mrx_t_last = clock64()
+// marks accumulate in LDS (fire-and-forget ds_add) so that a mark never waits on global memory
+#define MRX_PHASE_INIT()                                                    \
+    __shared__ unsigned long long mrx_lds_ticks[64];                        \
+    if (threadIdx.x < 64) mrx_lds_ticks[threadIdx.x] = 0;                   \
+    unsigned long long mrx_t_last = clock64()
 #define MRX_PHASE(i)                                                        \
     do {                                                                    \
         if (blockIdx.x == 0 && threadIdx.x == 0) {                          \
             const unsigned long long mrx_t_now = clock64();                 \
-            mrx_phase_ticks[i] += mrx_t_now - mrx_t_last;                   \
+            __hip_atomic_fetch_add(&mrx_lds_ticks[i], mrx_t_now - mrx_t_last, __ATOMIC_RELAXED, \
+                                   __HIP_MEMORY_SCOPE_WORKGROUP);           \
             mrx_t_last = mrx_t_now;                                         \
         }                                                                   \
+    } while (0)
+#define MRX_PHASE_FLUSH()                                                   \
+    do {                                                                    \
+        if (blockIdx.x == 0 && threadIdx.x < 64) mrx_phase_ticks[threadIdx.x] += mrx_lds_ticks[threadIdx.x]; \
     } while (0)
 #else
 #define MRX_WG_BEGIN() do { } while (0)
 #define MRX_WG_END() do { } while (0)
 #define MRX_PHASE_INIT() do { } while (0)
 #define MRX_PHASE(i) do { } while (0)
+#define MRX_PHASE_FLUSH() do { } while (0)
 #endif
