@@ -92,34 +92,53 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     typename IO::Regs rq, rk, rv;
     uint32_t rbeta = 0u, rdone = 0u;
     uint32_t rbrow[IO::PASSES];  // beta of the rows this thread stages
-    auto prefetch = [&](int c) {
-        const int t0 = c * C;
-        IO::load(rq, q + base, rs, t0, Tlen, tid);
-        IO::load(rk, k + base, rs, t0, Tlen, tid);
-        IO::load(rv, v + base, rs, t0, Tlen, tid);
+    // Element offsets of what this thread loads for the chunk about to be prefetched; they advance
+    // by one chunk per call (64-bit adds instead of per-chunk index multiplications).
+    int64_t roff[IO::PASSES], boff[IO::PASSES];
+#pragma unroll
+    for (int p = 0; p < IO::PASSES; ++p) {
+        const int r = IO::row_of(tid, p);
+        roff[p] = base + (int64_t)r * rs + (tid % IO::SEGS) * IO::KP;  // q/k/v: row r, this thread's 16-byte segment
+        boff[p] = ((int64_t)b * Tlen + r) * H + h;                     // beta of row r
+    }
+    int64_t doff = (int64_t)b * Tlen + lane;  // done of chunk row `lane`
+    int tpre = 0;                             // first time step of the chunk about to be prefetched
+    auto prefetch = [&]() {
+        typename IO::F z;
+#pragma unroll
+        for (int e = 0; e < IO::KP; ++e) z[e] = (T)0.f;
+#pragma unroll
+        for (int p = 0; p < IO::PASSES; ++p) {
+            const bool in = tpre + IO::row_of(tid, p) < Tlen;
+            rq.v[p] = in ? *reinterpret_cast<const typename IO::F *>(q + roff[p]) : z;
+            rk.v[p] = in ? *reinterpret_cast<const typename IO::F *>(k + roff[p]) : z;
+            rv.v[p] = in ? *reinterpret_cast<const typename IO::F *>(v + roff[p]) : z;
+            if (DELTA) rbrow[p] = in ? load_raw<T>(beta + boff[p]) : 0u;
+            roff[p] += (int64_t)C * rs;
+            boff[p] += (int64_t)C * H;
+        }
         rdone = 0u;
         rbeta = 0u;
-        if (DELTA) {
-#pragma unroll
-            for (int p = 0; p < IO::PASSES; ++p) {
-                const int t = t0 + IO::row_of(tid, p);
-                rbrow[p] = t < Tlen ? load_raw<T>(beta + ((int64_t)b * Tlen + t) * H + h) : 0u;
-            }
+        if (lane < C && tpre + lane < Tlen) {
+            rdone = done_raw(done, done_f32, doff);
+            if (DELTA && w == 0) rbeta = load_raw<T>(beta + doff * H + h);
         }
-        if (lane < C && t0 + lane < Tlen) {
-            const int64_t bt = (int64_t)b * Tlen + t0 + lane;
-            rdone = done_raw(done, done_f32, bt);
-            if (DELTA && w == 0) rbeta = load_raw<T>(beta + bt * H + h);
-        }
+        doff += C;
+        tpre += C;
     };
-    prefetch(0);
+    prefetch();
     if (DELTA) {
         // blocks above the block diagonal of Tm are never written again
         for (int idx = tid; idx < C * LDC * (int)sizeof(T) / 4; idx += NTHR) reinterpret_cast<uint32_t *>(sTm)[idx] = 0u;
     }
     MRX_PHASE_INIT();
 
-    for (int c = 0; c < NC; ++c) {
+    static_assert(C * C / 4 % NTHR == 0, "Tm tile copy assumes whole passes");
+    // running element offsets of this thread's stores, advanced by one chunk per iteration
+    int64_t o_off = base + (int64_t)li * rs + TMO::mt(w) * 16 + 4 * lg;                              // o[t0 + li][dv0..]
+    int64_t schk_off = (int64_t)bh * NC * HD * HD + li * HD + TMS::mt(w) * 16 + 4 * lg;                  // S_chk[c][li][dk0..]
+    int64_t tmchk_off = (int64_t)bh * NC * C * C + (int64_t)tid * 4;                                  // row-major C x C
+    for (int c = 0; c < NC; ++c, o_off += (int64_t)C * rs, schk_off += HD * HD, tmchk_off += C * C) {
         const int t0 = c * C;
         const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
@@ -151,17 +170,14 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             if (pass != 0) zero_acc<TMS::TPW>(Sacc);  // an episode that starts in the chunk starts from 0
             store_acc<T, HD, HD, NW>(Sacc, sS, LDD, w, lane);  // sS[dv][dk]
             if (S_chk && pass == 0) {
-                T *dst = S_chk + ((int64_t)bh * NC + c) * HD * HD;
 #pragma unroll
-                for (int j = 0; j < TMS::TPW; ++j) {
-                    const int dk0 = TMS::mt(w) * 16 + 4 * lg, dv = TMS::nt(w, j) * 16 + li;
-                    *reinterpret_cast<P4 *>(dst + dv * HD + dk0) =
+                for (int j = 0; j < TMS::TPW; ++j)
+                    *reinterpret_cast<P4 *>(S_chk + schk_off + TMS::nt(w, j) * 16 * HD) =
                         TT<T>::pack(Sacc[j][0], Sacc[j][1], Sacc[j][2], Sacc[j][3]);
-                }
             }
             sync_lds();
             MRX_PHASE(1);
-            if (pass == nres && c + 1 < NC) prefetch(c + 1);
+            if (pass == nres && c + 1 < NC) prefetch();
 
             // ---- O^T[dv][i] = S Q^T ; A[i][j] = beta_i (k_i . k_j), j < i ---------------
             f32x4 Oacc[TMO::TPW];
@@ -216,10 +232,12 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 if (Tm_chk) {
                     // residual for the backward call: the rows of this pass's episode (rows past
                     // the end of the sequence count as the last episode: identity rows)
-                    T *dst = Tm_chk + ((int64_t)bh * NC + c) * C * C;
-                    for (int idx = tid; idx < C * C / 4; idx += NTHR) {
-                        const int i = idx / (C / 4), j = (idx % (C / 4)) * 4;
-                        if (live(i)) *reinterpret_cast<P4 *>(dst + i * C + j) = *reinterpret_cast<const P4 *>(sTm + i * LDC + j);
+#pragma unroll
+                    for (int it = 0; it < C * C / 4 / NTHR; ++it) {
+                        const int idx = tid + it * NTHR, i = idx / (C / 4), j = (idx % (C / 4)) * 4;
+                        if (live(i))
+                            *reinterpret_cast<P4 *>(Tm_chk + tmchk_off + it * NTHR * 4) =
+                                *reinterpret_cast<const P4 *>(sTm + i * LDC + j);
                     }
                 }
                 sync_lds();  // sW, sAqk visible; every wave is done with sQ
@@ -240,9 +258,9 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             gemm<T, HD, C, C, KROW, ROWK, NW>(Oacc, sU, LDD, sAqk, LDC, w, lane);
 #pragma unroll
             for (int j = 0; j < TMO::TPW; ++j) {
-                const int dv0 = TMO::mt(w) * 16 + 4 * lg, cc = TMO::nt(w, j) * 16 + li;
+                const int cc = TMO::nt(w, j) * 16 + li;
                 if (t0 + cc < Tlen && live(cc))
-                    *reinterpret_cast<P4 *>(o + base + (int64_t)(t0 + cc) * rs + dv0) =
+                    *reinterpret_cast<P4 *>(o + o_off + (int64_t)(TMO::nt(w, j) * 16) * rs) =
                         TT<T>::pack(Oacc[j][0], Oacc[j][1], Oacc[j][2], Oacc[j][3]);
             }
             // ---- S^T[dk][dv] += sum_c K[c][dk] U'[c][dv]  (only the episode that leaves the chunk)
