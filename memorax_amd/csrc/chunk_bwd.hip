@@ -55,7 +55,7 @@ __device__ __forceinline__ void store_rows_global(const f32x4 *acc, T *base, int
     const int li = lane & 15, lg = lane >> 4;
 #pragma unroll
     for (int j = 0; j < TM::TPW; ++j) {
-        const int d0 = TM::mt(w) * 16 + 4 * lg, r = TM::nt(w, j) * 16 + li;
+        const int d0 = TM::mt(w, j) * 16 + 4 * lg, r = TM::nt(w, j) * 16 + li;
         if (t0 + r < Tlen && keep(r)) {
             const f32x4 s = scale(r, d0);
             *reinterpret_cast<P4 *>(base + (int64_t)(t0 + r) * rs + d0) =
@@ -111,7 +111,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     f32x4 dSacc[TMS::TPW];  // dS^T: m = dk, n = dv
 #pragma unroll
     for (int j = 0; j < TMS::TPW; ++j) {
-        const int dk0 = TMS::mt(w) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
+        const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
         dSacc[j] = dS_last ? *reinterpret_cast<const f32x4 *>(dS_last + ((int64_t)bh * HD + dvv) * HD + dk0)
                            : f32x4{0.f, 0.f, 0.f, 0.f};
     }
@@ -215,7 +215,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     if (dS0) {
 #pragma unroll
         for (int j = 0; j < TMS::TPW; ++j) {
-            const int dk0 = TMS::mt(w) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
+            const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
             *reinterpret_cast<f32x4 *>(dS0 + ((int64_t)bh * HD + dvv) * HD + dk0) = dSacc[j];
         }
     }
@@ -279,7 +279,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     f32x4 dSacc[TMS::TPW];  // dS^T: m = dk, n = dv
 #pragma unroll
     for (int j = 0; j < TMS::TPW; ++j) {
-        const int dk0 = TMS::mt(w) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
+        const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
         dSacc[j] = dS_last ? *reinterpret_cast<const f32x4 *>(dS_last + ((int64_t)bh * HD + dvv) * HD + dk0)
                            : f32x4{0.f, 0.f, 0.f, 0.f};
     }
@@ -432,7 +432,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             auto rowdot = [&](const f32x4 *acc, const T *X) {
 #pragma unroll
                 for (int j = 0; j < TMR::TPW; ++j) {
-                    const int d0 = TMR::mt(w) * 16 + 4 * lg, r = TMR::nt(w, j) * 16 + li;
+                    const int d0 = TMR::mt(w, j) * 16 + 4 * lg, r = TMR::nt(w, j) * 16 + li;
                     const P4 x = *reinterpret_cast<const P4 *>(X + r * LDD + d0);
                     dbp[j] += acc[j][0] * (float)x[0] + acc[j][1] * (float)x[1] + acc[j][2] * (float)x[2] +
                               acc[j][3] * (float)x[3];
@@ -502,7 +502,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 float x = dbp[j];
                 x += __shfl_xor(x, 16);
                 x += __shfl_xor(x, 32);
-                if (lg == 0) sDb[TMR::mt(w) * C + TMR::nt(w, j) * 16 + li] = x;
+                if (lg == 0) sDb[TMR::mt(w, j) * C + TMR::nt(w, j) * 16 + li] = x;
             }
             sync_lds();
             MRX_PHASE(23);
@@ -518,7 +518,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     if (dS0) {
 #pragma unroll
         for (int j = 0; j < TMS::TPW; ++j) {
-            const int dk0 = TMS::mt(w) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
+            const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
             *reinterpret_cast<f32x4 *>(dS0 + ((int64_t)bh * HD + dvv) * HD + dk0) = dSacc[j];
         }
     }

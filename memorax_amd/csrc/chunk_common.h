@@ -106,32 +106,47 @@ template <> struct TT<float> {
 // 16-byte LDS row padding (in elements) keeps 16-lane fragment reads conflict free.
 template <typename T> constexpr int pad_of() { return 16 / (int)sizeof(T); }
 
-// Which 16x16 tiles of an M x N result a wave owns: slot j -> (mt, nt).
-template <int M, int N, int NW> struct TileMap {
+// Which 16x16 tiles of an M x N result a wave owns: slot j -> (mt, nt).  A wave owns a block of
+// MBW x NBW tiles, so that one k-step of a product reads MBW + NBW operand fragments from LDS
+// for MBW * NBW MFMAs: 2 x 2 blocks (four or more tiles per wave) halve the LDS traffic of a
+// 1 x 2 row of tiles.
+constexpr int default_mbw(int M, int N, int NW)
+{
+    const int mt = M / 16, nt = N / 16, tpw = mt * nt / NW;
+    return (tpw >= 4 && tpw % 2 == 0 && mt % 2 == 0 && nt % (tpw / 2) == 0 && (mt / 2) * (nt / (tpw / 2)) == NW) ? 2 : 1;
+}
+template <int M, int N, int NW, int MBW_ = 0> struct TileMap {
     static constexpr int MT = M / 16, NT = N / 16;
     static constexpr int TPW = MT * NT / NW;
-    static_assert(MT * NT % NW == 0 && TPW >= 1, "tiles must divide over the waves");
-    static_assert(NW % MT == 0 && NT % (NW / MT) == 0, "wave grid must tile the result");
-    static __device__ __forceinline__ int mt(int w) { return w % MT; }
-    static __device__ __forceinline__ int nt(int w, int j) { return (w / MT) * TPW + j; }
+    static constexpr int MBW = MBW_ > 0 ? MBW_ : default_mbw(M, N, NW);
+    static constexpr int NBW = TPW / MBW;
+    static constexpr int WM = MT / MBW, WN = NT / NBW;  // wave grid
+    static_assert(MT * NT % NW == 0 && TPW >= 1 && TPW % MBW == 0, "tiles must divide over the waves");
+    static_assert(MT % MBW == 0 && NT % NBW == 0 && WM * WN == NW, "wave grid must tile the result");
+    static __device__ __forceinline__ int mt(int w, int j) { return (w % WM) * MBW + j / NBW; }
+    static __device__ __forceinline__ int nt(int w, int j) { return (w / WM) * NBW + j % NBW; }
 };
 
-// acc[j] += sum_k X(mt rows, k) * Y(nt_j rows, k), k = 0..K-1.
-template <typename T, int M, int N, int K, int XM, int YM, int NW>
+// acc[j] += sum_k X(mt_j rows, k) * Y(nt_j rows, k), k = 0..K-1.
+template <typename T, int M, int N, int K, int XM, int YM, int NW, int MBW_ = 0>
 __device__ __forceinline__ void gemm(f32x4 *acc, const T *X, int ldx, const T *Y, int ldy, int w, int lane)
 {
-    using TM = TileMap<M, N, NW>;
+    using TM = TileMap<M, N, NW, MBW_>;
     using F = typename TT<T>::frag;
     constexpr int KB = TT<T>::KB;
     static_assert(K % KB == 0, "K must be a multiple of the fragment k extent");
-    const int m0 = TM::mt(w) * 16;
 #pragma unroll
     for (int kb = 0; kb < K / KB; ++kb) {
-        const F a = TT<T>::template load<XM>(X, ldx, m0, kb * KB, lane);
+        F a[TM::MBW];
 #pragma unroll
-        for (int j = 0; j < TM::TPW; ++j) {
-            const F b = TT<T>::template load<YM>(Y, ldy, TM::nt(w, j) * 16, kb * KB, lane);
-            acc[j] = TT<T>::mma(a, b, acc[j]);
+        for (int mi = 0; mi < TM::MBW; ++mi)
+            a[mi] = TT<T>::template load<XM>(X, ldx, TM::mt(w, mi * TM::NBW) * 16, kb * KB, lane);
+#pragma unroll
+        for (int ni = 0; ni < TM::NBW; ++ni) {
+            const F b = TT<T>::template load<YM>(Y, ldy, TM::nt(w, ni) * 16, kb * KB, lane);
+#pragma unroll
+            for (int mi = 0; mi < TM::MBW; ++mi)
+                acc[mi * TM::NBW + ni] = TT<T>::mma(a[mi], b, acc[mi * TM::NBW + ni]);
         }
     }
 }
@@ -143,15 +158,15 @@ template <int N> __device__ __forceinline__ void zero_acc(f32x4 *acc)
 }
 
 // Store an accumulator tile set as dst[n][m] (type T), f(m, n, x) applied per element.
-template <typename T, int M, int N, int NW, typename Fn>
+template <typename T, int M, int N, int NW, typename Fn, int MBW_ = 0>
 __device__ __forceinline__ void store_acc_f(const f32x4 *acc, T *dst, int ld, int w, int lane, Fn f)
 {
-    using TM = TileMap<M, N, NW>;
+    using TM = TileMap<M, N, NW, MBW_>;
     using P = typename TT<T>::pack4;
     const int i = lane & 15, g = lane >> 4;
 #pragma unroll
     for (int j = 0; j < TM::TPW; ++j) {
-        const int m = TM::mt(w) * 16 + 4 * g, n = TM::nt(w, j) * 16 + i;
+        const int m = TM::mt(w, j) * 16 + 4 * g, n = TM::nt(w, j) * 16 + i;
         *reinterpret_cast<P *>(dst + n * ld + m) =
             TT<T>::pack(f(m, n, acc[j][0]), f(m + 1, n, acc[j][1]), f(m + 2, n, acc[j][2]), f(m + 3, n, acc[j][3]));
     }

@@ -79,10 +79,11 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     using TMS = TileMap<HD, HD, NW>;  // S^T : m = dk, n = dv
     using TMO = TileMap<HD, C, NW>;   // X^T : m = feature, n = chunk row
     using TMA = TileMap<C, C, NW>;
+    using TMK = TileMap<C, C, NW, 1>;  // K K^T: a row of tiles per wave, so that every wave owns one diagonal tile
     f32x4 Sacc[TMS::TPW];
 #pragma unroll
     for (int j = 0; j < TMS::TPW; ++j) {
-        const int dk0 = TMS::mt(w) * 16 + 4 * lg, dv = TMS::nt(w, j) * 16 + li;
+        const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dv = TMS::nt(w, j) * 16 + li;
         Sacc[j] = S0 ? *reinterpret_cast<const f32x4 *>(S0 + ((int64_t)bh * HD + dv) * HD + dk0)
                      : f32x4{0.f, 0.f, 0.f, 0.f};
     }
@@ -135,8 +136,8 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 
     static_assert(C * C / 4 % NTHR == 0, "Tm tile copy assumes whole passes");
     // running element offsets of this thread's stores, advanced by one chunk per iteration
-    int64_t o_off = base + (int64_t)li * rs + TMO::mt(w) * 16 + 4 * lg;                              // o[t0 + li][dv0..]
-    int64_t schk_off = (int64_t)bh * NC * HD * HD + li * HD + TMS::mt(w) * 16 + 4 * lg;                  // S_chk[c][li][dk0..]
+    int64_t o_off = base + (int64_t)li * rs + 4 * lg;                               // o[t0 + li][4 lg..]
+    int64_t schk_off = (int64_t)bh * NC * HD * HD + li * HD + 4 * lg;                // S_chk[c][li][4 lg..]
     int64_t tmchk_off = (int64_t)bh * NC * C * C + (int64_t)tid * 4;                                  // row-major C x C
     for (int c = 0; c < NC; ++c, o_off += (int64_t)C * rs, schk_off += HD * HD, tmchk_off += C * C) {
         const int t0 = c * C;
@@ -172,7 +173,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             if (S_chk && pass == 0) {
 #pragma unroll
                 for (int j = 0; j < TMS::TPW; ++j)
-                    *reinterpret_cast<P4 *>(S_chk + schk_off + TMS::nt(w, j) * 16 * HD) =
+                    *reinterpret_cast<P4 *>(S_chk + schk_off + TMS::nt(w, j) * 16 * HD + TMS::mt(w, j) * 16) =
                         TT<T>::pack(Sacc[j][0], Sacc[j][1], Sacc[j][2], Sacc[j][3]);
             }
             sync_lds();
@@ -184,13 +185,13 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             zero_acc<TMO::TPW>(Oacc);
             gemm<T, HD, C, HD, ROWK, ROWK, NW>(Oacc, sS, LDD, sQ, LDD, w, lane);
             if (DELTA) {
-                f32x4 acc[TMA::TPW];
-                zero_acc<TMA::TPW>(acc);
-                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sK, LDD, sK, LDD, w, lane);  // D[m = j][n = i]
+                f32x4 acc[TMK::TPW];
+                zero_acc<TMK::TPW>(acc);
+                gemm<T, C, C, HD, ROWK, ROWK, NW, 1>(acc, sK, LDD, sK, LDD, w, lane);  // D[m = j][n = i]
                 // sA[i][j] = beta_i (k_i . k_j) for j < i, else 0 (beta read once per tile, then selects)
 #pragma unroll
-                for (int j = 0; j < TMA::TPW; ++j) {
-                    const int m = TMA::mt(w) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
+                for (int j = 0; j < TMK::TPW; ++j) {
+                    const int m = TMK::mt(w, j) * 16 + 4 * lg, n = TMK::nt(w, j) * 16 + li;
                     const float bn = sBeta[n];
                     f32x4 a;
 #pragma unroll
@@ -201,8 +202,8 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 int diag = -1;
                 f32x4 kk = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int j = 0; j < TMA::TPW; ++j)
-                    if (TMA::nt(w, j) == TMA::mt(w)) { diag = TMA::mt(w); kk = acc[j]; }
+                for (int j = 0; j < TMK::TPW; ++j)
+                    if (TMK::nt(w, j) == TMK::mt(w, j)) { diag = TMK::mt(w, j); kk = acc[j]; }
                 f32x4 Xcc = {0.f, 0.f, 0.f, 0.f};
                 if (diag >= 0) Xcc = tri_diag_block<T>(kk, sBeta, diag, sA, LDA, sTm, LDC, lane);
                 sync_lds();
@@ -260,7 +261,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             for (int j = 0; j < TMO::TPW; ++j) {
                 const int cc = TMO::nt(w, j) * 16 + li;
                 if (t0 + cc < Tlen && live(cc))
-                    *reinterpret_cast<P4 *>(o + o_off + (int64_t)(TMO::nt(w, j) * 16) * rs) =
+                    *reinterpret_cast<P4 *>(o + o_off + (int64_t)(TMO::nt(w, j) * 16) * rs + TMO::mt(w, j) * 16) =
                         TT<T>::pack(Oacc[j][0], Oacc[j][1], Oacc[j][2], Oacc[j][3]);
             }
             // ---- S^T[dk][dv] += sum_c K[c][dk] U'[c][dv]  (only the episode that leaves the chunk)
@@ -275,7 +276,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     if (S_last) {
 #pragma unroll
         for (int j = 0; j < TMS::TPW; ++j) {
-            const int dk0 = TMS::mt(w) * 16 + 4 * lg, dv = TMS::nt(w, j) * 16 + li;
+            const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dv = TMS::nt(w, j) * 16 + li;
             *reinterpret_cast<f32x4 *>(S_last + ((int64_t)bh * HD + dv) * HD + dk0) = Sacc[j];
         }
     }
