@@ -225,7 +225,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 // delta rule: fifteen LDS tiles (138 KB for bf16 / C = 64, 133 KB for fp32 / C = 32; one
 // workgroup per CU), two of them reused once their first tenant is dead; NW waves
 // =====================================================================================
-template <typename T, int C, int NW> struct DeltaBwdSmem : BwdDims<T, C> {
+template <typename T, int C, int NW, bool SPLIT> struct DeltaBwdSmem : BwdDims<T, C> {
     using D = BwdDims<T, C>;
     // ten [C][64] tiles, two [64][64], three [C][C]; Y1 and dA reuse the dO and S tiles
     static_assert(D::szCC <= D::szRD && D::szCC <= D::szDD, "reused regions must hold a [C][C] tile");
@@ -233,10 +233,12 @@ template <typename T, int C, int NW> struct DeltaBwdSmem : BwdDims<T, C> {
                          oW = oDO + D::szRD, oBK = oW + D::szRD, oBV = oBK + D::szRD, oU = oBV + D::szRD,
                          oDU = oU + D::szRD, oDW = oDU + D::szRD, oS = oDW + D::szRD, oDS = oS + D::szDD,
                          oAqk = oDS + D::szDD, oTm = oAqk + D::szCC, oDT = oTm + D::szCC,
-                         oBeta = oDT + D::szCC, oDb = oBeta + C * 4, total = oDb + 4 * C * 4;
+                         oBeta = oDT + D::szCC, oDb = oBeta + C * 4;
+    static constexpr int NSLOT = (SPLIT ? 2 : 1) * TileMap<HD, C, SPLIT ? NW / 2 : NW>::WM;
+    static constexpr int total = oDb + NSLOT * C * 4;
 };
 
-template <typename T, int C, int NW>
+template <typename T, int C, int NW, bool SPLIT>
 __global__ void __launch_bounds__(64 * NW)
 delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
@@ -246,7 +248,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                  float *__restrict__ dS0, int Tlen, int H)
 {
     constexpr int NTHR = 64 * NW;
-    using L = DeltaBwdSmem<T, C, NW>;
+    using L = DeltaBwdSmem<T, C, NW, SPLIT>;
     using IO = TileIO<T, C, NTHR>;
     using IOS = TileIO<T, HD, NTHR>;
     using IOT = TileIO<T, C, NTHR, C>;  // the [C][C] triangular factor
@@ -263,25 +265,39 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     T *sAqk = at(L::oAqk), *sDAqk = at(L::oAqk);          // Aqk[i][j] -> dAqk[i][j]
     T *sTm = at(L::oTm), *sDT = at(L::oDT);               // Tm[i][j], dT[a][b]
     float *sBeta = reinterpret_cast<float *>(smem + L::oBeta);
-    float *sDb = reinterpret_cast<float *>(smem + L::oDb);  // [4 feature tiles][C] dbeta partials
+    float *sDb = reinterpret_cast<float *>(smem + L::oDb);  // [NSLOT][C] dbeta partials
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // SPLIT: the waves form two groups.  Most phases hold two independent products of the same
+    // size: each group takes one of them whole, so that a wave owns a 2 x 2 block of result tiles
+    // and reads one operand fragment per MFMA from LDS (a 1 x 2 row of tiles needs 1.5).
+    // Without SPLIT every wave works on every product (one group of NW waves).
+    constexpr int GW = SPLIT ? NW / 2 : NW;
+    const int grp = w / GW, wl = w % GW;
+    const bool g0 = !SPLIT || grp == 0, g1 = !SPLIT || grp == 1;
     const int li = lane & 15, lg = lane >> 4;
     const int bh = blockIdx.x, b = bh / H, h = bh % H;
     const int64_t rs = (int64_t)H * HD;
     const int64_t base = ((int64_t)b * Tlen * H + h) * HD;
     const int NC = (Tlen + C - 1) / C;
 
-    using TMS = TileMap<HD, HD, NW>;
-    using TMA = TileMap<C, C, NW>;
-    using TMR = TileMap<HD, C, NW>;
-    f32x4 dSacc[TMS::TPW];  // dS^T: m = dk, n = dv
+    using TMA = TileMap<C, C, NW>;   // products without a partner: all waves
+    using GS = TileMap<HD, HD, GW>;  // group maps
+    using GA = TileMap<C, C, GW>;
+    using GR = TileMap<HD, C, GW>;
+    constexpr int NSLOT = L::NSLOT;  // dbeta partials per row: one per group and feature block
+    static_assert(NSLOT == (SPLIT ? 2 : 1) * GR::WM, "sDb slots");
+    constexpr int LDR = HD + 4;      // fp32 R tile over the dead Q (and dO) tiles
+    static_assert(C * LDR * 4 <= 2 * L::szRD && L::oDO == L::oQ + L::szRD, "R tile must fit");
+    float *sR = reinterpret_cast<float *>(smem + L::oQ);
+
+    f32x4 dSacc[GS::TPW];  // dS^T: m = dk, n = dv (group 0)
 #pragma unroll
-    for (int j = 0; j < TMS::TPW; ++j) {
-        const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
-        dSacc[j] = dS_last ? *reinterpret_cast<const f32x4 *>(dS_last + ((int64_t)bh * HD + dvv) * HD + dk0)
-                           : f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < GS::TPW; ++j) {
+        const int dk0 = GS::mt(wl, j) * 16 + 4 * lg, dvv = GS::nt(wl, j) * 16 + li;
+        dSacc[j] = (dS_last && g0) ? *reinterpret_cast<const f32x4 *>(dS_last + ((int64_t)bh * HD + dvv) * HD + dk0)
+                                         : f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
     typename IO::Regs rq, rk, rv, rdo;
@@ -345,124 +361,130 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 IOT::to_lds(rTm, sTm, LDC, tid);  // Tm[i][j] from the forward call (block diagonal by episode)
             }
             if (tid < C) sBeta[tid] = live(tid) ? raw_to_float<T>(rbeta) : 0.f;
-            if (pass != nres) zero_acc<TMS::TPW>(dSacc);
-            store_acc<T, HD, HD, NW>(dSacc, sDS, LDD, w, lane);  // dS[dv][dk]
+            if (pass != nres) zero_acc<GS::TPW>(dSacc);
+            if (g0) store_acc<T, HD, HD, GW>(dSacc, sDS, LDD, wl, lane);  // dS[dv][dk]
             sync_lds();
             MRX_PHASE(11);
             if (pass == 0 && c > 0) prefetch(c - 1);
 
-            // ---- Aqk[i][j] (j <= i) ; W^T[dk][c] = sum_j beta_j K[j][dk] Tm[c][j] -> sW[c][dk] ----
-            {
-                f32x4 acc[TMA::TPW];
-                zero_acc<TMA::TPW>(acc);
-                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sK, LDD, sQ, LDD, w, lane);  // D[m = j][n = i]
-                store_acc_f<T, C, C, NW>(acc, sAqk, LDC, w, lane, [](int m, int n, float x) { return m <= n ? x : 0.f; });
+            auto tril = [](int m, int n, float x) { return m <= n ? x : 0.f; };
+            if (g0) {
+                // ---- Aqk[i][j] = q_i . k_j, j <= i : D[m = j][n = i] -> sAqk[i][j] ------------------
+                f32x4 acc[GA::TPW];
+                zero_acc<GA::TPW>(acc);
+                gemm<T, C, C, HD, ROWK, ROWK, GW>(acc, sK, LDD, sQ, LDD, wl, lane);
+                store_acc_f<T, C, C, GW>(acc, sAqk, LDC, wl, lane, tril);
             }
-            {
-                f32x4 acc[TMR::TPW];
-                zero_acc<TMR::TPW>(acc);
-                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sBK, LDD, sTm, LDC, w, lane);  // D[m = dk][n = c]
-                store_acc<T, HD, C, NW>(acc, sW, LDD, w, lane);
+            if (g1) {
+                // ---- W^T[dk][c] = sum_j beta_j K[j][dk] Tm[c][j] -> sW[c][dk] -----------------------
+                f32x4 acc[GR::TPW];
+                zero_acc<GR::TPW>(acc);
+                gemm<T, HD, C, C, KROW, ROWK, GW>(acc, sBK, LDD, sTm, LDC, wl, lane);
+                store_acc<T, HD, C, GW>(acc, sW, LDD, wl, lane);
             }
             sync_lds();
             MRX_PHASE(15);
-            // ---- U'^T[dv][c] = sum_j beta_j V[j][dv] Tm[c][j] - sum_dk S[dv][dk] W[c][dk] -> sU[c][dv]
-            {
-                f32x4 acc[TMR::TPW], acc2[TMR::TPW];
-                zero_acc<TMR::TPW>(acc);
-                zero_acc<TMR::TPW>(acc2);
-                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sBV, LDD, sTm, LDC, w, lane);
-                gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc2, sS, LDD, sW, LDD, w, lane);
+            if (g0) {
+                // ---- U'^T[dv][c] = sum_j beta_j V[j][dv] Tm[c][j] - sum_dk S[dv][dk] W[c][dk] -> sU[c][dv]
+                f32x4 acc[GR::TPW], acc2[GR::TPW];
+                zero_acc<GR::TPW>(acc);
+                zero_acc<GR::TPW>(acc2);
+                gemm<T, HD, C, C, KROW, ROWK, GW>(acc, sBV, LDD, sTm, LDC, wl, lane);
+                gemm<T, HD, C, HD, ROWK, ROWK, GW>(acc2, sS, LDD, sW, LDD, wl, lane);
 #pragma unroll
-                for (int j = 0; j < TMR::TPW; ++j) acc[j] -= acc2[j];
-                store_acc<T, HD, C, NW>(acc, sU, LDD, w, lane);
+                for (int j = 0; j < GR::TPW; ++j) acc[j] -= acc2[j];
+                store_acc<T, HD, C, GW>(acc, sU, LDD, wl, lane);
             }
-            // ---- dU'^T[dv][j] = sum_i dO[i][dv] Aqk[i][j] + sum_dk dS[dv][dk] K[j][dk] -> sDU[j][dv]
-            {
-                f32x4 acc[TMR::TPW];
-                zero_acc<TMR::TPW>(acc);
-                gemm<T, HD, C, C, KROW, KROW, NW>(acc, sDO, LDD, sAqk, LDC, w, lane);
-                gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc, sDS, LDD, sK, LDD, w, lane);
-                store_acc<T, HD, C, NW>(acc, sDU, LDD, w, lane);
+            if (g1) {
+                // ---- dU'^T[dv][j] = sum_i dO[i][dv] Aqk[i][j] + sum_dk dS[dv][dk] K[j][dk] -> sDU[j][dv]
+                f32x4 acc[GR::TPW];
+                zero_acc<GR::TPW>(acc);
+                gemm<T, HD, C, C, KROW, KROW, GW>(acc, sDO, LDD, sAqk, LDC, wl, lane);
+                gemm<T, HD, C, HD, ROWK, ROWK, GW>(acc, sDS, LDD, sK, LDD, wl, lane);
+                store_acc<T, HD, C, GW>(acc, sDU, LDD, wl, lane);
             }
             sync_lds();  // sU, sDU visible; sAqk dead
             MRX_PHASE(16);
-            // ---- dAqk[i][j] = do_i . u'_j, j <= i -> sDAqk (over sAqk) ------------------------
-            {
-                f32x4 acc[TMA::TPW];
-                zero_acc<TMA::TPW>(acc);
-                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sU, LDD, sDO, LDD, w, lane);  // D[m = j][n = i]
-                store_acc_f<T, C, C, NW>(acc, sDAqk, LDC, w, lane, [](int m, int n, float x) { return m <= n ? x : 0.f; });
+            if (g0) {
+                // ---- dAqk[i][j] = do_i . u'_j, j <= i -> sDAqk (over sAqk) ------------------------
+                f32x4 acc[GA::TPW];
+                zero_acc<GA::TPW>(acc);
+                gemm<T, C, C, HD, ROWK, ROWK, GW>(acc, sU, LDD, sDO, LDD, wl, lane);  // D[m = j][n = i]
+                store_acc_f<T, C, C, GW>(acc, sDAqk, LDC, wl, lane, tril);
             }
-            // ---- dW^T[dk][c] = -sum_dv S[dv][dk] dU'[c][dv] -> sDW[c][dk] -----------------------
-            {
-                f32x4 acc[TMR::TPW];
-                zero_acc<TMR::TPW>(acc);
-                gemm<T, HD, C, HD, KROW, ROWK, NW>(acc, sS, LDD, sDU, LDD, w, lane);
-                store_acc_f<T, HD, C, NW>(acc, sDW, LDD, w, lane, [](int, int, float x) { return -x; });
+            if (g1) {
+                // ---- dW^T[dk][c] = -sum_dv S[dv][dk] dU'[c][dv] -> sDW[c][dk] -----------------------
+                f32x4 acc[GR::TPW];
+                zero_acc<GR::TPW>(acc);
+                gemm<T, HD, C, HD, KROW, ROWK, GW>(acc, sS, LDD, sDU, LDD, wl, lane);
+                store_acc_f<T, HD, C, GW>(acc, sDW, LDD, wl, lane, [](int, int, float x) { return -x; });
             }
             sync_lds();
             MRX_PHASE(17);
             auto one = [](int, int) { return f32x4{1.f, 1.f, 1.f, 1.f}; };
-            // ---- dQ^T[dk][i] = sum_dv S[dv][dk] dO[i][dv] + sum_j K[j][dk] dAqk[i][j] -> global ----
-            {
-                f32x4 acc[TMR::TPW];
-                zero_acc<TMR::TPW>(acc);
-                gemm<T, HD, C, HD, KROW, ROWK, NW>(acc, sS, LDD, sDO, LDD, w, lane);
-                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sK, LDD, sDAqk, LDC, w, lane);
-                store_rows_global<T, C, NW>(acc, dq + base, rs, t0, Tlen, w, lane, one, live);
-            }
-            // ---- dK^T[dk][j] = sum_i Q[i][dk] dAqk[i][j] + sum_dv dS[dv][dk] U'[j][dv] (registers) --
-            f32x4 dKacc[TMR::TPW];
-            zero_acc<TMR::TPW>(dKacc);
-            gemm<T, HD, C, C, KROW, KROW, NW>(dKacc, sQ, LDD, sDAqk, LDC, w, lane);
-            gemm<T, HD, C, HD, KROW, ROWK, NW>(dKacc, sDS, LDD, sU, LDD, w, lane);
-            // ---- dS^T[dk][dv] += sum_c Q[c][dk] dO[c][dv] - sum_c W[c][dk] dU'[c][dv] ---------------
-            {
-                f32x4 acc[TMS::TPW];
-                zero_acc<TMS::TPW>(acc);
-                gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, sQ, LDD, sDO, LDD, w, lane);
-                gemm<T, HD, HD, C, KROW, KROW, NW>(acc, sW, LDD, sDU, LDD, w, lane);
+            auto beta_of = [&](int r, int) { const float bb = sBeta[r]; return f32x4{bb, bb, bb, bb}; };
+            float dbp[GR::NBW];  // per-lane partials of dbeta for rows nt * 16 + li of the wave's tile columns
 #pragma unroll
-                for (int j = 0; j < TMS::TPW; ++j) dSacc[j] -= acc[j];
-            }
-            float dbp[TMR::TPW];  // per-lane partial of dbeta for row nt*16 + li
-#pragma unroll
-            for (int j = 0; j < TMR::TPW; ++j) dbp[j] = 0.f;
+            for (int j = 0; j < GR::NBW; ++j) dbp[j] = 0.f;
             auto rowdot = [&](const f32x4 *acc, const T *X) {
 #pragma unroll
-                for (int j = 0; j < TMR::TPW; ++j) {
-                    const int d0 = TMR::mt(w, j) * 16 + 4 * lg, r = TMR::nt(w, j) * 16 + li;
+                for (int j = 0; j < GR::TPW; ++j) {
+                    const int d0 = GR::mt(wl, j) * 16 + 4 * lg, r = GR::nt(wl, j) * 16 + li;
                     const P4 x = *reinterpret_cast<const P4 *>(X + r * LDD + d0);
-                    dbp[j] += acc[j][0] * (float)x[0] + acc[j][1] * (float)x[1] + acc[j][2] * (float)x[2] +
-                              acc[j][3] * (float)x[3];
+                    dbp[j % GR::NBW] += acc[j][0] * (float)x[0] + acc[j][1] * (float)x[1] + acc[j][2] * (float)x[2] +
+                                        acc[j][3] * (float)x[3];
                 }
             };
-            auto beta_of = [&](int r, int) { const float bb = sBeta[r]; return f32x4{bb, bb, bb, bb}; };
-            // ---- Zu^T[dv][j] = sum_i dU'[i][dv] Tm[i][j] -> dV = beta_j Zu ; dbeta += V_j . Zu_j ------
-            {
-                f32x4 acc[TMR::TPW];
-                zero_acc<TMR::TPW>(acc);
-                gemm<T, HD, C, C, KROW, KROW, NW>(acc, sDU, LDD, sTm, LDC, w, lane);
-                rowdot(acc, sV);
-                store_rows_global<T, C, NW>(acc, dv + base, rs, t0, Tlen, w, lane, beta_of, live);
-            }
-            // ---- Zw^T[dk][j] = sum_i dW[i][dk] Tm[i][j] -> dK += beta_j Zw ; dbeta += K_j . Zw_j ------
-            {
-                f32x4 acc[TMR::TPW];
-                zero_acc<TMR::TPW>(acc);
-                gemm<T, HD, C, C, KROW, KROW, NW>(acc, sDW, LDD, sTm, LDC, w, lane);
-                rowdot(acc, sK);
+            f32x4 dKacc[GR::TPW];  // dK^T[dk][j] (group 1)
+            zero_acc<GR::TPW>(dKacc);
+            if (g0) {
+                // ---- dQ^T[dk][i] = sum_dv S[dv][dk] dO[i][dv] + sum_j K[j][dk] dAqk[i][j] -> global ----
+                {
+                    f32x4 acc[GR::TPW];
+                    zero_acc<GR::TPW>(acc);
+                    gemm<T, HD, C, HD, KROW, ROWK, GW>(acc, sS, LDD, sDO, LDD, wl, lane);
+                    gemm<T, HD, C, C, KROW, ROWK, GW>(acc, sK, LDD, sDAqk, LDC, wl, lane);
+                    store_rows_global<T, C, GW>(acc, dq + base, rs, t0, Tlen, wl, lane, one, live);
+                }
+                // ---- dS^T[dk][dv] += sum_c Q[c][dk] dO[c][dv] - sum_c W[c][dk] dU'[c][dv] ---------------
+                {
+                    f32x4 acc[GS::TPW];
+                    zero_acc<GS::TPW>(acc);
+                    gemm<T, HD, HD, C, KROW, KROW, GW>(dSacc, sQ, LDD, sDO, LDD, wl, lane);
+                    gemm<T, HD, HD, C, KROW, KROW, GW>(acc, sW, LDD, sDU, LDD, wl, lane);
 #pragma unroll
-                for (int j = 0; j < TMR::TPW; ++j) dKacc[j] += acc[j] * sBeta[TMR::nt(w, j) * 16 + li];
+                    for (int j = 0; j < GS::TPW; ++j) dSacc[j] -= acc[j];
+                }
+                // ---- Zu^T[dv][j] = sum_i dU'[i][dv] Tm[i][j] -> dV = beta_j Zu ; dbeta += V_j . Zu_j ------
+                {
+                    f32x4 acc[GR::TPW];
+                    zero_acc<GR::TPW>(acc);
+                    gemm<T, HD, C, C, KROW, KROW, GW>(acc, sDU, LDD, sTm, LDC, wl, lane);
+                    rowdot(acc, sV);
+                    store_rows_global<T, C, GW>(acc, dv + base, rs, t0, Tlen, wl, lane, beta_of, live);
+                }
             }
-            // ---- dT[a][b] = dw_a . k_b + du'_a . v_b, a >= b : D[m = b][n = a] -> sDT[a][b] ------------
-            {
-                f32x4 acc[TMA::TPW];
-                zero_acc<TMA::TPW>(acc);
-                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sK, LDD, sDW, LDD, w, lane);
-                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sV, LDD, sDU, LDD, w, lane);
-                store_acc_f<T, C, C, NW>(acc, sDT, LDC, w, lane, [](int m, int n, float x) { return m <= n ? x : 0.f; });
+            if (g1) {
+                // ---- dK^T[dk][j] = sum_i Q[i][dk] dAqk[i][j] + sum_dv dS[dv][dk] U'[j][dv] (registers) --
+                gemm<T, HD, C, C, KROW, KROW, GW>(dKacc, sQ, LDD, sDAqk, LDC, wl, lane);
+                gemm<T, HD, C, HD, KROW, ROWK, GW>(dKacc, sDS, LDD, sU, LDD, wl, lane);
+                // ---- Zw^T[dk][j] = sum_i dW[i][dk] Tm[i][j] -> dK += beta_j Zw ; dbeta += K_j . Zw_j ------
+                {
+                    f32x4 acc[GR::TPW];
+                    zero_acc<GR::TPW>(acc);
+                    gemm<T, HD, C, C, KROW, KROW, GW>(acc, sDW, LDD, sTm, LDC, wl, lane);
+                    rowdot(acc, sK);
+#pragma unroll
+                    for (int j = 0; j < GR::TPW; ++j) dKacc[j] += acc[j] * sBeta[GR::nt(wl, j) * 16 + li];
+                }
+                // ---- dT[a][b] = dw_a . k_b + du'_a . v_b, a >= b : D[m = b][n = a] -> sDT[a][b] ------------
+                {
+                    f32x4 acc[GA::TPW];
+                    zero_acc<GA::TPW>(acc);
+                    gemm<T, C, C, HD, ROWK, ROWK, GW>(acc, sK, LDD, sDW, LDD, wl, lane);
+                    gemm<T, C, C, HD, ROWK, ROWK, GW>(acc, sV, LDD, sDU, LDD, wl, lane);
+                    store_acc_f<T, C, C, GW>(acc, sDT, LDC, wl, lane, tril);
+                }
             }
             sync_lds();  // sDT visible; sQ, sDO, sS, sDS, sDAqk dead
             MRX_PHASE(20);
@@ -484,30 +506,45 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();
             MRX_PHASE(22);
-            // ---- R^T[dk][i] = sum_j K[j][dk] dA[i][j] -> dK += beta_i R ; dbeta += K_i . R_i ;
-            //      dK^T[dk][j] += sum_i beta_i K[i][dk] dA[i][j] ------------------------------------------
-            {
-                f32x4 acc[TMR::TPW];
-                zero_acc<TMR::TPW>(acc);
-                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sK, LDD, sDA, LDC, w, lane);
+            if (g0) {
+                // ---- R^T[dk][i] = sum_j K[j][dk] dA[i][j] ; dbeta += K_i . R_i ; beta_i R -> sR[i][dk] (fp32)
+                f32x4 acc[GR::TPW];
+                zero_acc<GR::TPW>(acc);
+                gemm<T, HD, C, C, KROW, ROWK, GW>(acc, sK, LDD, sDA, LDC, wl, lane);
                 rowdot(acc, sK);
 #pragma unroll
-                for (int j = 0; j < TMR::TPW; ++j) dKacc[j] += acc[j] * sBeta[TMR::nt(w, j) * 16 + li];
-                gemm<T, HD, C, C, KROW, KROW, NW>(dKacc, sBK, LDD, sDA, LDC, w, lane);
-                store_rows_global<T, C, NW>(dKacc, dk + base, rs, t0, Tlen, w, lane, one, live);
+                for (int j = 0; j < GR::TPW; ++j) {
+                    const int d0 = GR::mt(wl, j) * 16 + 4 * lg, r = GR::nt(wl, j) * 16 + li;
+                    *reinterpret_cast<f32x4 *>(sR + r * LDR + d0) = acc[j] * sBeta[r];
+                }
             }
-            // ---- dbeta: reduce the partials over lane groups, then over feature tiles through LDS ----
+            if (g1) {
+                // ---- dK^T[dk][j] += sum_i beta_i K[i][dk] dA[i][j] ---------------------------------------
+                gemm<T, HD, C, C, KROW, KROW, GW>(dKacc, sBK, LDD, sDA, LDC, wl, lane);
+            }
+            // ---- dbeta: reduce the partials over lane groups, then over waves through LDS -----------
 #pragma unroll
-            for (int j = 0; j < TMR::TPW; ++j) {
+            for (int j = 0; j < GR::NBW; ++j) {
                 float x = dbp[j];
                 x += __shfl_xor(x, 16);
                 x += __shfl_xor(x, 32);
-                if (lg == 0) sDb[TMR::mt(w, j) * C + TMR::nt(w, j) * 16 + li] = x;
+                if (lg == 0) sDb[((SPLIT ? grp * GR::WM : 0) + wl % GR::WM) * C + GR::nt(wl, j) * 16 + li] = x;
             }
             sync_lds();
             MRX_PHASE(23);
+            if (g1) {
+                // ---- dK += beta_i R -> global ---------------------------------------------------------
+#pragma unroll
+                for (int j = 0; j < GR::TPW; ++j) {
+                    const int d0 = GR::mt(wl, j) * 16 + 4 * lg, r = GR::nt(wl, j) * 16 + li;
+                    dKacc[j] += *reinterpret_cast<const f32x4 *>(sR + r * LDR + d0);
+                }
+                store_rows_global<T, C, GW>(dKacc, dk + base, rs, t0, Tlen, wl, lane, one, live);
+            }
             if (tid < C && t0 + tid < Tlen && live(tid)) {
-                const float x = sDb[tid] + sDb[C + tid] + sDb[2 * C + tid] + sDb[3 * C + tid];
+                float x = 0.f;
+#pragma unroll
+                for (int sl = 0; sl < NSLOT; ++sl) x += sDb[sl * C + tid];
                 dbeta[((int64_t)b * Tlen + t0 + tid) * H + h] = (T)x;
             }
             sync_lds();
@@ -515,10 +552,10 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         }
     }
     MRX_PHASE_FLUSH();
-    if (dS0) {
+    if (dS0 && g0) {
 #pragma unroll
-        for (int j = 0; j < TMS::TPW; ++j) {
-            const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
+        for (int j = 0; j < GS::TPW; ++j) {
+            const int dk0 = GS::mt(wl, j) * 16 + 4 * lg, dvv = GS::nt(wl, j) * 16 + li;
             *reinterpret_cast<f32x4 *>(dS0 + ((int64_t)bh * HD + dvv) * HD + dk0) = dSacc[j];
         }
     }
@@ -603,8 +640,8 @@ extern "C" int mrx_delta_rule_bwd(void *stream, const void *q, const void *k, co
     hipStream_t st = (hipStream_t)stream;
     if (dtype == MRX_BF16) {
         constexpr int NW = MRX_DELTA_BWD_WAVES;
-        auto kern = delta_bwd_kernel<__bf16, 64, NW>;
-        constexpr int smem = DeltaBwdSmem<__bf16, 64, NW>::total;
+        auto kern = delta_bwd_kernel<__bf16, 64, NW, true>;
+        constexpr int smem = DeltaBwdSmem<__bf16, 64, NW, true>::total;
         static bool attr_set = false;
         if (set_smem(kern, smem, attr_set) != MRX_OK) return MRX_ERR_LAUNCH;
         hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(64 * NW), smem, st, (const __bf16 *)q,
@@ -614,8 +651,8 @@ extern "C" int mrx_delta_rule_bwd(void *stream, const void *q, const void *k, co
                            (__bf16 *)dbeta, (float *)dS0, (int)T, (int)H);
     } else {
         constexpr int NW = 4;
-        auto kern = delta_bwd_kernel<float, 32, NW>;
-        constexpr int smem = DeltaBwdSmem<float, 32, NW>::total;
+        auto kern = delta_bwd_kernel<float, 32, NW, false>;
+        constexpr int smem = DeltaBwdSmem<float, 32, NW, false>::total;
         static bool attr_set = false;
         if (set_smem(kern, smem, attr_set) != MRX_OK) return MRX_ERR_LAUNCH;
         hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(64 * NW), smem, st, (const float *)q,

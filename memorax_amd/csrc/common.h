@@ -57,16 +57,17 @@ extern __device__ unsigned long long mrx_wg_trace[4096 * 3];
     do {                                                                                  \
         if (threadIdx.x == 0 && blockIdx.x < 4096) mrx_wg_trace[blockIdx.x * 3 + 1] = wall_clock64(); \
     } while (0)
-// marks accumulate in LDS (fire-and-forget ds_add) so that a mark never waits on global memory
+// marks (i < 32; thread 0 -> slot i, thread 256 -> slot 32 + i) accumulate in LDS
+// (fire-and-forget ds_add) so that a mark never waits on global memory
 #define MRX_PHASE_INIT()                                                    \
     __shared__ unsigned long long mrx_lds_ticks[64];                        \
     if (threadIdx.x < 64) mrx_lds_ticks[threadIdx.x] = 0;                   \
     unsigned long long mrx_t_last = clock64()
 #define MRX_PHASE(i)                                                        \
     do {                                                                    \
-        if (blockIdx.x == 0 && threadIdx.x == 0) {                          \
+        if (blockIdx.x == 0 && (threadIdx.x == 0 || threadIdx.x == 256)) {  \
             const unsigned long long mrx_t_now = clock64();                 \
-            __hip_atomic_fetch_add(&mrx_lds_ticks[i], mrx_t_now - mrx_t_last, __ATOMIC_RELAXED, \
+            __hip_atomic_fetch_add(&mrx_lds_ticks[(i) + (threadIdx.x ? 32 : 0)], mrx_t_now - mrx_t_last, __ATOMIC_RELAXED, \
                                    __HIP_MEMORY_SCOPE_WORKGROUP);           \
             mrx_t_last = mrx_t_now;                                         \
         }                                                                   \
