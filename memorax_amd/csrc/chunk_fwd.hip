@@ -65,7 +65,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     float *sA = reinterpret_cast<float *>(smem + L::oA);
     T *sAqk = reinterpret_cast<T *>(smem + L::oA);
     T *sW = reinterpret_cast<T *>(smem + L::oA + L::szCC);
-    T *sU = DELTA ? sQ : sV;                         // U' [C][dv]
+    T *sU = sV;                                      // U' [C][dv] (delta rule: over beta V once U is taken)
     float *sBeta = reinterpret_cast<float *>(smem + L::oBeta);
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -178,12 +178,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();
             MRX_PHASE(1);
-            if (pass == nres && c + 1 < NC) prefetch();
-
-            // ---- O^T[dv][i] = S Q^T ; A[i][j] = beta_i (k_i . k_j), j < i ---------------
-            f32x4 Oacc[TMO::TPW];
-            zero_acc<TMO::TPW>(Oacc);
-            gemm<T, HD, C, HD, ROWK, ROWK, NW>(Oacc, sS, LDD, sQ, LDD, w, lane);
+            // ---- A[i][j] = beta_i (k_i . k_j), j < i ----------------------------------
             if (DELTA) {
                 f32x4 acc[TMK::TPW];
                 zero_acc<TMK::TPW>(acc);
@@ -241,9 +236,10 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                                 *reinterpret_cast<const P4 *>(sTm + i * LDC + j);
                     }
                 }
-                sync_lds();  // sW, sAqk visible; every wave is done with sQ
+                sync_lds();  // sW, sAqk visible; every wave is done with beta V
                 MRX_PHASE(5);
-                // U'^T[dv][c] = U^T - S W^T -> sU[c][dv] (over sQ)
+                if (pass == nres && c + 1 < NC) prefetch();
+                // U'^T[dv][c] = U^T - S W^T -> sU[c][dv] (over beta V)
                 {
                     f32x4 acc[TMO::TPW];
                     zero_acc<TMO::TPW>(acc);
@@ -255,7 +251,11 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();
             MRX_PHASE(7);
-            // ---- O^T[dv][i] += sum_j U'[j][dv] Aqk[i][j] ; store O ------------------------------
+            // ---- O^T[dv][i] = sum_dk S[dv][dk] Q[i][dk] + sum_j U'[j][dv] Aqk[i][j] ; store O -------
+            if (!DELTA && pass == nres && c + 1 < NC) prefetch();
+            f32x4 Oacc[TMO::TPW];
+            zero_acc<TMO::TPW>(Oacc);
+            gemm<T, HD, C, HD, ROWK, ROWK, NW>(Oacc, sS, LDD, sQ, LDD, w, lane);
             gemm<T, HD, C, C, KROW, ROWK, NW>(Oacc, sU, LDD, sAqk, LDC, w, lane);
 #pragma unroll
             for (int j = 0; j < TMO::TPW; ++j) {
