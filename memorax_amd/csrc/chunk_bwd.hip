@@ -64,6 +64,26 @@ __device__ __forceinline__ void store_rows_global(const f32x4 *acc, T *base, int
     }
 }
 
+// Same, addressed by a running pointer: `row` points at feature 4 * (lane >> 4) of chunk row
+// (lane & 15); the tile offsets are wave-uniform.
+template <typename T, int C, int NW, typename ScaleF, typename KeepF>
+__device__ __forceinline__ void store_rows_at(const f32x4 *acc, T *row, int64_t rs, int t0, int Tlen, int w,
+                                              int lane, ScaleF scale, KeepF keep)
+{
+    using TM = TileMap<HD, C, NW>;
+    using P4 = typename TT<T>::pack4;
+    const int li = lane & 15, lg = lane >> 4;
+#pragma unroll
+    for (int j = 0; j < TM::TPW; ++j) {
+        const int d0 = TM::mt(w, j) * 16 + 4 * lg, r = TM::nt(w, j) * 16 + li;
+        if (t0 + r < Tlen && keep(r)) {
+            const f32x4 s = scale(r, d0);
+            *reinterpret_cast<P4 *>(row + (int64_t)(TM::nt(w, j) * 16) * rs + TM::mt(w, j) * 16) =
+                TT<T>::pack(acc[j][0] * s[0], acc[j][1] * s[1], acc[j][2] * s[2], acc[j][3] * s[3]);
+        }
+    }
+}
+
 // =====================================================================================
 // linear attention: 8 tiles, two workgroups per CU
 // =====================================================================================
@@ -305,31 +325,67 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     typename IOT::Regs rTm;
     uint32_t rdone = 0u, rbeta = 0u;  // raw bits, converted when the chunk is staged
     uint32_t rbrow[IO::PASSES];       // beta of the rows this thread stages
-    auto prefetch = [&](int c) {
-        const int t0 = c * C;
-        IO::load(rq, q + base, rs, t0, Tlen, tid);
-        IO::load(rk, k + base, rs, t0, Tlen, tid);
-        IO::load(rv, v + base, rs, t0, Tlen, tid);
-        IO::load(rdo, dout + base, rs, t0, Tlen, tid);
-        IOS::load(rS, S_chk + ((int64_t)bh * NC + c) * HD * HD, HD, 0, HD, tid);
-        IOT::load(rTm, Tm_chk + ((int64_t)bh * NC + c) * C * C, C, 0, C, tid);
+    // Running element offsets of this thread's loads and stores, stepped back by one chunk per
+    // iteration (64-bit adds instead of per-chunk index multiplications).
+    const int tlast = (NC - 1) * C;
+    int64_t roff[IO::PASSES], boff[IO::PASSES];
 #pragma unroll
-        for (int p = 0; p < IO::PASSES; ++p) {
-            const int t = t0 + IO::row_of(tid, p);
-            rbrow[p] = t < Tlen ? load_raw<T>(beta + ((int64_t)b * Tlen + t) * H + h) : 0u;
-        }
-        rdone = 0u;
-        rbeta = 0u;
-        if (lane < C && t0 + lane < Tlen) {
-            const int64_t bt = (int64_t)b * Tlen + t0 + lane;
-            rdone = done_raw(done, done_f32, bt);
-            if (w == 0) rbeta = load_raw<T>(beta + bt * H + h);
+    for (int p = 0; p < IO::PASSES; ++p) {
+        const int r = tlast + IO::row_of(tid, p);
+        roff[p] = base + (int64_t)r * rs + (tid % IO::SEGS) * IO::KP;  // q/k/v/dout: row r, this thread's segment
+        boff[p] = ((int64_t)b * Tlen + r) * H + h;                     // beta of row r
+    }
+    int64_t soff = ((int64_t)bh * NC + NC - 1) * HD * HD + (tid / IOS::SEGS) * HD + (tid % IOS::SEGS) * IOS::KP;
+    int64_t tmoff = ((int64_t)bh * NC + NC - 1) * C * C + (tid / IOT::SEGS) * C + (tid % IOT::SEGS) * IOT::KP;
+    int64_t doff = (int64_t)b * Tlen + tlast + lane;  // done/beta of chunk row `lane`
+    int tpre = tlast;                                 // first time step of the chunk about to be prefetched
+    // The prefetch of the next chunk is issued in parts, one per phase, so that the address unit
+    // works through the loads beside the phases' LDS and MFMA work instead of stalling every wave
+    // at one point.  part 0: q, 1: k, 2: v, 3: dout, 4: S, 5: Tm and the per-row scalars.
+    auto prefetch_part = [&](int part) {
+        typename IO::F z;
+#pragma unroll
+        for (int e = 0; e < IO::KP; ++e) z[e] = (T)0.f;
+        if (part < 4) {
+            const T *src = part == 0 ? q : part == 1 ? k : part == 2 ? v : dout;
+            typename IO::Regs &dst = part == 0 ? rq : part == 1 ? rk : part == 2 ? rv : rdo;
+#pragma unroll
+            for (int p = 0; p < IO::PASSES; ++p)
+                dst.v[p] = tpre + IO::row_of(tid, p) < Tlen ? *reinterpret_cast<const typename IO::F *>(src + roff[p]) : z;
+        } else if (part == 4) {
+#pragma unroll
+            for (int p = 0; p < IOS::PASSES; ++p)
+                rS.v[p] = *reinterpret_cast<const typename IOS::F *>(S_chk + soff + p * IOS::RPP * HD);
+        } else {
+#pragma unroll
+            for (int p = 0; p < IOT::PASSES; ++p)
+                rTm.v[p] = *reinterpret_cast<const typename IOT::F *>(Tm_chk + tmoff + p * IOT::RPP * C);
+#pragma unroll
+            for (int p = 0; p < IO::PASSES; ++p) {
+                rbrow[p] = tpre + IO::row_of(tid, p) < Tlen ? load_raw<T>(beta + boff[p]) : 0u;
+                roff[p] -= (int64_t)C * rs;
+                boff[p] -= (int64_t)C * H;
+            }
+            rdone = 0u;
+            rbeta = 0u;
+            if (lane < C && tpre + lane < Tlen) {
+                rdone = done_raw(done, done_f32, doff);
+                if (w == 0) rbeta = load_raw<T>(beta + doff * H + h);
+            }
+            soff -= HD * HD;
+            tmoff -= C * C;
+            doff -= C;
+            tpre -= C;
         }
     };
-    prefetch(NC - 1);
+#pragma unroll
+    for (int part = 0; part < 6; ++part) prefetch_part(part);
+    // stores: row li of the chunk, this lane's 4 features (tile offsets are added per tile)
+    int64_t goff = base + (int64_t)(tlast + li) * rs + 4 * lg;
+    int64_t dboff = ((int64_t)b * Tlen + tlast + tid) * H + h;
     MRX_PHASE_INIT();
 
-    for (int c = NC - 1; c >= 0; --c) {
+    for (int c = NC - 1; c >= 0; --c, goff -= (int64_t)C * rs, dboff -= (int64_t)C * H) {
         const int t0 = c * C;
         const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
@@ -365,7 +421,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             if (g0) store_acc<T, HD, HD, GW>(dSacc, sDS, LDD, wl, lane);  // dS[dv][dk]
             sync_lds();
             MRX_PHASE(11);
-            if (pass == 0 && c > 0) prefetch(c - 1);
+            const bool pre = pass == 0 && c > 0;
+            if (pre) prefetch_part(0);
 
             auto tril = [](int m, int n, float x) { return m <= n ? x : 0.f; };
             if (g0) {
@@ -384,6 +441,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();
             MRX_PHASE(15);
+            if (pre) prefetch_part(1);
             if (g0) {
                 // ---- U'^T[dv][c] = sum_j beta_j V[j][dv] Tm[c][j] - sum_dk S[dv][dk] W[c][dk] -> sU[c][dv]
                 f32x4 acc[GR::TPW], acc2[GR::TPW];
@@ -405,6 +463,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();  // sU, sDU visible; sAqk dead
             MRX_PHASE(16);
+            if (pre) prefetch_part(2);
             if (g0) {
                 // ---- dAqk[i][j] = do_i . u'_j, j <= i -> sDAqk (over sAqk) ------------------------
                 f32x4 acc[GA::TPW];
@@ -421,6 +480,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();
             MRX_PHASE(17);
+            if (pre) prefetch_part(3);
             auto one = [](int, int) { return f32x4{1.f, 1.f, 1.f, 1.f}; };
             auto beta_of = [&](int r, int) { const float bb = sBeta[r]; return f32x4{bb, bb, bb, bb}; };
             float dbp[GR::NBW];  // per-lane partials of dbeta for rows nt * 16 + li of the wave's tile columns
@@ -444,7 +504,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     zero_acc<GR::TPW>(acc);
                     gemm<T, HD, C, HD, KROW, ROWK, GW>(acc, sS, LDD, sDO, LDD, wl, lane);
                     gemm<T, HD, C, C, KROW, ROWK, GW>(acc, sK, LDD, sDAqk, LDC, wl, lane);
-                    store_rows_global<T, C, GW>(acc, dq + base, rs, t0, Tlen, wl, lane, one, live);
+                    store_rows_at<T, C, GW>(acc, dq + goff, rs, t0, Tlen, wl, lane, one, live);
                 }
                 // ---- dS^T[dk][dv] += sum_c Q[c][dk] dO[c][dv] - sum_c W[c][dk] dU'[c][dv] ---------------
                 {
@@ -461,7 +521,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     zero_acc<GR::TPW>(acc);
                     gemm<T, HD, C, C, KROW, KROW, GW>(acc, sDU, LDD, sTm, LDC, wl, lane);
                     rowdot(acc, sV);
-                    store_rows_global<T, C, GW>(acc, dv + base, rs, t0, Tlen, wl, lane, beta_of, live);
+                    store_rows_at<T, C, GW>(acc, dv + goff, rs, t0, Tlen, wl, lane, beta_of, live);
                 }
             }
             if (g1) {
@@ -488,6 +548,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();  // sDT visible; sQ, sDO, sS, sDS, sDAqk dead
             MRX_PHASE(20);
+            if (pre) prefetch_part(4);
             // ---- Y1[j][b] = beta_b sum_a Tm[a][j] dT[a][b] : D[m = b][n = j] -> sY1[j][b] ---------------
             {
                 f32x4 acc[TMA::TPW];
@@ -497,6 +558,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();
             MRX_PHASE(21);
+            if (pre) prefetch_part(5);
             // ---- dA[i][j] = -sum_b Y1[i][b] Tm[j][b], j < i : D[m = j][n = i] -> sDA[i][j] --------------
             {
                 f32x4 acc[TMA::TPW];
@@ -539,13 +601,13 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     const int d0 = GR::mt(wl, j) * 16 + 4 * lg, r = GR::nt(wl, j) * 16 + li;
                     dKacc[j] += *reinterpret_cast<const f32x4 *>(sR + r * LDR + d0);
                 }
-                store_rows_global<T, C, GW>(dKacc, dk + base, rs, t0, Tlen, wl, lane, one, live);
+                store_rows_at<T, C, GW>(dKacc, dk + goff, rs, t0, Tlen, wl, lane, one, live);
             }
             if (tid < C && t0 + tid < Tlen && live(tid)) {
                 float x = 0.f;
 #pragma unroll
                 for (int sl = 0; sl < NSLOT; ++sl) x += sDb[sl * C + tid];
-                dbeta[((int64_t)b * Tlen + t0 + tid) * H + h] = (T)x;
+                dbeta[dboff] = (T)x;
             }
             sync_lds();
             MRX_PHASE(24);
