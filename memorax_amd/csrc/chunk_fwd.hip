@@ -104,30 +104,37 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     }
     int64_t doff = (int64_t)b * Tlen + lane;  // done of chunk row `lane`
     int tpre = 0;                             // first time step of the chunk about to be prefetched
-    auto prefetch = [&]() {
+    // The prefetch is issued in parts spread over the phases, so that the address unit works
+    // through the loads beside LDS and MFMA work.  part 0: q, 1: k, 2: v, 3: per-row scalars.
+    auto prefetch_part = [&](int part) {
         typename IO::F z;
 #pragma unroll
         for (int e = 0; e < IO::KP; ++e) z[e] = (T)0.f;
+        if (part < 3) {
+            const T *src = part == 0 ? q : part == 1 ? k : v;
+            typename IO::Regs &dst = part == 0 ? rq : part == 1 ? rk : rv;
 #pragma unroll
-        for (int p = 0; p < IO::PASSES; ++p) {
-            const bool in = tpre + IO::row_of(tid, p) < Tlen;
-            rq.v[p] = in ? *reinterpret_cast<const typename IO::F *>(q + roff[p]) : z;
-            rk.v[p] = in ? *reinterpret_cast<const typename IO::F *>(k + roff[p]) : z;
-            rv.v[p] = in ? *reinterpret_cast<const typename IO::F *>(v + roff[p]) : z;
-            if (DELTA) rbrow[p] = in ? load_raw<T>(beta + boff[p]) : 0u;
-            roff[p] += (int64_t)C * rs;
-            boff[p] += (int64_t)C * H;
+            for (int p = 0; p < IO::PASSES; ++p)
+                dst.v[p] = tpre + IO::row_of(tid, p) < Tlen ? *reinterpret_cast<const typename IO::F *>(src + roff[p]) : z;
+        } else {
+#pragma unroll
+            for (int p = 0; p < IO::PASSES; ++p) {
+                if (DELTA) rbrow[p] = tpre + IO::row_of(tid, p) < Tlen ? load_raw<T>(beta + boff[p]) : 0u;
+                roff[p] += (int64_t)C * rs;
+                boff[p] += (int64_t)C * H;
+            }
+            rdone = 0u;
+            rbeta = 0u;
+            if (lane < C && tpre + lane < Tlen) {
+                rdone = done_raw(done, done_f32, doff);
+                if (DELTA && w == 0) rbeta = load_raw<T>(beta + doff * H + h);
+            }
+            doff += C;
+            tpre += C;
         }
-        rdone = 0u;
-        rbeta = 0u;
-        if (lane < C && tpre + lane < Tlen) {
-            rdone = done_raw(done, done_f32, doff);
-            if (DELTA && w == 0) rbeta = load_raw<T>(beta + doff * H + h);
-        }
-        doff += C;
-        tpre += C;
     };
-    prefetch();
+#pragma unroll
+    for (int part = 0; part < 4; ++part) prefetch_part(part);
     if (DELTA) {
         // blocks above the block diagonal of Tm are never written again
         for (int idx = tid; idx < C * LDC * (int)sizeof(T) / 4; idx += NTHR) reinterpret_cast<uint32_t *>(sTm)[idx] = 0u;
@@ -178,6 +185,9 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();
             MRX_PHASE(1);
+            const bool pre = pass == nres && c + 1 < NC;
+            if (pre) prefetch_part(0);
+            if (!DELTA && pre) prefetch_part(1);
             // ---- A[i][j] = beta_i (k_i . k_j), j < i ----------------------------------
             if (DELTA) {
                 f32x4 acc[TMK::TPW];
@@ -203,9 +213,11 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 if (diag >= 0) Xcc = tri_diag_block<T>(kk, sBeta, diag, sA, LDA, sTm, LDC, lane);
                 sync_lds();
                 MRX_PHASE(2);
+                if (pre) prefetch_part(1);
                 if (diag >= 0) tri_block_column<C, T>(sA, LDA, sTm, LDC, diag, Xcc, lane);
                 sync_lds();
                 MRX_PHASE(3);
+                if (pre) prefetch_part(2);
             }
             // ---- Aqk[i][j] = (q_i . k_j), j <= i ; delta rule: W = Tm (beta K), U = Tm (beta V) ----
             {
@@ -238,7 +250,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 }
                 sync_lds();  // sW, sAqk visible; every wave is done with beta V
                 MRX_PHASE(5);
-                if (pass == nres && c + 1 < NC) prefetch();
+                if (pre) prefetch_part(3);
                 // U'^T[dv][c] = U^T - S W^T -> sU[c][dv] (over beta V)
                 {
                     f32x4 acc[TMO::TPW];
@@ -252,7 +264,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             sync_lds();
             MRX_PHASE(7);
             // ---- O^T[dv][i] = sum_dk S[dv][dk] Q[i][dk] + sum_j U'[j][dv] Aqk[i][j] ; store O -------
-            if (!DELTA && pass == nres && c + 1 < NC) prefetch();
+            if (!DELTA && pre) { prefetch_part(2); prefetch_part(3); }
             f32x4 Oacc[TMO::TPW];
             zero_acc<TMO::TPW>(Oacc);
             gemm<T, HD, C, HD, ROWK, ROWK, NW>(Oacc, sS, LDD, sQ, LDD, w, lane);
