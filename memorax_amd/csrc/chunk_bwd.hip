@@ -308,9 +308,11 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     using GR = TileMap<HD, C, GW>;
     constexpr int NSLOT = L::NSLOT;  // dbeta partials per row: one per group and feature block
     static_assert(NSLOT == (SPLIT ? 2 : 1) * GR::WM, "sDb slots");
-    constexpr int LDR = HD + 4;      // fp32 R tile over the dead Q (and dO) tiles
-    static_assert(C * LDR * 4 <= 2 * L::szRD && L::oDO == L::oQ + L::szRD, "R tile must fit");
-    float *sR = reinterpret_cast<float *>(smem + L::oQ);
+    // fp32 R tile over the U' and dU' tiles: both are dead by then and neither is written before
+    // the second barrier of the next pass, so no barrier is needed after the last phase
+    constexpr int LDR = HD + 4;
+    static_assert(C * LDR * 4 <= 2 * L::szRD && L::oDU == L::oU + L::szRD, "R tile must fit");
+    float *sR = reinterpret_cast<float *>(smem + L::oU);
 
     f32x4 dSacc[GS::TPW];  // dS^T: m = dk, n = dv (group 0)
 #pragma unroll
@@ -609,8 +611,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 for (int sl = 0; sl < NSLOT; ++sl) x += sDb[sl * C + tid];
                 dbeta[dboff] = (T)x;
             }
-            sync_lds();
-            MRX_PHASE(24);
+            MRX_PHASE(24);  // no barrier: what this phase reads (sR, sDb) is not written by the next staging step
         }
     }
     MRX_PHASE_FLUSH();
