@@ -134,6 +134,7 @@ def main() -> int:
     if args.all:
         out["linear_attention"] = bench_linear_attention(torch, K, M, dev)
         out["torso"] = bench_torso(torch, K)
+        out["step"] = bench_step(torch, K)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(np, M, x, do_np)
     print(json.dumps(out))
@@ -198,6 +199,34 @@ def bench_linear_attention(torch, K, M, dev):
     ms = _time_ms(torch, f3, iters=5)
     res["cfg3_bf16_B32of256_4096x8x64"] = {"ms": ms, "tokens/s": Bn * Tn / ms * 1e3,
                                            "GB/s": 1408 * Bn * Tn * Hn / ms / 1e6}
+    return res
+
+
+def bench_step(torch, K):
+    """Acting path: one time step for 1024 environments x 4 heads (the rollout of configuration 5),
+    state updated in place.  Bytes = the fp32 state read once and written once (32 KiB per (b,h))
+    plus q, k, v, o.  The chunked forward kernel at T = 1 is timed beside it."""
+    Bn, Hn, d = 1024, 4, 64
+    bf = torch.bfloat16
+    q, k, v = (torch.randn((Bn, Hn, d), device="cuda").to(bf) for _ in range(3))
+    k = torch.nn.functional.normalize(k.float(), dim=-1).to(bf)
+    beta = torch.rand((Bn, Hn), device="cuda").to(bf)
+    dn = torch.rand((Bn,), device="cuda") < 0.01
+    S = torch.zeros((Bn, Hn, d, d), device="cuda")
+    z = torch.zeros((Bn, Hn, d), device="cuda")
+    by = Bn * Hn * (2 * d * d * 4 + 4 * d * 2)
+    res = {}
+    ms = _time_ms(torch, lambda: K.delta_rule_step(q, k, v, beta, dn, S, inplace=True), iters=50, warm=5)
+    res["delta_rule_step_1024x4x64"] = {"ms": ms, "GB/s": by / ms / 1e6, "frac_hbm": by / ms / 1e6 / HBM_PEAK_GBS,
+                                        "env_steps/s": Bn / ms * 1e3}
+    ms = _time_ms(torch, lambda: K.linear_attn_step(q, k, v, dn, S, z, "elu1", True, 1e-6, True), iters=50, warm=5)
+    res["linear_attn_step_normalised_1024x4x64"] = {"ms": ms, "GB/s": by / ms / 1e6,
+                                                    "frac_hbm": by / ms / 1e6 / HBM_PEAK_GBS,
+                                                    "env_steps/s": Bn / ms * 1e3}
+    q1, k1, v1, b1, d1 = q[:, None].contiguous(), k[:, None].contiguous(), v[:, None].contiguous(), \
+        beta[:, None].contiguous(), dn[:, None].contiguous()
+    ms = _time_ms(torch, lambda: K.delta_rule_fwd(q1, k1, v1, b1, d1, S, save_chk=False), iters=50, warm=5)
+    res["chunk_kernel_at_T1_for_comparison"] = {"ms": ms}
     return res
 
 

@@ -136,6 +136,33 @@ int mrx_delta_rule_bwd(void *stream, const void *q, const void *k,
                        void *dbeta, void *dS0, int64_t B, int64_t T, int64_t H,
                        int64_t dk, int64_t dv, int dtype, int done_dtype);
 
+/* ---- Single time step (rollout / acting) ------------------------------------
+ * What Memoroid.__call__ (memoroid.py:93-109) computes when T = 1, as PPO's rollout
+ * does once per environment step (algorithms/ppo.py:105-143): one update of the
+ * carry fused with the read-out, without the chunk machinery.
+ *   q,k,v,o: (B,1,H,64) = (B,H,64) in `dtype`; done: (B,) ; S_in/S_out: (B,H,dv,dk) fp32.
+ * S_in may be NULL (zero state) and may equal S_out (update in place).
+ *
+ * Linear attention (linear_attention.py:62-117):
+ *     S' = (done ? 0 : S) + v phi(k)^T ;  o = S' phi(q)
+ * and, when z_out is given (z_in/z_out: (B,H,dk) fp32, z_in nullable, may alias), the
+ * normaliser of LinearAttentionCell.read (linear_attention.py:100-110):
+ *     z' = (done ? 0 : z) + phi(k) ;  o = S' phi(q) / max(phi(q) . z', eps). */
+int mrx_linear_attn_step(void *stream, const void *q, const void *k,
+                         const void *v, const void *done, const float *S_in,
+                         const float *z_in, void *o, float *S_out, float *z_out,
+                         int64_t B, int64_t H, int64_t dk, int64_t dv, int dtype,
+                         int done_dtype, int feature_map, float eps);
+
+/* Delta rule (no counterpart in the reference; the T = 1 case of mrx_delta_rule_fwd):
+ *     S0 = done ? 0 : S ;  u = beta (v - S0 k) ;  S' = S0 + u k^T ;  o = S' q
+ * beta: (B,H) in `dtype`. */
+int mrx_delta_rule_step(void *stream, const void *q, const void *k,
+                        const void *v, const void *beta, const void *done,
+                        const float *S_in, void *o, float *S_out, int64_t B,
+                        int64_t H, int64_t dk, int64_t dv, int dtype,
+                        int done_dtype);
+
 #ifdef __cplusplus
 }
 #endif

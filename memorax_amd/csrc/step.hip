@@ -1,0 +1,158 @@
+// Single-step (T = 1) state updates for acting/rollout loops: one time step of the linear
+// attention and of the delta-rule recurrence per (b, h) sequence, fused with the read-out.
+//
+//   linear attention : S' = (done ? 0 : S) + v phi(k)^T ,  z' = (done ? 0 : z) + phi(k)
+//                      o = S' phi(q)            [ / max(phi(q) . z', eps) when z is given ]
+//   delta rule       : S0 = done ? 0 : S ,  u = beta (v - S0 k) ,  S' = S0 + u k^T ,  o = S' q
+//
+// The state S:(B,H,64,64) fp32 ([dv][dk]) is read once and written once; everything else is a
+// few hundred bytes per sequence, so the kernels are bound by HBM traffic of the state
+// (32 KiB per (b,h)).  One workgroup of 256 threads per (b,h): thread t owns the four
+// consecutive dk = 4 (t & 15).. of rows dv = (t >> 4) + 16 p, p = 0..3, so that every load and
+// store of S is a fully coalesced 16-byte access; row dot products reduce over 16 lanes.
+// Follows what Memoroid.__call__ computes for T = 1 (memoroid.py:93-109 with the cell algebra of
+// linear_attention.py:62-117) and the delta-rule recurrence of the chunked kernels.
+#include "chunk_common.h"
+
+namespace {
+
+using namespace mrx;
+
+__device__ __forceinline__ float reduce16(float x)
+{
+    x += __shfl_xor(x, 1);
+    x += __shfl_xor(x, 2);
+    x += __shfl_xor(x, 4);
+    x += __shfl_xor(x, 8);
+    return x;
+}
+
+template <typename T> __device__ __forceinline__ f32x4 load4(const T *p);
+template <> __device__ __forceinline__ f32x4 load4<float>(const float *p) { return *reinterpret_cast<const f32x4 *>(p); }
+template <> __device__ __forceinline__ f32x4 load4<__bf16>(const __bf16 *p)
+{
+    const bf16x4 x = *reinterpret_cast<const bf16x4 *>(p);
+    return f32x4{(float)x[0], (float)x[1], (float)x[2], (float)x[3]};
+}
+
+__device__ __forceinline__ float dot4(const f32x4 &a, const f32x4 &b)
+{
+    return a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
+}
+
+template <typename T, bool DELTA, bool FMAP>
+__global__ void __launch_bounds__(256)
+step_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
+            const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
+            const float *S_in, const float *z_in, T *__restrict__ o, float *S_out, float *z_out, int H,
+            float eps)  // S_in/S_out and z_in/z_out may alias (update in place)
+{
+    const int tid = threadIdx.x, c4 = tid & 15, r0 = tid >> 4;
+    const int64_t bh = blockIdx.x;
+    const int b = (int)(bh / H);
+    const bool reset = done_at(done, done_f32, b);
+    const T *qp = q + bh * HD, *kp = k + bh * HD, *vp = v + bh * HD;
+
+    f32x4 k4 = load4<T>(kp + 4 * c4), q4 = load4<T>(qp + 4 * c4);
+    if (FMAP) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            k4[e] = elu1(k4[e]);
+            q4[e] = elu1(q4[e]);
+        }
+    }
+    const float *Sp = S_in ? S_in + bh * HD * HD : nullptr;
+    f32x4 s[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int row = r0 + 16 * p;
+        s[p] = (Sp && !reset) ? *reinterpret_cast<const f32x4 *>(Sp + row * HD + 4 * c4) : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    float u[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) u[p] = (float)vp[r0 + 16 * p];
+    if (DELTA) {
+        const float bb = (float)beta[bh];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) u[p] = bb * (u[p] - reduce16(dot4(s[p], k4)));
+    }
+    float den = 1.f;
+    if (!DELTA && z_out) {
+        // every 16-lane group recomputes the normaliser of the sequence; group 0 stores it
+        f32x4 z4 = (z_in && !reset) ? *reinterpret_cast<const f32x4 *>(z_in + bh * HD + 4 * c4) : f32x4{0.f, 0.f, 0.f, 0.f};
+        z4 += k4;
+        if (r0 == 0) *reinterpret_cast<f32x4 *>(z_out + bh * HD + 4 * c4) = z4;
+        den = fmaxf(reduce16(dot4(z4, q4)), eps);
+    }
+    float *So = S_out + bh * HD * HD;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int row = r0 + 16 * p;
+        s[p] += k4 * u[p];
+        *reinterpret_cast<f32x4 *>(So + row * HD + 4 * c4) = s[p];
+        const float x = reduce16(dot4(s[p], q4));
+        if (c4 == 0) o[bh * HD + row] = (T)(x / den);
+    }
+}
+
+int check_step(const void *q, const void *k, const void *v, const void *done, const void *S_in,
+               const void *o, const void *S_out, int64_t B, int64_t H, int64_t dk, int64_t dv, int dtype,
+               int done_dtype)
+{
+    if (!q || !k || !v || !done || !o || !S_out) return MRX_ERR_INVALID_ARG;
+    if (B <= 0 || H <= 0 || dk <= 0 || dv <= 0) return MRX_ERR_INVALID_ARG;
+    if (dtype != MRX_F32 && dtype != MRX_BF16) return dtype == MRX_C64 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
+    if (done_dtype != MRX_DONE_U8 && done_dtype != MRX_DONE_F32) return MRX_ERR_INVALID_ARG;
+    if (dk != HD || dv != HD) return MRX_ERR_UNSUPPORTED;
+    if (B * H >= (1ll << 31)) return MRX_ERR_INVALID_ARG;
+    const void *ps[] = {q, k, v, S_in, o, S_out};
+    for (const void *p : ps)
+        if (!aligned(p, 16)) return MRX_ERR_INVALID_ARG;
+    if (done_dtype == MRX_DONE_F32 && !aligned(done, 4)) return MRX_ERR_INVALID_ARG;
+    return MRX_OK;
+}
+
+template <typename T, bool DELTA, bool FMAP>
+int launch_step(hipStream_t st, const void *q, const void *k, const void *v, const void *beta, const void *done,
+                int done_f32, const float *S_in, const float *z_in, void *o, float *S_out, float *z_out,
+                int64_t B, int64_t H, float eps)
+{
+    hipLaunchKernelGGL((step_kernel<T, DELTA, FMAP>), dim3((unsigned)(B * H)), dim3(256), 0, st, (const T *)q,
+                       (const T *)k, (const T *)v, (const T *)beta, done, done_f32, S_in, z_in, (T *)o, S_out,
+                       z_out, (int)H, eps);
+    return launch_status();
+}
+
+}  // namespace
+
+extern "C" int mrx_linear_attn_step(void *stream, const void *q, const void *k, const void *v, const void *done,
+                                    const float *S_in, const float *z_in, void *o, float *S_out, float *z_out,
+                                    int64_t B, int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype,
+                                    int feature_map, float eps)
+{
+    const int rc = check_step(q, k, v, done, S_in, o, S_out, B, H, dk, dv, dtype, done_dtype);
+    if (rc != MRX_OK) return rc;
+    if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
+    if ((z_in && !z_out) || !aligned(z_in, 16) || !aligned(z_out, 16)) return MRX_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const bool fm = feature_map == MRX_FMAP_ELU1;
+    const int df = done_dtype == MRX_DONE_F32;
+#define MRX_ARGS st, q, k, v, nullptr, done, df, S_in, z_in, o, S_out, z_out, B, H, eps
+    if (dtype == MRX_BF16) return fm ? launch_step<__bf16, false, true>(MRX_ARGS) : launch_step<__bf16, false, false>(MRX_ARGS);
+    return fm ? launch_step<float, false, true>(MRX_ARGS) : launch_step<float, false, false>(MRX_ARGS);
+#undef MRX_ARGS
+}
+
+extern "C" int mrx_delta_rule_step(void *stream, const void *q, const void *k, const void *v, const void *beta,
+                                   const void *done, const float *S_in, void *o, float *S_out, int64_t B,
+                                   int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype)
+{
+    const int rc = check_step(q, k, v, done, S_in, o, S_out, B, H, dk, dv, dtype, done_dtype);
+    if (rc != MRX_OK) return rc;
+    if (!beta) return MRX_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const int df = done_dtype == MRX_DONE_F32;
+    if (dtype == MRX_BF16)
+        return launch_step<__bf16, true, false>(st, q, k, v, beta, done, df, S_in, nullptr, o, S_out, nullptr, B, H, 0.f);
+    return launch_step<float, true, false>(st, q, k, v, beta, done, df, S_in, nullptr, o, S_out, nullptr, B, H, 0.f);
+}

@@ -15,6 +15,7 @@ import torch
 from . import kernels as K
 
 _FMAP = {None: 0, "none": 0, 0: 0, "elu1": 1, 1: 1}
+_FMAP_NAME = {0: "none", 1: "elu1"}
 
 
 class _LinearScan(torch.autograd.Function):
@@ -59,6 +60,11 @@ class _LinearAttention(torch.autograd.Function):
         q_, k_, v_ = q.contiguous(), k.contiguous(), v.contiguous()
         S0_ = None if S0 is None else S0.contiguous().float()
         need = any(ctx.needs_input_grad)
+        if q_.shape[1] == 1 and not need:  # acting: one step, no residuals (memoroid.py:93-109 with T = 1)
+            o, S_last, _ = K.linear_attn_step(q_[:, 0], k_[:, 0], v_[:, 0], done[:, 0], S0_,
+                                              feature_map=_FMAP_NAME[fmap])
+            ctx.done, ctx.fmap, ctx.has_S0 = done, fmap, S0 is not None
+            return o[:, None], S_last
         o, S_last, S_chk = K.linear_attn_fwd(q_, k_, v_, done, S0_, fmap, save_chk=need)
         if need:
             ctx.save_for_backward(q_, k_, v_, S_chk)
@@ -87,6 +93,10 @@ class _DeltaRule(torch.autograd.Function):
         q_, k_, v_, b_ = q.contiguous(), k.contiguous(), v.contiguous(), beta.contiguous()
         S0_ = None if S0 is None else S0.contiguous().float()
         need = any(ctx.needs_input_grad)
+        if q_.shape[1] == 1 and not need:  # acting: one step, no residuals
+            o, S_last = K.delta_rule_step(q_[:, 0], k_[:, 0], v_[:, 0], b_[:, 0], done[:, 0], S0_)
+            ctx.done, ctx.has_S0 = done, S0 is not None
+            return o[:, None], S_last
         o, S_last, chk = K.delta_rule_fwd(q_, k_, v_, b_, done, S0_, save_chk=need)
         if need:
             ctx.save_for_backward(q_, k_, v_, b_, *chk)

@@ -198,3 +198,55 @@ def delta_rule_bwd(q, k, v, beta, done, chk, do, dS_last=None, want_dS0=True):
                                 _ptr(dv_), _ptr(dbeta), _ptr(dS0), B, T, H, dk, dv, _DT[dt], dd)
     _lib.check(st, "mrx_delta_rule_bwd")
     return dq, dk_, dv_, dbeta, dS0
+
+
+# ------------------------------------------------------------- single time step
+def _step_shapes(q, k, v):
+    if q.dim() != 3:
+        raise ValueError(f"q must be (B,H,d), got {tuple(q.shape)}")
+    B, H, dk = q.shape
+    dv = v.shape[-1]
+    dt = q.dtype
+    if dt not in (torch.float32, torch.bfloat16):
+        raise ValueError(f"unsupported dtype {dt}")
+    _chk(q, "q", dt, (B, H, dk))
+    _chk(k, "k", dt, (B, H, dk))
+    _chk(v, "v", dt, (B, H, dv))
+    return B, H, dk, dv, dt
+
+
+def linear_attn_step(q, k, v, done, S=None, z=None, feature_map="none", normalise=False, eps=1e-6,
+                     inplace=False):
+    """One time step.  q,k,v: (B,H,d); done: (B,); S: (B,H,dv,dk) fp32 or None; z: (B,H,dk) fp32 or
+    None.  Returns (o, S_new, z_new) (z_new None unless normalise).  inplace updates S and z."""
+    lib = _lib.load()
+    B, H, dk, dv, dt = _step_shapes(q, k, v)
+    _chk(S, "S", torch.float32, (B, H, dv, dk))
+    _chk(z, "z", torch.float32, (B, H, dk))
+    done, dd = _done(done.reshape(B, 1), B, 1)
+    o = torch.empty_like(v)
+    S_new = S if (inplace and S is not None) else torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
+    z_new = None
+    if normalise:
+        z_new = z if (inplace and z is not None) else torch.empty((B, H, dk), dtype=torch.float32, device=q.device)
+    fm = {"none": _lib.MRX_FMAP_NONE, "elu1": _lib.MRX_FMAP_ELU1}[feature_map]
+    st = lib.mrx_linear_attn_step(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(done), _ptr(S),
+                                  _ptr(z) if normalise else None, _ptr(o), _ptr(S_new), _ptr(z_new),
+                                  B, H, dk, dv, _DT[dt], dd, fm, float(eps))
+    _lib.check(st, "mrx_linear_attn_step")
+    return o, S_new, z_new
+
+
+def delta_rule_step(q, k, v, beta, done, S=None, inplace=False):
+    """One time step of the delta rule.  beta: (B,H).  Returns (o, S_new)."""
+    lib = _lib.load()
+    B, H, dk, dv, dt = _step_shapes(q, k, v)
+    _chk(beta, "beta", dt, (B, H))
+    _chk(S, "S", torch.float32, (B, H, dv, dk))
+    done, dd = _done(done.reshape(B, 1), B, 1)
+    o = torch.empty_like(v)
+    S_new = S if (inplace and S is not None) else torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
+    st = lib.mrx_delta_rule_step(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done), _ptr(S),
+                                 _ptr(o), _ptr(S_new), B, H, dk, dv, _DT[dt], dd)
+    _lib.check(st, "mrx_delta_rule_step")
+    return o, S_new

@@ -278,6 +278,22 @@ class LinearAttentionCell(MemoroidCellBase):
         out = (num.float() / den).reshape(*x.shape[:2], -1)
         return self.output_projection(self.norm(out).to(x.dtype))
 
+    def step(self, x, done, carry):
+        """Acting path (T = 1, no gradients): state update, normaliser and divide in one kernel
+        (what __call__, binary_operator and read of linear_attention.py:62-117 do for one step)."""
+        from . import kernels as K
+        S0, z0 = carry
+        v, k_raw = self(x)
+        q = self._heads(self.query(x))
+        B = x.shape[0]
+        o, S_new, z_new = K.linear_attn_step(
+            q[:, 0].contiguous(), k_raw[:, 0].contiguous(), v[:, 0].contiguous(), done.reshape(B),
+            S0[:, 0].float().contiguous(), z0[:, 0].float().contiguous(), feature_map="elu1",
+            normalise=True, eps=self.eps)
+        out = o.float().reshape(B, 1, -1)
+        y = self.output_projection(self.norm(out).to(x.dtype))
+        return (S_new[:, None], z_new[:, None]), y
+
     def initialize_carry(self, key, input_shape):
         *batch, _ = input_shape
         dev = self.key.weight.device
@@ -296,6 +312,8 @@ class LinearAttention(SequenceModel):
     def forward(self, inputs, done, initial_carry=None, **kwargs):
         if initial_carry is None:
             initial_carry = self.cell.initialize_carry(None, get_input_shape(inputs))
+        if inputs.shape[1] == 1 and not torch.is_grad_enabled():
+            return self.cell.step(inputs, done, initial_carry)
         z = self.cell(inputs)
         h, z_last = self.cell.scan(z, initial_carry, done)
         y = self.cell.read(h, inputs)

@@ -111,3 +111,26 @@ def test_deltanet_stack_carries_and_split_invariance():
     assert relerr(torch.cat([y1, y2], 1), _np(y)) <= 2e-2
     y.float().pow(2).mean().backward()
     assert all(torch.isfinite(p.grad).all() for p in stack.parameters() if p.grad is not None)
+
+
+def test_rollout_steps_equal_sequence_call():
+    """Acting (T = 1 calls under no_grad, carry fed back) takes the single-step kernels and must
+    give what one call over the whole sequence gives (memoroid.py:93-109 is the same code for both)."""
+    from memorax_amd import sequence_models as sm
+    torch.manual_seed(5)
+    B, T, Fe, H, d = 3, 20, 32, 2, 64
+    x, done = _inputs(B, T, Fe, 0.1, 6)
+    la = sm.LinearAttention(sm.LinearAttentionCell(Fe, d, H).cuda())
+    dn = sm.Memoroid(sm.DeltaNetCell(Fe, d, H, dtype=torch.float32)).cuda()
+    for model, tol in ((la, 2e-4), (dn, 2e-4)):
+        with torch.no_grad():
+            carry_seq, y_seq = model(x, done)
+            carry, ys = None, []
+            for t in range(T):
+                carry, y = model(x[:, t:t + 1], done[:, t:t + 1], carry)
+                ys.append(y)
+        y_roll = torch.cat(ys, 1)
+        assert relerr(y_roll, _np(y_seq)) <= tol, relerr(y_roll, _np(y_seq))
+        for a, b_ in zip(carry, carry_seq):
+            assert a.shape == b_.shape
+            assert relerr(a, _np(b_)) <= tol

@@ -1,0 +1,144 @@
+"""GPU parity of the single-step (T = 1) kernels, through the C ABI, against the oracle recurrences.
+
+A rollout calls the step T times, feeding the state back; the outputs and the final state must
+equal what the oracle computes for the whole (B,T,...) sequence, resets included."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import memoroid as M
+from gpu_util import TOL_BF16, TOL_F32, attn_inputs, bf16_round, dev, relerr
+
+pytestmark = pytest.mark.gpu
+
+
+def _roll(step, T):
+    outs = []
+    for t in range(T):
+        outs.append(step(t))
+    return torch.stack(outs, dim=1)
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (3, 9, 2), (2, 17, 4)])
+@pytest.mark.parametrize("p", [0.0, 0.2])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("fmap", ["none", "elu1"])
+def test_linear_attention_step_rollout(shape, p, dtype, fmap):
+    from memorax_amd import kernels as K
+    B, T, H = shape
+    x = attn_inputs(B, T, H, p=p, seed=11 * B + T + H, scale=1.0 / 8)
+    print(f"case la_step shape={shape} p={p} dtype={dtype} fmap={fmap}", flush=True)
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    if dtype == "bf16":
+        for n in ("q", "k", "v"):
+            x[n] = bf16_round(x[n])
+    q, k, v, done = dev(x["q"], td), dev(x["k"], td), dev(x["v"], td), dev(x["done"])
+    state = {"S": dev(x["S0"])}
+
+    def step(t):
+        o, state["S"], _ = K.linear_attn_step(q[:, t].contiguous(), k[:, t].contiguous(), v[:, t].contiguous(),
+                                              done[:, t].contiguous(), state["S"], feature_map=fmap)
+        return o
+
+    o = _roll(step, T)
+    ro, rS = M.linear_attention(x["q"], x["k"], x["v"], x["done"], x["S0"], fmap)
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    assert relerr(o, ro) <= tol, relerr(o, ro)
+    assert relerr(state["S"], rS) <= (1e-5 if dtype == "f32" else tol), relerr(state["S"], rS)
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (3, 9, 2), (2, 17, 4)])
+@pytest.mark.parametrize("p", [0.0, 0.2])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_delta_rule_step_rollout(shape, p, dtype):
+    from memorax_amd import kernels as K
+    B, T, H = shape
+    x = attn_inputs(B, T, H, p=p, seed=13 * B + T + H, delta=True)
+    print(f"case delta_step shape={shape} p={p} dtype={dtype}", flush=True)
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    if dtype == "bf16":
+        for n in ("q", "k", "v", "beta"):
+            x[n] = bf16_round(x[n])
+    q, k, v, beta = (dev(x[n], td) for n in ("q", "k", "v", "beta"))
+    done = dev(x["done"])
+    state = {"S": dev(x["S0"])}
+
+    def step(t):
+        o, state["S"] = K.delta_rule_step(q[:, t].contiguous(), k[:, t].contiguous(), v[:, t].contiguous(),
+                                          beta[:, t].contiguous(), done[:, t].contiguous(), state["S"])
+        return o
+
+    o = _roll(step, T)
+    ro, rS = M.delta_rule(x["q"], x["k"], x["v"], x["beta"], x["done"], x["S0"])
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    assert relerr(o, ro) <= tol, relerr(o, ro)
+    assert relerr(state["S"], rS) <= (1e-5 if dtype == "f32" else tol), relerr(state["S"], rS)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_linear_attention_step_normalised(dtype):
+    """Fused denominator of LinearAttentionCell.read: o = S q / max(q . z, eps), z the running sum of phi(k)."""
+    from memorax_amd import kernels as K
+    B, T, H, d = 2, 12, 3, 64
+    x = attn_inputs(B, T, H, p=0.15, seed=5, scale=1.0 / 8)
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    if dtype == "bf16":
+        for n in ("q", "k", "v"):
+            x[n] = bf16_round(x[n])
+    q, k, v, done = dev(x["q"], td), dev(x["k"], td), dev(x["v"], td), dev(x["done"])
+    z0 = np.abs(np.random.default_rng(1).standard_normal((B, H, d))).astype(np.float32)
+    S, z = dev(x["S0"]), dev(z0)
+    outs = []
+    for t in range(T):
+        o, S, z = K.linear_attn_step(q[:, t].contiguous(), k[:, t].contiguous(), v[:, t].contiguous(),
+                                     done[:, t].contiguous(), S, z, feature_map="elu1", normalise=True, eps=1e-6)
+        outs.append(o)
+    o = torch.stack(outs, dim=1)
+    # oracle: numerator from the recurrence, normaliser = segmented running sum of phi(k) with carry z0
+    num, _ = M.linear_attention(x["q"], x["k"], x["v"], x["done"], x["S0"], "elu1")
+    fk, fq = M.elu1(x["k"].astype(np.float64)), M.elu1(x["q"].astype(np.float64))
+    zz = z0.astype(np.float64).copy()
+    ref = np.zeros_like(num)
+    for t in range(T):
+        zz = np.where(x["done"][:, t, None, None], 0.0, zz) + fk[:, t]
+        den = np.maximum((fq[:, t] * zz).sum(-1, keepdims=True), 1e-6)
+        ref[:, t] = num[:, t] / den
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    assert relerr(o, ref) <= tol, relerr(o, ref)
+    assert relerr(z, zz) <= 1e-5, relerr(z, zz)
+
+
+def test_step_inplace_zero_state_and_float_done():
+    from memorax_amd import kernels as K
+    B, H, d = 4, 2, 64
+    x = attn_inputs(B, 1, H, p=0.0, seed=3, delta=True)
+    q, k, v, beta = (dev(x[n][:, 0]) for n in ("q", "k", "v", "beta"))
+    done_f = torch.tensor([0.0, 1.0, 0.0, 1.0], device="cuda")
+    S = dev(x["S0"])
+    S_keep = S.clone()
+    o_ref, S_ref = K.delta_rule_step(q, k, v, beta, done_f, S)          # out of place, float32 done
+    assert torch.equal(S, S_keep)
+    o2, S2 = K.delta_rule_step(q, k, v, beta, done_f != 0, S, inplace=True)  # in place, bool done
+    assert S2.data_ptr() == S.data_ptr()
+    assert torch.equal(o2, o_ref) and torch.equal(S, S_ref)
+    # rows whose done flag is set behave as if the state were absent
+    o3, S3 = K.delta_rule_step(q, k, v, beta, torch.zeros(B, device="cuda"), None)
+    assert torch.equal(o3[1], o_ref[1]) and torch.equal(S3[3], S_ref[3])
+    # one step equals the chunked forward kernel at T = 1
+    o4, S4, _ = K.delta_rule_fwd(q[:, None].contiguous(), k[:, None].contiguous(), v[:, None].contiguous(),
+                                 beta[:, None].contiguous(), (done_f != 0)[:, None], S_keep, save_chk=False)
+    assert relerr(o4[:, 0], o_ref.cpu().numpy()) <= 1e-5
+    assert relerr(S4, S_ref.cpu().numpy()) <= 1e-5
+
+
+def test_step_rejects_bad_arguments():
+    from memorax_amd import _lib
+    lib = _lib.load()
+    t = torch.zeros(64 * 64, device="cuda")
+    p = t.data_ptr()
+    args = lambda dk: (None, p, p, p, p, p, p, p, p, 1, 1, dk, 64, 0, 0)
+    assert lib.mrx_delta_rule_step(*args(64)) == 0
+    assert lib.mrx_delta_rule_step(*args(32)) == -2          # unsupported head dim
+    assert lib.mrx_delta_rule_step(None, p, p, p, None, p, p, p, p, 1, 1, 64, 64, 0, 0) == -1  # beta missing
+    assert lib.mrx_linear_attn_step(None, p, p, p, p, p, None, p, p, None, 1, 1, 64, 64, 0, 0, 7, 1e-6) == -1
+    torch.cuda.synchronize()
