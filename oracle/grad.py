@@ -66,6 +66,20 @@ def linear_attention_t(q, k, v, done, S0, feature_map="none"):
     return torch.stack(os_, 1), S
 
 
+def gated_linear_attention_t(q, k, v, g, done, S0, feature_map="none"):
+    if feature_map in ("elu1", 1):
+        q, k = elu1_t(q), elu1_t(k)
+    B, T, H, dk = q.shape
+    S = S0
+    os_ = []
+    for t in range(T):
+        r = done[:, t][:, None, None, None]
+        S = torch.where(r, torch.zeros_like(S), torch.exp(g[:, t])[:, :, None, None] * S)
+        S = S + torch.einsum("bhi,bhj->bhij", v[:, t], k[:, t])
+        os_.append(torch.einsum("bhij,bhj->bhi", S, q[:, t]))
+    return torch.stack(os_, 1), S
+
+
 def delta_rule_t(q, k, v, beta, done, S0):
     B, T, H, dk = q.shape
     S = S0
@@ -121,3 +135,17 @@ def delta_rule_grads(q, k, v, beta, done, S0, do, dS_last=None):
     L.backward()
     return dict(o=_np(o), S_last=_np(Sl), dq=_np(q_.grad), dk=_np(k_.grad),
                 dv=_np(v_.grad), dbeta=_np(b_.grad), dS0=_np(S0_.grad))
+
+
+def gated_linear_attention_grads(q, k, v, g, done, S0, do, dS_last=None, feature_map="none"):
+    """Returns dict(o, S_last, dq, dk, dv, dg, dS0) for L = sum(do*o) + sum(dS_last*S_last)."""
+    q_, k_, v_, g_ = _t(q, True), _t(k, True), _t(v, True), _t(g, True)
+    B, T, H, dk = q_.shape
+    S0_ = _t(np.zeros((B, H, v_.shape[-1], dk)) if S0 is None else S0, True)
+    o, Sl = gated_linear_attention_t(q_, k_, v_, g_, _done(done), S0_, feature_map)
+    L = (o * _t(do)).sum()
+    if dS_last is not None:
+        L = L + (Sl * _t(dS_last)).sum()
+    L.backward()
+    return dict(o=_np(o), S_last=_np(Sl), dq=_np(q_.grad), dk=_np(k_.grad), dv=_np(v_.grad),
+                dg=_np(g_.grad), dS0=_np(S0_.grad))

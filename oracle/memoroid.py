@@ -319,6 +319,66 @@ def linear_attention_memoroid(q, k, v, done, carry=None, feature_map="none"):
     return nxt, num, den
 
 
+def gated_linear_attention(q, k, v, g, done, S0=None, feature_map="none"):
+    """Recurrent form with a scalar log-decay per step and head:
+        S_t = r_t exp(g_t) S_{t-1} + v_t k_t^T ;  o_t = S_t q_t.
+    This is the Mamba cell's algebra (mamba.py:109-122: elements (h = (B dt) (x) x,
+    decay = exp(dt A)), binary_operator (decay_j h_i + h_j, decay_j decay_i)) with
+    k = B dt, v = x, q = C and the state stored as (d_v, d_k); g = log decay (B,T,H)."""
+    q = _fmap(q, feature_map)
+    k = _fmap(k, feature_map)
+    v = np.asarray(v, dtype=np.float64)
+    g = np.asarray(g, dtype=np.float64)
+    B, T, H, dk = q.shape
+    dv = v.shape[-1]
+    S = np.zeros((B, H, dv, dk)) if S0 is None else np.asarray(S0, np.float64).copy()
+    done = np.asarray(done) != 0
+    o = np.empty((B, T, H, dv))
+    for t in range(T):
+        r = done[:, t][:, None, None, None]
+        S = np.where(r, 0.0, np.exp(g[:, t])[:, :, None, None] * S)
+        S = S + np.einsum("bhi,bhj->bhij", v[:, t], k[:, t])
+        o[:, t] = np.einsum("bhij,bhj->bhi", S, q[:, t])
+    return o, S
+
+
+def gated_linear_attention_memoroid(q, k, v, g, done, carry=None):
+    """The reference's own route for the Mamba cell: materialise h_t = v_t k_t^T and the decay leaf
+    and scan them with the diagonal operator (mamba.py:109-122 under memoroid.py:60-91).
+    Returns (next_carry, o) with carry = (S (B,1,H,dv,dk), decay (B,1,H,1,1))."""
+    q, k, v, g = (np.asarray(x, np.float64) for x in (q, k, v, g))
+    B, T, H, dk = q.shape
+    dv = v.shape[-1]
+    h = np.einsum("bthi,bthj->bthij", v, k)
+    decay = np.exp(g)[..., None, None]
+    if carry is None:
+        carry = (np.zeros((B, 1, H, dv, dk)), np.ones((B, 1, H, 1, 1)))
+    (Sc, _), nxt = scan_fn_tree((h, np.broadcast_to(decay, h.shape).copy()), (carry[0], np.broadcast_to(carry[1], carry[0].shape).copy()), done, diag_operator)
+    o = np.einsum("bthij,bthj->bthi", Sc, q)
+    return nxt, o
+
+
+def gated_linear_attention_quadratic(q, k, v, g, done, S0=None, feature_map="none"):
+    """Masked-matmul form: o_i = sum_{j<=i, same episode} exp(G_i - G_j) (q_i . k_j) v_j
+    + [episode 0] exp(G_i) S0 q_i, with G the cumulative sum of g inside the episode (the
+    decay of an episode's first step multiplies a zero state and drops out)."""
+    q = _fmap(q, feature_map)
+    k = _fmap(k, feature_map)
+    v = np.asarray(v, dtype=np.float64)
+    g = np.asarray(g, dtype=np.float64)
+    B, T, H, dk = q.shape
+    seg = segment_ids(done)
+    Gc = np.cumsum(g, axis=1)                                 # (B,T,H) global cumulative sum
+    M = (seg[:, :, None] == seg[:, None, :]) & np.tril(np.ones((T, T), bool))[None]
+    D = np.exp(np.where(M[:, None], (Gc.transpose(0, 2, 1)[:, :, :, None] - Gc.transpose(0, 2, 1)[:, :, None, :]), -np.inf))
+    A = np.einsum("bihd,bjhd->bhij", q, k) * D
+    o = np.einsum("bhij,bjhe->bihe", A, v)
+    if S0 is not None:
+        m = (seg == 0)[:, :, None, None]
+        o = o + m * np.exp(Gc)[..., None] * np.einsum("bihd,bhed->bihe", q, np.asarray(S0, np.float64))
+    return o
+
+
 def segment_ids(done):
     """Inclusive cumsum of done along time: rows with equal id share an episode."""
     return np.cumsum(np.asarray(done) != 0, axis=1)

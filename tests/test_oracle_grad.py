@@ -101,3 +101,45 @@ def test_delta_rule_grads_fd():
     ag = G.delta_rule_grads(q, k, v, beta, d, S0, do, dSl)
     for name, x in (("dq", q), ("dk", k), ("dv", v), ("dbeta", beta), ("dS0", S0)):
         np.testing.assert_allclose(ag[name], fd(L, x), rtol=1e-6, atol=1e-8, err_msg=name)
+
+
+def test_gated_linear_attention_grads_finite_differences_and_rowdot_identity():
+    """dg equals, inside each episode, the suffix sum of q_t . dq_t - k_t . dk_t (what the kernels
+    use); all gradients agree with central finite differences."""
+    from oracle import grad as G
+    rng = np.random.default_rng(4)
+    B, T, H, d = 1, 7, 2, 3
+    q, k, v = (rng.standard_normal((B, T, H, d)) for _ in range(3))
+    g = -np.abs(rng.standard_normal((B, T, H))) * 0.4
+    done = np.zeros((B, T), bool)
+    done[0, 3] = True
+    S0 = rng.standard_normal((B, H, d, d))
+    do = rng.standard_normal((B, T, H, d))
+    dSl = rng.standard_normal((B, H, d, d))
+    r = G.gated_linear_attention_grads(q, k, v, g, done, S0, do, dSl)
+
+    def loss(q_, k_, v_, g_, S0_):
+        o, S = M.gated_linear_attention(q_, k_, v_, g_, done, S0_)
+        return (o * do).sum() + (S * dSl).sum()
+
+    eps = 1e-6
+    for name, arr in (("dq", q), ("dk", k), ("dv", v), ("dg", g), ("dS0", S0)):
+        idx = tuple(rng.integers(0, s) for s in arr.shape)
+        args = dict(q_=q, k_=k, v_=v, g_=g, S0_=S0)
+        key = {"dq": "q_", "dk": "k_", "dv": "v_", "dg": "g_", "dS0": "S0_"}[name]
+        up, dn = arr.copy(), arr.copy()
+        up[idx] += eps
+        dn[idx] -= eps
+        fd = (loss(**{**args, key: up}) - loss(**{**args, key: dn})) / (2 * eps)
+        assert abs(fd - r[name][idx]) <= 1e-6 * max(1.0, abs(fd)), (name, fd, r[name][idx])
+    e = (q * r["dq"]).sum(-1) - (k * r["dk"]).sum(-1)      # (B,T,H)
+    # the final state's own dependence on g enters through dS_last: include it
+    _, S_last = M.gated_linear_attention(q, k, v, g, done, S0)
+    tail = (S_last * dSl).sum((-1, -2))                    # d/dG_last of <S_last, dS_last>
+    ref = np.zeros_like(g)
+    acc = tail.copy()
+    for t in range(T - 1, -1, -1):
+        acc = acc + e[:, t]
+        ref[:, t] = np.where(done[:, t][:, None], 0.0, acc)
+        acc = np.where(done[:, t][:, None], 0.0, acc)
+    np.testing.assert_allclose(r["dg"], ref, rtol=1e-9, atol=1e-9)

@@ -270,3 +270,59 @@ def test_make_inputs_shapes_and_determinism():
         np.testing.assert_array_equal(x[key], y[key])
     np.testing.assert_allclose(np.linalg.norm(x["k"], axis=-1), 1.0, rtol=1e-5)
     assert M.make_inputs(1)["a"].shape == (32, 128, 256)
+
+
+# ---- gated linear attention (the Mamba cell's algebra) -------------------------------------
+def _gla_inputs(B=2, T=13, H=2, d=4, p=0.2, seed=0):
+    rng = np.random.default_rng(seed)
+    q, k, v = (rng.standard_normal((B, T, H, d)) for _ in range(3))
+    g = -np.abs(rng.standard_normal((B, T, H))) * 0.5
+    done = rng.random((B, T)) < p
+    S0 = rng.standard_normal((B, H, d, d))
+    return q, k, v, g, done, S0
+
+
+def test_gated_linear_attention_forms_agree():
+    q, k, v, g, done, S0 = _gla_inputs()
+    o, S = M.gated_linear_attention(q, k, v, g, done, S0)
+    oq = M.gated_linear_attention_quadratic(q, k, v, g, done, S0)
+    np.testing.assert_allclose(o, oq, rtol=1e-11, atol=1e-11)
+    carry = (S0[:, None], np.ones((2, 1, 2, 1, 1)))
+    nxt, om = M.gated_linear_attention_memoroid(q, k, v, g, done, carry)
+    np.testing.assert_allclose(o, om, rtol=1e-11, atol=1e-11)
+    np.testing.assert_allclose(S, nxt[0][:, 0], rtol=1e-11, atol=1e-11)
+
+
+def test_gated_linear_attention_special_cases():
+    q, k, v, g, done, S0 = _gla_inputs(seed=1)
+    # zero log-decay is plain linear attention
+    o0, S0l = M.gated_linear_attention(q, k, v, 0 * g, done, S0)
+    o1, S1l = M.linear_attention(q, k, v, done, S0)
+    np.testing.assert_allclose(o0, o1, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(S0l, S1l, rtol=1e-12, atol=1e-12)
+    # constant decay, k = q = e_1, no resets: o[..., i] is a first-order IIR filter of v[..., i]
+    from scipy.signal import lfilter
+    B, T, H, d = q.shape
+    e1 = np.zeros_like(q)
+    e1[..., 0] = 1.0
+    a = 0.8
+    o, _ = M.gated_linear_attention(e1, e1, v, np.full_like(g, np.log(a)), np.zeros((B, T), bool))
+    ref = lfilter([1.0], [1.0, -a], v, axis=1)
+    np.testing.assert_allclose(o, ref, rtol=1e-11, atol=1e-11)
+    # the decay of an episode's first step has no effect
+    g2 = g.copy()
+    g2[done] = -7.0
+    oa, Sa = M.gated_linear_attention(q, k, v, g, done, None)
+    ob, Sb = M.gated_linear_attention(q, k, v, g2, done, None)
+    bt0 = np.cumsum(done, 1) > 0    # steps whose history does not reach the carry
+    np.testing.assert_allclose(oa[bt0], ob[bt0], rtol=1e-12, atol=1e-12)
+
+
+def test_gated_linear_attention_split_invariance():
+    q, k, v, g, done, S0 = _gla_inputs(T=11, seed=2)
+    o, S = M.gated_linear_attention(q, k, v, g, done, S0)
+    for s in range(1, 11):
+        o1, S1 = M.gated_linear_attention(q[:, :s], k[:, :s], v[:, :s], g[:, :s], done[:, :s], S0)
+        o2, S2 = M.gated_linear_attention(q[:, s:], k[:, s:], v[:, s:], g[:, s:], done[:, s:], S1)
+        np.testing.assert_allclose(np.concatenate([o1, o2], 1), o, rtol=1e-11, atol=1e-11)
+        np.testing.assert_allclose(S2, S, rtol=1e-11, atol=1e-11)
