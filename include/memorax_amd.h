@@ -136,6 +136,32 @@ int mrx_delta_rule_bwd(void *stream, const void *q, const void *k,
                        void *dbeta, void *dS0, int64_t B, int64_t T, int64_t H,
                        int64_t dk, int64_t dv, int dtype, int done_dtype);
 
+/* ---- Gated linear attention: linear attention with a scalar decay per step and head ----
+ * The Mamba cell's algebra (mamba.py:109-122: elements (h_t = (B_t dt_t) (x) x_t, decay_t =
+ * exp(dt_t A)), binary_operator (decay_j h_i + h_j, decay_j decay_i), read y_t = C_t . h_t), scanned
+ * by memoroid.py:60-91, with k = B dt, v = x, q = C and the state kept as (d_v, d_k):
+ *     S' = done_t ? 0 : exp(g_t) S_{t-1} ;  S_t = S' + v_t phi(k_t)^T ;  o_t = S_t phi(q_t)
+ * g: (B,T,H) float32 log-decay (<= 0 for a contracting state).  Other arguments as for
+ * mrx_linear_attn_fwd; S_chk is the residual for the backward call. */
+int mrx_gated_linear_attn_fwd(void *stream, const void *q, const void *k,
+                              const void *v, const void *g, const void *done,
+                              const void *S0, void *o, void *S_last, void *S_chk,
+                              int64_t B, int64_t T, int64_t H, int64_t dk, int64_t dv,
+                              int dtype, int done_dtype, int feature_map);
+
+/* Gradients w.r.t. q,k,v (pre-feature-map, in `dtype`) and S0 (fp32, nullable), and
+ * edot: (B,T,H) float32 with edot_t = phi(q_t) . dphi(q)_t - phi(k_t) . dphi(k)_t.  The gradient of
+ * the log-decay is its reverse cumulative sum inside each episode,
+ *     dg_t = done_t ? 0 : sum over i >= t of t's episode of edot_i  (+ <S_last, dS_last> when the
+ *     episode reaches the end),
+ * which the caller takes with mrx_linear_scan_fwd on the time-reversed array (decay 1). */
+int mrx_gated_linear_attn_bwd(void *stream, const void *q, const void *k,
+                              const void *v, const void *g, const void *done,
+                              const void *S_chk, const void *dout, const void *dS_last,
+                              void *dq, void *dk_out, void *dv_out, void *edot, void *dS0,
+                              int64_t B, int64_t T, int64_t H, int64_t dk, int64_t dv,
+                              int dtype, int done_dtype, int feature_map);
+
 /* ---- Single time step (rollout / acting) ------------------------------------
  * What Memoroid.__call__ (memoroid.py:93-109) computes when T = 1, as PPO's rollout
  * does once per environment step (algorithms/ppo.py:105-143): one update of the

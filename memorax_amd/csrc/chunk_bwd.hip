@@ -85,24 +85,34 @@ __device__ __forceinline__ void store_rows_at(const f32x4 *acc, T *row, int64_t 
 }
 
 // =====================================================================================
-// linear attention: 8 tiles, two workgroups per CU
+// linear attention: 8 tiles, two workgroups per CU; with a per-step decay (GATED) one tile more
 // =====================================================================================
-template <typename T, int C> struct LaBwdSmem : BwdDims<T, C> {
+template <typename T, int C, bool GATED = false> struct LaBwdSmem : BwdDims<T, C> {
     using D = BwdDims<T, C>;
     static constexpr int oQ = 0, oK = oQ + D::szRD, oV = oK + D::szRD, oDO = oV + D::szRD,
                          oS = oDO + D::szRD, oDS = oS + D::szDD, oAqk = oDS + D::szDD,
-                         oDAqk = oAqk + D::szCC, total = oDAqk + D::szCC;
+                         oDAqk = oAqk + D::szCC, oQa = oDAqk + D::szCC,    // gated: exp(G_i) Q_i
+                         oG = oQa + (GATED ? D::szRD : 0),                 // gated: G[C], then [WM][C] row-dot partials
+                         total = oG + (GATED ? (1 + TileMap<HD, C, 4>::WM) * C * 4 : 0);
 };
 
-template <typename T, int C, bool FMAP>
+// GATED: S_t = r_t exp(g_t) S_{t-1} + v_t k_t^T.  With G the cumulative log-decay inside the chunk
+// (per episode), a_i = exp(G_i), b_j = exp(G_last - G_j), c = exp(G_last), D_ij = exp(G_i - G_j):
+//   Aqk, dAqk carry the factor D;  dV = Aqk^T dO + diag(b) K dS^T;  dQ = diag(a) dO S + dAqk K;
+//   dK = dAqk^T Q + diag(b) V dS;  dS <- c dS + (diag(a) Q)^T dO.
+// The gradient of the log-decays follows from edot_i = q_i . dq_i - k_i . dk_i (taken on the
+// feature-mapped q, k and their gradients): dg_t is the sum of edot over the rows i >= t of t's
+// episode (plus <S_last, dS_last> at the end); the kernel writes edot, the caller sums.
+template <typename T, int C, bool FMAP, bool GATED>
 __global__ void __launch_bounds__(256, 2)
 la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
-              const void *__restrict__ done, int done_f32, const T *__restrict__ S_chk,
-              const T *__restrict__ dout, const float *__restrict__ dS_last, T *__restrict__ dq,
-              T *__restrict__ dk, T *__restrict__ dv, float *__restrict__ dS0, int Tlen, int H)
+              const float *__restrict__ glog, const void *__restrict__ done, int done_f32,
+              const T *__restrict__ S_chk, const T *__restrict__ dout, const float *__restrict__ dS_last,
+              T *__restrict__ dq, T *__restrict__ dk, T *__restrict__ dv, float *__restrict__ edot,
+              float *__restrict__ dS0, int Tlen, int H)
 {
     constexpr int NW = 4, NTHR = 64 * NW;
-    using L = LaBwdSmem<T, C>;
+    using L = LaBwdSmem<T, C, GATED>;
     using IO = TileIO<T, C, NTHR>;
     using IOS = TileIO<T, HD, NTHR>;
     using P4 = typename TT<T>::pack4;
@@ -116,6 +126,9 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     T *sDS = reinterpret_cast<T *>(smem + L::oDS);
     T *sAqk = reinterpret_cast<T *>(smem + L::oAqk);
     T *sDAqk = reinterpret_cast<T *>(smem + L::oDAqk);
+    T *sQa = reinterpret_cast<T *>(smem + L::oQa);
+    float *sG = reinterpret_cast<float *>(smem + L::oG);
+    float *sE = sG + C;  // [WM][C] partial row dots
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -139,6 +152,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     typename IO::Regs rq, rk, rv, rdo;
     typename IOS::Regs rS;
     uint32_t rdone = 0u;  // raw bits, tested when the chunk is staged
+    float rg = 0.f;       // log-decay of chunk row `lane` (gated)
     auto prefetch = [&](int c) {
         const int t0 = c * C;
         IO::load(rq, q + base, rs, t0, Tlen, tid);
@@ -147,7 +161,11 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
         IO::load(rdo, dout + base, rs, t0, Tlen, tid);
         IOS::load(rS, S_chk + ((int64_t)bh * NC + c) * HD * HD, HD, 0, HD, tid);
         rdone = 0u;
-        if (lane < C && t0 + lane < Tlen) rdone = done_raw(done, done_f32, (int64_t)b * Tlen + t0 + lane);
+        rg = 0.f;
+        if (lane < C && t0 + lane < Tlen) {
+            rdone = done_raw(done, done_f32, (int64_t)b * Tlen + t0 + lane);
+            if (GATED) rg = glog[((int64_t)b * Tlen + t0 + lane) * H + h];
+        }
     };
     prefetch(NC - 1);
 
@@ -157,6 +175,18 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
         const int nres = __popcll(dmask);
         for (int pass = nres; pass >= 0; --pass) {
             auto live = [&](int r) { return nres == 0 || episode_of(dmask, r) == pass; };
+            // gated: cumulative log-decay of this pass's episode (as in the forward kernel)
+            float G = 0.f, Glast = 0.f;
+            if (GATED) {
+                G = (lane < C && live(lane) && !((dmask >> lane) & 1ull)) ? rg : 0.f;
+#pragma unroll
+                for (int off = 1; off < C; off <<= 1) {
+                    const float up = __shfl_up(G, off);
+                    if (lane >= off) G += up;
+                }
+                Glast = __shfl(G, C - 1);
+                if (w == 0 && lane < C) sG[lane] = G;
+            }
             // ---- stage -------------------------------------------------------------
             {
                 typename IO::Regs fq = rq, fk = rk, fv = rv, fdo = rdo;
@@ -169,6 +199,13 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     IO::mask_rows(fdo, tid, live);
                 }
                 IO::to_lds(fq, sQ, LDD, tid);
+                if (GATED) {
+                    float af[IO::PASSES];
+#pragma unroll
+                    for (int p = 0; p < IO::PASSES; ++p) af[p] = __expf(__shfl(G, IO::row_of(tid, p)));
+                    IO::scale_rows(fq, af);
+                    IO::to_lds(fq, sQa, LDD, tid);
+                }
                 IO::to_lds(fk, sK, LDD, tid);
                 IO::to_lds(fv, sV, LDD, tid);
                 IO::to_lds(fdo, sDO, LDD, tid);
@@ -185,20 +222,57 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             {
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
+                // masked store; gated: times exp(G_i - G_j) (exponent <= 0 where kept)
+                auto store_tril = [&](const f32x4 *a, T *dst) {
+#pragma unroll
+                    for (int j = 0; j < TMA::TPW; ++j) {
+                        const int m = TMA::mt(w, j) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
+                        float x[4];
+                        if (GATED) {
+                            const float gn = sG[n];
+                            const f32x4 gm = *reinterpret_cast<const f32x4 *>(sG + m);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) x[e] = (m + e <= n) ? a[j][e] * __expf(gn - gm[e]) : 0.f;
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) x[e] = (m + e <= n) ? a[j][e] : 0.f;
+                        }
+                        *reinterpret_cast<P4 *>(dst + n * LDC + m) = TT<T>::pack(x[0], x[1], x[2], x[3]);
+                    }
+                };
                 gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sK, LDD, sQ, LDD, w, lane);  // D[m = j][n = i]
-                store_acc_f<T, C, C, NW>(acc, sAqk, LDC, w, lane, [](int m, int n, float x) { return m <= n ? x : 0.f; });
+                store_tril(acc, sAqk);
                 zero_acc<TMA::TPW>(acc);
                 gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sV, LDD, sDO, LDD, w, lane);  // D[m = j][n = i]
-                store_acc_f<T, C, C, NW>(acc, sDAqk, LDC, w, lane, [](int m, int n, float x) { return m <= n ? x : 0.f; });
+                store_tril(acc, sDAqk);
             }
             sync_lds();
             auto one = [](int, int) { return f32x4{1.f, 1.f, 1.f, 1.f}; };
+            float ep[TMR::NBW];  // gated: per-lane partials of edot for rows nt * 16 + li
+#pragma unroll
+            for (int j = 0; j < TMR::NBW; ++j) ep[j] = 0.f;
+            auto rowdot = [&](const f32x4 *acc, const T *X, float sign) {
+#pragma unroll
+                for (int j = 0; j < TMR::TPW; ++j) {
+                    const int d0 = TMR::mt(w, j) * 16 + 4 * lg, r = TMR::nt(w, j) * 16 + li;
+                    const P4 x = *reinterpret_cast<const P4 *>(X + r * LDD + d0);
+                    ep[j % TMR::NBW] += sign * (acc[j][0] * (float)x[0] + acc[j][1] * (float)x[1] +
+                                                acc[j][2] * (float)x[2] + acc[j][3] * (float)x[3]);
+                }
+            };
             // ---- dV^T[dv][j] = sum_i dO[i][dv] Aqk[i][j] + sum_dk dS[dv][dk] K[j][dk] -------
             {
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
-                gemm<T, HD, C, C, KROW, KROW, NW>(acc, sDO, LDD, sAqk, LDC, w, lane);
-                gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc, sDS, LDD, sK, LDD, w, lane);
+                if (GATED) {  // the state term of row j carries b_j = exp(G_last - G_j)
+                    gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc, sDS, LDD, sK, LDD, w, lane);
+#pragma unroll
+                    for (int j = 0; j < TMR::TPW; ++j) acc[j] *= __expf(Glast - sG[TMR::nt(w, j) * 16 + li]);
+                    gemm<T, HD, C, C, KROW, KROW, NW>(acc, sDO, LDD, sAqk, LDC, w, lane);
+                } else {
+                    gemm<T, HD, C, C, KROW, KROW, NW>(acc, sDO, LDD, sAqk, LDC, w, lane);
+                    gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc, sDS, LDD, sK, LDD, w, lane);
+                }
                 store_rows_global<T, C, NW>(acc, dv + base, rs, t0, Tlen, w, lane, one, live);
             }
             // ---- dQ^T[dk][i] = sum_dv S[dv][dk] dO[i][dv] + sum_j K[j][dk] dAqk[i][j] ---------
@@ -206,7 +280,12 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
                 gemm<T, HD, C, HD, KROW, ROWK, NW>(acc, sS, LDD, sDO, LDD, w, lane);
+                if (GATED) {  // the incoming state reaches row i decayed by a_i = exp(G_i)
+#pragma unroll
+                    for (int j = 0; j < TMR::TPW; ++j) acc[j] *= __expf(sG[TMR::nt(w, j) * 16 + li]);
+                }
                 gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sK, LDD, sDAqk, LDC, w, lane);
+                if (GATED) rowdot(acc, sQ, 1.f);
                 auto sc = [&](int r, int d0) {
                     const P4 x = *reinterpret_cast<const P4 *>(sQ + r * LDD + d0);
                     return f32x4{fmap_grad<FMAP>((float)x[0]), fmap_grad<FMAP>((float)x[1]),
@@ -218,8 +297,16 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             {
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
-                gemm<T, HD, C, C, KROW, KROW, NW>(acc, sQ, LDD, sDAqk, LDC, w, lane);
-                gemm<T, HD, C, HD, KROW, ROWK, NW>(acc, sDS, LDD, sV, LDD, w, lane);
+                if (GATED) {
+                    gemm<T, HD, C, HD, KROW, ROWK, NW>(acc, sDS, LDD, sV, LDD, w, lane);
+#pragma unroll
+                    for (int j = 0; j < TMR::TPW; ++j) acc[j] *= __expf(Glast - sG[TMR::nt(w, j) * 16 + li]);
+                    gemm<T, HD, C, C, KROW, KROW, NW>(acc, sQ, LDD, sDAqk, LDC, w, lane);
+                    rowdot(acc, sK, -1.f);
+                } else {
+                    gemm<T, HD, C, C, KROW, KROW, NW>(acc, sQ, LDD, sDAqk, LDC, w, lane);
+                    gemm<T, HD, C, HD, KROW, ROWK, NW>(acc, sDS, LDD, sV, LDD, w, lane);
+                }
                 auto sc = [&](int r, int d0) {
                     const P4 x = *reinterpret_cast<const P4 *>(sK + r * LDD + d0);
                     return f32x4{fmap_grad<FMAP>((float)x[0]), fmap_grad<FMAP>((float)x[1]),
@@ -227,9 +314,27 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 };
                 store_rows_global<T, C, NW>(acc, dk + base, rs, t0, Tlen, w, lane, sc, live);
             }
-            // ---- dS^T[dk][dv] += sum_c Q[c][dk] dO[c][dv] -----------------------------------------
-            gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, sQ, LDD, sDO, LDD, w, lane);
+            // ---- dS^T[dk][dv] += sum_c Q[c][dk] dO[c][dv]  (gated: c dS + sum_c a_c Q[c] dO[c]) -----
+            if (GATED) {
+                const float cl = __expf(Glast);
+#pragma unroll
+                for (int j = 0; j < TMS::TPW; ++j) dSacc[j] *= cl;
+#pragma unroll
+                for (int j = 0; j < TMR::NBW; ++j) {
+                    float x = ep[j];
+                    x += __shfl_xor(x, 16);
+                    x += __shfl_xor(x, 32);
+                    if (lg == 0) sE[(w % TMR::WM) * C + TMR::nt(w, j) * 16 + li] = x;
+                }
+            }
+            gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, GATED ? sQa : sQ, LDD, sDO, LDD, w, lane);
             sync_lds();
+            if (GATED && tid < C && t0 + tid < Tlen && live(tid)) {
+                float x = 0.f;
+#pragma unroll
+                for (int sl = 0; sl < TMR::WM; ++sl) x += sE[sl * C + tid];
+                edot[((int64_t)b * Tlen + t0 + tid) * H + h] = x;
+            }
         }
     }
     if (dS0) {
@@ -635,18 +740,19 @@ template <typename K> int set_smem(K kern, int smem, bool &flag)
     return MRX_OK;
 }
 
-template <typename T, int C, bool FMAP>
+template <typename T, int C, bool FMAP, bool GATED = false>
 int launch_la(hipStream_t st, const void *q, const void *k, const void *v, const void *done,
               int done_f32, const void *S_chk, const void *dout, const void *dS_last, void *dq,
-              void *dk, void *dv, void *dS0, int64_t B, int64_t Tlen, int64_t H)
+              void *dk, void *dv, void *dS0, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr,
+              void *edot = nullptr)
 {
-    auto kern = la_bwd_kernel<T, C, FMAP>;
-    constexpr int smem = LaBwdSmem<T, C>::total;
+    auto kern = la_bwd_kernel<T, C, FMAP, GATED>;
+    constexpr int smem = LaBwdSmem<T, C, GATED>::total;
     static bool attr_set = false;
     if (set_smem(kern, smem, attr_set) != MRX_OK) return MRX_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(256), smem, st, (const T *)q,
-                       (const T *)k, (const T *)v, done, done_f32, (const T *)S_chk,
-                       (const T *)dout, (const float *)dS_last, (T *)dq, (T *)dk, (T *)dv,
+                       (const T *)k, (const T *)v, (const float *)glog, done, done_f32, (const T *)S_chk,
+                       (const T *)dout, (const float *)dS_last, (T *)dq, (T *)dk, (T *)dv, (float *)edot,
                        (float *)dS0, (int)Tlen, (int)H);
     return launch_status();
 }
@@ -686,6 +792,26 @@ extern "C" int mrx_linear_attn_bwd(void *stream, const void *q, const void *k, c
 #define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H
     if (dtype == MRX_BF16) return fm ? launch_la<__bf16, 64, true>(MRX_ARGS) : launch_la<__bf16, 64, false>(MRX_ARGS);
     return fm ? launch_la<float, 32, true>(MRX_ARGS) : launch_la<float, 32, false>(MRX_ARGS);
+#undef MRX_ARGS
+}
+
+extern "C" int mrx_gated_linear_attn_bwd(void *stream, const void *q, const void *k, const void *v,
+                                         const void *g, const void *done, const void *S_chk,
+                                         const void *dout, const void *dS_last, void *dq, void *dk_out,
+                                         void *dv_out, void *edot, void *dS0, int64_t B, int64_t T, int64_t H,
+                                         int64_t dk, int64_t dv, int dtype, int done_dtype, int feature_map)
+{
+    const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
+                             dv, dtype, done_dtype);
+    if (rc != MRX_OK) return rc;
+    if (!g || !edot || !aligned(g, 4) || !aligned(edot, 4)) return MRX_ERR_INVALID_ARG;
+    if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const bool fm = feature_map == MRX_FMAP_ELU1;
+#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, g, edot
+    if (dtype == MRX_BF16)
+        return fm ? launch_la<__bf16, 64, true, true>(MRX_ARGS) : launch_la<__bf16, 64, false, true>(MRX_ARGS);
+    return fm ? launch_la<float, 32, true, true>(MRX_ARGS) : launch_la<float, 32, false, true>(MRX_ARGS);
 #undef MRX_ARGS
 }
 

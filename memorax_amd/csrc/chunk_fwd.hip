@@ -21,7 +21,7 @@ using namespace mrx;
 constexpr int NW = 4;             // waves per workgroup
 constexpr int NTHR = 64 * NW;
 
-template <typename T, int C, bool DELTA> struct FwdSmem {
+template <typename T, int C, bool DELTA, bool GATED = false> struct FwdSmem {
     static constexpr int PAD = pad_of<T>();
     static constexpr int LDD = HD + PAD;  // tiles with 64 columns
     static constexpr int LDC = C + PAD;   // tiles with C columns
@@ -36,22 +36,25 @@ template <typename T, int C, bool DELTA> struct FwdSmem {
     static constexpr int oQ = 0;                          // Q [C][dk], later U' [C][dv]
     static constexpr int oK = oQ + szRD;                  // K [C][dk]
     static constexpr int oV = oK + szRD;                  // V [C][dv]  (delta rule: beta_j V_j)
-    static constexpr int oBK = oV + szRD;                 // beta_j K_j [C][dk]  (delta rule only)
-    static constexpr int oS = oBK + (DELTA ? szRD : 0);   // S [dv][dk]
+    static constexpr int oBK = oV + szRD;                 // beta_j K_j [C][dk] (delta rule) / decayed K (gated)
+    static constexpr int oS = oBK + ((DELTA || GATED) ? szRD : 0);   // S [dv][dk]
     static constexpr int oTm = oS + szDD;                 // Tm [C][C]  (delta rule only)
     static constexpr int oA = oTm + (DELTA ? szCC : 0);
     static constexpr int oBeta = oA + szRA;
-    static constexpr int total = oBeta + C * 4;
+    static constexpr int oG = oBeta + C * 4;              // cumulative log-decay of the chunk rows (gated)
+    static constexpr int total = oG + C * 4;
 };
 
-template <typename T, int C, bool DELTA, bool FMAP>
+template <typename T, int C, bool DELTA, bool FMAP, bool GATED>
 __global__ void __launch_bounds__(NTHR, 2)  // 2 waves per SIMD: two workgroups share a CU
 chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
-                 const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
+                 const T *__restrict__ beta, const float *__restrict__ glog,
+                 const void *__restrict__ done, int done_f32,
                  const float *__restrict__ S0, T *__restrict__ o, float *__restrict__ S_last,
                  T *__restrict__ S_chk, T *__restrict__ Tm_chk, int Tlen, int H)
 {
-    using L = FwdSmem<T, C, DELTA>;
+    static_assert(!(DELTA && GATED), "the gated variant is linear attention with a decay");
+    using L = FwdSmem<T, C, DELTA, GATED>;
     using IO = TileIO<T, C, NTHR>;
     using P4 = typename TT<T>::pack4;
     constexpr int LDD = L::LDD, LDC = L::LDC, LDA = L::LDA;
@@ -67,6 +70,8 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     T *sW = reinterpret_cast<T *>(smem + L::oA + L::szCC);
     T *sU = sV;                                      // U' [C][dv] (delta rule: over beta V once U is taken)
     float *sBeta = reinterpret_cast<float *>(smem + L::oBeta);
+    float *sG = reinterpret_cast<float *>(smem + L::oG);
+    T *sKd = sBK;                                    // gated: K_j exp(G_last - G_j)
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -92,6 +97,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     // register prefetch of the next chunk (raw bits only: no arithmetic on in-flight loads)
     typename IO::Regs rq, rk, rv;
     uint32_t rbeta = 0u, rdone = 0u;
+    float rg = 0.f;  // log-decay of chunk row `lane` (gated)
     uint32_t rbrow[IO::PASSES];  // beta of the rows this thread stages
     // Element offsets of what this thread loads for the chunk about to be prefetched; they advance
     // by one chunk per call (64-bit adds instead of per-chunk index multiplications).
@@ -125,9 +131,11 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             rdone = 0u;
             rbeta = 0u;
+            rg = 0.f;
             if (lane < C && tpre + lane < Tlen) {
                 rdone = done_raw(done, done_f32, doff);
                 if (DELTA && w == 0) rbeta = load_raw<T>(beta + doff * H + h);
+                if (GATED) rg = glog[doff * H + h];
             }
             doff += C;
             tpre += C;
@@ -152,6 +160,19 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         const int nres = __popcll(dmask);
         for (int pass = 0; pass <= nres; ++pass) {
             auto live = [&](int r) { return nres == 0 || episode_of(dmask, r) == pass; };
+            // gated: G_i = sum of the log-decays of this pass's episode up to row i (the decay of an
+            // episode's first step multiplies a zero state and is left out); every wave scans its copy
+            float G = 0.f, Glast = 0.f;
+            if (GATED) {
+                G = (lane < C && live(lane) && !((dmask >> lane) & 1ull)) ? rg : 0.f;
+#pragma unroll
+                for (int off = 1; off < C; off <<= 1) {
+                    const float up = __shfl_up(G, off);
+                    if (lane >= off) G += up;
+                }
+                Glast = __shfl(G, C - 1);
+                if (w == 0 && lane < C) sG[lane] = G;
+            }
             // ---- stage the chunk ---------------------------------------------------
             {
                 typename IO::Regs fq = rq, fk = rk, fv = rv;
@@ -171,6 +192,13 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     IO::scale_rows(fk, bf);
                     IO::scale_rows(fv, bf);
                     IO::to_lds(fk, sBK, LDD, tid);
+                }
+                if (GATED) {
+                    float bf[IO::PASSES];
+#pragma unroll
+                    for (int p = 0; p < IO::PASSES; ++p) bf[p] = __expf(Glast - __shfl(G, IO::row_of(tid, p)));
+                    IO::scale_rows(fk, bf);
+                    IO::to_lds(fk, sKd, LDD, tid);
                 }
                 IO::to_lds(fv, sV, LDD, tid);
             }
@@ -224,8 +252,22 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
                 gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sK, LDD, sQ, LDD, w, lane);  // D[m = j][n = i]
-                store_acc_f<T, C, C, NW>(acc, sAqk, LDC, w, lane,
-                                         [](int m, int n, float x) { return m <= n ? x : 0.f; });
+                if (GATED) {
+                    // Aqk[i][j] = exp(G_i - G_j) (q_i . k_j), j <= i (exponent <= 0 for log-decays <= 0)
+#pragma unroll
+                    for (int j = 0; j < TMA::TPW; ++j) {
+                        const int m = TMA::mt(w, j) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
+                        const float gn = sG[n];
+                        const f32x4 gm = *reinterpret_cast<const f32x4 *>(sG + m);
+                        float x[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) x[e] = (m + e <= n) ? acc[j][e] * __expf(gn - gm[e]) : 0.f;
+                        *reinterpret_cast<P4 *>(sAqk + n * LDC + m) = TT<T>::pack(x[0], x[1], x[2], x[3]);
+                    }
+                } else {
+                    store_acc_f<T, C, C, NW>(acc, sAqk, LDC, w, lane,
+                                             [](int m, int n, float x) { return m <= n ? x : 0.f; });
+                }
             }
             if (DELTA) {
                 f32x4 Uacc[TMO::TPW];
@@ -268,6 +310,10 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             f32x4 Oacc[TMO::TPW];
             zero_acc<TMO::TPW>(Oacc);
             gemm<T, HD, C, HD, ROWK, ROWK, NW>(Oacc, sS, LDD, sQ, LDD, w, lane);
+            if (GATED) {  // the incoming state reaches row i decayed by exp(G_i)
+#pragma unroll
+                for (int j = 0; j < TMO::TPW; ++j) Oacc[j] *= __expf(sG[TMO::nt(w, j) * 16 + li]);
+            }
             gemm<T, HD, C, C, KROW, ROWK, NW>(Oacc, sU, LDD, sAqk, LDC, w, lane);
 #pragma unroll
             for (int j = 0; j < TMO::TPW; ++j) {
@@ -277,7 +323,14 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                         TT<T>::pack(Oacc[j][0], Oacc[j][1], Oacc[j][2], Oacc[j][3]);
             }
             // ---- S^T[dk][dv] += sum_c K[c][dk] U'[c][dv]  (only the episode that leaves the chunk)
-            if (pass == nres) gemm<T, HD, HD, C, KROW, KROW, NW>(Sacc, sK, LDD, sU, LDD, w, lane);
+            if (pass == nres) {
+                if (GATED) {  // S <- exp(G_last) S + sum_c exp(G_last - G_c) K[c] U'[c]
+                    const float cl = __expf(Glast);
+#pragma unroll
+                    for (int j = 0; j < TMS::TPW; ++j) Sacc[j] *= cl;
+                }
+                gemm<T, HD, HD, C, KROW, KROW, NW>(Sacc, GATED ? sKd : sK, LDD, sU, LDD, w, lane);
+            }
             sync_lds();
             MRX_PHASE(8);
         }
@@ -294,13 +347,13 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     }
 }
 
-template <typename T, int C, bool DELTA, bool FMAP>
+template <typename T, int C, bool DELTA, bool FMAP, bool GATED = false>
 int launch(hipStream_t st, const void *q, const void *k, const void *v, const void *beta,
            const void *done, int done_f32, const void *S0, void *o, void *S_last, void *S_chk,
-           void *Tm_chk, int64_t B, int64_t Tlen, int64_t H)
+           void *Tm_chk, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr)
 {
-    auto kern = chunk_fwd_kernel<T, C, DELTA, FMAP>;
-    constexpr int smem = FwdSmem<T, C, DELTA>::total;
+    auto kern = chunk_fwd_kernel<T, C, DELTA, FMAP, GATED>;
+    constexpr int smem = FwdSmem<T, C, DELTA, GATED>::total;
     static bool attr_set = false;  // idempotent; a race only repeats the call
     if (!attr_set) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -309,7 +362,7 @@ int launch(hipStream_t st, const void *q, const void *k, const void *v, const vo
         attr_set = true;
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(NTHR), smem, st, (const T *)q,
-                       (const T *)k, (const T *)v, (const T *)beta, done, done_f32,
+                       (const T *)k, (const T *)v, (const T *)beta, (const float *)glog, done, done_f32,
                        (const float *)S0, (T *)o, (float *)S_last, (T *)S_chk, (T *)Tm_chk, (int)Tlen, (int)H);
     return launch_status();
 }
@@ -364,4 +417,22 @@ extern "C" int mrx_delta_rule_fwd(void *stream, const void *q, const void *k, co
     if (dtype == MRX_BF16)
         return launch<__bf16, 64, true, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H);
     return launch<float, 32, true, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H);
+}
+
+extern "C" int mrx_gated_linear_attn_fwd(void *stream, const void *q, const void *k, const void *v,
+                                         const void *g, const void *done, const void *S0, void *o,
+                                         void *S_last, void *S_chk, int64_t B, int64_t T, int64_t H,
+                                         int64_t dk, int64_t dv, int dtype, int done_dtype, int feature_map)
+{
+    const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
+    if (rc != MRX_OK) return rc;
+    if (!g || !aligned(g, 4)) return MRX_ERR_INVALID_ARG;
+    if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const bool fm = feature_map == MRX_FMAP_ELU1;
+#define MRX_ARGS st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H, g
+    if (dtype == MRX_BF16)
+        return fm ? launch<__bf16, 64, false, true, true>(MRX_ARGS) : launch<__bf16, 64, false, false, true>(MRX_ARGS);
+    return fm ? launch<float, 32, false, true, true>(MRX_ARGS) : launch<float, 32, false, false, true>(MRX_ARGS);
+#undef MRX_ARGS
 }

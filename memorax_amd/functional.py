@@ -87,6 +87,36 @@ def linear_attention(q, k, v, done, S0=None, feature_map="none"):
     return _LinearAttention.apply(q, k, v, done, S0, _FMAP[feature_map])
 
 
+class _GatedLinearAttention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, g, done, S0, fmap):
+        q_, k_, v_ = q.contiguous(), k.contiguous(), v.contiguous()
+        g_ = g.contiguous().float()
+        S0_ = None if S0 is None else S0.contiguous().float()
+        need = any(ctx.needs_input_grad)
+        o, S_last, S_chk = K.gated_linear_attn_fwd(q_, k_, v_, g_, done, S0_, fmap, save_chk=need)
+        if need:
+            ctx.save_for_backward(q_, k_, v_, g_, S_chk, S_last)
+        ctx.done, ctx.fmap, ctx.has_S0 = done, fmap, S0 is not None
+        return o, S_last
+
+    @staticmethod
+    def backward(ctx, do, dS_last):
+        q, k, v, g, S_chk, S_last = ctx.saved_tensors
+        do = torch.zeros_like(v) if do is None else do.contiguous()
+        dS_last = None if dS_last is None else dS_last.contiguous().float()
+        dq, dk, dv, dg, dS0 = K.gated_linear_attn_bwd(q, k, v, g, ctx.done, S_chk, do, dS_last, ctx.fmap,
+                                                      want_dS0=ctx.has_S0, S_last=S_last)
+        return dq, dk, dv, dg, None, (dS0 if ctx.has_S0 else None), None
+
+
+def gated_linear_attention(q, k, v, g, done, S0=None, feature_map="none"):
+    """Linear attention with a scalar log-decay g:(B,T,H) per step and head:
+    S_t = r_t exp(g_t) S_{t-1} + v_t phi(k_t)^T, o_t = S_t phi(q_t) -- the Mamba cell's algebra
+    (mamba.py:109-122) in chunked form.  Returns (o, S_last)."""
+    return _GatedLinearAttention.apply(q, k, v, g, done, S0, _FMAP[feature_map])
+
+
 class _DeltaRule(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, beta, done, S0):
