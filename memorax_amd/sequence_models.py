@@ -27,7 +27,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .functional import delta_rule, linear_attention, linear_scan
+from .functional import delta_rule, gated_linear_attention, linear_attention, linear_scan
 
 
 # ----------------------------------------------------------------------------------
@@ -371,6 +371,103 @@ class DeltaNetCell(MemoroidCellBase):
         *batch, _ = input_shape
         dev = self.key.weight.device
         return (torch.zeros(*batch, 1, self.num_heads, self.head_dim, self.head_dim, device=dev),)
+
+
+class MambaCell(MemoroidCellBase):
+    """Mamba-2 style selective state space cell (mamba.py:33-144).  Elements are
+    (h_t = (B_t dt_t) (x) x_t : (H,N,P), decay_t = exp(dt_t A) : (H,1,1)) combined by the diagonal
+    operator; read is y_t = C_t . h_t + D x_t, gated by silu(z) after RMSNorm.  The reference
+    materialises h (B,T,H,N,P); here the scan and the C-contraction run in the gated chunked
+    kernel with k = B dt, v = x, q = C and log-decay g = dt A (needs state_dim = head_dim = 64).
+    Carry: (h (B,1,H,N,P), decay (B,1,H,1,1)), the reference's shapes."""
+
+    def __init__(self, features, num_heads=8, head_dim=64, state_dim=64, conv_dim=4, in_features=None):
+        super().__init__()
+        in_features = features if in_features is None else in_features
+        self.features, self.num_heads, self.head_dim = features, num_heads, head_dim
+        self.state_dim, self.conv_dim = state_dim, conv_dim
+        hidden, sp = num_heads * head_dim, num_heads * state_dim
+        conv_channels = hidden + 2 * sp
+        self.A_log = nn.Parameter(torch.empty(num_heads).uniform_(math.log(1.0), math.log(16.0)))
+        self.D = nn.Parameter(torch.ones(num_heads))
+        dt = torch.exp(torch.rand(num_heads) * (math.log(0.1) - math.log(0.001)) + math.log(0.001))
+        self.dt_bias = nn.Parameter(dt + torch.log(-torch.expm1(-dt)))
+        self.input_projection = nn.Linear(in_features, hidden * 2, bias=False)
+        self.B = nn.Linear(in_features, sp, bias=False)
+        self.C = nn.Linear(in_features, sp, bias=False)
+        self.dt = nn.Linear(in_features, num_heads, bias=False)
+        self.conv = nn.Conv1d(conv_channels, conv_channels, conv_dim, groups=conv_channels)
+        self.norm = _RMSNorm(hidden)
+        self.output_projection = nn.Linear(hidden, features)
+
+    def _project(self, x):
+        Bn, T, _ = x.shape
+        H, P, N = self.num_heads, self.head_dim, self.state_dim
+        hidden, z = self.input_projection(x).chunk(2, dim=-1)
+        ci = torch.cat([hidden, self.B(x), self.C(x)], dim=-1).transpose(1, 2)      # (B, channels, T)
+        ci = F.silu(self.conv(F.pad(ci, (self.conv_dim - 1, 0)))).transpose(1, 2)   # causal, per call
+        hidden = ci[..., :H * P].reshape(Bn, T, H, P)
+        B_proj = ci[..., H * P:H * P + H * N].reshape(Bn, T, H, N)
+        C_proj = ci[..., H * P + H * N:].reshape(Bn, T, H, N)
+        dt = F.softplus(self.dt(x) + self.dt_bias)
+        return hidden, B_proj, C_proj, z, dt
+
+    def forward(self, x, **kwargs):
+        """Elements in kernel form: (k = B dt, v = x, log-decay g = dt A); the reference's
+        (h, decay) are v (x) k and exp(g)."""
+        hidden, B_proj, _, _, dt = self._project(x)
+        g = dt * (-torch.exp(self.A_log))[None, None, :]
+        return (B_proj * dt[..., None], hidden, g)
+
+    def binary_operator(self, a, b):
+        h_i, decay_i = a
+        h_j, decay_j = b
+        return (decay_j * h_i + h_j, decay_j * decay_i)
+
+    def scan(self, z, initial_carry, done, q=None):
+        k, v, g = z
+        h0, decay0 = initial_carry                      # (B,1,H,N,P), (B,1,H,1,1)
+        S0 = h0[:, 0].transpose(-1, -2).float().contiguous()   # kernel state is (P, N) = (d_v, d_k)
+        o, S_last = gated_linear_attention(q.contiguous(), k.contiguous(), v.contiguous(), g.float(), done, S0)
+        Bn, T, H = g.shape
+        ones = torch.ones(H, device=g.device)
+        _, G_last, _ = linear_scan(ones, g.float().contiguous(), done,
+                                   torch.log(decay0[:, 0, :, 0, 0].float()).contiguous())
+        carry = (S_last.transpose(-1, -2)[:, None], torch.exp(G_last)[:, None, :, None, None])
+        return o, carry
+
+    def read(self, o, x, **kwargs):
+        Bn, T, _ = x.shape
+        hidden, _, _, z, _ = self._project(x)
+        y = o.float() + self.D[None, None, :, None] * hidden
+        y = y.reshape(Bn, T, self.num_heads * self.head_dim)
+        return self.output_projection((self.norm(y) * F.silu(z)).to(x.dtype))
+
+    def initialize_carry(self, key, input_shape):
+        *batch, _ = input_shape
+        dev = self.A_log.device
+        return (torch.zeros(*batch, 1, self.num_heads, self.state_dim, self.head_dim, device=dev),
+                torch.ones(*batch, 1, self.num_heads, 1, 1, device=dev))
+
+
+class Mamba(SequenceModel):
+    """Memoroid(MambaCell): the query (C projection) joins the scan because the kernel fuses the
+    contraction y_t = C_t . h_t into it."""
+
+    def __init__(self, cell: MambaCell):
+        super().__init__()
+        self.cell = cell
+
+    def forward(self, inputs, done, initial_carry=None, **kwargs):
+        if initial_carry is None:
+            initial_carry = self.cell.initialize_carry(None, get_input_shape(inputs))
+        z = self.cell(inputs)
+        _, _, C_proj, _, _ = self.cell._project(inputs)
+        o, carry = self.cell.scan(z, initial_carry, done, q=C_proj)
+        return carry, self.cell.read(o, inputs)
+
+    def initialize_carry(self, key, input_shape):
+        return self.cell.initialize_carry(key, input_shape)
 
 
 # ----------------------------------------------------------------------------------

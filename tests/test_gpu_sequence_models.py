@@ -134,3 +134,38 @@ def test_rollout_steps_equal_sequence_call():
         for a, b_ in zip(carry, carry_seq):
             assert a.shape == b_.shape
             assert relerr(a, _np(b_)) <= tol
+
+
+def test_mamba_model_matches_materialise_and_scan_reference():
+    """Mamba(MambaCell) against the reference's own route: materialise h_t = (B dt) (x) x and the
+    decay leaf, scan with the diagonal operator (mamba.py:109-135 under memoroid.py:60-91)."""
+    from memorax_amd import sequence_models as sm
+    torch.manual_seed(7)
+    B, T, Fe, H, d = 2, 90, 32, 2, 64
+    cell = sm.MambaCell(Fe, num_heads=H, head_dim=d, state_dim=d).cuda()
+    model = sm.Mamba(cell)
+    x, done = _inputs(B, T, Fe, 0.04, 8)
+    carry, y = model(x, done)
+    assert carry[0].shape == (B, 1, H, d, d) and carry[1].shape == (B, 1, H, 1, 1)
+    with torch.no_grad():
+        hidden, B_proj, C_proj, z, dt = cell._project(x)
+        g = dt * (-torch.exp(cell.A_log))[None, None, :]
+        k = B_proj * dt[..., None]
+    nxt, o = M.gated_linear_attention_memoroid(_np(C_proj), _np(k), _np(hidden), _np(g), _np(done.float()))
+    yy = o + _np(cell.D)[None, None, :, None] * _np(hidden)
+    yy = yy.reshape(B, T, H * d)
+    yy = yy / np.sqrt((yy ** 2).mean(-1, keepdims=True) + 1e-6) * _np(cell.norm.scale)
+    zz = _np(z)
+    yy = yy * (zz / (1 + np.exp(-zz)))
+    ry = yy @ _np(cell.output_projection.weight).T + _np(cell.output_projection.bias)
+    assert relerr(y, ry) <= 2e-4, relerr(y, ry)
+    # carry leaves in the reference's layout: h is (N, P) = k (x) v, decay the product since the last reset
+    assert relerr(carry[0][:, 0], nxt[0][:, 0].transpose(0, 1, 3, 2)) <= 2e-4
+    assert relerr(carry[1][:, 0, :, 0, 0], nxt[1][:, 0, :, 0, 0]) <= 1e-5
+    # carry threading and gradients
+    c1, y1 = model(x[:, :50], done[:, :50])
+    c2, y2 = model(x[:, 50:], done[:, 50:], c1)
+    assert relerr(c2[0], _np(carry[0])) <= 2e-4
+    y.pow(2).mean().backward()
+    assert torch.isfinite(cell.A_log.grad).all() and cell.A_log.grad.abs().sum() > 0
+    assert cell.dt.weight.grad.abs().sum() > 0 and cell.C.weight.grad.abs().sum() > 0
