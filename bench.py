@@ -199,6 +199,15 @@ def bench_linear_attention(torch, K, M, dev):
     ms = _time_ms(torch, f3, iters=5)
     res["cfg3_bf16_B32of256_4096x8x64"] = {"ms": ms, "tokens/s": Bn * Tn / ms * 1e3,
                                            "GB/s": 1408 * Bn * Tn * Hn / ms / 1e6}
+    # the same shape with a per-step scalar decay (Mamba cell algebra); + g in, edot out: 8 B more per token-head
+    g = -torch.rand((Bn, Tn, Hn), device="cuda") * 0.1
+
+    def f3g():
+        o, Sl, chk = K.gated_linear_attn_fwd(q, k, v, g, dn, None, 0)
+        K.gated_linear_attn_bwd(q, k, v, g, dn, chk, do, None, 0, want_dS0=False)
+    ms = _time_ms(torch, f3g, iters=5)
+    res["gated_bf16_B32_4096x8x64"] = {"ms": ms, "tokens/s": Bn * Tn / ms * 1e3,
+                                       "GB/s": (1408 + 12) * Bn * Tn * Hn / ms / 1e6}
     return res
 
 
