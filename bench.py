@@ -135,6 +135,7 @@ def main() -> int:
         out["linear_attention"] = bench_linear_attention(torch, K, M, dev)
         out["torso"] = bench_torso(torch, K)
         out["step"] = bench_step(torch, K)
+        out["rtrl"] = bench_rtrl(torch, K)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(np, M, x, do_np)
     print(json.dumps(out))
@@ -209,6 +210,28 @@ def bench_linear_attention(torch, K, M, dev):
     res["gated_bf16_B32_4096x8x64"] = {"ms": ms, "tokens/s": Bn * Tn / ms * 1e3,
                                        "GB/s": (1408 + 12) * Bn * Tn * Hn / ms / 1e6}
     return res
+
+
+def bench_rtrl(torch, K):
+    """RTRL sensitivity update (memoroid.py:114-141): final state of a diagonal scan over
+    H * param_size channels with the decay shared by param_size channels.  Bytes = one read of
+    the Jacobians (+ decay, carry in and out).  Beside it: the reference's formulation on the
+    general scan kernel (decay repeated param_size times, all states written)."""
+    Bn, Tn, Hn, ps = 64, 128, 256, 64
+    D = Hn * ps
+    decay = torch.rand((Bn, Tn, Hn), device="cuda") * 0.1 + 0.9
+    J = torch.randn((Bn, Tn, D), device="cuda")
+    S = torch.randn((Bn, D), device="cuda")
+    dn = torch.rand((Bn, Tn), device="cuda") < 0.01
+    by = 4 * (Bn * Tn * D + Bn * Tn * Hn + 2 * Bn * D)
+    ms = _time_ms(torch, lambda: K.linear_scan_last(decay, J, dn, S), iters=10)
+
+    def general():
+        a = decay.repeat_interleave(ps, dim=-1)
+        K.linear_scan_fwd(a, J, dn, S, want_P=False)
+    ms2 = _time_ms(torch, general, iters=5)
+    return {"scan_last_64x128x(256x64)": {"ms": ms, "GB/s": by / ms / 1e6, "frac_hbm": by / ms / 1e6 / HBM_PEAK_GBS},
+            "repeat_and_general_scan_ms": ms2}
 
 
 def bench_step(torch, K):

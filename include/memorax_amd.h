@@ -136,6 +136,18 @@ int mrx_delta_rule_bwd(void *stream, const void *q, const void *k,
                        void *dbeta, void *dS0, int64_t B, int64_t T, int64_t H,
                        int64_t dk, int64_t dv, int dtype, int done_dtype);
 
+/* Final state only, one decay per `a_group` consecutive channels: h_T of
+ *     h_t = done_t ? b_t : a_t h_{t-1} + b_t ,  a: (B,T,D/a_group), b: (B,T,D), h0 (nullable), h_last: (B,D).
+ * The sensitivity propagation of real-time recurrent learning, Memoroid._propagate_sensitivities
+ * (memoroid.py:114-141): there a = where(done, 0, repeat(decay, param_size)), b = the local
+ * Jacobians (B,T,H*param_size), h0 = the carried sensitivity and only last(state) is kept; here the
+ * repeated decay and the per-step states are never materialised (a_group = param_size).
+ * dtype: MRX_F32 or MRX_C64. */
+int mrx_linear_scan_last(void *stream, const void *a, const void *b,
+                         const void *done, const void *h0, void *h_last, int64_t B,
+                         int64_t T, int64_t D, int64_t a_group, int dtype,
+                         int done_dtype);
+
 /* ---- Gated linear attention: linear attention with a scalar decay per step and head ----
  * The Mamba cell's algebra (mamba.py:109-122: elements (h_t = (B_t dt_t) (x) x_t, decay_t =
  * exp(dt_t A)), binary_operator (decay_j h_i + h_j, decay_j decay_i), read y_t = C_t . h_t), scanned

@@ -396,6 +396,63 @@ diag_scan_fwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ b,
     if (P_last) *reinterpret_cast<V *>(P_last + bi * D + col) = cp;
 }
 
+// ---- final state only, decay shared by groups of channels ---------------------------
+// h_T of h_t = done_t ? b_t : a_t h_{t-1} + b_t where a:(B,T,D/a_group) holds one decay per
+// a_group consecutive channels.  Nothing but the last state is written, so the traffic is one
+// read of b.  This is the real-time-recurrent-learning sensitivity update
+// (memoroid.py:114-141: S <- last(scan(a = where(done, 0, repeat(decay, param_size)), J))),
+// without materialising the repeated decay or the per-step states.
+template <typename E, int VEC, int SG>
+__global__ void __launch_bounds__(256)
+diag_scan_last_kernel(const E *__restrict__ a, const E *__restrict__ b, const void *__restrict__ done,
+                      int done_f32, const E *__restrict__ h0, E *__restrict__ h_last, int64_t B, int T,
+                      int64_t D, int64_t cols_per_row, int64_t a_group)
+{
+    using V = Vec<E, VEC>;
+    using O = Ops<E>;
+    const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t bi = gid / cols_per_row;
+    const int64_t col = (gid % cols_per_row) * VEC;
+    if (bi >= B) return;  // padding threads of the last workgroup (this kernel has no barriers)
+    const int64_t row0 = bi * T, Da = D / a_group, acol = col / a_group;  // VEC divides a_group
+    V ch = vfill<E, VEC>(O::zero());
+    if (h0) ch = *reinterpret_cast<const V *>(h0 + bi * D + col);
+
+    E xa[SG], na[SG];
+    V xb[SG], nb[SG];
+    uint32_t xd[SG], nd[SG];
+    auto load = [&](int t0, E *pa, V *pb, uint32_t *pd) {
+#pragma unroll
+        for (int s = 0; s < SG; ++s) {
+            const int t = t0 + s;
+            pd[s] = 0u;
+            if (t < T) {
+                pa[s] = a[(row0 + t) * Da + acol];
+                pb[s] = *reinterpret_cast<const V *>(b + (row0 + t) * D + col);
+                pd[s] = done_raw(done, done_f32, row0 + t);
+            }
+        }
+    };
+    load(0, xa, xb, xd);
+    for (int t0 = 0; t0 < T; t0 += SG) {
+        if (t0 + SG < T) load(t0 + SG, na, nb, nd);
+#pragma unroll
+        for (int s = 0; s < SG; ++s) {
+            if (t0 + s < T) {
+                const bool r = done_test(xd[s], done_f32);
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) {
+                    const E hn = O::madd(xa[s], ch.v[i], xb[s].v[i]);
+                    ch.v[i] = r ? xb[s].v[i] : hn;
+                }
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < SG; ++s) { xa[s] = na[s]; xb[s] = nb[s]; xd[s] = nd[s]; }
+    }
+    *reinterpret_cast<V *>(h_last + bi * D + col) = ch;
+}
+
 template <typename E, int VEC, int SG>
 __global__ void __launch_bounds__(256)
 diag_scan_bwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ hfw,
@@ -575,6 +632,31 @@ int launch_bwd(hipStream_t st, const void *a, const void *h, const void *done,
     return launch_status();
 }
 
+template <typename E>
+int launch_last(hipStream_t st, const void *a, const void *b, const void *done, int done_f32,
+                const void *h0, void *h_last, int64_t B, int64_t T, int64_t D, int64_t a_group)
+{
+    const int maxvec = (int)(16 / sizeof(E));
+    int vec = 1;
+    for (int v = maxvec; v >= 1; v >>= 1) {
+        const size_t bytes = sizeof(E) * v;
+        if (D % v == 0 && a_group % v == 0 && aligned(b, bytes) && aligned(h0, bytes) && aligned(h_last, bytes)) {
+            vec = v;
+            break;
+        }
+    }
+    while (vec > 1 && B * (D / vec) < 2048 * 64) vec >>= 1;  // keep at least 2048 waves when the shape allows
+    const int64_t cpr = D / vec;
+    const dim3 grid((unsigned)((B * cpr + 255) / 256)), block(256);
+    vec_switch<E>(vec, [&](auto vc) {
+        constexpr int VEC = decltype(vc)::value;
+        hipLaunchKernelGGL((diag_scan_last_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8)>), grid, block, 0, st,
+                           (const E *)a, (const E *)b, done, done_f32, (const E *)h0, (E *)h_last, B, (int)T, D,
+                           cpr, a_group);
+    });
+    return launch_status();
+}
+
 bool scan_shape_ok(int64_t B, int64_t T, int64_t D)
 {
     return B > 0 && T > 0 && D > 0 && T < (1ll << 30) && B * ((D + 63) / 64) < (1ll << 31);
@@ -627,6 +709,27 @@ extern "C" int mrx_linear_scan_bwd(void *stream, const void *a, const void *h, c
             !aligned(db, 8) || !aligned(h0, 8) || !aligned(g_last, 8) || !aligned(dh0, 8))
             return MRX_ERR_INVALID_ARG;
         return launch_bwd<c64>(st, a, h, done, done_dtype, h0, g, g_last, da, db, dh0, B, T, D, ti);
+    }
+    return dtype == MRX_BF16 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
+}
+
+extern "C" int mrx_linear_scan_last(void *stream, const void *a, const void *b, const void *done,
+                                    const void *h0, void *h_last, int64_t B, int64_t T, int64_t D,
+                                    int64_t a_group, int dtype, int done_dtype)
+{
+    if (!a || !b || !done || !h_last) return MRX_ERR_INVALID_ARG;
+    if (!scan_shape_ok(B, T, D) || a_group <= 0 || D % a_group != 0) return MRX_ERR_INVALID_ARG;
+    if (B * D >= (1ll << 38)) return MRX_ERR_INVALID_ARG;  // grid size
+    if (done_dtype != MRX_DONE_U8 && done_dtype != MRX_DONE_F32) return MRX_ERR_INVALID_ARG;
+    if (done_dtype == MRX_DONE_F32 && !aligned(done, 4)) return MRX_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == MRX_F32) {
+        if (!aligned(a, 4) || !aligned(b, 4) || !aligned(h0, 4) || !aligned(h_last, 4)) return MRX_ERR_INVALID_ARG;
+        return launch_last<float>(st, a, b, done, done_dtype, h0, h_last, B, T, D, a_group);
+    }
+    if (dtype == MRX_C64) {
+        if (!aligned(a, 8) || !aligned(b, 8) || !aligned(h0, 8) || !aligned(h_last, 8)) return MRX_ERR_INVALID_ARG;
+        return launch_last<c64>(st, a, b, done, done_dtype, h0, h_last, B, T, D, a_group);
     }
     return dtype == MRX_BF16 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
 }

@@ -147,3 +147,24 @@ def delta_rule(q, k, v, beta, done, S0=None):
     """DeltaNet recurrence S_t = r_t S_{t-1}(I - beta_t k_t k_t^T) + beta_t v_t k_t^T,
     o_t = S_t q_t, in chunked WY form.  Returns (o, S_last)."""
     return _DeltaRule.apply(q, k, v, beta, done, S0)
+
+
+def propagate_sensitivities(decay, jacobians, sensitivity, done):
+    """Real-time recurrent learning: carry the parameter sensitivities of a diagonal recurrence
+    over a (B,T) block of steps -- Memoroid._propagate_sensitivities (memoroid.py:114-141).
+    decay: (B,T,H); jacobians[name]: (B,T,H,*param_shape) local Jacobians; sensitivity[name]:
+    (B,1,H,*param_shape).  Returns the sensitivities after the last step, same shapes.  The
+    reference repeats the decay param_size times and scans the concatenated (B,T+1,H*param_size)
+    array; the kernel reads the Jacobians once and writes only the final state."""
+    import math
+    B, T, H = decay.shape
+    decay = decay.contiguous()
+    out = {}
+    for name in sorted(jacobians.keys()):
+        J, S = jacobians[name], sensitivity[name]
+        param_shape = tuple(J.shape[3:])
+        ps = math.prod(param_shape)
+        last = K.linear_scan_last(decay.to(J.dtype), J.reshape(B, T, H * ps).contiguous(), done,
+                                  S.reshape(B, H * ps).to(J.dtype).contiguous())
+        out[name] = last.reshape(B, 1, H, *param_shape)
+    return out

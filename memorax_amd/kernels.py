@@ -80,6 +80,27 @@ def linear_scan_fwd(a, b, done, h0=None, P0=None, want_P=True):
     return h, h_last, P_last
 
 
+def linear_scan_last(a, b, done, h0=None):
+    """Final state of h_t = done ? b_t : a_t h_{t-1} + b_t with one decay per group of channels:
+    a: (B,T,D/group), b: (B,T,D), h0: (B,D) or None.  Returns h_last (B,D)."""
+    lib = _lib.load()
+    B, T, D = b.shape
+    dt = b.dtype
+    if dt not in (torch.float32, torch.complex64):
+        raise ValueError("linear_scan_last supports float32 and complex64")
+    if a.dim() != 3 or a.shape[:2] != (B, T) or D % a.shape[2] != 0:
+        raise ValueError(f"a must be (B,T,D/group), got {tuple(a.shape)} for b {tuple(b.shape)}")
+    _chk(a, "a", dt)
+    _chk(b, "b", dt)
+    _chk(h0, "h0", dt, (B, D))
+    done, dd = _done(done, B, T)
+    h_last = torch.empty((B, D), dtype=dt, device=b.device)
+    st = lib.mrx_linear_scan_last(_stream(), _ptr(a), _ptr(b), _ptr(done), _ptr(h0), _ptr(h_last), B, T, D,
+                                  D // a.shape[2], _DT[dt], dd)
+    _lib.check(st, "mrx_linear_scan_last")
+    return h_last
+
+
 def linear_scan_bwd(a, h, done, h0, g, g_last=None):
     """Returns (da (B,T,D) per step, db, dh0)."""
     lib = _lib.load()

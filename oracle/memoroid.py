@@ -220,6 +220,32 @@ def diag_scan_bwd(a, h, done, g, h0=None, g_last=None):
 # --------------------------------------------------------------------------
 
 
+def propagate_sensitivities(decay, jacobians, sensitivity, done):
+    """Memoroid._propagate_sensitivities (memoroid.py:114-141), restated step by step: per name the
+    Jacobians (B,T,H,*param_shape) are flattened to H*param_size channels, the decay is repeated
+    param_size times and zeroed where done, the carried sensitivity is prepended with decay 1, the
+    diagonal operator is scanned and the last state kept."""
+    decay = np.asarray(decay)
+    B, T, H = decay.shape
+    d = (np.asarray(done) != 0)[..., None]
+    out = {}
+    for name in sorted(jacobians.keys()):
+        J = np.asarray(jacobians[name])
+        param_shape = J.shape[3:]
+        ps = int(np.prod(param_shape)) if param_shape else 1
+        ct = np.complex128 if np.iscomplexobj(J) or np.iscomplexobj(decay) else np.float64
+        Jf = J.reshape(B, T, H * ps).astype(ct)
+        S = np.asarray(sensitivity[name]).reshape(B, 1, H * ps).astype(ct)
+        a = np.where(d, 0, np.repeat(decay, ps, axis=-1)).astype(ct)
+        state = np.concatenate([S, Jf], axis=1)
+        a = np.concatenate([np.ones_like(S), a], axis=1)
+        s_acc, a_acc = state[:, 0], a[:, 0]
+        for t in range(1, T + 1):  # left fold of (decay_j * state_i + state_j, decay_j * decay_i)
+            s_acc, a_acc = a[:, t] * s_acc + state[:, t], a[:, t] * a_acc
+        out[name] = s_acc.reshape(B, 1, H, *param_shape)
+    return out
+
+
 def softplus(x):
     return np.logaddexp(0.0, x)
 

@@ -132,3 +132,27 @@ def test_linear_scan_autograd_function():
     ag = G.diag_scan_grads(a, b, done, h0, g, gl)
     assert relerr(ta.grad, ag["da"]) <= TOL and relerr(tb.grad, ag["db"]) <= TOL
     assert relerr(th0.grad, ag["dh0"]) <= TOL
+
+
+@pytest.mark.parametrize("dtype", ["f32", "c64"])
+@pytest.mark.parametrize("shape", [(2, 9, 3, (2, 2)), (3, 130, 16, (8,)), (1, 1, 4, ()), (2, 64, 5, (3,)), (4, 257, 32, (16, 4))])
+def test_propagate_sensitivities(dtype, shape):
+    """RTRL sensitivity update (memoroid.py:114-141) through mrx_linear_scan_last."""
+    from memorax_amd.functional import propagate_sensitivities
+    B, T, H, ps = shape
+    rng = np.random.default_rng(B * 7 + T + H)
+    cplx = dtype == "c64"
+    rnd = (lambda *s: (rng.standard_normal(s) + 1j * rng.standard_normal(s)).astype(np.complex64)) if cplx \
+        else (lambda *s: rng.standard_normal(s).astype(np.float32))
+    decay = (rng.uniform(0.6, 1.0, (B, T, H)) * (np.exp(1j * rng.uniform(0, 6.28, (B, T, H))) if cplx else 1.0))
+    decay = decay.astype(np.complex64 if cplx else np.float32)
+    J = {"w": rnd(B, T, H, *ps), "u": rnd(B, T, H)}
+    S = {"w": rnd(B, 1, H, *ps), "u": rnd(B, 1, H)}
+    done = rng.random((B, T)) < 0.05
+    print(f"case rtrl dtype={dtype} shape={shape}", flush=True)
+    out = propagate_sensitivities(dev(decay), {k: dev(v) for k, v in J.items()}, {k: dev(v) for k, v in S.items()},
+                                  dev(done))
+    ref = M.propagate_sensitivities(decay, J, S, done)
+    for name in J:
+        assert out[name].shape == S[name].shape
+        assert relerr(out[name], ref[name]) <= 1e-4, (name, relerr(out[name], ref[name]))

@@ -326,3 +326,23 @@ def test_gated_linear_attention_split_invariance():
         o2, S2 = M.gated_linear_attention(q[:, s:], k[:, s:], v[:, s:], g[:, s:], done[:, s:], S1)
         np.testing.assert_allclose(np.concatenate([o1, o2], 1), o, rtol=1e-11, atol=1e-11)
         np.testing.assert_allclose(S2, S, rtol=1e-11, atol=1e-11)
+
+
+def test_propagate_sensitivities_is_the_diagonal_scan_with_repeated_decay():
+    rng = np.random.default_rng(8)
+    B, T, H, ps = 2, 9, 3, (2, 2)
+    decay = rng.uniform(0.5, 1.0, (B, T, H))
+    J = {"w": rng.standard_normal((B, T, H, *ps)), "b": rng.standard_normal((B, T, H))}
+    S = {"w": rng.standard_normal((B, 1, H, *ps)), "b": rng.standard_normal((B, 1, H))}
+    done = rng.random((B, T)) < 0.25
+    out = M.propagate_sensitivities(decay, J, S, done)
+    for name, n in (("w", 4), ("b", 1)):
+        a = np.repeat(decay, n, axis=-1)
+        h, h_last, _ = M.diag_scan(a, J[name].reshape(B, T, H * n), done, S[name].reshape(B, H * n))
+        np.testing.assert_allclose(out[name].reshape(B, H * n), h_last, rtol=1e-12, atol=1e-12)
+    # no resets, constant decay: closed form sum_s a^(T-s) J_s + a^T S
+    a0 = 0.9
+    o2 = M.propagate_sensitivities(np.full((B, T, H), a0), {"b": J["b"]}, {"b": S["b"]}, np.zeros((B, T), bool))
+    w = a0 ** np.arange(T - 1, -1, -1)
+    ref = (J["b"] * w[None, :, None]).sum(1) + a0 ** T * S["b"][:, 0]
+    np.testing.assert_allclose(o2["b"][:, 0], ref, rtol=1e-12, atol=1e-12)
