@@ -156,6 +156,76 @@ class LRUCell(_DiagonalCell):
                 torch.ones(*batch, 1, self.hidden_dim, dtype=torch.complex64, device=dev))
 
 
+def _dplr_hippo(n):
+    """Eigenvalues and eigenvectors of the normal part of the HiPPO-LegS matrix
+    (networks/hippo.py:6-37), in float64 NumPy."""
+    import numpy as np
+    p = np.sqrt(1.0 + 2.0 * np.arange(n))
+    a = -(np.tril(p[:, None] * p[None, :]) - np.diag(np.arange(n)))
+    pl = np.sqrt(np.arange(n) + 0.5)
+    sm = a + pl[:, None] * pl[None, :]
+    lam_real = np.full(n, np.mean(np.diag(sm)))
+    lam_imag, v = np.linalg.eigh(sm * (-1j))
+    return lam_real + 1j * lam_imag, v
+
+
+class S5Cell(_DiagonalCell):
+    """S5: diagonal state space model with HiPPO-N initialised eigenvalues, discretised with a
+    learned per-state step (s5.py:28-149).  As for the LRU the discretised decay is time-invariant
+    and goes to the kernel as an (N,) vector instead of being broadcast (s5.py:127)."""
+
+    def __init__(self, features, state_size, discretization="zoh", dt_min=0.001, dt_max=0.1,
+                 clip_eigens=False, step_rescale=1.0):
+        super().__init__()
+        import numpy as np
+        self.features, self.state_size = features, state_size
+        self.discretization, self.clip_eigens, self.step_rescale = discretization, clip_eigens, step_rescale
+        lam, v = _dplr_hippo(state_size)
+        v_inv = torch.from_numpy(v.conj().T.copy())
+        vt = torch.from_numpy(v.copy())
+        self.lambda_real = nn.Parameter(torch.from_numpy(lam.real.copy()).float())
+        self.lambda_imag = nn.Parameter(torch.from_numpy(lam.imag.copy()).float())
+        b = (v_inv @ (torch.randn(state_size, features, dtype=torch.float64) / math.sqrt(features)).to(v_inv.dtype))
+        c = (torch.randn(features, state_size, dtype=torch.float64).clamp(-2, 2).to(vt.dtype) @ vt)
+        self.B = nn.Parameter(torch.stack([b.real, b.imag], -1).float())     # (N, F, 2)
+        self.C = nn.Parameter(torch.stack([c.real, c.imag], -1).float())     # (F, N, 2)
+        self.d = nn.Parameter(torch.randn(features))
+        self.log_step = nn.Parameter(torch.rand(state_size, 1) * (math.log(dt_max) - math.log(dt_min)) + math.log(dt_min))
+
+    def _discretized_params(self):
+        lr = torch.clamp(self.lambda_real, max=-1e-4) if self.clip_eigens else self.lambda_real
+        lam = torch.complex(lr, self.lambda_imag)
+        b_tilde = torch.complex(self.B[..., 0], self.B[..., 1])
+        c_tilde = torch.complex(self.C[..., 0], self.C[..., 1])
+        step = (self.step_rescale * torch.exp(self.log_step[:, 0])).to(torch.complex64)
+        if self.discretization == "zoh":          # hippo.py:51-57
+            lambda_bar = torch.exp(lam * step)
+            b_bar = ((lambda_bar - 1.0) / lam)[:, None] * b_tilde
+        elif self.discretization == "bilinear":   # hippo.py:40-48
+            bl = 1.0 / (1.0 - (step / 2.0) * lam)
+            lambda_bar = bl * (1.0 + (step / 2.0) * lam)
+            b_bar = (bl * step)[:, None] * b_tilde
+        else:
+            raise ValueError(f"Invalid discretization: {self.discretization}")
+        return lambda_bar, b_bar, c_tilde
+
+    def forward(self, x, **kwargs):
+        lambda_bar, b_bar, _ = self._discretized_params()
+        state = x.to(torch.complex64) @ b_bar.T
+        return (state.contiguous(), lambda_bar.to(torch.complex64))
+
+    def read(self, h, x, **kwargs):
+        _, _, c_tilde = self._discretized_params()
+        state, _ = h
+        return (state @ c_tilde.T).real + self.d * x
+
+    def initialize_carry(self, key, input_shape):
+        *batch, _ = input_shape
+        dev = self.d.device
+        return (torch.zeros(*batch, 1, self.state_size, dtype=torch.complex64, device=dev),
+                torch.ones(*batch, 1, self.state_size, dtype=torch.complex64, device=dev))
+
+
 class MinGRUCell(_DiagonalCell):
     """MinGRU (min_gru.py:14-90).  The reference scans (log_state, log_decay) with
     logaddexp; the same recurrence in linear space is h_t = sigma(-z) h_{t-1} +

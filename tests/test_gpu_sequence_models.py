@@ -169,3 +169,26 @@ def test_mamba_model_matches_materialise_and_scan_reference():
     y.pow(2).mean().backward()
     assert torch.isfinite(cell.A_log.grad).all() and cell.A_log.grad.abs().sum() > 0
     assert cell.dt.weight.grad.abs().sum() > 0 and cell.C.weight.grad.abs().sum() > 0
+
+
+@pytest.mark.parametrize("disc", ["zoh", "bilinear"])
+def test_s5_memoroid_matches_generic_scan(disc):
+    from memorax_amd import sequence_models as sm
+    torch.manual_seed(9)
+    B, T, Fe, N = 2, 80, 10, 16
+    model = sm.Memoroid(sm.S5Cell(Fe, N, discretization=disc)).cuda()
+    x, done = _inputs(B, T, Fe, 0.05, 10)
+    carry, y = model(x, done)
+    assert carry[0].shape == (B, 1, N) and carry[0].dtype == torch.complex64 and y.shape == (B, T, Fe)
+    state, lam = model.cell(x)
+    el = (_np(state), np.broadcast_to(_np(lam), (B, T, N)).copy())
+    c0 = (np.zeros((B, 1, N), complex), np.ones((B, 1, N), complex))
+    (hs, _), nxt = M.scan_fn_tree(el, c0, _np(done.float()), M.diag_operator)
+    _, _, c_tilde = model.cell._discretized_params()
+    ry = (hs @ _np(c_tilde).T).real + _np(model.cell.d) * _np(x)
+    assert relerr(y, ry) <= 1e-4
+    assert relerr(carry[0], nxt[0]) <= 1e-4 and relerr(carry[1], nxt[1]) <= 1e-4
+    # the discretised decay is a contraction (HiPPO eigenvalues have negative real part)
+    assert (lam.abs() < 1).all()
+    y.sum().backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in model.parameters())
