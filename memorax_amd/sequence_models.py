@@ -540,6 +540,152 @@ class Mamba(SequenceModel):
         return self.cell.initialize_carry(key, input_shape)
 
 
+class _BlockDiagonalDense(nn.Module):
+    """One dense map per head (layers/block_diagonal_dense.py:10-50), no bias."""
+
+    def __init__(self, features, num_heads):
+        super().__init__()
+        bs = features // num_heads
+        self.num_heads = num_heads
+        self.kernel = nn.Parameter(torch.randn(num_heads, bs, bs) * math.sqrt(2.0 / (5.0 * bs)))
+
+    def forward(self, x):
+        *batch, f = x.shape
+        y = torch.einsum("...hd,hod->...ho", x.reshape(*batch, self.num_heads, -1), self.kernel)
+        return y.reshape(*batch, f)
+
+
+class mLSTMCell(MemoroidCellBase):
+    """Matrix LSTM (mlstm.py:31-240).  Elements (C = k (x) v, log_f, n = k, m = log_i) combine by the
+    max-stabilised gated sum of mlstm.py:190-206; read divides q C by max(|q . n|, exp(-m)) + 1e-6.
+    The stabiliser only rescales C and n by exp(-m), so the same numbers come from the plain gated
+    recurrence C~_t = f_t C~_{t-1} + i_t k_t v_t^T taken in units of exp(c) with one constant
+    c = max(log i, carried m) per sequence and head (every weight exp(log i - c) <= 1):
+        h = q C' / (max(|q . n'|, exp(-c)) + 1e-6 exp(m - c)).
+    q C' runs in the gated chunked kernel (k' = k exp(log i - c), log-decay log f), n' in the diagonal
+    scan, and m_t = max(m_{t-1} + log f_t, log i_t) is a cumulative maximum in log space.  Gates more
+    than about 80 nats below the running maximum underflow (the reference keeps them finite).
+    Carry: (C (B,1,H,d,d), log_f (B,1,H,1,1), n (B,1,H,d,1), m (B,1,H,1,1)) as in the reference."""
+
+    def __init__(self, features, hidden_dim, num_heads=4, conv_kernel_size=4, in_features=None):
+        super().__init__()
+        if hidden_dim % num_heads != 0:
+            raise ValueError(f"hidden_dim ({hidden_dim}) must be divisible by num_heads ({num_heads}).")
+        in_features = features if in_features is None else in_features
+        self.features, self.hidden_dim, self.num_heads = features, hidden_dim, num_heads
+        self.conv_kernel_size = conv_kernel_size
+        self.up_projection = nn.Linear(in_features, 2 * hidden_dim, bias=False)
+        self.causal_conv = nn.Conv1d(hidden_dim, hidden_dim, conv_kernel_size, groups=hidden_dim)
+        self.query = _BlockDiagonalDense(hidden_dim, num_heads)
+        self.key = _BlockDiagonalDense(hidden_dim, num_heads)
+        self.value = _BlockDiagonalDense(hidden_dim, num_heads)
+        self.i_gate = nn.Linear(3 * hidden_dim, num_heads)
+        self.f_gate = nn.Linear(3 * hidden_dim, num_heads)
+        with torch.no_grad():
+            self.i_gate.weight.zero_()
+            self.i_gate.bias.normal_(std=0.1)
+            self.f_gate.weight.zero_()
+            self.f_gate.bias.copy_(torch.linspace(3.0, 6.0, num_heads))
+        self.learnable_skip = nn.Parameter(torch.ones(hidden_dim))
+        self.norm_weight = nn.Parameter(torch.zeros(num_heads, hidden_dim // num_heads))
+        self.output_projection = nn.Linear(hidden_dim, features, bias=False)
+
+    def _project(self, x):
+        Bn, T, _ = x.shape
+        d = self.hidden_dim // self.num_heads
+        x_mlstm, z = self.up_projection(x).chunk(2, dim=-1)
+        u = F.silu(self.causal_conv(F.pad(x_mlstm.transpose(1, 2), (self.conv_kernel_size - 1, 0))).transpose(1, 2))
+        heads = lambda t: t.reshape(Bn, T, self.num_heads, d)  # noqa: E731
+        return heads(self.query(u)), heads(self.key(u)), heads(self.value(x_mlstm)), z, u
+
+    def forward(self, x, **kwargs):
+        """Elements in kernel form: (k / sqrt(d), v, log_i, log_f)."""
+        Bn, T, _ = x.shape
+        q, k, v, _, _ = self._project(x)
+        gate_input = torch.cat([q, k, v], dim=-1).reshape(Bn, T, -1)
+        log_i = self.i_gate(gate_input).float()
+        log_f = -F.softplus(-self.f_gate(gate_input).float())
+        return (k / math.sqrt(k.shape[-1]), v, log_i, log_f)
+
+    def binary_operator(self, a, b):
+        C_a, log_f_a, n_a, m_a = a
+        C_b, log_f_b, n_b, m_b = b
+        m_a_decayed = m_a + log_f_b
+        m = torch.maximum(m_a_decayed, m_b)
+        sa, sb = torch.exp(m_a_decayed - m), torch.exp(m_b - m)
+        return (sa * C_a + sb * C_b, log_f_a + log_f_b, sa * n_a + sb * n_b, m)
+
+    def scan(self, z, initial_carry, done, q=None):
+        k, v, log_i, log_f = z
+        C0, lf0, n0, m0 = initial_carry
+        Bn, T, H, d = k.shape
+        m0_ = m0[:, 0, :, 0, 0].float()                                        # (B,H)
+        c = torch.maximum(log_i.max(dim=1).values, m0_).detach()                # (B,H)
+        k_in = k.float() * torch.exp(log_i - c[:, None])[..., None]
+        w0 = torch.exp(m0_ - c)                                                 # <= 1; 0 for the initial carry
+        S0 = (C0[:, 0].float() * w0[..., None, None]).transpose(-1, -2).contiguous()
+        num, S_last = gated_linear_attention(q.float().contiguous(), k_in.contiguous(), v.float().contiguous(),
+                                             log_f.contiguous(), done, S0)
+        a = torch.exp(log_f)[..., None].expand(Bn, T, H, d).reshape(Bn, T, H * d).contiguous()
+        nvec, n_last, _ = linear_scan(a, k_in.reshape(Bn, T, H * d).contiguous(), done,
+                                      (n0[:, 0, :, :, 0].float() * w0[..., None]).reshape(Bn, H * d).contiguous())
+        qn = (q.float() * nvec.view(Bn, T, H, d)).sum(-1)                        # (B,T,H)
+        # m_t = max(m_{t-1} + log f_t, log i_t), restarted at resets: F_t + running max of (log i - F)
+        ones = torch.ones(H, device=k.device)
+        Fc, _, _ = linear_scan(ones, log_f.contiguous(), done, torch.zeros(Bn, H, device=k.device))
+        dn = done != 0
+        seg = torch.cumsum(dn.to(torch.float64), dim=1)[..., None]                # (B,T,1)
+        u = (log_i - Fc).double()
+        big = 2.0 * (u.max() - u.min()).detach() + 1.0
+        cm = torch.cummax(u + big * seg, dim=1).values - big * seg
+        cm = torch.where(seg == 0, torch.maximum(cm, m0_[:, None].double()), cm)
+        m = (Fc.double() + cm).float()                                          # (B,T,H)
+        den = torch.maximum(qn.abs(), torch.exp(-c)[:, None]) + 1e-6 * torch.exp(m - c[:, None])
+        h_tilde = num / den[..., None]
+        # carry in the reference's (stabilised) units
+        m_T = m[:, -1]
+        back = torch.exp(torch.clamp(c - m_T, max=80.0))
+        _, lf_last, _ = linear_scan(ones, log_f.contiguous(), done, lf0[:, 0, :, 0, 0].float().contiguous())
+        carry = ((S_last.transpose(-1, -2) * back[..., None, None])[:, None],
+                 lf_last[:, None, :, None, None],
+                 (n_last.view(Bn, H, d) * back[..., None])[:, None, :, :, None],
+                 m_T[:, None, :, None, None])
+        return h_tilde, carry
+
+    def read(self, h_tilde, x, **kwargs):
+        Bn, T, _ = x.shape
+        _, _, _, z, u = self._project(x)
+        y = F.layer_norm(h_tilde, (h_tilde.shape[-1],), eps=1e-5) * (1.0 + self.norm_weight)[None, None]
+        y = y.reshape(Bn, T, self.hidden_dim) + self.learnable_skip * u
+        return self.output_projection((y * F.silu(z)).to(x.dtype))
+
+    def initialize_carry(self, key, input_shape):
+        *batch, _ = input_shape
+        H, d = self.num_heads, self.hidden_dim // self.num_heads
+        dev = self.learnable_skip.device
+        return (torch.zeros(*batch, 1, H, d, d, device=dev), torch.zeros(*batch, 1, H, 1, 1, device=dev),
+                torch.zeros(*batch, 1, H, d, 1, device=dev), torch.full((*batch, 1, H, 1, 1), -1e9, device=dev))
+
+
+class mLSTM(SequenceModel):
+    """Memoroid(mLSTMCell) with the query inside the scan (the kernel fuses q C into it)."""
+
+    def __init__(self, cell: mLSTMCell):
+        super().__init__()
+        self.cell = cell
+
+    def forward(self, inputs, done, initial_carry=None, **kwargs):
+        if initial_carry is None:
+            initial_carry = self.cell.initialize_carry(None, get_input_shape(inputs))
+        z = self.cell(inputs)
+        q = self.cell._project(inputs)[0]
+        h_tilde, carry = self.cell.scan(z, initial_carry, done, q=q)
+        return carry, self.cell.read(h_tilde, inputs)
+
+    def initialize_carry(self, key, input_shape):
+        return self.cell.initialize_carry(key, input_shape)
+
+
 # ----------------------------------------------------------------------------------
 # block composition used by the torso configuration (blocks/{stack,residual,normalization}.py)
 # ----------------------------------------------------------------------------------

@@ -74,6 +74,18 @@ def delta_operator(a, b):
     return (B_i @ A_j + B_j, A_i @ A_j)
 
 
+def mlstm_operator(a, b):
+    """mlstm.py:190-206: max-stabilised gated sum of (C, log_f, n, m)."""
+    C_a, log_f_a, n_a, m_a = a
+    C_b, log_f_b, n_b, m_b = b
+    log_f = log_f_a + log_f_b
+    m_a_decayed = m_a + log_f_b
+    m_combined = np.maximum(m_a_decayed, m_b)
+    scale_a = np.exp(m_a_decayed - m_combined)
+    scale_b = np.exp(m_b - m_combined)
+    return (scale_a * C_a + scale_b * C_b, log_f, scale_a * n_a + scale_b * n_b, m_combined)
+
+
 # --------------------------------------------------------------------------
 # Memoroid.scan_fn, two independent formulations
 # --------------------------------------------------------------------------
@@ -403,6 +415,62 @@ def gated_linear_attention_quadratic(q, k, v, g, done, S0=None, feature_map="non
         m = (seg == 0)[:, :, None, None]
         o = o + m * np.exp(Gc)[..., None] * np.einsum("bihd,bhed->bihe", q, np.asarray(S0, np.float64))
     return o
+
+
+def mlstm_elements(q, k, v, i_gate, f_gate):
+    """mlstm.py:163-188: elements (C = k (x) v, log_f, n = k, m = log_i) with k pre-scaled by
+    1/sqrt(head_dim); q,k,v: (B,T,H,d), gates (B,T,H)."""
+    k = np.asarray(k, np.float64) / np.sqrt(k.shape[-1])
+    v = np.asarray(v, np.float64)
+    log_f = -softplus(-np.asarray(f_gate, np.float64))
+    log_i = np.asarray(i_gate, np.float64)
+    C = np.einsum("...i,...j->...ij", k, v)
+    return (C, log_f[..., None, None], k[..., None], log_i[..., None, None])
+
+
+def mlstm_read(h, q):
+    """mlstm.py:208-221 up to the division: h_tilde = q C / (max(|q . n|, exp(-m)) + 1e-6)."""
+    C, _, n, m = h
+    q = np.asarray(q, np.float64)
+    den = np.maximum(np.abs(np.einsum("...i,...i->...", q, n[..., 0])), np.exp(-m[..., 0, 0]))[..., None]
+    return np.einsum("...j,...jk->...k", q, C) / (den + 1e-6)
+
+
+def mlstm(q, k, v, i_gate, f_gate, done, carry=None, tree=True):
+    """The reference's route: scan the elements with the stabilised operator (memoroid.py:60-91),
+    read.  Returns (next_carry, h_tilde (B,T,H,d))."""
+    z = mlstm_elements(q, k, v, i_gate, f_gate)
+    B, T, H, d = np.asarray(q).shape
+    if carry is None:
+        carry = (np.zeros((B, 1, H, d, d)), np.zeros((B, 1, H, 1, 1)), np.zeros((B, 1, H, d, 1)),
+                 np.full((B, 1, H, 1, 1), -1e9))
+    scan = scan_fn_tree if tree else scan_fn_sequential
+    h, nxt = scan(z, carry, done, mlstm_operator)
+    return nxt, mlstm_read(h, q)
+
+
+def mlstm_unstabilised(q, k, v, i_gate, f_gate, done):
+    """The recurrence the docstring of mlstm.py:8-11 states, without the stabiliser:
+    C~_t = f_t C~_{t-1} + i_t k_t v_t^T, n~_t = f_t n~_{t-1} + i_t k_t (zero carry),
+    h = q C~ / (max(|q . n~|, 1) + 1e-6 exp(m_t)), m_t = max(m_{t-1} + log f_t, log i_t)."""
+    q, v = np.asarray(q, np.float64), np.asarray(v, np.float64)
+    k = np.asarray(k, np.float64) / np.sqrt(q.shape[-1])
+    log_f = -softplus(-np.asarray(f_gate, np.float64))
+    log_i = np.asarray(i_gate, np.float64)
+    B, T, H, d = q.shape
+    done = np.asarray(done) != 0
+    C = np.zeros((B, H, d, d)); n = np.zeros((B, H, d)); m = np.full((B, H), -1e9)
+    out = np.empty((B, T, H, d))
+    for t in range(T):
+        r = done[:, t]
+        f = np.where(r[:, None], 0.0, np.exp(log_f[:, t]))
+        i = np.exp(log_i[:, t])
+        C = f[..., None, None] * C + i[..., None, None] * np.einsum("bhi,bhj->bhij", k[:, t], v[:, t])
+        n = f[..., None] * n + i[..., None] * k[:, t]
+        m = np.where(r[:, None], log_i[:, t], np.maximum(m + log_f[:, t], log_i[:, t]))
+        den = np.maximum(np.abs((q[:, t] * n).sum(-1)), 1.0) + 1e-6 * np.exp(m)
+        out[:, t] = np.einsum("bhj,bhjk->bhk", q[:, t], C) / den[..., None]
+    return out
 
 
 def segment_ids(done):

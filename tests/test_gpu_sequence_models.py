@@ -192,3 +192,42 @@ def test_s5_memoroid_matches_generic_scan(disc):
     assert (lam.abs() < 1).all()
     y.sum().backward()
     assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in model.parameters())
+
+
+def test_mlstm_model_matches_stabilised_reference_scan():
+    """mLSTM(mLSTMCell) against the reference's route: elements (C, log_f, n, m) scanned with the
+    max-stabilised operator (mlstm.py:163-229 under memoroid.py:60-91), carry included."""
+    from memorax_amd import sequence_models as sm
+    torch.manual_seed(11)
+    B, T, Fe, H, d = 2, 100, 24, 2, 64
+    cell = sm.mLSTMCell(Fe, hidden_dim=H * d, num_heads=H).cuda()
+    with torch.no_grad():   # give the gates some input dependence (they start as pure biases)
+        cell.i_gate.weight.normal_(std=0.05)
+        cell.f_gate.weight.normal_(std=0.05)
+    model = sm.mLSTM(cell)
+    x, done = _inputs(B, T, Fe, 0.04, 12)
+    carry, y = model(x, done)
+    with torch.no_grad():
+        q, k, v, z, u = cell._project(x)
+        gi = torch.cat([q, k, v], dim=-1).reshape(B, T, -1)
+        ig, fg = cell.i_gate(gi), cell.f_gate(gi)
+    nxt, h_ref = M.mlstm(_np(q), _np(k), _np(v), _np(ig), _np(fg), _np(done.float()))
+    with torch.no_grad():
+        h_gpu, _ = cell.scan(cell(x), cell.initialize_carry(None, (B, Fe)), done, q=q)
+    assert relerr(h_gpu, h_ref) <= 2e-4, relerr(h_gpu, h_ref)
+    # carry leaves in the reference's stabilised units and shapes
+    for got, ref, tol in zip(carry, nxt, (2e-4, 1e-5, 2e-4, 1e-5)):
+        assert got.shape == ref.shape, (got.shape, ref.shape)
+        assert relerr(got, ref) <= tol, relerr(got, ref)
+    # split invariance through the carry, and gradients reach the gates
+    # (on the scan: the cell's causal convolution restarts at every call, in the reference too)
+    with torch.no_grad():
+        zz = cell(x)
+        h1, c1 = cell.scan(tuple(t[:, :37] for t in zz), cell.initialize_carry(None, (B, Fe)), done[:, :37], q=q[:, :37])
+        h2, c2 = cell.scan(tuple(t[:, 37:] for t in zz), c1, done[:, 37:], q=q[:, 37:])
+    assert relerr(torch.cat([h1, h2], 1), h_ref) <= 2e-4
+    for got, ref in zip(c2, nxt):
+        assert relerr(got, ref) <= 2e-4
+    y.pow(2).mean().backward()
+    assert cell.f_gate.bias.grad.abs().sum() > 0 and cell.i_gate.bias.grad.abs().sum() > 0
+    assert all(torch.isfinite(p.grad).all() for p in cell.parameters() if p.grad is not None)

@@ -346,3 +346,41 @@ def test_propagate_sensitivities_is_the_diagonal_scan_with_repeated_decay():
     w = a0 ** np.arange(T - 1, -1, -1)
     ref = (J["b"] * w[None, :, None]).sum(1) + a0 ** T * S["b"][:, 0]
     np.testing.assert_allclose(o2["b"][:, 0], ref, rtol=1e-12, atol=1e-12)
+
+
+# ---- mLSTM (stabilised gated linear attention) -------------------------------------------------
+def _mlstm_inputs(B=2, T=12, H=2, d=3, p=0.2, seed=0):
+    rng = np.random.default_rng(seed)
+    q, k, v = (rng.standard_normal((B, T, H, d)) for _ in range(3))
+    ig = rng.standard_normal((B, T, H)) * 2.0
+    fg = rng.standard_normal((B, T, H)) * 2.0 + 2.0
+    done = rng.random((B, T)) < p
+    return q, k, v, ig, fg, done
+
+
+def test_mlstm_operator_is_associative_and_orders_agree():
+    rng = np.random.default_rng(3)
+    def el():
+        return (rng.standard_normal((2, 1, 2, 3, 3)), -np.abs(rng.standard_normal((2, 1, 2, 1, 1))),
+                rng.standard_normal((2, 1, 2, 3, 1)), rng.standard_normal((2, 1, 2, 1, 1)) * 3)
+    a, b, c = el(), el(), el()
+    l = M.mlstm_operator(M.mlstm_operator(a, b), c)
+    r = M.mlstm_operator(a, M.mlstm_operator(b, c))
+    for x, y in zip(l, r):
+        np.testing.assert_allclose(x, y, rtol=1e-12, atol=1e-12)
+    q, k, v, ig, fg, done = _mlstm_inputs()
+    n1, h1 = M.mlstm(q, k, v, ig, fg, done, tree=True)
+    n2, h2 = M.mlstm(q, k, v, ig, fg, done, tree=False)
+    np.testing.assert_allclose(h1, h2, rtol=1e-10, atol=1e-12)
+    for x, y in zip(n1, n2):
+        np.testing.assert_allclose(x, y, rtol=1e-10, atol=1e-12)
+
+
+def test_mlstm_stabilised_scan_equals_plain_recurrence():
+    q, k, v, ig, fg, done = _mlstm_inputs(seed=4)
+    _, h = M.mlstm(q, k, v, ig, fg, done)
+    np.testing.assert_allclose(h, M.mlstm_unstabilised(q, k, v, ig, fg, done), rtol=1e-9, atol=1e-12)
+    # split invariance through the carry
+    nxt, ha = M.mlstm(q[:, :5], k[:, :5], v[:, :5], ig[:, :5], fg[:, :5], done[:, :5])
+    _, hb = M.mlstm(q[:, 5:], k[:, 5:], v[:, 5:], ig[:, 5:], fg[:, 5:], done[:, 5:], nxt)
+    np.testing.assert_allclose(np.concatenate([ha, hb], 1), h, rtol=1e-9, atol=1e-12)
