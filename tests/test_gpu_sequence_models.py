@@ -162,10 +162,14 @@ def test_mamba_model_matches_materialise_and_scan_reference():
     # carry leaves in the reference's layout: h is (N, P) = k (x) v, decay the product since the last reset
     assert relerr(carry[0][:, 0], nxt[0][:, 0].transpose(0, 1, 3, 2)) <= 2e-4
     assert relerr(carry[1][:, 0, :, 0, 0], nxt[1][:, 0, :, 0, 0]) <= 1e-5
-    # carry threading and gradients
-    c1, y1 = model(x[:, :50], done[:, :50])
-    c2, y2 = model(x[:, 50:], done[:, 50:], c1)
-    assert relerr(c2[0], _np(carry[0])) <= 2e-4
+    # carry threading (on the scan: the cell's causal convolution restarts at every call, in the
+    # reference too) and gradients
+    with torch.no_grad():
+        zz = cell(x)
+        o1, c1 = cell.scan(tuple(t[:, :50] for t in zz), cell.initialize_carry(None, (B, Fe)), done[:, :50], q=C_proj[:, :50])
+        o2, c2 = cell.scan(tuple(t[:, 50:] for t in zz), c1, done[:, 50:], q=C_proj[:, 50:])
+    assert relerr(torch.cat([o1, o2], 1), o) <= 2e-4
+    assert relerr(c2[0], _np(carry[0])) <= 2e-4 and relerr(c2[1], _np(carry[1])) <= 1e-5
     y.pow(2).mean().backward()
     assert torch.isfinite(cell.A_log.grad).all() and cell.A_log.grad.abs().sum() > 0
     assert cell.dt.weight.grad.abs().sum() > 0 and cell.C.weight.grad.abs().sum() > 0
