@@ -729,17 +729,6 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     }
 }
 
-template <typename K> int set_smem(K kern, int smem, bool &flag)
-{
-    if (!flag) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess)
-            return MRX_ERR_LAUNCH;
-        flag = true;
-    }
-    return MRX_OK;
-}
-
 template <typename T, int C, bool FMAP, bool GATED = false>
 int launch_la(hipStream_t st, const void *q, const void *k, const void *v, const void *done,
               int done_f32, const void *S_chk, const void *dout, const void *dS_last, void *dq,
@@ -748,8 +737,8 @@ int launch_la(hipStream_t st, const void *q, const void *k, const void *v, const
 {
     auto kern = la_bwd_kernel<T, C, FMAP, GATED>;
     constexpr int smem = LaBwdSmem<T, C, GATED>::total;
-    static bool attr_set = false;
-    if (set_smem(kern, smem, attr_set) != MRX_OK) return MRX_ERR_LAUNCH;
+    static unsigned long long lds_set = 0ull;
+    if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(256), smem, st, (const T *)q,
                        (const T *)k, (const T *)v, (const float *)glog, done, done_f32, (const T *)S_chk,
                        (const T *)dout, (const float *)dS_last, (T *)dq, (T *)dk, (T *)dv, (float *)edot,
@@ -831,8 +820,8 @@ extern "C" int mrx_delta_rule_bwd(void *stream, const void *q, const void *k, co
         constexpr int NW = MRX_DELTA_BWD_WAVES;
         auto kern = delta_bwd_kernel<__bf16, 64, NW, true>;
         constexpr int smem = DeltaBwdSmem<__bf16, 64, NW, true>::total;
-        static bool attr_set = false;
-        if (set_smem(kern, smem, attr_set) != MRX_OK) return MRX_ERR_LAUNCH;
+        static unsigned long long lds_set = 0ull;
+        if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
         hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(64 * NW), smem, st, (const __bf16 *)q,
                            (const __bf16 *)k, (const __bf16 *)v, (const __bf16 *)beta, done, done_dtype,
                            (const __bf16 *)S_chk, (const __bf16 *)Tm_chk, (const __bf16 *)dout,
@@ -842,8 +831,8 @@ extern "C" int mrx_delta_rule_bwd(void *stream, const void *q, const void *k, co
         constexpr int NW = 4;
         auto kern = delta_bwd_kernel<float, 32, NW, false>;
         constexpr int smem = DeltaBwdSmem<float, 32, NW, false>::total;
-        static bool attr_set = false;
-        if (set_smem(kern, smem, attr_set) != MRX_OK) return MRX_ERR_LAUNCH;
+        static unsigned long long lds_set = 0ull;
+        if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
         hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(64 * NW), smem, st, (const float *)q,
                            (const float *)k, (const float *)v, (const float *)beta, done, done_dtype,
                            (const float *)S_chk, (const float *)Tm_chk, (const float *)dout,

@@ -354,13 +354,8 @@ int launch(hipStream_t st, const void *q, const void *k, const void *v, const vo
 {
     auto kern = chunk_fwd_kernel<T, C, DELTA, FMAP, GATED>;
     constexpr int smem = FwdSmem<T, C, DELTA, GATED>::total;
-    static bool attr_set = false;  // idempotent; a race only repeats the call
-    if (!attr_set) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess)
-            return MRX_ERR_LAUNCH;
-        attr_set = true;
-    }
+    static unsigned long long lds_set = 0ull;
+    if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(NTHR), smem, st, (const T *)q,
                        (const T *)k, (const T *)v, (const T *)beta, (const float *)glog, done, done_f32,
                        (const float *)S0, (T *)o, (float *)S_last, (T *)S_chk, (T *)Tm_chk, (int)Tlen, (int)H);

@@ -32,6 +32,23 @@ inline int launch_status()
     return hipGetLastError() == hipSuccess ? MRX_OK : MRX_ERR_LAUNCH;
 }
 
+// Raises a kernel's dynamic LDS limit once per device (the attribute belongs to the device's
+// copy of the kernel).  `done` is a per-kernel bit mask indexed by device id; setting it twice
+// from racing threads only repeats an idempotent call.
+template <typename K> inline int ensure_lds_limit(K kern, int bytes, unsigned long long &done)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return MRX_ERR_LAUNCH;
+    const unsigned long long bit = 1ull << (dev & 63);
+    if (!(done & bit)) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                bytes) != hipSuccess)
+            return MRX_ERR_LAUNCH;
+        done |= bit;
+    }
+    return MRX_OK;
+}
+
 inline bool aligned(const void *p, size_t n)
 {
     return (reinterpret_cast<uintptr_t>(p) % n) == 0;
