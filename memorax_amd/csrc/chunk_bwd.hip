@@ -153,21 +153,53 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     typename IOS::Regs rS;
     uint32_t rdone = 0u;  // raw bits, tested when the chunk is staged
     float rg = 0.f;       // log-decay of chunk row `lane` (gated)
-    auto prefetch = [&](int c) {
-        const int t0 = c * C;
-        IO::load(rq, q + base, rs, t0, Tlen, tid);
-        IO::load(rk, k + base, rs, t0, Tlen, tid);
-        IO::load(rv, v + base, rs, t0, Tlen, tid);
-        IO::load(rdo, dout + base, rs, t0, Tlen, tid);
-        IOS::load(rS, S_chk + ((int64_t)bh * NC + c) * HD * HD, HD, 0, HD, tid);
-        rdone = 0u;
-        rg = 0.f;
-        if (lane < C && t0 + lane < Tlen) {
-            rdone = done_raw(done, done_f32, (int64_t)b * Tlen + t0 + lane);
-            if (GATED) rg = glog[((int64_t)b * Tlen + t0 + lane) * H + h];
+    // Running element offsets of this thread's loads, stepped back by one chunk per prefetch
+    // (64-bit adds instead of per-chunk index multiplications).  The prefetch is issued in parts
+    // spread over the phases so that the address unit works beside LDS and MFMA work:
+    // part 0: q, k; 1: v, dout; 2: S and the per-row scalars.
+    const int tlast = (NC - 1) * C;
+    int64_t roff[IO::PASSES];
+#pragma unroll
+    for (int p = 0; p < IO::PASSES; ++p)
+        roff[p] = base + (int64_t)(tlast + IO::row_of(tid, p)) * rs + (tid % IO::SEGS) * IO::KP;
+    int64_t soff = ((int64_t)bh * NC + NC - 1) * HD * HD + (tid / IOS::SEGS) * HD + (tid % IOS::SEGS) * IOS::KP;
+    int64_t doff = (int64_t)b * Tlen + tlast + lane;
+    int tpre = tlast;
+    auto prefetch_part = [&](int part) {
+        typename IO::F z;
+#pragma unroll
+        for (int e = 0; e < IO::KP; ++e) z[e] = (T)0.f;
+        if (part < 2) {
+#pragma unroll
+            for (int p = 0; p < IO::PASSES; ++p) {
+                const bool in = tpre + IO::row_of(tid, p) < Tlen;
+                if (part == 0) {
+                    rq.v[p] = in ? *reinterpret_cast<const typename IO::F *>(q + roff[p]) : z;
+                    rk.v[p] = in ? *reinterpret_cast<const typename IO::F *>(k + roff[p]) : z;
+                } else {
+                    rv.v[p] = in ? *reinterpret_cast<const typename IO::F *>(v + roff[p]) : z;
+                    rdo.v[p] = in ? *reinterpret_cast<const typename IO::F *>(dout + roff[p]) : z;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < IOS::PASSES; ++p)
+                rS.v[p] = *reinterpret_cast<const typename IOS::F *>(S_chk + soff + p * IOS::RPP * HD);
+            rdone = 0u;
+            rg = 0.f;
+            if (lane < C && tpre + lane < Tlen) {
+                rdone = done_raw(done, done_f32, doff);
+                if (GATED) rg = glog[doff * H + h];
+            }
+#pragma unroll
+            for (int p = 0; p < IO::PASSES; ++p) roff[p] -= (int64_t)C * rs;
+            soff -= HD * HD;
+            doff -= C;
+            tpre -= C;
         }
     };
-    prefetch(NC - 1);
+#pragma unroll
+    for (int part = 0; part < 3; ++part) prefetch_part(part);
 
     for (int c = NC - 1; c >= 0; --c) {
         const int t0 = c * C;
@@ -216,7 +248,8 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             if (pass != nres) zero_acc<TMS::TPW>(dSacc);  // an episode that ends inside the chunk
             store_acc<T, HD, HD, NW>(dSacc, sDS, LDD, w, lane);  // dS[dv][dk]
             sync_lds();
-            if (pass == 0 && c > 0) prefetch(c - 1);
+            const bool pre = pass == 0 && c > 0;
+            if (pre) prefetch_part(0);
 
             // ---- Aqk[i][j] = q_i.k_j, dAqk[i][j] = do_i.v_j, both j <= i ------------------
             {
@@ -247,6 +280,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 store_tril(acc, sDAqk);
             }
             sync_lds();
+            if (pre) prefetch_part(1);
             auto one = [](int, int) { return f32x4{1.f, 1.f, 1.f, 1.f}; };
             float ep[TMR::NBW];  // gated: per-lane partials of edot for rows nt * 16 + li
 #pragma unroll
@@ -275,6 +309,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 }
                 store_rows_global<T, C, NW>(acc, dv + base, rs, t0, Tlen, w, lane, one, live);
             }
+            if (pre) prefetch_part(2);
             // ---- dQ^T[dk][i] = sum_dv S[dv][dk] dO[i][dv] + sum_j K[j][dk] dAqk[i][j] ---------
             {
                 f32x4 acc[TMR::TPW];
