@@ -55,9 +55,12 @@ const char *mrx_status_string(int status);
 /* Library version, major*10000 + minor*100 + patch. */
 int mrx_version(void);
 
-/* Time-chunk length the chunked kernels use for `dtype`; fixes the layout of the
- * per-chunk state checkpoints S_chk: (B, H, ceil(T/chunk), dv, dk). */
+/* Time-chunk length the (gated) linear-attention kernels use for `dtype`; fixes the layout
+ * of the per-chunk state checkpoints S_chk: (B, H, ceil(T/chunk), dv, dk). */
 int64_t mrx_chunk_size(int dtype);
+
+/* The same for the delta-rule kernels (S_chk and Tm_chk of mrx_delta_rule_fwd/_bwd). */
+int64_t mrx_delta_chunk_size(int dtype);
 
 /* ---- diagonal linear recurrence --------------------------------------------
  * Replaces Memoroid.scan_fn (memoroid.py:60-91) driven by the diagonal algebra
@@ -118,7 +121,7 @@ int mrx_linear_attn_bwd(void *stream, const void *q, const void *k,
  *     S' = done_t ? 0 : S_{t-1} ;  S_t = S'(I - beta_t k_t k_t^T) + beta_t v_t k_t^T ;
  *     o_t = S_t q_t
  * beta: (B,T,H) in `dtype`; other arguments as for linear attention.
- * Tm_chk (nullable): (B,H,ceil(T/chunk),chunk,chunk) in `dtype`, receives each
+ * Tm_chk (nullable): (B,H,ceil(T/chunk),chunk,chunk) in `dtype` (chunk = mrx_delta_chunk_size), receives each
  * chunk's unit-lower-triangular factor (I + tril(diag(beta) K K^T, -1))^-1, block
  * diagonal by episode; like S_chk it is a residual the backward call requires. */
 int mrx_delta_rule_fwd(void *stream, const void *q, const void *k,

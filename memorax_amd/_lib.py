@@ -24,6 +24,7 @@ SIGNATURES = {
     "mrx_status_string": (ctypes.c_char_p, [_I]),
     "mrx_version": (_I, []),
     "mrx_chunk_size": (_L, [_I]),
+    "mrx_delta_chunk_size": (_L, [_I]),
     "mrx_linear_scan_fwd": (_I, [_P] * 9 + [_L] * 3 + [_I] * 3),
     "mrx_linear_scan_bwd": (_I, [_P] * 10 + [_L] * 3 + [_I] * 3),
     "mrx_linear_attn_fwd": (_I, [_P] * 9 + [_L] * 5 + [_I] * 3),

@@ -399,7 +399,7 @@ template <typename T, int C, int NW, bool SPLIT> struct DeltaBwdSmem : BwdDims<T
 };
 
 template <typename T, int C, int NW, bool SPLIT>
-__global__ void __launch_bounds__(64 * NW)
+__global__ void __launch_bounds__(64 * NW, (SPLIT && NW == 4) ? 2 : 1)  // bf16 with 32-step chunks: two workgroups per CU
 delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
                  const T *__restrict__ S_chk, const T *__restrict__ Tm_chk,
@@ -501,7 +501,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         } else {
 #pragma unroll
             for (int p = 0; p < IOT::PASSES; ++p)
-                rTm.v[p] = *reinterpret_cast<const typename IOT::F *>(Tm_chk + tmoff + p * IOT::RPP * C);
+                if (IOT::FULL || IOT::row_of(tid, p) < C)  // a [C][C] tile may have fewer segments than threads
+                    rTm.v[p] = *reinterpret_cast<const typename IOT::F *>(Tm_chk + tmoff + p * IOT::RPP * C);
 #pragma unroll
             for (int p = 0; p < IO::PASSES; ++p) {
                 rbrow[p] = tpre + IO::row_of(tid, p) < Tlen ? load_raw<T>(beta + boff[p]) : 0u;
@@ -814,7 +815,7 @@ extern "C" int mrx_linear_attn_bwd(void *stream, const void *q, const void *k, c
     hipStream_t st = (hipStream_t)stream;
     const bool fm = feature_map == MRX_FMAP_ELU1;
 #define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H
-    if (dtype == MRX_BF16) return fm ? launch_la<__bf16, 64, true>(MRX_ARGS) : launch_la<__bf16, 64, false>(MRX_ARGS);
+    if (dtype == MRX_BF16) return fm ? launch_la<__bf16, LA_BF16_CHUNK, true>(MRX_ARGS) : launch_la<__bf16, LA_BF16_CHUNK, false>(MRX_ARGS);
     return fm ? launch_la<float, 32, true>(MRX_ARGS) : launch_la<float, 32, false>(MRX_ARGS);
 #undef MRX_ARGS
 }
@@ -834,7 +835,7 @@ extern "C" int mrx_gated_linear_attn_bwd(void *stream, const void *q, const void
     const bool fm = feature_map == MRX_FMAP_ELU1;
 #define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, g, edot
     if (dtype == MRX_BF16)
-        return fm ? launch_la<__bf16, 64, true, true>(MRX_ARGS) : launch_la<__bf16, 64, false, true>(MRX_ARGS);
+        return fm ? launch_la<__bf16, LA_BF16_CHUNK, true, true>(MRX_ARGS) : launch_la<__bf16, LA_BF16_CHUNK, false, true>(MRX_ARGS);
     return fm ? launch_la<float, 32, true, true>(MRX_ARGS) : launch_la<float, 32, false, true>(MRX_ARGS);
 #undef MRX_ARGS
 }
@@ -852,9 +853,9 @@ extern "C" int mrx_delta_rule_bwd(void *stream, const void *q, const void *k, co
     if (!beta || !dbeta || !Tm_chk || !aligned(Tm_chk, 16)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == MRX_BF16) {
-        constexpr int NW = MRX_DELTA_BWD_WAVES;
-        auto kern = delta_bwd_kernel<__bf16, 64, NW, true>;
-        constexpr int smem = DeltaBwdSmem<__bf16, 64, NW, true>::total;
+        constexpr int NW = DELTA_BF16_CHUNK == 64 ? MRX_DELTA_BWD_WAVES : 4;
+        auto kern = delta_bwd_kernel<__bf16, DELTA_BF16_CHUNK, NW, true>;
+        constexpr int smem = DeltaBwdSmem<__bf16, DELTA_BF16_CHUNK, NW, true>::total;
         static unsigned long long lds_set = 0ull;
         if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
         hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(64 * NW), smem, st, (const __bf16 *)q,

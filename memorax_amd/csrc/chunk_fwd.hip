@@ -381,7 +381,9 @@ int check_common(const void *q, const void *k, const void *v, const void *done, 
 
 }  // namespace
 
-extern "C" int64_t mrx_chunk_size(int dtype) { return dtype == MRX_BF16 ? 64 : (dtype == MRX_F32 ? 32 : 0); }
+extern "C" int64_t mrx_chunk_size(int dtype) { return dtype == MRX_BF16 ? LA_BF16_CHUNK : (dtype == MRX_F32 ? 32 : 0); }
+
+extern "C" int64_t mrx_delta_chunk_size(int dtype) { return dtype == MRX_BF16 ? DELTA_BF16_CHUNK : (dtype == MRX_F32 ? 32 : 0); }
 
 extern "C" int mrx_linear_attn_fwd(void *stream, const void *q, const void *k, const void *v,
                                    const void *done, const void *S0, void *o, void *S_last,
@@ -394,8 +396,8 @@ extern "C" int mrx_linear_attn_fwd(void *stream, const void *q, const void *k, c
     hipStream_t st = (hipStream_t)stream;
     const bool fm = feature_map == MRX_FMAP_ELU1;
     if (dtype == MRX_BF16)
-        return fm ? launch<__bf16, 64, false, true>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H)
-                  : launch<__bf16, 64, false, false>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H);
+        return fm ? launch<__bf16, LA_BF16_CHUNK, false, true>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H)
+                  : launch<__bf16, LA_BF16_CHUNK, false, false>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H);
     return fm ? launch<float, 32, false, true>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H)
               : launch<float, 32, false, false>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H);
 }
@@ -410,7 +412,7 @@ extern "C" int mrx_delta_rule_fwd(void *stream, const void *q, const void *k, co
     if (!beta || !aligned(Tm_chk, 16)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == MRX_BF16)
-        return launch<__bf16, 64, true, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H);
+        return launch<__bf16, DELTA_BF16_CHUNK, true, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H);
     return launch<float, 32, true, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H);
 }
 
@@ -427,7 +429,7 @@ extern "C" int mrx_gated_linear_attn_fwd(void *stream, const void *q, const void
     const bool fm = feature_map == MRX_FMAP_ELU1;
 #define MRX_ARGS st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H, g
     if (dtype == MRX_BF16)
-        return fm ? launch<__bf16, 64, false, true, true>(MRX_ARGS) : launch<__bf16, 64, false, false, true>(MRX_ARGS);
+        return fm ? launch<__bf16, LA_BF16_CHUNK, false, true, true>(MRX_ARGS) : launch<__bf16, LA_BF16_CHUNK, false, false, true>(MRX_ARGS);
     return fm ? launch<float, 32, false, true, true>(MRX_ARGS) : launch<float, 32, false, false, true>(MRX_ARGS);
 #undef MRX_ARGS
 }

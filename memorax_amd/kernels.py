@@ -52,8 +52,10 @@ def _done(done, B, T):
     return done, _lib.MRX_DONE_U8
 
 
-def chunk_size(dtype) -> int:
-    return int(_lib.load().mrx_chunk_size(_DT[dtype]))
+def chunk_size(dtype, delta=False) -> int:
+    """Chunk length of the (gated) linear-attention kernels, or of the delta-rule kernels."""
+    lib = _lib.load()
+    return int((lib.mrx_delta_chunk_size if delta else lib.mrx_chunk_size)(_DT[dtype]))
 
 
 # ----------------------------------------------------------------- diagonal scan
@@ -136,8 +138,8 @@ def _attn_shapes(q, k, v):
     return B, T, H, dk, dv, dt
 
 
-def _n_chunks(T, dt):
-    C = chunk_size(dt)
+def _n_chunks(T, dt, delta=False):
+    C = chunk_size(dt, delta)
     return (T + C - 1) // C
 
 
@@ -176,21 +178,31 @@ def linear_attn_bwd(q, k, v, done, S_chk, do, dS_last=None, feature_map=0, want_
     return dq, dk_, dv_, dS0
 
 
-def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True):
+def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None):
     """Returns (o, S_last fp32, chk) where chk = (S_chk, Tm_chk) are the residuals the
-    backward call needs, or None."""
+    backward call needs, or None.  out = (o, S_last, S_chk, Tm_chk) reuses buffers of an earlier
+    call with the same shapes instead of allocating."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
     _chk(beta, "beta", dt, (B, T, H))
     _chk(S0, "S0", torch.float32, (B, H, dv, dk))
     done, dd = _done(done, B, T)
-    o = torch.empty_like(v)
-    S_last = torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
-    S_chk = Tm_chk = None
-    if save_chk:
-        C, NC = chunk_size(dt), _n_chunks(T, dt)
-        S_chk = torch.empty((B, H, NC, dv, dk), dtype=dt, device=q.device)
-        Tm_chk = torch.empty((B, H, NC, C, C), dtype=dt, device=q.device)
+    if out is not None:
+        o, S_last, S_chk, Tm_chk = out
+        C, NC = chunk_size(dt, True), _n_chunks(T, dt, True)
+        _chk(o, "out o", dt, (B, T, H, dv))
+        _chk(S_last, "out S_last", torch.float32, (B, H, dv, dk))
+        _chk(S_chk, "out S_chk", dt, (B, H, NC, dv, dk))
+        _chk(Tm_chk, "out Tm_chk", dt, (B, H, NC, C, C))
+        save_chk = S_chk is not None
+    else:
+        o = torch.empty_like(v)
+        S_last = torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
+        S_chk = Tm_chk = None
+        if save_chk:
+            C, NC = chunk_size(dt, True), _n_chunks(T, dt, True)
+            S_chk = torch.empty((B, H, NC, dv, dk), dtype=dt, device=q.device)
+            Tm_chk = torch.empty((B, H, NC, C, C), dtype=dt, device=q.device)
     st = lib.mrx_delta_rule_fwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done),
                                 _ptr(S0), _ptr(o), _ptr(S_last), _ptr(S_chk), _ptr(Tm_chk), B, T, H,
                                 dk, dv, _DT[dt], dd)
@@ -198,22 +210,29 @@ def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True):
     return o, S_last, ((S_chk, Tm_chk) if save_chk else None)
 
 
-def delta_rule_bwd(q, k, v, beta, done, chk, do, dS_last=None, want_dS0=True):
-    """chk = (S_chk, Tm_chk) from delta_rule_fwd.  Returns (dq, dk, dv, dbeta, dS0)."""
+def delta_rule_bwd(q, k, v, beta, done, chk, do, dS_last=None, want_dS0=True, out=None):
+    """chk = (S_chk, Tm_chk) from delta_rule_fwd.  Returns (dq, dk, dv, dbeta, dS0).
+    out = (dq, dk, dv, dbeta, dS0) reuses buffers instead of allocating."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
     S_chk, Tm_chk = chk
-    C = chunk_size(dt)
-    _chk(Tm_chk, "Tm_chk", dt, (B, H, _n_chunks(T, dt), C, C))
+    C = chunk_size(dt, True)
+    _chk(Tm_chk, "Tm_chk", dt, (B, H, _n_chunks(T, dt, True), C, C))
     _chk(beta, "beta", dt, (B, T, H))
     _chk(do, "do", dt, (B, T, H, dv))
-    _chk(S_chk, "S_chk", dt, (B, H, _n_chunks(T, dt), dv, dk))
+    _chk(S_chk, "S_chk", dt, (B, H, _n_chunks(T, dt, True), dv, dk))
     _chk(dS_last, "dS_last", torch.float32, (B, H, dv, dk))
     done, dd = _done(done, B, T)
-    dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    dbeta = torch.empty_like(beta)
-    dS0 = (torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
-           if want_dS0 else None)
+    if out is not None:
+        dq, dk_, dv_, dbeta, dS0 = out
+        for t_, n_, ref in ((dq, "out dq", q), (dk_, "out dk", k), (dv_, "out dv", v), (dbeta, "out dbeta", beta)):
+            _chk(t_, n_, dt, tuple(ref.shape))
+        _chk(dS0, "out dS0", torch.float32, (B, H, dv, dk))
+    else:
+        dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        dbeta = torch.empty_like(beta)
+        dS0 = (torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
+               if want_dS0 else None)
     st = lib.mrx_delta_rule_bwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done),
                                 _ptr(S_chk), _ptr(Tm_chk), _ptr(do), _ptr(dS_last), _ptr(dq), _ptr(dk_),
                                 _ptr(dv_), _ptr(dbeta), _ptr(dS0), B, T, H, dk, dv, _DT[dt], dd)

@@ -26,7 +26,7 @@ def _declared():
 def test_header_declares_the_expected_entry_points():
     names = set(_declared())
     assert {"mrx_linear_scan_fwd", "mrx_linear_scan_bwd", "mrx_linear_attn_fwd", "mrx_linear_attn_bwd",
-            "mrx_delta_rule_fwd", "mrx_delta_rule_bwd", "mrx_chunk_size", "mrx_status_string",
+            "mrx_delta_rule_fwd", "mrx_delta_rule_bwd", "mrx_chunk_size", "mrx_delta_chunk_size", "mrx_status_string",
             "mrx_version"} <= names
 
 
@@ -52,6 +52,7 @@ def test_status_strings_and_chunk_size_without_gpu():
     assert lib.mrx_status_string(0) == b"ok"
     assert b"unsupported" in lib.mrx_status_string(-2)
     assert lib.mrx_chunk_size(_lib.MRX_BF16) == 64 and lib.mrx_chunk_size(_lib.MRX_F32) == 32
+    assert lib.mrx_delta_chunk_size(_lib.MRX_BF16) == 32 and lib.mrx_delta_chunk_size(_lib.MRX_F32) == 32
     assert lib.mrx_version() >= 100
 
 
