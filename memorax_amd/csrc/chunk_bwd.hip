@@ -399,7 +399,7 @@ template <typename T, int C, int NW, bool SPLIT> struct DeltaBwdSmem : BwdDims<T
 };
 
 template <typename T, int C, int NW, bool SPLIT>
-__global__ void __launch_bounds__(64 * NW, (SPLIT && NW == 4) ? 2 : 1)  // bf16 with 32-step chunks: two workgroups per CU
+__global__ void __launch_bounds__(64 * NW, (sizeof(T) == 2 && NW == 4) ? 2 : 1)  // bf16 with 32-step chunks: two workgroups per CU
 delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
                  const T *__restrict__ S_chk, const T *__restrict__ Tm_chk,
@@ -853,9 +853,12 @@ extern "C" int mrx_delta_rule_bwd(void *stream, const void *q, const void *k, co
     if (!beta || !dbeta || !Tm_chk || !aligned(Tm_chk, 16)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == MRX_BF16) {
+        // 64-step chunks: 8 waves in two groups, one workgroup per CU; 32-step chunks: 4 waves, one
+        // group (measured 2 % faster than two groups of 2), two workgroups per CU
         constexpr int NW = DELTA_BF16_CHUNK == 64 ? MRX_DELTA_BWD_WAVES : 4;
-        auto kern = delta_bwd_kernel<__bf16, DELTA_BF16_CHUNK, NW, true>;
-        constexpr int smem = DeltaBwdSmem<__bf16, DELTA_BF16_CHUNK, NW, true>::total;
+        constexpr bool SPLIT = DELTA_BF16_CHUNK == 64;
+        auto kern = delta_bwd_kernel<__bf16, DELTA_BF16_CHUNK, NW, SPLIT>;
+        constexpr int smem = DeltaBwdSmem<__bf16, DELTA_BF16_CHUNK, NW, SPLIT>::total;
         static unsigned long long lds_set = 0ull;
         if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
         hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(64 * NW), smem, st, (const __bf16 *)q,
