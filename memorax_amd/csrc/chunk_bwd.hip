@@ -720,12 +720,14 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                 for (int j = 0; j < GR::TPW; ++j) {
                     const int d0 = GR::mt(wl, j) * 16 + 4 * lg, r = GR::nt(wl, j) * 16 + li;
-                    *reinterpret_cast<f32x4 *>(sR + r * LDR + d0) = acc[j] * sBeta[r];
+                    if (SPLIT) *reinterpret_cast<f32x4 *>(sR + r * LDR + d0) = acc[j] * sBeta[r];
+                    else dKacc[j] += acc[j] * sBeta[r];  // one group: the wave holds the matching dK tiles itself
                 }
             }
             if (g1) {
                 // ---- dK^T[dk][j] += sum_i beta_i K[i][dk] dA[i][j] ---------------------------------------
                 gemm<T, HD, C, C, KROW, KROW, GW>(dKacc, sBK, LDD, sDA, LDC, wl, lane);
+                if (!SPLIT) store_rows_at<T, C, GW>(dKacc, dk + goff, rs, t0, Tlen, wl, lane, one, live);
             }
             // ---- dbeta: reduce the partials over lane groups, then over waves through LDS -----------
 #pragma unroll
@@ -737,7 +739,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();
             MRX_PHASE(23);
-            if (g1) {
+            if (SPLIT && g1) {
                 // ---- dK += beta_i R -> global ---------------------------------------------------------
 #pragma unroll
                 for (int j = 0; j < GR::TPW; ++j) {
