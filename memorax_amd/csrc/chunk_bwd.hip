@@ -3,30 +3,21 @@
 // Chunks are walked from the last to the first with dS (gradient of the state
 // leaving the chunk) carried in MFMA accumulators; the state entering each chunk
 // comes from the checkpoints the forward call wrote (S_chk), as does the delta rule's
-// triangular factor Tm (Tm_chk); everything else of the forward (W, U', masked QK^T) is
+// triangular factor Tm (Tm_chk); everything else of the forward (U', masked QK^T) is
 // recomputed per chunk.  A chunk that
 // contains resets is processed once per episode, last episode first, with the rows
 // of the other episodes zeroed by select; dS only flows into the episode that
 // leaves the chunk and only out of the episode that enters it.
 //
-// Per pass (rows i >= j; all rows of one episode):
-//   Aqk = tril(Q K^T)                      dU' = Aqk^T dO + K dS^T
-//   dAqk = tril(dO U'^T)                   dQ  = dO S + dAqk K
-//   dK  = dAqk^T Q + U' dS                 dS <- dS + Q^T dO - W^T dU'   (stored as dS^T)
-//   linear attention: U' = V, dV = dU', W = 0.
-//   delta rule:  A = tril(diag(beta) K K^T, -1), Tm = (I+A)^-1 (from the forward call), T = Tm diag(beta),
-//     W = T K, U' = T V - W S^T, dW = -dU' S, Zu = Tm^T dU', Zw = Tm^T dW,
-//     dV = diag(beta) Zu, dK += diag(beta) Zw, dbeta = rowdot(V, Zu) + rowdot(K, Zw),
-//     dT = tril(dW K^T + dU' V^T), dA = -tril((Tm^T dT) T^T, -1),
-//     R = dA K, dbeta += rowdot(K, R), dK += diag(beta) R + dA^T (diag(beta) K).
-// The products with T are taken as Tm times the row-scaled tiles beta_j K_j, beta_j V_j.
+// Linear attention per pass (rows i >= j; all rows of one episode):
+//   Aqk = tril(Q K^T)                      dV  = Aqk^T dO + K dS^T
+//   dAqk = tril(dO V^T)                    dQ  = dO S + dAqk K
+//   dK  = dAqk^T Q + V dS                  dS <- dS + Q^T dO            (stored as dS^T)
+// The delta rule's formulas stand at its kernel.
 // Every tile lives in LDS once, in its natural orientation; products that contract over
 // the row index read it through transpose loads (KROW operands).
 #include "chunk_common.h"
 
-#ifndef MRX_DELTA_BWD_WAVES
-#define MRX_DELTA_BWD_WAVES 8  // waves per workgroup of the delta-rule backward kernel (4 or 8)
-#endif
 
 namespace {
 
@@ -382,24 +373,33 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 }
 
 // =====================================================================================
-// delta rule: fifteen LDS tiles (138 KB for bf16 / C = 64, 133 KB for fp32 / C = 32; one
-// workgroup per CU), two of them reused once their first tenant is dead; NW waves
+// delta rule: fourteen LDS tiles (68 KB for bf16, 127 KB for fp32, C = 32), three of them reused
+// once their first tenant is dead.  bf16: two workgroups per CU.
+//
+// Per pass, with S the state entering the chunk, Tm = (I + A)^-1 from the forward call:
+//   V0 = V - K S^T,  V~ = diag(beta) V0,  U' = Tm V~            (W = T K and U = T V are never formed)
+//   Aqk = tril(Q K^T),  dU' = Aqk^T dO + K dS^T,  dAqk = tril(dO U'^T)
+//   Z = Tm^T dU',  dV = diag(beta) Z,  dbeta = rowdot(Z, V0) + rowdot(K, R)
+//   dTm = tril(dU' V~^T),  dA = -tril((Tm^T dTm) Tm^T, -1),  R = dA K
+//   dQ = dO S + dAqk K
+//   dK = dAqk^T Q + U' dS - (diag(beta) Z) S + diag(beta) R + dA^T (diag(beta) K)
+//   dS <- dS + Q^T dO - K^T (diag(beta) Z)                       (stored as dS^T)
 // =====================================================================================
-template <typename T, int C, int NW, bool SPLIT> struct DeltaBwdSmem : BwdDims<T, C> {
+template <typename T, int C, int NW> struct DeltaBwdSmem : BwdDims<T, C> {
     using D = BwdDims<T, C>;
-    // ten [C][64] tiles, two [64][64], three [C][C]; Y1 and dA reuse the dO and S tiles
     static_assert(D::szCC <= D::szRD && D::szCC <= D::szDD, "reused regions must hold a [C][C] tile");
+    // nine [C][64] tiles, two [64][64], three [C][C]
     static constexpr int oK = 0, oV = oK + D::szRD, oQ = oV + D::szRD, oDO = oQ + D::szRD,
-                         oW = oDO + D::szRD, oBK = oW + D::szRD, oBV = oBK + D::szRD, oU = oBV + D::szRD,
-                         oDU = oU + D::szRD, oDW = oDU + D::szRD, oS = oDW + D::szRD, oDS = oS + D::szDD,
+                         oBK = oDO + D::szRD, oVt = oBK + D::szRD, oU = oVt + D::szRD, oDU = oU + D::szRD,
+                         oZb = oDU + D::szRD, oS = oZb + D::szRD, oDS = oS + D::szDD,
                          oAqk = oDS + D::szDD, oTm = oAqk + D::szCC, oDT = oTm + D::szCC,
                          oBeta = oDT + D::szCC, oDb = oBeta + C * 4;
-    static constexpr int NSLOT = (SPLIT ? 2 : 1) * TileMap<HD, C, SPLIT ? NW / 2 : NW>::WM;
+    static constexpr int NSLOT = TileMap<HD, C, NW>::WM;  // dbeta partials per row: one per feature block
     static constexpr int total = oDb + NSLOT * C * 4;
 };
 
-template <typename T, int C, int NW, bool SPLIT>
-__global__ void __launch_bounds__(64 * NW, (sizeof(T) == 2 && NW == 4) ? 2 : 1)  // bf16 with 32-step chunks: two workgroups per CU
+template <typename T, int C, int NW>
+__global__ void __launch_bounds__(64 * NW, sizeof(T) == 2 ? 2 : 1)
 delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
                  const T *__restrict__ S_chk, const T *__restrict__ Tm_chk,
@@ -408,7 +408,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                  float *__restrict__ dS0, int Tlen, int H)
 {
     constexpr int NTHR = 64 * NW;
-    using L = DeltaBwdSmem<T, C, NW, SPLIT>;
+    using L = DeltaBwdSmem<T, C, NW>;
     using IO = TileIO<T, C, NTHR>;
     using IOS = TileIO<T, HD, NTHR>;
     using IOT = TileIO<T, C, NTHR, C>;  // the [C][C] triangular factor
@@ -416,50 +416,36 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     constexpr int LDD = L::LDD, LDC = L::LDC;
     extern __shared__ __align__(16) unsigned char smem[];
     auto at = [&](int off) { return reinterpret_cast<T *>(smem + off); };
-    T *sK = at(L::oK), *sV = at(L::oV), *sQ = at(L::oQ), *sW = at(L::oW);
-    T *sBK = at(L::oBK), *sBV = at(L::oBV);               // beta_j K_j, beta_j V_j
-    T *sU = at(L::oU), *sDU = at(L::oDU), *sDW = at(L::oDW);
-    T *sDO = at(L::oDO), *sY1 = at(L::oDO);               // dO[c][dv] -> Y1[j][b] beta_b
+    T *sK = at(L::oK), *sQ = at(L::oQ), *sDO = at(L::oDO), *sBK = at(L::oBK);
+    T *sV = at(L::oV);                                    // V[c][dv] -> V0 = V - K S^T (in place)
+    T *sVt = at(L::oVt), *sY1 = at(L::oVt);               // V~ = beta V0 -> Y1[j][b]
+    T *sU = at(L::oU), *sDU = at(L::oDU), *sZb = at(L::oZb);
     T *sS = at(L::oS), *sDA = at(L::oS);                  // S[dv][dk] -> dA[i][j]
     T *sDS = at(L::oDS);                                  // dS[dv][dk]
     T *sAqk = at(L::oAqk), *sDAqk = at(L::oAqk);          // Aqk[i][j] -> dAqk[i][j]
-    T *sTm = at(L::oTm), *sDT = at(L::oDT);               // Tm[i][j], dT[a][b]
+    T *sTm = at(L::oTm), *sDT = at(L::oDT);               // Tm[i][j], dTm[a][b]
     float *sBeta = reinterpret_cast<float *>(smem + L::oBeta);
     float *sDb = reinterpret_cast<float *>(smem + L::oDb);  // [NSLOT][C] dbeta partials
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // SPLIT: the waves form two groups.  Most phases hold two independent products of the same
-    // size: each group takes one of them whole, so that a wave owns a 2 x 2 block of result tiles
-    // and reads one operand fragment per MFMA from LDS (a 1 x 2 row of tiles needs 1.5).
-    // Without SPLIT every wave works on every product (one group of NW waves).
-    constexpr int GW = SPLIT ? NW / 2 : NW;
-    const int grp = w / GW, wl = w % GW;
-    const bool g0 = !SPLIT || grp == 0, g1 = !SPLIT || grp == 1;
     const int li = lane & 15, lg = lane >> 4;
     const int bh = blockIdx.x, b = bh / H, h = bh % H;
     const int64_t rs = (int64_t)H * HD;
     const int64_t base = ((int64_t)b * Tlen * H + h) * HD;
     const int NC = (Tlen + C - 1) / C;
 
-    using TMA = TileMap<C, C, NW>;   // products without a partner: all waves
-    using GS = TileMap<HD, HD, GW>;  // group maps
-    using GA = TileMap<C, C, GW>;
-    using GR = TileMap<HD, C, GW>;
-    constexpr int NSLOT = L::NSLOT;  // dbeta partials per row: one per group and feature block
-    static_assert(NSLOT == (SPLIT ? 2 : 1) * GR::WM, "sDb slots");
-    // fp32 R tile over the U' and dU' tiles: both are dead by then and neither is written before
-    // the second barrier of the next pass, so no barrier is needed after the last phase
-    constexpr int LDR = HD + 4;
-    static_assert(C * LDR * 4 <= 2 * L::szRD && L::oDU == L::oU + L::szRD, "R tile must fit");
-    float *sR = reinterpret_cast<float *>(smem + L::oU);
+    using TMS = TileMap<HD, HD, NW>;
+    using TMA = TileMap<C, C, NW>;
+    using TMR = TileMap<HD, C, NW>;
+    constexpr int NSLOT = L::NSLOT;
 
-    f32x4 dSacc[GS::TPW];  // dS^T: m = dk, n = dv (group 0)
+    f32x4 dSacc[TMS::TPW];  // dS^T: m = dk, n = dv
 #pragma unroll
-    for (int j = 0; j < GS::TPW; ++j) {
-        const int dk0 = GS::mt(wl, j) * 16 + 4 * lg, dvv = GS::nt(wl, j) * 16 + li;
-        dSacc[j] = (dS_last && g0) ? *reinterpret_cast<const f32x4 *>(dS_last + ((int64_t)bh * HD + dvv) * HD + dk0)
-                                         : f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < TMS::TPW; ++j) {
+        const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
+        dSacc[j] = dS_last ? *reinterpret_cast<const f32x4 *>(dS_last + ((int64_t)bh * HD + dvv) * HD + dk0)
+                           : f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
     typename IO::Regs rq, rk, rv, rdo;
@@ -551,158 +537,151 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                 for (int p = 0; p < IO::PASSES; ++p) bf[p] = raw_to_float<T>(rbrow[p]);
                 IO::scale_rows(fk, bf);
-                IO::scale_rows(fv, bf);
                 IO::to_lds(fk, sBK, LDD, tid);
-                IO::to_lds(fv, sBV, LDD, tid);
                 typename IOS::Regs fS = rS;
                 if (pass != 0) IOS::zero(fS);
                 IOS::to_lds(fS, sS, LDD, tid);
                 IOT::to_lds(rTm, sTm, LDC, tid);  // Tm[i][j] from the forward call (block diagonal by episode)
             }
             if (tid < C) sBeta[tid] = live(tid) ? raw_to_float<T>(rbeta) : 0.f;
-            if (pass != nres) zero_acc<GS::TPW>(dSacc);
-            if (g0) store_acc<T, HD, HD, GW>(dSacc, sDS, LDD, wl, lane);  // dS[dv][dk]
+            if (pass != nres) zero_acc<TMS::TPW>(dSacc);
+            store_acc<T, HD, HD, NW>(dSacc, sDS, LDD, w, lane);  // dS[dv][dk]
             sync_lds();
             MRX_PHASE(11);
             const bool pre = pass == 0 && c > 0;
             if (pre) prefetch_part(0);
 
             auto tril = [](int m, int n, float x) { return m <= n ? x : 0.f; };
-            if (g0) {
-                // ---- Aqk[i][j] = q_i . k_j, j <= i : D[m = j][n = i] -> sAqk[i][j] ------------------
-                f32x4 acc[GA::TPW];
-                zero_acc<GA::TPW>(acc);
-                gemm<T, C, C, HD, ROWK, ROWK, GW>(acc, sK, LDD, sQ, LDD, wl, lane);
-                store_acc_f<T, C, C, GW>(acc, sAqk, LDC, wl, lane, tril);
+            // ---- Aqk[i][j] = q_i . k_j, j <= i : D[m = j][n = i] -> sAqk[i][j] ----------------------
+            {
+                f32x4 acc[TMA::TPW];
+                zero_acc<TMA::TPW>(acc);
+                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sK, LDD, sQ, LDD, w, lane);
+                store_acc_f<T, C, C, NW>(acc, sAqk, LDC, w, lane, tril);
             }
-            if (g1) {
-                // ---- W^T[dk][c] = sum_j beta_j K[j][dk] Tm[c][j] -> sW[c][dk] -----------------------
-                f32x4 acc[GR::TPW];
-                zero_acc<GR::TPW>(acc);
-                gemm<T, HD, C, C, KROW, ROWK, GW>(acc, sBK, LDD, sTm, LDC, wl, lane);
-                store_acc<T, HD, C, GW>(acc, sW, LDD, wl, lane);
+            // ---- V0[c][dv] = V[c][dv] - sum_dk S[dv][dk] K[c][dk] (in place), V~ = beta_c V0 -> sVt ---
+            {
+                f32x4 acc[TMR::TPW];
+                zero_acc<TMR::TPW>(acc);
+                gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc, sS, LDD, sK, LDD, w, lane);  // D[m = dv][n = c]
+#pragma unroll
+                for (int j = 0; j < TMR::TPW; ++j) {
+                    const int d0 = TMR::mt(w, j) * 16 + 4 * lg, r = TMR::nt(w, j) * 16 + li;
+                    const P4 x = *reinterpret_cast<const P4 *>(sV + r * LDD + d0);  // each lane rewrites what it read
+                    const float bb = sBeta[r];
+                    float y[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) y[e] = (float)x[e] - acc[j][e];
+                    const P4 v0 = TT<T>::pack(y[0], y[1], y[2], y[3]);
+                    *reinterpret_cast<P4 *>(sV + r * LDD + d0) = v0;
+                    // V~ from the rounded V0, so that dbeta = rowdot(Z, V0) matches what U' was built from
+                    *reinterpret_cast<P4 *>(sVt + r * LDD + d0) =
+                        TT<T>::pack(bb * (float)v0[0], bb * (float)v0[1], bb * (float)v0[2], bb * (float)v0[3]);
+                }
             }
             sync_lds();
             MRX_PHASE(15);
             if (pre) prefetch_part(1);
-            if (g0) {
-                // ---- U'^T[dv][c] = sum_j beta_j V[j][dv] Tm[c][j] - sum_dk S[dv][dk] W[c][dk] -> sU[c][dv]
-                f32x4 acc[GR::TPW], acc2[GR::TPW];
-                zero_acc<GR::TPW>(acc);
-                zero_acc<GR::TPW>(acc2);
-                gemm<T, HD, C, C, KROW, ROWK, GW>(acc, sBV, LDD, sTm, LDC, wl, lane);
-                gemm<T, HD, C, HD, ROWK, ROWK, GW>(acc2, sS, LDD, sW, LDD, wl, lane);
-#pragma unroll
-                for (int j = 0; j < GR::TPW; ++j) acc[j] -= acc2[j];
-                store_acc<T, HD, C, GW>(acc, sU, LDD, wl, lane);
+            // ---- U'^T[dv][c] = sum_j V~[j][dv] Tm[c][j] -> sU[c][dv] ----------------------------------
+            {
+                f32x4 acc[TMR::TPW];
+                zero_acc<TMR::TPW>(acc);
+                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sVt, LDD, sTm, LDC, w, lane);
+                store_acc<T, HD, C, NW>(acc, sU, LDD, w, lane);
             }
-            if (g1) {
-                // ---- dU'^T[dv][j] = sum_i dO[i][dv] Aqk[i][j] + sum_dk dS[dv][dk] K[j][dk] -> sDU[j][dv]
-                f32x4 acc[GR::TPW];
-                zero_acc<GR::TPW>(acc);
-                gemm<T, HD, C, C, KROW, KROW, GW>(acc, sDO, LDD, sAqk, LDC, wl, lane);
-                gemm<T, HD, C, HD, ROWK, ROWK, GW>(acc, sDS, LDD, sK, LDD, wl, lane);
-                store_acc<T, HD, C, GW>(acc, sDU, LDD, wl, lane);
+            // ---- dU'^T[dv][j] = sum_i dO[i][dv] Aqk[i][j] + sum_dk dS[dv][dk] K[j][dk] -> sDU[j][dv]
+            {
+                f32x4 acc[TMR::TPW];
+                zero_acc<TMR::TPW>(acc);
+                gemm<T, HD, C, C, KROW, KROW, NW>(acc, sDO, LDD, sAqk, LDC, w, lane);
+                gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc, sDS, LDD, sK, LDD, w, lane);
+                store_acc<T, HD, C, NW>(acc, sDU, LDD, w, lane);
             }
             sync_lds();  // sU, sDU visible; sAqk dead
             MRX_PHASE(16);
             if (pre) prefetch_part(2);
-            if (g0) {
-                // ---- dAqk[i][j] = do_i . u'_j, j <= i -> sDAqk (over sAqk) ------------------------
-                f32x4 acc[GA::TPW];
-                zero_acc<GA::TPW>(acc);
-                gemm<T, C, C, HD, ROWK, ROWK, GW>(acc, sU, LDD, sDO, LDD, wl, lane);  // D[m = j][n = i]
-                store_acc_f<T, C, C, GW>(acc, sDAqk, LDC, wl, lane, tril);
-            }
-            if (g1) {
-                // ---- dW^T[dk][c] = -sum_dv S[dv][dk] dU'[c][dv] -> sDW[c][dk] -----------------------
-                f32x4 acc[GR::TPW];
-                zero_acc<GR::TPW>(acc);
-                gemm<T, HD, C, HD, KROW, ROWK, GW>(acc, sS, LDD, sDU, LDD, wl, lane);
-                store_acc_f<T, HD, C, GW>(acc, sDW, LDD, wl, lane, [](int, int, float x) { return -x; });
-            }
-            sync_lds();
-            MRX_PHASE(17);
-            if (pre) prefetch_part(3);
-            auto one = [](int, int) { return f32x4{1.f, 1.f, 1.f, 1.f}; };
-            auto beta_of = [&](int r, int) { const float bb = sBeta[r]; return f32x4{bb, bb, bb, bb}; };
-            float dbp[GR::NBW];  // per-lane partials of dbeta for rows nt * 16 + li of the wave's tile columns
+            float dbp[TMR::NBW];  // per-lane partials of dbeta for rows nt * 16 + li of the wave's tile columns
 #pragma unroll
-            for (int j = 0; j < GR::NBW; ++j) dbp[j] = 0.f;
+            for (int j = 0; j < TMR::NBW; ++j) dbp[j] = 0.f;
             auto rowdot = [&](const f32x4 *acc, const T *X) {
 #pragma unroll
-                for (int j = 0; j < GR::TPW; ++j) {
-                    const int d0 = GR::mt(wl, j) * 16 + 4 * lg, r = GR::nt(wl, j) * 16 + li;
+                for (int j = 0; j < TMR::TPW; ++j) {
+                    const int d0 = TMR::mt(w, j) * 16 + 4 * lg, r = TMR::nt(w, j) * 16 + li;
                     const P4 x = *reinterpret_cast<const P4 *>(X + r * LDD + d0);
-                    dbp[j % GR::NBW] += acc[j][0] * (float)x[0] + acc[j][1] * (float)x[1] + acc[j][2] * (float)x[2] +
-                                        acc[j][3] * (float)x[3];
+                    dbp[j % TMR::NBW] += acc[j][0] * (float)x[0] + acc[j][1] * (float)x[1] + acc[j][2] * (float)x[2] +
+                                         acc[j][3] * (float)x[3];
                 }
             };
-            f32x4 dKacc[GR::TPW];  // dK^T[dk][j] (group 1)
-            zero_acc<GR::TPW>(dKacc);
-            if (g0) {
-                // ---- dQ^T[dk][i] = sum_dv S[dv][dk] dO[i][dv] + sum_j K[j][dk] dAqk[i][j] -> global ----
-                {
-                    f32x4 acc[GR::TPW];
-                    zero_acc<GR::TPW>(acc);
-                    gemm<T, HD, C, HD, KROW, ROWK, GW>(acc, sS, LDD, sDO, LDD, wl, lane);
-                    gemm<T, HD, C, C, KROW, ROWK, GW>(acc, sK, LDD, sDAqk, LDC, wl, lane);
-                    store_rows_at<T, C, GW>(acc, dq + goff, rs, t0, Tlen, wl, lane, one, live);
-                }
-                // ---- dS^T[dk][dv] += sum_c Q[c][dk] dO[c][dv] - sum_c W[c][dk] dU'[c][dv] ---------------
-                {
-                    f32x4 acc[GS::TPW];
-                    zero_acc<GS::TPW>(acc);
-                    gemm<T, HD, HD, C, KROW, KROW, GW>(dSacc, sQ, LDD, sDO, LDD, wl, lane);
-                    gemm<T, HD, HD, C, KROW, KROW, GW>(acc, sW, LDD, sDU, LDD, wl, lane);
-#pragma unroll
-                    for (int j = 0; j < GS::TPW; ++j) dSacc[j] -= acc[j];
-                }
-                // ---- Zu^T[dv][j] = sum_i dU'[i][dv] Tm[i][j] -> dV = beta_j Zu ; dbeta += V_j . Zu_j ------
-                {
-                    f32x4 acc[GR::TPW];
-                    zero_acc<GR::TPW>(acc);
-                    gemm<T, HD, C, C, KROW, KROW, GW>(acc, sDU, LDD, sTm, LDC, wl, lane);
-                    rowdot(acc, sV);
-                    store_rows_at<T, C, GW>(acc, dv + goff, rs, t0, Tlen, wl, lane, beta_of, live);
-                }
+            auto one = [](int, int) { return f32x4{1.f, 1.f, 1.f, 1.f}; };
+            // ---- dAqk[i][j] = do_i . u'_j, j <= i -> sDAqk (over sAqk) ------------------------------
+            {
+                f32x4 acc[TMA::TPW];
+                zero_acc<TMA::TPW>(acc);
+                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sU, LDD, sDO, LDD, w, lane);  // D[m = j][n = i]
+                store_acc_f<T, C, C, NW>(acc, sDAqk, LDC, w, lane, tril);
             }
-            if (g1) {
-                // ---- dK^T[dk][j] = sum_i Q[i][dk] dAqk[i][j] + sum_dv dS[dv][dk] U'[j][dv] (registers) --
-                gemm<T, HD, C, C, KROW, KROW, GW>(dKacc, sQ, LDD, sDAqk, LDC, wl, lane);
-                gemm<T, HD, C, HD, KROW, ROWK, GW>(dKacc, sDS, LDD, sU, LDD, wl, lane);
-                // ---- Zw^T[dk][j] = sum_i dW[i][dk] Tm[i][j] -> dK += beta_j Zw ; dbeta += K_j . Zw_j ------
-                {
-                    f32x4 acc[GR::TPW];
-                    zero_acc<GR::TPW>(acc);
-                    gemm<T, HD, C, C, KROW, KROW, GW>(acc, sDW, LDD, sTm, LDC, wl, lane);
-                    rowdot(acc, sK);
+            // ---- Z^T[dv][j] = sum_i dU'[i][dv] Tm[i][j] : dV = beta_j Z -> global and sZb ; dbeta += Z_j . V0_j
+            {
+                f32x4 acc[TMR::TPW];
+                zero_acc<TMR::TPW>(acc);
+                gemm<T, HD, C, C, KROW, KROW, NW>(acc, sDU, LDD, sTm, LDC, w, lane);
+                rowdot(acc, sV);
 #pragma unroll
-                    for (int j = 0; j < GR::TPW; ++j) dKacc[j] += acc[j] * sBeta[GR::nt(wl, j) * 16 + li];
-                }
-                // ---- dT[a][b] = dw_a . k_b + du'_a . v_b, a >= b : D[m = b][n = a] -> sDT[a][b] ------------
-                {
-                    f32x4 acc[GA::TPW];
-                    zero_acc<GA::TPW>(acc);
-                    gemm<T, C, C, HD, ROWK, ROWK, GW>(acc, sK, LDD, sDW, LDD, wl, lane);
-                    gemm<T, C, C, HD, ROWK, ROWK, GW>(acc, sV, LDD, sDU, LDD, wl, lane);
-                    store_acc_f<T, C, C, GW>(acc, sDT, LDC, wl, lane, tril);
-                }
+                for (int j = 0; j < TMR::TPW; ++j) acc[j] *= sBeta[TMR::nt(w, j) * 16 + li];
+                store_acc<T, HD, C, NW>(acc, sZb, LDD, w, lane);
+                store_rows_at<T, C, NW>(acc, dv + goff, rs, t0, Tlen, w, lane, one, live);
             }
-            sync_lds();  // sDT visible; sQ, sDO, sS, sDS, sDAqk dead
-            MRX_PHASE(20);
-            if (pre) prefetch_part(4);
-            // ---- Y1[j][b] = beta_b sum_a Tm[a][j] dT[a][b] : D[m = b][n = j] -> sY1[j][b] ---------------
+            // ---- dTm[a][b] = du'_a . v~_b, b <= a : D[m = b][n = a] -> sDT[a][b] ---------------------
+            {
+                f32x4 acc[TMA::TPW];
+                zero_acc<TMA::TPW>(acc);
+                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sVt, LDD, sDU, LDD, w, lane);
+                store_acc_f<T, C, C, NW>(acc, sDT, LDC, w, lane, tril);
+            }
+            sync_lds();  // sDAqk, sZb, sDT visible; sVt dead
+            MRX_PHASE(17);
+            if (pre) prefetch_part(3);
+            // ---- dQ^T[dk][i] = sum_dv S[dv][dk] dO[i][dv] + sum_j K[j][dk] dAqk[i][j] -> global ----
+            {
+                f32x4 acc[TMR::TPW];
+                zero_acc<TMR::TPW>(acc);
+                gemm<T, HD, C, HD, KROW, ROWK, NW>(acc, sS, LDD, sDO, LDD, w, lane);
+                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sK, LDD, sDAqk, LDC, w, lane);
+                store_rows_at<T, C, NW>(acc, dq + goff, rs, t0, Tlen, w, lane, one, live);
+            }
+            // ---- dK^T[dk][j] = sum_i Q[i][dk] dAqk[i][j] + sum_dv dS[dv][dk] U'[j][dv]
+            //                    - sum_dv S[dv][dk] (beta Z)[j][dv]   (kept in registers) ---------------
+            f32x4 dKacc[TMR::TPW];
+            {
+                f32x4 acc[TMR::TPW];
+                zero_acc<TMR::TPW>(acc);
+                zero_acc<TMR::TPW>(dKacc);
+                gemm<T, HD, C, HD, KROW, ROWK, NW>(acc, sS, LDD, sZb, LDD, w, lane);
+                gemm<T, HD, C, C, KROW, KROW, NW>(dKacc, sQ, LDD, sDAqk, LDC, w, lane);
+                gemm<T, HD, C, HD, KROW, ROWK, NW>(dKacc, sDS, LDD, sU, LDD, w, lane);
+#pragma unroll
+                for (int j = 0; j < TMR::TPW; ++j) dKacc[j] -= acc[j];
+            }
+            // ---- dS^T[dk][dv] += sum_c Q[c][dk] dO[c][dv] - sum_c K[c][dk] (beta Z)[c][dv] -----------
+            {
+                f32x4 acc[TMS::TPW];
+                zero_acc<TMS::TPW>(acc);
+                gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, sQ, LDD, sDO, LDD, w, lane);
+                gemm<T, HD, HD, C, KROW, KROW, NW>(acc, sK, LDD, sZb, LDD, w, lane);
+#pragma unroll
+                for (int j = 0; j < TMS::TPW; ++j) dSacc[j] -= acc[j];
+            }
+            // ---- Y1[j][b] = sum_a Tm[a][j] dTm[a][b] : D[m = b][n = j] -> sY1[j][b] (over sVt) ----------
             {
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
                 gemm<T, C, C, C, KROW, KROW, NW>(acc, sDT, LDC, sTm, LDC, w, lane);
-                store_acc_f<T, C, C, NW>(acc, sY1, LDC, w, lane, [&](int m, int, float x) { return x * sBeta[m]; });
+                store_acc<T, C, C, NW>(acc, sY1, LDC, w, lane);
             }
-            sync_lds();
-            MRX_PHASE(21);
-            if (pre) prefetch_part(5);
-            // ---- dA[i][j] = -sum_b Y1[i][b] Tm[j][b], j < i : D[m = j][n = i] -> sDA[i][j] --------------
+            sync_lds();  // sY1 visible; sQ, sDO, sS, sDS, sDAqk, sZb dead
+            MRX_PHASE(20);
+            if (pre) prefetch_part(4);
+            // ---- dA[i][j] = -sum_b Y1[i][b] Tm[j][b], j < i : D[m = j][n = i] -> sDA[i][j] (over sS) ----
             {
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
@@ -711,57 +690,43 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();
             MRX_PHASE(22);
-            if (g0) {
-                // ---- R^T[dk][i] = sum_j K[j][dk] dA[i][j] ; dbeta += K_i . R_i ; beta_i R -> sR[i][dk] (fp32)
-                f32x4 acc[GR::TPW];
-                zero_acc<GR::TPW>(acc);
-                gemm<T, HD, C, C, KROW, ROWK, GW>(acc, sK, LDD, sDA, LDC, wl, lane);
+            if (pre) prefetch_part(5);
+            // ---- R^T[dk][i] = sum_j K[j][dk] dA[i][j] : dbeta += K_i . R_i ; dK += beta_i R ;
+            //      dK^T[dk][j] += sum_i beta_i K[i][dk] dA[i][j] -> global -------------------------------
+            {
+                f32x4 acc[TMR::TPW];
+                zero_acc<TMR::TPW>(acc);
+                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sK, LDD, sDA, LDC, w, lane);
                 rowdot(acc, sK);
 #pragma unroll
-                for (int j = 0; j < GR::TPW; ++j) {
-                    const int d0 = GR::mt(wl, j) * 16 + 4 * lg, r = GR::nt(wl, j) * 16 + li;
-                    if (SPLIT) *reinterpret_cast<f32x4 *>(sR + r * LDR + d0) = acc[j] * sBeta[r];
-                    else dKacc[j] += acc[j] * sBeta[r];  // one group: the wave holds the matching dK tiles itself
-                }
-            }
-            if (g1) {
-                // ---- dK^T[dk][j] += sum_i beta_i K[i][dk] dA[i][j] ---------------------------------------
-                gemm<T, HD, C, C, KROW, KROW, GW>(dKacc, sBK, LDD, sDA, LDC, wl, lane);
-                if (!SPLIT) store_rows_at<T, C, GW>(dKacc, dk + goff, rs, t0, Tlen, wl, lane, one, live);
+                for (int j = 0; j < TMR::TPW; ++j) dKacc[j] += acc[j] * sBeta[TMR::nt(w, j) * 16 + li];
+                gemm<T, HD, C, C, KROW, KROW, NW>(dKacc, sBK, LDD, sDA, LDC, w, lane);
+                store_rows_at<T, C, NW>(dKacc, dk + goff, rs, t0, Tlen, w, lane, one, live);
             }
             // ---- dbeta: reduce the partials over lane groups, then over waves through LDS -----------
 #pragma unroll
-            for (int j = 0; j < GR::NBW; ++j) {
+            for (int j = 0; j < TMR::NBW; ++j) {
                 float x = dbp[j];
                 x += __shfl_xor(x, 16);
                 x += __shfl_xor(x, 32);
-                if (lg == 0) sDb[((SPLIT ? grp * GR::WM : 0) + wl % GR::WM) * C + GR::nt(wl, j) * 16 + li] = x;
+                if (lg == 0) sDb[(w % TMR::WM) * C + TMR::nt(w, j) * 16 + li] = x;
             }
             sync_lds();
             MRX_PHASE(23);
-            if (SPLIT && g1) {
-                // ---- dK += beta_i R -> global ---------------------------------------------------------
-#pragma unroll
-                for (int j = 0; j < GR::TPW; ++j) {
-                    const int d0 = GR::mt(wl, j) * 16 + 4 * lg, r = GR::nt(wl, j) * 16 + li;
-                    dKacc[j] += *reinterpret_cast<const f32x4 *>(sR + r * LDR + d0);
-                }
-                store_rows_at<T, C, GW>(dKacc, dk + goff, rs, t0, Tlen, wl, lane, one, live);
-            }
             if (tid < C && t0 + tid < Tlen && live(tid)) {
                 float x = 0.f;
 #pragma unroll
                 for (int sl = 0; sl < NSLOT; ++sl) x += sDb[sl * C + tid];
                 dbeta[dboff] = (T)x;
             }
-            MRX_PHASE(24);  // no barrier: what this phase reads (sR, sDb) is not written by the next staging step
+            MRX_PHASE(24);  // no barrier: sDb is not written again before the next pass's last phase
         }
     }
     MRX_PHASE_FLUSH();
-    if (dS0 && g0) {
+    if (dS0) {
 #pragma unroll
-        for (int j = 0; j < GS::TPW; ++j) {
-            const int dk0 = GS::mt(wl, j) * 16 + 4 * lg, dvv = GS::nt(wl, j) * 16 + li;
+        for (int j = 0; j < TMS::TPW; ++j) {
+            const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
             *reinterpret_cast<f32x4 *>(dS0 + ((int64_t)bh * HD + dvv) * HD + dk0) = dSacc[j];
         }
     }
@@ -854,13 +819,10 @@ extern "C" int mrx_delta_rule_bwd(void *stream, const void *q, const void *k, co
     if (rc != MRX_OK) return rc;
     if (!beta || !dbeta || !Tm_chk || !aligned(Tm_chk, 16)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
+    constexpr int NW = 4;
     if (dtype == MRX_BF16) {
-        // 64-step chunks: 8 waves in two groups, one workgroup per CU; 32-step chunks: 4 waves, one
-        // group (measured 2 % faster than two groups of 2), two workgroups per CU
-        constexpr int NW = DELTA_BF16_CHUNK == 64 ? MRX_DELTA_BWD_WAVES : 4;
-        constexpr bool SPLIT = DELTA_BF16_CHUNK == 64;
-        auto kern = delta_bwd_kernel<__bf16, DELTA_BF16_CHUNK, NW, SPLIT>;
-        constexpr int smem = DeltaBwdSmem<__bf16, DELTA_BF16_CHUNK, NW, SPLIT>::total;
+        auto kern = delta_bwd_kernel<__bf16, DELTA_BF16_CHUNK, NW>;
+        constexpr int smem = DeltaBwdSmem<__bf16, DELTA_BF16_CHUNK, NW>::total;
         static unsigned long long lds_set = 0ull;
         if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
         hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(64 * NW), smem, st, (const __bf16 *)q,
@@ -869,9 +831,8 @@ extern "C" int mrx_delta_rule_bwd(void *stream, const void *q, const void *k, co
                            (const float *)dS_last, (__bf16 *)dq, (__bf16 *)dk_out, (__bf16 *)dv_out,
                            (__bf16 *)dbeta, (float *)dS0, (int)T, (int)H);
     } else {
-        constexpr int NW = 4;
-        auto kern = delta_bwd_kernel<float, 32, NW, false>;
-        constexpr int smem = DeltaBwdSmem<float, 32, NW, false>::total;
+        auto kern = delta_bwd_kernel<float, 32, NW>;
+        constexpr int smem = DeltaBwdSmem<float, 32, NW>::total;
         static unsigned long long lds_set = 0ull;
         if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
         hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(64 * NW), smem, st, (const float *)q,
