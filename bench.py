@@ -214,6 +214,14 @@ def bench_linear_attention(torch, K, M, dev):
     ms = _time_ms(torch, f3g, iters=5)
     res["gated_bf16_256x4096x8x64"] = {"ms": ms, "tokens/s": Bn * Tn / ms * 1e3,
                                        "GB/s": (1408 + 12) * Bn * Tn * Hn / ms / 1e6}
+    # the same shape with the normalised read-out of LinearAttentionCell.read fused (elu+1 feature map);
+    # + o read back in the backward call, den written and read: 136 B more per token-head
+    def f3n():
+        o, den, Sl, zl, chk = K.linear_attn_norm_fwd(q, k, v, dn, None, None, 1, 1e-6)
+        K.linear_attn_norm_bwd(q, k, v, dn, chk, o, den, do, None, None, 1, 1e-6, want_d0=False)
+    ms = _time_ms(torch, f3n, iters=5)
+    res["normalised_bf16_256x4096x8x64"] = {"ms": ms, "tokens/s": Bn * Tn / ms * 1e3,
+                                            "GB/s": (1408 + 136) * Bn * Tn * Hn / ms / 1e6}
     return res
 
 

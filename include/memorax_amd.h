@@ -114,6 +114,34 @@ int mrx_linear_attn_bwd(void *stream, const void *q, const void *k,
                         int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                         int done_dtype, int feature_map);
 
+/* ---- linear attention with the normalised read-out fused ----------------------
+ * Replaces, in addition to the above, LinearAttentionCell.read's denominator and
+ * divide (linear_attention.py:107-110) and the z leaf of the carry
+ * (linear_attention.py:62-86):
+ *     z_t = (done_t ? 0 : z_{t-1}) + phi(k_t) ;  den_t = max(phi(q_t) . z_t, eps)
+ *     o_t = S_t phi(q_t) / den_t
+ * z0 (nullable = 0), z_last (nullable): (B,H,dk) fp32.  den: (B,T,H) fp32, the clamped
+ * denominators, and z_chk (nullable): (B,H,ceil(T/chunk),dk) fp32, z entering each
+ * chunk, are residuals of the backward call together with o and S_chk. */
+int mrx_linear_attn_norm_fwd(void *stream, const void *q, const void *k,
+                             const void *v, const void *done, const void *S0,
+                             const float *z0, void *o, float *den, void *S_last,
+                             float *z_last, void *S_chk, float *z_chk, int64_t B,
+                             int64_t T, int64_t H, int64_t dk, int64_t dv,
+                             int dtype, int done_dtype, int feature_map, float eps);
+
+/* Gradients of the above w.r.t. q,k,v (pre-feature-map), S0 and z0, given
+ * dout = dL/do (gradient of the normalised output), dS_last and dz_last (nullable).
+ * Where the clamp is active (den == eps) the denominator passes no gradient. */
+int mrx_linear_attn_norm_bwd(void *stream, const void *q, const void *k,
+                             const void *v, const void *done, const void *S_chk,
+                             const float *z_chk, const void *o, const float *den,
+                             const void *dout, const void *dS_last,
+                             const float *dz_last, void *dq, void *dk_out,
+                             void *dv_out, void *dS0, float *dz0, int64_t B,
+                             int64_t T, int64_t H, int64_t dk, int64_t dv,
+                             int dtype, int done_dtype, int feature_map, float eps);
+
 /* ---- DeltaNet delta rule, chunked WY/UT form --------------------------------
  * No counterpart in the reference; written in its cell idiom it would be a
  * MemoroidCellBase scanned by memoroid.py:60-91 with elements

@@ -78,32 +78,64 @@ __device__ __forceinline__ void store_rows_at(const f32x4 *acc, T *row, int64_t 
 // =====================================================================================
 // linear attention: 8 tiles, two workgroups per CU; with a per-step decay (GATED) one tile more
 // =====================================================================================
-template <typename T, int C, bool GATED = false> struct LaBwdSmem : BwdDims<T, C> {
+template <typename T, int C, bool GATED = false, bool NORM = false> struct LaBwdSmem : BwdDims<T, C> {
     using D = BwdDims<T, C>;
     static constexpr int oQ = 0, oK = oQ + D::szRD, oV = oK + D::szRD, oDO = oV + D::szRD,
                          oS = oDO + D::szRD, oDS = oS + D::szDD, oAqk = oDS + D::szDD,
                          oDAqk = oAqk + D::szCC, oQa = oDAqk + D::szCC,    // gated: exp(G_i) Q_i
                          oG = oQa + (GATED ? D::szRD : 0),                 // gated: G[C], then [WM][C] row-dot partials
-                         total = oG + (GATED ? (1 + TileMap<HD, C, 4>::WM) * C * 4 : 0);
+                         oN = oG + (GATED ? (1 + TileMap<HD, C, 4>::WM) * C * 4 : 0),
+                         // normalised read-out: dden fp32 [C], dden T-typed [C] (C * 4 bytes kept), z fp32 [64], dz fp32 [64]
+                         total = oN + (NORM ? 2 * C * 4 + 2 * HD * 4 : 0);
 };
+
+// What the normalised read-out adds to the backward argument list.
+struct NormBwdArgs {
+    const void *o;        // (B,T,H,64) T-typed: the normalised outputs of the forward call
+    const float *den;     // (B,T,H): the clamped denominators
+    const float *z_chk;   // (B,H,NC,64): z entering each chunk
+    const float *dz_last; // (B,H,64) or null
+    float *dz0;           // (B,H,64) or null
+    float eps;
+};
+
+// Sum over the SEGS consecutive lanes that share a tile row (8 or 16), by data-parallel
+// primitives; every lane of the group ends with the total.
+template <int SEGS> __device__ __forceinline__ float seg_sum(float x)
+{
+    static_assert(SEGS == 8 || SEGS == 16, "a row is 8 or 16 segments");
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xF, 0xF, true));  // row_half_mirror
+    if (SEGS == 16)
+        x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x140, 0xF, 0xF, true));  // row_mirror
+    return x;
+}
 
 // GATED: S_t = r_t exp(g_t) S_{t-1} + v_t k_t^T.  With G the cumulative log-decay inside the chunk
 // (per episode), a_i = exp(G_i), b_j = exp(G_last - G_j), c = exp(G_last), D_ij = exp(G_i - G_j):
 //   Aqk, dAqk carry the factor D;  dV = Aqk^T dO + diag(b) K dS^T;  dQ = diag(a) dO S + dAqk K;
 //   dK = dAqk^T Q + diag(b) V dS;  dS <- c dS + (diag(a) Q)^T dO.
+// NORM (normalised read-out o_i = num_i / den_i, den_i = max(q_i . z_i, eps), z the running sum of
+// the keys of the episode): with dnum_i = dout_i / den_i taking the place of dO and
+// dden_i = -(dout_i . o_i) / den_i (0 where the clamp is active),
+//   dAqk_ij += dden_i (j <= i);  dQ_i += dden_i z_in;  dK_j += dz;  dz <- dz + sum_i dden_i Q_i,
+// z_in the sum entering the chunk (first episode only), dz the gradient of the sum leaving it.
 // The gradient of the log-decays follows from edot_i = q_i . dq_i - k_i . dk_i (taken on the
 // feature-mapped q, k and their gradients): dg_t is the sum of edot over the rows i >= t of t's
 // episode (plus <S_last, dS_last> at the end); the kernel writes edot, the caller sums.
-template <typename T, int C, bool FMAP, bool GATED>
+template <typename T, int C, bool FMAP, bool GATED, bool NORM>
 __global__ void __launch_bounds__(256, 2)
 la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
               const float *__restrict__ glog, const void *__restrict__ done, int done_f32,
               const T *__restrict__ S_chk, const T *__restrict__ dout, const float *__restrict__ dS_last,
               T *__restrict__ dq, T *__restrict__ dk, T *__restrict__ dv, float *__restrict__ edot,
-              float *__restrict__ dS0, int Tlen, int H)
+              float *__restrict__ dS0, int Tlen, int H, NormBwdArgs na)
 {
+    static_assert(!(GATED && NORM), "the normalised read-out belongs to plain linear attention");
     constexpr int NW = 4, NTHR = 64 * NW;
-    using L = LaBwdSmem<T, C, GATED>;
+    using L = LaBwdSmem<T, C, GATED, NORM>;
+    using Frag = typename TT<T>::frag;
     using IO = TileIO<T, C, NTHR>;
     using IOS = TileIO<T, HD, NTHR>;
     using P4 = typename TT<T>::pack4;
@@ -120,6 +152,10 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     T *sQa = reinterpret_cast<T *>(smem + L::oQa);
     float *sG = reinterpret_cast<float *>(smem + L::oG);
     float *sE = sG + C;  // [WM][C] partial row dots
+    float *sDd = reinterpret_cast<float *>(smem + L::oN);       // dden[C]
+    T *sDdT = reinterpret_cast<T *>(smem + L::oN + C * 4);      // dden[C], T-typed (MFMA operand)
+    float *sZf = reinterpret_cast<float *>(smem + L::oN + 2 * C * 4);  // z entering the chunk
+    float *sDZ = sZf + HD;                                      // dz leaving the pass
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -140,7 +176,18 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                            : f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    typename IO::Regs rq, rk, rv, rdo;
+    // normalised read-out: dz[dk], held like a column of dS^T (see the forward kernel's z)
+    f32x4 dzacc[TMS::MBW];
+#pragma unroll
+    for (int mi = 0; mi < TMS::MBW; ++mi) {
+        const int dk0 = TMS::mt(w, mi * TMS::NBW) * 16 + 4 * lg;
+        dzacc[mi] = (NORM && na.dz_last) ? *reinterpret_cast<const f32x4 *>(na.dz_last + (int64_t)bh * HD + dk0)
+                                         : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    typename IO::Regs rq, rk, rv, rdo, ro;
+    float rden[IO::PASSES];
+    f32x4 rz = {0.f, 0.f, 0.f, 0.f};
     typename IOS::Regs rS;
     uint32_t rdone = 0u;  // raw bits, tested when the chunk is staged
     float rg = 0.f;       // log-decay of chunk row `lane` (gated)
@@ -155,6 +202,10 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
         roff[p] = base + (int64_t)(tlast + IO::row_of(tid, p)) * rs + (tid % IO::SEGS) * IO::KP;
     int64_t soff = ((int64_t)bh * NC + NC - 1) * HD * HD + (tid / IOS::SEGS) * HD + (tid % IOS::SEGS) * IOS::KP;
     int64_t doff = (int64_t)b * Tlen + tlast + lane;
+    int64_t noff[IO::PASSES];  // den of the rows this thread stages
+#pragma unroll
+    for (int p = 0; p < IO::PASSES; ++p) noff[p] = ((int64_t)b * Tlen + tlast + IO::row_of(tid, p)) * H + h;
+    int64_t zoff = ((int64_t)bh * NC + NC - 1) * HD + 4 * (tid & 15);
     int tpre = tlast;
     auto prefetch_part = [&](int part) {
         typename IO::F z;
@@ -170,6 +221,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 } else {
                     rv.v[p] = in ? *reinterpret_cast<const typename IO::F *>(v + roff[p]) : z;
                     rdo.v[p] = in ? *reinterpret_cast<const typename IO::F *>(dout + roff[p]) : z;
+                    if (NORM) ro.v[p] = in ? *reinterpret_cast<const typename IO::F *>((const T *)na.o + roff[p]) : z;
                 }
             }
         } else {
@@ -181,6 +233,15 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             if (lane < C && tpre + lane < Tlen) {
                 rdone = done_raw(done, done_f32, doff);
                 if (GATED) rg = glog[doff * H + h];
+            }
+            if (NORM) {
+#pragma unroll
+                for (int p = 0; p < IO::PASSES; ++p) {
+                    rden[p] = tpre + IO::row_of(tid, p) < Tlen ? na.den[noff[p]] : 1.f;
+                    noff[p] -= (int64_t)C * H;
+                }
+                rz = *reinterpret_cast<const f32x4 *>(na.z_chk + zoff);
+                zoff -= HD;
             }
 #pragma unroll
             for (int p = 0; p < IO::PASSES; ++p) roff[p] -= (int64_t)C * rs;
@@ -221,6 +282,27 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     IO::mask_rows(fv, tid, live);
                     IO::mask_rows(fdo, tid, live);
                 }
+                if (NORM) {
+                    // dden_i = -(dout_i . o_i) / den_i where the clamp is inactive; dO <- dout / den
+                    float inv[IO::PASSES];
+#pragma unroll
+                    for (int p = 0; p < IO::PASSES; ++p) {
+                        float dot = 0.f;
+#pragma unroll
+                        for (int e = 0; e < IO::KP; ++e) dot += (float)rdo.v[p][e] * (float)ro.v[p][e];
+                        dot = seg_sum<IO::SEGS>(dot);
+                        const int r = IO::row_of(tid, p);
+                        const bool on = (IO::FULL || r < C) && live(r);
+                        inv[p] = on ? 1.f / rden[p] : 1.f;
+                        const float dd = (on && rden[p] > na.eps) ? -dot * inv[p] : 0.f;
+                        if (tid % IO::SEGS == 0 && (IO::FULL || r < C)) {
+                            sDd[r] = dd;
+                            sDdT[r] = (T)dd;
+                        }
+                    }
+                    IO::scale_rows(fdo, inv);
+                    if (tid < 16) *reinterpret_cast<f32x4 *>(sZf + 4 * tid) = rz;
+                }
                 IO::to_lds(fq, sQ, LDD, tid);
                 if (GATED) {
                     float af[IO::PASSES];
@@ -238,6 +320,14 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             }
             if (pass != nres) zero_acc<TMS::TPW>(dSacc);  // an episode that ends inside the chunk
             store_acc<T, HD, HD, NW>(dSacc, sDS, LDD, w, lane);  // dS[dv][dk]
+            if (NORM) {
+                if (pass != nres) zero_acc<TMS::MBW>(dzacc);
+                if (w < TMS::WM && li == 0) {
+#pragma unroll
+                    for (int mi = 0; mi < TMS::MBW; ++mi)
+                        *reinterpret_cast<f32x4 *>(sDZ + TMS::mt(w, mi * TMS::NBW) * 16 + 4 * lg) = dzacc[mi];
+                }
+            }
             sync_lds();
             const bool pre = pass == 0 && c > 0;
             if (pre) prefetch_part(0);
@@ -247,11 +337,12 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
                 // masked store; gated: times exp(G_i - G_j) (exponent <= 0 where kept)
-                auto store_tril = [&](const f32x4 *a, T *dst) {
+                auto store_tril = [&](const f32x4 *a, T *dst, bool add_dden) {
 #pragma unroll
                     for (int j = 0; j < TMA::TPW; ++j) {
                         const int m = TMA::mt(w, j) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
                         float x[4];
+                        const float dd = (NORM && add_dden) ? sDd[n] : 0.f;
                         if (GATED) {
                             const float gn = sG[n];
                             const f32x4 gm = *reinterpret_cast<const f32x4 *>(sG + m);
@@ -259,16 +350,16 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                             for (int e = 0; e < 4; ++e) x[e] = (m + e <= n) ? a[j][e] * __expf(gn - gm[e]) : 0.f;
                         } else {
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) x[e] = (m + e <= n) ? a[j][e] : 0.f;
+                            for (int e = 0; e < 4; ++e) x[e] = (m + e <= n) ? a[j][e] + dd : 0.f;
                         }
                         *reinterpret_cast<P4 *>(dst + n * LDC + m) = TT<T>::pack(x[0], x[1], x[2], x[3]);
                     }
                 };
                 gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sK, LDD, sQ, LDD, w, lane);  // D[m = j][n = i]
-                store_tril(acc, sAqk);
+                store_tril(acc, sAqk, false);
                 zero_acc<TMA::TPW>(acc);
                 gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sV, LDD, sDO, LDD, w, lane);  // D[m = j][n = i]
-                store_tril(acc, sDAqk);
+                store_tril(acc, sDAqk, true);
             }
             sync_lds();
             if (pre) prefetch_part(1);
@@ -312,6 +403,13 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 }
                 gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sK, LDD, sDAqk, LDC, w, lane);
                 if (GATED) rowdot(acc, sQ, 1.f);
+                if (NORM && pass == 0) {  // den_i = q_i . (z_in + ...): dQ_i += dden_i z_in
+#pragma unroll
+                    for (int j = 0; j < TMR::TPW; ++j) {
+                        const f32x4 zz = *reinterpret_cast<const f32x4 *>(sZf + TMR::mt(w, j) * 16 + 4 * lg);
+                        acc[j] += zz * sDd[TMR::nt(w, j) * 16 + li];
+                    }
+                }
                 auto sc = [&](int r, int d0) {
                     const P4 x = *reinterpret_cast<const P4 *>(sQ + r * LDD + d0);
                     return f32x4{fmap_grad<FMAP>((float)x[0]), fmap_grad<FMAP>((float)x[1]),
@@ -333,6 +431,11 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     gemm<T, HD, C, C, KROW, KROW, NW>(acc, sQ, LDD, sDAqk, LDC, w, lane);
                     gemm<T, HD, C, HD, KROW, ROWK, NW>(acc, sDS, LDD, sV, LDD, w, lane);
                 }
+                if (NORM && pass == nres) {  // every key of the leaving episode is part of the z that leaves
+#pragma unroll
+                    for (int j = 0; j < TMR::TPW; ++j)
+                        acc[j] += *reinterpret_cast<const f32x4 *>(sDZ + TMR::mt(w, j) * 16 + 4 * lg);
+                }
                 auto sc = [&](int r, int d0) {
                     const P4 x = *reinterpret_cast<const P4 *>(sK + r * LDD + d0);
                     return f32x4{fmap_grad<FMAP>((float)x[0]), fmap_grad<FMAP>((float)x[1]),
@@ -353,7 +456,10 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     if (lg == 0) sE[(w % TMR::WM) * C + TMR::nt(w, j) * 16 + li] = x;
                 }
             }
-            gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, GATED ? sQa : sQ, LDD, sDO, LDD, w, lane);
+            auto dz_q = [&](int mi, int kb, const Frag &xq) {  // dz[dk] += sum_i Q[i][dk] dden_i
+                if (NORM) dzacc[mi] = TT<T>::mma(xq, TT<T>::template load<ROWK>(sDdT, 0, 0, kb * TT<T>::KB, lane), dzacc[mi]);
+            };
+            gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, GATED ? sQa : sQ, LDD, sDO, LDD, w, lane, dz_q);
             sync_lds();
             if (GATED && tid < C && t0 + tid < Tlen && live(tid)) {
                 float x = 0.f;
@@ -369,6 +475,11 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
             *reinterpret_cast<f32x4 *>(dS0 + ((int64_t)bh * HD + dvv) * HD + dk0) = dSacc[j];
         }
+    }
+    if (NORM && na.dz0 && w < TMS::WM && li == 0) {
+#pragma unroll
+        for (int mi = 0; mi < TMS::MBW; ++mi)
+            *reinterpret_cast<f32x4 *>(na.dz0 + (int64_t)bh * HD + TMS::mt(w, mi * TMS::NBW) * 16 + 4 * lg) = dzacc[mi];
     }
 }
 
@@ -732,20 +843,20 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     }
 }
 
-template <typename T, int C, bool FMAP, bool GATED = false>
+template <typename T, int C, bool FMAP, bool GATED = false, bool NORM = false>
 int launch_la(hipStream_t st, const void *q, const void *k, const void *v, const void *done,
               int done_f32, const void *S_chk, const void *dout, const void *dS_last, void *dq,
               void *dk, void *dv, void *dS0, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr,
-              void *edot = nullptr)
+              void *edot = nullptr, NormBwdArgs na = NormBwdArgs{})
 {
-    auto kern = la_bwd_kernel<T, C, FMAP, GATED>;
-    constexpr int smem = LaBwdSmem<T, C, GATED>::total;
+    auto kern = la_bwd_kernel<T, C, FMAP, GATED, NORM>;
+    constexpr int smem = LaBwdSmem<T, C, GATED, NORM>::total;
     static unsigned long long lds_set = 0ull;
     if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(256), smem, st, (const T *)q,
                        (const T *)k, (const T *)v, (const float *)glog, done, done_f32, (const T *)S_chk,
                        (const T *)dout, (const float *)dS_last, (T *)dq, (T *)dk, (T *)dv, (float *)edot,
-                       (float *)dS0, (int)Tlen, (int)H);
+                       (float *)dS0, (int)Tlen, (int)H, na);
     return launch_status();
 }
 
@@ -784,6 +895,32 @@ extern "C" int mrx_linear_attn_bwd(void *stream, const void *q, const void *k, c
 #define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H
     if (dtype == MRX_BF16) return fm ? launch_la<__bf16, LA_BF16_CHUNK, true>(MRX_ARGS) : launch_la<__bf16, LA_BF16_CHUNK, false>(MRX_ARGS);
     return fm ? launch_la<float, 32, true>(MRX_ARGS) : launch_la<float, 32, false>(MRX_ARGS);
+#undef MRX_ARGS
+}
+
+extern "C" int mrx_linear_attn_norm_bwd(void *stream, const void *q, const void *k, const void *v,
+                                        const void *done, const void *S_chk, const float *z_chk,
+                                        const void *o, const float *den, const void *dout,
+                                        const void *dS_last, const float *dz_last, void *dq, void *dk_out,
+                                        void *dv_out, void *dS0, float *dz0, int64_t B, int64_t T, int64_t H,
+                                        int64_t dk, int64_t dv, int dtype, int done_dtype, int feature_map,
+                                        float eps)
+{
+    const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
+                             dv, dtype, done_dtype);
+    if (rc != MRX_OK) return rc;
+    if (!z_chk || !o || !den) return MRX_ERR_INVALID_ARG;
+    if (!aligned(z_chk, 16) || !aligned(o, 16) || !aligned(den, 4) || !aligned(dz_last, 16) || !aligned(dz0, 16))
+        return MRX_ERR_INVALID_ARG;
+    if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const bool fm = feature_map == MRX_FMAP_ELU1;
+    const NormBwdArgs na{o, den, z_chk, dz_last, dz0, eps};
+#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, nullptr, nullptr, na
+    if (dtype == MRX_BF16)
+        return fm ? launch_la<__bf16, LA_BF16_CHUNK, true, false, true>(MRX_ARGS)
+                  : launch_la<__bf16, LA_BF16_CHUNK, false, false, true>(MRX_ARGS);
+    return fm ? launch_la<float, 32, true, false, true>(MRX_ARGS) : launch_la<float, 32, false, false, true>(MRX_ARGS);
 #undef MRX_ARGS
 }
 

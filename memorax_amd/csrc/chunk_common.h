@@ -65,6 +65,13 @@ template <> struct TT<__bf16> {
         r[0] = (__bf16)a; r[1] = (__bf16)b; r[2] = (__bf16)c; r[3] = (__bf16)d;
         return r;
     }
+    static __device__ __forceinline__ frag ones()
+    {
+        frag r;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) r[e] = (__bf16)1.f;
+        return r;
+    }
     // 16 rows r0.., k block k0..k0+31; lane (i, g) gets k = k0 + 8g + 0..7 of row r0 + i
     template <int MODE>
     static __device__ __forceinline__ frag load(const __bf16 *tile, int ld, int r0, int k0, int lane)
@@ -104,6 +111,7 @@ template <> struct TT<float> {
         pack4 r = {a, b, c, d};
         return r;
     }
+    static __device__ __forceinline__ frag ones() { return frag{1.f, 1.f, 1.f, 1.f}; }
     template <int MODE>
     static __device__ __forceinline__ frag load(const float *tile, int ld, int r0, int k0, int lane)
     {
@@ -140,9 +148,16 @@ template <int M, int N, int NW, int MBW_ = 0> struct TileMap {
     static __device__ __forceinline__ int nt(int w, int j) { return (w / WM) * NBW + j % NBW; }
 };
 
+struct NoHook {
+    template <typename F> __device__ __forceinline__ void operator()(int, int, const F &) const {}
+};
+
 // acc[j] += sum_k X(mt_j rows, k) * Y(nt_j rows, k), k = 0..K-1.
-template <typename T, int M, int N, int K, int XM, int YM, int NW, int MBW_ = 0>
-__device__ __forceinline__ void gemm(f32x4 *acc, const T *X, int ldx, const T *Y, int ldy, int w, int lane)
+// hx(mi, kb, fragment) / hy(ni, kb, fragment) see every operand fragment as it is loaded, so that
+// a rank-one by-product (a row or column sum, a product with one more vector) costs MFMAs only.
+template <typename T, int M, int N, int K, int XM, int YM, int NW, int MBW_ = 0, typename HX = NoHook, typename HY = NoHook>
+__device__ __forceinline__ void gemm(f32x4 *acc, const T *X, int ldx, const T *Y, int ldy, int w, int lane,
+                                     HX hx = HX(), HY hy = HY())
 {
     using TM = TileMap<M, N, NW, MBW_>;
     using F = typename TT<T>::frag;
@@ -153,10 +168,14 @@ __device__ __forceinline__ void gemm(f32x4 *acc, const T *X, int ldx, const T *Y
         F a[TM::MBW];
 #pragma unroll
         for (int mi = 0; mi < TM::MBW; ++mi)
+        {
             a[mi] = TT<T>::template load<XM>(X, ldx, TM::mt(w, mi * TM::NBW) * 16, kb * KB, lane);
+            hx(mi, kb, a[mi]);
+        }
 #pragma unroll
         for (int ni = 0; ni < TM::NBW; ++ni) {
             const F b = TT<T>::template load<YM>(Y, ldy, TM::nt(w, ni) * 16, kb * KB, lane);
+            hy(ni, kb, b);
 #pragma unroll
             for (int mi = 0; mi < TM::MBW; ++mi)
                 acc[mi * TM::NBW + ni] = TT<T>::mma(a[mi], b, acc[mi * TM::NBW + ni]);

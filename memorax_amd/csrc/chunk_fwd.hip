@@ -5,6 +5,8 @@
 //   delta rule:        A  = tril(diag(beta) K K^T, -1),  Tm = (I + A)^-1,  T = Tm diag(beta)
 //                      W  = T K,  U' = T V - W S^T
 //   both:              O  = Q S^T + tril(Q K^T) U' ,   S <- S + U'^T K
+//   normalised read-out (linear attention only): z <- z + sum_j K_j,
+//                      den_i = max(Q_i . z + sum_{j<=i} (Q K^T)_ij, eps),  O_i <- O_i / den_i
 // Episode resets: a chunk that contains resets is processed once per episode ("pass")
 // with the rows of all other episodes replaced by zeros *by select*; the episode that
 // enters the chunk sees S, later episodes start from 0, and only the episode that
@@ -21,7 +23,7 @@ using namespace mrx;
 constexpr int NW = 4;             // waves per workgroup
 constexpr int NTHR = 64 * NW;
 
-template <typename T, int C, bool DELTA, bool GATED = false> struct FwdSmem {
+template <typename T, int C, bool DELTA, bool GATED = false, bool NORM = false> struct FwdSmem {
     static constexpr int PAD = pad_of<T>();
     static constexpr int LDD = HD + PAD;  // tiles with 64 columns
     static constexpr int LDC = C + PAD;   // tiles with C columns
@@ -42,19 +44,31 @@ template <typename T, int C, bool DELTA, bool GATED = false> struct FwdSmem {
     static constexpr int oA = oTm + (DELTA ? szCC : 0);
     static constexpr int oBeta = oA + szRA;
     static constexpr int oG = oBeta + C * 4;              // cumulative log-decay of the chunk rows (gated)
-    static constexpr int total = oG + C * 4;
+    static constexpr int oZ = oG + C * 4;                 // z entering the pass, T-typed row of 64 (normalised read-out)
+    static constexpr int total = oZ + (NORM ? HD * (int)sizeof(T) : 0);
 };
 
-template <typename T, int C, bool DELTA, bool FMAP, bool GATED>
+// What the normalised read-out adds to the argument list.
+struct NormArgs {
+    const float *z0;  // (B,H,64) or null
+    float *den;       // (B,T,H): the clamped denominators (residual of the backward call)
+    float *z_last;    // (B,H,64) or null
+    float *z_chk;     // (B,H,NC,64) or null: z entering each chunk
+    float eps;
+};
+
+template <typename T, int C, bool DELTA, bool FMAP, bool GATED, bool NORM>
 __global__ void __launch_bounds__(NTHR, 2)  // 2 waves per SIMD: two workgroups share a CU
 chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const float *__restrict__ glog,
                  const void *__restrict__ done, int done_f32,
                  const float *__restrict__ S0, T *__restrict__ o, float *__restrict__ S_last,
-                 T *__restrict__ S_chk, T *__restrict__ Tm_chk, int Tlen, int H)
+                 T *__restrict__ S_chk, T *__restrict__ Tm_chk, int Tlen, int H, NormArgs na)
 {
     static_assert(!(DELTA && GATED), "the gated variant is linear attention with a decay");
-    using L = FwdSmem<T, C, DELTA, GATED>;
+    static_assert(!NORM || (!DELTA && !GATED), "the normalised read-out belongs to plain linear attention");
+    using L = FwdSmem<T, C, DELTA, GATED, NORM>;
+    using Frag = typename TT<T>::frag;
     using IO = TileIO<T, C, NTHR>;
     using P4 = typename TT<T>::pack4;
     constexpr int LDD = L::LDD, LDC = L::LDC, LDA = L::LDA;
@@ -72,6 +86,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     float *sBeta = reinterpret_cast<float *>(smem + L::oBeta);
     float *sG = reinterpret_cast<float *>(smem + L::oG);
     T *sKd = sBK;                                    // gated: K_j exp(G_last - G_j)
+    T *sZ = reinterpret_cast<T *>(smem + L::oZ);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -92,6 +107,18 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         Sacc[j] = S0 ? *reinterpret_cast<const f32x4 *>(S0 + ((int64_t)bh * HD + dv) * HD + dk0)
                      : f32x4{0.f, 0.f, 0.f, 0.f};
     }
+
+    // normalised read-out: z[dk] of the running episode, held like a column of S^T (every lane
+    // of a 16-lane group carries the same four dk of each of the wave's m-tiles)
+    f32x4 zacc[TMS::MBW];
+#pragma unroll
+    for (int mi = 0; mi < TMS::MBW; ++mi) {
+        const int dk0 = TMS::mt(w, mi * TMS::NBW) * 16 + 4 * lg;
+        zacc[mi] = (NORM && na.z0) ? *reinterpret_cast<const f32x4 *>(na.z0 + (int64_t)bh * HD + dk0)
+                                   : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    const Frag ones = TT<T>::ones();
+    int64_t den_off = ((int64_t)b * Tlen + li) * H + h;  // den[t0 + li]
 
     MRX_WG_BEGIN();
     // register prefetch of the next chunk (raw bits only: no arithmetic on in-flight loads)
@@ -154,7 +181,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     int64_t o_off = base + (int64_t)li * rs + 4 * lg;                               // o[t0 + li][4 lg..]
     int64_t schk_off = (int64_t)bh * NC * HD * HD + li * HD + 4 * lg;                // S_chk[c][li][4 lg..]
     int64_t tmchk_off = (int64_t)bh * NC * C * C + (int64_t)tid * 4;                                  // row-major C x C
-    for (int c = 0; c < NC; ++c, o_off += (int64_t)C * rs, schk_off += HD * HD, tmchk_off += C * C) {
+    for (int c = 0; c < NC; ++c, o_off += (int64_t)C * rs, schk_off += HD * HD, tmchk_off += C * C, den_off += (int64_t)C * H) {
         const int t0 = c * C;
         const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
@@ -183,6 +210,8 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     IO::mask_rows(fk, tid, live);
                     IO::mask_rows(fv, tid, live);
                 }
+                // rows past the end of the sequence: phi(0) = 1 must not count towards z
+                if (NORM && FMAP && t0 + C > Tlen) IO::mask_rows(fk, tid, [&](int r) { return t0 + r < Tlen; });
                 IO::to_lds(fq, sQ, LDD, tid);
                 IO::to_lds(fk, sK, LDD, tid);
                 if (DELTA) {
@@ -210,6 +239,18 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 for (int j = 0; j < TMS::TPW; ++j)
                     *reinterpret_cast<P4 *>(S_chk + schk_off + TMS::nt(w, j) * 16 * HD + TMS::mt(w, j) * 16) =
                         TT<T>::pack(Sacc[j][0], Sacc[j][1], Sacc[j][2], Sacc[j][3]);
+            }
+            if (NORM) {
+                if (pass != 0) zero_acc<TMS::MBW>(zacc);
+                if (w < TMS::WM && li == 0) {
+#pragma unroll
+                    for (int mi = 0; mi < TMS::MBW; ++mi) {
+                        const int dk0 = TMS::mt(w, mi * TMS::NBW) * 16 + 4 * lg;
+                        *reinterpret_cast<P4 *>(sZ + dk0) = TT<T>::pack(zacc[mi][0], zacc[mi][1], zacc[mi][2], zacc[mi][3]);
+                        if (na.z_chk && pass == 0)
+                            *reinterpret_cast<f32x4 *>(na.z_chk + ((int64_t)bh * NC + c) * HD + dk0) = zacc[mi];
+                    }
+                }
             }
             sync_lds();
             MRX_PHASE(1);
@@ -309,18 +350,34 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             if (!DELTA && pre) { prefetch_part(2); prefetch_part(3); }
             f32x4 Oacc[TMO::TPW];
             zero_acc<TMO::TPW>(Oacc);
-            gemm<T, HD, C, HD, ROWK, ROWK, NW>(Oacc, sS, LDD, sQ, LDD, w, lane);
+            // normalised read-out: den_i = Q_i . z + sum_j Aqk[i][j], taken from the Q and Aqk
+            // fragments the two products load anyway (z as a tile of equal rows, a tile of ones)
+            f32x4 dacc[TMO::NBW];
+            zero_acc<TMO::NBW>(dacc);
+            auto den_q = [&](int ni, int kb, const Frag &yq) {
+                if (NORM) dacc[ni] = TT<T>::mma(TT<T>::template load<ROWK>(sZ, 0, 0, kb * TT<T>::KB, lane), yq, dacc[ni]);
+            };
+            auto den_a = [&](int ni, int, const Frag &ya) {
+                if (NORM) dacc[ni] = TT<T>::mma(ones, ya, dacc[ni]);
+            };
+            gemm<T, HD, C, HD, ROWK, ROWK, NW>(Oacc, sS, LDD, sQ, LDD, w, lane, NoHook(), den_q);
             if (GATED) {  // the incoming state reaches row i decayed by exp(G_i)
 #pragma unroll
                 for (int j = 0; j < TMO::TPW; ++j) Oacc[j] *= __expf(sG[TMO::nt(w, j) * 16 + li]);
             }
-            gemm<T, HD, C, C, KROW, ROWK, NW>(Oacc, sU, LDD, sAqk, LDC, w, lane);
+            gemm<T, HD, C, C, KROW, ROWK, NW>(Oacc, sU, LDD, sAqk, LDC, w, lane, NoHook(), den_a);
 #pragma unroll
             for (int j = 0; j < TMO::TPW; ++j) {
                 const int cc = TMO::nt(w, j) * 16 + li;
-                if (t0 + cc < Tlen && live(cc))
+                if (t0 + cc < Tlen && live(cc)) {
+                    if (NORM) {
+                        const float den = fmaxf(dacc[j % TMO::NBW][0], na.eps);
+                        Oacc[j] *= 1.f / den;
+                        if (TMO::mt(w, j) == 0 && lg == 0) na.den[den_off + (int64_t)(TMO::nt(w, j) * 16) * H] = den;
+                    }
                     *reinterpret_cast<P4 *>(o + o_off + (int64_t)(TMO::nt(w, j) * 16) * rs + TMO::mt(w, j) * 16) =
                         TT<T>::pack(Oacc[j][0], Oacc[j][1], Oacc[j][2], Oacc[j][3]);
+                }
             }
             // ---- S^T[dk][dv] += sum_c K[c][dk] U'[c][dv]  (only the episode that leaves the chunk)
             if (pass == nres) {
@@ -329,7 +386,10 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                     for (int j = 0; j < TMS::TPW; ++j) Sacc[j] *= cl;
                 }
-                gemm<T, HD, HD, C, KROW, KROW, NW>(Sacc, GATED ? sKd : sK, LDD, sU, LDD, w, lane);
+                auto z_k = [&](int mi, int, const Frag &xk) {  // z[dk] += sum_c K[c][dk]
+                    if (NORM) zacc[mi] = TT<T>::mma(xk, ones, zacc[mi]);
+                };
+                gemm<T, HD, HD, C, KROW, KROW, NW>(Sacc, GATED ? sKd : sK, LDD, sU, LDD, w, lane, z_k);
             }
             sync_lds();
             MRX_PHASE(8);
@@ -345,20 +405,25 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             *reinterpret_cast<f32x4 *>(S_last + ((int64_t)bh * HD + dv) * HD + dk0) = Sacc[j];
         }
     }
+    if (NORM && na.z_last && w < TMS::WM && li == 0) {
+#pragma unroll
+        for (int mi = 0; mi < TMS::MBW; ++mi)
+            *reinterpret_cast<f32x4 *>(na.z_last + (int64_t)bh * HD + TMS::mt(w, mi * TMS::NBW) * 16 + 4 * lg) = zacc[mi];
+    }
 }
 
-template <typename T, int C, bool DELTA, bool FMAP, bool GATED = false>
+template <typename T, int C, bool DELTA, bool FMAP, bool GATED = false, bool NORM = false>
 int launch(hipStream_t st, const void *q, const void *k, const void *v, const void *beta,
            const void *done, int done_f32, const void *S0, void *o, void *S_last, void *S_chk,
-           void *Tm_chk, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr)
+           void *Tm_chk, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr, NormArgs na = NormArgs{})
 {
-    auto kern = chunk_fwd_kernel<T, C, DELTA, FMAP, GATED>;
-    constexpr int smem = FwdSmem<T, C, DELTA, GATED>::total;
+    auto kern = chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM>;
+    constexpr int smem = FwdSmem<T, C, DELTA, GATED, NORM>::total;
     static unsigned long long lds_set = 0ull;
     if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(NTHR), smem, st, (const T *)q,
                        (const T *)k, (const T *)v, (const T *)beta, (const float *)glog, done, done_f32,
-                       (const float *)S0, (T *)o, (float *)S_last, (T *)S_chk, (T *)Tm_chk, (int)Tlen, (int)H);
+                       (const float *)S0, (T *)o, (float *)S_last, (T *)S_chk, (T *)Tm_chk, (int)Tlen, (int)H, na);
     return launch_status();
 }
 
@@ -431,5 +496,27 @@ extern "C" int mrx_gated_linear_attn_fwd(void *stream, const void *q, const void
     if (dtype == MRX_BF16)
         return fm ? launch<__bf16, LA_BF16_CHUNK, false, true, true>(MRX_ARGS) : launch<__bf16, LA_BF16_CHUNK, false, false, true>(MRX_ARGS);
     return fm ? launch<float, 32, false, true, true>(MRX_ARGS) : launch<float, 32, false, false, true>(MRX_ARGS);
+#undef MRX_ARGS
+}
+
+extern "C" int mrx_linear_attn_norm_fwd(void *stream, const void *q, const void *k, const void *v,
+                                        const void *done, const void *S0, const float *z0, void *o,
+                                        float *den, void *S_last, float *z_last, void *S_chk, float *z_chk,
+                                        int64_t B, int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
+                                        int done_dtype, int feature_map, float eps)
+{
+    const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
+    if (rc != MRX_OK) return rc;
+    if (!den || !aligned(den, 4) || !aligned(z0, 16) || !aligned(z_last, 16) || !aligned(z_chk, 16))
+        return MRX_ERR_INVALID_ARG;
+    if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const bool fm = feature_map == MRX_FMAP_ELU1;
+    const NormArgs na{z0, den, z_last, z_chk, eps};
+#define MRX_ARGS st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H, nullptr, na
+    if (dtype == MRX_BF16)
+        return fm ? launch<__bf16, LA_BF16_CHUNK, false, true, false, true>(MRX_ARGS)
+                  : launch<__bf16, LA_BF16_CHUNK, false, false, false, true>(MRX_ARGS);
+    return fm ? launch<float, 32, false, true, false, true>(MRX_ARGS) : launch<float, 32, false, false, false, true>(MRX_ARGS);
 #undef MRX_ARGS
 }

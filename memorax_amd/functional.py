@@ -87,6 +87,41 @@ def linear_attention(q, k, v, done, S0=None, feature_map="none"):
     return _LinearAttention.apply(q, k, v, done, S0, _FMAP[feature_map])
 
 
+class _NormalisedLinearAttention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, done, S0, z0, fmap, eps):
+        q_, k_, v_ = q.contiguous(), k.contiguous(), v.contiguous()
+        S0_ = None if S0 is None else S0.contiguous().float()
+        z0_ = None if z0 is None else z0.contiguous().float()
+        need = any(ctx.needs_input_grad)
+        ctx.done, ctx.fmap, ctx.eps, ctx.has_0 = done, fmap, eps, (S0 is not None, z0 is not None)
+        if q_.shape[1] == 1 and not need:  # acting: one fused step
+            o, S_last, z_last = K.linear_attn_step(q_[:, 0], k_[:, 0], v_[:, 0], done[:, 0], S0_, z0_,
+                                                   feature_map=_FMAP_NAME[fmap], normalise=True, eps=eps)
+            return o[:, None], S_last, z_last
+        o, den, S_last, z_last, chk = K.linear_attn_norm_fwd(q_, k_, v_, done, S0_, z0_, fmap, eps, save_chk=need)
+        if need:
+            ctx.save_for_backward(q_, k_, v_, o, den, *chk)
+        return o, S_last, z_last
+
+    @staticmethod
+    def backward(ctx, do, dS_last, dz_last):
+        q, k, v, o, den, S_chk, z_chk = ctx.saved_tensors
+        do = torch.zeros_like(v) if do is None else do.contiguous()
+        dS_last = None if dS_last is None else dS_last.contiguous().float()
+        dz_last = None if dz_last is None else dz_last.contiguous().float()
+        dq, dk, dv, dS0, dz0 = K.linear_attn_norm_bwd(q, k, v, ctx.done, (S_chk, z_chk), o, den, do, dS_last,
+                                                      dz_last, ctx.fmap, ctx.eps, want_d0=any(ctx.has_0))
+        return dq, dk, dv, None, (dS0 if ctx.has_0[0] else None), (dz0 if ctx.has_0[1] else None), None, None
+
+
+def normalised_linear_attention(q, k, v, done, S0=None, z0=None, feature_map="elu1", eps=1e-6):
+    """Causal linear attention with the normalised read-out of LinearAttentionCell.read
+    (linear_attention.py:93-110) in the same kernel: z_t = r_t z_{t-1} + phi(k_t),
+    o_t = S_t phi(q_t) / max(phi(q_t) . z_t, eps).  Returns (o, S_last, z_last)."""
+    return _NormalisedLinearAttention.apply(q, k, v, done, S0, z0, _FMAP[feature_map], float(eps))
+
+
 class _GatedLinearAttention(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, g, done, S0, fmap):

@@ -178,6 +178,54 @@ def linear_attn_bwd(q, k, v, done, S_chk, do, dS_last=None, feature_map=0, want_
     return dq, dk_, dv_, dS0
 
 
+def linear_attn_norm_fwd(q, k, v, done, S0=None, z0=None, feature_map=0, eps=1e-6, save_chk=True):
+    """Linear attention with the normalised read-out fused.
+    Returns (o, den fp32 (B,T,H), S_last fp32, z_last fp32, (S_chk, z_chk) or None)."""
+    lib = _lib.load()
+    B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
+    _chk(S0, "S0", torch.float32, (B, H, dv, dk))
+    _chk(z0, "z0", torch.float32, (B, H, dk))
+    done, dd = _done(done, B, T)
+    o = torch.empty_like(v)
+    den = torch.empty((B, T, H), dtype=torch.float32, device=q.device)
+    S_last = torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
+    z_last = torch.empty((B, H, dk), dtype=torch.float32, device=q.device)
+    nc = _n_chunks(T, dt)
+    S_chk = torch.empty((B, H, nc, dv, dk), dtype=dt, device=q.device) if save_chk else None
+    z_chk = torch.empty((B, H, nc, dk), dtype=torch.float32, device=q.device) if save_chk else None
+    st = lib.mrx_linear_attn_norm_fwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(done), _ptr(S0), _ptr(z0),
+                                      _ptr(o), _ptr(den), _ptr(S_last), _ptr(z_last), _ptr(S_chk), _ptr(z_chk),
+                                      B, T, H, dk, dv, _DT[dt], dd, int(feature_map), float(eps))
+    _lib.check(st, "mrx_linear_attn_norm_fwd")
+    return o, den, S_last, z_last, ((S_chk, z_chk) if save_chk else None)
+
+
+def linear_attn_norm_bwd(q, k, v, done, chk, o, den, do, dS_last=None, dz_last=None, feature_map=0, eps=1e-6,
+                         want_d0=True):
+    """Returns (dq, dk, dv, dS0, dz0)."""
+    lib = _lib.load()
+    B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
+    S_chk, z_chk = chk
+    nc = _n_chunks(T, dt)
+    _chk(do, "do", dt, (B, T, H, dv))
+    _chk(o, "o", dt, (B, T, H, dv))
+    _chk(den, "den", torch.float32, (B, T, H))
+    _chk(S_chk, "S_chk", dt, (B, H, nc, dv, dk))
+    _chk(z_chk, "z_chk", torch.float32, (B, H, nc, dk))
+    _chk(dS_last, "dS_last", torch.float32, (B, H, dv, dk))
+    _chk(dz_last, "dz_last", torch.float32, (B, H, dk))
+    done, dd = _done(done, B, T)
+    dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dS0 = torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device) if want_d0 else None
+    dz0 = torch.empty((B, H, dk), dtype=torch.float32, device=q.device) if want_d0 else None
+    st = lib.mrx_linear_attn_norm_bwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(done), _ptr(S_chk), _ptr(z_chk),
+                                      _ptr(o), _ptr(den), _ptr(do), _ptr(dS_last), _ptr(dz_last), _ptr(dq),
+                                      _ptr(dk_), _ptr(dv_), _ptr(dS0), _ptr(dz0), B, T, H, dk, dv, _DT[dt], dd,
+                                      int(feature_map), float(eps))
+    _lib.check(st, "mrx_linear_attn_norm_bwd")
+    return dq, dk_, dv_, dS0, dz0
+
+
 def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None):
     """Returns (o, S_last fp32, chk) where chk = (S_chk, Tm_chk) are the residuals the
     backward call needs, or None.  out = (o, S_last, S_chk, Tm_chk) reuses buffers of an earlier

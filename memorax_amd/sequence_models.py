@@ -27,7 +27,8 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .functional import delta_rule, gated_linear_attention, linear_attention, linear_scan
+from .functional import (delta_rule, gated_linear_attention, linear_attention, linear_scan,
+                         normalised_linear_attention)
 
 
 # ----------------------------------------------------------------------------------
@@ -304,8 +305,8 @@ class _RMSNorm(nn.Module):
 class LinearAttentionCell(MemoroidCellBase):
     """Causal linear attention with phi = elu + 1 (linear_attention.py:14-124).
     Elements are (v phi(k)^T, phi(k)) combined by addition; the reference materialises
-    S (B,T,H,d,d), here the numerator S_t phi(q_t) comes from the chunked kernel and the
-    normaliser z_t = sum phi(k) from the diagonal scan with decay 1."""
+    S (B,T,H,d,d); here the recurrence, the key sum z and the normalised read-out run in one
+    chunked kernel per direction."""
 
     def __init__(self, features, head_dim, num_heads, in_features=None, eps=1e-6):
         super().__init__()
@@ -329,23 +330,18 @@ class LinearAttentionCell(MemoroidCellBase):
         return tuple(x + y for x, y in zip(a, b))
 
     def scan(self, z, initial_carry, done):
-        """Returns h = (v, k_raw, z_cum) for read(), which needs the query."""
+        """Returns h = (v, k_raw, S0, z0, done) for read(): the numerator needs the query, so the
+        recurrence, the running key sum and the read-out all run in read's one kernel."""
         v, k_raw = z
         S0, z0 = initial_carry            # (B,1,H,dv,dk), (B,1,H,dk)
-        B, T, H, d = k_raw.shape
-        kf = (F.elu(k_raw.float()) + 1).reshape(B, T, H * d)
-        ones = torch.ones(H * d, device=kf.device)
-        zc, z_last, _ = linear_scan(ones, kf, done, z0[:, 0].reshape(B, H * d).float().contiguous())
-        return (v, k_raw, zc.view(B, T, H, d), S0[:, 0], done), z_last.view(B, 1, H, d)
+        return (v, k_raw, S0[:, 0], z0[:, 0], done), None
 
     def read(self, h, x, **kwargs):
-        v, k_raw, zc, S0, done = h
+        v, k_raw, S0, z0, done = h
         q = self._heads(self.query(x))
-        num, S_last = linear_attention(q, k_raw, v, done, S0.float(), "elu1")
-        self._S_last = S_last
-        qf = F.elu(q.float()) + 1
-        den = torch.clamp((qf * zc).sum(-1), min=self.eps)[..., None]
-        out = (num.float() / den).reshape(*x.shape[:2], -1)
+        out, S_last, z_last = normalised_linear_attention(q, k_raw, v, done, S0.float(), z0.float(), "elu1", self.eps)
+        self._carry = (S_last[:, None], z_last[:, None])
+        out = out.float().reshape(*x.shape[:2], -1)
         return self.output_projection(self.norm(out).to(x.dtype))
 
     def step(self, x, done, carry):
@@ -385,9 +381,9 @@ class LinearAttention(SequenceModel):
         if inputs.shape[1] == 1 and not torch.is_grad_enabled():
             return self.cell.step(inputs, done, initial_carry)
         z = self.cell(inputs)
-        h, z_last = self.cell.scan(z, initial_carry, done)
+        h, _ = self.cell.scan(z, initial_carry, done)
         y = self.cell.read(h, inputs)
-        return (self.cell._S_last[:, None], z_last), y
+        return self.cell._carry, y
 
     def initialize_carry(self, key, input_shape):
         return self.cell.initialize_carry(key, input_shape)

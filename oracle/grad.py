@@ -66,6 +66,21 @@ def linear_attention_t(q, k, v, done, S0, feature_map="none"):
     return torch.stack(os_, 1), S
 
 
+def normalised_linear_attention_t(q, k, v, done, S0, z0, feature_map="elu1", eps=1e-6):
+    if feature_map in ("elu1", 1):
+        q, k = elu1_t(q), elu1_t(k)
+    B, T, H, dk = q.shape
+    S, z = S0, z0
+    os_ = []
+    for t in range(T):
+        r = done[:, t]
+        S = torch.where(r[:, None, None, None], torch.zeros_like(S), S) + torch.einsum("bhi,bhj->bhij", v[:, t], k[:, t])
+        z = torch.where(r[:, None, None], torch.zeros_like(z), z) + k[:, t]
+        den = torch.clamp((q[:, t] * z).sum(-1), min=eps)
+        os_.append(torch.einsum("bhij,bhj->bhi", S, q[:, t]) / den[..., None])
+    return torch.stack(os_, 1), S, z
+
+
 def gated_linear_attention_t(q, k, v, g, done, S0, feature_map="none"):
     if feature_map in ("elu1", 1):
         q, k = elu1_t(q), elu1_t(k)
@@ -121,6 +136,25 @@ def linear_attention_grads(q, k, v, done, S0, do, dS_last=None, feature_map="non
     L.backward()
     return dict(o=_np(o), S_last=_np(Sl), dq=_np(q_.grad), dk=_np(k_.grad),
                 dv=_np(v_.grad), dS0=_np(S0_.grad))
+
+
+def normalised_linear_attention_grads(q, k, v, done, S0, z0, do, dS_last=None, dz_last=None,
+                                      feature_map="elu1", eps=1e-6):
+    """Returns dict(o, S_last, z_last, dq, dk, dv, dS0, dz0) for
+    L = sum(do*o) + sum(dS_last*S_last) + sum(dz_last*z_last)."""
+    q_, k_, v_ = _t(q, True), _t(k, True), _t(v, True)
+    B, T, H, dk = q_.shape
+    S0_ = _t(np.zeros((B, H, v_.shape[-1], dk)) if S0 is None else S0, True)
+    z0_ = _t(np.zeros((B, H, dk)) if z0 is None else z0, True)
+    o, Sl, zl = normalised_linear_attention_t(q_, k_, v_, _done(done), S0_, z0_, feature_map, eps)
+    L = (o * _t(do)).sum()
+    if dS_last is not None:
+        L = L + (Sl * _t(dS_last)).sum()
+    if dz_last is not None:
+        L = L + (zl * _t(dz_last)).sum()
+    L.backward()
+    return dict(o=_np(o), S_last=_np(Sl), z_last=_np(zl), dq=_np(q_.grad), dk=_np(k_.grad),
+                dv=_np(v_.grad), dS0=_np(S0_.grad), dz0=_np(z0_.grad))
 
 
 def delta_rule_grads(q, k, v, beta, done, S0, do, dS_last=None):

@@ -357,6 +357,31 @@ def linear_attention_memoroid(q, k, v, done, carry=None, feature_map="none"):
     return nxt, num, den
 
 
+def normalised_linear_attention(q, k, v, done, S0=None, z0=None, feature_map="elu1", eps=1e-6):
+    """Recurrent form of the cell with its read-out (linear_attention.py:62-86 for the
+    elements, :93-110 for the read-out, scanned by memoroid.py:60-91):
+        S_t = r_t S_{t-1} + v_t k_t^T ;  z_t = r_t z_{t-1} + k_t ;
+        o_t = S_t q_t / max(q_t . z_t, eps)          (q, k after the feature map).
+    Returns (o (B,T,H,dv), den (B,T,H) clamped, S_last (B,H,dv,dk), z_last (B,H,dk))."""
+    q = _fmap(q, feature_map)
+    k = _fmap(k, feature_map)
+    v = np.asarray(v, dtype=np.float64)
+    B, T, H, dk = q.shape
+    dv = v.shape[-1]
+    S = np.zeros((B, H, dv, dk)) if S0 is None else np.asarray(S0, np.float64).copy()
+    z = np.zeros((B, H, dk)) if z0 is None else np.asarray(z0, np.float64).copy()
+    done = np.asarray(done) != 0
+    o = np.empty((B, T, H, dv))
+    den = np.empty((B, T, H))
+    for t in range(T):
+        r = done[:, t]
+        S = np.where(r[:, None, None, None], 0.0, S) + np.einsum("bhi,bhj->bhij", v[:, t], k[:, t])
+        z = np.where(r[:, None, None], 0.0, z) + k[:, t]
+        den[:, t] = np.maximum(np.einsum("bhd,bhd->bh", q[:, t], z), eps)
+        o[:, t] = np.einsum("bhij,bhj->bhi", S, q[:, t]) / den[:, t][..., None]
+    return o, den, S, z
+
+
 def gated_linear_attention(q, k, v, g, done, S0=None, feature_map="none"):
     """Recurrent form with a scalar log-decay per step and head:
         S_t = r_t exp(g_t) S_{t-1} + v_t k_t^T ;  o_t = S_t q_t.

@@ -86,6 +86,31 @@ def test_linear_attention_grads_fd(fmap):
     np.testing.assert_allclose(ag["S_last"], Sl, rtol=1e-12)
 
 
+@pytest.mark.parametrize("eps", [1e-6, 7.0])
+def test_normalised_linear_attention_grads_fd(eps):
+    """eps = 7 puts two of the seven rows under the clamp (no gradient through the denominator)."""
+    B, T, H, dk, dv = 1, 7, 1, 3, 2
+    r = np.random.default_rng(2)   # own stream: which rows the clamp catches must not depend on test order
+    rnd = lambda *s: r.standard_normal(s)  # noqa: E731
+    q, k, v, S0 = rnd(B, T, H, dk), rnd(B, T, H, dk), rnd(B, T, H, dv), rnd(B, H, dv, dk)
+    z0 = np.abs(rnd(B, H, dk))
+    do, dSl, dzl = rnd(B, T, H, dv), rnd(B, H, dv, dk), rnd(B, H, dk)
+    d = np.zeros((B, T), bool)
+    d[0, 3] = True
+
+    def L():
+        o, den, Sl, zl = M.normalised_linear_attention(q, k, v, d, S0, z0, "elu1", eps)
+        return (o * do).sum() + (Sl * dSl).sum() + (zl * dzl).sum()
+
+    _, den, _, _ = M.normalised_linear_attention(q, k, v, d, S0, z0, "elu1", eps)
+    if eps > 1:
+        assert (den == eps).any() and (den > eps).any()
+        assert np.abs(den[den > eps] - eps).min() > 1.0    # no row sits near the kink
+    ag = G.normalised_linear_attention_grads(q, k, v, d, S0, z0, do, dSl, dzl, "elu1", eps)
+    for name, x in (("dq", q), ("dk", k), ("dv", v), ("dS0", S0), ("dz0", z0)):
+        np.testing.assert_allclose(ag[name], fd(L, x), rtol=1e-5, atol=1e-7, err_msg=name)
+
+
 def test_delta_rule_grads_fd():
     B, T, H, dk, dv = 1, 7, 1, 3, 2
     q, k, v, S0 = rnd(B, T, H, dk), rnd(B, T, H, dk), rnd(B, T, H, dv), rnd(B, H, dv, dk)

@@ -191,6 +191,33 @@ def test_linear_attention_formulations(fmap, p):
     np.testing.assert_allclose(den, den2, rtol=1e-10, atol=1e-10)
 
 
+@pytest.mark.parametrize("p", [0.0, 0.15])
+def test_normalised_linear_attention_against_the_materialised_route_and_convexity(p):
+    B, T, H, dk, dv = 2, 29, 2, 5, 4
+    q, k, v = rnd(B, T, H, dk), rnd(B, T, H, dk), rnd(B, T, H, dv)
+    S0, z0 = rnd(B, H, dv, dk), np.abs(rnd(B, H, dk))
+    d = dones(B, T, p)
+    o, den, Sl, zl = M.normalised_linear_attention(q, k, v, d, S0, z0, "elu1", 1e-6)
+    # the reference's route: materialised outer products, additive tree scan, read-out
+    nxt, num, den2 = M.linear_attention_memoroid(q, k, v, d, (S0[:, None], z0[:, None]), "elu1")
+    np.testing.assert_allclose(den, np.maximum(den2, 1e-6), rtol=1e-10)
+    np.testing.assert_allclose(o, num / np.maximum(den2, 1e-6)[..., None], rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(Sl, nxt[0][:, 0], rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(zl, nxt[1][:, 0], rtol=1e-10, atol=1e-12)
+    # without carry the read-out is a convex combination of the episode's values:
+    # constant values come back unchanged, and every output lies within the values' range
+    c = rnd(dv)
+    oc, _, _, _ = M.normalised_linear_attention(q, k, np.broadcast_to(c, v.shape), d, None, None, "elu1", 1e-6)
+    np.testing.assert_allclose(oc, np.broadcast_to(c, v.shape), rtol=1e-10, atol=1e-12)
+    on, _, _, _ = M.normalised_linear_attention(q, k, v, d, None, None, "elu1", 1e-6)
+    assert on.max() <= v.max() + 1e-12 and on.min() >= v.min() - 1e-12
+    # the clamp: a denominator below eps is replaced by eps
+    ob, denb, _, _ = M.normalised_linear_attention(q, k, v, d, None, None, "elu1", 1e3)
+    assert (denb == 1e3).all()
+    num0, _ = M.linear_attention(q, k, v, d, None, "elu1")
+    np.testing.assert_allclose(ob, num0 / 1e3, rtol=1e-12)
+
+
 def test_linear_attention_cumsum_special_case():
     B, T, H, d = 1, 20, 1, 3
     e1 = np.zeros((B, T, H, d))
