@@ -16,6 +16,68 @@ from . import kernels as K
 
 _FMAP = {None: 0, "none": 0, 0: 0, "elu1": 1, 1: 1}
 _FMAP_NAME = {0: "none", 1: "elu1"}
+_HD = 64  # head dim of the kernels (d_k = d_v)
+
+
+class _Heads:
+    """Maps other head dims onto the kernels' d_k = d_v = 64 (the reference's cells take any
+    head_dim; its guides use 16).  d_k < 64 is zero-padded -- after the feature map, since
+    phi(0) = 1 would otherwise count -- and d_v is zero-padded to a multiple of 64 and split into
+    blocks that run as extra heads sharing q and k (rows of the state are independent recurrences).
+    Padding, blocks and slices are ordinary differentiable array ops around the kernel call."""
+
+    def __init__(self, q, v, fmap=0):
+        self.B, self.T, self.H, self.dk = q.shape
+        self.dv = v.shape[-1]
+        if self.dk > _HD:
+            raise ValueError(f"d_k = {self.dk} > {_HD} is not supported (d_v may be any size)")
+        self.nb = (self.dv + _HD - 1) // _HD
+        self.native = self.dk == _HD and self.dv == _HD
+        self.pre = fmap if self.dk != _HD else 0    # feature map applied here, before the padding
+        self.fmap = 0 if self.pre else fmap         # feature map left to the kernel
+
+    def _blocks(self, x):  # (B,T,H,64) -> (B,T,H*nb,64), every block a copy
+        if self.nb == 1:
+            return x
+        return x[:, :, :, None].expand(self.B, self.T, self.H, self.nb, _HD).reshape(self.B, self.T, self.H * self.nb, _HD)
+
+    def qk(self, x):
+        if self.native:
+            return x
+        if self.pre:
+            xf = x if x.dtype in (torch.float32, torch.float64) else x.float()
+            x = (torch.nn.functional.elu(xf) + 1).to(x.dtype)
+        return self._blocks(torch.nn.functional.pad(x, (0, _HD - self.dk)))
+
+    def v(self, x):
+        if self.native:
+            return x
+        x = torch.nn.functional.pad(x, (0, self.nb * _HD - self.dv))
+        return x.reshape(self.B, self.T, self.H * self.nb, _HD)
+
+    def per_head(self, x):  # (B,T,H) -> (B,T,H*nb)
+        return x if self.nb == 1 else x.repeat_interleave(self.nb, dim=2)
+
+    def state_in(self, S):  # (B,H,dv,dk) -> (B,H*nb,64,64)
+        if S is None or self.native:
+            return S
+        S = torch.nn.functional.pad(S, (0, _HD - self.dk, 0, self.nb * _HD - self.dv))
+        return S.reshape(self.B, self.H * self.nb, _HD, _HD)
+
+    def z_in(self, z):  # (B,H,dk) -> (B,H*nb,64)
+        if z is None or self.native:
+            return z
+        z = torch.nn.functional.pad(z, (0, _HD - self.dk))
+        return z if self.nb == 1 else z.repeat_interleave(self.nb, dim=1)
+
+    def out(self, o):  # (B,T,H*nb,64) -> (B,T,H,dv)
+        return o if self.native else o.reshape(self.B, o.shape[1], self.H, self.nb * _HD)[..., :self.dv]
+
+    def state_out(self, S):
+        return S if self.native else S.reshape(self.B, self.H, self.nb * _HD, _HD)[:, :, :self.dv, :self.dk]
+
+    def z_out(self, z):
+        return z if self.native else z.reshape(self.B, self.H, self.nb, _HD)[:, :, 0, :self.dk]
 
 
 class _LinearScan(torch.autograd.Function):
@@ -84,7 +146,9 @@ class _LinearAttention(torch.autograd.Function):
 def linear_attention(q, k, v, done, S0=None, feature_map="none"):
     """Causal unnormalised linear attention, chunked: S_t = r_t S_{t-1} + v_t phi(k_t)^T,
     o_t = S_t phi(q_t) (linear_attention.py:62-86,105).  Returns (o, S_last)."""
-    return _LinearAttention.apply(q, k, v, done, S0, _FMAP[feature_map])
+    hd = _Heads(q, v, _FMAP[feature_map])
+    o, S_last = _LinearAttention.apply(hd.qk(q), hd.qk(k), hd.v(v), done, hd.state_in(S0), hd.fmap)
+    return hd.out(o), hd.state_out(S_last)
 
 
 class _NormalisedLinearAttention(torch.autograd.Function):
@@ -119,7 +183,10 @@ def normalised_linear_attention(q, k, v, done, S0=None, z0=None, feature_map="el
     """Causal linear attention with the normalised read-out of LinearAttentionCell.read
     (linear_attention.py:93-110) in the same kernel: z_t = r_t z_{t-1} + phi(k_t),
     o_t = S_t phi(q_t) / max(phi(q_t) . z_t, eps).  Returns (o, S_last, z_last)."""
-    return _NormalisedLinearAttention.apply(q, k, v, done, S0, z0, _FMAP[feature_map], float(eps))
+    hd = _Heads(q, v, _FMAP[feature_map])
+    o, S_last, z_last = _NormalisedLinearAttention.apply(hd.qk(q), hd.qk(k), hd.v(v), done, hd.state_in(S0),
+                                                         hd.z_in(z0), hd.fmap, float(eps))
+    return hd.out(o), hd.state_out(S_last), hd.z_out(z_last)
 
 
 class _GatedLinearAttention(torch.autograd.Function):
@@ -149,7 +216,10 @@ def gated_linear_attention(q, k, v, g, done, S0=None, feature_map="none"):
     """Linear attention with a scalar log-decay g:(B,T,H) per step and head:
     S_t = r_t exp(g_t) S_{t-1} + v_t phi(k_t)^T, o_t = S_t phi(q_t) -- the Mamba cell's algebra
     (mamba.py:109-122) in chunked form.  Returns (o, S_last)."""
-    return _GatedLinearAttention.apply(q, k, v, g, done, S0, _FMAP[feature_map])
+    hd = _Heads(q, v, _FMAP[feature_map])
+    o, S_last = _GatedLinearAttention.apply(hd.qk(q), hd.qk(k), hd.v(v), hd.per_head(g), done, hd.state_in(S0),
+                                            hd.fmap)
+    return hd.out(o), hd.state_out(S_last)
 
 
 class _DeltaRule(torch.autograd.Function):
@@ -181,7 +251,9 @@ class _DeltaRule(torch.autograd.Function):
 def delta_rule(q, k, v, beta, done, S0=None):
     """DeltaNet recurrence S_t = r_t S_{t-1}(I - beta_t k_t k_t^T) + beta_t v_t k_t^T,
     o_t = S_t q_t, in chunked WY form.  Returns (o, S_last)."""
-    return _DeltaRule.apply(q, k, v, beta, done, S0)
+    hd = _Heads(q, v)
+    o, S_last = _DeltaRule.apply(hd.qk(q), hd.qk(k), hd.v(v), hd.per_head(beta), done, hd.state_in(S0))
+    return hd.out(o), hd.state_out(S_last)
 
 
 def propagate_sensitivities(decay, jacobians, sensitivity, done):

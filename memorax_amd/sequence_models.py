@@ -346,19 +346,11 @@ class LinearAttentionCell(MemoroidCellBase):
 
     def step(self, x, done, carry):
         """Acting path (T = 1, no gradients): state update, normaliser and divide in one kernel
-        (what __call__, binary_operator and read of linear_attention.py:62-117 do for one step)."""
-        from . import kernels as K
-        S0, z0 = carry
-        v, k_raw = self(x)
-        q = self._heads(self.query(x))
-        B = x.shape[0]
-        o, S_new, z_new = K.linear_attn_step(
-            q[:, 0].contiguous(), k_raw[:, 0].contiguous(), v[:, 0].contiguous(), done.reshape(B),
-            S0[:, 0].float().contiguous(), z0[:, 0].float().contiguous(), feature_map="elu1",
-            normalise=True, eps=self.eps)
-        out = o.float().reshape(B, 1, -1)
-        y = self.output_projection(self.norm(out).to(x.dtype))
-        return (S_new[:, None], z_new[:, None]), y
+        (what __call__, binary_operator and read of linear_attention.py:62-117 do for one step);
+        normalised_linear_attention picks the single-step kernel for such a call."""
+        h, _ = self.scan(self(x), carry, done)
+        y = self.read(h, x)
+        return self._carry, y
 
     def initialize_carry(self, key, input_shape):
         *batch, _ = input_shape
