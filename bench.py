@@ -84,7 +84,7 @@ def main() -> int:
 
     # per-kernel durations with HIP events on the stream the kernels are launched on
     ev = lambda: torch.cuda.Event(enable_timing=True)  # noqa: E731
-    tf = tb = 0.0
+    tfs, tbs = [], []
     for _ in range(args.steps):
         e0, e1, e2 = ev(), ev(), ev()
         e0.record()
@@ -93,9 +93,10 @@ def main() -> int:
         K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, out=bwd_out)
         e2.record()
         torch.cuda.synchronize()
-        tf += e0.elapsed_time(e1)
-        tb += e1.elapsed_time(e2)
-    tf_ms, tb_ms = tf / args.steps, tb / args.steps
+        tfs.append(e0.elapsed_time(e1))
+        tbs.append(e1.elapsed_time(e2))
+    tf_ms, tb_ms = sum(tfs) / args.steps, sum(tbs) / args.steps
+    pct = lambda xs: {f"p{p}_ms": float(np.percentile(xs, p)) for p in (10, 50, 90)}  # noqa: E731
     nth = B * T * H
     bwd_gbs = BYTES_BWD * nth / (tb_ms * 1e-3) / 1e9
     fwd_gbs = BYTES_FWD * nth / (tf_ms * 1e-3) / 1e9
@@ -121,8 +122,8 @@ def main() -> int:
             "launch_ms": tb_ms, "algorithmic_bytes": BYTES_BWD * nth,
         },
         "kernels": {
-            "delta_fwd": {"ms": tf_ms, "GB/s": fwd_gbs, "frac_hbm": fwd_gbs / HBM_PEAK_GBS},
-            "delta_bwd": {"ms": tb_ms, "GB/s": bwd_gbs, "frac_hbm": bwd_gbs / HBM_PEAK_GBS},
+            "delta_fwd": {"ms": tf_ms, "GB/s": fwd_gbs, "frac_hbm": fwd_gbs / HBM_PEAK_GBS, **pct(tfs)},
+            "delta_bwd": {"ms": tb_ms, "GB/s": bwd_gbs, "frac_hbm": bwd_gbs / HBM_PEAK_GBS, **pct(tbs)},
             "fwd+bwd": {"ms": tf_ms + tb_ms,
                         "GB/s": (BYTES_FWD + BYTES_BWD) * nth / ((tf_ms + tb_ms) * 1e-3) / 1e9},
         },
@@ -177,6 +178,21 @@ def bench_scan(torch, K, M, dev):
         res[name] = {"fwd_ms": ms, "fwd_GB/s": by / ms / 1e6, "fwd_frac_hbm": by / ms / 1e6 / HBM_PEAK_GBS,
                      "fwd_tokens/s": Bn * Tn / ms * 1e3,
                      "bwd_ms": msb, "bwd_GB/s": 20 * Bn * Tn * Dn / msb / 1e6}
+        if 12 * Bn * Tn * Dn < 256e6:
+            # the working set fits the 256 MB Infinity Cache: also time it with the inputs rotated
+            # through enough copies (> 512 MB) that every call reads them from HBM
+            nset = int(512e6 // (8 * Bn * Tn * Dn)) + 1
+            sets = [(a.clone(), b.clone()) for _ in range(nset)]
+            it = [0]
+
+            def rotated():
+                aa, bb = sets[it[0] % nset]
+                it[0] += 1
+                K.linear_scan_fwd(aa, bb, dn, want_P=False)
+            msr = _time_ms(torch, rotated, iters=2 * nset, warm=nset)
+            res[name]["fwd_ms_inputs_rotated"] = msr
+            res[name]["fwd_GB/s_inputs_rotated"] = by / msr / 1e6
+            del sets
         del a, b, g, h
     return res
 
