@@ -76,15 +76,15 @@ __device__ __forceinline__ void store_rows_at(const f32x4 *acc, T *row, int64_t 
 }
 
 // =====================================================================================
-// linear attention: 8 tiles, two workgroups per CU; with a per-step decay (GATED) one tile more
+// linear attention: 8 tiles, two workgroups per CU
 // =====================================================================================
 template <typename T, int C, bool GATED = false, bool NORM = false> struct LaBwdSmem : BwdDims<T, C> {
     using D = BwdDims<T, C>;
     static constexpr int oQ = 0, oK = oQ + D::szRD, oV = oK + D::szRD, oDO = oV + D::szRD,
                          oS = oDO + D::szRD, oDS = oS + D::szDD, oAqk = oDS + D::szDD,
-                         oDAqk = oAqk + D::szCC, oQa = oDAqk + D::szCC,    // gated: exp(G_i) Q_i
-                         oG = oQa + (GATED ? D::szRD : 0),                 // gated: G[C], then [WM][C] row-dot partials
-                         oN = oG + (GATED ? (1 + TileMap<HD, C, 4>::WM) * C * 4 : 0),
+                         oDAqk = oAqk + D::szCC,
+                         oG = oDAqk + D::szCC,    // gated: G[C], [WM][C] row-dot partials, exp(G)[C]
+                         oN = oG + (GATED ? (2 + TileMap<HD, C, 4>::WM) * C * 4 : 0),
                          // normalised read-out: dden fp32 [C], dden T-typed [C] (C * 4 bytes kept), z fp32 [64], dz fp32 [64]
                          total = oN + (NORM ? 2 * C * 4 + 2 * HD * 4 : 0);
 };
@@ -149,9 +149,9 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     T *sDS = reinterpret_cast<T *>(smem + L::oDS);
     T *sAqk = reinterpret_cast<T *>(smem + L::oAqk);
     T *sDAqk = reinterpret_cast<T *>(smem + L::oDAqk);
-    T *sQa = reinterpret_cast<T *>(smem + L::oQa);
     float *sG = reinterpret_cast<float *>(smem + L::oG);
     float *sE = sG + C;  // [WM][C] partial row dots
+    float *sEa = sE + TileMap<HD, C, 4>::WM * C;  // a_i = exp(G_i)
     float *sDd = reinterpret_cast<float *>(smem + L::oN);       // dden[C]
     T *sDdT = reinterpret_cast<T *>(smem + L::oN + C * 4);      // dden[C], T-typed (MFMA operand)
     float *sZf = reinterpret_cast<float *>(smem + L::oN + 2 * C * 4);  // z entering the chunk
@@ -269,7 +269,10 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     if (lane >= off) G += up;
                 }
                 Glast = __shfl(G, C - 1);
-                if (w == 0 && lane < C) sG[lane] = G;
+                if (w == 0 && lane < C) {
+                    sG[lane] = G;
+                    sEa[lane] = __expf(G);
+                }
             }
             // ---- stage -------------------------------------------------------------
             {
@@ -304,13 +307,6 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     if (tid < 16) *reinterpret_cast<f32x4 *>(sZf + 4 * tid) = rz;
                 }
                 IO::to_lds(fq, sQ, LDD, tid);
-                if (GATED) {
-                    float af[IO::PASSES];
-#pragma unroll
-                    for (int p = 0; p < IO::PASSES; ++p) af[p] = __expf(__shfl(G, IO::row_of(tid, p)));
-                    IO::scale_rows(fq, af);
-                    IO::to_lds(fq, sQa, LDD, tid);
-                }
                 IO::to_lds(fk, sK, LDD, tid);
                 IO::to_lds(fv, sV, LDD, tid);
                 IO::to_lds(fdo, sDO, LDD, tid);
@@ -456,10 +452,16 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     if (lg == 0) sE[(w % TMR::WM) * C + TMR::nt(w, j) * 16 + li] = x;
                 }
             }
-            auto dz_q = [&](int mi, int kb, const Frag &xq) {  // dz[dk] += sum_i Q[i][dk] dden_i
-                if (NORM) dzacc[mi] = TT<T>::mma(xq, TT<T>::template load<ROWK>(sDdT, 0, 0, kb * TT<T>::KB, lane), dzacc[mi]);
+            auto dz_q = [&](int mi, int kb, Frag &xq) {
+                if (NORM)  // dz[dk] += sum_i Q[i][dk] dden_i
+                    dzacc[mi] = TT<T>::mma(xq, TT<T>::template load<ROWK>(sDdT, 0, 0, kb * TT<T>::KB, lane), dzacc[mi]);
+                if (GATED) {  // row c of Q enters the state update as a_c Q[c]: scale the fragment along k
+                    const float *ea = sEa + kb * TT<T>::KB + TT<T>::KP * lg;
+#pragma unroll
+                    for (int e = 0; e < TT<T>::KP; ++e) xq[e] = (T)((float)xq[e] * ea[e]);
+                }
             };
-            gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, GATED ? sQa : sQ, LDD, sDO, LDD, w, lane, dz_q);
+            gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, sQ, LDD, sDO, LDD, w, lane, dz_q);
             sync_lds();
             if (GATED && tid < C && t0 + tid < Tlen && live(tid)) {
                 float x = 0.f;

@@ -149,12 +149,14 @@ template <int M, int N, int NW, int MBW_ = 0> struct TileMap {
 };
 
 struct NoHook {
-    template <typename F> __device__ __forceinline__ void operator()(int, int, const F &) const {}
+    template <typename F> __device__ __forceinline__ void operator()(int, int, F &) const {}
 };
 
 // acc[j] += sum_k X(mt_j rows, k) * Y(nt_j rows, k), k = 0..K-1.
 // hx(mi, kb, fragment) / hy(ni, kb, fragment) see every operand fragment as it is loaded, so that
-// a rank-one by-product (a row or column sum, a product with one more vector) costs MFMAs only.
+// a rank-one by-product (a row or column sum, a product with one more vector) costs MFMAs only;
+// a hook may also rewrite the fragment (scale it along k) before it is used.  Element e of a
+// fragment belongs to k = kb * KB + KP * (lane / 16) + e in both operand modes.
 template <typename T, int M, int N, int K, int XM, int YM, int NW, int MBW_ = 0, typename HX = NoHook, typename HY = NoHook>
 __device__ __forceinline__ void gemm(f32x4 *acc, const T *X, int ldx, const T *Y, int ldy, int w, int lane,
                                      HX hx = HX(), HY hy = HY())
@@ -174,7 +176,7 @@ __device__ __forceinline__ void gemm(f32x4 *acc, const T *X, int ldx, const T *Y
         }
 #pragma unroll
         for (int ni = 0; ni < TM::NBW; ++ni) {
-            const F b = TT<T>::template load<YM>(Y, ldy, TM::nt(w, ni) * 16, kb * KB, lane);
+            F b = TT<T>::template load<YM>(Y, ldy, TM::nt(w, ni) * 16, kb * KB, lane);
             hy(ni, kb, b);
 #pragma unroll
             for (int mi = 0; mi < TM::MBW; ++mi)

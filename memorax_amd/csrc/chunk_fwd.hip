@@ -38,13 +38,13 @@ template <typename T, int C, bool DELTA, bool GATED = false, bool NORM = false> 
     static constexpr int oQ = 0;                          // Q [C][dk], later U' [C][dv]
     static constexpr int oK = oQ + szRD;                  // K [C][dk]
     static constexpr int oV = oK + szRD;                  // V [C][dv]  (delta rule: beta_j V_j)
-    static constexpr int oBK = oV + szRD;                 // beta_j K_j [C][dk] (delta rule) / decayed K (gated)
-    static constexpr int oS = oBK + ((DELTA || GATED) ? szRD : 0);   // S [dv][dk]
+    static constexpr int oBK = oV + szRD;                 // beta_j K_j [C][dk] (delta rule)
+    static constexpr int oS = oBK + (DELTA ? szRD : 0);   // S [dv][dk]
     static constexpr int oTm = oS + szDD;                 // Tm [C][C]  (delta rule only)
     static constexpr int oA = oTm + (DELTA ? szCC : 0);
     static constexpr int oBeta = oA + szRA;
-    static constexpr int oG = oBeta + C * 4;              // cumulative log-decay of the chunk rows (gated)
-    static constexpr int oZ = oG + C * 4;                 // z entering the pass, T-typed row of 64 (normalised read-out)
+    static constexpr int oG = oBeta + C * 4;              // gated: cumulative log-decay G of the chunk rows, then exp(G_last - G)
+    static constexpr int oZ = oG + 2 * C * 4;             // z entering the pass, T-typed row of 64 (normalised read-out)
     static constexpr int total = oZ + (NORM ? HD * (int)sizeof(T) : 0);
 };
 
@@ -85,7 +85,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     T *sU = sV;                                      // U' [C][dv] (delta rule: over beta V once U is taken)
     float *sBeta = reinterpret_cast<float *>(smem + L::oBeta);
     float *sG = reinterpret_cast<float *>(smem + L::oG);
-    T *sKd = sBK;                                    // gated: K_j exp(G_last - G_j)
+    float *sEb = sG + C;                             // gated: b_j = exp(G_last - G_j)
     T *sZ = reinterpret_cast<T *>(smem + L::oZ);
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -198,7 +198,10 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     if (lane >= off) G += up;
                 }
                 Glast = __shfl(G, C - 1);
-                if (w == 0 && lane < C) sG[lane] = G;
+                if (w == 0 && lane < C) {
+                    sG[lane] = G;
+                    sEb[lane] = __expf(Glast - G);
+                }
             }
             // ---- stage the chunk ---------------------------------------------------
             {
@@ -221,13 +224,6 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     IO::scale_rows(fk, bf);
                     IO::scale_rows(fv, bf);
                     IO::to_lds(fk, sBK, LDD, tid);
-                }
-                if (GATED) {
-                    float bf[IO::PASSES];
-#pragma unroll
-                    for (int p = 0; p < IO::PASSES; ++p) bf[p] = __expf(Glast - __shfl(G, IO::row_of(tid, p)));
-                    IO::scale_rows(fk, bf);
-                    IO::to_lds(fk, sKd, LDD, tid);
                 }
                 IO::to_lds(fv, sV, LDD, tid);
             }
@@ -386,10 +382,15 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                     for (int j = 0; j < TMS::TPW; ++j) Sacc[j] *= cl;
                 }
-                auto z_k = [&](int mi, int, const Frag &xk) {  // z[dk] += sum_c K[c][dk]
-                    if (NORM) zacc[mi] = TT<T>::mma(xk, ones, zacc[mi]);
+                auto z_k = [&](int mi, int kb, Frag &xk) {
+                    if (NORM) zacc[mi] = TT<T>::mma(xk, ones, zacc[mi]);  // z[dk] += sum_c K[c][dk]
+                    if (GATED) {  // row c of K enters the state update as b_c K[c]: scale the fragment along k
+                        const float *eb = sEb + kb * TT<T>::KB + TT<T>::KP * lg;
+#pragma unroll
+                        for (int e = 0; e < TT<T>::KP; ++e) xk[e] = (T)((float)xk[e] * eb[e]);
+                    }
                 };
-                gemm<T, HD, HD, C, KROW, KROW, NW>(Sacc, GATED ? sKd : sK, LDD, sU, LDD, w, lane, z_k);
+                gemm<T, HD, HD, C, KROW, KROW, NW>(Sacc, sK, LDD, sU, LDD, w, lane, z_k);
             }
             sync_lds();
             MRX_PHASE(8);
