@@ -167,6 +167,26 @@ int mrx_delta_rule_bwd(void *stream, const void *q, const void *k,
                        void *dbeta, void *dS0, int64_t B, int64_t T, int64_t H,
                        int64_t dk, int64_t dv, int dtype, int done_dtype);
 
+/* ---- DeltaNet cell recurrence with its prologue fused -------------------------
+ * As mrx_delta_rule_fwd / _bwd, but on the raw projections: inside the kernels
+ *     k_t <- k_t / max(|k_t|, 1e-12)  (fp32, then rounded to `dtype`) ;  beta_t = sigmoid(beta_raw_t)
+ * so that the normalised keys and the gates are never written to memory, and the backward
+ * call returns the gradients w.r.t. the raw k and beta_raw.  Like the delta rule itself this
+ * has no counterpart in the reference; it is the prologue a DeltaNet cell written in the
+ * reference's cell idiom (projections -> elements, memoroid.py:20-33) would run per step.
+ * Residuals as for mrx_delta_rule_*. */
+int mrx_deltanet_fwd(void *stream, const void *q, const void *k, const void *v,
+                     const void *beta_raw, const void *done, const void *S0, void *o,
+                     void *S_last, void *S_chk, void *Tm_chk, int64_t B, int64_t T,
+                     int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype);
+
+int mrx_deltanet_bwd(void *stream, const void *q, const void *k, const void *v,
+                     const void *beta_raw, const void *done, const void *S_chk,
+                     const void *Tm_chk, const void *dout, const void *dS_last, void *dq,
+                     void *dk_out, void *dv_out, void *dbeta_raw, void *dS0, int64_t B,
+                     int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
+                     int done_dtype);
+
 /* Final state only, one decay per `a_group` consecutive channels: h_T of
  *     h_t = done_t ? b_t : a_t h_{t-1} + b_t ,  a: (B,T,D/a_group), b: (B,T,D), h0 (nullable), h_last: (B,D).
  * The sensitivity propagation of real-time recurrent learning, Memoroid._propagate_sensitivities

@@ -7,7 +7,7 @@ Layers:
   sequence_models  Memoroid-style modules: (inputs, done, initial_carry) -> (next_carry, y)
 """
 from . import _lib  # noqa: F401
-from .functional import (delta_rule, gated_linear_attention, linear_attention, linear_scan,  # noqa: F401
+from .functional import (delta_rule, deltanet, gated_linear_attention, linear_attention, linear_scan,  # noqa: F401
                          normalised_linear_attention)
 
-__all__ = ["linear_scan", "linear_attention", "normalised_linear_attention", "gated_linear_attention", "delta_rule"]
+__all__ = ["linear_scan", "linear_attention", "normalised_linear_attention", "gated_linear_attention", "delta_rule", "deltanet"]

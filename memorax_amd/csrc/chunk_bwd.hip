@@ -99,19 +99,6 @@ struct NormBwdArgs {
     float eps;
 };
 
-// Sum over the SEGS consecutive lanes that share a tile row (8 or 16), by data-parallel
-// primitives; every lane of the group ends with the total.
-template <int SEGS> __device__ __forceinline__ float seg_sum(float x)
-{
-    static_assert(SEGS == 8 || SEGS == 16, "a row is 8 or 16 segments");
-    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
-    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
-    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xF, 0xF, true));  // row_half_mirror
-    if (SEGS == 16)
-        x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x140, 0xF, 0xF, true));  // row_mirror
-    return x;
-}
-
 // GATED: S_t = r_t exp(g_t) S_{t-1} + v_t k_t^T.  With G the cumulative log-decay inside the chunk
 // (per episode), a_i = exp(G_i), b_j = exp(G_last - G_j), c = exp(G_last), D_ij = exp(G_i - G_j):
 //   Aqk, dAqk carry the factor D;  dV = Aqk^T dO + diag(b) K dS^T;  dQ = diag(a) dO S + dAqk K;
@@ -508,10 +495,15 @@ template <typename T, int C, int NW> struct DeltaBwdSmem : BwdDims<T, C> {
                          oAqk = oDS + D::szDD, oTm = oAqk + D::szCC, oDT = oTm + D::szCC,
                          oBeta = oDT + D::szCC, oDb = oBeta + C * 4;
     static constexpr int NSLOT = TileMap<HD, C, NW>::WM;  // dbeta partials per row: one per feature block
-    static constexpr int total = oDb + NSLOT * C * 4;
+    // prologue variant: 1 / |k| per row, then [NSLOT][C] partials of k_n . dk_n
+    static constexpr int oKinv = oDb + NSLOT * C * 4;
+    static constexpr int total = oKinv + (1 + NSLOT) * C * 4;
 };
 
-template <typename T, int C, int NW>
+// PRO: the cell's prologue is part of the call -- k_n = k / max(|k|, 1e-12), beta = sigmoid(b) are
+// formed while staging (as in the forward kernel) and the gradients are taken back through them:
+//   dk = (dk_n - k_n (k_n . dk_n)) / |k| ,   db = dbeta beta (1 - beta).
+template <typename T, int C, int NW, bool PRO>
 __global__ void __launch_bounds__(64 * NW, sizeof(T) == 2 ? 2 : 1)
 delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
@@ -539,6 +531,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     T *sTm = at(L::oTm), *sDT = at(L::oDT);               // Tm[i][j], dTm[a][b]
     float *sBeta = reinterpret_cast<float *>(smem + L::oBeta);
     float *sDb = reinterpret_cast<float *>(smem + L::oDb);  // [NSLOT][C] dbeta partials
+    float *sKinv = reinterpret_cast<float *>(smem + L::oKinv);  // prologue: 1 / |k_row|
+    float *sKd = sKinv + C;                                      // prologue: [NSLOT][C] partials of k_n . dk_n
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -642,21 +636,41 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     IO::mask_rows(fv, tid, live);
                     IO::mask_rows(fdo, tid, live);
                 }
+                if (PRO) {
+                    float kinv[IO::PASSES];
+#pragma unroll
+                    for (int p = 0; p < IO::PASSES; ++p) {
+                        float ss = 0.f;
+#pragma unroll
+                        for (int e = 0; e < IO::KP; ++e) ss += (float)fk.v[p][e] * (float)fk.v[p][e];
+                        kinv[p] = 1.f / fmaxf(sqrtf(seg_sum<IO::SEGS>(ss)), 1e-12f);
+                        const int r = IO::row_of(tid, p);
+                        if (tid % IO::SEGS == 0 && (IO::FULL || r < C)) sKinv[r] = kinv[p];
+                    }
+                    IO::scale_rows(fk, kinv);
+                }
                 IO::to_lds(fq, sQ, LDD, tid);
                 IO::to_lds(fk, sK, LDD, tid);
                 IO::to_lds(fv, sV, LDD, tid);
                 IO::to_lds(fdo, sDO, LDD, tid);
                 float bf[IO::PASSES];
 #pragma unroll
-                for (int p = 0; p < IO::PASSES; ++p) bf[p] = raw_to_float<T>(rbrow[p]);
+                for (int p = 0; p < IO::PASSES; ++p)
+                    bf[p] = !live(IO::row_of(tid, p)) ? 0.f  // by select: a NaN gate of another episode must not meet a zeroed row
+                            : PRO ? sigmoidf(raw_to_float<T>(rbrow[p])) : raw_to_float<T>(rbrow[p]);
                 IO::scale_rows(fk, bf);
                 IO::to_lds(fk, sBK, LDD, tid);
                 typename IOS::Regs fS = rS;
                 if (pass != 0) IOS::zero(fS);
                 IOS::to_lds(fS, sS, LDD, tid);
-                IOT::to_lds(rTm, sTm, LDC, tid);  // Tm[i][j] from the forward call (block diagonal by episode)
+                // Tm[i][j] from the forward call (block diagonal by episode).  Rows of other episodes
+                // are cleared by select: they only ever meet zeros, but a NaN key or gate of another
+                // episode sits in them and must not meet those zeros.
+                typename IOT::Regs fTm = rTm;
+                if (nres != 0) IOT::mask_rows(fTm, tid, live);
+                IOT::to_lds(fTm, sTm, LDC, tid);
             }
-            if (tid < C) sBeta[tid] = live(tid) ? raw_to_float<T>(rbeta) : 0.f;
+            if (tid < C) sBeta[tid] = !live(tid) ? 0.f : PRO ? sigmoidf(raw_to_float<T>(rbeta)) : raw_to_float<T>(rbeta);
             if (pass != nres) zero_acc<TMS::TPW>(dSacc);
             store_acc<T, HD, HD, NW>(dSacc, sDS, LDD, w, lane);  // dS[dv][dk]
             sync_lds();
@@ -814,7 +828,32 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                 for (int j = 0; j < TMR::TPW; ++j) dKacc[j] += acc[j] * sBeta[TMR::nt(w, j) * 16 + li];
                 gemm<T, HD, C, C, KROW, KROW, NW>(dKacc, sBK, LDD, sDA, LDC, w, lane);
-                store_rows_at<T, C, NW>(dKacc, dk + goff, rs, t0, Tlen, w, lane, one, live);
+                if (!PRO) store_rows_at<T, C, NW>(dKacc, dk + goff, rs, t0, Tlen, w, lane, one, live);
+            }
+            // prologue: dKacc holds the gradient of the normalised keys; its component along k_n is
+            // removed once the row dots k_n . dk_n are summed over the feature blocks (after the barrier).
+            // The k_n values and 1 / |k| are taken into registers now: sK is restaged right after.
+            P4 kn[TMR::TPW];
+            float kiv[TMR::NBW];
+            if (PRO) {
+                float sp[TMR::NBW];
+#pragma unroll
+                for (int j = 0; j < TMR::NBW; ++j) sp[j] = 0.f;
+#pragma unroll
+                for (int j = 0; j < TMR::TPW; ++j) {
+                    const int d0 = TMR::mt(w, j) * 16 + 4 * lg, r = TMR::nt(w, j) * 16 + li;
+                    kn[j] = *reinterpret_cast<const P4 *>(sK + r * LDD + d0);
+                    sp[j % TMR::NBW] += dKacc[j][0] * (float)kn[j][0] + dKacc[j][1] * (float)kn[j][1] +
+                                        dKacc[j][2] * (float)kn[j][2] + dKacc[j][3] * (float)kn[j][3];
+                }
+#pragma unroll
+                for (int j = 0; j < TMR::NBW; ++j) {
+                    float x = sp[j];
+                    x += __shfl_xor(x, 16);
+                    x += __shfl_xor(x, 32);
+                    if (lg == 0) sKd[(w % TMR::WM) * C + TMR::nt(w, j) * 16 + li] = x;
+                    kiv[j] = sKinv[TMR::nt(w, j) * 16 + li];
+                }
             }
             // ---- dbeta: reduce the partials over lane groups, then over waves through LDS -----------
 #pragma unroll
@@ -826,13 +865,26 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();
             MRX_PHASE(23);
+            if (PRO) {
+#pragma unroll
+                for (int j = 0; j < TMR::TPW; ++j) {
+                    const int r = TMR::nt(w, j) * 16 + li;
+                    float sd = 0.f;
+#pragma unroll
+                    for (int sl = 0; sl < NSLOT; ++sl) sd += sKd[sl * C + r];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) dKacc[j][e] = (dKacc[j][e] - (float)kn[j][e] * sd) * kiv[j % TMR::NBW];
+                }
+                store_rows_at<T, C, NW>(dKacc, dk + goff, rs, t0, Tlen, w, lane, one, live);
+            }
             if (tid < C && t0 + tid < Tlen && live(tid)) {
                 float x = 0.f;
 #pragma unroll
                 for (int sl = 0; sl < NSLOT; ++sl) x += sDb[sl * C + tid];
+                if (PRO) x *= sBeta[tid] * (1.f - sBeta[tid]);
                 dbeta[dboff] = (T)x;
             }
-            MRX_PHASE(24);  // no barrier: sDb is not written again before the next pass's last phase
+            MRX_PHASE(24);  // no barrier: sDb, sKd are not written again before the next pass's last phase
         }
     }
     MRX_PHASE_FLUSH();
@@ -946,6 +998,46 @@ extern "C" int mrx_gated_linear_attn_bwd(void *stream, const void *q, const void
 #undef MRX_ARGS
 }
 
+namespace {
+
+template <typename T, int C, bool PRO>
+int launch_delta_bwd(hipStream_t st, const void *q, const void *k, const void *v, const void *beta,
+                     const void *done, int done_dtype, const void *S_chk, const void *Tm_chk, const void *dout,
+                     const void *dS_last, void *dq, void *dk_out, void *dv_out, void *dbeta, void *dS0, int64_t B,
+                     int64_t T_, int64_t H)
+{
+    constexpr int NW = 4;
+    auto kern = delta_bwd_kernel<T, C, NW, PRO>;
+    constexpr int smem = DeltaBwdSmem<T, C, NW>::total;
+    static unsigned long long lds_set = 0ull;
+    if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(64 * NW), smem, st, (const T *)q, (const T *)k,
+                       (const T *)v, (const T *)beta, done, done_dtype, (const T *)S_chk, (const T *)Tm_chk,
+                       (const T *)dout, (const float *)dS_last, (T *)dq, (T *)dk_out, (T *)dv_out, (T *)dbeta,
+                       (float *)dS0, (int)T_, (int)H);
+    return launch_status();
+}
+
+template <bool PRO>
+int delta_bwd_entry(void *stream, const void *q, const void *k, const void *v, const void *beta, const void *done,
+                    const void *S_chk, const void *Tm_chk, const void *dout, const void *dS_last, void *dq,
+                    void *dk_out, void *dv_out, void *dbeta, void *dS0, int64_t B, int64_t T, int64_t H,
+                    int64_t dk, int64_t dv, int dtype, int done_dtype)
+{
+    const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
+                             dv, dtype, done_dtype);
+    if (rc != MRX_OK) return rc;
+    if (!beta || !dbeta || !Tm_chk || !aligned(Tm_chk, 16)) return MRX_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == MRX_BF16)
+        return launch_delta_bwd<__bf16, DELTA_BF16_CHUNK, PRO>(st, q, k, v, beta, done, done_dtype, S_chk, Tm_chk, dout,
+                                                               dS_last, dq, dk_out, dv_out, dbeta, dS0, B, T, H);
+    return launch_delta_bwd<float, 32, PRO>(st, q, k, v, beta, done, done_dtype, S_chk, Tm_chk, dout, dS_last, dq,
+                                            dk_out, dv_out, dbeta, dS0, B, T, H);
+}
+
+}  // namespace
+
 extern "C" int mrx_delta_rule_bwd(void *stream, const void *q, const void *k, const void *v,
                                   const void *beta, const void *done, const void *S_chk,
                                   const void *Tm_chk, const void *dout, const void *dS_last, void *dq,
@@ -953,32 +1045,17 @@ extern "C" int mrx_delta_rule_bwd(void *stream, const void *q, const void *k, co
                                   int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                                   int done_dtype)
 {
-    const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
-                             dv, dtype, done_dtype);
-    if (rc != MRX_OK) return rc;
-    if (!beta || !dbeta || !Tm_chk || !aligned(Tm_chk, 16)) return MRX_ERR_INVALID_ARG;
-    hipStream_t st = (hipStream_t)stream;
-    constexpr int NW = 4;
-    if (dtype == MRX_BF16) {
-        auto kern = delta_bwd_kernel<__bf16, DELTA_BF16_CHUNK, NW>;
-        constexpr int smem = DeltaBwdSmem<__bf16, DELTA_BF16_CHUNK, NW>::total;
-        static unsigned long long lds_set = 0ull;
-        if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
-        hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(64 * NW), smem, st, (const __bf16 *)q,
-                           (const __bf16 *)k, (const __bf16 *)v, (const __bf16 *)beta, done, done_dtype,
-                           (const __bf16 *)S_chk, (const __bf16 *)Tm_chk, (const __bf16 *)dout,
-                           (const float *)dS_last, (__bf16 *)dq, (__bf16 *)dk_out, (__bf16 *)dv_out,
-                           (__bf16 *)dbeta, (float *)dS0, (int)T, (int)H);
-    } else {
-        auto kern = delta_bwd_kernel<float, 32, NW>;
-        constexpr int smem = DeltaBwdSmem<float, 32, NW>::total;
-        static unsigned long long lds_set = 0ull;
-        if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
-        hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(64 * NW), smem, st, (const float *)q,
-                           (const float *)k, (const float *)v, (const float *)beta, done, done_dtype,
-                           (const float *)S_chk, (const float *)Tm_chk, (const float *)dout,
-                           (const float *)dS_last, (float *)dq, (float *)dk_out, (float *)dv_out,
-                           (float *)dbeta, (float *)dS0, (int)T, (int)H);
-    }
-    return launch_status();
+    return delta_bwd_entry<false>(stream, q, k, v, beta, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out,
+                                  dbeta, dS0, B, T, H, dk, dv, dtype, done_dtype);
+}
+
+extern "C" int mrx_deltanet_bwd(void *stream, const void *q, const void *k, const void *v,
+                                const void *beta_raw, const void *done, const void *S_chk,
+                                const void *Tm_chk, const void *dout, const void *dS_last, void *dq,
+                                void *dk_out, void *dv_out, void *dbeta_raw, void *dS0, int64_t B,
+                                int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
+                                int done_dtype)
+{
+    return delta_bwd_entry<true>(stream, q, k, v, beta_raw, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out,
+                                 dbeta_raw, dS0, B, T, H, dk, dv, dtype, done_dtype);
 }

@@ -309,6 +309,21 @@ template <typename T, int R, int NTHR, int COLS = HD> struct TileIO {
     }
 };
 
+// Sum over the SEGS consecutive lanes that share a tile row (8 or 16), by data-parallel
+// primitives; every lane of the group ends with the total.
+template <int SEGS> __device__ __forceinline__ float seg_sum(float x)
+{
+    static_assert(SEGS == 8 || SEGS == 16, "a row is 8 or 16 segments");
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xF, 0xF, true));  // row_half_mirror
+    if (SEGS == 16)
+        x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x140, 0xF, 0xF, true));  // row_mirror
+    return x;
+}
+
+__device__ __forceinline__ float sigmoidf(float x) { return 1.f / (1.f + __expf(-x)); }
+
 // ---- per-chunk reset bookkeeping ------------------------------------------------
 // dmask has bit r set when row r of the chunk starts a new episode.  episode_of(r)
 // counts the resets at rows <= r; rows interact iff they have the same count.

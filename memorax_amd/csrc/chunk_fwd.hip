@@ -57,7 +57,9 @@ struct NormArgs {
     float eps;
 };
 
-template <typename T, int C, bool DELTA, bool FMAP, bool GATED, bool NORM>
+// PRO (delta rule): the cell's prologue runs on the staged rows -- keys are L2-normalised
+// (k / max(|k|, 1e-12), in fp32, then rounded to T) and beta = sigmoid(raw beta).
+template <typename T, int C, bool DELTA, bool FMAP, bool GATED, bool NORM, bool PRO = false>
 __global__ void __launch_bounds__(NTHR, 2)  // 2 waves per SIMD: two workgroups share a CU
 chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const float *__restrict__ glog,
@@ -67,6 +69,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 {
     static_assert(!(DELTA && GATED), "the gated variant is linear attention with a decay");
     static_assert(!NORM || (!DELTA && !GATED), "the normalised read-out belongs to plain linear attention");
+    static_assert(!PRO || DELTA, "the prologue belongs to the delta rule");
     using L = FwdSmem<T, C, DELTA, GATED, NORM>;
     using Frag = typename TT<T>::frag;
     using IO = TileIO<T, C, NTHR>;
@@ -213,6 +216,17 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     IO::mask_rows(fk, tid, live);
                     IO::mask_rows(fv, tid, live);
                 }
+                if (PRO) {
+                    float kinv[IO::PASSES];
+#pragma unroll
+                    for (int p = 0; p < IO::PASSES; ++p) {
+                        float ss = 0.f;
+#pragma unroll
+                        for (int e = 0; e < IO::KP; ++e) ss += (float)fk.v[p][e] * (float)fk.v[p][e];
+                        kinv[p] = 1.f / fmaxf(sqrtf(seg_sum<IO::SEGS>(ss)), 1e-12f);
+                    }
+                    IO::scale_rows(fk, kinv);
+                }
                 // rows past the end of the sequence: phi(0) = 1 must not count towards z
                 if (NORM && FMAP && t0 + C > Tlen) IO::mask_rows(fk, tid, [&](int r) { return t0 + r < Tlen; });
                 IO::to_lds(fq, sQ, LDD, tid);
@@ -220,14 +234,17 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 if (DELTA) {
                     float bf[IO::PASSES];
 #pragma unroll
-                    for (int p = 0; p < IO::PASSES; ++p) bf[p] = raw_to_float<T>(rbrow[p]);
+                    for (int p = 0; p < IO::PASSES; ++p)
+                        bf[p] = !live(IO::row_of(tid, p)) ? 0.f  // by select: a NaN gate of another episode must not meet a zeroed row
+                            : PRO ? sigmoidf(raw_to_float<T>(rbrow[p])) : raw_to_float<T>(rbrow[p]);
                     IO::scale_rows(fk, bf);
                     IO::scale_rows(fv, bf);
                     IO::to_lds(fk, sBK, LDD, tid);
                 }
                 IO::to_lds(fv, sV, LDD, tid);
             }
-            if (DELTA && tid < C) sBeta[tid] = live(tid) ? raw_to_float<T>(rbeta) : 0.f;
+            if (DELTA && tid < C)
+                sBeta[tid] = !live(tid) ? 0.f : PRO ? sigmoidf(raw_to_float<T>(rbeta)) : raw_to_float<T>(rbeta);
             if (pass != 0) zero_acc<TMS::TPW>(Sacc);  // an episode that starts in the chunk starts from 0
             store_acc<T, HD, HD, NW>(Sacc, sS, LDD, w, lane);  // sS[dv][dk]
             if (S_chk && pass == 0) {
@@ -413,12 +430,12 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     }
 }
 
-template <typename T, int C, bool DELTA, bool FMAP, bool GATED = false, bool NORM = false>
+template <typename T, int C, bool DELTA, bool FMAP, bool GATED = false, bool NORM = false, bool PRO = false>
 int launch(hipStream_t st, const void *q, const void *k, const void *v, const void *beta,
            const void *done, int done_f32, const void *S0, void *o, void *S_last, void *S_chk,
            void *Tm_chk, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr, NormArgs na = NormArgs{})
 {
-    auto kern = chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM>;
+    auto kern = chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO>;
     constexpr int smem = FwdSmem<T, C, DELTA, GATED, NORM>::total;
     static unsigned long long lds_set = 0ull;
     if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
@@ -520,4 +537,18 @@ extern "C" int mrx_linear_attn_norm_fwd(void *stream, const void *q, const void 
                   : launch<__bf16, LA_BF16_CHUNK, false, false, false, true>(MRX_ARGS);
     return fm ? launch<float, 32, false, true, false, true>(MRX_ARGS) : launch<float, 32, false, false, false, true>(MRX_ARGS);
 #undef MRX_ARGS
+}
+
+extern "C" int mrx_deltanet_fwd(void *stream, const void *q, const void *k, const void *v,
+                                const void *beta_raw, const void *done, const void *S0, void *o,
+                                void *S_last, void *S_chk, void *Tm_chk, int64_t B, int64_t T,
+                                int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype)
+{
+    const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
+    if (rc != MRX_OK) return rc;
+    if (!beta_raw || !aligned(Tm_chk, 16)) return MRX_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == MRX_BF16)
+        return launch<__bf16, DELTA_BF16_CHUNK, true, false, false, false, true>(st, q, k, v, beta_raw, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H);
+    return launch<float, 32, true, false, false, false, true>(st, q, k, v, beta_raw, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H);
 }

@@ -4,6 +4,7 @@ the role jax.custom_vjp would in a JAX host).
     linear_scan(a, b, done, h0=None, P0=None)            -> (h, h_last, P_last)
     linear_attention(q, k, v, done, S0=None, feature_map) -> (o, S_last)
     delta_rule(q, k, v, beta, done, S0=None)             -> (o, S_last)
+    deltanet(q, k, v, beta_raw, done, S0=None)           -> (o, S_last)   (key L2-norm and sigmoid fused)
 
 Layouts follow the reference: (B,T,D) / (B,T,H,d), state (B,H,d_v,d_k), done (B,T)
 bool or float where nonzero clears the carry before step t (memoroid.py:60-91).
@@ -224,18 +225,21 @@ def gated_linear_attention(q, k, v, g, done, S0=None, feature_map="none"):
 
 class _DeltaRule(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, beta, done, S0):
+    def forward(ctx, q, k, v, beta, done, S0, prologue=False):
         q_, k_, v_, b_ = q.contiguous(), k.contiguous(), v.contiguous(), beta.contiguous()
         S0_ = None if S0 is None else S0.contiguous().float()
         need = any(ctx.needs_input_grad)
+        ctx.done, ctx.has_S0, ctx.prologue = done, S0 is not None, prologue
         if q_.shape[1] == 1 and not need:  # acting: one step, no residuals
-            o, S_last = K.delta_rule_step(q_[:, 0], k_[:, 0], v_[:, 0], b_[:, 0], done[:, 0], S0_)
-            ctx.done, ctx.has_S0 = done, S0 is not None
+            k1, b1 = k_[:, 0], b_[:, 0]
+            if prologue:  # a (B,H,d) array: the prologue as array ops costs nothing here
+                k1 = torch.nn.functional.normalize(k1.float(), dim=-1).to(k_.dtype)
+                b1 = torch.sigmoid(b1.float()).to(b_.dtype)
+            o, S_last = K.delta_rule_step(q_[:, 0], k1, v_[:, 0], b1, done[:, 0], S0_)
             return o[:, None], S_last
-        o, S_last, chk = K.delta_rule_fwd(q_, k_, v_, b_, done, S0_, save_chk=need)
+        o, S_last, chk = K.delta_rule_fwd(q_, k_, v_, b_, done, S0_, save_chk=need, prologue=prologue)
         if need:
             ctx.save_for_backward(q_, k_, v_, b_, *chk)
-        ctx.done, ctx.has_S0 = done, S0 is not None
         return o, S_last
 
     @staticmethod
@@ -244,8 +248,8 @@ class _DeltaRule(torch.autograd.Function):
         do = torch.zeros_like(v) if do is None else do.contiguous()
         dS_last = None if dS_last is None else dS_last.contiguous().float()
         dq, dk, dv, db, dS0 = K.delta_rule_bwd(q, k, v, beta, ctx.done, (S_chk, Tm_chk), do, dS_last,
-                                               want_dS0=ctx.has_S0)
-        return dq, dk, dv, db, None, (dS0 if ctx.has_S0 else None)
+                                               want_dS0=ctx.has_S0, prologue=ctx.prologue)
+        return dq, dk, dv, db, None, (dS0 if ctx.has_S0 else None), None
 
 
 def delta_rule(q, k, v, beta, done, S0=None):
@@ -253,6 +257,15 @@ def delta_rule(q, k, v, beta, done, S0=None):
     o_t = S_t q_t, in chunked WY form.  Returns (o, S_last)."""
     hd = _Heads(q, v)
     o, S_last = _DeltaRule.apply(hd.qk(q), hd.qk(k), hd.v(v), hd.per_head(beta), done, hd.state_in(S0))
+    return hd.out(o), hd.state_out(S_last)
+
+
+def deltanet(q, k, v, beta_raw, done, S0=None):
+    """The DeltaNet cell's recurrence on its raw projections: delta_rule with
+    k / max(|k|, 1e-12) and sigmoid(beta_raw) formed inside the kernels (the normalised keys and
+    the gates never reach memory; gradients come back w.r.t. the raw arrays).  Returns (o, S_last)."""
+    hd = _Heads(q, v)   # zero-padding the keys leaves their norm unchanged
+    o, S_last = _DeltaRule.apply(hd.qk(q), hd.qk(k), hd.v(v), hd.per_head(beta_raw), done, hd.state_in(S0), True)
     return hd.out(o), hd.state_out(S_last)
 
 

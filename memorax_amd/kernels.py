@@ -226,10 +226,11 @@ def linear_attn_norm_bwd(q, k, v, done, chk, o, den, do, dS_last=None, dz_last=N
     return dq, dk_, dv_, dS0, dz0
 
 
-def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None):
+def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prologue=False):
     """Returns (o, S_last fp32, chk) where chk = (S_chk, Tm_chk) are the residuals the
     backward call needs, or None.  out = (o, S_last, S_chk, Tm_chk) reuses buffers of an earlier
-    call with the same shapes instead of allocating."""
+    call with the same shapes instead of allocating.  prologue=True: k is L2-normalised and
+    beta = sigmoid(beta) inside the kernel (mrx_deltanet_fwd)."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
     _chk(beta, "beta", dt, (B, T, H))
@@ -251,16 +252,18 @@ def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None):
             C, NC = chunk_size(dt, True), _n_chunks(T, dt, True)
             S_chk = torch.empty((B, H, NC, dv, dk), dtype=dt, device=q.device)
             Tm_chk = torch.empty((B, H, NC, C, C), dtype=dt, device=q.device)
-    st = lib.mrx_delta_rule_fwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done),
-                                _ptr(S0), _ptr(o), _ptr(S_last), _ptr(S_chk), _ptr(Tm_chk), B, T, H,
-                                dk, dv, _DT[dt], dd)
-    _lib.check(st, "mrx_delta_rule_fwd")
+    name = "mrx_deltanet_fwd" if prologue else "mrx_delta_rule_fwd"
+    st = getattr(lib, name)(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done),
+                            _ptr(S0), _ptr(o), _ptr(S_last), _ptr(S_chk), _ptr(Tm_chk), B, T, H,
+                            dk, dv, _DT[dt], dd)
+    _lib.check(st, name)
     return o, S_last, ((S_chk, Tm_chk) if save_chk else None)
 
 
-def delta_rule_bwd(q, k, v, beta, done, chk, do, dS_last=None, want_dS0=True, out=None):
+def delta_rule_bwd(q, k, v, beta, done, chk, do, dS_last=None, want_dS0=True, out=None, prologue=False):
     """chk = (S_chk, Tm_chk) from delta_rule_fwd.  Returns (dq, dk, dv, dbeta, dS0).
-    out = (dq, dk, dv, dbeta, dS0) reuses buffers instead of allocating."""
+    out = (dq, dk, dv, dbeta, dS0) reuses buffers instead of allocating.  prologue=True pairs with
+    delta_rule_fwd(prologue=True): k and beta are the raw projections and so are dk and dbeta."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
     S_chk, Tm_chk = chk
@@ -281,10 +284,11 @@ def delta_rule_bwd(q, k, v, beta, done, chk, do, dS_last=None, want_dS0=True, ou
         dbeta = torch.empty_like(beta)
         dS0 = (torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
                if want_dS0 else None)
-    st = lib.mrx_delta_rule_bwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done),
-                                _ptr(S_chk), _ptr(Tm_chk), _ptr(do), _ptr(dS_last), _ptr(dq), _ptr(dk_),
-                                _ptr(dv_), _ptr(dbeta), _ptr(dS0), B, T, H, dk, dv, _DT[dt], dd)
-    _lib.check(st, "mrx_delta_rule_bwd")
+    name = "mrx_deltanet_bwd" if prologue else "mrx_delta_rule_bwd"
+    st = getattr(lib, name)(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done),
+                            _ptr(S_chk), _ptr(Tm_chk), _ptr(do), _ptr(dS_last), _ptr(dq), _ptr(dk_),
+                            _ptr(dv_), _ptr(dbeta), _ptr(dS0), B, T, H, dk, dv, _DT[dt], dd)
+    _lib.check(st, name)
     return dq, dk_, dv_, dbeta, dS0
 
 

@@ -27,7 +27,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .functional import (delta_rule, gated_linear_attention, linear_attention, linear_scan,
+from .functional import (deltanet, gated_linear_attention, linear_attention, linear_scan,
                          normalised_linear_attention)
 
 
@@ -383,7 +383,7 @@ class LinearAttention(SequenceModel):
 
 class DeltaNetCell(MemoroidCellBase):
     """DeltaNet: S_t = S_{t-1}(I - beta_t k_t k_t^T) + beta_t v_t k_t^T, o_t = S_t q_t with
-    L2-normalised keys and beta = sigmoid(.).  Not in the reference; written in its cell
+    L2-normalised keys and beta = sigmoid(.) (both formed inside the kernels).  Not in the reference; written in its cell
     idiom the elements are the affine maps (beta v k^T, I - beta k k^T) with
     binary_operator(a, b) = (B_a A_b + B_b, A_a A_b).  The carry is (S (B,1,H,d,d),)."""
 
@@ -403,12 +403,11 @@ class DeltaNetCell(MemoroidCellBase):
         return x.view(*x.shape[:2], self.num_heads, self.head_dim)
 
     def forward(self, x, **kwargs):
-        q = self._heads(self.query(x))
-        k = F.normalize(self._heads(self.key(x)).float(), dim=-1)
-        v = self._heads(self.value(x))
-        beta = torch.sigmoid(self.beta(x).float())
+        """The raw projections (q, k, v, beta logits): the key normalisation and the sigmoid run
+        inside the kernels."""
         dt = self.dtype
-        return (q.to(dt), k.to(dt), v.to(dt), beta.to(dt))
+        return (self._heads(self.query(x)).to(dt), self._heads(self.key(x)).to(dt),
+                self._heads(self.value(x)).to(dt), self.beta(x).to(dt))
 
     def binary_operator(self, a, b):
         B_i, A_i = a
@@ -416,9 +415,9 @@ class DeltaNetCell(MemoroidCellBase):
         return (B_i @ A_j + B_j, A_i @ A_j)
 
     def scan(self, z, initial_carry, done):
-        q, k, v, beta = z
+        q, k, v, beta_raw = z
         (S0,) = initial_carry
-        o, S_last = delta_rule(q, k, v, beta, done, S0[:, 0].float())
+        o, S_last = deltanet(q, k, v, beta_raw, done, S0[:, 0].float())
         return o, (S_last[:, None],)
 
     def read(self, h, x, **kwargs):

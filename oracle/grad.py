@@ -171,6 +171,21 @@ def delta_rule_grads(q, k, v, beta, done, S0, do, dS_last=None):
                 dv=_np(v_.grad), dbeta=_np(b_.grad), dS0=_np(S0_.grad))
 
 
+def deltanet_grads(q, k, v, beta_raw, done, S0, do, dS_last=None):
+    """Returns dict(o, S_last, dq, dk, dv, dbeta, dS0) w.r.t. the raw k and beta_raw."""
+    q_, k_, v_, b_ = _t(q, True), _t(k, True), _t(v, True), _t(beta_raw, True)
+    B, T, H, dk = q_.shape
+    S0_ = _t(np.zeros((B, H, v_.shape[-1], dk)) if S0 is None else S0, True)
+    kn = k_ / torch.clamp(k_.norm(dim=-1, keepdim=True), min=1e-12)
+    o, Sl = delta_rule_t(q_, kn, v_, torch.sigmoid(b_), _done(done), S0_)
+    L = (o * _t(do)).sum()
+    if dS_last is not None:
+        L = L + (Sl * _t(dS_last)).sum()
+    L.backward()
+    return dict(o=_np(o), S_last=_np(Sl), dq=_np(q_.grad), dk=_np(k_.grad), dv=_np(v_.grad),
+                dbeta=_np(b_.grad), dS0=_np(S0_.grad))
+
+
 def gated_linear_attention_grads(q, k, v, g, done, S0, do, dS_last=None, feature_map="none"):
     """Returns dict(o, S_last, dq, dk, dv, dg, dS0) for L = sum(do*o) + sum(dS_last*S_last)."""
     q_, k_, v_, g_ = _t(q, True), _t(k, True), _t(v, True), _t(g, True)

@@ -357,6 +357,14 @@ def linear_attention_memoroid(q, k, v, done, carry=None, feature_map="none"):
     return nxt, num, den
 
 
+def deltanet(q, k, v, beta_raw, done, S0=None):
+    """DeltaNet cell on raw projections: delta_rule on k / max(|k|, 1e-12) and sigmoid(beta_raw)
+    (the prologue a cell in the idiom of memoroid.py:20-33 runs before it emits its elements)."""
+    k = np.asarray(k, dtype=np.float64)
+    kn = k / np.maximum(np.linalg.norm(k, axis=-1, keepdims=True), 1e-12)
+    return delta_rule(q, kn, v, sigmoid(np.asarray(beta_raw, dtype=np.float64)), done, S0)
+
+
 def normalised_linear_attention(q, k, v, done, S0=None, z0=None, feature_map="elu1", eps=1e-6):
     """Recurrent form of the cell with its read-out (linear_attention.py:62-86 for the
     elements, :93-110 for the read-out, scanned by memoroid.py:60-91):

@@ -94,7 +94,9 @@ def test_bwd_reset_isolation():
     for n in ("q", "k", "v", "beta"):
         x[n] = bf16_round(x[n])
     do = bf16_round(np.random.default_rng(2).standard_normal((B, T, H, 64)).astype(np.float32))
-    do[0, 150] = np.nan      # poison in the later episode
+    do[0, 150] = np.nan      # poison in the later episode: gradient, key and gate
+    x["k"][0, 120] = np.nan
+    x["beta"][0, 110] = np.nan
     bf = torch.bfloat16
     tq, tk, tv, tb, tdo = (dev(a, bf) for a in (x["q"], x["k"], x["v"], x["beta"], do))
     o, Sl, chk = K.delta_rule_fwd(tq, tk, tv, tb, dev(x["done"]))

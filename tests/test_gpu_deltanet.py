@@ -1,0 +1,125 @@
+"""GPU parity of the DeltaNet entry points with the prologue fused (key L2-normalisation and
+sigmoid gate inside the kernels) against the oracle composition and its torch-fp64 autograd."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import grad as G
+from oracle import memoroid as M
+from gpu_util import TOL_BF16, TOL_F32, bf16_round, dev, relerr
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(1, 64, 1), (2, 128, 2), (1, 1, 1), (2, 7, 1), (1, 65, 2), (2, 200, 3), (1, 33, 1)]
+
+
+def _raw_inputs(B, T, H, p, seed, dtype, d=64):
+    r = np.random.default_rng(seed)
+    x = dict(q=r.standard_normal((B, T, H, d)), v=r.standard_normal((B, T, H, d)),
+             k=r.standard_normal((B, T, H, d)) * np.exp(r.standard_normal((B, T, H, 1))),   # norms spread over a decade
+             beta=r.standard_normal((B, T, H)) * 1.5, do=r.standard_normal((B, T, H, d)),
+             S0=r.standard_normal((B, H, d, d)) * 0.1, dSl=r.standard_normal((B, H, d, d)) * 0.1)
+    x = {n: a.astype(np.float32) for n, a in x.items()}
+    x["done"] = r.random((B, T)) < p
+    if dtype == "bf16":
+        for n in ("q", "k", "v", "beta", "do"):
+            x[n] = bf16_round(x[n])
+    return x
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("p", [0.0, 0.05])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_deltanet_fwd_bwd(shape, p, dtype):
+    from memorax_amd import kernels as K
+    B, T, H = shape
+    x = _raw_inputs(B, T, H, p, B * 100 + T + H + 91, dtype)
+    print(f"case deltanet shape={shape} p={p} dtype={dtype}", flush=True)
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    tq, tk, tv, tb, tdo = (dev(x[n], td) for n in ("q", "k", "v", "beta", "do"))
+    dn = dev(x["done"])
+    o, Sl, chk = K.delta_rule_fwd(tq, tk, tv, tb, dn, dev(x["S0"]), prologue=True)
+    got = K.delta_rule_bwd(tq, tk, tv, tb, dn, chk, tdo, dev(x["dSl"]), prologue=True)
+    ref = G.deltanet_grads(x["q"], x["k"], x["v"], x["beta"], x["done"], x["S0"], x["do"], x["dSl"])
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    errs = {"o": relerr(o, ref["o"]), "S_last": relerr(Sl, ref["S_last"])}
+    errs.update({n: relerr(g, ref[n]) for n, g in zip(("dq", "dk", "dv", "dbeta", "dS0"), got)})
+    assert all(e <= tol for e in errs.values()), errs
+    # fp32: the prologue done by the caller and the plain entry points give the same numbers
+    if dtype == "f32":
+        kn = torch.nn.functional.normalize(tk, dim=-1)
+        o2, Sl2, _ = K.delta_rule_fwd(tq, kn, tv, torch.sigmoid(tb), dn, dev(x["S0"]))
+        assert relerr(o, o2.cpu().numpy()) <= 1e-5 and relerr(Sl, Sl2.cpu().numpy()) <= 1e-5
+
+
+def test_deltanet_key_gradient_is_orthogonal_to_the_key_at_the_benchmark_shape():
+    """Size-independent property at BASELINE configuration 4's shape: the output is invariant to
+    the scale of each key, so dk . k = 0 row by row (up to bf16 rounding of the two factors)."""
+    from memorax_amd import kernels as K
+    B, T, H = 64, 1024, 8
+    g = torch.Generator(device="cuda").manual_seed(3)
+    bf = torch.bfloat16
+    q, k, v, do = (torch.randn((B, T, H, 64), device="cuda", generator=g).to(bf) for _ in range(4))
+    k = (k.float() * torch.exp(torch.randn((B, T, H, 1), device="cuda", generator=g))).to(bf)
+    braw = torch.randn((B, T, H), device="cuda", generator=g).to(bf)
+    done = torch.rand((B, T), device="cuda", generator=g) < 0.002
+    o, Sl, chk = K.delta_rule_fwd(q, k, v, braw, done, None, prologue=True)
+    dq, dk, dv, db, _ = K.delta_rule_bwd(q, k, v, braw, done, chk, do, None, want_dS0=False, prologue=True)
+    assert all(torch.isfinite(t.float()).all() for t in (o, Sl, dq, dk, dv, db))
+    kf, dkf = k.float(), dk.float()
+    cos = (kf * dkf).sum(-1).abs() / (kf.norm(dim=-1) * dkf.norm(dim=-1) + 1e-30)
+    assert float(cos.max()) <= 2e-2, float(cos.max())
+    # scaling the keys by powers of two changes nothing at all
+    o2, Sl2, _ = K.delta_rule_fwd(q, (k.float() * 4).to(bf), v, braw, done, None, save_chk=False, prologue=True)
+    assert torch.equal(o, o2) and torch.equal(Sl, Sl2)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_deltanet_functional_autograd_rollout_and_other_head_dims(dtype):
+    from memorax_amd import functional as F
+    B, T, H, d = 2, 40, 2, 32
+    x = _raw_inputs(B, T, H, 0.05, 7, dtype, d=d)
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    q, k, v, b = (dev(x[n], td).requires_grad_() for n in ("q", "k", "v", "beta"))
+    S0 = dev(x["S0"]).requires_grad_()
+    o, Sl = F.deltanet(q, k, v, b, dev(x["done"]), S0)
+    ((o.float() * dev(x["do"])).sum() + (Sl * dev(x["dSl"])).sum()).backward()
+    ref = G.deltanet_grads(x["q"], x["k"], x["v"], x["beta"], x["done"], x["S0"], x["do"], x["dSl"])
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    errs = {"o": relerr(o, ref["o"]), "S_last": relerr(Sl, ref["S_last"])}
+    errs.update({n: relerr(t.grad, ref[n]) for n, t in (("dq", q), ("dk", k), ("dv", v), ("dbeta", b), ("dS0", S0))})
+    assert all(e <= tol for e in errs.values()), errs
+    # acting: T = 1 calls without gradients, state fed back
+    with torch.no_grad():
+        S, outs = S0.detach(), []
+        for t in range(T):
+            o1, S = F.deltanet(q[:, t:t + 1].detach(), k[:, t:t + 1].detach(), v[:, t:t + 1].detach(),
+                               b[:, t:t + 1].detach(), dev(x["done"])[:, t:t + 1], S)
+            outs.append(o1)
+    assert relerr(torch.cat(outs, 1), ref["o"]) <= tol and relerr(S, ref["S_last"]) <= tol
+
+
+def test_deltanet_poison_does_not_cross_episodes():
+    from memorax_amd import kernels as K
+    B, T, H = 1, 100, 1
+    x = _raw_inputs(B, T, H, 0.0, 13, "f32")
+    done = np.zeros((B, T), bool)
+    done[0, 40] = True
+    done[0, 70] = True
+    clean = {n: dev(x[n]) for n in ("q", "k", "v", "beta", "do")}
+    bad = {n: t.clone() for n, t in clean.items()}
+    for n in bad:
+        bad[n][0, 40:70] = float("nan")
+    outs = []
+    for inp in (clean, bad):
+        o, Sl, chk = K.delta_rule_fwd(inp["q"], inp["k"], inp["v"], inp["beta"], dev(done), dev(x["S0"]), prologue=True)
+        g = K.delta_rule_bwd(inp["q"], inp["k"], inp["v"], inp["beta"], dev(done), chk, inp["do"], dev(x["dSl"]),
+                             prologue=True)
+        outs.append((o, Sl) + tuple(g))
+    keep = np.ones(T, bool)
+    keep[40:70] = False
+    for name, a, b_ in zip(("o", "S_last", "dq", "dk", "dv", "dbeta", "dS0"), outs[0], outs[1]):
+        if a.dim() >= 3 and a.shape[1] == T:
+            a, b_ = a[:, keep], b_[:, keep]
+        bad_at = (a != b_).nonzero()
+        assert bad_at.numel() == 0, (name, bad_at[:4].tolist(), a[a != b_][:4].tolist(), b_[a != b_][:4].tolist())

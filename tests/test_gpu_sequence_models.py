@@ -101,8 +101,8 @@ def test_deltanet_stack_carries_and_split_invariance():
     # DeltaNet block alone against the oracle on its own projections
     cell = blocks[0].module.module.cell
     xn = blocks[0].module.norm(x)
-    qq, kk, vv, bb = (t.float() for t in cell(xn))
-    ro, rS = M.delta_rule(_np(qq), _np(kk), _np(vv), _np(bb), _np(done.float()))
+    qq, kk, vv, bb = (t.float() for t in cell(xn))   # raw projections: keys not normalised, gates as logits
+    ro, rS = M.deltanet(_np(qq), _np(kk), _np(vv), _np(bb), _np(done.float()))
     o, c = cell.scan(cell(xn), cell.initialize_carry(None, (B, Fe)), done)
     assert relerr(o, ro) <= 2e-2 and relerr(c[0][:, 0], rS) <= 2e-2
     # carry threading: two halves == one pass (bf16 kernel tolerance)

@@ -111,6 +111,38 @@ def test_normalised_linear_attention_grads_fd(eps):
         np.testing.assert_allclose(ag[name], fd(L, x), rtol=1e-5, atol=1e-7, err_msg=name)
 
 
+def test_deltanet_prologue_grads_fd_scale_invariance_and_orthogonality():
+    """The fused prologue (k / |k|, sigmoid(beta_raw)) in front of the delta rule: finite
+    differences; the output does not change when a key is rescaled, hence (Euler, degree 0)
+    every key's gradient is orthogonal to the key."""
+    r = np.random.default_rng(5)
+    B, T, H, dk, dv = 1, 7, 2, 3, 2
+    q, k, v = r.standard_normal((B, T, H, dk)), r.standard_normal((B, T, H, dk)) * 3, r.standard_normal((B, T, H, dv))
+    braw, S0 = r.standard_normal((B, T, H)), r.standard_normal((B, H, dv, dk))
+    do, dSl = r.standard_normal((B, T, H, dv)), r.standard_normal((B, H, dv, dk))
+    d = np.zeros((B, T), bool)
+    d[0, 4] = True
+
+    def L():
+        o, Sl = M.deltanet(q, k, v, braw, d, S0)
+        return (o * do).sum() + (Sl * dSl).sum()
+
+    ag = G.deltanet_grads(q, k, v, braw, d, S0, do, dSl)
+    for name, x in (("dq", q), ("dk", k), ("dv", v), ("dbeta", braw), ("dS0", S0)):
+        np.testing.assert_allclose(ag[name], fd(L, x), rtol=1e-5, atol=1e-7, err_msg=name)
+    o, Sl = M.deltanet(q, k, v, braw, d, S0)
+    np.testing.assert_allclose(ag["o"], o, rtol=1e-12)
+    scale = np.exp(r.standard_normal((B, T, H, 1)))
+    o2, Sl2 = M.deltanet(q, k * scale, v, braw, d, S0)
+    np.testing.assert_allclose(o2, o, rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(Sl2, Sl, rtol=1e-10, atol=1e-12)
+    assert np.abs((ag["dk"] * k).sum(-1)).max() <= 1e-10 * np.abs(ag["dk"]).max() * np.abs(k).max()
+    # on unit keys and gates given as logits it is the plain delta rule
+    kn = k / np.linalg.norm(k, axis=-1, keepdims=True)
+    o3, Sl3 = M.delta_rule(q, kn, v, M.sigmoid(braw), d, S0)
+    np.testing.assert_allclose(o3, o, rtol=1e-12, atol=1e-12)
+
+
 def test_delta_rule_grads_fd():
     B, T, H, dk, dv = 1, 7, 1, 3, 2
     q, k, v, S0 = rnd(B, T, H, dk), rnd(B, T, H, dk), rnd(B, T, H, dv), rnd(B, H, dv, dk)
