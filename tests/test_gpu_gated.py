@@ -106,3 +106,34 @@ def test_gated_autograd_function_and_split_invariance():
         o2, S2 = gated_linear_attention(q[:, 40:], k[:, 40:], v[:, 40:], g[:, 40:], dn[:, 40:], S1, "elu1")
     assert relerr(torch.cat([o1, o2], 1), o.detach().cpu().numpy()) <= TOL_F32
     assert relerr(S2, Sl.detach().cpu().numpy()) <= TOL_F32
+
+
+def test_gated_poison_does_not_cross_episodes():
+    """NaN in one episode (inputs, log-decays, output gradient) leaves every other episode's
+    outputs and gradients bit-identical, including dg (reverse reset-aware sum of the row dots)."""
+    from memorax_amd import kernels as K
+    B, T, H = 1, 200, 2
+    x = attn_inputs(B, T, H, p=0.0, seed=17, scale=1.0 / 8)
+    rng = np.random.default_rng(18)
+    g = (-np.abs(rng.standard_normal((B, T, H))) * 0.1).astype(np.float32)
+    do = rng.standard_normal((B, T, H, 64)).astype(np.float32)
+    dSl = (rng.standard_normal((B, H, 64, 64)) * 0.1).astype(np.float32)
+    done = np.zeros((B, T), bool)
+    done[0, 70] = True
+    done[0, 130] = True
+    clean = dict(q=dev(x["q"]), k=dev(x["k"]), v=dev(x["v"]), g=dev(g), do=dev(do))
+    bad = {n: t.clone() for n, t in clean.items()}
+    for n in bad:
+        bad[n][0, 70:130] = float("nan")
+    outs = []
+    for inp in (clean, bad):
+        o, Sl, chk = K.gated_linear_attn_fwd(inp["q"], inp["k"], inp["v"], inp["g"], dev(done), dev(x["S0"]), 1)
+        gr = K.gated_linear_attn_bwd(inp["q"], inp["k"], inp["v"], inp["g"], dev(done), chk, inp["do"], dev(dSl), 1,
+                                     S_last=Sl)
+        outs.append((o, Sl) + tuple(gr))
+    keep = np.ones(T, bool)
+    keep[70:130] = False
+    for name, a, b_ in zip(("o", "S_last", "dq", "dk", "dv", "dg", "dS0"), outs[0], outs[1]):
+        if a.dim() >= 3 and a.shape[1] == T:
+            a, b_ = a[:, keep], b_[:, keep]
+        assert torch.equal(a, b_), name
