@@ -75,6 +75,25 @@ __device__ __forceinline__ void store_rows_at(const f32x4 *acc, T *row, int64_t 
     }
 }
 
+// Rows of an LDS tile [C][64] to a (B,T,H,64) array, 16 bytes per thread: eight (sixteen) threads
+// write one whole row, so a wave instruction covers full 128-byte lines -- against the four-feature
+// pieces (16 rows x 32 bytes per instruction) of a store from accumulators.  `g` points at row 0 of
+// the chunk.
+template <typename T, int C, int NTHR, typename KeepF>
+__device__ __forceinline__ void tile_rows_to_global(const T *tile, int ld, T *g, int64_t rs, int t0, int Tlen, int tid,
+                                                    KeepF keep)
+{
+    using IO = TileIO<T, C, NTHR>;
+    const int seg = tid % IO::SEGS;
+#pragma unroll
+    for (int p = 0; p < IO::PASSES; ++p) {
+        const int r = IO::row_of(tid, p);
+        if ((IO::FULL || r < C) && t0 + r < Tlen && keep(r))
+            *reinterpret_cast<typename IO::F *>(g + (int64_t)r * rs + seg * IO::KP) =
+                *reinterpret_cast<const typename IO::F *>(tile + r * ld + seg * IO::KP);
+    }
+}
+
 // =====================================================================================
 // linear attention: 8 tiles, two workgroups per CU
 // =====================================================================================
@@ -616,12 +635,32 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     };
 #pragma unroll
     for (int part = 0; part < 6; ++part) prefetch_part(part);
-    // stores: row li of the chunk, this lane's 4 features (tile offsets are added per tile)
-    int64_t goff = base + (int64_t)(tlast + li) * rs + 4 * lg;
     int64_t dboff = ((int64_t)b * Tlen + tlast + tid) * H + h;
     MRX_PHASE_INIT();
 
-    for (int c = NC - 1; c >= 0; --c, goff -= (int64_t)C * rs, dboff -= (int64_t)C * H) {
+    // Gradients leave through LDS: an accumulator tile holds four features of sixteen rows per lane
+    // group, so a store from accumulators writes 16 pieces of 32 bytes per instruction; written to a
+    // dead LDS tile first (dV is there anyway) and read back row-wise, every instruction writes whole
+    // 128-byte rows (measured: the three stores from accumulators cost a third of the kernel).
+    // dK is complete only in a pass's last phase; it waits in sU -- not written again before the
+    // next pass's second phase -- and goes to memory after the next pass has been staged, so that no
+    // store is issued right before the wait for the prefetched loads.  dbeta waits in a register.
+    unsigned long long pend_dmask = 0ull;
+    int pend_nres = 0, pend_pass = 0, pend_t0 = -1;
+    int64_t pend_dboff = 0;
+    float pend_db = 0.f;
+    bool pend_db_on = false;
+    auto flush_pending = [&]() {  // call after a barrier that follows the writes to sU
+        if (pend_t0 >= 0) {
+            auto keep = [&](int r) { return pend_nres == 0 || episode_of(pend_dmask, r) == pend_pass; };
+            tile_rows_to_global<T, C, NTHR>(sU, LDD, dk + base + (int64_t)pend_t0 * rs, rs, pend_t0, Tlen, tid, keep);
+        }
+        if (pend_db_on) dbeta[pend_dboff] = (T)pend_db;
+        pend_t0 = -1;
+        pend_db_on = false;
+    };
+
+    for (int c = NC - 1; c >= 0; --c, dboff -= (int64_t)C * H) {
         const int t0 = c * C;
         const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
@@ -675,6 +714,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             store_acc<T, HD, HD, NW>(dSacc, sDS, LDD, w, lane);  // dS[dv][dk]
             sync_lds();
             MRX_PHASE(11);
+            flush_pending();
             const bool pre = pass == 0 && c > 0;
             if (pre) prefetch_part(0);
 
@@ -739,7 +779,6 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                                          acc[j][3] * (float)x[3];
                 }
             };
-            auto one = [](int, int) { return f32x4{1.f, 1.f, 1.f, 1.f}; };
             // ---- dAqk[i][j] = do_i . u'_j, j <= i -> sDAqk (over sAqk) ------------------------------
             {
                 f32x4 acc[TMA::TPW];
@@ -755,8 +794,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 rowdot(acc, sV);
 #pragma unroll
                 for (int j = 0; j < TMR::TPW; ++j) acc[j] *= sBeta[TMR::nt(w, j) * 16 + li];
-                store_acc<T, HD, C, NW>(acc, sZb, LDD, w, lane);
-                store_rows_at<T, C, NW>(acc, dv + goff, rs, t0, Tlen, w, lane, one, live);
+                store_acc<T, HD, C, NW>(acc, sZb, LDD, w, lane);  // = dV, written to memory from here after the barrier
             }
             // ---- dTm[a][b] = du'_a . v~_b, b <= a : D[m = b][n = a] -> sDT[a][b] ---------------------
             {
@@ -768,13 +806,14 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             sync_lds();  // sDAqk, sZb, sDT visible; sVt dead
             MRX_PHASE(17);
             if (pre) prefetch_part(3);
+            tile_rows_to_global<T, C, NTHR>(sZb, LDD, dv + base + (int64_t)t0 * rs, rs, t0, Tlen, tid, live);
             // ---- dQ^T[dk][i] = sum_dv S[dv][dk] dO[i][dv] + sum_j K[j][dk] dAqk[i][j] -> global ----
             {
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
                 gemm<T, HD, C, HD, KROW, ROWK, NW>(acc, sS, LDD, sDO, LDD, w, lane);
                 gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sK, LDD, sDAqk, LDC, w, lane);
-                store_rows_at<T, C, NW>(acc, dq + goff, rs, t0, Tlen, w, lane, one, live);
+                store_acc<T, HD, C, NW>(acc, sDU, LDD, w, lane);  // dU' is dead; to memory after the barrier
             }
             // ---- dK^T[dk][j] = sum_i Q[i][dk] dAqk[i][j] + sum_dv dS[dv][dk] U'[j][dv]
             //                    - sum_dv S[dv][dk] (beta Z)[j][dv]   (kept in registers) ---------------
@@ -808,6 +847,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             sync_lds();  // sY1 visible; sQ, sDO, sS, sDS, sDAqk, sZb dead
             MRX_PHASE(20);
             if (pre) prefetch_part(4);
+            tile_rows_to_global<T, C, NTHR>(sDU, LDD, dq + base + (int64_t)t0 * rs, rs, t0, Tlen, tid, live);
             // ---- dA[i][j] = -sum_b Y1[i][b] Tm[j][b], j < i : D[m = j][n = i] -> sDA[i][j] (over sS) ----
             {
                 f32x4 acc[TMA::TPW];
@@ -828,7 +868,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                 for (int j = 0; j < TMR::TPW; ++j) dKacc[j] += acc[j] * sBeta[TMR::nt(w, j) * 16 + li];
                 gemm<T, HD, C, C, KROW, KROW, NW>(dKacc, sBK, LDD, sDA, LDC, w, lane);
-                if (!PRO) store_rows_at<T, C, NW>(dKacc, dk + goff, rs, t0, Tlen, w, lane, one, live);
+                if (!PRO) store_acc<T, HD, C, NW>(dKacc, sU, LDD, w, lane);
             }
             // prologue: dKacc holds the gradient of the normalised keys; its component along k_n is
             // removed once the row dots k_n . dk_n are summed over the feature blocks (after the barrier).
@@ -875,18 +915,26 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                     for (int e = 0; e < 4; ++e) dKacc[j][e] = (dKacc[j][e] - (float)kn[j][e] * sd) * kiv[j % TMR::NBW];
                 }
-                store_rows_at<T, C, NW>(dKacc, dk + goff, rs, t0, Tlen, w, lane, one, live);
+                store_acc<T, HD, C, NW>(dKacc, sU, LDD, w, lane);
             }
+            pend_dmask = dmask;
+            pend_nres = nres;
+            pend_pass = pass;
+            pend_t0 = t0;
             if (tid < C && t0 + tid < Tlen && live(tid)) {
                 float x = 0.f;
 #pragma unroll
                 for (int sl = 0; sl < NSLOT; ++sl) x += sDb[sl * C + tid];
                 if (PRO) x *= sBeta[tid] * (1.f - sBeta[tid]);
-                dbeta[dboff] = (T)x;
+                pend_db = x;
+                pend_dboff = dboff;
+                pend_db_on = true;
             }
             MRX_PHASE(24);  // no barrier: sDb, sKd are not written again before the next pass's last phase
         }
     }
+    sync_lds();
+    flush_pending();
     MRX_PHASE_FLUSH();
     if (dS0) {
 #pragma unroll
