@@ -75,25 +75,6 @@ __device__ __forceinline__ void store_rows_at(const f32x4 *acc, T *row, int64_t 
     }
 }
 
-// Rows of an LDS tile [C][64] to a (B,T,H,64) array, 16 bytes per thread: eight (sixteen) threads
-// write one whole row, so a wave instruction covers full 128-byte lines -- against the four-feature
-// pieces (16 rows x 32 bytes per instruction) of a store from accumulators.  `g` points at row 0 of
-// the chunk.
-template <typename T, int C, int NTHR, typename KeepF>
-__device__ __forceinline__ void tile_rows_to_global(const T *tile, int ld, T *g, int64_t rs, int t0, int Tlen, int tid,
-                                                    KeepF keep)
-{
-    using IO = TileIO<T, C, NTHR>;
-    const int seg = tid % IO::SEGS;
-#pragma unroll
-    for (int p = 0; p < IO::PASSES; ++p) {
-        const int r = IO::row_of(tid, p);
-        if ((IO::FULL || r < C) && t0 + r < Tlen && keep(r))
-            *reinterpret_cast<typename IO::F *>(g + (int64_t)r * rs + seg * IO::KP) =
-                *reinterpret_cast<const typename IO::F *>(tile + r * ld + seg * IO::KP);
-    }
-}
-
 // =====================================================================================
 // linear attention: 8 tiles, two workgroups per CU
 // =====================================================================================

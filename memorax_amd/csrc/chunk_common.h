@@ -324,6 +324,25 @@ template <int SEGS> __device__ __forceinline__ float seg_sum(float x)
 
 __device__ __forceinline__ float sigmoidf(float x) { return 1.f / (1.f + __expf(-x)); }
 
+// Rows of an LDS tile [C][64] to a (B,T,H,64) array, 16 bytes per thread: eight (sixteen) threads
+// write one whole row, so a wave instruction covers full 128-byte lines -- against the four-feature
+// pieces (16 rows x 32 bytes per instruction) of a store from accumulators.  `g` points at row 0 of
+// the chunk.
+template <typename T, int C, int NTHR, typename KeepF>
+__device__ __forceinline__ void tile_rows_to_global(const T *tile, int ld, T *g, int64_t rs, int t0, int Tlen, int tid,
+                                                    KeepF keep)
+{
+    using IO = TileIO<T, C, NTHR>;
+    const int seg = tid % IO::SEGS;
+#pragma unroll
+    for (int p = 0; p < IO::PASSES; ++p) {
+        const int r = IO::row_of(tid, p);
+        if ((IO::FULL || r < C) && t0 + r < Tlen && keep(r))
+            *reinterpret_cast<typename IO::F *>(g + (int64_t)r * rs + seg * IO::KP) =
+                *reinterpret_cast<const typename IO::F *>(tile + r * ld + seg * IO::KP);
+    }
+}
+
 // ---- per-chunk reset bookkeeping ------------------------------------------------
 // dmask has bit r set when row r of the chunk starts a new episode.  episode_of(r)
 // counts the resets at rows <= r; rows interact iff they have the same count.

@@ -45,7 +45,8 @@ template <typename T, int C, bool DELTA, bool GATED = false, bool NORM = false> 
     static constexpr int oBeta = oA + szRA;
     static constexpr int oG = oBeta + C * 4;              // gated: cumulative log-decay G of the chunk rows, then exp(G_last - G)
     static constexpr int oZ = oG + 2 * C * 4;             // z entering the pass, T-typed row of 64 (normalised read-out)
-    static constexpr int total = oZ + (NORM ? HD * (int)sizeof(T) : 0);
+    static constexpr int oO = oZ + (NORM ? HD * (int)sizeof(T) : 0);  // O [C][dv] on its way to memory
+    static constexpr int total = oO + szRD;
 };
 
 // What the normalised read-out adds to the argument list.
@@ -90,6 +91,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     float *sG = reinterpret_cast<float *>(smem + L::oG);
     float *sEb = sG + C;                             // gated: b_j = exp(G_last - G_j)
     T *sZ = reinterpret_cast<T *>(smem + L::oZ);
+    T *sO = reinterpret_cast<T *>(smem + L::oO);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -181,10 +183,18 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 
     static_assert(C * C / 4 % NTHR == 0, "Tm tile copy assumes whole passes");
     // running element offsets of this thread's stores, advanced by one chunk per iteration
-    int64_t o_off = base + (int64_t)li * rs + 4 * lg;                               // o[t0 + li][4 lg..]
-    int64_t schk_off = (int64_t)bh * NC * HD * HD + li * HD + 4 * lg;                // S_chk[c][li][4 lg..]
+    unsigned long long pend_dmask = 0ull;  // the unit whose output waits in sO
+    int pend_nres = 0, pend_pass = 0, pend_t0 = -1;
+    auto flush_o = [&]() {  // call after a barrier that follows the writes to sO
+        if (pend_t0 >= 0) {
+            auto keep = [&](int r) { return pend_nres == 0 || episode_of(pend_dmask, r) == pend_pass; };
+            tile_rows_to_global<T, C, NTHR>(sO, LDD, o + base + (int64_t)pend_t0 * rs, rs, pend_t0, Tlen, tid, keep);
+        }
+        pend_t0 = -1;
+    };
+    int64_t schk_off = (int64_t)bh * NC * HD * HD;                                   // S_chk[c]
     int64_t tmchk_off = (int64_t)bh * NC * C * C + (int64_t)tid * 4;                                  // row-major C x C
-    for (int c = 0; c < NC; ++c, o_off += (int64_t)C * rs, schk_off += HD * HD, tmchk_off += C * C, den_off += (int64_t)C * H) {
+    for (int c = 0; c < NC; ++c, schk_off += HD * HD, tmchk_off += C * C, den_off += (int64_t)C * H) {
         const int t0 = c * C;
         const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
@@ -247,12 +257,6 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 sBeta[tid] = !live(tid) ? 0.f : PRO ? sigmoidf(raw_to_float<T>(rbeta)) : raw_to_float<T>(rbeta);
             if (pass != 0) zero_acc<TMS::TPW>(Sacc);  // an episode that starts in the chunk starts from 0
             store_acc<T, HD, HD, NW>(Sacc, sS, LDD, w, lane);  // sS[dv][dk]
-            if (S_chk && pass == 0) {
-#pragma unroll
-                for (int j = 0; j < TMS::TPW; ++j)
-                    *reinterpret_cast<P4 *>(S_chk + schk_off + TMS::nt(w, j) * 16 * HD + TMS::mt(w, j) * 16) =
-                        TT<T>::pack(Sacc[j][0], Sacc[j][1], Sacc[j][2], Sacc[j][3]);
-            }
             if (NORM) {
                 if (pass != 0) zero_acc<TMS::MBW>(zacc);
                 if (w < TMS::WM && li == 0) {
@@ -267,6 +271,19 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();
             MRX_PHASE(1);
+            // Outputs leave through LDS as whole rows (an accumulator tile would write 16 pieces of
+            // 32 bytes per instruction): the output of the previous unit, parked in sO at its end, and
+            // the state checkpoint from the copy of S that has just been staged.
+            flush_o();
+            if (S_chk && pass == 0) {
+                using IOS = TileIO<T, HD, NTHR>;
+#pragma unroll
+                for (int p = 0; p < IOS::PASSES; ++p) {
+                    const int r = IOS::row_of(tid, p), seg = tid % IOS::SEGS;
+                    *reinterpret_cast<typename IOS::F *>(S_chk + schk_off + r * HD + seg * IOS::KP) =
+                        *reinterpret_cast<const typename IOS::F *>(sS + r * LDD + seg * IOS::KP);
+                }
+            }
             const bool pre = pass == nres && c + 1 < NC;
             if (pre) prefetch_part(0);
             if (!DELTA && pre) prefetch_part(1);
@@ -379,19 +396,21 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 for (int j = 0; j < TMO::TPW; ++j) Oacc[j] *= __expf(sG[TMO::nt(w, j) * 16 + li]);
             }
             gemm<T, HD, C, C, KROW, ROWK, NW>(Oacc, sU, LDD, sAqk, LDC, w, lane, NoHook(), den_a);
+            if (NORM) {
 #pragma unroll
-            for (int j = 0; j < TMO::TPW; ++j) {
-                const int cc = TMO::nt(w, j) * 16 + li;
-                if (t0 + cc < Tlen && live(cc)) {
-                    if (NORM) {
-                        const float den = fmaxf(dacc[j % TMO::NBW][0], na.eps);
-                        Oacc[j] *= 1.f / den;
-                        if (TMO::mt(w, j) == 0 && lg == 0) na.den[den_off + (int64_t)(TMO::nt(w, j) * 16) * H] = den;
-                    }
-                    *reinterpret_cast<P4 *>(o + o_off + (int64_t)(TMO::nt(w, j) * 16) * rs + TMO::mt(w, j) * 16) =
-                        TT<T>::pack(Oacc[j][0], Oacc[j][1], Oacc[j][2], Oacc[j][3]);
+                for (int j = 0; j < TMO::TPW; ++j) {
+                    const int cc = TMO::nt(w, j) * 16 + li;
+                    const float den = fmaxf(dacc[j % TMO::NBW][0], na.eps);
+                    Oacc[j] *= 1.f / den;
+                    if (t0 + cc < Tlen && live(cc) && TMO::mt(w, j) == 0 && lg == 0)
+                        na.den[den_off + (int64_t)(TMO::nt(w, j) * 16) * H] = den;
                 }
             }
+            store_acc<T, HD, C, NW>(Oacc, sO, LDD, w, lane);  // to memory once the next unit has been staged
+            pend_dmask = dmask;
+            pend_nres = nres;
+            pend_pass = pass;
+            pend_t0 = t0;
             // ---- S^T[dk][dv] += sum_c K[c][dk] U'[c][dv]  (only the episode that leaves the chunk)
             if (pass == nres) {
                 if (GATED) {  // S <- exp(G_last) S + sum_c exp(G_last - G_c) K[c] U'[c]
@@ -413,6 +432,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             MRX_PHASE(8);
         }
     }
+    flush_o();  // the last unit ended with a barrier
     MRX_WG_END();
     MRX_PHASE_FLUSH();
 
