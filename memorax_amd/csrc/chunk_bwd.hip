@@ -240,6 +240,37 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 #pragma unroll
     for (int part = 0; part < 3; ++part) prefetch_part(part);
 
+    // Gradients leave through LDS as whole rows (a store from accumulators writes 16 pieces of 32 bytes
+    // per instruction): at the end of a pass, once every product has read its operands, dV, dQ, dK are
+    // written over V, Q, K; the next pass reads them back row-wise -- each thread exactly the 16 bytes it
+    // is about to restage, so no barrier is needed in between -- after it has consumed its prefetched
+    // registers (the wait for those then does not cover these stores).
+    unsigned long long pend_dmask = 0ull;
+    int pend_nres = 0, pend_pass = 0, pend_t0 = -1;
+    auto flush_pending = [&]() {
+        if (pend_t0 >= 0) {
+            auto keep = [&](int r) { return pend_nres == 0 || episode_of(pend_dmask, r) == pend_pass; };
+            const int64_t off = base + (int64_t)pend_t0 * rs;
+            tile_rows_to_global<T, C, NTHR>(sV, LDD, dv + off, rs, pend_t0, Tlen, tid, keep);
+            tile_rows_to_global<T, C, NTHR>(sQ, LDD, dq + off, rs, pend_t0, Tlen, tid, keep);
+            tile_rows_to_global<T, C, NTHR>(sK, LDD, dk + off, rs, pend_t0, Tlen, tid, keep);
+        }
+        pend_t0 = -1;
+    };
+    P4 hV[TMR::TPW], hQ[TMR::TPW], hK[TMR::TPW];  // the three gradients of a pass, rounded, until its operands are dead
+    auto hold = [&](const f32x4 *acc, P4 *h, auto scale) {
+#pragma unroll
+        for (int j = 0; j < TMR::TPW; ++j) {
+            const f32x4 sc = scale(TMR::nt(w, j) * 16 + li, TMR::mt(w, j) * 16 + 4 * lg);
+            h[j] = TT<T>::pack(acc[j][0] * sc[0], acc[j][1] * sc[1], acc[j][2] * sc[2], acc[j][3] * sc[3]);
+        }
+    };
+    auto park = [&](const P4 *h, T *dst) {
+#pragma unroll
+        for (int j = 0; j < TMR::TPW; ++j)
+            *reinterpret_cast<P4 *>(dst + (TMR::nt(w, j) * 16 + li) * LDD + TMR::mt(w, j) * 16 + 4 * lg) = h[j];
+    };
+
     for (int c = NC - 1; c >= 0; --c) {
         const int t0 = c * C;
         const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
@@ -293,6 +324,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     IO::scale_rows(fdo, inv);
                     if (tid < 16) *reinterpret_cast<f32x4 *>(sZf + 4 * tid) = rz;
                 }
+                flush_pending();  // reads what this thread is about to overwrite in sV, sQ, sK
                 IO::to_lds(fq, sQ, LDD, tid);
                 IO::to_lds(fk, sK, LDD, tid);
                 IO::to_lds(fv, sV, LDD, tid);
@@ -372,7 +404,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     gemm<T, HD, C, C, KROW, KROW, NW>(acc, sDO, LDD, sAqk, LDC, w, lane);
                     gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc, sDS, LDD, sK, LDD, w, lane);
                 }
-                store_rows_global<T, C, NW>(acc, dv + base, rs, t0, Tlen, w, lane, one, live);
+                hold(acc, hV, one);
             }
             if (pre) prefetch_part(2);
             // ---- dQ^T[dk][i] = sum_dv S[dv][dk] dO[i][dv] + sum_j K[j][dk] dAqk[i][j] ---------
@@ -398,7 +430,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     return f32x4{fmap_grad<FMAP>((float)x[0]), fmap_grad<FMAP>((float)x[1]),
                                  fmap_grad<FMAP>((float)x[2]), fmap_grad<FMAP>((float)x[3])};
                 };
-                store_rows_global<T, C, NW>(acc, dq + base, rs, t0, Tlen, w, lane, sc, live);
+                hold(acc, hQ, sc);
             }
             // ---- dK^T[dk][j] = sum_i Q[i][dk] dAqk[i][j] + sum_dv dS[dv][dk] V[j][dv] -----------
             {
@@ -424,7 +456,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     return f32x4{fmap_grad<FMAP>((float)x[0]), fmap_grad<FMAP>((float)x[1]),
                                  fmap_grad<FMAP>((float)x[2]), fmap_grad<FMAP>((float)x[3])};
                 };
-                store_rows_global<T, C, NW>(acc, dk + base, rs, t0, Tlen, w, lane, sc, live);
+                hold(acc, hK, sc);
             }
             // ---- dS^T[dk][dv] += sum_c Q[c][dk] dO[c][dv]  (gated: c dS + sum_c a_c Q[c] dO[c]) -----
             if (GATED) {
@@ -449,6 +481,14 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 }
             };
             gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, sQ, LDD, sDO, LDD, w, lane, dz_q);
+            sync_lds();  // every product has read its operands
+            park(hV, sV);
+            park(hQ, sQ);
+            park(hK, sK);
+            pend_dmask = dmask;
+            pend_nres = nres;
+            pend_pass = pass;
+            pend_t0 = t0;
             sync_lds();
             if (GATED && tid < C && t0 + tid < Tlen && live(tid)) {
                 float x = 0.f;
@@ -458,6 +498,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             }
         }
     }
+    flush_pending();  // the last pass ended with a barrier
     if (dS0) {
 #pragma unroll
         for (int j = 0; j < TMS::TPW; ++j) {
