@@ -15,7 +15,8 @@
 //   dK  = dAqk^T Q + V dS                  dS <- dS + Q^T dO            (stored as dS^T)
 // The delta rule's formulas stand at its kernel.
 // Every tile lives in LDS once, in its natural orientation; products that contract over
-// the row index read it through transpose loads (KROW operands).
+// the row index read it through transpose loads (KROW operands).  Gradients leave through dead
+// LDS tiles and are written to memory row-wise (tile_rows_to_global).
 #include "chunk_common.h"
 
 
@@ -34,46 +35,6 @@ template <typename T, int C> struct BwdDims {
 
 // d(phi)/dx recovered from the staged phi(x): phi > 1 <=> x > 0 (derivative 1), else phi' = phi.
 template <bool FMAP> __device__ __forceinline__ float fmap_grad(float phi) { return FMAP ? (phi > 1.f ? 1.f : phi) : 1.f; }
-
-// Write an accumulator set holding X^T (m = feature, n = chunk row) to a (B,T,H,64)
-// array: 4 consecutive features per lane.  scale(row, d0) multiplies, keep(row) gates.
-template <typename T, int C, int NW, typename ScaleF, typename KeepF>
-__device__ __forceinline__ void store_rows_global(const f32x4 *acc, T *base, int64_t rs, int t0, int Tlen,
-                                                  int w, int lane, ScaleF scale, KeepF keep)
-{
-    using TM = TileMap<HD, C, NW>;
-    using P4 = typename TT<T>::pack4;
-    const int li = lane & 15, lg = lane >> 4;
-#pragma unroll
-    for (int j = 0; j < TM::TPW; ++j) {
-        const int d0 = TM::mt(w, j) * 16 + 4 * lg, r = TM::nt(w, j) * 16 + li;
-        if (t0 + r < Tlen && keep(r)) {
-            const f32x4 s = scale(r, d0);
-            *reinterpret_cast<P4 *>(base + (int64_t)(t0 + r) * rs + d0) =
-                TT<T>::pack(acc[j][0] * s[0], acc[j][1] * s[1], acc[j][2] * s[2], acc[j][3] * s[3]);
-        }
-    }
-}
-
-// Same, addressed by a running pointer: `row` points at feature 4 * (lane >> 4) of chunk row
-// (lane & 15); the tile offsets are wave-uniform.
-template <typename T, int C, int NW, typename ScaleF, typename KeepF>
-__device__ __forceinline__ void store_rows_at(const f32x4 *acc, T *row, int64_t rs, int t0, int Tlen, int w,
-                                              int lane, ScaleF scale, KeepF keep)
-{
-    using TM = TileMap<HD, C, NW>;
-    using P4 = typename TT<T>::pack4;
-    const int li = lane & 15, lg = lane >> 4;
-#pragma unroll
-    for (int j = 0; j < TM::TPW; ++j) {
-        const int d0 = TM::mt(w, j) * 16 + 4 * lg, r = TM::nt(w, j) * 16 + li;
-        if (t0 + r < Tlen && keep(r)) {
-            const f32x4 s = scale(r, d0);
-            *reinterpret_cast<P4 *>(row + (int64_t)(TM::nt(w, j) * 16) * rs + TM::mt(w, j) * 16) =
-                TT<T>::pack(acc[j][0] * s[0], acc[j][1] * s[1], acc[j][2] * s[2], acc[j][3] * s[3]);
-        }
-    }
-}
 
 // =====================================================================================
 // linear attention: 8 tiles, two workgroups per CU
