@@ -576,9 +576,10 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     int64_t tmoff = ((int64_t)bh * NC + NC - 1) * C * C + (tid / IOT::SEGS) * C + (tid % IOT::SEGS) * IOT::KP;
     int64_t doff = (int64_t)b * Tlen + tlast + lane;  // done/beta of chunk row `lane`
     int tpre = tlast;                                 // first time step of the chunk about to be prefetched
-    // The prefetch of the next chunk is issued in parts, one per phase, so that the address unit
-    // works through the loads beside the phases' LDS and MFMA work instead of stalling every wave
-    // at one point.  part 0: q, 1: k, 2: v, 3: dout, 4: S, 5: Tm and the per-row scalars.
+    // The prefetch of the next chunk is issued in parts, two in each of the first three phases, so
+    // that the address unit works through the loads beside the phases' LDS and MFMA work instead of
+    // stalling every wave at one point, and all of them are under way before the first store of the
+    // pass.  part 0: q, 1: k, 2: v, 3: dout, 4: S, 5: Tm and the per-row scalars.
     auto prefetch_part = [&](int part) {
         typename IO::F z;
 #pragma unroll
@@ -699,7 +700,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             MRX_PHASE(11);
             flush_pending();
             const bool pre = pass == 0 && c > 0;
-            if (pre) prefetch_part(0);
+            if (pre) { prefetch_part(0); prefetch_part(1); }
 
             auto tril = [](int m, int n, float x) { return m <= n ? x : 0.f; };
             // ---- Aqk[i][j] = q_i . k_j, j <= i : D[m = j][n = i] -> sAqk[i][j] ----------------------
@@ -731,7 +732,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();
             MRX_PHASE(15);
-            if (pre) prefetch_part(1);
+            if (pre) { prefetch_part(2); prefetch_part(3); }
             // ---- U'^T[dv][c] = sum_j V~[j][dv] Tm[c][j] -> sU[c][dv] ----------------------------------
             {
                 f32x4 acc[TMR::TPW];
@@ -749,7 +750,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();  // sU, sDU visible; sAqk dead
             MRX_PHASE(16);
-            if (pre) prefetch_part(2);
+            if (pre) { prefetch_part(4); prefetch_part(5); }
             float dbp[TMR::NBW];  // per-lane partials of dbeta for rows nt * 16 + li of the wave's tile columns
 #pragma unroll
             for (int j = 0; j < TMR::NBW; ++j) dbp[j] = 0.f;
@@ -788,7 +789,6 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();  // sDAqk, sZb, sDT visible; sVt dead
             MRX_PHASE(17);
-            if (pre) prefetch_part(3);
             tile_rows_to_global<T, C, NTHR>(sZb, LDD, dv + base + (int64_t)t0 * rs, rs, t0, Tlen, tid, live);
             // ---- dQ^T[dk][i] = sum_dv S[dv][dk] dO[i][dv] + sum_j K[j][dk] dAqk[i][j] -> global ----
             {
@@ -829,7 +829,6 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();  // sY1 visible; sQ, sDO, sS, sDS, sDAqk, sZb dead
             MRX_PHASE(20);
-            if (pre) prefetch_part(4);
             tile_rows_to_global<T, C, NTHR>(sDU, LDD, dq + base + (int64_t)t0 * rs, rs, t0, Tlen, tid, live);
             // ---- dA[i][j] = -sum_b Y1[i][b] Tm[j][b], j < i : D[m = j][n = i] -> sDA[i][j] (over sS) ----
             {
@@ -840,7 +839,6 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             sync_lds();
             MRX_PHASE(22);
-            if (pre) prefetch_part(5);
             // ---- R^T[dk][i] = sum_j K[j][dk] dA[i][j] : dbeta += K_i . R_i ; dK += beta_i R ;
             //      dK^T[dk][j] += sum_i beta_i K[i][dk] dA[i][j] -> global -------------------------------
             {

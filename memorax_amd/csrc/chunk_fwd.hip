@@ -142,7 +142,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     }
     int64_t doff = (int64_t)b * Tlen + lane;  // done of chunk row `lane`
     int tpre = 0;                             // first time step of the chunk about to be prefetched
-    // The prefetch is issued in parts spread over the phases, so that the address unit works
+    // The prefetch is issued in parts spread over the first phases, so that the address unit works
     // through the loads beside LDS and MFMA work.  part 0: q, 1: k, 2: v, 3: per-row scalars.
     auto prefetch_part = [&](int part) {
         typename IO::F z;
@@ -285,8 +285,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 }
             }
             const bool pre = pass == nres && c + 1 < NC;
-            if (pre) prefetch_part(0);
-            if (!DELTA && pre) prefetch_part(1);
+            if (pre) { prefetch_part(0); prefetch_part(1); }
             // ---- A[i][j] = beta_i (k_i . k_j), j < i ----------------------------------
             if (DELTA) {
                 f32x4 acc[TMK::TPW];
@@ -312,11 +311,10 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 if (diag >= 0) Xcc = tri_diag_block<T>(kk, sBeta, diag, sA, LDA, sTm, LDC, lane);
                 sync_lds();
                 MRX_PHASE(2);
-                if (pre) prefetch_part(1);
+                if (pre) { prefetch_part(2); prefetch_part(3); }
                 if (diag >= 0) tri_block_column<C, T>(sA, LDA, sTm, LDC, diag, Xcc, lane);
                 sync_lds();
                 MRX_PHASE(3);
-                if (pre) prefetch_part(2);
             }
             // ---- Aqk[i][j] = (q_i . k_j), j <= i ; delta rule: W = Tm (beta K), U = Tm (beta V) ----
             {
@@ -363,7 +361,6 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 }
                 sync_lds();  // sW, sAqk visible; every wave is done with beta V
                 MRX_PHASE(5);
-                if (pre) prefetch_part(3);
                 // U'^T[dv][c] = U^T - S W^T -> sU[c][dv] (over beta V)
                 {
                     f32x4 acc[TMO::TPW];
