@@ -137,3 +137,25 @@ def test_gated_poison_does_not_cross_episodes():
         if a.dim() >= 3 and a.shape[1] == T:
             a, b_ = a[:, keep], b_[:, keep]
         assert torch.equal(a, b_), name
+
+
+def test_gated_with_zero_log_decay_is_linear_attention_at_full_size():
+    """Size-independent property at configuration 3's per-sequence shape: g = 0 reduces the gated
+    kernels to the plain ones (same products, decay factors exactly 1)."""
+    from memorax_amd import kernels as K
+    B, T, H = 8, 4096, 8
+    gen = torch.Generator(device="cuda").manual_seed(12)
+    bf = torch.bfloat16
+    q, k, v, do = (torch.randn((B, T, H, 64), device="cuda", generator=gen).div_(8).to(bf) for _ in range(4))
+    done = torch.rand((B, T), device="cuda", generator=gen) < 0.002
+    g0 = torch.zeros((B, T, H), device="cuda")
+    o, Sl, chk = K.gated_linear_attn_fwd(q, k, v, g0, done, None, 1)
+    dq, dk, dv, dg, _ = K.gated_linear_attn_bwd(q, k, v, g0, done, chk, do, None, 1, want_dS0=False)
+    o2, Sl2, chk2 = K.linear_attn_fwd(q, k, v, done, None, 1)
+    dq2, dk2, dv2, _ = K.linear_attn_bwd(q, k, v, done, chk2, do, None, 1, want_dS0=False)
+    assert relerr(Sl, Sl2.cpu().numpy()) <= 1e-5
+    # bf16 outputs: the gated kernels add the two terms of dV and dK in the other order, so a result may
+    # round to the neighbouring bf16 value (2^-8 relative)
+    for a, b_ in ((o, o2), (dq, dq2), (dk, dk2), (dv, dv2)):
+        assert relerr(a, b_.float().cpu().numpy()) <= 2.0 ** -8
+    assert torch.isfinite(dg).all()

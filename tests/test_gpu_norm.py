@@ -213,3 +213,21 @@ def test_normalised_rejects_bad_arguments():
                                                   1, 4, 1, 64, 64, 0, 0, 1, 1e-6)
     assert bwd(None) == -1            # z_chk is required
     torch.cuda.synchronize()
+
+
+def test_normalised_constant_values_come_back_at_full_size():
+    """Size-independent property at configuration 3's per-sequence shape (T = 4096, bf16): without a
+    carry the normalised read-out is a convex combination of the episode's values, so values that
+    are constant along time come back unchanged, resets or not."""
+    from memorax_amd import kernels as K
+    B, T, H = 8, 4096, 8
+    g = torch.Generator(device="cuda").manual_seed(11)
+    bf = torch.bfloat16
+    q, k = (torch.randn((B, T, H, 64), device="cuda", generator=g).div_(8).to(bf) for _ in range(2))
+    c = torch.randn((B, 1, H, 64), device="cuda", generator=g).to(bf)
+    v = c.expand(B, T, H, 64).contiguous()
+    done = torch.rand((B, T), device="cuda", generator=g) < 0.002
+    o, den, Sl, zl, _ = K.linear_attn_norm_fwd(q, k, v, done, None, None, 1, 1e-6, save_chk=False)
+    err = (o.float() - v.float()).abs().max() / v.float().abs().max()
+    assert float(err) <= TOL_BF16, float(err)
+    assert float(den.min()) > 0.5   # phi > 0: every denominator is at least one key's worth
