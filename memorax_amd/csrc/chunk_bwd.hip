@@ -124,13 +124,18 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                            : f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    // normalised read-out: dz[dk], held like a column of dS^T (see the forward kernel's z)
+    // normalised read-out: dz[dk], held like a column of dS^T; fp32 (VN): component 0 holds
+    // dz[dk = 16 mt + li] and the sums run on the vector ALU (see the forward kernel's z)
+    constexpr bool VN = sizeof(T) == 4;
     f32x4 dzacc[TMS::MBW];
 #pragma unroll
     for (int mi = 0; mi < TMS::MBW; ++mi) {
-        const int dk0 = TMS::mt(w, mi * TMS::NBW) * 16 + 4 * lg;
-        dzacc[mi] = (NORM && na.dz_last) ? *reinterpret_cast<const f32x4 *>(na.dz_last + (int64_t)bh * HD + dk0)
-                                         : f32x4{0.f, 0.f, 0.f, 0.f};
+        const int dkt = TMS::mt(w, mi * TMS::NBW) * 16;
+        dzacc[mi] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (NORM && na.dz_last) {
+            if (VN) dzacc[mi][0] = na.dz_last[(int64_t)bh * HD + dkt + li];
+            else dzacc[mi] = *reinterpret_cast<const f32x4 *>(na.dz_last + (int64_t)bh * HD + dkt + 4 * lg);
+        }
     }
 
     typename IO::Regs rq, rk, rv, rdo, ro;
@@ -298,10 +303,13 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             store_acc<T, HD, HD, NW>(dSacc, sDS, LDD, w, lane);  // dS[dv][dk]
             if (NORM) {
                 if (pass != nres) zero_acc<TMS::MBW>(dzacc);
-                if (w < TMS::WM && li == 0) {
+                if (w < TMS::WM && (VN ? lg == 0 : li == 0)) {
 #pragma unroll
-                    for (int mi = 0; mi < TMS::MBW; ++mi)
-                        *reinterpret_cast<f32x4 *>(sDZ + TMS::mt(w, mi * TMS::NBW) * 16 + 4 * lg) = dzacc[mi];
+                    for (int mi = 0; mi < TMS::MBW; ++mi) {
+                        float *dst = sDZ + TMS::mt(w, mi * TMS::NBW) * 16;
+                        if (VN) dst[li] = dzacc[mi][0];
+                        else *reinterpret_cast<f32x4 *>(dst + 4 * lg) = dzacc[mi];
+                    }
                 }
             }
             sync_lds();
@@ -432,9 +440,19 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     if (lg == 0) sE[(w % TMR::WM) * C + TMR::nt(w, j) * 16 + li] = x;
                 }
             }
+            float dzpart[TMS::MBW];  // fp32: per-lane partial sums over the lane's k slots
+#pragma unroll
+            for (int mi = 0; mi < TMS::MBW; ++mi) dzpart[mi] = 0.f;
             auto dz_q = [&](int mi, int kb, Frag &xq) {
-                if (NORM)  // dz[dk] += sum_i Q[i][dk] dden_i
-                    dzacc[mi] = TT<T>::mma(xq, TT<T>::template load<ROWK>(sDdT, 0, 0, kb * TT<T>::KB, lane), dzacc[mi]);
+                if (NORM) {  // dz[dk] += sum_i Q[i][dk] dden_i
+                    if (VN) {
+                        const float *dd = sDd + kb * TT<T>::KB + TT<T>::KP * lg;
+#pragma unroll
+                        for (int e = 0; e < TT<T>::KP; ++e) dzpart[mi] += (float)xq[e] * dd[e];
+                    } else {
+                        dzacc[mi] = TT<T>::mma(xq, TT<T>::template load<ROWK>(sDdT, 0, 0, kb * TT<T>::KB, lane), dzacc[mi]);
+                    }
+                }
                 if (GATED) {  // row c of Q enters the state update as a_c Q[c]: scale the fragment along k
                     const float *ea = sEa + kb * TT<T>::KB + TT<T>::KP * lg;
 #pragma unroll
@@ -442,6 +460,15 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 }
             };
             gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, sQ, LDD, sDO, LDD, w, lane, dz_q);
+            if (NORM && VN) {
+#pragma unroll
+                for (int mi = 0; mi < TMS::MBW; ++mi) {
+                    float x = dzpart[mi];
+                    x += __shfl_xor(x, 16);
+                    x += __shfl_xor(x, 32);
+                    dzacc[mi][0] += x;
+                }
+            }
             sync_lds();  // every product has read its operands
             park(hV, sV);
             park(hQ, sQ);
@@ -467,10 +494,13 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             *reinterpret_cast<f32x4 *>(dS0 + ((int64_t)bh * HD + dvv) * HD + dk0) = dSacc[j];
         }
     }
-    if (NORM && na.dz0 && w < TMS::WM && li == 0) {
+    if (NORM && na.dz0 && w < TMS::WM && (VN ? lg == 0 : li == 0)) {
 #pragma unroll
-        for (int mi = 0; mi < TMS::MBW; ++mi)
-            *reinterpret_cast<f32x4 *>(na.dz0 + (int64_t)bh * HD + TMS::mt(w, mi * TMS::NBW) * 16 + 4 * lg) = dzacc[mi];
+        for (int mi = 0; mi < TMS::MBW; ++mi) {
+            float *dst = na.dz0 + (int64_t)bh * HD + TMS::mt(w, mi * TMS::NBW) * 16;
+            if (VN) dst[li] = dzacc[mi][0];
+            else *reinterpret_cast<f32x4 *>(dst + 4 * lg) = dzacc[mi];
+        }
     }
 }
 

@@ -113,14 +113,21 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                      : f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    // normalised read-out: z[dk] of the running episode, held like a column of S^T (every lane
-    // of a 16-lane group carries the same four dk of each of the wave's m-tiles)
+    // normalised read-out: z[dk] of the running episode.  bf16: held like a column of S^T (every
+    // lane of a 16-lane group carries the same four dk = 4 lg + v of each of the wave's m-tiles) and
+    // maintained with MFMAs on a tile of ones.  fp32 (VN): a 16x16x4 MFMA per four terms of a row
+    // sum is a bad trade, so the sums run on the vector ALU over the same fragments and component 0
+    // holds z[dk = 16 mt + li] (every lane group the same).
+    constexpr bool VN = sizeof(T) == 4;
     f32x4 zacc[TMS::MBW];
 #pragma unroll
     for (int mi = 0; mi < TMS::MBW; ++mi) {
-        const int dk0 = TMS::mt(w, mi * TMS::NBW) * 16 + 4 * lg;
-        zacc[mi] = (NORM && na.z0) ? *reinterpret_cast<const f32x4 *>(na.z0 + (int64_t)bh * HD + dk0)
-                                   : f32x4{0.f, 0.f, 0.f, 0.f};
+        const int dkt = TMS::mt(w, mi * TMS::NBW) * 16;
+        zacc[mi] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (NORM && na.z0) {
+            if (VN) zacc[mi][0] = na.z0[(int64_t)bh * HD + dkt + li];
+            else zacc[mi] = *reinterpret_cast<const f32x4 *>(na.z0 + (int64_t)bh * HD + dkt + 4 * lg);
+        }
     }
     const Frag ones = TT<T>::ones();
     int64_t den_off = ((int64_t)b * Tlen + li) * H + h;  // den[t0 + li]
@@ -259,13 +266,18 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             store_acc<T, HD, HD, NW>(Sacc, sS, LDD, w, lane);  // sS[dv][dk]
             if (NORM) {
                 if (pass != 0) zero_acc<TMS::MBW>(zacc);
-                if (w < TMS::WM && li == 0) {
+                if (w < TMS::WM && (VN ? lg == 0 : li == 0)) {
 #pragma unroll
                     for (int mi = 0; mi < TMS::MBW; ++mi) {
-                        const int dk0 = TMS::mt(w, mi * TMS::NBW) * 16 + 4 * lg;
-                        *reinterpret_cast<P4 *>(sZ + dk0) = TT<T>::pack(zacc[mi][0], zacc[mi][1], zacc[mi][2], zacc[mi][3]);
-                        if (na.z_chk && pass == 0)
-                            *reinterpret_cast<f32x4 *>(na.z_chk + ((int64_t)bh * NC + c) * HD + dk0) = zacc[mi];
+                        const int dkt = TMS::mt(w, mi * TMS::NBW) * 16;
+                        float *zc = (na.z_chk && pass == 0) ? na.z_chk + ((int64_t)bh * NC + c) * HD + dkt : nullptr;
+                        if (VN) {
+                            sZ[dkt + li] = (T)zacc[mi][0];
+                            if (zc) zc[li] = zacc[mi][0];
+                        } else {
+                            *reinterpret_cast<P4 *>(sZ + dkt + 4 * lg) = TT<T>::pack(zacc[mi][0], zacc[mi][1], zacc[mi][2], zacc[mi][3]);
+                            if (zc) *reinterpret_cast<f32x4 *>(zc + 4 * lg) = zacc[mi];
+                        }
                     }
                 }
             }
@@ -382,10 +394,23 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             f32x4 dacc[TMO::NBW];
             zero_acc<TMO::NBW>(dacc);
             auto den_q = [&](int ni, int kb, const Frag &yq) {
-                if (NORM) dacc[ni] = TT<T>::mma(TT<T>::template load<ROWK>(sZ, 0, 0, kb * TT<T>::KB, lane), yq, dacc[ni]);
+                if (!NORM) return;
+                const Frag zf = TT<T>::template load<ROWK>(sZ, 0, 0, kb * TT<T>::KB, lane);  // z[k], the lane's k slots
+                if (VN) {
+#pragma unroll
+                    for (int e = 0; e < TT<T>::KP; ++e) dacc[ni][0] += (float)zf[e] * (float)yq[e];
+                } else {
+                    dacc[ni] = TT<T>::mma(zf, yq, dacc[ni]);
+                }
             };
             auto den_a = [&](int ni, int, const Frag &ya) {
-                if (NORM) dacc[ni] = TT<T>::mma(ones, ya, dacc[ni]);
+                if (!NORM) return;
+                if (VN) {
+#pragma unroll
+                    for (int e = 0; e < TT<T>::KP; ++e) dacc[ni][0] += (float)ya[e];
+                } else {
+                    dacc[ni] = TT<T>::mma(ones, ya, dacc[ni]);
+                }
             };
             gemm<T, HD, C, HD, ROWK, ROWK, NW>(Oacc, sS, LDD, sQ, LDD, w, lane, NoHook(), den_q);
             if (GATED) {  // the incoming state reaches row i decayed by exp(G_i)
@@ -394,6 +419,15 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             gemm<T, HD, C, C, KROW, ROWK, NW>(Oacc, sU, LDD, sAqk, LDC, w, lane, NoHook(), den_a);
             if (NORM) {
+                if (VN) {  // the lane groups hold partial sums over their k slots
+#pragma unroll
+                    for (int ni = 0; ni < TMO::NBW; ++ni) {
+                        float x = dacc[ni][0];
+                        x += __shfl_xor(x, 16);
+                        x += __shfl_xor(x, 32);
+                        dacc[ni][0] = x;
+                    }
+                }
 #pragma unroll
                 for (int j = 0; j < TMO::TPW; ++j) {
                     const int cc = TMO::nt(w, j) * 16 + li;
@@ -415,8 +449,18 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                     for (int j = 0; j < TMS::TPW; ++j) Sacc[j] *= cl;
                 }
+                float zpart[TMS::MBW];  // fp32: per-lane partial column sums of K over the lane's k slots
+#pragma unroll
+                for (int mi = 0; mi < TMS::MBW; ++mi) zpart[mi] = 0.f;
                 auto z_k = [&](int mi, int kb, Frag &xk) {
-                    if (NORM) zacc[mi] = TT<T>::mma(xk, ones, zacc[mi]);  // z[dk] += sum_c K[c][dk]
+                    if (NORM) {  // z[dk] += sum_c K[c][dk]
+                        if (VN) {
+#pragma unroll
+                            for (int e = 0; e < TT<T>::KP; ++e) zpart[mi] += (float)xk[e];
+                        } else {
+                            zacc[mi] = TT<T>::mma(xk, ones, zacc[mi]);
+                        }
+                    }
                     if (GATED) {  // row c of K enters the state update as b_c K[c]: scale the fragment along k
                         const float *eb = sEb + kb * TT<T>::KB + TT<T>::KP * lg;
 #pragma unroll
@@ -424,6 +468,15 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     }
                 };
                 gemm<T, HD, HD, C, KROW, KROW, NW>(Sacc, sK, LDD, sU, LDD, w, lane, z_k);
+                if (NORM && VN) {
+#pragma unroll
+                    for (int mi = 0; mi < TMS::MBW; ++mi) {
+                        float x = zpart[mi];
+                        x += __shfl_xor(x, 16);
+                        x += __shfl_xor(x, 32);
+                        zacc[mi][0] += x;
+                    }
+                }
             }
             sync_lds();
             MRX_PHASE(8);
@@ -440,10 +493,13 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             *reinterpret_cast<f32x4 *>(S_last + ((int64_t)bh * HD + dv) * HD + dk0) = Sacc[j];
         }
     }
-    if (NORM && na.z_last && w < TMS::WM && li == 0) {
+    if (NORM && na.z_last && w < TMS::WM && (VN ? lg == 0 : li == 0)) {
 #pragma unroll
-        for (int mi = 0; mi < TMS::MBW; ++mi)
-            *reinterpret_cast<f32x4 *>(na.z_last + (int64_t)bh * HD + TMS::mt(w, mi * TMS::NBW) * 16 + 4 * lg) = zacc[mi];
+        for (int mi = 0; mi < TMS::MBW; ++mi) {
+            float *zl = na.z_last + (int64_t)bh * HD + TMS::mt(w, mi * TMS::NBW) * 16;
+            if (VN) zl[li] = zacc[mi][0];
+            else *reinterpret_cast<f32x4 *>(zl + 4 * lg) = zacc[mi];
+        }
     }
 }
 
