@@ -373,6 +373,37 @@ __device__ __forceinline__ f32x4 mm16(const f32x4 &xt, const f32x4 &y, f32x4 c)
     return c;
 }
 
+// The same product on the bf16 pipe, operands split into a high and a low bf16 half
+// (x = xh + xl up to 2^-16 relative): c + Xh Yh + Xl Yh + Xh Yl.  The 32 k-slots of a 16x16x32
+// MFMA hold the 16 contraction indices twice -- slot (g, e) is index 4 g + e % 4, the high half
+// for e < 4 and the second operand's choice for e >= 4 -- so the fp32 accumulator layout is the
+// operand layout and nothing moves between lanes.  Two MFMAs of 16 cycles instead of four of 32;
+// the dropped Xl Yl term is 2^-16 of a result that is rounded to bf16 in the end.
+__device__ __forceinline__ f32x4 mm16_split(const f32x4 &xt, const f32x4 &y, f32x4 c)
+{
+    bf16x8 a1, b1, a2, b2;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const __bf16 xh = (__bf16)xt[e], yh = (__bf16)y[e];
+        a1[e] = xh;
+        a1[4 + e] = (__bf16)(xt[e] - (float)xh);
+        b1[e] = yh;
+        b1[4 + e] = yh;
+        a2[e] = xh;
+        a2[4 + e] = (__bf16)0.f;
+        b2[e] = (__bf16)(y[e] - (float)yh);
+        b2[4 + e] = (__bf16)0.f;
+    }
+    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1, c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2, b2, c, 0, 0, 0);
+}
+
+// bf16 kernels take the split product (their factor is rounded to bf16 anyway), fp32 kernels the exact one
+template <typename T> __device__ __forceinline__ f32x4 mm16_for(const f32x4 &xt, const f32x4 &y, f32x4 c)
+{
+    return sizeof(T) == 2 ? mm16_split(xt, y, c) : mm16(xt, y, c);
+}
+
 // kk[v] = (K K^T)[16b + i][16b + 4g + v] (symmetric); sBeta indexed by chunk row
 template <typename T>
 __device__ __forceinline__ f32x4 tri_diag_block(const f32x4 &kk, const float *sBeta, int b, float *sA, int lda,
@@ -394,10 +425,10 @@ __device__ __forceinline__ f32x4 tri_diag_block(const f32x4 &kk, const float *sB
     }
 #pragma unroll
     for (int k = 0; k < 3; ++k) {
-        const f32x4 M2 = mm16(Mt, M, zero);    // N^2  : X = M,  Y = M
-        const f32x4 M2t = mm16(M, Mt, zero);   // (N^2)^T = M^T M^T
-        const f32x4 R2 = mm16(Rt, M2, R);      // R + R M2
-        const f32x4 R2t = mm16(M2, Rt, Rt);    // R^T + M2^T R^T
+        const f32x4 M2 = mm16_for<T>(Mt, M, zero);    // N^2  : X = M,  Y = M
+        const f32x4 M2t = mm16_for<T>(M, Mt, zero);   // (N^2)^T = M^T M^T
+        const f32x4 R2 = mm16_for<T>(Rt, M2, R);      // R + R M2
+        const f32x4 R2t = mm16_for<T>(M2, Rt, Rt);    // R^T + M2^T R^T
         M = M2; Mt = M2t; R = R2; Rt = R2t;
     }
     float *blk = sA + (16 * b) * lda + 16 * b;
@@ -425,13 +456,13 @@ __device__ __forceinline__ void tri_block_column(const float *sA, int lda, T *sX
 #pragma unroll
             for (int kk = 0; kk < r; ++kk) {  // k = c + kk
                 const f32x4 a4 = *reinterpret_cast<const f32x4 *>(sA + (16 * b + i) * lda + 16 * (c + kk) + 4 * g);
-                part[kk] = mm16(a4, Xc[kk], zero);
+                part[kk] = mm16_for<T>(a4, Xc[kk], zero);
             }
             f32x4 tmp = part[0];
 #pragma unroll
             for (int kk = 1; kk < r; ++kk) tmp += part[kk];
             const f32x4 d4 = *reinterpret_cast<const f32x4 *>(sA + (16 * b + i) * lda + 16 * b + 4 * g);
-            Xc[r] = -mm16(d4, tmp, zero);
+            Xc[r] = -mm16_for<T>(d4, tmp, zero);
 #pragma unroll
             for (int v = 0; v < 4; ++v) sX[(16 * b + 4 * g + v) * ldx + 16 * c + i] = (T)Xc[r][v];
         }
