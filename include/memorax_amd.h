@@ -151,7 +151,12 @@ int mrx_linear_attn_norm_bwd(void *stream, const void *q, const void *k,
  * beta: (B,T,H) in `dtype`; other arguments as for linear attention.
  * Tm_chk (nullable): (B,H,ceil(T/chunk),chunk,chunk) in `dtype` (chunk = mrx_delta_chunk_size), receives each
  * chunk's unit-lower-triangular factor (I + tril(diag(beta) K K^T, -1))^-1, block
- * diagonal by episode; like S_chk it is a residual the backward call requires. */
+ * diagonal by episode; like S_chk it is a residual the backward call requires.
+ * It may be given without S_chk: the forward call also works through it.  With the buffer and
+ * B*H <= 2 x the device's compute units the factors of all chunks are computed by a chunk-parallel
+ * kernel first and the sequential kernel reads them (up to a third faster while the device is not
+ * full); otherwise the sequential kernel inverts in place.  Both ways fill Tm_chk with the same
+ * factors up to rounding. */
 int mrx_delta_rule_fwd(void *stream, const void *q, const void *k,
                        const void *v, const void *beta, const void *done,
                        const void *S0, void *o, void *S_last, void *S_chk,

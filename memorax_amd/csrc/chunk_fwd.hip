@@ -15,6 +15,7 @@
 // The state is kept transposed (S^T, d_k x d_v) in MFMA accumulators for the whole
 // sequence and re-staged to LDS as a T-typed d_v x d_k tile once per chunk.
 #include "chunk_common.h"
+#include "delta_tm.h"
 
 namespace {
 
@@ -60,7 +61,10 @@ struct NormArgs {
 
 // PRO (delta rule): the cell's prologue runs on the staged rows -- keys are L2-normalised
 // (k / max(|k|, 1e-12), in fp32, then rounded to T) and beta = sigmoid(raw beta).
-template <typename T, int C, bool DELTA, bool FMAP, bool GATED, bool NORM, bool PRO = false>
+// TMIN (delta rule): the triangular factors have been computed by delta_tm_kernel and are read from
+// Tm_chk like any other input; the kernel then has neither the K K^T product nor the inverse and
+// a chunk costs four barriers.  Without it (no Tm_chk buffer given) the inverse runs in here.
+template <typename T, int C, bool DELTA, bool FMAP, bool GATED, bool NORM, bool PRO = false, bool TMIN = false>
 __global__ void __launch_bounds__(NTHR, 2)  // 2 waves per SIMD: two workgroups share a CU
 chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const float *__restrict__ glog,
@@ -71,6 +75,8 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     static_assert(!(DELTA && GATED), "the gated variant is linear attention with a decay");
     static_assert(!NORM || (!DELTA && !GATED), "the normalised read-out belongs to plain linear attention");
     static_assert(!PRO || DELTA, "the prologue belongs to the delta rule");
+    static_assert(!TMIN || (DELTA && C == 32), "precomputed factors belong to the delta rule's 32-row chunks");
+    using IOT = TileIO<T, C, NTHR, C>;  // the [C][C] triangular factor
     using L = FwdSmem<T, C, DELTA, GATED, NORM>;
     using Frag = typename TT<T>::frag;
     using IO = TileIO<T, C, NTHR>;
@@ -149,6 +155,8 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     }
     int64_t doff = (int64_t)b * Tlen + lane;  // done of chunk row `lane`
     int tpre = 0;                             // first time step of the chunk about to be prefetched
+    typename IOT::Regs rTm;                   // TMIN: the factor of the chunk about to be staged
+    int64_t tmoff = (int64_t)bh * ((Tlen + C - 1) / C) * C * C + (tid / IOT::SEGS) * C + (tid % IOT::SEGS) * IOT::KP;
     // The prefetch is issued in parts spread over the first phases, so that the address unit works
     // through the loads beside LDS and MFMA work.  part 0: q, 1: k, 2: v, 3: per-row scalars.
     auto prefetch_part = [&](int part) {
@@ -168,12 +176,19 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 roff[p] += (int64_t)C * rs;
                 boff[p] += (int64_t)C * H;
             }
+            if (TMIN) {
+#pragma unroll
+                for (int p = 0; p < IOT::PASSES; ++p)
+                    if (IOT::FULL || IOT::row_of(tid, p) < C)  // a [C][C] tile may have fewer segments than threads
+                        rTm.v[p] = *reinterpret_cast<const typename IOT::F *>(Tm_chk + tmoff + p * IOT::RPP * C);
+                tmoff += C * C;
+            }
             rdone = 0u;
             rbeta = 0u;
             rg = 0.f;
             if (lane < C && tpre + lane < Tlen) {
                 rdone = done_raw(done, done_f32, doff);
-                if (DELTA && w == 0) rbeta = load_raw<T>(beta + doff * H + h);
+                if (DELTA && !TMIN && w == 0) rbeta = load_raw<T>(beta + doff * H + h);
                 if (GATED) rg = glog[doff * H + h];
             }
             doff += C;
@@ -182,7 +197,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     };
 #pragma unroll
     for (int part = 0; part < 4; ++part) prefetch_part(part);
-    if (DELTA) {
+    if (DELTA && !TMIN) {
         // blocks above the block diagonal of Tm are never written again
         for (int idx = tid; idx < C * LDC * (int)sizeof(T) / 4; idx += NTHR) reinterpret_cast<uint32_t *>(sTm)[idx] = 0u;
     }
@@ -260,8 +275,15 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 }
                 IO::to_lds(fv, sV, LDD, tid);
             }
-            if (DELTA && tid < C)
+            if (DELTA && !TMIN && tid < C)
                 sBeta[tid] = !live(tid) ? 0.f : PRO ? sigmoidf(raw_to_float<T>(rbeta)) : raw_to_float<T>(rbeta);
+            if (TMIN) {
+                // rows of other episodes are cleared by select: they only ever meet zeros, but a NaN key
+                // or gate of another episode sits in them
+                typename IOT::Regs fTm = rTm;
+                if (nres != 0) IOT::mask_rows(fTm, tid, live);
+                IOT::to_lds(fTm, sTm, LDC, tid);
+            }
             if (pass != 0) zero_acc<TMS::TPW>(Sacc);  // an episode that starts in the chunk starts from 0
             store_acc<T, HD, HD, NW>(Sacc, sS, LDD, w, lane);  // sS[dv][dk]
             if (NORM) {
@@ -298,8 +320,9 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             }
             const bool pre = pass == nres && c + 1 < NC;
             if (pre) { prefetch_part(0); prefetch_part(1); }
+            if (TMIN && pre) { prefetch_part(2); prefetch_part(3); }
             // ---- A[i][j] = beta_i (k_i . k_j), j < i ----------------------------------
-            if (DELTA) {
+            if (DELTA && !TMIN) {
                 f32x4 acc[TMK::TPW];
                 zero_acc<TMK::TPW>(acc);
                 gemm<T, C, C, HD, ROWK, ROWK, NW, 1>(acc, sK, LDD, sK, LDD, w, lane);  // D[m = j][n = i]
@@ -360,7 +383,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sBK, LDD, sTm, LDC, w, lane);  // W^T[dk][c]
                     store_acc<T, HD, C, NW>(acc, sW, LDD, w, lane);
                 }
-                if (Tm_chk) {
+                if (Tm_chk && !TMIN) {
                     // residual for the backward call: the rows of this pass's episode (rows past
                     // the end of the sequence count as the last episode: identity rows)
 #pragma unroll
@@ -503,12 +526,13 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     }
 }
 
-template <typename T, int C, bool DELTA, bool FMAP, bool GATED = false, bool NORM = false, bool PRO = false>
+template <typename T, int C, bool DELTA, bool FMAP, bool GATED = false, bool NORM = false, bool PRO = false,
+          bool TMIN = false>
 int launch(hipStream_t st, const void *q, const void *k, const void *v, const void *beta,
            const void *done, int done_f32, const void *S0, void *o, void *S_last, void *S_chk,
            void *Tm_chk, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr, NormArgs na = NormArgs{})
 {
-    auto kern = chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO>;
+    auto kern = chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN>;
     constexpr int smem = FwdSmem<T, C, DELTA, GATED, NORM>::total;
     static unsigned long long lds_set = 0ull;
     if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
@@ -533,6 +557,49 @@ int check_common(const void *q, const void *k, const void *v, const void *done, 
         return MRX_ERR_INVALID_ARG;
     if (done_dtype == MRX_DONE_F32 && !aligned(done, 4)) return MRX_ERR_INVALID_ARG;
     return MRX_OK;
+}
+
+// Compute units of the current device (0 if the query fails), asked once per device.
+int compute_units()
+{
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
+// Two ways to the triangular factors.  With a buffer for them and at most two workgroups per compute
+// unit, the chunk-parallel kernel fills the buffer and the sequential kernel reads it: the
+// sequential kernel loses half of its per-chunk dependency chain, which is what bounds it while
+// the device is not full.  With more sequences than that the device is bound by memory traffic,
+// other workgroups hide the inverse, and the second pass over the keys plus the round trip of the
+// factors (a fifth more traffic) would only cost: the sequential kernel inverts in place then, as it
+// does when there is no buffer.
+template <bool PRO>
+int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void *v, const void *beta, const void *done,
+                       int done_dtype, const void *S0, void *o, void *S_last, void *S_chk, void *Tm_chk, int64_t B,
+                       int64_t T, int64_t H, int dtype)
+{
+    static_assert(DELTA_BF16_CHUNK == 32, "delta_tm_kernel is written for 32-row chunks");
+    if (Tm_chk && B * H <= 2 * (int64_t)compute_units()) {
+        const int rc = launch_delta_tm(st, k, beta, done, done_dtype, Tm_chk, B, T, H, dtype, PRO);
+        if (rc != MRX_OK) return rc;
+        if (dtype == MRX_BF16)
+            return launch<__bf16, 32, true, false, false, false, PRO, true>(st, q, k, v, beta, done, done_dtype, S0, o,
+                                                                           S_last, S_chk, Tm_chk, B, T, H);
+        return launch<float, 32, true, false, false, false, PRO, true>(st, q, k, v, beta, done, done_dtype, S0, o, S_last,
+                                                                       S_chk, Tm_chk, B, T, H);
+    }
+    if (dtype == MRX_BF16)
+        return launch<__bf16, 32, true, false, false, false, PRO, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last,
+                                                                        S_chk, Tm_chk, B, T, H);
+    return launch<float, 32, true, false, false, false, PRO, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last,
+                                                                    S_chk, Tm_chk, B, T, H);
 }
 
 }  // namespace
@@ -567,9 +634,7 @@ extern "C" int mrx_delta_rule_fwd(void *stream, const void *q, const void *k, co
     if (rc != MRX_OK) return rc;
     if (!beta || !aligned(Tm_chk, 16)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
-    if (dtype == MRX_BF16)
-        return launch<__bf16, DELTA_BF16_CHUNK, true, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H);
-    return launch<float, 32, true, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H);
+    return delta_fwd_dispatch<false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H, dtype);
 }
 
 extern "C" int mrx_gated_linear_attn_fwd(void *stream, const void *q, const void *k, const void *v,
@@ -621,7 +686,5 @@ extern "C" int mrx_deltanet_fwd(void *stream, const void *q, const void *k, cons
     if (rc != MRX_OK) return rc;
     if (!beta_raw || !aligned(Tm_chk, 16)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
-    if (dtype == MRX_BF16)
-        return launch<__bf16, DELTA_BF16_CHUNK, true, false, false, false, true>(st, q, k, v, beta_raw, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H);
-    return launch<float, 32, true, false, false, false, true>(st, q, k, v, beta_raw, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H);
+    return delta_fwd_dispatch<true>(st, q, k, v, beta_raw, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H, dtype);
 }

@@ -226,11 +226,14 @@ def linear_attn_norm_bwd(q, k, v, done, chk, o, den, do, dS_last=None, dz_last=N
     return dq, dk_, dv_, dS0, dz0
 
 
-def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prologue=False):
+def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prologue=False, tm_scratch=None):
     """Returns (o, S_last fp32, chk) where chk = (S_chk, Tm_chk) are the residuals the
     backward call needs, or None.  out = (o, S_last, S_chk, Tm_chk) reuses buffers of an earlier
     call with the same shapes instead of allocating.  prologue=True: k is L2-normalised and
-    beta = sigmoid(beta) inside the kernel (mrx_deltanet_fwd)."""
+    beta = sigmoid(beta) inside the kernel (mrx_deltanet_fwd).
+    tm_scratch (only without residuals): give the library a buffer for the triangular factors
+    anyway, which lets it compute them chunk-parallel while the device is not full.  None: when
+    B*H is at most two sequences per compute unit, which is when the library uses it."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
     _chk(beta, "beta", dt, (B, T, H))
@@ -252,6 +255,12 @@ def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prolog
             C, NC = chunk_size(dt, True), _n_chunks(T, dt, True)
             S_chk = torch.empty((B, H, NC, dv, dk), dtype=dt, device=q.device)
             Tm_chk = torch.empty((B, H, NC, C, C), dtype=dt, device=q.device)
+        else:
+            if tm_scratch is None:
+                tm_scratch = B * H <= 2 * torch.cuda.get_device_properties(q.device).multi_processor_count
+            if tm_scratch:
+                C, NC = chunk_size(dt, True), _n_chunks(T, dt, True)
+                Tm_chk = torch.empty((B, H, NC, C, C), dtype=dt, device=q.device)
     name = "mrx_deltanet_fwd" if prologue else "mrx_delta_rule_fwd"
     st = getattr(lib, name)(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done),
                             _ptr(S0), _ptr(o), _ptr(S_last), _ptr(S_chk), _ptr(Tm_chk), B, T, H,

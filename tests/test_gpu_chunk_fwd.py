@@ -42,17 +42,21 @@ def test_linear_attention_fwd(shape, p, dtype, fmap):
 @pytest.mark.parametrize("shape", SHAPES)
 @pytest.mark.parametrize("p", [0.0, 0.05])
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
-def test_delta_rule_fwd(shape, p, dtype):
+@pytest.mark.parametrize("save_chk", [True, False])
+def test_delta_rule_fwd(shape, p, dtype, save_chk):
+    """save_chk=True: the triangular factors come from the chunk-parallel kernel and the sequential
+    kernel reads them; False (and no scratch for them): the sequential kernel inverts in place."""
     from memorax_amd import kernels as K
     B, T, H = shape
     x = attn_inputs(B, T, H, p=p, seed=B * 100 + T + H + 7, delta=True)
-    print(f"case delta_fwd shape={shape} p={p} dtype={dtype}", flush=True)
+    print(f"case delta_fwd shape={shape} p={p} dtype={dtype} save_chk={save_chk}", flush=True)
     td = torch.bfloat16 if dtype == "bf16" else torch.float32
     if dtype == "bf16":
         for n in ("q", "k", "v", "beta"):
             x[n] = bf16_round(x[n])
     o, Sl, chk = K.delta_rule_fwd(dev(x["q"], td), dev(x["k"], td), dev(x["v"], td), dev(x["beta"], td),
-                                  dev(x["done"]), dev(x["S0"]))
+                                  dev(x["done"]), dev(x["S0"]), save_chk=save_chk, tm_scratch=False)
+    assert (chk is not None) == save_chk
     ro, rSl = M.delta_rule(x["q"], x["k"], x["v"], x["beta"], x["done"], x["S0"])
     tol = TOL_BF16 if dtype == "bf16" else TOL_F32
     assert relerr(o, ro) <= tol, relerr(o, ro)
@@ -92,3 +96,43 @@ def test_config_shapes_small_batch():
                                 dev(x["done"]))
     ro, rSl = clib.delta_rule_fwd(xb["q"], xb["k"], xb["v"], xb["beta"], x["done"])
     assert relerr(o, ro) <= TOL_BF16 and relerr(Sl, rSl) <= TOL_BF16
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("prologue", [False, True])
+def test_delta_rule_factor_paths_agree(dtype, prologue):
+    """The triangular factors of a chunk depend on its keys, gates and resets only.  Three ways to
+    them: the chunk-parallel kernel (residuals asked, device not full), the sequential kernel with
+    the factors stored (more than two sequences per compute unit) and without.  A batch large
+    enough for the second way is cut into slices small enough for the first: same outputs and the
+    same stored factors, up to rounding; and the backward call accepts either."""
+    from memorax_amd import kernels as K
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    H, T = 8, 70
+    B = 2 * cus // H + 3  # B*H just above two sequences per compute unit
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    g = torch.Generator(device="cuda").manual_seed(11)
+    q, k, v, do = (torch.randn((B, T, H, 64), device="cuda", generator=g).to(td) for _ in range(4))
+    if not prologue:
+        k = torch.nn.functional.normalize(k.float(), dim=-1).to(td)
+    beta = torch.randn((B, T, H), device="cuda", generator=g)
+    beta = (beta if prologue else torch.sigmoid(beta)).to(td)
+    done = torch.rand((B, T), device="cuda", generator=g) < 0.05
+    print(f"case factor_paths dtype={dtype} prologue={prologue} B={B}", flush=True)
+    o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done, prologue=prologue)            # stored, in place
+    o2, Sl2, _ = K.delta_rule_fwd(q, k, v, beta, done, save_chk=False, prologue=prologue, tm_scratch=False)
+    assert torch.equal(o, o2) and torch.equal(Sl, Sl2)  # the same kernel with and without the stores
+    grads = K.delta_rule_bwd(q, k, v, beta, done, chk, do, prologue=prologue)
+    for lo in range(0, B, 32):
+        sl = slice(lo, min(lo + 32, B))
+        args = (q[sl].contiguous(), k[sl].contiguous(), v[sl].contiguous(), beta[sl].contiguous(), done[sl].contiguous())
+        o3, Sl3, chk3 = K.delta_rule_fwd(*args, prologue=prologue)                   # chunk-parallel
+        o4, Sl4, _ = K.delta_rule_fwd(*args, save_chk=False, prologue=prologue)      # the same through scratch
+        assert torch.equal(o3, o4) and torch.equal(Sl3, Sl4)
+        assert relerr(o3, o[sl].float().cpu().numpy()) <= tol and relerr(Sl3, Sl[sl].cpu().numpy()) <= tol
+        assert relerr(chk3[1], chk[1][sl].float().cpu().numpy()) <= tol
+        assert relerr(chk3[0], chk[0][sl].float().cpu().numpy()) <= tol
+        g3 = K.delta_rule_bwd(*args, chk3, do[sl].contiguous(), prologue=prologue)
+        for a, b_ in zip(g3, grads):
+            assert relerr(a, b_[sl].float().cpu().numpy()) <= tol

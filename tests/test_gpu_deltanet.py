@@ -45,6 +45,9 @@ def test_deltanet_fwd_bwd(shape, p, dtype):
     errs = {"o": relerr(o, ref["o"]), "S_last": relerr(Sl, ref["S_last"])}
     errs.update({n: relerr(g, ref[n]) for n, g in zip(("dq", "dk", "dv", "dbeta", "dS0"), got)})
     assert all(e <= tol for e in errs.values()), errs
+    # without a buffer for the triangular factors the sequential kernel inverts in place
+    o3, Sl3, _ = K.delta_rule_fwd(tq, tk, tv, tb, dn, dev(x["S0"]), save_chk=False, prologue=True, tm_scratch=False)
+    assert relerr(o3, ref["o"]) <= tol and relerr(Sl3, ref["S_last"]) <= tol
     # fp32: the prologue done by the caller and the plain entry points give the same numbers
     if dtype == "f32":
         kn = torch.nn.functional.normalize(tk, dim=-1)
@@ -70,7 +73,7 @@ def test_deltanet_key_gradient_is_orthogonal_to_the_key_at_the_benchmark_shape()
     cos = (kf * dkf).sum(-1).abs() / (kf.norm(dim=-1) * dkf.norm(dim=-1) + 1e-30)
     assert float(cos.max()) <= 2e-2, float(cos.max())
     # scaling the keys by powers of two changes nothing at all
-    o2, Sl2, _ = K.delta_rule_fwd(q, (k.float() * 4).to(bf), v, braw, done, None, save_chk=False, prologue=True)
+    o2, Sl2, _ = K.delta_rule_fwd(q, (k.float() * 4).to(bf), v, braw, done, None, prologue=True)
     assert torch.equal(o, o2) and torch.equal(Sl, Sl2)
 
 
