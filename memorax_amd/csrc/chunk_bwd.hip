@@ -505,14 +505,17 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 }
 
 // =====================================================================================
-// delta rule: fourteen LDS tiles (68 KB for bf16, 127 KB for fp32, C = 32), three of them reused
+// delta rule: fourteen LDS tiles (68 KB for bf16, 127 KB for fp32, C = 32), two of them reused
 // once their first tenant is dead.  bf16: two workgroups per CU.
 //
 // Per pass, with S the state entering the chunk, Tm = (I + A)^-1 from the forward call:
 //   V0 = V - K S^T,  V~ = diag(beta) V0,  U' = Tm V~            (W = T K and U = T V are never formed)
 //   Aqk = tril(Q K^T),  dU' = Aqk^T dO + K dS^T,  dAqk = tril(dO U'^T)
 //   Z = Tm^T dU',  dV = diag(beta) Z,  dbeta = rowdot(Z, V0) + rowdot(K, R)
-//   dTm = tril(dU' V~^T),  dA = -tril((Tm^T dTm) Tm^T, -1),  R = dA K
+//   dA = -tril(Z U'^T, -1),  R = dA K
+//     (dTm = dU' V~^T and dA = -Tm^T dTm Tm^T = -(Tm^T dU')(Tm V~)^T; the part of dTm above the
+//      diagonal, which is no parameter, only reaches the part of dA above the diagonal, so neither
+//      dTm nor the two products with Tm^T are formed)
 //   dQ = dO S + dAqk K
 //   dK = dAqk^T Q + U' dS - (diag(beta) Z) S + diag(beta) R + dA^T (diag(beta) K)
 //   dS <- dS + Q^T dO - K^T (diag(beta) Z)                       (stored as dS^T)
@@ -555,12 +558,12 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     auto at = [&](int off) { return reinterpret_cast<T *>(smem + off); };
     T *sK = at(L::oK), *sQ = at(L::oQ), *sDO = at(L::oDO), *sBK = at(L::oBK);
     T *sV = at(L::oV);                                    // V[c][dv] -> V0 = V - K S^T (in place)
-    T *sVt = at(L::oVt), *sY1 = at(L::oVt);               // V~ = beta V0 -> Y1[j][b]
+    T *sVt = at(L::oVt), *sZ = at(L::oVt);                // V~ = beta V0 -> Z[c][dv]
     T *sU = at(L::oU), *sDU = at(L::oDU), *sZb = at(L::oZb);
-    T *sS = at(L::oS), *sDA = at(L::oS);                  // S[dv][dk] -> dA[i][j]
+    T *sS = at(L::oS);                                    // S[dv][dk]
     T *sDS = at(L::oDS);                                  // dS[dv][dk]
     T *sAqk = at(L::oAqk), *sDAqk = at(L::oAqk);          // Aqk[i][j] -> dAqk[i][j]
-    T *sTm = at(L::oTm), *sDT = at(L::oDT);               // Tm[i][j], dTm[a][b]
+    T *sTm = at(L::oTm), *sDA = at(L::oDT);               // Tm[i][j], dA[i][j]
     float *sBeta = reinterpret_cast<float *>(smem + L::oBeta);
     float *sDb = reinterpret_cast<float *>(smem + L::oDb);  // [NSLOT][C] dbeta partials
     float *sKinv = reinterpret_cast<float *>(smem + L::oKinv);  // prologue: 1 / |k_row|
@@ -806,18 +809,12 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 zero_acc<TMR::TPW>(acc);
                 gemm<T, HD, C, C, KROW, KROW, NW>(acc, sDU, LDD, sTm, LDC, w, lane);
                 rowdot(acc, sV);
+                store_acc<T, HD, C, NW>(acc, sZ, LDD, w, lane);  // V~ is dead: every wave has formed its U'
 #pragma unroll
                 for (int j = 0; j < TMR::TPW; ++j) acc[j] *= sBeta[TMR::nt(w, j) * 16 + li];
                 store_acc<T, HD, C, NW>(acc, sZb, LDD, w, lane);  // = dV, written to memory from here after the barrier
             }
-            // ---- dTm[a][b] = du'_a . v~_b, b <= a : D[m = b][n = a] -> sDT[a][b] ---------------------
-            {
-                f32x4 acc[TMA::TPW];
-                zero_acc<TMA::TPW>(acc);
-                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sVt, LDD, sDU, LDD, w, lane);
-                store_acc_f<T, C, C, NW>(acc, sDT, LDC, w, lane, tril);
-            }
-            sync_lds();  // sDAqk, sZb, sDT visible; sVt dead
+            sync_lds();  // sDAqk, sZ, sZb visible
             MRX_PHASE(17);
             tile_rows_to_global<T, C, NTHR>(sZb, LDD, dv + base + (int64_t)t0 * rs, rs, t0, Tlen, tid, live);
             // ---- dQ^T[dk][i] = sum_dv S[dv][dk] dO[i][dv] + sum_j K[j][dk] dAqk[i][j] -> global ----
@@ -850,25 +847,16 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                 for (int j = 0; j < TMS::TPW; ++j) dSacc[j] -= acc[j];
             }
-            // ---- Y1[j][b] = sum_a Tm[a][j] dTm[a][b] : D[m = b][n = j] -> sY1[j][b] (over sVt) ----------
+            // ---- dA[i][j] = -z_i . u'_j, j < i : D[m = j][n = i] -> sDA[i][j] ---------------------------
             {
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
-                gemm<T, C, C, C, KROW, KROW, NW>(acc, sDT, LDC, sTm, LDC, w, lane);
-                store_acc<T, C, C, NW>(acc, sY1, LDC, w, lane);
-            }
-            sync_lds();  // sY1 visible; sQ, sDO, sS, sDS, sDAqk, sZb dead
-            MRX_PHASE(20);
-            tile_rows_to_global<T, C, NTHR>(sDU, LDD, dq + base + (int64_t)t0 * rs, rs, t0, Tlen, tid, live);
-            // ---- dA[i][j] = -sum_b Y1[i][b] Tm[j][b], j < i : D[m = j][n = i] -> sDA[i][j] (over sS) ----
-            {
-                f32x4 acc[TMA::TPW];
-                zero_acc<TMA::TPW>(acc);
-                gemm<T, C, C, C, ROWK, ROWK, NW>(acc, sTm, LDC, sY1, LDC, w, lane);
+                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sU, LDD, sZ, LDD, w, lane);
                 store_acc_f<T, C, C, NW>(acc, sDA, LDC, w, lane, [](int m, int n, float x) { return m < n ? -x : 0.f; });
             }
-            sync_lds();
-            MRX_PHASE(22);
+            sync_lds();  // sDA visible; sQ, sDO, sS, sDS, sDAqk, sZ, sZb dead
+            MRX_PHASE(20);
+            tile_rows_to_global<T, C, NTHR>(sDU, LDD, dq + base + (int64_t)t0 * rs, rs, t0, Tlen, tid, live);
             // ---- R^T[dk][i] = sum_j K[j][dk] dA[i][j] : dbeta += K_i . R_i ; dK += beta_i R ;
             //      dK^T[dk][j] += sum_i beta_i K[i][dk] dA[i][j] -> global -------------------------------
             {
