@@ -4,6 +4,8 @@
 // registers costs four extra moves.
 #include "delta_tm.h"
 
+#include <type_traits>
+
 #include "chunk_common.h"
 
 namespace mrx {
@@ -131,8 +133,11 @@ delta_tm_kernel(const T *__restrict__ k, const T *__restrict__ beta, const void 
         for (int e = 0; e < 4; ++e) beta_r[bb][e] = __shfl(bl, 16 * bb + 4 * lg + e);
     }
     T *out = Tm_chk + ((int64_t)bh * NC + c) * (C * C);
-    for (int pass = 0; pass <= nres; ++pass) {
-        auto live = [&](int r) { return nres == 0 || episode_of(dmask, r) == pass; };
+    // One episode of the chunk.  RES false: the chunk has no reset, every row is live and the code
+    // carries no masks (the common case gets a copy of its own: this kernel is bound by the vector ALU).
+    auto episode = [&](auto res_tag, const int pass) {
+        constexpr bool RES = decltype(res_tag)::value;
+        auto live = [&](int r) { return !RES || episode_of(dmask, r) == pass; };
         // N = -A_bb (strictly lower) and R = I + N, each with its transpose, in accumulator layout.
         // mm(P, Q) = P^T Q, so a product and its transpose come from the same two operands swapped.
         f32x4 M[2], Mt[2], R[2], Rt[2];
@@ -185,6 +190,11 @@ delta_tm_kernel(const T *__restrict__ k, const T *__restrict__ beta, const void 
             *reinterpret_cast<P4 *>(out + (16 + li) * C + 4 * lg) = TT<T>::pack(-x10t[0], -x10t[1], -x10t[2], -x10t[3]);
             *reinterpret_cast<P4 *>(out + (16 + li) * C + 16 + 4 * lg) = TT<T>::pack(Rt[1][0], Rt[1][1], Rt[1][2], Rt[1][3]);
         }
+    };
+    if (nres == 0) {
+        episode(std::false_type{}, 0);
+    } else {
+        for (int pass = 0; pass <= nres; ++pass) episode(std::true_type{}, pass);
     }
 }
 
