@@ -156,7 +156,10 @@ int mrx_linear_attn_norm_bwd(void *stream, const void *q, const void *k,
  * B*H <= 2 x the device's compute units the factors of all chunks are computed by a chunk-parallel
  * kernel first and the sequential kernel reads them (up to a third faster while the device is not
  * full); otherwise the sequential kernel inverts in place.  Both ways fill Tm_chk with the same
- * factors up to rounding. */
+ * factors up to rounding.  The environment variable MRX_DELTA_FACTORS (read once per process)
+ * overrides the rule: "parallel" takes the chunk-parallel kernel whenever the buffer is given --
+ * worth it on a full device too when episodes end every hundred steps or so, which the library
+ * cannot see from the host -- and "inline" never does. */
 int mrx_delta_rule_fwd(void *stream, const void *q, const void *k,
                        const void *v, const void *beta, const void *done,
                        const void *S0, void *o, void *S_last, void *S_chk,

@@ -14,6 +14,9 @@
 // non-finite value can never meet a masked-out zero inside a matrix product.
 // The state is kept transposed (S^T, d_k x d_v) in MFMA accumulators for the whole
 // sequence and re-staged to LDS as a T-typed d_v x d_k tile once per chunk.
+#include <cstdlib>
+#include <cstring>
+
 #include "chunk_common.h"
 #include "delta_tm.h"
 
@@ -573,6 +576,21 @@ int compute_units()
     return cached[dev];
 }
 
+// MRX_DELTA_FACTORS in the environment overrides the rule below: "parallel" = the chunk-parallel
+// kernel whenever there is a buffer, "inline" = never.  Read once.  For callers who know what the
+// host cannot see: with frequent resets (every hundred steps or so) the chunk-parallel kernel wins
+// on a full device too, because a chunk with resets repeats the in-kernel inverse per episode.
+int factor_policy()
+{
+    static const int policy = [] {
+        const char *e = getenv("MRX_DELTA_FACTORS");
+        if (e && !strcmp(e, "parallel")) return 1;
+        if (e && !strcmp(e, "inline")) return 2;
+        return 0;
+    }();
+    return policy;
+}
+
 // Two ways to the triangular factors.  With a buffer for them and at most two workgroups per compute
 // unit, the chunk-parallel kernel fills the buffer and the sequential kernel reads it: the
 // sequential kernel loses half of its per-chunk dependency chain, which is what bounds it while
@@ -586,7 +604,8 @@ int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void 
                        int64_t T, int64_t H, int dtype)
 {
     static_assert(DELTA_BF16_CHUNK == 32, "delta_tm_kernel is written for 32-row chunks");
-    if (Tm_chk && B * H <= 2 * (int64_t)compute_units()) {
+    const int policy = factor_policy();
+    if (Tm_chk && policy != 2 && (policy == 1 || B * H <= 2 * (int64_t)compute_units())) {
         const int rc = launch_delta_tm(st, k, beta, done, done_dtype, Tm_chk, B, T, H, dtype, PRO);
         if (rc != MRX_OK) return rc;
         if (dtype == MRX_BF16)
