@@ -373,36 +373,53 @@ __device__ __forceinline__ f32x4 mm16(const f32x4 &xt, const f32x4 &y, f32x4 c)
     return c;
 }
 
-// The same product on the bf16 pipe, operands split into a high and a low bf16 half
-// (x = xh + xl up to 2^-16 relative): c + Xh Yh + Xl Yh + Xh Yl.  The 32 k-slots of a 16x16x32
-// MFMA hold the 16 contraction indices twice -- slot (g, e) is index 4 g + e % 4, the high half
-// for e < 4 and the second operand's choice for e >= 4 -- so the fp32 accumulator layout is the
-// operand layout and nothing moves between lanes.  Two MFMAs of 16 cycles instead of four of 32;
-// the dropped Xl Yl term is 2^-16 of a result that is rounded to bf16 in the end.
-__device__ __forceinline__ f32x4 mm16_split(const f32x4 &xt, const f32x4 &y, f32x4 c)
-{
-    bf16x8 a1, b1, a2, b2;
+// A 16x16 matrix in accumulator layout prepared as an operand of such a product.  fp32 kernels take
+// the exact fp32 MFMAs.  bf16 kernels run the product on the bf16 pipe with each operand split
+// once into a high and a low bf16 half (x = xh + xl up to 2^-16): Xh Yh + Xl Yh + Xh Yl as three
+// 16x16x16 MFMAs whose operands are those halves as they are (slot (g, e) of the 16 k-slots is
+// contraction index 4 g + e, so the fp32 accumulator layout is the operand layout and nothing moves
+// between lanes); a matrix is converted once however many products use it, and the dropped Xl Yl
+// term is 2^-16 of a result that is rounded to bf16 in the end.  The low halves are needed: with
+// keys correlated 0.9 from step to step the repeated squaring cancels, and high halves alone leave
+// an error of 0.19 in a factor whose entries are of order one (2e-3 with the split).
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+template <typename T> struct Op16;
+template <> struct Op16<float> {
+    f32x4 x;
+    static __device__ __forceinline__ Op16 of(const f32x4 &z) { return Op16{z}; }
+    // c + P^T Q for P, Q the matrices whose accumulator layouts were prepared
+    static __device__ __forceinline__ f32x4 mm(const Op16 &p, const Op16 &q, f32x4 c) { return mm16(p.x, q.x, c); }
+};
+template <> struct Op16<__bf16> {
+    bf16x4 h, l;
+    static __device__ __forceinline__ Op16 of(const f32x4 &z)
+    {
+        // pairs, so that each conversion is one packed instruction; the high half is widened
+        // again with a shift or a mask of the packed word
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+        u32x2 hw, lw;  // whole words: element-wise access would undo the packed conversions
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        const __bf16 xh = (__bf16)xt[e], yh = (__bf16)y[e];
-        a1[e] = xh;
-        a1[4 + e] = (__bf16)(xt[e] - (float)xh);
-        b1[e] = yh;
-        b1[4 + e] = yh;
-        a2[e] = xh;
-        a2[4 + e] = (__bf16)0.f;
-        b2[e] = (__bf16)(y[e] - (float)yh);
-        b2[4 + e] = (__bf16)0.f;
+        for (int p = 0; p < 2; ++p) {
+            const f32x2 x = {z[2 * p], z[2 * p + 1]};
+            const uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+            const f32x2 rest = {x[0] - __uint_as_float(w << 16), x[1] - __uint_as_float(w & 0xffff0000u)};
+            hw[p] = w;
+            lw[p] = __builtin_bit_cast(uint32_t, __builtin_convertvector(rest, bf16x2));
+        }
+        Op16 o;
+        o.h = __builtin_bit_cast(bf16x4, hw);
+        o.l = __builtin_bit_cast(bf16x4, lw);
+        return o;
     }
-    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1, c, 0, 0, 0);
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2, b2, c, 0, 0, 0);
-}
-
-// bf16 kernels take the split product (their factor is rounded to bf16 anyway), fp32 kernels the exact one
-template <typename T> __device__ __forceinline__ f32x4 mm16_for(const f32x4 &xt, const f32x4 &y, f32x4 c)
-{
-    return sizeof(T) == 2 ? mm16_split(xt, y, c) : mm16(xt, y, c);
-}
+    static __device__ __forceinline__ f32x4 mm(const Op16 &p, const Op16 &q, f32x4 c)
+    {
+        c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(p.h, q.h, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(p.l, q.h, c, 0, 0, 0);
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(p.h, q.l, c, 0, 0, 0);
+    }
+};
 
 // kk[v] = (K K^T)[16b + i][16b + 4g + v] (symmetric); sBeta indexed by chunk row
 template <typename T>
@@ -423,13 +440,16 @@ __device__ __forceinline__ f32x4 tri_diag_block(const f32x4 &kk, const float *sB
         R[v] = M[v] + (r == i ? 1.f : 0.f);
         Rt[v] = Mt[v] + (r == i ? 1.f : 0.f);
     }
+    using Op = Op16<T>;
+    Op oM = Op::of(M), oMt = Op::of(Mt);
 #pragma unroll
     for (int k = 0; k < 3; ++k) {
-        const f32x4 M2 = mm16_for<T>(Mt, M, zero);    // N^2  : X = M,  Y = M
-        const f32x4 M2t = mm16_for<T>(M, Mt, zero);   // (N^2)^T = M^T M^T
-        const f32x4 R2 = mm16_for<T>(Rt, M2, R);      // R + R M2
-        const f32x4 R2t = mm16_for<T>(M2, Rt, Rt);    // R^T + M2^T R^T
-        M = M2; Mt = M2t; R = R2; Rt = R2t;
+        const f32x4 M2 = Op::mm(oMt, oM, zero);       // N^2  : X = M,  Y = M
+        const Op oRt = Op::of(Rt), oM2 = Op::of(M2);
+        R = Op::mm(oRt, oM2, R);                      // R + R M2
+        Rt = Op::mm(oM2, oRt, Rt);                    // R^T + M2^T R^T
+        if (k < 2) oMt = Op::of(Op::mm(oM, oMt, zero));  // (N^2)^T = M^T M^T
+        oM = oM2;
     }
     float *blk = sA + (16 * b) * lda + 16 * b;
 #pragma unroll
@@ -456,13 +476,13 @@ __device__ __forceinline__ void tri_block_column(const float *sA, int lda, T *sX
 #pragma unroll
             for (int kk = 0; kk < r; ++kk) {  // k = c + kk
                 const f32x4 a4 = *reinterpret_cast<const f32x4 *>(sA + (16 * b + i) * lda + 16 * (c + kk) + 4 * g);
-                part[kk] = mm16_for<T>(a4, Xc[kk], zero);
+                part[kk] = Op16<T>::mm(Op16<T>::of(a4), Op16<T>::of(Xc[kk]), zero);
             }
             f32x4 tmp = part[0];
 #pragma unroll
             for (int kk = 1; kk < r; ++kk) tmp += part[kk];
             const f32x4 d4 = *reinterpret_cast<const f32x4 *>(sA + (16 * b + i) * lda + 16 * b + 4 * g);
-            Xc[r] = -mm16_for<T>(d4, tmp, zero);
+            Xc[r] = -Op16<T>::mm(Op16<T>::of(d4), Op16<T>::of(tmp), zero);
 #pragma unroll
             for (int v = 0; v < 4; ++v) sX[(16 * b + 4 * g + v) * ldx + 16 * c + i] = (T)Xc[r][v];
         }

@@ -10,47 +10,6 @@
 
 namespace mrx {
 
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-
-// A 16x16 matrix in accumulator layout (lane (i, g) holds Z[4 g + v][i]) prepared as an MFMA operand.
-template <typename T> struct Op16;
-template <> struct Op16<float> {
-    f32x4 x;
-    static __device__ __forceinline__ Op16 of(const f32x4 &z) { return Op16{z}; }
-    // c + P^T Q for P, Q the matrices whose accumulator layouts were prepared
-    static __device__ __forceinline__ f32x4 mm(const Op16 &p, const Op16 &q, f32x4 c) { return mm16(p.x, q.x, c); }
-};
-template <> struct Op16<__bf16> {
-    bf16x4 h, l;
-    static __device__ __forceinline__ Op16 of(const f32x4 &z)
-    {
-        // pairs, so that each conversion is one packed instruction; the high half is widened
-        // again with a shift or a mask of the packed word
-        typedef float f32x2 __attribute__((ext_vector_type(2)));
-        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-        u32x2 hw, lw;  // whole words: element-wise access would undo the packed conversions
-#pragma unroll
-        for (int p = 0; p < 2; ++p) {
-            const f32x2 x = {z[2 * p], z[2 * p + 1]};
-            const uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
-            const f32x2 rest = {x[0] - __uint_as_float(w << 16), x[1] - __uint_as_float(w & 0xffff0000u)};
-            hw[p] = w;
-            lw[p] = __builtin_bit_cast(uint32_t, __builtin_convertvector(rest, bf16x2));
-        }
-        Op16 o;
-        o.h = __builtin_bit_cast(bf16x4, hw);
-        o.l = __builtin_bit_cast(bf16x4, lw);
-        return o;
-    }
-    static __device__ __forceinline__ f32x4 mm(const Op16 &p, const Op16 &q, f32x4 c)
-    {
-        c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(p.h, q.h, c, 0, 0, 0);
-        c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(p.l, q.h, c, 0, 0, 0);
-        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(p.h, q.l, c, 0, 0, 0);
-    }
-};
-
 template <typename T, bool PRO>
 __global__ void __launch_bounds__(256)
 delta_tm_kernel(const T *__restrict__ k, const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
