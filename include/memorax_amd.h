@@ -157,9 +157,9 @@ int mrx_linear_attn_norm_bwd(void *stream, const void *q, const void *k,
  * kernel first and the sequential kernel reads them (up to a third faster while the device is not
  * full); otherwise the sequential kernel inverts in place.  Both ways fill Tm_chk with the same
  * factors up to rounding.  The environment variable MRX_DELTA_FACTORS (read once per process)
- * overrides the rule: "parallel" takes the chunk-parallel kernel whenever the buffer is given --
- * worth it on a full device too when episodes end every hundred steps or so, which the library
- * cannot see from the host -- and "inline" never does. */
+ * overrides the rule: "parallel" takes the chunk-parallel kernel whenever the buffer is given
+ * (on a full device that is level with the default when episodes end every hundred steps or so,
+ * and slower when resets are rare), "inline" never does. */
 int mrx_delta_rule_fwd(void *stream, const void *q, const void *k,
                        const void *v, const void *beta, const void *done,
                        const void *S0, void *o, void *S_last, void *S_chk,

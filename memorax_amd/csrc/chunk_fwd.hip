@@ -577,9 +577,9 @@ int compute_units()
 }
 
 // MRX_DELTA_FACTORS in the environment overrides the rule below: "parallel" = the chunk-parallel
-// kernel whenever there is a buffer, "inline" = never.  Read once.  For callers who know what the
-// host cannot see: with frequent resets (every hundred steps or so) the chunk-parallel kernel wins
-// on a full device too, because a chunk with resets repeats the in-kernel inverse per episode.
+// kernel whenever there is a buffer, "inline" = never.  Read once.  A tuning knob: the reset rate,
+// which the host cannot see, moves the break-even point (a chunk with resets repeats the in-kernel
+// inverse per episode, the chunk-parallel kernel does that off the sequential path).
 int factor_policy()
 {
     static const int policy = [] {
