@@ -1,0 +1,112 @@
+"""The benchmark configurations at their full sizes, through the C ABI.
+
+The C oracle (fp64 state, OpenMP over the sequences) does configuration 4's whole batch in well
+under a second, so configurations 2, 4 and 5 are compared with it outright; on top of that,
+properties that hold at any size: split invariance (two calls with the carried state equal one),
+linearity of the backward pass in the incoming gradients, the two routes to the triangular factors."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import clib
+from oracle import memoroid as M
+from gpu_util import TOL_BF16, TOL_F32, bf16_round, dev, relerr
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+
+
+def _cfg4(B=64, T=1024, H=8, p_seed=4):
+    x = M.make_inputs(p_seed, (B, T, H, 64))
+    xb = {n: bf16_round(x[n]) for n in ("q", "k", "v", "beta")}
+    do = bf16_round(np.random.default_rng(1).standard_normal(x["v"].shape).astype(np.float32))
+    return x, xb, do
+
+
+def test_config4_delta_rule_full_batch_against_the_c_oracle():
+    from memorax_amd import kernels as K
+    x, xb, do = _cfg4()
+    print("case full cfg4 delta rule fwd+bwd", flush=True)
+    tq, tk, tv, tb, tdo = (dev(a, BF) for a in (xb["q"], xb["k"], xb["v"], xb["beta"], do))
+    dn = dev(x["done"])
+    o, Sl, chk = K.delta_rule_fwd(tq, tk, tv, tb, dn)
+    got = K.delta_rule_bwd(tq, tk, tv, tb, dn, chk, tdo)
+    ro, rSl = clib.delta_rule_fwd(xb["q"], xb["k"], xb["v"], xb["beta"], x["done"])
+    ref = clib.delta_rule_bwd(xb["q"], xb["k"], xb["v"], xb["beta"], x["done"], None, do)
+    errs = {"o": relerr(o, ro), "S_last": relerr(Sl, rSl)}
+    errs.update({n: relerr(g, r) for n, g, r in zip(("dq", "dk", "dv", "dbeta", "dS0"), got, ref)})
+    assert all(e <= TOL_BF16 for e in errs.values()), errs
+
+
+def test_config5_shape_delta_rule_against_the_c_oracle():
+    """One block of configuration 5: 1024 environments x 4 heads, T = 128, resets every hundred steps
+    (more sequences than two per compute unit: the sequential kernel inverts in place)."""
+    from memorax_amd import kernels as K
+    rng = np.random.default_rng(1005)
+    shp = (1024, 128, 4, 64)
+    x = {"q": rng.standard_normal(shp).astype(np.float32), "k": rng.standard_normal(shp).astype(np.float32),
+         "v": rng.standard_normal(shp).astype(np.float32),
+         "beta": (1.0 / (1.0 + np.exp(-rng.standard_normal(shp[:3])))).astype(np.float32),
+         "done": rng.random(shp[:2]) < 0.01}
+    x["k"] /= np.linalg.norm(x["k"], axis=-1, keepdims=True)
+    xb = {n: bf16_round(x[n]) for n in ("q", "k", "v", "beta")}
+    do = bf16_round(np.random.default_rng(2).standard_normal(x["v"].shape).astype(np.float32))
+    print("case full cfg5 delta rule fwd+bwd", flush=True)
+    tq, tk, tv, tb, tdo = (dev(a, BF) for a in (xb["q"], xb["k"], xb["v"], xb["beta"], do))
+    dn = dev(x["done"])
+    o, Sl, chk = K.delta_rule_fwd(tq, tk, tv, tb, dn)
+    got = K.delta_rule_bwd(tq, tk, tv, tb, dn, chk, tdo)
+    ro, rSl = clib.delta_rule_fwd(xb["q"], xb["k"], xb["v"], xb["beta"], x["done"])
+    ref = clib.delta_rule_bwd(xb["q"], xb["k"], xb["v"], xb["beta"], x["done"], None, do)
+    errs = {"o": relerr(o, ro), "S_last": relerr(Sl, rSl)}
+    errs.update({n: relerr(g, r) for n, g, r in zip(("dq", "dk", "dv", "dbeta", "dS0"), got, ref)})
+    assert all(e <= TOL_BF16 for e in errs.values()), errs
+
+
+def test_config2_linear_attention_full_batch_against_the_c_oracle():
+    from memorax_amd import kernels as K
+    x = M.make_inputs(2, (64, 256, 4, 64))
+    do = np.random.default_rng(0).standard_normal(x["v"].shape).astype(np.float32)
+    print("case full cfg2 linear attention fwd+bwd", flush=True)
+    tq, tk, tv, tdo = (dev(a) for a in (x["q"], x["k"], x["v"], do))
+    o, Sl, chk = K.linear_attn_fwd(tq, tk, tv, dev(x["done"]), None, 1)
+    got = K.linear_attn_bwd(tq, tk, tv, dev(x["done"]), chk, tdo, None, 1)
+    ro, rSl = clib.linear_attn_fwd(x["q"], x["k"], x["v"], x["done"], None, 1)
+    ref = clib.linear_attn_bwd(x["q"], x["k"], x["v"], x["done"], None, do, None, 1)
+    errs = {"o": relerr(o, ro), "S_last": relerr(Sl, rSl)}
+    errs.update({n: relerr(g, r) for n, g, r in zip(("dq", "dk", "dv", "dS0"), got, ref)})
+    assert all(e <= TOL_F32 for e in errs.values()), errs
+
+
+def test_config4_split_invariance_is_exact():
+    """Steps [0, 512) and then [512, 1024) from the carried fp32 state give the outputs and the final
+    state of one call bit for bit (the split falls on a chunk boundary)."""
+    from memorax_amd import kernels as K
+    x, xb, _ = _cfg4()
+    tq, tk, tv, tb = (dev(a, BF) for a in (xb["q"], xb["k"], xb["v"], xb["beta"]))
+    dn = dev(x["done"])
+    o, Sl, _ = K.delta_rule_fwd(tq, tk, tv, tb, dn, save_chk=False)
+    h = 512
+    a = [t[:, :h].contiguous() for t in (tq, tk, tv, tb, dn)]
+    b = [t[:, h:].contiguous() for t in (tq, tk, tv, tb, dn)]
+    o1, S1, _ = K.delta_rule_fwd(*a, save_chk=False)
+    o2, S2, _ = K.delta_rule_fwd(*b, S1, save_chk=False)
+    assert torch.equal(torch.cat((o1, o2), dim=1), o) and torch.equal(S2, Sl)
+
+
+def test_config4_backward_is_linear_in_the_incoming_gradients():
+    from memorax_amd import kernels as K
+    x, xb, do = _cfg4()
+    tq, tk, tv, tb = (dev(a, BF) for a in (xb["q"], xb["k"], xb["v"], xb["beta"]))
+    dn = dev(x["done"])
+    g = torch.Generator(device="cuda").manual_seed(9)
+    d1 = dev(do, BF)
+    d2 = torch.randn(d1.shape, device="cuda", generator=g).to(BF)
+    s1 = torch.randn((64, 8, 64, 64), device="cuda", generator=g)
+    s2 = torch.randn((64, 8, 64, 64), device="cuda", generator=g)
+    _, _, chk = K.delta_rule_fwd(tq, tk, tv, tb, dn)
+    ga = K.delta_rule_bwd(tq, tk, tv, tb, dn, chk, d1, s1)
+    gb = K.delta_rule_bwd(tq, tk, tv, tb, dn, chk, d2, s2)
+    gs = K.delta_rule_bwd(tq, tk, tv, tb, dn, chk, (d1.float() + d2.float()).to(BF), s1 + s2)
+    for n, u, v_, w in zip(("dq", "dk", "dv", "dbeta", "dS0"), ga, gb, gs):
+        assert relerr(w, (u.float() + v_.float()).cpu().numpy()) <= TOL_BF16, n
