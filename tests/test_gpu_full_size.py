@@ -110,3 +110,36 @@ def test_config4_backward_is_linear_in_the_incoming_gradients():
     gs = K.delta_rule_bwd(tq, tk, tv, tb, dn, chk, (d1.float() + d2.float()).to(BF), s1 + s2)
     for n, u, v_, w in zip(("dq", "dk", "dv", "dbeta", "dS0"), ga, gb, gs):
         assert relerr(w, (u.float() + v_.float()).cpu().numpy()) <= TOL_BF16, n
+
+
+def test_config3_linear_attention_full_size_properties():
+    """Configuration 3 (B=256, T=4096, H=8, bf16, no resets; 1 GiB per tensor) is too large for the
+    CPU oracle in a test: split invariance (exact) and linearity of the backward at full size, and the
+    first two batch rows against the C oracle."""
+    from memorax_amd import kernels as K
+    B, T, H = 256, 4096, 8
+    g = torch.Generator(device="cuda").manual_seed(1003)
+    q, k, v, d1, d2 = ((torch.randn((B, T, H, 64), device="cuda", generator=g) / 8).to(BF) for _ in range(5))
+    dn = torch.zeros((B, T), device="cuda", dtype=torch.uint8)
+    print("case full cfg3 linear attention", flush=True)
+    o, Sl, chk = K.linear_attn_fwd(q, k, v, dn, None, 0)
+    h = T // 2
+    o1, S1, _ = K.linear_attn_fwd(q[:, :h].contiguous(), k[:, :h].contiguous(), v[:, :h].contiguous(), dn[:, :h].contiguous(),
+                                  None, 0, save_chk=False)
+    o2, S2, _ = K.linear_attn_fwd(q[:, h:].contiguous(), k[:, h:].contiguous(), v[:, h:].contiguous(), dn[:, h:].contiguous(),
+                                  S1, 0, save_chk=False)
+    assert torch.equal(o[:, :h], o1) and torch.equal(o[:, h:], o2) and torch.equal(S2, Sl)
+    del o1, o2
+    ga = K.linear_attn_bwd(q, k, v, dn, chk, d1, None, 0)
+    gb = K.linear_attn_bwd(q, k, v, dn, chk, d2, None, 0)
+    gs = K.linear_attn_bwd(q, k, v, dn, chk, (d1.float() + d2.float()).to(BF), None, 0)
+    for n, u, w_, s_ in zip(("dq", "dk", "dv"), ga, gb, gs):
+        err = float((s_.float() - (u.float() + w_.float())).abs().max() / (u.float() + w_.float()).abs().max())
+        assert err <= TOL_BF16, (n, err)
+    nb = 2
+    xs = [t[:nb].float().cpu().numpy() for t in (q, k, v, d1)]
+    ro, rSl = clib.linear_attn_fwd(xs[0], xs[1], xs[2], np.zeros((nb, T), bool), None, 0)
+    ref = clib.linear_attn_bwd(xs[0], xs[1], xs[2], np.zeros((nb, T), bool), None, xs[3], None, 0)
+    assert relerr(o[:nb], ro) <= TOL_BF16 and relerr(Sl[:nb], rSl) <= TOL_BF16
+    for n, u, r in zip(("dq", "dk", "dv"), ga, ref):
+        assert relerr(u[:nb], r) <= TOL_BF16, n
