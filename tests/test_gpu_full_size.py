@@ -143,3 +143,42 @@ def test_config3_linear_attention_full_size_properties():
     assert relerr(o[:nb], ro) <= TOL_BF16 and relerr(Sl[:nb], rSl) <= TOL_BF16
     for n, u, r in zip(("dq", "dk", "dv"), ga, ref):
         assert relerr(u[:nb], r) <= TOL_BF16, n
+
+
+def test_config5_scan_shape_against_the_oracle():
+    """The diagonal scan at configuration 5's shape (1024, 128, 256), resets every hundred steps:
+    forward and backward against the NumPy oracle (streaming kernels: enough columns to fill the chip)."""
+    from memorax_amd import kernels as K
+    shape = (1024, 128, 256)
+    rng = np.random.default_rng(1005)
+    a = rng.uniform(0.9, 0.999, shape).astype(np.float32)
+    b = rng.standard_normal(shape).astype(np.float32)
+    g = rng.standard_normal(shape).astype(np.float32)
+    done = rng.random(shape[:2]) < 0.01
+    print("case full cfg5 scan", flush=True)
+    h, hl, Pl = K.linear_scan_fwd(dev(a), dev(b), dev(done))
+    rh, rhl, rPl = M.diag_scan(a, b, done)
+    assert relerr(h, rh) <= TOL_F32 and relerr(hl, rhl) <= TOL_F32 and relerr(Pl, rPl) <= TOL_F32
+    da, db, _ = K.linear_scan_bwd(dev(a), h, dev(done), None, dev(g), None)
+    rda, rdb, _ = M.diag_scan_bwd(a, rh, done, g)
+    assert relerr(da, rda) <= TOL_F32 and relerr(db, rdb) <= TOL_F32
+
+
+def test_scan_sweep_shape_properties():
+    """512 x 1024 x 1024 fp32 (2 GiB per tensor), the shape the scan's bandwidth is quoted on: split
+    invariance at full size and one batch row against the oracle."""
+    from memorax_amd import kernels as K
+    B, T, D = 512, 1024, 1024
+    g = torch.Generator(device="cuda").manual_seed(7)
+    a = torch.rand((B, T, D), device="cuda", generator=g) * 0.099 + 0.9
+    b = torch.randn((B, T, D), device="cuda", generator=g)
+    done = torch.rand((B, T), device="cuda", generator=g) < 0.002
+    print("case scan sweep shape", flush=True)
+    h, hl, Pl = K.linear_scan_fwd(a, b, done)
+    s = 500  # not a multiple of anything the kernels block by
+    h1, hl1, Pl1 = K.linear_scan_fwd(a[:, :s].contiguous(), b[:, :s].contiguous(), done[:, :s].contiguous())
+    h2, hl2, Pl2 = K.linear_scan_fwd(a[:, s:].contiguous(), b[:, s:].contiguous(), done[:, s:].contiguous(), hl1, Pl1)
+    err = float((torch.cat((h1, h2), dim=1) - h).abs().max() / h.abs().max())
+    assert err <= 1e-6 and float((hl2 - hl).abs().max()) <= 1e-5 * float(hl.abs().max()), err
+    rh, rhl, rPl = M.diag_scan(a[:1].cpu().numpy(), b[:1].cpu().numpy(), done[:1].cpu().numpy())
+    assert relerr(h[:1], rh) <= TOL_F32 and relerr(hl[:1], rhl) <= TOL_F32 and relerr(Pl[:1], rPl) <= TOL_F32
