@@ -61,9 +61,15 @@ template <> struct TT<__bf16> {
     }
     static __device__ __forceinline__ pack4 pack(float a, float b, float c, float d)
     {
-        pack4 r;
-        r[0] = (__bf16)a; r[1] = (__bf16)b; r[2] = (__bf16)c; r[3] = (__bf16)d;
-        return r;
+        // Two packed conversions on whole words: element-wise conversions compile to four single
+        // converts and two byte permutes.
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+        u32x2 w;
+        w[0] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
+        w[1] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{c, d}, bf16x2));
+        return __builtin_bit_cast(pack4, w);
     }
     static __device__ __forceinline__ frag ones()
     {
