@@ -172,3 +172,42 @@ np.savez(sys.argv[1], o=o.float().cpu().numpy(), Sl=Sl.cpu().numpy(), Tm=chk[1].
     assert not np.array_equal(a["Tm"], b["Tm"])  # two different kernels made the factors
     for n in ("o", "Sl", "Tm"):
         assert relerr(torch.from_numpy(a[n]), b[n]) <= TOL_BF16, n
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("tm_path", ["parallel", "inline"])
+def test_delta_rule_correlated_keys(dtype, tm_path):
+    """Keys that change slowly from step to step (AR(1), rho = 0.95, normalised) and gates near one make
+    I + tril(diag(beta) K K^T) badly conditioned for repeated squaring: the powers of N grow and cancel.
+    Both routes to the triangular factors must hold the tolerance there (forward and backward)."""
+    from memorax_amd import kernels as K
+    from oracle import grad as G
+    B, T, H = 2, 96, 2
+    rng = np.random.default_rng(42)
+    z = rng.standard_normal((B, T, H, 64))
+    for t in range(1, T):
+        z[:, t] = 0.95 * z[:, t - 1] + np.sqrt(1 - 0.95 ** 2) * z[:, t]
+    k = (z / np.linalg.norm(z, axis=-1, keepdims=True)).astype(np.float32)
+    q = rng.standard_normal((B, T, H, 64)).astype(np.float32)
+    v = rng.standard_normal((B, T, H, 64)).astype(np.float32)
+    beta = rng.uniform(0.5, 1.0, (B, T, H)).astype(np.float32)
+    do = rng.standard_normal((B, T, H, 64)).astype(np.float32)
+    done = np.zeros((B, T), bool)
+    done[1, 40] = True
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    if dtype == "bf16":
+        q, k, v, beta, do = (bf16_round(a) for a in (q, k, v, beta, do))
+    print(f"case correlated keys dtype={dtype} path={tm_path}", flush=True)
+    tq, tk, tv, tb, tdo = (dev(a, td) for a in (q, k, v, beta, do))
+    if tm_path == "parallel":
+        o, Sl, chk = K.delta_rule_fwd(tq, tk, tv, tb, dev(done))
+    else:
+        o, Sl, _ = K.delta_rule_fwd(tq, tk, tv, tb, dev(done), save_chk=False, tm_scratch=False)
+        chk = None
+    ref = G.delta_rule_grads(q, k, v, beta, done, None, do)
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    assert relerr(o, ref["o"]) <= tol and relerr(Sl, ref["S_last"]) <= tol, (relerr(o, ref["o"]), relerr(Sl, ref["S_last"]))
+    if chk is not None:
+        got = K.delta_rule_bwd(tq, tk, tv, tb, dev(done), chk, tdo)
+        errs = {n: relerr(g, ref[n]) for n, g in zip(("dq", "dk", "dv", "dbeta", "dS0"), got)}
+        assert all(e <= tol for e in errs.values()), errs
