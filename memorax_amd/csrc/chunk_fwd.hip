@@ -605,7 +605,7 @@ int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void 
 {
     static_assert(DELTA_BF16_CHUNK == 32, "delta_tm_kernel is written for 32-row chunks");
     const int policy = factor_policy();
-    if (Tm_chk && policy != 2 && (policy == 1 || B * H <= 2 * (int64_t)compute_units())) {
+    if (Tm_chk && policy != 2 && T <= DELTA_TM_MAX_T && (policy == 1 || B * H <= 2 * (int64_t)compute_units())) {
         const int rc = launch_delta_tm(st, k, beta, done, done_dtype, Tm_chk, B, T, H, dtype, PRO);
         if (rc != MRX_OK) return rc;
         if (dtype == MRX_BF16)

@@ -79,3 +79,23 @@ def test_diagonal_scan_beyond_32_bit_offsets():
     errs = {"h": relerr(h[-NB:], rh), "h_last": relerr(hl[-NB:], rhl), "P_last": relerr(Pl[-NB:], rPl),
             "da": relerr(da[-NB:], rda), "db": relerr(db[-NB:], rdb), "last": relerr(last[-NB:], rhl)}
     assert all(e <= TOL_F32 for e in errs.values()), errs
+
+
+def test_delta_rule_sequence_longer_than_the_factor_kernel_covers():
+    """One sequence of more steps than the chunk-parallel factor kernel's grid covers: the call falls
+    back to the in-kernel inverse instead of failing, and since the recurrence is causal its first
+    steps equal a call on those steps alone (same kernel, bit for bit)."""
+    from memorax_amd import kernels as K
+    T, n = 4 * 65535 * 32 + 32, 2048
+    g = torch.Generator(device="cuda").manual_seed(34)
+    print("case long sequence delta rule", T, flush=True)
+    q, v = (torch.randn((1, T, 1, 64), device="cuda", generator=g).to(BF) for _ in range(2))
+    k = torch.nn.functional.normalize(torch.randn((1, T, 1, 64), device="cuda", generator=g), dim=-1).to(BF)
+    beta = torch.sigmoid(torch.randn((1, T, 1), device="cuda", generator=g)).to(BF)
+    done = torch.rand((1, T), device="cuda", generator=g) < 0.002
+    o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(o.float()).all()) and bool(torch.isfinite(Sl).all())
+    o1, _, _ = K.delta_rule_fwd(q[:, :n].contiguous(), k[:, :n].contiguous(), v[:, :n].contiguous(),
+                                beta[:, :n].contiguous(), done[:, :n].contiguous(), save_chk=False, tm_scratch=False)
+    assert torch.equal(o[:, :n], o1)
