@@ -674,7 +674,7 @@ class mLSTM(SequenceModel):
 
 
 # ----------------------------------------------------------------------------------
-# block composition used by the torso configuration (blocks/{stack,residual,normalization}.py)
+# block composition used by the torso configuration (blocks/{stack,residual,normalization,ffn}.py)
 # ----------------------------------------------------------------------------------
 class PreNorm(nn.Module):
     """normalization.py:10-35: norm, then the wrapped sequence model."""
@@ -705,6 +705,69 @@ class Residual(nn.Module):
         return self.module.initialize_carry(key, input_shape)
 
 
+class GatedResidual(nn.Module):
+    """residual.py:33-63: x + gate(Dense(x)) * module(x), the gate a dense layer of the block's width
+    (with bias) on the block's input."""
+
+    def __init__(self, module, dim, gate=torch.sigmoid):
+        super().__init__()
+        self.module, self.gate, self.gate_fn = module, nn.Linear(dim, dim), gate
+
+    def forward(self, inputs, done=None, initial_carry=None, **kwargs):
+        carry, y = self.module(inputs, done, initial_carry, **kwargs)
+        return carry, inputs + self.gate_fn(self.gate(inputs)) * y
+
+    def initialize_carry(self, key, input_shape):
+        return self.module.initialize_carry(key, input_shape)
+
+
+class _Stateless(nn.Module):
+    """Blocks without a recurrence (blocks/base.py:6-21): the carry is None on the way in and out."""
+
+    def initialize_carry(self, key, input_shape):
+        return None
+
+
+class FFN(_Stateless):
+    """ffn.py:11-50: Dense -> activation -> dropout -> Dense, hidden width features * expansion_factor."""
+
+    def __init__(self, features, expansion_factor=4, activation=F.gelu, dropout_rate=0.0):
+        super().__init__()
+        self.up = nn.Linear(features, features * expansion_factor)
+        self.down = nn.Linear(features * expansion_factor, features)
+        self.activation, self.dropout = activation, nn.Dropout(dropout_rate)
+
+    def forward(self, inputs, done=None, initial_carry=None, **kwargs):
+        return None, self.down(self.dropout(self.activation(self.up(inputs))))
+
+
+class Projection(_Stateless):
+    """ffn.py:53-79: a single dense layer."""
+
+    def __init__(self, in_features, features, use_bias=True):
+        super().__init__()
+        self.proj = nn.Linear(in_features, features, bias=use_bias)
+
+    def forward(self, inputs, done=None, initial_carry=None, **kwargs):
+        return None, self.proj(inputs)
+
+
+class GLU(_Stateless):
+    """ffn.py:82-123: up_proj to 2 * hidden, split into (gate, value) in that order,
+    activation(gate) * value, dropout, down_proj; no biases by default."""
+
+    def __init__(self, features, expansion_factor=4, activation=F.gelu, dropout_rate=0.0, use_bias=False):
+        super().__init__()
+        hidden = features * expansion_factor
+        self.up_proj = nn.Linear(features, 2 * hidden, bias=use_bias)
+        self.down_proj = nn.Linear(hidden, features, bias=use_bias)
+        self.activation, self.dropout = activation, nn.Dropout(dropout_rate)
+
+    def forward(self, inputs, done=None, initial_carry=None, **kwargs):
+        gate, value = self.up_proj(inputs).chunk(2, dim=-1)
+        return None, self.down_proj(self.dropout(self.activation(gate) * value))
+
+
 class Stack(nn.Module):
     """stack.py:10-60: one carry per block, threaded as a tuple."""
 
@@ -722,4 +785,5 @@ class Stack(nn.Module):
         return tuple(carries), x
 
     def initialize_carry(self, key, input_shape):
-        return tuple(b.initialize_carry(key, input_shape) for b in self.blocks)
+        return tuple(b.initialize_carry(key, input_shape) if hasattr(b, "initialize_carry") else None
+                     for b in self.blocks)
