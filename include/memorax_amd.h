@@ -207,6 +207,29 @@ int mrx_linear_scan_last(void *stream, const void *a, const void *b,
                          int64_t T, int64_t D, int64_t a_group, int dtype,
                          int done_dtype);
 
+/* ---- MinGRU: the diagonal scan with the cell's gate arithmetic inside ----
+ * MinGRUCell (min_gru.py:49-78) maps the step's two projections z and h~ to the elements
+ * (log sigma(z) + log g(h~), log sigma(-z)), g(x) = x + 0.5 (x >= 0) | sigma(x), scans them with the
+ * log-space operator (logaddexp(decay_j + state_i, state_j), decay_i + decay_j) through
+ * Memoroid.scan_fn (memoroid.py:60-91) and reads exp(state).  In linear space that is
+ *     h_t = done_t ? b_t : a_t h_{t-1} + b_t ,   a_t = sigma(-z_t),  b_t = sigma(z_t) g(h~_t),
+ * which these entry points compute from z and h~ directly: a and b are never written to memory,
+ * and the backward call returns dL/dz and dL/dh~ instead of dL/da and dL/db.
+ * z, h_tilde, h, g, dz, dh_tilde: (B,T,D) fp32.  h0, P0 (nullable), h_last, P_last (nullable),
+ * g_last (nullable), dh0 (nullable): (B,D) fp32, linear space: h0 = exp(carried log state) (0 for
+ * the cell's initial -inf), P = the cumulative decay since the last reset, whose log is the carry's
+ * second leaf (a product below the fp32 range underflows to 0, i.e. a log of -inf; the leaf never
+ * reaches h).  No counterpart as one function in the reference (which leaves the fusion to XLA). */
+int mrx_mingru_scan_fwd(void *stream, const void *z, const void *h_tilde, const void *done,
+                        const void *h0, const void *P0, void *h, void *h_last, void *P_last,
+                        int64_t B, int64_t T, int64_t D, int done_dtype);
+
+/* h: the states the forward call wrote.  dz, dh_tilde: gradients with respect to the projections. */
+int mrx_mingru_scan_bwd(void *stream, const void *z, const void *h_tilde, const void *h,
+                        const void *done, const void *h0, const void *g, const void *g_last,
+                        void *dz, void *dh_tilde, void *dh0, int64_t B, int64_t T, int64_t D,
+                        int done_dtype);
+
 /* ---- Gated linear attention: linear attention with a scalar decay per step and head ----
  * The Mamba cell's algebra (mamba.py:109-122: elements (h_t = (B_t dt_t) (x) x_t, decay_t =
  * exp(dt_t A)), binary_operator (decay_j h_i + h_j, decay_j decay_i), read y_t = C_t . h_t), scanned

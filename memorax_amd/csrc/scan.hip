@@ -9,6 +9,7 @@
 // summaries to its left into a carry-in and fixes its slice up by *select*
 // (a reset inside the slice wins over the carry, so NaN/Inf never cross a reset).
 // One pass over HBM in either case.
+#include <initializer_list>
 #include <type_traits>
 
 #include "common.h"
@@ -56,11 +57,49 @@ template <typename E, int VEC> __device__ __forceinline__ Vec<E, VEC> vfill(E x)
     return r;
 }
 
+// MinGRU in linear space.  The reference scans (log h, log decay) with logaddexp
+// (min_gru.py:49-78); the same recurrence is h_t = a_t h_{t-1} + b_t with, from the step's two
+// projections z and x = h~:  a = sigma(-z),  b = sigma(z) g(x),  g(x) = x + 0.5 (x >= 0) | sigma(x).
+// The kernels below take z and x in place of a and b when MG is set, so the coefficients never
+// exist in memory; the backward kernels then emit dz and dx instead of da and db.
+struct MinGru {
+    // s = sigma(z) and a = sigma(-z), each from exp(-|z|): neither is 1 - the other, so a small
+    // gate keeps its relative precision (the cumulative decay is a product of them)
+    static __device__ __forceinline__ void gates(float z, float &s, float &a)
+    {
+        const float e = expf(-fabsf(z)), r = 1.0f / (1.0f + e), q = e * r;
+        s = z >= 0.0f ? r : q;
+        a = z >= 0.0f ? q : r;
+    }
+    static __device__ __forceinline__ float g(float x) { return x >= 0.0f ? x + 0.5f : 1.0f / (1.0f + expf(-x)); }
+    static __device__ __forceinline__ float dg(float x)
+    {
+        const float sx = 1.0f / (1.0f + expf(-x));
+        return x >= 0.0f ? 1.0f : sx * (1.0f - sx);
+    }
+    // (z, x) -> (a, b) in place
+    static __device__ __forceinline__ void coeffs(float &za, float &xb)
+    {
+        float s, a;
+        gates(za, s, a);
+        xb = s * g(xb);
+        za = a;
+    }
+    // gradients of one step: lam = dL/db_t, da = dL/da_t (0 at a reset) -> dz, dx
+    static __device__ __forceinline__ void grads(float z, float x, float lam, float da, float &dz, float &dx)
+    {
+        float s, a;
+        gates(z, s, a);
+        dz = s * a * (g(x) * lam - da);  // sigma'(z) = s a; b = s g(x), a = 1 - s
+        dx = lam * s * dg(x);
+    }
+};
+
 constexpr int TS = 8;  // time steps a wave holds in registers per super-step
 
 // Forward.  grid = B * tiles workgroups, block = 64 * NW threads.
 // smem: sH[2][NW][64] Vec, sP[2][NW][64] Vec, sF[2][NW] int.
-template <typename E, int VEC>
+template <typename E, int VEC, bool MG = false>
 __global__ void __launch_bounds__(512)
 diag_scan_fwd_kernel(const E *__restrict__ a, const E *__restrict__ b,
                      const void *__restrict__ done, int done_f32,
@@ -103,6 +142,10 @@ diag_scan_fwd_kernel(const E *__restrict__ a, const E *__restrict__ b,
                 const int64_t off = (row0 + t) * D + col;
                 p[s] = *reinterpret_cast<const V *>(a + (a_ti ? col : off));
                 x[s] = *reinterpret_cast<const V *>(b + off);
+                if constexpr (MG) {
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) MinGru::coeffs(p[s].v[i], x[s].v[i]);
+                }
             } else {
                 p[s] = vfill<E, VEC>(O::one());
                 x[s] = vfill<E, VEC>(O::zero());
@@ -186,9 +229,10 @@ diag_scan_fwd_kernel(const E *__restrict__ a, const E *__restrict__ b,
 
 // Backward: the same scan walked from t = T-1 down with coefficient conj(a_{t+1}),
 // cut where done_{t+1}; reversed index r = T-1-t runs forward.
-template <typename E, int VEC>
+// MG: a holds z, hx holds x = h~; da receives dz and db receives dx.
+template <typename E, int VEC, bool MG = false>
 __global__ void __launch_bounds__(512)
-diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hfw,
+diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hx, const E *__restrict__ hfw,
                      const void *__restrict__ done, int done_f32,
                      const E *__restrict__ h0, const E *__restrict__ g,
                      const E *__restrict__ g_last, E *__restrict__ da,
@@ -232,7 +276,14 @@ diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hfw,
                     if (t + 1 < T) {
                         V av = *reinterpret_cast<const V *>(a + (a_ti ? col : off + D));
 #pragma unroll
-                        for (int i = 0; i < VEC; ++i) p[s].v[i] = O::conj(av.v[i]);
+                        for (int i = 0; i < VEC; ++i) {
+                            if constexpr (MG) {
+                                float sg;
+                                MinGru::gates(av.v[i], sg, p[s].v[i]);
+                            } else {
+                                p[s].v[i] = O::conj(av.v[i]);
+                            }
+                        }
                     }
                 }
                 if (t + 1 < T && done_at(done, done_f32, row0 + t + 1)) cmask |= 1u << s;
@@ -312,15 +363,31 @@ diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hfw,
                     const E prod = O::mul(x[s].v[i], O::conj(hp.v[i]));
                     o.v[i] = dn ? O::zero() : prod;
                 }
-                *reinterpret_cast<V *>(db + off) = x[s];
-                *reinterpret_cast<V *>(da + off) = o;
+                if constexpr (MG) {
+                    const V zt = *reinterpret_cast<const V *>(a + off), xt = *reinterpret_cast<const V *>(hx + off);
+                    V oz, ox;
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) MinGru::grads(zt.v[i], xt.v[i], x[s].v[i], o.v[i], oz.v[i], ox.v[i]);
+                    *reinterpret_cast<V *>(db + off) = ox;
+                    *reinterpret_cast<V *>(da + off) = oz;
+                } else {
+                    *reinterpret_cast<V *>(db + off) = x[s];
+                    *reinterpret_cast<V *>(da + off) = o;
+                }
             }
         }
     }
     if (w == 0 && act && dh0) {
         // carry = lam_0 ; dh0 = done_0 ? 0 : conj(a_0) lam_0
         const bool d0 = done_at(done, done_f32, row0);
-        const V a0 = *reinterpret_cast<const V *>(a + (a_ti ? col : row0 * D + col));
+        V a0 = *reinterpret_cast<const V *>(a + (a_ti ? col : row0 * D + col));
+        if constexpr (MG) {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                float sg;
+                MinGru::gates(a0.v[i], sg, a0.v[i]);
+            }
+        }
         V o;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
@@ -337,7 +404,7 @@ diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hfw,
 // with the loads of the next group issued before the current group is consumed
 // (register double buffering), so a wave always has 2*SG (forward) / 3*SG (backward)
 // row loads in flight.  done flags are prefetched as raw bits with the data.
-template <typename E, int VEC, int SG>
+template <typename E, int VEC, int SG, bool MG = false>
 __global__ void __launch_bounds__(256)
 diag_scan_fwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ b,
                             const void *__restrict__ done, int done_f32,
@@ -379,6 +446,10 @@ diag_scan_fwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ b,
         for (int s = 0; s < SG; ++s) {
             if (t0 + s < T) {
                 const bool r = done_test(xd[s], done_f32);
+                if constexpr (MG) {  // here, not at the load: the loads stay in flight
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) MinGru::coeffs(xa[s].v[i], xb[s].v[i]);
+                }
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) {
                     const E hn = O::madd(xa[s].v[i], ch.v[i], xb[s].v[i]);
@@ -453,9 +524,10 @@ diag_scan_last_kernel(const E *__restrict__ a, const E *__restrict__ b, const vo
     *reinterpret_cast<V *>(h_last + bi * D + col) = ch;
 }
 
-template <typename E, int VEC, int SG>
+// MG: a holds z, hx holds x = h~ (a fourth load per step); da receives dz and db receives dx.
+template <typename E, int VEC, int SG, bool MG = false>
 __global__ void __launch_bounds__(256)
-diag_scan_bwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ hfw,
+diag_scan_bwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ hx, const E *__restrict__ hfw,
                             const void *__restrict__ done, int done_f32,
                             const E *__restrict__ h0, const E *__restrict__ g,
                             const E *__restrict__ g_last, E *__restrict__ da, E *__restrict__ db,
@@ -473,8 +545,9 @@ diag_scan_bwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ hfw,
 
     // step r (reversed index), t = T-1-r: needs g_t, a_t (for the carry to t-1), h_{t-1}, done_t
     V xg[SG], xa[SG], xh[SG], ng[SG], na[SG], nh[SG];
+    V xx[MG ? SG : 1], nx[MG ? SG : 1];
     uint32_t xd[SG], nd[SG];
-    auto load = [&](int r0, V *pg, V *pa, V *ph, uint32_t *pd) {
+    auto load = [&](int r0, V *pg, V *pa, V *ph, V *px, uint32_t *pd) {
 #pragma unroll
         for (int s = 0; s < SG; ++s) {
             const int t = T - 1 - (r0 + s);
@@ -484,15 +557,16 @@ diag_scan_bwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ hfw,
                 const int64_t off = (row0 + t) * D + col;
                 pg[s] = *reinterpret_cast<const V *>(g + off);
                 pa[s] = *reinterpret_cast<const V *>(a + (a_ti ? col : off));
+                if constexpr (MG) px[s] = *reinterpret_cast<const V *>(hx + off);
                 if (t > 0) ph[s] = *reinterpret_cast<const V *>(hfw + off - D);
                 else if (h0) ph[s] = *reinterpret_cast<const V *>(h0 + bi * D + col);
                 pd[s] = done_raw(done, done_f32, row0 + t);
             }
         }
     };
-    load(0, xg, xa, xh, xd);
+    load(0, xg, xa, xh, xx, xd);
     for (int r0 = 0; r0 < T; r0 += SG) {
-        if (r0 + SG < T) load(r0 + SG, ng, na, nh, nd);
+        if (r0 + SG < T) load(r0 + SG, ng, na, nh, nx, nd);
 #pragma unroll
         for (int s = 0; s < SG; ++s) {
             const int t = T - 1 - (r0 + s);
@@ -505,8 +579,17 @@ diag_scan_bwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ hfw,
                     l.v[i] = O::madd(O::one(), xg[s].v[i], lam.v[i]);  // lam_t = g_t + carried term
                     const E prod = O::mul(l.v[i], O::conj(xh[s].v[i]));
                     o.v[i] = dn ? O::zero() : prod;
-                    const E nxt = O::mul(O::conj(xa[s].v[i]), l.v[i]);
-                    lam.v[i] = dn ? O::zero() : nxt;               // conj(abar_t) lam_t for step t-1
+                    if constexpr (MG) {
+                        float sg, at, dz, dx;
+                        MinGru::gates(xa[s].v[i], sg, at);
+                        MinGru::grads(xa[s].v[i], xx[s].v[i], l.v[i], o.v[i], dz, dx);
+                        lam.v[i] = dn ? 0.0f : at * l.v[i];
+                        o.v[i] = dz;
+                        l.v[i] = dx;
+                    } else {
+                        const E nxt = O::mul(O::conj(xa[s].v[i]), l.v[i]);
+                        lam.v[i] = dn ? O::zero() : nxt;           // conj(abar_t) lam_t for step t-1
+                    }
                 }
                 *reinterpret_cast<V *>(db + off) = l;
                 *reinterpret_cast<V *>(da + off) = o;
@@ -514,6 +597,10 @@ diag_scan_bwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ hfw,
         }
 #pragma unroll
         for (int s = 0; s < SG; ++s) { xg[s] = ng[s]; xa[s] = na[s]; xh[s] = nh[s]; xd[s] = nd[s]; }
+        if constexpr (MG) {
+#pragma unroll
+            for (int s = 0; s < SG; ++s) xx[s] = nx[s];
+        }
     }
     if (dh0) *reinterpret_cast<V *>(dh0 + bi * D + col) = lam;  // conj(abar_0) lam_0
 }
@@ -567,7 +654,8 @@ template <typename E, typename F> void vec_switch(int vec, F f)
     }
 }
 
-template <typename E>
+// MG (E = float): a and b hold the MinGRU projections z and h~.
+template <typename E, bool MG = false>
 int launch_fwd(hipStream_t st, const void *a, const void *b, const void *done,
                int done_f32, const void *h0, const void *P0, void *h, void *h_last,
                void *P_last, int64_t B, int64_t T, int64_t D, int a_ti)
@@ -582,7 +670,7 @@ int launch_fwd(hipStream_t st, const void *a, const void *b, const void *done,
         const dim3 grid((unsigned)((B * cpr + 255) / 256)), block(256);
         vec_switch<E>(pl.vec, [&](auto vc) {
             constexpr int VEC = decltype(vc)::value;
-            hipLaunchKernelGGL((diag_scan_fwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8)>), grid, block, 0, st,
+            hipLaunchKernelGGL((diag_scan_fwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8), MG>), grid, block, 0, st,
                                (const E *)a, (const E *)b, done, done_f32, (const E *)h0, (const E *)P0,
                                (E *)h, (E *)h_last, (E *)P_last, B, (int)T, D, cpr, a_ti);
         });
@@ -591,7 +679,7 @@ int launch_fwd(hipStream_t st, const void *a, const void *b, const void *done,
         const size_t smem = scan_smem(pl.nw, sizeof(E) * pl.vec);
         vec_switch<E>(pl.vec, [&](auto vc) {
             constexpr int VEC = decltype(vc)::value;
-            hipLaunchKernelGGL((diag_scan_fwd_kernel<E, VEC>), grid, block, smem, st, (const E *)a,
+            hipLaunchKernelGGL((diag_scan_fwd_kernel<E, VEC, MG>), grid, block, smem, st, (const E *)a,
                                (const E *)b, done, done_f32, (const E *)h0, (const E *)P0, (E *)h,
                                (E *)h_last, (E *)P_last, (int)T, D, pl.tiles, pl.nw, a_ti);
         });
@@ -599,14 +687,15 @@ int launch_fwd(hipStream_t st, const void *a, const void *b, const void *done,
     return launch_status();
 }
 
-template <typename E>
-int launch_bwd(hipStream_t st, const void *a, const void *h, const void *done,
+// MG (E = float): a holds z, hx holds h~ (else unused), da and db receive dz and dh~.
+template <typename E, bool MG = false>
+int launch_bwd(hipStream_t st, const void *a, const void *hx, const void *h, const void *done,
                int done_f32, const void *h0, const void *g, const void *g_last, void *da,
                void *db, void *dh0, int64_t B, int64_t T, int64_t D, int a_ti)
 {
-    const bool al16 = aligned(a, 16) && aligned(h, 16) && aligned(g, 16) && aligned(h0, 16) &&
+    const bool al16 = aligned(a, 16) && aligned(hx, 16) && aligned(h, 16) && aligned(g, 16) && aligned(h0, 16) &&
                       aligned(g_last, 16) && aligned(da, 16) && aligned(db, 16) && aligned(dh0, 16);
-    const bool al8 = aligned(a, 8) && aligned(h, 8) && aligned(g, 8) && aligned(h0, 8) &&
+    const bool al8 = aligned(a, 8) && aligned(hx, 8) && aligned(h, 8) && aligned(g, 8) && aligned(h0, 8) &&
                      aligned(g_last, 8) && aligned(da, 8) && aligned(db, 8) && aligned(dh0, 8);
     const ScanPlan pl = plan_scan(B, T, D, sizeof(E), al16, al8, true);
     if (pl.stream) {
@@ -614,8 +703,8 @@ int launch_bwd(hipStream_t st, const void *a, const void *h, const void *done,
         const dim3 grid((unsigned)((B * cpr + 255) / 256)), block(256);
         vec_switch<E>(pl.vec, [&](auto vc) {
             constexpr int VEC = decltype(vc)::value;
-            hipLaunchKernelGGL((diag_scan_bwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8)>), grid, block, 0, st,
-                               (const E *)a, (const E *)h, done, done_f32, (const E *)h0, (const E *)g,
+            hipLaunchKernelGGL((diag_scan_bwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8), MG>), grid, block, 0, st,
+                               (const E *)a, (const E *)hx, (const E *)h, done, done_f32, (const E *)h0, (const E *)g,
                                (const E *)g_last, (E *)da, (E *)db, (E *)dh0, B, (int)T, D, cpr, a_ti);
         });
     } else {
@@ -623,8 +712,8 @@ int launch_bwd(hipStream_t st, const void *a, const void *h, const void *done,
         const size_t smem = scan_smem(pl.nw, sizeof(E) * pl.vec);
         vec_switch<E>(pl.vec, [&](auto vc) {
             constexpr int VEC = decltype(vc)::value;
-            hipLaunchKernelGGL((diag_scan_bwd_kernel<E, VEC>), grid, block, smem, st, (const E *)a,
-                               (const E *)h, done, done_f32, (const E *)h0, (const E *)g,
+            hipLaunchKernelGGL((diag_scan_bwd_kernel<E, VEC, MG>), grid, block, smem, st, (const E *)a,
+                               (const E *)hx, (const E *)h, done, done_f32, (const E *)h0, (const E *)g,
                                (const E *)g_last, (E *)da, (E *)db, (E *)dh0, (int)T, D, pl.tiles,
                                pl.nw, a_ti);
         });
@@ -702,13 +791,13 @@ extern "C" int mrx_linear_scan_bwd(void *stream, const void *a, const void *h, c
     if (dtype == MRX_F32) {
         if (!aligned(a, 4) || !aligned(h, 4) || !aligned(g, 4) || !aligned(da, 4) || !aligned(db, 4))
             return MRX_ERR_INVALID_ARG;
-        return launch_bwd<float>(st, a, h, done, done_dtype, h0, g, g_last, da, db, dh0, B, T, D, ti);
+        return launch_bwd<float>(st, a, nullptr, h, done, done_dtype, h0, g, g_last, da, db, dh0, B, T, D, ti);
     }
     if (dtype == MRX_C64) {
         if (!aligned(a, 8) || !aligned(h, 8) || !aligned(g, 8) || !aligned(da, 8) ||
             !aligned(db, 8) || !aligned(h0, 8) || !aligned(g_last, 8) || !aligned(dh0, 8))
             return MRX_ERR_INVALID_ARG;
-        return launch_bwd<c64>(st, a, h, done, done_dtype, h0, g, g_last, da, db, dh0, B, T, D, ti);
+        return launch_bwd<c64>(st, a, nullptr, h, done, done_dtype, h0, g, g_last, da, db, dh0, B, T, D, ti);
     }
     return dtype == MRX_BF16 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
 }
@@ -732,4 +821,33 @@ extern "C" int mrx_linear_scan_last(void *stream, const void *a, const void *b, 
         return launch_last<c64>(st, a, b, done, done_dtype, h0, h_last, B, T, D, a_group);
     }
     return dtype == MRX_BF16 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
+}
+
+extern "C" int mrx_mingru_scan_fwd(void *stream, const void *z, const void *h_tilde, const void *done,
+                                   const void *h0, const void *P0, void *h, void *h_last, void *P_last,
+                                   int64_t B, int64_t T, int64_t D, int done_dtype)
+{
+    if (!z || !h_tilde || !done || !h) return MRX_ERR_INVALID_ARG;
+    if (!scan_shape_ok(B, T, D)) return MRX_ERR_INVALID_ARG;
+    if (done_dtype != MRX_DONE_U8 && done_dtype != MRX_DONE_F32) return MRX_ERR_INVALID_ARG;
+    if (done_dtype == MRX_DONE_F32 && !aligned(done, 4)) return MRX_ERR_INVALID_ARG;
+    for (const void *p : {z, h_tilde, h0, P0, (const void *)h, (const void *)h_last, (const void *)P_last})
+        if (!aligned(p, 4)) return MRX_ERR_INVALID_ARG;
+    return launch_fwd<float, true>((hipStream_t)stream, z, h_tilde, done, done_dtype, h0, P0, h, h_last, P_last, B, T,
+                                   D, 0);
+}
+
+extern "C" int mrx_mingru_scan_bwd(void *stream, const void *z, const void *h_tilde, const void *h,
+                                   const void *done, const void *h0, const void *g, const void *g_last,
+                                   void *dz, void *dh_tilde, void *dh0, int64_t B, int64_t T, int64_t D,
+                                   int done_dtype)
+{
+    if (!z || !h_tilde || !h || !done || !g || !dz || !dh_tilde) return MRX_ERR_INVALID_ARG;
+    if (!scan_shape_ok(B, T, D)) return MRX_ERR_INVALID_ARG;
+    if (done_dtype != MRX_DONE_U8 && done_dtype != MRX_DONE_F32) return MRX_ERR_INVALID_ARG;
+    if (done_dtype == MRX_DONE_F32 && !aligned(done, 4)) return MRX_ERR_INVALID_ARG;
+    for (const void *p : {z, h_tilde, h, h0, g, g_last, (const void *)dz, (const void *)dh_tilde, (const void *)dh0})
+        if (!aligned(p, 4)) return MRX_ERR_INVALID_ARG;
+    return launch_bwd<float, true>((hipStream_t)stream, z, h_tilde, h, done, done_dtype, h0, g, g_last, dz, dh_tilde,
+                                   dh0, B, T, D, 0);
 }

@@ -2,6 +2,7 @@
 the role jax.custom_vjp would in a JAX host).
 
     linear_scan(a, b, done, h0=None, P0=None)            -> (h, h_last, P_last)
+    mingru_scan(z, h_tilde, done, h0=None, P0=None)      -> (h, h_last, P_last)  (gates fused)
     linear_attention(q, k, v, done, S0=None, feature_map) -> (o, S_last)
     delta_rule(q, k, v, beta, done, S0=None)             -> (o, S_last)
     deltanet(q, k, v, beta_raw, done, S0=None)           -> (o, S_last)   (key L2-norm and sigmoid fused)
@@ -115,6 +116,41 @@ def linear_scan(a, b, done, h0=None, P0=None):
     by memoroid.py:60-91).  a: (B,T,D) or (D,); b: (B,T,D); h0,P0: (B,D).
     P_last (the cumulative-decay leaf of the carry) is not differentiable."""
     return _LinearScan.apply(a, b, done, h0, P0)
+
+
+class _MinGRUScan(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, z, h_tilde, done, h0, P0):
+        z_, x_ = z.contiguous(), h_tilde.contiguous()
+        h0_ = None if h0 is None else h0.contiguous()
+        P0_ = None if P0 is None else P0.contiguous()
+        h, h_last, P_last = K.mingru_scan_fwd(z_, x_, done, h0_, P0_)
+        ctx.save_for_backward(z_, x_, h, h0_ if h0_ is not None else torch.empty(0, device=z.device))
+        ctx.done = done
+        ctx.has_h0 = h0 is not None
+        ctx.mark_non_differentiable(P_last)
+        return h, h_last, P_last
+
+    @staticmethod
+    def backward(ctx, g, g_last, _gP):
+        z, x, h, h0 = ctx.saved_tensors
+        h0 = h0 if ctx.has_h0 else None
+        g = torch.zeros_like(h) if g is None else g.contiguous()
+        g_last = None if g_last is None else g_last.contiguous()
+        dz, dx, dh0 = K.mingru_scan_bwd(z, x, h, ctx.done, h0, g, g_last)
+        return (dz if ctx.needs_input_grad[0] else None,
+                dx if ctx.needs_input_grad[1] else None,
+                None,
+                dh0 if (ctx.has_h0 and ctx.needs_input_grad[3]) else None,
+                None)
+
+
+def mingru_scan(z, h_tilde, done, h0=None, P0=None):
+    """MinGRU from its two projections (min_gru.py:49-78 scanned by memoroid.py:60-91), linear space:
+    h_t = sigmoid(-z_t) h_{t-1} + sigmoid(z_t) g(h~_t), g(x) = x + 0.5 (x >= 0) | sigmoid(x), with the
+    gate arithmetic inside the scan kernels.  z, h_tilde: (B,T,D) fp32; h0, P0: (B,D).
+    Returns (h, h_last, P_last); P_last is not differentiable."""
+    return _MinGRUScan.apply(z, h_tilde, done, h0, P0)
 
 
 class _LinearAttention(torch.autograd.Function):

@@ -125,6 +125,45 @@ def linear_scan_bwd(a, h, done, h0, g, g_last=None):
     return da, db, dh0
 
 
+def mingru_scan_fwd(z, h_tilde, done, h0=None, P0=None, want_P=True):
+    """MinGRU recurrence from its two projections (min_gru.py:49-78, in linear space):
+    h_t = done ? b_t : a_t h_{t-1} + b_t with a = sigmoid(-z), b = sigmoid(z) g(h~) formed inside
+    the kernel.  z, h_tilde: (B,T,D) fp32; h0, P0: (B,D) linear space.  Returns (h, h_last, P_last)."""
+    lib = _lib.load()
+    B, T, D = z.shape
+    if z.dtype != torch.float32:
+        raise ValueError("mingru_scan supports float32")
+    _chk(z, "z", torch.float32)
+    _chk(h_tilde, "h_tilde", torch.float32, (B, T, D))
+    _chk(h0, "h0", torch.float32, (B, D))
+    _chk(P0, "P0", torch.float32, (B, D))
+    done, dd = _done(done, B, T)
+    h = torch.empty_like(z)
+    h_last = torch.empty((B, D), dtype=torch.float32, device=z.device)
+    P_last = torch.empty((B, D), dtype=torch.float32, device=z.device) if want_P else None
+    st = lib.mrx_mingru_scan_fwd(_stream(), _ptr(z), _ptr(h_tilde), _ptr(done), _ptr(h0), _ptr(P0), _ptr(h),
+                                 _ptr(h_last), _ptr(P_last), B, T, D, dd)
+    _lib.check(st, "mrx_mingru_scan_fwd")
+    return h, h_last, P_last
+
+
+def mingru_scan_bwd(z, h_tilde, h, done, h0, g, g_last=None):
+    """Returns (dz, dh_tilde, dh0) for the states h of mingru_scan_fwd and their gradients g."""
+    lib = _lib.load()
+    B, T, D = g.shape
+    for t_, n_ in ((z, "z"), (h_tilde, "h_tilde"), (h, "h"), (g, "g")):
+        _chk(t_, n_, torch.float32, (B, T, D))
+    _chk(h0, "h0", torch.float32, (B, D))
+    _chk(g_last, "g_last", torch.float32, (B, D))
+    done, dd = _done(done, B, T)
+    dz, dx = torch.empty_like(g), torch.empty_like(g)
+    dh0 = torch.empty((B, D), dtype=torch.float32, device=g.device)
+    st = lib.mrx_mingru_scan_bwd(_stream(), _ptr(z), _ptr(h_tilde), _ptr(h), _ptr(done), _ptr(h0), _ptr(g),
+                                 _ptr(g_last), _ptr(dz), _ptr(dx), _ptr(dh0), B, T, D, dd)
+    _lib.check(st, "mrx_mingru_scan_bwd")
+    return dz, dx, dh0
+
+
 # ----------------------------------------------------------------- chunked attention
 def _attn_shapes(q, k, v):
     B, T, H, dk = q.shape

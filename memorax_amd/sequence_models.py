@@ -27,7 +27,9 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .functional import (deltanet, gated_linear_attention, linear_attention, linear_scan,
+from typing import NamedTuple
+
+from .functional import (deltanet, gated_linear_attention, linear_attention, linear_scan, mingru_scan,
                          normalised_linear_attention)
 
 
@@ -227,15 +229,25 @@ class S5Cell(_DiagonalCell):
                 torch.ones(*batch, 1, self.state_size, dtype=torch.complex64, device=dev))
 
 
+class MinGRUProjections(NamedTuple):
+    """MinGRU's elements before the element map: the step's two projections.  ``MinGRUCell.scan``
+    hands them to the kernel that applies the map (a = sigma(-z), b = sigma(z) g(h~)) itself."""
+    z: torch.Tensor
+    h_tilde: torch.Tensor
+
+
 class MinGRUCell(_DiagonalCell):
     """MinGRU (min_gru.py:14-90).  The reference scans (log_state, log_decay) with
     logaddexp; the same recurrence in linear space is h_t = sigma(-z) h_{t-1} +
     sigma(z) g(h~), g(x) = x + 0.5 (x >= 0) | sigma(x), which is what the kernel scans.
-    The carry keeps the reference's log-space leaves: (log h_T, sum of log decays)."""
+    The carry keeps the reference's log-space leaves: (log h_T, sum of log decays).
+    fused (default): the cell returns the projections and the scan kernel forms the coefficients,
+    so neither they nor the half dozen elementwise intermediates behind them exist in memory;
+    fused=False returns the linear-space elements (b, a) for the generic diagonal scan."""
 
-    def __init__(self, features, in_features=None):
+    def __init__(self, features, in_features=None, fused=True):
         super().__init__()
-        self.features = features
+        self.features, self.fused = features, fused
         in_features = features if in_features is None else in_features
         self.z = nn.Linear(in_features, features, bias=False)
         self.h = nn.Linear(in_features, features, bias=False)
@@ -243,14 +255,21 @@ class MinGRUCell(_DiagonalCell):
 
     def forward(self, x, **kwargs):
         z, h_tilde = self.z(x), self.h(x)
+        self.intermediates["gate"] = z.mean().detach()   # min_gru.py:63 sows the mean gate
+        if self.fused and z.dtype == torch.float32:
+            return MinGRUProjections(z, h_tilde)
         a = torch.sigmoid(-z)
         g = torch.where(h_tilde >= 0, torch.relu(h_tilde) + 0.5, torch.sigmoid(h_tilde))
-        self.intermediates["gate"] = z.mean().detach()   # min_gru.py:63 sows the mean gate
         return ((torch.sigmoid(z) * g).contiguous(), a.contiguous())
 
     def scan(self, z, initial_carry, done):
         log_state, log_decay = initial_carry
-        (h, _), (h_last, P_last) = super().scan(z, (torch.exp(log_state), torch.exp(log_decay)), done)
+        h0, P0 = torch.exp(log_state), torch.exp(log_decay)
+        if isinstance(z, MinGRUProjections):
+            h, h_last, P_last = mingru_scan(z.z, z.h_tilde, done, h0[:, 0].contiguous(), P0[:, 0].contiguous())
+            h_last, P_last = h_last[:, None], P_last[:, None]
+        else:
+            (h, _), (h_last, P_last) = super().scan(z, (h0, P0), done)
         return (h, None), (torch.log(h_last), torch.log(P_last))
 
     def read(self, h, x, **kwargs):

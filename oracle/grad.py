@@ -48,6 +48,23 @@ def diag_scan_t(a, b, done, h0, P0=None):
     return torch.stack(hs, 1), h, P
 
 
+def mingru_scan_t(z, h_tilde, done, h0=None):
+    """MinGRU in the reference's log space (elements min_gru.py:52-65, operator :67-74, read :76-78),
+    folded sequentially with select resets (memoroid.py:79-83).  h0: linear-space carry (B,F) > 0,
+    or None for the cell's initial (-inf, 0).  Returns (h (B,T,F), h_last)."""
+    sp = torch.nn.functional.softplus
+    log_b = -sp(-z) + torch.where(h_tilde >= 0, torch.log(torch.relu(h_tilde) + 0.5), -sp(-h_tilde))
+    log_a = -sp(z)
+    B, T, F = z.shape
+    ls = torch.full((B, F), -float("inf"), dtype=z.dtype) if h0 is None else torch.log(h0)
+    out = []
+    for t in range(T):
+        r = done[:, t][:, None]
+        ls = torch.where(r, log_b[:, t], torch.logaddexp(log_a[:, t] + ls, log_b[:, t]))
+        out.append(ls)
+    return torch.exp(torch.stack(out, 1)), torch.exp(ls)
+
+
 def elu1_t(x):
     return torch.where(x > 0, x + 1.0, torch.exp(torch.clamp(x, max=0.0)))
 
@@ -122,6 +139,18 @@ def diag_scan_grads(a, b, done, h0, g, g_last=None):
         L = L + ((hl * _t(g_last).conj()).sum().real if hl.is_complex() else (hl * _t(g_last)).sum())
     L.backward()
     return dict(da=_np(a_.grad), db=_np(b_.grad), dh0=_np(h0_.grad))
+
+
+def mingru_grads(z, h_tilde, done, h0, g, g_last=None):
+    """Returns dict(dz, dh_tilde, dh0) for L = sum(g*h) + sum(g_last*h_last); h0 linear space or None."""
+    z_, x_ = _t(z, True), _t(h_tilde, True)
+    h0_ = None if h0 is None else _t(h0, True)
+    h, hl = mingru_scan_t(z_, x_, _done(done), h0_)
+    L = (h * _t(g)).sum()
+    if g_last is not None:
+        L = L + (hl * _t(g_last)).sum()
+    L.backward()
+    return dict(dz=_np(z_.grad), dh_tilde=_np(x_.grad), dh0=None if h0_ is None else _np(h0_.grad))
 
 
 def linear_attention_grads(q, k, v, done, S0, do, dS_last=None, feature_map="none"):

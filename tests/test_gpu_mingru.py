@@ -1,0 +1,135 @@
+"""GPU parity of the MinGRU scan with the gate arithmetic inside (mrx_mingru_scan_fwd / _bwd, through
+the C ABI) against the oracle's log-space route (the reference's own formulation) and its gradients."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import grad as G
+from oracle import memoroid as M
+from gpu_util import TOL_F32 as TOL, dev, relerr
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [
+    (32, 128, 256),   # time split over waves
+    (1, 1, 1), (2, 1, 64), (3, 7, 5), (2, 9, 130), (5, 200, 64), (4, 300, 258),
+    (64, 64, 1024),   # streaming kernels, 16-byte vectors
+    (40, 50, 516),    # D a multiple of 4 but not of 64: a partly filled last tile
+    (2, 1000, 8),
+]
+
+
+def _ref(z, x, done, h0, P0):
+    carry = None if h0 is None else (np.log(h0)[:, None], np.log(P0)[:, None])
+    nxt, h = M.mingru_scan(z, x, done, carry)
+    return h, np.exp(nxt[0][:, 0]), np.exp(nxt[1][:, 0])
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("p", [0.0, 0.05])
+def test_mingru_scan_fwd_bwd(shape, p):
+    from memorax_amd import kernels as K
+    B, T, D = shape
+    rng = np.random.default_rng(B * 1000 + T * 10 + D)
+    z = (2 * rng.standard_normal(shape)).astype(np.float32)
+    x = (2 * rng.standard_normal(shape)).astype(np.float32)
+    h0 = np.exp(rng.standard_normal((B, D))).astype(np.float32)
+    P0 = rng.uniform(0.5, 1.0, (B, D)).astype(np.float32)
+    done = rng.random((B, T)) < p
+    print(f"case mingru shape={shape} p={p}", flush=True)
+    h, hl, Pl = K.mingru_scan_fwd(dev(z), dev(x), dev(done), dev(h0), dev(P0))
+    rh, rhl, rPl = _ref(z, x, done, h0, P0)
+    assert relerr(h, rh) <= TOL and relerr(hl, rhl) <= TOL and relerr(Pl, rPl) <= TOL
+    g = rng.standard_normal(shape).astype(np.float32)
+    gl = rng.standard_normal((B, D)).astype(np.float32)
+    dz, dx, dh0 = K.mingru_scan_bwd(dev(z), dev(x), h, dev(done), dev(h0), dev(g), dev(gl))
+    # reference gradients from the linear-space closed form (pinned against autograd through the
+    # log-space restatement and finite differences on the CPU), in fp64 on the oracle's states
+    a, b = M.mingru_linear_coeffs(z, x)
+    hh, _, _ = M.diag_scan(a, b, done, h0)
+    da, lam, rdh0 = M.diag_scan_bwd(a, hh, done, g, h0, gl)
+    s = M.sigmoid(z.astype(np.float64))
+    x64 = x.astype(np.float64)
+    rdz = s * (1 - s) * (np.where(x64 >= 0, x64 + 0.5, M.sigmoid(x64)) * lam - da)
+    rdx = lam * s * np.where(x64 >= 0, 1.0, M.sigmoid(x64) * (1 - M.sigmoid(x64)))
+    assert relerr(dz, rdz) <= TOL and relerr(dx, rdx) <= TOL and relerr(dh0, rdh0) <= TOL
+
+
+def test_mingru_autograd_function_against_the_log_space_autograd_oracle():
+    import memorax_amd as mx
+    B, T, D = 4, 50, 32
+    rng = np.random.default_rng(3)
+    z = (2 * rng.standard_normal((B, T, D))).astype(np.float32)
+    x = (2 * rng.standard_normal((B, T, D))).astype(np.float32)
+    h0 = np.exp(rng.standard_normal((B, D))).astype(np.float32)
+    g = rng.standard_normal((B, T, D)).astype(np.float32)
+    gl = rng.standard_normal((B, D)).astype(np.float32)
+    done = rng.random((B, T)) < 0.05
+    tz, tx, th0 = (dev(v).requires_grad_() for v in (z, x, h0))
+    h, hl, _ = mx.functional.mingru_scan(tz, tx, dev(done), th0)
+    ((h * dev(g)).sum() + (hl * dev(gl)).sum()).backward()
+    ag = G.mingru_grads(z, x, done, h0, g, gl)
+    assert relerr(tz.grad, ag["dz"]) <= TOL and relerr(tx.grad, ag["dh_tilde"]) <= TOL
+    assert relerr(th0.grad, ag["dh0"]) <= TOL
+
+
+@pytest.mark.parametrize("done_dtype", ["bool", "float32"])
+def test_mingru_null_carry_extreme_gates_and_reset_isolation(done_dtype):
+    """The cell's initial carry (h0 = 0: exp(-inf)), gates far in both tails (sigma(-z) must stay a
+    relative-precision small number, not 1 - sigma(z)), and NaN before a reset staying there."""
+    from memorax_amd import kernels as K
+    B, T, D = 4, 96, 64
+    rng = np.random.default_rng(5)
+    z = (3 * rng.standard_normal((B, T, D))).astype(np.float32)
+    x = (3 * rng.standard_normal((B, T, D))).astype(np.float32)
+    z[:, 50] = 30.0     # sigma(-30) = 9.4e-14
+    z[:, 60] = -40.0
+    x[:, 70] = -100.0   # g = sigma(-100) = 0 in fp32
+    done = np.zeros((B, T), bool)
+    done[:, 40] = True
+    done[1, 0] = True
+    zp, xp = z.copy(), x.copy()
+    zp[:, 13] = np.nan
+    xp[:, 20] = np.inf
+    dd = done if done_dtype == "bool" else done.astype(np.float32)
+    h, hl, Pl = K.mingru_scan_fwd(dev(zp), dev(xp), dev(dd))
+    hn = h.cpu().numpy()
+    assert np.isfinite(hn[:, 40:]).all() and np.isfinite(hl.cpu().numpy()).all() and np.isfinite(Pl.cpu().numpy()).all()
+    rh, rhl, rPl = _ref(z[:, 40:], x[:, 40:], done[:, 40:], None, None)
+    assert relerr(hn[:, 40:], rh) <= TOL and relerr(hl, rhl) <= TOL
+    # the cumulative decay spans 50 orders of magnitude: compare its logarithm where fp32 can hold
+    # the product, and expect an underflow towards 0 where it cannot (a linear-space leaf)
+    Pn = Pl.cpu().numpy().astype(np.float64)
+    ok = rPl > 1e-30
+    assert (Pn[~ok] <= 1e-29).all() and (not ok.any() or np.abs(np.log(Pn[ok]) - np.log(rPl[ok])).max() <= 1e-3)
+    # steps 48..55 alone hold sigma(-30) among ordinary gates: a product fp32 can hold
+    _, _, Ps = K.mingru_scan_fwd(dev(z[:, 48:56]), dev(x[:, 48:56]), dev(dd[:, 48:56]))
+    _, _, rPs = _ref(z[:, 48:56], x[:, 48:56], done[:, 48:56], None, None)
+    assert rPs.min() > 1e-30 and np.abs(np.log(Ps.cpu().numpy().astype(np.float64)) - np.log(rPs)).max() <= 1e-3
+    g = rng.standard_normal((B, T, D)).astype(np.float32)
+    dz, dx, _ = K.mingru_scan_bwd(dev(zp), dev(xp), h, dev(dd), None, dev(g))
+    assert np.isfinite(dz.cpu().numpy()[:, 40:]).all() and np.isfinite(dx.cpu().numpy()[:, 40:]).all()
+    ag = G.mingru_grads(z[:, 40:], x[:, 40:], done[:, 40:], None, g[:, 40:])
+    assert relerr(dz[:, 40:], ag["dz"]) <= TOL and relerr(dx[:, 40:], ag["dh_tilde"]) <= TOL
+
+
+def test_mingru_cell_fused_and_unfused_agree_and_match_the_reference_route():
+    from memorax_amd import sequence_models as sm
+    torch.manual_seed(1)
+    B, T, Fe = 4, 90, 16
+    cell = sm.MinGRUCell(Fe).cuda()
+    model = sm.Memoroid(cell)
+    x = torch.randn(B, T, Fe, device="cuda")
+    done = torch.rand(B, T, device="cuda") < 0.04
+    carry, y = model(x, done)
+    y.sum().backward()
+    gz, gh = cell.z.weight.grad.clone(), cell.h.weight.grad.clone()
+    cell.zero_grad()
+    cell.fused = False
+    carry2, y2 = model(x, done)
+    y2.sum().backward()
+    assert relerr(y, y2.detach().cpu().numpy()) <= 1e-5
+    assert relerr(carry[0], carry2[0].detach().cpu().numpy()) <= 1e-5 and relerr(carry[1], carry2[1].detach().cpu().numpy()) <= 1e-5
+    assert relerr(gz, cell.z.weight.grad.cpu().numpy()) <= 1e-4 and relerr(gh, cell.h.weight.grad.cpu().numpy()) <= 1e-4
+    nxt, rh = M.mingru_scan(cell.z(x).detach().cpu().numpy(), cell.h(x).detach().cpu().numpy(), done.float().cpu().numpy())
+    assert relerr(y, rh) <= TOL and relerr(carry[0], nxt[0]) <= TOL and relerr(carry[1], nxt[1]) <= TOL

@@ -52,6 +52,43 @@ def test_diag_grads_fd_and_analytic():
     np.testing.assert_allclose(dh0, ag["dh0"], rtol=1e-12, atol=1e-13)
 
 
+def test_mingru_grads_fd_and_the_linear_space_formulas():
+    """Autograd through the log-space restatement vs finite differences of the NumPy log-space scan,
+    and vs the closed form the fused kernel uses: with (lam, da) the reverse scan of the linear-space
+    coefficients, dz = s (1 - s) (g(h~) lam - da), dh~ = lam s g'(h~), s = sigma(z)."""
+    B, T, F = 2, 9, 3
+    z, x = 2 * rnd(B, T, F), 2 * rnd(B, T, F)
+    x[0, 3, 0], x[1, 5, 2] = 0.7, -0.4   # both branches of g near the kink stay on their side under fd
+    h0 = np.exp(rnd(B, F))
+    g, gl = rnd(B, T, F), rnd(B, F)
+    d = np.zeros((B, T), bool)
+    d[0, 4] = True
+    d[1, 0] = True
+
+    def L():
+        nxt, h = M.mingru_scan(z, x, d, (np.log(h0)[:, None], np.zeros((B, 1, F))))
+        return (h * g).sum() + (np.exp(nxt[0][:, 0]) * gl).sum()
+
+    ag = G.mingru_grads(z, x, d, h0, g, gl)
+    np.testing.assert_allclose(ag["dz"], fd(L, z), rtol=1e-6, atol=1e-8)
+    np.testing.assert_allclose(ag["dh_tilde"], fd(L, x), rtol=1e-6, atol=1e-8)
+    np.testing.assert_allclose(ag["dh0"], fd(L, h0), rtol=1e-6, atol=1e-8)
+    a, b = M.mingru_linear_coeffs(z, x)
+    h, _, _ = M.diag_scan(a, b, d, h0)
+    da, lam, dh0 = M.diag_scan_bwd(a, h, d, g, h0, gl)
+    s = M.sigmoid(z)
+    gx = np.where(x >= 0, x + 0.5, M.sigmoid(x))
+    dgx = np.where(x >= 0, 1.0, M.sigmoid(x) * (1 - M.sigmoid(x)))
+    np.testing.assert_allclose(s * (1 - s) * (gx * lam - da), ag["dz"], rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(lam * s * dgx, ag["dh_tilde"], rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(dh0, ag["dh0"], rtol=1e-10, atol=1e-12)
+    # the cell's initial carry (-inf, 0): the first step is b_1 whatever z says about the decay
+    ag0 = G.mingru_grads(z, x, d, None, g)
+    h00, _, _ = M.diag_scan(a, b, d)
+    da0, lam0, _ = M.diag_scan_bwd(a, h00, d, g)
+    np.testing.assert_allclose(s * (1 - s) * (gx * lam0 - da0), ag0["dz"], rtol=1e-10, atol=1e-12)
+
+
 def test_diag_grads_complex_analytic_matches_autograd():
     B, T, D = 2, 8, 3
     a = 0.9 * np.exp(1j * RNG.uniform(0, 3, (B, T, D)))
