@@ -194,6 +194,33 @@ def bench_scan(torch, K, M, dev):
             res[name]["fwd_GB/s_inputs_rotated"] = by / msr / 1e6
             del sets
         del a, b, g, h
+    # MinGRU at the torso shape: gate arithmetic inside the scan kernels against the same recurrence
+    # with the coefficients formed by elementwise torch kernels around the plain scan
+    import memorax_amd.functional as Fn
+    shape = (1024, 128, 256)
+    z = torch.randn(shape, device="cuda").requires_grad_()
+    x = torch.randn(shape, device="cuda").requires_grad_()
+    dn = torch.rand(shape[:2], device="cuda") < 0.01
+    g = torch.randn(shape, device="cuda")
+
+    def fused():
+        h, _, _ = Fn.mingru_scan(z, x, dn)
+        h.backward(g)
+        z.grad = x.grad = None
+
+    def unfused():
+        gx = torch.where(x >= 0, torch.relu(x) + 0.5, torch.sigmoid(x))
+        h, _, _ = Fn.linear_scan(torch.sigmoid(-z), torch.sigmoid(z) * gx, dn)
+        h.backward(g)
+        z.grad = x.grad = None
+    zd, xd = z.detach(), x.detach()
+    h, _, _ = K.mingru_scan_fwd(zd, xd, dn, want_P=False)
+    n = shape[0] * shape[1] * shape[2]
+    mf = _time_ms(torch, lambda: K.mingru_scan_fwd(zd, xd, dn, want_P=False), iters=10)
+    mb = _time_ms(torch, lambda: K.mingru_scan_bwd(zd, xd, h, dn, None, g), iters=10)
+    res["mingru_1024x128x256"] = {"fwd_ms": mf, "fwd_GB/s": 12 * n / mf / 1e6, "bwd_ms": mb, "bwd_GB/s": 24 * n / mb / 1e6,
+                                  "fwd+bwd_ms_fused_autograd": _time_ms(torch, fused, iters=10),
+                                  "fwd+bwd_ms_elementwise_torch_around_the_plain_scan": _time_ms(torch, unfused, iters=10)}
     return res
 
 

@@ -65,17 +65,25 @@ template <typename E, int VEC> __device__ __forceinline__ Vec<E, VEC> vfill(E x)
 struct MinGru {
     // s = sigma(z) and a = sigma(-z), each from exp(-|z|): neither is 1 - the other, so a small
     // gate keeps its relative precision (the cumulative decay is a product of them)
+    // The hardware exponential and reciprocal (a few ulp) instead of the library routines: the
+    // kernels stream at HBM rate only if a step costs a handful of instructions per element.
+    static __device__ __forceinline__ float rcp(float x) { return __builtin_amdgcn_rcpf(x); }
     static __device__ __forceinline__ void gates(float z, float &s, float &a)
     {
-        const float e = expf(-fabsf(z)), r = 1.0f / (1.0f + e), q = e * r;
+        const float e = __expf(-fabsf(z)), r = rcp(1.0f + e), q = e * r;
         s = z >= 0.0f ? r : q;
         a = z >= 0.0f ? q : r;
     }
-    static __device__ __forceinline__ float g(float x) { return x >= 0.0f ? x + 0.5f : 1.0f / (1.0f + expf(-x)); }
+    // sigma(x) for x < 0 from exp(x) <= 1 (no overflow however negative x is)
+    static __device__ __forceinline__ float g(float x)
+    {
+        const float e = __expf(-fabsf(x));
+        return x >= 0.0f ? x + 0.5f : e * rcp(1.0f + e);
+    }
     static __device__ __forceinline__ float dg(float x)
     {
-        const float sx = 1.0f / (1.0f + expf(-x));
-        return x >= 0.0f ? 1.0f : sx * (1.0f - sx);
+        const float e = __expf(-fabsf(x)), r = rcp(1.0f + e);
+        return x >= 0.0f ? 1.0f : e * r * r;  // sigma (1 - sigma) = e / (1 + e)^2
     }
     // (z, x) -> (a, b) in place
     static __device__ __forceinline__ void coeffs(float &za, float &xb)
@@ -142,15 +150,20 @@ diag_scan_fwd_kernel(const E *__restrict__ a, const E *__restrict__ b,
                 const int64_t off = (row0 + t) * D + col;
                 p[s] = *reinterpret_cast<const V *>(a + (a_ti ? col : off));
                 x[s] = *reinterpret_cast<const V *>(b + off);
-                if constexpr (MG) {
-#pragma unroll
-                    for (int i = 0; i < VEC; ++i) MinGru::coeffs(p[s].v[i], x[s].v[i]);
-                }
             } else {
                 p[s] = vfill<E, VEC>(O::one());
                 x[s] = vfill<E, VEC>(O::zero());
             }
             if (t < T && done_at(done, done_f32, row0 + t)) rmask |= 1u << s;
+        }
+        if constexpr (MG) {  // after every load of the super-step has been issued
+#pragma unroll
+            for (int s = 0; s < TS; ++s) {
+                if (ts + s < T && act) {
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) MinGru::coeffs(p[s].v[i], x[s].v[i]);
+                }
+            }
         }
         if (NW == 1) {
             // no time split: continue straight from the carry
@@ -276,18 +289,24 @@ diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hx, const E 
                     if (t + 1 < T) {
                         V av = *reinterpret_cast<const V *>(a + (a_ti ? col : off + D));
 #pragma unroll
-                        for (int i = 0; i < VEC; ++i) {
-                            if constexpr (MG) {
-                                float sg;
-                                MinGru::gates(av.v[i], sg, p[s].v[i]);
-                            } else {
-                                p[s].v[i] = O::conj(av.v[i]);
-                            }
-                        }
+                        for (int i = 0; i < VEC; ++i) p[s].v[i] = MG ? av.v[i] : O::conj(av.v[i]);  // MG: z_{t+1} for now
                     }
                 }
                 if (t + 1 < T && done_at(done, done_f32, row0 + t + 1)) cmask |= 1u << s;
                 if (done_at(done, done_f32, row0 + t)) dmask |= 1u << s;
+            }
+        }
+        if constexpr (MG) {  // a_{t+1} = sigma(-z_{t+1}), after every load of the super-step has been issued
+#pragma unroll
+            for (int s = 0; s < TS; ++s) {
+                const int t = T - 1 - (rs + s);
+                if (t >= 0 && t + 1 < T && act) {
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) {
+                        float sg;
+                        MinGru::gates(p[s].v[i], sg, p[s].v[i]);
+                    }
+                }
             }
         }
         V my = carry;
