@@ -336,12 +336,16 @@ def bench_torso(torch, K):
     x = torch.randn(B, T, Fe, device="cuda")
     done = torch.rand(B, T, device="cuda") < 0.01
 
-    def full():
+    def full(autocast=True):
         for p in torso.parameters():
             p.grad = None
-        _, y = torso(x, done)
+        # configuration 5 names bf16 weights: the dense projections run under bf16 autocast, the
+        # recurrences in the precision their kernels take (bf16 in / fp32 state; fp32 for the scan)
+        with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+            _, y = torso(x, done)
         y.float().pow(2).mean().backward()
     ms_full = _time_ms(torch, full, iters=5, warm=2)
+    ms_full32 = _time_ms(torch, lambda: full(False), iters=3, warm=1)
 
     bf = torch.bfloat16
     q, k, v = (torch.randn(B, T, H, d, device="cuda").to(bf) for _ in range(3))
@@ -359,6 +363,7 @@ def bench_torso(torch, K):
             K.linear_scan_bwd(a, h, done, None, g)
     ms_k = _time_ms(torch, kernels_only, iters=5, warm=2)
     return {"full_torso_ms": ms_full, "full_torso_tokens/s": B * T / ms_full * 1e3,
+            "full_torso_ms_fp32_projections": ms_full32,
             "sequence_kernels_ms": ms_k, "sequence_kernels_tokens/s": B * T / ms_k * 1e3}
 
 

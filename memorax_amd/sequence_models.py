@@ -256,8 +256,9 @@ class MinGRUCell(_DiagonalCell):
     def forward(self, x, **kwargs):
         z, h_tilde = self.z(x), self.h(x)
         self.intermediates["gate"] = z.mean().detach()   # min_gru.py:63 sows the mean gate
-        if self.fused and z.dtype == torch.float32:
-            return MinGRUProjections(z, h_tilde)
+        if self.fused:   # the recurrence runs in fp32 whatever the projections' dtype (autocast)
+            return MinGRUProjections(z.float(), h_tilde.float())
+        z, h_tilde = z.float(), h_tilde.float()
         a = torch.sigmoid(-z)
         g = torch.where(h_tilde >= 0, torch.relu(h_tilde) + 0.5, torch.sigmoid(h_tilde))
         return ((torch.sigmoid(z) * g).contiguous(), a.contiguous())
