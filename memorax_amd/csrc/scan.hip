@@ -9,6 +9,7 @@
 // summaries to its left into a carry-in and fixes its slice up by *select*
 // (a reset inside the slice wins over the carry, so NaN/Inf never cross a reset).
 // One pass over HBM in either case.
+// With MG set the kernels take the MinGRU cell's two projections and form a_t, b_t in registers.
 #include <initializer_list>
 #include <type_traits>
 
