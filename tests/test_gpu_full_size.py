@@ -182,3 +182,28 @@ def test_scan_sweep_shape_properties():
     assert err <= 1e-6 and float((hl2 - hl).abs().max()) <= 1e-5 * float(hl.abs().max()), err
     rh, rhl, rPl = M.diag_scan(a[:1].cpu().numpy(), b[:1].cpu().numpy(), done[:1].cpu().numpy())
     assert relerr(h[:1], rh) <= TOL_F32 and relerr(hl[:1], rhl) <= TOL_F32 and relerr(Pl[:1], rPl) <= TOL_F32
+
+
+def test_config5_mingru_shape_against_the_oracle():
+    """The MinGRU recurrence with the gate arithmetic inside the kernels at configuration 5's shape
+    (1024, 128, 256): states against the oracle's log-space route (the reference's formulation),
+    gradients against the closed form over the oracle's reverse scan."""
+    from memorax_amd import kernels as K
+    shape = (1024, 128, 256)
+    rng = np.random.default_rng(2005)
+    z = (2 * rng.standard_normal(shape)).astype(np.float32)
+    x = (2 * rng.standard_normal(shape)).astype(np.float32)
+    g = rng.standard_normal(shape).astype(np.float32)
+    done = rng.random(shape[:2]) < 0.01
+    print("case full cfg5 mingru", flush=True)
+    h, hl, _ = K.mingru_scan_fwd(dev(z), dev(x), dev(done))
+    dz, dx, _ = K.mingru_scan_bwd(dev(z), dev(x), h, dev(done), None, dev(g))
+    nxt, rh = M.mingru_scan(z, x, done)
+    assert relerr(h, rh) <= TOL_F32 and relerr(hl, np.exp(nxt[0][:, 0])) <= TOL_F32
+    a, b = M.mingru_linear_coeffs(z, x)
+    da, lam, _ = M.diag_scan_bwd(a, rh, done, g)
+    z64, x64 = z.astype(np.float64), x.astype(np.float64)
+    s = M.sigmoid(z64)
+    rdz = s * (1 - s) * (np.where(x64 >= 0, x64 + 0.5, M.sigmoid(x64)) * lam - da)
+    rdx = lam * s * np.where(x64 >= 0, 1.0, M.sigmoid(x64) * (1 - M.sigmoid(x64)))
+    assert relerr(dz, rdz) <= TOL_F32 and relerr(dx, rdx) <= TOL_F32
