@@ -12,6 +12,8 @@ bool or float where nonzero clears the carry before step t (memoroid.py:60-91).
 """
 from __future__ import annotations
 
+import functools
+
 import torch
 
 from . import kernels as K
@@ -19,6 +21,34 @@ from . import kernels as K
 _FMAP = {None: 0, "none": 0, 0: 0, "elu1": 1, 1: 1}
 _FMAP_NAME = {0: "none", 1: "elu1"}
 _HD = 64  # head dim of the kernels (d_k = d_v)
+
+
+def _batched(core_rank, ref):
+    """Extra leading axes on the arguments (what jax.vmap over seeds or agents adds around the
+    reference's calls, examples/ppo_popjym.py:84-85, mappo.py:21-27) are folded into the batch axis
+    for the kernel call and restored on the results.  ``ref``: index of the argument whose rank tells
+    (its rank without extra axes is ``core_rank``); arguments that do not carry the leading axes
+    (a time-invariant decay, scalars) pass through."""
+    def deco(fn):
+        @functools.wraps(fn)
+        def wrapper(*args, **kwargs):
+            extra = args[ref].dim() - core_rank
+            if extra <= 0:
+                return fn(*args, **kwargs)
+            lead = tuple(args[ref].shape[:extra + 1])
+
+            def fold(x):
+                if torch.is_tensor(x) and x.dim() > extra and tuple(x.shape[:extra + 1]) == lead:
+                    return x.reshape(-1, *x.shape[extra + 1:])
+                return x
+
+            def unfold(y):
+                return y.reshape(*lead, *y.shape[1:]) if torch.is_tensor(y) else y
+
+            out = fn(*[fold(a) for a in args], **{k: fold(v) for k, v in kwargs.items()})
+            return tuple(unfold(y) for y in out) if isinstance(out, tuple) else unfold(out)
+        return wrapper
+    return deco
 
 
 class _Heads:
@@ -111,6 +141,7 @@ class _LinearScan(torch.autograd.Function):
                 None)
 
 
+@_batched(3, 1)
 def linear_scan(a, b, done, h0=None, P0=None):
     """Reset-aware diagonal recurrence h_t = a_t h_{t-1} + b_t (lru.py:92-95 scanned
     by memoroid.py:60-91).  a: (B,T,D) or (D,); b: (B,T,D); h0,P0: (B,D).
@@ -145,6 +176,7 @@ class _MinGRUScan(torch.autograd.Function):
                 None)
 
 
+@_batched(3, 0)
 def mingru_scan(z, h_tilde, done, h0=None, P0=None):
     """MinGRU from its two projections (min_gru.py:49-78 scanned by memoroid.py:60-91), linear space:
     h_t = sigmoid(-z_t) h_{t-1} + sigmoid(z_t) g(h~_t), g(x) = x + 0.5 (x >= 0) | sigmoid(x), with the
@@ -180,6 +212,7 @@ class _LinearAttention(torch.autograd.Function):
         return dq, dk, dv, None, (dS0 if ctx.has_S0 else None), None
 
 
+@_batched(4, 0)
 def linear_attention(q, k, v, done, S0=None, feature_map="none"):
     """Causal unnormalised linear attention, chunked: S_t = r_t S_{t-1} + v_t phi(k_t)^T,
     o_t = S_t phi(q_t) (linear_attention.py:62-86,105).  Returns (o, S_last)."""
@@ -216,6 +249,7 @@ class _NormalisedLinearAttention(torch.autograd.Function):
         return dq, dk, dv, None, (dS0 if ctx.has_0[0] else None), (dz0 if ctx.has_0[1] else None), None, None
 
 
+@_batched(4, 0)
 def normalised_linear_attention(q, k, v, done, S0=None, z0=None, feature_map="elu1", eps=1e-6):
     """Causal linear attention with the normalised read-out of LinearAttentionCell.read
     (linear_attention.py:93-110) in the same kernel: z_t = r_t z_{t-1} + phi(k_t),
@@ -249,6 +283,7 @@ class _GatedLinearAttention(torch.autograd.Function):
         return dq, dk, dv, dg, None, (dS0 if ctx.has_S0 else None), None
 
 
+@_batched(4, 0)
 def gated_linear_attention(q, k, v, g, done, S0=None, feature_map="none"):
     """Linear attention with a scalar log-decay g:(B,T,H) per step and head:
     S_t = r_t exp(g_t) S_{t-1} + v_t phi(k_t)^T, o_t = S_t phi(q_t) -- the Mamba cell's algebra
@@ -288,6 +323,7 @@ class _DeltaRule(torch.autograd.Function):
         return dq, dk, dv, db, None, (dS0 if ctx.has_S0 else None), None
 
 
+@_batched(4, 0)
 def delta_rule(q, k, v, beta, done, S0=None):
     """DeltaNet recurrence S_t = r_t S_{t-1}(I - beta_t k_t k_t^T) + beta_t v_t k_t^T,
     o_t = S_t q_t, in chunked WY form.  Returns (o, S_last)."""
@@ -296,6 +332,7 @@ def delta_rule(q, k, v, beta, done, S0=None):
     return hd.out(o), hd.state_out(S_last)
 
 
+@_batched(4, 0)
 def deltanet(q, k, v, beta_raw, done, S0=None):
     """The DeltaNet cell's recurrence on its raw projections: delta_rule with
     k / max(|k|, 1e-12) and sigmoid(beta_raw) formed inside the kernels (the normalised keys and

@@ -100,3 +100,37 @@ def test_linear_attention_model_at_the_reference_guides_head_dim():
     assert c2[0].shape == carry[0].shape and torch.isfinite(y2).all()
     y.pow(2).mean().backward()
     assert cell.key.weight.grad.abs().sum() > 0
+
+
+def test_extra_leading_axes_fold_into_the_batch():
+    """What jax.vmap over seeds adds around the reference's calls: a leading axis on every argument."""
+    import memorax_amd as mx
+    g = torch.Generator(device="cuda").manual_seed(0)
+    S, B, T, H, d = 3, 2, 70, 2, 64
+    q, k, v = (torch.randn((S, B, T, H, d), device="cuda", generator=g) / 8 for _ in range(3))
+    beta = torch.rand((S, B, T, H), device="cuda", generator=g)
+    done = torch.rand((S, B, T), device="cuda", generator=g) < 0.05
+    S0 = torch.randn((S, B, H, d, d), device="cuda", generator=g) * 0.1
+    kn = torch.nn.functional.normalize(k, dim=-1)
+    o, Sl = mx.delta_rule(q, kn, v, beta, done, S0)
+    assert o.shape == (S, B, T, H, d) and Sl.shape == (S, B, H, d, d)
+    for s in range(S):
+        o1, S1 = mx.delta_rule(q[s], kn[s], v[s], beta[s], done[s], S0[s])
+        assert torch.equal(o[s], o1) and torch.equal(Sl[s], S1)
+    o, Sl = mx.linear_attention(q, k, v, done, None, "elu1")
+    o1, S1 = mx.linear_attention(q[1], k[1], v[1], done[1], None, "elu1")
+    assert torch.equal(o[1], o1) and torch.equal(Sl[1], S1)
+    a = torch.rand((S, B, T, 48), device="cuda", generator=g) * 0.1 + 0.9
+    b = torch.randn((S, B, T, 48), device="cuda", generator=g).requires_grad_()
+    lam = torch.rand((48,), device="cuda", generator=g)     # a time-invariant decay carries no leading axes
+    h, hl, Pl = mx.linear_scan(a, b, done)
+    h1, hl1, _ = mx.linear_scan(a[2], b[2], done[2])
+    assert h.shape == (S, B, T, 48) and torch.equal(h[2], h1) and torch.equal(hl[2], hl1)
+    h, _, _ = mx.linear_scan(lam, b, done)
+    h2, _, _ = mx.linear_scan(lam, b[0], done[0])
+    assert torch.equal(h[0], h2)
+    h.sum().backward()
+    assert b.grad.shape == b.shape
+    hm, _, _ = mx.mingru_scan(a, b.detach(), done)
+    hm1, _, _ = mx.mingru_scan(a[1], b.detach()[1], done[1])
+    assert torch.equal(hm[1], hm1)
