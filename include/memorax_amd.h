@@ -12,7 +12,14 @@
  *    kernels on `stream` (a hipStream_t passed as void*, NULL = default stream)
  *    and returns.
  *  - Return value: MRX_OK (0) or a negative mrx_status; never throws.
- *    mrx_status_string() names a code.  Arguments are checked before any launch.
+ *    mrx_status_string() names a code.  Arguments are checked before any launch;
+ *    the status of a launch is the launch call's own return code (the runtime's
+ *    sticky last-error state is neither read nor cleared).  An entry point that
+ *    enqueues two kernels (mrx_delta_rule_fwd with the chunk-parallel factors)
+ *    may return MRX_ERR_LAUNCH after the first has been enqueued.
+ *  - The library keeps no state between calls apart from what mrx_init() sets up
+ *    once per device (below); calls are re-entrant and may be captured in a HIP
+ *    graph once the device has been set up.
  *  - Layouts are the reference's: time on axis 1, features last, row-major,
  *    densely packed.  `done` is (B,T); nonzero at (b,t) clears the carried state
  *    before step t consumes its input (select semantics, memoroid.py:79-83).
@@ -50,7 +57,22 @@ typedef enum {
     MRX_FMAP_ELU1 = 1 /* phi(x) = elu(x) + 1 applied to q and k (linear_attention.py:58-60) */
 } mrx_feature_map;
 
+/* How mrx_delta_rule_fwd / mrx_deltanet_fwd obtain the per-chunk triangular factors. */
+typedef enum {
+    MRX_FACTORS_AUTO = 0,     /* by occupancy: chunk-parallel kernel iff a buffer is given and B*H <= 2 x compute units */
+    MRX_FACTORS_PARALLEL = 1, /* chunk-parallel kernel whenever a buffer is given */
+    MRX_FACTORS_INLINE = 2    /* inverted inside the sequential kernel */
+} mrx_factor_path;
+
 const char *mrx_status_string(int status);
+
+/* Per-device set-up: raises the dynamic-LDS limit of every kernel that needs more than the
+ * default and caches the device's compute-unit count.  Idempotent and thread-safe; the caller's current device
+ * is left as it was.  Calling it is optional -- the first launch on a device does the same --
+ * but a caller that captures its first call on a device into a HIP graph must call it before
+ * the capture begins (the set-up calls are not stream operations).  No counterpart in the
+ * reference (which has no native code). */
+int mrx_init(int device);
 
 /* Library version, major*10000 + minor*100 + patch. */
 int mrx_version(void);
@@ -156,15 +178,15 @@ int mrx_linear_attn_norm_bwd(void *stream, const void *q, const void *k,
  * B*H <= 2 x the device's compute units the factors of all chunks are computed by a chunk-parallel
  * kernel first and the sequential kernel reads them (up to a third faster while the device is not
  * full); otherwise the sequential kernel inverts in place.  Both ways fill Tm_chk with the same
- * factors up to rounding.  The environment variable MRX_DELTA_FACTORS (read once per process)
- * overrides the rule: "parallel" takes the chunk-parallel kernel whenever the buffer is given
- * (on a full device that is level with the default when episodes end every hundred steps or so,
- * and slower when resets are rare), "inline" never does. */
+ * factors up to rounding.  factor_path (mrx_factor_path) overrides the rule:
+ * MRX_FACTORS_PARALLEL takes the chunk-parallel kernel whenever the buffer is given (on a full
+ * device that is level with the default when episodes end every hundred steps or so, and slower
+ * when resets are rare), MRX_FACTORS_INLINE never does. */
 int mrx_delta_rule_fwd(void *stream, const void *q, const void *k,
                        const void *v, const void *beta, const void *done,
                        const void *S0, void *o, void *S_last, void *S_chk,
                        void *Tm_chk, int64_t B, int64_t T, int64_t H, int64_t dk,
-                       int64_t dv, int dtype, int done_dtype);
+                       int64_t dv, int dtype, int done_dtype, int factor_path);
 
 /* Gradients w.r.t. q,k,v,beta (in `dtype`) and S0 (fp32, nullable).  S_chk and
  * Tm_chk are the residuals written by mrx_delta_rule_fwd on the same inputs. */
@@ -186,7 +208,8 @@ int mrx_delta_rule_bwd(void *stream, const void *q, const void *k,
 int mrx_deltanet_fwd(void *stream, const void *q, const void *k, const void *v,
                      const void *beta_raw, const void *done, const void *S0, void *o,
                      void *S_last, void *S_chk, void *Tm_chk, int64_t B, int64_t T,
-                     int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype);
+                     int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype,
+                     int factor_path);
 
 int mrx_deltanet_bwd(void *stream, const void *q, const void *k, const void *v,
                      const void *beta_raw, const void *done, const void *S_chk,

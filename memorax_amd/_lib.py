@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmemorax_amd.so")
 MRX_F32, MRX_BF16, MRX_C64 = 0, 1, 2
 MRX_DONE_U8, MRX_DONE_F32 = 0, 1
 MRX_FMAP_NONE, MRX_FMAP_ELU1 = 0, 1
+MRX_FACTORS_AUTO, MRX_FACTORS_PARALLEL, MRX_FACTORS_INLINE = 0, 1, 2
 
 _P = ctypes.c_void_p
 _I = ctypes.c_int
@@ -23,6 +24,7 @@ _L = ctypes.c_int64
 SIGNATURES = {
     "mrx_status_string": (ctypes.c_char_p, [_I]),
     "mrx_version": (_I, []),
+    "mrx_init": (_I, [_I]),
     "mrx_chunk_size": (_L, [_I]),
     "mrx_delta_chunk_size": (_L, [_I]),
     "mrx_linear_scan_fwd": (_I, [_P] * 9 + [_L] * 3 + [_I] * 3),
@@ -31,9 +33,9 @@ SIGNATURES = {
     "mrx_linear_attn_bwd": (_I, [_P] * 12 + [_L] * 5 + [_I] * 3),
     "mrx_linear_attn_norm_fwd": (_I, [_P] * 13 + [_L] * 5 + [_I] * 3 + [ctypes.c_float]),
     "mrx_linear_attn_norm_bwd": (_I, [_P] * 17 + [_L] * 5 + [_I] * 3 + [ctypes.c_float]),
-    "mrx_delta_rule_fwd": (_I, [_P] * 11 + [_L] * 5 + [_I] * 2),
+    "mrx_delta_rule_fwd": (_I, [_P] * 11 + [_L] * 5 + [_I] * 3),
     "mrx_delta_rule_bwd": (_I, [_P] * 15 + [_L] * 5 + [_I] * 2),
-    "mrx_deltanet_fwd": (_I, [_P] * 11 + [_L] * 5 + [_I] * 2),
+    "mrx_deltanet_fwd": (_I, [_P] * 11 + [_L] * 5 + [_I] * 3),
     "mrx_deltanet_bwd": (_I, [_P] * 15 + [_L] * 5 + [_I] * 2),
     "mrx_linear_scan_last": (_I, [_P] * 6 + [_L] * 4 + [_I] * 2),
     "mrx_mingru_scan_fwd": (_I, [_P] * 9 + [_L] * 3 + [_I]),

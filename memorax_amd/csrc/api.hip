@@ -1,5 +1,48 @@
-// Library-level entry points of the C ABI (status strings, version, chunk size).
+// Library-level entry points of the C ABI: status strings, version, per-device set-up.
+#include <atomic>
+#include <mutex>
+
 #include "common.h"
+
+namespace mrx {
+
+namespace {
+KernelNode *g_kernels = nullptr;               // filled while the library is loaded, read-only afterwards
+std::atomic<unsigned long long> g_ready{0ull};  // bit d: device d has been set up
+std::mutex g_setup;
+int g_cus[64] = {0};
+}  // namespace
+
+void register_kernel(KernelNode *node)
+{
+    node->next = g_kernels;
+    g_kernels = node;
+}
+
+int prepare_device(int *cus, int *dev_out)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return MRX_ERR_LAUNCH;
+    if (dev < 0 || dev >= 64) return MRX_ERR_UNSUPPORTED;
+    const unsigned long long bit = 1ull << dev;
+    if (!(g_ready.load(std::memory_order_acquire) & bit)) {
+        std::lock_guard<std::mutex> lock(g_setup);
+        if (!(g_ready.load(std::memory_order_relaxed) & bit)) {
+            for (const KernelNode *n = g_kernels; n; n = n->next)
+                if (hipFuncSetAttribute(n->fn, hipFuncAttributeMaxDynamicSharedMemorySize, n->lds_bytes) != hipSuccess)
+                    return MRX_ERR_LAUNCH;
+            int n_cu = 0;
+            if (hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return MRX_ERR_LAUNCH;
+            g_cus[dev] = n_cu;
+            g_ready.fetch_or(bit, std::memory_order_release);
+        }
+    }
+    if (cus) *cus = g_cus[dev];
+    if (dev_out) *dev_out = dev;
+    return MRX_OK;
+}
+
+}  // namespace mrx
 
 extern "C" const char *mrx_status_string(int status)
 {
@@ -12,22 +55,15 @@ extern "C" const char *mrx_status_string(int status)
     }
 }
 
-extern "C" int mrx_version(void) { return 100; }
+extern "C" int mrx_version(void) { return 200; }
 
-#ifdef MRX_PHASE_TIMING
-__device__ unsigned long long mrx_phase_ticks[64];
-__device__ unsigned long long mrx_wg_trace[4096 * 3];
-extern "C" int mrx_wg_trace_read(unsigned long long *host)
+extern "C" int mrx_init(int device)
 {
-    return hipMemcpyFromSymbol(host, HIP_SYMBOL(mrx_wg_trace), sizeof(unsigned long long) * 4096 * 3) == hipSuccess ? 0 : -1;
+    int prev = 0;
+    if (hipGetDevice(&prev) != hipSuccess) return MRX_ERR_LAUNCH;
+    if (device < 0 || device >= 64) return MRX_ERR_INVALID_ARG;
+    if (device != prev && hipSetDevice(device) != hipSuccess) return MRX_ERR_INVALID_ARG;
+    const int rc = mrx::prepare_device();
+    if (device != prev && hipSetDevice(prev) != hipSuccess) return MRX_ERR_LAUNCH;
+    return rc;
 }
-extern "C" int mrx_phase_read(unsigned long long *host, int reset)
-{
-    if (hipMemcpyFromSymbol(host, HIP_SYMBOL(mrx_phase_ticks), sizeof(unsigned long long) * 64) != hipSuccess) return -1;
-    if (reset) {
-        unsigned long long z[64] = {0};
-        if (hipMemcpyToSymbol(HIP_SYMBOL(mrx_phase_ticks), z, sizeof(z)) != hipSuccess) return -1;
-    }
-    return 0;
-}
-#endif

@@ -653,7 +653,6 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
     for (int part = 0; part < 6; ++part) prefetch_part(part);
     int64_t dboff = ((int64_t)b * Tlen + tlast + tid) * H + h;
-    MRX_PHASE_INIT();
 
     // Gradients leave through LDS: an accumulator tile holds four features of sixteen rows per lane
     // group, so a store from accumulators writes 16 pieces of 32 bytes per instruction; written to a
@@ -730,7 +729,6 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             if (pass != nres) zero_acc<TMS::TPW>(dSacc);
             store_acc<T, HD, HD, NW>(dSacc, sDS, LDD, w, lane);  // dS[dv][dk]
             sync_lds();
-            MRX_PHASE(11);
             flush_pending();
             const bool pre = pass == 0 && c > 0;
             if (pre) { prefetch_part(0); prefetch_part(1); }
@@ -764,7 +762,6 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 }
             }
             sync_lds();
-            MRX_PHASE(15);
             if (pre) { prefetch_part(2); prefetch_part(3); }
             // ---- U'^T[dv][c] = sum_j V~[j][dv] Tm[c][j] -> sU[c][dv] ----------------------------------
             {
@@ -782,7 +779,6 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 store_acc<T, HD, C, NW>(acc, sDU, LDD, w, lane);
             }
             sync_lds();  // sU, sDU visible; sAqk dead
-            MRX_PHASE(16);
             if (pre) { prefetch_part(4); prefetch_part(5); }
             float dbp[TMR::NBW];  // per-lane partials of dbeta for rows nt * 16 + li of the wave's tile columns
 #pragma unroll
@@ -815,7 +811,6 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 store_acc<T, HD, C, NW>(acc, sZb, LDD, w, lane);  // = dV, written to memory from here after the barrier
             }
             sync_lds();  // sDAqk, sZ, sZb visible
-            MRX_PHASE(17);
             tile_rows_to_global<T, C, NTHR>(sZb, LDD, dv + base + (int64_t)t0 * rs, rs, t0, Tlen, tid, live);
             // ---- dQ^T[dk][i] = sum_dv S[dv][dk] dO[i][dv] + sum_j K[j][dk] dAqk[i][j] -> global ----
             {
@@ -855,7 +850,6 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 store_acc_f<T, C, C, NW>(acc, sDA, LDC, w, lane, [](int m, int n, float x) { return m < n ? -x : 0.f; });
             }
             sync_lds();  // sDA visible; sQ, sDO, sS, sDS, sDAqk, sZ, sZb dead
-            MRX_PHASE(20);
             tile_rows_to_global<T, C, NTHR>(sDU, LDD, dq + base + (int64_t)t0 * rs, rs, t0, Tlen, tid, live);
             // ---- R^T[dk][i] = sum_j K[j][dk] dA[i][j] : dbeta += K_i . R_i ; dK += beta_i R ;
             //      dK^T[dk][j] += sum_i beta_i K[i][dk] dA[i][j] -> global -------------------------------
@@ -903,7 +897,6 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 if (lg == 0) sDb[(w % TMR::WM) * C + TMR::nt(w, j) * 16 + li] = x;
             }
             sync_lds();
-            MRX_PHASE(23);
             if (PRO) {
 #pragma unroll
                 for (int j = 0; j < TMR::TPW; ++j) {
@@ -929,12 +922,11 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 pend_dboff = dboff;
                 pend_db_on = true;
             }
-            MRX_PHASE(24);  // no barrier: sDb, sKd are not written again before the next pass's last phase
+            // no barrier: sDb, sKd are not written again before the next pass's last phase
         }
     }
     sync_lds();
     flush_pending();
-    MRX_PHASE_FLUSH();
     if (dS0) {
 #pragma unroll
         for (int j = 0; j < TMS::TPW; ++j) {
@@ -944,21 +936,24 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     }
 }
 
+template <typename T, int C, bool FMAP, bool GATED, bool NORM> struct LaBwdReg {
+    static constexpr int smem = LaBwdSmem<T, C, GATED, NORM>::total;
+    static inline KernelRegistrar reg{reinterpret_cast<const void *>(la_bwd_kernel<T, C, FMAP, GATED, NORM>), smem};
+};
+
 template <typename T, int C, bool FMAP, bool GATED = false, bool NORM = false>
 int launch_la(hipStream_t st, const void *q, const void *k, const void *v, const void *done,
               int done_f32, const void *S_chk, const void *dout, const void *dS_last, void *dq,
               void *dk, void *dv, void *dS0, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr,
               void *edot = nullptr, NormBwdArgs na = NormBwdArgs{})
 {
-    auto kern = la_bwd_kernel<T, C, FMAP, GATED, NORM>;
-    constexpr int smem = LaBwdSmem<T, C, GATED, NORM>::total;
-    static unsigned long long lds_set = 0ull;
-    if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(256), smem, st, (const T *)q,
-                       (const T *)k, (const T *)v, (const float *)glog, done, done_f32, (const T *)S_chk,
-                       (const T *)dout, (const float *)dS_last, (T *)dq, (T *)dk, (T *)dv, (float *)edot,
-                       (float *)dS0, (int)Tlen, (int)H, na);
-    return launch_status();
+    using Reg = LaBwdReg<T, C, FMAP, GATED, NORM>;
+    (void)&Reg::reg;  // the kernel is on the list mrx_init() walks
+    if (const int rc = prepare_device(); rc != MRX_OK) return rc;
+    return launch_kernel(la_bwd_kernel<T, C, FMAP, GATED, NORM>, dim3((unsigned)(B * H)), dim3(256), Reg::smem, st,
+                         (const T *)q, (const T *)k, (const T *)v, (const float *)glog, done, done_f32,
+                         (const T *)S_chk, (const T *)dout, (const float *)dS_last, (T *)dq, (T *)dk, (T *)dv,
+                         (float *)edot, (float *)dS0, (int)Tlen, (int)H, na);
 }
 
 int check_bwd(const void *q, const void *k, const void *v, const void *done, const void *S_chk,
@@ -1047,22 +1042,25 @@ extern "C" int mrx_gated_linear_attn_bwd(void *stream, const void *q, const void
 
 namespace {
 
+template <typename T, int C, bool PRO> struct DeltaBwdReg {
+    static constexpr int NW = 4;
+    static constexpr int smem = DeltaBwdSmem<T, C, NW>::total;
+    static inline KernelRegistrar reg{reinterpret_cast<const void *>(delta_bwd_kernel<T, C, NW, PRO>), smem};
+};
+
 template <typename T, int C, bool PRO>
 int launch_delta_bwd(hipStream_t st, const void *q, const void *k, const void *v, const void *beta,
                      const void *done, int done_dtype, const void *S_chk, const void *Tm_chk, const void *dout,
                      const void *dS_last, void *dq, void *dk_out, void *dv_out, void *dbeta, void *dS0, int64_t B,
                      int64_t T_, int64_t H)
 {
-    constexpr int NW = 4;
-    auto kern = delta_bwd_kernel<T, C, NW, PRO>;
-    constexpr int smem = DeltaBwdSmem<T, C, NW>::total;
-    static unsigned long long lds_set = 0ull;
-    if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(64 * NW), smem, st, (const T *)q, (const T *)k,
-                       (const T *)v, (const T *)beta, done, done_dtype, (const T *)S_chk, (const T *)Tm_chk,
-                       (const T *)dout, (const float *)dS_last, (T *)dq, (T *)dk_out, (T *)dv_out, (T *)dbeta,
-                       (float *)dS0, (int)T_, (int)H);
-    return launch_status();
+    using Reg = DeltaBwdReg<T, C, PRO>;
+    (void)&Reg::reg;  // the kernel is on the list mrx_init() walks
+    if (const int rc = prepare_device(); rc != MRX_OK) return rc;
+    return launch_kernel(delta_bwd_kernel<T, C, Reg::NW, PRO>, dim3((unsigned)(B * H)), dim3(64 * Reg::NW), Reg::smem, st,
+                         (const T *)q, (const T *)k, (const T *)v, (const T *)beta, done, done_dtype,
+                         (const T *)S_chk, (const T *)Tm_chk, (const T *)dout, (const float *)dS_last, (T *)dq,
+                         (T *)dk_out, (T *)dv_out, (T *)dbeta, (float *)dS0, (int)T_, (int)H);
 }
 
 template <bool PRO>

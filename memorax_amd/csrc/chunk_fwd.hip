@@ -14,9 +14,6 @@
 // non-finite value can never meet a masked-out zero inside a matrix product.
 // The state is kept transposed (S^T, d_k x d_v) in MFMA accumulators for the whole
 // sequence and re-staged to LDS as a T-typed d_v x d_k tile once per chunk.
-#include <cstdlib>
-#include <cstring>
-
 #include "chunk_common.h"
 #include "delta_tm.h"
 
@@ -141,7 +138,6 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     const Frag ones = TT<T>::ones();
     int64_t den_off = ((int64_t)b * Tlen + li) * H + h;  // den[t0 + li]
 
-    MRX_WG_BEGIN();
     // register prefetch of the next chunk (raw bits only: no arithmetic on in-flight loads)
     typename IO::Regs rq, rk, rv;
     uint32_t rbeta = 0u, rdone = 0u;
@@ -204,7 +200,6 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         // blocks above the block diagonal of Tm are never written again
         for (int idx = tid; idx < C * LDC * (int)sizeof(T) / 4; idx += NTHR) reinterpret_cast<uint32_t *>(sTm)[idx] = 0u;
     }
-    MRX_PHASE_INIT();
 
     static_assert(C * C / 4 % NTHR == 0, "Tm tile copy assumes whole passes");
     // running element offsets of this thread's stores, advanced by one chunk per iteration
@@ -307,7 +302,6 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 }
             }
             sync_lds();
-            MRX_PHASE(1);
             // Outputs leave through LDS as whole rows (an accumulator tile would write 16 pieces of
             // 32 bytes per instruction): the output of the previous unit, parked in sO at its end, and
             // the state checkpoint from the copy of S that has just been staged.
@@ -348,11 +342,9 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 f32x4 Xcc = {0.f, 0.f, 0.f, 0.f};
                 if (diag >= 0) Xcc = tri_diag_block<T>(kk, sBeta, diag, sA, LDA, sTm, LDC, lane);
                 sync_lds();
-                MRX_PHASE(2);
                 if (pre) { prefetch_part(2); prefetch_part(3); }
                 if (diag >= 0) tri_block_column<C, T>(sA, LDA, sTm, LDC, diag, Xcc, lane);
                 sync_lds();
-                MRX_PHASE(3);
             }
             // ---- Aqk[i][j] = (q_i . k_j), j <= i ; delta rule: W = Tm (beta K), U = Tm (beta V) ----
             {
@@ -398,7 +390,6 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     }
                 }
                 sync_lds();  // sW, sAqk visible; every wave is done with beta V
-                MRX_PHASE(5);
                 // U'^T[dv][c] = U^T - S W^T -> sU[c][dv] (over beta V)
                 {
                     f32x4 acc[TMO::TPW];
@@ -410,7 +401,6 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 }
             }
             sync_lds();
-            MRX_PHASE(7);
             // ---- O^T[dv][i] = sum_dk S[dv][dk] Q[i][dk] + sum_j U'[j][dv] Aqk[i][j] ; store O -------
             if (!DELTA && pre) { prefetch_part(2); prefetch_part(3); }
             f32x4 Oacc[TMO::TPW];
@@ -505,12 +495,9 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 }
             }
             sync_lds();
-            MRX_PHASE(8);
         }
     }
     flush_o();  // the last unit ended with a barrier
-    MRX_WG_END();
-    MRX_PHASE_FLUSH();
 
     if (S_last) {
 #pragma unroll
@@ -529,20 +516,25 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     }
 }
 
+template <typename T, int C, bool DELTA, bool FMAP, bool GATED, bool NORM, bool PRO, bool TMIN> struct FwdReg {
+    static constexpr int smem = FwdSmem<T, C, DELTA, GATED, NORM>::total;
+    static inline KernelRegistrar reg{
+        reinterpret_cast<const void *>(chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN>), smem};
+};
+
 template <typename T, int C, bool DELTA, bool FMAP, bool GATED = false, bool NORM = false, bool PRO = false,
           bool TMIN = false>
 int launch(hipStream_t st, const void *q, const void *k, const void *v, const void *beta,
            const void *done, int done_f32, const void *S0, void *o, void *S_last, void *S_chk,
            void *Tm_chk, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr, NormArgs na = NormArgs{})
 {
-    auto kern = chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN>;
-    constexpr int smem = FwdSmem<T, C, DELTA, GATED, NORM>::total;
-    static unsigned long long lds_set = 0ull;
-    if (ensure_lds_limit(kern, smem, lds_set) != MRX_OK) return MRX_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(NTHR), smem, st, (const T *)q,
-                       (const T *)k, (const T *)v, (const T *)beta, (const float *)glog, done, done_f32,
-                       (const float *)S0, (T *)o, (float *)S_last, (T *)S_chk, (T *)Tm_chk, (int)Tlen, (int)H, na);
-    return launch_status();
+    using Reg = FwdReg<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN>;
+    (void)&Reg::reg;  // the kernel is on the list mrx_init() walks
+    if (const int rc = prepare_device(); rc != MRX_OK) return rc;
+    return launch_kernel(chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN>, dim3((unsigned)(B * H)),
+                         dim3(NTHR), Reg::smem, st, (const T *)q, (const T *)k, (const T *)v, (const T *)beta,
+                         (const float *)glog, done, done_f32, (const float *)S0, (T *)o, (float *)S_last, (T *)S_chk,
+                         (T *)Tm_chk, (int)Tlen, (int)H, na);
 }
 
 int check_common(const void *q, const void *k, const void *v, const void *done, const void *o,
@@ -562,50 +554,26 @@ int check_common(const void *q, const void *k, const void *v, const void *done, 
     return MRX_OK;
 }
 
-// Compute units of the current device (0 if the query fails), asked once per device.
-int compute_units()
-{
-    static int cached[64] = {0};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
-    if (cached[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-        cached[dev] = n;
-    }
-    return cached[dev];
-}
-
-// MRX_DELTA_FACTORS in the environment overrides the rule below: "parallel" = the chunk-parallel
-// kernel whenever there is a buffer, "inline" = never.  Read once.  A tuning knob: the reset rate,
-// which the host cannot see, moves the break-even point (a chunk with resets repeats the in-kernel
-// inverse per episode, the chunk-parallel kernel does that off the sequential path).
-int factor_policy()
-{
-    static const int policy = [] {
-        const char *e = getenv("MRX_DELTA_FACTORS");
-        if (e && !strcmp(e, "parallel")) return 1;
-        if (e && !strcmp(e, "inline")) return 2;
-        return 0;
-    }();
-    return policy;
-}
-
 // Two ways to the triangular factors.  With a buffer for them and at most two workgroups per compute
 // unit, the chunk-parallel kernel fills the buffer and the sequential kernel reads it: the
 // sequential kernel loses half of its per-chunk dependency chain, which is what bounds it while
 // the device is not full.  With more sequences than that the device is bound by memory traffic,
 // other workgroups hide the inverse, and the second pass over the keys plus the round trip of the
 // factors (a fifth more traffic) would only cost: the sequential kernel inverts in place then, as it
-// does when there is no buffer.
+// does when there is no buffer.  factor_path (mrx_factor_path) overrides the rule: the reset rate,
+// which the host cannot see, moves the break-even point (a chunk with resets repeats the in-kernel
+// inverse per episode, the chunk-parallel kernel does that off the sequential path).
 template <bool PRO>
 int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void *v, const void *beta, const void *done,
                        int done_dtype, const void *S0, void *o, void *S_last, void *S_chk, void *Tm_chk, int64_t B,
-                       int64_t T, int64_t H, int dtype)
+                       int64_t T, int64_t H, int dtype, int factor_path)
 {
     static_assert(DELTA_BF16_CHUNK == 32, "delta_tm_kernel is written for 32-row chunks");
-    const int policy = factor_policy();
-    if (Tm_chk && policy != 2 && T <= DELTA_TM_MAX_T && (policy == 1 || B * H <= 2 * (int64_t)compute_units())) {
+    int cus = 0;
+    if (const int rc = prepare_device(&cus); rc != MRX_OK) return rc;
+    const bool parallel = Tm_chk && factor_path != MRX_FACTORS_INLINE && T <= DELTA_TM_MAX_T &&
+                          (factor_path == MRX_FACTORS_PARALLEL || B * H <= 2 * (int64_t)cus);
+    if (parallel) {
         const int rc = launch_delta_tm(st, k, beta, done, done_dtype, Tm_chk, B, T, H, dtype, PRO);
         if (rc != MRX_OK) return rc;
         if (dtype == MRX_BF16)
@@ -620,6 +588,8 @@ int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void 
     return launch<float, 32, true, false, false, false, PRO, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last,
                                                                     S_chk, Tm_chk, B, T, H);
 }
+
+bool factor_path_ok(int f) { return f == MRX_FACTORS_AUTO || f == MRX_FACTORS_PARALLEL || f == MRX_FACTORS_INLINE; }
 
 }  // namespace
 
@@ -647,13 +617,14 @@ extern "C" int mrx_linear_attn_fwd(void *stream, const void *q, const void *k, c
 extern "C" int mrx_delta_rule_fwd(void *stream, const void *q, const void *k, const void *v,
                                   const void *beta, const void *done, const void *S0, void *o,
                                   void *S_last, void *S_chk, void *Tm_chk, int64_t B, int64_t T,
-                                  int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype)
+                                  int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype, int factor_path)
 {
     const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
-    if (!beta || !aligned(Tm_chk, 16)) return MRX_ERR_INVALID_ARG;
+    if (!beta || !aligned(Tm_chk, 16) || !factor_path_ok(factor_path)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
-    return delta_fwd_dispatch<false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H, dtype);
+    return delta_fwd_dispatch<false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H, dtype,
+                                     factor_path);
 }
 
 extern "C" int mrx_gated_linear_attn_fwd(void *stream, const void *q, const void *k, const void *v,
@@ -699,11 +670,12 @@ extern "C" int mrx_linear_attn_norm_fwd(void *stream, const void *q, const void 
 extern "C" int mrx_deltanet_fwd(void *stream, const void *q, const void *k, const void *v,
                                 const void *beta_raw, const void *done, const void *S0, void *o,
                                 void *S_last, void *S_chk, void *Tm_chk, int64_t B, int64_t T,
-                                int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype)
+                                int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype, int factor_path)
 {
     const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
-    if (!beta_raw || !aligned(Tm_chk, 16)) return MRX_ERR_INVALID_ARG;
+    if (!beta_raw || !aligned(Tm_chk, 16) || !factor_path_ok(factor_path)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
-    return delta_fwd_dispatch<true>(st, q, k, v, beta_raw, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H, dtype);
+    return delta_fwd_dispatch<true>(st, q, k, v, beta_raw, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H, dtype,
+                                    factor_path);
 }

@@ -3,6 +3,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <tuple>
+#include <utility>
+
 #include "memorax_amd.h"
 
 namespace mrx {
@@ -27,27 +30,44 @@ __device__ __forceinline__ bool done_test(uint32_t raw, int is_f32)
     return is_f32 ? (__uint_as_float(raw) != 0.0f) : (raw != 0u);
 }
 
-inline int launch_status()
+// Launches `kern` and returns MRX_OK or MRX_ERR_LAUNCH from the launch call's own return code.
+// The runtime's sticky "last error" is neither read nor cleared, so an error left behind by other
+// code in the process is not mistaken for this launch's, and is still there for its owner.
+template <typename... KArgs, size_t... I>
+inline int launch_impl(void (*kern)(KArgs...), dim3 grid, dim3 block, size_t lds_bytes, hipStream_t st,
+                       std::tuple<KArgs...> &vals, std::index_sequence<I...>)
 {
-    return hipGetLastError() == hipSuccess ? MRX_OK : MRX_ERR_LAUNCH;
+    void *ptrs[] = {static_cast<void *>(&std::get<I>(vals))...};
+    return hipLaunchKernel(reinterpret_cast<const void *>(kern), grid, block, ptrs, lds_bytes, st) == hipSuccess
+               ? MRX_OK
+               : MRX_ERR_LAUNCH;
+}
+template <typename... KArgs, typename... Args>
+inline int launch_kernel(void (*kern)(KArgs...), dim3 grid, dim3 block, size_t lds_bytes, hipStream_t st, Args... args)
+{
+    static_assert(sizeof...(KArgs) == sizeof...(Args), "one argument per kernel parameter");
+    std::tuple<KArgs...> vals(static_cast<KArgs>(args)...);
+    return launch_impl(kern, grid, block, lds_bytes, st, vals, std::index_sequence_for<KArgs...>{});
 }
 
-// Raises a kernel's dynamic LDS limit once per device (the attribute belongs to the device's
-// copy of the kernel).  `done` is a per-kernel bit mask indexed by device id; setting it twice
-// from racing threads only repeats an idempotent call.
-template <typename K> inline int ensure_lds_limit(K kern, int bytes, unsigned long long &done)
-{
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return MRX_ERR_LAUNCH;
-    const unsigned long long bit = 1ull << (dev & 63);
-    if (!(done & bit)) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                bytes) != hipSuccess)
-            return MRX_ERR_LAUNCH;
-        done |= bit;
-    }
-    return MRX_OK;
-}
+// Per-device set-up, done once per device by mrx_init() or by the first launch on it: every kernel
+// that needs more than the default 64 KB of dynamic LDS gets its limit raised (the attribute belongs
+// to the device's copy of the kernel) and the number of compute units is cached.  Kernels enter the list through a
+// KernelRegistrar with static storage, i.e. while the library is being loaded; after that the list
+// is read-only.
+struct KernelNode {
+    const void *fn;
+    int lds_bytes;
+    KernelNode *next;
+};
+void register_kernel(KernelNode *node);
+struct KernelRegistrar {
+    KernelNode node;
+    KernelRegistrar(const void *fn, int lds_bytes) : node{fn, lds_bytes, nullptr} { register_kernel(&node); }
+};
+// Makes the current device ready (see above).  Returns an MRX_* status; *cus (if given) receives the
+// device's compute-unit count, *dev its index.
+int prepare_device(int *cus = nullptr, int *dev = nullptr);
 
 inline bool aligned(const void *p, size_t n)
 {
@@ -55,48 +75,3 @@ inline bool aligned(const void *p, size_t n)
 }
 
 }  // namespace mrx
-
-// Phase timing for kernel tuning: compiled in only with -DMRX_PHASE_TIMING (never in
-// the shipped library).  Workgroup 0 / thread 0 accumulates the shader-clock ticks
-// spent between consecutive MRX_PHASE marks; MRX_PHASE_FLUSH adds them to mrx_phase_ticks[].
-#ifdef MRX_PHASE_TIMING
-extern __device__ unsigned long long mrx_phase_ticks[64];
-extern __device__ unsigned long long mrx_wg_trace[4096 * 3];
-#define MRX_WG_BEGIN()                                                                    \
-    do {                                                                                  \
-        if (threadIdx.x == 0 && blockIdx.x < 4096) {                                      \
-            mrx_wg_trace[blockIdx.x * 3 + 0] = wall_clock64();                            \
-            mrx_wg_trace[blockIdx.x * 3 + 2] = __builtin_amdgcn_s_getreg((4) | (0 << 6) | (31 << 11)) \
-                | ((unsigned long long)__builtin_amdgcn_s_getreg((20) | (0 << 6) | (31 << 11)) << 32); \
-        }                                                                                 \
-    } while (0)
-#define MRX_WG_END()                                                                      \
-    do {                                                                                  \
-        if (threadIdx.x == 0 && blockIdx.x < 4096) mrx_wg_trace[blockIdx.x * 3 + 1] = wall_clock64(); \
-    } while (0)
-// marks (i < 32; thread 0 -> slot i, thread 256 -> slot 32 + i) accumulate in LDS
-// (fire-and-forget ds_add) so that a mark never waits on global memory
-#define MRX_PHASE_INIT()                                                    \
-    __shared__ unsigned long long mrx_lds_ticks[64];                        \
-    if (threadIdx.x < 64) mrx_lds_ticks[threadIdx.x] = 0;                   \
-    unsigned long long mrx_t_last = clock64()
-#define MRX_PHASE(i)                                                        \
-    do {                                                                    \
-        if (blockIdx.x == 0 && (threadIdx.x == 0 || threadIdx.x == 256)) {  \
-            const unsigned long long mrx_t_now = clock64();                 \
-            __hip_atomic_fetch_add(&mrx_lds_ticks[(i) + (threadIdx.x ? 32 : 0)], mrx_t_now - mrx_t_last, __ATOMIC_RELAXED, \
-                                   __HIP_MEMORY_SCOPE_WORKGROUP);           \
-            mrx_t_last = mrx_t_now;                                         \
-        }                                                                   \
-    } while (0)
-#define MRX_PHASE_FLUSH()                                                   \
-    do {                                                                    \
-        if (blockIdx.x == 0 && threadIdx.x < 64) mrx_phase_ticks[threadIdx.x] += mrx_lds_ticks[threadIdx.x]; \
-    } while (0)
-#else
-#define MRX_WG_BEGIN() do { } while (0)
-#define MRX_WG_END() do { } while (0)
-#define MRX_PHASE_INIT() do { } while (0)
-#define MRX_PHASE(i) do { } while (0)
-#define MRX_PHASE_FLUSH() do { } while (0)
-#endif

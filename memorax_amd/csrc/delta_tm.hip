@@ -164,9 +164,8 @@ int launch_tm(hipStream_t st, const void *k, const void *beta, const void *done,
 {
     const int64_t NC = (Tlen + 31) / 32, groups = (NC + 3) / 4;
     if (B * H > 0x7fffffffLL || groups > 65535) return MRX_ERR_INVALID_ARG;
-    hipLaunchKernelGGL((delta_tm_kernel<T, PRO>), dim3((unsigned)(B * H), (unsigned)groups), dim3(256), 0, st,
-                       (const T *)k, (const T *)beta, done, done_f32, (T *)Tm_chk, (int)Tlen, (int)H, (int)NC);
-    return launch_status();
+    return launch_kernel((delta_tm_kernel<T, PRO>), dim3((unsigned)(B * H), (unsigned)groups), dim3(256), 0, st,
+                         (const T *)k, (const T *)beta, done, done_f32, (T *)Tm_chk, (int)Tlen, (int)H, (int)NC);
 }
 }  // namespace
 

@@ -685,12 +685,13 @@ int launch_fwd(hipStream_t st, const void *a, const void *b, const void *done,
     const bool al8 = aligned(a, 8) && aligned(b, 8) && aligned(h, 8) && aligned(h0, 8) &&
                      aligned(P0, 8) && aligned(h_last, 8) && aligned(P_last, 8);
     const ScanPlan pl = plan_scan(B, T, D, sizeof(E), al16, al8, false);
+    int rc = MRX_ERR_LAUNCH;
     if (pl.stream) {
         const int64_t cpr = D / pl.vec;
         const dim3 grid((unsigned)((B * cpr + 255) / 256)), block(256);
         vec_switch<E>(pl.vec, [&](auto vc) {
             constexpr int VEC = decltype(vc)::value;
-            hipLaunchKernelGGL((diag_scan_fwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8), MG>), grid, block, 0, st,
+            rc = launch_kernel((diag_scan_fwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8), MG>), grid, block, 0, st,
                                (const E *)a, (const E *)b, done, done_f32, (const E *)h0, (const E *)P0,
                                (E *)h, (E *)h_last, (E *)P_last, B, (int)T, D, cpr, a_ti);
         });
@@ -699,12 +700,12 @@ int launch_fwd(hipStream_t st, const void *a, const void *b, const void *done,
         const size_t smem = scan_smem(pl.nw, sizeof(E) * pl.vec);
         vec_switch<E>(pl.vec, [&](auto vc) {
             constexpr int VEC = decltype(vc)::value;
-            hipLaunchKernelGGL((diag_scan_fwd_kernel<E, VEC, MG>), grid, block, smem, st, (const E *)a,
+            rc = launch_kernel((diag_scan_fwd_kernel<E, VEC, MG>), grid, block, smem, st, (const E *)a,
                                (const E *)b, done, done_f32, (const E *)h0, (const E *)P0, (E *)h,
                                (E *)h_last, (E *)P_last, (int)T, D, pl.tiles, pl.nw, a_ti);
         });
     }
-    return launch_status();
+    return rc;
 }
 
 // MG (E = float): a holds z, hx holds h~ (else unused), da and db receive dz and dh~.
@@ -718,12 +719,13 @@ int launch_bwd(hipStream_t st, const void *a, const void *hx, const void *h, con
     const bool al8 = aligned(a, 8) && aligned(hx, 8) && aligned(h, 8) && aligned(g, 8) && aligned(h0, 8) &&
                      aligned(g_last, 8) && aligned(da, 8) && aligned(db, 8) && aligned(dh0, 8);
     const ScanPlan pl = plan_scan(B, T, D, sizeof(E), al16, al8, true);
+    int rc = MRX_ERR_LAUNCH;
     if (pl.stream) {
         const int64_t cpr = D / pl.vec;
         const dim3 grid((unsigned)((B * cpr + 255) / 256)), block(256);
         vec_switch<E>(pl.vec, [&](auto vc) {
             constexpr int VEC = decltype(vc)::value;
-            hipLaunchKernelGGL((diag_scan_bwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8), MG>), grid, block, 0, st,
+            rc = launch_kernel((diag_scan_bwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8), MG>), grid, block, 0, st,
                                (const E *)a, (const E *)hx, (const E *)h, done, done_f32, (const E *)h0, (const E *)g,
                                (const E *)g_last, (E *)da, (E *)db, (E *)dh0, B, (int)T, D, cpr, a_ti);
         });
@@ -732,13 +734,13 @@ int launch_bwd(hipStream_t st, const void *a, const void *hx, const void *h, con
         const size_t smem = scan_smem(pl.nw, sizeof(E) * pl.vec);
         vec_switch<E>(pl.vec, [&](auto vc) {
             constexpr int VEC = decltype(vc)::value;
-            hipLaunchKernelGGL((diag_scan_bwd_kernel<E, VEC, MG>), grid, block, smem, st, (const E *)a,
+            rc = launch_kernel((diag_scan_bwd_kernel<E, VEC, MG>), grid, block, smem, st, (const E *)a,
                                (const E *)hx, (const E *)h, done, done_f32, (const E *)h0, (const E *)g,
                                (const E *)g_last, (E *)da, (E *)db, (E *)dh0, (int)T, D, pl.tiles,
                                pl.nw, a_ti);
         });
     }
-    return launch_status();
+    return rc;
 }
 
 template <typename E>
@@ -757,13 +759,14 @@ int launch_last(hipStream_t st, const void *a, const void *b, const void *done, 
     while (vec > 1 && B * (D / vec) < 2048 * 64) vec >>= 1;  // keep at least 2048 waves when the shape allows
     const int64_t cpr = D / vec;
     const dim3 grid((unsigned)((B * cpr + 255) / 256)), block(256);
+    int rc = MRX_ERR_LAUNCH;
     vec_switch<E>(vec, [&](auto vc) {
         constexpr int VEC = decltype(vc)::value;
-        hipLaunchKernelGGL((diag_scan_last_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8)>), grid, block, 0, st,
+        rc = launch_kernel((diag_scan_last_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8)>), grid, block, 0, st,
                            (const E *)a, (const E *)b, done, done_f32, (const E *)h0, (E *)h_last, B, (int)T, D,
                            cpr, a_group);
     });
-    return launch_status();
+    return rc;
 }
 
 bool scan_shape_ok(int64_t B, int64_t T, int64_t D)

@@ -117,10 +117,9 @@ int launch_step(hipStream_t st, const void *q, const void *k, const void *v, con
                 int done_f32, const float *S_in, const float *z_in, void *o, float *S_out, float *z_out,
                 int64_t B, int64_t H, float eps)
 {
-    hipLaunchKernelGGL((step_kernel<T, DELTA, FMAP>), dim3((unsigned)(B * H)), dim3(256), 0, st, (const T *)q,
-                       (const T *)k, (const T *)v, (const T *)beta, done, done_f32, S_in, z_in, (T *)o, S_out,
-                       z_out, (int)H, eps);
-    return launch_status();
+    return launch_kernel((step_kernel<T, DELTA, FMAP>), dim3((unsigned)(B * H)), dim3(256), 0, st, (const T *)q,
+                         (const T *)k, (const T *)v, (const T *)beta, done, done_f32, S_in, z_in, (T *)o, S_out,
+                         z_out, (int)H, eps);
 }
 
 }  // namespace

@@ -265,14 +265,28 @@ def linear_attn_norm_bwd(q, k, v, done, chk, o, den, do, dS_last=None, dz_last=N
     return dq, dk_, dv_, dS0, dz0
 
 
-def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prologue=False, tm_scratch=None):
+_FACTORS = {None: _lib.MRX_FACTORS_AUTO, "auto": _lib.MRX_FACTORS_AUTO, "parallel": _lib.MRX_FACTORS_PARALLEL,
+            "inline": _lib.MRX_FACTORS_INLINE}
+
+
+def init(device=None):
+    """Per-device set-up of the library (mrx_init): optional, the first launch on a device does
+    the same, but it must precede a HIP-graph capture that holds the first call on that device."""
+    lib = _lib.load()
+    dev = torch.cuda.current_device() if device is None else int(device)
+    _lib.check(lib.mrx_init(dev), "mrx_init")
+
+
+def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prologue=False, tm_scratch=None,
+                   factor_path=None):
     """Returns (o, S_last fp32, chk) where chk = (S_chk, Tm_chk) are the residuals the
     backward call needs, or None.  out = (o, S_last, S_chk, Tm_chk) reuses buffers of an earlier
     call with the same shapes instead of allocating.  prologue=True: k is L2-normalised and
     beta = sigmoid(beta) inside the kernel (mrx_deltanet_fwd).
     tm_scratch (only without residuals): give the library a buffer for the triangular factors
     anyway, which lets it compute them chunk-parallel while the device is not full.  None: when
-    B*H is at most two sequences per compute unit, which is when the library uses it."""
+    B*H is at most two sequences per compute unit, which is when the library uses it.
+    factor_path: None / "auto" (by occupancy), "parallel" or "inline" (mrx_factor_path)."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
     _chk(beta, "beta", dt, (B, T, H))
@@ -303,7 +317,7 @@ def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prolog
     name = "mrx_deltanet_fwd" if prologue else "mrx_delta_rule_fwd"
     st = getattr(lib, name)(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done),
                             _ptr(S0), _ptr(o), _ptr(S_last), _ptr(S_chk), _ptr(Tm_chk), B, T, H,
-                            dk, dv, _DT[dt], dd)
+                            dk, dv, _DT[dt], dd, _FACTORS[factor_path])
     _lib.check(st, name)
     return o, S_last, ((S_chk, Tm_chk) if save_chk else None)
 

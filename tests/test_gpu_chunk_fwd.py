@@ -138,40 +138,31 @@ def test_delta_rule_factor_paths_agree(dtype, prologue):
             assert relerr(a, b_[sl].float().cpu().numpy()) <= tol
 
 
-def test_factor_policy_from_the_environment(tmp_path):
-    """MRX_DELTA_FACTORS=parallel takes the chunk-parallel factor kernel on a batch above the
-    occupancy threshold (read once per process, hence the child process); same results as the
-    default route up to rounding."""
-    import os
-    import subprocess
-    import sys
+def test_factor_path_argument():
+    """factor_path = parallel takes the chunk-parallel factor kernel on a batch above the occupancy
+    threshold, inline never does; same results as each other up to rounding, and the automatic
+    choice above the threshold is the inline one bit for bit."""
     from memorax_amd import kernels as K
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     H, T = 8, 70
     B = 2 * cus // H + 3
-    script = f"""
-import sys, numpy as np, torch
-sys.path.insert(0, {os.path.dirname(os.path.dirname(os.path.abspath(__file__)))!r})
-from memorax_amd import kernels as K
-g = torch.Generator(device="cuda").manual_seed(5)
-q, k, v = (torch.randn(({B}, {T}, {H}, 64), device="cuda", generator=g).to(torch.bfloat16) for _ in range(3))
-k = torch.nn.functional.normalize(k.float(), dim=-1).to(torch.bfloat16)
-beta = torch.rand(({B}, {T}, {H}), device="cuda", generator=g).to(torch.bfloat16)
-done = torch.rand(({B}, {T}), device="cuda", generator=g) < 0.05
-o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done)
-np.savez(sys.argv[1], o=o.float().cpu().numpy(), Sl=Sl.cpu().numpy(), Tm=chk[1].float().cpu().numpy())
-"""
+    g = torch.Generator(device="cuda").manual_seed(5)
+    q, k, v = (torch.randn((B, T, H, 64), device="cuda", generator=g).to(torch.bfloat16) for _ in range(3))
+    k = torch.nn.functional.normalize(k.float(), dim=-1).to(torch.bfloat16)
+    beta = torch.rand((B, T, H), device="cuda", generator=g).to(torch.bfloat16)
+    done = torch.rand((B, T), device="cuda", generator=g) < 0.05
     out = {}
-    for policy in ("inline", "parallel"):
-        path = str(tmp_path / f"{policy}.npz")
-        env = dict(os.environ, MRX_DELTA_FACTORS=policy)
-        print(f"case factor_policy {policy}", flush=True)
-        subprocess.run([sys.executable, "-c", script, path], env=env, check=True, timeout=100)
-        out[policy] = np.load(path)
+    for path in ("inline", "parallel", "auto"):
+        print(f"case factor_path {path}", flush=True)
+        o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done, factor_path=path)
+        out[path] = dict(o=o.float().cpu().numpy(), Sl=Sl.cpu().numpy(), Tm=chk[1].float().cpu().numpy())
     a, b = out["inline"], out["parallel"]
     assert not np.array_equal(a["Tm"], b["Tm"])  # two different kernels made the factors
     for n in ("o", "Sl", "Tm"):
         assert relerr(torch.from_numpy(a[n]), b[n]) <= TOL_BF16, n
+        assert np.array_equal(out["auto"][n], a[n]), n
+    with pytest.raises(KeyError):
+        K.delta_rule_fwd(q, k, v, beta, done, factor_path="sideways")
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])

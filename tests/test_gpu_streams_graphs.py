@@ -41,8 +41,10 @@ def test_side_stream_equals_default_stream():
 
 def test_graph_replays_of_forward_and_backward():
     from memorax_amd import kernels as K
+    K.init()   # per-device set-up (LDS limits of every kernel) before anything is captured; idempotent
+    K.init(torch.cuda.current_device())
     static = _delta_inputs(2)
-    # first calls outside the capture: they set the kernels' LDS limits and size the buffers
+    # first calls outside the capture: they size the buffers
     o, Sl, chk = K.delta_rule_fwd(static["q"], static["k"], static["v"], static["beta"], static["done"])
     fwd_out = (o, Sl, chk[0], chk[1])
     bwd_out = K.delta_rule_bwd(static["q"], static["k"], static["v"], static["beta"], static["done"], chk,
