@@ -7,6 +7,10 @@ One "step" = one forward + backward pass of the DeltaNet delta rule over the
 synthetic batch of BASELINE configuration 4 (B=64, H=8, T=1024, d=64, bf16 inputs,
 fp32 state, reset mask Bernoulli(0.002)); inputs are resident in HBM before the
 timed region.  Prints ONE JSON line.  Only one GPU is used: --gpus > 1 exits.
+
+The other configurations (diagonal scan: configs[0]; linear attention: configs[1], configs[2];
+the sequence kernels of the torso: configs[4]) are timed first and reported as secondary blocks of
+the same line; the headline step is timed after them, on a device that is already at its clocks.
 """
 from __future__ import annotations
 
@@ -19,7 +23,9 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
+MFMA_BF16_PEAK = 2.5e15    # MI355X dense bf16 matrix peak, flop/s, published
+MFMA_F32_PEAK = 157.3e12   # MI355X fp32 matrix peak, flop/s, published
 # Algorithmic HBM bytes per (b, t, h) token-head, d = 64, bf16:
 #   forward : read q,k,v (3*128) + beta (2), write o (128)                    = 514
 #   backward: read q,k,v,do (4*128) + beta (2), write dq,dk,dv (3*128) + dbeta (2) = 900
@@ -29,6 +35,41 @@ BYTES_FWD, BYTES_BWD = 514, 900
 # (summary kept under profiles/).  The excess over the algorithmic bytes is the forward's
 # per-chunk residuals (state checkpoints and triangular factors) being read back.
 TRAFFIC_BWD_BYTES = 655.1e6
+# Matrix-pipe busy fraction of delta_bwd_kernel from rocprofv3 --pmc (SQ_VALU_MFMA_BUSY_CYCLES over
+# SQ_BUSY_CYCLES per SIMD), same workload; summary and command under profiles/.
+MFMA_BUSY_BWD = 0.149
+MFMA_BUSY_SOURCE = "profiles/delta_rule_kernels_counters_B64_T1024_H8_d64_bf16.md"
+CLOCK_RAMP_S = 0.1         # untimed load before the warm-up steps, so that short runs see a device at its clocks
+
+
+def delta_flops(C, d=64):
+    """Matrix flops per (b, t, h) token-head of the delta rule in WY chunk form with C-step chunks
+    (dense, no causal skip): forward 10 C d + 6 d^2 + 2/3 C^2, backward 2.5 x forward."""
+    fwd = 10 * C * d + 6 * d * d + 2.0 * C * C / 3.0
+    return fwd, 2.5 * fwd
+
+
+def linear_attn_flops(C, d=64):
+    """Chunk-form linear attention: forward 4 C d + 4 d^2, backward 10 C d + 10 d^2 per token-head."""
+    return 4 * C * d + 4 * d * d, 10 * C * d + 10 * d * d
+
+
+def synthetic(np, cfg, shape=None):
+    """Seeded fp32 inputs of BASELINE configuration cfg (1-based index into its list)."""
+    rng = np.random.default_rng(1000 + cfg)
+    if cfg == 2:
+        B, T, H, d = shape or (64, 256, 4, 64)
+        q, k, v = ((rng.standard_normal((B, T, H, d)) / 8.0).astype(np.float32) for _ in range(3))
+        return dict(q=q, k=k, v=v, done=rng.random((B, T)) < 0.005)
+    if cfg == 4:
+        B, T, H, d = shape or (64, 1024, 8, 64)
+        q = rng.standard_normal((B, T, H, d)).astype(np.float32)
+        k = rng.standard_normal((B, T, H, d)).astype(np.float32)
+        k /= np.linalg.norm(k, axis=-1, keepdims=True)
+        v = rng.standard_normal((B, T, H, d)).astype(np.float32)
+        beta = (1.0 / (1.0 + np.exp(-rng.standard_normal((B, T, H))))).astype(np.float32)
+        return dict(q=q, k=k, v=v, beta=beta, done=rng.random((B, T)) < 0.002)
+    raise ValueError(cfg)
 
 
 def main() -> int:
@@ -37,7 +78,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--all", action="store_true", help="also time the other configurations")
+    ap.add_argument("--all", action="store_true",
+                    help="also time the whole torso with its dense layers, the single-step kernels and the RTRL scan")
+    ap.add_argument("--headline-only", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain elementwise kernel of known size (256 MiB read, 256 MiB "
                          "written) so that a rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE run can be scaled")
@@ -51,15 +94,34 @@ def main() -> int:
     import torch
 
     from memorax_amd import kernels as K
-    from oracle import memoroid as M
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
+    K.init()
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()  # noqa: E731
+
+    secondary = {}
+    if not args.headline_only:
+        secondary["scan"] = bench_scan(torch, K)
+        secondary["linear_attention"] = bench_linear_attention(torch, K, np, dev)
+        secondary["torso"] = bench_torso_kernels(torch, K)
+        if args.all:
+            secondary["torso"].update(bench_torso_full(torch, K))
+            secondary["step"] = bench_step(torch, K)
+            secondary["rtrl"] = bench_rtrl(torch, K)
+        torch.cuda.empty_cache()
+    if args.calibrate:
+        cx = torch.zeros(64 * 1024 * 1024, device="cuda")  # 256 MiB fp32
+        cy = torch.empty_like(cx)
+        for _ in range(3):
+            torch.add(cx, 1.0, out=cy)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del cx, cy
+
     bf = torch.bfloat16
     B, T, H, d = 64, 1024, 8, 64
-    x = M.make_inputs(4, (B, T, H, d))
+    x = synthetic(np, 4, (B, T, H, d))
     do_np = np.random.default_rng(2004).standard_normal((B, T, H, d)).astype(np.float32)
-    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()  # noqa: E731
     q, k, v, beta, do = (dev(a).to(bf) for a in (x["q"], x["k"], x["v"], x["beta"], do_np))
     done = dev(x["done"])
     torch.cuda.synchronize()
@@ -73,6 +135,14 @@ def main() -> int:
         K.delta_rule_fwd(q, k, v, beta, done, out=fwd_out)
         return K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, out=bwd_out)
 
+    # The device needs some 30 ms of continuous load to reach its clocks (measured: 20-step batches
+    # right after an idle stretch read 0.32, 0.29, 0.28, 0.27, 0.27 ms per step): an untimed ramp of the
+    # same work comes first, outside the W warm-up steps and the K timed ones.
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < CLOCK_RAMP_S:
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -85,7 +155,7 @@ def main() -> int:
     # per-kernel durations with HIP events on the stream the kernels are launched on
     ev = lambda: torch.cuda.Event(enable_timing=True)  # noqa: E731
     tfs, tbs = [], []
-    for _ in range(args.steps):
+    for _ in range(max(args.steps, 50)):
         e0, e1, e2 = ev(), ev(), ev()
         e0.record()
         K.delta_rule_fwd(q, k, v, beta, done, out=fwd_out)
@@ -95,11 +165,14 @@ def main() -> int:
         torch.cuda.synchronize()
         tfs.append(e0.elapsed_time(e1))
         tbs.append(e1.elapsed_time(e2))
-    tf_ms, tb_ms = sum(tfs) / args.steps, sum(tbs) / args.steps
+    tf_ms, tb_ms = sum(tfs) / len(tfs), sum(tbs) / len(tbs)
     pct = lambda xs: {f"p{p}_ms": float(np.percentile(xs, p)) for p in (10, 50, 90)}  # noqa: E731
     nth = B * T * H
     bwd_gbs = BYTES_BWD * nth / (tb_ms * 1e-3) / 1e9
     fwd_gbs = BYTES_FWD * nth / (tf_ms * 1e-3) / 1e9
+    C = K.chunk_size(bf, delta=True)
+    fl_f, fl_b = delta_flops(C)
+    mfma = lambda fl, ms: fl * nth / (ms * 1e-3) / MFMA_BF16_PEAK  # noqa: E731
 
     out = {
         "metric": "tokens/sec (B×T) fwd+bwd + % HBM/MFMA roofline, DeltaNet T=1024 on 1 GPU",
@@ -114,36 +187,31 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
+        "clock_ramp_ms": CLOCK_RAMP_S * 1e3,
         "config": {"workload": "configs[3]: DeltaNet delta rule fwd+bwd, B=64 H=8 T=1024 d=64, "
-                               "bf16 in / fp32 state, chunk 32, resets p=0.002"},
+                               f"bf16 in / fp32 state, chunk {C}, resets p=0.002"},
         "roofline": {
             "bound": "hbm", "kernel": "delta_bwd_kernel", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": TRAFFIC_BWD_BYTES,
             "launch_ms": tb_ms, "algorithmic_bytes": BYTES_BWD * nth,
+            # the matrix-pipe side of the same launch: chunk-form flops at the kernel's chunk length
+            # over the launch time, against the dense bf16 peak; and the pipe's busy fraction by counter
+            "mfma_frac": mfma(fl_b, tb_ms), "mfma_flops": fl_b * nth, "mfma_peak": MFMA_BF16_PEAK,
+            "mfma_busy": MFMA_BUSY_BWD, "mfma_busy_source": MFMA_BUSY_SOURCE,
         },
         "kernels": {
-            "delta_fwd": {"ms": tf_ms, "GB/s": fwd_gbs, "frac_hbm": fwd_gbs / HBM_PEAK_GBS, **pct(tfs)},
-            "delta_bwd": {"ms": tb_ms, "GB/s": bwd_gbs, "frac_hbm": bwd_gbs / HBM_PEAK_GBS, **pct(tbs)},
+            "delta_fwd": {"ms": tf_ms, "GB/s": fwd_gbs, "frac_hbm": fwd_gbs / HBM_PEAK_GBS,
+                          "frac_mfma": mfma(fl_f, tf_ms), **pct(tfs)},
+            "delta_bwd": {"ms": tb_ms, "GB/s": bwd_gbs, "frac_hbm": bwd_gbs / HBM_PEAK_GBS,
+                          "frac_mfma": mfma(fl_b, tb_ms), **pct(tbs)},
             "fwd+bwd": {"ms": tf_ms + tb_ms,
-                        "GB/s": (BYTES_FWD + BYTES_BWD) * nth / ((tf_ms + tb_ms) * 1e-3) / 1e9},
+                        "GB/s": (BYTES_FWD + BYTES_BWD) * nth / ((tf_ms + tb_ms) * 1e-3) / 1e9,
+                        "frac_mfma": mfma(fl_f + fl_b, tf_ms + tb_ms)},
         },
     }
-
-    if args.calibrate:
-        cx = torch.zeros(64 * 1024 * 1024, device="cuda")  # 256 MiB fp32
-        cy = torch.empty_like(cx)
-        for _ in range(3):
-            torch.add(cx, 1.0, out=cy)  # reads 256 MiB, writes 256 MiB
-        torch.cuda.synchronize()
-        del cx, cy
-    out["scan"] = bench_scan(torch, K, M, dev)
-    if args.all:
-        out["linear_attention"] = bench_linear_attention(torch, K, M, dev)
-        out["torso"] = bench_torso(torch, K)
-        out["step"] = bench_step(torch, K)
-        out["rtrl"] = bench_rtrl(torch, K)
+    out.update(secondary)
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(np, M, x, do_np)
+        out["cpu_baseline"] = cpu_baseline(np, x, do_np)
     print(json.dumps(out))
     return 0
 
@@ -161,7 +229,7 @@ def _time_ms(torch, fn, iters=20, warm=3):
     return e0.elapsed_time(e1) / iters
 
 
-def bench_scan(torch, K, M, dev):
+def bench_scan(torch, K):
     """Diagonal scan forward: configuration 1 (32,128,256) and a shape that saturates HBM."""
     res = {}
     for name, shape in (("cfg1_32x128x256", (32, 128, 256)), ("torso_1024x128x256", (1024, 128, 256)),
@@ -224,10 +292,12 @@ def bench_scan(torch, K, M, dev):
     return res
 
 
-def bench_linear_attention(torch, K, M, dev):
-    """Configuration 2 (fp32, elu+1, resets) and configuration 3 (bf16, no resets)."""
+def bench_linear_attention(torch, K, np, dev):
+    """Configuration 2 (configs[1]: fp32, elu+1, resets) and configuration 3 (configs[2]: bf16, no resets),
+    forward + backward, with the fractions of the roofline that binds each on paper: the fp32 matrix
+    peak for configuration 2 (41 flop/B against a balance of 20), HBM for configuration 3."""
     res = {}
-    x = M.make_inputs(2)
+    x = synthetic(np, 2)
     q, k, v = (dev(x[n]) for n in ("q", "k", "v"))
     dn = dev(x["done"])
     do = torch.randn_like(v)
@@ -236,8 +306,12 @@ def bench_linear_attention(torch, K, M, dev):
         o, Sl, chk = K.linear_attn_fwd(q, k, v, dn, None, 1)
         K.linear_attn_bwd(q, k, v, dn, chk, do, None, 1, want_dS0=False)
     ms = _time_ms(torch, f2)
-    res["cfg2_f32_64x256x4x64"] = {"ms": ms, "tokens/s": 64 * 256 / ms * 1e3,
-                                   "GB/s": 2816 * 64 * 256 * 4 / ms / 1e6}
+    nth = 64 * 256 * 4
+    ff, fb = linear_attn_flops(K.chunk_size(torch.float32))
+    res["cfg2_f32_64x256x4x64"] = {"ms": ms, "tokens/s": 64 * 256 / ms * 1e3, "GB/s": 2816 * nth / ms / 1e6,
+                                   "frac_hbm": 2816 * nth / ms / 1e6 / HBM_PEAK_GBS,
+                                   "frac_mfma_f32": (ff + fb) * nth / (ms * 1e-3) / MFMA_F32_PEAK}
+    del q, k, v, do
     Bn, Tn, Hn = 256, 4096, 8   # configuration 3 at full size (11.8 GB of q, k, v, do, o, dq, dk, dv)
     q, k, v, do = (torch.randn((Bn, Tn, Hn, 64), device="cuda").div_(8).to(torch.bfloat16) for _ in range(4))
     dn = torch.zeros((Bn, Tn), dtype=torch.bool, device="cuda")
@@ -246,8 +320,11 @@ def bench_linear_attention(torch, K, M, dev):
         o, Sl, chk = K.linear_attn_fwd(q, k, v, dn, None, 0)
         K.linear_attn_bwd(q, k, v, dn, chk, do, None, 0, want_dS0=False)
     ms = _time_ms(torch, f3, iters=5)
-    res["cfg3_bf16_256x4096x8x64"] = {"ms": ms, "tokens/s": Bn * Tn / ms * 1e3,
-                                           "GB/s": 1408 * Bn * Tn * Hn / ms / 1e6}
+    nth = Bn * Tn * Hn
+    ff, fb = linear_attn_flops(K.chunk_size(torch.bfloat16))
+    res["cfg3_bf16_256x4096x8x64"] = {"ms": ms, "tokens/s": Bn * Tn / ms * 1e3, "GB/s": 1408 * nth / ms / 1e6,
+                                      "frac_hbm": 1408 * nth / ms / 1e6 / HBM_PEAK_GBS,
+                                      "frac_mfma": (ff + fb) * nth / (ms * 1e-3) / MFMA_BF16_PEAK}
     # the same shape with a per-step scalar decay (Mamba cell algebra); + g in, edot out: 8 B more per token-head
     g = -torch.rand((Bn, Tn, Hn), device="cuda") * 0.1
 
@@ -318,17 +395,41 @@ def bench_step(torch, K):
     return res
 
 
-def bench_torso(torch, K):
-    """Configuration 5: 4 blocks of [RMSNorm -> DeltaNet(H=4, d=64) -> +x ; RMSNorm -> gated
-    linear recurrence -> +x], d_model 256, B=1024 envs x T=128, weights N(0, 0.02), done p=0.01.
-    Reports the whole torso (dense projections in torch included) and the sequence kernels alone."""
+def bench_torso_kernels(torch, K):
+    """Configuration 5 (configs[4]), the sequence kernels of one update: 4 blocks x (DeltaNet H=4, d=64
+    forward + backward, diagonal recurrence forward + backward) over B=1024 envs x T=128, done p=0.01."""
+    B, T, Fe, H, d = 1024, 128, 256, 4, 64
+    bf = torch.bfloat16
+    done = torch.rand(B, T, device="cuda") < 0.01
+    q, k, v = (torch.randn(B, T, H, d, device="cuda").to(bf) for _ in range(3))
+    k = torch.nn.functional.normalize(k.float(), dim=-1).to(bf)
+    beta = torch.rand(B, T, H, device="cuda").to(bf)
+    do = torch.randn_like(v)
+    z, hx, g = (torch.randn(B, T, Fe, device="cuda") for _ in range(3))
+
+    def kernels_only():
+        for _ in range(4):
+            o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done)
+            K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False)
+            h, _, _ = K.mingru_scan_fwd(z, hx, done, want_P=False)
+            K.mingru_scan_bwd(z, hx, h, done, None, g)
+    ms_k = _time_ms(torch, kernels_only, iters=10, warm=3)
+    by = 4 * ((BYTES_FWD + BYTES_BWD) * B * T * H + 36 * B * T * Fe)   # + MinGRU scan: 12 B fwd, 24 B bwd per element
+    return {"sequence_kernels_ms": ms_k, "sequence_kernels_tokens/s": B * T / ms_k * 1e3,
+            "sequence_kernels_GB/s": by / ms_k / 1e6, "sequence_kernels_frac_hbm": by / ms_k / 1e6 / HBM_PEAK_GBS}
+
+
+def bench_torso_full(torch, K):
+    """Configuration 5 through the host mirror, dense projections in torch included: 4 blocks of
+    [RMSNorm -> DeltaNet(H=4, d=64) -> +x ; RMSNorm -> gated linear recurrence -> +x], d_model 256,
+    weights N(0, 0.02)."""
     from memorax_amd import sequence_models as sm
     B, T, Fe, H, d = 1024, 128, 256, 4, 64
     torch.manual_seed(5)
     blocks = []
     for _ in range(4):
-        blocks += [sm.Residual(sm.PreNorm(sm.Memoroid(sm.DeltaNetCell(Fe, d, H)), Fe)),
-                   sm.Residual(sm.PreNorm(sm.GatedLinearRecurrence(Fe), Fe))]
+        blocks += [sm.Residual(sm.PreNorm(sm.Memoroid(sm.DeltaNetCell(Fe, d, H)), Fe, norm=sm.RMSNorm)),
+                   sm.Residual(sm.PreNorm(sm.GatedLinearRecurrence(Fe), Fe, norm=sm.RMSNorm))]
     torso = sm.Stack(blocks).cuda()
     for p in torso.parameters():
         if p.dim() > 1:
@@ -346,28 +447,11 @@ def bench_torso(torch, K):
         y.float().pow(2).mean().backward()
     ms_full = _time_ms(torch, full, iters=5, warm=2)
     ms_full32 = _time_ms(torch, lambda: full(False), iters=3, warm=1)
-
-    bf = torch.bfloat16
-    q, k, v = (torch.randn(B, T, H, d, device="cuda").to(bf) for _ in range(3))
-    k = torch.nn.functional.normalize(k.float(), dim=-1).to(bf)
-    beta = torch.rand(B, T, H, device="cuda").to(bf)
-    do = torch.randn_like(v)
-    a = torch.rand(B, T, Fe, device="cuda") * 0.099 + 0.9
-    bb, g = torch.randn(B, T, Fe, device="cuda"), torch.randn(B, T, Fe, device="cuda")
-
-    def kernels_only():
-        for _ in range(4):
-            o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done)
-            K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False)
-            h, _, _ = K.linear_scan_fwd(a, bb, done, want_P=False)
-            K.linear_scan_bwd(a, h, done, None, g)
-    ms_k = _time_ms(torch, kernels_only, iters=5, warm=2)
     return {"full_torso_ms": ms_full, "full_torso_tokens/s": B * T / ms_full * 1e3,
-            "full_torso_ms_fp32_projections": ms_full32,
-            "sequence_kernels_ms": ms_k, "sequence_kernels_tokens/s": B * T / ms_k * 1e3}
+            "full_torso_ms_fp32_projections": ms_full32}
 
 
-def cpu_baseline(np, M, x, do_np):
+def cpu_baseline(np, x, do_np):
     """The C restatement (oracle/c, fp32 state, OpenMP) on a bounded sample of the same
     workload (configuration 4, forward + backward, one pass)."""
     from oracle import clib

@@ -106,10 +106,12 @@ struct MinGru {
 
 constexpr int TS = 8;  // time steps a wave holds in registers per super-step
 
-// Forward.  grid = B * tiles workgroups, block = 64 * NW threads.
+// Forward.  grid = B * tiles workgroups, block = 64 * NW threads, NW <= MAXW (8, or 16 for the
+// one-vector-lane instances that small shapes take: with 16 waves of 8 steps a sequence of up to 128
+// steps is one super-step, every load of the workgroup in flight at once and a single barrier).
 // smem: sH[2][NW][64] Vec, sP[2][NW][64] Vec, sF[2][NW] int.
-template <typename E, int VEC, bool MG = false>
-__global__ void __launch_bounds__(512)
+template <typename E, int VEC, bool MG = false, int MAXW = 8>
+__global__ void __launch_bounds__(64 * MAXW)
 diag_scan_fwd_kernel(const E *__restrict__ a, const E *__restrict__ b,
                      const void *__restrict__ done, int done_f32,
                      const E *__restrict__ h0, const E *__restrict__ P0,
@@ -244,8 +246,8 @@ diag_scan_fwd_kernel(const E *__restrict__ a, const E *__restrict__ b,
 // Backward: the same scan walked from t = T-1 down with coefficient conj(a_{t+1}),
 // cut where done_{t+1}; reversed index r = T-1-t runs forward.
 // MG: a holds z, hx holds x = h~; da receives dz and db receives dx.
-template <typename E, int VEC, bool MG = false>
-__global__ void __launch_bounds__(512)
+template <typename E, int VEC, bool MG = false, int MAXW = 8>
+__global__ void __launch_bounds__(64 * MAXW)
 diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hx, const E *__restrict__ hfw,
                      const void *__restrict__ done, int done_f32,
                      const E *__restrict__ h0, const E *__restrict__ g,
@@ -275,7 +277,11 @@ diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hx, const E 
     int buf = 0;
     for (int r0 = 0; r0 < T; r0 += span) {
         const int rs = r0 + w * TS;
-        V x[TS], p[TS];
+        // Everything the super-step reads is requested here, before the barrier: h_{t-1} (and the
+        // MinGRU projections of step t) are only needed once lam_t is known, but a load issued after the
+        // barrier would be a second trip to memory on the critical path.
+        V x[TS], p[TS], hp[TS];
+        V zt[MG ? TS : 1], xt[MG ? TS : 1];
         unsigned cmask = 0;  // bit s: chain cut between step t and t+1 (done_{t+1})
         unsigned dmask = 0;  // bit s: done_t
 #pragma unroll
@@ -283,6 +289,7 @@ diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hx, const E 
             const int t = T - 1 - (rs + s);
             p[s] = vfill<E, VEC>(O::one());
             x[s] = vfill<E, VEC>(O::zero());
+            hp[s] = vfill<E, VEC>(O::zero());
             if (t >= 0) {
                 if (act) {
                     const int64_t off = (row0 + t) * D + col;
@@ -291,6 +298,14 @@ diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hx, const E 
                         V av = *reinterpret_cast<const V *>(a + (a_ti ? col : off + D));
 #pragma unroll
                         for (int i = 0; i < VEC; ++i) p[s].v[i] = MG ? av.v[i] : O::conj(av.v[i]);  // MG: z_{t+1} for now
+                    }
+                    if (t > 0)
+                        hp[s] = *reinterpret_cast<const V *>(hfw + off - D);
+                    else if (h0)
+                        hp[s] = *reinterpret_cast<const V *>(h0 + bi * D + col);
+                    if constexpr (MG) {
+                        zt[s] = *reinterpret_cast<const V *>(a + off);
+                        xt[s] = *reinterpret_cast<const V *>(hx + off);
                     }
                 }
                 if (t + 1 < T && done_at(done, done_f32, row0 + t + 1)) cmask |= 1u << s;
@@ -371,23 +386,17 @@ diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hx, const E 
             const int t = T - 1 - (rs + s);
             if (t >= 0 && act) {
                 const int64_t off = (row0 + t) * D + col;
-                V hp = vfill<E, VEC>(O::zero());
-                if (t > 0)
-                    hp = *reinterpret_cast<const V *>(hfw + off - D);
-                else if (h0)
-                    hp = *reinterpret_cast<const V *>(h0 + bi * D + col);
                 const bool dn = (dmask >> s) & 1u;
                 V o;
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) {
-                    const E prod = O::mul(x[s].v[i], O::conj(hp.v[i]));
+                    const E prod = O::mul(x[s].v[i], O::conj(hp[s].v[i]));
                     o.v[i] = dn ? O::zero() : prod;
                 }
                 if constexpr (MG) {
-                    const V zt = *reinterpret_cast<const V *>(a + off), xt = *reinterpret_cast<const V *>(hx + off);
                     V oz, ox;
 #pragma unroll
-                    for (int i = 0; i < VEC; ++i) MinGru::grads(zt.v[i], xt.v[i], x[s].v[i], o.v[i], oz.v[i], ox.v[i]);
+                    for (int i = 0; i < VEC; ++i) MinGru::grads(zt[s].v[i], xt[s].v[i], x[s].v[i], o.v[i], oz.v[i], ox.v[i]);
                     *reinterpret_cast<V *>(db + off) = ox;
                     *reinterpret_cast<V *>(da + off) = oz;
                 } else {
@@ -634,7 +643,10 @@ struct ScanPlan {
 //  - widest vector the shapes/alignments allow, narrowed until there are >= 2048 wave columns;
 //  - forward: split time over up to 8 waves until ~8192 waves exist (the wave-split kernel at
 //    4 waves reached 5.7 TB/s on the 6.4 GB shape, the streaming kernel 5.1 TB/s); with no
-//    split left to do, stream;
+//    split left to do, stream; shapes so small that eight waves per workgroup still leave the
+//    device short of waves (one vector lane per thread by then) take sixteen, which makes a
+//    sequence of up to 128 steps a single super-step: the kernel's time is then one trip to
+//    memory and back instead of one per super-step;
 //  - backward (three loads per step): the streaming kernel wins whenever the columns alone
 //    give >= 2048 waves; below that, the wave-split kernel.
 ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, bool al8, bool bwd)
@@ -651,7 +663,8 @@ ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, boo
     const int tiles = (int)ntiles(vec);
     const int64_t waves = B * tiles;
     int nw = 1;
-    while (nw < 8 && waves * nw < 8192 && (int64_t)nw * TS < T) nw <<= 1;
+    const int maxw = vec == 1 ? 16 : 8;
+    while (nw < maxw && waves * nw < 8192 && (int64_t)nw * TS < T) nw <<= 1;
     const bool stream = bwd ? waves >= 2048 : nw == 1;
     return {vec, stream ? 1 : nw, tiles, stream};
 }
@@ -700,6 +713,14 @@ int launch_fwd(hipStream_t st, const void *a, const void *b, const void *done,
         const size_t smem = scan_smem(pl.nw, sizeof(E) * pl.vec);
         vec_switch<E>(pl.vec, [&](auto vc) {
             constexpr int VEC = decltype(vc)::value;
+            if constexpr (VEC == 1) {
+                if (pl.nw == 16) {
+                    rc = launch_kernel((diag_scan_fwd_kernel<E, 1, MG, 16>), grid, block, smem, st, (const E *)a,
+                                       (const E *)b, done, done_f32, (const E *)h0, (const E *)P0, (E *)h,
+                                       (E *)h_last, (E *)P_last, (int)T, D, pl.tiles, pl.nw, a_ti);
+                    return;
+                }
+            }
             rc = launch_kernel((diag_scan_fwd_kernel<E, VEC, MG>), grid, block, smem, st, (const E *)a,
                                (const E *)b, done, done_f32, (const E *)h0, (const E *)P0, (E *)h,
                                (E *)h_last, (E *)P_last, (int)T, D, pl.tiles, pl.nw, a_ti);
@@ -734,6 +755,15 @@ int launch_bwd(hipStream_t st, const void *a, const void *hx, const void *h, con
         const size_t smem = scan_smem(pl.nw, sizeof(E) * pl.vec);
         vec_switch<E>(pl.vec, [&](auto vc) {
             constexpr int VEC = decltype(vc)::value;
+            if constexpr (VEC == 1) {
+                if (pl.nw == 16) {
+                    rc = launch_kernel((diag_scan_bwd_kernel<E, 1, MG, 16>), grid, block, smem, st, (const E *)a,
+                                       (const E *)hx, (const E *)h, done, done_f32, (const E *)h0, (const E *)g,
+                                       (const E *)g_last, (E *)da, (E *)db, (E *)dh0, (int)T, D, pl.tiles,
+                                       pl.nw, a_ti);
+                    return;
+                }
+            }
             rc = launch_kernel((diag_scan_bwd_kernel<E, VEC, MG>), grid, block, smem, st, (const E *)a,
                                (const E *)hx, (const E *)h, done, done_f32, (const E *)h0, (const E *)g,
                                (const E *)g_last, (E *)da, (E *)db, (E *)dh0, (int)T, D, pl.tiles,

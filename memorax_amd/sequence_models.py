@@ -81,7 +81,10 @@ class MemoroidCellBase(nn.Module):
 
 
 class Memoroid(SequenceModel):
-    """memoroid.py:57-112 (without the RTRL hooks)."""
+    """memoroid.py:57-112 (without the RTRL hooks).  Works for every cell of this module: the
+    matrix-state cells (linear attention, Mamba, mLSTM) put the query among their elements, because
+    their kernels fuse the read-out contraction into the scan, so that ``scan`` returns the carry
+    like any other cell's."""
 
     def __init__(self, cell: MemoroidCellBase):
         super().__init__()
@@ -343,34 +346,27 @@ class LinearAttentionCell(MemoroidCellBase):
         return x.view(*x.shape[:2], self.num_heads, self.head_dim)
 
     def forward(self, x, **kwargs):
-        # pre-feature-map keys: phi is applied inside the kernel (and here for z)
-        return (self._heads(self.value(x)), self._heads(self.key(x)))
+        """Elements in kernel form: (v, k, q), keys and queries before the feature map (phi is applied
+        inside the kernel).  The reference's elements are (v phi(k)^T, phi(k)); the query joins them here
+        because the kernel contracts the state with it as it goes."""
+        return (self._heads(self.value(x)), self._heads(self.key(x)), self._heads(self.query(x)))
 
     def binary_operator(self, a, b):
         return tuple(x + y for x, y in zip(a, b))
 
     def scan(self, z, initial_carry, done):
-        """Returns h = (v, k_raw, S0, z0, done) for read(): the numerator needs the query, so the
-        recurrence, the running key sum and the read-out all run in read's one kernel."""
-        v, k_raw = z
-        S0, z0 = initial_carry            # (B,1,H,dv,dk), (B,1,H,dk)
-        return (v, k_raw, S0[:, 0], z0[:, 0], done), None
+        """The recurrence, the running key sum and the normalised read-out in one kernel per direction
+        (the single-step kernel when T = 1 and no gradient is asked for).  Returns h = the normalised
+        numerator (B,T,H,dv) and the carry (S (B,1,H,dv,dk), z (B,1,H,dk))."""
+        v, k_raw, q = z
+        S0, z0 = initial_carry
+        out, S_last, z_last = normalised_linear_attention(q, k_raw, v, done, S0[:, 0].float(), z0[:, 0].float(),
+                                                          "elu1", self.eps)
+        return out, (S_last[:, None], z_last[:, None])
 
     def read(self, h, x, **kwargs):
-        v, k_raw, S0, z0, done = h
-        q = self._heads(self.query(x))
-        out, S_last, z_last = normalised_linear_attention(q, k_raw, v, done, S0.float(), z0.float(), "elu1", self.eps)
-        self._carry = (S_last[:, None], z_last[:, None])
-        out = out.float().reshape(*x.shape[:2], -1)
+        out = h.float().reshape(*x.shape[:2], -1)
         return self.output_projection(self.norm(out).to(x.dtype))
-
-    def step(self, x, done, carry):
-        """Acting path (T = 1, no gradients): state update, normaliser and divide in one kernel
-        (what __call__, binary_operator and read of linear_attention.py:62-117 do for one step);
-        normalised_linear_attention picks the single-step kernel for such a call."""
-        h, _ = self.scan(self(x), carry, done)
-        y = self.read(h, x)
-        return self._carry, y
 
     def initialize_carry(self, key, input_shape):
         *batch, _ = input_shape
@@ -379,26 +375,11 @@ class LinearAttentionCell(MemoroidCellBase):
                 torch.zeros(*batch, 1, self.num_heads, self.head_dim, device=dev))
 
 
-class LinearAttention(SequenceModel):
-    """Memoroid(LinearAttentionCell) with the read-out fused around the kernel call: the
-    numerator needs q, k, v together, so the state leaf of the carry is produced by read."""
+class LinearAttention(Memoroid):
+    """Memoroid(LinearAttentionCell) under its own name."""
 
     def __init__(self, cell: LinearAttentionCell):
-        super().__init__()
-        self.cell = cell
-
-    def forward(self, inputs, done, initial_carry=None, **kwargs):
-        if initial_carry is None:
-            initial_carry = self.cell.initialize_carry(None, get_input_shape(inputs))
-        if inputs.shape[1] == 1 and not torch.is_grad_enabled():
-            return self.cell.step(inputs, done, initial_carry)
-        z = self.cell(inputs)
-        h, _ = self.cell.scan(z, initial_carry, done)
-        y = self.cell.read(h, inputs)
-        return self.cell._carry, y
-
-    def initialize_carry(self, key, input_shape):
-        return self.cell.initialize_carry(key, input_shape)
+        super().__init__(cell)
 
 
 class DeltaNetCell(MemoroidCellBase):
@@ -490,19 +471,20 @@ class MambaCell(MemoroidCellBase):
         return hidden, B_proj, C_proj, z, dt
 
     def forward(self, x, **kwargs):
-        """Elements in kernel form: (k = B dt, v = x, log-decay g = dt A); the reference's
-        (h, decay) are v (x) k and exp(g)."""
-        hidden, B_proj, _, _, dt = self._project(x)
+        """Elements in kernel form: (k = B dt, v = x, log-decay g = dt A, q = C); the reference's
+        (h, decay) are v (x) k and exp(g), and the C projection joins them because the kernel fuses the
+        contraction y_t = C_t . h_t into the scan."""
+        hidden, B_proj, C_proj, _, dt = self._project(x)
         g = dt * (-torch.exp(self.A_log))[None, None, :]
-        return (B_proj * dt[..., None], hidden, g)
+        return (B_proj * dt[..., None], hidden, g, C_proj)
 
     def binary_operator(self, a, b):
         h_i, decay_i = a
         h_j, decay_j = b
         return (decay_j * h_i + h_j, decay_j * decay_i)
 
-    def scan(self, z, initial_carry, done, q=None):
-        k, v, g = z
+    def scan(self, z, initial_carry, done):
+        k, v, g, q = z
         h0, decay0 = initial_carry                      # (B,1,H,N,P), (B,1,H,1,1)
         S0 = h0[:, 0].transpose(-1, -2).float().contiguous()   # kernel state is (P, N) = (d_v, d_k)
         o, S_last = gated_linear_attention(q.contiguous(), k.contiguous(), v.contiguous(), g.float(), done, S0)
@@ -527,24 +509,11 @@ class MambaCell(MemoroidCellBase):
                 torch.ones(*batch, 1, self.num_heads, 1, 1, device=dev))
 
 
-class Mamba(SequenceModel):
-    """Memoroid(MambaCell): the query (C projection) joins the scan because the kernel fuses the
-    contraction y_t = C_t . h_t into it."""
+class Mamba(Memoroid):
+    """Memoroid(MambaCell) under its own name."""
 
     def __init__(self, cell: MambaCell):
-        super().__init__()
-        self.cell = cell
-
-    def forward(self, inputs, done, initial_carry=None, **kwargs):
-        if initial_carry is None:
-            initial_carry = self.cell.initialize_carry(None, get_input_shape(inputs))
-        z = self.cell(inputs)
-        _, _, C_proj, _, _ = self.cell._project(inputs)
-        o, carry = self.cell.scan(z, initial_carry, done, q=C_proj)
-        return carry, self.cell.read(o, inputs)
-
-    def initialize_carry(self, key, input_shape):
-        return self.cell.initialize_carry(key, input_shape)
+        super().__init__(cell)
 
 
 class _BlockDiagonalDense(nn.Module):
@@ -565,13 +534,14 @@ class _BlockDiagonalDense(nn.Module):
 class mLSTMCell(MemoroidCellBase):
     """Matrix LSTM (mlstm.py:31-240).  Elements (C = k (x) v, log_f, n = k, m = log_i) combine by the
     max-stabilised gated sum of mlstm.py:190-206; read divides q C by max(|q . n|, exp(-m)) + 1e-6.
-    The stabiliser only rescales C and n by exp(-m), so the same numbers come from the plain gated
-    recurrence C~_t = f_t C~_{t-1} + i_t k_t v_t^T taken in units of exp(c) with one constant
-    c = max(log i, carried m) per sequence and head (every weight exp(log i - c) <= 1):
-        h = q C' / (max(|q . n'|, exp(-c)) + 1e-6 exp(m - c)).
-    q C' runs in the gated chunked kernel (k' = k exp(log i - c), log-decay log f), n' in the diagonal
-    scan, and m_t = max(m_{t-1} + log f_t, log i_t) is a cumulative maximum in log space.  Gates more
-    than about 80 nats below the running maximum underflow (the reference keeps them finite).
+    Unrolled, that operator is the recurrence
+        m_t = max(m_{t-1} + log f_t, log i_t)
+        C_t = exp(log f_t + m_{t-1} - m_t) C_{t-1} + exp(log i_t - m_t) k_t v_t^T      (n_t alike),
+    a gated linear recurrence whose log-decay g_t = log f_t + m_{t-1} - m_t and key weight
+    exp(log i_t - m_t) are both <= 1 whatever the gates do: m_t is a cumulative maximum in log space
+    (taken per episode), g and the weights follow from it elementwise, q C runs in the gated chunked
+    kernel and n in the diagonal scan.  State, normaliser and m come out in the reference's stabilised
+    units, step by step, so gates may drift by any amount inside an episode.
     Carry: (C (B,1,H,d,d), log_f (B,1,H,1,1), n (B,1,H,d,1), m (B,1,H,1,1)) as in the reference."""
 
     def __init__(self, features, hidden_dim, num_heads=4, conv_kernel_size=4, in_features=None):
@@ -606,13 +576,13 @@ class mLSTMCell(MemoroidCellBase):
         return heads(self.query(u)), heads(self.key(u)), heads(self.value(x_mlstm)), z, u
 
     def forward(self, x, **kwargs):
-        """Elements in kernel form: (k / sqrt(d), v, log_i, log_f)."""
+        """Elements in kernel form: (k / sqrt(d), v, log_i, log_f, q)."""
         Bn, T, _ = x.shape
         q, k, v, _, _ = self._project(x)
         gate_input = torch.cat([q, k, v], dim=-1).reshape(Bn, T, -1)
         log_i = self.i_gate(gate_input).float()
         log_f = -F.softplus(-self.f_gate(gate_input).float())
-        return (k / math.sqrt(k.shape[-1]), v, log_i, log_f)
+        return (k / math.sqrt(k.shape[-1]), v, log_i, log_f, q)
 
     def binary_operator(self, a, b):
         C_a, log_f_a, n_a, m_a = a
@@ -622,41 +592,44 @@ class mLSTMCell(MemoroidCellBase):
         sa, sb = torch.exp(m_a_decayed - m), torch.exp(m_b - m)
         return (sa * C_a + sb * C_b, log_f_a + log_f_b, sa * n_a + sb * n_b, m)
 
-    def scan(self, z, initial_carry, done, q=None):
-        k, v, log_i, log_f = z
+    # A log-decay below this is a state multiplied by exp(-60) < 1e-26 next to a new term of weight one:
+    # clamping keeps the in-chunk prefix sums of the kernel small (no cancellation between them).
+    _G_FLOOR = -60.0
+
+    def scan(self, z, initial_carry, done):
+        k, v, log_i, log_f, q = z
         C0, lf0, n0, m0 = initial_carry
         Bn, T, H, d = k.shape
-        m0_ = m0[:, 0, :, 0, 0].float()                                        # (B,H)
-        c = torch.maximum(log_i.max(dim=1).values, m0_).detach()                # (B,H)
-        k_in = k.float() * torch.exp(log_i - c[:, None])[..., None]
-        w0 = torch.exp(m0_ - c)                                                 # <= 1; 0 for the initial carry
-        S0 = (C0[:, 0].float() * w0[..., None, None]).transpose(-1, -2).contiguous()
-        num, S_last = gated_linear_attention(q.float().contiguous(), k_in.contiguous(), v.float().contiguous(),
-                                             log_f.contiguous(), done, S0)
-        a = torch.exp(log_f)[..., None].expand(Bn, T, H, d).reshape(Bn, T, H * d).contiguous()
-        nvec, n_last, _ = linear_scan(a, k_in.reshape(Bn, T, H * d).contiguous(), done,
-                                      (n0[:, 0, :, :, 0].float() * w0[..., None]).reshape(Bn, H * d).contiguous())
-        qn = (q.float() * nvec.view(Bn, T, H, d)).sum(-1)                        # (B,T,H)
-        # m_t = max(m_{t-1} + log f_t, log i_t), restarted at resets: F_t + running max of (log i - F)
         ones = torch.ones(H, device=k.device)
+        dn = (done != 0)
+        m0_ = m0[:, 0, :, 0, 0].float()                                          # (B,H)
+        # m_t = max(m_{t-1} + log f_t, log i_t), restarted at resets: with F the cumulative log f of the
+        # episode, m_t = F_t + max(m_0 [first episode], running max of (log i - F))
         Fc, _, _ = linear_scan(ones, log_f.contiguous(), done, torch.zeros(Bn, H, device=k.device))
-        dn = done != 0
         seg = torch.cumsum(dn.to(torch.float64), dim=1)[..., None]                # (B,T,1)
         u = (log_i - Fc).double()
         big = 2.0 * (u.max() - u.min()).detach() + 1.0
         cm = torch.cummax(u + big * seg, dim=1).values - big * seg
         cm = torch.where(seg == 0, torch.maximum(cm, m0_[:, None].double()), cm)
-        m = (Fc.double() + cm).float()                                          # (B,T,H)
-        den = torch.maximum(qn.abs(), torch.exp(-c)[:, None]) + 1e-6 * torch.exp(m - c[:, None])
+        m = (Fc.double() + cm).float()                                            # (B,T,H)
+        m_prev = torch.cat([m0_[:, None], m[:, :-1]], dim=1)
+        g = log_f + m_prev - m                                                    # <= 0
+        g = torch.where(dn[..., None], torch.zeros_like(g), g).clamp(min=self._G_FLOOR)   # a reset zeroes the state anyway
+        k_in = k.float() * torch.exp(log_i - m)[..., None]                        # weights <= 1
+        S0 = C0[:, 0].float().transpose(-1, -2).contiguous()
+        num, S_last = gated_linear_attention(q.float().contiguous(), k_in.contiguous(), v.float().contiguous(),
+                                             g.contiguous(), done, S0)
+        a = torch.exp(g)[..., None].expand(Bn, T, H, d).reshape(Bn, T, H * d).contiguous()
+        nvec, n_last, _ = linear_scan(a, k_in.reshape(Bn, T, H * d).contiguous(), done,
+                                      n0[:, 0, :, :, 0].float().reshape(Bn, H * d).contiguous())
+        qn = (q.float() * nvec.view(Bn, T, H, d)).sum(-1)                         # (B,T,H)
+        den = torch.maximum(qn.abs(), torch.exp(-m)) + 1e-6
         h_tilde = num / den[..., None]
-        # carry in the reference's (stabilised) units
-        m_T = m[:, -1]
-        back = torch.exp(torch.clamp(c - m_T, max=80.0))
         _, lf_last, _ = linear_scan(ones, log_f.contiguous(), done, lf0[:, 0, :, 0, 0].float().contiguous())
-        carry = ((S_last.transpose(-1, -2) * back[..., None, None])[:, None],
+        carry = (S_last.transpose(-1, -2)[:, None],
                  lf_last[:, None, :, None, None],
-                 (n_last.view(Bn, H, d) * back[..., None])[:, None, :, :, None],
-                 m_T[:, None, :, None, None])
+                 n_last.view(Bn, H, d)[:, None, :, :, None],
+                 m[:, -1][:, None, :, None, None])
         return h_tilde, carry
 
     def read(self, h_tilde, x, **kwargs):
@@ -674,37 +647,51 @@ class mLSTMCell(MemoroidCellBase):
                 torch.zeros(*batch, 1, H, d, 1, device=dev), torch.full((*batch, 1, H, 1, 1), -1e9, device=dev))
 
 
-class mLSTM(SequenceModel):
-    """Memoroid(mLSTMCell) with the query inside the scan (the kernel fuses q C into it)."""
+class mLSTM(Memoroid):
+    """Memoroid(mLSTMCell) under its own name."""
 
     def __init__(self, cell: mLSTMCell):
-        super().__init__()
-        self.cell = cell
-
-    def forward(self, inputs, done, initial_carry=None, **kwargs):
-        if initial_carry is None:
-            initial_carry = self.cell.initialize_carry(None, get_input_shape(inputs))
-        z = self.cell(inputs)
-        q = self.cell._project(inputs)[0]
-        h_tilde, carry = self.cell.scan(z, initial_carry, done, q=q)
-        return carry, self.cell.read(h_tilde, inputs)
-
-    def initialize_carry(self, key, input_shape):
-        return self.cell.initialize_carry(key, input_shape)
+        super().__init__(cell)
 
 
 # ----------------------------------------------------------------------------------
 # block composition used by the torso configuration (blocks/{stack,residual,normalization,ffn}.py)
 # ----------------------------------------------------------------------------------
-class PreNorm(nn.Module):
-    """normalization.py:10-35: norm, then the wrapped sequence model."""
+def LayerNorm(dim):
+    """flax.linen.LayerNorm with its defaults: mean and variance over the last axis, eps = 1e-6,
+    learned scale and bias -- the default norm of the reference's PreNorm / PostNorm."""
+    return nn.LayerNorm(dim, eps=1e-6)
 
-    def __init__(self, module, dim):
+
+RMSNorm = _RMSNorm
+
+
+class PreNorm(nn.Module):
+    """normalization.py:10-35: norm, then the wrapped sequence model.  ``norm`` is a constructor taking
+    the feature width (the reference's flax modules infer it); default LayerNorm as in the reference,
+    ``norm=RMSNorm`` for the torso configuration."""
+
+    def __init__(self, module, dim, norm=LayerNorm):
         super().__init__()
-        self.module, self.norm = module, _RMSNorm(dim)
+        self.module, self.norm = module, norm(dim)
 
     def forward(self, inputs, done=None, initial_carry=None, **kwargs):
         return self.module(self.norm(inputs), done, initial_carry, **kwargs)
+
+    def initialize_carry(self, key, input_shape):
+        return self.module.initialize_carry(key, input_shape)
+
+
+class PostNorm(nn.Module):
+    """normalization.py:38-65: the wrapped sequence model, then norm."""
+
+    def __init__(self, module, dim, norm=LayerNorm):
+        super().__init__()
+        self.module, self.norm = module, norm(dim)
+
+    def forward(self, inputs, done=None, initial_carry=None, **kwargs):
+        carry, y = self.module(inputs, done, initial_carry, **kwargs)
+        return carry, self.norm(y)
 
     def initialize_carry(self, key, input_shape):
         return self.module.initialize_carry(key, input_shape)

@@ -227,3 +227,49 @@ def gated_linear_attention_grads(q, k, v, g, done, S0, do, dS_last=None, feature
     L.backward()
     return dict(o=_np(o), S_last=_np(Sl), dq=_np(q_.grad), dk=_np(k_.grad), dv=_np(v_.grad),
                 dg=_np(g_.grad), dS0=_np(S0_.grad))
+
+
+# --------------------------------------------------------------------------
+# The torso block of configuration 5, composed from the reference's parts:
+# PreNorm (blocks/normalization.py:30-31) with RMSNorm, Residual (blocks/residual.py:23-26),
+# Stack (blocks/stack.py:40-51), a DeltaNet cell in the Memoroid idiom (memoroid.py:93-109) and a
+# MinGRU recurrence (min_gru.py:49-78) inside the gating pattern of GLU (blocks/ffn.py:82-123).
+# Dense algebra around recurrences that are pinned on their own (delta_rule_t, mingru_scan_t).
+# --------------------------------------------------------------------------
+def rms_norm_t(x, scale, eps=1e-6):
+    """flax.linen.RMSNorm defaults: x * rsqrt(mean(x^2) + eps) * scale."""
+    return x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * scale
+
+
+def gated_linear_recurrence_t(x, done, Wz, Wh, Wg, Wo, carry=None):
+    """y = Wo( mingru(Wz x, Wh x) * silu(Wg x) ); carry = (log h_T, log of the cumulative decay since
+    the last reset), both (B,1,F) as MinGRUCell.initialize_carry gives them (-inf, 0).
+    Returns ((log_state, log_decay), y)."""
+    z, ht = x @ Wz.T, x @ Wh.T
+    B, T, F = z.shape
+    if carry is None:
+        h0, ld = None, torch.zeros(B, F, dtype=x.dtype)
+    else:
+        h0, ld = torch.exp(carry[0][:, 0]), carry[1][:, 0]
+        if bool(torch.isinf(carry[0]).all()):
+            h0 = None
+    h, h_last = mingru_scan_t(z, ht, done, h0)
+    log_a = -torch.nn.functional.softplus(z)
+    for t in range(T):
+        ld = torch.where(done[:, t][:, None], log_a[:, t], ld + log_a[:, t])
+    y = (h * torch.nn.functional.silu(x @ Wg.T)) @ Wo.T
+    return (torch.log(h_last)[:, None], ld[:, None]), y
+
+
+def deltanet_cell_t(x, done, Wq, Wk, Wv, Wb, norm_scale, Wout, bout, H, S0=None):
+    """DeltaNet cell: projections, L2-normalised keys, beta = sigmoid, delta rule, RMSNorm over the
+    heads' concatenated outputs, output projection.  Returns ((S (B,1,H,d,d),), y)."""
+    B, T, _ = x.shape
+    heads = lambda t: t.reshape(B, T, H, -1)  # noqa: E731
+    q, k, v = heads(x @ Wq.T), heads(x @ Wk.T), heads(x @ Wv.T)
+    d = q.shape[-1]
+    kn = k / torch.clamp(k.norm(dim=-1, keepdim=True), min=1e-12)
+    S0 = torch.zeros(B, H, d, d, dtype=x.dtype) if S0 is None else S0[:, 0]
+    o, S = delta_rule_t(q, kn, v, torch.sigmoid(x @ Wb.T), done, S0)
+    y = rms_norm_t(o.reshape(B, T, H * d), norm_scale) @ Wout.T + bout
+    return (S[:, None],), y

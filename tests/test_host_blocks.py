@@ -68,3 +68,25 @@ def test_stack_threads_one_carry_per_block_and_none_for_stateless_blocks():
     c1, y1 = stack(x[:, :2], initial_carry=init)
     c2, y2 = stack(x[:, 2:], initial_carry=c1)
     assert torch.allclose(torch.cat((y1, y2), dim=1), y) and torch.allclose(c2[1], carries[1])
+
+
+def test_prenorm_defaults_to_layer_norm_and_takes_rms_norm():
+    """normalization.py:22 defaults to flax's LayerNorm: mean subtracted, variance normalised with
+    eps = 1e-6, learned scale and bias; the torso configuration passes RMSNorm explicitly."""
+    inner = sm.Projection(8, 8).double()
+    x = _x(seed=4) * 3 + 1.5
+    m = sm.PreNorm(inner, 8).double()
+    with torch.no_grad():
+        m.norm.weight.copy_(torch.linspace(0.5, 1.5, 8))
+        m.norm.bias.copy_(torch.linspace(-0.2, 0.2, 8))
+    mu, var = x.mean(-1, keepdim=True), x.var(-1, unbiased=False, keepdim=True)
+    xn = (x - mu) / torch.sqrt(var + 1e-6) * m.norm.weight + m.norm.bias
+    carry, y = m(x)
+    assert carry is None and torch.allclose(y, inner(xn)[1], atol=1e-12)
+    r = sm.PreNorm(inner, 8, norm=sm.RMSNorm).double()
+    xr = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-6) * r.norm.scale
+    assert torch.allclose(r(x)[1], inner(xr)[1], atol=1e-6)   # the RMS statistics are taken in fp32
+    p = sm.PostNorm(inner, 8).double()                         # normalization.py:38-65
+    yi = inner(x)[1]
+    want = (yi - yi.mean(-1, keepdim=True)) / torch.sqrt(yi.var(-1, unbiased=False, keepdim=True) + 1e-6)
+    assert torch.allclose(p(x)[1], want * p.norm.weight + p.norm.bias, atol=1e-12)

@@ -237,3 +237,47 @@ def test_gated_linear_attention_grads_finite_differences_and_rowdot_identity():
         ref[:, t] = np.where(done[:, t][:, None], 0.0, acc)
         acc = np.where(done[:, t][:, None], 0.0, acc)
     np.testing.assert_allclose(r["dg"], ref, rtol=1e-9, atol=1e-9)
+
+
+def test_torso_parts_of_the_gradient_oracle():
+    """rms_norm_t against the closed form; gated_linear_recurrence_t: values against the NumPy
+    log-space MinGRU (oracle.memoroid.mingru_scan) composed with the gating by hand, carry against
+    the cumulative product of decays since the last reset, and split invariance through the carry;
+    deltanet_cell_t against the NumPy composition."""
+    import torch
+    from oracle import grad as G
+    from oracle import memoroid as M
+    rng = np.random.default_rng(77)
+    B, T, Fe, H, d = 2, 23, 6, 2, 4
+    x = rng.standard_normal((B, T, Fe))
+    done = rng.random((B, T)) < 0.15
+    done[0, 0] = False
+    scale = rng.uniform(0.5, 1.5, Fe)
+    xn = x / np.sqrt((x ** 2).mean(-1, keepdims=True) + 1e-6) * scale
+    assert np.allclose(G.rms_norm_t(torch.from_numpy(x), torch.from_numpy(scale)).numpy(), xn, atol=1e-13)
+    Wz, Wh, Wg, Wo = (rng.standard_normal((Fe, Fe)) * 0.7 for _ in range(4))
+    t = torch.from_numpy
+    carry, y = G.gated_linear_recurrence_t(t(x), t(done), t(Wz), t(Wh), t(Wg), t(Wo))
+    z, ht, gt = x @ Wz.T, x @ Wh.T, x @ Wg.T
+    nxt, h = M.mingru_scan(z, ht, done.astype(np.float64))
+    want = (h * (gt / (1 + np.exp(-gt)))) @ Wo.T
+    assert np.allclose(y.numpy(), want, atol=1e-12)
+    assert np.allclose(carry[0].numpy(), nxt[0], atol=1e-12) and np.allclose(carry[1].numpy(), nxt[1], atol=1e-12)
+    a = 1 / (1 + np.exp(z))   # sigma(-z); cumulative product since the last reset, by brute force
+    for b in range(B):
+        last = max([i for i in range(T) if done[b, i]] + [0])
+        assert np.allclose(np.exp(carry[1].numpy()[b, 0]), a[b, last:].prod(0), atol=1e-13)
+    for s in (1, 9, 22):
+        c1, y1 = G.gated_linear_recurrence_t(t(x[:, :s]), t(done[:, :s]), t(Wz), t(Wh), t(Wg), t(Wo))
+        c2, y2 = G.gated_linear_recurrence_t(t(x[:, s:]), t(done[:, s:]), t(Wz), t(Wh), t(Wg), t(Wo), c1)
+        assert np.allclose(np.concatenate([y1.numpy(), y2.numpy()], 1), want, atol=1e-11)
+        assert np.allclose(c2[0].numpy(), nxt[0], atol=1e-11) and np.allclose(c2[1].numpy(), nxt[1], atol=1e-11)
+    Wq, Wk, Wv = (rng.standard_normal((H * d, Fe)) for _ in range(3))
+    Wb, ns = rng.standard_normal((H, Fe)), rng.uniform(0.5, 1.5, H * d)
+    Wout, bout = rng.standard_normal((Fe, H * d)), rng.standard_normal(Fe)
+    (S,), yd = G.deltanet_cell_t(t(x), t(done), t(Wq), t(Wk), t(Wv), t(Wb), t(ns), t(Wout), t(bout), H)
+    hv = lambda w: (x @ w.T).reshape(B, T, H, d)  # noqa: E731
+    o, Sl = M.deltanet(hv(Wq), hv(Wk), hv(Wv), x @ Wb.T, done.astype(np.float64))
+    o = o.reshape(B, T, H * d)
+    o = o / np.sqrt((o ** 2).mean(-1, keepdims=True) + 1e-6) * ns
+    assert np.allclose(yd.numpy(), o @ Wout.T + bout, atol=1e-11) and np.allclose(S.numpy()[:, 0], Sl, atol=1e-12)
