@@ -38,7 +38,8 @@ typedef enum {
     MRX_OK = 0,
     MRX_ERR_INVALID_ARG = -1, /* null pointer, non-positive size, bad enum, misalignment */
     MRX_ERR_UNSUPPORTED = -2, /* valid request the kernels do not cover (e.g. head dim != 64) */
-    MRX_ERR_LAUNCH = -3       /* the HIP runtime rejected the launch */
+    MRX_ERR_LAUNCH = -3,      /* the HIP runtime rejected the launch */
+    MRX_ERR_SCRATCH = -4      /* the problem exceeds the library's static scratch buffer (mrx_delta_rule_fwd_noalloc) */
 } mrx_status;
 
 typedef enum {
@@ -67,7 +68,8 @@ typedef enum {
 const char *mrx_status_string(int status);
 
 /* Per-device set-up: raises the dynamic-LDS limit of every kernel that needs more than the
- * default and caches the device's compute-unit count.  Idempotent and thread-safe; the caller's current device
+ * default, caches the device's compute-unit count and resolves the address of the library's
+ * static scratch array on that device.  Idempotent and thread-safe; the caller's current device
  * is left as it was.  Calling it is optional -- the first launch on a device does the same --
  * but a caller that captures its first call on a device into a HIP graph must call it before
  * the capture begins (the set-up calls are not stream operations).  No counterpart in the
@@ -187,6 +189,25 @@ int mrx_delta_rule_fwd(void *stream, const void *q, const void *k,
                        const void *S0, void *o, void *S_last, void *S_chk,
                        void *Tm_chk, int64_t B, int64_t T, int64_t H, int64_t dk,
                        int64_t dv, int dtype, int done_dtype, int factor_path);
+
+/* mrx_delta_rule_fwd without residuals for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the triangular
+ * factors, which mrx_delta_rule_fwd keeps in the caller's Tm_chk buffer, go to a static device
+ * array inside the library instead (MRX_NOALLOC_SCRATCH_BYTES per device, held until the process
+ * ends), and the chunk-parallel factor kernel always runs.  No counterpart in the reference.
+ * Same results as mrx_delta_rule_fwd(..., S_chk = NULL, Tm_chk = buffer, MRX_FACTORS_PARALLEL).
+ * Limit: B * H * ceil(T / 32) * 32 * 32 * sizeof(element) <= MRX_NOALLOC_SCRATCH_BYTES, i.e. 16384
+ * chunks of bf16 or 8192 of fp32 (B=64, H=8, T=1024 in bf16 fits exactly); beyond it the call
+ * returns MRX_ERR_SCRATCH and launches nothing.  The call allocates and frees nothing.  All calls
+ * on one device share that device's array: calls that overlap in time on one device (different
+ * streams, or graphs replayed concurrently) race; calls ordered on one stream do not.  Nothing in
+ * the array needs clearing between calls: every factor a call reads, it has written itself. */
+#define MRX_NOALLOC_SCRATCH_BYTES (32u << 20)
+int mrx_delta_rule_fwd_noalloc(void *stream, const void *q, const void *k,
+                               const void *v, const void *beta, const void *done,
+                               const void *S0, void *o, void *S_last, int64_t B,
+                               int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
+                               int done_dtype);
 
 /* Gradients w.r.t. q,k,v,beta (in `dtype`) and S0 (fp32, nullable).  S_chk and
  * Tm_chk are the residuals written by mrx_delta_rule_fwd on the same inputs. */

@@ -15,6 +15,7 @@ MRX_F32, MRX_BF16, MRX_C64 = 0, 1, 2
 MRX_DONE_U8, MRX_DONE_F32 = 0, 1
 MRX_FMAP_NONE, MRX_FMAP_ELU1 = 0, 1
 MRX_FACTORS_AUTO, MRX_FACTORS_PARALLEL, MRX_FACTORS_INLINE = 0, 1, 2
+MRX_NOALLOC_SCRATCH_BYTES = 32 << 20
 
 _P = ctypes.c_void_p
 _I = ctypes.c_int
@@ -34,6 +35,7 @@ SIGNATURES = {
     "mrx_linear_attn_norm_fwd": (_I, [_P] * 13 + [_L] * 5 + [_I] * 3 + [ctypes.c_float]),
     "mrx_linear_attn_norm_bwd": (_I, [_P] * 17 + [_L] * 5 + [_I] * 3 + [ctypes.c_float]),
     "mrx_delta_rule_fwd": (_I, [_P] * 11 + [_L] * 5 + [_I] * 3),
+    "mrx_delta_rule_fwd_noalloc": (_I, [_P] * 9 + [_L] * 5 + [_I] * 2),
     "mrx_delta_rule_bwd": (_I, [_P] * 15 + [_L] * 5 + [_I] * 2),
     "mrx_deltanet_fwd": (_I, [_P] * 11 + [_L] * 5 + [_I] * 3),
     "mrx_deltanet_bwd": (_I, [_P] * 15 + [_L] * 5 + [_I] * 2),

@@ -34,6 +34,7 @@ int prepare_device(int *cus, int *dev_out)
             int n_cu = 0;
             if (hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return MRX_ERR_LAUNCH;
             g_cus[dev] = n_cu;
+            if (const int rc = resolve_scratch(dev); rc != MRX_OK) return rc;
             g_ready.fetch_or(bit, std::memory_order_release);
         }
     }
@@ -51,6 +52,7 @@ extern "C" const char *mrx_status_string(int status)
     case MRX_ERR_INVALID_ARG: return "invalid argument";
     case MRX_ERR_UNSUPPORTED: return "unsupported configuration";
     case MRX_ERR_LAUNCH: return "kernel launch failed";
+    case MRX_ERR_SCRATCH: return "problem exceeds the library's static scratch buffer";
     default: return "unknown status";
     }
 }

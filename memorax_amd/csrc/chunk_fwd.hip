@@ -591,7 +591,23 @@ int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void 
 
 bool factor_path_ok(int f) { return f == MRX_FACTORS_AUTO || f == MRX_FACTORS_PARALLEL || f == MRX_FACTORS_INLINE; }
 
+// ---- static scratch of the entry point that allocates nothing --------------------------------------
+// Room for the triangular factors of MRX_NOALLOC_SCRATCH_BYTES / (32 * 32 * sizeof(element)) chunks.
+// Every device the library runs on holds its own copy at its own address; host code only ever uses
+// the address resolve_scratch() obtained for the current device, never the array's name.
+static __device__ __align__(256) unsigned char scratch[MRX_NOALLOC_SCRATCH_BYTES];
+void *g_scratch_ptr[64] = {nullptr};
+
 }  // namespace
+
+int mrx::resolve_scratch(int dev)
+{
+    if (dev < 0 || dev >= 64) return MRX_ERR_UNSUPPORTED;
+    void *p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return MRX_ERR_LAUNCH;
+    g_scratch_ptr[dev] = p;
+    return MRX_OK;
+}
 
 extern "C" int64_t mrx_chunk_size(int dtype) { return dtype == MRX_BF16 ? LA_BF16_CHUNK : (dtype == MRX_F32 ? 32 : 0); }
 
@@ -625,6 +641,25 @@ extern "C" int mrx_delta_rule_fwd(void *stream, const void *q, const void *k, co
     hipStream_t st = (hipStream_t)stream;
     return delta_fwd_dispatch<false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H, dtype,
                                      factor_path);
+}
+
+extern "C" int mrx_delta_rule_fwd_noalloc(void *stream, const void *q, const void *k, const void *v,
+                                          const void *beta, const void *done, const void *S0, void *o,
+                                          void *S_last, int64_t B, int64_t T, int64_t H, int64_t dk,
+                                          int64_t dv, int dtype, int done_dtype)
+{
+    const int rc = check_common(q, k, v, done, o, S0, S_last, nullptr, B, T, H, dk, dv, dtype, done_dtype);
+    if (rc != MRX_OK) return rc;
+    if (!beta) return MRX_ERR_INVALID_ARG;
+    const int64_t NC = (T + 31) / 32, esize = dtype == MRX_BF16 ? 2 : 4;
+    if (T > DELTA_TM_MAX_T || B * H * NC > (int64_t)MRX_NOALLOC_SCRATCH_BYTES / (32 * 32 * esize)) return MRX_ERR_SCRATCH;
+    int dev = -1;
+    if (const int rc2 = prepare_device(nullptr, &dev); rc2 != MRX_OK) return rc2;
+    void *factors = g_scratch_ptr[dev];  // this device's copy of the array, resolved at set-up
+    if (!factors) return MRX_ERR_LAUNCH;
+    hipStream_t st = (hipStream_t)stream;
+    return delta_fwd_dispatch<false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, nullptr, factors, B, T, H, dtype,
+                                     MRX_FACTORS_PARALLEL);
 }
 
 extern "C" int mrx_gated_linear_attn_fwd(void *stream, const void *q, const void *k, const void *v,

@@ -52,7 +52,8 @@ inline int launch_kernel(void (*kern)(KArgs...), dim3 grid, dim3 block, size_t l
 
 // Per-device set-up, done once per device by mrx_init() or by the first launch on it: every kernel
 // that needs more than the default 64 KB of dynamic LDS gets its limit raised (the attribute belongs
-// to the device's copy of the kernel) and the number of compute units is cached.  Kernels enter the list through a
+// to the device's copy of the kernel), the number of compute units is cached, and the address of the
+// library's static scratch array on that device is resolved.  Kernels enter the list through a
 // KernelRegistrar with static storage, i.e. while the library is being loaded; after that the list
 // is read-only.
 struct KernelNode {
@@ -68,6 +69,8 @@ struct KernelRegistrar {
 // Makes the current device ready (see above).  Returns an MRX_* status; *cus (if given) receives the
 // device's compute-unit count, *dev its index.
 int prepare_device(int *cus = nullptr, int *dev = nullptr);
+// Defined beside the scratch array (chunk_fwd.hip): resolves its address on the current device.
+int resolve_scratch(int dev);
 
 inline bool aligned(const void *p, size_t n)
 {

@@ -277,6 +277,28 @@ def init(device=None):
     _lib.check(lib.mrx_init(dev), "mrx_init")
 
 
+def delta_rule_fwd_noalloc(q, k, v, beta, done, S0=None, out=None):
+    """mrx_delta_rule_fwd_noalloc: forward without residuals, the triangular factors in the
+    library's static scratch array (nothing is allocated by the library; this wrapper allocates
+    o and S_last unless out = (o, S_last) is given).  Returns (o, S_last)."""
+    lib = _lib.load()
+    B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
+    _chk(beta, "beta", dt, (B, T, H))
+    _chk(S0, "S0", torch.float32, (B, H, dv, dk))
+    done, dd = _done(done, B, T)
+    if out is not None:
+        o, S_last = out
+        _chk(o, "out o", dt, (B, T, H, dv))
+        _chk(S_last, "out S_last", torch.float32, (B, H, dv, dk))
+    else:
+        o = torch.empty_like(v)
+        S_last = torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
+    st = lib.mrx_delta_rule_fwd_noalloc(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done), _ptr(S0),
+                                        _ptr(o), _ptr(S_last), B, T, H, dk, dv, _DT[dt], dd)
+    _lib.check(st, "mrx_delta_rule_fwd_noalloc")
+    return o, S_last
+
+
 def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prologue=False, tm_scratch=None,
                    factor_path=None):
     """Returns (o, S_last fp32, chk) where chk = (S_chk, Tm_chk) are the residuals the
