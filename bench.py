@@ -81,6 +81,8 @@ def main() -> int:
     ap.add_argument("--all", action="store_true",
                     help="also time the whole torso with its dense layers, the single-step kernels and the RTRL scan")
     ap.add_argument("--headline-only", action="store_true", help="skip the secondary configurations")
+    ap.add_argument("--ramp-ms", type=float, default=CLOCK_RAMP_S * 1e3,
+                    help="untimed load before the warm-up steps (0 under a counter-collecting profiler)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain elementwise kernel of known size (256 MiB read, 256 MiB "
                          "written) so that a rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE run can be scaled")
@@ -139,7 +141,7 @@ def main() -> int:
     # right after an idle stretch read 0.32, 0.29, 0.28, 0.27, 0.27 ms per step): an untimed ramp of the
     # same work comes first, outside the W warm-up steps and the K timed ones.
     t_ramp = time.perf_counter()
-    while time.perf_counter() - t_ramp < CLOCK_RAMP_S:
+    while time.perf_counter() - t_ramp < args.ramp_ms * 1e-3:
         for _ in range(10):
             step()
         torch.cuda.synchronize()
@@ -187,7 +189,7 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "clock_ramp_ms": CLOCK_RAMP_S * 1e3,
+        "clock_ramp_ms": args.ramp_ms,
         "config": {"workload": "configs[3]: DeltaNet delta rule fwd+bwd, B=64 H=8 T=1024 d=64, "
                                f"bf16 in / fp32 state, chunk {C}, resets p=0.002"},
         "roofline": {

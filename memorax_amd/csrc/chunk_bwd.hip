@@ -562,7 +562,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     T *sU = at(L::oU), *sDU = at(L::oDU), *sZb = at(L::oZb);
     T *sS = at(L::oS);                                    // S[dv][dk]
     T *sDS = at(L::oDS);                                  // dS[dv][dk]
-    T *sAqk = at(L::oAqk), *sDAqk = at(L::oAqk);          // Aqk[i][j] -> dAqk[i][j]
+    T *sAqk = at(L::oAqk), *sDAqk = at(L::oAqk);          // Aqk^T[j][i] -> dAqk[i][j]
     T *sTm = at(L::oTm), *sDA = at(L::oDT);               // Tm[i][j], dA[i][j]
     float *sBeta = reinterpret_cast<float *>(smem + L::oBeta);
     float *sDb = reinterpret_cast<float *>(smem + L::oDb);  // [NSLOT][C] dbeta partials
@@ -734,12 +734,13 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             if (pre) { prefetch_part(0); prefetch_part(1); }
 
             auto tril = [](int m, int n, float x) { return m <= n ? x : 0.f; };
-            // ---- Aqk[i][j] = q_i . k_j, j <= i : D[m = j][n = i] -> sAqk[i][j] ----------------------
+            // ---- Aqk[i][j] = q_i . k_j, j <= i, stored transposed: D[m = i][n = j] -> sAqk[j][i], the
+            //      orientation its one consumer (dU') contracts over without transpose reads -------------
             {
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
-                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sK, LDD, sQ, LDD, w, lane);
-                store_acc_f<T, C, C, NW>(acc, sAqk, LDC, w, lane, tril);
+                gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sQ, LDD, sK, LDD, w, lane);
+                store_acc_f<T, C, C, NW>(acc, sAqk, LDC, w, lane, [](int m, int n, float x) { return m >= n ? x : 0.f; });
             }
             // ---- V0[c][dv] = V[c][dv] - sum_dk S[dv][dk] K[c][dk] (in place), V~ = beta_c V0 -> sVt ---
             {
@@ -774,7 +775,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             {
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
-                gemm<T, HD, C, C, KROW, KROW, NW>(acc, sDO, LDD, sAqk, LDC, w, lane);
+                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sDO, LDD, sAqk, LDC, w, lane);
                 gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc, sDS, LDD, sK, LDD, w, lane);
                 store_acc<T, HD, C, NW>(acc, sDU, LDD, w, lane);
             }
