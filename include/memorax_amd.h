@@ -183,11 +183,17 @@ int mrx_linear_attn_norm_bwd(void *stream, const void *q, const void *k,
  * factors up to rounding.  factor_path (mrx_factor_path) overrides the rule:
  * MRX_FACTORS_PARALLEL takes the chunk-parallel kernel whenever the buffer is given (on a full
  * device that is level with the default when episodes end every hundred steps or so, and slower
- * when resets are rare), MRX_FACTORS_INLINE never does. */
+ * when resets are rare), MRX_FACTORS_INLINE never does.
+ * U_chk (nullable; required with S_chk): (B,T,H,dv) in `dtype`, receives U'_t = the rows of
+ * Tm diag(beta) (V - K S^T), the chunk's increments: S_leaving = S_entering + U'^T K.  The backward
+ * call undoes that update chunk by chunk (S_c = S_{c+1} - U'_c^T K_c, in fp32), so S_chk is
+ * written SPARSELY: only the slot of the last chunk and the slots of chunks that contain a reset
+ * (whose entering state the leaving one does not determine) are touched; the other slots keep
+ * whatever the buffer held.  Per 32-step chunk that is 4 KB of residual each way instead of 8. */
 int mrx_delta_rule_fwd(void *stream, const void *q, const void *k,
                        const void *v, const void *beta, const void *done,
                        const void *S0, void *o, void *S_last, void *S_chk,
-                       void *Tm_chk, int64_t B, int64_t T, int64_t H, int64_t dk,
+                       void *Tm_chk, void *U_chk, int64_t B, int64_t T, int64_t H, int64_t dk,
                        int64_t dv, int dtype, int done_dtype, int factor_path);
 
 /* mrx_delta_rule_fwd without residuals for callers that cannot allocate device memory (code under
@@ -209,11 +215,11 @@ int mrx_delta_rule_fwd_noalloc(void *stream, const void *q, const void *k,
                                int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                                int done_dtype);
 
-/* Gradients w.r.t. q,k,v,beta (in `dtype`) and S0 (fp32, nullable).  S_chk and
- * Tm_chk are the residuals written by mrx_delta_rule_fwd on the same inputs. */
+/* Gradients w.r.t. q,k,v,beta (in `dtype`) and S0 (fp32, nullable).  S_chk, Tm_chk and
+ * U_chk are the residuals written by mrx_delta_rule_fwd on the same inputs. */
 int mrx_delta_rule_bwd(void *stream, const void *q, const void *k,
                        const void *v, const void *beta, const void *done,
-                       const void *S_chk, const void *Tm_chk, const void *dout,
+                       const void *S_chk, const void *Tm_chk, const void *U_chk, const void *dout,
                        const void *dS_last, void *dq, void *dk_out, void *dv_out,
                        void *dbeta, void *dS0, int64_t B, int64_t T, int64_t H,
                        int64_t dk, int64_t dv, int dtype, int done_dtype);
@@ -228,13 +234,13 @@ int mrx_delta_rule_bwd(void *stream, const void *q, const void *k,
  * Residuals as for mrx_delta_rule_*. */
 int mrx_deltanet_fwd(void *stream, const void *q, const void *k, const void *v,
                      const void *beta_raw, const void *done, const void *S0, void *o,
-                     void *S_last, void *S_chk, void *Tm_chk, int64_t B, int64_t T,
+                     void *S_last, void *S_chk, void *Tm_chk, void *U_chk, int64_t B, int64_t T,
                      int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype,
                      int factor_path);
 
 int mrx_deltanet_bwd(void *stream, const void *q, const void *k, const void *v,
                      const void *beta_raw, const void *done, const void *S_chk,
-                     const void *Tm_chk, const void *dout, const void *dS_last, void *dq,
+                     const void *Tm_chk, const void *U_chk, const void *dout, const void *dS_last, void *dq,
                      void *dk_out, void *dv_out, void *dbeta_raw, void *dS0, int64_t B,
                      int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                      int done_dtype);

@@ -132,7 +132,9 @@ def test_delta_rule_factor_paths_agree(dtype, prologue):
         assert torch.equal(o3, o4) and torch.equal(Sl3, Sl4)
         assert relerr(o3, o[sl].float().cpu().numpy()) <= tol and relerr(Sl3, Sl[sl].cpu().numpy()) <= tol
         assert relerr(chk3[1], chk[1][sl].float().cpu().numpy()) <= tol
-        assert relerr(chk3[0], chk[0][sl].float().cpu().numpy()) <= tol
+        assert relerr(chk3[2], chk[2][sl].float().cpu().numpy()) <= tol  # U'
+        # the state checkpoints are sparse; the one of the last chunk is always written
+        assert relerr(chk3[0][:, :, -1], chk[0][sl][:, :, -1].float().cpu().numpy()) <= tol
         g3 = K.delta_rule_bwd(*args, chk3, do[sl].contiguous(), prologue=prologue)
         for a, b_ in zip(g3, grads):
             assert relerr(a, b_[sl].float().cpu().numpy()) <= tol
