@@ -80,7 +80,15 @@ int mrx_init(int device);
 int mrx_version(void);
 
 /* Time-chunk length the (gated) linear-attention kernels use for `dtype`; fixes the layout
- * of the per-chunk state checkpoints S_chk: (B, H, ceil(T/chunk), dv, dk). */
+ * of the per-chunk state checkpoints S_chk: (B, H, ceil(T/chunk), dv, dk).
+ *
+ * State checkpoints.  The backward calls need the state entering every chunk.  Where the chunk's
+ * update can be undone (plain and normalised linear attention: S_c = S_{c+1} - V_c^T K_c; delta rule:
+ * S_c = S_{c+1} - U'_c^T K_c) they walk it back in fp32 from the forward call's S_last, which is
+ * then an INPUT of the backward call, and S_chk is a float32 buffer that the forward call writes
+ * SPARSELY: only the slots of chunks that contain a reset -- whose entering state the leaving one does
+ * not determine -- are written and read; the other slots keep whatever the buffer held.  The gated
+ * kernels (whose decayed update is not undone) keep one checkpoint per chunk in `dtype`. */
 int64_t mrx_chunk_size(int dtype);
 
 /* The same for the delta-rule kernels (S_chk and Tm_chk of mrx_delta_rule_fwd/_bwd). */
@@ -120,8 +128,9 @@ int mrx_linear_scan_bwd(void *stream, const void *a, const void *h,
  *     S_t = (done_t ? 0 : S_{t-1}) + v_t phi(k_t)^T ;   o_t = S_t phi(q_t)
  * q,k: (B,T,H,dk); v,o: (B,T,H,dv) in `dtype` (MRX_F32 or MRX_BF16).
  * S0 (nullable = 0), S_last (nullable): (B,H,dv,dk) fp32.
- * S_chk (nullable): (B,H,ceil(T/chunk),dv,dk) in `dtype`, receives the state
- * entering each chunk; required by the backward call.  dk = dv = 64. */
+ * S_chk (nullable): (B,H,ceil(T/chunk),dv,dk) float32, sparse (see mrx_chunk_size): receives the
+ * state entering each chunk that contains a reset; required by the backward call together with
+ * S_last.  dk = dv = 64. */
 int mrx_linear_attn_fwd(void *stream, const void *q, const void *k,
                         const void *v, const void *done, const void *S0,
                         void *o, void *S_last, void *S_chk, int64_t B,
@@ -130,10 +139,11 @@ int mrx_linear_attn_fwd(void *stream, const void *q, const void *k,
 
 /* Gradients of the above w.r.t. q,k,v (pre-feature-map) and S0, given
  * dout = dL/do (B,T,H,dv) and dS_last = dL/dS_last (nullable).
+ * S_chk, S_last: as the forward call on the same inputs left them.
  * dq,dk,dv in `dtype`; dS0 (nullable) fp32. */
 int mrx_linear_attn_bwd(void *stream, const void *q, const void *k,
                         const void *v, const void *done, const void *S_chk,
-                        const void *dout, const void *dS_last, void *dq,
+                        const float *S_last, const void *dout, const void *dS_last, void *dq,
                         void *dk_out, void *dv_out, void *dS0, int64_t B,
                         int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                         int done_dtype, int feature_map);
@@ -159,7 +169,7 @@ int mrx_linear_attn_norm_fwd(void *stream, const void *q, const void *k,
  * Where the clamp is active (den == eps) the denominator passes no gradient. */
 int mrx_linear_attn_norm_bwd(void *stream, const void *q, const void *k,
                              const void *v, const void *done, const void *S_chk,
-                             const float *z_chk, const void *o, const float *den,
+                             const float *S_last, const float *z_chk, const void *o, const float *den,
                              const void *dout, const void *dS_last,
                              const float *dz_last, void *dq, void *dk_out,
                              void *dv_out, void *dS0, float *dz0, int64_t B,
@@ -186,10 +196,9 @@ int mrx_linear_attn_norm_bwd(void *stream, const void *q, const void *k,
  * when resets are rare), MRX_FACTORS_INLINE never does.
  * U_chk (nullable; required with S_chk): (B,T,H,dv) in `dtype`, receives U'_t = the rows of
  * Tm diag(beta) (V - K S^T), the chunk's increments: S_leaving = S_entering + U'^T K.  The backward
- * call undoes that update chunk by chunk (S_c = S_{c+1} - U'_c^T K_c, in fp32), so S_chk is
- * written SPARSELY: only the slot of the last chunk and the slots of chunks that contain a reset
- * (whose entering state the leaving one does not determine) are touched; the other slots keep
- * whatever the buffer held.  Per 32-step chunk that is 4 KB of residual each way instead of 8. */
+ * call undoes that update chunk by chunk (S_c = S_{c+1} - U'_c^T K_c, in fp32, from S_last), so
+ * S_chk (float32) is written sparsely, as for linear attention (see mrx_chunk_size).  Per 32-step
+ * chunk that is 4 KB of residual each way instead of the 8 KB of a state checkpoint. */
 int mrx_delta_rule_fwd(void *stream, const void *q, const void *k,
                        const void *v, const void *beta, const void *done,
                        const void *S0, void *o, void *S_last, void *S_chk,
@@ -215,11 +224,12 @@ int mrx_delta_rule_fwd_noalloc(void *stream, const void *q, const void *k,
                                int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                                int done_dtype);
 
-/* Gradients w.r.t. q,k,v,beta (in `dtype`) and S0 (fp32, nullable).  S_chk, Tm_chk and
- * U_chk are the residuals written by mrx_delta_rule_fwd on the same inputs. */
+/* Gradients w.r.t. q,k,v,beta (in `dtype`) and S0 (fp32, nullable).  S_chk, Tm_chk,
+ * U_chk and S_last are what mrx_delta_rule_fwd wrote on the same inputs. */
 int mrx_delta_rule_bwd(void *stream, const void *q, const void *k,
                        const void *v, const void *beta, const void *done,
-                       const void *S_chk, const void *Tm_chk, const void *U_chk, const void *dout,
+                       const void *S_chk, const void *Tm_chk, const void *U_chk,
+                       const float *S_last, const void *dout,
                        const void *dS_last, void *dq, void *dk_out, void *dv_out,
                        void *dbeta, void *dS0, int64_t B, int64_t T, int64_t H,
                        int64_t dk, int64_t dv, int dtype, int done_dtype);
@@ -240,7 +250,8 @@ int mrx_deltanet_fwd(void *stream, const void *q, const void *k, const void *v,
 
 int mrx_deltanet_bwd(void *stream, const void *q, const void *k, const void *v,
                      const void *beta_raw, const void *done, const void *S_chk,
-                     const void *Tm_chk, const void *U_chk, const void *dout, const void *dS_last, void *dq,
+                     const void *Tm_chk, const void *U_chk, const float *S_last, const void *dout,
+                     const void *dS_last, void *dq,
                      void *dk_out, void *dv_out, void *dbeta_raw, void *dS0, int64_t B,
                      int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                      int done_dtype);

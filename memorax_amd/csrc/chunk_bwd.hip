@@ -76,8 +76,8 @@ template <typename T, int C, bool FMAP, bool GATED, bool NORM>
 __global__ void __launch_bounds__(256, 2)
 la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
               const float *__restrict__ glog, const void *__restrict__ done, int done_f32,
-              const T *__restrict__ S_chk, const T *__restrict__ dout, const float *__restrict__ dS_last,
-              T *__restrict__ dq, T *__restrict__ dk, T *__restrict__ dv, float *__restrict__ edot,
+              const void *__restrict__ S_chk, const float *__restrict__ S_last, const T *__restrict__ dout,
+              const float *__restrict__ dS_last, T *__restrict__ dq, T *__restrict__ dk, T *__restrict__ dv, float *__restrict__ edot,
               float *__restrict__ dS0, int Tlen, int H, NormBwdArgs na)
 {
     static_assert(!(GATED && NORM), "the normalised read-out belongs to plain linear attention");
@@ -138,11 +138,34 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
         }
     }
 
+    // The state leaving, then entering, the chunk at hand (S^T, in the layout of dS^T).  Without a decay
+    // the update of a chunk can be undone, S_c = S_{c+1} - V_c^T K_c, so the state is walked back in
+    // fp32 registers from the forward call's S_last and read from the forward call's (fp32) checkpoints
+    // only where the walk cannot pass: chunks with resets, the only ones the forward call writes then.
+    // Gated: every chunk has a checkpoint in the I/O type, staged row-wise.
+    constexpr bool WALK = !GATED;
+    constexpr int NSA = WALK ? TMS::TPW : 1;
+    f32x4 Sacc[NSA], rS32[NSA];
+    zero_acc<NSA>(Sacc);
+    zero_acc<NSA>(rS32);
+    if (WALK) {
+#pragma unroll
+        for (int j = 0; j < NSA; ++j) {
+            const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
+            Sacc[j] = *reinterpret_cast<const f32x4 *>(S_last + ((int64_t)bh * HD + dvv) * HD + dk0);
+        }
+    }
+
     typename IO::Regs rq, rk, rv, rdo, ro;
     float rden[IO::PASSES];
     f32x4 rz = {0.f, 0.f, 0.f, 0.f};
     typename IOS::Regs rS;
-    uint32_t rdone = 0u;  // raw bits, tested when the chunk is staged
+    // raw bits, tested when the chunk is staged; the reset flags of the chunk after the next one too:
+    // whether its checkpoint must be fetched is known when the next prefetch starts
+    uint32_t rdone = 0u, rdone2 = 0u;
+    // Does the chunk about to be prefetched take its entering state from S_chk?  Not known for the
+    // first one (its reset flags are part of the same prefetch): read then, used only if it applies.
+    bool need_S = true;
     float rg = 0.f;       // log-decay of chunk row `lane` (gated)
     // Running element offsets of this thread's loads, stepped back by one chunk per prefetch
     // (64-bit adds instead of per-chunk index multiplications).  The prefetch is issued in parts
@@ -153,7 +176,8 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 #pragma unroll
     for (int p = 0; p < IO::PASSES; ++p)
         roff[p] = base + (int64_t)(tlast + IO::row_of(tid, p)) * rs + (tid % IO::SEGS) * IO::KP;
-    int64_t soff = ((int64_t)bh * NC + NC - 1) * HD * HD + (tid / IOS::SEGS) * HD + (tid % IOS::SEGS) * IOS::KP;
+    int64_t soff = ((int64_t)bh * NC + NC - 1) * HD * HD +
+                   (WALK ? li * HD + 4 * lg : (tid / IOS::SEGS) * HD + (tid % IOS::SEGS) * IOS::KP);
     int64_t doff = (int64_t)b * Tlen + tlast + lane;
     int64_t noff[IO::PASSES];  // den of the rows this thread stages
 #pragma unroll
@@ -178,15 +202,24 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 }
             }
         } else {
+            if (!WALK) {
 #pragma unroll
-            for (int p = 0; p < IOS::PASSES; ++p)
-                rS.v[p] = *reinterpret_cast<const typename IOS::F *>(S_chk + soff + p * IOS::RPP * HD);
+                for (int p = 0; p < IOS::PASSES; ++p)
+                    rS.v[p] = *reinterpret_cast<const typename IOS::F *>(reinterpret_cast<const T *>(S_chk) + soff + p * IOS::RPP * HD);
+            } else if (need_S) {
+#pragma unroll
+                for (int j = 0; j < NSA; ++j)
+                    rS32[j] = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(S_chk) + soff +
+                                                               TMS::nt(w, j) * 16 * HD + TMS::mt(w, j) * 16);
+            }
             rdone = 0u;
+            rdone2 = 0u;
             rg = 0.f;
             if (lane < C && tpre + lane < Tlen) {
                 rdone = done_raw(done, done_f32, doff);
                 if (GATED) rg = glog[doff * H + h];
             }
+            if (WALK && lane < C && tpre >= C) rdone2 = done_raw(done, done_f32, doff - C);
             if (NORM) {
 #pragma unroll
                 for (int p = 0; p < IO::PASSES; ++p) {
@@ -241,6 +274,8 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
         const int t0 = c * C;
         const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
+        const bool ckpt = !WALK || nres != 0;  // the entering state comes from S_chk
+        if (WALK) need_S = __ballot(done_test(rdone2, done_f32) && lane < C) != 0ull;  // for the chunk prefetched during this one
         for (int pass = nres; pass >= 0; --pass) {
             auto live = [&](int r) { return nres == 0 || episode_of(dmask, r) == pass; };
             // gated: cumulative log-decay of this pass's episode (as in the forward kernel)
@@ -295,9 +330,11 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 IO::to_lds(fk, sK, LDD, tid);
                 IO::to_lds(fv, sV, LDD, tid);
                 IO::to_lds(fdo, sDO, LDD, tid);
-                typename IOS::Regs fS = rS;
-                if (pass != 0) IOS::zero(fS);
-                IOS::to_lds(fS, sS, LDD, tid);  // S[dv][dk]
+                if (!WALK) {
+                    typename IOS::Regs fS = rS;
+                    if (pass != 0) IOS::zero(fS);
+                    IOS::to_lds(fS, sS, LDD, tid);  // S[dv][dk]
+                }
             }
             if (pass != nres) zero_acc<TMS::TPW>(dSacc);  // an episode that ends inside the chunk
             store_acc<T, HD, HD, NW>(dSacc, sDS, LDD, w, lane);  // dS[dv][dk]
@@ -344,6 +381,27 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 zero_acc<TMA::TPW>(acc);
                 gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sV, LDD, sDO, LDD, w, lane);  // D[m = j][n = i]
                 store_tril(acc, sDAqk, true);
+            }
+            // ---- the state entering the chunk, S^T[dk][dv] = S_leaving^T - sum_c K[c][dk] V[c][dv], or the
+            //      forward call's checkpoint (first episode of a chunk with resets; the later ones start
+            //      from zero); rounded into sS[dv][dk] -----------------------------------------------------
+            if (WALK) {
+                if (!ckpt) {
+                    f32x4 acc[TMS::TPW];
+                    zero_acc<TMS::TPW>(acc);
+                    gemm<T, HD, HD, C, KROW, KROW, NW>(acc, sK, LDD, sV, LDD, w, lane);
+#pragma unroll
+                    for (int j = 0; j < NSA; ++j) Sacc[j] -= acc[j];
+                    store_acc<T, HD, HD, NW>(Sacc, sS, LDD, w, lane);
+                } else if (pass == 0) {
+#pragma unroll
+                    for (int j = 0; j < NSA; ++j) Sacc[j] = rS32[j];
+                    store_acc<T, HD, HD, NW>(Sacc, sS, LDD, w, lane);
+                } else {
+                    f32x4 zero[TMS::TPW];
+                    zero_acc<TMS::TPW>(zero);
+                    store_acc<T, HD, HD, NW>(zero, sS, LDD, w, lane);
+                }
             }
             sync_lds();
             if (pre) prefetch_part(1);
@@ -509,9 +567,10 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 // once their first tenant is dead.  bf16: two workgroups per CU.
 //
 // Per pass, with Tm = (I + A)^-1 and U' (= Tm diag(beta) (V - K S^T)) from the forward call and S the
-// state entering the chunk -- walked back from the state entering the next chunk,
-// S_c = S_{c+1} - U'_c^T K_c, in fp32 registers; read from the forward call's checkpoint where the walk
-// cannot pass (the last chunk; a chunk with resets, whose entering state the leaving one does not fix):
+// state entering the chunk -- walked back from the state leaving it, S_c = S_{c+1} - U'_c^T K_c, in
+// fp32 registers that start from the forward call's S_last; read from the forward call's (fp32)
+// checkpoint where the walk cannot pass (a chunk with resets, whose entering state the leaving one
+// does not determine):
 //   V0 = V - K S^T                                                 (for dbeta only)
 //   Aqk = tril(Q K^T),  dU' = Aqk^T dO + K dS^T,  dAqk = tril(dO U'^T)
 //   Z = Tm^T dU',  dV = diag(beta) Z,  dbeta = rowdot(Z, V0) + rowdot(K, R)
@@ -545,15 +604,14 @@ template <typename T, int C, int NW, bool PRO>
 __global__ void __launch_bounds__(64 * NW, sizeof(T) == 2 ? 2 : 1)
 delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
-                 const T *__restrict__ S_chk, const T *__restrict__ Tm_chk, const T *__restrict__ U_chk,
-                 const T *__restrict__ dout, const float *__restrict__ dS_last, T *__restrict__ dq,
+                 const float *__restrict__ S_chk, const T *__restrict__ Tm_chk, const T *__restrict__ U_chk,
+                 const float *__restrict__ S_last, const T *__restrict__ dout, const float *__restrict__ dS_last, T *__restrict__ dq,
                  T *__restrict__ dk, T *__restrict__ dv, T *__restrict__ dbeta,
                  float *__restrict__ dS0, int Tlen, int H)
 {
     constexpr int NTHR = 64 * NW;
     using L = DeltaBwdSmem<T, C, NW>;
     using IO = TileIO<T, C, NTHR>;
-    using IOS = TileIO<T, HD, NTHR>;
     using IOT = TileIO<T, C, NTHR, C>;  // the [C][C] triangular factor
     using P4 = typename TT<T>::pack4;
     constexpr int LDD = L::LDD, LDC = L::LDC;
@@ -593,16 +651,22 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                            : f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    f32x4 Sacc[TMS::TPW];  // S^T entering the chunk at hand, in the layout of dS^T
-    zero_acc<TMS::TPW>(Sacc);
+    f32x4 Sacc[TMS::TPW];  // S^T leaving, then entering, the chunk at hand; in the layout of dS^T
+#pragma unroll
+    for (int j = 0; j < TMS::TPW; ++j) {
+        const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
+        Sacc[j] = *reinterpret_cast<const f32x4 *>(S_last + ((int64_t)bh * HD + dvv) * HD + dk0);
+    }
 
     typename IO::Regs rq, rk, rv, rdo, ru;
-    typename IOS::Regs rS;
+    f32x4 rS[TMS::TPW];  // a checkpoint, in the layout of Sacc
     typename IOT::Regs rTm;
     // raw bits, converted when the chunk is staged; the reset flags of the chunk after the next one as
     // well: whether its checkpoint must be fetched is known when the next prefetch starts
     uint32_t rdone = 0u, rdone2 = 0u, rbeta = 0u;
-    bool need_S = true;  // the chunk about to be prefetched takes its entering state from S_chk
+    // Does the chunk about to be prefetched take its entering state from S_chk?  Not known for the
+    // first one (its reset flags are part of the same prefetch): read then, used only if it applies.
+    bool need_S = true;
     uint32_t rbrow[IO::PASSES];       // beta of the rows this thread stages
     // Running element offsets of this thread's loads and stores, stepped back by one chunk per
     // iteration (64-bit adds instead of per-chunk index multiplications).
@@ -614,7 +678,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         roff[p] = base + (int64_t)r * rs + (tid % IO::SEGS) * IO::KP;  // q/k/v/dout: row r, this thread's segment
         boff[p] = ((int64_t)b * Tlen + r) * H + h;                     // beta of row r
     }
-    int64_t soff = ((int64_t)bh * NC + NC - 1) * HD * HD + (tid / IOS::SEGS) * HD + (tid % IOS::SEGS) * IOS::KP;
+    int64_t soff = ((int64_t)bh * NC + NC - 1) * HD * HD + li * HD + 4 * lg;
     int64_t tmoff = ((int64_t)bh * NC + NC - 1) * C * C + (tid / IOT::SEGS) * C + (tid % IOT::SEGS) * IOT::KP;
     int64_t doff = (int64_t)b * Tlen + tlast + lane;  // done/beta of chunk row `lane`
     int tpre = tlast;                                 // first time step of the chunk about to be prefetched
@@ -638,8 +702,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 ru.v[p] = tpre + IO::row_of(tid, p) < Tlen ? *reinterpret_cast<const typename IO::F *>(U_chk + roff[p]) : z;
             if (need_S) {
 #pragma unroll
-                for (int p = 0; p < IOS::PASSES; ++p)
-                    rS.v[p] = *reinterpret_cast<const typename IOS::F *>(S_chk + soff + p * IOS::RPP * HD);
+                for (int j = 0; j < TMS::TPW; ++j)
+                    rS[j] = *reinterpret_cast<const f32x4 *>(S_chk + soff + TMS::nt(w, j) * 16 * HD + TMS::mt(w, j) * 16);
             }
         } else {
 #pragma unroll
@@ -697,7 +761,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
         // where the state entering this chunk comes from: the forward call's checkpoint, or the walk
-        const bool ckpt = nres != 0 || c == NC - 1;
+        const bool ckpt = nres != 0;
         need_S = __ballot(done_test(rdone2, done_f32) && lane < C) != 0ull;  // for the chunk prefetched during this one
         for (int pass = nres; pass >= 0; --pass) {
             auto live = [&](int r) { return nres == 0 || episode_of(dmask, r) == pass; };
@@ -736,11 +800,6 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                             : PRO ? sigmoidf(raw_to_float<T>(rbrow[p])) : raw_to_float<T>(rbrow[p]);
                 IO::scale_rows(fk, bf);
                 IO::to_lds(fk, sBK, LDD, tid);
-                if (ckpt) {
-                    typename IOS::Regs fS = rS;
-                    if (pass != 0) IOS::zero(fS);
-                    IOS::to_lds(fS, sS, LDD, tid);
-                }
                 // Tm[i][j] from the forward call (block diagonal by episode).  Rows of other episodes
                 // are cleared by select: they only ever meet zeros, but a NaN key or gate of another
                 // episode sits in them and must not meet those zeros.
@@ -765,8 +824,9 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sQ, LDD, sK, LDD, w, lane);
                 store_acc_f<T, C, C, NW>(acc, sAqk, LDC, w, lane, [](int m, int n, float x) { return m >= n ? x : 0.f; });
             }
-            // ---- the state entering the chunk: S^T[dk][dv] = S_next^T - sum_c K[c][dk] U'[c][dv], rounded
-            //      into sS[dv][dk]; or, where the forward call left a checkpoint, that (staged above) -------
+            // ---- the state entering the chunk, S^T[dk][dv] = S_leaving^T - sum_c K[c][dk] U'[c][dv], or the
+            //      forward call's checkpoint (first episode of a chunk with resets; the later ones start
+            //      from zero); rounded into sS[dv][dk] -----------------------------------------------------
             if (!ckpt) {
                 f32x4 acc[TMS::TPW];
                 zero_acc<TMS::TPW>(acc);
@@ -776,11 +836,12 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 store_acc<T, HD, HD, NW>(Sacc, sS, LDD, w, lane);
             } else if (pass == 0) {
 #pragma unroll
-                for (int j = 0; j < TMS::TPW; ++j) {
-                    const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
-                    const P4 x = *reinterpret_cast<const P4 *>(sS + dvv * LDD + dk0);
-                    Sacc[j] = f32x4{(float)x[0], (float)x[1], (float)x[2], (float)x[3]};
-                }
+                for (int j = 0; j < TMS::TPW; ++j) Sacc[j] = rS[j];
+                store_acc<T, HD, HD, NW>(Sacc, sS, LDD, w, lane);
+            } else {
+                f32x4 zero[TMS::TPW];
+                zero_acc<TMS::TPW>(zero);
+                store_acc<T, HD, HD, NW>(zero, sS, LDD, w, lane);
             }
             sync_lds();
             if (pre) { prefetch_part(2); prefetch_part(3); }
@@ -970,7 +1031,7 @@ template <typename T, int C, bool FMAP, bool GATED, bool NORM> struct LaBwdReg {
 
 template <typename T, int C, bool FMAP, bool GATED = false, bool NORM = false>
 int launch_la(hipStream_t st, const void *q, const void *k, const void *v, const void *done,
-              int done_f32, const void *S_chk, const void *dout, const void *dS_last, void *dq,
+              int done_f32, const void *S_chk, const void *S_last, const void *dout, const void *dS_last, void *dq,
               void *dk, void *dv, void *dS0, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr,
               void *edot = nullptr, NormBwdArgs na = NormBwdArgs{})
 {
@@ -979,7 +1040,7 @@ int launch_la(hipStream_t st, const void *q, const void *k, const void *v, const
     if (const int rc = prepare_device(); rc != MRX_OK) return rc;
     return launch_kernel(la_bwd_kernel<T, C, FMAP, GATED, NORM>, dim3((unsigned)(B * H)), dim3(256), Reg::smem, st,
                          (const T *)q, (const T *)k, (const T *)v, (const float *)glog, done, done_f32,
-                         (const T *)S_chk, (const T *)dout, (const float *)dS_last, (T *)dq, (T *)dk, (T *)dv,
+                         S_chk, (const float *)S_last, (const T *)dout, (const float *)dS_last, (T *)dq, (T *)dk, (T *)dv,
                          (float *)edot, (float *)dS0, (int)Tlen, (int)H, na);
 }
 
@@ -1004,7 +1065,7 @@ int check_bwd(const void *q, const void *k, const void *v, const void *done, con
 }  // namespace
 
 extern "C" int mrx_linear_attn_bwd(void *stream, const void *q, const void *k, const void *v,
-                                   const void *done, const void *S_chk, const void *dout,
+                                   const void *done, const void *S_chk, const float *S_last, const void *dout,
                                    const void *dS_last, void *dq, void *dk_out, void *dv_out,
                                    void *dS0, int64_t B, int64_t T, int64_t H, int64_t dk, int64_t dv,
                                    int dtype, int done_dtype, int feature_map)
@@ -1012,17 +1073,18 @@ extern "C" int mrx_linear_attn_bwd(void *stream, const void *q, const void *k, c
     const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
                              dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
+    if (!S_last || !aligned(S_last, 16)) return MRX_ERR_INVALID_ARG;
     if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     const bool fm = feature_map == MRX_FMAP_ELU1;
-#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H
+#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, S_last, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H
     if (dtype == MRX_BF16) return fm ? launch_la<__bf16, LA_BF16_CHUNK, true>(MRX_ARGS) : launch_la<__bf16, LA_BF16_CHUNK, false>(MRX_ARGS);
     return fm ? launch_la<float, 32, true>(MRX_ARGS) : launch_la<float, 32, false>(MRX_ARGS);
 #undef MRX_ARGS
 }
 
 extern "C" int mrx_linear_attn_norm_bwd(void *stream, const void *q, const void *k, const void *v,
-                                        const void *done, const void *S_chk, const float *z_chk,
+                                        const void *done, const void *S_chk, const float *S_last, const float *z_chk,
                                         const void *o, const float *den, const void *dout,
                                         const void *dS_last, const float *dz_last, void *dq, void *dk_out,
                                         void *dv_out, void *dS0, float *dz0, int64_t B, int64_t T, int64_t H,
@@ -1032,14 +1094,14 @@ extern "C" int mrx_linear_attn_norm_bwd(void *stream, const void *q, const void 
     const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
                              dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
-    if (!z_chk || !o || !den) return MRX_ERR_INVALID_ARG;
+    if (!z_chk || !o || !den || !S_last || !aligned(S_last, 16)) return MRX_ERR_INVALID_ARG;
     if (!aligned(z_chk, 16) || !aligned(o, 16) || !aligned(den, 4) || !aligned(dz_last, 16) || !aligned(dz0, 16))
         return MRX_ERR_INVALID_ARG;
     if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     const bool fm = feature_map == MRX_FMAP_ELU1;
     const NormBwdArgs na{o, den, z_chk, dz_last, dz0, eps};
-#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, nullptr, nullptr, na
+#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, S_last, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, nullptr, nullptr, na
     if (dtype == MRX_BF16)
         return fm ? launch_la<__bf16, LA_BF16_CHUNK, true, false, true>(MRX_ARGS)
                   : launch_la<__bf16, LA_BF16_CHUNK, false, false, true>(MRX_ARGS);
@@ -1060,7 +1122,7 @@ extern "C" int mrx_gated_linear_attn_bwd(void *stream, const void *q, const void
     if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     const bool fm = feature_map == MRX_FMAP_ELU1;
-#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, g, edot
+#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, nullptr, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, g, edot
     if (dtype == MRX_BF16)
         return fm ? launch_la<__bf16, LA_BF16_CHUNK, true, true>(MRX_ARGS) : launch_la<__bf16, LA_BF16_CHUNK, false, true>(MRX_ARGS);
     return fm ? launch_la<float, 32, true, true>(MRX_ARGS) : launch_la<float, 32, false, true>(MRX_ARGS);
@@ -1078,7 +1140,7 @@ template <typename T, int C, bool PRO> struct DeltaBwdReg {
 template <typename T, int C, bool PRO>
 int launch_delta_bwd(hipStream_t st, const void *q, const void *k, const void *v, const void *beta,
                      const void *done, int done_dtype, const void *S_chk, const void *Tm_chk, const void *U_chk,
-                     const void *dout, const void *dS_last, void *dq, void *dk_out, void *dv_out, void *dbeta, void *dS0,
+                     const void *S_last, const void *dout, const void *dS_last, void *dq, void *dk_out, void *dv_out, void *dbeta, void *dS0,
                      int64_t B, int64_t T_, int64_t H)
 {
     using Reg = DeltaBwdReg<T, C, PRO>;
@@ -1086,25 +1148,27 @@ int launch_delta_bwd(hipStream_t st, const void *q, const void *k, const void *v
     if (const int rc = prepare_device(); rc != MRX_OK) return rc;
     return launch_kernel(delta_bwd_kernel<T, C, Reg::NW, PRO>, dim3((unsigned)(B * H)), dim3(64 * Reg::NW), Reg::smem, st,
                          (const T *)q, (const T *)k, (const T *)v, (const T *)beta, done, done_dtype,
-                         (const T *)S_chk, (const T *)Tm_chk, (const T *)U_chk, (const T *)dout, (const float *)dS_last, (T *)dq,
+                         (const float *)S_chk, (const T *)Tm_chk, (const T *)U_chk, (const float *)S_last, (const T *)dout,
+                         (const float *)dS_last, (T *)dq,
                          (T *)dk_out, (T *)dv_out, (T *)dbeta, (float *)dS0, (int)T_, (int)H);
 }
 
 template <bool PRO>
 int delta_bwd_entry(void *stream, const void *q, const void *k, const void *v, const void *beta, const void *done,
-                    const void *S_chk, const void *Tm_chk, const void *U_chk, const void *dout, const void *dS_last,
-                    void *dq, void *dk_out, void *dv_out, void *dbeta, void *dS0, int64_t B, int64_t T, int64_t H,
+                    const void *S_chk, const void *Tm_chk, const void *U_chk, const void *S_last, const void *dout,
+                    const void *dS_last, void *dq, void *dk_out, void *dv_out, void *dbeta, void *dS0, int64_t B, int64_t T, int64_t H,
                     int64_t dk, int64_t dv, int dtype, int done_dtype)
 {
     const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
                              dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
-    if (!beta || !dbeta || !Tm_chk || !aligned(Tm_chk, 16) || !U_chk || !aligned(U_chk, 16)) return MRX_ERR_INVALID_ARG;
+    if (!beta || !dbeta || !Tm_chk || !aligned(Tm_chk, 16) || !U_chk || !aligned(U_chk, 16) || !S_last || !aligned(S_last, 16))
+        return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == MRX_BF16)
         return launch_delta_bwd<__bf16, DELTA_BF16_CHUNK, PRO>(st, q, k, v, beta, done, done_dtype, S_chk, Tm_chk, U_chk,
-                                                               dout, dS_last, dq, dk_out, dv_out, dbeta, dS0, B, T, H);
-    return launch_delta_bwd<float, 32, PRO>(st, q, k, v, beta, done, done_dtype, S_chk, Tm_chk, U_chk, dout, dS_last, dq,
+                                                               S_last, dout, dS_last, dq, dk_out, dv_out, dbeta, dS0, B, T, H);
+    return launch_delta_bwd<float, 32, PRO>(st, q, k, v, beta, done, done_dtype, S_chk, Tm_chk, U_chk, S_last, dout, dS_last, dq,
                                             dk_out, dv_out, dbeta, dS0, B, T, H);
 }
 
@@ -1112,22 +1176,22 @@ int delta_bwd_entry(void *stream, const void *q, const void *k, const void *v, c
 
 extern "C" int mrx_delta_rule_bwd(void *stream, const void *q, const void *k, const void *v,
                                   const void *beta, const void *done, const void *S_chk,
-                                  const void *Tm_chk, const void *U_chk, const void *dout, const void *dS_last,
-                                  void *dq, void *dk_out, void *dv_out, void *dbeta, void *dS0, int64_t B,
-                                  int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
+                                  const void *Tm_chk, const void *U_chk, const float *S_last, const void *dout,
+                                  const void *dS_last, void *dq, void *dk_out, void *dv_out, void *dbeta, void *dS0,
+                                  int64_t B, int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                                   int done_dtype)
 {
-    return delta_bwd_entry<false>(stream, q, k, v, beta, done, S_chk, Tm_chk, U_chk, dout, dS_last, dq, dk_out, dv_out,
+    return delta_bwd_entry<false>(stream, q, k, v, beta, done, S_chk, Tm_chk, U_chk, S_last, dout, dS_last, dq, dk_out, dv_out,
                                   dbeta, dS0, B, T, H, dk, dv, dtype, done_dtype);
 }
 
 extern "C" int mrx_deltanet_bwd(void *stream, const void *q, const void *k, const void *v,
                                 const void *beta_raw, const void *done, const void *S_chk,
-                                const void *Tm_chk, const void *U_chk, const void *dout, const void *dS_last,
-                                void *dq, void *dk_out, void *dv_out, void *dbeta_raw, void *dS0, int64_t B,
-                                int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
+                                const void *Tm_chk, const void *U_chk, const float *S_last, const void *dout,
+                                const void *dS_last, void *dq, void *dk_out, void *dv_out, void *dbeta_raw, void *dS0,
+                                int64_t B, int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                                 int done_dtype)
 {
-    return delta_bwd_entry<true>(stream, q, k, v, beta_raw, done, S_chk, Tm_chk, U_chk, dout, dS_last, dq, dk_out, dv_out,
+    return delta_bwd_entry<true>(stream, q, k, v, beta_raw, done, S_chk, Tm_chk, U_chk, S_last, dout, dS_last, dq, dk_out, dv_out,
                                  dbeta_raw, dS0, B, T, H, dk, dv, dtype, done_dtype);
 }

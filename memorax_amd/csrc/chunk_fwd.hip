@@ -70,7 +70,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                  const T *__restrict__ beta, const float *__restrict__ glog,
                  const void *__restrict__ done, int done_f32,
                  const float *__restrict__ S0, T *__restrict__ o, float *__restrict__ S_last,
-                 T *__restrict__ S_chk, T *__restrict__ Tm_chk, T *__restrict__ U_chk, int Tlen, int H, NormArgs na)
+                 void *__restrict__ S_chk, T *__restrict__ Tm_chk, T *__restrict__ U_chk, int Tlen, int H, NormArgs na)
 {
     static_assert(!(DELTA && GATED), "the gated variant is linear attention with a decay");
     static_assert(!NORM || (!DELTA && !GATED), "the normalised read-out belongs to plain linear attention");
@@ -315,18 +315,28 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             // 32 bytes per instruction): the output of the previous unit, parked in sO at its end, and
             // the state checkpoint from the copy of S that has just been staged.
             flush_o();
-            // The backward call walks the state back from chunk to chunk (S_c = S_{c+1} - U'_c^T K_c, the
-            // update it can undo from U' and K), so a checkpoint is written only where that walk has to
-            // start again: for the last chunk and for a chunk with resets, whose entering state the state
-            // that leaves it does not determine.  The decayed update of the gated variant is not undone
-            // (dividing by the decay), so there every chunk is written.
-            if (S_chk && pass == 0 && (GATED || !DELTA || nres != 0 || c == NC - 1)) {
-                using IOS = TileIO<T, HD, NTHR>;
+            // The backward call walks the state back from chunk to chunk in fp32, starting from S_last
+            // (S_c = S_{c+1} - U'_c^T K_c: the update it can undo from U' -- V for linear attention -- and
+            // K), so a checkpoint is written only where that walk cannot pass: for a chunk with resets,
+            // whose entering state the state that leaves it does not determine.  Those are written in fp32
+            // from the accumulators (rare, and the walk carries their rounding to the chunks before).  The
+            // decayed update of the gated variant is not undone (it would divide by the decay): there every
+            // chunk is written, in the I/O type, from the copy of S that has just been staged.
+            if (S_chk && pass == 0 && (GATED || nres != 0)) {
+                if (GATED) {
+                    using IOS = TileIO<T, HD, NTHR>;
 #pragma unroll
-                for (int p = 0; p < IOS::PASSES; ++p) {
-                    const int r = IOS::row_of(tid, p), seg = tid % IOS::SEGS;
-                    *reinterpret_cast<typename IOS::F *>(S_chk + schk_off + r * HD + seg * IOS::KP) =
-                        *reinterpret_cast<const typename IOS::F *>(sS + r * LDD + seg * IOS::KP);
+                    for (int p = 0; p < IOS::PASSES; ++p) {
+                        const int r = IOS::row_of(tid, p), seg = tid % IOS::SEGS;
+                        *reinterpret_cast<typename IOS::F *>(reinterpret_cast<T *>(S_chk) + schk_off + r * HD + seg * IOS::KP) =
+                            *reinterpret_cast<const typename IOS::F *>(sS + r * LDD + seg * IOS::KP);
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < TMS::TPW; ++j) {
+                        const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dv = TMS::nt(w, j) * 16 + li;
+                        *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(S_chk) + schk_off + dv * HD + dk0) = Sacc[j];
+                    }
                 }
             }
             const bool pre = pass == nres && c + 1 < NC;
@@ -558,7 +568,7 @@ int launch(hipStream_t st, const void *q, const void *k, const void *v, const vo
     if (const int rc = prepare_device(); rc != MRX_OK) return rc;
     return launch_kernel(chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN>, dim3((unsigned)(B * H)),
                          dim3(NTHR), Reg::smem, st, (const T *)q, (const T *)k, (const T *)v, (const T *)beta,
-                         (const float *)glog, done, done_f32, (const float *)S0, (T *)o, (float *)S_last, (T *)S_chk,
+                         (const float *)glog, done, done_f32, (const float *)S0, (T *)o, (float *)S_last, S_chk,
                          (T *)Tm_chk, (T *)U_chk, (int)Tlen, (int)H, na);
 }
 

@@ -196,18 +196,18 @@ class _LinearAttention(torch.autograd.Function):
                                               feature_map=_FMAP_NAME[fmap])
             ctx.done, ctx.fmap, ctx.has_S0 = done, fmap, S0 is not None
             return o[:, None], S_last
-        o, S_last, S_chk = K.linear_attn_fwd(q_, k_, v_, done, S0_, fmap, save_chk=need)
+        o, S_last, chk = K.linear_attn_fwd(q_, k_, v_, done, S0_, fmap, save_chk=need)
         if need:
-            ctx.save_for_backward(q_, k_, v_, S_chk)
+            ctx.save_for_backward(q_, k_, v_, *chk)
         ctx.done, ctx.fmap, ctx.has_S0 = done, fmap, S0 is not None
         return o, S_last
 
     @staticmethod
     def backward(ctx, do, dS_last):
-        q, k, v, S_chk = ctx.saved_tensors
+        q, k, v, S_chk, S_last = ctx.saved_tensors
         do = torch.zeros_like(v) if do is None else do.contiguous()
         dS_last = None if dS_last is None else dS_last.contiguous().float()
-        dq, dk, dv, dS0 = K.linear_attn_bwd(q, k, v, ctx.done, S_chk, do, dS_last, ctx.fmap,
+        dq, dk, dv, dS0 = K.linear_attn_bwd(q, k, v, ctx.done, (S_chk, S_last), do, dS_last, ctx.fmap,
                                             want_dS0=ctx.has_S0)
         return dq, dk, dv, None, (dS0 if ctx.has_S0 else None), None
 
@@ -240,11 +240,11 @@ class _NormalisedLinearAttention(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, do, dS_last, dz_last):
-        q, k, v, o, den, S_chk, z_chk = ctx.saved_tensors
+        q, k, v, o, den, S_chk, z_chk, S_last = ctx.saved_tensors
         do = torch.zeros_like(v) if do is None else do.contiguous()
         dS_last = None if dS_last is None else dS_last.contiguous().float()
         dz_last = None if dz_last is None else dz_last.contiguous().float()
-        dq, dk, dv, dS0, dz0 = K.linear_attn_norm_bwd(q, k, v, ctx.done, (S_chk, z_chk), o, den, do, dS_last,
+        dq, dk, dv, dS0, dz0 = K.linear_attn_norm_bwd(q, k, v, ctx.done, (S_chk, z_chk, S_last), o, den, do, dS_last,
                                                       dz_last, ctx.fmap, ctx.eps, want_d0=any(ctx.has_0))
         return dq, dk, dv, None, (dS0 if ctx.has_0[0] else None), (dz0 if ctx.has_0[1] else None), None, None
 
@@ -315,10 +315,10 @@ class _DeltaRule(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, do, dS_last):
-        q, k, v, beta, S_chk, Tm_chk, U_chk = ctx.saved_tensors
+        q, k, v, beta, S_chk, Tm_chk, U_chk, S_last = ctx.saved_tensors
         do = torch.zeros_like(v) if do is None else do.contiguous()
         dS_last = None if dS_last is None else dS_last.contiguous().float()
-        dq, dk, dv, db, dS0 = K.delta_rule_bwd(q, k, v, beta, ctx.done, (S_chk, Tm_chk, U_chk), do, dS_last,
+        dq, dk, dv, db, dS0 = K.delta_rule_bwd(q, k, v, beta, ctx.done, (S_chk, Tm_chk, U_chk, S_last), do, dS_last,
                                                want_dS0=ctx.has_S0, prologue=ctx.prologue)
         return dq, dk, dv, db, None, (dS0 if ctx.has_S0 else None), None
 

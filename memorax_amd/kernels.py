@@ -183,34 +183,38 @@ def _n_chunks(T, dt, delta=False):
 
 
 def linear_attn_fwd(q, k, v, done, S0=None, feature_map=0, save_chk=True):
-    """Returns (o, S_last fp32, S_chk or None)."""
+    """Returns (o, S_last fp32, chk) with chk = (S_chk, S_last), what the backward call needs, or None.
+    S_chk is float32 and sparse: the library writes only the slots of chunks that contain a reset (the
+    backward call walks the state back from S_last through the others)."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
     _chk(S0, "S0", torch.float32, (B, H, dv, dk))
     done, dd = _done(done, B, T)
     o = torch.empty_like(v)
     S_last = torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
-    S_chk = (torch.empty((B, H, _n_chunks(T, dt), dv, dk), dtype=dt, device=q.device)
+    S_chk = (torch.empty((B, H, _n_chunks(T, dt), dv, dk), dtype=torch.float32, device=q.device)
              if save_chk else None)
     st = lib.mrx_linear_attn_fwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(done), _ptr(S0),
                                  _ptr(o), _ptr(S_last), _ptr(S_chk), B, T, H, dk, dv, _DT[dt], dd,
                                  int(feature_map))
     _lib.check(st, "mrx_linear_attn_fwd")
-    return o, S_last, S_chk
+    return o, S_last, ((S_chk, S_last) if save_chk else None)
 
 
-def linear_attn_bwd(q, k, v, done, S_chk, do, dS_last=None, feature_map=0, want_dS0=True):
-    """Returns (dq, dk, dv, dS0)."""
+def linear_attn_bwd(q, k, v, done, chk, do, dS_last=None, feature_map=0, want_dS0=True):
+    """chk = (S_chk, S_last) from linear_attn_fwd.  Returns (dq, dk, dv, dS0)."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
+    S_chk, S_last = chk
     _chk(do, "do", dt, (B, T, H, dv))
-    _chk(S_chk, "S_chk", dt, (B, H, _n_chunks(T, dt), dv, dk))
+    _chk(S_chk, "S_chk", torch.float32, (B, H, _n_chunks(T, dt), dv, dk))
+    _chk(S_last, "S_last", torch.float32, (B, H, dv, dk))
     _chk(dS_last, "dS_last", torch.float32, (B, H, dv, dk))
     done, dd = _done(done, B, T)
     dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dS0 = (torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
            if want_dS0 else None)
-    st = lib.mrx_linear_attn_bwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(done), _ptr(S_chk),
+    st = lib.mrx_linear_attn_bwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(done), _ptr(S_chk), _ptr(S_last),
                                  _ptr(do), _ptr(dS_last), _ptr(dq), _ptr(dk_), _ptr(dv_),
                                  _ptr(dS0), B, T, H, dk, dv, _DT[dt], dd, int(feature_map))
     _lib.check(st, "mrx_linear_attn_bwd")
@@ -219,7 +223,8 @@ def linear_attn_bwd(q, k, v, done, S_chk, do, dS_last=None, feature_map=0, want_
 
 def linear_attn_norm_fwd(q, k, v, done, S0=None, z0=None, feature_map=0, eps=1e-6, save_chk=True):
     """Linear attention with the normalised read-out fused.
-    Returns (o, den fp32 (B,T,H), S_last fp32, z_last fp32, (S_chk, z_chk) or None)."""
+    Returns (o, den fp32 (B,T,H), S_last fp32, z_last fp32, (S_chk, z_chk, S_last) or None); S_chk as for
+    linear_attn_fwd."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
     _chk(S0, "S0", torch.float32, (B, H, dv, dk))
@@ -230,13 +235,13 @@ def linear_attn_norm_fwd(q, k, v, done, S0=None, z0=None, feature_map=0, eps=1e-
     S_last = torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
     z_last = torch.empty((B, H, dk), dtype=torch.float32, device=q.device)
     nc = _n_chunks(T, dt)
-    S_chk = torch.empty((B, H, nc, dv, dk), dtype=dt, device=q.device) if save_chk else None
+    S_chk = torch.empty((B, H, nc, dv, dk), dtype=torch.float32, device=q.device) if save_chk else None
     z_chk = torch.empty((B, H, nc, dk), dtype=torch.float32, device=q.device) if save_chk else None
     st = lib.mrx_linear_attn_norm_fwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(done), _ptr(S0), _ptr(z0),
                                       _ptr(o), _ptr(den), _ptr(S_last), _ptr(z_last), _ptr(S_chk), _ptr(z_chk),
                                       B, T, H, dk, dv, _DT[dt], dd, int(feature_map), float(eps))
     _lib.check(st, "mrx_linear_attn_norm_fwd")
-    return o, den, S_last, z_last, ((S_chk, z_chk) if save_chk else None)
+    return o, den, S_last, z_last, ((S_chk, z_chk, S_last) if save_chk else None)
 
 
 def linear_attn_norm_bwd(q, k, v, done, chk, o, den, do, dS_last=None, dz_last=None, feature_map=0, eps=1e-6,
@@ -244,12 +249,13 @@ def linear_attn_norm_bwd(q, k, v, done, chk, o, den, do, dS_last=None, dz_last=N
     """Returns (dq, dk, dv, dS0, dz0)."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
-    S_chk, z_chk = chk
+    S_chk, z_chk, S_last = chk
     nc = _n_chunks(T, dt)
+    _chk(S_last, "S_last", torch.float32, (B, H, dv, dk))
     _chk(do, "do", dt, (B, T, H, dv))
     _chk(o, "o", dt, (B, T, H, dv))
     _chk(den, "den", torch.float32, (B, T, H))
-    _chk(S_chk, "S_chk", dt, (B, H, nc, dv, dk))
+    _chk(S_chk, "S_chk", torch.float32, (B, H, nc, dv, dk))
     _chk(z_chk, "z_chk", torch.float32, (B, H, nc, dk))
     _chk(dS_last, "dS_last", torch.float32, (B, H, dv, dk))
     _chk(dz_last, "dz_last", torch.float32, (B, H, dk))
@@ -257,7 +263,7 @@ def linear_attn_norm_bwd(q, k, v, done, chk, o, den, do, dS_last=None, dz_last=N
     dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dS0 = torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device) if want_d0 else None
     dz0 = torch.empty((B, H, dk), dtype=torch.float32, device=q.device) if want_d0 else None
-    st = lib.mrx_linear_attn_norm_bwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(done), _ptr(S_chk), _ptr(z_chk),
+    st = lib.mrx_linear_attn_norm_bwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(done), _ptr(S_chk), _ptr(S_last), _ptr(z_chk),
                                       _ptr(o), _ptr(den), _ptr(do), _ptr(dS_last), _ptr(dz_last), _ptr(dq),
                                       _ptr(dk_), _ptr(dv_), _ptr(dS0), _ptr(dz0), B, T, H, dk, dv, _DT[dt], dd,
                                       int(feature_map), float(eps))
@@ -301,10 +307,10 @@ def delta_rule_fwd_noalloc(q, k, v, beta, done, S0=None, out=None):
 
 def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prologue=False, tm_scratch=None,
                    factor_path=None):
-    """Returns (o, S_last fp32, chk) where chk = (S_chk, Tm_chk, U_chk) are the residuals the
-    backward call needs, or None: the states entering the chunks (written only for the last chunk and
-    for chunks with resets -- the backward call walks the state back through the others), the
-    triangular factors and U' (B,T,H,dv).  out = (o, S_last, S_chk, Tm_chk, U_chk) reuses buffers of an
+    """Returns (o, S_last fp32, chk) where chk = (S_chk, Tm_chk, U_chk, S_last) is what the
+    backward call needs, or None: the states entering the chunks (float32; written only for chunks with
+    resets -- the backward call walks the state back from S_last through the others), the triangular
+    factors and U' (B,T,H,dv).  out = (o, S_last, S_chk, Tm_chk, U_chk, ...) reuses buffers of an
     earlier call with the same shapes instead of allocating.  prologue=True: k is L2-normalised and
     beta = sigmoid(beta) inside the kernel (mrx_deltanet_fwd).
     tm_scratch (only without residuals): give the library a buffer for the triangular factors
@@ -317,11 +323,11 @@ def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prolog
     _chk(S0, "S0", torch.float32, (B, H, dv, dk))
     done, dd = _done(done, B, T)
     if out is not None:
-        o, S_last, S_chk, Tm_chk, U_chk = out
+        o, S_last, S_chk, Tm_chk, U_chk = out[:5]
         C, NC = chunk_size(dt, True), _n_chunks(T, dt, True)
         _chk(o, "out o", dt, (B, T, H, dv))
         _chk(S_last, "out S_last", torch.float32, (B, H, dv, dk))
-        _chk(S_chk, "out S_chk", dt, (B, H, NC, dv, dk))
+        _chk(S_chk, "out S_chk", torch.float32, (B, H, NC, dv, dk))
         _chk(Tm_chk, "out Tm_chk", dt, (B, H, NC, C, C))
         _chk(U_chk, "out U_chk", dt, (B, T, H, dv))
         save_chk = S_chk is not None
@@ -331,7 +337,7 @@ def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prolog
         S_chk = Tm_chk = U_chk = None
         if save_chk:
             C, NC = chunk_size(dt, True), _n_chunks(T, dt, True)
-            S_chk = torch.empty((B, H, NC, dv, dk), dtype=dt, device=q.device)
+            S_chk = torch.empty((B, H, NC, dv, dk), dtype=torch.float32, device=q.device)
             U_chk = torch.empty_like(v)
             Tm_chk = torch.empty((B, H, NC, C, C), dtype=dt, device=q.device)
         else:
@@ -345,22 +351,23 @@ def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prolog
                             _ptr(S0), _ptr(o), _ptr(S_last), _ptr(S_chk), _ptr(Tm_chk), _ptr(U_chk), B, T, H,
                             dk, dv, _DT[dt], dd, _FACTORS[factor_path])
     _lib.check(st, name)
-    return o, S_last, ((S_chk, Tm_chk, U_chk) if save_chk else None)
+    return o, S_last, ((S_chk, Tm_chk, U_chk, S_last) if save_chk else None)
 
 
 def delta_rule_bwd(q, k, v, beta, done, chk, do, dS_last=None, want_dS0=True, out=None, prologue=False):
-    """chk = (S_chk, Tm_chk, U_chk) from delta_rule_fwd.  Returns (dq, dk, dv, dbeta, dS0).
+    """chk = (S_chk, Tm_chk, U_chk, S_last) from delta_rule_fwd.  Returns (dq, dk, dv, dbeta, dS0).
     out = (dq, dk, dv, dbeta, dS0) reuses buffers instead of allocating.  prologue=True pairs with
     delta_rule_fwd(prologue=True): k and beta are the raw projections and so are dk and dbeta."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
-    S_chk, Tm_chk, U_chk = chk
+    S_chk, Tm_chk, U_chk, S_last = chk
     C = chunk_size(dt, True)
+    _chk(S_last, "S_last", torch.float32, (B, H, dv, dk))
     _chk(U_chk, "U_chk", dt, (B, T, H, dv))
     _chk(Tm_chk, "Tm_chk", dt, (B, H, _n_chunks(T, dt, True), C, C))
     _chk(beta, "beta", dt, (B, T, H))
     _chk(do, "do", dt, (B, T, H, dv))
-    _chk(S_chk, "S_chk", dt, (B, H, _n_chunks(T, dt, True), dv, dk))
+    _chk(S_chk, "S_chk", torch.float32, (B, H, _n_chunks(T, dt, True), dv, dk))
     _chk(dS_last, "dS_last", torch.float32, (B, H, dv, dk))
     done, dd = _done(done, B, T)
     if out is not None:
@@ -375,7 +382,8 @@ def delta_rule_bwd(q, k, v, beta, done, chk, do, dS_last=None, want_dS0=True, ou
                if want_dS0 else None)
     name = "mrx_deltanet_bwd" if prologue else "mrx_delta_rule_bwd"
     st = getattr(lib, name)(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done),
-                            _ptr(S_chk), _ptr(Tm_chk), _ptr(U_chk), _ptr(do), _ptr(dS_last), _ptr(dq), _ptr(dk_),
+                            _ptr(S_chk), _ptr(Tm_chk), _ptr(U_chk), _ptr(S_last), _ptr(do), _ptr(dS_last), _ptr(dq),
+                            _ptr(dk_),
                             _ptr(dv_), _ptr(dbeta), _ptr(dS0), B, T, H, dk, dv, _DT[dt], dd)
     _lib.check(st, name)
     return dq, dk_, dv_, dbeta, dS0

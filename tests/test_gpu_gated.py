@@ -155,7 +155,8 @@ def test_gated_with_zero_log_decay_is_linear_attention_at_full_size():
     dq2, dk2, dv2, _ = K.linear_attn_bwd(q, k, v, done, chk2, do, None, 1, want_dS0=False)
     assert relerr(Sl, Sl2.cpu().numpy()) <= 1e-5
     # bf16 outputs: the gated kernels add the two terms of dV and dK in the other order, so a result may
-    # round to the neighbouring bf16 value (2^-8 relative)
+    # round to the neighbouring bf16 value (2^-8 relative); and their backward takes the state entering
+    # a chunk from a bf16 checkpoint where the plain kernel walks it back in fp32 (another 2^-9 on dq)
     for a, b_ in ((o, o2), (dq, dq2), (dk, dk2), (dv, dv2)):
-        assert relerr(a, b_.float().cpu().numpy()) <= 2.0 ** -8
+        assert relerr(a, b_.float().cpu().numpy()) <= 2.0 ** -7
     assert torch.isfinite(dg).all()
