@@ -130,7 +130,7 @@ def main() -> int:
 
     # outputs and residuals are allocated once and reused, as a training loop's caching allocator does
     o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done)
-    fwd_out = (o, Sl, *chk)
+    fwd_out = (o, Sl, chk[0], chk[1])
     bwd_out = K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False)
 
     def step():

@@ -83,12 +83,14 @@ int mrx_version(void);
  * of the per-chunk state checkpoints S_chk: (B, H, ceil(T/chunk), dv, dk).
  *
  * State checkpoints.  The backward calls need the state entering every chunk.  Where the chunk's
- * update can be undone (plain and normalised linear attention: S_c = S_{c+1} - V_c^T K_c; delta rule:
- * S_c = S_{c+1} - U'_c^T K_c) they walk it back in fp32 from the forward call's S_last, which is
+ * update can be undone cheaply (plain and normalised linear attention: S_c = S_{c+1} - V_c^T K_c)
+ * they walk it back in fp32 from the forward call's S_last, which is
  * then an INPUT of the backward call, and S_chk is a float32 buffer that the forward call writes
  * SPARSELY: only the slots of chunks that contain a reset -- whose entering state the leaving one does
  * not determine -- are written and read; the other slots keep whatever the buffer held.  The gated
- * kernels (whose decayed update is not undone) keep one checkpoint per chunk in `dtype`. */
+ * kernels (whose decayed update is not undone) and the delta rule (where the walk would need U' as a
+ * further residual and one more product per chunk: measured slower) keep one checkpoint per chunk
+ * in `dtype`. */
 int64_t mrx_chunk_size(int dtype);
 
 /* The same for the delta-rule kernels (S_chk and Tm_chk of mrx_delta_rule_fwd/_bwd). */
@@ -194,15 +196,11 @@ int mrx_linear_attn_norm_bwd(void *stream, const void *q, const void *k,
  * MRX_FACTORS_PARALLEL takes the chunk-parallel kernel whenever the buffer is given (on a full
  * device that is level with the default when episodes end every hundred steps or so, and slower
  * when resets are rare), MRX_FACTORS_INLINE never does.
- * U_chk (nullable; required with S_chk): (B,T,H,dv) in `dtype`, receives U'_t = the rows of
- * Tm diag(beta) (V - K S^T), the chunk's increments: S_leaving = S_entering + U'^T K.  The backward
- * call undoes that update chunk by chunk (S_c = S_{c+1} - U'_c^T K_c, in fp32, from S_last), so
- * S_chk (float32) is written sparsely, as for linear attention (see mrx_chunk_size).  Per 32-step
- * chunk that is 4 KB of residual each way instead of the 8 KB of a state checkpoint. */
+ * S_chk: (B,H,ceil(T/chunk),dv,dk) in `dtype`, one checkpoint per chunk (dense; see mrx_chunk_size). */
 int mrx_delta_rule_fwd(void *stream, const void *q, const void *k,
                        const void *v, const void *beta, const void *done,
                        const void *S0, void *o, void *S_last, void *S_chk,
-                       void *Tm_chk, void *U_chk, int64_t B, int64_t T, int64_t H, int64_t dk,
+                       void *Tm_chk, int64_t B, int64_t T, int64_t H, int64_t dk,
                        int64_t dv, int dtype, int done_dtype, int factor_path);
 
 /* mrx_delta_rule_fwd without residuals for callers that cannot allocate device memory (code under
@@ -224,12 +222,11 @@ int mrx_delta_rule_fwd_noalloc(void *stream, const void *q, const void *k,
                                int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                                int done_dtype);
 
-/* Gradients w.r.t. q,k,v,beta (in `dtype`) and S0 (fp32, nullable).  S_chk, Tm_chk,
- * U_chk and S_last are what mrx_delta_rule_fwd wrote on the same inputs. */
+/* Gradients w.r.t. q,k,v,beta (in `dtype`) and S0 (fp32, nullable).  S_chk and
+ * Tm_chk are the residuals written by mrx_delta_rule_fwd on the same inputs. */
 int mrx_delta_rule_bwd(void *stream, const void *q, const void *k,
                        const void *v, const void *beta, const void *done,
-                       const void *S_chk, const void *Tm_chk, const void *U_chk,
-                       const float *S_last, const void *dout,
+                       const void *S_chk, const void *Tm_chk, const void *dout,
                        const void *dS_last, void *dq, void *dk_out, void *dv_out,
                        void *dbeta, void *dS0, int64_t B, int64_t T, int64_t H,
                        int64_t dk, int64_t dv, int dtype, int done_dtype);
@@ -244,14 +241,13 @@ int mrx_delta_rule_bwd(void *stream, const void *q, const void *k,
  * Residuals as for mrx_delta_rule_*. */
 int mrx_deltanet_fwd(void *stream, const void *q, const void *k, const void *v,
                      const void *beta_raw, const void *done, const void *S0, void *o,
-                     void *S_last, void *S_chk, void *Tm_chk, void *U_chk, int64_t B, int64_t T,
+                     void *S_last, void *S_chk, void *Tm_chk, int64_t B, int64_t T,
                      int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype,
                      int factor_path);
 
 int mrx_deltanet_bwd(void *stream, const void *q, const void *k, const void *v,
                      const void *beta_raw, const void *done, const void *S_chk,
-                     const void *Tm_chk, const void *U_chk, const float *S_last, const void *dout,
-                     const void *dS_last, void *dq,
+                     const void *Tm_chk, const void *dout, const void *dS_last, void *dq,
                      void *dk_out, void *dv_out, void *dbeta_raw, void *dS0, int64_t B,
                      int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                      int done_dtype);

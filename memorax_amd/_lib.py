@@ -34,11 +34,11 @@ SIGNATURES = {
     "mrx_linear_attn_bwd": (_I, [_P] * 13 + [_L] * 5 + [_I] * 3),
     "mrx_linear_attn_norm_fwd": (_I, [_P] * 13 + [_L] * 5 + [_I] * 3 + [ctypes.c_float]),
     "mrx_linear_attn_norm_bwd": (_I, [_P] * 18 + [_L] * 5 + [_I] * 3 + [ctypes.c_float]),
-    "mrx_delta_rule_fwd": (_I, [_P] * 12 + [_L] * 5 + [_I] * 3),
+    "mrx_delta_rule_fwd": (_I, [_P] * 11 + [_L] * 5 + [_I] * 3),
     "mrx_delta_rule_fwd_noalloc": (_I, [_P] * 9 + [_L] * 5 + [_I] * 2),
-    "mrx_delta_rule_bwd": (_I, [_P] * 17 + [_L] * 5 + [_I] * 2),
-    "mrx_deltanet_fwd": (_I, [_P] * 12 + [_L] * 5 + [_I] * 3),
-    "mrx_deltanet_bwd": (_I, [_P] * 17 + [_L] * 5 + [_I] * 2),
+    "mrx_delta_rule_bwd": (_I, [_P] * 15 + [_L] * 5 + [_I] * 2),
+    "mrx_deltanet_fwd": (_I, [_P] * 11 + [_L] * 5 + [_I] * 3),
+    "mrx_deltanet_bwd": (_I, [_P] * 15 + [_L] * 5 + [_I] * 2),
     "mrx_linear_scan_last": (_I, [_P] * 6 + [_L] * 4 + [_I] * 2),
     "mrx_mingru_scan_fwd": (_I, [_P] * 9 + [_L] * 3 + [_I]),
     "mrx_mingru_scan_bwd": (_I, [_P] * 11 + [_L] * 3 + [_I]),

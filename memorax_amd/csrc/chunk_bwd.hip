@@ -164,8 +164,9 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     // whether its checkpoint must be fetched is known when the next prefetch starts
     uint32_t rdone = 0u, rdone2 = 0u;
     // Does the chunk about to be prefetched take its entering state from S_chk?  Not known for the
-    // first one (its reset flags are part of the same prefetch): read then, used only if it applies.
-    bool need_S = true;
+    // first one (its reset flags are part of the same prefetch): if it does, the checkpoint is fetched
+    // when the chunk is reached.
+    bool need_S = false;
     float rg = 0.f;       // log-decay of chunk row `lane` (gated)
     // Running element offsets of this thread's loads, stepped back by one chunk per prefetch
     // (64-bit adds instead of per-chunk index multiplications).  The prefetch is issued in parts
@@ -394,6 +395,13 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     for (int j = 0; j < NSA; ++j) Sacc[j] -= acc[j];
                     store_acc<T, HD, HD, NW>(Sacc, sS, LDD, w, lane);
                 } else if (pass == 0) {
+                    if (c == NC - 1) {  // the one checkpoint no prefetch could know of
+#pragma unroll
+                        for (int j = 0; j < NSA; ++j)
+                            rS32[j] = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(S_chk) +
+                                                                       ((int64_t)bh * NC + c) * HD * HD + li * HD + 4 * lg +
+                                                                       TMS::nt(w, j) * 16 * HD + TMS::mt(w, j) * 16);
+                    }
 #pragma unroll
                     for (int j = 0; j < NSA; ++j) Sacc[j] = rS32[j];
                     store_acc<T, HD, HD, NW>(Sacc, sS, LDD, w, lane);
@@ -566,12 +574,8 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 // delta rule: fourteen LDS tiles (68 KB for bf16, 127 KB for fp32, C = 32), two of them reused
 // once their first tenant is dead.  bf16: two workgroups per CU.
 //
-// Per pass, with Tm = (I + A)^-1 and U' (= Tm diag(beta) (V - K S^T)) from the forward call and S the
-// state entering the chunk -- walked back from the state leaving it, S_c = S_{c+1} - U'_c^T K_c, in
-// fp32 registers that start from the forward call's S_last; read from the forward call's (fp32)
-// checkpoint where the walk cannot pass (a chunk with resets, whose entering state the leaving one
-// does not determine):
-//   V0 = V - K S^T                                                 (for dbeta only)
+// Per pass, with S the state entering the chunk, Tm = (I + A)^-1 from the forward call:
+//   V0 = V - K S^T,  V~ = diag(beta) V0,  U' = Tm V~            (W = T K and U = T V are never formed)
 //   Aqk = tril(Q K^T),  dU' = Aqk^T dO + K dS^T,  dAqk = tril(dO U'^T)
 //   Z = Tm^T dU',  dV = diag(beta) Z,  dbeta = rowdot(Z, V0) + rowdot(K, R)
 //   dA = -tril(Z U'^T, -1),  R = dA K
@@ -587,7 +591,7 @@ template <typename T, int C, int NW> struct DeltaBwdSmem : BwdDims<T, C> {
     static_assert(D::szCC <= D::szRD && D::szCC <= D::szDD, "reused regions must hold a [C][C] tile");
     // nine [C][64] tiles, two [64][64], three [C][C]
     static constexpr int oK = 0, oV = oK + D::szRD, oQ = oV + D::szRD, oDO = oQ + D::szRD,
-                         oBK = oDO + D::szRD, oZ = oBK + D::szRD, oU = oZ + D::szRD, oDU = oU + D::szRD,
+                         oBK = oDO + D::szRD, oVt = oBK + D::szRD, oU = oVt + D::szRD, oDU = oU + D::szRD,
                          oZb = oDU + D::szRD, oS = oZb + D::szRD, oDS = oS + D::szDD,
                          oAqk = oDS + D::szDD, oTm = oAqk + D::szCC, oDT = oTm + D::szCC,
                          oBeta = oDT + D::szCC, oDb = oBeta + C * 4;
@@ -604,14 +608,15 @@ template <typename T, int C, int NW, bool PRO>
 __global__ void __launch_bounds__(64 * NW, sizeof(T) == 2 ? 2 : 1)
 delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
-                 const float *__restrict__ S_chk, const T *__restrict__ Tm_chk, const T *__restrict__ U_chk,
-                 const float *__restrict__ S_last, const T *__restrict__ dout, const float *__restrict__ dS_last, T *__restrict__ dq,
+                 const T *__restrict__ S_chk, const T *__restrict__ Tm_chk,
+                 const T *__restrict__ dout, const float *__restrict__ dS_last, T *__restrict__ dq,
                  T *__restrict__ dk, T *__restrict__ dv, T *__restrict__ dbeta,
                  float *__restrict__ dS0, int Tlen, int H)
 {
     constexpr int NTHR = 64 * NW;
     using L = DeltaBwdSmem<T, C, NW>;
     using IO = TileIO<T, C, NTHR>;
+    using IOS = TileIO<T, HD, NTHR>;
     using IOT = TileIO<T, C, NTHR, C>;  // the [C][C] triangular factor
     using P4 = typename TT<T>::pack4;
     constexpr int LDD = L::LDD, LDC = L::LDC;
@@ -619,8 +624,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     auto at = [&](int off) { return reinterpret_cast<T *>(smem + off); };
     T *sK = at(L::oK), *sQ = at(L::oQ), *sDO = at(L::oDO), *sBK = at(L::oBK);
     T *sV = at(L::oV);                                    // V[c][dv] -> V0 = V - K S^T (in place)
-    T *sZ = at(L::oZ);                                    // Z[c][dv], then the pass's dK on its way to memory
-    T *sU = at(L::oU), *sDU = at(L::oDU), *sZb = at(L::oZb);  // U'[c][dv] as the forward call left it
+    T *sVt = at(L::oVt), *sZ = at(L::oVt);                // V~ = beta V0 -> Z[c][dv]
+    T *sU = at(L::oU), *sDU = at(L::oDU), *sZb = at(L::oZb);
     T *sS = at(L::oS);                                    // S[dv][dk]
     T *sDS = at(L::oDS);                                  // dS[dv][dk]
     T *sAqk = at(L::oAqk), *sDAqk = at(L::oAqk);          // Aqk^T[j][i] -> dAqk[i][j]
@@ -651,22 +656,10 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                            : f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    f32x4 Sacc[TMS::TPW];  // S^T leaving, then entering, the chunk at hand; in the layout of dS^T
-#pragma unroll
-    for (int j = 0; j < TMS::TPW; ++j) {
-        const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
-        Sacc[j] = *reinterpret_cast<const f32x4 *>(S_last + ((int64_t)bh * HD + dvv) * HD + dk0);
-    }
-
-    typename IO::Regs rq, rk, rv, rdo, ru;
-    f32x4 rS[TMS::TPW];  // a checkpoint, in the layout of Sacc
+    typename IO::Regs rq, rk, rv, rdo;
+    typename IOS::Regs rS;
     typename IOT::Regs rTm;
-    // raw bits, converted when the chunk is staged; the reset flags of the chunk after the next one as
-    // well: whether its checkpoint must be fetched is known when the next prefetch starts
-    uint32_t rdone = 0u, rdone2 = 0u, rbeta = 0u;
-    // Does the chunk about to be prefetched take its entering state from S_chk?  Not known for the
-    // first one (its reset flags are part of the same prefetch): read then, used only if it applies.
-    bool need_S = true;
+    uint32_t rdone = 0u, rbeta = 0u;  // raw bits, converted when the chunk is staged
     uint32_t rbrow[IO::PASSES];       // beta of the rows this thread stages
     // Running element offsets of this thread's loads and stores, stepped back by one chunk per
     // iteration (64-bit adds instead of per-chunk index multiplications).
@@ -678,14 +671,14 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         roff[p] = base + (int64_t)r * rs + (tid % IO::SEGS) * IO::KP;  // q/k/v/dout: row r, this thread's segment
         boff[p] = ((int64_t)b * Tlen + r) * H + h;                     // beta of row r
     }
-    int64_t soff = ((int64_t)bh * NC + NC - 1) * HD * HD + li * HD + 4 * lg;
+    int64_t soff = ((int64_t)bh * NC + NC - 1) * HD * HD + (tid / IOS::SEGS) * HD + (tid % IOS::SEGS) * IOS::KP;
     int64_t tmoff = ((int64_t)bh * NC + NC - 1) * C * C + (tid / IOT::SEGS) * C + (tid % IOT::SEGS) * IOT::KP;
     int64_t doff = (int64_t)b * Tlen + tlast + lane;  // done/beta of chunk row `lane`
     int tpre = tlast;                                 // first time step of the chunk about to be prefetched
     // The prefetch of the next chunk is issued in parts, two in each of the first three phases, so
     // that the address unit works through the loads beside the phases' LDS and MFMA work instead of
     // stalling every wave at one point, and all of them are under way before the first store of the
-    // pass.  part 0: q, 1: k, 2: v, 3: dout, 4: U' (and S where checkpointed), 5: Tm and the per-row scalars.
+    // pass.  part 0: q, 1: k, 2: v, 3: dout, 4: S, 5: Tm and the per-row scalars.
     auto prefetch_part = [&](int part) {
         typename IO::F z;
 #pragma unroll
@@ -698,13 +691,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 dst.v[p] = tpre + IO::row_of(tid, p) < Tlen ? *reinterpret_cast<const typename IO::F *>(src + roff[p]) : z;
         } else if (part == 4) {
 #pragma unroll
-            for (int p = 0; p < IO::PASSES; ++p)
-                ru.v[p] = tpre + IO::row_of(tid, p) < Tlen ? *reinterpret_cast<const typename IO::F *>(U_chk + roff[p]) : z;
-            if (need_S) {
-#pragma unroll
-                for (int j = 0; j < TMS::TPW; ++j)
-                    rS[j] = *reinterpret_cast<const f32x4 *>(S_chk + soff + TMS::nt(w, j) * 16 * HD + TMS::mt(w, j) * 16);
-            }
+            for (int p = 0; p < IOS::PASSES; ++p)
+                rS.v[p] = *reinterpret_cast<const typename IOS::F *>(S_chk + soff + p * IOS::RPP * HD);
         } else {
 #pragma unroll
             for (int p = 0; p < IOT::PASSES; ++p)
@@ -717,13 +705,11 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 boff[p] -= (int64_t)C * H;
             }
             rdone = 0u;
-            rdone2 = 0u;
             rbeta = 0u;
             if (lane < C && tpre + lane < Tlen) {
                 rdone = done_raw(done, done_f32, doff);
                 if (w == 0) rbeta = load_raw<T>(beta + doff * H + h);
             }
-            if (lane < C && tpre >= C) rdone2 = done_raw(done, done_f32, doff - C);
             soff -= HD * HD;
             tmoff -= C * C;
             doff -= C;
@@ -738,18 +724,18 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     // group, so a store from accumulators writes 16 pieces of 32 bytes per instruction; written to a
     // dead LDS tile first (dV is there anyway) and read back row-wise, every instruction writes whole
     // 128-byte rows (measured: the three stores from accumulators cost a third of the kernel).
-    // dK is complete only in a pass's last phase; it waits in sZ -- not written again before the
-    // next pass's third phase -- and goes to memory after the next pass has been staged, so that no
+    // dK is complete only in a pass's last phase; it waits in sU -- not written again before the
+    // next pass's second phase -- and goes to memory after the next pass has been staged, so that no
     // store is issued right before the wait for the prefetched loads.  dbeta waits in a register.
     unsigned long long pend_dmask = 0ull;
     int pend_nres = 0, pend_pass = 0, pend_t0 = -1;
     int64_t pend_dboff = 0;
     float pend_db = 0.f;
     bool pend_db_on = false;
-    auto flush_pending = [&]() {  // call after a barrier that follows the writes to sZ
+    auto flush_pending = [&]() {  // call after a barrier that follows the writes to sU
         if (pend_t0 >= 0) {
             auto keep = [&](int r) { return pend_nres == 0 || episode_of(pend_dmask, r) == pend_pass; };
-            tile_rows_to_global<T, C, NTHR>(sZ, LDD, dk + base + (int64_t)pend_t0 * rs, rs, pend_t0, Tlen, tid, keep);
+            tile_rows_to_global<T, C, NTHR>(sU, LDD, dk + base + (int64_t)pend_t0 * rs, rs, pend_t0, Tlen, tid, keep);
         }
         if (pend_db_on) dbeta[pend_dboff] = (T)pend_db;
         pend_t0 = -1;
@@ -760,22 +746,17 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         const int t0 = c * C;
         const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
-        // where the state entering this chunk comes from: the forward call's checkpoint, or the walk
-        const bool ckpt = nres != 0;
-        need_S = __ballot(done_test(rdone2, done_f32) && lane < C) != 0ull;  // for the chunk prefetched during this one
         for (int pass = nres; pass >= 0; --pass) {
             auto live = [&](int r) { return nres == 0 || episode_of(dmask, r) == pass; };
             // ---- stage ---------------------------------------------------------------
             {
-                typename IO::Regs fq = rq, fk = rk, fv = rv, fdo = rdo, fu = ru;
+                typename IO::Regs fq = rq, fk = rk, fv = rv, fdo = rdo;
                 if (nres != 0) {
                     IO::mask_rows(fq, tid, live);
                     IO::mask_rows(fk, tid, live);
                     IO::mask_rows(fv, tid, live);
                     IO::mask_rows(fdo, tid, live);
-                    IO::mask_rows(fu, tid, live);
                 }
-                IO::to_lds(fu, sU, LDD, tid);
                 if (PRO) {
                     float kinv[IO::PASSES];
 #pragma unroll
@@ -800,6 +781,9 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                             : PRO ? sigmoidf(raw_to_float<T>(rbrow[p])) : raw_to_float<T>(rbrow[p]);
                 IO::scale_rows(fk, bf);
                 IO::to_lds(fk, sBK, LDD, tid);
+                typename IOS::Regs fS = rS;
+                if (pass != 0) IOS::zero(fS);
+                IOS::to_lds(fS, sS, LDD, tid);
                 // Tm[i][j] from the forward call (block diagonal by episode).  Rows of other episodes
                 // are cleared by select: they only ever meet zeros, but a NaN key or gate of another
                 // episode sits in them and must not meet those zeros.
@@ -824,28 +808,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sQ, LDD, sK, LDD, w, lane);
                 store_acc_f<T, C, C, NW>(acc, sAqk, LDC, w, lane, [](int m, int n, float x) { return m >= n ? x : 0.f; });
             }
-            // ---- the state entering the chunk, S^T[dk][dv] = S_leaving^T - sum_c K[c][dk] U'[c][dv], or the
-            //      forward call's checkpoint (first episode of a chunk with resets; the later ones start
-            //      from zero); rounded into sS[dv][dk] -----------------------------------------------------
-            if (!ckpt) {
-                f32x4 acc[TMS::TPW];
-                zero_acc<TMS::TPW>(acc);
-                gemm<T, HD, HD, C, KROW, KROW, NW>(acc, sK, LDD, sU, LDD, w, lane);
-#pragma unroll
-                for (int j = 0; j < TMS::TPW; ++j) Sacc[j] -= acc[j];
-                store_acc<T, HD, HD, NW>(Sacc, sS, LDD, w, lane);
-            } else if (pass == 0) {
-#pragma unroll
-                for (int j = 0; j < TMS::TPW; ++j) Sacc[j] = rS[j];
-                store_acc<T, HD, HD, NW>(Sacc, sS, LDD, w, lane);
-            } else {
-                f32x4 zero[TMS::TPW];
-                zero_acc<TMS::TPW>(zero);
-                store_acc<T, HD, HD, NW>(zero, sS, LDD, w, lane);
-            }
-            sync_lds();
-            if (pre) { prefetch_part(2); prefetch_part(3); }
-            // ---- V0[c][dv] = V[c][dv] - sum_dk S[dv][dk] K[c][dk] (in place; dbeta needs it) -----------
+            // ---- V0[c][dv] = V[c][dv] - sum_dk S[dv][dk] K[c][dk] (in place), V~ = beta_c V0 -> sVt ---
             {
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
@@ -854,9 +817,25 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 for (int j = 0; j < TMR::TPW; ++j) {
                     const int d0 = TMR::mt(w, j) * 16 + 4 * lg, r = TMR::nt(w, j) * 16 + li;
                     const P4 x = *reinterpret_cast<const P4 *>(sV + r * LDD + d0);  // each lane rewrites what it read
-                    *reinterpret_cast<P4 *>(sV + r * LDD + d0) = TT<T>::pack((float)x[0] - acc[j][0], (float)x[1] - acc[j][1],
-                                                                            (float)x[2] - acc[j][2], (float)x[3] - acc[j][3]);
+                    const float bb = sBeta[r];
+                    float y[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) y[e] = (float)x[e] - acc[j][e];
+                    const P4 v0 = TT<T>::pack(y[0], y[1], y[2], y[3]);
+                    *reinterpret_cast<P4 *>(sV + r * LDD + d0) = v0;
+                    // V~ from the rounded V0, so that dbeta = rowdot(Z, V0) matches what U' was built from
+                    *reinterpret_cast<P4 *>(sVt + r * LDD + d0) =
+                        TT<T>::pack(bb * (float)v0[0], bb * (float)v0[1], bb * (float)v0[2], bb * (float)v0[3]);
                 }
+            }
+            sync_lds();
+            if (pre) { prefetch_part(2); prefetch_part(3); }
+            // ---- U'^T[dv][c] = sum_j V~[j][dv] Tm[c][j] -> sU[c][dv] ----------------------------------
+            {
+                f32x4 acc[TMR::TPW];
+                zero_acc<TMR::TPW>(acc);
+                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sVt, LDD, sTm, LDC, w, lane);
+                store_acc<T, HD, C, NW>(acc, sU, LDD, w, lane);
             }
             // ---- dU'^T[dv][j] = sum_i dO[i][dv] Aqk[i][j] + sum_dk dS[dv][dk] K[j][dk] -> sDU[j][dv]
             {
@@ -893,7 +872,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 zero_acc<TMR::TPW>(acc);
                 gemm<T, HD, C, C, KROW, KROW, NW>(acc, sDU, LDD, sTm, LDC, w, lane);
                 rowdot(acc, sV);
-                store_acc<T, HD, C, NW>(acc, sZ, LDD, w, lane);  // the dK parked there left after the staging barrier
+                store_acc<T, HD, C, NW>(acc, sZ, LDD, w, lane);  // V~ is dead: every wave has formed its U'
 #pragma unroll
                 for (int j = 0; j < TMR::TPW; ++j) acc[j] *= sBeta[TMR::nt(w, j) * 16 + li];
                 store_acc<T, HD, C, NW>(acc, sZb, LDD, w, lane);  // = dV, written to memory from here after the barrier
@@ -949,7 +928,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                 for (int j = 0; j < TMR::TPW; ++j) dKacc[j] += acc[j] * sBeta[TMR::nt(w, j) * 16 + li];
                 gemm<T, HD, C, C, KROW, KROW, NW>(dKacc, sBK, LDD, sDA, LDC, w, lane);
-                if (!PRO) store_acc<T, HD, C, NW>(dKacc, sZ, LDD, w, lane);  // Z is dead since the last barrier
+                if (!PRO) store_acc<T, HD, C, NW>(dKacc, sU, LDD, w, lane);
             }
             // prologue: dKacc holds the gradient of the normalised keys; its component along k_n is
             // removed once the row dots k_n . dk_n are summed over the feature blocks (after the barrier).
@@ -995,7 +974,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                     for (int e = 0; e < 4; ++e) dKacc[j][e] = (dKacc[j][e] - (float)kn[j][e] * sd) * kiv[j % TMR::NBW];
                 }
-                store_acc<T, HD, C, NW>(dKacc, sZ, LDD, w, lane);
+                store_acc<T, HD, C, NW>(dKacc, sU, LDD, w, lane);
             }
             pend_dmask = dmask;
             pend_nres = nres;
@@ -1139,36 +1118,34 @@ template <typename T, int C, bool PRO> struct DeltaBwdReg {
 
 template <typename T, int C, bool PRO>
 int launch_delta_bwd(hipStream_t st, const void *q, const void *k, const void *v, const void *beta,
-                     const void *done, int done_dtype, const void *S_chk, const void *Tm_chk, const void *U_chk,
-                     const void *S_last, const void *dout, const void *dS_last, void *dq, void *dk_out, void *dv_out, void *dbeta, void *dS0,
-                     int64_t B, int64_t T_, int64_t H)
+                     const void *done, int done_dtype, const void *S_chk, const void *Tm_chk, const void *dout,
+                     const void *dS_last, void *dq, void *dk_out, void *dv_out, void *dbeta, void *dS0, int64_t B,
+                     int64_t T_, int64_t H)
 {
     using Reg = DeltaBwdReg<T, C, PRO>;
     (void)&Reg::reg;  // the kernel is on the list mrx_init() walks
     if (const int rc = prepare_device(); rc != MRX_OK) return rc;
     return launch_kernel(delta_bwd_kernel<T, C, Reg::NW, PRO>, dim3((unsigned)(B * H)), dim3(64 * Reg::NW), Reg::smem, st,
                          (const T *)q, (const T *)k, (const T *)v, (const T *)beta, done, done_dtype,
-                         (const float *)S_chk, (const T *)Tm_chk, (const T *)U_chk, (const float *)S_last, (const T *)dout,
-                         (const float *)dS_last, (T *)dq,
+                         (const T *)S_chk, (const T *)Tm_chk, (const T *)dout, (const float *)dS_last, (T *)dq,
                          (T *)dk_out, (T *)dv_out, (T *)dbeta, (float *)dS0, (int)T_, (int)H);
 }
 
 template <bool PRO>
 int delta_bwd_entry(void *stream, const void *q, const void *k, const void *v, const void *beta, const void *done,
-                    const void *S_chk, const void *Tm_chk, const void *U_chk, const void *S_last, const void *dout,
-                    const void *dS_last, void *dq, void *dk_out, void *dv_out, void *dbeta, void *dS0, int64_t B, int64_t T, int64_t H,
+                    const void *S_chk, const void *Tm_chk, const void *dout, const void *dS_last, void *dq,
+                    void *dk_out, void *dv_out, void *dbeta, void *dS0, int64_t B, int64_t T, int64_t H,
                     int64_t dk, int64_t dv, int dtype, int done_dtype)
 {
     const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
                              dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
-    if (!beta || !dbeta || !Tm_chk || !aligned(Tm_chk, 16) || !U_chk || !aligned(U_chk, 16) || !S_last || !aligned(S_last, 16))
-        return MRX_ERR_INVALID_ARG;
+    if (!beta || !dbeta || !Tm_chk || !aligned(Tm_chk, 16)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == MRX_BF16)
-        return launch_delta_bwd<__bf16, DELTA_BF16_CHUNK, PRO>(st, q, k, v, beta, done, done_dtype, S_chk, Tm_chk, U_chk,
-                                                               S_last, dout, dS_last, dq, dk_out, dv_out, dbeta, dS0, B, T, H);
-    return launch_delta_bwd<float, 32, PRO>(st, q, k, v, beta, done, done_dtype, S_chk, Tm_chk, U_chk, S_last, dout, dS_last, dq,
+        return launch_delta_bwd<__bf16, DELTA_BF16_CHUNK, PRO>(st, q, k, v, beta, done, done_dtype, S_chk, Tm_chk, dout,
+                                                               dS_last, dq, dk_out, dv_out, dbeta, dS0, B, T, H);
+    return launch_delta_bwd<float, 32, PRO>(st, q, k, v, beta, done, done_dtype, S_chk, Tm_chk, dout, dS_last, dq,
                                             dk_out, dv_out, dbeta, dS0, B, T, H);
 }
 
@@ -1176,22 +1153,22 @@ int delta_bwd_entry(void *stream, const void *q, const void *k, const void *v, c
 
 extern "C" int mrx_delta_rule_bwd(void *stream, const void *q, const void *k, const void *v,
                                   const void *beta, const void *done, const void *S_chk,
-                                  const void *Tm_chk, const void *U_chk, const float *S_last, const void *dout,
-                                  const void *dS_last, void *dq, void *dk_out, void *dv_out, void *dbeta, void *dS0,
-                                  int64_t B, int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
+                                  const void *Tm_chk, const void *dout, const void *dS_last, void *dq,
+                                  void *dk_out, void *dv_out, void *dbeta, void *dS0, int64_t B,
+                                  int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                                   int done_dtype)
 {
-    return delta_bwd_entry<false>(stream, q, k, v, beta, done, S_chk, Tm_chk, U_chk, S_last, dout, dS_last, dq, dk_out, dv_out,
+    return delta_bwd_entry<false>(stream, q, k, v, beta, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out,
                                   dbeta, dS0, B, T, H, dk, dv, dtype, done_dtype);
 }
 
 extern "C" int mrx_deltanet_bwd(void *stream, const void *q, const void *k, const void *v,
                                 const void *beta_raw, const void *done, const void *S_chk,
-                                const void *Tm_chk, const void *U_chk, const float *S_last, const void *dout,
-                                const void *dS_last, void *dq, void *dk_out, void *dv_out, void *dbeta_raw, void *dS0,
-                                int64_t B, int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
+                                const void *Tm_chk, const void *dout, const void *dS_last, void *dq,
+                                void *dk_out, void *dv_out, void *dbeta_raw, void *dS0, int64_t B,
+                                int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                                 int done_dtype)
 {
-    return delta_bwd_entry<true>(stream, q, k, v, beta_raw, done, S_chk, Tm_chk, U_chk, S_last, dout, dS_last, dq, dk_out, dv_out,
+    return delta_bwd_entry<true>(stream, q, k, v, beta_raw, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out,
                                  dbeta_raw, dS0, B, T, H, dk, dv, dtype, done_dtype);
 }

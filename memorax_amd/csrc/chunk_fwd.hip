@@ -70,7 +70,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                  const T *__restrict__ beta, const float *__restrict__ glog,
                  const void *__restrict__ done, int done_f32,
                  const float *__restrict__ S0, T *__restrict__ o, float *__restrict__ S_last,
-                 void *__restrict__ S_chk, T *__restrict__ Tm_chk, T *__restrict__ U_chk, int Tlen, int H, NormArgs na)
+                 void *__restrict__ S_chk, T *__restrict__ Tm_chk, int Tlen, int H, NormArgs na)
 {
     static_assert(!(DELTA && GATED), "the gated variant is linear attention with a decay");
     static_assert(!NORM || (!DELTA && !GATED), "the normalised read-out belongs to plain linear attention");
@@ -205,19 +205,10 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     // running element offsets of this thread's stores, advanced by one chunk per iteration
     unsigned long long pend_dmask = 0ull;  // the unit whose output waits in sO
     int pend_nres = 0, pend_pass = 0, pend_t0 = -1;
-    typename IO::Regs hu;  // delta rule: this thread's 16 bytes of the unit's U' rows, on their way to U_chk
     auto flush_o = [&]() {  // call after a barrier that follows the writes to sO
         if (pend_t0 >= 0) {
             auto keep = [&](int r) { return pend_nres == 0 || episode_of(pend_dmask, r) == pend_pass; };
             tile_rows_to_global<T, C, NTHR>(sO, LDD, o + base + (int64_t)pend_t0 * rs, rs, pend_t0, Tlen, tid, keep);
-            if (DELTA && U_chk) {
-#pragma unroll
-                for (int p = 0; p < IO::PASSES; ++p) {
-                    const int r = IO::row_of(tid, p);
-                    if ((IO::FULL || r < C) && pend_t0 + r < Tlen && keep(r))
-                        *reinterpret_cast<typename IO::F *>(U_chk + base + (int64_t)(pend_t0 + r) * rs + (tid % IO::SEGS) * IO::KP) = hu.v[p];
-                }
-            }
         }
         pend_t0 = -1;
     };
@@ -315,15 +306,17 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             // 32 bytes per instruction): the output of the previous unit, parked in sO at its end, and
             // the state checkpoint from the copy of S that has just been staged.
             flush_o();
-            // The backward call walks the state back from chunk to chunk in fp32, starting from S_last
-            // (S_c = S_{c+1} - U'_c^T K_c: the update it can undo from U' -- V for linear attention -- and
-            // K), so a checkpoint is written only where that walk cannot pass: for a chunk with resets,
-            // whose entering state the state that leaves it does not determine.  Those are written in fp32
-            // from the accumulators (rare, and the walk carries their rounding to the chunks before).  The
-            // decayed update of the gated variant is not undone (it would divide by the decay): there every
-            // chunk is written, in the I/O type, from the copy of S that has just been staged.
-            if (S_chk && pass == 0 && (GATED || nres != 0)) {
-                if (GATED) {
+            // Plain and normalised linear attention: the backward call walks the state back from chunk to
+            // chunk in fp32, starting from S_last (S_c = S_{c+1} - V_c^T K_c undoes a chunk's update), so a
+            // checkpoint is written only where that walk cannot pass: for a chunk with resets, whose entering
+            // state the state that leaves it does not determine.  Those are written in fp32 from the
+            // accumulators (rare; the walk carries their rounding to the chunks before).  The decayed update
+            // of the gated variant is not undone (it would divide by the decay), and for the delta rule the
+            // walk needs U' as a residual and an extra product, which measured slower than reading the
+            // states: there every chunk is written, in the I/O type, from the copy of S just staged.
+            constexpr bool DENSE_CHK = GATED || DELTA;
+            if (S_chk && pass == 0 && (DENSE_CHK || nres != 0)) {
+                if (DENSE_CHK) {
                     using IOS = TileIO<T, HD, NTHR>;
 #pragma unroll
                     for (int p = 0; p < IOS::PASSES; ++p) {
@@ -425,16 +418,6 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 }
             }
             sync_lds();
-            // residual for the backward call: the rows of U' of this pass's episode, taken row-wise from the
-            // tile now and written with the unit's output, once the next unit has been staged (a store
-            // issued here would still be in flight at the wait for the prefetched loads)
-            if (DELTA && U_chk) {
-#pragma unroll
-                for (int p = 0; p < IO::PASSES; ++p) {
-                    const int r = IO::row_of(tid, p);
-                    if (IO::FULL || r < C) hu.v[p] = *reinterpret_cast<const typename IO::F *>(sU + r * LDD + (tid % IO::SEGS) * IO::KP);
-                }
-            }
             // ---- O^T[dv][i] = sum_dk S[dv][dk] Q[i][dk] + sum_j U'[j][dv] Aqk[i][j] ; store O -------
             if (!DELTA && pre) { prefetch_part(2); prefetch_part(3); }
             f32x4 Oacc[TMO::TPW];
@@ -560,8 +543,7 @@ template <typename T, int C, bool DELTA, bool FMAP, bool GATED = false, bool NOR
           bool TMIN = false>
 int launch(hipStream_t st, const void *q, const void *k, const void *v, const void *beta,
            const void *done, int done_f32, const void *S0, void *o, void *S_last, void *S_chk,
-           void *Tm_chk, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr, NormArgs na = NormArgs{},
-           void *U_chk = nullptr)
+           void *Tm_chk, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr, NormArgs na = NormArgs{})
 {
     using Reg = FwdReg<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN>;
     (void)&Reg::reg;  // the kernel is on the list mrx_init() walks
@@ -569,7 +551,7 @@ int launch(hipStream_t st, const void *q, const void *k, const void *v, const vo
     return launch_kernel(chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN>, dim3((unsigned)(B * H)),
                          dim3(NTHR), Reg::smem, st, (const T *)q, (const T *)k, (const T *)v, (const T *)beta,
                          (const float *)glog, done, done_f32, (const float *)S0, (T *)o, (float *)S_last, S_chk,
-                         (T *)Tm_chk, (T *)U_chk, (int)Tlen, (int)H, na);
+                         (T *)Tm_chk, (int)Tlen, (int)H, na);
 }
 
 int check_common(const void *q, const void *k, const void *v, const void *done, const void *o,
@@ -600,8 +582,8 @@ int check_common(const void *q, const void *k, const void *v, const void *done, 
 // inverse per episode, the chunk-parallel kernel does that off the sequential path).
 template <bool PRO>
 int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void *v, const void *beta, const void *done,
-                       int done_dtype, const void *S0, void *o, void *S_last, void *S_chk, void *Tm_chk, void *U_chk,
-                       int64_t B, int64_t T, int64_t H, int dtype, int factor_path)
+                       int done_dtype, const void *S0, void *o, void *S_last, void *S_chk, void *Tm_chk, int64_t B,
+                       int64_t T, int64_t H, int dtype, int factor_path)
 {
     static_assert(DELTA_BF16_CHUNK == 32, "delta_tm_kernel is written for 32-row chunks");
     int cus = 0;
@@ -613,16 +595,15 @@ int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void 
         if (rc != MRX_OK) return rc;
         if (dtype == MRX_BF16)
             return launch<__bf16, 32, true, false, false, false, PRO, true>(st, q, k, v, beta, done, done_dtype, S0, o,
-                                                                           S_last, S_chk, Tm_chk, B, T, H, nullptr,
-                                                                           NormArgs{}, U_chk);
+                                                                           S_last, S_chk, Tm_chk, B, T, H);
         return launch<float, 32, true, false, false, false, PRO, true>(st, q, k, v, beta, done, done_dtype, S0, o, S_last,
-                                                                       S_chk, Tm_chk, B, T, H, nullptr, NormArgs{}, U_chk);
+                                                                       S_chk, Tm_chk, B, T, H);
     }
     if (dtype == MRX_BF16)
         return launch<__bf16, 32, true, false, false, false, PRO, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last,
-                                                                        S_chk, Tm_chk, B, T, H, nullptr, NormArgs{}, U_chk);
+                                                                        S_chk, Tm_chk, B, T, H);
     return launch<float, 32, true, false, false, false, PRO, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last,
-                                                                    S_chk, Tm_chk, B, T, H, nullptr, NormArgs{}, U_chk);
+                                                                    S_chk, Tm_chk, B, T, H);
 }
 
 bool factor_path_ok(int f) { return f == MRX_FACTORS_AUTO || f == MRX_FACTORS_PARALLEL || f == MRX_FACTORS_INLINE; }
@@ -668,16 +649,15 @@ extern "C" int mrx_linear_attn_fwd(void *stream, const void *q, const void *k, c
 
 extern "C" int mrx_delta_rule_fwd(void *stream, const void *q, const void *k, const void *v,
                                   const void *beta, const void *done, const void *S0, void *o,
-                                  void *S_last, void *S_chk, void *Tm_chk, void *U_chk, int64_t B, int64_t T,
+                                  void *S_last, void *S_chk, void *Tm_chk, int64_t B, int64_t T,
                                   int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype, int factor_path)
 {
     const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
-    if (!beta || !aligned(Tm_chk, 16) || !aligned(U_chk, 16) || !factor_path_ok(factor_path)) return MRX_ERR_INVALID_ARG;
-    if (S_chk && !U_chk) return MRX_ERR_INVALID_ARG;  // the state checkpoints are sparse: of no use without U'
+    if (!beta || !aligned(Tm_chk, 16) || !factor_path_ok(factor_path)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
-    return delta_fwd_dispatch<false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, U_chk, B, T, H,
-                                     dtype, factor_path);
+    return delta_fwd_dispatch<false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H, dtype,
+                                     factor_path);
 }
 
 extern "C" int mrx_delta_rule_fwd_noalloc(void *stream, const void *q, const void *k, const void *v,
@@ -695,8 +675,8 @@ extern "C" int mrx_delta_rule_fwd_noalloc(void *stream, const void *q, const voi
     void *factors = g_scratch_ptr[dev];  // this device's copy of the array, resolved at set-up
     if (!factors) return MRX_ERR_LAUNCH;
     hipStream_t st = (hipStream_t)stream;
-    return delta_fwd_dispatch<false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, nullptr, factors, nullptr, B, T, H,
-                                     dtype, MRX_FACTORS_PARALLEL);
+    return delta_fwd_dispatch<false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, nullptr, factors, B, T, H, dtype,
+                                     MRX_FACTORS_PARALLEL);
 }
 
 extern "C" int mrx_gated_linear_attn_fwd(void *stream, const void *q, const void *k, const void *v,
@@ -741,14 +721,13 @@ extern "C" int mrx_linear_attn_norm_fwd(void *stream, const void *q, const void 
 
 extern "C" int mrx_deltanet_fwd(void *stream, const void *q, const void *k, const void *v,
                                 const void *beta_raw, const void *done, const void *S0, void *o,
-                                void *S_last, void *S_chk, void *Tm_chk, void *U_chk, int64_t B, int64_t T,
+                                void *S_last, void *S_chk, void *Tm_chk, int64_t B, int64_t T,
                                 int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype, int factor_path)
 {
     const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
-    if (!beta_raw || !aligned(Tm_chk, 16) || !aligned(U_chk, 16) || !factor_path_ok(factor_path)) return MRX_ERR_INVALID_ARG;
-    if (S_chk && !U_chk) return MRX_ERR_INVALID_ARG;
+    if (!beta_raw || !aligned(Tm_chk, 16) || !factor_path_ok(factor_path)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
-    return delta_fwd_dispatch<true>(st, q, k, v, beta_raw, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, U_chk, B, T, H,
-                                    dtype, factor_path);
+    return delta_fwd_dispatch<true>(st, q, k, v, beta_raw, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H, dtype,
+                                    factor_path);
 }

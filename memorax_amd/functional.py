@@ -315,10 +315,10 @@ class _DeltaRule(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, do, dS_last):
-        q, k, v, beta, S_chk, Tm_chk, U_chk, S_last = ctx.saved_tensors
+        q, k, v, beta, S_chk, Tm_chk = ctx.saved_tensors
         do = torch.zeros_like(v) if do is None else do.contiguous()
         dS_last = None if dS_last is None else dS_last.contiguous().float()
-        dq, dk, dv, db, dS0 = K.delta_rule_bwd(q, k, v, beta, ctx.done, (S_chk, Tm_chk, U_chk, S_last), do, dS_last,
+        dq, dk, dv, db, dS0 = K.delta_rule_bwd(q, k, v, beta, ctx.done, (S_chk, Tm_chk), do, dS_last,
                                                want_dS0=ctx.has_S0, prologue=ctx.prologue)
         return dq, dk, dv, db, None, (dS0 if ctx.has_S0 else None), None
 

@@ -307,11 +307,9 @@ def delta_rule_fwd_noalloc(q, k, v, beta, done, S0=None, out=None):
 
 def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prologue=False, tm_scratch=None,
                    factor_path=None):
-    """Returns (o, S_last fp32, chk) where chk = (S_chk, Tm_chk, U_chk, S_last) is what the
-    backward call needs, or None: the states entering the chunks (float32; written only for chunks with
-    resets -- the backward call walks the state back from S_last through the others), the triangular
-    factors and U' (B,T,H,dv).  out = (o, S_last, S_chk, Tm_chk, U_chk, ...) reuses buffers of an
-    earlier call with the same shapes instead of allocating.  prologue=True: k is L2-normalised and
+    """Returns (o, S_last fp32, chk) where chk = (S_chk, Tm_chk) are the residuals the
+    backward call needs, or None.  out = (o, S_last, S_chk, Tm_chk) reuses buffers of an earlier
+    call with the same shapes instead of allocating.  prologue=True: k is L2-normalised and
     beta = sigmoid(beta) inside the kernel (mrx_deltanet_fwd).
     tm_scratch (only without residuals): give the library a buffer for the triangular factors
     anyway, which lets it compute them chunk-parallel while the device is not full.  None: when
@@ -323,22 +321,20 @@ def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prolog
     _chk(S0, "S0", torch.float32, (B, H, dv, dk))
     done, dd = _done(done, B, T)
     if out is not None:
-        o, S_last, S_chk, Tm_chk, U_chk = out[:5]
+        o, S_last, S_chk, Tm_chk = out
         C, NC = chunk_size(dt, True), _n_chunks(T, dt, True)
         _chk(o, "out o", dt, (B, T, H, dv))
         _chk(S_last, "out S_last", torch.float32, (B, H, dv, dk))
-        _chk(S_chk, "out S_chk", torch.float32, (B, H, NC, dv, dk))
+        _chk(S_chk, "out S_chk", dt, (B, H, NC, dv, dk))
         _chk(Tm_chk, "out Tm_chk", dt, (B, H, NC, C, C))
-        _chk(U_chk, "out U_chk", dt, (B, T, H, dv))
         save_chk = S_chk is not None
     else:
         o = torch.empty_like(v)
         S_last = torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
-        S_chk = Tm_chk = U_chk = None
+        S_chk = Tm_chk = None
         if save_chk:
             C, NC = chunk_size(dt, True), _n_chunks(T, dt, True)
-            S_chk = torch.empty((B, H, NC, dv, dk), dtype=torch.float32, device=q.device)
-            U_chk = torch.empty_like(v)
+            S_chk = torch.empty((B, H, NC, dv, dk), dtype=dt, device=q.device)
             Tm_chk = torch.empty((B, H, NC, C, C), dtype=dt, device=q.device)
         else:
             if tm_scratch is None:
@@ -348,26 +344,24 @@ def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prolog
                 Tm_chk = torch.empty((B, H, NC, C, C), dtype=dt, device=q.device)
     name = "mrx_deltanet_fwd" if prologue else "mrx_delta_rule_fwd"
     st = getattr(lib, name)(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done),
-                            _ptr(S0), _ptr(o), _ptr(S_last), _ptr(S_chk), _ptr(Tm_chk), _ptr(U_chk), B, T, H,
+                            _ptr(S0), _ptr(o), _ptr(S_last), _ptr(S_chk), _ptr(Tm_chk), B, T, H,
                             dk, dv, _DT[dt], dd, _FACTORS[factor_path])
     _lib.check(st, name)
-    return o, S_last, ((S_chk, Tm_chk, U_chk, S_last) if save_chk else None)
+    return o, S_last, ((S_chk, Tm_chk) if save_chk else None)
 
 
 def delta_rule_bwd(q, k, v, beta, done, chk, do, dS_last=None, want_dS0=True, out=None, prologue=False):
-    """chk = (S_chk, Tm_chk, U_chk, S_last) from delta_rule_fwd.  Returns (dq, dk, dv, dbeta, dS0).
+    """chk = (S_chk, Tm_chk) from delta_rule_fwd.  Returns (dq, dk, dv, dbeta, dS0).
     out = (dq, dk, dv, dbeta, dS0) reuses buffers instead of allocating.  prologue=True pairs with
     delta_rule_fwd(prologue=True): k and beta are the raw projections and so are dk and dbeta."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
-    S_chk, Tm_chk, U_chk, S_last = chk
+    S_chk, Tm_chk = chk
     C = chunk_size(dt, True)
-    _chk(S_last, "S_last", torch.float32, (B, H, dv, dk))
-    _chk(U_chk, "U_chk", dt, (B, T, H, dv))
     _chk(Tm_chk, "Tm_chk", dt, (B, H, _n_chunks(T, dt, True), C, C))
     _chk(beta, "beta", dt, (B, T, H))
     _chk(do, "do", dt, (B, T, H, dv))
-    _chk(S_chk, "S_chk", torch.float32, (B, H, _n_chunks(T, dt, True), dv, dk))
+    _chk(S_chk, "S_chk", dt, (B, H, _n_chunks(T, dt, True), dv, dk))
     _chk(dS_last, "dS_last", torch.float32, (B, H, dv, dk))
     done, dd = _done(done, B, T)
     if out is not None:
@@ -382,8 +376,7 @@ def delta_rule_bwd(q, k, v, beta, done, chk, do, dS_last=None, want_dS0=True, ou
                if want_dS0 else None)
     name = "mrx_deltanet_bwd" if prologue else "mrx_delta_rule_bwd"
     st = getattr(lib, name)(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done),
-                            _ptr(S_chk), _ptr(Tm_chk), _ptr(U_chk), _ptr(S_last), _ptr(do), _ptr(dS_last), _ptr(dq),
-                            _ptr(dk_),
+                            _ptr(S_chk), _ptr(Tm_chk), _ptr(do), _ptr(dS_last), _ptr(dq), _ptr(dk_),
                             _ptr(dv_), _ptr(dbeta), _ptr(dS0), B, T, H, dk, dv, _DT[dt], dd)
     _lib.check(st, name)
     return dq, dk_, dv_, dbeta, dS0

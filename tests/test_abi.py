@@ -66,16 +66,10 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mrx_linear_scan_fwd(n, one, one, one, n, n, one, n, n, 0, 4, 4, 0, 0, 0) == -1
     assert lib.mrx_linear_scan_fwd(n, one, one, one, n, n, one, n, n, 2, 4, 4, 1, 0, 0) == -2  # bf16 scan
     assert lib.mrx_linear_attn_fwd(n, one, one, one, one, n, one, n, n, 1, 8, 1, 32, 64, 1, 0, 0) == -2  # dk != 64
-    assert lib.mrx_delta_rule_bwd(n, one, one, one, one, one, one, n, one, one, one, n, one, one, one, one, n,
+    assert lib.mrx_delta_rule_bwd(n, one, one, one, one, one, one, n, one, n, one, one, one, one, n,
                                   1, 8, 1, 64, 64, 0, 0) == -1  # residual Tm_chk missing
-    assert lib.mrx_delta_rule_bwd(n, one, one, one, one, one, one, one, n, one, one, n, one, one, one, one, n,
-                                  1, 8, 1, 64, 64, 0, 0) == -1  # residual U_chk missing
-    assert lib.mrx_delta_rule_bwd(n, one, one, one, one, one, one, one, one, n, one, n, one, one, one, one, n,
-                                  1, 8, 1, 64, 64, 0, 0) == -1  # S_last, where the walk back starts, missing
     assert lib.mrx_linear_attn_bwd(n, one, one, one, one, one, n, one, n, one, one, one, n,
                                    1, 8, 1, 64, 64, 0, 0, 0) == -1  # S_last missing
-    assert lib.mrx_delta_rule_fwd(n, one, one, one, one, one, n, one, n, one, one, n,
-                                  1, 8, 1, 64, 64, 0, 0, 0) == -1  # state checkpoints asked without U_chk
 
 
 def test_host_layer_has_no_cpu_fallback():

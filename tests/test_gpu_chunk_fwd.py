@@ -145,13 +145,7 @@ def test_delta_rule_factor_paths_agree(dtype, prologue):
         assert torch.equal(o3, o4) and torch.equal(Sl3, Sl4)
         assert relerr(o3, o[sl].float().cpu().numpy()) <= tol and relerr(Sl3, Sl[sl].cpu().numpy()) <= tol
         assert relerr(chk3[1], chk[1][sl].float().cpu().numpy()) <= tol
-        assert relerr(chk3[2], chk[2][sl].float().cpu().numpy()) <= tol  # U'
-        # the state checkpoints are sparse: written where the chunk contains a reset
-        C = 32
-        pad = (-T) % C
-        dch = torch.nn.functional.pad(done[sl], (0, pad)).reshape(done[sl].shape[0], -1, C).any(-1)  # (b, NC)
-        for b_i, c_i in dch.nonzero().tolist():
-            assert relerr(chk3[0][b_i, :, c_i], chk[0][sl][b_i, :, c_i].cpu().numpy()) <= tol
+        assert relerr(chk3[0], chk[0][sl].float().cpu().numpy()) <= tol
         g3 = K.delta_rule_bwd(*args, chk3, do[sl].contiguous(), prologue=prologue)
         for a, b_ in zip(g3, grads):
             assert relerr(a, b_[sl].float().cpu().numpy()) <= tol

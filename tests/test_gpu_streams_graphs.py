@@ -46,7 +46,7 @@ def test_graph_replays_of_forward_and_backward():
     static = _delta_inputs(2)
     # first calls outside the capture: they size the buffers
     o, Sl, chk = K.delta_rule_fwd(static["q"], static["k"], static["v"], static["beta"], static["done"])
-    fwd_out = (o, Sl, *chk)
+    fwd_out = (o, Sl, chk[0], chk[1])
     bwd_out = K.delta_rule_bwd(static["q"], static["k"], static["v"], static["beta"], static["done"], chk,
                                static["do"], None, want_dS0=False)
     sa = torch.rand(4, 96, 128, device="cuda")
