@@ -145,9 +145,8 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     // Gated: every chunk has a checkpoint in the I/O type, staged row-wise.
     constexpr bool WALK = !GATED;
     constexpr int NSA = WALK ? TMS::TPW : 1;
-    f32x4 Sacc[NSA], rS32[NSA];
+    f32x4 Sacc[NSA];
     zero_acc<NSA>(Sacc);
-    zero_acc<NSA>(rS32);
     if (WALK) {
 #pragma unroll
         for (int j = 0; j < NSA; ++j) {
@@ -208,9 +207,11 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 for (int p = 0; p < IOS::PASSES; ++p)
                     rS.v[p] = *reinterpret_cast<const typename IOS::F *>(reinterpret_cast<const T *>(S_chk) + soff + p * IOS::RPP * HD);
             } else if (need_S) {
+                // straight into the state registers: the chunk at hand has formed its state (the first
+                // phase), and the next chunk, taking a checkpoint, does not walk back from it
 #pragma unroll
                 for (int j = 0; j < NSA; ++j)
-                    rS32[j] = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(S_chk) + soff +
+                    Sacc[j] = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(S_chk) + soff +
                                                                TMS::nt(w, j) * 16 * HD + TMS::mt(w, j) * 16);
             }
             rdone = 0u;
@@ -398,12 +399,10 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     if (c == NC - 1) {  // the one checkpoint no prefetch could know of
 #pragma unroll
                         for (int j = 0; j < NSA; ++j)
-                            rS32[j] = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(S_chk) +
+                            Sacc[j] = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(S_chk) +
                                                                        ((int64_t)bh * NC + c) * HD * HD + li * HD + 4 * lg +
                                                                        TMS::nt(w, j) * 16 * HD + TMS::mt(w, j) * 16);
-                    }
-#pragma unroll
-                    for (int j = 0; j < NSA; ++j) Sacc[j] = rS32[j];
+                    }  // else the prefetch of the chunk before has left the checkpoint in Sacc
                     store_acc<T, HD, HD, NW>(Sacc, sS, LDD, w, lane);
                 } else {
                     f32x4 zero[TMS::TPW];
