@@ -83,6 +83,9 @@ def main() -> int:
     ap.add_argument("--headline-only", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--ramp-ms", type=float, default=CLOCK_RAMP_S * 1e3,
                     help="untimed load before the warm-up steps (0 under a counter-collecting profiler)")
+    ap.add_argument("--lib", default=None,
+                    help="path of another build of the library to load (bench.py --all times the build with "
+                         "64-step delta-rule chunks through this, in a child process)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain elementwise kernel of known size (256 MiB read, 256 MiB "
                          "written) so that a rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE run can be scaled")
@@ -95,6 +98,9 @@ def main() -> int:
     import numpy as np
     import torch
 
+    if args.lib:
+        from memorax_amd import _lib
+        _lib.LIB_PATH = os.path.abspath(args.lib)
     from memorax_amd import kernels as K
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
@@ -111,6 +117,7 @@ def main() -> int:
             secondary["torso"].update(bench_torso_full(torch, K))
             secondary["step"] = bench_step(torch, K)
             secondary["rtrl"] = bench_rtrl(torch, K)
+            secondary["delta_rule_chunk64"] = bench_delta_chunk64()
         torch.cuda.empty_cache()
     if args.calibrate:
         cx = torch.zeros(64 * 1024 * 1024, device="cuda")  # 256 MiB fp32
@@ -216,6 +223,24 @@ def main() -> int:
         out["cpu_baseline"] = cpu_baseline(np, x, do_np)
     print(json.dumps(out))
     return 0
+
+
+def bench_delta_chunk64():
+    """The headline step on the build whose bf16 delta-rule kernels use 64-step chunks (the chunk length
+    BASELINE configuration 4 names; the library's default is 32), timed by this script in a child process
+    that loads memorax_amd/csrc/libmemorax_amd_c64.so.  That build has no chunk-parallel factor kernel:
+    the triangular inverse runs inside the sequential forward kernel."""
+    import subprocess
+    lib = os.path.join(ROOT, "memorax_amd", "csrc", "libmemorax_amd_c64.so")
+    if not os.path.exists(lib):
+        return {"skipped": "libmemorax_amd_c64.so not built"}
+    r = subprocess.run([sys.executable, os.path.abspath(__file__), "--lib", lib, "--headline-only", "--no-cpu"],
+                       capture_output=True, text=True, timeout=300)
+    if r.returncode != 0:
+        return {"failed": r.stderr[-300:]}
+    d = json.loads(r.stdout.strip().splitlines()[-1])
+    return {"workload": d["config"]["workload"], "ms_per_step": d["ms_per_step"], "tokens/s": d["value"],
+            "fwd_ms": d["kernels"]["delta_fwd"]["ms"], "bwd_ms": d["kernels"]["delta_bwd"]["ms"]}
 
 
 def _time_ms(torch, fn, iters=20, warm=3):

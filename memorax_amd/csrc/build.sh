@@ -1,24 +1,31 @@
 #!/usr/bin/env bash
-# Builds libmemorax_amd.so (HIP kernels + C ABI) for gfx950, in-tree.
+# Builds, in-tree and for gfx950:
+#   libmemorax_amd.so      the library (HIP kernels + C ABI)
+#   libmemorax_amd_c64.so  the same sources with the delta rule's bf16 kernels on 64-step chunks; only
+#                          bench.py --all loads it, to time that chunk length beside the default 32
 #   memorax_amd/csrc/build.sh
 set -euo pipefail
 cd "$(dirname "$0")"
 HIPCC=${HIPCC:-/opt/rocm/bin/hipcc}
 FLAGS=(--offload-arch=gfx950 -O3 -std=c++17 -fPIC -I../../include
        -Xclang -target-feature -Xclang -packed-fp32-ops -Wall -Wno-unused-function)
-objs=()
+SRCS=(api.hip scan.hip chunk_fwd.hip chunk_bwd.hip step.hip delta_tm.hip)
 pids=()
-for src in api.hip scan.hip chunk_fwd.hip chunk_bwd.hip step.hip delta_tm.hip; do
-    [ -f "$src" ] || continue
-    obj="${src%.hip}.o"
-    extra=()
-    # delta_tm.hip: MFMA results feed the vector ALU at once, keep them out of accumulation registers
-    [ "$src" = delta_tm.hip ] && extra=(-mllvm -amdgpu-mfma-vgpr-form)
-    "$HIPCC" "${FLAGS[@]}" "${extra[@]}" -c "$src" -o "$obj" 2> >(grep -v "packed-fp32-ops' is not a recognized feature" >&2) &
-    pids+=($!)
-    objs+=("$obj")
-done
+compile() {  # compile <object suffix> <extra flags...>
+    local suf=$1; shift
+    for src in "${SRCS[@]}"; do
+        local extra=()
+        # delta_tm.hip: MFMA results feed the vector ALU at once, keep them out of accumulation registers
+        [ "$src" = delta_tm.hip ] && extra=(-mllvm -amdgpu-mfma-vgpr-form)
+        "$HIPCC" "${FLAGS[@]}" "${extra[@]}" "$@" -c "$src" -o "${src%.hip}$suf.o" \
+            2> >(grep -v "packed-fp32-ops' is not a recognized feature" >&2) &
+        pids+=($!)
+    done
+}
+compile ""
+compile _c64 -DMRX_DELTA_BF16_CHUNK=64
 for p in "${pids[@]}"; do wait "$p"; done
-"$HIPCC" --offload-arch=gfx950 -shared -fPIC -o libmemorax_amd.so "${objs[@]}"
-rm -f "${objs[@]}"
-echo "built $(pwd)/libmemorax_amd.so"
+"$HIPCC" --offload-arch=gfx950 -shared -fPIC -o libmemorax_amd.so $(printf '%s.o ' "${SRCS[@]%.hip}")
+"$HIPCC" --offload-arch=gfx950 -shared -fPIC -o libmemorax_amd_c64.so $(printf '%s_c64.o ' "${SRCS[@]%.hip}")
+rm -f ./*.o
+echo "built $(pwd)/libmemorax_amd.so and libmemorax_amd_c64.so"

@@ -585,12 +585,15 @@ int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void 
                        int done_dtype, const void *S0, void *o, void *S_last, void *S_chk, void *Tm_chk, int64_t B,
                        int64_t T, int64_t H, int dtype, int factor_path)
 {
-    static_assert(DELTA_BF16_CHUNK == 32, "delta_tm_kernel is written for 32-row chunks");
+    // delta_tm_kernel is written for 32-row chunks: a build with 64-row bf16 chunks (the measurement
+    // variant, MRX_DELTA_BF16_CHUNK=64) always inverts inside the sequential kernel
+    constexpr bool TM_KERNEL = DELTA_BF16_CHUNK == 32;
     int cus = 0;
     if (const int rc = prepare_device(&cus); rc != MRX_OK) return rc;
     const bool parallel = Tm_chk && factor_path != MRX_FACTORS_INLINE && T <= DELTA_TM_MAX_T &&
                           (factor_path == MRX_FACTORS_PARALLEL || B * H <= 2 * (int64_t)cus);
-    if (parallel) {
+    if (!TM_KERNEL && factor_path == MRX_FACTORS_PARALLEL) return MRX_ERR_UNSUPPORTED;
+    if constexpr (TM_KERNEL) if (parallel) {
         const int rc = launch_delta_tm(st, k, beta, done, done_dtype, Tm_chk, B, T, H, dtype, PRO);
         if (rc != MRX_OK) return rc;
         if (dtype == MRX_BF16)
@@ -600,8 +603,8 @@ int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void 
                                                                        S_chk, Tm_chk, B, T, H);
     }
     if (dtype == MRX_BF16)
-        return launch<__bf16, 32, true, false, false, false, PRO, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last,
-                                                                        S_chk, Tm_chk, B, T, H);
+        return launch<__bf16, DELTA_BF16_CHUNK, true, false, false, false, PRO, false>(st, q, k, v, beta, done, done_dtype, S0, o,
+                                                                                      S_last, S_chk, Tm_chk, B, T, H);
     return launch<float, 32, true, false, false, false, PRO, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last,
                                                                     S_chk, Tm_chk, B, T, H);
 }

@@ -126,3 +126,53 @@ def test_deltanet_poison_does_not_cross_episodes():
             a, b_ = a[:, keep], b_[:, keep]
         bad_at = (a != b_).nonzero()
         assert bad_at.numel() == 0, (name, bad_at[:4].tolist(), a[a != b_][:4].tolist(), b_[a != b_][:4].tolist())
+
+
+def test_chunk64_build_agrees_with_the_default_build():
+    """libmemorax_amd_c64.so (the delta rule's bf16 kernels on 64-step chunks, loaded only by
+    bench.py --all) computes the same function: forward and backward through its C ABI against the
+    default library on the same inputs, ragged length, resets, non-zero initial state."""
+    import ctypes
+    import os
+    from memorax_amd import _lib
+    from memorax_amd import kernels as K
+    path = os.path.join(os.path.dirname(_lib.LIB_PATH), "libmemorax_amd_c64.so")
+    if not os.path.exists(path):
+        pytest.skip("libmemorax_amd_c64.so not built")
+    lib = ctypes.CDLL(path)
+    for name in ("mrx_delta_rule_fwd", "mrx_delta_rule_bwd", "mrx_delta_chunk_size"):
+        res, args = _lib.SIGNATURES[name]
+        getattr(lib, name).restype, getattr(lib, name).argtypes = res, args
+    assert lib.mrx_delta_chunk_size(_lib.MRX_BF16) == 64
+    B, T, H = 3, 200, 2
+    bf = torch.bfloat16
+    g = torch.Generator(device="cuda").manual_seed(64)
+    q, k, v, do = (torch.randn((B, T, H, 64), device="cuda", generator=g).to(bf) for _ in range(4))
+    k = torch.nn.functional.normalize(k.float(), dim=-1).to(bf)
+    beta = torch.rand((B, T, H), device="cuda", generator=g).to(bf)
+    done = (torch.rand((B, T), device="cuda", generator=g) < 0.02).view(torch.uint8).contiguous()
+    S0 = torch.randn((B, H, 64, 64), device="cuda", generator=g) * 0.1
+    print("case chunk64 build", flush=True)
+    o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done, S0)
+    ref = (o, Sl) + tuple(K.delta_rule_bwd(q, k, v, beta, done, chk, do))
+    NC = (T + 63) // 64
+    p = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+    st = torch.cuda.current_stream().cuda_stream
+    o2, Sl2 = torch.empty_like(v), torch.empty_like(S0)
+    S_chk = torch.empty((B, H, NC, 64, 64), dtype=bf, device="cuda")
+    Tm_chk = torch.empty((B, H, NC, 64, 64), dtype=bf, device="cuda")
+    rc = lib.mrx_delta_rule_fwd(st, p(q), p(k), p(v), p(beta), p(done), p(S0), p(o2), p(Sl2), p(S_chk), p(Tm_chk),
+                                B, T, H, 64, 64, _lib.MRX_BF16, _lib.MRX_DONE_U8, _lib.MRX_FACTORS_AUTO)
+    assert rc == 0, rc
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    db, dS0 = torch.empty_like(beta), torch.empty_like(S0)
+    rc = lib.mrx_delta_rule_bwd(st, p(q), p(k), p(v), p(beta), p(done), p(S_chk), p(Tm_chk), p(do), None, p(dq), p(dk),
+                                p(dv), p(db), p(dS0), B, T, H, 64, 64, _lib.MRX_BF16, _lib.MRX_DONE_U8)
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    for name, a, b_ in zip(("o", "S_last", "dq", "dk", "dv", "dbeta", "dS0"), (o2, Sl2, dq, dk, dv, db, dS0), ref):
+        assert relerr(a, b_.float().cpu().numpy()) <= TOL_BF16, name
+    # the chunk-parallel factor kernel exists for 32-step chunks only
+    rc = lib.mrx_delta_rule_fwd(st, p(q), p(k), p(v), p(beta), p(done), p(S0), p(o2), p(Sl2), p(S_chk), p(Tm_chk),
+                                B, T, H, 64, 64, _lib.MRX_BF16, _lib.MRX_DONE_U8, _lib.MRX_FACTORS_PARALLEL)
+    assert rc == -2, rc
