@@ -647,9 +647,15 @@ struct ScanPlan {
 //    device short of waves (one vector lane per thread by then) take sixteen, which makes a
 //    sequence of up to 128 steps a single super-step: the kernel's time is then one trip to
 //    memory and back instead of one per super-step;
-//  - backward (three loads per step): the streaming kernel wins whenever the columns alone
-//    give >= 2048 waves; below that, the wave-split kernel.
-ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, bool al8, bool bwd)
+//  - backward (three loads per step) prefers wide vectors: the widest one that still gives 4096 waves
+//    with the time axis split over eight waves -- or, for one or two lanes per thread, sixteen --
+//    takes the wave-split kernel (512x1024x1024: 1.91 ms = 5.6 TB/s against 2.12 ms streaming;
+//    1024x128x256: 135 us either way; 256x128x256: 28 against 39 us; 64x512x512: 77 against 111 us);
+//    shapes too small for that fall to the rule of the forward pass, and otherwise the streaming
+//    kernel runs whenever the columns alone give >= 2048 waves.  With the MinGRU map inside (a
+//    fourth stream and the map's arithmetic per element) the eight-wave split loses to streaming at
+//    1024x128x256 (202 vs 165 us; level at the large shape), so that case keeps the rule it had.
+ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, bool al8, bool bwd, bool mg = false)
 {
     const int maxvec = (int)(16 / esize);
     int vec = 1;
@@ -659,6 +665,13 @@ ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, boo
         if (D % v == 0 && ok_al) { vec = v; break; }
     }
     auto ntiles = [&](int v) { return (D + 64 * (int64_t)v - 1) / (64 * (int64_t)v); };
+    if (bwd && !mg && esize == 4) {
+        for (int v = vec; v >= 1; v >>= 1) {
+            const int64_t cols = B * ntiles(v);
+            if (cols * 8 >= 4096 && T >= 8 * TS) return {v, 8, (int)ntiles(v), false};
+            if (v <= 2 && cols * 16 >= 4096 && T >= 16 * TS) return {v, 16, (int)ntiles(v), false};
+        }
+    }
     while (vec > 1 && B * ntiles(vec) < 2048) vec >>= 1;
     const int tiles = (int)ntiles(vec);
     const int64_t waves = B * tiles;
@@ -739,7 +752,7 @@ int launch_bwd(hipStream_t st, const void *a, const void *hx, const void *h, con
                       aligned(g_last, 16) && aligned(da, 16) && aligned(db, 16) && aligned(dh0, 16);
     const bool al8 = aligned(a, 8) && aligned(hx, 8) && aligned(h, 8) && aligned(g, 8) && aligned(h0, 8) &&
                      aligned(g_last, 8) && aligned(da, 8) && aligned(db, 8) && aligned(dh0, 8);
-    const ScanPlan pl = plan_scan(B, T, D, sizeof(E), al16, al8, true);
+    const ScanPlan pl = plan_scan(B, T, D, sizeof(E), al16, al8, true, MG);
     int rc = MRX_ERR_LAUNCH;
     if (pl.stream) {
         const int64_t cpr = D / pl.vec;
@@ -755,9 +768,9 @@ int launch_bwd(hipStream_t st, const void *a, const void *hx, const void *h, con
         const size_t smem = scan_smem(pl.nw, sizeof(E) * pl.vec);
         vec_switch<E>(pl.vec, [&](auto vc) {
             constexpr int VEC = decltype(vc)::value;
-            if constexpr (VEC == 1) {
+            if constexpr (VEC == 1 || (VEC == 2 && sizeof(E) == 4 && !MG)) {
                 if (pl.nw == 16) {
-                    rc = launch_kernel((diag_scan_bwd_kernel<E, 1, MG, 16>), grid, block, smem, st, (const E *)a,
+                    rc = launch_kernel((diag_scan_bwd_kernel<E, VEC, MG, 16>), grid, block, smem, st, (const E *)a,
                                        (const E *)hx, (const E *)h, done, done_f32, (const E *)h0, (const E *)g,
                                        (const E *)g_last, (E *)da, (E *)db, (E *)dh0, (int)T, D, pl.tiles,
                                        pl.nw, a_ti);
