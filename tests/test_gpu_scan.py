@@ -22,7 +22,8 @@ def dev(x):
 SHAPES = [
     (32, 128, 256),   # benchmark configuration 1 (time split over waves)
     (1, 1, 1), (2, 1, 64), (3, 7, 5), (2, 9, 130), (5, 200, 64), (4, 300, 258),
-    (64, 64, 1024),   # wide: vectorised, no time split
+    (64, 64, 1024),   # wide: vectorised, no time split (backward: two lanes per thread, eight waves)
+    (32, 160, 1024),  # backward: two lanes per thread, time split over sixteen waves, ragged second super-step
     (2, 1000, 8),
 ]
 
