@@ -460,26 +460,33 @@ def bench_step(torch, K):
 
 def bench_torso_kernels(torch, K):
     """Configuration 5 (configs[4]), the sequence kernels of one update: 4 blocks x (DeltaNet H=4, d=64
-    forward + backward, diagonal recurrence forward + backward) over B=1024 envs x T=128, done p=0.01."""
+    forward + backward, diagonal recurrence forward + backward) over B=1024 envs x T=128, done p=0.01.
+    The DeltaNet cell calls the kernels with its prologue inside (key normalisation and gate sigmoid on
+    the raw projections, gradients taken back through them): that is the figure reported; the plain
+    delta rule on ready-made unit keys and gates is timed beside it."""
     B, T, Fe, H, d = 1024, 128, 256, 4, 64
     bf = torch.bfloat16
     done = torch.rand(B, T, device="cuda") < 0.01
-    q, k, v = (torch.randn(B, T, H, d, device="cuda").to(bf) for _ in range(3))
-    k = torch.nn.functional.normalize(k.float(), dim=-1).to(bf)
-    beta = torch.rand(B, T, H, device="cuda").to(bf)
+    q, k_raw, v = (torch.randn(B, T, H, d, device="cuda").to(bf) for _ in range(3))
+    k_unit = torch.nn.functional.normalize(k_raw.float(), dim=-1).to(bf)
+    b_raw = torch.randn(B, T, H, device="cuda").to(bf)
+    beta = torch.sigmoid(b_raw.float()).to(bf)
     do = torch.randn_like(v)
     z, hx, g = (torch.randn(B, T, Fe, device="cuda") for _ in range(3))
 
-    def kernels_only():
+    def kernels_only(prologue):
+        kk, bb = (k_raw, b_raw) if prologue else (k_unit, beta)
         for _ in range(4):
-            o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done)
-            K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False)
+            o, Sl, chk = K.delta_rule_fwd(q, kk, v, bb, done, prologue=prologue)
+            K.delta_rule_bwd(q, kk, v, bb, done, chk, do, None, want_dS0=False, prologue=prologue)
             h, _, _ = K.mingru_scan_fwd(z, hx, done, want_P=False)
             K.mingru_scan_bwd(z, hx, h, done, None, g)
-    ms_k = _time_ms(torch, kernels_only, iters=10, warm=3)
+    ms_k = _time_ms(torch, lambda: kernels_only(True), iters=10, warm=3)
+    ms_p = _time_ms(torch, lambda: kernels_only(False), iters=10, warm=3)
     by = 4 * ((BYTES_FWD + BYTES_BWD) * B * T * H + 36 * B * T * Fe)   # + MinGRU scan: 12 B fwd, 24 B bwd per element
     return {"sequence_kernels_ms": ms_k, "sequence_kernels_tokens/s": B * T / ms_k * 1e3,
-            "sequence_kernels_GB/s": by / ms_k / 1e6, "sequence_kernels_frac_hbm": by / ms_k / 1e6 / HBM_PEAK_GBS}
+            "sequence_kernels_GB/s": by / ms_k / 1e6, "sequence_kernels_frac_hbm": by / ms_k / 1e6 / HBM_PEAK_GBS,
+            "sequence_kernels_ms_plain_delta_rule": ms_p}
 
 
 def bench_torso_full(torch, K):

@@ -328,7 +328,11 @@ template <int SEGS> __device__ __forceinline__ float seg_sum(float x)
     return x;
 }
 
-__device__ __forceinline__ float sigmoidf(float x) { return 1.f / (1.f + __expf(-x)); }
+// The prologue's two scalar functions on the hardware reciprocal / reciprocal square root (1 ulp): a
+// full-precision division is some ten instructions, and these sit in every thread's staging path.
+__device__ __forceinline__ float sigmoidf(float x) { return __builtin_amdgcn_rcpf(1.f + __expf(-x)); }
+// 1 / max(|k|, 1e-12) from the row's sum of squares
+__device__ __forceinline__ float inv_norm(float ss) { return __builtin_amdgcn_rsqf(fmaxf(ss, 1e-24f)); }
 
 // Rows of an LDS tile [C][64] to a (B,T,H,64) array, 16 bytes per thread: eight (sixteen) threads
 // write one whole row, so a wave instruction covers full 128-byte lines -- against the four-feature

@@ -253,7 +253,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                         float ss = 0.f;
 #pragma unroll
                         for (int e = 0; e < IO::KP; ++e) ss += (float)fk.v[p][e] * (float)fk.v[p][e];
-                        kinv[p] = 1.f / fmaxf(sqrtf(seg_sum<IO::SEGS>(ss)), 1e-12f);
+                        kinv[p] = inv_norm(seg_sum<IO::SEGS>(ss));
                     }
                     IO::scale_rows(fk, kinv);
                 }

@@ -67,7 +67,7 @@ delta_tm_kernel(const T *__restrict__ k, const T *__restrict__ beta, const void 
             }
             float tot = tq[0] + tq[1];
             if (NKB == 4) tot += tq[2] + tq[3];
-            const float inv = 1.f / fmaxf(sqrtf(tot), 1e-12f);
+            const float inv = inv_norm(tot);
 #pragma unroll
             for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
