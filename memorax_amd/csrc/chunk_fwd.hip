@@ -102,7 +102,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lg = lane >> 4;
-    const int bh = blockIdx.x, b = bh / H, h = bh % H;
+    const int bh = sequence_of_block(blockIdx.x, gridDim.x, H), b = bh / H, h = bh % H;
     const int64_t rs = (int64_t)H * HD;  // row stride of q/k/v/o
     const int64_t base = ((int64_t)b * Tlen * H + h) * HD;
     const int NC = (Tlen + C - 1) / C;
