@@ -149,3 +149,37 @@ def test_autograd_functions():
     (o2 * dev(do)).sum().backward()
     ref = G.linear_attention_grads(x["q"] / 8, x["k"] / 8, x["v"] / 8, x["done"], None, do, None, "elu1")
     _check((tq2.grad, tk2.grad, tv2.grad), ref, TOL_F32, ("dq", "dk", "dv"))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_linear_attention_state_walk_back_over_a_long_sequence(dtype):
+    """The backward call recovers the state entering every chunk by undoing the chunks' updates from
+    S_last in fp32.  With the elu+1 feature map the state grows with every step, so the first chunks
+    hold a state hundreds of times smaller than the one the walk starts from: their dq (= dO S + ...)
+    is where an error of the walk would show.  4096 steps, resets in the middle (one chunk with two of
+    them), a non-zero initial state; dq is checked on the first chunks against their own scale."""
+    from memorax_amd import kernels as K
+    B, T, H = 2, 4096, 2
+    rng = np.random.default_rng(77)
+    q, k, v, do = ((rng.standard_normal((B, T, H, 64)) / 8).astype(np.float32) for _ in range(4))
+    S0 = (rng.standard_normal((B, H, 64, 64)) * 0.1).astype(np.float32)
+    done = np.zeros((B, T), bool)
+    done[0, [1500, 1510, 3000]] = True
+    done[1, 2047] = True
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    if dtype == "bf16":
+        q, k, v, do = (bf16_round(a) for a in (q, k, v, do))
+    print(f"case la walk-back dtype={dtype}", flush=True)
+    tq, tk, tv, tdo = (dev(a, td) for a in (q, k, v, do))
+    o, Sl, chk = K.linear_attn_fwd(tq, tk, tv, dev(done), dev(S0), 1)
+    got = K.linear_attn_bwd(tq, tk, tv, dev(done), chk, tdo, None, 1)
+    ref = clib.linear_attn_bwd(q, k, v, done, S0, do, None, 1)
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    for name, a, r in zip(("dq", "dk", "dv", "dS0"), got, ref):
+        assert relerr(a, r) <= tol, name
+    # the first 128 steps on their own scale (the state there is a thirtieth of the final one)
+    for name, a, r in zip(("dq", "dk", "dv"), got, ref):
+        assert relerr(a[:, :128], r[:, :128]) <= tol, name
+    # and the steps right after each reset, where the state has just restarted from zero
+    for b_, t_ in ((0, 1500), (0, 1510), (0, 3000), (1, 2047)):
+        assert relerr(got[0][b_, t_:t_ + 32], ref[0][b_, t_:t_ + 32]) <= tol, (b_, t_)
