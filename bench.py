@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--all]
 
 One "step" = one forward + backward pass of the DeltaNet delta rule over the
-synthetic batch of BASELINE configuration 4 (B=64, H=8, T=1024, d=64, bf16 inputs,
+synthetic batch of benchmark configuration 4 (B=64, H=8, T=1024, d=64, bf16 inputs,
 fp32 state, reset mask Bernoulli(0.002)); inputs are resident in HBM before the
 timed region.  Prints ONE JSON line.  Only one GPU is used: --gpus > 1 exits.
 
@@ -55,7 +55,7 @@ def linear_attn_flops(C, d=64):
 
 
 def synthetic(np, cfg, shape=None):
-    """Seeded fp32 inputs of BASELINE configuration cfg (1-based index into its list)."""
+    """Seeded fp32 inputs of benchmark configuration cfg (1-based index into its list)."""
     rng = np.random.default_rng(1000 + cfg)
     if cfg == 2:
         B, T, H, d = shape or (64, 256, 4, 64)
@@ -227,7 +227,7 @@ def main() -> int:
 
 def bench_delta_chunk64():
     """The headline step on the build whose bf16 delta-rule kernels use 64-step chunks (the chunk length
-    BASELINE configuration 4 names; the library's default is 32), timed by this script in a child process
+    benchmark configuration 4 names; the library's default is 32), timed by this script in a child process
     that loads memorax_amd/csrc/libmemorax_amd_c64.so.  That build has no chunk-parallel factor kernel:
     the triangular inverse runs inside the sequential forward kernel."""
     import subprocess

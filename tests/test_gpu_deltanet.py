@@ -56,7 +56,7 @@ def test_deltanet_fwd_bwd(shape, p, dtype):
 
 
 def test_deltanet_key_gradient_is_orthogonal_to_the_key_at_the_benchmark_shape():
-    """Size-independent property at BASELINE configuration 4's shape: the output is invariant to
+    """Size-independent property at benchmark configuration 4's shape: the output is invariant to
     the scale of each key, so dk . k = 0 row by row (up to bf16 rounding of the two factors)."""
     from memorax_amd import kernels as K
     B, T, H = 64, 1024, 8
