@@ -156,9 +156,9 @@ int mrx_linear_attn_bwd(void *stream, const void *q, const void *k,
  * (linear_attention.py:62-86):
  *     z_t = (done_t ? 0 : z_{t-1}) + phi(k_t) ;  den_t = max(phi(q_t) . z_t, eps)
  *     o_t = S_t phi(q_t) / den_t
- * z0 (nullable = 0), z_last (nullable): (B,H,dk) fp32.  den: (B,T,H) fp32, the clamped
- * denominators, and z_chk (nullable): (B,H,ceil(T/chunk),dk) fp32, z entering each
- * chunk, are residuals of the backward call together with o and S_chk. */
+ * z0 (nullable = 0), z_last (nullable): (B,H,dk) fp32.  den: (B,H,T) fp32 (contiguous in time per
+ * sequence: a residual, written and read back a chunk at a time), the clamped denominators, and
+ * z_chk (nullable): (B,H,ceil(T/chunk),dk) fp32, z entering each chunk, are residuals of the backward call together with o and S_chk. */
 int mrx_linear_attn_norm_fwd(void *stream, const void *q, const void *k,
                              const void *v, const void *done, const void *S0,
                              const float *z0, void *o, float *den, void *S_last,

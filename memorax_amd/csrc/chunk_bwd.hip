@@ -181,7 +181,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     int64_t doff = (int64_t)b * Tlen + tlast + lane;
     int64_t noff[IO::PASSES];  // den of the rows this thread stages
 #pragma unroll
-    for (int p = 0; p < IO::PASSES; ++p) noff[p] = ((int64_t)b * Tlen + tlast + IO::row_of(tid, p)) * H + h;
+    for (int p = 0; p < IO::PASSES; ++p) noff[p] = (int64_t)bh * Tlen + tlast + IO::row_of(tid, p);  // den: (B,H,T)
     int64_t zoff = ((int64_t)bh * NC + NC - 1) * HD + 4 * (tid & 15);
     int tpre = tlast;
     auto prefetch_part = [&](int part) {
@@ -226,7 +226,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 #pragma unroll
                 for (int p = 0; p < IO::PASSES; ++p) {
                     rden[p] = tpre + IO::row_of(tid, p) < Tlen ? na.den[noff[p]] : 1.f;
-                    noff[p] -= (int64_t)C * H;
+                    noff[p] -= C;
                 }
                 rz = *reinterpret_cast<const f32x4 *>(na.z_chk + zoff);
                 zoff -= HD;

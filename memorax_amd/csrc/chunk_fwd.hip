@@ -136,7 +136,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         }
     }
     const Frag ones = TT<T>::ones();
-    int64_t den_off = ((int64_t)b * Tlen + li) * H + h;  // den[t0 + li]
+    int64_t den_off = (int64_t)bh * Tlen + li;  // den[b][h][t0 + li]: contiguous in time per sequence
 
     // register prefetch of the next chunk (raw bits only: no arithmetic on in-flight loads)
     typename IO::Regs rq, rk, rv;
@@ -214,7 +214,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     };
     int64_t schk_off = (int64_t)bh * NC * HD * HD;                                   // S_chk[c]
     int64_t tmchk_off = (int64_t)bh * NC * C * C + (int64_t)tid * 4;                                  // row-major C x C
-    for (int c = 0; c < NC; ++c, schk_off += HD * HD, tmchk_off += C * C, den_off += (int64_t)C * H) {
+    for (int c = 0; c < NC; ++c, schk_off += HD * HD, tmchk_off += C * C, den_off += C) {
         const int t0 = c * C;
         const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
@@ -467,7 +467,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     const float den = fmaxf(dacc[j % TMO::NBW][0], na.eps);
                     Oacc[j] *= 1.f / den;
                     if (t0 + cc < Tlen && live(cc) && TMO::mt(w, j) == 0 && lg == 0)
-                        na.den[den_off + (int64_t)(TMO::nt(w, j) * 16) * H] = den;
+                        na.den[den_off + TMO::nt(w, j) * 16] = den;
                 }
             }
             store_acc<T, HD, C, NW>(Oacc, sO, LDD, w, lane);  // to memory once the next unit has been staged

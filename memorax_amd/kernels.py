@@ -223,7 +223,7 @@ def linear_attn_bwd(q, k, v, done, chk, do, dS_last=None, feature_map=0, want_dS
 
 def linear_attn_norm_fwd(q, k, v, done, S0=None, z0=None, feature_map=0, eps=1e-6, save_chk=True):
     """Linear attention with the normalised read-out fused.
-    Returns (o, den fp32 (B,T,H), S_last fp32, z_last fp32, (S_chk, z_chk, S_last) or None); S_chk as for
+    Returns (o, den fp32 (B,H,T), S_last fp32, z_last fp32, (S_chk, z_chk, S_last) or None); S_chk as for
     linear_attn_fwd."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
@@ -231,7 +231,7 @@ def linear_attn_norm_fwd(q, k, v, done, S0=None, z0=None, feature_map=0, eps=1e-
     _chk(z0, "z0", torch.float32, (B, H, dk))
     done, dd = _done(done, B, T)
     o = torch.empty_like(v)
-    den = torch.empty((B, T, H), dtype=torch.float32, device=q.device)
+    den = torch.empty((B, H, T), dtype=torch.float32, device=q.device)
     S_last = torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
     z_last = torch.empty((B, H, dk), dtype=torch.float32, device=q.device)
     nc = _n_chunks(T, dt)
@@ -254,7 +254,7 @@ def linear_attn_norm_bwd(q, k, v, done, chk, o, den, do, dS_last=None, dz_last=N
     _chk(S_last, "S_last", torch.float32, (B, H, dv, dk))
     _chk(do, "do", dt, (B, T, H, dv))
     _chk(o, "o", dt, (B, T, H, dv))
-    _chk(den, "den", torch.float32, (B, T, H))
+    _chk(den, "den", torch.float32, (B, H, T))
     _chk(S_chk, "S_chk", torch.float32, (B, H, nc, dv, dk))
     _chk(z_chk, "z_chk", torch.float32, (B, H, nc, dk))
     _chk(dS_last, "dS_last", torch.float32, (B, H, dv, dk))
