@@ -34,7 +34,7 @@ BYTES_FWD, BYTES_BWD = 514, 900
 # FETCH_SIZE and WRITE_SIZE runs scaled by a plain elementwise kernel of known size
 # (summary kept under profiles/).  The excess over the algorithmic bytes is the forward's
 # per-chunk residuals (state checkpoints and triangular factors) being read back.
-TRAFFIC_BWD_BYTES = 655.1e6
+TRAFFIC_BWD_BYTES = 640.1e6
 # Matrix-pipe busy fraction of delta_bwd_kernel from rocprofv3 --pmc (SQ_VALU_MFMA_BUSY_CYCLES over
 # SQ_BUSY_CYCLES per SIMD), same workload; summary and command under profiles/.
 MFMA_BUSY_BWD = 0.149
