@@ -375,6 +375,21 @@ def bench_linear_attention(torch, K, np, dev):
                                    "frac_hbm": 2816 * nth / ms / 1e6 / HBM_PEAK_GBS,
                                    "frac_mfma_f32": (ff + fb) * nth / (ms * 1e-3) / MFMA_F32_PEAK}
     del q, k, v, do
+    # a grid that does not fill the device (32 sequences of 4096 steps, bf16): one workgroup per sequence
+    # against the chunk-parallel pair the library's rule picks there
+    Bn, Tn, Hn = 8, 4096, 4
+    q, k, v, do = (torch.randn((Bn, Tn, Hn, 64), device="cuda").div_(8).to(torch.bfloat16) for _ in range(4))
+    dn = torch.zeros((Bn, Tn), dtype=torch.bool, device="cuda")
+    small = {}
+    for name, par in (("ms_one_workgroup_per_sequence", False), ("ms_chunk_parallel", True)):
+        def fs():
+            o, Sl, chk = K.linear_attn_fwd(q, k, v, dn, None, 0, chunk_parallel=par)
+            K.linear_attn_bwd(q, k, v, dn, chk, do, None, 0, want_dS0=False)
+        small[name] = _time_ms(torch, fs)
+    small["rule_picks_chunk_parallel"] = bool(K.linear_attn_chunk_parallel_pays(Bn, Tn, Hn, torch.bfloat16))
+    small["tokens/s"] = Bn * Tn / min(small["ms_one_workgroup_per_sequence"], small["ms_chunk_parallel"]) * 1e3
+    res["small_grid_bf16_8x4096x4x64"] = small
+    del q, k, v, do
     Bn, Tn, Hn = 256, 4096, 8   # configuration 3 at full size (11.8 GB of q, k, v, do, o, dq, dk, dv)
     q, k, v, do = (torch.randn((Bn, Tn, Hn, 64), device="cuda").div_(8).to(torch.bfloat16) for _ in range(4))
     dn = torch.zeros((Bn, Tn), dtype=torch.bool, device="cuda")

@@ -150,6 +150,33 @@ int mrx_linear_attn_bwd(void *stream, const void *q, const void *k,
                         int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                         int done_dtype, int feature_map);
 
+/* ---- the same function cut along time: one workgroup per chunk -------------------
+ * mrx_linear_attn_fwd / _bwd give every (batch, head) sequence one workgroup that walks its chunks
+ * in order; with fewer sequences than the device has room for, most of it idles behind that walk.
+ * The state of linear attention is additive (memoroid.py:60-91 scanning the operator of
+ * linear_attention.py:82-86), so the pair below first forms every chunk's own contribution to the
+ * state in parallel, sums those per sequence, and then treats every chunk of every sequence as an
+ * independent workgroup.  Same arguments, results and accuracy class as the pair above, except:
+ *   S_chk (required): (B,H,ceil(T/chunk),dv,dk) float32, dense: the forward call leaves the state
+ *     entering every chunk in it, and the backward call reads all of it (the two calls of a pair must
+ *     be of the same kind: the sequential backward call does not take these, and vice versa);
+ *   workspace (backward, required): (B,H,ceil(T/chunk),dv,dk) float32 scratch, overwritten;
+ *   S_last is not an input of the backward call.
+ * mrx_linear_attn_chunk_parallel_pays: 1 when the library's own rule (at most one sequence per two
+ * compute units of the current device and at least eight chunks each) prefers this pair, else 0. */
+int mrx_linear_attn_fwd_chunk_parallel(void *stream, const void *q, const void *k,
+                                       const void *v, const void *done, const void *S0,
+                                       void *o, void *S_last, float *S_chk, int64_t B,
+                                       int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
+                                       int done_dtype, int feature_map);
+int mrx_linear_attn_bwd_chunk_parallel(void *stream, const void *q, const void *k,
+                                       const void *v, const void *done, const float *S_chk,
+                                       const void *dout, const void *dS_last, void *dq,
+                                       void *dk_out, void *dv_out, void *dS0, float *workspace,
+                                       int64_t B, int64_t T, int64_t H, int64_t dk, int64_t dv,
+                                       int dtype, int done_dtype, int feature_map);
+int mrx_linear_attn_chunk_parallel_pays(int64_t B, int64_t T, int64_t H, int dtype);
+
 /* ---- linear attention with the normalised read-out fused ----------------------
  * Replaces, in addition to the above, LinearAttentionCell.read's denominator and
  * divide (linear_attention.py:107-110) and the z leaf of the carry

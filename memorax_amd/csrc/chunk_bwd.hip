@@ -18,6 +18,7 @@
 // the row index read it through transpose loads (KROW operands).  Gradients leave through dead
 // LDS tiles and are written to memory row-wise (tile_rows_to_global).
 #include "chunk_common.h"
+#include "la_states.h"
 
 
 namespace {
@@ -72,7 +73,11 @@ struct NormBwdArgs {
 // The gradient of the log-decays follows from edot_i = q_i . dq_i - k_i . dk_i (taken on the
 // feature-mapped q, k and their gradients): dg_t is the sum of edot over the rows i >= t of t's
 // episode (plus <S_last, dS_last> at the end); the kernel writes edot, the caller sums.
-template <typename T, int C, bool FMAP, bool GATED, bool NORM>
+// PAR (plain linear attention): one workgroup per chunk (grid.y = chunk).  Slot c of S_chk holds, in
+// fp32, the state entering chunk c and slot c of dS_last -- then a (B,H,NC,64,64) array -- the gradient
+// of the state leaving it (la_states.h); the workgroup forms the chunk's dQ, dK, dV from them and neither
+// walks the state nor accumulates its gradient.
+template <typename T, int C, bool FMAP, bool GATED, bool NORM, bool PAR = false>
 __global__ void __launch_bounds__(256, 2)
 la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
               const float *__restrict__ glog, const void *__restrict__ done, int done_f32,
@@ -81,6 +86,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
               float *__restrict__ dS0, int Tlen, int H, NormBwdArgs na)
 {
     static_assert(!(GATED && NORM), "the normalised read-out belongs to plain linear attention");
+    static_assert(!PAR || (!GATED && !NORM), "one workgroup per chunk: plain linear attention only");
     constexpr int NW = 4, NTHR = 64 * NW;
     using L = LaBwdSmem<T, C, GATED, NORM>;
     using Frag = typename TT<T>::frag;
@@ -112,6 +118,8 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     const int64_t rs = (int64_t)H * HD;
     const int64_t base = ((int64_t)b * Tlen * H + h) * HD;
     const int NC = (Tlen + C - 1) / C;
+    const int c_hi = PAR ? (int)blockIdx.y : NC - 1, c_lo = PAR ? c_hi : 0;  // the chunks this workgroup walks, downwards
+    const int64_t slot = PAR ? ((int64_t)bh * NC + c_hi) * HD : (int64_t)bh * HD;  // in rows of 64 floats
 
     using TMS = TileMap<HD, HD, NW>;
     using TMA = TileMap<C, C, NW>;
@@ -120,7 +128,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 #pragma unroll
     for (int j = 0; j < TMS::TPW; ++j) {
         const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
-        dSacc[j] = dS_last ? *reinterpret_cast<const f32x4 *>(dS_last + ((int64_t)bh * HD + dvv) * HD + dk0)
+        dSacc[j] = dS_last ? *reinterpret_cast<const f32x4 *>(dS_last + (slot + dvv) * HD + dk0)
                            : f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
@@ -151,7 +159,8 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 #pragma unroll
         for (int j = 0; j < NSA; ++j) {
             const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
-            Sacc[j] = *reinterpret_cast<const f32x4 *>(S_last + ((int64_t)bh * HD + dvv) * HD + dk0);
+            Sacc[j] = *reinterpret_cast<const f32x4 *>((PAR ? reinterpret_cast<const float *>(S_chk) : S_last) +
+                                                       (slot + dvv) * HD + dk0);
         }
     }
 
@@ -171,18 +180,18 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     // (64-bit adds instead of per-chunk index multiplications).  The prefetch is issued in parts
     // spread over the phases so that the address unit works beside LDS and MFMA work:
     // part 0: q, k; 1: v, dout; 2: S and the per-row scalars.
-    const int tlast = (NC - 1) * C;
+    const int tlast = c_hi * C;
     int64_t roff[IO::PASSES];
 #pragma unroll
     for (int p = 0; p < IO::PASSES; ++p)
         roff[p] = base + (int64_t)(tlast + IO::row_of(tid, p)) * rs + (tid % IO::SEGS) * IO::KP;
-    int64_t soff = ((int64_t)bh * NC + NC - 1) * HD * HD +
+    int64_t soff = ((int64_t)bh * NC + c_hi) * HD * HD +
                    (WALK ? li * HD + 4 * lg : (tid / IOS::SEGS) * HD + (tid % IOS::SEGS) * IOS::KP);
     int64_t doff = (int64_t)b * Tlen + tlast + lane;
     int64_t noff[IO::PASSES];  // den of the rows this thread stages
 #pragma unroll
     for (int p = 0; p < IO::PASSES; ++p) noff[p] = (int64_t)bh * Tlen + tlast + IO::row_of(tid, p);  // den: (B,H,T)
-    int64_t zoff = ((int64_t)bh * NC + NC - 1) * HD + 4 * (tid & 15);
+    int64_t zoff = ((int64_t)bh * NC + c_hi) * HD + 4 * (tid & 15);
     int tpre = tlast;
     auto prefetch_part = [&](int part) {
         typename IO::F z;
@@ -221,7 +230,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 rdone = done_raw(done, done_f32, doff);
                 if (GATED) rg = glog[doff * H + h];
             }
-            if (WALK && lane < C && tpre >= C) rdone2 = done_raw(done, done_f32, doff - C);
+            if (WALK && !PAR && lane < C && tpre >= C) rdone2 = done_raw(done, done_f32, doff - C);
             if (NORM) {
 #pragma unroll
                 for (int p = 0; p < IO::PASSES; ++p) {
@@ -272,12 +281,12 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             *reinterpret_cast<P4 *>(dst + (TMR::nt(w, j) * 16 + li) * LDD + TMR::mt(w, j) * 16 + 4 * lg) = h[j];
     };
 
-    for (int c = NC - 1; c >= 0; --c) {
+    for (int c = c_hi; c >= c_lo; --c) {
         const int t0 = c * C;
         const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
-        const bool ckpt = !WALK || nres != 0;  // the entering state comes from S_chk
-        if (WALK) need_S = __ballot(done_test(rdone2, done_f32) && lane < C) != 0ull;  // for the chunk prefetched during this one
+        const bool ckpt = PAR || !WALK || nres != 0;  // the entering state comes from S_chk
+        if (WALK && !PAR) need_S = __ballot(done_test(rdone2, done_f32) && lane < C) != 0ull;  // for the chunk prefetched during this one
         for (int pass = nres; pass >= 0; --pass) {
             auto live = [&](int r) { return nres == 0 || episode_of(dmask, r) == pass; };
             // gated: cumulative log-decay of this pass's episode (as in the forward kernel)
@@ -352,7 +361,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 }
             }
             sync_lds();
-            const bool pre = pass == 0 && c > 0;
+            const bool pre = pass == 0 && c > c_lo;
             if (pre) prefetch_part(0);
 
             // ---- Aqk[i][j] = q_i.k_j, dAqk[i][j] = do_i.v_j, both j <= i ------------------
@@ -396,7 +405,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     for (int j = 0; j < NSA; ++j) Sacc[j] -= acc[j];
                     store_acc<T, HD, HD, NW>(Sacc, sS, LDD, w, lane);
                 } else if (pass == 0) {
-                    if (c == NC - 1) {  // the one checkpoint no prefetch could know of
+                    if (!PAR && c == NC - 1) {  // the one checkpoint no prefetch could know of (PAR: loaded at the start)
 #pragma unroll
                         for (int j = 0; j < NSA; ++j)
                             Sacc[j] = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(S_chk) +
@@ -524,7 +533,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     for (int e = 0; e < TT<T>::KP; ++e) xq[e] = (T)((float)xq[e] * ea[e]);
                 }
             };
-            gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, sQ, LDD, sDO, LDD, w, lane, dz_q);
+            if (!PAR) gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, sQ, LDD, sDO, LDD, w, lane, dz_q);
             if (NORM && VN) {
 #pragma unroll
                 for (int mi = 0; mi < TMS::MBW; ++mi) {
@@ -552,7 +561,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
         }
     }
     flush_pending();  // the last pass ended with a barrier
-    if (dS0) {
+    if (dS0 && !PAR) {
 #pragma unroll
         for (int j = 0; j < TMS::TPW; ++j) {
             const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
@@ -1002,21 +1011,24 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     }
 }
 
-template <typename T, int C, bool FMAP, bool GATED, bool NORM> struct LaBwdReg {
+template <typename T, int C, bool FMAP, bool GATED, bool NORM, bool PAR> struct LaBwdReg {
     static constexpr int smem = LaBwdSmem<T, C, GATED, NORM>::total;
-    static inline KernelRegistrar reg{reinterpret_cast<const void *>(la_bwd_kernel<T, C, FMAP, GATED, NORM>), smem};
+    static inline KernelRegistrar reg{reinterpret_cast<const void *>(la_bwd_kernel<T, C, FMAP, GATED, NORM, PAR>), smem};
 };
 
-template <typename T, int C, bool FMAP, bool GATED = false, bool NORM = false>
+template <typename T, int C, bool FMAP, bool GATED = false, bool NORM = false, bool PAR = false>
 int launch_la(hipStream_t st, const void *q, const void *k, const void *v, const void *done,
               int done_f32, const void *S_chk, const void *S_last, const void *dout, const void *dS_last, void *dq,
               void *dk, void *dv, void *dS0, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr,
               void *edot = nullptr, NormBwdArgs na = NormBwdArgs{})
 {
-    using Reg = LaBwdReg<T, C, FMAP, GATED, NORM>;
+    using Reg = LaBwdReg<T, C, FMAP, GATED, NORM, PAR>;
     (void)&Reg::reg;  // the kernel is on the list mrx_init() walks
     if (const int rc = prepare_device(); rc != MRX_OK) return rc;
-    return launch_kernel(la_bwd_kernel<T, C, FMAP, GATED, NORM>, dim3((unsigned)(B * H)), dim3(256), Reg::smem, st,
+    const int64_t NC = (Tlen + C - 1) / C;
+    if (PAR && NC > 65535) return MRX_ERR_INVALID_ARG;
+    return launch_kernel(la_bwd_kernel<T, C, FMAP, GATED, NORM, PAR>, dim3((unsigned)(B * H), PAR ? (unsigned)NC : 1u),
+                         dim3(256), Reg::smem, st,
                          (const T *)q, (const T *)k, (const T *)v, (const float *)glog, done, done_f32,
                          S_chk, (const float *)S_last, (const T *)dout, (const float *)dS_last, (T *)dq, (T *)dk, (T *)dv,
                          (float *)edot, (float *)dS0, (int)Tlen, (int)H, na);
@@ -1058,6 +1070,35 @@ extern "C" int mrx_linear_attn_bwd(void *stream, const void *q, const void *k, c
 #define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, S_last, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H
     if (dtype == MRX_BF16) return fm ? launch_la<__bf16, LA_BF16_CHUNK, true>(MRX_ARGS) : launch_la<__bf16, LA_BF16_CHUNK, false>(MRX_ARGS);
     return fm ? launch_la<float, 32, true>(MRX_ARGS) : launch_la<float, 32, false>(MRX_ARGS);
+#undef MRX_ARGS
+}
+
+extern "C" int mrx_linear_attn_bwd_chunk_parallel(void *stream, const void *q, const void *k, const void *v,
+                                                  const void *done, const float *S_chk, const void *dout,
+                                                  const void *dS_last, void *dq, void *dk_out, void *dv_out,
+                                                  void *dS0, float *workspace, int64_t B, int64_t T, int64_t H,
+                                                  int64_t dk, int64_t dv, int dtype, int done_dtype, int feature_map)
+{
+    const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
+                             dv, dtype, done_dtype);
+    if (rc != MRX_OK) return rc;
+    if (!workspace || !aligned(workspace, 16)) return MRX_ERR_INVALID_ARG;
+    if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const bool fm = feature_map == MRX_FMAP_ELU1;
+    const int C = (int)mrx_chunk_size(dtype);
+    if ((T + C - 1) / C > 65535) return MRX_ERR_INVALID_ARG;
+    // per-chunk sums of do phi(q)^T -> gradients of the states leaving the chunks (and dS0) -> dQ, dK, dV
+    int rc2 = launch_la_chunk_states(st, q, dout, done, done_dtype, workspace, B, T, H, dtype, fm, true);
+    if (rc2 != MRX_OK) return rc2;
+    rc2 = launch_la_state_scan(st, workspace, (const float *)dS_last, (float *)dS0, done, done_dtype, B, T, H, C, true);
+    if (rc2 != MRX_OK) return rc2;
+#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, nullptr, dout, workspace, dq, dk_out, dv_out, nullptr, B, T, H
+    if (dtype == MRX_BF16)
+        return fm ? launch_la<__bf16, LA_BF16_CHUNK, true, false, false, true>(MRX_ARGS)
+                  : launch_la<__bf16, LA_BF16_CHUNK, false, false, false, true>(MRX_ARGS);
+    return fm ? launch_la<float, 32, true, false, false, true>(MRX_ARGS)
+              : launch_la<float, 32, false, false, false, true>(MRX_ARGS);
 #undef MRX_ARGS
 }
 

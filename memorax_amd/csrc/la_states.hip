@@ -1,0 +1,132 @@
+// The kernels declared in la_states.h.
+#include "la_states.h"
+
+#include "chunk_common.h"
+
+namespace mrx {
+
+namespace {
+
+// One workgroup = one chunk of one sequence: slot <- sum over the kept rows r of y_r phi(x_r)^T,
+// kept = the chunk's last episode (forward: what the chunk adds to the state that leaves it) or its
+// first episode (backward: what it adds to the gradient of the state that enters it).
+template <typename T, int C, bool FMAP, bool BWD>
+__global__ void __launch_bounds__(256)
+la_chunk_state_kernel(const T *__restrict__ x, const T *__restrict__ y, const void *__restrict__ done, int done_f32,
+                      float *__restrict__ slots, int Tlen, int H, int NC)
+{
+    constexpr int NW = 4, NTHR = 64 * NW, LDD = HD + pad_of<T>();
+    using IO = TileIO<T, C, NTHR>;
+    using TMS = TileMap<HD, HD, NW>;
+    __shared__ __align__(16) T sX[C * LDD];
+    __shared__ __align__(16) T sY[C * LDD];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15, lg = lane >> 4;
+    const int bh = blockIdx.x, c = blockIdx.y, b = bh / H, h = bh % H;
+    const int t0 = c * C;
+    const int64_t rs = (int64_t)H * HD;
+    const int64_t base = ((int64_t)b * Tlen * H + h) * HD;
+
+    typename IO::Regs rx, ry;
+    IO::load(rx, x + base, rs, t0, Tlen, tid);
+    IO::load(ry, y + base, rs, t0, Tlen, tid);
+    const bool dn = lane < C && t0 + lane < Tlen && done_at(done, done_f32, (int64_t)b * Tlen + t0 + lane);
+    const unsigned long long dmask = __ballot(dn);
+    const int nres = __popcll(dmask);
+    IO::template fmap<FMAP>(rx);
+    if (nres != 0) {  // rows of other episodes leave by select: what they hold must not meet a zero in a product
+        const int ep = BWD ? 0 : nres;
+        auto keep = [&](int r) { return episode_of(dmask, r) == ep; };
+        IO::mask_rows(rx, tid, keep);
+        IO::mask_rows(ry, tid, keep);
+    }
+    // rows past the end of the sequence: y is zero there, and phi(0) = 1 in x is finite
+    IO::to_lds(rx, sX, LDD, tid);
+    IO::to_lds(ry, sY, LDD, tid);
+    sync_lds();
+    f32x4 acc[TMS::TPW];  // S^T: m = dk, n = dv
+    zero_acc<TMS::TPW>(acc);
+    gemm<T, HD, HD, C, KROW, KROW, NW>(acc, sX, LDD, sY, LDD, w, lane);
+    float *slot = slots + ((int64_t)bh * NC + c) * (HD * HD);
+#pragma unroll
+    for (int j = 0; j < TMS::TPW; ++j) {
+        const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dv = TMS::nt(w, j) * 16 + li;
+        *reinterpret_cast<f32x4 *>(slot + dv * HD + dk0) = acc[j];
+    }
+}
+
+// grid (B * H, 4): each thread carries four of the 4096 state elements through the chunks.  The loads of
+// a group of four chunks are issued together; only the additions are sequential.
+__global__ void __launch_bounds__(256)
+la_state_scan_kernel(float *__restrict__ slots, const float *__restrict__ init, float *__restrict__ fin,
+                     const void *__restrict__ done, int done_f32, int Tlen, int H, int NC, int C, int backward)
+{
+    constexpr int Q = HD * HD / 4;  // f32x4 per state
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int bh = blockIdx.x, b = bh / H;
+    const int idx = blockIdx.y * 256 + tid;
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    f32x4 S = init ? reinterpret_cast<const f32x4 *>(init)[(int64_t)bh * Q + idx] : zero;
+    f32x4 *p = reinterpret_cast<f32x4 *>(slots) + (int64_t)bh * NC * Q + idx;
+    for (int s0 = 0; s0 < NC; s0 += 4) {
+        f32x4 t[4];
+        bool cut[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int s = s0 + u, c = backward ? NC - 1 - s : s;
+            t[u] = zero;
+            cut[u] = false;
+            if (s < NC) {  // uniform over the workgroup
+                t[u] = p[(int64_t)c * Q];
+                const int tt = c * C + lane;
+                cut[u] = __ballot(lane < C && tt < Tlen && done_at(done, done_f32, (int64_t)b * Tlen + tt)) != 0ull;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int s = s0 + u, c = backward ? NC - 1 - s : s;
+            if (s < NC) {
+                p[(int64_t)c * Q] = S;
+                S = cut[u] ? t[u] : S + t[u];
+            }
+        }
+    }
+    if (fin) reinterpret_cast<f32x4 *>(fin)[(int64_t)bh * Q + idx] = S;
+}
+
+template <typename T, int C>
+int launch_states(hipStream_t st, const void *x, const void *y, const void *done, int done_f32, float *slots, int64_t B,
+                  int64_t Tlen, int64_t H, bool fmap, bool backward)
+{
+    const int64_t NC = (Tlen + C - 1) / C;
+    if (B * H > 0x7fffffffLL || NC > 65535) return MRX_ERR_INVALID_ARG;
+    const dim3 grid((unsigned)(B * H), (unsigned)NC), block(256);
+#define MRX_LAUNCH(FM, BW)                                                                                             \
+    launch_kernel((la_chunk_state_kernel<T, C, FM, BW>), grid, block, 0, st, (const T *)x, (const T *)y, done, done_f32, \
+                  slots, (int)Tlen, (int)H, (int)NC)
+    if (fmap) return backward ? MRX_LAUNCH(true, true) : MRX_LAUNCH(true, false);
+    return backward ? MRX_LAUNCH(false, true) : MRX_LAUNCH(false, false);
+#undef MRX_LAUNCH
+}
+
+}  // namespace
+
+int launch_la_chunk_states(hipStream_t st, const void *x, const void *y, const void *done, int done_f32, float *slots,
+                           int64_t B, int64_t Tlen, int64_t H, int dtype, bool fmap, bool backward)
+{
+    if (dtype == MRX_BF16)
+        return launch_states<__bf16, LA_BF16_CHUNK>(st, x, y, done, done_f32, slots, B, Tlen, H, fmap, backward);
+    return launch_states<float, 32>(st, x, y, done, done_f32, slots, B, Tlen, H, fmap, backward);
+}
+
+int launch_la_state_scan(hipStream_t st, float *slots, const float *init, float *fin, const void *done, int done_f32,
+                         int64_t B, int64_t Tlen, int64_t H, int C, bool backward)
+{
+    const int64_t NC = (Tlen + C - 1) / C;
+    if (B * H > 0x7fffffffLL) return MRX_ERR_INVALID_ARG;
+    return launch_kernel(la_state_scan_kernel, dim3((unsigned)(B * H), 4), dim3(256), 0, st, slots, init, fin, done,
+                         done_f32, (int)Tlen, (int)H, (int)NC, C, backward ? 1 : 0);
+}
+
+}  // namespace mrx

@@ -197,18 +197,18 @@ class _LinearAttention(torch.autograd.Function):
             ctx.done, ctx.fmap, ctx.has_S0 = done, fmap, S0 is not None
             return o[:, None], S_last
         o, S_last, chk = K.linear_attn_fwd(q_, k_, v_, done, S0_, fmap, save_chk=need)
-        if need:
-            ctx.save_for_backward(q_, k_, v_, *chk)
+        if need:  # chk[1] (S_last) is None when the chunk-parallel pair of kernels ran
+            ctx.save_for_backward(q_, k_, v_, *(t for t in chk if t is not None))
         ctx.done, ctx.fmap, ctx.has_S0 = done, fmap, S0 is not None
         return o, S_last
 
     @staticmethod
     def backward(ctx, do, dS_last):
-        q, k, v, S_chk, S_last = ctx.saved_tensors
+        q, k, v, S_chk, *rest = ctx.saved_tensors
         do = torch.zeros_like(v) if do is None else do.contiguous()
         dS_last = None if dS_last is None else dS_last.contiguous().float()
-        dq, dk, dv, dS0 = K.linear_attn_bwd(q, k, v, ctx.done, (S_chk, S_last), do, dS_last, ctx.fmap,
-                                            want_dS0=ctx.has_S0)
+        dq, dk, dv, dS0 = K.linear_attn_bwd(q, k, v, ctx.done, (S_chk, rest[0] if rest else None), do, dS_last,
+                                            ctx.fmap, want_dS0=ctx.has_S0)
         return dq, dk, dv, None, (dS0 if ctx.has_S0 else None), None
 
 

@@ -182,18 +182,34 @@ def _n_chunks(T, dt, delta=False):
     return (T + C - 1) // C
 
 
-def linear_attn_fwd(q, k, v, done, S0=None, feature_map=0, save_chk=True):
+def linear_attn_chunk_parallel_pays(B, T, H, dtype):
+    """The library's rule: cut the work along time (one workgroup per chunk) instead of along sequences."""
+    return bool(_lib.load().mrx_linear_attn_chunk_parallel_pays(B, T, H, _DT[dtype]))
+
+
+def linear_attn_fwd(q, k, v, done, S0=None, feature_map=0, save_chk=True, chunk_parallel=None):
     """Returns (o, S_last fp32, chk) with chk = (S_chk, S_last), what the backward call needs, or None.
-    S_chk is float32 and sparse: the library writes only the slots of chunks that contain a reset (the
-    backward call walks the state back from S_last through the others)."""
+    Sequential form (one workgroup per sequence): S_chk is float32 and sparse -- the library writes only
+    the slots of chunks that contain a reset (the backward call walks the state back from S_last through
+    the others).  Chunk-parallel form (chunk_parallel=True, or None and the library's rule prefers it:
+    few sequences, several chunks each): S_chk is dense and chk = (S_chk, None); linear_attn_bwd takes
+    either."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
     _chk(S0, "S0", torch.float32, (B, H, dv, dk))
     done, dd = _done(done, B, T)
+    if chunk_parallel is None:
+        chunk_parallel = linear_attn_chunk_parallel_pays(B, T, H, dt)
     o = torch.empty_like(v)
     S_last = torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
     S_chk = (torch.empty((B, H, _n_chunks(T, dt), dv, dk), dtype=torch.float32, device=q.device)
-             if save_chk else None)
+             if save_chk or chunk_parallel else None)
+    if chunk_parallel:
+        st = lib.mrx_linear_attn_fwd_chunk_parallel(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(done), _ptr(S0),
+                                                    _ptr(o), _ptr(S_last), _ptr(S_chk), B, T, H, dk, dv, _DT[dt],
+                                                    dd, int(feature_map))
+        _lib.check(st, "mrx_linear_attn_fwd_chunk_parallel")
+        return o, S_last, ((S_chk, None) if save_chk else None)
     st = lib.mrx_linear_attn_fwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(done), _ptr(S0),
                                  _ptr(o), _ptr(S_last), _ptr(S_chk), B, T, H, dk, dv, _DT[dt], dd,
                                  int(feature_map))
@@ -202,7 +218,8 @@ def linear_attn_fwd(q, k, v, done, S0=None, feature_map=0, save_chk=True):
 
 
 def linear_attn_bwd(q, k, v, done, chk, do, dS_last=None, feature_map=0, want_dS0=True):
-    """chk = (S_chk, S_last) from linear_attn_fwd.  Returns (dq, dk, dv, dS0)."""
+    """chk = (S_chk, S_last) from linear_attn_fwd (S_last None: the chunk-parallel pair).
+    Returns (dq, dk, dv, dS0)."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
     S_chk, S_last = chk
@@ -214,6 +231,14 @@ def linear_attn_bwd(q, k, v, done, chk, do, dS_last=None, feature_map=0, want_dS
     dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dS0 = (torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
            if want_dS0 else None)
+    if S_last is None:
+        ws = torch.empty_like(S_chk)
+        st = lib.mrx_linear_attn_bwd_chunk_parallel(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(done), _ptr(S_chk),
+                                                    _ptr(do), _ptr(dS_last), _ptr(dq), _ptr(dk_), _ptr(dv_),
+                                                    _ptr(dS0), _ptr(ws), B, T, H, dk, dv, _DT[dt], dd,
+                                                    int(feature_map))
+        _lib.check(st, "mrx_linear_attn_bwd_chunk_parallel")
+        return dq, dk_, dv_, dS0
     st = lib.mrx_linear_attn_bwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(done), _ptr(S_chk), _ptr(S_last),
                                  _ptr(do), _ptr(dS_last), _ptr(dq), _ptr(dk_), _ptr(dv_),
                                  _ptr(dS0), B, T, H, dk, dv, _DT[dt], dd, int(feature_map))

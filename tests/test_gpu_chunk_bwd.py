@@ -171,7 +171,7 @@ def test_linear_attention_state_walk_back_over_a_long_sequence(dtype):
         q, k, v, do = (bf16_round(a) for a in (q, k, v, do))
     print(f"case la walk-back dtype={dtype}", flush=True)
     tq, tk, tv, tdo = (dev(a, td) for a in (q, k, v, do))
-    o, Sl, chk = K.linear_attn_fwd(tq, tk, tv, dev(done), dev(S0), 1)
+    o, Sl, chk = K.linear_attn_fwd(tq, tk, tv, dev(done), dev(S0), 1, chunk_parallel=False)  # the sequential pair
     got = K.linear_attn_bwd(tq, tk, tv, dev(done), chk, tdo, None, 1)
     ref = clib.linear_attn_bwd(q, k, v, done, S0, do, None, 1)
     tol = TOL_BF16 if dtype == "bf16" else TOL_F32
