@@ -662,7 +662,11 @@ ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, boo
     for (int v = maxvec; v >= 1; v >>= 1) {
         const size_t bytes = esize * v;
         const bool ok_al = bytes == 16 ? al16 : (bytes == 8 ? al8 : true);
-        if (D % v == 0 && ok_al) { vec = v; break; }
+        // a vector so wide that the waves covering a row are less than three quarters full wastes the
+        // idle lanes' share of every load (rows of 128 floats, backward: 0.87 -> 0.57 ms at 16384x64x128
+        // with two floats per lane instead of four; rows of 64: 0.75 -> 0.36 ms)
+        const int64_t covered = ((D + 64 * (int64_t)v - 1) / (64 * (int64_t)v)) * 64 * v;
+        if (D % v == 0 && ok_al && (v == 1 || 4 * D >= 3 * covered)) { vec = v; break; }
     }
     auto ntiles = [&](int v) { return (D + 64 * (int64_t)v - 1) / (64 * (int64_t)v); };
     if (bwd && !mg && esize == 4) {
