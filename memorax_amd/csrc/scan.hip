@@ -669,11 +669,21 @@ ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, boo
         if (D % v == 0 && ok_al && (v == 1 || 4 * D >= 3 * covered)) { vec = v; break; }
     }
     auto ntiles = [&](int v) { return (D + 64 * (int64_t)v - 1) / (64 * (int64_t)v); };
-    if (bwd && !mg && esize == 4) {
-        for (int v = vec; v >= 1; v >>= 1) {
+    // complex64: where the columns alone give the streaming kernel its 2048 waves it stays ahead (measured
+    // at 128 steps: 0.28 against 0.57 ms at 4096x128x64, 0.27 against 0.32 ms at 1024x128x256); below
+    // that the wide vectors win as they do for floats (256x1024x256: 0.99 -> 0.59 ms)
+    bool wide = bwd && !mg;
+    if (wide && esize == 8) {
+        int v2 = vec;
+        while (v2 > 1 && B * ntiles(v2) < 2048) v2 >>= 1;
+        wide = B * ntiles(v2) < 2048;
+    }
+    if (wide) {
+        for (int v = vec; v >= (esize == 8 ? 2 : 1); v >>= 1) {  // complex64: the 16-byte vector or the rule below
             const int64_t cols = B * ntiles(v);
             if (cols * 8 >= 4096 && T >= 8 * TS) return {v, 8, (int)ntiles(v), false};
-            if (v <= 2 && cols * 16 >= 4096 && T >= 16 * TS) return {v, 16, (int)ntiles(v), false};
+            // sixteen waves: instances exist for one lane per thread, and for two floats
+            if ((v == 1 || (v == 2 && esize == 4)) && cols * 16 >= 4096 && T >= 16 * TS) return {v, 16, (int)ntiles(v), false};
         }
     }
     while (vec > 1 && B * ntiles(vec) < 2048) vec >>= 1;
