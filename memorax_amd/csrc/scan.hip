@@ -669,21 +669,26 @@ ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, boo
         if (D % v == 0 && ok_al && (v == 1 || 4 * D >= 3 * covered)) { vec = v; break; }
     }
     auto ntiles = [&](int v) { return (D + 64 * (int64_t)v - 1) / (64 * (int64_t)v); };
-    // complex64: where the columns alone give the streaming kernel its 2048 waves it stays ahead (measured
-    // at 128 steps: 0.28 against 0.57 ms at 4096x128x64, 0.27 against 0.32 ms at 1024x128x256); below
-    // that the wide vectors win as they do for floats (256x1024x256: 0.99 -> 0.59 ms)
-    bool wide = bwd && !mg;
-    if (wide && esize == 8) {
-        int v2 = vec;
-        while (v2 > 1 && B * ntiles(v2) < 2048) v2 >>= 1;
-        wide = B * ntiles(v2) < 2048;
+    // complex64 (measured on 1024x128x{64,128,256}, 4096x128x64, 256x1024x{64,256}, 64x4096x256): one
+    // element per lane is the width the column rule below arrives at for most shapes, and at that width
+    // the streaming kernel is ahead of the wave-split one as soon as the columns give it 2048 waves
+    // (forward 111 -> 93 us at 1024x128x128, 242 -> 180 us at 4096x128x64) or, backward, 1024 waves
+    // (146 -> 70 us at 1024x128x64; 990 -> 520 us at 256x1024x256); where the 16-byte vector would be
+    // narrowed for lack of columns but eight waves along time make up for them, it is kept (forward
+    // 399 -> 328 us at 256x1024x256).
+    if (esize == 8 && !mg) {
+        int v1 = vec;
+        while (v1 > 1 && B * ntiles(v1) < 2048) v1 >>= 1;
+        const int64_t waves1 = B * ntiles(v1);
+        if (v1 == 1 && waves1 >= (bwd ? 1024 : 2048)) return {1, 1, (int)ntiles(1), true};
+        if (vec == 2 && v1 == 1 && B * ntiles(2) * 8 >= 4096 && T >= 8 * TS) return {2, 8, (int)ntiles(2), false};
     }
-    if (wide) {
-        for (int v = vec; v >= (esize == 8 ? 2 : 1); v >>= 1) {  // complex64: the 16-byte vector or the rule below
+    // floats, backward: see above
+    if (bwd && !mg && esize == 4) {
+        for (int v = vec; v >= 1; v >>= 1) {
             const int64_t cols = B * ntiles(v);
             if (cols * 8 >= 4096 && T >= 8 * TS) return {v, 8, (int)ntiles(v), false};
-            // sixteen waves: instances exist for one lane per thread, and for two floats
-            if ((v == 1 || (v == 2 && esize == 4)) && cols * 16 >= 4096 && T >= 16 * TS) return {v, 16, (int)ntiles(v), false};
+            if (v <= 2 && cols * 16 >= 4096 && T >= 16 * TS) return {v, 16, (int)ntiles(v), false};
         }
     }
     while (vec > 1 && B * ntiles(vec) < 2048) vec >>= 1;
