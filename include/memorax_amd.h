@@ -14,7 +14,8 @@
  *  - Return value: MRX_OK (0) or a negative mrx_status; never throws.
  *    mrx_status_string() names a code.  Arguments are checked before any launch;
  *    the status of a launch is the launch call's own return code (the runtime's
- *    sticky last-error state is neither read nor cleared).  An entry point that
+ *    sticky last-error state is not consulted; only the record of a launch that
+ *    was itself refused, and reported as MRX_ERR_LAUNCH, is cleared).  An entry point that
  *    enqueues two kernels (mrx_delta_rule_fwd with the chunk-parallel factors)
  *    may return MRX_ERR_LAUNCH after the first has been enqueued.
  *  - The library keeps no state between calls apart from what mrx_init() sets up

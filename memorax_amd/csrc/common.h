@@ -31,16 +31,19 @@ __device__ __forceinline__ bool done_test(uint32_t raw, int is_f32)
 }
 
 // Launches `kern` and returns MRX_OK or MRX_ERR_LAUNCH from the launch call's own return code.
-// The runtime's sticky "last error" is neither read nor cleared, so an error left behind by other
-// code in the process is not mistaken for this launch's, and is still there for its owner.
+// The runtime's sticky "last error" is not consulted, so an error left behind by other code in the
+// process is not mistaken for this launch's, and is still there for its owner.  When the launch
+// itself is refused, the error it has just recorded is this call's own and is reported through the
+// return value: it is taken off the runtime's record, or the next runtime call of the host
+// framework would report it a second time as its own.
 template <typename... KArgs, size_t... I>
 inline int launch_impl(void (*kern)(KArgs...), dim3 grid, dim3 block, size_t lds_bytes, hipStream_t st,
                        std::tuple<KArgs...> &vals, std::index_sequence<I...>)
 {
     void *ptrs[] = {static_cast<void *>(&std::get<I>(vals))...};
-    return hipLaunchKernel(reinterpret_cast<const void *>(kern), grid, block, ptrs, lds_bytes, st) == hipSuccess
-               ? MRX_OK
-               : MRX_ERR_LAUNCH;
+    if (hipLaunchKernel(reinterpret_cast<const void *>(kern), grid, block, ptrs, lds_bytes, st) == hipSuccess) return MRX_OK;
+    (void)hipGetLastError();
+    return MRX_ERR_LAUNCH;
 }
 template <typename... KArgs, typename... Args>
 inline int launch_kernel(void (*kern)(KArgs...), dim3 grid, dim3 block, size_t lds_bytes, hipStream_t st, Args... args)

@@ -683,7 +683,11 @@ ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, boo
         if (v1 == 1 && waves1 >= (bwd ? 1024 : 2048)) return {1, 1, (int)ntiles(1), true};
         if (vec == 2 && v1 == 1 && B * ntiles(2) * 8 >= 4096 && T >= 8 * TS) return {2, 8, (int)ntiles(2), false};
     }
-    // floats, backward: see above
+    // floats, backward: see above; rows of up to 128 floats first -- there a wave's loads in the
+    // wave-split kernel are short pieces, and one column per lane in the streaming kernel is ahead
+    // wherever it gets 1024 waves (4096x128x64: 193 -> 137 us, 1024x1024x64: 456 -> 303 us,
+    // 1024x128x128: 84 -> 69 us, 8192x128x128: 585 -> 545 us)
+    if (bwd && !mg && esize == 4 && D <= 128 && B * ntiles(1) >= 1024) return {1, 1, (int)ntiles(1), true};
     if (bwd && !mg && esize == 4) {
         for (int v = vec; v >= 1; v >>= 1) {
             const int64_t cols = B * ntiles(v);
