@@ -702,6 +702,9 @@ ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, boo
     const int maxw = vec == 1 ? 16 : 8;
     while (nw < maxw && waves * nw < 8192 && (int64_t)nw * TS < T) nw <<= 1;
     const bool stream = bwd ? waves >= 2048 : nw == 1;
+    // MinGRU backward short of columns for that: one column per lane still streams ahead of the wave-split
+    // kernel from 1024 waves (1024x128x64: 55 -> 45 us, 256x1024x256: 472 -> 332 us)
+    if (bwd && mg && !stream && B * ntiles(1) >= 1024) return {1, 1, (int)ntiles(1), true};
     return {vec, stream ? 1 : nw, tiles, stream};
 }
 
