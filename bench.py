@@ -403,7 +403,7 @@ def bench_linear_attention(torch, K, np, dev):
     res["cfg3_bf16_256x4096x8x64"] = {"ms": ms, "tokens/s": Bn * Tn / ms * 1e3, "GB/s": 1408 * nth / ms / 1e6,
                                       "frac_hbm": 1408 * nth / ms / 1e6 / HBM_PEAK_GBS,
                                       "frac_mfma": (ff + fb) * nth / (ms * 1e-3) / MFMA_BF16_PEAK}
-    # the same shape with a per-step scalar decay (Mamba cell algebra); + g in, edot out: 8 B more per token-head
+    # the same shape with a per-step scalar decay (Mamba cell algebra); + g in, dg out: 8 B more per token-head
     g = -torch.rand((Bn, Tn, Hn), device="cuda") * 0.1
 
     def f3g():

@@ -328,18 +328,18 @@ int mrx_gated_linear_attn_fwd(void *stream, const void *q, const void *k,
                               int64_t B, int64_t T, int64_t H, int64_t dk, int64_t dv,
                               int dtype, int done_dtype, int feature_map);
 
-/* Gradients w.r.t. q,k,v (pre-feature-map, in `dtype`) and S0 (fp32, nullable), and
- * edot: (B,T,H) float32 with edot_t = phi(q_t) . dphi(q)_t - phi(k_t) . dphi(k)_t.  The gradient of
- * the log-decay is its reverse cumulative sum inside each episode,
+/* Gradients w.r.t. q,k,v (pre-feature-map, in `dtype`), S0 (fp32, nullable) and the log-decay:
+ * dg: (B,T,H) float32.  With edot_t = phi(q_t) . dphi(q)_t - phi(k_t) . dphi(k)_t,
  *     dg_t = done_t ? 0 : sum over i >= t of t's episode of edot_i  (+ <S_last, dS_last> when the
  *     episode reaches the end),
- * which the caller takes with mrx_linear_scan_fwd on the time-reversed array (decay 1). */
+ * summed inside the kernel, which walks the time axis from the end.  S_last: the forward call's
+ * output, read only when dS_last is given (nullable otherwise). */
 int mrx_gated_linear_attn_bwd(void *stream, const void *q, const void *k,
                               const void *v, const void *g, const void *done,
-                              const void *S_chk, const void *dout, const void *dS_last,
-                              void *dq, void *dk_out, void *dv_out, void *edot, void *dS0,
-                              int64_t B, int64_t T, int64_t H, int64_t dk, int64_t dv,
-                              int dtype, int done_dtype, int feature_map);
+                              const void *S_chk, const float *S_last, const void *dout,
+                              const void *dS_last, void *dq, void *dk_out, void *dv_out,
+                              float *dg, void *dS0, int64_t B, int64_t T, int64_t H, int64_t dk,
+                              int64_t dv, int dtype, int done_dtype, int feature_map);
 
 /* ---- Single time step (rollout / acting) ------------------------------------
  * What Memoroid.__call__ (memoroid.py:93-109) computes when T = 1, as PPO's rollout

@@ -46,7 +46,7 @@ SIGNATURES = {
     "mrx_mingru_scan_fwd": (_I, [_P] * 9 + [_L] * 3 + [_I]),
     "mrx_mingru_scan_bwd": (_I, [_P] * 11 + [_L] * 3 + [_I]),
     "mrx_gated_linear_attn_fwd": (_I, [_P] * 10 + [_L] * 5 + [_I] * 3),
-    "mrx_gated_linear_attn_bwd": (_I, [_P] * 14 + [_L] * 5 + [_I] * 3),
+    "mrx_gated_linear_attn_bwd": (_I, [_P] * 15 + [_L] * 5 + [_I] * 3),
     "mrx_linear_attn_step": (_I, [_P] * 10 + [_L] * 4 + [_I] * 3 + [ctypes.c_float]),
     "mrx_delta_rule_step": (_I, [_P] * 9 + [_L] * 4 + [_I] * 2),
 }

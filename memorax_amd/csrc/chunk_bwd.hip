@@ -72,7 +72,10 @@ struct NormBwdArgs {
 // z_in the sum entering the chunk (first episode only), dz the gradient of the sum leaving it.
 // The gradient of the log-decays follows from edot_i = q_i . dq_i - k_i . dk_i (taken on the
 // feature-mapped q, k and their gradients): dg_t is the sum of edot over the rows i >= t of t's
-// episode (plus <S_last, dS_last> at the end); the kernel writes edot, the caller sums.
+// episode (plus <S_last, dS_last> when the episode reaches the end), 0 at a reset step.  The kernel
+// walks the chunks and their episodes from the end anyway, so wave 0 carries that running sum in
+// a register (a reverse cumulative sum over the chunk's rows by lane shuffles, cut at resets) and
+// writes dg itself.
 // PAR (plain linear attention): one workgroup per chunk (grid.y = chunk).  Slot c of S_chk holds, in
 // fp32, the state entering chunk c and slot c of dS_last -- then a (B,H,NC,64,64) array -- the gradient
 // of the state leaving it (la_states.h); the workgroup forms the chunk's dQ, dK, dV from them and neither
@@ -82,7 +85,7 @@ __global__ void __launch_bounds__(256, 2)
 la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
               const float *__restrict__ glog, const void *__restrict__ done, int done_f32,
               const void *__restrict__ S_chk, const float *__restrict__ S_last, const T *__restrict__ dout,
-              const float *__restrict__ dS_last, T *__restrict__ dq, T *__restrict__ dk, T *__restrict__ dv, float *__restrict__ edot,
+              const float *__restrict__ dS_last, T *__restrict__ dq, T *__restrict__ dk, T *__restrict__ dv, float *__restrict__ dg,
               float *__restrict__ dS0, int Tlen, int H, NormBwdArgs na)
 {
     static_assert(!(GATED && NORM), "the normalised read-out belongs to plain linear attention");
@@ -162,6 +165,24 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             Sacc[j] = *reinterpret_cast<const f32x4 *>((PAR ? reinterpret_cast<const float *>(S_chk) : S_last) +
                                                        (slot + dvv) * HD + dk0);
         }
+    }
+
+    // gated: the running sum behind dg, held by wave 0; it starts from <S_last, dS_last>
+    float dg_carry = 0.f;
+    if (GATED && dS_last && S_last) {
+        float part = 0.f;
+#pragma unroll
+        for (int j = 0; j < TMS::TPW; ++j) {
+            const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
+            const f32x4 sl = *reinterpret_cast<const f32x4 *>(S_last + ((int64_t)bh * HD + dvv) * HD + dk0);
+            part += dSacc[j][0] * sl[0] + dSacc[j][1] * sl[1] + dSacc[j][2] * sl[2] + dSacc[j][3] * sl[3];
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) part += __shfl_xor(part, off);
+        if (lane == 0) sE[w] = part;
+        sync_lds();
+        dg_carry = sE[0] + sE[1] + sE[2] + sE[3];
+        sync_lds();  // sE is written again by the first pass
     }
 
     typename IO::Regs rq, rk, rv, rdo, ro;
@@ -552,11 +573,22 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             pend_pass = pass;
             pend_t0 = t0;
             sync_lds();
-            if (GATED && tid < C && t0 + tid < Tlen && live(tid)) {
+            if (GATED && w == 0) {
+                const bool on = lane < C && live(lane);  // rows past the end of the sequence hold zeros
                 float x = 0.f;
+                if (on) {
 #pragma unroll
-                for (int sl = 0; sl < TMR::WM; ++sl) x += sE[sl * C + tid];
-                edot[((int64_t)b * Tlen + t0 + tid) * H + h] = x;
+                    for (int sl = 0; sl < TMR::WM; ++sl) x += sE[sl * C + lane];
+                }
+                // x_r <- sum over the rows i >= r of this pass's episode (its rows are consecutive)
+#pragma unroll
+                for (int off = 1; off < C; off <<= 1) {
+                    const float up = __shfl_down(x, off);
+                    if (lane + off < C) x += up;
+                }
+                if (pass == nres) x += dg_carry;  // the episode that reaches the end of the chunk goes on into the later steps
+                if (on && t0 + lane < Tlen) dg[((int64_t)b * Tlen + t0 + lane) * H + h] = ((dmask >> lane) & 1ull) ? 0.f : x;
+                if (pass == 0) dg_carry = (dmask & 1ull) ? 0.f : __shfl(x, 0);  // cut where the chunk opens with a reset
             }
         }
     }
@@ -1020,7 +1052,7 @@ template <typename T, int C, bool FMAP, bool GATED = false, bool NORM = false, b
 int launch_la(hipStream_t st, const void *q, const void *k, const void *v, const void *done,
               int done_f32, const void *S_chk, const void *S_last, const void *dout, const void *dS_last, void *dq,
               void *dk, void *dv, void *dS0, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr,
-              void *edot = nullptr, NormBwdArgs na = NormBwdArgs{})
+              void *dg = nullptr, NormBwdArgs na = NormBwdArgs{})
 {
     using Reg = LaBwdReg<T, C, FMAP, GATED, NORM, PAR>;
     (void)&Reg::reg;  // the kernel is on the list mrx_init() walks
@@ -1031,7 +1063,7 @@ int launch_la(hipStream_t st, const void *q, const void *k, const void *v, const
                          dim3(256), Reg::smem, st,
                          (const T *)q, (const T *)k, (const T *)v, (const float *)glog, done, done_f32,
                          S_chk, (const float *)S_last, (const T *)dout, (const float *)dS_last, (T *)dq, (T *)dk, (T *)dv,
-                         (float *)edot, (float *)dS0, (int)Tlen, (int)H, na);
+                         (float *)dg, (float *)dS0, (int)Tlen, (int)H, na);
 }
 
 int check_bwd(const void *q, const void *k, const void *v, const void *done, const void *S_chk,
@@ -1129,19 +1161,20 @@ extern "C" int mrx_linear_attn_norm_bwd(void *stream, const void *q, const void 
 }
 
 extern "C" int mrx_gated_linear_attn_bwd(void *stream, const void *q, const void *k, const void *v,
-                                         const void *g, const void *done, const void *S_chk,
+                                         const void *g, const void *done, const void *S_chk, const float *S_last,
                                          const void *dout, const void *dS_last, void *dq, void *dk_out,
-                                         void *dv_out, void *edot, void *dS0, int64_t B, int64_t T, int64_t H,
+                                         void *dv_out, float *dg, void *dS0, int64_t B, int64_t T, int64_t H,
                                          int64_t dk, int64_t dv, int dtype, int done_dtype, int feature_map)
 {
     const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
                              dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
-    if (!g || !edot || !aligned(g, 4) || !aligned(edot, 4)) return MRX_ERR_INVALID_ARG;
+    if (!g || !dg || !aligned(g, 4) || !aligned(dg, 4) || !aligned(S_last, 16)) return MRX_ERR_INVALID_ARG;
+    if (dS_last && !S_last) return MRX_ERR_INVALID_ARG;  // <S_last, dS_last> enters dg at the last step
     if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     const bool fm = feature_map == MRX_FMAP_ELU1;
-#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, nullptr, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, g, edot
+#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, S_last, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, g, dg
     if (dtype == MRX_BF16)
         return fm ? launch_la<__bf16, LA_BF16_CHUNK, true, true>(MRX_ARGS) : launch_la<__bf16, LA_BF16_CHUNK, false, true>(MRX_ARGS);
     return fm ? launch_la<float, 32, true, true>(MRX_ARGS) : launch_la<float, 32, false, true>(MRX_ARGS);

@@ -428,36 +428,25 @@ def gated_linear_attn_fwd(q, k, v, g, done, S0=None, feature_map=0, save_chk=Tru
 
 def gated_linear_attn_bwd(q, k, v, g, done, S_chk, do, dS_last=None, feature_map=0, want_dS0=True,
                           S_last=None):
-    """Returns (dq, dk, dv, dg, dS0).  dg is the reverse cumulative sum, inside each episode, of the
-    row dots the kernel writes (one reset-aware scan over the time-reversed (B,T,H) array); S_last
-    is needed when dS_last is given (its inner product with dS_last enters at the last step)."""
+    """Returns (dq, dk, dv, dg, dS0).  S_last (the forward call's) is needed when dS_last is given: its
+    inner product with dS_last enters dg at the last step."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
     _chk(g, "g", torch.float32, (B, T, H))
     _chk(do, "do", dt, (B, T, H, dv))
     _chk(S_chk, "S_chk", dt, (B, H, _n_chunks(T, dt), dv, dk))
     _chk(dS_last, "dS_last", torch.float32, (B, H, dv, dk))
+    _chk(S_last, "S_last", torch.float32, (B, H, dv, dk))
+    if dS_last is not None and S_last is None:
+        raise ValueError("S_last is required with dS_last")
     done_u, dd = _done(done, B, T)
     dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    edot = torch.empty((B, T, H), dtype=torch.float32, device=q.device)
+    dg = torch.empty((B, T, H), dtype=torch.float32, device=q.device)
     dS0 = (torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device) if want_dS0 else None)
     st = lib.mrx_gated_linear_attn_bwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(g), _ptr(done_u), _ptr(S_chk),
-                                       _ptr(do), _ptr(dS_last), _ptr(dq), _ptr(dk_), _ptr(dv_), _ptr(edot),
-                                       _ptr(dS0), B, T, H, dk, dv, _DT[dt], dd, int(feature_map))
+                                       _ptr(S_last), _ptr(do), _ptr(dS_last), _ptr(dq), _ptr(dk_), _ptr(dv_),
+                                       _ptr(dg), _ptr(dS0), B, T, H, dk, dv, _DT[dt], dd, int(feature_map))
     _lib.check(st, "mrx_gated_linear_attn_bwd")
-    # reverse scan: acc_t = edot_t + (done_{t+1} ? 0 : acc_{t+1}); dg_t = done_t ? 0 : acc_t
-    dn = done_u != 0 if done_u.dtype != torch.float32 else done_u != 0
-    tail = None
-    if dS_last is not None:
-        if S_last is None:
-            raise ValueError("S_last is required with dS_last")
-        tail = (S_last * dS_last).sum((-1, -2)).contiguous()
-    flags = torch.zeros((B, T), dtype=torch.bool, device=q.device)
-    if T > 1:
-        flags[:, 1:] = dn.flip(1)[:, :-1]
-    ones = torch.ones(H, dtype=torch.float32, device=q.device)
-    acc, _, _ = linear_scan_fwd(ones, edot.flip(1).contiguous(), flags, tail, want_P=False)
-    dg = torch.where(dn[:, :, None], torch.zeros((), device=q.device), acc.flip(1))
     return dq, dk_, dv_, dg, dS0
 
 
