@@ -61,7 +61,7 @@ typedef enum {
 
 /* How mrx_delta_rule_fwd / mrx_deltanet_fwd obtain the per-chunk triangular factors. */
 typedef enum {
-    MRX_FACTORS_AUTO = 0,     /* by occupancy: chunk-parallel kernel iff a buffer is given and B*H <= 2 x compute units */
+    MRX_FACTORS_AUTO = 0,     /* chunk-parallel kernel iff a buffer is given and (float32, or B*H <= 2 x compute units) */
     MRX_FACTORS_PARALLEL = 1, /* chunk-parallel kernel whenever a buffer is given */
     MRX_FACTORS_INLINE = 2    /* inverted inside the sequential kernel */
 } mrx_factor_path;

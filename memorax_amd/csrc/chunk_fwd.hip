@@ -604,8 +604,11 @@ int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void 
     constexpr bool TM_KERNEL = DELTA_BF16_CHUNK == 32;
     int cus = 0;
     if (const int rc = prepare_device(&cus); rc != MRX_OK) return rc;
+    // fp32: the in-kernel inverse is the longer part of a chunk's chain at any occupancy (measured on
+    // full devices, 1024 to 8192 sequences: 8 % faster with the chunk-parallel kernel), so the rule by
+    // occupancy is the bf16 kernels' only
     const bool parallel = Tm_chk && factor_path != MRX_FACTORS_INLINE && T <= DELTA_TM_MAX_T &&
-                          (factor_path == MRX_FACTORS_PARALLEL || B * H <= 2 * (int64_t)cus);
+                          (factor_path == MRX_FACTORS_PARALLEL || dtype == MRX_F32 || B * H <= 2 * (int64_t)cus);
     if (!TM_KERNEL && factor_path == MRX_FACTORS_PARALLEL) return MRX_ERR_UNSUPPORTED;
     if constexpr (TM_KERNEL) if (parallel) {
         const int rc = launch_delta_tm(st, k, beta, done, done_dtype, Tm_chk, B, T, H, dtype, PRO);

@@ -337,8 +337,8 @@ def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prolog
     call with the same shapes instead of allocating.  prologue=True: k is L2-normalised and
     beta = sigmoid(beta) inside the kernel (mrx_deltanet_fwd).
     tm_scratch (only without residuals): give the library a buffer for the triangular factors
-    anyway, which lets it compute them chunk-parallel while the device is not full.  None: when
-    B*H is at most two sequences per compute unit, which is when the library uses it.
+    anyway, which lets it compute them chunk-parallel.  None: when the library would use it (float32;
+    bf16 with B*H at most two sequences per compute unit).
     factor_path: None / "auto" (by occupancy), "parallel" or "inline" (mrx_factor_path)."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
@@ -363,7 +363,8 @@ def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prolog
             Tm_chk = torch.empty((B, H, NC, C, C), dtype=dt, device=q.device)
         else:
             if tm_scratch is None:
-                tm_scratch = B * H <= 2 * torch.cuda.get_device_properties(q.device).multi_processor_count
+                tm_scratch = (dt == torch.float32 or
+                              B * H <= 2 * torch.cuda.get_device_properties(q.device).multi_processor_count)
             if tm_scratch:
                 C, NC = chunk_size(dt, True), _n_chunks(T, dt, True)
                 Tm_chk = torch.empty((B, H, NC, C, C), dtype=dt, device=q.device)

@@ -116,7 +116,7 @@ def test_config_shapes_small_batch():
 def test_delta_rule_factor_paths_agree(dtype, prologue):
     """The triangular factors of a chunk depend on its keys, gates and resets only.  Three ways to
     them: the chunk-parallel kernel (residuals asked, device not full), the sequential kernel with
-    the factors stored (more than two sequences per compute unit) and without.  A batch large
+    the factors stored (bf16: more than two sequences per compute unit) and without.  A batch large
     enough for the second way is cut into slices small enough for the first: same outputs and the
     same stored factors, up to rounding; and the backward call accepts either."""
     from memorax_amd import kernels as K
@@ -133,7 +133,9 @@ def test_delta_rule_factor_paths_agree(dtype, prologue):
     beta = (beta if prologue else torch.sigmoid(beta)).to(td)
     done = torch.rand((B, T), device="cuda", generator=g) < 0.05
     print(f"case factor_paths dtype={dtype} prologue={prologue} B={B}", flush=True)
-    o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done, prologue=prologue)            # stored, in place
+    # stored, in place (what the automatic rule picks for bf16 on a full device; float32 always takes the
+    # chunk-parallel kernel when it has a buffer, so the path is named)
+    o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done, prologue=prologue, factor_path="inline")
     o2, Sl2, _ = K.delta_rule_fwd(q, k, v, beta, done, save_chk=False, prologue=prologue, tm_scratch=False)
     assert torch.equal(o, o2) and torch.equal(Sl, Sl2)  # the same kernel with and without the stores
     grads = K.delta_rule_bwd(q, k, v, beta, done, chk, do, prologue=prologue)
