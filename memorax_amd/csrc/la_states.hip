@@ -56,38 +56,53 @@ la_chunk_state_kernel(const T *__restrict__ x, const T *__restrict__ y, const vo
     }
 }
 
-// grid (B * H, 4): each thread carries four of the 4096 state elements through the chunks.  The loads of
-// a group of four chunks are issued together; only the additions are sequential.
+// grid (B * H, 4): each thread carries four of the 4096 state elements through the chunks.  Only the
+// additions are sequential: the slots (and the reset flags) of the next group of eight chunks are
+// requested before the current group is summed and written back, so that one trip to memory is exposed
+// per sequence, not one per group.
 __global__ void __launch_bounds__(256)
 la_state_scan_kernel(float *__restrict__ slots, const float *__restrict__ init, float *__restrict__ fin,
                      const void *__restrict__ done, int done_f32, int Tlen, int H, int NC, int C, int backward)
 {
     constexpr int Q = HD * HD / 4;  // f32x4 per state
+    constexpr int G = 8;            // chunks per group
     const int tid = threadIdx.x, lane = tid & 63;
     const int bh = blockIdx.x, b = bh / H;
     const int idx = blockIdx.y * 256 + tid;
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
     f32x4 S = init ? reinterpret_cast<const f32x4 *>(init)[(int64_t)bh * Q + idx] : zero;
     f32x4 *p = reinterpret_cast<f32x4 *>(slots) + (int64_t)bh * NC * Q + idx;
-    for (int s0 = 0; s0 < NC; s0 += 4) {
-        f32x4 t[4];
-        bool cut[4];
+    auto chunk_of = [&](int s) { return backward ? NC - 1 - s : s; };
+    f32x4 nt[G];
+    uint32_t nd[G];  // raw reset flag of chunk row `lane`
+    auto fetch = [&](int s0) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int s = s0 + u, c = backward ? NC - 1 - s : s;
-            t[u] = zero;
-            cut[u] = false;
+        for (int u = 0; u < G; ++u) {
+            const int s = s0 + u, c = chunk_of(s);
+            nt[u] = zero;
+            nd[u] = 0u;
             if (s < NC) {  // uniform over the workgroup
-                t[u] = p[(int64_t)c * Q];
+                nt[u] = p[(int64_t)c * Q];
                 const int tt = c * C + lane;
-                cut[u] = __ballot(lane < C && tt < Tlen && done_at(done, done_f32, (int64_t)b * Tlen + tt)) != 0ull;
+                if (lane < C && tt < Tlen) nd[u] = done_raw(done, done_f32, (int64_t)b * Tlen + tt);
             }
         }
+    };
+    fetch(0);
+    for (int s0 = 0; s0 < NC; s0 += G) {
+        f32x4 t[G];
+        bool cut[G];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int s = s0 + u, c = backward ? NC - 1 - s : s;
+        for (int u = 0; u < G; ++u) {
+            t[u] = nt[u];
+            cut[u] = __ballot(done_test(nd[u], done_f32)) != 0ull;
+        }
+        if (s0 + G < NC) fetch(s0 + G);
+#pragma unroll
+        for (int u = 0; u < G; ++u) {
+            const int s = s0 + u;
             if (s < NC) {
-                p[(int64_t)c * Q] = S;
+                p[(int64_t)chunk_of(s) * Q] = S;
                 S = cut[u] ? t[u] : S + t[u];
             }
         }
