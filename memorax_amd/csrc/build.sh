@@ -22,10 +22,16 @@ compile() {  # compile <object suffix> <extra flags...>
         pids+=($!)
     done
 }
+# the chunked and single-step kernels once more for head dim 32 (hd.h); both libraries link these objects
+HD32_SRCS=(chunk_fwd.hip chunk_bwd.hip step.hip delta_tm.hip la_states.hip)
 compile ""
 compile _c64 -DMRX_DELTA_BF16_CHUNK=64
+ALL_SRCS=("${SRCS[@]}"); SRCS=("${HD32_SRCS[@]}")
+compile _hd32 -DMRX_HD=32
+SRCS=("${ALL_SRCS[@]}")
 for p in "${pids[@]}"; do wait "$p"; done
-"$HIPCC" --offload-arch=gfx950 -shared -fPIC -o libmemorax_amd.so $(printf '%s.o ' "${SRCS[@]%.hip}")
-"$HIPCC" --offload-arch=gfx950 -shared -fPIC -o libmemorax_amd_c64.so $(printf '%s_c64.o ' "${SRCS[@]%.hip}")
+HD32_OBJS=$(printf '%s_hd32.o ' "${HD32_SRCS[@]%.hip}")
+"$HIPCC" --offload-arch=gfx950 -shared -fPIC -o libmemorax_amd.so $(printf '%s.o ' "${SRCS[@]%.hip}") $HD32_OBJS
+"$HIPCC" --offload-arch=gfx950 -shared -fPIC -o libmemorax_amd_c64.so $(printf '%s_c64.o ' "${SRCS[@]%.hip}") $HD32_OBJS
 rm -f ./*.o
 echo "built $(pwd)/libmemorax_amd.so and libmemorax_amd_c64.so"

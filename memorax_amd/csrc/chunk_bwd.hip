@@ -19,6 +19,9 @@
 // LDS tiles and are written to memory row-wise (tile_rows_to_global).
 #include "chunk_common.h"
 #include "la_states.h"
+#if MRX_HD == 64
+#include "hd32_api.h"
+#endif
 
 
 namespace {
@@ -212,7 +215,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     int64_t noff[IO::PASSES];  // den of the rows this thread stages
 #pragma unroll
     for (int p = 0; p < IO::PASSES; ++p) noff[p] = (int64_t)bh * Tlen + tlast + IO::row_of(tid, p);  // den: (B,H,T)
-    int64_t zoff = ((int64_t)bh * NC + c_hi) * HD + 4 * (tid & 15);
+    int64_t zoff = ((int64_t)bh * NC + c_hi) * HD + 4 * (tid % (HD / 4));
     int tpre = tlast;
     auto prefetch_part = [&](int part) {
         typename IO::F z;
@@ -221,7 +224,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
         if (part < 2) {
 #pragma unroll
             for (int p = 0; p < IO::PASSES; ++p) {
-                const bool in = tpre + IO::row_of(tid, p) < Tlen;
+                const bool in = (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen;
                 if (part == 0) {
                     rq.v[p] = in ? *reinterpret_cast<const typename IO::F *>(q + roff[p]) : z;
                     rk.v[p] = in ? *reinterpret_cast<const typename IO::F *>(k + roff[p]) : z;
@@ -235,7 +238,8 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             if (!WALK) {
 #pragma unroll
                 for (int p = 0; p < IOS::PASSES; ++p)
-                    rS.v[p] = *reinterpret_cast<const typename IOS::F *>(reinterpret_cast<const T *>(S_chk) + soff + p * IOS::RPP * HD);
+                    if (IOS::FULL || IOS::row_of(tid, p) < HD)  // a [32][32] tile has fewer segments than threads
+                        rS.v[p] = *reinterpret_cast<const typename IOS::F *>(reinterpret_cast<const T *>(S_chk) + soff + p * IOS::RPP * HD);
             } else if (need_S) {
                 // straight into the state registers: the chunk at hand has formed its state (the first
                 // phase), and the next chunk, taking a checkpoint, does not walk back from it
@@ -255,7 +259,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             if (NORM) {
 #pragma unroll
                 for (int p = 0; p < IO::PASSES; ++p) {
-                    rden[p] = tpre + IO::row_of(tid, p) < Tlen ? na.den[noff[p]] : 1.f;
+                    rden[p] = (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen ? na.den[noff[p]] : 1.f;
                     noff[p] -= C;
                 }
                 rz = *reinterpret_cast<const f32x4 *>(na.z_chk + zoff);
@@ -355,7 +359,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                         }
                     }
                     IO::scale_rows(fdo, inv);
-                    if (tid < 16) *reinterpret_cast<f32x4 *>(sZf + 4 * tid) = rz;
+                    if (tid < HD / 4) *reinterpret_cast<f32x4 *>(sZf + 4 * tid) = rz;
                 }
                 flush_pending();  // reads what this thread is about to overwrite in sV, sQ, sK
                 IO::to_lds(fq, sQ, LDD, tid);
@@ -728,11 +732,13 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             typename IO::Regs &dst = part == 0 ? rq : part == 1 ? rk : part == 2 ? rv : rdo;
 #pragma unroll
             for (int p = 0; p < IO::PASSES; ++p)
-                dst.v[p] = tpre + IO::row_of(tid, p) < Tlen ? *reinterpret_cast<const typename IO::F *>(src + roff[p]) : z;
+                dst.v[p] = (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen
+                               ? *reinterpret_cast<const typename IO::F *>(src + roff[p]) : z;
         } else if (part == 4) {
 #pragma unroll
             for (int p = 0; p < IOS::PASSES; ++p)
-                rS.v[p] = *reinterpret_cast<const typename IOS::F *>(S_chk + soff + p * IOS::RPP * HD);
+                if (IOS::FULL || IOS::row_of(tid, p) < HD)
+                    rS.v[p] = *reinterpret_cast<const typename IOS::F *>(S_chk + soff + p * IOS::RPP * HD);
         } else {
 #pragma unroll
             for (int p = 0; p < IOT::PASSES; ++p)
@@ -740,7 +746,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     rTm.v[p] = *reinterpret_cast<const typename IOT::F *>(Tm_chk + tmoff + p * IOT::RPP * C);
 #pragma unroll
             for (int p = 0; p < IO::PASSES; ++p) {
-                rbrow[p] = tpre + IO::row_of(tid, p) < Tlen ? load_raw<T>(beta + boff[p]) : 0u;
+                rbrow[p] = (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen ? load_raw<T>(beta + boff[p]) : 0u;
                 roff[p] -= (int64_t)C * rs;
                 boff[p] -= (int64_t)C * H;
             }
@@ -1086,12 +1092,15 @@ int check_bwd(const void *q, const void *k, const void *v, const void *done, con
 
 }  // namespace
 
-extern "C" int mrx_linear_attn_bwd(void *stream, const void *q, const void *k, const void *v,
+MRX_EXPORT int MRX_API(mrx_linear_attn_bwd)(void *stream, const void *q, const void *k, const void *v,
                                    const void *done, const void *S_chk, const float *S_last, const void *dout,
                                    const void *dS_last, void *dq, void *dk_out, void *dv_out,
                                    void *dS0, int64_t B, int64_t T, int64_t H, int64_t dk, int64_t dv,
                                    int dtype, int done_dtype, int feature_map)
 {
+#if MRX_HD == 64
+    if (dk == 32 && dv == 32) return mrx_linear_attn_bwd_hd32(stream, q, k, v, done, S_chk, S_last, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk, dv, dtype, done_dtype, feature_map);
+#endif
     const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
                              dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
@@ -1105,12 +1114,15 @@ extern "C" int mrx_linear_attn_bwd(void *stream, const void *q, const void *k, c
 #undef MRX_ARGS
 }
 
-extern "C" int mrx_linear_attn_bwd_chunk_parallel(void *stream, const void *q, const void *k, const void *v,
+MRX_EXPORT int MRX_API(mrx_linear_attn_bwd_chunk_parallel)(void *stream, const void *q, const void *k, const void *v,
                                                   const void *done, const float *S_chk, const void *dout,
                                                   const void *dS_last, void *dq, void *dk_out, void *dv_out,
                                                   void *dS0, float *workspace, int64_t B, int64_t T, int64_t H,
                                                   int64_t dk, int64_t dv, int dtype, int done_dtype, int feature_map)
 {
+#if MRX_HD == 64
+    if (dk == 32 && dv == 32) return mrx_linear_attn_bwd_chunk_parallel_hd32(stream, q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, workspace, B, T, H, dk, dv, dtype, done_dtype, feature_map);
+#endif
     const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
                              dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
@@ -1134,7 +1146,7 @@ extern "C" int mrx_linear_attn_bwd_chunk_parallel(void *stream, const void *q, c
 #undef MRX_ARGS
 }
 
-extern "C" int mrx_linear_attn_norm_bwd(void *stream, const void *q, const void *k, const void *v,
+MRX_EXPORT int MRX_API(mrx_linear_attn_norm_bwd)(void *stream, const void *q, const void *k, const void *v,
                                         const void *done, const void *S_chk, const float *S_last, const float *z_chk,
                                         const void *o, const float *den, const void *dout,
                                         const void *dS_last, const float *dz_last, void *dq, void *dk_out,
@@ -1142,6 +1154,9 @@ extern "C" int mrx_linear_attn_norm_bwd(void *stream, const void *q, const void 
                                         int64_t dk, int64_t dv, int dtype, int done_dtype, int feature_map,
                                         float eps)
 {
+#if MRX_HD == 64
+    if (dk == 32 && dv == 32) return mrx_linear_attn_norm_bwd_hd32(stream, q, k, v, done, S_chk, S_last, z_chk, o, den, dout, dS_last, dz_last, dq, dk_out, dv_out, dS0, dz0, B, T, H, dk, dv, dtype, done_dtype, feature_map, eps);
+#endif
     const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
                              dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
@@ -1160,12 +1175,15 @@ extern "C" int mrx_linear_attn_norm_bwd(void *stream, const void *q, const void 
 #undef MRX_ARGS
 }
 
-extern "C" int mrx_gated_linear_attn_bwd(void *stream, const void *q, const void *k, const void *v,
+MRX_EXPORT int MRX_API(mrx_gated_linear_attn_bwd)(void *stream, const void *q, const void *k, const void *v,
                                          const void *g, const void *done, const void *S_chk, const float *S_last,
                                          const void *dout, const void *dS_last, void *dq, void *dk_out,
                                          void *dv_out, float *dg, void *dS0, int64_t B, int64_t T, int64_t H,
                                          int64_t dk, int64_t dv, int dtype, int done_dtype, int feature_map)
 {
+#if MRX_HD == 64
+    if (dk == 32 && dv == 32) return mrx_gated_linear_attn_bwd_hd32(stream, q, k, v, g, done, S_chk, S_last, dout, dS_last, dq, dk_out, dv_out, dg, dS0, B, T, H, dk, dv, dtype, done_dtype, feature_map);
+#endif
     const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
                              dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
@@ -1224,24 +1242,30 @@ int delta_bwd_entry(void *stream, const void *q, const void *k, const void *v, c
 
 }  // namespace
 
-extern "C" int mrx_delta_rule_bwd(void *stream, const void *q, const void *k, const void *v,
+MRX_EXPORT int MRX_API(mrx_delta_rule_bwd)(void *stream, const void *q, const void *k, const void *v,
                                   const void *beta, const void *done, const void *S_chk,
                                   const void *Tm_chk, const void *dout, const void *dS_last, void *dq,
                                   void *dk_out, void *dv_out, void *dbeta, void *dS0, int64_t B,
                                   int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                                   int done_dtype)
 {
+#if MRX_HD == 64
+    if (dk == 32 && dv == 32) return mrx_delta_rule_bwd_hd32(stream, q, k, v, beta, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out, dbeta, dS0, B, T, H, dk, dv, dtype, done_dtype);
+#endif
     return delta_bwd_entry<false>(stream, q, k, v, beta, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out,
                                   dbeta, dS0, B, T, H, dk, dv, dtype, done_dtype);
 }
 
-extern "C" int mrx_deltanet_bwd(void *stream, const void *q, const void *k, const void *v,
+MRX_EXPORT int MRX_API(mrx_deltanet_bwd)(void *stream, const void *q, const void *k, const void *v,
                                 const void *beta_raw, const void *done, const void *S_chk,
                                 const void *Tm_chk, const void *dout, const void *dS_last, void *dq,
                                 void *dk_out, void *dv_out, void *dbeta_raw, void *dS0, int64_t B,
                                 int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                                 int done_dtype)
 {
+#if MRX_HD == 64
+    if (dk == 32 && dv == 32) return mrx_deltanet_bwd_hd32(stream, q, k, v, beta_raw, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out, dbeta_raw, dS0, B, T, H, dk, dv, dtype, done_dtype);
+#endif
     return delta_bwd_entry<true>(stream, q, k, v, beta_raw, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out,
                                  dbeta_raw, dS0, B, T, H, dk, dv, dtype, done_dtype);
 }

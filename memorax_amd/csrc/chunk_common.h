@@ -15,6 +15,7 @@
 // result is stored with one 8/16-byte write per lane as the matrix dst[n][m].
 #pragma once
 #include "common.h"
+#include "hd.h"
 
 namespace mrx {
 
@@ -32,7 +33,10 @@ __device__ __forceinline__ void sync_lds()
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-constexpr int HD = 64;  // head dim (d_k = d_v)
+// Head dim (d_k = d_v) of the chunked and single-step kernels: 64, or 32 in the library's second build
+// of these sources (hd.h).
+constexpr int HD = MRX_HD;
+static_assert(HD == 64 || HD == 32, "tile maps exist for head dims 64 and 32");
 
 // Time steps per chunk of the bf16 kernels.  Linear attention: 64 (two workgroups per CU fit at 64
 // and larger chunks amortise the per-chunk staging of S).  Delta rule: 32 -- the backward's fifteen
@@ -315,14 +319,15 @@ template <typename T, int R, int NTHR, int COLS = HD> struct TileIO {
     }
 };
 
-// Sum over the SEGS consecutive lanes that share a tile row (8 or 16), by data-parallel
+// Sum over the SEGS consecutive lanes that share a tile row (4, 8 or 16), by data-parallel
 // primitives; every lane of the group ends with the total.
 template <int SEGS> __device__ __forceinline__ float seg_sum(float x)
 {
-    static_assert(SEGS == 8 || SEGS == 16, "a row is 8 or 16 segments");
+    static_assert(SEGS == 4 || SEGS == 8 || SEGS == 16, "a row is 4, 8 or 16 segments");
     x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
     x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
-    x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xF, 0xF, true));  // row_half_mirror
+    if (SEGS >= 8)
+        x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xF, 0xF, true));  // row_half_mirror
     if (SEGS == 16)
         x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x140, 0xF, 0xF, true));  // row_mirror
     return x;

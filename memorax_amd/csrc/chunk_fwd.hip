@@ -17,6 +17,9 @@
 #include "chunk_common.h"
 #include "delta_tm.h"
 #include "la_states.h"
+#if MRX_HD == 64
+#include "hd32_api.h"
+#endif
 
 namespace {
 
@@ -178,11 +181,12 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             typename IO::Regs &dst = part == 0 ? rq : part == 1 ? rk : rv;
 #pragma unroll
             for (int p = 0; p < IO::PASSES; ++p)
-                dst.v[p] = tpre + IO::row_of(tid, p) < Tlen ? *reinterpret_cast<const typename IO::F *>(src + roff[p]) : z;
+                dst.v[p] = (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen
+                               ? *reinterpret_cast<const typename IO::F *>(src + roff[p]) : z;
         } else {
 #pragma unroll
             for (int p = 0; p < IO::PASSES; ++p) {
-                if (DELTA) rbrow[p] = tpre + IO::row_of(tid, p) < Tlen ? load_raw<T>(beta + boff[p]) : 0u;
+                if (DELTA) rbrow[p] = (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen ? load_raw<T>(beta + boff[p]) : 0u;
                 roff[p] += (int64_t)C * rs;
                 boff[p] += (int64_t)C * H;
             }
@@ -332,8 +336,9 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                     for (int p = 0; p < IOS::PASSES; ++p) {
                         const int r = IOS::row_of(tid, p), seg = tid % IOS::SEGS;
-                        *reinterpret_cast<typename IOS::F *>(reinterpret_cast<T *>(S_chk) + schk_off + r * HD + seg * IOS::KP) =
-                            *reinterpret_cast<const typename IOS::F *>(sS + r * LDD + seg * IOS::KP);
+                        if (IOS::FULL || r < HD)  // a [32][32] tile has fewer segments than threads
+                            *reinterpret_cast<typename IOS::F *>(reinterpret_cast<T *>(S_chk) + schk_off + r * HD + seg * IOS::KP) =
+                                *reinterpret_cast<const typename IOS::F *>(sS + r * LDD + seg * IOS::KP);
                     }
                 } else {
 #pragma unroll
@@ -628,6 +633,7 @@ int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void 
 
 bool factor_path_ok(int f) { return f == MRX_FACTORS_AUTO || f == MRX_FACTORS_PARALLEL || f == MRX_FACTORS_INLINE; }
 
+#if MRX_HD == 64
 // ---- static scratch of the entry point that allocates nothing --------------------------------------
 // Room for the triangular factors of MRX_NOALLOC_SCRATCH_BYTES / (32 * 32 * sizeof(element)) chunks.
 // Every device the library runs on holds its own copy at its own address; host code only ever uses
@@ -635,8 +641,10 @@ bool factor_path_ok(int f) { return f == MRX_FACTORS_AUTO || f == MRX_FACTORS_PA
 static __device__ __align__(256) unsigned char scratch[MRX_NOALLOC_SCRATCH_BYTES];
 void *g_scratch_ptr[64] = {nullptr};
 
+#endif
 }  // namespace
 
+#if MRX_HD == 64
 int mrx::resolve_scratch(int dev)
 {
     if (dev < 0 || dev >= 64) return MRX_ERR_UNSUPPORTED;
@@ -650,11 +658,16 @@ extern "C" int64_t mrx_chunk_size(int dtype) { return dtype == MRX_BF16 ? LA_BF1
 
 extern "C" int64_t mrx_delta_chunk_size(int dtype) { return dtype == MRX_BF16 ? DELTA_BF16_CHUNK : (dtype == MRX_F32 ? 32 : 0); }
 
-extern "C" int mrx_linear_attn_fwd(void *stream, const void *q, const void *k, const void *v,
+#endif
+
+MRX_EXPORT int MRX_API(mrx_linear_attn_fwd)(void *stream, const void *q, const void *k, const void *v,
                                    const void *done, const void *S0, void *o, void *S_last,
                                    void *S_chk, int64_t B, int64_t T, int64_t H, int64_t dk,
                                    int64_t dv, int dtype, int done_dtype, int feature_map)
 {
+#if MRX_HD == 64
+    if (dk == 32 && dv == 32) return mrx_linear_attn_fwd_hd32(stream, q, k, v, done, S0, o, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, feature_map);
+#endif
     const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
     if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
@@ -667,11 +680,14 @@ extern "C" int mrx_linear_attn_fwd(void *stream, const void *q, const void *k, c
               : launch<float, 32, false, false>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H);
 }
 
-extern "C" int mrx_linear_attn_fwd_chunk_parallel(void *stream, const void *q, const void *k, const void *v,
+MRX_EXPORT int MRX_API(mrx_linear_attn_fwd_chunk_parallel)(void *stream, const void *q, const void *k, const void *v,
                                                   const void *done, const void *S0, void *o, void *S_last,
                                                   float *S_chk, int64_t B, int64_t T, int64_t H, int64_t dk,
                                                   int64_t dv, int dtype, int done_dtype, int feature_map)
 {
+#if MRX_HD == 64
+    if (dk == 32 && dv == 32) return mrx_linear_attn_fwd_chunk_parallel_hd32(stream, q, k, v, done, S0, o, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, feature_map);
+#endif
     const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
     if (!S_chk) return MRX_ERR_INVALID_ARG;  // the per-chunk states live there
@@ -694,6 +710,7 @@ extern "C" int mrx_linear_attn_fwd_chunk_parallel(void *stream, const void *q, c
 #undef MRX_ARGS
 }
 
+#if MRX_HD == 64
 extern "C" int mrx_linear_attn_chunk_parallel_pays(int64_t B, int64_t T, int64_t H, int dtype)
 {
     const int64_t C = mrx_chunk_size(dtype);
@@ -707,12 +724,16 @@ extern "C" int mrx_linear_attn_chunk_parallel_pays(int64_t B, int64_t T, int64_t
     // than the idle compute units, and with fewer chunks the two extra launches do.
     return 2 * B * H <= (int64_t)cus && NC >= 8 && NC <= 65535;
 }
+#endif
 
-extern "C" int mrx_delta_rule_fwd(void *stream, const void *q, const void *k, const void *v,
+MRX_EXPORT int MRX_API(mrx_delta_rule_fwd)(void *stream, const void *q, const void *k, const void *v,
                                   const void *beta, const void *done, const void *S0, void *o,
                                   void *S_last, void *S_chk, void *Tm_chk, int64_t B, int64_t T,
                                   int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype, int factor_path)
 {
+#if MRX_HD == 64
+    if (dk == 32 && dv == 32) return mrx_delta_rule_fwd_hd32(stream, q, k, v, beta, done, S0, o, S_last, S_chk, Tm_chk, B, T, H, dk, dv, dtype, done_dtype, factor_path);
+#endif
     const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
     if (!beta || !aligned(Tm_chk, 16) || !factor_path_ok(factor_path)) return MRX_ERR_INVALID_ARG;
@@ -721,6 +742,7 @@ extern "C" int mrx_delta_rule_fwd(void *stream, const void *q, const void *k, co
                                      factor_path);
 }
 
+#if MRX_HD == 64
 extern "C" int mrx_delta_rule_fwd_noalloc(void *stream, const void *q, const void *k, const void *v,
                                           const void *beta, const void *done, const void *S0, void *o,
                                           void *S_last, int64_t B, int64_t T, int64_t H, int64_t dk,
@@ -739,12 +761,16 @@ extern "C" int mrx_delta_rule_fwd_noalloc(void *stream, const void *q, const voi
     return delta_fwd_dispatch<false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, nullptr, factors, B, T, H, dtype,
                                      MRX_FACTORS_PARALLEL);
 }
+#endif
 
-extern "C" int mrx_gated_linear_attn_fwd(void *stream, const void *q, const void *k, const void *v,
+MRX_EXPORT int MRX_API(mrx_gated_linear_attn_fwd)(void *stream, const void *q, const void *k, const void *v,
                                          const void *g, const void *done, const void *S0, void *o,
                                          void *S_last, void *S_chk, int64_t B, int64_t T, int64_t H,
                                          int64_t dk, int64_t dv, int dtype, int done_dtype, int feature_map)
 {
+#if MRX_HD == 64
+    if (dk == 32 && dv == 32) return mrx_gated_linear_attn_fwd_hd32(stream, q, k, v, g, done, S0, o, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, feature_map);
+#endif
     const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
     if (!g || !aligned(g, 4)) return MRX_ERR_INVALID_ARG;
@@ -758,12 +784,15 @@ extern "C" int mrx_gated_linear_attn_fwd(void *stream, const void *q, const void
 #undef MRX_ARGS
 }
 
-extern "C" int mrx_linear_attn_norm_fwd(void *stream, const void *q, const void *k, const void *v,
+MRX_EXPORT int MRX_API(mrx_linear_attn_norm_fwd)(void *stream, const void *q, const void *k, const void *v,
                                         const void *done, const void *S0, const float *z0, void *o,
                                         float *den, void *S_last, float *z_last, void *S_chk, float *z_chk,
                                         int64_t B, int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                                         int done_dtype, int feature_map, float eps)
 {
+#if MRX_HD == 64
+    if (dk == 32 && dv == 32) return mrx_linear_attn_norm_fwd_hd32(stream, q, k, v, done, S0, z0, o, den, S_last, z_last, S_chk, z_chk, B, T, H, dk, dv, dtype, done_dtype, feature_map, eps);
+#endif
     const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
     if (!den || !aligned(den, 4) || !aligned(z0, 16) || !aligned(z_last, 16) || !aligned(z_chk, 16))
@@ -780,11 +809,14 @@ extern "C" int mrx_linear_attn_norm_fwd(void *stream, const void *q, const void 
 #undef MRX_ARGS
 }
 
-extern "C" int mrx_deltanet_fwd(void *stream, const void *q, const void *k, const void *v,
+MRX_EXPORT int MRX_API(mrx_deltanet_fwd)(void *stream, const void *q, const void *k, const void *v,
                                 const void *beta_raw, const void *done, const void *S0, void *o,
                                 void *S_last, void *S_chk, void *Tm_chk, int64_t B, int64_t T,
                                 int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype, int factor_path)
 {
+#if MRX_HD == 64
+    if (dk == 32 && dv == 32) return mrx_deltanet_fwd_hd32(stream, q, k, v, beta_raw, done, S0, o, S_last, S_chk, Tm_chk, B, T, H, dk, dv, dtype, done_dtype, factor_path);
+#endif
     const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
     if (!beta_raw || !aligned(Tm_chk, 16) || !factor_path_ok(factor_path)) return MRX_ERR_INVALID_ARG;

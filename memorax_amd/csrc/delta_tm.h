@@ -21,7 +21,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "hd.h"
+
 namespace mrx {
+inline namespace MRX_HD_NS {
 
 // Longest sequence the launch covers: four chunks per workgroup, 65535 workgroups along the grid's y.
 constexpr int64_t DELTA_TM_MAX_T = 4ll * 65535 * 32;
@@ -32,4 +35,5 @@ constexpr int64_t DELTA_TM_MAX_T = 4ll * 65535 * 32;
 int launch_delta_tm(hipStream_t st, const void *k, const void *beta, const void *done, int done_f32, void *Tm_chk,
                     int64_t B, int64_t Tlen, int64_t H, int dtype, bool prologue);
 
+}  // namespace MRX_HD_NS
 }  // namespace mrx

@@ -9,6 +9,7 @@
 #include "chunk_common.h"
 
 namespace mrx {
+inline namespace MRX_HD_NS {
 
 template <typename T, bool PRO>
 __global__ void __launch_bounds__(256)
@@ -65,8 +66,9 @@ delta_tm_kernel(const T *__restrict__ k, const T *__restrict__ beta, const void 
                 ss += __shfl_xor(ss, 32);
                 tq[kb] = ss;
             }
-            float tot = tq[0] + tq[1];
-            if (NKB == 4) tot += tq[2] + tq[3];
+            float tot = tq[0];  // pairs, then pairs of pairs: the staging code's order
+            if (NKB >= 2) tot += tq[NKB >= 2 ? 1 : 0];
+            if (NKB == 4) tot += tq[NKB == 4 ? 2 : 0] + tq[NKB == 4 ? 3 : 0];
             const float inv = inv_norm(tot);
 #pragma unroll
             for (int kb = 0; kb < NKB; ++kb)
@@ -179,4 +181,5 @@ int launch_delta_tm(hipStream_t st, const void *k, const void *beta, const void 
                     : launch_tm<float, false>(st, k, beta, done, done_f32, Tm_chk, B, Tlen, H);
 }
 
+}  // namespace MRX_HD_NS
 }  // namespace mrx

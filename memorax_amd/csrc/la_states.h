@@ -18,7 +18,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "hd.h"
+
 namespace mrx {
+inline namespace MRX_HD_NS {
 
 // slots[B][H][NC][64][64] fp32 <- per-chunk contributions.  x: keys (forward) or queries (backward),
 // y: values (forward) or output gradients (backward), both (B,T,H,64) of `dtype`; fmap: elu+1 on x.
@@ -31,4 +34,5 @@ int launch_la_chunk_states(hipStream_t st, const void *x, const void *y, const v
 int launch_la_state_scan(hipStream_t st, float *slots, const float *init, float *fin, const void *done, int done_f32,
                          int64_t B, int64_t Tlen, int64_t H, int C, bool backward);
 
+}  // namespace MRX_HD_NS
 }  // namespace mrx

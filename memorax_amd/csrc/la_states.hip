@@ -4,6 +4,7 @@
 #include "chunk_common.h"
 
 namespace mrx {
+inline namespace MRX_HD_NS {
 
 namespace {
 
@@ -56,7 +57,7 @@ la_chunk_state_kernel(const T *__restrict__ x, const T *__restrict__ y, const vo
     }
 }
 
-// grid (B * H, 4): each thread carries four of the 4096 state elements through the chunks.  Only the
+// grid (B * H, d * d / 1024): each thread carries four of the d x d state elements through the chunks.  Only the
 // additions are sequential: the slots (and the reset flags) of the next group of eight chunks are
 // requested before the current group is summed and written back, so that one trip to memory is exposed
 // per sequence, not one per group.
@@ -140,8 +141,9 @@ int launch_la_state_scan(hipStream_t st, float *slots, const float *init, float 
 {
     const int64_t NC = (Tlen + C - 1) / C;
     if (B * H > 0x7fffffffLL) return MRX_ERR_INVALID_ARG;
-    return launch_kernel(la_state_scan_kernel, dim3((unsigned)(B * H), 4), dim3(256), 0, st, slots, init, fin, done,
+    return launch_kernel(la_state_scan_kernel, dim3((unsigned)(B * H), HD * HD / 1024), dim3(256), 0, st, slots, init, fin, done,
                          done_f32, (int)Tlen, (int)H, (int)NC, C, backward ? 1 : 0);
 }
 
+}  // namespace MRX_HD_NS
 }  // namespace mrx

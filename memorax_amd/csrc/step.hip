@@ -5,25 +5,33 @@
 //                      o = S' phi(q)            [ / max(phi(q) . z', eps) when z is given ]
 //   delta rule       : S0 = done ? 0 : S ,  u = beta (v - S0 k) ,  S' = S0 + u k^T ,  o = S' q
 //
-// The state S:(B,H,64,64) fp32 ([dv][dk]) is read once and written once; everything else is a
-// few hundred bytes per sequence, so the kernels are bound by HBM traffic of the state
-// (32 KiB per (b,h)).  One workgroup of 256 threads per (b,h): thread t owns the four
-// consecutive dk = 4 (t & 15).. of rows dv = (t >> 4) + 16 p, p = 0..3, so that every load and
-// store of S is a fully coalesced 16-byte access; row dot products reduce over 16 lanes.
+// The state S:(B,H,d,d) fp32 ([dv][dk], d = 64 or 32) is read once and written once; everything else
+// is a few hundred bytes per sequence, so the kernels are bound by HBM traffic of the state
+// (32 KiB per (b,h) at d = 64).  One workgroup of 256 threads per (b,h): a row of the state is d / 4
+// lanes of four consecutive dk each, the 256 threads cover 1024 / d rows at a time (d = 64: thread t
+// owns dk = 4 (t & 15).. of rows dv = (t >> 4) + 16 p, p = 0..3), so that every load and store of S is a
+// fully coalesced 16-byte access; row dot products reduce over the lanes of a row.
 // Follows what Memoroid.__call__ computes for T = 1 (memoroid.py:93-109 with the cell algebra of
 // linear_attention.py:62-117) and the delta-rule recurrence of the chunked kernels.
 #include "chunk_common.h"
+#if MRX_HD == 64
+#include "hd32_api.h"
+#endif
 
 namespace {
 
 using namespace mrx;
 
-__device__ __forceinline__ float reduce16(float x)
+constexpr int LPR = HD / 4;    // lanes per row of the state
+constexpr int RPP = 256 / LPR;  // rows the workgroup covers at a time
+constexpr int NP = HD / RPP;    // times it does so
+
+__device__ __forceinline__ float reduce_row(float x)
 {
     x += __shfl_xor(x, 1);
     x += __shfl_xor(x, 2);
     x += __shfl_xor(x, 4);
-    x += __shfl_xor(x, 8);
+    if (LPR == 16) x += __shfl_xor(x, 8);
     return x;
 }
 
@@ -47,7 +55,7 @@ step_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restric
             const float *S_in, const float *z_in, T *__restrict__ o, float *S_out, float *z_out, int H,
             float eps)  // S_in/S_out and z_in/z_out may alias (update in place)
 {
-    const int tid = threadIdx.x, c4 = tid & 15, r0 = tid >> 4;
+    const int tid = threadIdx.x, c4 = tid % LPR, r0 = tid / LPR;
     const int64_t bh = blockIdx.x;
     const int b = (int)(bh / H);
     const bool reset = done_at(done, done_f32, b);
@@ -62,35 +70,35 @@ step_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restric
         }
     }
     const float *Sp = S_in ? S_in + bh * HD * HD : nullptr;
-    f32x4 s[4];
+    f32x4 s[NP];
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const int row = r0 + 16 * p;
+    for (int p = 0; p < NP; ++p) {
+        const int row = r0 + RPP * p;
         s[p] = (Sp && !reset) ? *reinterpret_cast<const f32x4 *>(Sp + row * HD + 4 * c4) : f32x4{0.f, 0.f, 0.f, 0.f};
     }
-    float u[4];
+    float u[NP];
 #pragma unroll
-    for (int p = 0; p < 4; ++p) u[p] = (float)vp[r0 + 16 * p];
+    for (int p = 0; p < NP; ++p) u[p] = (float)vp[r0 + RPP * p];
     if (DELTA) {
         const float bb = (float)beta[bh];
 #pragma unroll
-        for (int p = 0; p < 4; ++p) u[p] = bb * (u[p] - reduce16(dot4(s[p], k4)));
+        for (int p = 0; p < NP; ++p) u[p] = bb * (u[p] - reduce_row(dot4(s[p], k4)));
     }
     float den = 1.f;
     if (!DELTA && z_out) {
-        // every 16-lane group recomputes the normaliser of the sequence; group 0 stores it
+        // every row's lanes recompute the normaliser of the sequence; row 0 stores it
         f32x4 z4 = (z_in && !reset) ? *reinterpret_cast<const f32x4 *>(z_in + bh * HD + 4 * c4) : f32x4{0.f, 0.f, 0.f, 0.f};
         z4 += k4;
         if (r0 == 0) *reinterpret_cast<f32x4 *>(z_out + bh * HD + 4 * c4) = z4;
-        den = fmaxf(reduce16(dot4(z4, q4)), eps);
+        den = fmaxf(reduce_row(dot4(z4, q4)), eps);
     }
     float *So = S_out + bh * HD * HD;
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const int row = r0 + 16 * p;
+    for (int p = 0; p < NP; ++p) {
+        const int row = r0 + RPP * p;
         s[p] += k4 * u[p];
         *reinterpret_cast<f32x4 *>(So + row * HD + 4 * c4) = s[p];
-        const float x = reduce16(dot4(s[p], q4));
+        const float x = reduce_row(dot4(s[p], q4));
         if (c4 == 0) o[bh * HD + row] = (T)(x / den);
     }
 }
@@ -124,11 +132,14 @@ int launch_step(hipStream_t st, const void *q, const void *k, const void *v, con
 
 }  // namespace
 
-extern "C" int mrx_linear_attn_step(void *stream, const void *q, const void *k, const void *v, const void *done,
+MRX_EXPORT int MRX_API(mrx_linear_attn_step)(void *stream, const void *q, const void *k, const void *v, const void *done,
                                     const float *S_in, const float *z_in, void *o, float *S_out, float *z_out,
                                     int64_t B, int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype,
                                     int feature_map, float eps)
 {
+#if MRX_HD == 64
+    if (dk == 32 && dv == 32) return mrx_linear_attn_step_hd32(stream, q, k, v, done, S_in, z_in, o, S_out, z_out, B, H, dk, dv, dtype, done_dtype, feature_map, eps);
+#endif
     const int rc = check_step(q, k, v, done, S_in, o, S_out, B, H, dk, dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
     if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
@@ -142,10 +153,13 @@ extern "C" int mrx_linear_attn_step(void *stream, const void *q, const void *k, 
 #undef MRX_ARGS
 }
 
-extern "C" int mrx_delta_rule_step(void *stream, const void *q, const void *k, const void *v, const void *beta,
+MRX_EXPORT int MRX_API(mrx_delta_rule_step)(void *stream, const void *q, const void *k, const void *v, const void *beta,
                                    const void *done, const float *S_in, void *o, float *S_out, int64_t B,
                                    int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype)
 {
+#if MRX_HD == 64
+    if (dk == 32 && dv == 32) return mrx_delta_rule_step_hd32(stream, q, k, v, beta, done, S_in, o, S_out, B, H, dk, dv, dtype, done_dtype);
+#endif
     const int rc = check_step(q, k, v, done, S_in, o, S_out, B, H, dk, dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
     if (!beta) return MRX_ERR_INVALID_ARG;

@@ -20,7 +20,7 @@ from . import kernels as K
 
 _FMAP = {None: 0, "none": 0, 0: 0, "elu1": 1, 1: 1}
 _FMAP_NAME = {0: "none", 1: "elu1"}
-_HD = 64  # head dim of the kernels (d_k = d_v)
+_HD = 64  # widest head dim of the kernels (d_k = d_v = 64 or 32)
 
 
 def _batched(core_rank, ref):
@@ -52,10 +52,11 @@ def _batched(core_rank, ref):
 
 
 class _Heads:
-    """Maps other head dims onto the kernels' d_k = d_v = 64 (the reference's cells take any
-    head_dim; its guides use 16).  d_k < 64 is zero-padded -- after the feature map, since
-    phi(0) = 1 would otherwise count -- and d_v is zero-padded to a multiple of 64 and split into
-    blocks that run as extra heads sharing q and k (rows of the state are independent recurrences).
+    """Maps other head dims onto the kernels' d_k = d_v = 64 or 32 (the reference's cells take any
+    head_dim; its guides use 16): the 32-wide kernels serve d_k <= 32, the 64-wide ones the rest.
+    d_k below the kernel's width is zero-padded -- after the feature map, since phi(0) = 1 would
+    otherwise count -- and d_v is zero-padded to a multiple of that width and split into blocks that
+    run as extra heads sharing q and k (rows of the state are independent recurrences).
     Padding, blocks and slices are ordinary differentiable array ops around the kernel call."""
 
     def __init__(self, q, v, fmap=0):
@@ -63,15 +64,16 @@ class _Heads:
         self.dv = v.shape[-1]
         if self.dk > _HD:
             raise ValueError(f"d_k = {self.dk} > {_HD} is not supported (d_v may be any size)")
-        self.nb = (self.dv + _HD - 1) // _HD
-        self.native = self.dk == _HD and self.dv == _HD
-        self.pre = fmap if self.dk != _HD else 0    # feature map applied here, before the padding
-        self.fmap = 0 if self.pre else fmap         # feature map left to the kernel
+        self.hd = 32 if self.dk <= 32 else _HD
+        self.nb = (self.dv + self.hd - 1) // self.hd
+        self.native = self.dk == self.hd and self.dv == self.hd
+        self.pre = fmap if self.dk != self.hd else 0    # feature map applied here, before the padding
+        self.fmap = 0 if self.pre else fmap             # feature map left to the kernel
 
-    def _blocks(self, x):  # (B,T,H,64) -> (B,T,H*nb,64), every block a copy
+    def _blocks(self, x):  # (B,T,H,hd) -> (B,T,H*nb,hd), every block a copy
         if self.nb == 1:
             return x
-        return x[:, :, :, None].expand(self.B, self.T, self.H, self.nb, _HD).reshape(self.B, self.T, self.H * self.nb, _HD)
+        return x[:, :, :, None].expand(self.B, self.T, self.H, self.nb, self.hd).reshape(self.B, self.T, self.H * self.nb, self.hd)
 
     def qk(self, x):
         if self.native:
@@ -79,37 +81,37 @@ class _Heads:
         if self.pre:
             xf = x if x.dtype in (torch.float32, torch.float64) else x.float()
             x = (torch.nn.functional.elu(xf) + 1).to(x.dtype)
-        return self._blocks(torch.nn.functional.pad(x, (0, _HD - self.dk)))
+        return self._blocks(torch.nn.functional.pad(x, (0, self.hd - self.dk)))
 
     def v(self, x):
         if self.native:
             return x
-        x = torch.nn.functional.pad(x, (0, self.nb * _HD - self.dv))
-        return x.reshape(self.B, self.T, self.H * self.nb, _HD)
+        x = torch.nn.functional.pad(x, (0, self.nb * self.hd - self.dv))
+        return x.reshape(self.B, self.T, self.H * self.nb, self.hd)
 
     def per_head(self, x):  # (B,T,H) -> (B,T,H*nb)
         return x if self.nb == 1 else x.repeat_interleave(self.nb, dim=2)
 
-    def state_in(self, S):  # (B,H,dv,dk) -> (B,H*nb,64,64)
+    def state_in(self, S):  # (B,H,dv,dk) -> (B,H*nb,hd,hd)
         if S is None or self.native:
             return S
-        S = torch.nn.functional.pad(S, (0, _HD - self.dk, 0, self.nb * _HD - self.dv))
-        return S.reshape(self.B, self.H * self.nb, _HD, _HD)
+        S = torch.nn.functional.pad(S, (0, self.hd - self.dk, 0, self.nb * self.hd - self.dv))
+        return S.reshape(self.B, self.H * self.nb, self.hd, self.hd)
 
-    def z_in(self, z):  # (B,H,dk) -> (B,H*nb,64)
+    def z_in(self, z):  # (B,H,dk) -> (B,H*nb,hd)
         if z is None or self.native:
             return z
-        z = torch.nn.functional.pad(z, (0, _HD - self.dk))
+        z = torch.nn.functional.pad(z, (0, self.hd - self.dk))
         return z if self.nb == 1 else z.repeat_interleave(self.nb, dim=1)
 
-    def out(self, o):  # (B,T,H*nb,64) -> (B,T,H,dv)
-        return o if self.native else o.reshape(self.B, o.shape[1], self.H, self.nb * _HD)[..., :self.dv]
+    def out(self, o):  # (B,T,H*nb,hd) -> (B,T,H,dv)
+        return o if self.native else o.reshape(self.B, o.shape[1], self.H, self.nb * self.hd)[..., :self.dv]
 
     def state_out(self, S):
-        return S if self.native else S.reshape(self.B, self.H, self.nb * _HD, _HD)[:, :, :self.dv, :self.dk]
+        return S if self.native else S.reshape(self.B, self.H, self.nb * self.hd, self.hd)[:, :, :self.dv, :self.dk]
 
     def z_out(self, z):
-        return z if self.native else z.reshape(self.B, self.H, self.nb, _HD)[:, :, 0, :self.dk]
+        return z if self.native else z.reshape(self.B, self.H, self.nb, self.hd)[:, :, 0, :self.dk]
 
 
 class _LinearScan(torch.autograd.Function):

@@ -1,4 +1,4 @@
-"""Host logic that maps other head dims onto the kernels' d_k = d_v = 64 (CPU: the oracle
+"""Host logic that maps other head dims onto the kernels' d_k = d_v = 64 or 32 (CPU: the oracle
 recurrences stand in for the kernels, so the test pins the padding/blocking algebra itself)."""
 import numpy as np
 import pytest
@@ -12,7 +12,7 @@ def _rand(*s, seed=0):
     return torch.from_numpy(np.random.default_rng(seed).standard_normal(s))
 
 
-@pytest.mark.parametrize("dk,dv", [(16, 16), (32, 64), (64, 96), (16, 130), (64, 64)])
+@pytest.mark.parametrize("dk,dv", [(16, 16), (32, 64), (64, 96), (16, 130), (64, 64), (32, 32), (33, 20)])
 @pytest.mark.parametrize("op", ["linear", "normalised", "gated", "delta"])
 def test_padding_and_value_blocks_reproduce_the_native_recurrence(dk, dv, op):
     B, T, H = 2, 9, 2
@@ -22,10 +22,11 @@ def test_padding_and_value_blocks_reproduce_the_native_recurrence(dk, dv, op):
     done = torch.from_numpy(np.random.default_rng(8).random((B, T)) < 0.2)
     fm = "none" if op == "delta" else "elu1"
     hd = _Heads(q, v, 0 if op == "delta" else 1)
-    assert hd.native == (dk == 64 and dv == 64) and hd.nb == -(-dv // 64)
+    w = 32 if dk <= 32 else 64  # the 32-wide kernels serve keys of up to 32 features
+    assert hd.hd == w and hd.native == (dk == w and dv == w) and hd.nb == -(-dv // w)
     kfm = "elu1" if hd.fmap else "none"   # the feature map the kernel would be asked to apply
     qq, kk, vv, SS = hd.qk(q), hd.qk(k), hd.v(v), hd.state_in(S0)
-    assert qq.shape == (B, T, H * hd.nb, 64) and vv.shape == qq.shape and SS.shape == (B, H * hd.nb, 64, 64)
+    assert qq.shape == (B, T, H * hd.nb, w) and vv.shape == qq.shape and SS.shape == (B, H * hd.nb, w, w)
     if op == "linear":
         o, Sl = G.linear_attention_t(qq, kk, vv, done, SS, kfm)
         ro, rS = G.linear_attention_t(q, k, v, done, S0, fm)
