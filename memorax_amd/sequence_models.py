@@ -436,7 +436,8 @@ class MambaCell(MemoroidCellBase):
     (h_t = (B_t dt_t) (x) x_t : (H,N,P), decay_t = exp(dt_t A) : (H,1,1)) combined by the diagonal
     operator; read is y_t = C_t . h_t + D x_t, gated by silu(z) after RMSNorm.  The reference
     materialises h (B,T,H,N,P); here the scan and the C-contraction run in the gated chunked
-    kernel with k = B dt, v = x, q = C and log-decay g = dt A (needs state_dim = head_dim = 64).
+    kernel with k = B dt, v = x, q = C and log-decay g = dt A (native at state_dim = head_dim = 64 or
+    32; other sizes are padded by the op, state_dim up to 64).
     Carry: (h (B,1,H,N,P), decay (B,1,H,1,1)), the reference's shapes."""
 
     def __init__(self, features, num_heads=8, head_dim=64, state_dim=64, conv_dim=4, in_features=None):
