@@ -390,6 +390,21 @@ def bench_linear_attention(torch, K, np, dev):
     small["tokens/s"] = Bn * Tn / min(small["ms_one_workgroup_per_sequence"], small["ms_chunk_parallel"]) * 1e3
     res["small_grid_bf16_8x4096x4x64"] = small
     del q, k, v, do
+    # head dim 32 (the library's second build of the kernels) at 1024 environments x 128 steps x 4 heads,
+    # beside the same token-heads at head dim 64 (what a 32-wide model paid when it was padded)
+    Bn, Tn, Hn = 1024, 128, 4
+    dn = torch.rand((Bn, Tn), device="cuda") < 0.01
+    hd = {}
+    for d in (32, 64):
+        q, k, v, do = (torch.randn((Bn, Tn, Hn, d), device="cuda").div_(8).to(torch.bfloat16) for _ in range(4))
+
+        def fh():
+            o, Sl, chk = K.linear_attn_fwd(q, k, v, dn, None, 1)
+            K.linear_attn_bwd(q, k, v, dn, chk, do, None, 1, want_dS0=False)
+        hd[f"ms_d{d}"] = _time_ms(torch, fh)
+        del q, k, v, do
+    hd["tokens/s"] = Bn * Tn / hd["ms_d32"] * 1e3
+    res["head_dim_32_bf16_1024x128x4"] = hd
     Bn, Tn, Hn = 256, 4096, 8   # configuration 3 at full size (11.8 GB of q, k, v, do, o, dq, dk, dv)
     q, k, v, do = (torch.randn((Bn, Tn, Hn, 64), device="cuda").div_(8).to(torch.bfloat16) for _ in range(4))
     dn = torch.zeros((Bn, Tn), dtype=torch.bool, device="cuda")
