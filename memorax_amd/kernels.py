@@ -13,7 +13,14 @@ from . import _lib
 _DT = {torch.float32: _lib.MRX_F32, torch.bfloat16: _lib.MRX_BF16, torch.complex64: _lib.MRX_C64}
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream():
+    """The current device's current stream as a raw handle (the short way where torch has it: building
+    a torch.cuda.Stream object per call costs several microseconds of a 15-microsecond call)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -52,10 +59,16 @@ def _done(done, B, T):
     return done, _lib.MRX_DONE_U8
 
 
+_chunk_sizes = {}
+
+
 def chunk_size(dtype, delta=False) -> int:
     """Chunk length of the (gated) linear-attention kernels, or of the delta-rule kernels."""
-    lib = _lib.load()
-    return int((lib.mrx_delta_chunk_size if delta else lib.mrx_chunk_size)(_DT[dtype]))
+    c = _chunk_sizes.get((dtype, delta))
+    if c is None:
+        lib = _lib.load()
+        c = _chunk_sizes[(dtype, delta)] = int((lib.mrx_delta_chunk_size if delta else lib.mrx_chunk_size)(_DT[dtype]))
+    return c
 
 
 # ----------------------------------------------------------------- diagonal scan
