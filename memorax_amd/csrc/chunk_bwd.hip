@@ -25,6 +25,7 @@
 
 
 namespace {
+inline namespace MRX_HD_NS {
 
 using namespace mrx;
 
@@ -1090,6 +1091,7 @@ int check_bwd(const void *q, const void *k, const void *v, const void *done, con
     return MRX_OK;
 }
 
+}  // namespace MRX_HD_NS
 }  // namespace
 
 MRX_EXPORT int MRX_API(mrx_linear_attn_bwd)(void *stream, const void *q, const void *k, const void *v,
@@ -1200,6 +1202,7 @@ MRX_EXPORT int MRX_API(mrx_gated_linear_attn_bwd)(void *stream, const void *q, c
 }
 
 namespace {
+inline namespace MRX_HD_NS {
 
 template <typename T, int C, bool PRO> struct DeltaBwdReg {
     static constexpr int NW = 4;
@@ -1240,6 +1243,7 @@ int delta_bwd_entry(void *stream, const void *q, const void *k, const void *v, c
                                             dk_out, dv_out, dbeta, dS0, B, T, H);
 }
 
+}  // namespace MRX_HD_NS
 }  // namespace
 
 MRX_EXPORT int MRX_API(mrx_delta_rule_bwd)(void *stream, const void *q, const void *k, const void *v,

@@ -22,6 +22,7 @@
 #endif
 
 namespace {
+inline namespace MRX_HD_NS {
 
 using namespace mrx;
 
@@ -642,6 +643,7 @@ static __device__ __align__(256) unsigned char scratch[MRX_NOALLOC_SCRATCH_BYTES
 void *g_scratch_ptr[64] = {nullptr};
 
 #endif
+}  // namespace MRX_HD_NS
 }  // namespace
 
 #if MRX_HD == 64

@@ -19,6 +19,7 @@
 #endif
 
 namespace {
+inline namespace MRX_HD_NS {
 
 using namespace mrx;
 
@@ -130,6 +131,7 @@ int launch_step(hipStream_t st, const void *q, const void *k, const void *v, con
                          z_out, (int)H, eps);
 }
 
+}  // namespace MRX_HD_NS
 }  // namespace
 
 MRX_EXPORT int MRX_API(mrx_linear_attn_step)(void *stream, const void *q, const void *k, const void *v, const void *done,
