@@ -89,3 +89,51 @@ def test_graph_replays_of_forward_and_backward():
         ref = [ef[0], ef[1]] + list(eb[:4]) + [eh]
         for i, (a, b) in enumerate(zip(got, ref)):
             assert torch.equal(a, b), (rep, i)
+
+
+def test_graph_replays_of_the_chunk_parallel_pair_and_the_gated_backward():
+    """The chunk-parallel pair enqueues three kernels per call, the gated backward carries its running
+    sum for dg across chunks, and head dim 32 runs the library's second build: captured once, replayed
+    on fresh inputs with eager work in between, every replay equal to the eager calls bit for bit."""
+    from memorax_amd import kernels as K
+    K.init()
+    B, T, H, d = 2, 700, 2, 32
+    gen = torch.Generator(device="cuda").manual_seed(3)
+
+    def fresh():
+        x = {n: (torch.randn((B, T, H, d), device="cuda", generator=gen) / 6).to(torch.bfloat16) for n in ("q", "k", "v", "do")}
+        x["g"] = -torch.rand((B, T, H), device="cuda", generator=gen) * 0.3
+        x["done"] = (torch.rand((B, T), device="cuda", generator=gen) < 0.01).to(torch.uint8)
+        return x
+
+    static = fresh()
+
+    def work():
+        o, Sl, chk = K.linear_attn_fwd(static["q"], static["k"], static["v"], static["done"], None, 1, chunk_parallel=True)
+        gr = K.linear_attn_bwd(static["q"], static["k"], static["v"], static["done"], chk, static["do"], Sl, 1)
+        o2, Sl2, chk2 = K.gated_linear_attn_fwd(static["q"], static["k"], static["v"], static["g"], static["done"], None, 0)
+        gr2 = K.gated_linear_attn_bwd(static["q"], static["k"], static["v"], static["g"], static["done"], chk2,
+                                      static["do"], Sl2, 0, S_last=Sl2)
+        return [o, Sl, *gr, o2, Sl2, *gr2]
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        work()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        outs = work()
+    for rep in range(3):
+        new = fresh()
+        for n, t in new.items():
+            static[n].copy_(t)
+        g.replay()
+        torch.cuda.synchronize()
+        got = [x.clone() for x in outs]
+        _ = (torch.randn(128, 128, device="cuda") @ torch.randn(128, 128, device="cuda")).sum().item()
+        ref = work()
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip(got, ref)):
+            assert torch.equal(a, b), (rep, i)
