@@ -38,7 +38,7 @@ extern "C" {
 typedef enum {
     MRX_OK = 0,
     MRX_ERR_INVALID_ARG = -1, /* null pointer, non-positive size, bad enum, misalignment */
-    MRX_ERR_UNSUPPORTED = -2, /* valid request the kernels do not cover (e.g. a head dim other than 64 or 32) */
+    MRX_ERR_UNSUPPORTED = -2, /* valid request the kernels do not cover (e.g. a head dim the kernels are not built for) */
     MRX_ERR_LAUNCH = -3,      /* the HIP runtime rejected the launch */
     MRX_ERR_SCRATCH = -4      /* the problem exceeds the library's static scratch buffer (mrx_delta_rule_fwd_noalloc) */
 } mrx_status;
@@ -134,7 +134,13 @@ int mrx_linear_scan_bwd(void *stream, const void *a, const void *h,
  * S_chk (nullable): (B,H,ceil(T/chunk),dv,dk) float32, sparse (see mrx_chunk_size): receives the
  * state entering each chunk that contains a reset; required by the backward call together with
  * S_last.  dk = dv = 64 or dk = dv = 32 (here and in every chunked and single-step entry point below;
- * the library holds a build of those kernels for either width; mrx_delta_rule_fwd_noalloc: 64 only). */
+ * the library holds a build of those kernels for either width; mrx_delta_rule_fwd_noalloc: 64 only).
+ * Narrow heads: the linear-attention family -- mrx_linear_attn_*, mrx_gated_linear_attn_*,
+ * mrx_linear_attn_norm_*, mrx_linear_attn_*_chunk_parallel and mrx_linear_attn_step -- also takes any
+ * dk <= 32 and dv <= 32, independent of one another, whose rows are a whole number of 16-byte segments
+ * (multiples of 4 in float32, of 8 in bfloat16; the reference's guides use head_dim = 16).  Every array
+ * keeps its dense (.., dv, dk) / (.., dk) / (.., dv) layout at those widths; the 32-wide kernels pad
+ * on the fly.  The delta-rule entry points keep to 64 and 32. */
 int mrx_linear_attn_fwd(void *stream, const void *q, const void *k,
                         const void *v, const void *done, const void *S0,
                         void *o, void *S_last, void *S_chk, int64_t B,
@@ -346,7 +352,8 @@ int mrx_gated_linear_attn_bwd(void *stream, const void *q, const void *k,
  * What Memoroid.__call__ (memoroid.py:93-109) computes when T = 1, as PPO's rollout
  * does once per environment step (algorithms/ppo.py:105-143): one update of the
  * carry fused with the read-out, without the chunk machinery.
- *   q,k,v,o: (B,1,H,d) = (B,H,d) in `dtype`, d = 64 or 32; done: (B,) ; S_in/S_out: (B,H,dv,dk) fp32.
+ *   q,k,v,o: (B,1,H,d) = (B,H,d) in `dtype`, d = 64 or 32 (mrx_linear_attn_step: narrow heads too, see
+ *   mrx_linear_attn_fwd); done: (B,) ; S_in/S_out: (B,H,dv,dk) fp32.
  * S_in may be NULL (zero state) and may equal S_out (update in place).
  *
  * Linear attention (linear_attention.py:62-117):

@@ -17,6 +17,8 @@
 // Every tile lives in LDS once, in its natural orientation; products that contract over
 // the row index read it through transpose loads (KROW operands).  Gradients leave through dead
 // LDS tiles and are written to memory row-wise (tile_rows_to_global).
+#include <type_traits>
+
 #include "chunk_common.h"
 #include "la_states.h"
 #if MRX_HD == 64
@@ -84,13 +86,16 @@ struct NormBwdArgs {
 // fp32, the state entering chunk c and slot c of dS_last -- then a (B,H,NC,64,64) array -- the gradient
 // of the state leaving it (la_states.h); the workgroup forms the chunk's dQ, dK, dV from them and neither
 // walks the state nor accumulates its gradient.
-template <typename T, int C, bool FMAP, bool GATED, bool NORM, bool PAR = false>
+// RAG: narrow heads, as in the forward kernel: q, k and their gradients are dka wide in memory, v, dout, o and
+// dv dva, states [dva][dka], z [dka]; tiles keep the build's width, zero beyond, and only the rows' own
+// width is ever stored.
+template <typename T, int C, bool FMAP, bool GATED, bool NORM, bool PAR = false, bool RAG = false>
 __global__ void __launch_bounds__(256, 2)
 la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
               const float *__restrict__ glog, const void *__restrict__ done, int done_f32,
               const void *__restrict__ S_chk, const float *__restrict__ S_last, const T *__restrict__ dout,
               const float *__restrict__ dS_last, T *__restrict__ dq, T *__restrict__ dk, T *__restrict__ dv, float *__restrict__ dg,
-              float *__restrict__ dS0, int Tlen, int H, NormBwdArgs na)
+              float *__restrict__ dS0, int Tlen, int H, NormBwdArgs na, int dka, int dva)
 {
     static_assert(!(GATED && NORM), "the normalised read-out belongs to plain linear attention");
     static_assert(!PAR || (!GATED && !NORM), "one workgroup per chunk: plain linear attention only");
@@ -122,11 +127,15 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lg = lane >> 4;
     const int bh = sequence_of_block(blockIdx.x, gridDim.x, H), b = bh / H, h = bh % H;
-    const int64_t rs = (int64_t)H * HD;
-    const int64_t base = ((int64_t)b * Tlen * H + h) * HD;
+    const int dkw = RAG ? dka : HD, dvw = RAG ? dva : HD;  // row widths in memory
+    const int64_t rs = (int64_t)H * dkw, rsv = (int64_t)H * dvw;  // row strides of q, k / v, dout, o
+    const int64_t base = ((int64_t)b * Tlen * H + h) * dkw, basev = ((int64_t)b * Tlen * H + h) * dvw;
+    const bool segk = !RAG || (tid % (HD / TT<T>::KP)) * TT<T>::KP < dkw;  // this thread's 16-byte segment lies inside a q/k row
+    const bool segv = !RAG || (tid % (HD / TT<T>::KP)) * TT<T>::KP < dvw;  // ... inside a v row
     const int NC = (Tlen + C - 1) / C;
     const int c_hi = PAR ? (int)blockIdx.y : NC - 1, c_lo = PAR ? c_hi : 0;  // the chunks this workgroup walks, downwards
-    const int64_t slot = PAR ? ((int64_t)bh * NC + c_hi) * HD : (int64_t)bh * HD;  // in rows of 64 floats
+    const int64_t slot = PAR ? ((int64_t)bh * NC + c_hi) * dvw : (int64_t)bh * dvw;  // in state rows
+    auto in_state = [&](int dvv, int dk0) { return !RAG || (dvv < dvw && dk0 < dkw); };
 
     using TMS = TileMap<HD, HD, NW>;
     using TMA = TileMap<C, C, NW>;
@@ -135,8 +144,8 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 #pragma unroll
     for (int j = 0; j < TMS::TPW; ++j) {
         const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
-        dSacc[j] = dS_last ? *reinterpret_cast<const f32x4 *>(dS_last + (slot + dvv) * HD + dk0)
-                           : f32x4{0.f, 0.f, 0.f, 0.f};
+        dSacc[j] = dS_last && in_state(dvv, dk0) ? *reinterpret_cast<const f32x4 *>(dS_last + (slot + dvv) * dkw + dk0)
+                                                 : f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
     // normalised read-out: dz[dk], held like a column of dS^T; fp32 (VN): component 0 holds
@@ -148,8 +157,8 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
         const int dkt = TMS::mt(w, mi * TMS::NBW) * 16;
         dzacc[mi] = f32x4{0.f, 0.f, 0.f, 0.f};
         if (NORM && na.dz_last) {
-            if (VN) dzacc[mi][0] = na.dz_last[(int64_t)bh * HD + dkt + li];
-            else dzacc[mi] = *reinterpret_cast<const f32x4 *>(na.dz_last + (int64_t)bh * HD + dkt + 4 * lg);
+            if (VN) { if (!RAG || dkt + li < dkw) dzacc[mi][0] = na.dz_last[(int64_t)bh * dkw + dkt + li]; }
+            else if (!RAG || dkt + 4 * lg < dkw) dzacc[mi] = *reinterpret_cast<const f32x4 *>(na.dz_last + (int64_t)bh * dkw + dkt + 4 * lg);
         }
     }
 
@@ -166,8 +175,9 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 #pragma unroll
         for (int j = 0; j < NSA; ++j) {
             const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
-            Sacc[j] = *reinterpret_cast<const f32x4 *>((PAR ? reinterpret_cast<const float *>(S_chk) : S_last) +
-                                                       (slot + dvv) * HD + dk0);
+            if (in_state(dvv, dk0))
+                Sacc[j] = *reinterpret_cast<const f32x4 *>((PAR ? reinterpret_cast<const float *>(S_chk) : S_last) +
+                                                           (slot + dvv) * dkw + dk0);
         }
     }
 
@@ -178,7 +188,8 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 #pragma unroll
         for (int j = 0; j < TMS::TPW; ++j) {
             const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
-            const f32x4 sl = *reinterpret_cast<const f32x4 *>(S_last + ((int64_t)bh * HD + dvv) * HD + dk0);
+            if (!in_state(dvv, dk0)) continue;
+            const f32x4 sl = *reinterpret_cast<const f32x4 *>(S_last + ((int64_t)bh * dvw + dvv) * dkw + dk0);
             part += dSacc[j][0] * sl[0] + dSacc[j][1] * sl[1] + dSacc[j][2] * sl[2] + dSacc[j][3] * sl[3];
         }
 #pragma unroll
@@ -207,16 +218,19 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     // part 0: q, k; 1: v, dout; 2: S and the per-row scalars.
     const int tlast = c_hi * C;
     int64_t roff[IO::PASSES];
+    int64_t roffv[RAG ? IO::PASSES : 1];  // v, dout, o where their rows are not as wide as those of q and k
 #pragma unroll
-    for (int p = 0; p < IO::PASSES; ++p)
+    for (int p = 0; p < IO::PASSES; ++p) {
         roff[p] = base + (int64_t)(tlast + IO::row_of(tid, p)) * rs + (tid % IO::SEGS) * IO::KP;
-    int64_t soff = ((int64_t)bh * NC + c_hi) * HD * HD +
-                   (WALK ? li * HD + 4 * lg : (tid / IOS::SEGS) * HD + (tid % IOS::SEGS) * IOS::KP);
+        if (RAG) roffv[p] = basev + (int64_t)(tlast + IO::row_of(tid, p)) * rsv + (tid % IO::SEGS) * IO::KP;
+    }
+    int64_t soff = ((int64_t)bh * NC + c_hi) * dvw * dkw +
+                   (WALK ? li * dkw + 4 * lg : (tid / IOS::SEGS) * dkw + (tid % IOS::SEGS) * IOS::KP);
     int64_t doff = (int64_t)b * Tlen + tlast + lane;
     int64_t noff[IO::PASSES];  // den of the rows this thread stages
 #pragma unroll
     for (int p = 0; p < IO::PASSES; ++p) noff[p] = (int64_t)bh * Tlen + tlast + IO::row_of(tid, p);  // den: (B,H,T)
-    int64_t zoff = ((int64_t)bh * NC + c_hi) * HD + 4 * (tid % (HD / 4));
+    int64_t zoff = ((int64_t)bh * NC + c_hi) * dkw + 4 * (tid % (HD / 4));
     int tpre = tlast;
     auto prefetch_part = [&](int part) {
         typename IO::F z;
@@ -227,27 +241,35 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             for (int p = 0; p < IO::PASSES; ++p) {
                 const bool in = (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen;
                 if (part == 0) {
-                    rq.v[p] = in ? *reinterpret_cast<const typename IO::F *>(q + roff[p]) : z;
-                    rk.v[p] = in ? *reinterpret_cast<const typename IO::F *>(k + roff[p]) : z;
+                    rq.v[p] = in && segk ? *reinterpret_cast<const typename IO::F *>(q + roff[p]) : z;
+                    rk.v[p] = in && segk ? *reinterpret_cast<const typename IO::F *>(k + roff[p]) : z;
                 } else {
-                    rv.v[p] = in ? *reinterpret_cast<const typename IO::F *>(v + roff[p]) : z;
-                    rdo.v[p] = in ? *reinterpret_cast<const typename IO::F *>(dout + roff[p]) : z;
-                    if (NORM) ro.v[p] = in ? *reinterpret_cast<const typename IO::F *>((const T *)na.o + roff[p]) : z;
+                    const int64_t ov = RAG ? roffv[p] : roff[p];
+                    rv.v[p] = in && segv ? *reinterpret_cast<const typename IO::F *>(v + ov) : z;
+                    rdo.v[p] = in && segv ? *reinterpret_cast<const typename IO::F *>(dout + ov) : z;
+                    if (NORM) ro.v[p] = in && segv ? *reinterpret_cast<const typename IO::F *>((const T *)na.o + ov) : z;
                 }
             }
         } else {
             if (!WALK) {
 #pragma unroll
                 for (int p = 0; p < IOS::PASSES; ++p)
-                    if (IOS::FULL || IOS::row_of(tid, p) < HD)  // a [32][32] tile has fewer segments than threads
-                        rS.v[p] = *reinterpret_cast<const typename IOS::F *>(reinterpret_cast<const T *>(S_chk) + soff + p * IOS::RPP * HD);
+                    if (IOS::FULL || IOS::row_of(tid, p) < HD) {  // a [32][32] tile has fewer segments than threads
+                        if (!RAG || (IOS::row_of(tid, p) < dvw && (tid % IOS::SEGS) * IOS::KP < dkw))
+                            rS.v[p] = *reinterpret_cast<const typename IOS::F *>(reinterpret_cast<const T *>(S_chk) + soff + p * IOS::RPP * dkw);
+                        else
+                            rS.v[p] = z;
+                    }
             } else if (need_S) {
                 // straight into the state registers: the chunk at hand has formed its state (the first
                 // phase), and the next chunk, taking a checkpoint, does not walk back from it
 #pragma unroll
                 for (int j = 0; j < NSA; ++j)
-                    Sacc[j] = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(S_chk) + soff +
-                                                               TMS::nt(w, j) * 16 * HD + TMS::mt(w, j) * 16);
+                    if (in_state(TMS::nt(w, j) * 16 + li, TMS::mt(w, j) * 16 + 4 * lg))
+                        Sacc[j] = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(S_chk) + soff +
+                                                                   TMS::nt(w, j) * 16 * dkw + TMS::mt(w, j) * 16);
+                    else
+                        Sacc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
             rdone = 0u;
             rdone2 = 0u;
@@ -263,12 +285,15 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     rden[p] = (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen ? na.den[noff[p]] : 1.f;
                     noff[p] -= C;
                 }
-                rz = *reinterpret_cast<const f32x4 *>(na.z_chk + zoff);
-                zoff -= HD;
+                if (!RAG || 4 * (tid % (HD / 4)) < dkw) rz = *reinterpret_cast<const f32x4 *>(na.z_chk + zoff);
+                zoff -= dkw;
             }
 #pragma unroll
-            for (int p = 0; p < IO::PASSES; ++p) roff[p] -= (int64_t)C * rs;
-            soff -= HD * HD;
+            for (int p = 0; p < IO::PASSES; ++p) {
+                roff[p] -= (int64_t)C * rs;
+                if (RAG) roffv[p] -= (int64_t)C * rsv;
+            }
+            soff -= dvw * dkw;
             doff -= C;
             tpre -= C;
         }
@@ -287,9 +312,9 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
         if (pend_t0 >= 0) {
             auto keep = [&](int r) { return pend_nres == 0 || episode_of(pend_dmask, r) == pend_pass; };
             const int64_t off = base + (int64_t)pend_t0 * rs;
-            tile_rows_to_global<T, C, NTHR>(sV, LDD, dv + off, rs, pend_t0, Tlen, tid, keep);
-            tile_rows_to_global<T, C, NTHR>(sQ, LDD, dq + off, rs, pend_t0, Tlen, tid, keep);
-            tile_rows_to_global<T, C, NTHR>(sK, LDD, dk + off, rs, pend_t0, Tlen, tid, keep);
+            tile_rows_to_global<T, C, NTHR>(sV, LDD, dv + basev + (int64_t)pend_t0 * rsv, rsv, pend_t0, Tlen, tid, keep, dvw);
+            tile_rows_to_global<T, C, NTHR>(sQ, LDD, dq + off, rs, pend_t0, Tlen, tid, keep, dkw);
+            tile_rows_to_global<T, C, NTHR>(sK, LDD, dk + off, rs, pend_t0, Tlen, tid, keep, dkw);
         }
         pend_t0 = -1;
     };
@@ -333,8 +358,10 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             // ---- stage -------------------------------------------------------------
             {
                 typename IO::Regs fq = rq, fk = rk, fv = rv, fdo = rdo;
-                IO::template fmap<FMAP>(fq);
-                IO::template fmap<FMAP>(fk);
+                if (segk) {  // columns beyond a narrow head's width stay zero: phi(0) = 1 must not count
+                    IO::template fmap<FMAP>(fq);
+                    IO::template fmap<FMAP>(fk);
+                }
                 if (nres != 0) {
                     IO::mask_rows(fq, tid, live);
                     IO::mask_rows(fk, tid, live);
@@ -434,9 +461,12 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     if (!PAR && c == NC - 1) {  // the one checkpoint no prefetch could know of (PAR: loaded at the start)
 #pragma unroll
                         for (int j = 0; j < NSA; ++j)
-                            Sacc[j] = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(S_chk) +
-                                                                       ((int64_t)bh * NC + c) * HD * HD + li * HD + 4 * lg +
-                                                                       TMS::nt(w, j) * 16 * HD + TMS::mt(w, j) * 16);
+                            if (in_state(TMS::nt(w, j) * 16 + li, TMS::mt(w, j) * 16 + 4 * lg))
+                                Sacc[j] = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(S_chk) +
+                                                                           ((int64_t)bh * NC + c) * dvw * dkw + li * dkw + 4 * lg +
+                                                                           TMS::nt(w, j) * 16 * dkw + TMS::mt(w, j) * 16);
+                            else
+                                Sacc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
                     }  // else the prefetch of the chunk before has left the checkpoint in Sacc
                     store_acc<T, HD, HD, NW>(Sacc, sS, LDD, w, lane);
                 } else {
@@ -602,15 +632,16 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 #pragma unroll
         for (int j = 0; j < TMS::TPW; ++j) {
             const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
-            *reinterpret_cast<f32x4 *>(dS0 + ((int64_t)bh * HD + dvv) * HD + dk0) = dSacc[j];
+            if (in_state(dvv, dk0)) *reinterpret_cast<f32x4 *>(dS0 + ((int64_t)bh * dvw + dvv) * dkw + dk0) = dSacc[j];
         }
     }
     if (NORM && na.dz0 && w < TMS::WM && (VN ? lg == 0 : li == 0)) {
 #pragma unroll
         for (int mi = 0; mi < TMS::MBW; ++mi) {
-            float *dst = na.dz0 + (int64_t)bh * HD + TMS::mt(w, mi * TMS::NBW) * 16;
-            if (VN) dst[li] = dzacc[mi][0];
-            else *reinterpret_cast<f32x4 *>(dst + 4 * lg) = dzacc[mi];
+            const int dkt = TMS::mt(w, mi * TMS::NBW) * 16;
+            float *dst = na.dz0 + (int64_t)bh * dkw + dkt;
+            if (VN) { if (!RAG || dkt + li < dkw) dst[li] = dzacc[mi][0]; }
+            else if (!RAG || dkt + 4 * lg < dkw) *reinterpret_cast<f32x4 *>(dst + 4 * lg) = dzacc[mi];
         }
     }
 }
@@ -1050,39 +1081,49 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     }
 }
 
-template <typename T, int C, bool FMAP, bool GATED, bool NORM, bool PAR> struct LaBwdReg {
+template <typename T, int C, bool FMAP, bool GATED, bool NORM, bool PAR, bool RAG> struct LaBwdReg {
     static constexpr int smem = LaBwdSmem<T, C, GATED, NORM>::total;
-    static inline KernelRegistrar reg{reinterpret_cast<const void *>(la_bwd_kernel<T, C, FMAP, GATED, NORM, PAR>), smem};
+    static inline KernelRegistrar reg{reinterpret_cast<const void *>(la_bwd_kernel<T, C, FMAP, GATED, NORM, PAR, RAG>), smem};
 };
 
 template <typename T, int C, bool FMAP, bool GATED = false, bool NORM = false, bool PAR = false>
 int launch_la(hipStream_t st, const void *q, const void *k, const void *v, const void *done,
               int done_f32, const void *S_chk, const void *S_last, const void *dout, const void *dS_last, void *dq,
               void *dk, void *dv, void *dS0, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr,
-              void *dg = nullptr, NormBwdArgs na = NormBwdArgs{})
+              void *dg = nullptr, NormBwdArgs na = NormBwdArgs{}, int64_t dka = HD, int64_t dva = HD)
 {
-    using Reg = LaBwdReg<T, C, FMAP, GATED, NORM, PAR>;
-    (void)&Reg::reg;  // the kernel is on the list mrx_init() walks
     if (const int rc = prepare_device(); rc != MRX_OK) return rc;
     const int64_t NC = (Tlen + C - 1) / C;
     if (PAR && NC > 65535) return MRX_ERR_INVALID_ARG;
-    return launch_kernel(la_bwd_kernel<T, C, FMAP, GATED, NORM, PAR>, dim3((unsigned)(B * H), PAR ? (unsigned)NC : 1u),
-                         dim3(256), Reg::smem, st,
-                         (const T *)q, (const T *)k, (const T *)v, (const float *)glog, done, done_f32,
-                         S_chk, (const float *)S_last, (const T *)dout, (const float *)dS_last, (T *)dq, (T *)dk, (T *)dv,
-                         (float *)dg, (float *)dS0, (int)Tlen, (int)H, na);
+    auto go = [&](auto rag) {
+        constexpr bool RAG = decltype(rag)::value;
+        using Reg = LaBwdReg<T, C, FMAP, GATED, NORM, PAR, RAG>;
+        (void)&Reg::reg;  // the kernel is on the list mrx_init() walks
+        return launch_kernel(la_bwd_kernel<T, C, FMAP, GATED, NORM, PAR, RAG>,
+                             dim3((unsigned)(B * H), PAR ? (unsigned)NC : 1u), dim3(256), Reg::smem, st, (const T *)q,
+                             (const T *)k, (const T *)v, (const float *)glog, done, done_f32, S_chk,
+                             (const float *)S_last, (const T *)dout, (const float *)dS_last, (T *)dq, (T *)dk, (T *)dv,
+                             (float *)dg, (float *)dS0, (int)Tlen, (int)H, na, (int)dka, (int)dva);
+    };
+    if constexpr (MRX_HD == 32) {
+        if (dka != HD || dva != HD) return go(std::true_type{});  // narrow heads
+    }
+    return go(std::false_type{});
 }
 
 int check_bwd(const void *q, const void *k, const void *v, const void *done, const void *S_chk,
               const void *dout, const void *dS_last, const void *dq, const void *dk_out,
               const void *dv_out, const void *dS0, int64_t B, int64_t T, int64_t H, int64_t dk,
-              int64_t dv, int dtype, int done_dtype)
+              int64_t dv, int dtype, int done_dtype, bool narrow = false)
 {
     if (!q || !k || !v || !done || !S_chk || !dout || !dq || !dk_out || !dv_out) return MRX_ERR_INVALID_ARG;
     if (B <= 0 || T <= 0 || H <= 0 || dk <= 0 || dv <= 0) return MRX_ERR_INVALID_ARG;
     if (dtype != MRX_F32 && dtype != MRX_BF16) return dtype == MRX_C64 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
     if (done_dtype != MRX_DONE_U8 && done_dtype != MRX_DONE_F32) return MRX_ERR_INVALID_ARG;
-    if (dk != HD || dv != HD) return MRX_ERR_UNSUPPORTED;
+    // narrow: linear attention in the head dim 32 build also takes narrower rows of whole 16-byte segments
+    const int64_t seg = dtype == MRX_BF16 ? 8 : 4;
+    const bool narrow_ok = narrow && MRX_HD == 32 && dk <= HD && dv <= HD && dk % seg == 0 && dv % seg == 0;
+    if ((dk != HD || dv != HD) && !narrow_ok) return MRX_ERR_UNSUPPORTED;
     if (B * H >= (1ll << 31) || T >= (1ll << 30)) return MRX_ERR_INVALID_ARG;
     const void *ps[] = {q, k, v, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0};
     for (const void *p : ps)
@@ -1101,16 +1142,16 @@ MRX_EXPORT int MRX_API(mrx_linear_attn_bwd)(void *stream, const void *q, const v
                                    int dtype, int done_dtype, int feature_map)
 {
 #if MRX_HD == 64
-    if (dk == 32 && dv == 32) return mrx_linear_attn_bwd_hd32(stream, q, k, v, done, S_chk, S_last, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk, dv, dtype, done_dtype, feature_map);
+    if (dk <= 32 && dv <= 32) return mrx_linear_attn_bwd_hd32(stream, q, k, v, done, S_chk, S_last, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk, dv, dtype, done_dtype, feature_map);
 #endif
     const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
-                             dv, dtype, done_dtype);
+                             dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
     if (!S_last || !aligned(S_last, 16)) return MRX_ERR_INVALID_ARG;
     if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     const bool fm = feature_map == MRX_FMAP_ELU1;
-#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, S_last, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H
+#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, S_last, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, nullptr, nullptr, NormBwdArgs{}, dk, dv
     if (dtype == MRX_BF16) return fm ? launch_la<__bf16, LA_BF16_CHUNK, true>(MRX_ARGS) : launch_la<__bf16, LA_BF16_CHUNK, false>(MRX_ARGS);
     return fm ? launch_la<float, 32, true>(MRX_ARGS) : launch_la<float, 32, false>(MRX_ARGS);
 #undef MRX_ARGS
@@ -1123,10 +1164,10 @@ MRX_EXPORT int MRX_API(mrx_linear_attn_bwd_chunk_parallel)(void *stream, const v
                                                   int64_t dk, int64_t dv, int dtype, int done_dtype, int feature_map)
 {
 #if MRX_HD == 64
-    if (dk == 32 && dv == 32) return mrx_linear_attn_bwd_chunk_parallel_hd32(stream, q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, workspace, B, T, H, dk, dv, dtype, done_dtype, feature_map);
+    if (dk <= 32 && dv <= 32) return mrx_linear_attn_bwd_chunk_parallel_hd32(stream, q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, workspace, B, T, H, dk, dv, dtype, done_dtype, feature_map);
 #endif
     const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
-                             dv, dtype, done_dtype);
+                             dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
     if (!workspace || !aligned(workspace, 16)) return MRX_ERR_INVALID_ARG;
     if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
@@ -1135,11 +1176,11 @@ MRX_EXPORT int MRX_API(mrx_linear_attn_bwd_chunk_parallel)(void *stream, const v
     const int C = (int)mrx_chunk_size(dtype);
     if ((T + C - 1) / C > 65535) return MRX_ERR_INVALID_ARG;
     // per-chunk sums of do phi(q)^T -> gradients of the states leaving the chunks (and dS0) -> dQ, dK, dV
-    int rc2 = launch_la_chunk_states(st, q, dout, done, done_dtype, workspace, B, T, H, dtype, fm, true);
+    int rc2 = launch_la_chunk_states(st, q, dout, done, done_dtype, workspace, B, T, H, dtype, fm, true, dk, dv);
     if (rc2 != MRX_OK) return rc2;
-    rc2 = launch_la_state_scan(st, workspace, (const float *)dS_last, (float *)dS0, done, done_dtype, B, T, H, C, true);
+    rc2 = launch_la_state_scan(st, workspace, (const float *)dS_last, (float *)dS0, done, done_dtype, B, T, H, C, true, dk, dv);
     if (rc2 != MRX_OK) return rc2;
-#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, nullptr, dout, workspace, dq, dk_out, dv_out, nullptr, B, T, H
+#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, nullptr, dout, workspace, dq, dk_out, dv_out, nullptr, B, T, H, nullptr, nullptr, NormBwdArgs{}, dk, dv
     if (dtype == MRX_BF16)
         return fm ? launch_la<__bf16, LA_BF16_CHUNK, true, false, false, true>(MRX_ARGS)
                   : launch_la<__bf16, LA_BF16_CHUNK, false, false, false, true>(MRX_ARGS);
@@ -1157,10 +1198,10 @@ MRX_EXPORT int MRX_API(mrx_linear_attn_norm_bwd)(void *stream, const void *q, co
                                         float eps)
 {
 #if MRX_HD == 64
-    if (dk == 32 && dv == 32) return mrx_linear_attn_norm_bwd_hd32(stream, q, k, v, done, S_chk, S_last, z_chk, o, den, dout, dS_last, dz_last, dq, dk_out, dv_out, dS0, dz0, B, T, H, dk, dv, dtype, done_dtype, feature_map, eps);
+    if (dk <= 32 && dv <= 32) return mrx_linear_attn_norm_bwd_hd32(stream, q, k, v, done, S_chk, S_last, z_chk, o, den, dout, dS_last, dz_last, dq, dk_out, dv_out, dS0, dz0, B, T, H, dk, dv, dtype, done_dtype, feature_map, eps);
 #endif
     const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
-                             dv, dtype, done_dtype);
+                             dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
     if (!z_chk || !o || !den || !S_last || !aligned(S_last, 16)) return MRX_ERR_INVALID_ARG;
     if (!aligned(z_chk, 16) || !aligned(o, 16) || !aligned(den, 4) || !aligned(dz_last, 16) || !aligned(dz0, 16))
@@ -1169,7 +1210,7 @@ MRX_EXPORT int MRX_API(mrx_linear_attn_norm_bwd)(void *stream, const void *q, co
     hipStream_t st = (hipStream_t)stream;
     const bool fm = feature_map == MRX_FMAP_ELU1;
     const NormBwdArgs na{o, den, z_chk, dz_last, dz0, eps};
-#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, S_last, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, nullptr, nullptr, na
+#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, S_last, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, nullptr, nullptr, na, dk, dv
     if (dtype == MRX_BF16)
         return fm ? launch_la<__bf16, LA_BF16_CHUNK, true, false, true>(MRX_ARGS)
                   : launch_la<__bf16, LA_BF16_CHUNK, false, false, true>(MRX_ARGS);
@@ -1184,17 +1225,17 @@ MRX_EXPORT int MRX_API(mrx_gated_linear_attn_bwd)(void *stream, const void *q, c
                                          int64_t dk, int64_t dv, int dtype, int done_dtype, int feature_map)
 {
 #if MRX_HD == 64
-    if (dk == 32 && dv == 32) return mrx_gated_linear_attn_bwd_hd32(stream, q, k, v, g, done, S_chk, S_last, dout, dS_last, dq, dk_out, dv_out, dg, dS0, B, T, H, dk, dv, dtype, done_dtype, feature_map);
+    if (dk <= 32 && dv <= 32) return mrx_gated_linear_attn_bwd_hd32(stream, q, k, v, g, done, S_chk, S_last, dout, dS_last, dq, dk_out, dv_out, dg, dS0, B, T, H, dk, dv, dtype, done_dtype, feature_map);
 #endif
     const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
-                             dv, dtype, done_dtype);
+                             dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
     if (!g || !dg || !aligned(g, 4) || !aligned(dg, 4) || !aligned(S_last, 16)) return MRX_ERR_INVALID_ARG;
     if (dS_last && !S_last) return MRX_ERR_INVALID_ARG;  // <S_last, dS_last> enters dg at the last step
     if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     const bool fm = feature_map == MRX_FMAP_ELU1;
-#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, S_last, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, g, dg
+#define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, S_last, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, g, dg, NormBwdArgs{}, dk, dv
     if (dtype == MRX_BF16)
         return fm ? launch_la<__bf16, LA_BF16_CHUNK, true, true>(MRX_ARGS) : launch_la<__bf16, LA_BF16_CHUNK, false, true>(MRX_ARGS);
     return fm ? launch_la<float, 32, true, true>(MRX_ARGS) : launch_la<float, 32, false, true>(MRX_ARGS);

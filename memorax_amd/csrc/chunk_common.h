@@ -343,12 +343,14 @@ __device__ __forceinline__ float inv_norm(float ss) { return __builtin_amdgcn_rs
 // write one whole row, so a wave instruction covers full 128-byte lines -- against the four-feature
 // pieces (16 rows x 32 bytes per instruction) of a store from accumulators.  `g` points at row 0 of
 // the chunk.
+// ncols: width of the rows in memory when it is less than the tile's (narrow heads: the tile's further columns are padding).
 template <typename T, int C, int NTHR, typename KeepF>
 __device__ __forceinline__ void tile_rows_to_global(const T *tile, int ld, T *g, int64_t rs, int t0, int Tlen, int tid,
-                                                    KeepF keep)
+                                                    KeepF keep, int ncols = HD)
 {
     using IO = TileIO<T, C, NTHR>;
     const int seg = tid % IO::SEGS;
+    if (seg * IO::KP >= ncols) return;
 #pragma unroll
     for (int p = 0; p < IO::PASSES; ++p) {
         const int r = IO::row_of(tid, p);

@@ -14,6 +14,8 @@
 // non-finite value can never meet a masked-out zero inside a matrix product.
 // The state is kept transposed (S^T, d_k x d_v) in MFMA accumulators for the whole
 // sequence and re-staged to LDS as a T-typed d_v x d_k tile once per chunk.
+#include <type_traits>
+
 #include "chunk_common.h"
 #include "delta_tm.h"
 #include "la_states.h"
@@ -72,15 +74,21 @@ struct NormArgs {
 // PAR (plain linear attention): one workgroup per chunk (grid.y = chunk) instead of one per sequence.
 // S_chk then is an input: slot c holds, in fp32, the state entering chunk c (la_states.h); the
 // workgroup forms the chunk's outputs from it and neither updates nor writes any state.
+// RAG (linear attention, all variants): narrow heads.  Keys and queries are dka wide in memory, values
+// and outputs dva (both at most the head dim of the build, whole 16-byte segments), and so are the
+// states (B,H,dva,dka) and z (B,H,dka).  Tiles in LDS and registers keep the build's width: what lies
+// beyond the rows' width is loaded as zero (after the feature map, phi(0) = 1 must not count) and never
+// stored.
 template <typename T, int C, bool DELTA, bool FMAP, bool GATED, bool NORM, bool PRO = false, bool TMIN = false,
-          bool PAR = false>
+          bool PAR = false, bool RAG = false>
 __global__ void __launch_bounds__(NTHR, 2)  // 2 waves per SIMD: two workgroups share a CU
 chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const float *__restrict__ glog,
                  const void *__restrict__ done, int done_f32,
                  const float *__restrict__ S0, T *__restrict__ o, float *__restrict__ S_last,
-                 void *__restrict__ S_chk, T *__restrict__ Tm_chk, int Tlen, int H, NormArgs na)
+                 void *__restrict__ S_chk, T *__restrict__ Tm_chk, int Tlen, int H, NormArgs na, int dka, int dva)
 {
+    static_assert(!RAG || !DELTA, "narrow heads: linear attention only");
     static_assert(!(DELTA && GATED), "the gated variant is linear attention with a decay");
     static_assert(!NORM || (!DELTA && !GATED), "the normalised read-out belongs to plain linear attention");
     static_assert(!PRO || DELTA, "the prologue belongs to the delta rule");
@@ -113,8 +121,12 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lg = lane >> 4;
     const int bh = sequence_of_block(blockIdx.x, gridDim.x, H), b = bh / H, h = bh % H;
-    const int64_t rs = (int64_t)H * HD;  // row stride of q/k/v/o
-    const int64_t base = ((int64_t)b * Tlen * H + h) * HD;
+    const int dkw = RAG ? dka : HD, dvw = RAG ? dva : HD;  // row widths in memory
+    const int64_t rs = (int64_t)H * dkw;   // row stride of q/k
+    const int64_t rsv = (int64_t)H * dvw;  // ... of v/o
+    const int64_t base = ((int64_t)b * Tlen * H + h) * dkw, basev = ((int64_t)b * Tlen * H + h) * dvw;
+    const bool segk = !RAG || (tid % (HD / TT<T>::KP)) * TT<T>::KP < dkw;  // this thread's 16-byte segment lies inside a q/k row
+    const bool segv = !RAG || (tid % (HD / TT<T>::KP)) * TT<T>::KP < dvw;  // ... inside a v row
     const int NC = (Tlen + C - 1) / C;
     const int c_first = PAR ? (int)blockIdx.y : 0, c_end = PAR ? c_first + 1 : NC;  // the chunks this workgroup walks
 
@@ -126,12 +138,14 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
     for (int j = 0; j < TMS::TPW; ++j) {
         const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dv = TMS::nt(w, j) * 16 + li;
-        if (PAR)
-            Sacc[j] = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(S_chk) +
-                                                       (((int64_t)bh * NC + c_first) * HD + dv) * HD + dk0);
-        else
-            Sacc[j] = S0 ? *reinterpret_cast<const f32x4 *>(S0 + ((int64_t)bh * HD + dv) * HD + dk0)
-                         : f32x4{0.f, 0.f, 0.f, 0.f};
+        const bool in = !RAG || (dv < dvw && dk0 < dkw);
+        Sacc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (PAR) {
+            if (in) Sacc[j] = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(S_chk) +
+                                                              (((int64_t)bh * NC + c_first) * dvw + dv) * dkw + dk0);
+        } else if (S0 && in) {
+            Sacc[j] = *reinterpret_cast<const f32x4 *>(S0 + ((int64_t)bh * dvw + dv) * dkw + dk0);
+        }
     }
 
     // normalised read-out: z[dk] of the running episode.  bf16: held like a column of S^T (every
@@ -146,8 +160,8 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         const int dkt = TMS::mt(w, mi * TMS::NBW) * 16;
         zacc[mi] = f32x4{0.f, 0.f, 0.f, 0.f};
         if (NORM && na.z0) {
-            if (VN) zacc[mi][0] = na.z0[(int64_t)bh * HD + dkt + li];
-            else zacc[mi] = *reinterpret_cast<const f32x4 *>(na.z0 + (int64_t)bh * HD + dkt + 4 * lg);
+            if (VN) { if (!RAG || dkt + li < dkw) zacc[mi][0] = na.z0[(int64_t)bh * dkw + dkt + li]; }
+            else if (!RAG || dkt + 4 * lg < dkw) zacc[mi] = *reinterpret_cast<const f32x4 *>(na.z0 + (int64_t)bh * dkw + dkt + 4 * lg);
         }
     }
     const Frag ones = TT<T>::ones();
@@ -161,10 +175,12 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     // Element offsets of what this thread loads for the chunk about to be prefetched; they advance
     // by one chunk per call (64-bit adds instead of per-chunk index multiplications).
     int64_t roff[IO::PASSES], boff[IO::PASSES];
+    int64_t roffv[RAG ? IO::PASSES : 1];  // v, where its rows are not as wide as those of q and k
 #pragma unroll
     for (int p = 0; p < IO::PASSES; ++p) {
         const int r = IO::row_of(tid, p);
         roff[p] = base + (int64_t)(c_first * C + r) * rs + (tid % IO::SEGS) * IO::KP;  // q/k/v: row r, this thread's 16-byte segment
+        if (RAG) roffv[p] = basev + (int64_t)(c_first * C + r) * rsv + (tid % IO::SEGS) * IO::KP;
         boff[p] = ((int64_t)b * Tlen + c_first * C + r) * H + h;                       // beta of row r
     }
     int64_t doff = (int64_t)b * Tlen + c_first * C + lane;  // done of chunk row `lane`
@@ -180,15 +196,17 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         if (part < 3) {
             const T *src = part == 0 ? q : part == 1 ? k : v;
             typename IO::Regs &dst = part == 0 ? rq : part == 1 ? rk : rv;
+            const bool seg_in = part == 2 ? segv : segk;
 #pragma unroll
             for (int p = 0; p < IO::PASSES; ++p)
-                dst.v[p] = (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen
-                               ? *reinterpret_cast<const typename IO::F *>(src + roff[p]) : z;
+                dst.v[p] = seg_in && (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen
+                               ? *reinterpret_cast<const typename IO::F *>(src + (RAG && part == 2 ? roffv[p] : roff[p])) : z;
         } else {
 #pragma unroll
             for (int p = 0; p < IO::PASSES; ++p) {
                 if (DELTA) rbrow[p] = (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen ? load_raw<T>(beta + boff[p]) : 0u;
                 roff[p] += (int64_t)C * rs;
+                if (RAG) roffv[p] += (int64_t)C * rsv;
                 boff[p] += (int64_t)C * H;
             }
             if (TMIN) {
@@ -224,13 +242,13 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     auto flush_o = [&]() {  // call after a barrier that follows the writes to sO
         if (pend_t0 >= 0) {
             auto keep = [&](int r) { return pend_nres == 0 || episode_of(pend_dmask, r) == pend_pass; };
-            tile_rows_to_global<T, C, NTHR>(sO, LDD, o + base + (int64_t)pend_t0 * rs, rs, pend_t0, Tlen, tid, keep);
+            tile_rows_to_global<T, C, NTHR>(sO, LDD, o + basev + (int64_t)pend_t0 * rsv, rsv, pend_t0, Tlen, tid, keep, dvw);
         }
         pend_t0 = -1;
     };
-    int64_t schk_off = (int64_t)bh * NC * HD * HD;                                   // S_chk[c]
+    int64_t schk_off = (int64_t)bh * NC * dvw * dkw;                                 // S_chk[c]
     int64_t tmchk_off = (int64_t)bh * NC * C * C + (int64_t)tid * 4;                                  // row-major C x C
-    for (int c = c_first; c < c_end; ++c, schk_off += HD * HD, tmchk_off += C * C, den_off += C) {
+    for (int c = c_first; c < c_end; ++c, schk_off += dvw * dkw, tmchk_off += C * C, den_off += C) {
         const int t0 = c * C;
         const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
@@ -255,8 +273,10 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             // ---- stage the chunk ---------------------------------------------------
             {
                 typename IO::Regs fq = rq, fk = rk, fv = rv;
-                IO::template fmap<FMAP>(fq);
-                IO::template fmap<FMAP>(fk);
+                if (segk) {  // columns beyond a narrow head's width stay zero: phi(0) = 1 must not count
+                    IO::template fmap<FMAP>(fq);
+                    IO::template fmap<FMAP>(fk);
+                }
                 if (nres != 0) {
                     IO::mask_rows(fq, tid, live);
                     IO::mask_rows(fk, tid, live);
@@ -306,13 +326,13 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                     for (int mi = 0; mi < TMS::MBW; ++mi) {
                         const int dkt = TMS::mt(w, mi * TMS::NBW) * 16;
-                        float *zc = (na.z_chk && pass == 0) ? na.z_chk + ((int64_t)bh * NC + c) * HD + dkt : nullptr;
+                        float *zc = (na.z_chk && pass == 0) ? na.z_chk + ((int64_t)bh * NC + c) * dkw + dkt : nullptr;
                         if (VN) {
                             sZ[dkt + li] = (T)zacc[mi][0];
-                            if (zc) zc[li] = zacc[mi][0];
+                            if (zc && (!RAG || dkt + li < dkw)) zc[li] = zacc[mi][0];
                         } else {
                             *reinterpret_cast<P4 *>(sZ + dkt + 4 * lg) = TT<T>::pack(zacc[mi][0], zacc[mi][1], zacc[mi][2], zacc[mi][3]);
-                            if (zc) *reinterpret_cast<f32x4 *>(zc + 4 * lg) = zacc[mi];
+                            if (zc && (!RAG || dkt + 4 * lg < dkw)) *reinterpret_cast<f32x4 *>(zc + 4 * lg) = zacc[mi];
                         }
                     }
                 }
@@ -337,15 +357,16 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                     for (int p = 0; p < IOS::PASSES; ++p) {
                         const int r = IOS::row_of(tid, p), seg = tid % IOS::SEGS;
-                        if (IOS::FULL || r < HD)  // a [32][32] tile has fewer segments than threads
-                            *reinterpret_cast<typename IOS::F *>(reinterpret_cast<T *>(S_chk) + schk_off + r * HD + seg * IOS::KP) =
+                        if ((IOS::FULL || r < HD) && (!RAG || (r < dvw && seg * IOS::KP < dkw)))  // a [32][32] tile has fewer segments than threads
+                            *reinterpret_cast<typename IOS::F *>(reinterpret_cast<T *>(S_chk) + schk_off + r * dkw + seg * IOS::KP) =
                                 *reinterpret_cast<const typename IOS::F *>(sS + r * LDD + seg * IOS::KP);
                     }
                 } else {
 #pragma unroll
                     for (int j = 0; j < TMS::TPW; ++j) {
                         const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dv = TMS::nt(w, j) * 16 + li;
-                        *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(S_chk) + schk_off + dv * HD + dk0) = Sacc[j];
+                        if (!RAG || (dv < dvw && dk0 < dkw))
+                            *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(S_chk) + schk_off + dv * dkw + dk0) = Sacc[j];
                     }
                 }
             }
@@ -537,52 +558,68 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
         for (int j = 0; j < TMS::TPW; ++j) {
             const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dv = TMS::nt(w, j) * 16 + li;
-            *reinterpret_cast<f32x4 *>(S_last + ((int64_t)bh * HD + dv) * HD + dk0) = Sacc[j];
+            if (!RAG || (dv < dvw && dk0 < dkw))
+                *reinterpret_cast<f32x4 *>(S_last + ((int64_t)bh * dvw + dv) * dkw + dk0) = Sacc[j];
         }
     }
     if (NORM && na.z_last && w < TMS::WM && (VN ? lg == 0 : li == 0)) {
 #pragma unroll
         for (int mi = 0; mi < TMS::MBW; ++mi) {
-            float *zl = na.z_last + (int64_t)bh * HD + TMS::mt(w, mi * TMS::NBW) * 16;
-            if (VN) zl[li] = zacc[mi][0];
-            else *reinterpret_cast<f32x4 *>(zl + 4 * lg) = zacc[mi];
+            const int dkt = TMS::mt(w, mi * TMS::NBW) * 16;
+            float *zl = na.z_last + (int64_t)bh * dkw + dkt;
+            if (VN) { if (!RAG || dkt + li < dkw) zl[li] = zacc[mi][0]; }
+            else if (!RAG || dkt + 4 * lg < dkw) *reinterpret_cast<f32x4 *>(zl + 4 * lg) = zacc[mi];
         }
     }
 }
 
-template <typename T, int C, bool DELTA, bool FMAP, bool GATED, bool NORM, bool PRO, bool TMIN, bool PAR> struct FwdReg {
+template <typename T, int C, bool DELTA, bool FMAP, bool GATED, bool NORM, bool PRO, bool TMIN, bool PAR, bool RAG> struct FwdReg {
     static constexpr int smem = FwdSmem<T, C, DELTA, GATED, NORM>::total;
     static inline KernelRegistrar reg{
-        reinterpret_cast<const void *>(chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR>), smem};
+        reinterpret_cast<const void *>(chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR, RAG>), smem};
 };
 
+// dka, dva: widths of the q/k and v/o rows in memory; less than the build's head dim (narrow heads,
+// linear attention only, head dim 32 build) selects the kernel instance that pads on the fly.
 template <typename T, int C, bool DELTA, bool FMAP, bool GATED = false, bool NORM = false, bool PRO = false,
           bool TMIN = false, bool PAR = false>
 int launch(hipStream_t st, const void *q, const void *k, const void *v, const void *beta,
            const void *done, int done_f32, const void *S0, void *o, void *S_last, void *S_chk,
-           void *Tm_chk, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr, NormArgs na = NormArgs{})
+           void *Tm_chk, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr, NormArgs na = NormArgs{},
+           int64_t dka = HD, int64_t dva = HD)
 {
-    using Reg = FwdReg<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR>;
-    (void)&Reg::reg;  // the kernel is on the list mrx_init() walks
     if (const int rc = prepare_device(); rc != MRX_OK) return rc;
     const int64_t NC = (Tlen + C - 1) / C;
     if (PAR && NC > 65535) return MRX_ERR_INVALID_ARG;
-    return launch_kernel(chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR>,
-                         dim3((unsigned)(B * H), PAR ? (unsigned)NC : 1u),
-                         dim3(NTHR), Reg::smem, st, (const T *)q, (const T *)k, (const T *)v, (const T *)beta,
-                         (const float *)glog, done, done_f32, (const float *)S0, (T *)o, (float *)S_last, S_chk,
-                         (T *)Tm_chk, (int)Tlen, (int)H, na);
+    auto go = [&](auto rag) {
+        constexpr bool RAG = decltype(rag)::value;
+        using Reg = FwdReg<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR, RAG>;
+        (void)&Reg::reg;  // the kernel is on the list mrx_init() walks
+        return launch_kernel(chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR, RAG>,
+                             dim3((unsigned)(B * H), PAR ? (unsigned)NC : 1u), dim3(NTHR), Reg::smem, st, (const T *)q,
+                             (const T *)k, (const T *)v, (const T *)beta, (const float *)glog, done, done_f32,
+                             (const float *)S0, (T *)o, (float *)S_last, S_chk, (T *)Tm_chk, (int)Tlen, (int)H, na,
+                             (int)dka, (int)dva);
+    };
+    if constexpr (MRX_HD == 32 && !DELTA) {
+        if (dka != HD || dva != HD) return go(std::true_type{});
+    }
+    return go(std::false_type{});
 }
 
+// narrow: the entry point also serves heads narrower than the build's (linear attention in the head dim 32
+// build: rows of whole 16-byte segments, padded inside the kernels)
 int check_common(const void *q, const void *k, const void *v, const void *done, const void *o,
                  const void *S0, const void *S_last, const void *S_chk, int64_t B, int64_t T,
-                 int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype)
+                 int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype, bool narrow = false)
 {
     if (!q || !k || !v || !done || !o) return MRX_ERR_INVALID_ARG;
     if (B <= 0 || T <= 0 || H <= 0 || dk <= 0 || dv <= 0) return MRX_ERR_INVALID_ARG;
     if (dtype != MRX_F32 && dtype != MRX_BF16) return dtype == MRX_C64 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
     if (done_dtype != MRX_DONE_U8 && done_dtype != MRX_DONE_F32) return MRX_ERR_INVALID_ARG;
-    if (dk != HD || dv != HD) return MRX_ERR_UNSUPPORTED;
+    const int64_t seg = dtype == MRX_BF16 ? 8 : 4;  // elements per 16 bytes
+    const bool narrow_ok = narrow && MRX_HD == 32 && dk <= HD && dv <= HD && dk % seg == 0 && dv % seg == 0;
+    if ((dk != HD || dv != HD) && !narrow_ok) return MRX_ERR_UNSUPPORTED;
     if (B * H >= (1ll << 31) || T >= (1ll << 30)) return MRX_ERR_INVALID_ARG;
     if (!aligned(q, 16) || !aligned(k, 16) || !aligned(v, 16) || !aligned(o, 16) || !aligned(S0, 16) ||
         !aligned(S_last, 16) || !aligned(S_chk, 16))
@@ -668,18 +705,18 @@ MRX_EXPORT int MRX_API(mrx_linear_attn_fwd)(void *stream, const void *q, const v
                                    int64_t dv, int dtype, int done_dtype, int feature_map)
 {
 #if MRX_HD == 64
-    if (dk == 32 && dv == 32) return mrx_linear_attn_fwd_hd32(stream, q, k, v, done, S0, o, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, feature_map);
+    if (dk <= 32 && dv <= 32) return mrx_linear_attn_fwd_hd32(stream, q, k, v, done, S0, o, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, feature_map);
 #endif
-    const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
+    const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
     if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     const bool fm = feature_map == MRX_FMAP_ELU1;
     if (dtype == MRX_BF16)
-        return fm ? launch<__bf16, LA_BF16_CHUNK, false, true>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H)
-                  : launch<__bf16, LA_BF16_CHUNK, false, false>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H);
-    return fm ? launch<float, 32, false, true>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H)
-              : launch<float, 32, false, false>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H);
+        return fm ? launch<__bf16, LA_BF16_CHUNK, false, true>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H, nullptr, NormArgs{}, dk, dv)
+                  : launch<__bf16, LA_BF16_CHUNK, false, false>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H, nullptr, NormArgs{}, dk, dv);
+    return fm ? launch<float, 32, false, true>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H, nullptr, NormArgs{}, dk, dv)
+              : launch<float, 32, false, false>(st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H, nullptr, NormArgs{}, dk, dv);
 }
 
 MRX_EXPORT int MRX_API(mrx_linear_attn_fwd_chunk_parallel)(void *stream, const void *q, const void *k, const void *v,
@@ -688,9 +725,9 @@ MRX_EXPORT int MRX_API(mrx_linear_attn_fwd_chunk_parallel)(void *stream, const v
                                                   int64_t dv, int dtype, int done_dtype, int feature_map)
 {
 #if MRX_HD == 64
-    if (dk == 32 && dv == 32) return mrx_linear_attn_fwd_chunk_parallel_hd32(stream, q, k, v, done, S0, o, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, feature_map);
+    if (dk <= 32 && dv <= 32) return mrx_linear_attn_fwd_chunk_parallel_hd32(stream, q, k, v, done, S0, o, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, feature_map);
 #endif
-    const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
+    const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
     if (!S_chk) return MRX_ERR_INVALID_ARG;  // the per-chunk states live there
     if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
@@ -699,11 +736,11 @@ MRX_EXPORT int MRX_API(mrx_linear_attn_fwd_chunk_parallel)(void *stream, const v
     const int C = (int)mrx_chunk_size(dtype);
     if ((T + C - 1) / C > 65535) return MRX_ERR_INVALID_ARG;
     // per-chunk sums of v phi(k)^T -> states entering the chunks (and S_last) -> outputs, chunk by chunk
-    int rc2 = launch_la_chunk_states(st, k, v, done, done_dtype, S_chk, B, T, H, dtype, fm, false);
+    int rc2 = launch_la_chunk_states(st, k, v, done, done_dtype, S_chk, B, T, H, dtype, fm, false, dk, dv);
     if (rc2 != MRX_OK) return rc2;
-    rc2 = launch_la_state_scan(st, S_chk, (const float *)S0, (float *)S_last, done, done_dtype, B, T, H, C, false);
+    rc2 = launch_la_state_scan(st, S_chk, (const float *)S0, (float *)S_last, done, done_dtype, B, T, H, C, false, dk, dv);
     if (rc2 != MRX_OK) return rc2;
-#define MRX_ARGS st, q, k, v, nullptr, done, done_dtype, nullptr, o, nullptr, S_chk, nullptr, B, T, H
+#define MRX_ARGS st, q, k, v, nullptr, done, done_dtype, nullptr, o, nullptr, S_chk, nullptr, B, T, H, nullptr, NormArgs{}, dk, dv
     if (dtype == MRX_BF16)
         return fm ? launch<__bf16, LA_BF16_CHUNK, false, true, false, false, false, false, true>(MRX_ARGS)
                   : launch<__bf16, LA_BF16_CHUNK, false, false, false, false, false, false, true>(MRX_ARGS);
@@ -771,15 +808,15 @@ MRX_EXPORT int MRX_API(mrx_gated_linear_attn_fwd)(void *stream, const void *q, c
                                          int64_t dk, int64_t dv, int dtype, int done_dtype, int feature_map)
 {
 #if MRX_HD == 64
-    if (dk == 32 && dv == 32) return mrx_gated_linear_attn_fwd_hd32(stream, q, k, v, g, done, S0, o, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, feature_map);
+    if (dk <= 32 && dv <= 32) return mrx_gated_linear_attn_fwd_hd32(stream, q, k, v, g, done, S0, o, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, feature_map);
 #endif
-    const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
+    const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
     if (!g || !aligned(g, 4)) return MRX_ERR_INVALID_ARG;
     if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     const bool fm = feature_map == MRX_FMAP_ELU1;
-#define MRX_ARGS st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H, g
+#define MRX_ARGS st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H, g, NormArgs{}, dk, dv
     if (dtype == MRX_BF16)
         return fm ? launch<__bf16, LA_BF16_CHUNK, false, true, true>(MRX_ARGS) : launch<__bf16, LA_BF16_CHUNK, false, false, true>(MRX_ARGS);
     return fm ? launch<float, 32, false, true, true>(MRX_ARGS) : launch<float, 32, false, false, true>(MRX_ARGS);
@@ -793,9 +830,9 @@ MRX_EXPORT int MRX_API(mrx_linear_attn_norm_fwd)(void *stream, const void *q, co
                                         int done_dtype, int feature_map, float eps)
 {
 #if MRX_HD == 64
-    if (dk == 32 && dv == 32) return mrx_linear_attn_norm_fwd_hd32(stream, q, k, v, done, S0, z0, o, den, S_last, z_last, S_chk, z_chk, B, T, H, dk, dv, dtype, done_dtype, feature_map, eps);
+    if (dk <= 32 && dv <= 32) return mrx_linear_attn_norm_fwd_hd32(stream, q, k, v, done, S0, z0, o, den, S_last, z_last, S_chk, z_chk, B, T, H, dk, dv, dtype, done_dtype, feature_map, eps);
 #endif
-    const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
+    const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
     if (!den || !aligned(den, 4) || !aligned(z0, 16) || !aligned(z_last, 16) || !aligned(z_chk, 16))
         return MRX_ERR_INVALID_ARG;
@@ -803,7 +840,7 @@ MRX_EXPORT int MRX_API(mrx_linear_attn_norm_fwd)(void *stream, const void *q, co
     hipStream_t st = (hipStream_t)stream;
     const bool fm = feature_map == MRX_FMAP_ELU1;
     const NormArgs na{z0, den, z_last, z_chk, eps};
-#define MRX_ARGS st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H, nullptr, na
+#define MRX_ARGS st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H, nullptr, na, dk, dv
     if (dtype == MRX_BF16)
         return fm ? launch<__bf16, LA_BF16_CHUNK, false, true, false, true>(MRX_ARGS)
                   : launch<__bf16, LA_BF16_CHUNK, false, false, false, true>(MRX_ARGS);

@@ -23,16 +23,17 @@
 namespace mrx {
 inline namespace MRX_HD_NS {
 
-// slots[B][H][NC][64][64] fp32 <- per-chunk contributions.  x: keys (forward) or queries (backward),
-// y: values (forward) or output gradients (backward), both (B,T,H,64) of `dtype`; fmap: elu+1 on x.
+// slots[B][H][NC][dv][dk] fp32 <- per-chunk contributions.  x: keys (forward) or queries (backward),
+// (B,T,H,dk), y: values (forward) or output gradients (backward), (B,T,H,dv), of `dtype`; fmap: elu+1 on x.
+// dk, dv: the build's head dim, or less in whole 16-byte segments (narrow heads).
 // C is the chunk length of the linear-attention kernels for `dtype`.  Returns an MRX_* status.
 int launch_la_chunk_states(hipStream_t st, const void *x, const void *y, const void *done, int done_f32, float *slots,
-                           int64_t B, int64_t Tlen, int64_t H, int dtype, bool fmap, bool backward);
+                           int64_t B, int64_t Tlen, int64_t H, int dtype, bool fmap, bool backward, int64_t dk, int64_t dv);
 
-// In-place exclusive scan over the slots of every sequence (see above).  init: (B,H,64,64) fp32 or
-// null (zero); fin: (B,H,64,64) fp32 or null.  C: chunk length the slots were formed with.
+// In-place exclusive scan over the slots of every sequence (see above).  init: (B,H,dv,dk) fp32 or
+// null (zero); fin: (B,H,dv,dk) fp32 or null.  C: chunk length the slots were formed with.
 int launch_la_state_scan(hipStream_t st, float *slots, const float *init, float *fin, const void *done, int done_f32,
-                         int64_t B, int64_t Tlen, int64_t H, int C, bool backward);
+                         int64_t B, int64_t Tlen, int64_t H, int C, bool backward, int64_t dk, int64_t dv);
 
 }  // namespace MRX_HD_NS
 }  // namespace mrx

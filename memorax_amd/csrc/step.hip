@@ -13,6 +13,8 @@
 // fully coalesced 16-byte access; row dot products reduce over the lanes of a row.
 // Follows what Memoroid.__call__ computes for T = 1 (memoroid.py:93-109 with the cell algebra of
 // linear_attention.py:62-117) and the delta-rule recurrence of the chunked kernels.
+#include <type_traits>
+
 #include "chunk_common.h"
 #if MRX_HD == 64
 #include "hd32_api.h"
@@ -49,37 +51,43 @@ __device__ __forceinline__ float dot4(const f32x4 &a, const f32x4 &b)
     return a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
 }
 
-template <typename T, bool DELTA, bool FMAP>
+// RAG (linear attention, head dim 32 build): narrow heads -- q, k, z are dka wide, v, o dva, the state
+// [dva][dka]; lanes and rows beyond take no part.
+template <typename T, bool DELTA, bool FMAP, bool RAG = false>
 __global__ void __launch_bounds__(256)
 step_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
             const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
             const float *S_in, const float *z_in, T *__restrict__ o, float *S_out, float *z_out, int H,
-            float eps)  // S_in/S_out and z_in/z_out may alias (update in place)
+            float eps, int dka, int dva)  // S_in/S_out and z_in/z_out may alias (update in place)
 {
+    static_assert(!RAG || !DELTA, "narrow heads: linear attention only");
     const int tid = threadIdx.x, c4 = tid % LPR, r0 = tid / LPR;
     const int64_t bh = blockIdx.x;
     const int b = (int)(bh / H);
     const bool reset = done_at(done, done_f32, b);
-    const T *qp = q + bh * HD, *kp = k + bh * HD, *vp = v + bh * HD;
+    const int dkw = RAG ? dka : HD, dvw = RAG ? dva : HD;
+    const bool cin = !RAG || 4 * c4 < dkw;  // this lane's four dk lie inside a row
+    const T *qp = q + bh * dkw, *kp = k + bh * dkw, *vp = v + bh * dvw;
 
-    f32x4 k4 = load4<T>(kp + 4 * c4), q4 = load4<T>(qp + 4 * c4);
-    if (FMAP) {
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    f32x4 k4 = cin ? load4<T>(kp + 4 * c4) : zero4, q4 = cin ? load4<T>(qp + 4 * c4) : zero4;
+    if (FMAP && cin) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             k4[e] = elu1(k4[e]);
             q4[e] = elu1(q4[e]);
         }
     }
-    const float *Sp = S_in ? S_in + bh * HD * HD : nullptr;
+    const float *Sp = S_in ? S_in + bh * dvw * dkw : nullptr;
     f32x4 s[NP];
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
         const int row = r0 + RPP * p;
-        s[p] = (Sp && !reset) ? *reinterpret_cast<const f32x4 *>(Sp + row * HD + 4 * c4) : f32x4{0.f, 0.f, 0.f, 0.f};
+        s[p] = (Sp && !reset && cin && (!RAG || row < dvw)) ? *reinterpret_cast<const f32x4 *>(Sp + row * dkw + 4 * c4) : zero4;
     }
     float u[NP];
 #pragma unroll
-    for (int p = 0; p < NP; ++p) u[p] = (float)vp[r0 + RPP * p];
+    for (int p = 0; p < NP; ++p) u[p] = (!RAG || r0 + RPP * p < dvw) ? (float)vp[r0 + RPP * p] : 0.f;
     if (DELTA) {
         const float bb = (float)beta[bh];
 #pragma unroll
@@ -88,31 +96,35 @@ step_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restric
     float den = 1.f;
     if (!DELTA && z_out) {
         // every row's lanes recompute the normaliser of the sequence; row 0 stores it
-        f32x4 z4 = (z_in && !reset) ? *reinterpret_cast<const f32x4 *>(z_in + bh * HD + 4 * c4) : f32x4{0.f, 0.f, 0.f, 0.f};
+        f32x4 z4 = (z_in && !reset && cin) ? *reinterpret_cast<const f32x4 *>(z_in + bh * dkw + 4 * c4) : zero4;
         z4 += k4;
-        if (r0 == 0) *reinterpret_cast<f32x4 *>(z_out + bh * HD + 4 * c4) = z4;
+        if (r0 == 0 && cin) *reinterpret_cast<f32x4 *>(z_out + bh * dkw + 4 * c4) = z4;
         den = fmaxf(reduce_row(dot4(z4, q4)), eps);
     }
-    float *So = S_out + bh * HD * HD;
+    float *So = S_out + bh * dvw * dkw;
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
         const int row = r0 + RPP * p;
         s[p] += k4 * u[p];
-        *reinterpret_cast<f32x4 *>(So + row * HD + 4 * c4) = s[p];
+        const bool rin = !RAG || row < dvw;
+        if (cin && rin) *reinterpret_cast<f32x4 *>(So + row * dkw + 4 * c4) = s[p];
         const float x = reduce_row(dot4(s[p], q4));
-        if (c4 == 0) o[bh * HD + row] = (T)(x / den);
+        if (c4 == 0 && rin) o[bh * dvw + row] = (T)(x / den);
     }
 }
 
 int check_step(const void *q, const void *k, const void *v, const void *done, const void *S_in,
                const void *o, const void *S_out, int64_t B, int64_t H, int64_t dk, int64_t dv, int dtype,
-               int done_dtype)
+               int done_dtype, bool narrow = false)
 {
     if (!q || !k || !v || !done || !o || !S_out) return MRX_ERR_INVALID_ARG;
     if (B <= 0 || H <= 0 || dk <= 0 || dv <= 0) return MRX_ERR_INVALID_ARG;
     if (dtype != MRX_F32 && dtype != MRX_BF16) return dtype == MRX_C64 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
     if (done_dtype != MRX_DONE_U8 && done_dtype != MRX_DONE_F32) return MRX_ERR_INVALID_ARG;
-    if (dk != HD || dv != HD) return MRX_ERR_UNSUPPORTED;
+    // narrow: linear attention in the head dim 32 build also takes narrower rows of whole 16-byte segments
+    const int64_t seg = dtype == MRX_BF16 ? 8 : 4;
+    const bool narrow_ok = narrow && MRX_HD == 32 && dk <= HD && dv <= HD && dk % seg == 0 && dv % seg == 0;
+    if ((dk != HD || dv != HD) && !narrow_ok) return MRX_ERR_UNSUPPORTED;
     if (B * H >= (1ll << 31)) return MRX_ERR_INVALID_ARG;
     const void *ps[] = {q, k, v, S_in, o, S_out};
     for (const void *p : ps)
@@ -124,11 +136,17 @@ int check_step(const void *q, const void *k, const void *v, const void *done, co
 template <typename T, bool DELTA, bool FMAP>
 int launch_step(hipStream_t st, const void *q, const void *k, const void *v, const void *beta, const void *done,
                 int done_f32, const float *S_in, const float *z_in, void *o, float *S_out, float *z_out,
-                int64_t B, int64_t H, float eps)
+                int64_t B, int64_t H, float eps, int64_t dka = HD, int64_t dva = HD)
 {
-    return launch_kernel((step_kernel<T, DELTA, FMAP>), dim3((unsigned)(B * H)), dim3(256), 0, st, (const T *)q,
-                         (const T *)k, (const T *)v, (const T *)beta, done, done_f32, S_in, z_in, (T *)o, S_out,
-                         z_out, (int)H, eps);
+    auto go = [&](auto rag) {
+        return launch_kernel((step_kernel<T, DELTA, FMAP, decltype(rag)::value>), dim3((unsigned)(B * H)), dim3(256), 0, st,
+                             (const T *)q, (const T *)k, (const T *)v, (const T *)beta, done, done_f32, S_in, z_in,
+                             (T *)o, S_out, z_out, (int)H, eps, (int)dka, (int)dva);
+    };
+    if constexpr (MRX_HD == 32 && !DELTA) {
+        if (dka != HD || dva != HD) return go(std::true_type{});  // narrow heads
+    }
+    return go(std::false_type{});
 }
 
 }  // namespace MRX_HD_NS
@@ -140,16 +158,16 @@ MRX_EXPORT int MRX_API(mrx_linear_attn_step)(void *stream, const void *q, const 
                                     int feature_map, float eps)
 {
 #if MRX_HD == 64
-    if (dk == 32 && dv == 32) return mrx_linear_attn_step_hd32(stream, q, k, v, done, S_in, z_in, o, S_out, z_out, B, H, dk, dv, dtype, done_dtype, feature_map, eps);
+    if (dk <= 32 && dv <= 32) return mrx_linear_attn_step_hd32(stream, q, k, v, done, S_in, z_in, o, S_out, z_out, B, H, dk, dv, dtype, done_dtype, feature_map, eps);
 #endif
-    const int rc = check_step(q, k, v, done, S_in, o, S_out, B, H, dk, dv, dtype, done_dtype);
+    const int rc = check_step(q, k, v, done, S_in, o, S_out, B, H, dk, dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
     if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
     if ((z_in && !z_out) || !aligned(z_in, 16) || !aligned(z_out, 16)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     const bool fm = feature_map == MRX_FMAP_ELU1;
     const int df = done_dtype == MRX_DONE_F32;
-#define MRX_ARGS st, q, k, v, nullptr, done, df, S_in, z_in, o, S_out, z_out, B, H, eps
+#define MRX_ARGS st, q, k, v, nullptr, done, df, S_in, z_in, o, S_out, z_out, B, H, eps, dk, dv
     if (dtype == MRX_BF16) return fm ? launch_step<__bf16, false, true>(MRX_ARGS) : launch_step<__bf16, false, false>(MRX_ARGS);
     return fm ? launch_step<float, false, true>(MRX_ARGS) : launch_step<float, false, false>(MRX_ARGS);
 #undef MRX_ARGS

@@ -52,28 +52,34 @@ def _batched(core_rank, ref):
 
 
 class _Heads:
-    """Maps other head dims onto the kernels' d_k = d_v = 64 or 32 (the reference's cells take any
-    head_dim; its guides use 16): the 32-wide kernels serve d_k <= 32, the 64-wide ones the rest.
-    d_k below the kernel's width is zero-padded -- after the feature map, since phi(0) = 1 would
-    otherwise count -- and d_v is zero-padded to a multiple of that width and split into blocks that
-    run as extra heads sharing q and k (rows of the state are independent recurrences).
+    """Maps other head dims onto what the kernels take (the reference's cells take any head_dim; its
+    guides use 16).  The 32-wide kernels serve d_k <= 32, the 64-wide ones the rest.  The kernels of the
+    linear-attention family (`narrow`) in the 32-wide build take any d_k, d_v <= 32 that is a whole
+    number of 16-byte segments as it is; everything else goes through padding: d_k below the kernel's
+    width is zero-padded -- after the feature map, since phi(0) = 1 would otherwise count -- and d_v is
+    zero-padded to a multiple of the value width and split into blocks that run as extra heads sharing
+    q and k (rows of the state are independent recurrences).
     Padding, blocks and slices are ordinary differentiable array ops around the kernel call."""
 
-    def __init__(self, q, v, fmap=0):
+    def __init__(self, q, v, fmap=0, narrow=False):
         self.B, self.T, self.H, self.dk = q.shape
         self.dv = v.shape[-1]
         if self.dk > _HD:
             raise ValueError(f"d_k = {self.dk} > {_HD} is not supported (d_v may be any size)")
         self.hd = 32 if self.dk <= 32 else _HD
-        self.nb = (self.dv + self.hd - 1) // self.hd
-        self.native = self.dk == self.hd and self.dv == self.hd
-        self.pre = fmap if self.dk != self.hd else 0    # feature map applied here, before the padding
+        seg = 16 // q.element_size()                    # elements per 16 bytes
+        thin = narrow and self.hd == 32
+        self.kw = self.dk if thin and self.dk % seg == 0 else self.hd                          # key width the kernel sees
+        self.vw = self.dv if thin and self.dv <= self.hd and self.dv % seg == 0 else self.hd   # value width per block
+        self.nb = (self.dv + self.vw - 1) // self.vw
+        self.native = self.dk == self.kw and self.dv == self.vw
+        self.pre = fmap if self.dk != self.kw else 0    # feature map applied here, before the padding
         self.fmap = 0 if self.pre else fmap             # feature map left to the kernel
 
-    def _blocks(self, x):  # (B,T,H,hd) -> (B,T,H*nb,hd), every block a copy
+    def _blocks(self, x):  # (B,T,H,kw) -> (B,T,H*nb,kw), every block a copy
         if self.nb == 1:
             return x
-        return x[:, :, :, None].expand(self.B, self.T, self.H, self.nb, self.hd).reshape(self.B, self.T, self.H * self.nb, self.hd)
+        return x[:, :, :, None].expand(self.B, self.T, self.H, self.nb, self.kw).reshape(self.B, self.T, self.H * self.nb, self.kw)
 
     def qk(self, x):
         if self.native:
@@ -81,37 +87,37 @@ class _Heads:
         if self.pre:
             xf = x if x.dtype in (torch.float32, torch.float64) else x.float()
             x = (torch.nn.functional.elu(xf) + 1).to(x.dtype)
-        return self._blocks(torch.nn.functional.pad(x, (0, self.hd - self.dk)))
+        return self._blocks(torch.nn.functional.pad(x, (0, self.kw - self.dk)))
 
     def v(self, x):
         if self.native:
             return x
-        x = torch.nn.functional.pad(x, (0, self.nb * self.hd - self.dv))
-        return x.reshape(self.B, self.T, self.H * self.nb, self.hd)
+        x = torch.nn.functional.pad(x, (0, self.nb * self.vw - self.dv))
+        return x.reshape(self.B, self.T, self.H * self.nb, self.vw)
 
     def per_head(self, x):  # (B,T,H) -> (B,T,H*nb)
         return x if self.nb == 1 else x.repeat_interleave(self.nb, dim=2)
 
-    def state_in(self, S):  # (B,H,dv,dk) -> (B,H*nb,hd,hd)
+    def state_in(self, S):  # (B,H,dv,dk) -> (B,H*nb,vw,kw)
         if S is None or self.native:
             return S
-        S = torch.nn.functional.pad(S, (0, self.hd - self.dk, 0, self.nb * self.hd - self.dv))
-        return S.reshape(self.B, self.H * self.nb, self.hd, self.hd)
+        S = torch.nn.functional.pad(S, (0, self.kw - self.dk, 0, self.nb * self.vw - self.dv))
+        return S.reshape(self.B, self.H * self.nb, self.vw, self.kw)
 
-    def z_in(self, z):  # (B,H,dk) -> (B,H*nb,hd)
+    def z_in(self, z):  # (B,H,dk) -> (B,H*nb,kw)
         if z is None or self.native:
             return z
-        z = torch.nn.functional.pad(z, (0, self.hd - self.dk))
+        z = torch.nn.functional.pad(z, (0, self.kw - self.dk))
         return z if self.nb == 1 else z.repeat_interleave(self.nb, dim=1)
 
-    def out(self, o):  # (B,T,H*nb,hd) -> (B,T,H,dv)
-        return o if self.native else o.reshape(self.B, o.shape[1], self.H, self.nb * self.hd)[..., :self.dv]
+    def out(self, o):  # (B,T,H*nb,vw) -> (B,T,H,dv)
+        return o if self.native else o.reshape(self.B, o.shape[1], self.H, self.nb * self.vw)[..., :self.dv]
 
     def state_out(self, S):
-        return S if self.native else S.reshape(self.B, self.H, self.nb * self.hd, self.hd)[:, :, :self.dv, :self.dk]
+        return S if self.native else S.reshape(self.B, self.H, self.nb * self.vw, self.kw)[:, :, :self.dv, :self.dk]
 
     def z_out(self, z):
-        return z if self.native else z.reshape(self.B, self.H, self.nb, self.hd)[:, :, 0, :self.dk]
+        return z if self.native else z.reshape(self.B, self.H, self.nb, self.kw)[:, :, 0, :self.dk]
 
 
 class _LinearScan(torch.autograd.Function):
@@ -218,7 +224,7 @@ class _LinearAttention(torch.autograd.Function):
 def linear_attention(q, k, v, done, S0=None, feature_map="none"):
     """Causal unnormalised linear attention, chunked: S_t = r_t S_{t-1} + v_t phi(k_t)^T,
     o_t = S_t phi(q_t) (linear_attention.py:62-86,105).  Returns (o, S_last)."""
-    hd = _Heads(q, v, _FMAP[feature_map])
+    hd = _Heads(q, v, _FMAP[feature_map], narrow=True)
     o, S_last = _LinearAttention.apply(hd.qk(q), hd.qk(k), hd.v(v), done, hd.state_in(S0), hd.fmap)
     return hd.out(o), hd.state_out(S_last)
 
@@ -256,7 +262,7 @@ def normalised_linear_attention(q, k, v, done, S0=None, z0=None, feature_map="el
     """Causal linear attention with the normalised read-out of LinearAttentionCell.read
     (linear_attention.py:93-110) in the same kernel: z_t = r_t z_{t-1} + phi(k_t),
     o_t = S_t phi(q_t) / max(phi(q_t) . z_t, eps).  Returns (o, S_last, z_last)."""
-    hd = _Heads(q, v, _FMAP[feature_map])
+    hd = _Heads(q, v, _FMAP[feature_map], narrow=True)
     o, S_last, z_last = _NormalisedLinearAttention.apply(hd.qk(q), hd.qk(k), hd.v(v), done, hd.state_in(S0),
                                                          hd.z_in(z0), hd.fmap, float(eps))
     return hd.out(o), hd.state_out(S_last), hd.z_out(z_last)
@@ -290,7 +296,7 @@ def gated_linear_attention(q, k, v, g, done, S0=None, feature_map="none"):
     """Linear attention with a scalar log-decay g:(B,T,H) per step and head:
     S_t = r_t exp(g_t) S_{t-1} + v_t phi(k_t)^T, o_t = S_t phi(q_t) -- the Mamba cell's algebra
     (mamba.py:109-122) in chunked form.  Returns (o, S_last)."""
-    hd = _Heads(q, v, _FMAP[feature_map])
+    hd = _Heads(q, v, _FMAP[feature_map], narrow=True)
     o, S_last = _GatedLinearAttention.apply(hd.qk(q), hd.qk(k), hd.v(v), hd.per_head(g), done, hd.state_in(S0),
                                             hd.fmap)
     return hd.out(o), hd.state_out(S_last)

@@ -1,0 +1,147 @@
+"""GPU parity of the linear-attention family on heads narrower than the library's 32-wide build
+(d_k, d_v <= 32 in whole 16-byte segments, d_k and d_v independent): the kernels take such rows as they lie
+in memory and pad inside; results against the oracle at the same head dims."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import grad as G
+from gpu_util import TOL_BF16, TOL_F32, bf16_round, dev, relerr
+
+pytestmark = pytest.mark.gpu
+
+# (d_k, d_v): the reference guides' head_dim 16, unequal widths either way, one full and one narrow side
+DIMS = [(16, 16), (8, 24), (24, 8), (32, 16), (16, 32)]
+DIMS_F32_ONLY = [(12, 20), (4, 4)]  # whole 16-byte segments of float32 only
+SHAPES = [(3, 1, 2), (2, 65, 1), (2, 200, 3), (1, 1100, 2)]
+
+
+def _inputs(shape, dk, dv, p, dtype, seed):
+    B, T, H = shape
+    rng = np.random.default_rng(seed)
+    x = {n: (rng.standard_normal((B, T, H, d)) / 4).astype(np.float32)
+         for n, d in (("q", dk), ("k", dk), ("v", dv), ("do", dv))}
+    x["do"] *= 4
+    x["done"] = rng.random((B, T)) < p
+    x["S0"] = (rng.standard_normal((B, H, dv, dk)) * 0.1).astype(np.float32)
+    x["dSl"] = (rng.standard_normal((B, H, dv, dk)) * 0.1).astype(np.float32)
+    x["g"] = (-np.abs(rng.standard_normal((B, T, H))) * 0.2).astype(np.float32)
+    x["z0"] = np.abs(rng.standard_normal((B, H, dk))).astype(np.float32)
+    x["dzl"] = (rng.standard_normal((B, H, dk)) * 0.1).astype(np.float32)
+    if dtype == "bf16":
+        for n in ("q", "k", "v", "do"):
+            x[n] = bf16_round(x[n])
+    return x
+
+
+def _check(got, ref, names, tol):
+    errs = {n: relerr(g, ref[n]) for n, g in zip(names, got)}
+    assert all(e <= tol for e in errs.values()), errs
+
+
+def _cases():
+    return [(d, "f32") for d in DIMS + DIMS_F32_ONLY] + [(d, "bf16") for d in DIMS]
+
+
+@pytest.mark.parametrize("dims,dtype", _cases())
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("p", [0.0, 0.06])
+@pytest.mark.parametrize("par", [False, True])
+def test_linear_attention(dims, dtype, shape, p, par):
+    from memorax_amd import kernels as K
+    dk, dv = dims
+    x = _inputs(shape, dk, dv, p, dtype, seed=sum(shape) + dk + 3)
+    print(f"case narrow la dk={dk} dv={dv} shape={shape} p={p} dtype={dtype} chunk_parallel={par}", flush=True)
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    tq, tk, tv, tdo = (dev(x[n], td) for n in ("q", "k", "v", "do"))
+    for fm, name in ((1, "elu1"), (0, "none")):
+        o, Sl, chk = K.linear_attn_fwd(tq, tk, tv, dev(x["done"]), dev(x["S0"]), fm, chunk_parallel=par)
+        assert o.shape == (shape[0], shape[1], shape[2], dv) and Sl.shape == (shape[0], shape[2], dv, dk)
+        ref = G.linear_attention_grads(x["q"], x["k"], x["v"], x["done"], x["S0"], x["do"], x["dSl"], name)
+        _check((o, Sl), ref, ("o", "S_last"), tol)
+        got = K.linear_attn_bwd(tq, tk, tv, dev(x["done"]), chk, tdo, dev(x["dSl"]), fm)
+        _check(got, ref, ("dq", "dk", "dv", "dS0"), tol)
+
+
+@pytest.mark.parametrize("dims,dtype", _cases())
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("p", [0.0, 0.06])
+def test_gated_and_normalised_linear_attention(dims, dtype, shape, p):
+    from memorax_amd import kernels as K
+    dk, dv = dims
+    x = _inputs(shape, dk, dv, p, dtype, seed=sum(shape) + dk + 5)
+    print(f"case narrow gated/norm dk={dk} dv={dv} shape={shape} p={p} dtype={dtype}", flush=True)
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    tq, tk, tv, tdo = (dev(x[n], td) for n in ("q", "k", "v", "do"))
+    dn = dev(x["done"])
+    o, Sl, S_chk = K.gated_linear_attn_fwd(tq, tk, tv, dev(x["g"]), dn, dev(x["S0"]), 1)
+    ref = G.gated_linear_attention_grads(x["q"], x["k"], x["v"], x["g"], x["done"], x["S0"], x["do"], x["dSl"], "elu1")
+    _check((o, Sl), ref, ("o", "S_last"), tol)
+    got = K.gated_linear_attn_bwd(tq, tk, tv, dev(x["g"]), dn, S_chk, tdo, dev(x["dSl"]), 1, S_last=Sl)
+    _check(got, ref, ("dq", "dk", "dv", "dg", "dS0"), tol)
+    o, den, Sl, zl, chk = K.linear_attn_norm_fwd(tq, tk, tv, dn, dev(x["S0"]), dev(x["z0"]), 1, 1e-6)
+    ref = G.normalised_linear_attention_grads(x["q"], x["k"], x["v"], x["done"], x["S0"], x["z0"], x["do"], x["dSl"],
+                                              x["dzl"], "elu1", 1e-6)
+    _check((o, Sl, zl), ref, ("o", "S_last", "z_last"), tol)
+    got = K.linear_attn_norm_bwd(tq, tk, tv, dn, chk, o, den, tdo, dev(x["dSl"]), dev(x["dzl"]), 1, 1e-6)
+    _check(got, ref, ("dq", "dk", "dv", "dS0", "dz0"), tol)
+
+
+@pytest.mark.parametrize("dims,dtype", _cases())
+def test_single_steps_roll_out_to_the_sequence_results(dims, dtype):
+    from memorax_amd import kernels as K
+    dk, dv = dims
+    B, T, H = 3, 11, 2
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    print(f"case narrow steps dk={dk} dv={dv} dtype={dtype}", flush=True)
+    x = _inputs((B, T, H), dk, dv, 0.2, dtype, seed=21)
+    q, k, v, done = dev(x["q"], td), dev(x["k"], td), dev(x["v"], td), dev(x["done"])
+    for normalise in (True, False):
+        S, z, outs = dev(x["S0"]), dev(x["z0"]) if normalise else None, []
+        for t in range(T):
+            o, S, z = K.linear_attn_step(q[:, t].contiguous(), k[:, t].contiguous(), v[:, t].contiguous(),
+                                         done[:, t].contiguous(), S, z, "elu1", normalise)
+            outs.append(o)
+        args = [torch.from_numpy(x[n]).double() for n in ("q", "k", "v")] + [torch.from_numpy(x["done"]),
+                                                                              torch.from_numpy(x["S0"]).double()]
+        if normalise:
+            ro, rS, rz = (a.numpy() for a in G.normalised_linear_attention_t(*args, torch.from_numpy(x["z0"]).double(), "elu1"))
+            assert relerr(z, rz) <= tol
+        else:
+            ro, rS = (a.numpy() for a in G.linear_attention_t(*args, "elu1"))
+        assert outs[0].shape == (B, H, dv) and S.shape == (B, H, dv, dk)
+        assert relerr(torch.stack(outs, 1), ro) <= tol and relerr(S, rS) <= tol
+
+
+def test_what_is_not_a_narrow_head_is_refused():
+    from memorax_amd import _lib
+    lib = _lib.load()
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def la(dk, dv, dtype):
+        td = torch.bfloat16 if dtype else torch.float32
+        q = torch.zeros((1, 4, 1, dk), dtype=td, device="cuda")
+        v = torch.zeros((1, 4, 1, dv), dtype=td, device="cuda")
+        dn = torch.zeros((1, 4), dtype=torch.uint8, device="cuda")
+        o = torch.empty_like(v)
+        return lib.mrx_linear_attn_fwd(None, P(q), P(q), P(v), P(dn), None, P(o), None, None, 1, 4, 1, dk, dv, dtype, 0, 0)
+
+    assert la(16, 16, 0) == 0 and la(16, 16, 1) == 0 and la(12, 4, 0) == 0
+    assert la(12, 16, 1) == -2       # 12 bf16 are one and a half segments
+    assert la(6, 16, 0) == -2 and la(16, 10, 0) == -2
+    assert la(16, 64, 0) == -2 and la(64, 16, 0) == -2 and la(48, 48, 0) == -2 and la(32, 40, 0) == -2
+    # the delta rule keeps to the two head dims of the builds
+    q = torch.zeros((1, 4, 1, 16), device="cuda")
+    dn = torch.zeros((1, 4), dtype=torch.uint8, device="cuda")
+    beta = torch.zeros((1, 4, 1), device="cuda")
+    o = torch.empty_like(q)
+    assert lib.mrx_delta_rule_fwd(None, P(q), P(q), P(q), P(beta), P(dn), None, P(o), None, None, None, 1, 4, 1, 16, 16, 0, 0, 0) == -2
+    S = torch.zeros((1, 1, 16, 16), device="cuda")
+    assert lib.mrx_delta_rule_step(None, P(q[:, 0]), P(q[:, 0]), P(q[:, 0]), P(beta[:, 0]), P(dn[:, 0]), None, P(o[:, 0]), P(S),
+                                   1, 1, 16, 16, 0, 0) == -2
+    torch.cuda.synchronize()

@@ -1,5 +1,6 @@
-"""Host logic that maps other head dims onto the kernels' d_k = d_v = 64 or 32 (CPU: the oracle
-recurrences stand in for the kernels, so the test pins the padding/blocking algebra itself)."""
+"""Host logic that maps other head dims onto what the kernels take: d_k = d_v = 64 or 32, and for the
+linear-attention family any narrower head of whole 16-byte segments (CPU: the oracle recurrences stand in
+for the kernels, so the test pins the padding/blocking algebra itself)."""
 import numpy as np
 import pytest
 import torch
@@ -12,7 +13,7 @@ def _rand(*s, seed=0):
     return torch.from_numpy(np.random.default_rng(seed).standard_normal(s))
 
 
-@pytest.mark.parametrize("dk,dv", [(16, 16), (32, 64), (64, 96), (16, 130), (64, 64), (32, 32), (33, 20)])
+@pytest.mark.parametrize("dk,dv", [(16, 16), (32, 64), (64, 96), (16, 130), (64, 64), (32, 32), (33, 20), (24, 8), (15, 16), (16, 31)])
 @pytest.mark.parametrize("op", ["linear", "normalised", "gated", "delta"])
 def test_padding_and_value_blocks_reproduce_the_native_recurrence(dk, dv, op):
     B, T, H = 2, 9, 2
@@ -21,12 +22,16 @@ def test_padding_and_value_blocks_reproduce_the_native_recurrence(dk, dv, op):
     g, beta = -_rand(B, T, H, seed=6).abs() * 0.3, torch.sigmoid(_rand(B, T, H, seed=7))
     done = torch.from_numpy(np.random.default_rng(8).random((B, T)) < 0.2)
     fm = "none" if op == "delta" else "elu1"
-    hd = _Heads(q, v, 0 if op == "delta" else 1)
+    narrow = op != "delta"  # the linear-attention kernels of the 32-wide build take narrower heads as they are
+    hd = _Heads(q, v, 0 if op == "delta" else 1, narrow=narrow)
     w = 32 if dk <= 32 else 64  # the 32-wide kernels serve keys of up to 32 features
-    assert hd.hd == w and hd.native == (dk == w and dv == w) and hd.nb == -(-dv // w)
+    seg = 16 // q.element_size()
+    kw = dk if narrow and w == 32 and dk % seg == 0 else w
+    vw = dv if narrow and w == 32 and dv <= 32 and dv % seg == 0 else w
+    assert hd.hd == w and (hd.kw, hd.vw) == (kw, vw) and hd.native == (dk == kw and dv == vw) and hd.nb == -(-dv // vw)
     kfm = "elu1" if hd.fmap else "none"   # the feature map the kernel would be asked to apply
     qq, kk, vv, SS = hd.qk(q), hd.qk(k), hd.v(v), hd.state_in(S0)
-    assert qq.shape == (B, T, H * hd.nb, w) and vv.shape == qq.shape and SS.shape == (B, H * hd.nb, w, w)
+    assert qq.shape == (B, T, H * hd.nb, kw) and vv.shape == (B, T, H * hd.nb, vw) and SS.shape == (B, H * hd.nb, vw, kw)
     if op == "linear":
         o, Sl = G.linear_attention_t(qq, kk, vv, done, SS, kfm)
         ro, rS = G.linear_attention_t(q, k, v, done, S0, fm)
