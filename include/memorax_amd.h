@@ -136,7 +136,8 @@ int mrx_linear_scan_bwd(void *stream, const void *a, const void *h,
  * S_last.  dk = dv = 64 or dk = dv = 32 (here and in every chunked and single-step entry point below;
  * the library holds a build of those kernels for either width; mrx_delta_rule_fwd_noalloc: 64 only).
  * Narrow heads: the linear-attention family -- mrx_linear_attn_*, mrx_gated_linear_attn_*,
- * mrx_linear_attn_norm_*, mrx_linear_attn_*_chunk_parallel and mrx_linear_attn_step -- also takes any
+ * mrx_linear_attn_norm_*, mrx_linear_attn_*_chunk_parallel, mrx_linear_attn_step and
+ * mrx_gated_linear_attn_step -- also takes any
  * dk <= 32 and dv <= 32, independent of one another, whose rows are a whole number of 16-byte segments
  * (multiples of 4 in float32, of 8 in bfloat16; the reference's guides use head_dim = 16).  Every array
  * keeps its dense (.., dv, dk) / (.., dk) / (.., dv) layout at those widths; the 32-wide kernels pad
@@ -352,8 +353,8 @@ int mrx_gated_linear_attn_bwd(void *stream, const void *q, const void *k,
  * What Memoroid.__call__ (memoroid.py:93-109) computes when T = 1, as PPO's rollout
  * does once per environment step (algorithms/ppo.py:105-143): one update of the
  * carry fused with the read-out, without the chunk machinery.
- *   q,k,v,o: (B,1,H,d) = (B,H,d) in `dtype`, d = 64 or 32 (mrx_linear_attn_step: narrow heads too, see
- *   mrx_linear_attn_fwd); done: (B,) ; S_in/S_out: (B,H,dv,dk) fp32.
+ *   q,k,v,o: (B,1,H,d) = (B,H,d) in `dtype`, d = 64 or 32 (the two linear-attention steps: narrow heads
+ *   too, see mrx_linear_attn_fwd); done: (B,) ; S_in/S_out: (B,H,dv,dk) fp32.
  * S_in may be NULL (zero state) and may equal S_out (update in place).
  *
  * Linear attention (linear_attention.py:62-117):
@@ -366,6 +367,16 @@ int mrx_linear_attn_step(void *stream, const void *q, const void *k,
                          const float *z_in, void *o, float *S_out, float *z_out,
                          int64_t B, int64_t H, int64_t dk, int64_t dv, int dtype,
                          int done_dtype, int feature_map, float eps);
+
+/* Gated linear attention, the T = 1 case of mrx_gated_linear_attn_fwd (the Mamba cell's step,
+ * mamba.py:109-135, and the mLSTM cell's in its stabilised units, mlstm.py:163-229):
+ *     S' = (done ? 0 : exp(g) S) + v phi(k)^T ;  o = S' phi(q)
+ * g: (B,H) float32, the log-decay of the step. */
+int mrx_gated_linear_attn_step(void *stream, const void *q, const void *k,
+                               const void *v, const float *g, const void *done,
+                               const float *S_in, void *o, float *S_out, int64_t B,
+                               int64_t H, int64_t dk, int64_t dv, int dtype,
+                               int done_dtype, int feature_map);
 
 /* Delta rule (no counterpart in the reference; the T = 1 case of mrx_delta_rule_fwd):
  *     S0 = done ? 0 : S ;  u = beta (v - S0 k) ;  S' = S0 + u k^T ;  o = S' q

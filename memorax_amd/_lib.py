@@ -49,6 +49,7 @@ SIGNATURES = {
     "mrx_gated_linear_attn_bwd": (_I, [_P] * 15 + [_L] * 5 + [_I] * 3),
     "mrx_linear_attn_step": (_I, [_P] * 10 + [_L] * 4 + [_I] * 3 + [ctypes.c_float]),
     "mrx_delta_rule_step": (_I, [_P] * 9 + [_L] * 4 + [_I] * 2),
+    "mrx_gated_linear_attn_step": (_I, [_P] * 9 + [_L] * 4 + [_I] * 3),
 }
 
 _lib = None

@@ -3,6 +3,7 @@
 //
 //   linear attention : S' = (done ? 0 : S) + v phi(k)^T ,  z' = (done ? 0 : z) + phi(k)
 //                      o = S' phi(q)            [ / max(phi(q) . z', eps) when z is given ]
+//   gated            : S' = (done ? 0 : exp(g) S) + v phi(k)^T ,  o = S' phi(q)   (g a log-decay per sequence)
 //   delta rule       : S0 = done ? 0 : S ,  u = beta (v - S0 k) ,  S' = S0 + u k^T ,  o = S' q
 //
 // The state S:(B,H,d,d) fp32 ([dv][dk], d = 64 or 32) is read once and written once; everything else
@@ -56,7 +57,7 @@ __device__ __forceinline__ float dot4(const f32x4 &a, const f32x4 &b)
 template <typename T, bool DELTA, bool FMAP, bool RAG = false>
 __global__ void __launch_bounds__(256)
 step_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
-            const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
+            const T *__restrict__ beta, const float *__restrict__ glog, const void *__restrict__ done, int done_f32,
             const float *S_in, const float *z_in, T *__restrict__ o, float *S_out, float *z_out, int H,
             float eps, int dka, int dva)  // S_in/S_out and z_in/z_out may alias (update in place)
 {
@@ -79,11 +80,12 @@ step_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restric
         }
     }
     const float *Sp = S_in ? S_in + bh * dvw * dkw : nullptr;
+    const float decay = (!DELTA && glog) ? __expf(glog[bh]) : 1.f;  // gated linear attention: the carried state decays first
     f32x4 s[NP];
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
         const int row = r0 + RPP * p;
-        s[p] = (Sp && !reset && cin && (!RAG || row < dvw)) ? *reinterpret_cast<const f32x4 *>(Sp + row * dkw + 4 * c4) : zero4;
+        s[p] = (Sp && !reset && cin && (!RAG || row < dvw)) ? *reinterpret_cast<const f32x4 *>(Sp + row * dkw + 4 * c4) * decay : zero4;
     }
     float u[NP];
 #pragma unroll
@@ -136,11 +138,11 @@ int check_step(const void *q, const void *k, const void *v, const void *done, co
 template <typename T, bool DELTA, bool FMAP>
 int launch_step(hipStream_t st, const void *q, const void *k, const void *v, const void *beta, const void *done,
                 int done_f32, const float *S_in, const float *z_in, void *o, float *S_out, float *z_out,
-                int64_t B, int64_t H, float eps, int64_t dka = HD, int64_t dva = HD)
+                int64_t B, int64_t H, float eps, int64_t dka = HD, int64_t dva = HD, const float *glog = nullptr)
 {
     auto go = [&](auto rag) {
         return launch_kernel((step_kernel<T, DELTA, FMAP, decltype(rag)::value>), dim3((unsigned)(B * H)), dim3(256), 0, st,
-                             (const T *)q, (const T *)k, (const T *)v, (const T *)beta, done, done_f32, S_in, z_in,
+                             (const T *)q, (const T *)k, (const T *)v, (const T *)beta, glog, done, done_f32, S_in, z_in,
                              (T *)o, S_out, z_out, (int)H, eps, (int)dka, (int)dva);
     };
     if constexpr (MRX_HD == 32 && !DELTA) {
@@ -168,6 +170,27 @@ MRX_EXPORT int MRX_API(mrx_linear_attn_step)(void *stream, const void *q, const 
     const bool fm = feature_map == MRX_FMAP_ELU1;
     const int df = done_dtype == MRX_DONE_F32;
 #define MRX_ARGS st, q, k, v, nullptr, done, df, S_in, z_in, o, S_out, z_out, B, H, eps, dk, dv
+    if (dtype == MRX_BF16) return fm ? launch_step<__bf16, false, true>(MRX_ARGS) : launch_step<__bf16, false, false>(MRX_ARGS);
+    return fm ? launch_step<float, false, true>(MRX_ARGS) : launch_step<float, false, false>(MRX_ARGS);
+#undef MRX_ARGS
+}
+
+MRX_EXPORT int MRX_API(mrx_gated_linear_attn_step)(void *stream, const void *q, const void *k, const void *v,
+                                          const float *g, const void *done, const float *S_in, void *o, float *S_out,
+                                          int64_t B, int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype,
+                                          int feature_map)
+{
+#if MRX_HD == 64
+    if (dk <= 32 && dv <= 32) return mrx_gated_linear_attn_step_hd32(stream, q, k, v, g, done, S_in, o, S_out, B, H, dk, dv, dtype, done_dtype, feature_map);
+#endif
+    const int rc = check_step(q, k, v, done, S_in, o, S_out, B, H, dk, dv, dtype, done_dtype, true);
+    if (rc != MRX_OK) return rc;
+    if (!g || !aligned(g, 4)) return MRX_ERR_INVALID_ARG;
+    if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    const bool fm = feature_map == MRX_FMAP_ELU1;
+    const int df = done_dtype == MRX_DONE_F32;
+#define MRX_ARGS st, q, k, v, nullptr, done, df, S_in, nullptr, o, S_out, nullptr, B, H, 0.f, dk, dv, g
     if (dtype == MRX_BF16) return fm ? launch_step<__bf16, false, true>(MRX_ARGS) : launch_step<__bf16, false, false>(MRX_ARGS);
     return fm ? launch_step<float, false, true>(MRX_ARGS) : launch_step<float, false, false>(MRX_ARGS);
 #undef MRX_ARGS

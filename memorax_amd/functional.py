@@ -275,6 +275,11 @@ class _GatedLinearAttention(torch.autograd.Function):
         g_ = g.contiguous().float()
         S0_ = None if S0 is None else S0.contiguous().float()
         need = any(ctx.needs_input_grad)
+        if q_.shape[1] == 1 and not need:  # acting: one step, no residuals (memoroid.py:93-109 with T = 1)
+            o, S_last = K.gated_linear_attn_step(q_[:, 0], k_[:, 0], v_[:, 0], g_[:, 0], done[:, 0], S0_,
+                                                 feature_map=_FMAP_NAME[fmap])
+            ctx.done, ctx.fmap, ctx.has_S0 = done, fmap, S0 is not None
+            return o[:, None], S_last
         o, S_last, S_chk = K.gated_linear_attn_fwd(q_, k_, v_, g_, done, S0_, fmap, save_chk=need)
         if need:
             ctx.save_for_backward(q_, k_, v_, g_, S_chk, S_last)

@@ -501,6 +501,23 @@ def linear_attn_step(q, k, v, done, S=None, z=None, feature_map="none", normalis
     return o, S_new, z_new
 
 
+def gated_linear_attn_step(q, k, v, g, done, S=None, feature_map="none", inplace=False):
+    """One time step of gated linear attention.  q,k: (B,H,dk); v: (B,H,dv); g: (B,H) fp32 log-decay;
+    done: (B,); S: (B,H,dv,dk) fp32 or None.  Returns (o, S_new).  inplace updates S."""
+    lib = _lib.load()
+    B, H, dk, dv, dt = _step_shapes(q, k, v)
+    _chk(g, "g", torch.float32, (B, H))
+    _chk(S, "S", torch.float32, (B, H, dv, dk))
+    done, dd = _done(done.reshape(B, 1), B, 1)
+    o = torch.empty_like(v)
+    S_new = S if (inplace and S is not None) else torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device)
+    fm = {"none": _lib.MRX_FMAP_NONE, "elu1": _lib.MRX_FMAP_ELU1}[feature_map]
+    st = lib.mrx_gated_linear_attn_step(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(g), _ptr(done), _ptr(S), _ptr(o),
+                                        _ptr(S_new), B, H, dk, dv, _DT[dt], dd, fm)
+    _lib.check(st, "mrx_gated_linear_attn_step")
+    return o, S_new
+
+
 def delta_rule_step(q, k, v, beta, done, S=None, inplace=False):
     """One time step of the delta rule.  beta: (B,H).  Returns (o, S_new)."""
     lib = _lib.load()

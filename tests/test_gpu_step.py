@@ -75,6 +75,52 @@ def test_delta_rule_step_rollout(shape, p, dtype):
     assert relerr(state["S"], rS) <= (1e-5 if dtype == "f32" else tol), relerr(state["S"], rS)
 
 
+@pytest.mark.parametrize("dims", [(64, 64), (32, 32), (16, 16), (8, 24)])
+@pytest.mark.parametrize("p", [0.0, 0.2])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("fmap", ["none", "elu1"])
+def test_gated_linear_attention_step_rollout(dims, p, dtype, fmap):
+    """S' = (done ? 0 : exp(g) S) + v phi(k)^T, o = S' phi(q): a rollout of steps against the oracle's gated
+    recurrence over the whole sequence, and the host mirror's T = 1 route against the chunked kernel."""
+    from memorax_amd import functional as F
+    from memorax_amd import kernels as K
+    dk, dv = dims
+    B, T, H = 3, 13, 2
+    rng = np.random.default_rng(dk + dv + int(10 * p))
+    x = {n: (rng.standard_normal((B, T, H, d)) / 4).astype(np.float32) for n, d in (("q", dk), ("k", dk), ("v", dv))}
+    g = (-np.abs(rng.standard_normal((B, T, H))) * 0.5).astype(np.float32)
+    done = rng.random((B, T)) < p
+    S0 = (rng.standard_normal((B, H, dv, dk)) * 0.1).astype(np.float32)
+    print(f"case gated_step dims={dims} p={p} dtype={dtype} fmap={fmap}", flush=True)
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    if dtype == "bf16":
+        for n in ("q", "k", "v"):
+            x[n] = bf16_round(x[n])
+    q, k, v, tg, dn = dev(x["q"], td), dev(x["k"], td), dev(x["v"], td), dev(g), dev(done)
+    state = {"S": dev(S0)}
+
+    def step(t):
+        o, state["S"] = K.gated_linear_attn_step(q[:, t].contiguous(), k[:, t].contiguous(), v[:, t].contiguous(),
+                                                 tg[:, t].contiguous(), dn[:, t].contiguous(), state["S"],
+                                                 feature_map=fmap)
+        return o
+
+    o = _roll(step, T)
+    ro, rS = M.gated_linear_attention(x["q"], x["k"], x["v"], g, done, S0, fmap)
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    assert o.shape == (B, T, H, dv) and relerr(o, ro) <= tol, relerr(o, ro)
+    assert relerr(state["S"], rS) <= (1e-5 if dtype == "f32" else tol), relerr(state["S"], rS)
+    # the host mirror takes the step kernel for T = 1 without gradients; same numbers as the chunked kernel
+    S_mid = dev(S0)
+    with torch.no_grad():
+        o1, S1 = F.gated_linear_attention(q[:, :1], k[:, :1], v[:, :1], tg[:, :1], dn[:, :1], S_mid, fmap)
+    o2, S2, _ = K.gated_linear_attn_fwd(q[:, :1].contiguous(), k[:, :1].contiguous(), v[:, :1].contiguous(),
+                                        tg[:, :1].contiguous(), dn[:, :1].contiguous(), S_mid,
+                                        {"none": 0, "elu1": 1}[fmap], save_chk=False)
+    # (bf16: the chunked kernel rounds phi(k) to the I/O type before the products, the step kernel does not)
+    assert relerr(o1, o2.float().cpu().numpy()) <= tol and relerr(S1, S2.cpu().numpy()) <= (1e-5 if dtype == "f32" else tol)
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_linear_attention_step_normalised(dtype):
     """Fused denominator of LinearAttentionCell.read: o = S q / max(q . z, eps), z the running sum of phi(k)."""
@@ -141,4 +187,7 @@ def test_step_rejects_bad_arguments():
     assert lib.mrx_delta_rule_step(*args(32)) == -2          # unsupported head dim
     assert lib.mrx_delta_rule_step(None, p, p, p, None, p, p, p, p, 1, 1, 64, 64, 0, 0) == -1  # beta missing
     assert lib.mrx_linear_attn_step(None, p, p, p, p, p, None, p, p, None, 1, 1, 64, 64, 0, 0, 7, 1e-6) == -1
+    assert lib.mrx_gated_linear_attn_step(None, p, p, p, p, p, p, p, p, 1, 1, 64, 64, 0, 0, 0) == 0
+    assert lib.mrx_gated_linear_attn_step(None, p, p, p, None, p, p, p, p, 1, 1, 64, 64, 0, 0, 0) == -1  # g missing
+    assert lib.mrx_gated_linear_attn_step(None, p, p, p, p, p, p, p, p, 1, 1, 48, 48, 0, 0, 0) == -2
     torch.cuda.synchronize()
