@@ -65,17 +65,19 @@ la_chunk_state_kernel(const T *__restrict__ x, const T *__restrict__ y, const vo
 // additions are sequential: the slots (and the reset flags) of the next group of eight chunks are
 // requested before the current group is summed and written back, so that one trip to memory is exposed
 // per sequence, not one per group.
+// RAG: narrow heads, the state's size is a run-time value.
+template <bool RAG>
 __global__ void __launch_bounds__(256)
 la_state_scan_kernel(float *__restrict__ slots, const float *__restrict__ init, float *__restrict__ fin,
-                     const void *__restrict__ done, int done_f32, int Tlen, int H, int NC, int C, int backward, int Q)
+                     const void *__restrict__ done, int done_f32, int Tlen, int H, int NC, int C, int backward, int Qn)
 {
-    // Q: f32x4 per state (d_v * d_k / 4)
+    const int Q = RAG ? Qn : HD * HD / 4;  // f32x4 per state (d_v * d_k / 4)
     constexpr int G = 8;            // chunks per group
     const int tid = threadIdx.x, lane = tid & 63;
     const int bh = blockIdx.x, b = bh / H;
     const int idx = blockIdx.y * 256 + tid;
-    const bool act = idx < Q;  // a narrow state has fewer elements than the workgroup has threads; the idle lanes still
-                               // bring their reset flags to the ballots
+    const bool act = !RAG || idx < Q;  // a narrow state has fewer elements than the workgroup has threads; the idle lanes
+                                       // still bring their reset flags to the ballots
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
     f32x4 S = init && act ? reinterpret_cast<const f32x4 *>(init)[(int64_t)bh * Q + idx] : zero;
     f32x4 *p = reinterpret_cast<f32x4 *>(slots) + (int64_t)bh * NC * Q + idx;
@@ -154,8 +156,12 @@ int launch_la_state_scan(hipStream_t st, float *slots, const float *init, float 
     const int64_t NC = (Tlen + C - 1) / C;
     if (B * H > 0x7fffffffLL) return MRX_ERR_INVALID_ARG;
     const int Q = (int)(dk * dv / 4);
-    return launch_kernel(la_state_scan_kernel, dim3((unsigned)(B * H), (unsigned)((Q + 255) / 256)), dim3(256), 0, st, slots,
-                         init, fin, done, done_f32, (int)Tlen, (int)H, (int)NC, C, backward ? 1 : 0, Q);
+    const dim3 grid((unsigned)(B * H), (unsigned)((Q + 255) / 256));
+    if (dk != HD || dv != HD)
+        return launch_kernel(la_state_scan_kernel<true>, grid, dim3(256), 0, st, slots, init, fin, done, done_f32, (int)Tlen,
+                             (int)H, (int)NC, C, backward ? 1 : 0, Q);
+    return launch_kernel(la_state_scan_kernel<false>, grid, dim3(256), 0, st, slots, init, fin, done, done_f32, (int)Tlen,
+                         (int)H, (int)NC, C, backward ? 1 : 0, Q);
 }
 
 }  // namespace MRX_HD_NS
