@@ -58,63 +58,79 @@ class _Heads:
     number of 16-byte segments as it is; everything else goes through padding: d_k below the kernel's
     width is zero-padded -- after the feature map, since phi(0) = 1 would otherwise count -- and d_v is
     zero-padded to a multiple of the value width and split into blocks that run as extra heads sharing
-    q and k (rows of the state are independent recurrences).
-    Padding, blocks and slices are ordinary differentiable array ops around the kernel call."""
+    q and k (rows of the state are independent recurrences).  Where the output is linear in the state
+    (`split_k`: plain and gated linear attention), d_k > 64 is split the same way into key blocks
+    whose outputs add up (o = sum over blocks of S[:, block] q[block]); the delta rule and the
+    normalised read-out couple the key features and stay at d_k <= 64.
+    Padding, blocks, sums and slices are ordinary differentiable array ops around the kernel call."""
 
-    def __init__(self, q, v, fmap=0, narrow=False):
+    def __init__(self, q, v, fmap=0, narrow=False, split_k=False):
         self.B, self.T, self.H, self.dk = q.shape
         self.dv = v.shape[-1]
-        if self.dk > _HD:
-            raise ValueError(f"d_k = {self.dk} > {_HD} is not supported (d_v may be any size)")
+        if self.dk > _HD and not split_k:
+            raise ValueError(f"d_k = {self.dk} > {_HD} is not supported by this operator (d_v may be any size)")
         self.hd = 32 if self.dk <= 32 else _HD
         seg = 16 // q.element_size()                    # elements per 16 bytes
         thin = narrow and self.hd == 32
         self.kw = self.dk if thin and self.dk % seg == 0 else self.hd                          # key width the kernel sees
         self.vw = self.dv if thin and self.dv <= self.hd and self.dv % seg == 0 else self.hd   # value width per block
-        self.nb = (self.dv + self.vw - 1) // self.vw
+        self.nkb = (self.dk + self.kw - 1) // self.kw   # key blocks (1 unless d_k > 64)
+        self.nb = (self.dv + self.vw - 1) // self.vw    # value blocks
         self.native = self.dk == self.kw and self.dv == self.vw
-        self.pre = fmap if self.dk != self.kw else 0    # feature map applied here, before the padding
-        self.fmap = 0 if self.pre else fmap             # feature map left to the kernel
+        self.pre = fmap if self.dk != self.nkb * self.kw else 0    # feature map applied here, before the padding
+        self.fmap = 0 if self.pre else fmap                        # feature map left to the kernel
 
-    def _blocks(self, x):  # (B,T,H,kw) -> (B,T,H*nb,kw), every block a copy
-        if self.nb == 1:
-            return x
-        return x[:, :, :, None].expand(self.B, self.T, self.H, self.nb, self.kw).reshape(self.B, self.T, self.H * self.nb, self.kw)
-
-    def qk(self, x):
+    # the kernel's head axis is (H, nkb, nb) flattened
+    def qk(self, x):  # (B,T,H,dk) -> (B,T,H*nkb*nb,kw), every value block a copy
         if self.native:
             return x
         if self.pre:
             xf = x if x.dtype in (torch.float32, torch.float64) else x.float()
             x = (torch.nn.functional.elu(xf) + 1).to(x.dtype)
-        return self._blocks(torch.nn.functional.pad(x, (0, self.kw - self.dk)))
+        x = torch.nn.functional.pad(x, (0, self.nkb * self.kw - self.dk))
+        if self.nkb * self.nb == 1:
+            return x
+        x = x.reshape(self.B, self.T, self.H, self.nkb, 1, self.kw).expand(self.B, self.T, self.H, self.nkb, self.nb, self.kw)
+        return x.reshape(self.B, self.T, self.H * self.nkb * self.nb, self.kw)
 
-    def v(self, x):
+    def v(self, x):  # (B,T,H,dv) -> (B,T,H*nkb*nb,vw), every key block a copy
         if self.native:
             return x
         x = torch.nn.functional.pad(x, (0, self.nb * self.vw - self.dv))
-        return x.reshape(self.B, self.T, self.H * self.nb, self.vw)
+        x = x.reshape(self.B, self.T, self.H, 1, self.nb, self.vw).expand(self.B, self.T, self.H, self.nkb, self.nb, self.vw)
+        return x.reshape(self.B, self.T, self.H * self.nkb * self.nb, self.vw)
 
-    def per_head(self, x):  # (B,T,H) -> (B,T,H*nb)
-        return x if self.nb == 1 else x.repeat_interleave(self.nb, dim=2)
+    def per_head(self, x):  # (B,T,H) -> (B,T,H*nkb*nb)
+        return x if self.nkb * self.nb == 1 else x.repeat_interleave(self.nkb * self.nb, dim=2)
 
-    def state_in(self, S):  # (B,H,dv,dk) -> (B,H*nb,vw,kw)
+    def state_in(self, S):  # (B,H,dv,dk) -> (B,H*nkb*nb,vw,kw)
         if S is None or self.native:
             return S
-        S = torch.nn.functional.pad(S, (0, self.kw - self.dk, 0, self.nb * self.vw - self.dv))
-        return S.reshape(self.B, self.H * self.nb, self.vw, self.kw)
+        S = torch.nn.functional.pad(S, (0, self.nkb * self.kw - self.dk, 0, self.nb * self.vw - self.dv))
+        S = S.reshape(self.B, self.H, self.nb, self.vw, self.nkb, self.kw).permute(0, 1, 4, 2, 3, 5)
+        return S.reshape(self.B, self.H * self.nkb * self.nb, self.vw, self.kw)
 
-    def z_in(self, z):  # (B,H,dk) -> (B,H*nb,kw)
+    def z_in(self, z):  # (B,H,dk) -> (B,H*nb,kw)   (normalised read-out: one key block)
         if z is None or self.native:
             return z
         z = torch.nn.functional.pad(z, (0, self.kw - self.dk))
         return z if self.nb == 1 else z.repeat_interleave(self.nb, dim=1)
 
-    def out(self, o):  # (B,T,H*nb,vw) -> (B,T,H,dv)
-        return o if self.native else o.reshape(self.B, o.shape[1], self.H, self.nb * self.vw)[..., :self.dv]
+    def out(self, o):  # (B,T,H*nkb*nb,vw) -> (B,T,H,dv): the key blocks' outputs add up
+        if self.native:
+            return o
+        o = o.reshape(self.B, o.shape[1], self.H, self.nkb, self.nb * self.vw)
+        if self.nkb > 1:
+            o = (o if o.dtype in (torch.float32, torch.float64) else o.float()).sum(3).to(o.dtype)
+        else:
+            o = o[:, :, :, 0]
+        return o[..., :self.dv]
 
     def state_out(self, S):
-        return S if self.native else S.reshape(self.B, self.H, self.nb * self.vw, self.kw)[:, :, :self.dv, :self.dk]
+        if self.native:
+            return S
+        S = S.reshape(self.B, self.H, self.nkb, self.nb, self.vw, self.kw).permute(0, 1, 3, 4, 2, 5)
+        return S.reshape(self.B, self.H, self.nb * self.vw, self.nkb * self.kw)[:, :, :self.dv, :self.dk]
 
     def z_out(self, z):
         return z if self.native else z.reshape(self.B, self.H, self.nb, self.kw)[:, :, 0, :self.dk]
@@ -224,7 +240,7 @@ class _LinearAttention(torch.autograd.Function):
 def linear_attention(q, k, v, done, S0=None, feature_map="none"):
     """Causal unnormalised linear attention, chunked: S_t = r_t S_{t-1} + v_t phi(k_t)^T,
     o_t = S_t phi(q_t) (linear_attention.py:62-86,105).  Returns (o, S_last)."""
-    hd = _Heads(q, v, _FMAP[feature_map], narrow=True)
+    hd = _Heads(q, v, _FMAP[feature_map], narrow=True, split_k=True)
     o, S_last = _LinearAttention.apply(hd.qk(q), hd.qk(k), hd.v(v), done, hd.state_in(S0), hd.fmap)
     return hd.out(o), hd.state_out(S_last)
 
@@ -301,7 +317,7 @@ def gated_linear_attention(q, k, v, g, done, S0=None, feature_map="none"):
     """Linear attention with a scalar log-decay g:(B,T,H) per step and head:
     S_t = r_t exp(g_t) S_{t-1} + v_t phi(k_t)^T, o_t = S_t phi(q_t) -- the Mamba cell's algebra
     (mamba.py:109-122) in chunked form.  Returns (o, S_last)."""
-    hd = _Heads(q, v, _FMAP[feature_map], narrow=True)
+    hd = _Heads(q, v, _FMAP[feature_map], narrow=True, split_k=True)
     o, S_last = _GatedLinearAttention.apply(hd.qk(q), hd.qk(k), hd.v(v), hd.per_head(g), done, hd.state_in(S0),
                                             hd.fmap)
     return hd.out(o), hd.state_out(S_last)

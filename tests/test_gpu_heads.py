@@ -1,5 +1,5 @@
-"""GPU parity of the differentiable ops at head dims other than the kernels' 64 (zero-padded
-keys, value blocks as extra heads) against the oracle at the native dims."""
+"""GPU parity of the differentiable ops at head dims other than the kernels' own (zero-padded
+keys, value blocks and key blocks as extra heads) against the oracle at the native dims."""
 import numpy as np
 import pytest
 import torch
@@ -70,6 +70,43 @@ def test_other_head_dims(dk, dv, dtype, op):
         assert t.grad.shape == t.shape
         errs[n] = relerr(t.grad, ref[n])
     assert all(e <= tol for e in errs.values()), errs
+
+
+@pytest.mark.parametrize("dk,dv", [(128, 64), (96, 40), (130, 16)])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("op", ["linear", "gated"])
+def test_key_dims_above_64_run_as_key_blocks_whose_outputs_add_up(dk, dv, dtype, op):
+    """o = sum over 64-wide key blocks of S[:, block] q[block]: plain and gated linear attention, outputs,
+    state and every gradient against the oracle at the native dims."""
+    from memorax_amd import functional as F
+    B, T, H = 2, 75, 2
+    x = _data(B, T, H, dk, dv, dk * 3 + dv, dtype)
+    print(f"case key blocks op={op} dk={dk} dv={dv} dtype={dtype}", flush=True)
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    q, k, v = (dev(x[n], td).requires_grad_() for n in ("q", "k", "v"))
+    S0 = dev(x["S0"]).requires_grad_()
+    done = dev(x["done"])
+    extra = {}
+    if op == "linear":
+        o, Sl = F.linear_attention(q, k, v, done, S0, "elu1")
+        ref = G.linear_attention_grads(x["q"], x["k"], x["v"], x["done"], x["S0"], x["do"], x["dSl"], "elu1")
+    else:
+        g = dev(x["g"]).requires_grad_()
+        o, Sl = F.gated_linear_attention(q, k, v, g, done, S0, "elu1")
+        ref = G.gated_linear_attention_grads(x["q"], x["k"], x["v"], x["g"], x["done"], x["S0"], x["do"], x["dSl"], "elu1")
+        extra = {"dg": g}
+    assert o.shape == (B, T, H, dv) and Sl.shape == (B, H, dv, dk)
+    ((o.float() * dev(x["do"])).sum() + (Sl * dev(x["dSl"])).sum()).backward()
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    errs = {"o": relerr(o, ref["o"]), "S_last": relerr(Sl, ref["S_last"])}
+    for n, t in dict(dq=q, dk=k, dv=v, dS0=S0, **extra).items():
+        assert t.grad.shape == t.shape
+        errs[n] = relerr(t.grad, ref[n])
+    assert all(e <= tol for e in errs.values()), errs
+    with pytest.raises(ValueError):  # the normalised read-out and the delta rule couple the key features
+        F.normalised_linear_attention(q, k, v, done, None, None, "elu1", 1e-6)
+    with pytest.raises(ValueError):
+        F.delta_rule(q, k, v, dev(x["beta"], td), done, None)
 
 
 def test_linear_attention_model_at_the_reference_guides_head_dim():

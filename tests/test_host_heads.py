@@ -13,7 +13,8 @@ def _rand(*s, seed=0):
     return torch.from_numpy(np.random.default_rng(seed).standard_normal(s))
 
 
-@pytest.mark.parametrize("dk,dv", [(16, 16), (32, 64), (64, 96), (16, 130), (64, 64), (32, 32), (33, 20), (24, 8), (15, 16), (16, 31)])
+@pytest.mark.parametrize("dk,dv", [(16, 16), (32, 64), (64, 96), (16, 130), (64, 64), (32, 32), (33, 20), (24, 8), (15, 16), (16, 31),
+                                   (128, 64), (96, 40), (130, 130)])
 @pytest.mark.parametrize("op", ["linear", "normalised", "gated", "delta"])
 def test_padding_and_value_blocks_reproduce_the_native_recurrence(dk, dv, op):
     B, T, H = 2, 9, 2
@@ -23,15 +24,23 @@ def test_padding_and_value_blocks_reproduce_the_native_recurrence(dk, dv, op):
     done = torch.from_numpy(np.random.default_rng(8).random((B, T)) < 0.2)
     fm = "none" if op == "delta" else "elu1"
     narrow = op != "delta"  # the linear-attention kernels of the 32-wide build take narrower heads as they are
-    hd = _Heads(q, v, 0 if op == "delta" else 1, narrow=narrow)
+    split_k = op in ("linear", "gated")  # outputs linear in the state: key features beyond 64 run as further blocks
+    if dk > 64 and not split_k:
+        with pytest.raises(ValueError):
+            _Heads(q, v, 0 if op == "delta" else 1, narrow=narrow, split_k=split_k)
+        return
+    hd = _Heads(q, v, 0 if op == "delta" else 1, narrow=narrow, split_k=split_k)
     w = 32 if dk <= 32 else 64  # the 32-wide kernels serve keys of up to 32 features
     seg = 16 // q.element_size()
     kw = dk if narrow and w == 32 and dk % seg == 0 else w
     vw = dv if narrow and w == 32 and dv <= 32 and dv % seg == 0 else w
-    assert hd.hd == w and (hd.kw, hd.vw) == (kw, vw) and hd.native == (dk == kw and dv == vw) and hd.nb == -(-dv // vw)
+    nkb = -(-dk // kw)
+    assert hd.hd == w and (hd.kw, hd.vw) == (kw, vw) and hd.native == (dk == kw and dv == vw)
+    assert hd.nb == -(-dv // vw) and hd.nkb == nkb and (nkb == 1 or dk > 64)
     kfm = "elu1" if hd.fmap else "none"   # the feature map the kernel would be asked to apply
     qq, kk, vv, SS = hd.qk(q), hd.qk(k), hd.v(v), hd.state_in(S0)
-    assert qq.shape == (B, T, H * hd.nb, kw) and vv.shape == (B, T, H * hd.nb, vw) and SS.shape == (B, H * hd.nb, vw, kw)
+    nh = H * hd.nb * nkb
+    assert qq.shape == (B, T, nh, kw) and vv.shape == (B, T, nh, vw) and SS.shape == (B, nh, vw, kw)
     if op == "linear":
         o, Sl = G.linear_attention_t(qq, kk, vv, done, SS, kfm)
         ro, rS = G.linear_attention_t(q, k, v, done, S0, fm)
