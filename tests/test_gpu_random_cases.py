@@ -1,0 +1,101 @@
+"""Seeded random sweep of the chunked kernels against the oracle: shapes, head dims (64, 32 and, for the
+linear-attention family, narrow heads with d_k != d_v), dtypes, reset rates, feature maps, optional initial
+state and state gradient, every factor path of the delta rule -- combinations the hand-written case lists
+do not enumerate.  Every case is drawn from a fixed seed, so a failure names its case."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import grad as G
+from gpu_util import TOL_BF16, TOL_F32, bf16_round, dev, relerr
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = [1, 2, 31, 32, 33, 63, 64, 65, 96, 127, 130, 257, 300]
+CASES_PER_SEED = 16
+
+
+def _case(rng):
+    op = str(rng.choice(["la", "lapar", "gated", "norm", "delta", "deltanet"]))
+    dtype = str(rng.choice(["f32", "bf16"]))
+    if op in ("delta", "deltanet"):
+        dk = dv = int(rng.choice([32, 64]))
+    else:
+        seg = 8 if dtype == "bf16" else 4
+        kind = int(rng.integers(0, 3))
+        if kind == 0:
+            dk = dv = 64
+        elif kind == 1:
+            dk = dv = 32
+        else:  # narrow heads: whole 16-byte segments, widths independent of one another
+            dk, dv = (int(rng.integers(1, 32 // seg + 1)) * seg for _ in range(2))
+    return dict(op=op, dtype=dtype, dk=dk, dv=dv, B=int(rng.integers(1, 4)), H=int(rng.integers(1, 4)),
+                T=int(rng.choice(LENGTHS)), p=float(rng.choice([0.0, 0.01, 0.1, 0.5])), fm=int(rng.integers(0, 2)),
+                S0=bool(rng.integers(0, 2)), dSl=bool(rng.integers(0, 2)),
+                path=str(rng.choice(["auto", "parallel", "inline"])))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_cases(seed):
+    from memorax_amd import kernels as K
+    rng = np.random.default_rng(1000 + seed)
+    failures = []
+    for it in range(CASES_PER_SEED):
+        c = _case(rng)
+        op, dtype, dk, dv, B, T, H, fm = (c[n] for n in ("op", "dtype", "dk", "dv", "B", "T", "H", "fm"))
+        desc = f"seed={seed} it={it} " + " ".join(f"{k}={v}" for k, v in c.items())
+        print("case", desc, flush=True)
+        td = torch.bfloat16 if dtype == "bf16" else torch.float32
+        tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+        r = lambda *s: rng.standard_normal(s).astype(np.float32)
+        q, k, v, do = r(B, T, H, dk) / 6, r(B, T, H, dk) / 6, r(B, T, H, dv), r(B, T, H, dv)
+        S0 = r(B, H, dv, dk) * 0.1 if c["S0"] else None
+        dSl = r(B, H, dv, dk) * 0.1 if c["dSl"] else None
+        done = rng.random((B, T)) < c["p"]
+        g, beta, z0 = -np.abs(r(B, T, H)) * 0.3, r(B, T, H) * 1.5, np.abs(r(B, H, dk))
+        if op in ("delta", "deltanet"):
+            q, k = r(B, T, H, dk), r(B, T, H, dk)
+            if op == "delta":  # unit keys and gates in (0, 1); deltanet forms both inside the kernels
+                k, beta = k / np.linalg.norm(k, axis=-1, keepdims=True), 1 / (1 + np.exp(-beta))
+        if dtype == "bf16":
+            q, k, v, do, beta = (bf16_round(a) for a in (q, k, v, do, beta))
+        tq, tk, tv, tdo = (dev(a, td) for a in (q, k, v, do))
+        dn = dev(done)
+        tS0, tdSl = (None if a is None else dev(a) for a in (S0, dSl))
+        name = "elu1" if fm else "none"
+        if op in ("la", "lapar"):
+            o, Sl, chk = K.linear_attn_fwd(tq, tk, tv, dn, tS0, fm, chunk_parallel=(op == "lapar"))
+            got = K.linear_attn_bwd(tq, tk, tv, dn, chk, tdo, tdSl, fm)
+            ref = G.linear_attention_grads(q, k, v, done, S0, do, dSl, name)
+            names = ("dq", "dk", "dv", "dS0")
+        elif op == "gated":
+            o, Sl, chk = K.gated_linear_attn_fwd(tq, tk, tv, dev(g), dn, tS0, fm)
+            got = K.gated_linear_attn_bwd(tq, tk, tv, dev(g), dn, chk, tdo, tdSl, fm, S_last=Sl)
+            ref = G.gated_linear_attention_grads(q, k, v, g, done, S0, do, dSl, name)
+            names = ("dq", "dk", "dv", "dg", "dS0")
+        elif op == "norm":
+            o, den, Sl, zl, chk = K.linear_attn_norm_fwd(tq, tk, tv, dn, tS0, dev(z0), 1, 1e-6)
+            got = K.linear_attn_norm_bwd(tq, tk, tv, dn, chk, o, den, tdo, tdSl, None, 1, 1e-6)
+            ref = G.normalised_linear_attention_grads(q, k, v, done, S0, z0, do, dSl, None, "elu1", 1e-6)
+            names = ("dq", "dk", "dv", "dS0", "dz0")
+        else:
+            pro = op == "deltanet"
+            tb = dev(beta, td)
+            o, Sl, chk = K.delta_rule_fwd(tq, tk, tv, tb, dn, tS0, prologue=pro, factor_path=c["path"])
+            got = K.delta_rule_bwd(tq, tk, tv, tb, dn, chk, tdo, tdSl, prologue=pro)
+            ref = (G.deltanet_grads if pro else G.delta_rule_grads)(q, k, v, beta, done, S0, do, dSl)
+            names = ("dq", "dk", "dv", "dbeta", "dS0")
+        torch.cuda.synchronize()
+        errs = {"o": relerr(o, ref["o"]), "S_last": relerr(Sl, ref["S_last"])}
+        for n, a in zip(names, got):
+            if a is None or (B * T * H < 4 and n in ("dbeta", "dg")):  # a lone scalar has no scale to be judged against
+                continue
+            # a gradient that is exactly zero in the oracle (dg at reset steps only, say) has no scale of its own
+            scale = max(np.abs(ref[n]).max(), 1e-3 * max(np.abs(ref["dq"]).max(), 1e-30))
+            errs[n] = float(np.abs(a.float().cpu().numpy() - ref[n]).max() / scale)
+        # the normalised read-out divides by a bf16-rounded denominator: its gradients carry that rounding twice
+        lim = tol * (1.5 if op == "norm" and dtype == "bf16" else 1.0)
+        bad = {n: e for n, e in errs.items() if not e <= lim}
+        if bad:
+            failures.append((desc, bad))
+    assert not failures, failures
