@@ -136,24 +136,25 @@ def test_rollout_steps_equal_sequence_call():
             assert relerr(a, _np(b_)) <= tol
 
 
-def test_mamba_model_matches_materialise_and_scan_reference():
+@pytest.mark.parametrize("P,N", [(64, 64), (16, 16), (32, 16)])  # head_dim, state_dim; (16, 16): mamba.py:37-38
+def test_mamba_model_matches_materialise_and_scan_reference(P, N):
     """Mamba(MambaCell) against the reference's own route: materialise h_t = (B dt) (x) x and the
     decay leaf, scan with the diagonal operator (mamba.py:109-135 under memoroid.py:60-91)."""
     from memorax_amd import sequence_models as sm
     torch.manual_seed(7)
-    B, T, Fe, H, d = 2, 90, 32, 2, 64
-    cell = sm.MambaCell(Fe, num_heads=H, head_dim=d, state_dim=d).cuda()
+    B, T, Fe, H = 2, 90, 32, 2
+    cell = sm.MambaCell(Fe, num_heads=H, head_dim=P, state_dim=N).cuda()
     model = sm.Mamba(cell)
     x, done = _inputs(B, T, Fe, 0.04, 8)
     carry, y = model(x, done)
-    assert carry[0].shape == (B, 1, H, d, d) and carry[1].shape == (B, 1, H, 1, 1)
+    assert carry[0].shape == (B, 1, H, N, P) and carry[1].shape == (B, 1, H, 1, 1)
     with torch.no_grad():
         hidden, B_proj, C_proj, z, dt = cell._project(x)
         g = dt * (-torch.exp(cell.A_log))[None, None, :]
         k = B_proj * dt[..., None]
     nxt, o = M.gated_linear_attention_memoroid(_np(C_proj), _np(k), _np(hidden), _np(g), _np(done.float()))
     yy = o + _np(cell.D)[None, None, :, None] * _np(hidden)
-    yy = yy.reshape(B, T, H * d)
+    yy = yy.reshape(B, T, H * P)
     yy = yy / np.sqrt((yy ** 2).mean(-1, keepdims=True) + 1e-6) * _np(cell.norm.scale)
     zz = _np(z)
     yy = yy * (zz / (1 + np.exp(-zz)))
