@@ -391,11 +391,12 @@ def bench_linear_attention(torch, K, np, dev):
     res["small_grid_bf16_8x4096x4x64"] = small
     del q, k, v, do
     # head dim 32 (the library's second build of the kernels) at 1024 environments x 128 steps x 4 heads,
-    # beside the same token-heads at head dim 64 (what a 32-wide model paid when it was padded)
+    # beside the same token-heads at head dim 64 (what a 32-wide model paid when it was padded) and at
+    # head dim 16 (the reference guides' size, which the 32-wide kernels take as it lies in memory)
     Bn, Tn, Hn = 1024, 128, 4
     dn = torch.rand((Bn, Tn), device="cuda") < 0.01
     hd = {}
-    for d in (32, 64):
+    for d in (16, 32, 64):
         q, k, v, do = (torch.randn((Bn, Tn, Hn, d), device="cuda").div_(8).to(torch.bfloat16) for _ in range(4))
 
         def fh():
