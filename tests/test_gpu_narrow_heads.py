@@ -145,3 +145,39 @@ def test_what_is_not_a_narrow_head_is_refused():
     assert lib.mrx_delta_rule_step(None, P(q[:, 0]), P(q[:, 0]), P(q[:, 0]), P(beta[:, 0]), P(dn[:, 0]), None, P(o[:, 0]), P(S),
                                    1, 1, 16, 16, 0, 0) == -2
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_reference_default_head_dim_at_scale(dtype):
+    """1024 environments x 128 steps x 8 heads x 16 features (the Mamba cell's default heads, mamba.py:36-38):
+    two calls over [0, 64) and [64, 128) with the state carried equal one call bit for bit (chunk boundaries
+    coincide), the backward is linear in the incoming gradient, and two batch rows match the oracle."""
+    from memorax_amd import kernels as K
+    B, T, H, d = 1024, 128, 8, 16
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    g = torch.Generator(device="cuda").manual_seed(5)
+    q, k, v, do = (torch.randn((B, T, H, d), device="cuda", generator=g).div_(4).to(td) for _ in range(4))
+    glog = -torch.rand((B, T, H), device="cuda", generator=g) * 0.3
+    done = torch.rand((B, T), device="cuda", generator=g) < 0.01
+    S0 = torch.randn((B, H, d, d), device="cuda", generator=g) * 0.1
+    print(f"case narrow at scale dtype={dtype}", flush=True)
+    o, Sl, chk = K.gated_linear_attn_fwd(q, k, v, glog, done, S0, 1)
+    h = T // 2
+    o1, S1, _ = K.gated_linear_attn_fwd(q[:, :h].contiguous(), k[:, :h].contiguous(), v[:, :h].contiguous(),
+                                        glog[:, :h].contiguous(), done[:, :h].contiguous(), S0, 1, save_chk=False)
+    o2, S2, _ = K.gated_linear_attn_fwd(q[:, h:].contiguous(), k[:, h:].contiguous(), v[:, h:].contiguous(),
+                                        glog[:, h:].contiguous(), done[:, h:].contiguous(), S1, 1, save_chk=False)
+    assert torch.equal(torch.cat([o1, o2], 1), o) and torch.equal(S2, Sl)
+    g1 = K.gated_linear_attn_bwd(q, k, v, glog, done, chk, do, None, 1, S_last=Sl)
+    g2 = K.gated_linear_attn_bwd(q, k, v, glog, done, chk, (do.float() * 2).to(td), None, 1, S_last=Sl)
+    for a, b in zip(g1, g2):  # doubling is exact in either dtype
+        assert torch.equal((a.float() * 2).to(a.dtype), b)
+    rows = [3, B - 1]
+    x = {n: t[rows].float().cpu().numpy() for n, t in (("q", q), ("k", k), ("v", v), ("do", do))}
+    ref = G.gated_linear_attention_grads(x["q"], x["k"], x["v"], glog[rows].cpu().numpy(), done[rows].cpu().numpy(),
+                                         S0[rows].cpu().numpy(), x["do"], None, "elu1")
+    got = dict(zip(("dq", "dk", "dv", "dg", "dS0"), g1))
+    errs = {"o": relerr(o[rows], ref["o"]), "S_last": relerr(Sl[rows], ref["S_last"])}
+    errs.update({n: relerr(got[n][rows], ref[n]) for n in got})
+    assert all(e <= tol for e in errs.values()), errs
