@@ -51,6 +51,26 @@ def _batched(core_rank, ref):
     return deco
 
 
+def _no_steps(x):
+    """No sequences or no time steps: the reference's scan then hands the carry back unchanged
+    (memoroid.py:60-91 scans the carry prepended to T = 0 elements) and there is nothing to launch."""
+    return x.shape[0] == 0 or x.shape[1] == 0
+
+
+def _scan_without_steps(b, h0, P0):
+    B, _, D = b.shape
+    h_last = b.new_zeros((B, D)) if h0 is None else h0 + 0
+    P_last = b.new_ones((B, D)) if P0 is None else P0.detach().clone()
+    return b.new_zeros(b.shape), h_last, P_last
+
+
+def _attention_without_steps(q, v, S0):
+    B, T, H, dk = q.shape
+    dv = v.shape[-1]
+    S_last = q.new_zeros((B, H, dv, dk), dtype=torch.float32) if S0 is None else S0.float() + 0
+    return v.new_zeros((B, T, H, dv)), S_last
+
+
 class _Heads:
     """Maps other head dims onto what the kernels take (the reference's cells take any head_dim; its
     guides use 16).  The 32-wide kernels serve d_k <= 32, the 64-wide ones the rest.  The kernels of the
@@ -170,6 +190,8 @@ def linear_scan(a, b, done, h0=None, P0=None):
     """Reset-aware diagonal recurrence h_t = a_t h_{t-1} + b_t (lru.py:92-95 scanned
     by memoroid.py:60-91).  a: (B,T,D) or (D,); b: (B,T,D); h0,P0: (B,D).
     P_last (the cumulative-decay leaf of the carry) is not differentiable."""
+    if _no_steps(b):
+        return _scan_without_steps(b, h0, P0)
     return _LinearScan.apply(a, b, done, h0, P0)
 
 
@@ -206,6 +228,8 @@ def mingru_scan(z, h_tilde, done, h0=None, P0=None):
     h_t = sigmoid(-z_t) h_{t-1} + sigmoid(z_t) g(h~_t), g(x) = x + 0.5 (x >= 0) | sigmoid(x), with the
     gate arithmetic inside the scan kernels.  z, h_tilde: (B,T,D) fp32; h0, P0: (B,D).
     Returns (h, h_last, P_last); P_last is not differentiable."""
+    if _no_steps(z):
+        return _scan_without_steps(z, h0, P0)
     return _MinGRUScan.apply(z, h_tilde, done, h0, P0)
 
 
@@ -240,6 +264,8 @@ class _LinearAttention(torch.autograd.Function):
 def linear_attention(q, k, v, done, S0=None, feature_map="none"):
     """Causal unnormalised linear attention, chunked: S_t = r_t S_{t-1} + v_t phi(k_t)^T,
     o_t = S_t phi(q_t) (linear_attention.py:62-86,105).  Returns (o, S_last)."""
+    if _no_steps(q):
+        return _attention_without_steps(q, v, S0)
     hd = _Heads(q, v, _FMAP[feature_map], narrow=True, split_k=True)
     o, S_last = _LinearAttention.apply(hd.qk(q), hd.qk(k), hd.v(v), done, hd.state_in(S0), hd.fmap)
     return hd.out(o), hd.state_out(S_last)
@@ -278,6 +304,10 @@ def normalised_linear_attention(q, k, v, done, S0=None, z0=None, feature_map="el
     """Causal linear attention with the normalised read-out of LinearAttentionCell.read
     (linear_attention.py:93-110) in the same kernel: z_t = r_t z_{t-1} + phi(k_t),
     o_t = S_t phi(q_t) / max(phi(q_t) . z_t, eps).  Returns (o, S_last, z_last)."""
+    if _no_steps(q):
+        B, _, H, dk = q.shape
+        z_last = q.new_zeros((B, H, dk), dtype=torch.float32) if z0 is None else z0.float() + 0
+        return (*_attention_without_steps(q, v, S0), z_last)
     hd = _Heads(q, v, _FMAP[feature_map], narrow=True)
     o, S_last, z_last = _NormalisedLinearAttention.apply(hd.qk(q), hd.qk(k), hd.v(v), done, hd.state_in(S0),
                                                          hd.z_in(z0), hd.fmap, float(eps))
@@ -317,6 +347,8 @@ def gated_linear_attention(q, k, v, g, done, S0=None, feature_map="none"):
     """Linear attention with a scalar log-decay g:(B,T,H) per step and head:
     S_t = r_t exp(g_t) S_{t-1} + v_t phi(k_t)^T, o_t = S_t phi(q_t) -- the Mamba cell's algebra
     (mamba.py:109-122) in chunked form.  Returns (o, S_last)."""
+    if _no_steps(q):
+        return _attention_without_steps(q, v, S0)
     hd = _Heads(q, v, _FMAP[feature_map], narrow=True, split_k=True)
     o, S_last = _GatedLinearAttention.apply(hd.qk(q), hd.qk(k), hd.v(v), hd.per_head(g), done, hd.state_in(S0),
                                             hd.fmap)
@@ -356,6 +388,8 @@ class _DeltaRule(torch.autograd.Function):
 def delta_rule(q, k, v, beta, done, S0=None):
     """DeltaNet recurrence S_t = r_t S_{t-1}(I - beta_t k_t k_t^T) + beta_t v_t k_t^T,
     o_t = S_t q_t, in chunked WY form.  Returns (o, S_last)."""
+    if _no_steps(q):
+        return _attention_without_steps(q, v, S0)
     hd = _Heads(q, v)
     o, S_last = _DeltaRule.apply(hd.qk(q), hd.qk(k), hd.v(v), hd.per_head(beta), done, hd.state_in(S0))
     return hd.out(o), hd.state_out(S_last)
@@ -366,6 +400,8 @@ def deltanet(q, k, v, beta_raw, done, S0=None):
     """The DeltaNet cell's recurrence on its raw projections: delta_rule with
     k / max(|k|, 1e-12) and sigmoid(beta_raw) formed inside the kernels (the normalised keys and
     the gates never reach memory; gradients come back w.r.t. the raw arrays).  Returns (o, S_last)."""
+    if _no_steps(q):
+        return _attention_without_steps(q, v, S0)
     hd = _Heads(q, v)   # zero-padding the keys leaves their norm unchanged
     o, S_last = _DeltaRule.apply(hd.qk(q), hd.qk(k), hd.v(v), hd.per_head(beta_raw), done, hd.state_in(S0), True)
     return hd.out(o), hd.state_out(S_last)
@@ -380,6 +416,8 @@ def propagate_sensitivities(decay, jacobians, sensitivity, done):
     array; the kernel reads the Jacobians once and writes only the final state."""
     import math
     B, T, H = decay.shape
+    if B == 0 or T == 0:  # nothing to propagate through
+        return {name: sensitivity[name] for name in sorted(jacobians.keys())}
     decay = decay.contiguous()
     out = {}
     for name in sorted(jacobians.keys()):
