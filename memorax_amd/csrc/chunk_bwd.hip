@@ -86,10 +86,10 @@ struct NormBwdArgs {
 // fp32, the state entering chunk c and slot c of dS_last -- then a (B,H,NC,64,64) array -- the gradient
 // of the state leaving it (la_states.h); the workgroup forms the chunk's dQ, dK, dV from them and neither
 // walks the state nor accumulates its gradient.
-// RAG: narrow heads, as in the forward kernel: q, k and their gradients are dka wide in memory, v, dout, o and
+// NARROW: narrow heads, as in the forward kernel: q, k and their gradients are dka wide in memory, v, dout, o and
 // dv dva, states [dva][dka], z [dka]; tiles keep the build's width, zero beyond, and only the rows' own
 // width is ever stored.
-template <typename T, int C, bool FMAP, bool GATED, bool NORM, bool PAR = false, bool RAG = false>
+template <typename T, int C, bool FMAP, bool GATED, bool NORM, bool PAR = false, bool NARROW = false>
 __global__ void __launch_bounds__(256, 2)
 la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
               const float *__restrict__ glog, const void *__restrict__ done, int done_f32,
@@ -127,15 +127,15 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lg = lane >> 4;
     const int bh = sequence_of_block(blockIdx.x, gridDim.x, H), b = bh / H, h = bh % H;
-    const int dkw = RAG ? dka : HD, dvw = RAG ? dva : HD;  // row widths in memory
+    const int dkw = NARROW ? dka : HD, dvw = NARROW ? dva : HD;  // row widths in memory
     const int64_t rs = (int64_t)H * dkw, rsv = (int64_t)H * dvw;  // row strides of q, k / v, dout, o
     const int64_t base = ((int64_t)b * Tlen * H + h) * dkw, basev = ((int64_t)b * Tlen * H + h) * dvw;
-    const bool segk = !RAG || (tid % (HD / TT<T>::KP)) * TT<T>::KP < dkw;  // this thread's 16-byte segment lies inside a q/k row
-    const bool segv = !RAG || (tid % (HD / TT<T>::KP)) * TT<T>::KP < dvw;  // ... inside a v row
+    const bool segk = !NARROW || (tid % (HD / TT<T>::KP)) * TT<T>::KP < dkw;  // this thread's 16-byte segment lies inside a q/k row
+    const bool segv = !NARROW || (tid % (HD / TT<T>::KP)) * TT<T>::KP < dvw;  // ... inside a v row
     const int NC = (Tlen + C - 1) / C;
     const int c_hi = PAR ? (int)blockIdx.y : NC - 1, c_lo = PAR ? c_hi : 0;  // the chunks this workgroup walks, downwards
     const int64_t slot = PAR ? ((int64_t)bh * NC + c_hi) * dvw : (int64_t)bh * dvw;  // in state rows
-    auto in_state = [&](int dvv, int dk0) { return !RAG || (dvv < dvw && dk0 < dkw); };
+    auto in_state = [&](int dvv, int dk0) { return !NARROW || (dvv < dvw && dk0 < dkw); };
 
     using TMS = TileMap<HD, HD, NW>;
     using TMA = TileMap<C, C, NW>;
@@ -157,8 +157,8 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
         const int dkt = TMS::mt(w, mi * TMS::NBW) * 16;
         dzacc[mi] = f32x4{0.f, 0.f, 0.f, 0.f};
         if (NORM && na.dz_last) {
-            if (VN) { if (!RAG || dkt + li < dkw) dzacc[mi][0] = na.dz_last[(int64_t)bh * dkw + dkt + li]; }
-            else if (!RAG || dkt + 4 * lg < dkw) dzacc[mi] = *reinterpret_cast<const f32x4 *>(na.dz_last + (int64_t)bh * dkw + dkt + 4 * lg);
+            if (VN) { if (!NARROW || dkt + li < dkw) dzacc[mi][0] = na.dz_last[(int64_t)bh * dkw + dkt + li]; }
+            else if (!NARROW || dkt + 4 * lg < dkw) dzacc[mi] = *reinterpret_cast<const f32x4 *>(na.dz_last + (int64_t)bh * dkw + dkt + 4 * lg);
         }
     }
 
@@ -218,11 +218,11 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     // part 0: q, k; 1: v, dout; 2: S and the per-row scalars.
     const int tlast = c_hi * C;
     int64_t roff[IO::PASSES];
-    int64_t roffv[RAG ? IO::PASSES : 1];  // v, dout, o where their rows are not as wide as those of q and k
+    int64_t roffv[NARROW ? IO::PASSES : 1];  // v, dout, o where their rows are not as wide as those of q and k
 #pragma unroll
     for (int p = 0; p < IO::PASSES; ++p) {
         roff[p] = base + (int64_t)(tlast + IO::row_of(tid, p)) * rs + (tid % IO::SEGS) * IO::KP;
-        if (RAG) roffv[p] = basev + (int64_t)(tlast + IO::row_of(tid, p)) * rsv + (tid % IO::SEGS) * IO::KP;
+        if (NARROW) roffv[p] = basev + (int64_t)(tlast + IO::row_of(tid, p)) * rsv + (tid % IO::SEGS) * IO::KP;
     }
     int64_t soff = ((int64_t)bh * NC + c_hi) * dvw * dkw +
                    (WALK ? li * dkw + 4 * lg : (tid / IOS::SEGS) * dkw + (tid % IOS::SEGS) * IOS::KP);
@@ -244,7 +244,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     rq.v[p] = in && segk ? *reinterpret_cast<const typename IO::F *>(q + roff[p]) : z;
                     rk.v[p] = in && segk ? *reinterpret_cast<const typename IO::F *>(k + roff[p]) : z;
                 } else {
-                    const int64_t ov = RAG ? roffv[p] : roff[p];
+                    const int64_t ov = NARROW ? roffv[p] : roff[p];
                     rv.v[p] = in && segv ? *reinterpret_cast<const typename IO::F *>(v + ov) : z;
                     rdo.v[p] = in && segv ? *reinterpret_cast<const typename IO::F *>(dout + ov) : z;
                     if (NORM) ro.v[p] = in && segv ? *reinterpret_cast<const typename IO::F *>((const T *)na.o + ov) : z;
@@ -255,7 +255,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
 #pragma unroll
                 for (int p = 0; p < IOS::PASSES; ++p)
                     if (IOS::FULL || IOS::row_of(tid, p) < HD) {  // a [32][32] tile has fewer segments than threads
-                        if (!RAG || (IOS::row_of(tid, p) < dvw && (tid % IOS::SEGS) * IOS::KP < dkw))
+                        if (!NARROW || (IOS::row_of(tid, p) < dvw && (tid % IOS::SEGS) * IOS::KP < dkw))
                             rS.v[p] = *reinterpret_cast<const typename IOS::F *>(reinterpret_cast<const T *>(S_chk) + soff + p * IOS::RPP * dkw);
                         else
                             rS.v[p] = z;
@@ -285,13 +285,13 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                     rden[p] = (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen ? na.den[noff[p]] : 1.f;
                     noff[p] -= C;
                 }
-                if (!RAG || 4 * (tid % (HD / 4)) < dkw) rz = *reinterpret_cast<const f32x4 *>(na.z_chk + zoff);
+                if (!NARROW || 4 * (tid % (HD / 4)) < dkw) rz = *reinterpret_cast<const f32x4 *>(na.z_chk + zoff);
                 zoff -= dkw;
             }
 #pragma unroll
             for (int p = 0; p < IO::PASSES; ++p) {
                 roff[p] -= (int64_t)C * rs;
-                if (RAG) roffv[p] -= (int64_t)C * rsv;
+                if (NARROW) roffv[p] -= (int64_t)C * rsv;
             }
             soff -= dvw * dkw;
             doff -= C;
@@ -640,8 +640,8 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
         for (int mi = 0; mi < TMS::MBW; ++mi) {
             const int dkt = TMS::mt(w, mi * TMS::NBW) * 16;
             float *dst = na.dz0 + (int64_t)bh * dkw + dkt;
-            if (VN) { if (!RAG || dkt + li < dkw) dst[li] = dzacc[mi][0]; }
-            else if (!RAG || dkt + 4 * lg < dkw) *reinterpret_cast<f32x4 *>(dst + 4 * lg) = dzacc[mi];
+            if (VN) { if (!NARROW || dkt + li < dkw) dst[li] = dzacc[mi][0]; }
+            else if (!NARROW || dkt + 4 * lg < dkw) *reinterpret_cast<f32x4 *>(dst + 4 * lg) = dzacc[mi];
         }
     }
 }
@@ -1081,9 +1081,9 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     }
 }
 
-template <typename T, int C, bool FMAP, bool GATED, bool NORM, bool PAR, bool RAG> struct LaBwdReg {
+template <typename T, int C, bool FMAP, bool GATED, bool NORM, bool PAR, bool NARROW> struct LaBwdReg {
     static constexpr int smem = LaBwdSmem<T, C, GATED, NORM>::total;
-    static inline KernelRegistrar reg{reinterpret_cast<const void *>(la_bwd_kernel<T, C, FMAP, GATED, NORM, PAR, RAG>), smem};
+    static inline KernelRegistrar reg{reinterpret_cast<const void *>(la_bwd_kernel<T, C, FMAP, GATED, NORM, PAR, NARROW>), smem};
 };
 
 template <typename T, int C, bool FMAP, bool GATED = false, bool NORM = false, bool PAR = false>
@@ -1095,11 +1095,11 @@ int launch_la(hipStream_t st, const void *q, const void *k, const void *v, const
     if (const int rc = prepare_device(); rc != MRX_OK) return rc;
     const int64_t NC = (Tlen + C - 1) / C;
     if (PAR && NC > 65535) return MRX_ERR_INVALID_ARG;
-    auto go = [&](auto rag) {
-        constexpr bool RAG = decltype(rag)::value;
-        using Reg = LaBwdReg<T, C, FMAP, GATED, NORM, PAR, RAG>;
+    auto go = [&](auto narrow) {
+        constexpr bool NARROW = decltype(narrow)::value;
+        using Reg = LaBwdReg<T, C, FMAP, GATED, NORM, PAR, NARROW>;
         (void)&Reg::reg;  // the kernel is on the list mrx_init() walks
-        return launch_kernel(la_bwd_kernel<T, C, FMAP, GATED, NORM, PAR, RAG>,
+        return launch_kernel(la_bwd_kernel<T, C, FMAP, GATED, NORM, PAR, NARROW>,
                              dim3((unsigned)(B * H), PAR ? (unsigned)NC : 1u), dim3(256), Reg::smem, st, (const T *)q,
                              (const T *)k, (const T *)v, (const float *)glog, done, done_f32, S_chk,
                              (const float *)S_last, (const T *)dout, (const float *)dS_last, (T *)dq, (T *)dk, (T *)dv,

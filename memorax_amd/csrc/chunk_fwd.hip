@@ -74,13 +74,13 @@ struct NormArgs {
 // PAR (plain linear attention): one workgroup per chunk (grid.y = chunk) instead of one per sequence.
 // S_chk then is an input: slot c holds, in fp32, the state entering chunk c (la_states.h); the
 // workgroup forms the chunk's outputs from it and neither updates nor writes any state.
-// RAG (linear attention, all variants): narrow heads.  Keys and queries are dka wide in memory, values
+// NARROW (linear attention, all variants): narrow heads.  Keys and queries are dka wide in memory, values
 // and outputs dva (both at most the head dim of the build, whole 16-byte segments), and so are the
 // states (B,H,dva,dka) and z (B,H,dka).  Tiles in LDS and registers keep the build's width: what lies
 // beyond the rows' width is loaded as zero (after the feature map, phi(0) = 1 must not count) and never
 // stored.
 template <typename T, int C, bool DELTA, bool FMAP, bool GATED, bool NORM, bool PRO = false, bool TMIN = false,
-          bool PAR = false, bool RAG = false>
+          bool PAR = false, bool NARROW = false>
 __global__ void __launch_bounds__(NTHR, 2)  // 2 waves per SIMD: two workgroups share a CU
 chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const float *__restrict__ glog,
@@ -88,7 +88,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                  const float *__restrict__ S0, T *__restrict__ o, float *__restrict__ S_last,
                  void *__restrict__ S_chk, T *__restrict__ Tm_chk, int Tlen, int H, NormArgs na, int dka, int dva)
 {
-    static_assert(!RAG || !DELTA, "narrow heads: linear attention only");
+    static_assert(!NARROW || !DELTA, "narrow heads: linear attention only");
     static_assert(!(DELTA && GATED), "the gated variant is linear attention with a decay");
     static_assert(!NORM || (!DELTA && !GATED), "the normalised read-out belongs to plain linear attention");
     static_assert(!PRO || DELTA, "the prologue belongs to the delta rule");
@@ -121,12 +121,12 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lg = lane >> 4;
     const int bh = sequence_of_block(blockIdx.x, gridDim.x, H), b = bh / H, h = bh % H;
-    const int dkw = RAG ? dka : HD, dvw = RAG ? dva : HD;  // row widths in memory
+    const int dkw = NARROW ? dka : HD, dvw = NARROW ? dva : HD;  // row widths in memory
     const int64_t rs = (int64_t)H * dkw;   // row stride of q/k
     const int64_t rsv = (int64_t)H * dvw;  // ... of v/o
     const int64_t base = ((int64_t)b * Tlen * H + h) * dkw, basev = ((int64_t)b * Tlen * H + h) * dvw;
-    const bool segk = !RAG || (tid % (HD / TT<T>::KP)) * TT<T>::KP < dkw;  // this thread's 16-byte segment lies inside a q/k row
-    const bool segv = !RAG || (tid % (HD / TT<T>::KP)) * TT<T>::KP < dvw;  // ... inside a v row
+    const bool segk = !NARROW || (tid % (HD / TT<T>::KP)) * TT<T>::KP < dkw;  // this thread's 16-byte segment lies inside a q/k row
+    const bool segv = !NARROW || (tid % (HD / TT<T>::KP)) * TT<T>::KP < dvw;  // ... inside a v row
     const int NC = (Tlen + C - 1) / C;
     const int c_first = PAR ? (int)blockIdx.y : 0, c_end = PAR ? c_first + 1 : NC;  // the chunks this workgroup walks
 
@@ -138,7 +138,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
     for (int j = 0; j < TMS::TPW; ++j) {
         const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dv = TMS::nt(w, j) * 16 + li;
-        const bool in = !RAG || (dv < dvw && dk0 < dkw);
+        const bool in = !NARROW || (dv < dvw && dk0 < dkw);
         Sacc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
         if (PAR) {
             if (in) Sacc[j] = *reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(S_chk) +
@@ -160,8 +160,8 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         const int dkt = TMS::mt(w, mi * TMS::NBW) * 16;
         zacc[mi] = f32x4{0.f, 0.f, 0.f, 0.f};
         if (NORM && na.z0) {
-            if (VN) { if (!RAG || dkt + li < dkw) zacc[mi][0] = na.z0[(int64_t)bh * dkw + dkt + li]; }
-            else if (!RAG || dkt + 4 * lg < dkw) zacc[mi] = *reinterpret_cast<const f32x4 *>(na.z0 + (int64_t)bh * dkw + dkt + 4 * lg);
+            if (VN) { if (!NARROW || dkt + li < dkw) zacc[mi][0] = na.z0[(int64_t)bh * dkw + dkt + li]; }
+            else if (!NARROW || dkt + 4 * lg < dkw) zacc[mi] = *reinterpret_cast<const f32x4 *>(na.z0 + (int64_t)bh * dkw + dkt + 4 * lg);
         }
     }
     const Frag ones = TT<T>::ones();
@@ -175,12 +175,12 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     // Element offsets of what this thread loads for the chunk about to be prefetched; they advance
     // by one chunk per call (64-bit adds instead of per-chunk index multiplications).
     int64_t roff[IO::PASSES], boff[IO::PASSES];
-    int64_t roffv[RAG ? IO::PASSES : 1];  // v, where its rows are not as wide as those of q and k
+    int64_t roffv[NARROW ? IO::PASSES : 1];  // v, where its rows are not as wide as those of q and k
 #pragma unroll
     for (int p = 0; p < IO::PASSES; ++p) {
         const int r = IO::row_of(tid, p);
         roff[p] = base + (int64_t)(c_first * C + r) * rs + (tid % IO::SEGS) * IO::KP;  // q/k/v: row r, this thread's 16-byte segment
-        if (RAG) roffv[p] = basev + (int64_t)(c_first * C + r) * rsv + (tid % IO::SEGS) * IO::KP;
+        if (NARROW) roffv[p] = basev + (int64_t)(c_first * C + r) * rsv + (tid % IO::SEGS) * IO::KP;
         boff[p] = ((int64_t)b * Tlen + c_first * C + r) * H + h;                       // beta of row r
     }
     int64_t doff = (int64_t)b * Tlen + c_first * C + lane;  // done of chunk row `lane`
@@ -200,13 +200,13 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
             for (int p = 0; p < IO::PASSES; ++p)
                 dst.v[p] = seg_in && (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen
-                               ? *reinterpret_cast<const typename IO::F *>(src + (RAG && part == 2 ? roffv[p] : roff[p])) : z;
+                               ? *reinterpret_cast<const typename IO::F *>(src + (NARROW && part == 2 ? roffv[p] : roff[p])) : z;
         } else {
 #pragma unroll
             for (int p = 0; p < IO::PASSES; ++p) {
                 if (DELTA) rbrow[p] = (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen ? load_raw<T>(beta + boff[p]) : 0u;
                 roff[p] += (int64_t)C * rs;
-                if (RAG) roffv[p] += (int64_t)C * rsv;
+                if (NARROW) roffv[p] += (int64_t)C * rsv;
                 boff[p] += (int64_t)C * H;
             }
             if (TMIN) {
@@ -329,10 +329,10 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                         float *zc = (na.z_chk && pass == 0) ? na.z_chk + ((int64_t)bh * NC + c) * dkw + dkt : nullptr;
                         if (VN) {
                             sZ[dkt + li] = (T)zacc[mi][0];
-                            if (zc && (!RAG || dkt + li < dkw)) zc[li] = zacc[mi][0];
+                            if (zc && (!NARROW || dkt + li < dkw)) zc[li] = zacc[mi][0];
                         } else {
                             *reinterpret_cast<P4 *>(sZ + dkt + 4 * lg) = TT<T>::pack(zacc[mi][0], zacc[mi][1], zacc[mi][2], zacc[mi][3]);
-                            if (zc && (!RAG || dkt + 4 * lg < dkw)) *reinterpret_cast<f32x4 *>(zc + 4 * lg) = zacc[mi];
+                            if (zc && (!NARROW || dkt + 4 * lg < dkw)) *reinterpret_cast<f32x4 *>(zc + 4 * lg) = zacc[mi];
                         }
                     }
                 }
@@ -357,7 +357,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                     for (int p = 0; p < IOS::PASSES; ++p) {
                         const int r = IOS::row_of(tid, p), seg = tid % IOS::SEGS;
-                        if ((IOS::FULL || r < HD) && (!RAG || (r < dvw && seg * IOS::KP < dkw)))  // a [32][32] tile has fewer segments than threads
+                        if ((IOS::FULL || r < HD) && (!NARROW || (r < dvw && seg * IOS::KP < dkw)))  // a [32][32] tile has fewer segments than threads
                             *reinterpret_cast<typename IOS::F *>(reinterpret_cast<T *>(S_chk) + schk_off + r * dkw + seg * IOS::KP) =
                                 *reinterpret_cast<const typename IOS::F *>(sS + r * LDD + seg * IOS::KP);
                     }
@@ -365,7 +365,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
                     for (int j = 0; j < TMS::TPW; ++j) {
                         const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dv = TMS::nt(w, j) * 16 + li;
-                        if (!RAG || (dv < dvw && dk0 < dkw))
+                        if (!NARROW || (dv < dvw && dk0 < dkw))
                             *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(S_chk) + schk_off + dv * dkw + dk0) = Sacc[j];
                     }
                 }
@@ -558,7 +558,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
         for (int j = 0; j < TMS::TPW; ++j) {
             const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dv = TMS::nt(w, j) * 16 + li;
-            if (!RAG || (dv < dvw && dk0 < dkw))
+            if (!NARROW || (dv < dvw && dk0 < dkw))
                 *reinterpret_cast<f32x4 *>(S_last + ((int64_t)bh * dvw + dv) * dkw + dk0) = Sacc[j];
         }
     }
@@ -567,16 +567,16 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         for (int mi = 0; mi < TMS::MBW; ++mi) {
             const int dkt = TMS::mt(w, mi * TMS::NBW) * 16;
             float *zl = na.z_last + (int64_t)bh * dkw + dkt;
-            if (VN) { if (!RAG || dkt + li < dkw) zl[li] = zacc[mi][0]; }
-            else if (!RAG || dkt + 4 * lg < dkw) *reinterpret_cast<f32x4 *>(zl + 4 * lg) = zacc[mi];
+            if (VN) { if (!NARROW || dkt + li < dkw) zl[li] = zacc[mi][0]; }
+            else if (!NARROW || dkt + 4 * lg < dkw) *reinterpret_cast<f32x4 *>(zl + 4 * lg) = zacc[mi];
         }
     }
 }
 
-template <typename T, int C, bool DELTA, bool FMAP, bool GATED, bool NORM, bool PRO, bool TMIN, bool PAR, bool RAG> struct FwdReg {
+template <typename T, int C, bool DELTA, bool FMAP, bool GATED, bool NORM, bool PRO, bool TMIN, bool PAR, bool NARROW> struct FwdReg {
     static constexpr int smem = FwdSmem<T, C, DELTA, GATED, NORM>::total;
     static inline KernelRegistrar reg{
-        reinterpret_cast<const void *>(chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR, RAG>), smem};
+        reinterpret_cast<const void *>(chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR, NARROW>), smem};
 };
 
 // dka, dva: widths of the q/k and v/o rows in memory; less than the build's head dim (narrow heads,
@@ -591,11 +591,11 @@ int launch(hipStream_t st, const void *q, const void *k, const void *v, const vo
     if (const int rc = prepare_device(); rc != MRX_OK) return rc;
     const int64_t NC = (Tlen + C - 1) / C;
     if (PAR && NC > 65535) return MRX_ERR_INVALID_ARG;
-    auto go = [&](auto rag) {
-        constexpr bool RAG = decltype(rag)::value;
-        using Reg = FwdReg<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR, RAG>;
+    auto go = [&](auto narrow) {
+        constexpr bool NARROW = decltype(narrow)::value;
+        using Reg = FwdReg<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR, NARROW>;
         (void)&Reg::reg;  // the kernel is on the list mrx_init() walks
-        return launch_kernel(chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR, RAG>,
+        return launch_kernel(chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR, NARROW>,
                              dim3((unsigned)(B * H), PAR ? (unsigned)NC : 1u), dim3(NTHR), Reg::smem, st, (const T *)q,
                              (const T *)k, (const T *)v, (const T *)beta, (const float *)glog, done, done_f32,
                              (const float *)S0, (T *)o, (float *)S_last, S_chk, (T *)Tm_chk, (int)Tlen, (int)H, na,

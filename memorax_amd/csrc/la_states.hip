@@ -11,9 +11,9 @@ namespace {
 // One workgroup = one chunk of one sequence: slot <- sum over the kept rows r of y_r phi(x_r)^T,
 // kept = the chunk's last episode (forward: what the chunk adds to the state that leaves it) or its
 // first episode (backward: what it adds to the gradient of the state that enters it).
-// RAG: narrow heads -- x rows are dka wide in memory, y rows dva, a slot is [dva][dka]; the tiles keep the
+// NARROW: narrow heads -- x rows are dka wide in memory, y rows dva, a slot is [dva][dka]; the tiles keep the
 // build's width with zeros beyond (after the feature map).
-template <typename T, int C, bool FMAP, bool BWD, bool RAG>
+template <typename T, int C, bool FMAP, bool BWD, bool NARROW>
 __global__ void __launch_bounds__(256)
 la_chunk_state_kernel(const T *__restrict__ x, const T *__restrict__ y, const void *__restrict__ done, int done_f32,
                       float *__restrict__ slots, int Tlen, int H, int NC, int dka, int dva)
@@ -28,8 +28,8 @@ la_chunk_state_kernel(const T *__restrict__ x, const T *__restrict__ y, const vo
     const int li = lane & 15, lg = lane >> 4;
     const int bh = blockIdx.x, c = blockIdx.y, b = bh / H, h = bh % H;
     const int t0 = c * C;
-    const int dkw = RAG ? dka : HD, dvw = RAG ? dva : HD;
-    const bool segx = !RAG || (tid % IO::SEGS) * IO::KP < dkw, segy = !RAG || (tid % IO::SEGS) * IO::KP < dvw;
+    const int dkw = NARROW ? dka : HD, dvw = NARROW ? dva : HD;
+    const bool segx = !NARROW || (tid % IO::SEGS) * IO::KP < dkw, segy = !NARROW || (tid % IO::SEGS) * IO::KP < dvw;
 
     typename IO::Regs rx, ry;
     IO::zero(rx);
@@ -57,7 +57,7 @@ la_chunk_state_kernel(const T *__restrict__ x, const T *__restrict__ y, const vo
 #pragma unroll
     for (int j = 0; j < TMS::TPW; ++j) {
         const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dv = TMS::nt(w, j) * 16 + li;
-        if (!RAG || (dv < dvw && dk0 < dkw)) *reinterpret_cast<f32x4 *>(slot + dv * dkw + dk0) = acc[j];
+        if (!NARROW || (dv < dvw && dk0 < dkw)) *reinterpret_cast<f32x4 *>(slot + dv * dkw + dk0) = acc[j];
     }
 }
 
@@ -65,18 +65,18 @@ la_chunk_state_kernel(const T *__restrict__ x, const T *__restrict__ y, const vo
 // additions are sequential: the slots (and the reset flags) of the next group of eight chunks are
 // requested before the current group is summed and written back, so that one trip to memory is exposed
 // per sequence, not one per group.
-// RAG: narrow heads, the state's size is a run-time value.
-template <bool RAG>
+// NARROW: narrow heads, the state's size is a run-time value.
+template <bool NARROW>
 __global__ void __launch_bounds__(256)
 la_state_scan_kernel(float *__restrict__ slots, const float *__restrict__ init, float *__restrict__ fin,
                      const void *__restrict__ done, int done_f32, int Tlen, int H, int NC, int C, int backward, int Qn)
 {
-    const int Q = RAG ? Qn : HD * HD / 4;  // f32x4 per state (d_v * d_k / 4)
+    const int Q = NARROW ? Qn : HD * HD / 4;  // f32x4 per state (d_v * d_k / 4)
     constexpr int G = 8;            // chunks per group
     const int tid = threadIdx.x, lane = tid & 63;
     const int bh = blockIdx.x, b = bh / H;
     const int idx = blockIdx.y * 256 + tid;
-    const bool act = !RAG || idx < Q;  // a narrow state has fewer elements than the workgroup has threads; the idle lanes
+    const bool act = !NARROW || idx < Q;  // a narrow state has fewer elements than the workgroup has threads; the idle lanes
                                        // still bring their reset flags to the ballots
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
     f32x4 S = init && act ? reinterpret_cast<const f32x4 *>(init)[(int64_t)bh * Q + idx] : zero;

@@ -52,22 +52,22 @@ __device__ __forceinline__ float dot4(const f32x4 &a, const f32x4 &b)
     return a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
 }
 
-// RAG (linear attention, head dim 32 build): narrow heads -- q, k, z are dka wide, v, o dva, the state
+// NARROW (linear attention, head dim 32 build): narrow heads -- q, k, z are dka wide, v, o dva, the state
 // [dva][dka]; lanes and rows beyond take no part.
-template <typename T, bool DELTA, bool FMAP, bool RAG = false>
+template <typename T, bool DELTA, bool FMAP, bool NARROW = false>
 __global__ void __launch_bounds__(256)
 step_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
             const T *__restrict__ beta, const float *__restrict__ glog, const void *__restrict__ done, int done_f32,
             const float *S_in, const float *z_in, T *__restrict__ o, float *S_out, float *z_out, int H,
             float eps, int dka, int dva)  // S_in/S_out and z_in/z_out may alias (update in place)
 {
-    static_assert(!RAG || !DELTA, "narrow heads: linear attention only");
+    static_assert(!NARROW || !DELTA, "narrow heads: linear attention only");
     const int tid = threadIdx.x, c4 = tid % LPR, r0 = tid / LPR;
     const int64_t bh = blockIdx.x;
     const int b = (int)(bh / H);
     const bool reset = done_at(done, done_f32, b);
-    const int dkw = RAG ? dka : HD, dvw = RAG ? dva : HD;
-    const bool cin = !RAG || 4 * c4 < dkw;  // this lane's four dk lie inside a row
+    const int dkw = NARROW ? dka : HD, dvw = NARROW ? dva : HD;
+    const bool cin = !NARROW || 4 * c4 < dkw;  // this lane's four dk lie inside a row
     const T *qp = q + bh * dkw, *kp = k + bh * dkw, *vp = v + bh * dvw;
 
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -85,11 +85,11 @@ step_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restric
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
         const int row = r0 + RPP * p;
-        s[p] = (Sp && !reset && cin && (!RAG || row < dvw)) ? *reinterpret_cast<const f32x4 *>(Sp + row * dkw + 4 * c4) * decay : zero4;
+        s[p] = (Sp && !reset && cin && (!NARROW || row < dvw)) ? *reinterpret_cast<const f32x4 *>(Sp + row * dkw + 4 * c4) * decay : zero4;
     }
     float u[NP];
 #pragma unroll
-    for (int p = 0; p < NP; ++p) u[p] = (!RAG || r0 + RPP * p < dvw) ? (float)vp[r0 + RPP * p] : 0.f;
+    for (int p = 0; p < NP; ++p) u[p] = (!NARROW || r0 + RPP * p < dvw) ? (float)vp[r0 + RPP * p] : 0.f;
     if (DELTA) {
         const float bb = (float)beta[bh];
 #pragma unroll
@@ -108,7 +108,7 @@ step_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restric
     for (int p = 0; p < NP; ++p) {
         const int row = r0 + RPP * p;
         s[p] += k4 * u[p];
-        const bool rin = !RAG || row < dvw;
+        const bool rin = !NARROW || row < dvw;
         if (cin && rin) *reinterpret_cast<f32x4 *>(So + row * dkw + 4 * c4) = s[p];
         const float x = reduce_row(dot4(s[p], q4));
         if (c4 == 0 && rin) o[bh * dvw + row] = (T)(x / den);
@@ -140,8 +140,8 @@ int launch_step(hipStream_t st, const void *q, const void *k, const void *v, con
                 int done_f32, const float *S_in, const float *z_in, void *o, float *S_out, float *z_out,
                 int64_t B, int64_t H, float eps, int64_t dka = HD, int64_t dva = HD, const float *glog = nullptr)
 {
-    auto go = [&](auto rag) {
-        return launch_kernel((step_kernel<T, DELTA, FMAP, decltype(rag)::value>), dim3((unsigned)(B * H)), dim3(256), 0, st,
+    auto go = [&](auto narrow) {
+        return launch_kernel((step_kernel<T, DELTA, FMAP, decltype(narrow)::value>), dim3((unsigned)(B * H)), dim3(256), 0, st,
                              (const T *)q, (const T *)k, (const T *)v, (const T *)beta, glog, done, done_f32, S_in, z_in,
                              (T *)o, S_out, z_out, (int)H, eps, (int)dka, (int)dva);
     };
