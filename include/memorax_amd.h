@@ -138,10 +138,11 @@ int mrx_linear_scan_bwd(void *stream, const void *a, const void *h,
  * Narrow heads: the linear-attention family -- mrx_linear_attn_*, mrx_gated_linear_attn_*,
  * mrx_linear_attn_norm_*, mrx_linear_attn_*_chunk_parallel, mrx_linear_attn_step and
  * mrx_gated_linear_attn_step -- also takes any
- * dk <= 32 and dv <= 32, independent of one another, whose rows are a whole number of 16-byte segments
+ * dk <= 64 and dv <= 64, independent of one another, whose rows are a whole number of 16-byte segments
  * (multiples of 4 in float32, of 8 in bfloat16; the reference's guides use head_dim = 16).  Every array
- * keeps its dense (.., dv, dk) / (.., dk) / (.., dv) layout at those widths; the 32-wide kernels pad
- * on the fly.  The delta-rule entry points keep to 64 and 32. */
+ * keeps its dense (.., dv, dk) / (.., dk) / (.., dv) layout at those widths; the kernels pad on the fly
+ * (the 32-wide build when both widths are at most 32, else the 64-wide one).  The delta-rule entry
+ * points keep to 64 and 32. */
 int mrx_linear_attn_fwd(void *stream, const void *q, const void *k,
                         const void *v, const void *done, const void *S0,
                         void *o, void *S_last, void *S_chk, int64_t B,

@@ -1105,9 +1105,7 @@ int launch_la(hipStream_t st, const void *q, const void *k, const void *v, const
                              (const float *)S_last, (const T *)dout, (const float *)dS_last, (T *)dq, (T *)dk, (T *)dv,
                              (float *)dg, (float *)dS0, (int)Tlen, (int)H, na, (int)dka, (int)dva);
     };
-    if constexpr (MRX_HD == 32) {
-        if (dka != HD || dva != HD) return go(std::true_type{});  // narrow heads
-    }
+    if (dka != HD || dva != HD) return go(std::true_type{});  // narrow heads
     return go(std::false_type{});
 }
 
@@ -1120,9 +1118,9 @@ int check_bwd(const void *q, const void *k, const void *v, const void *done, con
     if (B <= 0 || T <= 0 || H <= 0 || dk <= 0 || dv <= 0) return MRX_ERR_INVALID_ARG;
     if (dtype != MRX_F32 && dtype != MRX_BF16) return dtype == MRX_C64 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
     if (done_dtype != MRX_DONE_U8 && done_dtype != MRX_DONE_F32) return MRX_ERR_INVALID_ARG;
-    // narrow: linear attention in the head dim 32 build also takes narrower rows of whole 16-byte segments
+    // narrow: linear attention also takes rows narrower than the build's head dim, in whole 16-byte segments
     const int64_t seg = dtype == MRX_BF16 ? 8 : 4;
-    const bool narrow_ok = narrow && MRX_HD == 32 && dk <= HD && dv <= HD && dk % seg == 0 && dv % seg == 0;
+    const bool narrow_ok = narrow && dk <= HD && dv <= HD && dk % seg == 0 && dv % seg == 0;
     if ((dk != HD || dv != HD) && !narrow_ok) return MRX_ERR_UNSUPPORTED;
     if (B * H >= (1ll << 31) || T >= (1ll << 30)) return MRX_ERR_INVALID_ARG;
     const void *ps[] = {q, k, v, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0};

@@ -580,7 +580,7 @@ template <typename T, int C, bool DELTA, bool FMAP, bool GATED, bool NORM, bool 
 };
 
 // dka, dva: widths of the q/k and v/o rows in memory; less than the build's head dim (narrow heads,
-// linear attention only, head dim 32 build) selects the kernel instance that pads on the fly.
+// linear attention only) selects the kernel instance that pads on the fly.
 template <typename T, int C, bool DELTA, bool FMAP, bool GATED = false, bool NORM = false, bool PRO = false,
           bool TMIN = false, bool PAR = false>
 int launch(hipStream_t st, const void *q, const void *k, const void *v, const void *beta,
@@ -601,14 +601,14 @@ int launch(hipStream_t st, const void *q, const void *k, const void *v, const vo
                              (const float *)S0, (T *)o, (float *)S_last, S_chk, (T *)Tm_chk, (int)Tlen, (int)H, na,
                              (int)dka, (int)dva);
     };
-    if constexpr (MRX_HD == 32 && !DELTA) {
+    if constexpr (!DELTA) {
         if (dka != HD || dva != HD) return go(std::true_type{});
     }
     return go(std::false_type{});
 }
 
-// narrow: the entry point also serves heads narrower than the build's (linear attention in the head dim 32
-// build: rows of whole 16-byte segments, padded inside the kernels)
+// narrow: the entry point also serves heads narrower than the build's (linear attention: rows of whole
+// 16-byte segments, padded inside the kernels)
 int check_common(const void *q, const void *k, const void *v, const void *done, const void *o,
                  const void *S0, const void *S_last, const void *S_chk, int64_t B, int64_t T,
                  int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype, bool narrow = false)
@@ -618,7 +618,7 @@ int check_common(const void *q, const void *k, const void *v, const void *done, 
     if (dtype != MRX_F32 && dtype != MRX_BF16) return dtype == MRX_C64 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
     if (done_dtype != MRX_DONE_U8 && done_dtype != MRX_DONE_F32) return MRX_ERR_INVALID_ARG;
     const int64_t seg = dtype == MRX_BF16 ? 8 : 4;  // elements per 16 bytes
-    const bool narrow_ok = narrow && MRX_HD == 32 && dk <= HD && dv <= HD && dk % seg == 0 && dv % seg == 0;
+    const bool narrow_ok = narrow && dk <= HD && dv <= HD && dk % seg == 0 && dv % seg == 0;
     if ((dk != HD || dv != HD) && !narrow_ok) return MRX_ERR_UNSUPPORTED;
     if (B * H >= (1ll << 31) || T >= (1ll << 30)) return MRX_ERR_INVALID_ARG;
     if (!aligned(q, 16) || !aligned(k, 16) || !aligned(v, 16) || !aligned(o, 16) || !aligned(S0, 16) ||

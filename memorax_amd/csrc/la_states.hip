@@ -129,11 +129,9 @@ int launch_states(hipStream_t st, const void *x, const void *y, const void *done
 #define MRX_LAUNCH(FM, BW, RG)                                                                                         \
     launch_kernel((la_chunk_state_kernel<T, C, FM, BW, RG>), grid, block, 0, st, (const T *)x, (const T *)y, done,       \
                   done_f32, slots, (int)Tlen, (int)H, (int)NC, (int)dk, (int)dv)
-    if constexpr (MRX_HD == 32) {
-        if (dk != HD || dv != HD) {  // narrow heads
-            if (fmap) return backward ? MRX_LAUNCH(true, true, true) : MRX_LAUNCH(true, false, true);
-            return backward ? MRX_LAUNCH(false, true, true) : MRX_LAUNCH(false, false, true);
-        }
+    if (dk != HD || dv != HD) {  // narrow heads
+        if (fmap) return backward ? MRX_LAUNCH(true, true, true) : MRX_LAUNCH(true, false, true);
+        return backward ? MRX_LAUNCH(false, true, true) : MRX_LAUNCH(false, false, true);
     }
     if (fmap) return backward ? MRX_LAUNCH(true, true, false) : MRX_LAUNCH(true, false, false);
     return backward ? MRX_LAUNCH(false, true, false) : MRX_LAUNCH(false, false, false);

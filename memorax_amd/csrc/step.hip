@@ -52,7 +52,7 @@ __device__ __forceinline__ float dot4(const f32x4 &a, const f32x4 &b)
     return a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
 }
 
-// NARROW (linear attention, head dim 32 build): narrow heads -- q, k, z are dka wide, v, o dva, the state
+// NARROW (linear attention): narrow heads -- q, k, z are dka wide, v, o dva, the state
 // [dva][dka]; lanes and rows beyond take no part.
 template <typename T, bool DELTA, bool FMAP, bool NARROW = false>
 __global__ void __launch_bounds__(256)
@@ -123,9 +123,9 @@ int check_step(const void *q, const void *k, const void *v, const void *done, co
     if (B <= 0 || H <= 0 || dk <= 0 || dv <= 0) return MRX_ERR_INVALID_ARG;
     if (dtype != MRX_F32 && dtype != MRX_BF16) return dtype == MRX_C64 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
     if (done_dtype != MRX_DONE_U8 && done_dtype != MRX_DONE_F32) return MRX_ERR_INVALID_ARG;
-    // narrow: linear attention in the head dim 32 build also takes narrower rows of whole 16-byte segments
+    // narrow: linear attention also takes rows narrower than the build's head dim, in whole 16-byte segments
     const int64_t seg = dtype == MRX_BF16 ? 8 : 4;
-    const bool narrow_ok = narrow && MRX_HD == 32 && dk <= HD && dv <= HD && dk % seg == 0 && dv % seg == 0;
+    const bool narrow_ok = narrow && dk <= HD && dv <= HD && dk % seg == 0 && dv % seg == 0;
     if ((dk != HD || dv != HD) && !narrow_ok) return MRX_ERR_UNSUPPORTED;
     if (B * H >= (1ll << 31)) return MRX_ERR_INVALID_ARG;
     const void *ps[] = {q, k, v, S_in, o, S_out};
@@ -145,7 +145,7 @@ int launch_step(hipStream_t st, const void *q, const void *k, const void *v, con
                              (const T *)q, (const T *)k, (const T *)v, (const T *)beta, glog, done, done_f32, S_in, z_in,
                              (T *)o, S_out, z_out, (int)H, eps, (int)dka, (int)dva);
     };
-    if constexpr (MRX_HD == 32 && !DELTA) {
+    if constexpr (!DELTA) {
         if (dka != HD || dva != HD) return go(std::true_type{});  // narrow heads
     }
     return go(std::false_type{});

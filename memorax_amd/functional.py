@@ -74,7 +74,7 @@ def _attention_without_steps(q, v, S0):
 class _Heads:
     """Maps other head dims onto what the kernels take (the reference's cells take any head_dim; its
     guides use 16).  The 32-wide kernels serve d_k <= 32, the 64-wide ones the rest.  The kernels of the
-    linear-attention family (`narrow`) in the 32-wide build take any d_k, d_v <= 32 that is a whole
+    linear-attention family (`narrow`) take any d_k, d_v up to their build's width that is a whole
     number of 16-byte segments as it is; everything else goes through padding: d_k below the kernel's
     width is zero-padded -- after the feature map, since phi(0) = 1 would otherwise count -- and d_v is
     zero-padded to a multiple of the value width and split into blocks that run as extra heads sharing
@@ -91,9 +91,8 @@ class _Heads:
             raise ValueError(f"d_k = {self.dk} > {_HD} is not supported by this operator (d_v may be any size)")
         self.hd = 32 if self.dk <= 32 else _HD
         seg = 16 // q.element_size()                    # elements per 16 bytes
-        thin = narrow and self.hd == 32
-        self.kw = self.dk if thin and self.dk % seg == 0 else self.hd                          # key width the kernel sees
-        self.vw = self.dv if thin and self.dv <= self.hd and self.dv % seg == 0 else self.hd   # value width per block
+        self.kw = self.dk if narrow and self.dk <= self.hd and self.dk % seg == 0 else self.hd   # key width the kernel sees
+        self.vw = self.dv if narrow and self.dv <= self.hd and self.dv % seg == 0 else self.hd   # value width per block
         self.nkb = (self.dk + self.kw - 1) // self.kw   # key blocks (1 unless d_k > 64)
         self.nb = (self.dv + self.vw - 1) // self.vw    # value blocks
         self.native = self.dk == self.kw and self.dv == self.vw

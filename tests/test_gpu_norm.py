@@ -209,7 +209,7 @@ def test_normalised_rejects_bad_arguments():
                                                            None, 1, 4, 1, dk, 64, dt, 0, 1, 1e-6)
     assert fwd(p, 64, 0) == 0
     assert fwd(None, 64, 0) == -1     # den is required
-    assert fwd(p, 32, 0) == -2        # unsupported head dim
+    assert fwd(p, 72, 0) == -2        # unsupported head dim
     assert fwd(p, 64, 2) == -2        # complex64
     bwd = lambda zc: lib.mrx_linear_attn_norm_bwd(None, p, p, p, p, p, p, zc, p, p, p, None, None, p, p, p, None, None,
                                                   1, 4, 1, 64, 64, 0, 0, 1, 1e-6)

@@ -22,13 +22,13 @@ def _case(rng):
         dk = dv = int(rng.choice([32, 64]))
     else:
         seg = 8 if dtype == "bf16" else 4
-        kind = int(rng.integers(0, 3))
+        kind = int(rng.integers(0, 4))
         if kind == 0:
             dk = dv = 64
         elif kind == 1:
             dk = dv = 32
-        else:  # narrow heads: whole 16-byte segments, widths independent of one another
-            dk, dv = (int(rng.integers(1, 32 // seg + 1)) * seg for _ in range(2))
+        else:  # narrow heads: whole 16-byte segments, widths independent of one another, up to 32 or up to 64
+            dk, dv = (int(rng.integers(1, (32 if kind == 2 else 64) // seg + 1)) * seg for _ in range(2))
     return dict(op=op, dtype=dtype, dk=dk, dv=dv, B=int(rng.integers(1, 4)), H=int(rng.integers(1, 4)),
                 T=int(rng.choice(LENGTHS)), p=float(rng.choice([0.0, 0.01, 0.1, 0.5])), fm=int(rng.integers(0, 2)),
                 S0=bool(rng.integers(0, 2)), dSl=bool(rng.integers(0, 2)),

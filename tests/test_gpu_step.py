@@ -189,5 +189,5 @@ def test_step_rejects_bad_arguments():
     assert lib.mrx_linear_attn_step(None, p, p, p, p, p, None, p, p, None, 1, 1, 64, 64, 0, 0, 7, 1e-6) == -1
     assert lib.mrx_gated_linear_attn_step(None, p, p, p, p, p, p, p, p, 1, 1, 64, 64, 0, 0, 0) == 0
     assert lib.mrx_gated_linear_attn_step(None, p, p, p, None, p, p, p, p, 1, 1, 64, 64, 0, 0, 0) == -1  # g missing
-    assert lib.mrx_gated_linear_attn_step(None, p, p, p, p, p, p, p, p, 1, 1, 48, 48, 0, 0, 0) == -2
+    assert lib.mrx_gated_linear_attn_step(None, p, p, p, p, p, p, p, p, 1, 1, 72, 72, 0, 0, 0) == -2
     torch.cuda.synchronize()

@@ -14,7 +14,7 @@ def _rand(*s, seed=0):
 
 
 @pytest.mark.parametrize("dk,dv", [(16, 16), (32, 64), (64, 96), (16, 130), (64, 64), (32, 32), (33, 20), (24, 8), (15, 16), (16, 31),
-                                   (128, 64), (96, 40), (130, 130)])
+                                   (128, 64), (96, 40), (130, 130), (48, 48), (40, 64), (64, 24)])
 @pytest.mark.parametrize("op", ["linear", "normalised", "gated", "delta"])
 def test_padding_and_value_blocks_reproduce_the_native_recurrence(dk, dv, op):
     B, T, H = 2, 9, 2
@@ -32,8 +32,8 @@ def test_padding_and_value_blocks_reproduce_the_native_recurrence(dk, dv, op):
     hd = _Heads(q, v, 0 if op == "delta" else 1, narrow=narrow, split_k=split_k)
     w = 32 if dk <= 32 else 64  # the 32-wide kernels serve keys of up to 32 features
     seg = 16 // q.element_size()
-    kw = dk if narrow and w == 32 and dk % seg == 0 else w
-    vw = dv if narrow and w == 32 and dv <= 32 and dv % seg == 0 else w
+    kw = dk if narrow and dk <= w and dk % seg == 0 else w
+    vw = dv if narrow and dv <= w and dv % seg == 0 else w
     nkb = -(-dk // kw)
     assert hd.hd == w and (hd.kw, hd.vw) == (kw, vw) and hd.native == (dk == kw and dv == vw)
     assert hd.nb == -(-dv // vw) and hd.nkb == nkb and (nkb == 1 or dk > 64)
