@@ -117,7 +117,11 @@ int mrx_linear_scan_fwd(void *stream, const void *a, const void *b,
  * (conj is the identity for MRX_F32; for MRX_C64 cotangents follow the
  * torch.autograd convention, the complex conjugate of JAX's).
  * h is the forward output; g = dL/dh (B,T,D); g_last = dL/dh_last (B,D, nullable).
- * da is per step (B,T,D) even when a is time-invariant (the caller reduces). */
+ * da is per step (B,T,D), also when a is time-invariant (a_time_invariant = 1: the caller reduces);
+ * with a_time_invariant = MRX_A_TIME_INVARIANT_SUM_DA the kernel sums the per-step terms over the
+ * sequence itself and da is (B,D) -- the gradient of the broadcast lambda of lru.py:86 / s5.py is then
+ * its sum over B, and the (B,T,D) array is neither written nor read back. */
+#define MRX_A_TIME_INVARIANT_SUM_DA 2
 int mrx_linear_scan_bwd(void *stream, const void *a, const void *h,
                         const void *done, const void *h0, const void *g,
                         const void *g_last, void *da, void *db, void *dh0,

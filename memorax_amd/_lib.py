@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libmemorax_amd.so")
 MRX_F32, MRX_BF16, MRX_C64 = 0, 1, 2
 MRX_DONE_U8, MRX_DONE_F32 = 0, 1
 MRX_FMAP_NONE, MRX_FMAP_ELU1 = 0, 1
+MRX_A_TIME_INVARIANT_SUM_DA = 2
 MRX_FACTORS_AUTO, MRX_FACTORS_PARALLEL, MRX_FACTORS_INLINE = 0, 1, 2
 MRX_NOALLOC_SCRATCH_BYTES = 32 << 20
 

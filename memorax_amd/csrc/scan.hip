@@ -253,7 +253,7 @@ diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hx, const E 
                      const E *__restrict__ h0, const E *__restrict__ g,
                      const E *__restrict__ g_last, E *__restrict__ da,
                      E *__restrict__ db, E *__restrict__ dh0, int T, int64_t D,
-                     int tiles, int NW, int a_ti)
+                     int tiles, int NW, int a_ti, int da_sum)
 {
     using V = Vec<E, VEC>;
     using O = Ops<E>;
@@ -272,6 +272,9 @@ diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hx, const E 
 
     V carry = vfill<E, VEC>(O::zero());  // lam_{t+1} entering from the right
     if (act && g_last) carry = *reinterpret_cast<const V *>(g_last + bi * D + col);
+    // da_sum (time-invariant a): da is (B,D), the sum of the per-step terms over the sequence -- what the
+    // gradient of a broadcast coefficient needs -- kept in registers instead of written per step
+    V dsum = vfill<E, VEC>(O::zero());
 
     const int span = NW * TS;
     int buf = 0;
@@ -401,10 +404,30 @@ diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hx, const E 
                     *reinterpret_cast<V *>(da + off) = oz;
                 } else {
                     *reinterpret_cast<V *>(db + off) = x[s];
-                    *reinterpret_cast<V *>(da + off) = o;
+                    if (da_sum) {
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) dsum.v[i] = O::madd(O::one(), dsum.v[i], o.v[i]);
+                    } else {
+                        *reinterpret_cast<V *>(da + off) = o;
+                    }
                 }
             }
         }
+    }
+    if (!MG && da_sum) {  // uniform over the workgroup
+        if (NW > 1) {
+            __syncthreads();  // the last fold has read sH
+            sH[w * 64 + lane] = dsum;
+            __syncthreads();
+            if (w == 0) {
+                for (int j = 1; j < NW; ++j) {
+                    const V dj = sH[j * 64 + lane];
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) dsum.v[i] = O::madd(O::one(), dsum.v[i], dj.v[i]);
+                }
+            }
+        }
+        if (w == 0 && act) *reinterpret_cast<V *>(da + bi * D + col) = dsum;
     }
     if (w == 0 && act && dh0) {
         // carry = lam_0 ; dh0 = done_0 ? 0 : conj(a_0) lam_0
@@ -560,7 +583,8 @@ diag_scan_bwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ hx, c
                             const void *__restrict__ done, int done_f32,
                             const E *__restrict__ h0, const E *__restrict__ g,
                             const E *__restrict__ g_last, E *__restrict__ da, E *__restrict__ db,
-                            E *__restrict__ dh0, int64_t B, int T, int64_t D, int64_t cols_per_row, int a_ti)
+                            E *__restrict__ dh0, int64_t B, int T, int64_t D, int64_t cols_per_row, int a_ti,
+                            int da_sum)
 {
     using V = Vec<E, VEC>;
     using O = Ops<E>;
@@ -569,6 +593,7 @@ diag_scan_bwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ hx, c
     const int64_t col = (gid % cols_per_row) * VEC;
     if (bi >= B) return;
     const int64_t row0 = bi * T;
+    V dsum = vfill<E, VEC>(O::zero());  // da_sum: the per-step terms summed over the sequence, da is (B,D)
     V lam = vfill<E, VEC>(O::zero());  // conj(abar_{t+1}) lam_{t+1} entering step t
     if (g_last) lam = *reinterpret_cast<const V *>(g_last + bi * D + col);
 
@@ -621,7 +646,12 @@ diag_scan_bwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ hx, c
                     }
                 }
                 *reinterpret_cast<V *>(db + off) = l;
-                *reinterpret_cast<V *>(da + off) = o;
+                if (!MG && da_sum) {
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) dsum.v[i] = O::madd(O::one(), dsum.v[i], o.v[i]);
+                } else {
+                    *reinterpret_cast<V *>(da + off) = o;
+                }
             }
         }
 #pragma unroll
@@ -631,6 +661,7 @@ diag_scan_bwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ hx, c
             for (int s = 0; s < SG; ++s) xx[s] = nx[s];
         }
     }
+    if (!MG && da_sum) *reinterpret_cast<V *>(da + bi * D + col) = dsum;
     if (dh0) *reinterpret_cast<V *>(dh0 + bi * D + col) = lam;  // conj(abar_0) lam_0
 }
 
@@ -772,7 +803,7 @@ int launch_fwd(hipStream_t st, const void *a, const void *b, const void *done,
 template <typename E, bool MG = false>
 int launch_bwd(hipStream_t st, const void *a, const void *hx, const void *h, const void *done,
                int done_f32, const void *h0, const void *g, const void *g_last, void *da,
-               void *db, void *dh0, int64_t B, int64_t T, int64_t D, int a_ti)
+               void *db, void *dh0, int64_t B, int64_t T, int64_t D, int a_ti, int da_sum = 0)
 {
     const bool al16 = aligned(a, 16) && aligned(hx, 16) && aligned(h, 16) && aligned(g, 16) && aligned(h0, 16) &&
                       aligned(g_last, 16) && aligned(da, 16) && aligned(db, 16) && aligned(dh0, 16);
@@ -787,7 +818,7 @@ int launch_bwd(hipStream_t st, const void *a, const void *hx, const void *h, con
             constexpr int VEC = decltype(vc)::value;
             rc = launch_kernel((diag_scan_bwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8), MG>), grid, block, 0, st,
                                (const E *)a, (const E *)hx, (const E *)h, done, done_f32, (const E *)h0, (const E *)g,
-                               (const E *)g_last, (E *)da, (E *)db, (E *)dh0, B, (int)T, D, cpr, a_ti);
+                               (const E *)g_last, (E *)da, (E *)db, (E *)dh0, B, (int)T, D, cpr, a_ti, da_sum);
         });
     } else {
         const dim3 grid((unsigned)(B * pl.tiles)), block(64 * pl.nw);
@@ -799,14 +830,14 @@ int launch_bwd(hipStream_t st, const void *a, const void *hx, const void *h, con
                     rc = launch_kernel((diag_scan_bwd_kernel<E, VEC, MG, 16>), grid, block, smem, st, (const E *)a,
                                        (const E *)hx, (const E *)h, done, done_f32, (const E *)h0, (const E *)g,
                                        (const E *)g_last, (E *)da, (E *)db, (E *)dh0, (int)T, D, pl.tiles,
-                                       pl.nw, a_ti);
+                                       pl.nw, a_ti, da_sum);
                     return;
                 }
             }
             rc = launch_kernel((diag_scan_bwd_kernel<E, VEC, MG>), grid, block, smem, st, (const E *)a,
                                (const E *)hx, (const E *)h, done, done_f32, (const E *)h0, (const E *)g,
                                (const E *)g_last, (E *)da, (E *)db, (E *)dh0, (int)T, D, pl.tiles,
-                               pl.nw, a_ti);
+                               pl.nw, a_ti, da_sum);
         });
     }
     return rc;
@@ -879,17 +910,19 @@ extern "C" int mrx_linear_scan_bwd(void *stream, const void *a, const void *h, c
     if (done_dtype != MRX_DONE_U8 && done_dtype != MRX_DONE_F32) return MRX_ERR_INVALID_ARG;
     if (done_dtype == MRX_DONE_F32 && !aligned(done, 4)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
+    if (a_time_invariant < 0 || a_time_invariant > MRX_A_TIME_INVARIANT_SUM_DA) return MRX_ERR_INVALID_ARG;
     const int ti = a_time_invariant != 0;
+    const int da_sum = a_time_invariant == MRX_A_TIME_INVARIANT_SUM_DA;
     if (dtype == MRX_F32) {
         if (!aligned(a, 4) || !aligned(h, 4) || !aligned(g, 4) || !aligned(da, 4) || !aligned(db, 4))
             return MRX_ERR_INVALID_ARG;
-        return launch_bwd<float>(st, a, nullptr, h, done, done_dtype, h0, g, g_last, da, db, dh0, B, T, D, ti);
+        return launch_bwd<float>(st, a, nullptr, h, done, done_dtype, h0, g, g_last, da, db, dh0, B, T, D, ti, da_sum);
     }
     if (dtype == MRX_C64) {
         if (!aligned(a, 8) || !aligned(h, 8) || !aligned(g, 8) || !aligned(da, 8) ||
             !aligned(db, 8) || !aligned(h0, 8) || !aligned(g_last, 8) || !aligned(dh0, 8))
             return MRX_ERR_INVALID_ARG;
-        return launch_bwd<c64>(st, a, nullptr, h, done, done_dtype, h0, g, g_last, da, db, dh0, B, T, D, ti);
+        return launch_bwd<c64>(st, a, nullptr, h, done, done_dtype, h0, g, g_last, da, db, dh0, B, T, D, ti, da_sum);
     }
     return dtype == MRX_BF16 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
 }

@@ -174,9 +174,10 @@ class _LinearScan(torch.autograd.Function):
         h0 = h0 if ctx.has_h0 else None
         g = torch.zeros_like(h) if g is None else g.contiguous()
         g_last = None if g_last is None else g_last.contiguous()
-        da, db, dh0 = K.linear_scan_bwd(a, h, ctx.done, h0, g, g_last)
-        if a.dim() == 1:
-            da = da.sum(dim=(0, 1))
+        ti = a.dim() == 1  # a broadcast coefficient: the kernel sums its gradient over time, the rest is (B,D)
+        da, db, dh0 = K.linear_scan_bwd(a, h, ctx.done, h0, g, g_last, sum_da=ti)
+        if ti:
+            da = da.sum(dim=0)
         return (da if ctx.needs_input_grad[0] else None,
                 db if ctx.needs_input_grad[1] else None,
                 None,

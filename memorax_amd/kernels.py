@@ -116,8 +116,9 @@ def linear_scan_last(a, b, done, h0=None):
     return h_last
 
 
-def linear_scan_bwd(a, h, done, h0, g, g_last=None):
-    """Returns (da (B,T,D) per step, db, dh0)."""
+def linear_scan_bwd(a, h, done, h0, g, g_last=None, sum_da=False):
+    """Returns (da (B,T,D) per step, db, dh0).  sum_da (time-invariant a only): da is (B,D), the per-step
+    terms summed over the sequence inside the kernel."""
     lib = _lib.load()
     B, T, D = g.shape
     dt = g.dtype
@@ -128,12 +129,14 @@ def linear_scan_bwd(a, h, done, h0, g, g_last=None):
     _chk(h0, "h0", dt, (B, D))
     _chk(g_last, "g_last", dt, (B, D))
     done, dd = _done(done, B, T)
-    da = torch.empty_like(g)
+    if sum_da and not ti:
+        raise ValueError("sum_da belongs to a time-invariant a")
+    da = torch.empty((B, D), dtype=dt, device=g.device) if sum_da else torch.empty_like(g)
     db = torch.empty_like(g)
     dh0 = torch.empty((B, D), dtype=dt, device=g.device)
     st = lib.mrx_linear_scan_bwd(_stream(), _ptr(a), _ptr(h), _ptr(done), _ptr(h0), _ptr(g),
                                  _ptr(g_last), _ptr(da), _ptr(db), _ptr(dh0), B, T, D, _DT[dt],
-                                 dd, int(ti))
+                                 dd, _lib.MRX_A_TIME_INVARIANT_SUM_DA if sum_da else int(ti))
     _lib.check(st, "mrx_linear_scan_bwd")
     return da, db, dh0
 

@@ -117,6 +117,33 @@ def test_scan_complex64(ti):
     assert relerr(da, ag["da"]) <= TOL and relerr(db, ag["db"]) <= TOL and relerr(dh0, ag["dh0"]) <= TOL
 
 
+@pytest.mark.parametrize("dtype", ["f32", "c64"])
+@pytest.mark.parametrize("shape", [(3, 77, 48), (2, 1, 5), (64, 128, 256), (1024, 128, 64), (4, 300, 1024), (2, 1000, 130)])
+def test_time_invariant_coefficient_gradient_summed_inside_the_kernel(dtype, shape):
+    """a_time_invariant = 2: da comes back as (B,D), the per-step terms summed over the sequence by the kernel
+    (both kernel families: the shapes cover the wave-split and the streaming plans) -- against the oracle's
+    gradient of the broadcast coefficient and against the per-step array summed afterwards."""
+    from memorax_amd import kernels as K
+    B, T, D = shape
+    rng = np.random.default_rng(B + T + D)
+    cplx = dtype == "c64"
+    rnd = (lambda *s: (rng.standard_normal(s) + 1j * rng.standard_normal(s)).astype(np.complex64)) if cplx \
+        else (lambda *s: rng.standard_normal(s).astype(np.float32))
+    lam = (rng.uniform(0.8, 0.999, D) * (np.exp(1j * rng.uniform(0, 3, D)) if cplx else 1.0)).astype(np.complex64 if cplx else np.float32)
+    b, g, h0, gl = rnd(B, T, D), rnd(B, T, D), rnd(B, D), rnd(B, D)
+    done = rng.random((B, T)) < 0.03
+    print(f"case scan da summed dtype={dtype} shape={shape}", flush=True)
+    h, _, _ = K.linear_scan_fwd(dev(lam), dev(b), dev(done), dev(h0))
+    da_steps, db1, dh01 = K.linear_scan_bwd(dev(lam), h, dev(done), dev(h0), dev(g), dev(gl))
+    da_sum, db2, dh02 = K.linear_scan_bwd(dev(lam), h, dev(done), dev(h0), dev(g), dev(gl), sum_da=True)
+    assert da_sum.shape == (B, D) and torch.equal(db1, db2) and torch.equal(dh01, dh02)
+    ref_steps = da_steps.cpu().numpy().astype(np.complex128 if cplx else np.float64).sum(1)
+    assert relerr(da_sum, ref_steps) <= TOL
+    if B * T * D <= 2_000_000:  # the oracle's autograd on the broadcast coefficient
+        ag = G.diag_scan_grads(np.broadcast_to(lam, (B, T, D)).copy(), b, done, h0, g, gl)
+        assert relerr(da_sum.sum(0), ag["da"].sum((0, 1))) <= TOL
+
+
 def test_linear_scan_autograd_function():
     import memorax_amd as mx
     B, T, D = 4, 50, 32
