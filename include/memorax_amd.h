@@ -139,14 +139,11 @@ int mrx_linear_scan_bwd(void *stream, const void *a, const void *h,
  * state entering each chunk that contains a reset; required by the backward call together with
  * S_last.  dk = dv = 64 or dk = dv = 32 (here and in every chunked and single-step entry point below;
  * the library holds a build of those kernels for either width; mrx_delta_rule_fwd_noalloc: 64 only).
- * Narrow heads: the linear-attention family -- mrx_linear_attn_*, mrx_gated_linear_attn_*,
- * mrx_linear_attn_norm_*, mrx_linear_attn_*_chunk_parallel, mrx_linear_attn_step and
- * mrx_gated_linear_attn_step -- also takes any
+ * Narrow heads: every chunked and single-step entry point but mrx_delta_rule_fwd_noalloc also takes any
  * dk <= 64 and dv <= 64, independent of one another, whose rows are a whole number of 16-byte segments
  * (multiples of 4 in float32, of 8 in bfloat16; the reference's guides use head_dim = 16).  Every array
  * keeps its dense (.., dv, dk) / (.., dk) / (.., dv) layout at those widths; the kernels pad on the fly
- * (the 32-wide build when both widths are at most 32, else the 64-wide one).  The delta-rule entry
- * points keep to 64 and 32. */
+ * (the 32-wide build when both widths are at most 32, else the 64-wide one). */
 int mrx_linear_attn_fwd(void *stream, const void *q, const void *k,
                         const void *v, const void *done, const void *S0,
                         void *o, void *S_last, void *S_chk, int64_t B,
@@ -358,8 +355,8 @@ int mrx_gated_linear_attn_bwd(void *stream, const void *q, const void *k,
  * What Memoroid.__call__ (memoroid.py:93-109) computes when T = 1, as PPO's rollout
  * does once per environment step (algorithms/ppo.py:105-143): one update of the
  * carry fused with the read-out, without the chunk machinery.
- *   q,k,v,o: (B,1,H,d) = (B,H,d) in `dtype`, d = 64 or 32 (the two linear-attention steps: narrow heads
- *   too, see mrx_linear_attn_fwd); done: (B,) ; S_in/S_out: (B,H,dv,dk) fp32.
+ *   q,k: (B,1,H,dk) = (B,H,dk), v,o: (B,H,dv) in `dtype` (head dims as for mrx_linear_attn_fwd);
+ *   done: (B,) ; S_in/S_out: (B,H,dv,dk) fp32.
  * S_in may be NULL (zero state) and may equal S_out (update in place).
  *
  * Linear attention (linear_attention.py:62-117):

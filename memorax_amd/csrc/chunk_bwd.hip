@@ -680,14 +680,16 @@ template <typename T, int C, int NW> struct DeltaBwdSmem : BwdDims<T, C> {
 // PRO: the cell's prologue is part of the call -- k_n = k / max(|k|, 1e-12), beta = sigmoid(b) are
 // formed while staging (as in the forward kernel) and the gradients are taken back through them:
 //   dk = (dk_n - k_n (k_n . dk_n)) / |k| ,   db = dbeta beta (1 - beta).
-template <typename T, int C, int NW, bool PRO>
+// NARROW: narrow heads, as in the linear-attention kernels -- q, k, dq, dk are dka wide in memory, v, dout, dv dva,
+// the states [dva][dka]; tiles keep the build's width with zeros beyond, only the rows' own width is stored.
+template <typename T, int C, int NW, bool PRO, bool NARROW = false>
 __global__ void __launch_bounds__(64 * NW, sizeof(T) == 2 ? 2 : 1)
 delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
                  const T *__restrict__ S_chk, const T *__restrict__ Tm_chk,
                  const T *__restrict__ dout, const float *__restrict__ dS_last, T *__restrict__ dq,
                  T *__restrict__ dk, T *__restrict__ dv, T *__restrict__ dbeta,
-                 float *__restrict__ dS0, int Tlen, int H)
+                 float *__restrict__ dS0, int Tlen, int H, int dka, int dva)
 {
     constexpr int NTHR = 64 * NW;
     using L = DeltaBwdSmem<T, C, NW>;
@@ -715,8 +717,12 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lg = lane >> 4;
     const int bh = sequence_of_block(blockIdx.x, gridDim.x, H), b = bh / H, h = bh % H;
-    const int64_t rs = (int64_t)H * HD;
-    const int64_t base = ((int64_t)b * Tlen * H + h) * HD;
+    const int dkw = NARROW ? dka : HD, dvw = NARROW ? dva : HD;  // row widths in memory
+    const int64_t rs = (int64_t)H * dkw, rsv = (int64_t)H * dvw;  // row strides of q, k / v, dout
+    const int64_t base = ((int64_t)b * Tlen * H + h) * dkw, basev = ((int64_t)b * Tlen * H + h) * dvw;
+    const bool segk = !NARROW || (tid % (HD / TT<T>::KP)) * TT<T>::KP < dkw;  // this thread's 16-byte segment lies inside a q/k row
+    const bool segv = !NARROW || (tid % (HD / TT<T>::KP)) * TT<T>::KP < dvw;  // ... inside a v row
+    auto in_state = [&](int dvv, int dk0) { return !NARROW || (dvv < dvw && dk0 < dkw); };
     const int NC = (Tlen + C - 1) / C;
 
     using TMS = TileMap<HD, HD, NW>;
@@ -728,8 +734,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
     for (int j = 0; j < TMS::TPW; ++j) {
         const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
-        dSacc[j] = dS_last ? *reinterpret_cast<const f32x4 *>(dS_last + ((int64_t)bh * HD + dvv) * HD + dk0)
-                           : f32x4{0.f, 0.f, 0.f, 0.f};
+        dSacc[j] = dS_last && in_state(dvv, dk0) ? *reinterpret_cast<const f32x4 *>(dS_last + ((int64_t)bh * dvw + dvv) * dkw + dk0)
+                                                 : f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
     typename IO::Regs rq, rk, rv, rdo;
@@ -741,13 +747,15 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     // iteration (64-bit adds instead of per-chunk index multiplications).
     const int tlast = (NC - 1) * C;
     int64_t roff[IO::PASSES], boff[IO::PASSES];
+    int64_t roffv[NARROW ? IO::PASSES : 1];  // v, dout where their rows are not as wide as those of q and k
 #pragma unroll
     for (int p = 0; p < IO::PASSES; ++p) {
         const int r = tlast + IO::row_of(tid, p);
         roff[p] = base + (int64_t)r * rs + (tid % IO::SEGS) * IO::KP;  // q/k/v/dout: row r, this thread's segment
+        if (NARROW) roffv[p] = basev + (int64_t)r * rsv + (tid % IO::SEGS) * IO::KP;
         boff[p] = ((int64_t)b * Tlen + r) * H + h;                     // beta of row r
     }
-    int64_t soff = ((int64_t)bh * NC + NC - 1) * HD * HD + (tid / IOS::SEGS) * HD + (tid % IOS::SEGS) * IOS::KP;
+    int64_t soff = ((int64_t)bh * NC + NC - 1) * dvw * dkw + (tid / IOS::SEGS) * dkw + (tid % IOS::SEGS) * IOS::KP;
     int64_t tmoff = ((int64_t)bh * NC + NC - 1) * C * C + (tid / IOT::SEGS) * C + (tid % IOT::SEGS) * IOT::KP;
     int64_t doff = (int64_t)b * Tlen + tlast + lane;  // done/beta of chunk row `lane`
     int tpre = tlast;                                 // first time step of the chunk about to be prefetched
@@ -762,15 +770,20 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         if (part < 4) {
             const T *src = part == 0 ? q : part == 1 ? k : part == 2 ? v : dout;
             typename IO::Regs &dst = part == 0 ? rq : part == 1 ? rk : part == 2 ? rv : rdo;
+            const bool seg_in = part < 2 ? segk : segv;
 #pragma unroll
             for (int p = 0; p < IO::PASSES; ++p)
-                dst.v[p] = (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen
-                               ? *reinterpret_cast<const typename IO::F *>(src + roff[p]) : z;
+                dst.v[p] = seg_in && (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen
+                               ? *reinterpret_cast<const typename IO::F *>(src + (NARROW && part >= 2 ? roffv[p] : roff[p])) : z;
         } else if (part == 4) {
 #pragma unroll
             for (int p = 0; p < IOS::PASSES; ++p)
-                if (IOS::FULL || IOS::row_of(tid, p) < HD)
-                    rS.v[p] = *reinterpret_cast<const typename IOS::F *>(S_chk + soff + p * IOS::RPP * HD);
+                if (IOS::FULL || IOS::row_of(tid, p) < HD) {
+                    if (!NARROW || (IOS::row_of(tid, p) < dvw && (tid % IOS::SEGS) * IOS::KP < dkw))
+                        rS.v[p] = *reinterpret_cast<const typename IOS::F *>(S_chk + soff + p * IOS::RPP * dkw);
+                    else
+                        rS.v[p] = z;
+                }
         } else {
 #pragma unroll
             for (int p = 0; p < IOT::PASSES; ++p)
@@ -780,6 +793,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             for (int p = 0; p < IO::PASSES; ++p) {
                 rbrow[p] = (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen ? load_raw<T>(beta + boff[p]) : 0u;
                 roff[p] -= (int64_t)C * rs;
+                if (NARROW) roffv[p] -= (int64_t)C * rsv;
                 boff[p] -= (int64_t)C * H;
             }
             rdone = 0u;
@@ -788,7 +802,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 rdone = done_raw(done, done_f32, doff);
                 if (w == 0) rbeta = load_raw<T>(beta + doff * H + h);
             }
-            soff -= HD * HD;
+            soff -= dvw * dkw;
             tmoff -= C * C;
             doff -= C;
             tpre -= C;
@@ -813,7 +827,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     auto flush_pending = [&]() {  // call after a barrier that follows the writes to sU
         if (pend_t0 >= 0) {
             auto keep = [&](int r) { return pend_nres == 0 || episode_of(pend_dmask, r) == pend_pass; };
-            tile_rows_to_global<T, C, NTHR>(sU, LDD, dk + base + (int64_t)pend_t0 * rs, rs, pend_t0, Tlen, tid, keep);
+            tile_rows_to_global<T, C, NTHR>(sU, LDD, dk + base + (int64_t)pend_t0 * rs, rs, pend_t0, Tlen, tid, keep, dkw);
         }
         if (pend_db_on) dbeta[pend_dboff] = (T)pend_db;
         pend_t0 = -1;
@@ -956,7 +970,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 store_acc<T, HD, C, NW>(acc, sZb, LDD, w, lane);  // = dV, written to memory from here after the barrier
             }
             sync_lds();  // sDAqk, sZ, sZb visible
-            tile_rows_to_global<T, C, NTHR>(sZb, LDD, dv + base + (int64_t)t0 * rs, rs, t0, Tlen, tid, live);
+            tile_rows_to_global<T, C, NTHR>(sZb, LDD, dv + basev + (int64_t)t0 * rsv, rsv, t0, Tlen, tid, live, dvw);
             // ---- dQ^T[dk][i] = sum_dv S[dv][dk] dO[i][dv] + sum_j K[j][dk] dAqk[i][j] -> global ----
             {
                 f32x4 acc[TMR::TPW];
@@ -995,7 +1009,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 store_acc_f<T, C, C, NW>(acc, sDA, LDC, w, lane, [](int m, int n, float x) { return m < n ? -x : 0.f; });
             }
             sync_lds();  // sDA visible; sQ, sDO, sS, sDS, sDAqk, sZ, sZb dead
-            tile_rows_to_global<T, C, NTHR>(sDU, LDD, dq + base + (int64_t)t0 * rs, rs, t0, Tlen, tid, live);
+            tile_rows_to_global<T, C, NTHR>(sDU, LDD, dq + base + (int64_t)t0 * rs, rs, t0, Tlen, tid, live, dkw);
             // ---- R^T[dk][i] = sum_j K[j][dk] dA[i][j] : dbeta += K_i . R_i ; dK += beta_i R ;
             //      dK^T[dk][j] += sum_i beta_i K[i][dk] dA[i][j] -> global -------------------------------
             {
@@ -1076,7 +1090,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
         for (int j = 0; j < TMS::TPW; ++j) {
             const int dk0 = TMS::mt(w, j) * 16 + 4 * lg, dvv = TMS::nt(w, j) * 16 + li;
-            *reinterpret_cast<f32x4 *>(dS0 + ((int64_t)bh * HD + dvv) * HD + dk0) = dSacc[j];
+            if (in_state(dvv, dk0)) *reinterpret_cast<f32x4 *>(dS0 + ((int64_t)bh * dvw + dvv) * dkw + dk0) = dSacc[j];
         }
     }
 }
@@ -1118,7 +1132,7 @@ int check_bwd(const void *q, const void *k, const void *v, const void *done, con
     if (B <= 0 || T <= 0 || H <= 0 || dk <= 0 || dv <= 0) return MRX_ERR_INVALID_ARG;
     if (dtype != MRX_F32 && dtype != MRX_BF16) return dtype == MRX_C64 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
     if (done_dtype != MRX_DONE_U8 && done_dtype != MRX_DONE_F32) return MRX_ERR_INVALID_ARG;
-    // narrow: linear attention also takes rows narrower than the build's head dim, in whole 16-byte segments
+    // narrow: rows narrower than the build's head dim, in whole 16-byte segments
     const int64_t seg = dtype == MRX_BF16 ? 8 : 4;
     const bool narrow_ok = narrow && dk <= HD && dv <= HD && dk % seg == 0 && dv % seg == 0;
     if ((dk != HD || dv != HD) && !narrow_ok) return MRX_ERR_UNSUPPORTED;
@@ -1243,25 +1257,30 @@ MRX_EXPORT int MRX_API(mrx_gated_linear_attn_bwd)(void *stream, const void *q, c
 namespace {
 inline namespace MRX_HD_NS {
 
-template <typename T, int C, bool PRO> struct DeltaBwdReg {
+template <typename T, int C, bool PRO, bool NARROW> struct DeltaBwdReg {
     static constexpr int NW = 4;
     static constexpr int smem = DeltaBwdSmem<T, C, NW>::total;
-    static inline KernelRegistrar reg{reinterpret_cast<const void *>(delta_bwd_kernel<T, C, NW, PRO>), smem};
+    static inline KernelRegistrar reg{reinterpret_cast<const void *>(delta_bwd_kernel<T, C, NW, PRO, NARROW>), smem};
 };
 
 template <typename T, int C, bool PRO>
 int launch_delta_bwd(hipStream_t st, const void *q, const void *k, const void *v, const void *beta,
                      const void *done, int done_dtype, const void *S_chk, const void *Tm_chk, const void *dout,
                      const void *dS_last, void *dq, void *dk_out, void *dv_out, void *dbeta, void *dS0, int64_t B,
-                     int64_t T_, int64_t H)
+                     int64_t T_, int64_t H, int64_t dka, int64_t dva)
 {
-    using Reg = DeltaBwdReg<T, C, PRO>;
-    (void)&Reg::reg;  // the kernel is on the list mrx_init() walks
     if (const int rc = prepare_device(); rc != MRX_OK) return rc;
-    return launch_kernel(delta_bwd_kernel<T, C, Reg::NW, PRO>, dim3((unsigned)(B * H)), dim3(64 * Reg::NW), Reg::smem, st,
-                         (const T *)q, (const T *)k, (const T *)v, (const T *)beta, done, done_dtype,
-                         (const T *)S_chk, (const T *)Tm_chk, (const T *)dout, (const float *)dS_last, (T *)dq,
-                         (T *)dk_out, (T *)dv_out, (T *)dbeta, (float *)dS0, (int)T_, (int)H);
+    auto go = [&](auto narrow) {
+        using Reg = DeltaBwdReg<T, C, PRO, decltype(narrow)::value>;
+        (void)&Reg::reg;  // the kernel is on the list mrx_init() walks
+        return launch_kernel(delta_bwd_kernel<T, C, Reg::NW, PRO, decltype(narrow)::value>, dim3((unsigned)(B * H)),
+                             dim3(64 * Reg::NW), Reg::smem, st, (const T *)q, (const T *)k, (const T *)v, (const T *)beta,
+                             done, done_dtype, (const T *)S_chk, (const T *)Tm_chk, (const T *)dout,
+                             (const float *)dS_last, (T *)dq, (T *)dk_out, (T *)dv_out, (T *)dbeta, (float *)dS0, (int)T_,
+                             (int)H, (int)dka, (int)dva);
+    };
+    if (dka != HD || dva != HD) return go(std::true_type{});  // narrow heads
+    return go(std::false_type{});
 }
 
 template <bool PRO>
@@ -1271,15 +1290,15 @@ int delta_bwd_entry(void *stream, const void *q, const void *k, const void *v, c
                     int64_t dk, int64_t dv, int dtype, int done_dtype)
 {
     const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
-                             dv, dtype, done_dtype);
+                             dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
     if (!beta || !dbeta || !Tm_chk || !aligned(Tm_chk, 16)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == MRX_BF16)
         return launch_delta_bwd<__bf16, DELTA_BF16_CHUNK, PRO>(st, q, k, v, beta, done, done_dtype, S_chk, Tm_chk, dout,
-                                                               dS_last, dq, dk_out, dv_out, dbeta, dS0, B, T, H);
+                                                               dS_last, dq, dk_out, dv_out, dbeta, dS0, B, T, H, dk, dv);
     return launch_delta_bwd<float, 32, PRO>(st, q, k, v, beta, done, done_dtype, S_chk, Tm_chk, dout, dS_last, dq,
-                                            dk_out, dv_out, dbeta, dS0, B, T, H);
+                                            dk_out, dv_out, dbeta, dS0, B, T, H, dk, dv);
 }
 
 }  // namespace MRX_HD_NS
@@ -1293,7 +1312,7 @@ MRX_EXPORT int MRX_API(mrx_delta_rule_bwd)(void *stream, const void *q, const vo
                                   int done_dtype)
 {
 #if MRX_HD == 64
-    if (dk == 32 && dv == 32) return mrx_delta_rule_bwd_hd32(stream, q, k, v, beta, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out, dbeta, dS0, B, T, H, dk, dv, dtype, done_dtype);
+    if (dk <= 32 && dv <= 32) return mrx_delta_rule_bwd_hd32(stream, q, k, v, beta, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out, dbeta, dS0, B, T, H, dk, dv, dtype, done_dtype);
 #endif
     return delta_bwd_entry<false>(stream, q, k, v, beta, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out,
                                   dbeta, dS0, B, T, H, dk, dv, dtype, done_dtype);
@@ -1307,7 +1326,7 @@ MRX_EXPORT int MRX_API(mrx_deltanet_bwd)(void *stream, const void *q, const void
                                 int done_dtype)
 {
 #if MRX_HD == 64
-    if (dk == 32 && dv == 32) return mrx_deltanet_bwd_hd32(stream, q, k, v, beta_raw, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out, dbeta_raw, dS0, B, T, H, dk, dv, dtype, done_dtype);
+    if (dk <= 32 && dv <= 32) return mrx_deltanet_bwd_hd32(stream, q, k, v, beta_raw, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out, dbeta_raw, dS0, B, T, H, dk, dv, dtype, done_dtype);
 #endif
     return delta_bwd_entry<true>(stream, q, k, v, beta_raw, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out,
                                  dbeta_raw, dS0, B, T, H, dk, dv, dtype, done_dtype);

@@ -74,7 +74,7 @@ struct NormArgs {
 // PAR (plain linear attention): one workgroup per chunk (grid.y = chunk) instead of one per sequence.
 // S_chk then is an input: slot c holds, in fp32, the state entering chunk c (la_states.h); the
 // workgroup forms the chunk's outputs from it and neither updates nor writes any state.
-// NARROW (linear attention, all variants): narrow heads.  Keys and queries are dka wide in memory, values
+// NARROW (every variant): narrow heads.  Keys and queries are dka wide in memory, values
 // and outputs dva (both at most the head dim of the build, whole 16-byte segments), and so are the
 // states (B,H,dva,dka) and z (B,H,dka).  Tiles in LDS and registers keep the build's width: what lies
 // beyond the rows' width is loaded as zero (after the feature map, phi(0) = 1 must not count) and never
@@ -88,7 +88,6 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                  const float *__restrict__ S0, T *__restrict__ o, float *__restrict__ S_last,
                  void *__restrict__ S_chk, T *__restrict__ Tm_chk, int Tlen, int H, NormArgs na, int dka, int dva)
 {
-    static_assert(!NARROW || !DELTA, "narrow heads: linear attention only");
     static_assert(!(DELTA && GATED), "the gated variant is linear attention with a decay");
     static_assert(!NORM || (!DELTA && !GATED), "the normalised read-out belongs to plain linear attention");
     static_assert(!PRO || DELTA, "the prologue belongs to the delta rule");
@@ -579,8 +578,8 @@ template <typename T, int C, bool DELTA, bool FMAP, bool GATED, bool NORM, bool 
         reinterpret_cast<const void *>(chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR, NARROW>), smem};
 };
 
-// dka, dva: widths of the q/k and v/o rows in memory; less than the build's head dim (narrow heads,
-// linear attention only) selects the kernel instance that pads on the fly.
+// dka, dva: widths of the q/k and v/o rows in memory; less than the build's head dim (narrow heads)
+// selects the kernel instance that pads on the fly.
 template <typename T, int C, bool DELTA, bool FMAP, bool GATED = false, bool NORM = false, bool PRO = false,
           bool TMIN = false, bool PAR = false>
 int launch(hipStream_t st, const void *q, const void *k, const void *v, const void *beta,
@@ -601,14 +600,12 @@ int launch(hipStream_t st, const void *q, const void *k, const void *v, const vo
                              (const float *)S0, (T *)o, (float *)S_last, S_chk, (T *)Tm_chk, (int)Tlen, (int)H, na,
                              (int)dka, (int)dva);
     };
-    if constexpr (!DELTA) {
-        if (dka != HD || dva != HD) return go(std::true_type{});
-    }
+    if (dka != HD || dva != HD) return go(std::true_type{});
     return go(std::false_type{});
 }
 
-// narrow: the entry point also serves heads narrower than the build's (linear attention: rows of whole
-// 16-byte segments, padded inside the kernels)
+// narrow: the entry point also serves heads narrower than the build's (rows of whole 16-byte segments,
+// padded inside the kernels)
 int check_common(const void *q, const void *k, const void *v, const void *done, const void *o,
                  const void *S0, const void *S_last, const void *S_chk, int64_t B, int64_t T,
                  int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype, bool narrow = false)
@@ -640,7 +637,7 @@ int check_common(const void *q, const void *k, const void *v, const void *done, 
 template <bool PRO>
 int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void *v, const void *beta, const void *done,
                        int done_dtype, const void *S0, void *o, void *S_last, void *S_chk, void *Tm_chk, int64_t B,
-                       int64_t T, int64_t H, int dtype, int factor_path)
+                       int64_t T, int64_t H, int dtype, int factor_path, int64_t dk = HD, int64_t dv = HD)
 {
     // delta_tm_kernel is written for 32-row chunks: a build with 64-row bf16 chunks (the measurement
     // variant, MRX_DELTA_BF16_CHUNK=64) always inverts inside the sequential kernel
@@ -654,19 +651,21 @@ int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void 
                           (factor_path == MRX_FACTORS_PARALLEL || dtype == MRX_F32 || B * H <= 2 * (int64_t)cus);
     if (!TM_KERNEL && factor_path == MRX_FACTORS_PARALLEL) return MRX_ERR_UNSUPPORTED;
     if constexpr (TM_KERNEL) if (parallel) {
-        const int rc = launch_delta_tm(st, k, beta, done, done_dtype, Tm_chk, B, T, H, dtype, PRO);
+        const int rc = launch_delta_tm(st, k, beta, done, done_dtype, Tm_chk, B, T, H, dtype, PRO, dk);
         if (rc != MRX_OK) return rc;
         if (dtype == MRX_BF16)
             return launch<__bf16, 32, true, false, false, false, PRO, true>(st, q, k, v, beta, done, done_dtype, S0, o,
-                                                                           S_last, S_chk, Tm_chk, B, T, H);
+                                                                           S_last, S_chk, Tm_chk, B, T, H, nullptr,
+                                                                           NormArgs{}, dk, dv);
         return launch<float, 32, true, false, false, false, PRO, true>(st, q, k, v, beta, done, done_dtype, S0, o, S_last,
-                                                                       S_chk, Tm_chk, B, T, H);
+                                                                       S_chk, Tm_chk, B, T, H, nullptr, NormArgs{}, dk, dv);
     }
     if (dtype == MRX_BF16)
         return launch<__bf16, DELTA_BF16_CHUNK, true, false, false, false, PRO, false>(st, q, k, v, beta, done, done_dtype, S0, o,
-                                                                                      S_last, S_chk, Tm_chk, B, T, H);
+                                                                                      S_last, S_chk, Tm_chk, B, T, H, nullptr,
+                                                                                      NormArgs{}, dk, dv);
     return launch<float, 32, true, false, false, false, PRO, false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last,
-                                                                    S_chk, Tm_chk, B, T, H);
+                                                                    S_chk, Tm_chk, B, T, H, nullptr, NormArgs{}, dk, dv);
 }
 
 bool factor_path_ok(int f) { return f == MRX_FACTORS_AUTO || f == MRX_FACTORS_PARALLEL || f == MRX_FACTORS_INLINE; }
@@ -771,14 +770,14 @@ MRX_EXPORT int MRX_API(mrx_delta_rule_fwd)(void *stream, const void *q, const vo
                                   int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype, int factor_path)
 {
 #if MRX_HD == 64
-    if (dk == 32 && dv == 32) return mrx_delta_rule_fwd_hd32(stream, q, k, v, beta, done, S0, o, S_last, S_chk, Tm_chk, B, T, H, dk, dv, dtype, done_dtype, factor_path);
+    if (dk <= 32 && dv <= 32) return mrx_delta_rule_fwd_hd32(stream, q, k, v, beta, done, S0, o, S_last, S_chk, Tm_chk, B, T, H, dk, dv, dtype, done_dtype, factor_path);
 #endif
-    const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
+    const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
     if (!beta || !aligned(Tm_chk, 16) || !factor_path_ok(factor_path)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     return delta_fwd_dispatch<false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H, dtype,
-                                     factor_path);
+                                     factor_path, dk, dv);
 }
 
 #if MRX_HD == 64
@@ -854,12 +853,12 @@ MRX_EXPORT int MRX_API(mrx_deltanet_fwd)(void *stream, const void *q, const void
                                 int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype, int factor_path)
 {
 #if MRX_HD == 64
-    if (dk == 32 && dv == 32) return mrx_deltanet_fwd_hd32(stream, q, k, v, beta_raw, done, S0, o, S_last, S_chk, Tm_chk, B, T, H, dk, dv, dtype, done_dtype, factor_path);
+    if (dk <= 32 && dv <= 32) return mrx_deltanet_fwd_hd32(stream, q, k, v, beta_raw, done, S0, o, S_last, S_chk, Tm_chk, B, T, H, dk, dv, dtype, done_dtype, factor_path);
 #endif
-    const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype);
+    const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
     if (!beta_raw || !aligned(Tm_chk, 16) || !factor_path_ok(factor_path)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     return delta_fwd_dispatch<true>(st, q, k, v, beta_raw, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H, dtype,
-                                    factor_path);
+                                    factor_path, dk, dv);
 }

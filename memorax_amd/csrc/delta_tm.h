@@ -29,11 +29,12 @@ inline namespace MRX_HD_NS {
 // Longest sequence the launch covers: four chunks per workgroup, 65535 workgroups along the grid's y.
 constexpr int64_t DELTA_TM_MAX_T = 4ll * 65535 * 32;
 
-// Fills Tm_chk[B][H][ceil(T / 32)][32][32] (dtype: MRX_F32 or MRX_BF16) from the keys [B][T][H][64],
+// Fills Tm_chk[B][H][ceil(T / 32)][32][32] (dtype: MRX_F32 or MRX_BF16) from the keys [B][T][H][dk],
 // the gates [B][T][H] and the reset flags [B][T].  prologue: keys are L2-normalised and gates go
-// through a sigmoid first.  Returns an MRX_* status (MRX_ERR_INVALID_ARG beyond DELTA_TM_MAX_T steps).
+// through a sigmoid first.  dk: the build's head dim, or less in whole 16-byte segments (narrow heads).
+// Returns an MRX_* status (MRX_ERR_INVALID_ARG beyond DELTA_TM_MAX_T steps).
 int launch_delta_tm(hipStream_t st, const void *k, const void *beta, const void *done, int done_f32, void *Tm_chk,
-                    int64_t B, int64_t Tlen, int64_t H, int dtype, bool prologue);
+                    int64_t B, int64_t Tlen, int64_t H, int dtype, bool prologue, int64_t dk);
 
 }  // namespace MRX_HD_NS
 }  // namespace mrx

@@ -11,10 +11,12 @@
 namespace mrx {
 inline namespace MRX_HD_NS {
 
-template <typename T, bool PRO>
+// NARROW: the key rows are dka wide in memory, less than the build's head dim; the fragments' further
+// columns are zeros.
+template <typename T, bool PRO, bool NARROW = false>
 __global__ void __launch_bounds__(256)
 delta_tm_kernel(const T *__restrict__ k, const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
-                T *__restrict__ Tm_chk, int Tlen, int H, int NC)
+                T *__restrict__ Tm_chk, int Tlen, int H, int NC, int dka)
 {
     constexpr int C = 32;
     using Frag = typename TT<T>::frag;
@@ -36,9 +38,10 @@ delta_tm_kernel(const T *__restrict__ k, const T *__restrict__ beta, const void 
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb) {
         const int t = t0 + 16 * rb + li;
-        const T *row = k + (((int64_t)b * Tlen + t) * H + h) * HD + KP * lg;
+        const T *row = k + (((int64_t)b * Tlen + t) * H + h) * (NARROW ? dka : HD) + KP * lg;
 #pragma unroll
-        for (int kb = 0; kb < NKB; ++kb) f[rb][kb] = t < Tlen ? *reinterpret_cast<const Frag *>(row + kb * KB) : zf;
+        for (int kb = 0; kb < NKB; ++kb)
+            f[rb][kb] = (t < Tlen && (!NARROW || kb * KB + KP * lg < dka)) ? *reinterpret_cast<const Frag *>(row + kb * KB) : zf;
     }
     // gates and reset flags of the 32 rows, one per lane
     float bl = 0.f;
@@ -162,23 +165,27 @@ delta_tm_kernel(const T *__restrict__ k, const T *__restrict__ beta, const void 
 namespace {
 template <typename T, bool PRO>
 int launch_tm(hipStream_t st, const void *k, const void *beta, const void *done, int done_f32, void *Tm_chk, int64_t B,
-              int64_t Tlen, int64_t H)
+              int64_t Tlen, int64_t H, int64_t dk)
 {
     const int64_t NC = (Tlen + 31) / 32, groups = (NC + 3) / 4;
     if (B * H > 0x7fffffffLL || groups > 65535) return MRX_ERR_INVALID_ARG;
-    return launch_kernel((delta_tm_kernel<T, PRO>), dim3((unsigned)(B * H), (unsigned)groups), dim3(256), 0, st,
-                         (const T *)k, (const T *)beta, done, done_f32, (T *)Tm_chk, (int)Tlen, (int)H, (int)NC);
+    const dim3 grid((unsigned)(B * H), (unsigned)groups);
+    if (dk != HD)
+        return launch_kernel((delta_tm_kernel<T, PRO, true>), grid, dim3(256), 0, st, (const T *)k, (const T *)beta, done,
+                             done_f32, (T *)Tm_chk, (int)Tlen, (int)H, (int)NC, (int)dk);
+    return launch_kernel((delta_tm_kernel<T, PRO, false>), grid, dim3(256), 0, st, (const T *)k, (const T *)beta, done,
+                         done_f32, (T *)Tm_chk, (int)Tlen, (int)H, (int)NC, (int)dk);
 }
 }  // namespace
 
 int launch_delta_tm(hipStream_t st, const void *k, const void *beta, const void *done, int done_f32, void *Tm_chk,
-                    int64_t B, int64_t Tlen, int64_t H, int dtype, bool prologue)
+                    int64_t B, int64_t Tlen, int64_t H, int dtype, bool prologue, int64_t dk)
 {
     if (dtype == MRX_BF16)
-        return prologue ? launch_tm<__bf16, true>(st, k, beta, done, done_f32, Tm_chk, B, Tlen, H)
-                        : launch_tm<__bf16, false>(st, k, beta, done, done_f32, Tm_chk, B, Tlen, H);
-    return prologue ? launch_tm<float, true>(st, k, beta, done, done_f32, Tm_chk, B, Tlen, H)
-                    : launch_tm<float, false>(st, k, beta, done, done_f32, Tm_chk, B, Tlen, H);
+        return prologue ? launch_tm<__bf16, true>(st, k, beta, done, done_f32, Tm_chk, B, Tlen, H, dk)
+                        : launch_tm<__bf16, false>(st, k, beta, done, done_f32, Tm_chk, B, Tlen, H, dk);
+    return prologue ? launch_tm<float, true>(st, k, beta, done, done_f32, Tm_chk, B, Tlen, H, dk)
+                    : launch_tm<float, false>(st, k, beta, done, done_f32, Tm_chk, B, Tlen, H, dk);
 }
 
 }  // namespace MRX_HD_NS

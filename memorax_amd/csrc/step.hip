@@ -52,7 +52,7 @@ __device__ __forceinline__ float dot4(const f32x4 &a, const f32x4 &b)
     return a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
 }
 
-// NARROW (linear attention): narrow heads -- q, k, z are dka wide, v, o dva, the state
+// NARROW: narrow heads -- q, k, z are dka wide, v, o dva, the state
 // [dva][dka]; lanes and rows beyond take no part.
 template <typename T, bool DELTA, bool FMAP, bool NARROW = false>
 __global__ void __launch_bounds__(256)
@@ -61,7 +61,6 @@ step_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restric
             const float *S_in, const float *z_in, T *__restrict__ o, float *S_out, float *z_out, int H,
             float eps, int dka, int dva)  // S_in/S_out and z_in/z_out may alias (update in place)
 {
-    static_assert(!NARROW || !DELTA, "narrow heads: linear attention only");
     const int tid = threadIdx.x, c4 = tid % LPR, r0 = tid / LPR;
     const int64_t bh = blockIdx.x;
     const int b = (int)(bh / H);
@@ -123,7 +122,7 @@ int check_step(const void *q, const void *k, const void *v, const void *done, co
     if (B <= 0 || H <= 0 || dk <= 0 || dv <= 0) return MRX_ERR_INVALID_ARG;
     if (dtype != MRX_F32 && dtype != MRX_BF16) return dtype == MRX_C64 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
     if (done_dtype != MRX_DONE_U8 && done_dtype != MRX_DONE_F32) return MRX_ERR_INVALID_ARG;
-    // narrow: linear attention also takes rows narrower than the build's head dim, in whole 16-byte segments
+    // narrow: rows narrower than the build's head dim, in whole 16-byte segments
     const int64_t seg = dtype == MRX_BF16 ? 8 : 4;
     const bool narrow_ok = narrow && dk <= HD && dv <= HD && dk % seg == 0 && dv % seg == 0;
     if ((dk != HD || dv != HD) && !narrow_ok) return MRX_ERR_UNSUPPORTED;
@@ -145,9 +144,7 @@ int launch_step(hipStream_t st, const void *q, const void *k, const void *v, con
                              (const T *)q, (const T *)k, (const T *)v, (const T *)beta, glog, done, done_f32, S_in, z_in,
                              (T *)o, S_out, z_out, (int)H, eps, (int)dka, (int)dva);
     };
-    if constexpr (!DELTA) {
-        if (dka != HD || dva != HD) return go(std::true_type{});  // narrow heads
-    }
+    if (dka != HD || dva != HD) return go(std::true_type{});  // narrow heads
     return go(std::false_type{});
 }
 
@@ -201,14 +198,14 @@ MRX_EXPORT int MRX_API(mrx_delta_rule_step)(void *stream, const void *q, const v
                                    int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype)
 {
 #if MRX_HD == 64
-    if (dk == 32 && dv == 32) return mrx_delta_rule_step_hd32(stream, q, k, v, beta, done, S_in, o, S_out, B, H, dk, dv, dtype, done_dtype);
+    if (dk <= 32 && dv <= 32) return mrx_delta_rule_step_hd32(stream, q, k, v, beta, done, S_in, o, S_out, B, H, dk, dv, dtype, done_dtype);
 #endif
-    const int rc = check_step(q, k, v, done, S_in, o, S_out, B, H, dk, dv, dtype, done_dtype);
+    const int rc = check_step(q, k, v, done, S_in, o, S_out, B, H, dk, dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
     if (!beta) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     const int df = done_dtype == MRX_DONE_F32;
     if (dtype == MRX_BF16)
-        return launch_step<__bf16, true, false>(st, q, k, v, beta, done, df, S_in, nullptr, o, S_out, nullptr, B, H, 0.f);
-    return launch_step<float, true, false>(st, q, k, v, beta, done, df, S_in, nullptr, o, S_out, nullptr, B, H, 0.f);
+        return launch_step<__bf16, true, false>(st, q, k, v, beta, done, df, S_in, nullptr, o, S_out, nullptr, B, H, 0.f, dk, dv);
+    return launch_step<float, true, false>(st, q, k, v, beta, done, df, S_in, nullptr, o, S_out, nullptr, B, H, 0.f, dk, dv);
 }

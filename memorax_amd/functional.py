@@ -390,7 +390,7 @@ def delta_rule(q, k, v, beta, done, S0=None):
     o_t = S_t q_t, in chunked WY form.  Returns (o, S_last)."""
     if _no_steps(q):
         return _attention_without_steps(q, v, S0)
-    hd = _Heads(q, v)
+    hd = _Heads(q, v, narrow=True)
     o, S_last = _DeltaRule.apply(hd.qk(q), hd.qk(k), hd.v(v), hd.per_head(beta), done, hd.state_in(S0))
     return hd.out(o), hd.state_out(S_last)
 
@@ -402,7 +402,7 @@ def deltanet(q, k, v, beta_raw, done, S0=None):
     the gates never reach memory; gradients come back w.r.t. the raw arrays).  Returns (o, S_last)."""
     if _no_steps(q):
         return _attention_without_steps(q, v, S0)
-    hd = _Heads(q, v)   # zero-padding the keys leaves their norm unchanged
+    hd = _Heads(q, v, narrow=True)   # where keys are padded: zeros leave their norm unchanged
     o, S_last = _DeltaRule.apply(hd.qk(q), hd.qk(k), hd.v(v), hd.per_head(beta_raw), done, hd.state_in(S0), True)
     return hd.out(o), hd.state_out(S_last)
 

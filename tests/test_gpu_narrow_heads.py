@@ -159,6 +159,89 @@ def test_single_steps_roll_out_to_the_sequence_results(dims, dtype):
         assert relerr(torch.stack(outs, 1), ro) <= tol and relerr(S, rS) <= tol
 
 
+def _delta_inputs(shape, dk, dv, p, dtype, seed):
+    B, T, H = shape
+    rng = np.random.default_rng(seed)
+    x = {"q": rng.standard_normal((B, T, H, dk)).astype(np.float32), "v": rng.standard_normal((B, T, H, dv)).astype(np.float32),
+         "do": rng.standard_normal((B, T, H, dv)).astype(np.float32)}
+    kk = rng.standard_normal((B, T, H, dk)).astype(np.float32)
+    x["k"] = kk / np.linalg.norm(kk, axis=-1, keepdims=True)
+    x["beta"] = (1 / (1 + np.exp(-rng.standard_normal((B, T, H))))).astype(np.float32)
+    x["kr"] = (x["k"] * (0.5 + rng.random((B, T, H, 1)))).astype(np.float32)   # raw keys and gate pre-activations
+    x["br"] = (rng.standard_normal((B, T, H)) * 1.5).astype(np.float32)
+    x["done"] = rng.random((B, T)) < p
+    x["S0"] = (rng.standard_normal((B, H, dv, dk)) * 0.1).astype(np.float32)
+    x["dSl"] = (rng.standard_normal((B, H, dv, dk)) * 0.1).astype(np.float32)
+    if dtype == "bf16":
+        for n in ("q", "k", "v", "do", "beta", "kr", "br"):
+            x[n] = bf16_round(x[n])
+    return x
+
+
+@pytest.mark.parametrize("dims,dtype", _cases())
+@pytest.mark.parametrize("shape", [(3, 1, 2), (2, 65, 1), (2, 200, 3), (1, 1100, 2)])
+@pytest.mark.parametrize("p", [0.0, 0.06])
+@pytest.mark.parametrize("path", ["parallel", "inline"])
+def test_delta_rule_and_deltanet(dims, dtype, shape, p, path):
+    from memorax_amd import kernels as K
+    dk, dv = dims
+    x = _delta_inputs(shape, dk, dv, p, dtype, seed=sum(shape) + dk + 9)
+    print(f"case narrow delta dk={dk} dv={dv} shape={shape} p={p} dtype={dtype} factors={path}", flush=True)
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    tq, tk, tv, tb, tdo = (dev(x[n], td) for n in ("q", "k", "v", "beta", "do"))
+    dn = dev(x["done"])
+    o, Sl, chk = K.delta_rule_fwd(tq, tk, tv, tb, dn, dev(x["S0"]), factor_path=path)
+    assert o.shape == (shape[0], shape[1], shape[2], dv) and Sl.shape == (shape[0], shape[2], dv, dk)
+    ref = G.delta_rule_grads(x["q"], x["k"], x["v"], x["beta"], x["done"], x["S0"], x["do"], x["dSl"])
+    _check((o, Sl), ref, ("o", "S_last"), tol)
+    got = K.delta_rule_bwd(tq, tk, tv, tb, dn, chk, tdo, dev(x["dSl"]))
+    _check(got, ref, ("dq", "dk", "dv", "dbeta", "dS0"), tol)
+    # the cell's prologue inside the kernels: raw keys and gate pre-activations
+    tk2, tb2 = dev(x["kr"], td), dev(x["br"], td)
+    o, Sl, chk = K.delta_rule_fwd(tq, tk2, tv, tb2, dn, dev(x["S0"]), prologue=True, factor_path=path)
+    ref = G.deltanet_grads(x["q"], x["kr"], x["v"], x["br"], x["done"], x["S0"], x["do"], x["dSl"])
+    _check((o, Sl), ref, ("o", "S_last"), tol)
+    got = K.delta_rule_bwd(tq, tk2, tv, tb2, dn, chk, tdo, dev(x["dSl"]), prologue=True)
+    _check(got, ref, ("dq", "dk", "dv", "dbeta", "dS0"), tol)
+
+
+@pytest.mark.parametrize("dims", [(16, 16), (8, 24), (40, 64), (48, 24)])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_narrow_delta_rule_equals_zero_padded_heads_bit_for_bit(dims, dtype):
+    """Zero key features change neither k k^T nor the key norm, zero value features add zero rows to the state:
+    a narrow call and the same call on zero-padded arrays at the build's full width give identical bits, with
+    either factor path, with and without the prologue, forward, backward and single steps."""
+    from memorax_amd import kernels as K
+    dk, dv = dims
+    W = 32 if max(dk, dv) <= 32 else 64
+    shape = (2, 200, 3)
+    x = _delta_inputs(shape, dk, dv, 0.05, dtype, seed=78)
+    td = torch.bfloat16 if dtype == "bf16" else torch.float32
+    print(f"case narrow delta vs padded dk={dk} dv={dv} dtype={dtype}", flush=True)
+    pad = lambda t, n: torch.nn.functional.pad(t, (0, n)).contiguous()
+    pad2 = lambda t: torch.nn.functional.pad(t, (0, W - dk, 0, W - dv)).contiguous()
+    tq, tv, tdo = dev(x["q"], td), dev(x["v"], td), dev(x["do"], td)
+    dn, S0, dSl = dev(x["done"]), dev(x["S0"]), dev(x["dSl"])
+    cut = {"k": lambda t: t[..., :dk], "v": lambda t: t[..., :dv], "s": lambda t: t[..., :dv, :dk], "": lambda t: t}
+    for pro, kn, bn in ((False, "k", "beta"), (True, "kr", "br")):
+        tk, tb = dev(x[kn], td), dev(x[bn], td)
+        for path in ("parallel", "inline"):
+            def run(q, k, v, do, S0, dSl):
+                o, Sl, chk = K.delta_rule_fwd(q, k, v, tb, dn, S0, prologue=pro, factor_path=path)
+                return (o, Sl) + tuple(K.delta_rule_bwd(q, k, v, tb, dn, chk, do, dSl, prologue=pro))
+            a = run(tq, tk, tv, tdo, S0, dSl)
+            b = run(pad(tq, W - dk), pad(tk, W - dk), pad(tv, W - dv), pad(tdo, W - dv), pad2(S0), pad2(dSl))
+            for i, (ta, tb_, kd) in enumerate(zip(a, b, ("v", "s", "k", "k", "v", "", "s"))):
+                assert torch.equal(ta, cut[kd](tb_)), (pro, path, i)
+    tk, tb = dev(x["k"], td), dev(x["beta"], td)
+    o1, S1 = K.delta_rule_step(tq[:, 0].contiguous(), tk[:, 0].contiguous(), tv[:, 0].contiguous(), tb[:, 0].contiguous(),
+                               dn[:, 0].contiguous(), S0)
+    o2, S2 = K.delta_rule_step(pad(tq[:, 0], W - dk), pad(tk[:, 0], W - dk), pad(tv[:, 0], W - dv), tb[:, 0].contiguous(),
+                               dn[:, 0].contiguous(), pad2(S0))
+    assert torch.equal(o1, o2[..., :dv]) and torch.equal(S1, S2[..., :dv, :dk])
+
+
 def test_what_is_not_a_narrow_head_is_refused():
     from memorax_amd import _lib
     lib = _lib.load()
@@ -177,15 +260,14 @@ def test_what_is_not_a_narrow_head_is_refused():
     assert la(6, 16, 0) == -2 and la(16, 10, 0) == -2
     assert la(16, 64, 0) == 0 and la(64, 16, 1) == 0 and la(48, 48, 0) == 0 and la(32, 40, 1) == 0  # the 64-wide kernels
     assert la(72, 64, 0) == -2 and la(64, 128, 0) == -2 and la(36, 36, 1) == -2
-    # the delta rule keeps to the two head dims of the builds
+    # the delta rule: the same widths; the variant with the static scratch array stays at 64
     q = torch.zeros((1, 4, 1, 16), device="cuda")
     dn = torch.zeros((1, 4), dtype=torch.uint8, device="cuda")
     beta = torch.zeros((1, 4, 1), device="cuda")
     o = torch.empty_like(q)
-    assert lib.mrx_delta_rule_fwd(None, P(q), P(q), P(q), P(beta), P(dn), None, P(o), None, None, None, 1, 4, 1, 16, 16, 0, 0, 0) == -2
-    S = torch.zeros((1, 1, 16, 16), device="cuda")
-    assert lib.mrx_delta_rule_step(None, P(q[:, 0]), P(q[:, 0]), P(q[:, 0]), P(beta[:, 0]), P(dn[:, 0]), None, P(o[:, 0]), P(S),
-                                   1, 1, 16, 16, 0, 0) == -2
+    assert lib.mrx_delta_rule_fwd(None, P(q), P(q), P(q), P(beta), P(dn), None, P(o), None, None, None, 1, 4, 1, 16, 16, 0, 0, 0) == 0
+    assert lib.mrx_delta_rule_fwd(None, P(q), P(q), P(q), P(beta), P(dn), None, P(o), None, None, None, 1, 4, 1, 16, 6, 0, 0, 0) == -2
+    assert lib.mrx_delta_rule_fwd_noalloc(None, P(q), P(q), P(q), P(beta), P(dn), None, P(o), None, 1, 4, 1, 16, 16, 0, 0) == -2
     torch.cuda.synchronize()
 
 

@@ -1,5 +1,5 @@
-"""Seeded random sweep of the chunked kernels against the oracle: shapes, head dims (64, 32 and, for the
-linear-attention family, narrow heads with d_k != d_v), dtypes, reset rates, feature maps, optional initial
+"""Seeded random sweep of the chunked kernels against the oracle: shapes, head dims (64, 32 and narrow heads
+with d_k != d_v), dtypes, reset rates, feature maps, optional initial
 state and state gradient, every factor path of the delta rule -- combinations the hand-written case lists
 do not enumerate.  Every case is drawn from a fixed seed, so a failure names its case."""
 import numpy as np
@@ -18,17 +18,14 @@ CASES_PER_SEED = 16
 def _case(rng):
     op = str(rng.choice(["la", "lapar", "gated", "norm", "delta", "deltanet"]))
     dtype = str(rng.choice(["f32", "bf16"]))
-    if op in ("delta", "deltanet"):
-        dk = dv = int(rng.choice([32, 64]))
-    else:
-        seg = 8 if dtype == "bf16" else 4
-        kind = int(rng.integers(0, 4))
-        if kind == 0:
-            dk = dv = 64
-        elif kind == 1:
-            dk = dv = 32
-        else:  # narrow heads: whole 16-byte segments, widths independent of one another, up to 32 or up to 64
-            dk, dv = (int(rng.integers(1, (32 if kind == 2 else 64) // seg + 1)) * seg for _ in range(2))
+    seg = 8 if dtype == "bf16" else 4
+    kind = int(rng.integers(0, 4))
+    if kind == 0:
+        dk = dv = 64
+    elif kind == 1:
+        dk = dv = 32
+    else:  # narrow heads: whole 16-byte segments, widths independent of one another, up to 32 or up to 64
+        dk, dv = (int(rng.integers(1, (32 if kind == 2 else 64) // seg + 1)) * seg for _ in range(2))
     return dict(op=op, dtype=dtype, dk=dk, dv=dv, B=int(rng.integers(1, 4)), H=int(rng.integers(1, 4)),
                 T=int(rng.choice(LENGTHS)), p=float(rng.choice([0.0, 0.01, 0.1, 0.5])), fm=int(rng.integers(0, 2)),
                 S0=bool(rng.integers(0, 2)), dSl=bool(rng.integers(0, 2)),

@@ -184,7 +184,7 @@ def test_step_rejects_bad_arguments():
     p = t.data_ptr()
     args = lambda dk: (None, p, p, p, p, p, p, p, p, 1, 1, dk, 64, 0, 0)
     assert lib.mrx_delta_rule_step(*args(64)) == 0
-    assert lib.mrx_delta_rule_step(*args(32)) == -2          # unsupported head dim
+    assert lib.mrx_delta_rule_step(*args(72)) == -2          # unsupported head dim
     assert lib.mrx_delta_rule_step(None, p, p, p, None, p, p, p, p, 1, 1, 64, 64, 0, 0) == -1  # beta missing
     assert lib.mrx_linear_attn_step(None, p, p, p, p, p, None, p, p, None, 1, 1, 64, 64, 0, 0, 7, 1e-6) == -1
     assert lib.mrx_gated_linear_attn_step(None, p, p, p, p, p, p, p, p, 1, 1, 64, 64, 0, 0, 0) == 0

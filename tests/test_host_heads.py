@@ -23,7 +23,7 @@ def test_padding_and_value_blocks_reproduce_the_native_recurrence(dk, dv, op):
     g, beta = -_rand(B, T, H, seed=6).abs() * 0.3, torch.sigmoid(_rand(B, T, H, seed=7))
     done = torch.from_numpy(np.random.default_rng(8).random((B, T)) < 0.2)
     fm = "none" if op == "delta" else "elu1"
-    narrow = op != "delta"  # the linear-attention kernels of the 32-wide build take narrower heads as they are
+    narrow = True  # the kernels take narrower heads as they are
     split_k = op in ("linear", "gated")  # outputs linear in the state: key features beyond 64 run as further blocks
     if dk > 64 and not split_k:
         with pytest.raises(ValueError):
