@@ -178,8 +178,13 @@ def _delta_inputs(shape, dk, dv, p, dtype, seed):
     return x
 
 
-@pytest.mark.parametrize("dims,dtype", _cases())
-@pytest.mark.parametrize("shape", [(3, 1, 2), (2, 65, 1), (2, 200, 3), (1, 1100, 2)])
+def _delta_cases():
+    # every width on the short shapes; the long sequence (35 chunks) on one width per build
+    short = [(d, t, s) for d, t in _cases() for s in [(3, 1, 2), (2, 65, 1), (2, 200, 3)]]
+    return short + [(d, t, (1, 1100, 2)) for d in [(16, 16), (40, 64)] for t in ("f32", "bf16")]
+
+
+@pytest.mark.parametrize("dims,dtype,shape", _delta_cases())
 @pytest.mark.parametrize("p", [0.0, 0.06])
 @pytest.mark.parametrize("path", ["parallel", "inline"])
 def test_delta_rule_and_deltanet(dims, dtype, shape, p, path):
