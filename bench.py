@@ -514,10 +514,14 @@ def bench_torso_kernels(torch, K):
             K.mingru_scan_bwd(z, hx, h, done, None, g)
     ms_k = _time_ms(torch, lambda: kernels_only(True), iters=10, warm=3)
     ms_p = _time_ms(torch, lambda: kernels_only(False), iters=10, warm=3)
+    # the same with the recurrence's arrays in bfloat16 (what a bf16 torso hands over; float32 arithmetic and
+    # carries inside the kernels): half the bytes of the scans
+    z, hx, g = (t.to(bf) for t in (z, hx, g))
+    ms_h = _time_ms(torch, lambda: kernels_only(True), iters=10, warm=3)
     by = 4 * ((BYTES_FWD + BYTES_BWD) * B * T * H + 36 * B * T * Fe)   # + MinGRU scan: 12 B fwd, 24 B bwd per element
     return {"sequence_kernels_ms": ms_k, "sequence_kernels_tokens/s": B * T / ms_k * 1e3,
             "sequence_kernels_GB/s": by / ms_k / 1e6, "sequence_kernels_frac_hbm": by / ms_k / 1e6 / HBM_PEAK_GBS,
-            "sequence_kernels_ms_plain_delta_rule": ms_p}
+            "sequence_kernels_ms_plain_delta_rule": ms_p, "sequence_kernels_ms_bf16_recurrence_arrays": ms_h}
 
 
 def bench_torso_full(torch, K):

@@ -104,7 +104,8 @@ int64_t mrx_delta_chunk_size(int dtype);
  *     P_t = done_t ? a_t : a_t * P_{t-1}          (cumulative-decay leaf)
  * a: (B,T,D), or (D,) when a_time_invariant != 0 (LRU/S5 broadcast lambda,
  * lru.py:86, never materialised here).  b,h: (B,T,D).  h0,P0 (nullable: 0 and 1),
- * h_last,P_last (nullable: not written): (B,D).  dtype: MRX_F32 or MRX_C64. */
+ * h_last,P_last (nullable: not written): (B,D).  dtype: MRX_F32, MRX_C64, or MRX_BF16: the (B,T,D) arrays
+ * (and a) in bfloat16, the arithmetic and the (B,D) carries in float32. */
 int mrx_linear_scan_fwd(void *stream, const void *a, const void *b,
                         const void *done, const void *h0, const void *P0,
                         void *h, void *h_last, void *P_last, int64_t B,
@@ -120,7 +121,8 @@ int mrx_linear_scan_fwd(void *stream, const void *a, const void *b,
  * da is per step (B,T,D), also when a is time-invariant (a_time_invariant = 1: the caller reduces);
  * with a_time_invariant = MRX_A_TIME_INVARIANT_SUM_DA the kernel sums the per-step terms over the
  * sequence itself and da is (B,D) -- the gradient of the broadcast lambda of lru.py:86 / s5.py is then
- * its sum over B, and the (B,T,D) array is neither written nor read back. */
+ * its sum over B, and the (B,T,D) array is neither written nor read back (MRX_BF16: this summed da is
+ * float32, like the carries). */
 #define MRX_A_TIME_INVARIANT_SUM_DA 2
 int mrx_linear_scan_bwd(void *stream, const void *a, const void *h,
                         const void *done, const void *h0, const void *g,
@@ -310,20 +312,21 @@ int mrx_linear_scan_last(void *stream, const void *a, const void *b,
  *     h_t = done_t ? b_t : a_t h_{t-1} + b_t ,   a_t = sigma(-z_t),  b_t = sigma(z_t) g(h~_t),
  * which these entry points compute from z and h~ directly: a and b are never written to memory,
  * and the backward call returns dL/dz and dL/dh~ instead of dL/da and dL/db.
- * z, h_tilde, h, g, dz, dh_tilde: (B,T,D) fp32.  h0, P0 (nullable), h_last, P_last (nullable),
- * g_last (nullable), dh0 (nullable): (B,D) fp32, linear space: h0 = exp(carried log state) (0 for
+ * z, h_tilde, h, g, dz, dh_tilde: (B,T,D) in `dtype`, MRX_F32 or MRX_BF16 (bfloat16 in memory, float32 in
+ * the kernels: half the traffic of a kernel bound by it).  h0, P0 (nullable), h_last, P_last (nullable),
+ * g_last (nullable), dh0 (nullable): (B,D) fp32 whatever `dtype` is, linear space: h0 = exp(carried log state) (0 for
  * the cell's initial -inf), P = the cumulative decay since the last reset, whose log is the carry's
  * second leaf (a product below the fp32 range underflows to 0, i.e. a log of -inf; the leaf never
  * reaches h).  No counterpart as one function in the reference (which leaves the fusion to XLA). */
 int mrx_mingru_scan_fwd(void *stream, const void *z, const void *h_tilde, const void *done,
                         const void *h0, const void *P0, void *h, void *h_last, void *P_last,
-                        int64_t B, int64_t T, int64_t D, int done_dtype);
+                        int64_t B, int64_t T, int64_t D, int dtype, int done_dtype);
 
 /* h: the states the forward call wrote.  dz, dh_tilde: gradients with respect to the projections. */
 int mrx_mingru_scan_bwd(void *stream, const void *z, const void *h_tilde, const void *h,
                         const void *done, const void *h0, const void *g, const void *g_last,
                         void *dz, void *dh_tilde, void *dh0, int64_t B, int64_t T, int64_t D,
-                        int done_dtype);
+                        int dtype, int done_dtype);
 
 /* ---- Gated linear attention: linear attention with a scalar decay per step and head ----
  * The Mamba cell's algebra (mamba.py:109-122: elements (h_t = (B_t dt_t) (x) x_t, decay_t =

@@ -44,8 +44,8 @@ SIGNATURES = {
     "mrx_deltanet_fwd": (_I, [_P] * 11 + [_L] * 5 + [_I] * 3),
     "mrx_deltanet_bwd": (_I, [_P] * 15 + [_L] * 5 + [_I] * 2),
     "mrx_linear_scan_last": (_I, [_P] * 6 + [_L] * 4 + [_I] * 2),
-    "mrx_mingru_scan_fwd": (_I, [_P] * 9 + [_L] * 3 + [_I]),
-    "mrx_mingru_scan_bwd": (_I, [_P] * 11 + [_L] * 3 + [_I]),
+    "mrx_mingru_scan_fwd": (_I, [_P] * 9 + [_L] * 3 + [_I] * 2),
+    "mrx_mingru_scan_bwd": (_I, [_P] * 11 + [_L] * 3 + [_I] * 2),
     "mrx_gated_linear_attn_fwd": (_I, [_P] * 10 + [_L] * 5 + [_I] * 3),
     "mrx_gated_linear_attn_bwd": (_I, [_P] * 15 + [_L] * 5 + [_I] * 3),
     "mrx_linear_attn_step": (_I, [_P] * 10 + [_L] * 4 + [_I] * 3 + [ctypes.c_float]),

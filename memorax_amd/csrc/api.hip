@@ -57,7 +57,7 @@ extern "C" const char *mrx_status_string(int status)
     }
 }
 
-extern "C" int mrx_version(void) { return 304; }
+extern "C" int mrx_version(void) { return 400; }
 
 extern "C" int mrx_init(int device)
 {

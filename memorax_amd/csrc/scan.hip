@@ -58,6 +58,32 @@ template <typename E, int VEC> __device__ __forceinline__ Vec<E, VEC> vfill(E x)
     return r;
 }
 
+// Storage and arithmetic types of the (B,T,D) arrays may differ: bfloat16 in memory, float in registers
+// (the carries -- h0, P0, h_last, P_last, g_last, dh0 -- are always in the arithmetic type).
+template <typename S, typename E, int VEC> __device__ __forceinline__ Vec<E, VEC> ldv(const S *p)
+{
+    if constexpr (std::is_same<S, E>::value) {
+        return *reinterpret_cast<const Vec<E, VEC> *>(p);
+    } else {
+        const Vec<S, VEC> raw = *reinterpret_cast<const Vec<S, VEC> *>(p);
+        Vec<E, VEC> r;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) r.v[i] = (E)raw.v[i];
+        return r;
+    }
+}
+template <typename S, typename E, int VEC> __device__ __forceinline__ void stv(S *p, const Vec<E, VEC> &x)
+{
+    if constexpr (std::is_same<S, E>::value) {
+        *reinterpret_cast<Vec<E, VEC> *>(p) = x;
+    } else {
+        Vec<S, VEC> raw;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) raw.v[i] = (S)x.v[i];
+        *reinterpret_cast<Vec<S, VEC> *>(p) = raw;
+    }
+}
+
 // MinGRU in linear space.  The reference scans (log h, log decay) with logaddexp
 // (min_gru.py:49-78); the same recurrence is h_t = a_t h_{t-1} + b_t with, from the step's two
 // projections z and x = h~:  a = sigma(-z),  b = sigma(z) g(x),  g(x) = x + 0.5 (x >= 0) | sigma(x).
@@ -110,12 +136,12 @@ constexpr int TS = 8;  // time steps a wave holds in registers per super-step
 // one-vector-lane instances that small shapes take: with 16 waves of 8 steps a sequence of up to 128
 // steps is one super-step, every load of the workgroup in flight at once and a single barrier).
 // smem: sH[2][NW][64] Vec, sP[2][NW][64] Vec, sF[2][NW] int.
-template <typename E, int VEC, bool MG = false, int MAXW = 8>
+template <typename E, int VEC, bool MG = false, int MAXW = 8, typename S = E>
 __global__ void __launch_bounds__(64 * MAXW)
-diag_scan_fwd_kernel(const E *__restrict__ a, const E *__restrict__ b,
+diag_scan_fwd_kernel(const S *__restrict__ a, const S *__restrict__ b,
                      const void *__restrict__ done, int done_f32,
                      const E *__restrict__ h0, const E *__restrict__ P0,
-                     E *__restrict__ h, E *__restrict__ h_last,
+                     S *__restrict__ h, E *__restrict__ h_last,
                      E *__restrict__ P_last, int T, int64_t D, int tiles, int NW,
                      int a_ti)
 {
@@ -151,8 +177,8 @@ diag_scan_fwd_kernel(const E *__restrict__ a, const E *__restrict__ b,
             const int t = ts + s;
             if (t < T && act) {
                 const int64_t off = (row0 + t) * D + col;
-                p[s] = *reinterpret_cast<const V *>(a + (a_ti ? col : off));
-                x[s] = *reinterpret_cast<const V *>(b + off);
+                p[s] = ldv<S, E, VEC>(a + (a_ti ? col : off));
+                x[s] = ldv<S, E, VEC>(b + off);
             } else {
                 p[s] = vfill<E, VEC>(O::one());
                 x[s] = vfill<E, VEC>(O::zero());
@@ -181,7 +207,7 @@ diag_scan_fwd_kernel(const E *__restrict__ a, const E *__restrict__ b,
                     carry_p.v[i] = r ? p[s].v[i] : pn;
                 }
                 if (ts + s < T && act)
-                    *reinterpret_cast<V *>(h + (row0 + ts + s) * D + col) = carry_h;
+                    stv<S, E, VEC>(h + (row0 + ts + s) * D + col, carry_h);
             }
             continue;
         }
@@ -233,7 +259,7 @@ diag_scan_fwd_kernel(const E *__restrict__ a, const E *__restrict__ b,
                 out.v[i] = seen ? x[s].v[i] : fx;
             }
             if (ts + s < T && act)
-                *reinterpret_cast<V *>(h + (row0 + ts + s) * D + col) = out;
+                stv<S, E, VEC>(h + (row0 + ts + s) * D + col, out);
         }
         buf ^= 1;
     }
@@ -246,13 +272,13 @@ diag_scan_fwd_kernel(const E *__restrict__ a, const E *__restrict__ b,
 // Backward: the same scan walked from t = T-1 down with coefficient conj(a_{t+1}),
 // cut where done_{t+1}; reversed index r = T-1-t runs forward.
 // MG: a holds z, hx holds x = h~; da receives dz and db receives dx.
-template <typename E, int VEC, bool MG = false, int MAXW = 8>
+template <typename E, int VEC, bool MG = false, int MAXW = 8, typename S = E>
 __global__ void __launch_bounds__(64 * MAXW)
-diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hx, const E *__restrict__ hfw,
+diag_scan_bwd_kernel(const S *__restrict__ a, const S *__restrict__ hx, const S *__restrict__ hfw,
                      const void *__restrict__ done, int done_f32,
-                     const E *__restrict__ h0, const E *__restrict__ g,
-                     const E *__restrict__ g_last, E *__restrict__ da,
-                     E *__restrict__ db, E *__restrict__ dh0, int T, int64_t D,
+                     const E *__restrict__ h0, const S *__restrict__ g,
+                     const E *__restrict__ g_last, S *__restrict__ da,
+                     S *__restrict__ db, E *__restrict__ dh0, int T, int64_t D,
                      int tiles, int NW, int a_ti, int da_sum)
 {
     using V = Vec<E, VEC>;
@@ -296,19 +322,19 @@ diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hx, const E 
             if (t >= 0) {
                 if (act) {
                     const int64_t off = (row0 + t) * D + col;
-                    x[s] = *reinterpret_cast<const V *>(g + off);
+                    x[s] = ldv<S, E, VEC>(g + off);
                     if (t + 1 < T) {
-                        V av = *reinterpret_cast<const V *>(a + (a_ti ? col : off + D));
+                        V av = ldv<S, E, VEC>(a + (a_ti ? col : off + D));
 #pragma unroll
                         for (int i = 0; i < VEC; ++i) p[s].v[i] = MG ? av.v[i] : O::conj(av.v[i]);  // MG: z_{t+1} for now
                     }
                     if (t > 0)
-                        hp[s] = *reinterpret_cast<const V *>(hfw + off - D);
+                        hp[s] = ldv<S, E, VEC>(hfw + off - D);
                     else if (h0)
                         hp[s] = *reinterpret_cast<const V *>(h0 + bi * D + col);
                     if constexpr (MG) {
-                        zt[s] = *reinterpret_cast<const V *>(a + off);
-                        xt[s] = *reinterpret_cast<const V *>(hx + off);
+                        zt[s] = ldv<S, E, VEC>(a + off);
+                        xt[s] = ldv<S, E, VEC>(hx + off);
                     }
                 }
                 if (t + 1 < T && done_at(done, done_f32, row0 + t + 1)) cmask |= 1u << s;
@@ -400,15 +426,15 @@ diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hx, const E 
                     V oz, ox;
 #pragma unroll
                     for (int i = 0; i < VEC; ++i) MinGru::grads(zt[s].v[i], xt[s].v[i], x[s].v[i], o.v[i], oz.v[i], ox.v[i]);
-                    *reinterpret_cast<V *>(db + off) = ox;
-                    *reinterpret_cast<V *>(da + off) = oz;
+                    stv<S, E, VEC>(db + off, ox);
+                    stv<S, E, VEC>(da + off, oz);
                 } else {
-                    *reinterpret_cast<V *>(db + off) = x[s];
+                    stv<S, E, VEC>(db + off, x[s]);
                     if (da_sum) {
 #pragma unroll
                         for (int i = 0; i < VEC; ++i) dsum.v[i] = O::madd(O::one(), dsum.v[i], o.v[i]);
                     } else {
-                        *reinterpret_cast<V *>(da + off) = o;
+                        stv<S, E, VEC>(da + off, o);
                     }
                 }
             }
@@ -427,12 +453,12 @@ diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hx, const E 
                 }
             }
         }
-        if (w == 0 && act) *reinterpret_cast<V *>(da + bi * D + col) = dsum;
+        if (w == 0 && act) *reinterpret_cast<V *>(reinterpret_cast<E *>(da) + bi * D + col) = dsum;  // (B,D), arithmetic type
     }
     if (w == 0 && act && dh0) {
         // carry = lam_0 ; dh0 = done_0 ? 0 : conj(a_0) lam_0
         const bool d0 = done_at(done, done_f32, row0);
-        V a0 = *reinterpret_cast<const V *>(a + (a_ti ? col : row0 * D + col));
+        V a0 = ldv<S, E, VEC>(a + (a_ti ? col : row0 * D + col));
         if constexpr (MG) {
 #pragma unroll
             for (int i = 0; i < VEC; ++i) {
@@ -456,12 +482,12 @@ diag_scan_bwd_kernel(const E *__restrict__ a, const E *__restrict__ hx, const E 
 // with the loads of the next group issued before the current group is consumed
 // (register double buffering), so a wave always has 2*SG (forward) / 3*SG (backward)
 // row loads in flight.  done flags are prefetched as raw bits with the data.
-template <typename E, int VEC, int SG, bool MG = false>
+template <typename E, int VEC, int SG, bool MG = false, typename S = E>
 __global__ void __launch_bounds__(256)
-diag_scan_fwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ b,
+diag_scan_fwd_stream_kernel(const S *__restrict__ a, const S *__restrict__ b,
                             const void *__restrict__ done, int done_f32,
                             const E *__restrict__ h0, const E *__restrict__ P0,
-                            E *__restrict__ h, E *__restrict__ h_last, E *__restrict__ P_last,
+                            S *__restrict__ h, E *__restrict__ h_last, E *__restrict__ P_last,
                             int64_t B, int T, int64_t D, int64_t cols_per_row, int a_ti)
 {
     using V = Vec<E, VEC>;
@@ -485,8 +511,8 @@ diag_scan_fwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ b,
             pd[s] = 0u;
             if (t < T) {
                 const int64_t off = (row0 + t) * D + col;
-                pa[s] = *reinterpret_cast<const V *>(a + (a_ti ? col : off));
-                pb[s] = *reinterpret_cast<const V *>(b + off);
+                pa[s] = ldv<S, E, VEC>(a + (a_ti ? col : off));
+                pb[s] = ldv<S, E, VEC>(b + off);
                 pd[s] = done_raw(done, done_f32, row0 + t);
             }
         }
@@ -509,7 +535,7 @@ diag_scan_fwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ b,
                     ch.v[i] = r ? xb[s].v[i] : hn;
                     cp.v[i] = r ? xa[s].v[i] : pn;
                 }
-                *reinterpret_cast<V *>(h + (row0 + t0 + s) * D + col) = ch;
+                stv<S, E, VEC>(h + (row0 + t0 + s) * D + col, ch);
             }
         }
 #pragma unroll
@@ -577,12 +603,12 @@ diag_scan_last_kernel(const E *__restrict__ a, const E *__restrict__ b, const vo
 }
 
 // MG: a holds z, hx holds x = h~ (a fourth load per step); da receives dz and db receives dx.
-template <typename E, int VEC, int SG, bool MG = false>
+template <typename E, int VEC, int SG, bool MG = false, typename S = E>
 __global__ void __launch_bounds__(256)
-diag_scan_bwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ hx, const E *__restrict__ hfw,
+diag_scan_bwd_stream_kernel(const S *__restrict__ a, const S *__restrict__ hx, const S *__restrict__ hfw,
                             const void *__restrict__ done, int done_f32,
-                            const E *__restrict__ h0, const E *__restrict__ g,
-                            const E *__restrict__ g_last, E *__restrict__ da, E *__restrict__ db,
+                            const E *__restrict__ h0, const S *__restrict__ g,
+                            const E *__restrict__ g_last, S *__restrict__ da, S *__restrict__ db,
                             E *__restrict__ dh0, int64_t B, int T, int64_t D, int64_t cols_per_row, int a_ti,
                             int da_sum)
 {
@@ -609,10 +635,10 @@ diag_scan_bwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ hx, c
             ph[s] = vfill<E, VEC>(O::zero());
             if (t >= 0) {
                 const int64_t off = (row0 + t) * D + col;
-                pg[s] = *reinterpret_cast<const V *>(g + off);
-                pa[s] = *reinterpret_cast<const V *>(a + (a_ti ? col : off));
-                if constexpr (MG) px[s] = *reinterpret_cast<const V *>(hx + off);
-                if (t > 0) ph[s] = *reinterpret_cast<const V *>(hfw + off - D);
+                pg[s] = ldv<S, E, VEC>(g + off);
+                pa[s] = ldv<S, E, VEC>(a + (a_ti ? col : off));
+                if constexpr (MG) px[s] = ldv<S, E, VEC>(hx + off);
+                if (t > 0) ph[s] = ldv<S, E, VEC>(hfw + off - D);
                 else if (h0) ph[s] = *reinterpret_cast<const V *>(h0 + bi * D + col);
                 pd[s] = done_raw(done, done_f32, row0 + t);
             }
@@ -645,12 +671,12 @@ diag_scan_bwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ hx, c
                         lam.v[i] = dn ? O::zero() : nxt;           // conj(abar_t) lam_t for step t-1
                     }
                 }
-                *reinterpret_cast<V *>(db + off) = l;
+                stv<S, E, VEC>(db + off, l);
                 if (!MG && da_sum) {
 #pragma unroll
                     for (int i = 0; i < VEC; ++i) dsum.v[i] = O::madd(O::one(), dsum.v[i], o.v[i]);
                 } else {
-                    *reinterpret_cast<V *>(da + off) = o;
+                    stv<S, E, VEC>(da + off, o);
                 }
             }
         }
@@ -661,7 +687,7 @@ diag_scan_bwd_stream_kernel(const E *__restrict__ a, const E *__restrict__ hx, c
             for (int s = 0; s < SG; ++s) xx[s] = nx[s];
         }
     }
-    if (!MG && da_sum) *reinterpret_cast<V *>(da + bi * D + col) = dsum;
+    if (!MG && da_sum) *reinterpret_cast<V *>(reinterpret_cast<E *>(da) + bi * D + col) = dsum;  // (B,D), arithmetic type
     if (dh0) *reinterpret_cast<V *>(dh0 + bi * D + col) = lam;  // conj(abar_0) lam_0
 }
 
@@ -686,7 +712,8 @@ struct ScanPlan {
 //    kernel runs whenever the columns alone give >= 2048 waves.  With the MinGRU map inside (a
 //    fourth stream and the map's arithmetic per element) the eight-wave split loses to streaming at
 //    1024x128x256 (202 vs 165 us; level at the large shape), so that case keeps the rule it had.
-ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, bool al8, bool bwd, bool mg = false)
+ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, bool al8, bool bwd, bool mg = false,
+                   bool half_storage = false)
 {
     const int maxvec = (int)(16 / esize);
     int vec = 1;
@@ -700,6 +727,17 @@ ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, boo
         if (D % v == 0 && ok_al && (v == 1 || 4 * D >= 3 * covered)) { vec = v; break; }
     }
     auto ntiles = [&](int v) { return (D + 64 * (int64_t)v - 1) / (64 * (int64_t)v); };
+    // bfloat16 arrays: a lane's loads are half as wide, so the widest vector stays (no narrowing for the sake
+    // of more columns); measured on the MinGRU kernels at 1024x128x256, 512x1024x1024, 256x128x256: with 1024
+    // waves of columns the streaming kernel is ahead or level (backward 186 -> 161 us, forward of the largest
+    // shape 1412 -> 875 us), below that eight waves along time (backward 88 -> 44 us at 256x128x256)
+    if (half_storage) {
+        const int64_t cols = B * ntiles(vec);
+        if (cols >= 1024) return {vec, 1, (int)ntiles(vec), true};
+        int nw = 1;
+        while (nw < 8 && cols * nw < 2048 && (int64_t)nw * TS < T) nw <<= 1;
+        return {vec, nw, (int)ntiles(vec), nw == 1};
+    }
     // complex64 (measured on 1024x128x{64,128,256}, 4096x128x64, 256x1024x{64,256}, 64x4096x256): one
     // element per lane is the width the column rule below arrives at for most shapes, and at that width
     // the streaming kernel is ahead of the wave-split one as soon as the columns give it 2048 waves
@@ -758,7 +796,8 @@ template <typename E, typename F> void vec_switch(int vec, F f)
 }
 
 // MG (E = float): a and b hold the MinGRU projections z and h~.
-template <typename E, bool MG = false>
+// S: storage type of the (B,T,D) arrays (E, or __bf16 with E = float).
+template <typename E, bool MG = false, typename S = E>
 int launch_fwd(hipStream_t st, const void *a, const void *b, const void *done,
                int done_f32, const void *h0, const void *P0, void *h, void *h_last,
                void *P_last, int64_t B, int64_t T, int64_t D, int a_ti)
@@ -767,16 +806,16 @@ int launch_fwd(hipStream_t st, const void *a, const void *b, const void *done,
                       aligned(P0, 16) && aligned(h_last, 16) && aligned(P_last, 16);
     const bool al8 = aligned(a, 8) && aligned(b, 8) && aligned(h, 8) && aligned(h0, 8) &&
                      aligned(P0, 8) && aligned(h_last, 8) && aligned(P_last, 8);
-    const ScanPlan pl = plan_scan(B, T, D, sizeof(E), al16, al8, false);
+    const ScanPlan pl = plan_scan(B, T, D, sizeof(E), al16, al8, false, MG, !std::is_same<S, E>::value);
     int rc = MRX_ERR_LAUNCH;
     if (pl.stream) {
         const int64_t cpr = D / pl.vec;
         const dim3 grid((unsigned)((B * cpr + 255) / 256)), block(256);
         vec_switch<E>(pl.vec, [&](auto vc) {
             constexpr int VEC = decltype(vc)::value;
-            rc = launch_kernel((diag_scan_fwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8), MG>), grid, block, 0, st,
-                               (const E *)a, (const E *)b, done, done_f32, (const E *)h0, (const E *)P0,
-                               (E *)h, (E *)h_last, (E *)P_last, B, (int)T, D, cpr, a_ti);
+            rc = launch_kernel((diag_scan_fwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8), MG, S>), grid, block, 0, st,
+                               (const S *)a, (const S *)b, done, done_f32, (const E *)h0, (const E *)P0,
+                               (S *)h, (E *)h_last, (E *)P_last, B, (int)T, D, cpr, a_ti);
         });
     } else {
         const dim3 grid((unsigned)(B * pl.tiles)), block(64 * pl.nw);
@@ -785,14 +824,14 @@ int launch_fwd(hipStream_t st, const void *a, const void *b, const void *done,
             constexpr int VEC = decltype(vc)::value;
             if constexpr (VEC == 1) {
                 if (pl.nw == 16) {
-                    rc = launch_kernel((diag_scan_fwd_kernel<E, 1, MG, 16>), grid, block, smem, st, (const E *)a,
-                                       (const E *)b, done, done_f32, (const E *)h0, (const E *)P0, (E *)h,
+                    rc = launch_kernel((diag_scan_fwd_kernel<E, 1, MG, 16, S>), grid, block, smem, st, (const S *)a,
+                                       (const S *)b, done, done_f32, (const E *)h0, (const E *)P0, (S *)h,
                                        (E *)h_last, (E *)P_last, (int)T, D, pl.tiles, pl.nw, a_ti);
                     return;
                 }
             }
-            rc = launch_kernel((diag_scan_fwd_kernel<E, VEC, MG>), grid, block, smem, st, (const E *)a,
-                               (const E *)b, done, done_f32, (const E *)h0, (const E *)P0, (E *)h,
+            rc = launch_kernel((diag_scan_fwd_kernel<E, VEC, MG, 8, S>), grid, block, smem, st, (const S *)a,
+                               (const S *)b, done, done_f32, (const E *)h0, (const E *)P0, (S *)h,
                                (E *)h_last, (E *)P_last, (int)T, D, pl.tiles, pl.nw, a_ti);
         });
     }
@@ -800,7 +839,7 @@ int launch_fwd(hipStream_t st, const void *a, const void *b, const void *done,
 }
 
 // MG (E = float): a holds z, hx holds h~ (else unused), da and db receive dz and dh~.
-template <typename E, bool MG = false>
+template <typename E, bool MG = false, typename S = E>
 int launch_bwd(hipStream_t st, const void *a, const void *hx, const void *h, const void *done,
                int done_f32, const void *h0, const void *g, const void *g_last, void *da,
                void *db, void *dh0, int64_t B, int64_t T, int64_t D, int a_ti, int da_sum = 0)
@@ -809,16 +848,16 @@ int launch_bwd(hipStream_t st, const void *a, const void *hx, const void *h, con
                       aligned(g_last, 16) && aligned(da, 16) && aligned(db, 16) && aligned(dh0, 16);
     const bool al8 = aligned(a, 8) && aligned(hx, 8) && aligned(h, 8) && aligned(g, 8) && aligned(h0, 8) &&
                      aligned(g_last, 8) && aligned(da, 8) && aligned(db, 8) && aligned(dh0, 8);
-    const ScanPlan pl = plan_scan(B, T, D, sizeof(E), al16, al8, true, MG);
+    const ScanPlan pl = plan_scan(B, T, D, sizeof(E), al16, al8, true, MG, !std::is_same<S, E>::value);
     int rc = MRX_ERR_LAUNCH;
     if (pl.stream) {
         const int64_t cpr = D / pl.vec;
         const dim3 grid((unsigned)((B * cpr + 255) / 256)), block(256);
         vec_switch<E>(pl.vec, [&](auto vc) {
             constexpr int VEC = decltype(vc)::value;
-            rc = launch_kernel((diag_scan_bwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8), MG>), grid, block, 0, st,
-                               (const E *)a, (const E *)hx, (const E *)h, done, done_f32, (const E *)h0, (const E *)g,
-                               (const E *)g_last, (E *)da, (E *)db, (E *)dh0, B, (int)T, D, cpr, a_ti, da_sum);
+            rc = launch_kernel((diag_scan_bwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8), MG, S>), grid, block, 0, st,
+                               (const S *)a, (const S *)hx, (const S *)h, done, done_f32, (const E *)h0, (const S *)g,
+                               (const E *)g_last, (S *)da, (S *)db, (E *)dh0, B, (int)T, D, cpr, a_ti, da_sum);
         });
     } else {
         const dim3 grid((unsigned)(B * pl.tiles)), block(64 * pl.nw);
@@ -827,16 +866,16 @@ int launch_bwd(hipStream_t st, const void *a, const void *hx, const void *h, con
             constexpr int VEC = decltype(vc)::value;
             if constexpr (VEC == 1 || (VEC == 2 && sizeof(E) == 4 && !MG)) {
                 if (pl.nw == 16) {
-                    rc = launch_kernel((diag_scan_bwd_kernel<E, VEC, MG, 16>), grid, block, smem, st, (const E *)a,
-                                       (const E *)hx, (const E *)h, done, done_f32, (const E *)h0, (const E *)g,
-                                       (const E *)g_last, (E *)da, (E *)db, (E *)dh0, (int)T, D, pl.tiles,
+                    rc = launch_kernel((diag_scan_bwd_kernel<E, VEC, MG, 16, S>), grid, block, smem, st, (const S *)a,
+                                       (const S *)hx, (const S *)h, done, done_f32, (const E *)h0, (const S *)g,
+                                       (const E *)g_last, (S *)da, (S *)db, (E *)dh0, (int)T, D, pl.tiles,
                                        pl.nw, a_ti, da_sum);
                     return;
                 }
             }
-            rc = launch_kernel((diag_scan_bwd_kernel<E, VEC, MG>), grid, block, smem, st, (const E *)a,
-                               (const E *)hx, (const E *)h, done, done_f32, (const E *)h0, (const E *)g,
-                               (const E *)g_last, (E *)da, (E *)db, (E *)dh0, (int)T, D, pl.tiles,
+            rc = launch_kernel((diag_scan_bwd_kernel<E, VEC, MG, 8, S>), grid, block, smem, st, (const S *)a,
+                               (const S *)hx, (const S *)h, done, done_f32, (const E *)h0, (const S *)g,
+                               (const E *)g_last, (S *)da, (S *)db, (E *)dh0, (int)T, D, pl.tiles,
                                pl.nw, a_ti, da_sum);
         });
     }
@@ -897,7 +936,13 @@ extern "C" int mrx_linear_scan_fwd(void *stream, const void *a, const void *b, c
             return MRX_ERR_INVALID_ARG;
         return launch_fwd<c64>(st, a, b, done, done_dtype, h0, P0, h, h_last, P_last, B, T, D, ti);
     }
-    return dtype == MRX_BF16 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
+    if (dtype == MRX_BF16) {  // a, b, h in bfloat16; arithmetic and carries in float32
+        if (!aligned(a, 2) || !aligned(b, 2) || !aligned(h, 2) || !aligned(h0, 4) || !aligned(P0, 4) ||
+            !aligned(h_last, 4) || !aligned(P_last, 4))
+            return MRX_ERR_INVALID_ARG;
+        return launch_fwd<float, false, __bf16>(st, a, b, done, done_dtype, h0, P0, h, h_last, P_last, B, T, D, ti);
+    }
+    return MRX_ERR_INVALID_ARG;
 }
 
 extern "C" int mrx_linear_scan_bwd(void *stream, const void *a, const void *h, const void *done,
@@ -924,7 +969,14 @@ extern "C" int mrx_linear_scan_bwd(void *stream, const void *a, const void *h, c
             return MRX_ERR_INVALID_ARG;
         return launch_bwd<c64>(st, a, nullptr, h, done, done_dtype, h0, g, g_last, da, db, dh0, B, T, D, ti, da_sum);
     }
-    return dtype == MRX_BF16 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
+    if (dtype == MRX_BF16) {  // a, h, g, da (per step), db in bfloat16; carries and a summed da in float32
+        if (!aligned(a, 2) || !aligned(h, 2) || !aligned(g, 2) || !aligned(da, da_sum ? 4 : 2) || !aligned(db, 2) ||
+            !aligned(h0, 4) || !aligned(g_last, 4) || !aligned(dh0, 4))
+            return MRX_ERR_INVALID_ARG;
+        return launch_bwd<float, false, __bf16>(st, a, nullptr, h, done, done_dtype, h0, g, g_last, da, db, dh0, B, T, D,
+                                                ti, da_sum);
+    }
+    return MRX_ERR_INVALID_ARG;
 }
 
 extern "C" int mrx_linear_scan_last(void *stream, const void *a, const void *b, const void *done,
@@ -950,14 +1002,21 @@ extern "C" int mrx_linear_scan_last(void *stream, const void *a, const void *b, 
 
 extern "C" int mrx_mingru_scan_fwd(void *stream, const void *z, const void *h_tilde, const void *done,
                                    const void *h0, const void *P0, void *h, void *h_last, void *P_last,
-                                   int64_t B, int64_t T, int64_t D, int done_dtype)
+                                   int64_t B, int64_t T, int64_t D, int dtype, int done_dtype)
 {
     if (!z || !h_tilde || !done || !h) return MRX_ERR_INVALID_ARG;
     if (!scan_shape_ok(B, T, D)) return MRX_ERR_INVALID_ARG;
+    if (dtype != MRX_F32 && dtype != MRX_BF16) return dtype == MRX_C64 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
     if (done_dtype != MRX_DONE_U8 && done_dtype != MRX_DONE_F32) return MRX_ERR_INVALID_ARG;
     if (done_dtype == MRX_DONE_F32 && !aligned(done, 4)) return MRX_ERR_INVALID_ARG;
-    for (const void *p : {z, h_tilde, h0, P0, (const void *)h, (const void *)h_last, (const void *)P_last})
+    const size_t ea = dtype == MRX_BF16 ? 2 : 4;  // z, h~, h in `dtype`; the carries in float32
+    for (const void *p : {z, h_tilde, (const void *)h})
+        if (!aligned(p, ea)) return MRX_ERR_INVALID_ARG;
+    for (const void *p : {h0, P0, (const void *)h_last, (const void *)P_last})
         if (!aligned(p, 4)) return MRX_ERR_INVALID_ARG;
+    if (dtype == MRX_BF16)
+        return launch_fwd<float, true, __bf16>((hipStream_t)stream, z, h_tilde, done, done_dtype, h0, P0, h, h_last,
+                                               P_last, B, T, D, 0);
     return launch_fwd<float, true>((hipStream_t)stream, z, h_tilde, done, done_dtype, h0, P0, h, h_last, P_last, B, T,
                                    D, 0);
 }
@@ -965,14 +1024,21 @@ extern "C" int mrx_mingru_scan_fwd(void *stream, const void *z, const void *h_ti
 extern "C" int mrx_mingru_scan_bwd(void *stream, const void *z, const void *h_tilde, const void *h,
                                    const void *done, const void *h0, const void *g, const void *g_last,
                                    void *dz, void *dh_tilde, void *dh0, int64_t B, int64_t T, int64_t D,
-                                   int done_dtype)
+                                   int dtype, int done_dtype)
 {
     if (!z || !h_tilde || !h || !done || !g || !dz || !dh_tilde) return MRX_ERR_INVALID_ARG;
     if (!scan_shape_ok(B, T, D)) return MRX_ERR_INVALID_ARG;
+    if (dtype != MRX_F32 && dtype != MRX_BF16) return dtype == MRX_C64 ? MRX_ERR_UNSUPPORTED : MRX_ERR_INVALID_ARG;
     if (done_dtype != MRX_DONE_U8 && done_dtype != MRX_DONE_F32) return MRX_ERR_INVALID_ARG;
     if (done_dtype == MRX_DONE_F32 && !aligned(done, 4)) return MRX_ERR_INVALID_ARG;
-    for (const void *p : {z, h_tilde, h, h0, g, g_last, (const void *)dz, (const void *)dh_tilde, (const void *)dh0})
+    const size_t ea = dtype == MRX_BF16 ? 2 : 4;  // z, h~, h, g, dz, dh~ in `dtype`; the carries in float32
+    for (const void *p : {z, h_tilde, h, g, (const void *)dz, (const void *)dh_tilde})
+        if (!aligned(p, ea)) return MRX_ERR_INVALID_ARG;
+    for (const void *p : {h0, g_last, (const void *)dh0})
         if (!aligned(p, 4)) return MRX_ERR_INVALID_ARG;
+    if (dtype == MRX_BF16)
+        return launch_bwd<float, true, __bf16>((hipStream_t)stream, z, h_tilde, h, done, done_dtype, h0, g, g_last, dz,
+                                               dh_tilde, dh0, B, T, D, 0);
     return launch_bwd<float, true>((hipStream_t)stream, z, h_tilde, h, done, done_dtype, h0, g, g_last, dz, dh_tilde,
                                    dh0, B, T, D, 0);
 }

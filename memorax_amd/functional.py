@@ -159,12 +159,14 @@ class _LinearScan(torch.autograd.Function):
     @staticmethod
     def forward(ctx, a, b, done, h0, P0):
         a_, b_ = a.contiguous(), b.contiguous()
-        h0_ = None if h0 is None else h0.contiguous()
-        P0_ = None if P0 is None else P0.contiguous()
+        carry = (lambda x: x.float()) if b.dtype == torch.bfloat16 else (lambda x: x)  # bfloat16 arrays: float32 carries
+        h0_ = None if h0 is None else carry(h0).contiguous()
+        P0_ = None if P0 is None else carry(P0).contiguous()
         h, h_last, P_last = K.linear_scan_fwd(a_, b_, done, h0_, P0_)
         ctx.save_for_backward(a_, h, h0_ if h0_ is not None else torch.empty(0, device=b.device))
         ctx.done = done
         ctx.has_h0 = h0 is not None
+        ctx.h0_dtype = None if h0 is None else h0.dtype
         ctx.mark_non_differentiable(P_last)
         return h, h_last, P_last
 
@@ -177,11 +179,11 @@ class _LinearScan(torch.autograd.Function):
         ti = a.dim() == 1  # a broadcast coefficient: the kernel sums its gradient over time, the rest is (B,D)
         da, db, dh0 = K.linear_scan_bwd(a, h, ctx.done, h0, g, g_last, sum_da=ti)
         if ti:
-            da = da.sum(dim=0)
+            da = da.sum(dim=0).to(a.dtype)
         return (da if ctx.needs_input_grad[0] else None,
                 db if ctx.needs_input_grad[1] else None,
                 None,
-                dh0 if (ctx.has_h0 and ctx.needs_input_grad[3]) else None,
+                dh0.to(ctx.h0_dtype) if (ctx.has_h0 and ctx.needs_input_grad[3]) else None,
                 None)
 
 
@@ -198,13 +200,14 @@ def linear_scan(a, b, done, h0=None, P0=None):
 class _MinGRUScan(torch.autograd.Function):
     @staticmethod
     def forward(ctx, z, h_tilde, done, h0, P0):
-        z_, x_ = z.contiguous(), h_tilde.contiguous()
-        h0_ = None if h0 is None else h0.contiguous()
-        P0_ = None if P0 is None else P0.contiguous()
+        z_, x_ = z.contiguous(), h_tilde.contiguous().to(z.dtype)
+        h0_ = None if h0 is None else h0.float().contiguous()   # the carries are float32 whatever the arrays are
+        P0_ = None if P0 is None else P0.float().contiguous()
         h, h_last, P_last = K.mingru_scan_fwd(z_, x_, done, h0_, P0_)
         ctx.save_for_backward(z_, x_, h, h0_ if h0_ is not None else torch.empty(0, device=z.device))
         ctx.done = done
         ctx.has_h0 = h0 is not None
+        ctx.h0_dtype = None if h0 is None else h0.dtype
         ctx.mark_non_differentiable(P_last)
         return h, h_last, P_last
 
@@ -218,7 +221,7 @@ class _MinGRUScan(torch.autograd.Function):
         return (dz if ctx.needs_input_grad[0] else None,
                 dx if ctx.needs_input_grad[1] else None,
                 None,
-                dh0 if (ctx.has_h0 and ctx.needs_input_grad[3]) else None,
+                dh0.to(ctx.h0_dtype) if (ctx.has_h0 and ctx.needs_input_grad[3]) else None,
                 None)
 
 
@@ -226,7 +229,8 @@ class _MinGRUScan(torch.autograd.Function):
 def mingru_scan(z, h_tilde, done, h0=None, P0=None):
     """MinGRU from its two projections (min_gru.py:49-78 scanned by memoroid.py:60-91), linear space:
     h_t = sigmoid(-z_t) h_{t-1} + sigmoid(z_t) g(h~_t), g(x) = x + 0.5 (x >= 0) | sigmoid(x), with the
-    gate arithmetic inside the scan kernels.  z, h_tilde: (B,T,D) fp32; h0, P0: (B,D).
+    gate arithmetic inside the scan kernels.  z, h_tilde: (B,T,D) float32 or bfloat16 (the arithmetic and the
+    carries are float32 either way); h0, P0: (B,D).
     Returns (h, h_last, P_last); P_last is not differentiable."""
     if _no_steps(z):
         return _scan_without_steps(z, h0, P0)

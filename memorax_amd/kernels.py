@@ -73,22 +73,24 @@ def chunk_size(dtype, delta=False) -> int:
 
 # ----------------------------------------------------------------- diagonal scan
 def linear_scan_fwd(a, b, done, h0=None, P0=None, want_P=True):
-    """h_t = done ? b_t : a_t h_{t-1} + b_t.  a: (B,T,D) or (D,) time-invariant.
+    """h_t = done ? b_t : a_t h_{t-1} + b_t.  a: (B,T,D) or (D,) time-invariant.  float32, complex64, or
+    bfloat16 arrays with float32 arithmetic and float32 carries (h0, P0, h_last, P_last).
     Returns (h, h_last, P_last)."""
     lib = _lib.load()
     B, T, D = b.shape
     dt = b.dtype
-    if dt not in (torch.float32, torch.complex64):
-        raise ValueError("linear_scan supports float32 and complex64")
+    if dt not in (torch.float32, torch.complex64, torch.bfloat16):
+        raise ValueError("linear_scan supports float32, complex64 and bfloat16")
+    ct = torch.float32 if dt == torch.bfloat16 else dt  # the carries' type
     ti = a.dim() == 1
     _chk(a, "a", dt, (D,) if ti else (B, T, D))
     _chk(b, "b", dt)
-    _chk(h0, "h0", dt, (B, D))
-    _chk(P0, "P0", dt, (B, D))
+    _chk(h0, "h0", ct, (B, D))
+    _chk(P0, "P0", ct, (B, D))
     done, dd = _done(done, B, T)
     h = torch.empty_like(b)
-    h_last = torch.empty((B, D), dtype=dt, device=b.device)
-    P_last = torch.empty((B, D), dtype=dt, device=b.device) if want_P else None
+    h_last = torch.empty((B, D), dtype=ct, device=b.device)
+    P_last = torch.empty((B, D), dtype=ct, device=b.device) if want_P else None
     st = lib.mrx_linear_scan_fwd(_stream(), _ptr(a), _ptr(b), _ptr(done), _ptr(h0), _ptr(P0),
                                  _ptr(h), _ptr(h_last), _ptr(P_last), B, T, D, _DT[dt], dd, int(ti))
     _lib.check(st, "mrx_linear_scan_fwd")
@@ -122,18 +124,19 @@ def linear_scan_bwd(a, h, done, h0, g, g_last=None, sum_da=False):
     lib = _lib.load()
     B, T, D = g.shape
     dt = g.dtype
+    ct = torch.float32 if dt == torch.bfloat16 else dt  # the carries' type (and a summed da's)
     ti = a.dim() == 1
     _chk(a, "a", dt, (D,) if ti else (B, T, D))
     _chk(h, "h", dt, (B, T, D))
     _chk(g, "g", dt)
-    _chk(h0, "h0", dt, (B, D))
-    _chk(g_last, "g_last", dt, (B, D))
+    _chk(h0, "h0", ct, (B, D))
+    _chk(g_last, "g_last", ct, (B, D))
     done, dd = _done(done, B, T)
     if sum_da and not ti:
         raise ValueError("sum_da belongs to a time-invariant a")
-    da = torch.empty((B, D), dtype=dt, device=g.device) if sum_da else torch.empty_like(g)
+    da = torch.empty((B, D), dtype=ct, device=g.device) if sum_da else torch.empty_like(g)
     db = torch.empty_like(g)
-    dh0 = torch.empty((B, D), dtype=dt, device=g.device)
+    dh0 = torch.empty((B, D), dtype=ct, device=g.device)
     st = lib.mrx_linear_scan_bwd(_stream(), _ptr(a), _ptr(h), _ptr(done), _ptr(h0), _ptr(g),
                                  _ptr(g_last), _ptr(da), _ptr(db), _ptr(dh0), B, T, D, _DT[dt],
                                  dd, _lib.MRX_A_TIME_INVARIANT_SUM_DA if sum_da else int(ti))
@@ -144,13 +147,14 @@ def linear_scan_bwd(a, h, done, h0, g, g_last=None, sum_da=False):
 def mingru_scan_fwd(z, h_tilde, done, h0=None, P0=None, want_P=True):
     """MinGRU recurrence from its two projections (min_gru.py:49-78, in linear space):
     h_t = done ? b_t : a_t h_{t-1} + b_t with a = sigmoid(-z), b = sigmoid(z) g(h~) formed inside
-    the kernel.  z, h_tilde: (B,T,D) fp32; h0, P0: (B,D) linear space.  Returns (h, h_last, P_last)."""
+    the kernel.  z, h_tilde: (B,T,D) float32 or bfloat16 (float32 arithmetic); h0, P0: (B,D) float32,
+    linear space.  Returns (h in the dtype of z, h_last, P_last)."""
     lib = _lib.load()
     B, T, D = z.shape
-    if z.dtype != torch.float32:
-        raise ValueError("mingru_scan supports float32")
-    _chk(z, "z", torch.float32)
-    _chk(h_tilde, "h_tilde", torch.float32, (B, T, D))
+    if z.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("mingru_scan supports float32 and bfloat16")
+    _chk(z, "z", z.dtype)
+    _chk(h_tilde, "h_tilde", z.dtype, (B, T, D))
     _chk(h0, "h0", torch.float32, (B, D))
     _chk(P0, "P0", torch.float32, (B, D))
     done, dd = _done(done, B, T)
@@ -158,7 +162,7 @@ def mingru_scan_fwd(z, h_tilde, done, h0=None, P0=None, want_P=True):
     h_last = torch.empty((B, D), dtype=torch.float32, device=z.device)
     P_last = torch.empty((B, D), dtype=torch.float32, device=z.device) if want_P else None
     st = lib.mrx_mingru_scan_fwd(_stream(), _ptr(z), _ptr(h_tilde), _ptr(done), _ptr(h0), _ptr(P0), _ptr(h),
-                                 _ptr(h_last), _ptr(P_last), B, T, D, dd)
+                                 _ptr(h_last), _ptr(P_last), B, T, D, _DT[z.dtype], dd)
     _lib.check(st, "mrx_mingru_scan_fwd")
     return h, h_last, P_last
 
@@ -167,15 +171,17 @@ def mingru_scan_bwd(z, h_tilde, h, done, h0, g, g_last=None):
     """Returns (dz, dh_tilde, dh0) for the states h of mingru_scan_fwd and their gradients g."""
     lib = _lib.load()
     B, T, D = g.shape
+    if g.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("mingru_scan supports float32 and bfloat16")
     for t_, n_ in ((z, "z"), (h_tilde, "h_tilde"), (h, "h"), (g, "g")):
-        _chk(t_, n_, torch.float32, (B, T, D))
+        _chk(t_, n_, g.dtype, (B, T, D))
     _chk(h0, "h0", torch.float32, (B, D))
     _chk(g_last, "g_last", torch.float32, (B, D))
     done, dd = _done(done, B, T)
     dz, dx = torch.empty_like(g), torch.empty_like(g)
     dh0 = torch.empty((B, D), dtype=torch.float32, device=g.device)
     st = lib.mrx_mingru_scan_bwd(_stream(), _ptr(z), _ptr(h_tilde), _ptr(h), _ptr(done), _ptr(h0), _ptr(g),
-                                 _ptr(g_last), _ptr(dz), _ptr(dx), _ptr(dh0), B, T, D, dd)
+                                 _ptr(g_last), _ptr(dz), _ptr(dx), _ptr(dh0), B, T, D, _DT[g.dtype], dd)
     _lib.check(st, "mrx_mingru_scan_bwd")
     return dz, dx, dh0
 

@@ -259,7 +259,10 @@ class MinGRUCell(_DiagonalCell):
     def forward(self, x, **kwargs):
         z, h_tilde = self.z(x), self.h(x)
         self.intermediates["gate"] = z.mean().detach()   # min_gru.py:63 sows the mean gate
-        if self.fused:   # the recurrence runs in fp32 whatever the projections' dtype (autocast)
+        if self.fused:   # the recurrence runs in fp32 whatever the projections' dtype (autocast): the kernels
+            # read bfloat16 projections as they are (and write bfloat16 states); anything else goes in as float32
+            if z.dtype == torch.bfloat16 and h_tilde.dtype == torch.bfloat16:
+                return MinGRUProjections(z, h_tilde)
             return MinGRUProjections(z.float(), h_tilde.float())
         z, h_tilde = z.float(), h_tilde.float()
         a = torch.sigmoid(-z)

@@ -64,7 +64,9 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mrx_linear_scan_fwd(n, n, n, n, n, n, n, n, n, 1, 1, 1, 0, 0, 0) == -1
     one = ctypes.c_void_p(16)
     assert lib.mrx_linear_scan_fwd(n, one, one, one, n, n, one, n, n, 0, 4, 4, 0, 0, 0) == -1
-    assert lib.mrx_linear_scan_fwd(n, one, one, one, n, n, one, n, n, 2, 4, 4, 1, 0, 0) == -2  # bf16 scan
+    assert lib.mrx_linear_scan_last(n, one, one, one, n, one, 2, 4, 4, 1, 1, 0) == -2  # bf16 final-state scan
+    assert lib.mrx_mingru_scan_fwd(n, one, one, one, n, n, one, n, n, 2, 4, 4, 2, 0) == -2  # complex64 MinGRU
+    assert lib.mrx_linear_scan_fwd(n, one, one, one, n, n, one, n, n, 2, 4, 4, 7, 0, 0) == -1  # no such dtype
     assert lib.mrx_linear_attn_fwd(n, one, one, one, one, n, one, n, n, 1, 8, 1, 72, 64, 1, 0, 0) == -2  # dk > 64
     assert lib.mrx_linear_attn_fwd(n, one, one, one, one, n, one, n, n, 1, 8, 1, 36, 64, 1, 0, 0) == -2  # 36 bf16: 4.5 segments
     assert lib.mrx_delta_rule_fwd(n, one, one, one, one, one, n, one, n, n, n, 1, 8, 1, 64, 72, 1, 0, 0) == -2  # dv > 64

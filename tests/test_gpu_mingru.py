@@ -133,3 +133,61 @@ def test_mingru_cell_fused_and_unfused_agree_and_match_the_reference_route():
     assert relerr(gz, cell.z.weight.grad.cpu().numpy()) <= 1e-4 and relerr(gh, cell.h.weight.grad.cpu().numpy()) <= 1e-4
     nxt, rh = M.mingru_scan(cell.z(x).detach().cpu().numpy(), cell.h(x).detach().cpu().numpy(), done.float().cpu().numpy())
     assert relerr(y, rh) <= TOL and relerr(carry[0], nxt[0]) <= TOL and relerr(carry[1], nxt[1]) <= TOL
+
+
+@pytest.mark.parametrize("shape", [(2, 1, 5), (3, 77, 48), (4, 300, 258), (64, 128, 256), (16, 1000, 130), (512, 128, 64)])
+@pytest.mark.parametrize("p", [0.0, 0.05])
+def test_bfloat16_arrays_float32_arithmetic(shape, p):
+    """z, h~, h, g, dz, dh~ in bfloat16, arithmetic and carries in float32: against the oracle on the rounded
+    inputs, within the bf16-in / fp32-accumulate tolerance (the backward walks the stored, rounded states, as
+    the gradient of a function with a rounded output does)."""
+    from memorax_amd import kernels as K
+    from gpu_util import TOL_BF16, bf16_round
+    B, T, D = shape
+    rng = np.random.default_rng(B * 1000 + T * 10 + D + 1)
+    z = bf16_round((2 * rng.standard_normal(shape)).astype(np.float32))
+    x = bf16_round((2 * rng.standard_normal(shape)).astype(np.float32))
+    g = bf16_round(rng.standard_normal(shape).astype(np.float32))
+    h0 = np.exp(rng.standard_normal((B, D))).astype(np.float32)
+    P0 = rng.uniform(0.5, 1.0, (B, D)).astype(np.float32)
+    gl = rng.standard_normal((B, D)).astype(np.float32)
+    done = rng.random((B, T)) < p
+    print(f"case mingru bf16 shape={shape} p={p}", flush=True)
+    bf = torch.bfloat16
+    h, hl, Pl = K.mingru_scan_fwd(dev(z).to(bf), dev(x).to(bf), dev(done), dev(h0), dev(P0))
+    assert h.dtype == bf and hl.dtype == torch.float32 and Pl.dtype == torch.float32
+    rh, rhl, rPl = _ref(z, x, done, h0, P0)
+    assert relerr(h.float(), rh) <= TOL_BF16 and relerr(hl, rhl) <= 1e-4 and relerr(Pl, rPl) <= 1e-4
+    dz, dx, dh0 = K.mingru_scan_bwd(dev(z).to(bf), dev(x).to(bf), h, dev(done), dev(h0), dev(g).to(bf), dev(gl))
+    assert dz.dtype == bf and dx.dtype == bf and dh0.dtype == torch.float32
+    a, b = M.mingru_linear_coeffs(z, x)
+    hh, _, _ = M.diag_scan(a, b, done, h0)
+    da, lam, rdh0 = M.diag_scan_bwd(a, hh, done, g, h0, gl)
+    s = M.sigmoid(z.astype(np.float64))
+    x64 = x.astype(np.float64)
+    rdz = s * (1 - s) * (np.where(x64 >= 0, x64 + 0.5, M.sigmoid(x64)) * lam - da)
+    rdx = lam * s * np.where(x64 >= 0, 1.0, M.sigmoid(x64) * (1 - M.sigmoid(x64)))
+    assert relerr(dz.float(), rdz) <= TOL_BF16 and relerr(dx.float(), rdx) <= TOL_BF16 and relerr(dh0, rdh0) <= TOL_BF16
+
+
+def test_bfloat16_autograd_function_and_cell():
+    """functional.mingru_scan on bfloat16 projections (what a bf16 torso hands over): states in bfloat16, carries
+    and their gradients in float32, the projections' gradients in bfloat16."""
+    import memorax_amd as mx
+    from gpu_util import TOL_BF16
+    B, T, D = 4, 90, 64
+    rng = np.random.default_rng(11)
+    z = torch.from_numpy((2 * rng.standard_normal((B, T, D))).astype(np.float32)).cuda().bfloat16().requires_grad_()
+    x = torch.from_numpy((2 * rng.standard_normal((B, T, D))).astype(np.float32)).cuda().bfloat16().requires_grad_()
+    h0 = torch.from_numpy(np.exp(rng.standard_normal((B, D))).astype(np.float32)).cuda().requires_grad_()
+    done = torch.from_numpy(rng.random((B, T)) < 0.05).cuda()
+    h, hl, Pl = mx.mingru_scan(z, x, done, h0)
+    assert h.dtype == torch.bfloat16 and hl.dtype == torch.float32
+    (h.float().sum() + hl.sum()).backward()
+    assert z.grad.dtype == torch.bfloat16 and x.grad.dtype == torch.bfloat16 and h0.grad.dtype == torch.float32
+    zf, xf, h0f = (t.detach().float().requires_grad_() for t in (z, x, h0))
+    hf, hlf, _ = mx.mingru_scan(zf, xf, done, h0f)
+    (hf.sum() + hlf.sum()).backward()
+    assert relerr(h.float(), hf.detach().cpu().numpy()) <= TOL_BF16
+    for a, b in ((z.grad, zf.grad), (x.grad, xf.grad), (h0.grad, h0f.grad)):
+        assert relerr(a.float(), b.cpu().numpy()) <= TOL_BF16

@@ -184,3 +184,32 @@ def test_propagate_sensitivities(dtype, shape):
     for name in J:
         assert out[name].shape == S[name].shape
         assert relerr(out[name], ref[name]) <= 1e-4, (name, relerr(out[name], ref[name]))
+
+
+@pytest.mark.parametrize("shape", [(3, 77, 48), (2, 1, 5), (64, 128, 256), (4, 300, 1024), (512, 128, 64)])
+@pytest.mark.parametrize("ti", [False, True])
+def test_scan_bfloat16_arrays_float32_arithmetic(shape, ti):
+    """a, b, h, g, da, db in bfloat16; arithmetic, carries and a summed da in float32."""
+    from memorax_amd import kernels as K
+    B, T, D = shape
+    rng = np.random.default_rng(B + 3 * T + D)
+    rb = lambda x: torch.from_numpy(x.astype(np.float32)).bfloat16().float().numpy()  # round to bfloat16
+    a = rb(rng.uniform(0.8, 0.999, (D,) if ti else shape))
+    b, g = rb(rng.standard_normal(shape)), rb(rng.standard_normal(shape))
+    h0, gl = rng.standard_normal((B, D)).astype(np.float32), rng.standard_normal((B, D)).astype(np.float32)
+    P0 = rng.uniform(0.5, 1.0, (B, D)).astype(np.float32)
+    done = rng.random((B, T)) < 0.04
+    print(f"case scan bf16 shape={shape} ti={ti}", flush=True)
+    bf = torch.bfloat16
+    h, hl, Pl = K.linear_scan_fwd(dev(a).to(bf), dev(b).to(bf), dev(done), dev(h0), dev(P0))
+    assert h.dtype == bf and hl.dtype == torch.float32 and Pl.dtype == torch.float32
+    rh, rhl, rPl = M.diag_scan(a, b, done, h0, P0)
+    assert relerr(h.float(), rh) <= 2e-2 and relerr(hl, rhl) <= TOL and relerr(Pl, rPl) <= TOL
+    da, db, dh0 = K.linear_scan_bwd(dev(a).to(bf), h, dev(done), dev(h0), dev(g).to(bf), dev(gl), sum_da=ti)
+    ag = G.diag_scan_grads(np.broadcast_to(a, shape).copy(), b, done, h0, g, gl)
+    assert db.dtype == bf and dh0.dtype == torch.float32 and da.dtype == (torch.float32 if ti else bf)
+    assert relerr(db.float(), ag["db"]) <= 2e-2 and relerr(dh0, ag["dh0"]) <= 2e-2
+    if ti:
+        assert da.shape == (B, D) and relerr(da.sum(0), ag["da"].sum((0, 1))) <= 2e-2
+    else:
+        assert relerr(da.float(), ag["da"]) <= 2e-2
