@@ -171,7 +171,8 @@ diag_scan_fwd_kernel(const S *__restrict__ a, const S *__restrict__ b,
     for (int t0 = 0; t0 < T; t0 += span) {
         const int ts = t0 + w * TS;
         V x[TS], p[TS];
-        unsigned rmask = 0;
+        // reset flags of the wave's TS steps: lane s fetches the flag of step ts + s, one ballot makes the mask
+        const unsigned rmask = (unsigned)__ballot(lane < TS && ts + lane < T && done_at(done, done_f32, row0 + ts + lane));
 #pragma unroll
         for (int s = 0; s < TS; ++s) {
             const int t = ts + s;
@@ -183,7 +184,6 @@ diag_scan_fwd_kernel(const S *__restrict__ a, const S *__restrict__ b,
                 p[s] = vfill<E, VEC>(O::one());
                 x[s] = vfill<E, VEC>(O::zero());
             }
-            if (t < T && done_at(done, done_f32, row0 + t)) rmask |= 1u << s;
         }
         if constexpr (MG) {  // after every load of the super-step has been issued
 #pragma unroll
@@ -311,8 +311,18 @@ diag_scan_bwd_kernel(const S *__restrict__ a, const S *__restrict__ hx, const S 
         // barrier would be a second trip to memory on the critical path.
         V x[TS], p[TS], hp[TS];
         V zt[MG ? TS : 1], xt[MG ? TS : 1];
-        unsigned cmask = 0;  // bit s: chain cut between step t and t+1 (done_{t+1})
-        unsigned dmask = 0;  // bit s: done_t
+        // reset flags: step s of the wave is t_s = T - 1 - (rs + s); lane l fetches done at T - rs - l, i.e.
+        // done_{t_0 + 1}, done_{t_0}, done_{t_1}, ..., and one ballot serves both masks (steps before the
+        // sequence's first, t_s < 0, take no bit: a cut there would drop the carry on its way to dh0)
+        unsigned cmask, dmask;  // bit s: chain cut between step t_s and t_s + 1 (done_{t_s + 1}) / done_{t_s}
+        {
+            const int tt = T - rs - lane;
+            const unsigned fl = (unsigned)__ballot(lane <= TS && tt >= 0 && tt < T && done_at(done, done_f32, row0 + tt));
+            const int nv = T - rs < TS ? (T - rs < 0 ? 0 : T - rs) : TS;  // steps of the wave inside the sequence
+            const unsigned vm = (1u << nv) - 1u;
+            cmask = fl & vm;
+            dmask = (fl >> 1) & vm;
+        }
 #pragma unroll
         for (int s = 0; s < TS; ++s) {
             const int t = T - 1 - (rs + s);
@@ -337,8 +347,6 @@ diag_scan_bwd_kernel(const S *__restrict__ a, const S *__restrict__ hx, const S 
                         xt[s] = ldv<S, E, VEC>(hx + off);
                     }
                 }
-                if (t + 1 < T && done_at(done, done_f32, row0 + t + 1)) cmask |= 1u << s;
-                if (done_at(done, done_f32, row0 + t)) dmask |= 1u << s;
             }
         }
         if constexpr (MG) {  // a_{t+1} = sigma(-z_{t+1}), after every load of the super-step has been issued
