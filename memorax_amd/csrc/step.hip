@@ -84,11 +84,15 @@ step_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restric
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
         const int row = r0 + RPP * p;
-        s[p] = (Sp && !reset && cin && (!NARROW || row < dvw)) ? *reinterpret_cast<const f32x4 *>(Sp + row * dkw + 4 * c4) * decay : zero4;
+        // the carried state is loaded whether or not the flag says reset, and dropped by select below: a load
+        // that waits for the flag would be a second trip to memory behind the first
+        s[p] = (Sp && cin && (!NARROW || row < dvw)) ? *reinterpret_cast<const f32x4 *>(Sp + row * dkw + 4 * c4) : zero4;
     }
     float u[NP];
 #pragma unroll
     for (int p = 0; p < NP; ++p) u[p] = (!NARROW || r0 + RPP * p < dvw) ? (float)vp[r0 + RPP * p] : 0.f;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) s[p] = reset ? zero4 : s[p] * decay;
     if (DELTA) {
         const float bb = (float)beta[bh];
 #pragma unroll
@@ -97,7 +101,8 @@ step_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restric
     float den = 1.f;
     if (!DELTA && z_out) {
         // every row's lanes recompute the normaliser of the sequence; row 0 stores it
-        f32x4 z4 = (z_in && !reset && cin) ? *reinterpret_cast<const f32x4 *>(z_in + bh * dkw + 4 * c4) : zero4;
+        f32x4 z4 = (z_in && cin) ? *reinterpret_cast<const f32x4 *>(z_in + bh * dkw + 4 * c4) : zero4;
+        if (reset) z4 = zero4;
         z4 += k4;
         if (r0 == 0 && cin) *reinterpret_cast<f32x4 *>(z_out + bh * dkw + 4 * c4) = z4;
         den = fmaxf(reduce_row(dot4(z4, q4)), eps);
