@@ -72,6 +72,47 @@ template <typename S, typename E, int VEC> __device__ __forceinline__ Vec<E, VEC
         return r;
     }
 }
+// The same in two steps, for prefetched values: the load leaves the stored bits in registers and the conversion
+// runs where the value is consumed -- arithmetic on a load still in flight makes the wave wait for it, and for
+// every load issued before it, in the middle of issuing a group of loads.
+// bfloat16 values wait as whole 32-bit words (a structure of 16-bit members would be taken apart, i.e. computed
+// on, the moment it arrives); a single one is widened by its load instruction.
+template <typename S, int VEC> struct RawVec {
+    using type = Vec<S, VEC>;
+};
+template <int VEC> struct alignas(VEC >= 2 ? 2 * VEC : 4) RawBf16 {
+    uint32_t w[VEC >= 2 ? VEC / 2 : 1];
+};
+template <int VEC> struct RawVec<__bf16, VEC> {
+    using type = RawBf16<VEC>;
+};
+template <typename S, int VEC> using raw_t = typename RawVec<S, VEC>::type;
+
+template <typename S, int VEC> __device__ __forceinline__ raw_t<S, VEC> ldraw(const S *p)
+{
+    if constexpr (std::is_same<S, __bf16>::value && VEC == 1) {
+        raw_t<S, VEC> r;
+        r.w[0] = *reinterpret_cast<const uint16_t *>(p);
+        return r;
+    } else {
+        return *reinterpret_cast<const raw_t<S, VEC> *>(p);
+    }
+}
+template <typename S, typename E, int VEC> __device__ __forceinline__ Vec<E, VEC> cvtv(const raw_t<S, VEC> &raw)
+{
+    if constexpr (std::is_same<S, E>::value) {
+        return raw;
+    } else {
+        static_assert(std::is_same<S, __bf16>::value && std::is_same<E, float>::value, "bfloat16 storage, float arithmetic");
+        Vec<E, VEC> r;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            const uint32_t word = raw.w[i >> 1];
+            r.v[i] = __builtin_bit_cast(float, (VEC == 1 || !(i & 1)) ? word << 16 : word & 0xffff0000u);
+        }
+        return r;
+    }
+}
 template <typename S, typename E, int VEC> __device__ __forceinline__ void stv(S *p, const Vec<E, VEC> &x)
 {
     if constexpr (std::is_same<S, E>::value) {
@@ -173,13 +214,21 @@ diag_scan_fwd_kernel(const S *__restrict__ a, const S *__restrict__ b,
         V x[TS], p[TS];
         // reset flags of the wave's TS steps: lane s fetches the flag of step ts + s, one ballot makes the mask
         const unsigned rmask = (unsigned)__ballot(lane < TS && ts + lane < T && done_at(done, done_f32, row0 + ts + lane));
+        raw_t<S, VEC> rp[TS], rx[TS];  // as stored; converted once every load of the super-step has been issued
 #pragma unroll
         for (int s = 0; s < TS; ++s) {
             const int t = ts + s;
             if (t < T && act) {
                 const int64_t off = (row0 + t) * D + col;
-                p[s] = ldv<S, E, VEC>(a + (a_ti ? col : off));
-                x[s] = ldv<S, E, VEC>(b + off);
+                rp[s] = ldraw<S, VEC>(a + (a_ti ? col : off));
+                rx[s] = ldraw<S, VEC>(b + off);
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < TS; ++s) {
+            if (ts + s < T && act) {
+                p[s] = cvtv<S, E, VEC>(rp[s]);
+                x[s] = cvtv<S, E, VEC>(rx[s]);
             } else {
                 p[s] = vfill<E, VEC>(O::one());
                 x[s] = vfill<E, VEC>(O::zero());
@@ -323,14 +372,14 @@ diag_scan_bwd_kernel(const S *__restrict__ a, const S *__restrict__ hx, const S 
             cmask = fl & vm;
             dmask = (fl >> 1) & vm;
         }
+        if constexpr (std::is_same<S, E>::value) {
 #pragma unroll
-        for (int s = 0; s < TS; ++s) {
-            const int t = T - 1 - (rs + s);
-            p[s] = vfill<E, VEC>(O::one());
-            x[s] = vfill<E, VEC>(O::zero());
-            hp[s] = vfill<E, VEC>(O::zero());
-            if (t >= 0) {
-                if (act) {
+            for (int s = 0; s < TS; ++s) {
+                const int t = T - 1 - (rs + s);
+                p[s] = vfill<E, VEC>(O::one());
+                x[s] = vfill<E, VEC>(O::zero());
+                hp[s] = vfill<E, VEC>(O::zero());
+                if (t >= 0 && act) {
                     const int64_t off = (row0 + t) * D + col;
                     x[s] = ldv<S, E, VEC>(g + off);
                     if (t + 1 < T) {
@@ -345,6 +394,46 @@ diag_scan_bwd_kernel(const S *__restrict__ a, const S *__restrict__ hx, const S 
                     if constexpr (MG) {
                         zt[s] = ldv<S, E, VEC>(a + off);
                         xt[s] = ldv<S, E, VEC>(hx + off);
+                    }
+                }
+            }
+        } else {
+            // narrower storage: the values wait as stored and are widened once every load has been issued
+            raw_t<S, VEC> rg[TS], ra[TS], rh[TS], rz[MG ? TS : 1], rxt[MG ? TS : 1];
+            V h0v = vfill<E, VEC>(O::zero());  // h_{-1}: what step 0 multiplies its lam with
+            if (act && h0 && T - 1 - rs - (TS - 1) <= 0) h0v = *reinterpret_cast<const V *>(h0 + bi * D + col);
+#pragma unroll
+            for (int s = 0; s < TS; ++s) {
+                const int t = T - 1 - (rs + s);
+                if (t >= 0 && act) {
+                    const int64_t off = (row0 + t) * D + col;
+                    rg[s] = ldraw<S, VEC>(g + off);
+                    if (t + 1 < T) ra[s] = ldraw<S, VEC>(a + (a_ti ? col : off + D));
+                    if (t > 0) rh[s] = ldraw<S, VEC>(hfw + off - D);
+                    if constexpr (MG) {
+                        rz[s] = ldraw<S, VEC>(a + off);
+                        rxt[s] = ldraw<S, VEC>(hx + off);
+                    }
+                }
+            }
+#pragma unroll
+            for (int s = 0; s < TS; ++s) {
+                const int t = T - 1 - (rs + s);
+                p[s] = vfill<E, VEC>(O::one());
+                x[s] = vfill<E, VEC>(O::zero());
+                hp[s] = vfill<E, VEC>(O::zero());
+                if (t >= 0 && act) {
+                    x[s] = cvtv<S, E, VEC>(rg[s]);
+                    if (t + 1 < T) {
+                        const V av = cvtv<S, E, VEC>(ra[s]);
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) p[s].v[i] = MG ? av.v[i] : O::conj(av.v[i]);  // MG: z_{t+1} for now
+                    }
+                    if (t > 0) hp[s] = cvtv<S, E, VEC>(rh[s]);
+                    else hp[s] = h0v;
+                    if constexpr (MG) {
+                        zt[s] = cvtv<S, E, VEC>(rz[s]);
+                        xt[s] = cvtv<S, E, VEC>(rxt[s]);
                     }
                 }
             }
@@ -490,16 +579,19 @@ diag_scan_bwd_kernel(const S *__restrict__ a, const S *__restrict__ hx, const S 
 // with the loads of the next group issued before the current group is consumed
 // (register double buffering), so a wave always has 2*SG (forward) / 3*SG (backward)
 // row loads in flight.  done flags are prefetched as raw bits with the data.
-template <typename E, int VEC, int SG, bool MG = false, typename S = E>
+template <typename E, int VEC, int SG, bool MG = false, typename S = E, bool DF = false>
 __global__ void __launch_bounds__(256)
 diag_scan_fwd_stream_kernel(const S *__restrict__ a, const S *__restrict__ b,
-                            const void *__restrict__ done, int done_f32,
+                            const void *__restrict__ done, int,
                             const E *__restrict__ h0, const E *__restrict__ P0,
                             S *__restrict__ h, E *__restrict__ h_last, E *__restrict__ P_last,
                             int64_t B, int T, int64_t D, int64_t cols_per_row, int a_ti)
 {
     using V = Vec<E, VEC>;
     using O = Ops<E>;
+    // the flags' type is a template parameter here: with both kinds of load in the code the compiler reuses
+    // registers of loads still in flight for the other kind's address and waits for them in mid-prefetch
+    constexpr int done_f32 = DF;
     // one thread per VEC channels of one batch row
     const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t bi = gid / cols_per_row;
@@ -510,17 +602,18 @@ diag_scan_fwd_stream_kernel(const S *__restrict__ a, const S *__restrict__ b,
     if (h0) ch = *reinterpret_cast<const V *>(h0 + bi * D + col);
     if (P0) cp = *reinterpret_cast<const V *>(P0 + bi * D + col);
 
-    V xa[SG], xb[SG], na[SG], nb[SG];
+    using R = raw_t<S, VEC>;  // prefetched values stay as stored until they are consumed
+    R xa[SG], xb[SG], na[SG], nb[SG];
     uint32_t xd[SG], nd[SG];
-    auto load = [&](int t0, V *pa, V *pb, uint32_t *pd) {
+    auto load = [&](int t0, R *pa, R *pb, uint32_t *pd) {
 #pragma unroll
         for (int s = 0; s < SG; ++s) {
             const int t = t0 + s;
             pd[s] = 0u;
             if (t < T) {
                 const int64_t off = (row0 + t) * D + col;
-                pa[s] = ldv<S, E, VEC>(a + (a_ti ? col : off));
-                pb[s] = ldv<S, E, VEC>(b + off);
+                pa[s] = ldraw<S, VEC>(a + (a_ti ? col : off));
+                pb[s] = ldraw<S, VEC>(b + off);
                 pd[s] = done_raw(done, done_f32, row0 + t);
             }
         }
@@ -532,16 +625,17 @@ diag_scan_fwd_stream_kernel(const S *__restrict__ a, const S *__restrict__ b,
         for (int s = 0; s < SG; ++s) {
             if (t0 + s < T) {
                 const bool r = done_test(xd[s], done_f32);
+                V va = cvtv<S, E, VEC>(xa[s]), vb = cvtv<S, E, VEC>(xb[s]);
                 if constexpr (MG) {  // here, not at the load: the loads stay in flight
 #pragma unroll
-                    for (int i = 0; i < VEC; ++i) MinGru::coeffs(xa[s].v[i], xb[s].v[i]);
+                    for (int i = 0; i < VEC; ++i) MinGru::coeffs(va.v[i], vb.v[i]);
                 }
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) {
-                    const E hn = O::madd(xa[s].v[i], ch.v[i], xb[s].v[i]);
-                    const E pn = O::mul(xa[s].v[i], cp.v[i]);
-                    ch.v[i] = r ? xb[s].v[i] : hn;
-                    cp.v[i] = r ? xa[s].v[i] : pn;
+                    const E hn = O::madd(va.v[i], ch.v[i], vb.v[i]);
+                    const E pn = O::mul(va.v[i], cp.v[i]);
+                    ch.v[i] = r ? vb.v[i] : hn;
+                    cp.v[i] = r ? va.v[i] : pn;
                 }
                 stv<S, E, VEC>(h + (row0 + t0 + s) * D + col, ch);
             }
@@ -611,10 +705,10 @@ diag_scan_last_kernel(const E *__restrict__ a, const E *__restrict__ b, const vo
 }
 
 // MG: a holds z, hx holds x = h~ (a fourth load per step); da receives dz and db receives dx.
-template <typename E, int VEC, int SG, bool MG = false, typename S = E>
+template <typename E, int VEC, int SG, bool MG = false, typename S = E, bool DF = false>
 __global__ void __launch_bounds__(256)
 diag_scan_bwd_stream_kernel(const S *__restrict__ a, const S *__restrict__ hx, const S *__restrict__ hfw,
-                            const void *__restrict__ done, int done_f32,
+                            const void *__restrict__ done, int,
                             const E *__restrict__ h0, const S *__restrict__ g,
                             const E *__restrict__ g_last, S *__restrict__ da, S *__restrict__ db,
                             E *__restrict__ dh0, int64_t B, int T, int64_t D, int64_t cols_per_row, int a_ti,
@@ -622,6 +716,9 @@ diag_scan_bwd_stream_kernel(const S *__restrict__ a, const S *__restrict__ hx, c
 {
     using V = Vec<E, VEC>;
     using O = Ops<E>;
+    // the flags' type is a template parameter here: with both kinds of load in the code the compiler reuses
+    // registers of loads still in flight for the other kind's address and waits for them in mid-prefetch
+    constexpr int done_f32 = DF;
     const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t bi = gid / cols_per_row;
     const int64_t col = (gid % cols_per_row) * VEC;
@@ -632,22 +729,23 @@ diag_scan_bwd_stream_kernel(const S *__restrict__ a, const S *__restrict__ hx, c
     if (g_last) lam = *reinterpret_cast<const V *>(g_last + bi * D + col);
 
     // step r (reversed index), t = T-1-r: needs g_t, a_t (for the carry to t-1), h_{t-1}, done_t
-    V xg[SG], xa[SG], xh[SG], ng[SG], na[SG], nh[SG];
-    V xx[MG ? SG : 1], nx[MG ? SG : 1];
+    using R = raw_t<S, VEC>;  // prefetched values stay as stored until they are consumed
+    R xg[SG], xa[SG], xh[SG], ng[SG], na[SG], nh[SG];
+    R xx[MG ? SG : 1], nx[MG ? SG : 1];
     uint32_t xd[SG], nd[SG];
-    auto load = [&](int r0, V *pg, V *pa, V *ph, V *px, uint32_t *pd) {
+    V h0v = vfill<E, VEC>(O::zero());  // h_{-1}: what step 0 multiplies its lam with
+    if (h0) h0v = *reinterpret_cast<const V *>(h0 + bi * D + col);
+    auto load = [&](int r0, R *pg, R *pa, R *ph, R *px, uint32_t *pd) {
 #pragma unroll
         for (int s = 0; s < SG; ++s) {
             const int t = T - 1 - (r0 + s);
             pd[s] = 0u;
-            ph[s] = vfill<E, VEC>(O::zero());
             if (t >= 0) {
                 const int64_t off = (row0 + t) * D + col;
-                pg[s] = ldv<S, E, VEC>(g + off);
-                pa[s] = ldv<S, E, VEC>(a + (a_ti ? col : off));
-                if constexpr (MG) px[s] = ldv<S, E, VEC>(hx + off);
-                if (t > 0) ph[s] = ldv<S, E, VEC>(hfw + off - D);
-                else if (h0) ph[s] = *reinterpret_cast<const V *>(h0 + bi * D + col);
+                pg[s] = ldraw<S, VEC>(g + off);
+                pa[s] = ldraw<S, VEC>(a + (a_ti ? col : off));
+                if constexpr (MG) px[s] = ldraw<S, VEC>(hx + off);
+                if (t > 0) ph[s] = ldraw<S, VEC>(hfw + off - D);
                 pd[s] = done_raw(done, done_f32, row0 + t);
             }
         }
@@ -661,21 +759,25 @@ diag_scan_bwd_stream_kernel(const S *__restrict__ a, const S *__restrict__ hx, c
             if (t >= 0) {
                 const bool dn = done_test(xd[s], done_f32);
                 const int64_t off = (row0 + t) * D + col;
+                const V vg = cvtv<S, E, VEC>(xg[s]), va = cvtv<S, E, VEC>(xa[s]);
+                V vh = h0v, vx;
+                if (t > 0) vh = cvtv<S, E, VEC>(xh[s]);
+                if constexpr (MG) vx = cvtv<S, E, VEC>(xx[s]);
                 V l, o;
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) {
-                    l.v[i] = O::madd(O::one(), xg[s].v[i], lam.v[i]);  // lam_t = g_t + carried term
-                    const E prod = O::mul(l.v[i], O::conj(xh[s].v[i]));
+                    l.v[i] = O::madd(O::one(), vg.v[i], lam.v[i]);  // lam_t = g_t + carried term
+                    const E prod = O::mul(l.v[i], O::conj(vh.v[i]));
                     o.v[i] = dn ? O::zero() : prod;
                     if constexpr (MG) {
                         float sg, at, dz, dx;
-                        MinGru::gates(xa[s].v[i], sg, at);
-                        MinGru::grads(xa[s].v[i], xx[s].v[i], l.v[i], o.v[i], dz, dx);
+                        MinGru::gates(va.v[i], sg, at);
+                        MinGru::grads(va.v[i], vx.v[i], l.v[i], o.v[i], dz, dx);
                         lam.v[i] = dn ? 0.0f : at * l.v[i];
                         o.v[i] = dz;
                         l.v[i] = dx;
                     } else {
-                        const E nxt = O::mul(O::conj(xa[s].v[i]), l.v[i]);
+                        const E nxt = O::mul(O::conj(va.v[i]), l.v[i]);
                         lam.v[i] = dn ? O::zero() : nxt;           // conj(abar_t) lam_t for step t-1
                     }
                 }
@@ -750,18 +852,14 @@ ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, boo
         // so few columns that eight waves along time leave most of the device idle: sixteen of one lane each
         if (T >= 16 * TS && cols(1) <= 256) return split(1, 16);
         if (half_storage) {
+            // (swept again once the bfloat16 values waited as stored bits: the wave-split kernels then lead
+            // forward at every size; four elements per lane, backward, do not fit the wave-split kernel's
+            // registers)
+            const int v = vec < 2 ? vec : 2;
+            if (!bwd) return split(v, cols(v) >= 1024 && nw8 > 4 ? 4 : nw8);
             // the streaming kernels lay their threads flat over (row, column): a row need not fill whole waves
-            const bool flat4 = D % 4 == 0 && al16;
-            const int64_t waves4 = flat4 ? B * D / 256 : 0;
-            if (waves4 >= (bwd ? 1024 : 2048)) return {4, 1, (int)ntiles(4), true};
-            if (!bwd) {
-                const int v = vec < 2 ? vec : 2;
-                return split(v, cols(v) >= 2048 && nw8 > 4 ? 4 : nw8);
-            }
-            if (vec < 4) return split(1, nw8);
-            int v = 4;
-            while (v > 1 && cols(v) < 256) v >>= 1;
-            return split(v, nw8);
+            if (D % 2 == 0 && al8 && B * D / 128 >= 2048) return {2, 1, (int)ntiles(2), true};
+            return split(v, cols(v) >= 512 && nw8 > 4 ? 4 : nw8);
         }
         if (esize == 8 && !mg) {
             if (!bwd && T <= 256) return split(1, nw8);
@@ -874,9 +972,13 @@ int launch_fwd(hipStream_t st, const void *a, const void *b, const void *done,
         const dim3 grid((unsigned)((B * cpr + 255) / 256)), block(256);
         vec_switch<E>(pl.vec, [&](auto vc) {
             constexpr int VEC = decltype(vc)::value;
-            rc = launch_kernel((diag_scan_fwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8), MG, S>), grid, block, 0, st,
-                               (const S *)a, (const S *)b, done, done_f32, (const E *)h0, (const E *)P0,
-                               (S *)h, (E *)h_last, (E *)P_last, B, (int)T, D, cpr, a_ti);
+            auto go = [&](auto df) {
+                rc = launch_kernel((diag_scan_fwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8), MG, S, decltype(df)::value>),
+                                   grid, block, 0, st, (const S *)a, (const S *)b, done, done_f32, (const E *)h0,
+                                   (const E *)P0, (S *)h, (E *)h_last, (E *)P_last, B, (int)T, D, cpr, a_ti);
+            };
+            if (done_f32) go(std::true_type{});
+            else go(std::false_type{});
         });
     } else {
         const dim3 grid((unsigned)(B * pl.tiles)), block(64 * pl.nw);
@@ -916,9 +1018,14 @@ int launch_bwd(hipStream_t st, const void *a, const void *hx, const void *h, con
         const dim3 grid((unsigned)((B * cpr + 255) / 256)), block(256);
         vec_switch<E>(pl.vec, [&](auto vc) {
             constexpr int VEC = decltype(vc)::value;
-            rc = launch_kernel((diag_scan_bwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8), MG, S>), grid, block, 0, st,
-                               (const S *)a, (const S *)hx, (const S *)h, done, done_f32, (const E *)h0, (const S *)g,
-                               (const E *)g_last, (S *)da, (S *)db, (E *)dh0, B, (int)T, D, cpr, a_ti, da_sum);
+            auto go = [&](auto df) {
+                rc = launch_kernel((diag_scan_bwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8), MG, S, decltype(df)::value>),
+                                   grid, block, 0, st, (const S *)a, (const S *)hx, (const S *)h, done, done_f32,
+                                   (const E *)h0, (const S *)g, (const E *)g_last, (S *)da, (S *)db, (E *)dh0, B, (int)T, D,
+                                   cpr, a_ti, da_sum);
+            };
+            if (done_f32) go(std::true_type{});
+            else go(std::false_type{});
         });
     } else {
         const dim3 grid((unsigned)(B * pl.tiles)), block(64 * pl.nw);
