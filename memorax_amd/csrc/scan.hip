@@ -806,7 +806,11 @@ struct ScanPlan {
     bool stream;  // streaming kernel (no time split) instead of the wave-split kernel
 };
 
-// Tuned on MI355X (fp32; 512x1024x1024, 1024x128x256, 64x512x512, 32x128x256):
+// Which kernel, how many elements per lane and how many waves along time.  Two layers of rules: the first
+// block in the function body (sequences of 32 steps and more) comes from one sweep over every plan and
+// takes precedence; what follows it are the earlier rules, which still decide the cases that block leaves
+// open and all shorter sequences.  The earlier rules, as they were derived
+// (fp32; 512x1024x1024, 1024x128x256, 64x512x512, 32x128x256):
 //  - widest vector the shapes/alignments allow, narrowed until there are >= 2048 wave columns;
 //  - forward: split time over up to 8 waves until ~8192 waves exist (the wave-split kernel at
 //    4 waves reached 5.7 TB/s on the 6.4 GB shape, the streaming kernel 5.1 TB/s); with no
