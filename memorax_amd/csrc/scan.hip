@@ -867,7 +867,7 @@ ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, boo
         }
         if (esize == 8 && !mg) {
             if (!bwd && T <= 256) return split(1, nw8);
-            if (bwd && vec == 2 && cols(2) >= 1024) return split(2, nw8);
+            if (bwd && vec == 2 && (cols(2) >= 1024 || (cols(2) >= 256 && T >= 64 * TS))) return split(2, nw8);
         }
         if (esize == 4) {
             if (!bwd) {
