@@ -521,7 +521,10 @@ def bench_torso_kernels(torch, K):
     by = 4 * ((BYTES_FWD + BYTES_BWD) * B * T * H + 36 * B * T * Fe)   # + MinGRU scan: 12 B fwd, 24 B bwd per element
     return {"sequence_kernels_ms": ms_k, "sequence_kernels_tokens/s": B * T / ms_k * 1e3,
             "sequence_kernels_GB/s": by / ms_k / 1e6, "sequence_kernels_frac_hbm": by / ms_k / 1e6 / HBM_PEAK_GBS,
-            "sequence_kernels_ms_plain_delta_rule": ms_p, "sequence_kernels_ms_bf16_recurrence_arrays": ms_h}
+            "sequence_kernels_ms_plain_delta_rule": ms_p, "sequence_kernels_ms_bf16_recurrence_arrays": ms_h,
+            "sequence_kernels_tokens/s_bf16_recurrence_arrays": B * T / ms_h * 1e3,
+            "sequence_kernels_frac_hbm_bf16_recurrence_arrays":
+                4 * ((BYTES_FWD + BYTES_BWD) * B * T * H + 18 * B * T * Fe) / ms_h / 1e6 / HBM_PEAK_GBS}
 
 
 def bench_torso_full(torch, K):
