@@ -86,6 +86,9 @@ def main() -> int:
     ap.add_argument("--lib", default=None,
                     help="path of another build of the library to load (bench.py --all times the build with "
                          "64-step delta-rule chunks through this, in a child process)")
+    ap.add_argument("--phase-clocks", action="store_true",
+                    help="with --lib <the measurement build>: run the headline backward and print the share of "
+                         "a wave's cycles spent inside matrix products (child process of the default run)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain elementwise kernel of known size (256 MiB read, 256 MiB "
                          "written) so that a rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE run can be scaled")
@@ -108,8 +111,12 @@ def main() -> int:
     K.init()
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()  # noqa: E731
 
+    if args.phase_clocks:
+        print(json.dumps(phase_clocks_child(np, torch, K, dev)))
+        return 0
     secondary = {}
     if not args.headline_only:
+        secondary["hbm_copy"] = bench_copy(torch)
         secondary["scan"] = bench_scan(torch, K)
         secondary["linear_attention"] = bench_linear_attention(torch, K, np, dev)
         secondary["torso"] = bench_torso_kernels(torch, K)
@@ -117,7 +124,7 @@ def main() -> int:
             secondary["torso"].update(bench_torso_full(torch, K))
             secondary["step"] = bench_step(torch, K)
             secondary["rtrl"] = bench_rtrl(torch, K)
-            secondary["delta_rule_chunk64"] = bench_delta_chunk64()
+        secondary["delta_rule_chunk64"] = bench_delta_chunk64()
         torch.cuda.empty_cache()
     if args.calibrate:
         cx = torch.zeros(64 * 1024 * 1024, device="cuda")  # 256 MiB fp32
@@ -218,11 +225,93 @@ def main() -> int:
                         "frac_mfma": mfma(fl_f + fl_b, tf_ms + tb_ms)},
         },
     }
+    if not args.headline_only:
+        out["roofline"].update(bench_gemm_phase(MFMA_BUSY_BWD))
+        if "hbm_copy" in secondary:
+            out["roofline"]["hbm_copy_GB/s"] = secondary["hbm_copy"]["GB/s"]
+            out["roofline"]["frac_of_copy_rate"] = bwd_gbs / secondary["hbm_copy"]["GB/s"]
     out.update(secondary)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(np, x, do_np)
     print(json.dumps(out))
     return 0
+
+
+def bench_copy(torch):
+    """What a plain streaming kernel reaches on this device: c = a + b over three float32 arrays of 512 MiB
+    (two reads, one write, 1.6 GB per launch, far beyond the 256 MB last-level cache) -- the practical
+    ceiling the HBM fractions of the bandwidth-bound kernels are to be read against."""
+    n = 128 * 1024 * 1024
+    a = torch.ones(n, device="cuda")
+    b = torch.ones(n, device="cuda")
+    c = torch.empty_like(a)
+    ms = _time_ms(torch, lambda: torch.add(a, b, out=c), iters=20, warm=5)
+    del a, b, c
+    return {"ms": ms, "bytes": 12 * n, "GB/s": 12 * n / ms / 1e6, "frac_hbm_peak": 12 * n / ms / 1e6 / HBM_PEAK_GBS,
+            "kernel": "torch.add(a, b, out=c), 3 x 512 MiB float32"}
+
+
+MFMA_CYCLES_16x16x32_BF16 = 16   # 16 384 flop at the SIMD's peak of 1 024 flop per cycle (2.5 PFLOP/s / 1 024 SIMDs / 2.4 GHz)
+MFMAS_PER_PASS_BWD = 48          # delta_bwd_kernel, bf16, 32-step chunks: MFMA instructions per wave and pass
+
+
+def phase_clocks_child(np, torch, K, dev):
+    """Runs in a child process on the measurement build (build.sh: MRX_PHASE_CLOCKS): the headline backward
+    with every matrix product bracketed by shader-clock reads; returns the clock totals."""
+    import ctypes
+    from memorax_amd import _lib
+    lib = _lib.load()
+    lib.mrx_phase_clocks.argtypes = [ctypes.POINTER(ctypes.c_ulonglong), ctypes.c_int]
+    lib.mrx_phase_clocks.restype = ctypes.c_int
+    bf = torch.bfloat16
+    B, T, H, d = 64, 1024, 8, 64
+    x = synthetic(np, 4, (B, T, H, d))
+    do_np = np.random.default_rng(2004).standard_normal((B, T, H, d)).astype(np.float32)
+    q, k, v, beta, do = (dev(a).to(bf) for a in (x["q"], x["k"], x["v"], x["beta"], do_np))
+    done = dev(x["done"])
+    o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done)
+    out = K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False)
+    for _ in range(20):
+        K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, out=out)
+    buf = (ctypes.c_ulonglong * 4)()
+    assert lib.mrx_phase_clocks(buf, 1) == 0
+    n = 20
+    for _ in range(n):
+        K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, out=out)
+    assert lib.mrx_phase_clocks(buf, 1) == 0
+    C = K.chunk_size(bf, delta=True)
+    dn = x["done"].reshape(B, T // C, C)
+    passes = float((1 + dn.sum(-1)).sum()) / B   # per sequence (every head of a batch row shares the resets)
+    return {"product_clocks": int(buf[0]), "wave_clocks": int(buf[1]), "workgroups": int(buf[2]), "launches": n,
+            "passes_per_sequence": passes}
+
+
+def bench_gemm_phase(mfma_busy):
+    """MFMA utilisation inside the product phases of delta_bwd_kernel.  The measurement build brackets every
+    matrix product of the kernel -- from before its first operand fragment is requested from LDS until its
+    accumulators are in hand -- with reads of the shader clock; product_phase_share is the share of a wave's
+    lifetime spent inside those brackets.  mfma_gemm_phase_frac is the rate at which a wave keeps its SIMD's
+    matrix pipe busy while inside them: MFMAs per wave (48 per pass) x 16 cycles each / bracketed cycles per wave.
+    Two waves share a SIMD at the headline shape, so the pipe's own utilisation while either is in a product
+    lies between this figure and twice it; mfma_busy / product_phase_share (the whole-kernel busy counter spread
+    over the product phases only) is reported beside it."""
+    import subprocess
+    lib = os.path.join(ROOT, "memorax_amd", "csrc", "libmemorax_amd_clk.so")
+    if not os.path.exists(lib):
+        return {"mfma_gemm_phase_frac": None, "mfma_gemm_phase_note": "libmemorax_amd_clk.so not built"}
+    r = subprocess.run([sys.executable, os.path.abspath(__file__), "--lib", lib, "--phase-clocks"],
+                       capture_output=True, text=True, timeout=300)
+    if r.returncode != 0:
+        return {"mfma_gemm_phase_frac": None, "mfma_gemm_phase_note": r.stderr[-300:]}
+    d = json.loads(r.stdout.strip().splitlines()[-1])
+    waves = 4 * d["workgroups"]
+    prod_per_wave = d["product_clocks"] / waves
+    share = d["product_clocks"] / d["wave_clocks"]
+    mfma_cycles = MFMAS_PER_PASS_BWD * d["passes_per_sequence"] * MFMA_CYCLES_16x16x32_BF16
+    return {"mfma_gemm_phase_frac": mfma_cycles / prod_per_wave, "product_phase_share": share,
+            "mfma_busy_over_product_phase_share": mfma_busy / share,
+            "mfma_gemm_phase_method": "shader-clock brackets around every product in the measurement build "
+                                      "(libmemorax_amd_clk.so), 20 launches; per wave: 48 MFMAs/pass x 16 cycles / bracketed cycles"}
 
 
 def bench_delta_chunk64():
@@ -289,12 +378,19 @@ def bench_scan(torch, K):
     Configuration 1 moves 12.6 MB per call: its kernels are timed back to back inside a HIP graph
     (the per-call host cost from Python is larger than the kernel), the larger shapes call by call."""
     res = {}
+    import numpy as np
     for name, shape in (("cfg1_32x128x256", (32, 128, 256)), ("torso_1024x128x256", (1024, 128, 256)),
                         ("sweep_512x1024x1024", (512, 1024, 1024))):
         Bn, Tn, Dn = shape
-        a = torch.rand(shape, device="cuda") * 0.099 + 0.9
-        b = torch.randn(shape, device="cuda")
-        dn = torch.rand((Bn, Tn), device="cuda") < 0.01
+        if name.startswith("cfg1"):  # the configuration's own seeded inputs: a ~ U(0.9, 0.999), b ~ N(0, 1), resets p = 0.01
+            rng = np.random.default_rng(1001)
+            a = torch.from_numpy(rng.uniform(0.9, 0.999, shape).astype(np.float32)).cuda()
+            b = torch.from_numpy(rng.standard_normal(shape).astype(np.float32)).cuda()
+            dn = torch.from_numpy(rng.random((Bn, Tn)) < 0.01).cuda()
+        else:                        # same distributions, drawn on the device (6.4 GB for the sweep shape)
+            a = torch.rand(shape, device="cuda") * 0.099 + 0.9
+            b = torch.randn(shape, device="cuda")
+            dn = torch.rand((Bn, Tn), device="cuda") < 0.01
         small = 12 * Bn * Tn * Dn < 256e6
         timer = _graph_time_ms if small else (lambda t_, f_: _time_ms(t_, f_, iters=10))
         ms = timer(torch, lambda: K.linear_scan_fwd(a, b, dn, want_P=False))

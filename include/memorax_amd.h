@@ -198,21 +198,28 @@ int mrx_linear_attn_chunk_parallel_pays(int64_t B, int64_t T, int64_t H, int dty
  *     o_t = S_t phi(q_t) / den_t
  * z0 (nullable = 0), z_last (nullable): (B,H,dk) fp32.  den: (B,H,T) fp32 (contiguous in time per
  * sequence: a residual, written and read back a chunk at a time), the clamped denominators, and
- * z_chk (nullable): (B,H,ceil(T/chunk),dk) fp32, z entering each chunk, are residuals of the backward call together with o and S_chk. */
+ * z_chk (nullable): (B,H,ceil(T/chunk),dk) fp32, z entering each chunk, are residuals of the backward call together with o and S_chk.
+ * ss (nullable): (B,H,T) fp32, ss_t = sum over the dv value features of o_t^2 (o as stored, i.e. rounded to
+ *   the I/O type), taken from the output tile before it leaves the kernel.  It is what the RMS norm over
+ *   all heads that follows the divide (linear_attention.py:114, `self.norm(output)` over H*dv) needs from
+ *   each head: mean square = sum_h ss[b,h,t] / (H dv), so the caller's side of the norm is one rescale of o
+ *   instead of a reduction pass plus a rescale. */
 int mrx_linear_attn_norm_fwd(void *stream, const void *q, const void *k,
                              const void *v, const void *done, const void *S0,
-                             const float *z0, void *o, float *den, void *S_last,
+                             const float *z0, void *o, float *den, float *ss, void *S_last,
                              float *z_last, void *S_chk, float *z_chk, int64_t B,
                              int64_t T, int64_t H, int64_t dk, int64_t dv,
                              int dtype, int done_dtype, int feature_map, float eps);
 
 /* Gradients of the above w.r.t. q,k,v (pre-feature-map), S0 and z0, given
  * dout = dL/do (gradient of the normalised output), dS_last and dz_last (nullable).
- * Where the clamp is active (den == eps) the denominator passes no gradient. */
+ * Where the clamp is active (den == eps) the denominator passes no gradient.
+ * d_ss (nullable = 0): (B,H,T) fp32, dL/dss of the forward call's sums of squares; the kernel adds
+ *   2 d_ss_t o_t to dout_t as it stages the chunk. */
 int mrx_linear_attn_norm_bwd(void *stream, const void *q, const void *k,
                              const void *v, const void *done, const void *S_chk,
                              const float *S_last, const float *z_chk, const void *o, const float *den,
-                             const void *dout, const void *dS_last,
+                             const void *dout, const float *d_ss, const void *dS_last,
                              const float *dz_last, void *dq, void *dk_out,
                              void *dv_out, void *dS0, float *dz0, int64_t B,
                              int64_t T, int64_t H, int64_t dk, int64_t dv,

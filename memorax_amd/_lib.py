@@ -36,8 +36,8 @@ SIGNATURES = {
     "mrx_linear_attn_fwd_chunk_parallel": (_I, [_P] * 9 + [_L] * 5 + [_I] * 3),
     "mrx_linear_attn_bwd_chunk_parallel": (_I, [_P] * 13 + [_L] * 5 + [_I] * 3),
     "mrx_linear_attn_chunk_parallel_pays": (_I, [_L] * 3 + [_I]),
-    "mrx_linear_attn_norm_fwd": (_I, [_P] * 13 + [_L] * 5 + [_I] * 3 + [ctypes.c_float]),
-    "mrx_linear_attn_norm_bwd": (_I, [_P] * 18 + [_L] * 5 + [_I] * 3 + [ctypes.c_float]),
+    "mrx_linear_attn_norm_fwd": (_I, [_P] * 14 + [_L] * 5 + [_I] * 3 + [ctypes.c_float]),
+    "mrx_linear_attn_norm_bwd": (_I, [_P] * 19 + [_L] * 5 + [_I] * 3 + [ctypes.c_float]),
     "mrx_delta_rule_fwd": (_I, [_P] * 11 + [_L] * 5 + [_I] * 3),
     "mrx_delta_rule_fwd_noalloc": (_I, [_P] * 9 + [_L] * 5 + [_I] * 2),
     "mrx_delta_rule_bwd": (_I, [_P] * 15 + [_L] * 5 + [_I] * 2),

@@ -28,11 +28,18 @@ int prepare_device(int *cus, int *dev_out)
     if (!(g_ready.load(std::memory_order_acquire) & bit)) {
         std::lock_guard<std::mutex> lock(g_setup);
         if (!(g_ready.load(std::memory_order_relaxed) & bit)) {
+            // a refused set-up call is reported through the return value and taken off the runtime's
+            // record, as a refused launch is (launch_kernel)
+            auto failed = [](hipError_t e) {
+                if (e == hipSuccess) return false;
+                (void)hipGetLastError();
+                return true;
+            };
             for (const KernelNode *n = g_kernels; n; n = n->next)
-                if (hipFuncSetAttribute(n->fn, hipFuncAttributeMaxDynamicSharedMemorySize, n->lds_bytes) != hipSuccess)
+                if (failed(hipFuncSetAttribute(n->fn, hipFuncAttributeMaxDynamicSharedMemorySize, n->lds_bytes)))
                     return MRX_ERR_LAUNCH;
             int n_cu = 0;
-            if (hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return MRX_ERR_LAUNCH;
+            if (failed(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev))) return MRX_ERR_LAUNCH;
             g_cus[dev] = n_cu;
             if (const int rc = resolve_scratch(dev); rc != MRX_OK) return rc;
             g_ready.fetch_or(bit, std::memory_order_release);

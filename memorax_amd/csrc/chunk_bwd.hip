@@ -65,6 +65,7 @@ struct NormBwdArgs {
     const float *dz_last; // (B,H,64) or null
     float *dz0;           // (B,H,64) or null
     float eps;
+    const float *d_ss;    // (B,H,T) or null: gradient of the forward call's sums of squares of the outputs
 };
 
 // GATED: S_t = r_t exp(g_t) S_{t-1} + v_t k_t^T.  With G the cumulative log-decay inside the chunk
@@ -72,7 +73,8 @@ struct NormBwdArgs {
 //   Aqk, dAqk carry the factor D;  dV = Aqk^T dO + diag(b) K dS^T;  dQ = diag(a) dO S + dAqk K;
 //   dK = dAqk^T Q + diag(b) V dS;  dS <- c dS + (diag(a) Q)^T dO.
 // NORM (normalised read-out o_i = num_i / den_i, den_i = max(q_i . z_i, eps), z the running sum of
-// the keys of the episode): with dnum_i = dout_i / den_i taking the place of dO and
+// the keys of the episode; a gradient d_ss of the forward call's row sums of squares ss_i = |o_i|^2
+// first joins the output gradient, dout_i <- dout_i + 2 d_ss_i o_i): with dnum_i = dout_i / den_i taking the place of dO and
 // dden_i = -(dout_i . o_i) / den_i (0 where the clamp is active),
 //   dAqk_ij += dden_i (j <= i);  dQ_i += dden_i z_in;  dK_j += dz;  dz <- dz + sum_i dden_i Q_i,
 // z_in the sum entering the chunk (first episode only), dz the gradient of the sum leaving it.
@@ -165,7 +167,8 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     // The state leaving, then entering, the chunk at hand (S^T, in the layout of dS^T).  Without a decay
     // the update of a chunk can be undone, S_c = S_{c+1} - V_c^T K_c, so the state is walked back in
     // fp32 registers from the forward call's S_last and read from the forward call's (fp32) checkpoints
-    // only where the walk cannot pass: chunks with resets, the only ones the forward call writes then.
+    // only where the walk cannot pass -- chunks with resets -- and at every walk_anchor()-th chunk, where it
+    // starts afresh from the exact state: the chunks the forward call writes then.
     // Gated: every chunk has a checkpoint in the I/O type, staged row-wise.
     constexpr bool WALK = !GATED;
     constexpr int NSA = WALK ? TMS::TPW : 1;
@@ -201,7 +204,9 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
     }
 
     typename IO::Regs rq, rk, rv, rdo, ro;
-    float rden[IO::PASSES];
+    float rden[IO::PASSES], rdss[IO::PASSES];
+#pragma unroll
+    for (int p = 0; p < IO::PASSES; ++p) rdss[p] = 0.f;
     f32x4 rz = {0.f, 0.f, 0.f, 0.f};
     typename IOS::Regs rS;
     // raw bits, tested when the chunk is staged; the reset flags of the chunk after the next one too:
@@ -282,7 +287,9 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
             if (NORM) {
 #pragma unroll
                 for (int p = 0; p < IO::PASSES; ++p) {
-                    rden[p] = (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen ? na.den[noff[p]] : 1.f;
+                    const bool in = (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen;
+                    rden[p] = in ? na.den[noff[p]] : 1.f;
+                    if (na.d_ss) rdss[p] = in ? na.d_ss[noff[p]] : 0.f;
                     noff[p] -= C;
                 }
                 if (!NARROW || 4 * (tid % (HD / 4)) < dkw) rz = *reinterpret_cast<const f32x4 *>(na.z_chk + zoff);
@@ -336,8 +343,9 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
         const int t0 = c * C;
         const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
-        const bool ckpt = PAR || !WALK || nres != 0;  // the entering state comes from S_chk
-        if (WALK && !PAR) need_S = __ballot(done_test(rdone2, done_f32) && lane < C) != 0ull;  // for the chunk prefetched during this one
+        const bool ckpt = PAR || !WALK || nres != 0 || c % walk_anchor<T>() == 0;  // the entering state comes from S_chk
+        if (WALK && !PAR)  // for the chunk prefetched during this one
+            need_S = __ballot(done_test(rdone2, done_f32) && lane < C) != 0ull || (c >= 1 && (c - 1) % walk_anchor<T>() == 0);
         for (int pass = nres; pass >= 0; --pass) {
             auto live = [&](int r) { return nres == 0 || episode_of(dmask, r) == pass; };
             // gated: cumulative log-decay of this pass's episode (as in the forward kernel)
@@ -379,6 +387,18 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                         dot = seg_sum<IO::SEGS>(dot);
                         const int r = IO::row_of(tid, p);
                         const bool on = (IO::FULL || r < C) && live(r);
+                        if (na.d_ss) {  // dout_i + 2 d_ss_i o_i takes the place of dout_i (live rows only, by select)
+                            float oo = 0.f;
+#pragma unroll
+                            for (int e = 0; e < IO::KP; ++e) oo += (float)ro.v[p][e] * (float)ro.v[p][e];
+                            oo = seg_sum<IO::SEGS>(oo);
+                            const float two = 2.f * rdss[p];
+                            dot += two * oo;
+                            if (on) {
+#pragma unroll
+                                for (int e = 0; e < IO::KP; ++e) fdo.v[p][e] = (T)(((float)rdo.v[p][e] + two * (float)ro.v[p][e]) / rden[p]);
+                            }
+                        }
                         inv[p] = on ? 1.f / rden[p] : 1.f;
                         const float dd = (on && rden[p] > na.eps) ? -dot * inv[p] : 0.f;
                         if (tid % IO::SEGS == 0 && (IO::FULL || r < C)) {
@@ -386,7 +406,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                             sDdT[r] = (T)dd;
                         }
                     }
-                    IO::scale_rows(fdo, inv);
+                    if (!na.d_ss) IO::scale_rows(fdo, inv);
                     if (tid < HD / 4) *reinterpret_cast<f32x4 *>(sZf + 4 * tid) = rz;
                 }
                 flush_pending();  // reads what this thread is about to overwrite in sV, sQ, sK
@@ -682,6 +702,12 @@ template <typename T, int C, int NW> struct DeltaBwdSmem : BwdDims<T, C> {
 //   dk = (dk_n - k_n (k_n . dk_n)) / |k| ,   db = dbeta beta (1 - beta).
 // NARROW: narrow heads, as in the linear-attention kernels -- q, k, dq, dk are dka wide in memory, v, dout, dv dva,
 // the states [dva][dka]; tiles keep the build's width with zeros beyond, only the rows' own width is stored.
+#ifdef MRX_PHASE_CLOCKS
+// [0] cycles inside matrix products, [1] cycles alive, both summed over the waves of every workgroup of
+// every delta_bwd_kernel launch since the last reset; [2] workgroups counted.
+static __device__ unsigned long long g_phase_clocks[4];
+#endif
+
 template <typename T, int C, int NW, bool PRO, bool NARROW = false>
 __global__ void __launch_bounds__(64 * NW, sizeof(T) == 2 ? 2 : 1)
 delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
@@ -729,6 +755,10 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     using TMA = TileMap<C, C, NW>;
     using TMR = TileMap<HD, C, NW>;
     constexpr int NSLOT = L::NSLOT;
+#ifdef MRX_PHASE_CLOCKS
+    if (tid == 0) wg_product_clocks = 0ull;  // the first product comes after the staging barrier
+    const long long kernel_clk0 = clock64();
+#endif
 
     f32x4 dSacc[TMS::TPW];  // dS^T: m = dk, n = dv
 #pragma unroll
@@ -1086,6 +1116,13 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     }
     sync_lds();
     flush_pending();
+#ifdef MRX_PHASE_CLOCKS
+    if (tid == 0) {  // the waves of a workgroup move from barrier to barrier together: wave 0's lifetime stands for all
+        atomicAdd(&g_phase_clocks[0], wg_product_clocks);
+        atomicAdd(&g_phase_clocks[1], (unsigned long long)NW * (unsigned long long)(clock64() - kernel_clk0));
+        atomicAdd(&g_phase_clocks[2], 1ull);
+    }
+#endif
     if (dS0) {
 #pragma unroll
         for (int j = 0; j < TMS::TPW; ++j) {
@@ -1203,25 +1240,25 @@ MRX_EXPORT int MRX_API(mrx_linear_attn_bwd_chunk_parallel)(void *stream, const v
 
 MRX_EXPORT int MRX_API(mrx_linear_attn_norm_bwd)(void *stream, const void *q, const void *k, const void *v,
                                         const void *done, const void *S_chk, const float *S_last, const float *z_chk,
-                                        const void *o, const float *den, const void *dout,
+                                        const void *o, const float *den, const void *dout, const float *d_ss,
                                         const void *dS_last, const float *dz_last, void *dq, void *dk_out,
                                         void *dv_out, void *dS0, float *dz0, int64_t B, int64_t T, int64_t H,
                                         int64_t dk, int64_t dv, int dtype, int done_dtype, int feature_map,
                                         float eps)
 {
 #if MRX_HD == 64
-    if (dk <= 32 && dv <= 32) return mrx_linear_attn_norm_bwd_hd32(stream, q, k, v, done, S_chk, S_last, z_chk, o, den, dout, dS_last, dz_last, dq, dk_out, dv_out, dS0, dz0, B, T, H, dk, dv, dtype, done_dtype, feature_map, eps);
+    if (dk <= 32 && dv <= 32) return mrx_linear_attn_norm_bwd_hd32(stream, q, k, v, done, S_chk, S_last, z_chk, o, den, dout, d_ss, dS_last, dz_last, dq, dk_out, dv_out, dS0, dz0, B, T, H, dk, dv, dtype, done_dtype, feature_map, eps);
 #endif
     const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
                              dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
     if (!z_chk || !o || !den || !S_last || !aligned(S_last, 16)) return MRX_ERR_INVALID_ARG;
-    if (!aligned(z_chk, 16) || !aligned(o, 16) || !aligned(den, 4) || !aligned(dz_last, 16) || !aligned(dz0, 16))
+    if (!aligned(z_chk, 16) || !aligned(o, 16) || !aligned(den, 4) || !aligned(d_ss, 4) || !aligned(dz_last, 16) || !aligned(dz0, 16))
         return MRX_ERR_INVALID_ARG;
     if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     const bool fm = feature_map == MRX_FMAP_ELU1;
-    const NormBwdArgs na{o, den, z_chk, dz_last, dz0, eps};
+    const NormBwdArgs na{o, den, z_chk, dz_last, dz0, eps, d_ss};
 #define MRX_ARGS st, q, k, v, done, done_dtype, S_chk, S_last, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, nullptr, nullptr, na, dk, dv
     if (dtype == MRX_BF16)
         return fm ? launch_la<__bf16, LA_BF16_CHUNK, true, false, true>(MRX_ARGS)
@@ -1331,3 +1368,20 @@ MRX_EXPORT int MRX_API(mrx_deltanet_bwd)(void *stream, const void *q, const void
     return delta_bwd_entry<true>(stream, q, k, v, beta_raw, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out,
                                  dbeta_raw, dS0, B, T, H, dk, dv, dtype, done_dtype);
 }
+
+#if defined(MRX_PHASE_CLOCKS) && MRX_HD == 64
+// Measurement build only: the clocks of delta_bwd_kernel (above), copied to out[0..2] after the device has
+// finished what was enqueued; reset != 0 clears them afterwards.  Synchronises: not for use beside real work.
+extern "C" int mrx_phase_clocks(unsigned long long *out, int reset)
+{
+    unsigned long long v[4] = {0ull, 0ull, 0ull, 0ull};
+    if (hipDeviceSynchronize() != hipSuccess) return MRX_ERR_LAUNCH;
+    if (hipMemcpyFromSymbol(v, HIP_SYMBOL(g_phase_clocks), sizeof(v)) != hipSuccess) return MRX_ERR_LAUNCH;
+    if (out) for (int i = 0; i < 3; ++i) out[i] = v[i];
+    if (reset) {
+        const unsigned long long z[4] = {0ull, 0ull, 0ull, 0ull};
+        if (hipMemcpyToSymbol(HIP_SYMBOL(g_phase_clocks), z, sizeof(z)) != hipSuccess) return MRX_ERR_LAUNCH;
+    }
+    return MRX_OK;
+}
+#endif

@@ -51,6 +51,16 @@ static_assert(HD == 64 || HD == 32, "tile maps exist for head dims 64 and 32");
 #endif
 constexpr int LA_BF16_CHUNK = MRX_LA_BF16_CHUNK, DELTA_BF16_CHUNK = MRX_DELTA_BF16_CHUNK;
 
+// Plain and normalised linear attention: the backward call walks the state back from chunk to chunk
+// (S_c = S_{c+1} - V_c^T K_c in fp32) instead of reading a checkpoint per chunk.  Every step of that walk
+// rounds at the magnitude of the late, large state, so its error relative to an early, small state grows
+// with the number of chunks walked (about eps N^1.5 for a state that grows linearly).  The forward
+// call therefore writes the exact fp32 state every WALK_ANCHOR chunks as well (besides the chunks
+// with resets) and the walk starts afresh there: 32 chunks keep fp32 at 1e-5 of the early states,
+// bf16 inputs (tolerance 2e-2, rounding 4e-3) are re-anchored every 128.  Extra traffic: one 16 KB
+// slot per 32 (128) chunks of 32 KB each way.
+template <typename T> constexpr int walk_anchor() { return sizeof(T) == 2 ? 128 : 32; }
+
 enum OpMode { ROWK = 0, KROW = 1 };
 
 template <typename T> struct TT;
@@ -162,6 +172,15 @@ struct NoHook {
     template <typename F> __device__ __forceinline__ void operator()(int, int, F &) const {}
 };
 
+#ifdef MRX_PHASE_CLOCKS
+// Measurement build (libmemorax_amd_clk.so): every matrix product is bracketed by reads of the shader
+// clock -- from before its first operand fragment is requested until its accumulators are in hand --
+// and the cycles are summed per workgroup here.  A kernel that reports them (delta_bwd_kernel) clears the
+// sum at its start and adds it to its device-wide totals at its end.  The brackets serialise a product
+// against what follows it, so this build is for the ratio of the two clocks only, never for timing.
+static __shared__ unsigned long long wg_product_clocks;
+#endif
+
 // acc[j] += sum_k X(mt_j rows, k) * Y(nt_j rows, k), k = 0..K-1.
 // hx(mi, kb, fragment) / hy(ni, kb, fragment) see every operand fragment as it is loaded, so that
 // a rank-one by-product (a row or column sum, a product with one more vector) costs MFMAs only;
@@ -175,6 +194,9 @@ __device__ __forceinline__ void gemm(f32x4 *acc, const T *X, int ldx, const T *Y
     using F = typename TT<T>::frag;
     constexpr int KB = TT<T>::KB;
     static_assert(K % KB == 0, "K must be a multiple of the fragment k extent");
+#ifdef MRX_PHASE_CLOCKS
+    const long long clk0 = clock64();
+#endif
 #pragma unroll
     for (int kb = 0; kb < K / KB; ++kb) {
         F a[TM::MBW];
@@ -193,6 +215,14 @@ __device__ __forceinline__ void gemm(f32x4 *acc, const T *X, int ldx, const T *Y
                 acc[mi * TM::NBW + ni] = TT<T>::mma(a[mi], b, acc[mi * TM::NBW + ni]);
         }
     }
+#ifdef MRX_PHASE_CLOCKS
+    float sink = 0.f;  // an ordinary read of every tile: the matrix pipe has delivered before the second clock
+#pragma unroll
+    for (int j = 0; j < TM::TPW; ++j) sink += acc[j][0] + acc[j][3];
+    asm volatile("" ::"v"(sink));
+    const long long clk1 = clock64();
+    if (lane == 0) atomicAdd(&wg_product_clocks, (unsigned long long)(clk1 - clk0));
+#endif
 }
 
 template <int N> __device__ __forceinline__ void zero_acc(f32x4 *acc)

@@ -53,7 +53,9 @@ template <typename T, int C, bool DELTA, bool GATED = false, bool NORM = false> 
     static constexpr int oBeta = oA + szRA;
     static constexpr int oG = oBeta + C * 4;              // gated: cumulative log-decay G of the chunk rows, then exp(G_last - G)
     static constexpr int oZ = oG + 2 * C * 4;             // z entering the pass, T-typed row of 64 (normalised read-out)
-    static constexpr int oO = oZ + (NORM ? HD * (int)sizeof(T) : 0);  // O [C][dv] on its way to memory
+    // normalised read-out: per-row partial sums of squares of the outputs, one slot per feature block of waves
+    static constexpr int oSS = oZ + (NORM ? HD * (int)sizeof(T) : 0);
+    static constexpr int oO = oSS + (NORM ? TileMap<HD, C, 4>::WM * C * 4 : 0);  // O [C][dv] on its way to memory
     static constexpr int total = oO + szRD;
 };
 
@@ -64,6 +66,7 @@ struct NormArgs {
     float *z_last;    // (B,H,64) or null
     float *z_chk;     // (B,H,NC,64) or null: z entering each chunk
     float eps;
+    float *ss;        // (B,H,T) or null: sum over the value features of the squared (rounded) outputs of each step
 };
 
 // PRO (delta rule): the cell's prologue runs on the staged rows -- keys are L2-normalised
@@ -114,6 +117,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     float *sG = reinterpret_cast<float *>(smem + L::oG);
     float *sEb = sG + C;                             // gated: b_j = exp(G_last - G_j)
     T *sZ = reinterpret_cast<T *>(smem + L::oZ);
+    float *sSS = reinterpret_cast<float *>(smem + L::oSS);
     T *sO = reinterpret_cast<T *>(smem + L::oO);
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -345,12 +349,13 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             // chunk in fp32, starting from S_last (S_c = S_{c+1} - V_c^T K_c undoes a chunk's update), so a
             // checkpoint is written only where that walk cannot pass: for a chunk with resets, whose entering
             // state the state that leaves it does not determine.  Those are written in fp32 from the
-            // accumulators (rare; the walk carries their rounding to the chunks before).  The decayed update
+            // accumulators (rare; the walk carries their rounding to the chunks before), as is every
+            // walk_anchor()-th chunk, where the walk starts afresh from the exact state.  The decayed update
             // of the gated variant is not undone (it would divide by the decay), and for the delta rule the
             // walk needs U' as a residual and an extra product, which measured slower than reading the
             // states: there every chunk is written, in the I/O type, from the copy of S just staged.
             constexpr bool DENSE_CHK = GATED || DELTA;
-            if (!PAR && S_chk && pass == 0 && (DENSE_CHK || nres != 0)) {
+            if (!PAR && S_chk && pass == 0 && (DENSE_CHK || nres != 0 || c % walk_anchor<T>() == 0)) {
                 if (DENSE_CHK) {
                     using IOS = TileIO<T, HD, NTHR>;
 #pragma unroll
@@ -508,6 +513,27 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 }
             }
             store_acc<T, HD, C, NW>(Oacc, sO, LDD, w, lane);  // to memory once the next unit has been staged
+            if (NORM && na.ss) {
+                // sum of squares of each output row as it is stored (rounded to T), for an RMS norm over the
+                // heads that follows the read-out (linear_attention.py:114): the wave's feature tiles, the four
+                // lane groups, then one slot per feature block of waves; summed after the unit's last barrier
+                float sq[TMO::NBW];
+#pragma unroll
+                for (int ni = 0; ni < TMO::NBW; ++ni) sq[ni] = 0.f;
+#pragma unroll
+                for (int j = 0; j < TMO::TPW; ++j) {
+                    const P4 r4 = TT<T>::pack(Oacc[j][0], Oacc[j][1], Oacc[j][2], Oacc[j][3]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) sq[j % TMO::NBW] += (float)r4[e] * (float)r4[e];
+                }
+#pragma unroll
+                for (int ni = 0; ni < TMO::NBW; ++ni) {
+                    float x = sq[ni];
+                    x += __shfl_xor(x, 16);
+                    x += __shfl_xor(x, 32);
+                    if (lg == 0) sSS[(w % TMO::WM) * C + TMO::nt(w, ni) * 16 + li] = x;
+                }
+            }
             pend_dmask = dmask;
             pend_nres = nres;
             pend_pass = pass;
@@ -549,6 +575,12 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 }
             }
             sync_lds();
+            if (NORM && na.ss && tid < C && t0 + tid < Tlen && live(tid)) {
+                float x = 0.f;
+#pragma unroll
+                for (int sl = 0; sl < TMO::WM; ++sl) x += sSS[sl * C + tid];
+                na.ss[(int64_t)bh * Tlen + t0 + tid] = x;  // the slots are next written after the next unit's barriers
+            }
         }
     }
     flush_o();  // the last unit ended with a barrier
@@ -675,7 +707,10 @@ bool factor_path_ok(int f) { return f == MRX_FACTORS_AUTO || f == MRX_FACTORS_PA
 // Room for the triangular factors of MRX_NOALLOC_SCRATCH_BYTES / (32 * 32 * sizeof(element)) chunks.
 // Every device the library runs on holds its own copy at its own address; host code only ever uses
 // the address resolve_scratch() obtained for the current device, never the array's name.
-static __device__ __align__(256) unsigned char scratch[MRX_NOALLOC_SCRATCH_BYTES];
+// The build with 64-step delta-rule chunks has no chunk-parallel factor kernel, hence no use for the
+// array (its mrx_delta_rule_fwd_noalloc answers MRX_ERR_UNSUPPORTED) and does not hold it.
+constexpr bool HAS_SCRATCH = DELTA_BF16_CHUNK == 32;
+static __device__ __align__(256) unsigned char scratch[HAS_SCRATCH ? MRX_NOALLOC_SCRATCH_BYTES : 256];
 void *g_scratch_ptr[64] = {nullptr};
 
 #endif
@@ -686,8 +721,12 @@ void *g_scratch_ptr[64] = {nullptr};
 int mrx::resolve_scratch(int dev)
 {
     if (dev < 0 || dev >= 64) return MRX_ERR_UNSUPPORTED;
+    if (!HAS_SCRATCH) return MRX_OK;
     void *p = nullptr;
-    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return MRX_ERR_LAUNCH;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+        (void)hipGetLastError();  // reported through the return value; not left for the host framework's next call
+        return MRX_ERR_LAUNCH;
+    }
     g_scratch_ptr[dev] = p;
     return MRX_OK;
 }
@@ -789,6 +828,7 @@ extern "C" int mrx_delta_rule_fwd_noalloc(void *stream, const void *q, const voi
     const int rc = check_common(q, k, v, done, o, S0, S_last, nullptr, B, T, H, dk, dv, dtype, done_dtype);
     if (rc != MRX_OK) return rc;
     if (!beta) return MRX_ERR_INVALID_ARG;
+    if (!HAS_SCRATCH) return MRX_ERR_UNSUPPORTED;
     const int64_t NC = (T + 31) / 32, esize = dtype == MRX_BF16 ? 2 : 4;
     if (T > DELTA_TM_MAX_T || B * H * NC > (int64_t)MRX_NOALLOC_SCRATCH_BYTES / (32 * 32 * esize)) return MRX_ERR_SCRATCH;
     int dev = -1;
@@ -824,21 +864,21 @@ MRX_EXPORT int MRX_API(mrx_gated_linear_attn_fwd)(void *stream, const void *q, c
 
 MRX_EXPORT int MRX_API(mrx_linear_attn_norm_fwd)(void *stream, const void *q, const void *k, const void *v,
                                         const void *done, const void *S0, const float *z0, void *o,
-                                        float *den, void *S_last, float *z_last, void *S_chk, float *z_chk,
+                                        float *den, float *ss, void *S_last, float *z_last, void *S_chk, float *z_chk,
                                         int64_t B, int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
                                         int done_dtype, int feature_map, float eps)
 {
 #if MRX_HD == 64
-    if (dk <= 32 && dv <= 32) return mrx_linear_attn_norm_fwd_hd32(stream, q, k, v, done, S0, z0, o, den, S_last, z_last, S_chk, z_chk, B, T, H, dk, dv, dtype, done_dtype, feature_map, eps);
+    if (dk <= 32 && dv <= 32) return mrx_linear_attn_norm_fwd_hd32(stream, q, k, v, done, S0, z0, o, den, ss, S_last, z_last, S_chk, z_chk, B, T, H, dk, dv, dtype, done_dtype, feature_map, eps);
 #endif
     const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
-    if (!den || !aligned(den, 4) || !aligned(z0, 16) || !aligned(z_last, 16) || !aligned(z_chk, 16))
+    if (!den || !aligned(den, 4) || !aligned(ss, 4) || !aligned(z0, 16) || !aligned(z_last, 16) || !aligned(z_chk, 16))
         return MRX_ERR_INVALID_ARG;
     if (feature_map != MRX_FMAP_NONE && feature_map != MRX_FMAP_ELU1) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     const bool fm = feature_map == MRX_FMAP_ELU1;
-    const NormArgs na{z0, den, z_last, z_chk, eps};
+    const NormArgs na{z0, den, z_last, z_chk, eps, ss};
 #define MRX_ARGS st, q, k, v, nullptr, done, done_dtype, S0, o, S_last, S_chk, nullptr, B, T, H, nullptr, na, dk, dv
     if (dtype == MRX_BF16)
         return fm ? launch<__bf16, LA_BF16_CHUNK, false, true, false, true>(MRX_ARGS)

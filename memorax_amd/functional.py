@@ -59,8 +59,9 @@ def _no_steps(x):
 
 def _scan_without_steps(b, h0, P0):
     B, _, D = b.shape
-    h_last = b.new_zeros((B, D)) if h0 is None else h0 + 0
-    P_last = b.new_ones((B, D)) if P0 is None else P0.detach().clone()
+    ct = torch.float32 if b.dtype == torch.bfloat16 else b.dtype   # bf16 arrays carry float32 state, as the kernels do
+    h_last = b.new_zeros((B, D), dtype=ct) if h0 is None else h0.to(ct) + 0
+    P_last = b.new_ones((B, D), dtype=ct) if P0 is None else P0.detach().to(ct).clone()
     return b.new_zeros(b.shape), h_last, P_last
 
 
@@ -277,7 +278,7 @@ def linear_attention(q, k, v, done, S0=None, feature_map="none"):
 
 class _NormalisedLinearAttention(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, done, S0, z0, fmap, eps):
+    def forward(ctx, q, k, v, done, S0, z0, fmap, eps, want_ss):
         q_, k_, v_ = q.contiguous(), k.contiguous(), v.contiguous()
         S0_ = None if S0 is None else S0.contiguous().float()
         z0_ = None if z0 is None else z0.contiguous().float()
@@ -286,36 +287,48 @@ class _NormalisedLinearAttention(torch.autograd.Function):
         if q_.shape[1] == 1 and not need:  # acting: one fused step
             o, S_last, z_last = K.linear_attn_step(q_[:, 0], k_[:, 0], v_[:, 0], done[:, 0], S0_, z0_,
                                                    feature_map=_FMAP_NAME[fmap], normalise=True, eps=eps)
-            return o[:, None], S_last, z_last
-        o, den, S_last, z_last, chk = K.linear_attn_norm_fwd(q_, k_, v_, done, S0_, z0_, fmap, eps, save_chk=need)
+            ss = o.float().square().sum(-1)[..., None] if want_ss else None   # (B,H,1)
+            return o[:, None], S_last, z_last, ss
+        o, den, S_last, z_last, chk, ss = K.linear_attn_norm_fwd(q_, k_, v_, done, S0_, z0_, fmap, eps, save_chk=need,
+                                                                 want_ss=True) if want_ss else \
+            (*K.linear_attn_norm_fwd(q_, k_, v_, done, S0_, z0_, fmap, eps, save_chk=need), None)
         if need:
             ctx.save_for_backward(q_, k_, v_, o, den, *chk)
-        return o, S_last, z_last
+        return o, S_last, z_last, ss
 
     @staticmethod
-    def backward(ctx, do, dS_last, dz_last):
+    def backward(ctx, do, dS_last, dz_last, d_ss):
         q, k, v, o, den, S_chk, z_chk, S_last = ctx.saved_tensors
         do = torch.zeros_like(v) if do is None else do.contiguous()
         dS_last = None if dS_last is None else dS_last.contiguous().float()
         dz_last = None if dz_last is None else dz_last.contiguous().float()
+        d_ss = None if d_ss is None else d_ss.contiguous().float()
         dq, dk, dv, dS0, dz0 = K.linear_attn_norm_bwd(q, k, v, ctx.done, (S_chk, z_chk, S_last), o, den, do, dS_last,
-                                                      dz_last, ctx.fmap, ctx.eps, want_d0=any(ctx.has_0))
-        return dq, dk, dv, None, (dS0 if ctx.has_0[0] else None), (dz0 if ctx.has_0[1] else None), None, None
+                                                      dz_last, ctx.fmap, ctx.eps, want_d0=any(ctx.has_0), d_ss=d_ss)
+        return dq, dk, dv, None, (dS0 if ctx.has_0[0] else None), (dz0 if ctx.has_0[1] else None), None, None, None
 
 
 @_batched(4, 0)
-def normalised_linear_attention(q, k, v, done, S0=None, z0=None, feature_map="elu1", eps=1e-6):
+def normalised_linear_attention(q, k, v, done, S0=None, z0=None, feature_map="elu1", eps=1e-6, return_ss=False):
     """Causal linear attention with the normalised read-out of LinearAttentionCell.read
     (linear_attention.py:93-110) in the same kernel: z_t = r_t z_{t-1} + phi(k_t),
-    o_t = S_t phi(q_t) / max(phi(q_t) . z_t, eps).  Returns (o, S_last, z_last)."""
+    o_t = S_t phi(q_t) / max(phi(q_t) . z_t, eps).  Returns (o, S_last, z_last), and with return_ss a
+    fourth result ss (B,T,H) float32, ss[b,t,h] = sum_d o[b,t,h,d]^2 from the kernel's output tile
+    (differentiable): what the RMS norm over all heads that follows (linear_attention.py:114) needs
+    from each head, so that its caller does one rescale of o and no reduction over it."""
     if _no_steps(q):
-        B, _, H, dk = q.shape
+        B, T, H, dk = q.shape
         z_last = q.new_zeros((B, H, dk), dtype=torch.float32) if z0 is None else z0.float() + 0
-        return (*_attention_without_steps(q, v, S0), z_last)
+        out = (*_attention_without_steps(q, v, S0), z_last)
+        return (*out, q.new_zeros((B, T, H), dtype=torch.float32)) if return_ss else out
     hd = _Heads(q, v, _FMAP[feature_map], narrow=True)
-    o, S_last, z_last = _NormalisedLinearAttention.apply(hd.qk(q), hd.qk(k), hd.v(v), done, hd.state_in(S0),
-                                                         hd.z_in(z0), hd.fmap, float(eps))
-    return hd.out(o), hd.state_out(S_last), hd.z_out(z_last)
+    o, S_last, z_last, ss = _NormalisedLinearAttention.apply(hd.qk(q), hd.qk(k), hd.v(v), done, hd.state_in(S0),
+                                                             hd.z_in(z0), hd.fmap, float(eps), bool(return_ss))
+    out = (hd.out(o), hd.state_out(S_last), hd.z_out(z_last))
+    if not return_ss:
+        return out
+    B, Hk, T = ss.shape   # kernel heads = (H, value blocks): a head's sum of squares is the sum over its blocks
+    return (*out, ss.view(B, hd.H, Hk // hd.H, T).sum(2).transpose(1, 2))
 
 
 class _GatedLinearAttention(torch.autograd.Function):

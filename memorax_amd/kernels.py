@@ -268,10 +268,11 @@ def linear_attn_bwd(q, k, v, done, chk, do, dS_last=None, feature_map=0, want_dS
     return dq, dk_, dv_, dS0
 
 
-def linear_attn_norm_fwd(q, k, v, done, S0=None, z0=None, feature_map=0, eps=1e-6, save_chk=True):
+def linear_attn_norm_fwd(q, k, v, done, S0=None, z0=None, feature_map=0, eps=1e-6, save_chk=True, want_ss=False):
     """Linear attention with the normalised read-out fused.
     Returns (o, den fp32 (B,H,T), S_last fp32, z_last fp32, (S_chk, z_chk, S_last) or None); S_chk as for
-    linear_attn_fwd."""
+    linear_attn_fwd.  want_ss: a sixth result, ss fp32 (B,H,T), the per-head sums of squares of the
+    outputs (what an RMS norm over the heads needs from each of them)."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
     _chk(S0, "S0", torch.float32, (B, H, dv, dk))
@@ -284,16 +285,18 @@ def linear_attn_norm_fwd(q, k, v, done, S0=None, z0=None, feature_map=0, eps=1e-
     nc = _n_chunks(T, dt)
     S_chk = torch.empty((B, H, nc, dv, dk), dtype=torch.float32, device=q.device) if save_chk else None
     z_chk = torch.empty((B, H, nc, dk), dtype=torch.float32, device=q.device) if save_chk else None
+    ss = torch.empty((B, H, T), dtype=torch.float32, device=q.device) if want_ss else None
     st = lib.mrx_linear_attn_norm_fwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(done), _ptr(S0), _ptr(z0),
-                                      _ptr(o), _ptr(den), _ptr(S_last), _ptr(z_last), _ptr(S_chk), _ptr(z_chk),
+                                      _ptr(o), _ptr(den), _ptr(ss), _ptr(S_last), _ptr(z_last), _ptr(S_chk), _ptr(z_chk),
                                       B, T, H, dk, dv, _DT[dt], dd, int(feature_map), float(eps))
     _lib.check(st, "mrx_linear_attn_norm_fwd")
-    return o, den, S_last, z_last, ((S_chk, z_chk, S_last) if save_chk else None)
+    chk = (S_chk, z_chk, S_last) if save_chk else None
+    return (o, den, S_last, z_last, chk, ss) if want_ss else (o, den, S_last, z_last, chk)
 
 
 def linear_attn_norm_bwd(q, k, v, done, chk, o, den, do, dS_last=None, dz_last=None, feature_map=0, eps=1e-6,
-                         want_d0=True):
-    """Returns (dq, dk, dv, dS0, dz0)."""
+                         want_d0=True, d_ss=None):
+    """Returns (dq, dk, dv, dS0, dz0).  d_ss: gradient of the forward call's ss, fp32 (B,H,T)."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
     S_chk, z_chk, S_last = chk
@@ -306,12 +309,13 @@ def linear_attn_norm_bwd(q, k, v, done, chk, o, den, do, dS_last=None, dz_last=N
     _chk(z_chk, "z_chk", torch.float32, (B, H, nc, dk))
     _chk(dS_last, "dS_last", torch.float32, (B, H, dv, dk))
     _chk(dz_last, "dz_last", torch.float32, (B, H, dk))
+    _chk(d_ss, "d_ss", torch.float32, (B, H, T))
     done, dd = _done(done, B, T)
     dq, dk_, dv_ = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dS0 = torch.empty((B, H, dv, dk), dtype=torch.float32, device=q.device) if want_d0 else None
     dz0 = torch.empty((B, H, dk), dtype=torch.float32, device=q.device) if want_d0 else None
     st = lib.mrx_linear_attn_norm_bwd(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(done), _ptr(S_chk), _ptr(S_last), _ptr(z_chk),
-                                      _ptr(o), _ptr(den), _ptr(do), _ptr(dS_last), _ptr(dz_last), _ptr(dq),
+                                      _ptr(o), _ptr(den), _ptr(do), _ptr(d_ss), _ptr(dS_last), _ptr(dz_last), _ptr(dq),
                                       _ptr(dk_), _ptr(dv_), _ptr(dS0), _ptr(dz0), B, T, H, dk, dv, _DT[dt], dd,
                                       int(feature_map), float(eps))
     _lib.check(st, "mrx_linear_attn_norm_bwd")

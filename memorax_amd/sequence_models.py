@@ -76,15 +76,67 @@ class MemoroidCellBase(nn.Module):
 
     def scan(self, z, initial_carry, done):
         """Reset-aware inclusive scan of the cell's algebra over time, carry-in
-        prepended (memoroid.py:60-91).  Returns (h, next_carry)."""
-        raise NotImplementedError
+        prepended (memoroid.py:60-91).  Returns (h, next_carry).
+
+        The cells of this module override it with a fused kernel.  This default serves any other
+        cell that only defines ``binary_operator``: the same scan with array operations, on whatever
+        device the elements live on (``generic_scan``)."""
+        return generic_scan(self.binary_operator, z, initial_carry, done)
+
+
+def _tree_map(fn, tree, *rest):
+    """fn over the leaves of nested tuples / lists / dicts (named tuples keep their type)."""
+    if isinstance(tree, dict):
+        return {k: _tree_map(fn, v, *(r[k] for r in rest)) for k, v in tree.items()}
+    if isinstance(tree, (tuple, list)):
+        out = [_tree_map(fn, v, *(r[i] for r in rest)) for i, v in enumerate(tree)]
+        return type(tree)(*out) if hasattr(tree, "_fields") else type(tree)(out)
+    return fn(tree, *rest)
+
+
+def broadcast_done(done, carry):
+    """utils/axes.py:64-68: trailing axes added to (or dropped from) done until its rank is the leaf's."""
+    while done.dim() != carry.dim():
+        done = done[..., None] if done.dim() < carry.dim() else done[..., 0]
+    return done
+
+
+def generic_scan(binary_operator, z, initial_carry, done):
+    """Memoroid.scan_fn (memoroid.py:60-91) for an arbitrary pytree algebra.
+
+    The carry becomes slot 0 of every leaf with reset flag 0; slots are combined with the augmented
+    operator ``(where(reset_b, b, a (+) b), max(reset_a, reset_b))`` -- the right element wins by
+    *select* when its reset flag is set -- and the result is split into the T prefixes and the last
+    one (time axis of size 1).  Instead of jax.lax.associative_scan's odd/even recursion the slots
+    are combined by doubling: ceil(log2(T + 1)) rounds, each one call of ``binary_operator`` on leaves
+    of shape (B, n, ...) (n slots at once; the reference maps the operator over B, so it sees
+    (n, ...)); there is no host loop over time steps, and autograd differentiates through it.
+    Leaves are (B, T, ...); ``done`` is (B, T), bool or float."""
+    zz = _tree_map(lambda c, e: torch.cat([c, e], dim=1), initial_carry, z)
+    first = zz
+    while isinstance(first, (tuple, list, dict)):
+        first = next(iter(first.values())) if isinstance(first, dict) else first[0]
+    reset = torch.cat([done.new_zeros((done.shape[0], 1), dtype=torch.bool), done != 0], dim=1)[..., None]
+    n, shift = first.shape[1], 1
+    while shift < n:
+        left = _tree_map(lambda x: x[:, :-shift], zz)
+        right = _tree_map(lambda x: x[:, shift:], zz)
+        rr = reset[:, shift:]
+        comb = binary_operator(left, right)
+        comb = _tree_map(lambda r, c: torch.where(broadcast_done(rr, r), r, c), right, comb)
+        zz = _tree_map(lambda x, c: torch.cat([x[:, :shift], c], dim=1), zz, comb)
+        reset = torch.cat([reset[:, :shift], reset[:, :-shift] | rr], dim=1)
+        shift *= 2
+    return _tree_map(lambda x: x[:, 1:], zz), _tree_map(lambda x: x[:, -1:], zz)
 
 
 class Memoroid(SequenceModel):
-    """memoroid.py:57-112 (without the RTRL hooks).  Works for every cell of this module: the
-    matrix-state cells (linear attention, Mamba, mLSTM) put the query among their elements, because
-    their kernels fuse the read-out contraction into the scan, so that ``scan`` returns the carry
-    like any other cell's."""
+    """memoroid.py:57-112 (without the RTRL hooks).  The cells of this module scan with their fused
+    kernels: the matrix-state cells (linear attention, Mamba, mLSTM) put the query among their elements,
+    because their kernels fuse the read-out contraction into the scan, so that ``scan`` returns the
+    carry like any other cell's.  Any other MemoroidCellBase -- a user's cell that defines only
+    ``binary_operator`` -- is scanned by the base class's generic ``scan``, as the reference scans
+    every cell."""
 
     def __init__(self, cell: MemoroidCellBase):
         super().__init__()
@@ -363,13 +415,18 @@ class LinearAttentionCell(MemoroidCellBase):
         numerator (B,T,H,dv) and the carry (S (B,1,H,dv,dk), z (B,1,H,dk))."""
         v, k_raw, q = z
         S0, z0 = initial_carry
-        out, S_last, z_last = normalised_linear_attention(q, k_raw, v, done, S0[:, 0].float(), z0[:, 0].float(),
-                                                          "elu1", self.eps)
-        return out, (S_last[:, None], z_last[:, None])
+        out, S_last, z_last, ss = normalised_linear_attention(q, k_raw, v, done, S0[:, 0].float(), z0[:, 0].float(),
+                                                              "elu1", self.eps, return_ss=True)
+        return (out, ss), (S_last[:, None], z_last[:, None])
 
     def read(self, h, x, **kwargs):
-        out = h.float().reshape(*x.shape[:2], -1)
-        return self.output_projection(self.norm(out).to(x.dtype))
+        """linear_attention.py:109-117: RMS norm over the heads' concatenated outputs, then the output
+        projection.  The kernel has left each head's sum of squares beside its outputs, so the norm is
+        one rescale: out * rsqrt(sum_h ss / (H d) + eps) * scale."""
+        out, ss = h
+        inv = torch.rsqrt(ss.sum(-1) / (self.num_heads * self.head_dim) + self.norm.eps)   # (B,T)
+        y = out.float() * inv[..., None, None] * self.norm.scale.float().view(self.num_heads, self.head_dim)
+        return self.output_projection(y.reshape(*x.shape[:2], -1).to(x.dtype))
 
     def initialize_carry(self, key, input_shape):
         *batch, _ = input_shape

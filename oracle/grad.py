@@ -48,12 +48,21 @@ def diag_scan_t(a, b, done, h0, P0=None):
     return torch.stack(hs, 1), h, P
 
 
-def mingru_scan_t(z, h_tilde, done, h0=None):
+def mingru_scan_t(z, h_tilde, done, h0=None, side=None):
     """MinGRU in the reference's log space (elements min_gru.py:52-65, operator :67-74, read :76-78),
     folded sequentially with select resets (memoroid.py:79-83).  h0: linear-space carry (B,F) > 0,
-    or None for the cell's initial (-inf, 0).  Returns (h (B,T,F), h_last)."""
+    or None for the cell's initial (-inf, 0).  Returns (h (B,T,F), h_last).
+    side (bool, optional): which branch of g(x) = x + 0.5 (x >= 0) | sigmoid(x) each element takes,
+    when it is not to be decided by the sign of this evaluation's own h_tilde: a test that compares
+    gradients with a lower-precision evaluation passes the sides that evaluation saw, so that an
+    element within rounding of the kink (slope 1/4 against 1) is differentiated on the same branch
+    on both sides of the comparison.  The value moves by at most 3/4 |x| there."""
     sp = torch.nn.functional.softplus
-    log_b = -sp(-z) + torch.where(h_tilde >= 0, torch.log(torch.relu(h_tilde) + 0.5), -sp(-h_tilde))
+    if side is None:
+        log_g = torch.where(h_tilde >= 0, torch.log(torch.relu(h_tilde) + 0.5), -sp(-h_tilde))
+    else:
+        log_g = torch.where(side, torch.log(torch.where(side, h_tilde, torch.zeros_like(h_tilde)) + 0.5), -sp(-h_tilde))
+    log_b = -sp(-z) + log_g
     log_a = -sp(z)
     B, T, F = z.shape
     ls = torch.full((B, F), -float("inf"), dtype=z.dtype) if h0 is None else torch.log(h0)
@@ -83,7 +92,25 @@ def linear_attention_t(q, k, v, done, S0, feature_map="none"):
     return torch.stack(os_, 1), S
 
 
-def normalised_linear_attention_t(q, k, v, done, S0, z0, feature_map="elu1", eps=1e-6):
+class _DivideKeepingStoredQuotient(torch.autograd.Function):
+    """num / den whose backward takes the quotient from a given array instead of recomputing it:
+    d num = g / den, d den = -(g . o_stored) / den.  With o_stored the outputs as a lower-precision
+    implementation stored them (and reads them back in its backward), the gradients are those of that
+    implementation's own formula on the same information, so that a comparison is not charged with the
+    rounding of o, which cancellation in g . o can amplify."""
+
+    @staticmethod
+    def forward(ctx, num, den, o_stored):
+        ctx.save_for_backward(den, o_stored)
+        return num / den[..., None]
+
+    @staticmethod
+    def backward(ctx, g):
+        den, o = ctx.saved_tensors
+        return g / den[..., None], -(g * o).sum(-1) / den, None
+
+
+def normalised_linear_attention_t(q, k, v, done, S0, z0, feature_map="elu1", eps=1e-6, o_stored=None):
     if feature_map in ("elu1", 1):
         q, k = elu1_t(q), elu1_t(k)
     B, T, H, dk = q.shape
@@ -94,7 +121,8 @@ def normalised_linear_attention_t(q, k, v, done, S0, z0, feature_map="elu1", eps
         S = torch.where(r[:, None, None, None], torch.zeros_like(S), S) + torch.einsum("bhi,bhj->bhij", v[:, t], k[:, t])
         z = torch.where(r[:, None, None], torch.zeros_like(z), z) + k[:, t]
         den = torch.clamp((q[:, t] * z).sum(-1), min=eps)
-        os_.append(torch.einsum("bhij,bhj->bhi", S, q[:, t]) / den[..., None])
+        num = torch.einsum("bhij,bhj->bhi", S, q[:, t])
+        os_.append(num / den[..., None] if o_stored is None else _DivideKeepingStoredQuotient.apply(num, den, o_stored[:, t]))
     return torch.stack(os_, 1), S, z
 
 
@@ -168,19 +196,24 @@ def linear_attention_grads(q, k, v, done, S0, do, dS_last=None, feature_map="non
 
 
 def normalised_linear_attention_grads(q, k, v, done, S0, z0, do, dS_last=None, dz_last=None,
-                                      feature_map="elu1", eps=1e-6):
+                                      feature_map="elu1", eps=1e-6, d_ss=None, o_stored=None):
     """Returns dict(o, S_last, z_last, dq, dk, dv, dS0, dz0) for
-    L = sum(do*o) + sum(dS_last*S_last) + sum(dz_last*z_last)."""
+    L = sum(do*o) + sum(dS_last*S_last) + sum(dz_last*z_last) + sum(d_ss * ss), ss[b,t,h] = |o[b,t,h]|^2
+    (d_ss (B,T,H): the per-head sums of squares an RMS norm over the heads is built from).
+    o_stored (B,T,H,dv): see _DivideKeepingStoredQuotient."""
     q_, k_, v_ = _t(q, True), _t(k, True), _t(v, True)
     B, T, H, dk = q_.shape
     S0_ = _t(np.zeros((B, H, v_.shape[-1], dk)) if S0 is None else S0, True)
     z0_ = _t(np.zeros((B, H, dk)) if z0 is None else z0, True)
-    o, Sl, zl = normalised_linear_attention_t(q_, k_, v_, _done(done), S0_, z0_, feature_map, eps)
+    o, Sl, zl = normalised_linear_attention_t(q_, k_, v_, _done(done), S0_, z0_, feature_map, eps,
+                                              None if o_stored is None else _t(o_stored))
     L = (o * _t(do)).sum()
     if dS_last is not None:
         L = L + (Sl * _t(dS_last)).sum()
     if dz_last is not None:
         L = L + (zl * _t(dz_last)).sum()
+    if d_ss is not None:
+        L = L + ((o * o).sum(-1) * _t(d_ss)).sum()
     L.backward()
     return dict(o=_np(o), S_last=_np(Sl), z_last=_np(zl), dq=_np(q_.grad), dk=_np(k_.grad),
                 dv=_np(v_.grad), dS0=_np(S0_.grad), dz0=_np(z0_.grad))
@@ -241,7 +274,7 @@ def rms_norm_t(x, scale, eps=1e-6):
     return x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * scale
 
 
-def gated_linear_recurrence_t(x, done, Wz, Wh, Wg, Wo, carry=None):
+def gated_linear_recurrence_t(x, done, Wz, Wh, Wg, Wo, carry=None, side=None):
     """y = Wo( mingru(Wz x, Wh x) * silu(Wg x) ); carry = (log h_T, log of the cumulative decay since
     the last reset), both (B,1,F) as MinGRUCell.initialize_carry gives them (-inf, 0).
     Returns ((log_state, log_decay), y)."""
@@ -253,12 +286,27 @@ def gated_linear_recurrence_t(x, done, Wz, Wh, Wg, Wo, carry=None):
         h0, ld = torch.exp(carry[0][:, 0]), carry[1][:, 0]
         if bool(torch.isinf(carry[0]).all()):
             h0 = None
-    h, h_last = mingru_scan_t(z, ht, done, h0)
+    h, h_last = mingru_scan_t(z, ht, done, h0, side)
     log_a = -torch.nn.functional.softplus(z)
     for t in range(T):
         ld = torch.where(done[:, t][:, None], log_a[:, t], ld + log_a[:, t])
     y = (h * torch.nn.functional.silu(x @ Wg.T)) @ Wo.T
     return (torch.log(h_last)[:, None], ld[:, None]), y
+
+
+def linear_attention_cell_t(x, done, Wq, Wk, Wv, norm_scale, Wout, bout, H, carry=None, eps=1e-6):
+    """LinearAttentionCell (linear_attention.py:58-117): projections, phi = elu + 1 on keys and queries,
+    the additive recurrence with the key sum, read-out num / max(q . z, eps), RMSNorm over the heads'
+    concatenated outputs, output projection.  Returns ((S (B,1,H,d,d), z (B,1,H,d)), y)."""
+    B, T, _ = x.shape
+    heads = lambda t: t.reshape(B, T, H, -1)  # noqa: E731
+    q, k, v = heads(x @ Wq.T), heads(x @ Wk.T), heads(x @ Wv.T)
+    d = q.shape[-1]
+    S0 = torch.zeros(B, H, d, d, dtype=x.dtype) if carry is None else carry[0][:, 0]
+    z0 = torch.zeros(B, H, d, dtype=x.dtype) if carry is None else carry[1][:, 0]
+    o, S, z = normalised_linear_attention_t(q, k, v, done, S0, z0, "elu1", eps)
+    y = rms_norm_t(o.reshape(B, T, H * d), norm_scale) @ Wout.T + bout
+    return (S[:, None], z[:, None]), y
 
 
 def deltanet_cell_t(x, done, Wq, Wk, Wv, Wb, norm_scale, Wout, bout, H, S0=None):

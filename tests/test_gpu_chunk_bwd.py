@@ -183,3 +183,48 @@ def test_linear_attention_state_walk_back_over_a_long_sequence(dtype):
     # and the steps right after each reset, where the state has just restarted from zero
     for b_, t_ in ((0, 1500), (0, 1510), (0, 3000), (1, 2047)):
         assert relerr(got[0][b_, t_:t_ + 32], ref[0][b_, t_:t_ + 32]) <= tol, (b_, t_)
+
+
+@pytest.mark.parametrize("feature_map", [1, 0])
+def test_linear_attention_walk_back_16k_steps_without_a_reset(feature_map):
+    """The worst case for the walk: no reset in 16 384 steps and values with a positive mean, so that the
+    state grows linearly to some five hundred times what the first chunk sees.  Undone chunk by chunk all
+    the way from S_last, the rounding of the late state (about eps (T/C)^1.5 relative to the early one)
+    would exceed 1e-4 in fp32; the walk starts afresh from the exact state the forward call leaves every
+    32 chunks, and dq, dk of the first chunks -- on their own scale -- stay inside the tolerance."""
+    from memorax_amd import kernels as K
+    B, T, H = 1, 16384, 2
+    rng = np.random.default_rng(91)
+    q, k, do = ((rng.standard_normal((B, T, H, 64)) / 8).astype(np.float32) for _ in range(3))
+    v = (rng.standard_normal((B, T, H, 64)) / 8 + 0.5).astype(np.float32)
+    done = np.zeros((B, T), bool)
+    print(f"case la walk-back 16k fmap={feature_map}", flush=True)
+    tq, tk, tv, tdo = (dev(a) for a in (q, k, v, do))
+    o, Sl, chk = K.linear_attn_fwd(tq, tk, tv, dev(done), None, feature_map, chunk_parallel=False)
+    got = K.linear_attn_bwd(tq, tk, tv, dev(done), chk, tdo, None, feature_map)
+    ref = clib.linear_attn_bwd(q, k, v, done, None, do, None, feature_map)
+    for name, a, r in zip(("dq", "dk", "dv"), got, ref):
+        assert relerr(a, r) <= TOL_F32, name
+        for lo in (0, 32, 992, 1024, 4064):   # first chunks, and the chunks on either side of an anchor
+            assert relerr(a[:, lo:lo + 32], r[:, lo:lo + 32]) <= TOL_F32, (name, lo)
+
+
+def test_normalised_read_out_walks_across_an_anchor():
+    """The normalised read-out's backward shares the walk and its anchors: 1 300 fp32 steps cross the
+    anchor at chunk 32 (step 1 024) and end in a ragged chunk; gradients against torch-fp64 autograd.
+    (Zero-mean values: with a common mean the normalised output hardly depends on the query and dq is
+    what a cancellation leaves, in any implementation.)"""
+    from memorax_amd import kernels as K
+    B, T, H = 1, 1300, 1
+    rng = np.random.default_rng(92)
+    q, k, v, do = ((rng.standard_normal((B, T, H, 64)) / 8).astype(np.float32) for _ in range(4))
+    done = np.zeros((B, T), bool)
+    print("case la_norm walk-back across an anchor", flush=True)
+    tq, tk, tv, tdo = (dev(a) for a in (q, k, v, do))
+    on, den, Sl, zl, chkn = K.linear_attn_norm_fwd(tq, tk, tv, dev(done), None, None, 1)
+    gn = K.linear_attn_norm_bwd(tq, tk, tv, dev(done), chkn, on, den, tdo, None, None, 1)
+    rn = G.normalised_linear_attention_grads(q, k, v, done, None, None, do, None, None, "elu1")
+    for name, a in zip(("dq", "dk", "dv"), gn):
+        assert relerr(a, rn[name]) <= TOL_F32, name
+        for lo in (0, 992, 1024):
+            assert relerr(a[:, lo:lo + 32], rn[name][:, lo:lo + 32]) <= TOL_F32, (name, lo)

@@ -72,6 +72,61 @@ def test_normalised_bwd(shape, p, dtype):
     assert all(e <= tol for e in errs.values()), errs
 
 
+@pytest.mark.parametrize("shape", [(2, 128, 2), (1, 65, 2), (2, 200, 3), (1, 1, 1)])
+@pytest.mark.parametrize("p", [0.0, 0.05])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_sums_of_squares_out_of_the_epilogue_and_their_gradient(shape, p, dtype):
+    """ss[b,h,t] = |o[b,t,h]|^2 written by the forward kernel from its output tile (what the RMS norm
+    over the heads, linear_attention.py:114, needs from each head) equals the sum of squares of the
+    outputs as stored; and the backward call given d_ss returns the gradients of
+    L = <do, o> + <dS_last, S_last> + <dz_last, z_last> + <d_ss, ss> (torch-fp64 autograd)."""
+    from memorax_amd import kernels as K
+    B, T, H = shape
+    x = _inputs(B, T, H, p, B * 100 + T + H + 31, dtype)
+    rng = np.random.default_rng(5)
+    d_ss = rng.standard_normal((B, T, H)).astype(np.float32)
+    print(f"case la_norm_ss shape={shape} p={p} dtype={dtype}", flush=True)
+    td = _td(dtype)
+    tq, tk, tv, tdo = (dev(x[n], td) for n in ("q", "k", "v", "do"))
+    o, den, Sl, zl, chk, ss = K.linear_attn_norm_fwd(tq, tk, tv, dev(x["done"]), dev(x["S0"]), dev(x["z0"]), 1, 1e-6,
+                                                     want_ss=True)
+    assert ss.shape == (B, H, T) and ss.dtype == torch.float32
+    want = o.float().square().sum(-1).transpose(1, 2)      # of the outputs as stored
+    assert relerr(ss, want.cpu().numpy()) <= 1e-6
+    o2 = K.linear_attn_norm_fwd(tq, tk, tv, dev(x["done"]), dev(x["S0"]), dev(x["z0"]), 1, 1e-6)[0]
+    assert torch.equal(o, o2)                              # asking for ss changes nothing else
+    got = K.linear_attn_norm_bwd(tq, tk, tv, dev(x["done"]), chk, o, den, tdo, dev(x["dSl"]), dev(x["dzl"]), 1, 1e-6,
+                                 d_ss=dev(np.ascontiguousarray(d_ss.transpose(0, 2, 1))))
+    ref = G.normalised_linear_attention_grads(x["q"], x["k"], x["v"], x["done"], x["S0"], x["z0"], x["do"],
+                                              x["dSl"], x["dzl"], "elu1", 1e-6, d_ss=d_ss)
+    tol = TOL_BF16 if dtype == "bf16" else TOL_F32
+    errs = {n: relerr(g, ref[n]) for n, g in zip(("dq", "dk", "dv", "dS0", "dz0"), got)}
+    assert all(e <= tol for e in errs.values()), errs
+    # d_ss = 0 is the call without it
+    z = K.linear_attn_norm_bwd(tq, tk, tv, dev(x["done"]), chk, o, den, tdo, dev(x["dSl"]), dev(x["dzl"]), 1, 1e-6,
+                               d_ss=torch.zeros_like(ss))
+    n = K.linear_attn_norm_bwd(tq, tk, tv, dev(x["done"]), chk, o, den, tdo, dev(x["dSl"]), dev(x["dzl"]), 1, 1e-6)
+    for a, b_ in zip(z, n):
+        assert relerr(a, b_.float().cpu().numpy()) <= (4e-3 if dtype == "bf16" else 1e-6)
+
+
+def test_sums_of_squares_do_not_cross_episodes():
+    """A NaN in the outputs of one episode (poisoned values before a reset) leaves ss and every gradient
+    of the later episode finite: the d_ss term joins dout by select on live rows only."""
+    from memorax_amd import kernels as K
+    B, T, H = 1, 96, 1
+    x = _inputs(B, T, H, 0.0, 77, "f32")
+    x["done"][0, 40] = True
+    x["v"][0, 10] = np.nan
+    tq, tk, tv, tdo = (dev(x[n]) for n in ("q", "k", "v", "do"))
+    o, den, Sl, zl, chk, ss = K.linear_attn_norm_fwd(tq, tk, tv, dev(x["done"]), None, None, 1, 1e-6, want_ss=True)
+    assert torch.isfinite(ss[0, 0, 40:]).all() and torch.isnan(ss[0, 0, 10:40]).all()
+    d_ss = torch.ones_like(ss)
+    got = K.linear_attn_norm_bwd(tq, tk, tv, dev(x["done"]), chk, o, den, tdo, None, None, 1, 1e-6, d_ss=d_ss)
+    for g in got[:3]:
+        assert torch.isfinite(g[0, 40:]).all()
+
+
 def test_normalised_clamp_and_plain_feature_map():
     """No feature map, so that denominators of either sign occur: rows under the clamp take
     den = eps and pass no gradient through the denominator.  fp32 only: the seed keeps every

@@ -73,7 +73,12 @@ def test_random_cases(seed):
         elif op == "norm":
             o, den, Sl, zl, chk = K.linear_attn_norm_fwd(tq, tk, tv, dn, tS0, dev(z0), 1, 1e-6)
             got = K.linear_attn_norm_bwd(tq, tk, tv, dn, chk, o, den, tdo, tdSl, None, 1, 1e-6)
-            ref = G.normalised_linear_attention_grads(q, k, v, done, S0, z0, do, dSl, None, "elu1", 1e-6)
+            # The backward call reads the quotient o back as the forward call stored it (bf16) and forms
+            # dden = -(dout . o) / den from it, a sum that can cancel; the oracle differentiates the divide on
+            # the same stored o (values are still compared with its own exact quotient), so that the
+            # tolerance is not charged with the rounding of a residual.
+            o_st = o.float().cpu().numpy().astype(np.float64) if dtype == "bf16" else None
+            ref = G.normalised_linear_attention_grads(q, k, v, done, S0, z0, do, dSl, None, "elu1", 1e-6, o_stored=o_st)
             names = ("dq", "dk", "dv", "dS0", "dz0")
         else:
             pro = op == "deltanet"
@@ -87,12 +92,17 @@ def test_random_cases(seed):
         for n, a in zip(names, got):
             if a is None or (B * T * H < 4 and n in ("dbeta", "dg")):  # a lone scalar has no scale to be judged against
                 continue
-            # a gradient that is exactly zero in the oracle (dg at reset steps only, say) has no scale of its own
-            scale = max(np.abs(ref[n]).max(), 1e-3 * max(np.abs(ref["dq"]).max(), 1e-30))
-            errs[n] = float(np.abs(a.float().cpu().numpy() - ref[n]).max() / scale)
-        # the normalised read-out divides by a bf16-rounded denominator: its gradients carry that rounding twice
-        lim = tol * (1.5 if op == "norm" and dtype == "bf16" else 1.0)
-        bad = {n: e for n, e in errs.items() if not e <= lim}
+            an, top = a.float().cpu().numpy(), np.abs(ref[n]).max()
+            if top == 0.0:
+                # a gradient that is exactly zero in the oracle (dg of a one-step sequence without an initial
+                # state, say) has no scale of its own: what the kernel returns must be rounding noise of the
+                # products behind it, bounded absolutely by their operands: eps(dtype) |dout|_max |q|_max |k|_max d
+                bound = (2.0 ** -8 if dtype == "bf16" else 2.0 ** -23) * np.abs(do).max() * max(np.abs(q).max(), 1.0) * \
+                    max(np.abs(k).max(), 1.0) * q.shape[-1]
+                errs[n] = 0.0 if np.abs(an).max() <= bound else float("inf")
+            else:
+                errs[n] = float(np.abs(an - ref[n]).max() / top)
+        bad = {n: e for n, e in errs.items() if not e <= tol}
         if bad:
             failures.append((desc, bad))
     assert not failures, failures

@@ -88,6 +88,45 @@ def test_linear_attention_model_matches_reference_readout():
     assert torch.isfinite(cell.query.weight.grad).all() and cell.key.weight.grad.abs().sum() > 0
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 2e-2)], ids=["f32", "bf16"])
+def test_linear_attention_cell_full_read_out_values_and_every_gradient(dtype, tol):
+    """LinearAttentionCell end to end (linear_attention.py:58-117): the recurrence, the divide, the RMS
+    norm over the heads -- built from the per-head sums of squares the kernel leaves beside its outputs --
+    and the output projection, against the torch-fp64 restatement: outputs, both carry leaves, the input
+    gradient and every parameter gradient; then split invariance through the carry."""
+    from memorax_amd import sequence_models as sm
+    from oracle import grad as G
+    torch.manual_seed(21)
+    B, T, Fe, H, d = 2, 150, 32, 2, 64
+    cell = sm.LinearAttentionCell(Fe, d, H).cuda()
+    with torch.no_grad():
+        cell.norm.scale.copy_(torch.rand(H * d) + 0.5)
+    model = sm.LinearAttention(cell)
+    x, done = _inputs(B, T, Fe, 0.03, 22)
+    x.requires_grad_()
+    gy = torch.randn(B, T, Fe, generator=torch.Generator().manual_seed(23)).cuda()
+    print(f"case la_cell dtype={dtype}", flush=True)
+    with torch.autocast("cuda", dtype=torch.bfloat16, enabled=dtype == torch.bfloat16):
+        carry, y = model(x, done)
+    (y.float() * gy).sum().backward()
+    ps = [_f64(p_).requires_grad_() for p_ in (cell.query.weight, cell.key.weight, cell.value.weight, cell.norm.scale,
+                                              cell.output_projection.weight, cell.output_projection.bias)]
+    xr = _f64(x).requires_grad_()
+    rc, ry = G.linear_attention_cell_t(xr, done.cpu(), *ps, H)
+    (ry * _f64(gy)).sum().backward()
+    assert relerr(y, ry.detach().numpy()) <= tol
+    assert relerr(carry[0], rc[0].detach().numpy()) <= tol and relerr(carry[1], rc[1].detach().numpy()) <= tol
+    assert relerr(x.grad, xr.grad.numpy()) <= tol
+    for p_, r_, n_ in zip((cell.query.weight, cell.key.weight, cell.value.weight, cell.norm.scale,
+                           cell.output_projection.weight, cell.output_projection.bias), ps,
+                          ("query", "key", "value", "norm.scale", "out.weight", "out.bias")):
+        assert relerr(p_.grad, r_.grad.numpy()) <= tol, n_
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16, enabled=dtype == torch.bfloat16):
+        c1, y1 = model(x[:, :70], done[:, :70])
+        c2, y2 = model(x[:, 70:], done[:, 70:], c1)
+    assert relerr(torch.cat([y1, y2], 1), y.detach().float().cpu().numpy()) <= tol
+
+
 def test_deltanet_stack_carries_and_split_invariance():
     from memorax_amd import sequence_models as sm
     torch.manual_seed(3)
@@ -368,9 +407,11 @@ def _torso(sm, Fe, H, d, nblocks, dtype, std):
     return torso
 
 
-def _torso_reference(G, torso, x, done, carries, H):
+def _torso_reference(G, torso, x, done, carries, H, sides=None):
     """The same stack in torch fp64 from the oracle's parts; parameters are fp64 leaf copies.
-    Returns (carries, y, params) with params a list parallel to torso.parameters()."""
+    Returns (carries, y, params) with params a list parallel to torso.parameters().
+    sides: per recurrence block, which branch of MinGRU's g the modules under test took for each
+    candidate pre-activation (oracle.grad.mingru_scan_t)."""
     params = [_f64(p).requires_grad_() for p in torso.parameters()]
     it = iter(params)
     out_carries = []
@@ -385,7 +426,8 @@ def _torso_reference(G, torso, x, done, carries, H):
                                        None if c is None else c[0])
         else:
             Wz, Wh, Wg, Wo, pn = (next(it) for _ in range(5))
-            nc, yb = G.gated_linear_recurrence_t(G.rms_norm_t(x, pn), done, Wz, Wh, Wg, Wo, c)
+            nc, yb = G.gated_linear_recurrence_t(G.rms_norm_t(x, pn), done, Wz, Wh, Wg, Wo, c,
+                                                 None if sides is None else sides[i // 2])
         x = x + yb
         out_carries.append(nc)
     return tuple(out_carries), x, params
@@ -416,10 +458,21 @@ def test_torso_stack_of_four_blocks_against_the_fp64_restatement(dtype, tol, std
     x.requires_grad_()
     gy = torch.randn(B, T, Fe, generator=torch.Generator().manual_seed(53)).cuda()
     print(f"case torso dtype={dtype}", flush=True)
+    # MinGRU's g(x) = x + 0.5 (x >= 0) | sigmoid(x) has a kink at 0 (slope 1/4 -> 1).  With bf16 cells upstream
+    # the candidate pre-activations differ from the fp64 ones by ~3e-3 at a spread of 0.3, so about one in a
+    # hundred sits on the other side of the kink, and the gradient of W_h -- a random-sign sum over tokens of
+    # terms carrying that slope -- would differ by some 10 %: a property of the function.  The restatement is
+    # therefore evaluated on the branches the modules themselves took (their own pre-activations, captured
+    # here), and every gradient is held to the one tolerance.
+    sides, hooks = [], []
+    for blk in torso.blocks[1::2]:
+        hooks.append(blk.module.module.cell.h.register_forward_hook(lambda m, i, out: sides.append((out.detach() >= 0).cpu())))
     carries, y = torso(x, done)
+    for h_ in hooks:
+        h_.remove()
     (y * gy).sum().backward()
     xr = _f64(x).requires_grad_()
-    rcar, ry, rparams = _torso_reference(G, torso, xr, done.cpu(), None, H)
+    rcar, ry, rparams = _torso_reference(G, torso, xr, done.cpu(), None, H, sides)
     (ry * _f64(gy)).sum().backward()
     assert relerr(y, ry.detach().numpy()) <= tol, relerr(y, ry.detach().numpy())
     assert len(carries) == 8
@@ -435,13 +488,7 @@ def test_torso_stack_of_four_blocks_against_the_fp64_restatement(dtype, tol, std
     for n, p, rp in zip(names, torso.parameters(), rparams):
         worst[n] = relerr(p.grad, rp.grad.numpy())
     print("largest gradient errors:", sorted(worst.items(), key=lambda kv: -kv[1])[:4], flush=True)
-    # MinGRU's g(x) = x + 0.5 (x >= 0) | sigmoid(x) has a kink at 0 (slope 1/4 -> 1).  With bf16 cells upstream the
-    # candidate pre-activations differ from the fp64 ones by ~3e-3 at a spread of 0.3, so about one in
-    # a hundred sits on the other side of the kink; the gradient of W_h is a random-sign sum over tokens
-    # of terms carrying that slope, and moves by sqrt(fraction) * 3/4 ~ 10 %.  A property of the function,
-    # not of the kernels: the fp32 case holds the same weights to 2e-3.
-    kink = (lambda n: n.endswith("cell.h.weight")) if dtype == torch.bfloat16 else (lambda n: False)
-    bad = {n: e for n, e in worst.items() if e > (0.25 if kink(n) else tol)}
+    bad = {n: e for n, e in worst.items() if e > tol}
     assert not bad, bad
     # split invariance through the carry tuple
     with torch.no_grad():

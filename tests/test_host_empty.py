@@ -7,6 +7,19 @@ import torch
 from memorax_amd import functional as F
 
 
+@pytest.mark.parametrize("B,T", [(0, 5), (3, 0)])
+def test_bf16_scans_without_steps_carry_float32_like_the_kernels(B, T):
+    D = 8
+    a, b = torch.rand(B, T, D).bfloat16(), torch.randn(B, T, D).bfloat16()
+    done = torch.zeros(B, T, dtype=torch.bool)
+    for op in (F.linear_scan, F.mingru_scan):
+        h, h_last, P_last = op(a, b, done)
+        assert h.dtype == torch.bfloat16 and h_last.dtype == torch.float32 and P_last.dtype == torch.float32
+        h0, P0 = torch.randn(B, D), torch.rand(B, D)
+        h, h_last, P_last = op(a, b, done, h0, P0)
+        assert h_last.dtype == torch.float32 and torch.equal(h_last, h0) and torch.equal(P_last, P0)
+
+
 @pytest.mark.parametrize("B,T", [(0, 5), (3, 0), (0, 0)])
 def test_scans_without_steps_return_the_carry(B, T):
     D = 6

@@ -281,3 +281,80 @@ def test_torso_parts_of_the_gradient_oracle():
     o = o.reshape(B, T, H * d)
     o = o / np.sqrt((o ** 2).mean(-1, keepdims=True) + 1e-6) * ns
     assert np.allclose(yd.numpy(), o @ Wout.T + bout, atol=1e-11) and np.allclose(S.numpy()[:, 0], Sl, atol=1e-12)
+
+
+def test_sum_of_squares_gradient_stored_quotient_and_g_side_options():
+    """The three options the GPU comparisons use.  d_ss: the term <d_ss, |o|^2> of the loss, by finite
+    differences.  o_stored: with the exact outputs it changes nothing; with perturbed ones only the
+    denominator's share of the gradients moves, by -(g . delta o) / den.  side: equal to the default
+    when it is the sign of h_tilde; an element within 1e-3 of the kink forced to the other branch moves
+    the values by at most 3/4 |x| and is differentiated with that branch's slope."""
+    import torch
+    B, T, H, dk, dv = 1, 6, 2, 3, 2
+    r = np.random.default_rng(4)
+    rnd = lambda *s: r.standard_normal(s)  # noqa: E731
+    q, k, v, S0 = rnd(B, T, H, dk), rnd(B, T, H, dk), rnd(B, T, H, dv), rnd(B, H, dv, dk)
+    z0 = np.abs(rnd(B, H, dk))
+    do, d_ss = rnd(B, T, H, dv), rnd(B, T, H)
+    d = np.zeros((B, T), bool)
+    d[0, 2] = True
+
+    def L():
+        o, den, Sl, zl = M.normalised_linear_attention(q, k, v, d, S0, z0, "elu1", 1e-6)
+        return (o * do).sum() + ((o * o).sum(-1) * d_ss).sum()
+
+    ag = G.normalised_linear_attention_grads(q, k, v, d, S0, z0, do, None, None, "elu1", 1e-6, d_ss=d_ss)
+    for name, x in (("dq", q), ("dk", k), ("dv", v), ("dS0", S0), ("dz0", z0)):
+        np.testing.assert_allclose(ag[name], fd(L, x), rtol=1e-5, atol=1e-7, err_msg=name)
+    same = G.normalised_linear_attention_grads(q, k, v, d, S0, z0, do, None, None, "elu1", 1e-6, d_ss=d_ss, o_stored=ag["o"])
+    for name in ("dq", "dk", "dv", "dS0", "dz0"):
+        np.testing.assert_allclose(same[name], ag[name], rtol=1e-12, atol=1e-13, err_msg=name)
+    base = G.normalised_linear_attention_grads(q, k, v, d, S0, z0, do)
+    off = G.normalised_linear_attention_grads(q, k, v, d, S0, z0, do, o_stored=base["o"] + 0.01)
+    np.testing.assert_allclose(off["dv"], base["dv"], rtol=1e-12, atol=1e-13)   # values never see the denominator
+    assert np.abs(off["dq"] - base["dq"]).max() > 1e-4                           # queries do
+
+    z, ht = rnd(2, 7, 3), rnd(2, 7, 3)
+    ht[0, 3, 1], ht[1, 5, 0] = 4e-4, -7e-4
+    done = np.zeros((2, 7), bool)
+    t = lambda a: torch.from_numpy(a)  # noqa: E731
+    h_def, _ = G.mingru_scan_t(t(z), t(ht), t(done))
+    h_same, _ = G.mingru_scan_t(t(z), t(ht), t(done), side=t(ht >= 0))
+    assert torch.equal(h_def, h_same)
+    side = ht >= 0
+    side[0, 3, 1], side[1, 5, 0] = False, True
+    htt = t(ht).requires_grad_()
+    h_flip, _ = G.mingru_scan_t(t(z), htt, t(done), side=t(side))
+    assert (h_flip - h_def).abs().max() <= 0.75 * 7e-4
+    h_flip[:, -1].sum().backward()
+    htd = t(ht).requires_grad_()
+    G.mingru_scan_t(t(z), htd, t(done))[0][:, -1].sum().backward()
+    ratio = (htt.grad / htd.grad).numpy()
+    assert abs(ratio[0, 3, 1] - 0.25) < 2e-3 and abs(ratio[1, 5, 0] - 4.0) < 2e-2   # slope 1/4 <-> 1
+    mask = np.ones_like(ratio, bool)
+    mask[0, 3, 1] = mask[1, 5, 0] = False
+    np.testing.assert_allclose(ratio[mask], 1.0, rtol=2e-3)
+
+
+def test_linear_attention_cell_of_the_gradient_oracle():
+    """linear_attention_cell_t against the NumPy composition: the reference's materialise-and-scan
+    route for numerator and denominator (linear_attention.py:62-110), RMS norm over the heads, projection."""
+    import torch
+    rng = np.random.default_rng(78)
+    B, T, Fe, H, d = 2, 17, 5, 2, 3
+    x = rng.standard_normal((B, T, Fe))
+    done = rng.random((B, T)) < 0.15
+    Wq, Wk, Wv = (rng.standard_normal((H * d, Fe)) for _ in range(3))
+    ns, Wout, bout = rng.uniform(0.5, 1.5, H * d), rng.standard_normal((Fe, H * d)), rng.standard_normal(Fe)
+    t = torch.from_numpy
+    (S, z), y = G.linear_attention_cell_t(t(x), t(done), t(Wq), t(Wk), t(Wv), t(ns), t(Wout), t(bout), H)
+    hv = lambda w: (x @ w.T).reshape(B, T, H, d)  # noqa: E731
+    nxt, num, den = M.linear_attention_memoroid(hv(Wq), hv(Wk), hv(Wv), done.astype(np.float64), None, "elu1")
+    out = (num / np.maximum(den, 1e-6)[..., None]).reshape(B, T, H * d)
+    out = out / np.sqrt((out ** 2).mean(-1, keepdims=True) + 1e-6) * ns
+    assert np.allclose(y.numpy(), out @ Wout.T + bout, atol=1e-11)
+    assert np.allclose(S.numpy(), nxt[0], atol=1e-12) and np.allclose(z.numpy(), nxt[1], atol=1e-12)
+    s = 6
+    c1, y1 = G.linear_attention_cell_t(t(x[:, :s]), t(done[:, :s]), t(Wq), t(Wk), t(Wv), t(ns), t(Wout), t(bout), H)
+    c2, y2 = G.linear_attention_cell_t(t(x[:, s:]), t(done[:, s:]), t(Wq), t(Wk), t(Wv), t(ns), t(Wout), t(bout), H, c1)
+    assert np.allclose(np.concatenate([y1.numpy(), y2.numpy()], 1), y.numpy(), atol=1e-11)
