@@ -260,15 +260,17 @@ def test_normalised_rejects_bad_arguments():
     lib = _lib.load()
     t = torch.zeros(64 * 64 * 4, device="cuda")
     p = t.data_ptr()
-    fwd = lambda den, dk, dt: lib.mrx_linear_attn_norm_fwd(None, p, p, p, p, None, None, p, den, None, None, None,
-                                                           None, 1, 4, 1, dk, 64, dt, 0, 1, 1e-6)
+    fwd = lambda den, dk, dt, ss=None: lib.mrx_linear_attn_norm_fwd(None, p, p, p, p, None, None, p, den, ss, None, None, None,
+                                                                    None, 1, 4, 1, dk, 64, dt, 0, 1, 1e-6)
     assert fwd(p, 64, 0) == 0
     assert fwd(None, 64, 0) == -1     # den is required
     assert fwd(p, 72, 0) == -2        # unsupported head dim
     assert fwd(p, 64, 2) == -2        # complex64
-    bwd = lambda zc: lib.mrx_linear_attn_norm_bwd(None, p, p, p, p, p, p, zc, p, p, p, None, None, p, p, p, None, None,
-                                                  1, 4, 1, 64, 64, 0, 0, 1, 1e-6)
+    assert fwd(p, 64, 0, p + 2) == -1  # ss must be aligned to its element size
+    bwd = lambda zc, dss=None: lib.mrx_linear_attn_norm_bwd(None, p, p, p, p, p, p, zc, p, p, p, dss, None, None, p, p, p,
+                                                            None, None, 1, 4, 1, 64, 64, 0, 0, 1, 1e-6)
     assert bwd(None) == -1            # z_chk is required
+    assert bwd(p, p + 2) == -1        # d_ss must be aligned to its element size
     torch.cuda.synchronize()
 
 
