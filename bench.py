@@ -89,6 +89,9 @@ def main() -> int:
     ap.add_argument("--phase-clocks", action="store_true",
                     help="with --lib <the measurement build>: run the headline backward and print the share of "
                          "a wave's cycles spent inside matrix products (child process of the default run)")
+    ap.add_argument("--no-children", action="store_true",
+                    help="skip the two measurements that run in child processes (64-step-chunk build, product-phase "
+                         "clocks): under a profiler the children would be traced into the same output")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain elementwise kernel of known size (256 MiB read, 256 MiB "
                          "written) so that a rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE run can be scaled")
@@ -124,7 +127,8 @@ def main() -> int:
             secondary["torso"].update(bench_torso_full(torch, K))
             secondary["step"] = bench_step(torch, K)
             secondary["rtrl"] = bench_rtrl(torch, K)
-        secondary["delta_rule_chunk64"] = bench_delta_chunk64()
+        if not args.no_children:
+            secondary["delta_rule_chunk64"] = bench_delta_chunk64()
         torch.cuda.empty_cache()
     if args.calibrate:
         cx = torch.zeros(64 * 1024 * 1024, device="cuda")  # 256 MiB fp32
@@ -226,7 +230,8 @@ def main() -> int:
         },
     }
     if not args.headline_only:
-        out["roofline"].update(bench_gemm_phase(MFMA_BUSY_BWD))
+        if not args.no_children:
+            out["roofline"].update(bench_gemm_phase(MFMA_BUSY_BWD))
         if "hbm_copy" in secondary:
             out["roofline"]["hbm_copy_GB/s"] = secondary["hbm_copy"]["GB/s"]
             out["roofline"]["frac_of_copy_rate"] = bwd_gbs / secondary["hbm_copy"]["GB/s"]
@@ -601,23 +606,29 @@ def bench_torso_kernels(torch, K):
     do = torch.randn_like(v)
     z, hx, g = (torch.randn(B, T, Fe, device="cuda") for _ in range(3))
 
-    def kernels_only(prologue):
+    def kernels_only(prologue, resets=None):
         kk, bb = (k_raw, b_raw) if prologue else (k_unit, beta)
         for _ in range(4):
-            o, Sl, chk = K.delta_rule_fwd(q, kk, v, bb, done, prologue=prologue)
-            K.delta_rule_bwd(q, kk, v, bb, done, chk, do, None, want_dS0=False, prologue=prologue)
+            o, Sl, chk = K.delta_rule_fwd(q, kk, v, bb, done, prologue=prologue, reset_path=resets)
+            K.delta_rule_bwd(q, kk, v, bb, done, chk, do, None, want_dS0=False, prologue=prologue, reset_path=resets)
             h, _, _ = K.mingru_scan_fwd(z, hx, done, want_P=False)
             K.mingru_scan_bwd(z, hx, h, done, None, g)
     ms_k = _time_ms(torch, lambda: kernels_only(True), iters=10, warm=3)
     ms_p = _time_ms(torch, lambda: kernels_only(False), iters=10, warm=3)
+    # episodes end every hundred steps here: the caller's choice of MRX_RESETS_MERGED (all episodes of a chunk in
+    # one unit of work, behind a screen of the chunk's inputs) against the default of one unit per episode
+    ms_m = _time_ms(torch, lambda: kernels_only(True, "merged"), iters=10, warm=3)
     # the same with the recurrence's arrays in bfloat16 (what a bf16 torso hands over; float32 arithmetic and
     # carries inside the kernels): half the bytes of the scans
     z, hx, g = (t.to(bf) for t in (z, hx, g))
     ms_h = _time_ms(torch, lambda: kernels_only(True), iters=10, warm=3)
+    ms_hm = _time_ms(torch, lambda: kernels_only(True, "merged"), iters=10, warm=3)
     by = 4 * ((BYTES_FWD + BYTES_BWD) * B * T * H + 36 * B * T * Fe)   # + MinGRU scan: 12 B fwd, 24 B bwd per element
     return {"sequence_kernels_ms": ms_k, "sequence_kernels_tokens/s": B * T / ms_k * 1e3,
             "sequence_kernels_GB/s": by / ms_k / 1e6, "sequence_kernels_frac_hbm": by / ms_k / 1e6 / HBM_PEAK_GBS,
+            "sequence_kernels_ms_merged_resets": ms_m, "sequence_kernels_tokens/s_merged_resets": B * T / ms_m * 1e3,
             "sequence_kernels_ms_plain_delta_rule": ms_p, "sequence_kernels_ms_bf16_recurrence_arrays": ms_h,
+            "sequence_kernels_ms_bf16_recurrence_arrays_merged_resets": ms_hm,
             "sequence_kernels_tokens/s_bf16_recurrence_arrays": B * T / ms_h * 1e3,
             "sequence_kernels_frac_hbm_bf16_recurrence_arrays":
                 4 * ((BYTES_FWD + BYTES_BWD) * B * T * H + 18 * B * T * Fe) / ms_h / 1e6 / HBM_PEAK_GBS}

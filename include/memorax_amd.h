@@ -66,6 +66,27 @@ typedef enum {
     MRX_FACTORS_INLINE = 2    /* inverted inside the sequential kernel */
 } mrx_factor_path;
 
+/* How the delta-rule kernels treat a chunk that holds episode resets.
+ * MRX_RESETS_PASSES: one unit of work per episode of the chunk, the rows of the other episodes replaced by
+ *   zeros by select -- exact whatever the data (a NaN or Inf of one episode never reaches another).
+ * MRX_RESETS_MERGED: one unit per chunk, the episodes kept apart by masks inside it.  A masked zero then
+ *   multiplies values of other episodes, which is exact while those are finite; the kernels therefore screen
+ *   every such chunk first (|q|, |k|, |v|, |beta|, |dout| and the factor's entries <= 2^6, the state's and its
+ *   gradient's <= 2^20: bounds under which no intermediate can leave the float32 range) and fall back to
+ *   the units per episode for a chunk that fails, so the results are those of MRX_RESETS_PASSES for any data.
+ *   For callers whose episodes end every hundred steps or so (ppo.py:181-190): a chunk with a reset
+ *   then costs what a chunk without one costs (measured, B=64 T=1024 H=8 bf16 at one reset per hundred steps:
+ *   backward 201 -> 170 us; at one per five hundred the two are level, without resets the merged instance
+ *   is 4 % behind).  The forward call merges where it takes the chunk-parallel factor kernel
+ *   (mrx_factor_path), the backward call always; head dim 64 at full width, 32-row chunks -- elsewhere the
+ *   argument is accepted and the units per episode run.  The two calls of a pair need not agree.
+ * MRX_RESETS_AUTO: MRX_RESETS_PASSES. */
+typedef enum {
+    MRX_RESETS_AUTO = 0,
+    MRX_RESETS_PASSES = 1,
+    MRX_RESETS_MERGED = 2
+} mrx_reset_path;
+
 const char *mrx_status_string(int status);
 
 /* Per-device set-up: raises the dynamic-LDS limit of every kernel that needs more than the
@@ -248,7 +269,7 @@ int mrx_delta_rule_fwd(void *stream, const void *q, const void *k,
                        const void *v, const void *beta, const void *done,
                        const void *S0, void *o, void *S_last, void *S_chk,
                        void *Tm_chk, int64_t B, int64_t T, int64_t H, int64_t dk,
-                       int64_t dv, int dtype, int done_dtype, int factor_path);
+                       int64_t dv, int dtype, int done_dtype, int factor_path, int reset_path);
 
 /* mrx_delta_rule_fwd without residuals for callers that cannot allocate device memory (code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the triangular
@@ -276,7 +297,7 @@ int mrx_delta_rule_bwd(void *stream, const void *q, const void *k,
                        const void *S_chk, const void *Tm_chk, const void *dout,
                        const void *dS_last, void *dq, void *dk_out, void *dv_out,
                        void *dbeta, void *dS0, int64_t B, int64_t T, int64_t H,
-                       int64_t dk, int64_t dv, int dtype, int done_dtype);
+                       int64_t dk, int64_t dv, int dtype, int done_dtype, int reset_path);
 
 /* ---- DeltaNet cell recurrence with its prologue fused -------------------------
  * As mrx_delta_rule_fwd / _bwd, but on the raw projections: inside the kernels
@@ -290,14 +311,14 @@ int mrx_deltanet_fwd(void *stream, const void *q, const void *k, const void *v,
                      const void *beta_raw, const void *done, const void *S0, void *o,
                      void *S_last, void *S_chk, void *Tm_chk, int64_t B, int64_t T,
                      int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype,
-                     int factor_path);
+                     int factor_path, int reset_path);
 
 int mrx_deltanet_bwd(void *stream, const void *q, const void *k, const void *v,
                      const void *beta_raw, const void *done, const void *S_chk,
                      const void *Tm_chk, const void *dout, const void *dS_last, void *dq,
                      void *dk_out, void *dv_out, void *dbeta_raw, void *dS0, int64_t B,
                      int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
-                     int done_dtype);
+                     int done_dtype, int reset_path);
 
 /* Final state only, one decay per `a_group` consecutive channels: h_T of
  *     h_t = done_t ? b_t : a_t h_{t-1} + b_t ,  a: (B,T,D/a_group), b: (B,T,D), h0 (nullable), h_last: (B,D).

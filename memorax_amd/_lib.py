@@ -16,6 +16,7 @@ MRX_DONE_U8, MRX_DONE_F32 = 0, 1
 MRX_FMAP_NONE, MRX_FMAP_ELU1 = 0, 1
 MRX_A_TIME_INVARIANT_SUM_DA = 2
 MRX_FACTORS_AUTO, MRX_FACTORS_PARALLEL, MRX_FACTORS_INLINE = 0, 1, 2
+MRX_RESETS_AUTO, MRX_RESETS_PASSES, MRX_RESETS_MERGED = 0, 1, 2
 MRX_NOALLOC_SCRATCH_BYTES = 32 << 20
 
 _P = ctypes.c_void_p
@@ -38,11 +39,11 @@ SIGNATURES = {
     "mrx_linear_attn_chunk_parallel_pays": (_I, [_L] * 3 + [_I]),
     "mrx_linear_attn_norm_fwd": (_I, [_P] * 14 + [_L] * 5 + [_I] * 3 + [ctypes.c_float]),
     "mrx_linear_attn_norm_bwd": (_I, [_P] * 19 + [_L] * 5 + [_I] * 3 + [ctypes.c_float]),
-    "mrx_delta_rule_fwd": (_I, [_P] * 11 + [_L] * 5 + [_I] * 3),
+    "mrx_delta_rule_fwd": (_I, [_P] * 11 + [_L] * 5 + [_I] * 4),
     "mrx_delta_rule_fwd_noalloc": (_I, [_P] * 9 + [_L] * 5 + [_I] * 2),
-    "mrx_delta_rule_bwd": (_I, [_P] * 15 + [_L] * 5 + [_I] * 2),
-    "mrx_deltanet_fwd": (_I, [_P] * 11 + [_L] * 5 + [_I] * 3),
-    "mrx_deltanet_bwd": (_I, [_P] * 15 + [_L] * 5 + [_I] * 2),
+    "mrx_delta_rule_bwd": (_I, [_P] * 15 + [_L] * 5 + [_I] * 3),
+    "mrx_deltanet_fwd": (_I, [_P] * 11 + [_L] * 5 + [_I] * 4),
+    "mrx_deltanet_bwd": (_I, [_P] * 15 + [_L] * 5 + [_I] * 3),
     "mrx_linear_scan_last": (_I, [_P] * 6 + [_L] * 4 + [_I] * 2),
     "mrx_mingru_scan_fwd": (_I, [_P] * 9 + [_L] * 3 + [_I] * 2),
     "mrx_mingru_scan_bwd": (_I, [_P] * 11 + [_L] * 3 + [_I] * 2),

@@ -343,9 +343,9 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
         const int t0 = c * C;
         const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
-        const bool ckpt = PAR || !WALK || nres != 0 || c % walk_anchor<T>() == 0;  // the entering state comes from S_chk
+        const bool ckpt = PAR || !WALK || nres != 0 || (c > 0 && c % walk_anchor<T>() == 0);  // the entering state comes from S_chk
         if (WALK && !PAR)  // for the chunk prefetched during this one
-            need_S = __ballot(done_test(rdone2, done_f32) && lane < C) != 0ull || (c >= 1 && (c - 1) % walk_anchor<T>() == 0);
+            need_S = __ballot(done_test(rdone2, done_f32) && lane < C) != 0ull || (c >= 2 && (c - 1) % walk_anchor<T>() == 0);
         for (int pass = nres; pass >= 0; --pass) {
             auto live = [&](int r) { return nres == 0 || episode_of(dmask, r) == pass; };
             // gated: cumulative log-decay of this pass's episode (as in the forward kernel)
@@ -694,7 +694,8 @@ template <typename T, int C, int NW> struct DeltaBwdSmem : BwdDims<T, C> {
     static constexpr int NSLOT = TileMap<HD, C, NW>::WM;  // dbeta partials per row: one per feature block
     // prologue variant: 1 / |k| per row, then [NSLOT][C] partials of k_n . dk_n
     static constexpr int oKinv = oDb + NSLOT * C * 4;
-    static constexpr int total = oKinv + (1 + NSLOT) * C * 4;
+    static constexpr int oFlag = oKinv + (1 + NSLOT) * C * 4;  // merged episodes: one screen flag per wave
+    static constexpr int total = oFlag + NW * 4;
 };
 
 // PRO: the cell's prologue is part of the call -- k_n = k / max(|k|, 1e-12), beta = sigmoid(b) are
@@ -708,7 +709,13 @@ template <typename T, int C, int NW> struct DeltaBwdSmem : BwdDims<T, C> {
 static __device__ unsigned long long g_phase_clocks[4];
 #endif
 
-template <typename T, int C, int NW, bool PRO, bool NARROW = false>
+// MERGE: a chunk that holds resets is done in ONE unit instead of one per episode, as in the forward kernel
+// (chunk_fwd_kernel): masks keep the episodes apart where they could meet -- Aqk, dAqk and dA (pairs of one
+// episode only), the three terms with the state entering the chunk (rows of the first episode), the two
+// terms with the gradient of the state leaving it (rows of the last episode) and the update of that
+// gradient (rows of the first episode) -- after a screen of the chunk's inputs that rules out any
+// non-finite intermediate (chunk_common.h); a chunk that fails the screen takes the units per episode.
+template <typename T, int C, int NW, bool PRO, bool NARROW = false, bool MERGE = false>
 __global__ void __launch_bounds__(64 * NW, sizeof(T) == 2 ? 2 : 1)
 delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const void *__restrict__ done, int done_f32,
@@ -738,6 +745,8 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     float *sDb = reinterpret_cast<float *>(smem + L::oDb);  // [NSLOT][C] dbeta partials
     float *sKinv = reinterpret_cast<float *>(smem + L::oKinv);  // prologue: 1 / |k_row|
     float *sKd = sKinv + C;                                      // prologue: [NSLOT][C] partials of k_n . dk_n
+    float *sFlag = reinterpret_cast<float *>(smem + L::oFlag);
+    static_assert(!MERGE || !NARROW, "merged episodes: full-width heads");
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -868,12 +877,88 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         const int t0 = c * C;
         const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
-        for (int pass = nres; pass >= 0; --pass) {
-            auto live = [&](int r) { return nres == 0 || episode_of(dmask, r) == pass; };
+        bool mg = false;  // this chunk's episodes in one unit
+        if constexpr (MERGE) {
+            if (nres != 0) {
+                bool ok = true;
+                auto small = [](float x, float lim) { return fabsf(x) <= lim; };  // false for NaN
+#pragma unroll
+                for (int p = 0; p < IO::PASSES; ++p) {
+#pragma unroll
+                    for (int e = 0; e < IO::KP; ++e)
+                        ok = ok && small((float)rq.v[p][e], MERGE_IN_MAX) && small((float)rk.v[p][e], MERGE_IN_MAX) &&
+                             small((float)rv.v[p][e], MERGE_IN_MAX) && small((float)rdo.v[p][e], MERGE_IN_MAX);
+                    ok = ok && small(raw_to_float<T>(rbrow[p]), MERGE_IN_MAX);
+                }
+#pragma unroll
+                for (int p = 0; p < IOT::PASSES; ++p)
+                    if (IOT::FULL || IOT::row_of(tid, p) < C) {
+#pragma unroll
+                        for (int e = 0; e < IOT::KP; ++e) ok = ok && small((float)rTm.v[p][e], MERGE_IN_MAX);
+                    }
+#pragma unroll
+                for (int p = 0; p < IOS::PASSES; ++p)
+                    if (IOS::FULL || IOS::row_of(tid, p) < HD) {
+#pragma unroll
+                        for (int e = 0; e < IOS::KP; ++e) ok = ok && small((float)rS.v[p][e], MERGE_STATE_MAX);
+                    }
+#pragma unroll
+                for (int j = 0; j < TMS::TPW; ++j)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) ok = ok && small(dSacc[j][e], MERGE_STATE_MAX);
+                if (lane == 0) sFlag[w] = __ballot(!ok) != 0ull ? 1.f : 0.f;
+                sync_lds();
+                float bad = 0.f;
+#pragma unroll
+                for (int j = 0; j < NW; ++j) bad += sFlag[j];
+                mg = bad == 0.f;
+            }
+        }
+        const int r_first = mg ? (int)__builtin_ctzll(dmask) : C;        // rows below it: the episode that enters the chunk
+        const int r_last = mg ? 63 - (int)__builtin_clzll(dmask) : 0;   // rows from it on: the episode that leaves it
+        auto one_episode = [&](int lo, int hi) { return (dmask & ((2ull << hi) - (2ull << lo))) == 0ull; };  // no reset in rows lo + 1 .. hi
+        // One unit of work: the rows of one episode of the chunk (`pass` counts the episodes), or -- merged
+        // episodes, MG -- all rows of a chunk that holds resets at once (pass 0).  In the instance that can
+        // merge, the masks are part of the straight-line code of every unit (all-pass values where there is
+        // nothing to mask): a branch per mask would cut the phases into pieces the scheduler cannot overlap
+        // (measured: 10 % on chunks without resets), two copies of the unit do not fit the registers.
+        const bool MG = MERGE && mg;
+        // ff / fl: 1 for the rows (nt * 16 + li of the wave's [C][64]-shaped tiles) of the first / last episode, else
+        // 0; cc: bit 4 j + e set when element e of the wave's [C][C] tile j pairs two rows of one episode
+        float ff[TMR::NBW], fl[TMR::NBW];
+        unsigned cc = 0u;
+        if constexpr (MERGE) {
+#pragma unroll
+            for (int ni = 0; ni < TMR::NBW; ++ni) {
+                const int r = TMR::nt(w, ni) * 16 + li;
+                ff[ni] = !MG || r < r_first ? 1.f : 0.f;
+                fl[ni] = !MG || r >= r_last ? 1.f : 0.f;
+            }
+#pragma unroll
+            for (int j = 0; j < TMA::TPW; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int m = TMA::mt(w, j) * 16 + 4 * lg + e, n = TMA::nt(w, j) * 16 + li;
+                    if (!MG || one_episode(m < n ? m : n, m < n ? n : m)) cc |= 1u << (4 * j + e);
+                }
+        }
+        // masked store of a [C][C] product as dst[n][m]: tri(m, n) and, merged, the pair's bit of cc
+        auto store_cc = [&](const f32x4 *acc, T *dst, auto tri, float sign) {
+#pragma unroll
+            for (int j = 0; j < TMA::TPW; ++j) {
+                const int m = TMA::mt(w, j) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
+                float x[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) x[e] = tri(m + e, n) && (!MERGE || ((cc >> (4 * j + e)) & 1u)) ? sign * acc[j][e] : 0.f;
+                *reinterpret_cast<P4 *>(dst + n * LDC + m) = TT<T>::pack(x[0], x[1], x[2], x[3]);
+            }
+        };
+        for (int pass = MG ? 0 : nres; pass >= 0; --pass) {
+            auto live = [&](int r) { return nres == 0 || MG || episode_of(dmask, r) == pass; };
             // ---- stage ---------------------------------------------------------------
             {
                 typename IO::Regs fq = rq, fk = rk, fv = rv, fdo = rdo;
-                if (nres != 0) {
+                if (nres != 0 && !MG) {
                     IO::mask_rows(fq, tid, live);
                     IO::mask_rows(fk, tid, live);
                     IO::mask_rows(fv, tid, live);
@@ -910,11 +995,11 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 // are cleared by select: they only ever meet zeros, but a NaN key or gate of another
                 // episode sits in them and must not meet those zeros.
                 typename IOT::Regs fTm = rTm;
-                if (nres != 0) IOT::mask_rows(fTm, tid, live);
+                if (nres != 0 && !MG) IOT::mask_rows(fTm, tid, live);
                 IOT::to_lds(fTm, sTm, LDC, tid);
             }
             if (tid < C) sBeta[tid] = !live(tid) ? 0.f : PRO ? sigmoidf(raw_to_float<T>(rbeta)) : raw_to_float<T>(rbeta);
-            if (pass != nres) zero_acc<TMS::TPW>(dSacc);
+            if (pass != nres && !MG) zero_acc<TMS::TPW>(dSacc);
             store_acc<T, HD, HD, NW>(dSacc, sDS, LDD, w, lane);  // dS[dv][dk]
             sync_lds();
             flush_pending();
@@ -928,7 +1013,10 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
                 gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sQ, LDD, sK, LDD, w, lane);
-                store_acc_f<T, C, C, NW>(acc, sAqk, LDC, w, lane, [](int m, int n, float x) { return m >= n ? x : 0.f; });
+                if constexpr (MERGE)
+                    store_cc(acc, sAqk, [](int m, int n) { return m >= n; }, 1.f);
+                else
+                    store_acc_f<T, C, C, NW>(acc, sAqk, LDC, w, lane, [](int m, int n, float x) { return m >= n ? x : 0.f; });
             }
             // ---- V0[c][dv] = V[c][dv] - sum_dk S[dv][dk] K[c][dk] (in place), V~ = beta_c V0 -> sVt ---
             {
@@ -941,8 +1029,10 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     const P4 x = *reinterpret_cast<const P4 *>(sV + r * LDD + d0);  // each lane rewrites what it read
                     const float bb = sBeta[r];
                     float y[4];
+                    // merged episodes: the first one alone sees the entering state (a factor 0 on finite values)
+                    const float sees_S = MERGE ? ff[j % TMR::NBW] : 1.f;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) y[e] = (float)x[e] - acc[j][e];
+                    for (int e = 0; e < 4; ++e) y[e] = MERGE ? (float)x[e] - sees_S * acc[j][e] : (float)x[e] - acc[j][e];
                     const P4 v0 = TT<T>::pack(y[0], y[1], y[2], y[3]);
                     *reinterpret_cast<P4 *>(sV + r * LDD + d0) = v0;
                     // V~ from the rounded V0, so that dbeta = rowdot(Z, V0) matches what U' was built from
@@ -963,8 +1053,15 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             {
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
-                gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sDO, LDD, sAqk, LDC, w, lane);
-                gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc, sDS, LDD, sK, LDD, w, lane);
+                if constexpr (MERGE) {  // the term with dS first, so that it can be confined to the rows of the last episode
+                    gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc, sDS, LDD, sK, LDD, w, lane);
+#pragma unroll
+                    for (int j = 0; j < TMR::TPW; ++j) acc[j] *= fl[j % TMR::NBW];
+                    gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sDO, LDD, sAqk, LDC, w, lane);
+                } else {
+                    gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sDO, LDD, sAqk, LDC, w, lane);
+                    gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc, sDS, LDD, sK, LDD, w, lane);
+                }
                 store_acc<T, HD, C, NW>(acc, sDU, LDD, w, lane);
             }
             sync_lds();  // sU, sDU visible; sAqk dead
@@ -986,7 +1083,10 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
                 gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sU, LDD, sDO, LDD, w, lane);  // D[m = j][n = i]
-                store_acc_f<T, C, C, NW>(acc, sDAqk, LDC, w, lane, tril);
+                if constexpr (MERGE)
+                    store_cc(acc, sDAqk, [](int m, int n) { return m <= n; }, 1.f);
+                else
+                    store_acc_f<T, C, C, NW>(acc, sDAqk, LDC, w, lane, tril);
             }
             // ---- Z^T[dv][j] = sum_i dU'[i][dv] Tm[i][j] : dV = beta_j Z -> global and sZb ; dbeta += Z_j . V0_j
             {
@@ -1006,6 +1106,10 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 f32x4 acc[TMR::TPW];
                 zero_acc<TMR::TPW>(acc);
                 gemm<T, HD, C, HD, KROW, ROWK, NW>(acc, sS, LDD, sDO, LDD, w, lane);
+                if constexpr (MERGE) {
+#pragma unroll
+                    for (int j = 0; j < TMR::TPW; ++j) acc[j] *= ff[j % TMR::NBW];
+                }
                 gemm<T, HD, C, C, KROW, ROWK, NW>(acc, sK, LDD, sDAqk, LDC, w, lane);
                 store_acc<T, HD, C, NW>(acc, sDU, LDD, w, lane);  // dU' is dead; to memory after the barrier
             }
@@ -1017,17 +1121,39 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 zero_acc<TMR::TPW>(acc);
                 zero_acc<TMR::TPW>(dKacc);
                 gemm<T, HD, C, HD, KROW, ROWK, NW>(acc, sS, LDD, sZb, LDD, w, lane);
-                gemm<T, HD, C, C, KROW, KROW, NW>(dKacc, sQ, LDD, sDAqk, LDC, w, lane);
-                gemm<T, HD, C, HD, KROW, ROWK, NW>(dKacc, sDS, LDD, sU, LDD, w, lane);
+                if constexpr (MERGE) {  // the term with dS first: rows of the last episode; the term with S: rows of the first
+                    gemm<T, HD, C, HD, KROW, ROWK, NW>(dKacc, sDS, LDD, sU, LDD, w, lane);
 #pragma unroll
-                for (int j = 0; j < TMR::TPW; ++j) dKacc[j] -= acc[j];
+                    for (int j = 0; j < TMR::TPW; ++j) dKacc[j] *= fl[j % TMR::NBW];
+                    gemm<T, HD, C, C, KROW, KROW, NW>(dKacc, sQ, LDD, sDAqk, LDC, w, lane);
+#pragma unroll
+                    for (int j = 0; j < TMR::TPW; ++j) dKacc[j] -= acc[j] * ff[j % TMR::NBW];
+                } else {
+                    gemm<T, HD, C, C, KROW, KROW, NW>(dKacc, sQ, LDD, sDAqk, LDC, w, lane);
+                    gemm<T, HD, C, HD, KROW, ROWK, NW>(dKacc, sDS, LDD, sU, LDD, w, lane);
+#pragma unroll
+                    for (int j = 0; j < TMR::TPW; ++j) dKacc[j] -= acc[j];
+                }
             }
             // ---- dS^T[dk][dv] += sum_c Q[c][dk] dO[c][dv] - sum_c K[c][dk] (beta Z)[c][dv] -----------
             {
                 f32x4 acc[TMS::TPW];
                 zero_acc<TMS::TPW>(acc);
-                gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, sQ, LDD, sDO, LDD, w, lane);
-                gemm<T, HD, HD, C, KROW, KROW, NW>(acc, sK, LDD, sZb, LDD, w, lane);
+                if (MG) {
+                    // a chunk with resets: what flows on to the chunk before is the first episode's own sum
+                    zero_acc<TMS::TPW>(dSacc);
+                    auto first_rows = [&](int, int kb, typename TT<T>::frag &x) {  // element e of the fragment is chunk row k0 + e
+                        const int k0 = kb * TT<T>::KB + TT<T>::KP * lg;
+#pragma unroll
+                        for (int e = 0; e < TT<T>::KP; ++e)
+                            if (k0 + e >= r_first) x[e] = (T)0.f;
+                    };
+                    gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, sQ, LDD, sDO, LDD, w, lane, first_rows);
+                    gemm<T, HD, HD, C, KROW, KROW, NW>(acc, sK, LDD, sZb, LDD, w, lane, first_rows);
+                } else {
+                    gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, sQ, LDD, sDO, LDD, w, lane);
+                    gemm<T, HD, HD, C, KROW, KROW, NW>(acc, sK, LDD, sZb, LDD, w, lane);
+                }
 #pragma unroll
                 for (int j = 0; j < TMS::TPW; ++j) dSacc[j] -= acc[j];
             }
@@ -1036,7 +1162,10 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 f32x4 acc[TMA::TPW];
                 zero_acc<TMA::TPW>(acc);
                 gemm<T, C, C, HD, ROWK, ROWK, NW>(acc, sU, LDD, sZ, LDD, w, lane);
-                store_acc_f<T, C, C, NW>(acc, sDA, LDC, w, lane, [](int m, int n, float x) { return m < n ? -x : 0.f; });
+                if constexpr (MERGE)
+                    store_cc(acc, sDA, [](int m, int n) { return m < n; }, -1.f);
+                else
+                    store_acc_f<T, C, C, NW>(acc, sDA, LDC, w, lane, [](int m, int n, float x) { return m < n ? -x : 0.f; });
             }
             sync_lds();  // sDA visible; sQ, sDO, sS, sDS, sDAqk, sZ, sZb dead
             tile_rows_to_global<T, C, NTHR>(sDU, LDD, dq + base + (int64_t)t0 * rs, rs, t0, Tlen, tid, live, dkw);
@@ -1099,7 +1228,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 store_acc<T, HD, C, NW>(dKacc, sU, LDD, w, lane);
             }
             pend_dmask = dmask;
-            pend_nres = nres;
+            pend_nres = MG ? 0 : nres;
             pend_pass = pass;
             pend_t0 = t0;
             if (tid < C && t0 + tid < Tlen && live(tid)) {
@@ -1294,13 +1423,13 @@ MRX_EXPORT int MRX_API(mrx_gated_linear_attn_bwd)(void *stream, const void *q, c
 namespace {
 inline namespace MRX_HD_NS {
 
-template <typename T, int C, bool PRO, bool NARROW> struct DeltaBwdReg {
+template <typename T, int C, bool PRO, bool NARROW, bool MERGE> struct DeltaBwdReg {
     static constexpr int NW = 4;
     static constexpr int smem = DeltaBwdSmem<T, C, NW>::total;
-    static inline KernelRegistrar reg{reinterpret_cast<const void *>(delta_bwd_kernel<T, C, NW, PRO, NARROW>), smem};
+    static inline KernelRegistrar reg{reinterpret_cast<const void *>(delta_bwd_kernel<T, C, NW, PRO, NARROW, MERGE>), smem};
 };
 
-template <typename T, int C, bool PRO>
+template <typename T, int C, bool PRO, bool MERGE = false>
 int launch_delta_bwd(hipStream_t st, const void *q, const void *k, const void *v, const void *beta,
                      const void *done, int done_dtype, const void *S_chk, const void *Tm_chk, const void *dout,
                      const void *dS_last, void *dq, void *dk_out, void *dv_out, void *dbeta, void *dS0, int64_t B,
@@ -1308,9 +1437,10 @@ int launch_delta_bwd(hipStream_t st, const void *q, const void *k, const void *v
 {
     if (const int rc = prepare_device(); rc != MRX_OK) return rc;
     auto go = [&](auto narrow) {
-        using Reg = DeltaBwdReg<T, C, PRO, decltype(narrow)::value>;
+        constexpr bool MG = MERGE && !decltype(narrow)::value;  // narrow heads keep the units per episode
+        using Reg = DeltaBwdReg<T, C, PRO, decltype(narrow)::value, MG>;
         (void)&Reg::reg;  // the kernel is on the list mrx_init() walks
-        return launch_kernel(delta_bwd_kernel<T, C, Reg::NW, PRO, decltype(narrow)::value>, dim3((unsigned)(B * H)),
+        return launch_kernel(delta_bwd_kernel<T, C, Reg::NW, PRO, decltype(narrow)::value, MG>, dim3((unsigned)(B * H)),
                              dim3(64 * Reg::NW), Reg::smem, st, (const T *)q, (const T *)k, (const T *)v, (const T *)beta,
                              done, done_dtype, (const T *)S_chk, (const T *)Tm_chk, (const T *)dout,
                              (const float *)dS_last, (T *)dq, (T *)dk_out, (T *)dv_out, (T *)dbeta, (float *)dS0, (int)T_,
@@ -1324,13 +1454,25 @@ template <bool PRO>
 int delta_bwd_entry(void *stream, const void *q, const void *k, const void *v, const void *beta, const void *done,
                     const void *S_chk, const void *Tm_chk, const void *dout, const void *dS_last, void *dq,
                     void *dk_out, void *dv_out, void *dbeta, void *dS0, int64_t B, int64_t T, int64_t H,
-                    int64_t dk, int64_t dv, int dtype, int done_dtype)
+                    int64_t dk, int64_t dv, int dtype, int done_dtype, int reset_path)
 {
     const int rc = check_bwd(q, k, v, done, S_chk, dout, dS_last, dq, dk_out, dv_out, dS0, B, T, H, dk,
                              dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
     if (!beta || !dbeta || !Tm_chk || !aligned(Tm_chk, 16)) return MRX_ERR_INVALID_ARG;
+    if (reset_path != MRX_RESETS_AUTO && reset_path != MRX_RESETS_PASSES && reset_path != MRX_RESETS_MERGED)
+        return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
+#if MRX_HD == 64
+    // merged episodes: the build with 32-row chunks, whose bounds the screen was derived for
+    if (reset_path == MRX_RESETS_MERGED && DELTA_BF16_CHUNK == 32) {
+        if (dtype == MRX_BF16)
+            return launch_delta_bwd<__bf16, 32, PRO, true>(st, q, k, v, beta, done, done_dtype, S_chk, Tm_chk, dout,
+                                                           dS_last, dq, dk_out, dv_out, dbeta, dS0, B, T, H, dk, dv);
+        return launch_delta_bwd<float, 32, PRO, true>(st, q, k, v, beta, done, done_dtype, S_chk, Tm_chk, dout, dS_last, dq,
+                                                      dk_out, dv_out, dbeta, dS0, B, T, H, dk, dv);
+    }
+#endif
     if (dtype == MRX_BF16)
         return launch_delta_bwd<__bf16, DELTA_BF16_CHUNK, PRO>(st, q, k, v, beta, done, done_dtype, S_chk, Tm_chk, dout,
                                                                dS_last, dq, dk_out, dv_out, dbeta, dS0, B, T, H, dk, dv);
@@ -1346,13 +1488,13 @@ MRX_EXPORT int MRX_API(mrx_delta_rule_bwd)(void *stream, const void *q, const vo
                                   const void *Tm_chk, const void *dout, const void *dS_last, void *dq,
                                   void *dk_out, void *dv_out, void *dbeta, void *dS0, int64_t B,
                                   int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
-                                  int done_dtype)
+                                  int done_dtype, int reset_path)
 {
 #if MRX_HD == 64
-    if (dk <= 32 && dv <= 32) return mrx_delta_rule_bwd_hd32(stream, q, k, v, beta, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out, dbeta, dS0, B, T, H, dk, dv, dtype, done_dtype);
+    if (dk <= 32 && dv <= 32) return mrx_delta_rule_bwd_hd32(stream, q, k, v, beta, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out, dbeta, dS0, B, T, H, dk, dv, dtype, done_dtype, reset_path);
 #endif
     return delta_bwd_entry<false>(stream, q, k, v, beta, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out,
-                                  dbeta, dS0, B, T, H, dk, dv, dtype, done_dtype);
+                                  dbeta, dS0, B, T, H, dk, dv, dtype, done_dtype, reset_path);
 }
 
 MRX_EXPORT int MRX_API(mrx_deltanet_bwd)(void *stream, const void *q, const void *k, const void *v,
@@ -1360,13 +1502,13 @@ MRX_EXPORT int MRX_API(mrx_deltanet_bwd)(void *stream, const void *q, const void
                                 const void *Tm_chk, const void *dout, const void *dS_last, void *dq,
                                 void *dk_out, void *dv_out, void *dbeta_raw, void *dS0, int64_t B,
                                 int64_t T, int64_t H, int64_t dk, int64_t dv, int dtype,
-                                int done_dtype)
+                                int done_dtype, int reset_path)
 {
 #if MRX_HD == 64
-    if (dk <= 32 && dv <= 32) return mrx_deltanet_bwd_hd32(stream, q, k, v, beta_raw, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out, dbeta_raw, dS0, B, T, H, dk, dv, dtype, done_dtype);
+    if (dk <= 32 && dv <= 32) return mrx_deltanet_bwd_hd32(stream, q, k, v, beta_raw, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out, dbeta_raw, dS0, B, T, H, dk, dv, dtype, done_dtype, reset_path);
 #endif
     return delta_bwd_entry<true>(stream, q, k, v, beta_raw, done, S_chk, Tm_chk, dout, dS_last, dq, dk_out, dv_out,
-                                 dbeta_raw, dS0, B, T, H, dk, dv, dtype, done_dtype);
+                                 dbeta_raw, dS0, B, T, H, dk, dv, dtype, done_dtype, reset_path);
 }
 
 #if defined(MRX_PHASE_CLOCKS) && MRX_HD == 64

@@ -55,11 +55,18 @@ constexpr int LA_BF16_CHUNK = MRX_LA_BF16_CHUNK, DELTA_BF16_CHUNK = MRX_DELTA_BF
 // (S_c = S_{c+1} - V_c^T K_c in fp32) instead of reading a checkpoint per chunk.  Every step of that walk
 // rounds at the magnitude of the late, large state, so its error relative to an early, small state grows
 // with the number of chunks walked (about eps N^1.5 for a state that grows linearly).  The forward
-// call therefore writes the exact fp32 state every WALK_ANCHOR chunks as well (besides the chunks
+// call therefore writes the exact fp32 state every walk_anchor() chunks as well (besides the chunks
 // with resets) and the walk starts afresh there: 32 chunks keep fp32 at 1e-5 of the early states,
 // bf16 inputs (tolerance 2e-2, rounding 4e-3) are re-anchored every 128.  Extra traffic: one 16 KB
 // slot per 32 (128) chunks of 32 KB each way.
 template <typename T> constexpr int walk_anchor() { return sizeof(T) == 2 ? 128 : 32; }
+
+// Bounds of the screen that lets the delta-rule kernels do all episodes of a chunk in one unit (template flag
+// MERGE): with |q|, |k|, |v|, |beta|, |dout| and the entries of the triangular factor at most 2^6 and the
+// entries of the state and of its gradient at most 2^20, the largest intermediate of a 32-row chunk at
+// head dim 64 stays below 2^123 (forward: the output, 2^5 x 2^18 x 2^50 and its state term; backward: the
+// row dots behind dbeta, 2^6 x 2^6 x 2^110), inside the float32 range.
+constexpr float MERGE_IN_MAX = 64.f, MERGE_STATE_MAX = 1048576.f;
 
 enum OpMode { ROWK = 0, KROW = 1 };
 

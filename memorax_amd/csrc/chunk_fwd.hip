@@ -82,8 +82,17 @@ struct NormArgs {
 // states (B,H,dva,dka) and z (B,H,dka).  Tiles in LDS and registers keep the build's width: what lies
 // beyond the rows' width is loaded as zero (after the feature map, phi(0) = 1 must not count) and never
 // stored.
+// MERGE (delta rule with TMIN): a chunk that holds resets is done in ONE unit instead of one per episode.  The
+// episodes are kept apart by masks on the three places where they could meet -- Q K^T (pairs of one episode
+// only), the terms with the state entering the chunk (rows of the first episode only) and the state update
+// (rows of the last episode only) -- and the triangular factor arrives block diagonal by episode.  A masked
+// zero then multiplies values of other episodes inside the products, which is exact as long as those
+// values are finite, so the chunk is screened first: every input of the chunk at most MERGE_IN_MAX in
+// magnitude and the state at most MERGE_STATE_MAX (bounds under which no intermediate of the chunk can
+// leave the float32 range, so a non-finite value cannot arise either), else the chunk takes the units
+// per episode, whose zeros are put in by select.  Results equal those of the units per episode.
 template <typename T, int C, bool DELTA, bool FMAP, bool GATED, bool NORM, bool PRO = false, bool TMIN = false,
-          bool PAR = false, bool NARROW = false>
+          bool PAR = false, bool NARROW = false, bool MERGE = false>
 __global__ void __launch_bounds__(NTHR, 2)  // 2 waves per SIMD: two workgroups share a CU
 chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v,
                  const T *__restrict__ beta, const float *__restrict__ glog,
@@ -96,6 +105,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     static_assert(!PRO || DELTA, "the prologue belongs to the delta rule");
     static_assert(!TMIN || (DELTA && C == 32), "precomputed factors belong to the delta rule's 32-row chunks");
     static_assert(!PAR || (!DELTA && !GATED && !NORM), "one workgroup per chunk: plain linear attention only");
+    static_assert(!MERGE || (TMIN && !NARROW), "merged episodes: the delta rule on precomputed factors, full-width heads");
     using IOT = TileIO<T, C, NTHR, C>;  // the [C][C] triangular factor
     using L = FwdSmem<T, C, DELTA, GATED, NORM>;
     using Frag = typename TT<T>::frag;
@@ -255,8 +265,40 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         const int t0 = c * C;
         const unsigned long long dmask = __ballot(done_test(rdone, done_f32) && lane < C);
         const int nres = __popcll(dmask);
-        for (int pass = 0; pass <= nres; ++pass) {
-            auto live = [&](int r) { return nres == 0 || episode_of(dmask, r) == pass; };
+        bool mg = false;  // this chunk's episodes in one unit
+        if constexpr (MERGE) {
+            if (nres != 0) {
+                bool ok = true;
+                auto small = [](float x, float lim) { return fabsf(x) <= lim; };  // false for NaN
+#pragma unroll
+                for (int p = 0; p < IO::PASSES; ++p) {
+#pragma unroll
+                    for (int e = 0; e < IO::KP; ++e)
+                        ok = ok && small((float)rq.v[p][e], MERGE_IN_MAX) && small((float)rk.v[p][e], MERGE_IN_MAX) &&
+                             small((float)rv.v[p][e], MERGE_IN_MAX);
+                    ok = ok && small(raw_to_float<T>(rbrow[p]), MERGE_IN_MAX);
+                }
+#pragma unroll
+                for (int p = 0; p < IOT::PASSES; ++p)
+                    if (IOT::FULL || IOT::row_of(tid, p) < C) {
+#pragma unroll
+                        for (int e = 0; e < IOT::KP; ++e) ok = ok && small((float)rTm.v[p][e], MERGE_IN_MAX);
+                    }
+#pragma unroll
+                for (int j = 0; j < TMS::TPW; ++j)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) ok = ok && small(Sacc[j][e], MERGE_STATE_MAX);
+                // sBeta is free in this variant (the factors arrive ready): one flag per wave
+                if (lane == 0) sBeta[w] = __ballot(!ok) != 0ull ? 1.f : 0.f;
+                sync_lds();
+                mg = sBeta[0] + sBeta[1] + sBeta[2] + sBeta[3] == 0.f;
+            }
+        }
+        const int npass = mg ? 0 : nres;
+        const int r_first = mg ? (int)__builtin_ctzll(dmask) : C;        // rows below it: the episode that enters the chunk
+        const int r_last = mg ? 63 - (int)__builtin_clzll(dmask) : 0;   // rows from it on: the episode that leaves it
+        for (int pass = 0; pass <= npass; ++pass) {
+            auto live = [&](int r) { return nres == 0 || mg || episode_of(dmask, r) == pass; };
             // gated: G_i = sum of the log-decays of this pass's episode up to row i (the decay of an
             // episode's first step multiplies a zero state and is left out); every wave scans its copy
             float G = 0.f, Glast = 0.f;
@@ -280,7 +322,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     IO::template fmap<FMAP>(fq);
                     IO::template fmap<FMAP>(fk);
                 }
-                if (nres != 0) {
+                if (nres != 0 && !mg) {
                     IO::mask_rows(fq, tid, live);
                     IO::mask_rows(fk, tid, live);
                     IO::mask_rows(fv, tid, live);
@@ -318,7 +360,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 // rows of other episodes are cleared by select: they only ever meet zeros, but a NaN key
                 // or gate of another episode sits in them
                 typename IOT::Regs fTm = rTm;
-                if (nres != 0) IOT::mask_rows(fTm, tid, live);
+                if (nres != 0 && !mg) IOT::mask_rows(fTm, tid, live);
                 IOT::to_lds(fTm, sTm, LDC, tid);
             }
             if (pass != 0) zero_acc<TMS::TPW>(Sacc);  // an episode that starts in the chunk starts from 0
@@ -355,7 +397,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             // walk needs U' as a residual and an extra product, which measured slower than reading the
             // states: there every chunk is written, in the I/O type, from the copy of S just staged.
             constexpr bool DENSE_CHK = GATED || DELTA;
-            if (!PAR && S_chk && pass == 0 && (DENSE_CHK || nres != 0 || c % walk_anchor<T>() == 0)) {
+            if (!PAR && S_chk && pass == 0 && (DENSE_CHK || nres != 0 || (c > 0 && c % walk_anchor<T>() == 0))) {
                 if (DENSE_CHK) {
                     using IOS = TileIO<T, HD, NTHR>;
 #pragma unroll
@@ -374,7 +416,7 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     }
                 }
             }
-            const bool pre = pass == nres && c + 1 < c_end;
+            const bool pre = pass == npass && c + 1 < c_end;
             if (pre) { prefetch_part(0); prefetch_part(1); }
             if (TMIN && pre) { prefetch_part(2); prefetch_part(3); }
             // ---- A[i][j] = beta_i (k_i . k_j), j < i ----------------------------------
@@ -422,6 +464,11 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                         for (int e = 0; e < 4; ++e) x[e] = (m + e <= n) ? acc[j][e] * __expf(gn - gm[e]) : 0.f;
                         *reinterpret_cast<P4 *>(sAqk + n * LDC + m) = TT<T>::pack(x[0], x[1], x[2], x[3]);
                     }
+                } else if (MERGE && mg) {
+                    // pairs (i = n, j = m <= n) of one episode only: no reset in rows m + 1 .. n
+                    store_acc_f<T, C, C, NW>(acc, sAqk, LDC, w, lane, [&](int m, int n, float x) {
+                        return m <= n && (dmask & ((2ull << n) - (2ull << m))) == 0ull ? x : 0.f;
+                    });
                 } else {
                     store_acc_f<T, C, C, NW>(acc, sAqk, LDC, w, lane,
                                              [](int m, int n, float x) { return m <= n ? x : 0.f; });
@@ -455,7 +502,10 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                     zero_acc<TMO::TPW>(acc);
                     gemm<T, HD, C, HD, ROWK, ROWK, NW>(acc, sS, LDD, sW, LDD, w, lane);
 #pragma unroll
-                    for (int j = 0; j < TMO::TPW; ++j) Uacc[j] -= acc[j];
+                    for (int j = 0; j < TMO::TPW; ++j) {
+                        // merged episodes: only the rows of the episode that entered the chunk see its state
+                        if (!(MERGE && mg) || TMO::nt(w, j) * 16 + li < r_first) Uacc[j] -= acc[j];
+                    }
                     store_acc<T, HD, C, NW>(Uacc, sU, LDD, w, lane);
                 }
             }
@@ -488,6 +538,11 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 }
             };
             gemm<T, HD, C, HD, ROWK, ROWK, NW>(Oacc, sS, LDD, sQ, LDD, w, lane, NoHook(), den_q);
+            if (MERGE && mg) {
+#pragma unroll
+                for (int j = 0; j < TMO::TPW; ++j)
+                    if (TMO::nt(w, j) * 16 + li >= r_first) Oacc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
             if (GATED) {  // the incoming state reaches row i decayed by exp(G_i)
 #pragma unroll
                 for (int j = 0; j < TMO::TPW; ++j) Oacc[j] *= __expf(sG[TMO::nt(w, j) * 16 + li]);
@@ -535,11 +590,12 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                 }
             }
             pend_dmask = dmask;
-            pend_nres = nres;
+            pend_nres = mg ? 0 : nres;
             pend_pass = pass;
             pend_t0 = t0;
             // ---- S^T[dk][dv] += sum_c K[c][dk] U'[c][dv]  (only the episode that leaves the chunk)
-            if (pass == nres && !PAR) {
+            if (pass == npass && !PAR) {
+                if (MERGE && mg) zero_acc<TMS::TPW>(Sacc);  // a chunk with resets: the state that leaves is the last episode's own
                 if (GATED) {  // S <- exp(G_last) S + sum_c exp(G_last - G_c) K[c] U'[c]
                     const float cl = __expf(Glast);
 #pragma unroll
@@ -561,6 +617,12 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
                         const float *eb = sEb + kb * TT<T>::KB + TT<T>::KP * lg;
 #pragma unroll
                         for (int e = 0; e < TT<T>::KP; ++e) xk[e] = (T)((float)xk[e] * eb[e]);
+                    }
+                    if (MERGE && mg) {  // rows of the last episode only (element e of the fragment is chunk row k0 + e)
+                        const int k0 = kb * TT<T>::KB + TT<T>::KP * lg;
+#pragma unroll
+                        for (int e = 0; e < TT<T>::KP; ++e)
+                            if (k0 + e < r_last) xk[e] = (T)0.f;
                     }
                 };
                 gemm<T, HD, HD, C, KROW, KROW, NW>(Sacc, sK, LDD, sU, LDD, w, lane, z_k);
@@ -604,16 +666,16 @@ chunk_fwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
     }
 }
 
-template <typename T, int C, bool DELTA, bool FMAP, bool GATED, bool NORM, bool PRO, bool TMIN, bool PAR, bool NARROW> struct FwdReg {
+template <typename T, int C, bool DELTA, bool FMAP, bool GATED, bool NORM, bool PRO, bool TMIN, bool PAR, bool NARROW, bool MERGE> struct FwdReg {
     static constexpr int smem = FwdSmem<T, C, DELTA, GATED, NORM>::total;
     static inline KernelRegistrar reg{
-        reinterpret_cast<const void *>(chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR, NARROW>), smem};
+        reinterpret_cast<const void *>(chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR, NARROW, MERGE>), smem};
 };
 
 // dka, dva: widths of the q/k and v/o rows in memory; less than the build's head dim (narrow heads)
 // selects the kernel instance that pads on the fly.
 template <typename T, int C, bool DELTA, bool FMAP, bool GATED = false, bool NORM = false, bool PRO = false,
-          bool TMIN = false, bool PAR = false>
+          bool TMIN = false, bool PAR = false, bool MERGE = false>
 int launch(hipStream_t st, const void *q, const void *k, const void *v, const void *beta,
            const void *done, int done_f32, const void *S0, void *o, void *S_last, void *S_chk,
            void *Tm_chk, int64_t B, int64_t Tlen, int64_t H, const void *glog = nullptr, NormArgs na = NormArgs{},
@@ -624,9 +686,10 @@ int launch(hipStream_t st, const void *q, const void *k, const void *v, const vo
     if (PAR && NC > 65535) return MRX_ERR_INVALID_ARG;
     auto go = [&](auto narrow) {
         constexpr bool NARROW = decltype(narrow)::value;
-        using Reg = FwdReg<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR, NARROW>;
+        constexpr bool MG = MERGE && !NARROW;  // narrow heads keep the units per episode
+        using Reg = FwdReg<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR, NARROW, MG>;
         (void)&Reg::reg;  // the kernel is on the list mrx_init() walks
-        return launch_kernel(chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR, NARROW>,
+        return launch_kernel(chunk_fwd_kernel<T, C, DELTA, FMAP, GATED, NORM, PRO, TMIN, PAR, NARROW, MG>,
                              dim3((unsigned)(B * H), PAR ? (unsigned)NC : 1u), dim3(NTHR), Reg::smem, st, (const T *)q,
                              (const T *)k, (const T *)v, (const T *)beta, (const float *)glog, done, done_f32,
                              (const float *)S0, (T *)o, (float *)S_last, S_chk, (T *)Tm_chk, (int)Tlen, (int)H, na,
@@ -669,7 +732,8 @@ int check_common(const void *q, const void *k, const void *v, const void *done, 
 template <bool PRO>
 int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void *v, const void *beta, const void *done,
                        int done_dtype, const void *S0, void *o, void *S_last, void *S_chk, void *Tm_chk, int64_t B,
-                       int64_t T, int64_t H, int dtype, int factor_path, int64_t dk = HD, int64_t dv = HD)
+                       int64_t T, int64_t H, int dtype, int factor_path, int64_t dk = HD, int64_t dv = HD,
+                       int reset_path = MRX_RESETS_AUTO)
 {
     // delta_tm_kernel is written for 32-row chunks: a build with 64-row bf16 chunks (the measurement
     // variant, MRX_DELTA_BF16_CHUNK=64) always inverts inside the sequential kernel
@@ -681,16 +745,24 @@ int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void 
     // occupancy is the bf16 kernels' only
     const bool parallel = Tm_chk && factor_path != MRX_FACTORS_INLINE && T <= DELTA_TM_MAX_T &&
                           (factor_path == MRX_FACTORS_PARALLEL || dtype == MRX_F32 || B * H <= 2 * (int64_t)cus);
+    // merged episodes run on precomputed factors (which arrive block diagonal by episode, and screened like any
+    // other input): where the factor path is the chunk-parallel kernel; with the inverse inside the sequential
+    // kernel the units per episode stay (on a full device, where that path is the rule, a chunk with resets
+    // costs the forward a few per cent, less than the factor kernel would)
+    const bool merged = MRX_HD == 64 && TM_KERNEL && reset_path == MRX_RESETS_MERGED && parallel;
     if (!TM_KERNEL && factor_path == MRX_FACTORS_PARALLEL) return MRX_ERR_UNSUPPORTED;
     if constexpr (TM_KERNEL) if (parallel) {
         const int rc = launch_delta_tm(st, k, beta, done, done_dtype, Tm_chk, B, T, H, dtype, PRO, dk);
         if (rc != MRX_OK) return rc;
-        if (dtype == MRX_BF16)
-            return launch<__bf16, 32, true, false, false, false, PRO, true>(st, q, k, v, beta, done, done_dtype, S0, o,
-                                                                           S_last, S_chk, Tm_chk, B, T, H, nullptr,
-                                                                           NormArgs{}, dk, dv);
-        return launch<float, 32, true, false, false, false, PRO, true>(st, q, k, v, beta, done, done_dtype, S0, o, S_last,
-                                                                       S_chk, Tm_chk, B, T, H, nullptr, NormArgs{}, dk, dv);
+#define MRX_ARGS st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H, nullptr, NormArgs{}, dk, dv
+#if MRX_HD == 64
+        if (merged)
+            return dtype == MRX_BF16 ? launch<__bf16, 32, true, false, false, false, PRO, true, false, true>(MRX_ARGS)
+                                     : launch<float, 32, true, false, false, false, PRO, true, false, true>(MRX_ARGS);
+#endif
+        if (dtype == MRX_BF16) return launch<__bf16, 32, true, false, false, false, PRO, true>(MRX_ARGS);
+        return launch<float, 32, true, false, false, false, PRO, true>(MRX_ARGS);
+#undef MRX_ARGS
     }
     if (dtype == MRX_BF16)
         return launch<__bf16, DELTA_BF16_CHUNK, true, false, false, false, PRO, false>(st, q, k, v, beta, done, done_dtype, S0, o,
@@ -701,6 +773,7 @@ int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void 
 }
 
 bool factor_path_ok(int f) { return f == MRX_FACTORS_AUTO || f == MRX_FACTORS_PARALLEL || f == MRX_FACTORS_INLINE; }
+bool reset_path_ok(int r) { return r == MRX_RESETS_AUTO || r == MRX_RESETS_PASSES || r == MRX_RESETS_MERGED; }
 
 #if MRX_HD == 64
 // ---- static scratch of the entry point that allocates nothing --------------------------------------
@@ -806,17 +879,18 @@ extern "C" int mrx_linear_attn_chunk_parallel_pays(int64_t B, int64_t T, int64_t
 MRX_EXPORT int MRX_API(mrx_delta_rule_fwd)(void *stream, const void *q, const void *k, const void *v,
                                   const void *beta, const void *done, const void *S0, void *o,
                                   void *S_last, void *S_chk, void *Tm_chk, int64_t B, int64_t T,
-                                  int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype, int factor_path)
+                                  int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype, int factor_path,
+                                  int reset_path)
 {
 #if MRX_HD == 64
-    if (dk <= 32 && dv <= 32) return mrx_delta_rule_fwd_hd32(stream, q, k, v, beta, done, S0, o, S_last, S_chk, Tm_chk, B, T, H, dk, dv, dtype, done_dtype, factor_path);
+    if (dk <= 32 && dv <= 32) return mrx_delta_rule_fwd_hd32(stream, q, k, v, beta, done, S0, o, S_last, S_chk, Tm_chk, B, T, H, dk, dv, dtype, done_dtype, factor_path, reset_path);
 #endif
     const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
-    if (!beta || !aligned(Tm_chk, 16) || !factor_path_ok(factor_path)) return MRX_ERR_INVALID_ARG;
+    if (!beta || !aligned(Tm_chk, 16) || !factor_path_ok(factor_path) || !reset_path_ok(reset_path)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     return delta_fwd_dispatch<false>(st, q, k, v, beta, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H, dtype,
-                                     factor_path, dk, dv);
+                                     factor_path, dk, dv, reset_path);
 }
 
 #if MRX_HD == 64
@@ -890,15 +964,16 @@ MRX_EXPORT int MRX_API(mrx_linear_attn_norm_fwd)(void *stream, const void *q, co
 MRX_EXPORT int MRX_API(mrx_deltanet_fwd)(void *stream, const void *q, const void *k, const void *v,
                                 const void *beta_raw, const void *done, const void *S0, void *o,
                                 void *S_last, void *S_chk, void *Tm_chk, int64_t B, int64_t T,
-                                int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype, int factor_path)
+                                int64_t H, int64_t dk, int64_t dv, int dtype, int done_dtype, int factor_path,
+                                int reset_path)
 {
 #if MRX_HD == 64
-    if (dk <= 32 && dv <= 32) return mrx_deltanet_fwd_hd32(stream, q, k, v, beta_raw, done, S0, o, S_last, S_chk, Tm_chk, B, T, H, dk, dv, dtype, done_dtype, factor_path);
+    if (dk <= 32 && dv <= 32) return mrx_deltanet_fwd_hd32(stream, q, k, v, beta_raw, done, S0, o, S_last, S_chk, Tm_chk, B, T, H, dk, dv, dtype, done_dtype, factor_path, reset_path);
 #endif
     const int rc = check_common(q, k, v, done, o, S0, S_last, S_chk, B, T, H, dk, dv, dtype, done_dtype, true);
     if (rc != MRX_OK) return rc;
-    if (!beta_raw || !aligned(Tm_chk, 16) || !factor_path_ok(factor_path)) return MRX_ERR_INVALID_ARG;
+    if (!beta_raw || !aligned(Tm_chk, 16) || !factor_path_ok(factor_path) || !reset_path_ok(reset_path)) return MRX_ERR_INVALID_ARG;
     hipStream_t st = (hipStream_t)stream;
     return delta_fwd_dispatch<true>(st, q, k, v, beta_raw, done, done_dtype, S0, o, S_last, S_chk, Tm_chk, B, T, H, dtype,
-                                    factor_path, dk, dv);
+                                    factor_path, dk, dv, reset_path);
 }

@@ -374,11 +374,11 @@ def gated_linear_attention(q, k, v, g, done, S0=None, feature_map="none"):
 
 class _DeltaRule(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, beta, done, S0, prologue=False):
+    def forward(ctx, q, k, v, beta, done, S0, prologue=False, resets=None):
         q_, k_, v_, b_ = q.contiguous(), k.contiguous(), v.contiguous(), beta.contiguous()
         S0_ = None if S0 is None else S0.contiguous().float()
         need = any(ctx.needs_input_grad)
-        ctx.done, ctx.has_S0, ctx.prologue = done, S0 is not None, prologue
+        ctx.done, ctx.has_S0, ctx.prologue, ctx.resets = done, S0 is not None, prologue, resets
         if q_.shape[1] == 1 and not need:  # acting: one step, no residuals
             k1, b1 = k_[:, 0], b_[:, 0]
             if prologue:  # a (B,H,d) array: the prologue as array ops costs nothing here
@@ -386,7 +386,7 @@ class _DeltaRule(torch.autograd.Function):
                 b1 = torch.sigmoid(b1.float()).to(b_.dtype)
             o, S_last = K.delta_rule_step(q_[:, 0], k1, v_[:, 0], b1, done[:, 0], S0_)
             return o[:, None], S_last
-        o, S_last, chk = K.delta_rule_fwd(q_, k_, v_, b_, done, S0_, save_chk=need, prologue=prologue)
+        o, S_last, chk = K.delta_rule_fwd(q_, k_, v_, b_, done, S0_, save_chk=need, prologue=prologue, reset_path=resets)
         if need:
             ctx.save_for_backward(q_, k_, v_, b_, *chk)
         return o, S_last
@@ -397,30 +397,32 @@ class _DeltaRule(torch.autograd.Function):
         do = torch.zeros_like(v) if do is None else do.contiguous()
         dS_last = None if dS_last is None else dS_last.contiguous().float()
         dq, dk, dv, db, dS0 = K.delta_rule_bwd(q, k, v, beta, ctx.done, (S_chk, Tm_chk), do, dS_last,
-                                               want_dS0=ctx.has_S0, prologue=ctx.prologue)
-        return dq, dk, dv, db, None, (dS0 if ctx.has_S0 else None), None
+                                               want_dS0=ctx.has_S0, prologue=ctx.prologue, reset_path=ctx.resets)
+        return dq, dk, dv, db, None, (dS0 if ctx.has_S0 else None), None, None
 
 
 @_batched(4, 0)
-def delta_rule(q, k, v, beta, done, S0=None):
+def delta_rule(q, k, v, beta, done, S0=None, resets=None):
     """DeltaNet recurrence S_t = r_t S_{t-1}(I - beta_t k_t k_t^T) + beta_t v_t k_t^T,
-    o_t = S_t q_t, in chunked WY form.  Returns (o, S_last)."""
+    o_t = S_t q_t, in chunked WY form.  Returns (o, S_last).
+    resets: None / "passes" / "merged" -- how the kernels treat a chunk that holds resets
+    (mrx_reset_path; "merged" for callers whose episodes end every hundred steps or so)."""
     if _no_steps(q):
         return _attention_without_steps(q, v, S0)
     hd = _Heads(q, v, narrow=True)
-    o, S_last = _DeltaRule.apply(hd.qk(q), hd.qk(k), hd.v(v), hd.per_head(beta), done, hd.state_in(S0))
+    o, S_last = _DeltaRule.apply(hd.qk(q), hd.qk(k), hd.v(v), hd.per_head(beta), done, hd.state_in(S0), False, resets)
     return hd.out(o), hd.state_out(S_last)
 
 
 @_batched(4, 0)
-def deltanet(q, k, v, beta_raw, done, S0=None):
+def deltanet(q, k, v, beta_raw, done, S0=None, resets=None):
     """The DeltaNet cell's recurrence on its raw projections: delta_rule with
     k / max(|k|, 1e-12) and sigmoid(beta_raw) formed inside the kernels (the normalised keys and
     the gates never reach memory; gradients come back w.r.t. the raw arrays).  Returns (o, S_last)."""
     if _no_steps(q):
         return _attention_without_steps(q, v, S0)
     hd = _Heads(q, v, narrow=True)   # where keys are padded: zeros leave their norm unchanged
-    o, S_last = _DeltaRule.apply(hd.qk(q), hd.qk(k), hd.v(v), hd.per_head(beta_raw), done, hd.state_in(S0), True)
+    o, S_last = _DeltaRule.apply(hd.qk(q), hd.qk(k), hd.v(v), hd.per_head(beta_raw), done, hd.state_in(S0), True, resets)
     return hd.out(o), hd.state_out(S_last)
 
 

@@ -324,6 +324,8 @@ def linear_attn_norm_bwd(q, k, v, done, chk, o, den, do, dS_last=None, dz_last=N
 
 _FACTORS = {None: _lib.MRX_FACTORS_AUTO, "auto": _lib.MRX_FACTORS_AUTO, "parallel": _lib.MRX_FACTORS_PARALLEL,
             "inline": _lib.MRX_FACTORS_INLINE}
+_RESETS = {None: _lib.MRX_RESETS_AUTO, "auto": _lib.MRX_RESETS_AUTO, "passes": _lib.MRX_RESETS_PASSES,
+           "merged": _lib.MRX_RESETS_MERGED}
 
 
 def init(device=None):
@@ -357,7 +359,7 @@ def delta_rule_fwd_noalloc(q, k, v, beta, done, S0=None, out=None):
 
 
 def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prologue=False, tm_scratch=None,
-                   factor_path=None):
+                   factor_path=None, reset_path=None):
     """Returns (o, S_last fp32, chk) where chk = (S_chk, Tm_chk) are the residuals the
     backward call needs, or None.  out = (o, S_last, S_chk, Tm_chk) reuses buffers of an earlier
     call with the same shapes instead of allocating.  prologue=True: k is L2-normalised and
@@ -365,7 +367,9 @@ def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prolog
     tm_scratch (only without residuals): give the library a buffer for the triangular factors
     anyway, which lets it compute them chunk-parallel.  None: when the library would use it (float32;
     bf16 with B*H at most two sequences per compute unit).
-    factor_path: None / "auto" (by occupancy), "parallel" or "inline" (mrx_factor_path)."""
+    factor_path: None / "auto" (by occupancy), "parallel" or "inline" (mrx_factor_path).
+    reset_path: None / "auto", "passes" (one unit of work per episode of a chunk) or "merged" (one per chunk
+    behind a screen of its inputs: mrx_reset_path); the backward call takes the same argument."""
     lib = _lib.load()
     B, T, H, dk, dv, dt = _attn_shapes(q, k, v)
     _chk(beta, "beta", dt, (B, T, H))
@@ -397,12 +401,13 @@ def delta_rule_fwd(q, k, v, beta, done, S0=None, save_chk=True, out=None, prolog
     name = "mrx_deltanet_fwd" if prologue else "mrx_delta_rule_fwd"
     st = getattr(lib, name)(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done),
                             _ptr(S0), _ptr(o), _ptr(S_last), _ptr(S_chk), _ptr(Tm_chk), B, T, H,
-                            dk, dv, _DT[dt], dd, _FACTORS[factor_path])
+                            dk, dv, _DT[dt], dd, _FACTORS[factor_path], _RESETS[reset_path])
     _lib.check(st, name)
     return o, S_last, ((S_chk, Tm_chk) if save_chk else None)
 
 
-def delta_rule_bwd(q, k, v, beta, done, chk, do, dS_last=None, want_dS0=True, out=None, prologue=False):
+def delta_rule_bwd(q, k, v, beta, done, chk, do, dS_last=None, want_dS0=True, out=None, prologue=False,
+                   reset_path=None):
     """chk = (S_chk, Tm_chk) from delta_rule_fwd.  Returns (dq, dk, dv, dbeta, dS0).
     out = (dq, dk, dv, dbeta, dS0) reuses buffers instead of allocating.  prologue=True pairs with
     delta_rule_fwd(prologue=True): k and beta are the raw projections and so are dk and dbeta."""
@@ -429,7 +434,7 @@ def delta_rule_bwd(q, k, v, beta, done, chk, do, dS_last=None, want_dS0=True, ou
     name = "mrx_deltanet_bwd" if prologue else "mrx_delta_rule_bwd"
     st = getattr(lib, name)(_stream(), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(done),
                             _ptr(S_chk), _ptr(Tm_chk), _ptr(do), _ptr(dS_last), _ptr(dq), _ptr(dk_),
-                            _ptr(dv_), _ptr(dbeta), _ptr(dS0), B, T, H, dk, dv, _DT[dt], dd)
+                            _ptr(dv_), _ptr(dbeta), _ptr(dS0), B, T, H, dk, dv, _DT[dt], dd, _RESETS[reset_path])
     _lib.check(st, name)
     return dq, dk_, dv_, dbeta, dS0
 

@@ -448,10 +448,11 @@ class DeltaNetCell(MemoroidCellBase):
     idiom the elements are the affine maps (beta v k^T, I - beta k k^T) with
     binary_operator(a, b) = (B_a A_b + B_b, A_a A_b).  The carry is (S (B,1,H,d,d),)."""
 
-    def __init__(self, features, head_dim, num_heads, in_features=None, dtype=torch.bfloat16):
+    def __init__(self, features, head_dim, num_heads, in_features=None, dtype=torch.bfloat16, resets=None):
         super().__init__()
         in_features = features if in_features is None else in_features
         self.features, self.head_dim, self.num_heads, self.dtype = features, head_dim, num_heads, dtype
+        self.resets = resets   # None / "passes" / "merged": mrx_reset_path, for rollouts whose episodes end often
         hidden = head_dim * num_heads
         self.query = nn.Linear(in_features, hidden, bias=False)
         self.key = nn.Linear(in_features, hidden, bias=False)
@@ -478,7 +479,7 @@ class DeltaNetCell(MemoroidCellBase):
     def scan(self, z, initial_carry, done):
         q, k, v, beta_raw = z
         (S0,) = initial_carry
-        o, S_last = deltanet(q, k, v, beta_raw, done, S0[:, 0].float())
+        o, S_last = deltanet(q, k, v, beta_raw, done, S0[:, 0].float(), resets=self.resets)
         return o, (S_last[:, None],)
 
     def read(self, h, x, **kwargs):

@@ -69,10 +69,11 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.mrx_linear_scan_fwd(n, one, one, one, n, n, one, n, n, 2, 4, 4, 7, 0, 0) == -1  # no such dtype
     assert lib.mrx_linear_attn_fwd(n, one, one, one, one, n, one, n, n, 1, 8, 1, 72, 64, 1, 0, 0) == -2  # dk > 64
     assert lib.mrx_linear_attn_fwd(n, one, one, one, one, n, one, n, n, 1, 8, 1, 36, 64, 1, 0, 0) == -2  # 36 bf16: 4.5 segments
-    assert lib.mrx_delta_rule_fwd(n, one, one, one, one, one, n, one, n, n, n, 1, 8, 1, 64, 72, 1, 0, 0) == -2  # dv > 64
+    assert lib.mrx_delta_rule_fwd(n, one, one, one, one, one, n, one, n, n, n, 1, 8, 1, 64, 72, 1, 0, 0, 0) == -2  # dv > 64
+    assert lib.mrx_delta_rule_fwd(n, one, one, one, one, one, n, one, n, n, n, 1, 8, 1, 64, 64, 1, 0, 0, 3) == -1  # no such reset path
     assert lib.mrx_delta_rule_fwd_noalloc(n, one, one, one, one, one, n, one, n, 1, 8, 1, 32, 32, 1, 0) == -2  # 64 only
     assert lib.mrx_delta_rule_bwd(n, one, one, one, one, one, one, n, one, n, one, one, one, one, n,
-                                  1, 8, 1, 64, 64, 0, 0) == -1  # residual Tm_chk missing
+                                  1, 8, 1, 64, 64, 0, 0, 0) == -1  # residual Tm_chk missing
     assert lib.mrx_linear_attn_bwd(n, one, one, one, one, one, n, one, n, one, one, one, n,
                                    1, 8, 1, 64, 64, 0, 0, 0) == -1  # S_last missing
 

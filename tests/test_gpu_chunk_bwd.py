@@ -224,7 +224,14 @@ def test_normalised_read_out_walks_across_an_anchor():
     on, den, Sl, zl, chkn = K.linear_attn_norm_fwd(tq, tk, tv, dev(done), None, None, 1)
     gn = K.linear_attn_norm_bwd(tq, tk, tv, dev(done), chkn, on, den, tdo, None, None, 1)
     rn = G.normalised_linear_attention_grads(q, k, v, done, None, None, do, None, None, "elu1")
-    for name, a in zip(("dq", "dk", "dv"), gn):
+    for name, a in zip(("dk", "dv"), gn[1:]):
         assert relerr(a, rn[name]) <= TOL_F32, name
         for lo in (0, 992, 1024):
             assert relerr(a[:, lo:lo + 32], rn[name][:, lo:lo + 32]) <= TOL_F32, (name, lo)
+    # dq of a normalised read-out is what two terms leave that cancel -- the output does not depend on the
+    # scale of the mapped query phi(q), and over a thousand steps S^T dnum and dden z are each a hundred times
+    # their difference -- and each has the size of dk: that is the scale its error is judged on
+    dq = gn[0].cpu().numpy()
+    for lo, hi in ((0, T), (0, 32), (992, 1024), (1024, 1056)):
+        scale = np.abs(rn["dk"][:, lo:hi]).max()
+        assert np.abs(dq[:, lo:hi] - rn["dq"][:, lo:hi]).max() <= TOL_F32 * scale, (lo, hi)

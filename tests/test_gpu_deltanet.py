@@ -162,17 +162,17 @@ def test_chunk64_build_agrees_with_the_default_build():
     S_chk = torch.empty((B, H, NC, 64, 64), dtype=bf, device="cuda")
     Tm_chk = torch.empty((B, H, NC, 64, 64), dtype=bf, device="cuda")
     rc = lib.mrx_delta_rule_fwd(st, p(q), p(k), p(v), p(beta), p(done), p(S0), p(o2), p(Sl2), p(S_chk), p(Tm_chk),
-                                B, T, H, 64, 64, _lib.MRX_BF16, _lib.MRX_DONE_U8, _lib.MRX_FACTORS_AUTO)
+                                B, T, H, 64, 64, _lib.MRX_BF16, _lib.MRX_DONE_U8, _lib.MRX_FACTORS_AUTO, _lib.MRX_RESETS_AUTO)
     assert rc == 0, rc
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     db, dS0 = torch.empty_like(beta), torch.empty_like(S0)
     rc = lib.mrx_delta_rule_bwd(st, p(q), p(k), p(v), p(beta), p(done), p(S_chk), p(Tm_chk), p(do), None, p(dq), p(dk),
-                                p(dv), p(db), p(dS0), B, T, H, 64, 64, _lib.MRX_BF16, _lib.MRX_DONE_U8)
+                                p(dv), p(db), p(dS0), B, T, H, 64, 64, _lib.MRX_BF16, _lib.MRX_DONE_U8, _lib.MRX_RESETS_AUTO)
     assert rc == 0, rc
     torch.cuda.synchronize()
     for name, a, b_ in zip(("o", "S_last", "dq", "dk", "dv", "dbeta", "dS0"), (o2, Sl2, dq, dk, dv, db, dS0), ref):
         assert relerr(a, b_.float().cpu().numpy()) <= TOL_BF16, name
     # the chunk-parallel factor kernel exists for 32-step chunks only
     rc = lib.mrx_delta_rule_fwd(st, p(q), p(k), p(v), p(beta), p(done), p(S0), p(o2), p(Sl2), p(S_chk), p(Tm_chk),
-                                B, T, H, 64, 64, _lib.MRX_BF16, _lib.MRX_DONE_U8, _lib.MRX_FACTORS_PARALLEL)
+                                B, T, H, 64, 64, _lib.MRX_BF16, _lib.MRX_DONE_U8, _lib.MRX_FACTORS_PARALLEL, _lib.MRX_RESETS_AUTO)
     assert rc == -2, rc

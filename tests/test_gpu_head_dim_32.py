@@ -157,6 +157,6 @@ def test_other_head_dims_are_still_refused_and_the_static_scratch_variant_is_64_
     o = torch.empty_like(q)
     assert lib.mrx_linear_attn_fwd(None, P(q), P(q), P(q), P(dn), None, P(o), None, None, 1, 4, 1, 32, 32, 0, 0, 0) == 0
     # nothing is launched on a refusal
-    assert lib.mrx_delta_rule_fwd(None, P(q), P(q), P(q), P(beta), P(dn), None, P(o), None, None, None, 1, 4, 1, 32, 72, 0, 0, 0) == -2
+    assert lib.mrx_delta_rule_fwd(None, P(q), P(q), P(q), P(beta), P(dn), None, P(o), None, None, None, 1, 4, 1, 32, 72, 0, 0, 0, 0) == -2
     assert lib.mrx_delta_rule_fwd_noalloc(None, P(q), P(q), P(q), P(beta), P(dn), None, P(o), None, 1, 4, 1, 32, 32, 0, 0) == -2
     torch.cuda.synchronize()

@@ -270,8 +270,8 @@ def test_what_is_not_a_narrow_head_is_refused():
     dn = torch.zeros((1, 4), dtype=torch.uint8, device="cuda")
     beta = torch.zeros((1, 4, 1), device="cuda")
     o = torch.empty_like(q)
-    assert lib.mrx_delta_rule_fwd(None, P(q), P(q), P(q), P(beta), P(dn), None, P(o), None, None, None, 1, 4, 1, 16, 16, 0, 0, 0) == 0
-    assert lib.mrx_delta_rule_fwd(None, P(q), P(q), P(q), P(beta), P(dn), None, P(o), None, None, None, 1, 4, 1, 16, 6, 0, 0, 0) == -2
+    assert lib.mrx_delta_rule_fwd(None, P(q), P(q), P(q), P(beta), P(dn), None, P(o), None, None, None, 1, 4, 1, 16, 16, 0, 0, 0, 0) == 0
+    assert lib.mrx_delta_rule_fwd(None, P(q), P(q), P(q), P(beta), P(dn), None, P(o), None, None, None, 1, 4, 1, 16, 6, 0, 0, 0, 0) == -2
     assert lib.mrx_delta_rule_fwd_noalloc(None, P(q), P(q), P(q), P(beta), P(dn), None, P(o), None, 1, 4, 1, 16, 16, 0, 0) == -2
     torch.cuda.synchronize()
 

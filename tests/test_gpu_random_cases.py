@@ -83,8 +83,11 @@ def test_random_cases(seed):
         else:
             pro = op == "deltanet"
             tb = dev(beta, td)
-            o, Sl, chk = K.delta_rule_fwd(tq, tk, tv, tb, dn, tS0, prologue=pro, factor_path=c["path"])
-            got = K.delta_rule_bwd(tq, tk, tv, tb, dn, chk, tdo, tdSl, prologue=pro)
+            # every second case with all episodes of a chunk in one unit (taken from the drawn sizes, so that
+            # the cases themselves stay what they were)
+            resets = "merged" if (B + T + H) % 2 else None
+            o, Sl, chk = K.delta_rule_fwd(tq, tk, tv, tb, dn, tS0, prologue=pro, factor_path=c["path"], reset_path=resets)
+            got = K.delta_rule_bwd(tq, tk, tv, tb, dn, chk, tdo, tdSl, prologue=pro, reset_path=resets)
             ref = (G.deltanet_grads if pro else G.delta_rule_grads)(q, k, v, beta, done, S0, do, dSl)
             names = ("dq", "dk", "dv", "dbeta", "dS0")
         torch.cuda.synchronize()

@@ -34,7 +34,7 @@ def _call_pair(lib, _lib, B, T, H, dtype, seed):
     o_ref, Sl_ref = torch.empty_like(v), torch.empty_like(S0)
     tm = torch.empty((B, H, NC, 32, 32), dtype=dtype, device="cuda")
     rc = lib.mrx_delta_rule_fwd(st, p(q), p(k), p(v), p(beta), p(done), p(S0), p(o_ref), p(Sl_ref), None, p(tm),
-                                B, T, H, 64, 64, dt, _lib.MRX_DONE_U8, _lib.MRX_FACTORS_PARALLEL)
+                                B, T, H, 64, 64, dt, _lib.MRX_DONE_U8, _lib.MRX_FACTORS_PARALLEL, _lib.MRX_RESETS_AUTO)
     assert rc == 0, rc
     # outputs pre-filled so that an entry point that wrote nothing cannot pass
     o, Sl = torch.full_like(v, float("nan")), torch.full_like(S0, float("nan"))
