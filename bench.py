@@ -147,13 +147,17 @@ def main() -> int:
     torch.cuda.synchronize()
 
     # outputs and residuals are allocated once and reused, as a training loop's caching allocator does
-    o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done)
+    # Episodes end every five hundred steps in this configuration: the step asks for all episodes of a chunk in
+    # one unit of work (MRX_RESETS_MERGED: same results, a chunk with a reset costs one unit instead of two);
+    # the library's default, one unit per episode, is timed beside it ("resets_per_episode").
+    RESETS = None if args.lib else "merged"   # the other builds of the library (64-step chunks, clocks) keep the default
+    o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done, reset_path=RESETS)
     fwd_out = (o, Sl, chk[0], chk[1])
-    bwd_out = K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False)
+    bwd_out = K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, reset_path=RESETS)
 
-    def step():
-        K.delta_rule_fwd(q, k, v, beta, done, out=fwd_out)
-        return K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, out=bwd_out)
+    def step(resets=RESETS):
+        K.delta_rule_fwd(q, k, v, beta, done, out=fwd_out, reset_path=resets)
+        return K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, out=bwd_out, reset_path=resets)
 
     # The device needs some 30 ms of continuous load to reach its clocks (measured: 20-step batches
     # right after an idle stretch read 0.32, 0.29, 0.28, 0.27, 0.27 ms per step): an untimed ramp of the
@@ -171,6 +175,14 @@ def main() -> int:
         step()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
+    for _ in range(10):
+        step(None)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(None)
+    torch.cuda.synchronize()
+    dt_passes = (time.perf_counter() - t0) / args.steps
 
     # per-kernel durations with HIP events on the stream the kernels are launched on
     ev = lambda: torch.cuda.Event(enable_timing=True)  # noqa: E731
@@ -178,9 +190,9 @@ def main() -> int:
     for _ in range(max(args.steps, 50)):
         e0, e1, e2 = ev(), ev(), ev()
         e0.record()
-        K.delta_rule_fwd(q, k, v, beta, done, out=fwd_out)
+        K.delta_rule_fwd(q, k, v, beta, done, out=fwd_out, reset_path=RESETS)
         e1.record()
-        K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, out=bwd_out)
+        K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, out=bwd_out, reset_path=RESETS)
         e2.record()
         torch.cuda.synchronize()
         tfs.append(e0.elapsed_time(e1))
@@ -209,7 +221,9 @@ def main() -> int:
         "data": "synthetic",
         "clock_ramp_ms": args.ramp_ms,
         "config": {"workload": "configs[3]: DeltaNet delta rule fwd+bwd, B=64 H=8 T=1024 d=64, "
-                               f"bf16 in / fp32 state, chunk {C}, resets p=0.002"},
+                               f"bf16 in / fp32 state, chunk {C}, resets p=0.002"
+                               + (", episodes of a chunk merged (MRX_RESETS_MERGED)" if RESETS else "")},
+        "ms_per_step_resets_per_episode": dt_passes * 1e3,
         "roofline": {
             "bound": "hbm", "kernel": "delta_bwd_kernel", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": TRAFFIC_BWD_BYTES,
@@ -274,19 +288,18 @@ def phase_clocks_child(np, torch, K, dev):
     do_np = np.random.default_rng(2004).standard_normal((B, T, H, d)).astype(np.float32)
     q, k, v, beta, do = (dev(a).to(bf) for a in (x["q"], x["k"], x["v"], x["beta"], do_np))
     done = dev(x["done"])
-    o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done)
-    out = K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False)
+    o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done, reset_path="merged")   # as the headline step calls it
+    out = K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, reset_path="merged")
     for _ in range(20):
-        K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, out=out)
+        K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, out=out, reset_path="merged")
     buf = (ctypes.c_ulonglong * 4)()
     assert lib.mrx_phase_clocks(buf, 1) == 0
     n = 20
     for _ in range(n):
-        K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, out=out)
+        K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, out=out, reset_path="merged")
     assert lib.mrx_phase_clocks(buf, 1) == 0
     C = K.chunk_size(bf, delta=True)
-    dn = x["done"].reshape(B, T // C, C)
-    passes = float((1 + dn.sum(-1)).sum()) / B   # per sequence (every head of a batch row shares the resets)
+    passes = float(T // C)   # units of work per sequence: one per chunk with the episodes merged
     return {"product_clocks": int(buf[0]), "wave_clocks": int(buf[1]), "workgroups": int(buf[2]), "launches": n,
             "passes_per_sequence": passes}
 

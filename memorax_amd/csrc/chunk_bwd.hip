@@ -924,33 +924,70 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
         // (measured: 10 % on chunks without resets), two copies of the unit do not fit the registers.
         const bool MG = MERGE && mg;
         // ff / fl: 1 for the rows (nt * 16 + li of the wave's [C][64]-shaped tiles) of the first / last episode, else
-        // 0; cc: bit 4 j + e set when element e of the wave's [C][C] tile j pairs two rows of one episode
-        float ff[TMR::NBW], fl[TMR::NBW];
-        unsigned cc = 0u;
-        if constexpr (MERGE) {
+        // 0; cw: the packed words of the wave's [C][C] tile j keep the bits of the elements that pair two rows of
+        // one episode; fw: the words of an operand fragment read along the chunk rows (element e of the fragment of k block kb is
+        // row kb KB + KP lg + e) keep the bits of the rows of the first episode; keep_dS: 0 where the gradient of
+        // the state that leaves the chunk does not flow on past it
+        constexpr int NKB = C / TT<T>::KB, WPF = TT<T>::KP * (int)sizeof(T) / 4;  // k blocks; 32-bit words per fragment
+        float ff[TMR::NBW], fl[TMR::NBW], keep_dS = 1.f;
+        constexpr int WPP = 4 * (int)sizeof(T) / 4;  // 32-bit words of four packed elements
+        unsigned cw[TMA::TPW][WPP], fw[NKB][WPF];
+#pragma unroll
+        for (int j = 0; j < TMA::TPW; ++j)
+#pragma unroll
+            for (int i = 0; i < WPP; ++i) cw[j][i] = ~0u;
+#pragma unroll
+        for (int ni = 0; ni < TMR::NBW; ++ni) ff[ni] = fl[ni] = 1.f;
+#pragma unroll
+        for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+            for (int i = 0; i < WPF; ++i) fw[kb][i] = ~0u;
+        if (MG) {  // once per chunk, outside the unit's phases
+            keep_dS = 0.f;
 #pragma unroll
             for (int ni = 0; ni < TMR::NBW; ++ni) {
                 const int r = TMR::nt(w, ni) * 16 + li;
-                ff[ni] = !MG || r < r_first ? 1.f : 0.f;
-                fl[ni] = !MG || r >= r_last ? 1.f : 0.f;
+                ff[ni] = r < r_first ? 1.f : 0.f;
+                fl[ni] = r >= r_last ? 1.f : 0.f;
             }
 #pragma unroll
-            for (int j = 0; j < TMA::TPW; ++j)
+            for (int j = 0; j < TMA::TPW; ++j) {
+                bool same[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int m = TMA::mt(w, j) * 16 + 4 * lg + e, n = TMA::nt(w, j) * 16 + li;
-                    if (!MG || one_episode(m < n ? m : n, m < n ? n : m)) cc |= 1u << (4 * j + e);
+                    same[e] = one_episode(m < n ? m : n, m < n ? n : m);
+                }
+#pragma unroll
+                for (int i = 0; i < WPP; ++i)
+                    cw[j][i] = sizeof(T) == 2 ? (same[2 * i] ? 0x0000ffffu : 0u) | (same[2 * i + 1] ? 0xffff0000u : 0u)
+                                              : (same[i % 4] ? ~0u : 0u);
+            }
+#pragma unroll
+            for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+                for (int i = 0; i < WPF; ++i) {
+                    const int k0 = kb * TT<T>::KB + TT<T>::KP * lg;
+                    if (sizeof(T) == 2)
+                        fw[kb][i] = (k0 + 2 * i < r_first ? 0x0000ffffu : 0u) | (k0 + 2 * i + 1 < r_first ? 0xffff0000u : 0u);
+                    else
+                        fw[kb][i] = k0 + i < r_first ? ~0u : 0u;
                 }
         }
-        // masked store of a [C][C] product as dst[n][m]: tri(m, n) and, merged, the pair's bit of cc
+        // masked store of a [C][C] product as dst[n][m]: tri(m, n) as in the other instance (a compile-time
+        // pattern for most tiles), then the packed words ANDed with the chunk's episode mask
         auto store_cc = [&](const f32x4 *acc, T *dst, auto tri, float sign) {
 #pragma unroll
             for (int j = 0; j < TMA::TPW; ++j) {
                 const int m = TMA::mt(w, j) * 16 + 4 * lg, n = TMA::nt(w, j) * 16 + li;
                 float x[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) x[e] = tri(m + e, n) && (!MERGE || ((cc >> (4 * j + e)) & 1u)) ? sign * acc[j][e] : 0.f;
-                *reinterpret_cast<P4 *>(dst + n * LDC + m) = TT<T>::pack(x[0], x[1], x[2], x[3]);
+                for (int e = 0; e < 4; ++e) x[e] = tri(m + e, n) ? sign * acc[j][e] : 0.f;
+                typedef uint32_t words_t __attribute__((ext_vector_type(WPP)));
+                words_t wv = __builtin_bit_cast(words_t, TT<T>::pack(x[0], x[1], x[2], x[3]));
+#pragma unroll
+                for (int i = 0; i < WPP; ++i) wv[i] &= cw[j][i];
+                *reinterpret_cast<words_t *>(dst + n * LDC + m) = wv;
             }
         };
         for (int pass = MG ? 0 : nres; pass >= 0; --pass) {
@@ -1139,14 +1176,18 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             {
                 f32x4 acc[TMS::TPW];
                 zero_acc<TMS::TPW>(acc);
-                if (MG) {
-                    // a chunk with resets: what flows on to the chunk before is the first episode's own sum
-                    zero_acc<TMS::TPW>(dSacc);
-                    auto first_rows = [&](int, int kb, typename TT<T>::frag &x) {  // element e of the fragment is chunk row k0 + e
-                        const int k0 = kb * TT<T>::KB + TT<T>::KP * lg;
+                if constexpr (MERGE) {
+                    // a merged chunk: what flows on to the chunk before is the first episode's own sum -- the
+                    // incoming gradient is dropped and the operand fragments keep the first episode's rows
+                    // (straight-line: all-pass values in every other chunk)
 #pragma unroll
-                        for (int e = 0; e < TT<T>::KP; ++e)
-                            if (k0 + e >= r_first) x[e] = (T)0.f;
+                    for (int j = 0; j < TMS::TPW; ++j) dSacc[j] *= keep_dS;
+                    auto first_rows = [&](int, int kb, typename TT<T>::frag &x) {
+                        typedef uint32_t words_t __attribute__((ext_vector_type(WPF)));
+                        words_t wv = __builtin_bit_cast(words_t, x);
+#pragma unroll
+                        for (int i = 0; i < WPF; ++i) wv[i] &= fw[kb][i];
+                        x = __builtin_bit_cast(typename TT<T>::frag, wv);
                     };
                     gemm<T, HD, HD, C, KROW, KROW, NW>(dSacc, sQ, LDD, sDO, LDD, w, lane, first_rows);
                     gemm<T, HD, HD, C, KROW, KROW, NW>(acc, sK, LDD, sZb, LDD, w, lane, first_rows);

@@ -750,6 +750,7 @@ int delta_fwd_dispatch(hipStream_t st, const void *q, const void *k, const void 
     // kernel the units per episode stay (on a full device, where that path is the rule, a chunk with resets
     // costs the forward a few per cent, less than the factor kernel would)
     const bool merged = MRX_HD == 64 && TM_KERNEL && reset_path == MRX_RESETS_MERGED && parallel;
+    (void)merged;  // the head-dim-32 build has no merged instances
     if (!TM_KERNEL && factor_path == MRX_FACTORS_PARALLEL) return MRX_ERR_UNSUPPORTED;
     if constexpr (TM_KERNEL) if (parallel) {
         const int rc = launch_delta_tm(st, k, beta, done, done_dtype, Tm_chk, B, T, H, dtype, PRO, dk);
