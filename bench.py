@@ -147,10 +147,11 @@ def main() -> int:
     torch.cuda.synchronize()
 
     # outputs and residuals are allocated once and reused, as a training loop's caching allocator does
-    # Episodes end every five hundred steps in this configuration: the step asks for all episodes of a chunk in
-    # one unit of work (MRX_RESETS_MERGED: same results, a chunk with a reset costs one unit instead of two);
-    # the library's default, one unit per episode, is timed beside it ("resets_per_episode").
-    RESETS = None if args.lib else "merged"   # the other builds of the library (64-step chunks, clocks) keep the default
+    # The step runs the library's defaults (one unit of work per episode of a chunk that holds resets).  Episodes
+    # end every five hundred steps in this configuration, where MRX_RESETS_MERGED (all episodes of a chunk in one
+    # unit) is level with the default; it is timed beside it ("ms_per_step_merged_resets") and pays at the
+    # torso's reset rate (the torso block).
+    RESETS = None
     o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done, reset_path=RESETS)
     fwd_out = (o, Sl, chk[0], chk[1])
     bwd_out = K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, reset_path=RESETS)
@@ -175,14 +176,16 @@ def main() -> int:
         step()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
-    for _ in range(10):
-        step(None)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step(None)
-    torch.cuda.synchronize()
-    dt_passes = (time.perf_counter() - t0) / args.steps
+    dt_merged = None
+    if not args.lib:   # the other builds of the library (64-step chunks, clocks) have no use for it
+        for _ in range(10):
+            step("merged")
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step("merged")
+        torch.cuda.synchronize()
+        dt_merged = (time.perf_counter() - t0) / args.steps
 
     # per-kernel durations with HIP events on the stream the kernels are launched on
     ev = lambda: torch.cuda.Event(enable_timing=True)  # noqa: E731
@@ -222,8 +225,8 @@ def main() -> int:
         "clock_ramp_ms": args.ramp_ms,
         "config": {"workload": "configs[3]: DeltaNet delta rule fwd+bwd, B=64 H=8 T=1024 d=64, "
                                f"bf16 in / fp32 state, chunk {C}, resets p=0.002"
-                               + (", episodes of a chunk merged (MRX_RESETS_MERGED)" if RESETS else "")},
-        "ms_per_step_resets_per_episode": dt_passes * 1e3,
+                               },
+        "ms_per_step_merged_resets": None if dt_merged is None else dt_merged * 1e3,
         "roofline": {
             "bound": "hbm", "kernel": "delta_bwd_kernel", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": TRAFFIC_BWD_BYTES,
@@ -288,18 +291,19 @@ def phase_clocks_child(np, torch, K, dev):
     do_np = np.random.default_rng(2004).standard_normal((B, T, H, d)).astype(np.float32)
     q, k, v, beta, do = (dev(a).to(bf) for a in (x["q"], x["k"], x["v"], x["beta"], do_np))
     done = dev(x["done"])
-    o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done, reset_path="merged")   # as the headline step calls it
-    out = K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, reset_path="merged")
+    o, Sl, chk = K.delta_rule_fwd(q, k, v, beta, done)
+    out = K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False)
     for _ in range(20):
-        K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, out=out, reset_path="merged")
+        K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, out=out)
     buf = (ctypes.c_ulonglong * 4)()
     assert lib.mrx_phase_clocks(buf, 1) == 0
     n = 20
     for _ in range(n):
-        K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, out=out, reset_path="merged")
+        K.delta_rule_bwd(q, k, v, beta, done, chk, do, None, want_dS0=False, out=out)
     assert lib.mrx_phase_clocks(buf, 1) == 0
     C = K.chunk_size(bf, delta=True)
-    passes = float(T // C)   # units of work per sequence: one per chunk with the episodes merged
+    dn = x["done"].reshape(B, T // C, C)
+    passes = float((1 + dn.sum(-1)).sum()) / B   # units of work per sequence (every head of a batch row shares the resets)
     return {"product_clocks": int(buf[0]), "wave_clocks": int(buf[1]), "workgroups": int(buf[2]), "launches": n,
             "passes_per_sequence": passes}
 
