@@ -261,7 +261,7 @@ la_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restr
                 for (int p = 0; p < IOS::PASSES; ++p)
                     if (IOS::FULL || IOS::row_of(tid, p) < HD) {  // a [32][32] tile has fewer segments than threads
                         if (!NARROW || (IOS::row_of(tid, p) < dvw && (tid % IOS::SEGS) * IOS::KP < dkw))
-                            rS.v[p] = *reinterpret_cast<const typename IOS::F *>(reinterpret_cast<const T *>(S_chk) + soff + p * IOS::RPP * dkw);
+                            rS.v[p] = load_once<typename IOS::F>(reinterpret_cast<const T *>(S_chk) + soff + p * IOS::RPP * dkw);
                         else
                             rS.v[p] = z;
                     }
@@ -819,7 +819,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
             for (int p = 0; p < IOS::PASSES; ++p)
                 if (IOS::FULL || IOS::row_of(tid, p) < HD) {
                     if (!NARROW || (IOS::row_of(tid, p) < dvw && (tid % IOS::SEGS) * IOS::KP < dkw))
-                        rS.v[p] = *reinterpret_cast<const typename IOS::F *>(S_chk + soff + p * IOS::RPP * dkw);
+                        rS.v[p] = load_once<typename IOS::F>(S_chk + soff + p * IOS::RPP * dkw);
                     else
                         rS.v[p] = z;
                 }
@@ -827,7 +827,7 @@ delta_bwd_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__re
 #pragma unroll
             for (int p = 0; p < IOT::PASSES; ++p)
                 if (IOT::FULL || IOT::row_of(tid, p) < C)  // a [C][C] tile may have fewer segments than threads
-                    rTm.v[p] = *reinterpret_cast<const typename IOT::F *>(Tm_chk + tmoff + p * IOT::RPP * C);
+                    rTm.v[p] = load_once<typename IOT::F>(Tm_chk + tmoff + p * IOT::RPP * C);
 #pragma unroll
             for (int p = 0; p < IO::PASSES; ++p) {
                 rbrow[p] = (IO::FULL || IO::row_of(tid, p) < C) && tpre + IO::row_of(tid, p) < Tlen ? load_raw<T>(beta + boff[p]) : 0u;

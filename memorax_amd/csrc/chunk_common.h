@@ -68,6 +68,16 @@ template <typename T> constexpr int walk_anchor() { return sizeof(T) == 2 ? 128 
 // row dots behind dbeta, 2^6 x 2^6 x 2^110), inside the float32 range.
 constexpr float MERGE_IN_MAX = 64.f, MERGE_STATE_MAX = 1048576.f;
 
+// A 16-byte global load of data that no later kernel reads again (the residuals a backward call consumes):
+// non-temporal, so that it does not displace what the next kernels will read -- inputs, and the residuals the
+// forward call has just written -- from the last-level cache.  Row stores of results take the same hint
+// (tile_rows_to_global).  Measured on the delta rule at 64 x 1024 x 8: forward + backward 0.266 -> 0.260 ms;
+// the same hint on the loads of q, k, v costs the forward 3 % there (it reads k right after the factor
+// kernel has), and on the stores of the residuals it costs the backward what it saves the forward.
+template <typename F, typename P> __device__ __forceinline__ F load_once(const P *p)
+{
+    return __builtin_nontemporal_load(reinterpret_cast<const F *>(p));
+}
 enum OpMode { ROWK = 0, KROW = 1 };
 
 template <typename T> struct TT;
@@ -391,9 +401,9 @@ __device__ __forceinline__ void tile_rows_to_global(const T *tile, int ld, T *g,
 #pragma unroll
     for (int p = 0; p < IO::PASSES; ++p) {
         const int r = IO::row_of(tid, p);
-        if ((IO::FULL || r < C) && t0 + r < Tlen && keep(r))
-            *reinterpret_cast<typename IO::F *>(g + (int64_t)r * rs + seg * IO::KP) =
-                *reinterpret_cast<const typename IO::F *>(tile + r * ld + seg * IO::KP);
+        if ((IO::FULL || r < C) && t0 + r < Tlen && keep(r))  // results are not read again by these kernels: non-temporal
+            __builtin_nontemporal_store(*reinterpret_cast<const typename IO::F *>(tile + r * ld + seg * IO::KP),
+                                        reinterpret_cast<typename IO::F *>(g + (int64_t)r * rs + seg * IO::KP));
     }
 }
 

@@ -58,14 +58,42 @@ template <typename E, int VEC> __device__ __forceinline__ Vec<E, VEC> vfill(E x)
     return r;
 }
 
+// Every (B,T,D) array is read or written once per launch and not again before the next kernel: its loads and
+// stores are non-temporal, so that the stream does not sit in the caches at the expense of itself (measured at
+// 512 x 1024 x 1024 float32: forward 5.77 -> 6.05 TB/s, backward 5.74 -> 6.27 TB/s).  The built-ins take
+// scalars and vectors of the language, so a Vec or a raw word group goes through a word type of its size.
+template <int BYTES> struct StreamWord;
+template <> struct StreamWord<2> { using type = uint16_t; };
+template <> struct StreamWord<4> { using type = uint32_t; };
+template <> struct StreamWord<8> { typedef uint32_t type __attribute__((ext_vector_type(2))); };
+template <> struct StreamWord<16> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
+template <typename X> __device__ __forceinline__ X ld_stream(const void *p)
+{
+    if constexpr (sizeof(X) <= 16) {
+        using W = typename StreamWord<sizeof(X)>::type;
+        return __builtin_bit_cast(X, __builtin_nontemporal_load(reinterpret_cast<const W *>(p)));
+    } else {
+        return *reinterpret_cast<const X *>(p);  // wider than one instruction moves (complex64 x 4)
+    }
+}
+template <typename X> __device__ __forceinline__ void st_stream(void *p, const X &x)
+{
+    if constexpr (sizeof(X) <= 16) {
+        using W = typename StreamWord<sizeof(X)>::type;
+        __builtin_nontemporal_store(__builtin_bit_cast(W, x), reinterpret_cast<W *>(p));
+    } else {
+        *reinterpret_cast<X *>(p) = x;
+    }
+}
+
 // Storage and arithmetic types of the (B,T,D) arrays may differ: bfloat16 in memory, float in registers
 // (the carries -- h0, P0, h_last, P_last, g_last, dh0 -- are always in the arithmetic type).
 template <typename S, typename E, int VEC> __device__ __forceinline__ Vec<E, VEC> ldv(const S *p)
 {
     if constexpr (std::is_same<S, E>::value) {
-        return *reinterpret_cast<const Vec<E, VEC> *>(p);
+        return ld_stream<Vec<E, VEC>>(p);
     } else {
-        const Vec<S, VEC> raw = *reinterpret_cast<const Vec<S, VEC> *>(p);
+        const Vec<S, VEC> raw = ld_stream<Vec<S, VEC>>(p);
         Vec<E, VEC> r;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) r.v[i] = (E)raw.v[i];
@@ -95,7 +123,7 @@ template <typename S, int VEC> __device__ __forceinline__ raw_t<S, VEC> ldraw(co
         r.w[0] = *reinterpret_cast<const uint16_t *>(p);
         return r;
     } else {
-        return *reinterpret_cast<const raw_t<S, VEC> *>(p);
+        return ld_stream<raw_t<S, VEC>>(p);
     }
 }
 template <typename S, typename E, int VEC> __device__ __forceinline__ Vec<E, VEC> cvtv(const raw_t<S, VEC> &raw)
@@ -116,12 +144,12 @@ template <typename S, typename E, int VEC> __device__ __forceinline__ Vec<E, VEC
 template <typename S, typename E, int VEC> __device__ __forceinline__ void stv(S *p, const Vec<E, VEC> &x)
 {
     if constexpr (std::is_same<S, E>::value) {
-        *reinterpret_cast<Vec<E, VEC> *>(p) = x;
+        st_stream(p, x);
     } else {
         Vec<S, VEC> raw;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) raw.v[i] = (S)x.v[i];
-        *reinterpret_cast<Vec<S, VEC> *>(p) = raw;
+        st_stream(p, raw);
     }
 }
 
