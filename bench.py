@@ -249,6 +249,14 @@ def main() -> int:
     if not args.headline_only:
         if not args.no_children:
             out["roofline"].update(bench_gemm_phase(MFMA_BUSY_BWD))
+            ap_ = out["roofline"].get("access_pattern")
+            if ap_:  # the kernels' times against what their access pattern alone costs (access_pattern_times)
+                out["roofline"]["access_pattern_ms"] = ap_["delta_bwd_ms"]
+                out["roofline"]["access_pattern_over_launch"] = ap_["delta_bwd_ms"] / tb_ms
+                la3 = secondary.get("linear_attention", {}).get("cfg3_bf16_256x4096x8x64")
+                if la3:
+                    la3["access_pattern_ms"] = ap_["cfg3_fwd_ms"] + ap_["cfg3_bwd_ms"]
+                    la3["access_pattern_over_ms"] = la3["access_pattern_ms"] / la3["ms"]
         if "hbm_copy" in secondary:
             out["roofline"]["hbm_copy_GB/s"] = secondary["hbm_copy"]["GB/s"]
             out["roofline"]["frac_of_copy_rate"] = bwd_gbs / secondary["hbm_copy"]["GB/s"]
@@ -304,8 +312,43 @@ def phase_clocks_child(np, torch, K, dev):
     C = K.chunk_size(bf, delta=True)
     dn = x["done"].reshape(B, T // C, C)
     passes = float((1 + dn.sum(-1)).sum()) / B   # units of work per sequence (every head of a batch row shares the resets)
+    del q, k, v, beta, do, o, Sl, chk, out
     return {"product_clocks": int(buf[0]), "wave_clocks": int(buf[1]), "workgroups": int(buf[2]), "launches": n,
-            "passes_per_sequence": passes}
+            "passes_per_sequence": passes, "access_pattern": access_pattern_times(torch, lib)}
+
+
+def access_pattern_times(torch, lib):
+    """What the chunked kernels' access pattern costs without their arithmetic (mrx_pattern_probe of the
+    measurement build: one workgroup of four waves per (b, h), two per compute unit, 128-byte rows H rows apart,
+    a chunk at a time with the next one requested ahead, results written row-wise; per-chunk residual blocks
+    each way).  Milliseconds per launch for the delta rule at the headline shape (sequential forward kernel:
+    q, k, v + 2 KB factor in, o + 8 KB checkpoint out per 32-row chunk; backward: q, k, v, dO + 10 KB in,
+    dq, dk, dv out, last chunk first) and for plain linear attention at configuration 3's size (64-row chunks)."""
+    import ctypes
+    f = lib.mrx_pattern_probe
+    vp, i64 = ctypes.c_void_p, ctypes.c_int64
+    f.argtypes = [vp, ctypes.POINTER(vp), ctypes.c_int, ctypes.POINTER(vp), ctypes.c_int, vp, ctypes.c_int, vp, ctypes.c_int,
+                  i64, i64, i64, ctypes.c_int, ctypes.c_int]
+    f.restype = ctypes.c_int
+
+    def time_case(B, T, H, C, n_in, n_out, res_in, res_out, reverse, iters):
+        arrs = [torch.empty((B, T, H, 64), dtype=torch.bfloat16, device="cuda").fill_(1.0) for _ in range(n_in + n_out)]
+        NC = T // C
+        rin = torch.zeros((B * H * NC * max(res_in, 16),), dtype=torch.uint8, device="cuda")
+        rout = torch.zeros((B * H * NC * max(res_out, 16),), dtype=torch.uint8, device="cuda")
+        ins = (vp * n_in)(*[a.data_ptr() for a in arrs[:n_in]])
+        outs = (vp * n_out)(*[a.data_ptr() for a in arrs[n_in:]])
+        st = torch.cuda.current_stream().cuda_stream
+
+        def go():
+            rc = f(st, ins, n_in, outs, n_out, rin.data_ptr(), res_in, rout.data_ptr(), res_out, B, T, H, C, reverse)
+            assert rc == 0, rc
+        return _time_ms(torch, go, iters=iters)
+    out = {"delta_fwd_sequential_ms": time_case(64, 1024, 8, 32, 3, 1, 2048, 8192, 0, 50),
+           "delta_bwd_ms": time_case(64, 1024, 8, 32, 4, 3, 10240, 0, 1, 50),
+           "cfg3_fwd_ms": time_case(256, 4096, 8, 64, 3, 1, 0, 0, 0, 5),
+           "cfg3_bwd_ms": time_case(256, 4096, 8, 64, 4, 3, 0, 0, 1, 5)}
+    return out
 
 
 def bench_gemm_phase(mfma_busy):
@@ -330,7 +373,8 @@ def bench_gemm_phase(mfma_busy):
     prod_per_wave = d["product_clocks"] / waves
     share = d["product_clocks"] / d["wave_clocks"]
     mfma_cycles = MFMAS_PER_PASS_BWD * d["passes_per_sequence"] * MFMA_CYCLES_16x16x32_BF16
-    return {"mfma_gemm_phase_frac": mfma_cycles / prod_per_wave, "product_phase_share": share,
+    return {"access_pattern": d.get("access_pattern"),
+            "mfma_gemm_phase_frac": mfma_cycles / prod_per_wave, "product_phase_share": share,
             "mfma_busy_over_product_phase_share": mfma_busy / share,
             "mfma_gemm_phase_method": "shader-clock brackets around every product in the measurement build "
                                       "(libmemorax_amd_clk.so), 20 launches; per wave: 48 MFMAs/pass x 16 cycles / bracketed cycles"}

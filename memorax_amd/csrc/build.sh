@@ -4,8 +4,10 @@
 #   libmemorax_amd_c64.so  the same sources with the delta rule's bf16 kernels on 64-step chunks; only
 #                          bench.py loads it, to time that chunk length beside the default 32
 #   libmemorax_amd_clk.so  the library with chunk_bwd.hip compiled for measurement (MRX_PHASE_CLOCKS: shader-clock
-#                          brackets around every matrix product); only bench.py loads it, for the share of a
-#                          wave's time that delta_bwd_kernel spends inside products
+#                          brackets around every matrix product) and with pattern_probe.hip (the memory side of the
+#                          chunked kernels without their arithmetic); only bench.py loads it, for the share of a
+#                          wave's time that delta_bwd_kernel spends inside products and for what the kernels'
+#                          access pattern alone costs
 #   memorax_amd/csrc/build.sh
 set -euo pipefail
 cd "$(dirname "$0")"
@@ -33,12 +35,14 @@ ALL_SRCS=("${SRCS[@]}"); SRCS=("${HD32_SRCS[@]}")
 compile _hd32 -DMRX_HD=32
 SRCS=(chunk_bwd.hip)
 compile _clk -DMRX_PHASE_CLOCKS=1
+SRCS=(pattern_probe.hip)
+compile ""
 SRCS=("${ALL_SRCS[@]}")
 for p in "${pids[@]}"; do wait "$p"; done
 HD32_OBJS=$(printf '%s_hd32.o ' "${HD32_SRCS[@]%.hip}")
 "$HIPCC" --offload-arch=gfx950 -shared -fPIC -o libmemorax_amd.so $(printf '%s.o ' "${SRCS[@]%.hip}") $HD32_OBJS
 "$HIPCC" --offload-arch=gfx950 -shared -fPIC -o libmemorax_amd_c64.so $(printf '%s_c64.o ' "${SRCS[@]%.hip}") $HD32_OBJS
 CLK_OBJS=$(printf '%s.o ' "${SRCS[@]%.hip}" | sed 's/chunk_bwd\.o/chunk_bwd_clk.o/')
-"$HIPCC" --offload-arch=gfx950 -shared -fPIC -o libmemorax_amd_clk.so $CLK_OBJS $HD32_OBJS
+"$HIPCC" --offload-arch=gfx950 -shared -fPIC -o libmemorax_amd_clk.so $CLK_OBJS pattern_probe.o $HD32_OBJS
 rm -f ./*.o
 echo "built $(pwd)/libmemorax_amd.so, libmemorax_amd_c64.so and libmemorax_amd_clk.so"
