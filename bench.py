@@ -34,10 +34,10 @@ BYTES_FWD, BYTES_BWD = 514, 900
 # FETCH_SIZE and WRITE_SIZE runs scaled by a plain elementwise kernel of known size
 # (summary kept under profiles/).  The excess over the algorithmic bytes is the forward's
 # per-chunk residuals (state checkpoints and triangular factors) being read back.
-TRAFFIC_BWD_BYTES = 640.1e6
+TRAFFIC_BWD_BYTES = 639.9e6
 # Matrix-pipe busy fraction of delta_bwd_kernel from rocprofv3 --pmc (SQ_VALU_MFMA_BUSY_CYCLES over
 # SQ_BUSY_CYCLES per SIMD), same workload; summary and command under profiles/.
-MFMA_BUSY_BWD = 0.149
+MFMA_BUSY_BWD = 0.150
 MFMA_BUSY_SOURCE = "profiles/delta_rule_kernels_counters_B64_T1024_H8_d64_bf16.md"
 CLOCK_RAMP_S = 0.1         # untimed load before the warm-up steps, so that short runs see a device at its clocks
 
