@@ -76,8 +76,8 @@ typedef enum {
  *   the units per episode for a chunk that fails, so the results are those of MRX_RESETS_PASSES for any data.
  *   For callers whose episodes end every hundred steps or so (ppo.py:181-190): a chunk with a reset
  *   then costs what a chunk without one costs (measured, B=64 T=1024 H=8 bf16 at one reset per hundred steps:
- *   backward 201 -> 170 us; at one per five hundred the two are level, without resets the merged instance
- *   is 4 % behind).  The forward call merges where it takes the chunk-parallel factor kernel
+ *   backward 197 -> 169 us; at one per five hundred the two are level, without resets the merged instance
+ *   is 5 % behind).  The forward call merges where it takes the chunk-parallel factor kernel
  *   (mrx_factor_path), the backward call always; head dim 64 at full width, 32-row chunks -- elsewhere the
  *   argument is accepted and the units per episode run.  The two calls of a pair need not agree.
  * MRX_RESETS_AUTO: MRX_RESETS_PASSES. */
