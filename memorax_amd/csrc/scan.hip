@@ -876,6 +876,9 @@ ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, boo
     // Geometric mean of time over the best plan's, these rules / the rules below alone: float32 1.00 / 1.07
     // forward and 1.02 / 1.04 backward, MinGRU 1.00 / 1.06 and 1.02 / 1.05, bfloat16 1.01 / 1.40 and
     // 1.00 / 1.21, complex64 1.01 / 1.08 and 1.03 / 1.07; no shape more than 9 % off its best plan but one.
+    // The sweep was repeated after the arrays' loads and stores had become non-temporal: two float32 rules
+    // changed (marked below); against the new timings the rules stand at 1.03 / 1.02 (float32), 1.03 / 1.02
+    // (MinGRU), 1.02 / 1.00 (bfloat16) and 1.02 / 1.01 (complex64).
     if (T >= 4 * TS) {
         auto cols = [&](int v) { return B * ntiles(v); };  // workgroups of the wave-split kernel
         auto split = [&](int v, int n) { return ScanPlan{v, n, (int)ntiles(v), false}; };
@@ -899,8 +902,10 @@ ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, boo
         }
         if (esize == 4) {
             if (!bwd) {
-                const int v = !mg && vec == 4 && cols(4) >= 2048 && T >= 8 * TS ? 4 : (vec < 2 ? vec : 2);
-                return split(v, nw8);
+                // (swept again once every array was loaded and stored non-temporally: two elements per lane
+                // then lead at the large shapes as well -- 512 x 1024 x 1024 forward 1067 -> 1009 us,
+                // 4096 x 128 x 256 291 -> 269 us -- where four used to)
+                return split(vec < 2 ? vec : 2, nw8);
             }
             if (mg) {
                 if (vec == 4 && cols(4) >= 2048 && T >= 8 * TS) return split(4, nw8 > 4 ? 4 : nw8);
@@ -909,7 +914,9 @@ ScanPlan plan_scan(int64_t B, int64_t T, int64_t D, size_t esize, bool al16, boo
                 if (D <= 128 && cols(1) >= 1024) return split(1, nw8);
                 if (T >= 8 * TS) {
                     for (int v = vec; v >= 1; v >>= 1) {
-                        if (cols(v) >= 1024) return split(v, 4);
+                        // rows of a single column tile take eight waves along time, wider rows four (the same
+                        // sweep: 8192 x 128 x 256 backward 1007 -> 920 us, 256 x 128 x 1024 149 -> 132 us)
+                        if (cols(v) >= 1024) return split(v, ntiles(v) == 1 ? 8 : 4);
                         if (cols(v) * 8 >= 4096) return split(v, 8);
                         if (v <= 2 && cols(v) * 16 >= 4096 && T >= 16 * TS) return split(v, 16);
                     }
