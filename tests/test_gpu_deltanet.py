@@ -176,3 +176,74 @@ def test_chunk64_build_agrees_with_the_default_build():
     rc = lib.mrx_delta_rule_fwd(st, p(q), p(k), p(v), p(beta), p(done), p(S0), p(o2), p(Sl2), p(S_chk), p(Tm_chk),
                                 B, T, H, 64, 64, _lib.MRX_BF16, _lib.MRX_DONE_U8, _lib.MRX_FACTORS_PARALLEL, _lib.MRX_RESETS_AUTO)
     assert rc == -2, rc
+
+
+def test_pattern_probe_of_the_measurement_build_moves_the_bytes_it_claims():
+    """mrx_pattern_probe (libmemorax_amd_clk.so, loaded only by bench.py) is what the kernels' times are read
+    against, so it has to touch what it says: every row of every output array is written (here: with the XOR of
+    the inputs' rows, segments rotated by one, XOR the residual block of the chunk), the residual block written
+    back, in both walking directions; bad arguments are refused before anything is launched."""
+    import ctypes
+    import os
+    from memorax_amd import _lib
+    path = os.path.join(os.path.dirname(_lib.LIB_PATH), "libmemorax_amd_clk.so")
+    if not os.path.exists(path):
+        pytest.skip("libmemorax_amd_clk.so not built")
+    lib = ctypes.CDLL(path)
+    vp, i64 = ctypes.c_void_p, ctypes.c_int64
+    f = lib.mrx_pattern_probe
+    f.argtypes = [vp, ctypes.POINTER(vp), ctypes.c_int, ctypes.POINTER(vp), ctypes.c_int, vp, ctypes.c_int, vp, ctypes.c_int,
+                  i64, i64, i64, ctypes.c_int, ctypes.c_int]
+    f.restype = ctypes.c_int
+    st = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator(device="cuda").manual_seed(7)
+    for (n_in, n_out, C, res_in, res_out, reverse) in ((3, 1, 64, 0, 0, 0), (4, 3, 32, 4096, 0, 1), (3, 1, 32, 2048, 8192, 0)):
+        B, T, H = 8, 4 * C, 2
+        NC = T // C
+        print(f"case pattern probe n_in={n_in} n_out={n_out} C={C}", flush=True)
+        ins = [torch.randint(-2**31, 2**31 - 1, (B, T, H, 32), dtype=torch.int32, device="cuda", generator=g) for _ in range(n_in)]
+        outs = [torch.zeros((B, T, H, 32), dtype=torch.int32, device="cuda") for _ in range(n_out)]
+        rin = torch.randint(-2**31, 2**31 - 1, (B * H, NC, max(res_in, 16) // 4), dtype=torch.int32, device="cuda", generator=g)
+        rout = torch.zeros((B * H, NC, max(res_out, 16) // 4), dtype=torch.int32, device="cuda")
+        pi = (vp * n_in)(*[a.data_ptr() for a in ins])
+        po = (vp * n_out)(*[a.data_ptr() for a in outs])
+        rc = f(st, pi, n_in, po, n_out, rin.data_ptr(), res_in, rout.data_ptr(), res_out, B, T, H, C, reverse)
+        assert rc == 0, rc
+        torch.cuda.synchronize()
+        x = ins[0]
+        for a in ins[1:]:
+            x = x ^ a
+        # rows as 8 segments of 4 words: segment s of the output holds segment (s + 1) % 8 of the XOR of the inputs
+        x = x.view(B, T, H, 8, 4).roll(-1, dims=3)
+        # ... XOR, per thread, the words of the residual block that thread took (thread = 8 * row-in-pass + segment)
+        if res_in:
+            segs = res_in // 16
+            r = rin.view(B, H, NC, segs, 4)
+            acc = torch.zeros((B, H, NC, 256, 4), dtype=torch.int32, device="cuda")
+            for s0 in range(0, segs, 256):
+                blk = r[:, :, :, s0:s0 + 256]
+                acc[:, :, :, :blk.shape[3]] ^= blk
+            # thread tid handles rows tid // 8 + 32 p of the chunk, segment tid % 8
+            acc = acc.view(B, H, NC, 32, 8, 4)                      # (row in pass, segment)
+            per_row = acc.repeat(1, 1, 1, C // 32, 1, 1).view(B, H, NC * C, 8, 4).permute(0, 2, 1, 3, 4)
+            x = x ^ per_row
+        for o_ in outs:
+            assert torch.equal(o_.view(B, T, H, 8, 4), x), (n_in, n_out, C)
+        if res_out:
+            want = torch.zeros_like(rout.view(B, H, NC, -1, 4))
+            if res_in:
+                segs_o = res_out // 16
+                acc2 = torch.zeros((B, H, NC, 256, 4), dtype=torch.int32, device="cuda")
+                r = rin.view(B, H, NC, res_in // 16, 4)
+                for s0 in range(0, res_in // 16, 256):
+                    blk = r[:, :, :, s0:s0 + 256]
+                    acc2[:, :, :, :blk.shape[3]] ^= blk
+                for s0 in range(0, segs_o, 256):
+                    n = min(256, segs_o - s0)
+                    want[:, :, :, s0:s0 + n] = acc2[:, :, :, :n]
+            assert torch.equal(rout.view(B, H, NC, -1, 4), want)
+    # refused: chunk length, ragged T, unsupported array counts, residual bytes without a pointer
+    assert f(st, pi, 3, po, 1, None, 0, None, 0, 8, 100, 2, 32, 0) == -1
+    assert f(st, pi, 3, po, 1, None, 0, None, 0, 8, 128, 2, 48, 0) == -1
+    assert f(st, pi, 2, po, 1, None, 0, None, 0, 8, 128, 2, 32, 0) == -2
+    assert f(st, pi, 3, po, 1, None, 64, None, 0, 8, 128, 2, 32, 0) == -1
