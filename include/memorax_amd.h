@@ -332,6 +332,28 @@ int mrx_linear_scan_last(void *stream, const void *a, const void *b,
                          int64_t T, int64_t D, int64_t a_group, int dtype,
                          int done_dtype);
 
+/* ---- mLSTM: the stabiliser of the cell's gates ---------------------------------
+ * mLSTMCell's elements (C, log_f, n, m) combine by the max-stabilised gated sum of mlstm.py:190-206
+ * (m = max(m_a + log_f_b, m_b), both sides rescaled by exp(. - m)) under Memoroid.scan_fn's select-reset
+ * operator (memoroid.py:60-91).  Unrolled over time the stabiliser is
+ *     m_t = done_t ? log_i_t : max(m_{t-1} + log_f_t, log_i_t)
+ * and C and n follow the gated linear recurrence that mrx_gated_linear_attn_* / mrx_linear_scan_* compute,
+ * with log-decay and key weight
+ *     g_t = done_t ? 0 : max(log_f_t + m_{t-1} - m_t, g_floor)   (<= 0) ,   w_t = exp(log_i_t - m_t)   (<= 1).
+ * These two calls produce m, g, w from the gate pre-activations in one pass per (b, h), and take the gradients
+ * back: dm (what the read-out's exp(-m) and the carried m contribute), dg, dw in (any of them nullable),
+ * dlog_i, dlog_f and dm0 (nullable) out.  log_i, log_f, m, g, w and their gradients: (B,T,H) float32;
+ * m0 (nullable: the cell's initial -1e9), dm0: (B,H); g_floor <= 0 (a decay below e^g_floor multiplies a state
+ * next to a new term of weight one: the cell passes -60). */
+int mrx_mlstm_gates_fwd(void *stream, const float *log_i, const float *log_f, const void *done,
+                        const float *m0, float *m, float *g, float *w, int64_t B, int64_t T,
+                        int64_t H, int done_dtype, float g_floor);
+
+int mrx_mlstm_gates_bwd(void *stream, const float *log_i, const float *log_f, const void *done,
+                        const float *m0, const float *m, const float *dm, const float *dg,
+                        const float *dw, float *dlog_i, float *dlog_f, float *dm0, int64_t B,
+                        int64_t T, int64_t H, int done_dtype, float g_floor);
+
 /* ---- MinGRU: the diagonal scan with the cell's gate arithmetic inside ----
  * MinGRUCell (min_gru.py:49-78) maps the step's two projections z and h~ to the elements
  * (log sigma(z) + log g(h~), log sigma(-z)), g(x) = x + 0.5 (x >= 0) | sigma(x), scans them with the

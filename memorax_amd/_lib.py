@@ -52,6 +52,8 @@ SIGNATURES = {
     "mrx_linear_attn_step": (_I, [_P] * 10 + [_L] * 4 + [_I] * 3 + [ctypes.c_float]),
     "mrx_delta_rule_step": (_I, [_P] * 9 + [_L] * 4 + [_I] * 2),
     "mrx_gated_linear_attn_step": (_I, [_P] * 9 + [_L] * 4 + [_I] * 3),
+    "mrx_mlstm_gates_fwd": (_I, [_P] * 8 + [_L] * 3 + [_I, ctypes.c_float]),
+    "mrx_mlstm_gates_bwd": (_I, [_P] * 12 + [_L] * 3 + [_I, ctypes.c_float]),
 }
 
 _lib = None

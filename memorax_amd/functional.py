@@ -426,6 +426,33 @@ def deltanet(q, k, v, beta_raw, done, S0=None, resets=None):
     return hd.out(o), hd.state_out(S_last)
 
 
+class _MlstmGates(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, log_i, log_f, done, m0, g_floor):
+        li, lf = log_i.contiguous().float(), log_f.contiguous().float()
+        m0_ = None if m0 is None else m0.contiguous().float()
+        m, g, w = K.mlstm_gates_fwd(li, lf, done, m0_, g_floor)
+        ctx.done, ctx.g_floor, ctx.has_m0 = done, g_floor, m0 is not None
+        ctx.save_for_backward(li, lf, m, *([m0_] if m0 is not None else []))
+        return m, g, w
+
+    @staticmethod
+    def backward(ctx, dm, dg, dw):
+        li, lf, m, *rest = ctx.saved_tensors
+        m0 = rest[0] if rest else None
+        c = lambda t: None if t is None else t.contiguous().float()  # noqa: E731
+        dli, dlf, dm0 = K.mlstm_gates_bwd(li, lf, ctx.done, m0, m, c(dm), c(dg), c(dw), ctx.g_floor, want_dm0=ctx.has_m0)
+        return dli, dlf, None, dm0, None
+
+
+def mlstm_gates(log_i, log_f, done, m0=None, g_floor=-60.0):
+    """The stabiliser of the mLSTM cell's gates (mlstm.py:190-206 unrolled over time, resets as memoroid.py:72-85):
+    m_t = done_t ? log_i_t : max(m_{t-1} + log_f_t, log_i_t); returns (m, g, w), each (B,T,H), with
+    g_t = log_f_t + m_{t-1} - m_t (0 at a reset, not below g_floor) and w_t = exp(log_i_t - m_t) -- the log-decay
+    and the key weight of the gated linear recurrence that carries the cell's C and n.  m0: (B,H) or None."""
+    return _MlstmGates.apply(log_i, log_f, done, m0, g_floor)
+
+
 def propagate_sensitivities(decay, jacobians, sensitivity, done):
     """Real-time recurrent learning: carry the parameter sensitivities of a diagonal recurrence
     over a (B,T) block of steps -- Memoroid._propagate_sensitivities (memoroid.py:114-141).

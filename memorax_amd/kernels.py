@@ -97,6 +97,39 @@ def linear_scan_fwd(a, b, done, h0=None, P0=None, want_P=True):
     return h, h_last, P_last
 
 
+def mlstm_gates_fwd(log_i, log_f, done, m0=None, g_floor=-60.0):
+    """The mLSTM cell's stabiliser in one pass (mrx_mlstm_gates_fwd): log_i, log_f (B,T,H) float32, m0 (B,H) or
+    None (the cell's initial -1e9).  Returns (m, g, w), each (B,T,H): the running maximum, the log-decay
+    g_t = log_f_t + m_{t-1} - m_t (0 at a reset, not below g_floor) and the key weight exp(log_i_t - m_t)."""
+    lib = _lib.load()
+    B, T, H = log_i.shape
+    _chk(log_i, "log_i", torch.float32)
+    _chk(log_f, "log_f", torch.float32, (B, T, H))
+    _chk(m0, "m0", torch.float32, (B, H))
+    done, dd = _done(done, B, T)
+    m, g, w = (torch.empty_like(log_i) for _ in range(3))
+    st = lib.mrx_mlstm_gates_fwd(_stream(), _ptr(log_i), _ptr(log_f), _ptr(done), _ptr(m0), _ptr(m), _ptr(g), _ptr(w),
+                                 B, T, H, dd, float(g_floor))
+    _lib.check(st, "mrx_mlstm_gates_fwd")
+    return m, g, w
+
+
+def mlstm_gates_bwd(log_i, log_f, done, m0, m, dm, dg, dw, g_floor=-60.0, want_dm0=True):
+    """Gradients of mlstm_gates_fwd: dm, dg, dw (each (B,T,H) or None) in, (dlog_i, dlog_f, dm0) out."""
+    lib = _lib.load()
+    B, T, H = log_i.shape
+    for t, n in ((log_i, "log_i"), (log_f, "log_f"), (m, "m"), (dm, "dm"), (dg, "dg"), (dw, "dw")):
+        _chk(t, n, torch.float32, (B, T, H))
+    _chk(m0, "m0", torch.float32, (B, H))
+    done, dd = _done(done, B, T)
+    dli, dlf = torch.empty_like(log_i), torch.empty_like(log_f)
+    dm0 = torch.empty((B, H), dtype=torch.float32, device=log_i.device) if want_dm0 else None
+    st = lib.mrx_mlstm_gates_bwd(_stream(), _ptr(log_i), _ptr(log_f), _ptr(done), _ptr(m0), _ptr(m), _ptr(dm), _ptr(dg),
+                                 _ptr(dw), _ptr(dli), _ptr(dlf), _ptr(dm0), B, T, H, dd, float(g_floor))
+    _lib.check(st, "mrx_mlstm_gates_bwd")
+    return dli, dlf, dm0
+
+
 def linear_scan_last(a, b, done, h0=None):
     """Final state of h_t = done ? b_t : a_t h_{t-1} + b_t with one decay per group of channels:
     a: (B,T,D/group), b: (B,T,D), h0: (B,D) or None.  Returns h_last (B,D)."""

@@ -29,7 +29,7 @@ import torch.nn.functional as F
 
 from typing import NamedTuple
 
-from .functional import (deltanet, gated_linear_attention, linear_attention, linear_scan, mingru_scan,
+from .functional import (deltanet, gated_linear_attention, linear_attention, linear_scan, mingru_scan, mlstm_gates,
                          normalised_linear_attention)
 
 
@@ -600,9 +600,9 @@ class mLSTMCell(MemoroidCellBase):
         m_t = max(m_{t-1} + log f_t, log i_t)
         C_t = exp(log f_t + m_{t-1} - m_t) C_{t-1} + exp(log i_t - m_t) k_t v_t^T      (n_t alike),
     a gated linear recurrence whose log-decay g_t = log f_t + m_{t-1} - m_t and key weight
-    exp(log i_t - m_t) are both <= 1 whatever the gates do: m_t is a cumulative maximum in log space
-    (taken per episode), g and the weights follow from it elementwise, q C runs in the gated chunked
-    kernel and n in the diagonal scan.  State, normaliser and m come out in the reference's stabilised
+    exp(log i_t - m_t) are both <= 1 whatever the gates do: m, g and the weights come from one pass per
+    (b, h) in the library (functional.mlstm_gates), q C runs in the gated chunked kernel and n in the
+    diagonal scan.  State, normaliser and m come out in the reference's stabilised
     units, step by step, so gates may drift by any amount inside an episode.
     Carry: (C (B,1,H,d,d), log_f (B,1,H,1,1), n (B,1,H,d,1), m (B,1,H,1,1)) as in the reference."""
 
@@ -663,21 +663,11 @@ class mLSTMCell(MemoroidCellBase):
         C0, lf0, n0, m0 = initial_carry
         Bn, T, H, d = k.shape
         ones = torch.ones(H, device=k.device)
-        dn = (done != 0)
         m0_ = m0[:, 0, :, 0, 0].float()                                          # (B,H)
-        # m_t = max(m_{t-1} + log f_t, log i_t), restarted at resets: with F the cumulative log f of the
-        # episode, m_t = F_t + max(m_0 [first episode], running max of (log i - F))
-        Fc, _, _ = linear_scan(ones, log_f.contiguous(), done, torch.zeros(Bn, H, device=k.device))
-        seg = torch.cumsum(dn.to(torch.float64), dim=1)[..., None]                # (B,T,1)
-        u = (log_i - Fc).double()
-        big = 2.0 * (u.max() - u.min()).detach() + 1.0
-        cm = torch.cummax(u + big * seg, dim=1).values - big * seg
-        cm = torch.where(seg == 0, torch.maximum(cm, m0_[:, None].double()), cm)
-        m = (Fc.double() + cm).float()                                            # (B,T,H)
-        m_prev = torch.cat([m0_[:, None], m[:, :-1]], dim=1)
-        g = log_f + m_prev - m                                                    # <= 0
-        g = torch.where(dn[..., None], torch.zeros_like(g), g).clamp(min=self._G_FLOOR)   # a reset zeroes the state anyway
-        k_in = k.float() * torch.exp(log_i - m)[..., None]                        # weights <= 1
+        # m_t = max(m_{t-1} + log f_t, log i_t), restarted at resets; g_t = log f_t + m_{t-1} - m_t (0 at a reset:
+        # it zeroes the state anyway) and the key weights exp(log i_t - m_t) <= 1: one pass per (b, h) in the library
+        m, g, wk = mlstm_gates(log_i, log_f, done, m0_, self._G_FLOOR)            # each (B,T,H)
+        k_in = k.float() * wk[..., None]
         S0 = C0[:, 0].float().transpose(-1, -2).contiguous()
         num, S_last = gated_linear_attention(q.float().contiguous(), k_in.contiguous(), v.float().contiguous(),
                                              g.contiguous(), done, S0)

@@ -74,6 +74,31 @@ def mingru_scan_t(z, h_tilde, done, h0=None, side=None):
     return torch.exp(torch.stack(out, 1)), torch.exp(ls)
 
 
+def mlstm_gates_t(log_i, log_f, done, m0=None, g_floor=-60.0):
+    """torch restatement of oracle.memoroid.mlstm_gates (differentiable)."""
+    B, T, H = log_i.shape
+    mp = torch.full((B, H), -1e9, dtype=log_i.dtype) if m0 is None else m0
+    ms, gs, ws = [], [], []
+    for t in range(T):
+        r = done[:, t][:, None]
+        mt = torch.where(r, log_i[:, t], torch.maximum(mp + log_f[:, t], log_i[:, t]))
+        gs.append(torch.where(r, torch.zeros_like(mt), torch.clamp(log_f[:, t] + mp - mt, min=g_floor)))
+        ws.append(torch.exp(log_i[:, t] - mt))
+        ms.append(mt)
+        mp = mt
+    return torch.stack(ms, 1), torch.stack(gs, 1), torch.stack(ws, 1)
+
+
+def mlstm_gates_grads(log_i, log_f, done, m0, dm, dg, dw, g_floor=-60.0):
+    """(dlog_i, dlog_f, dm0) of L = sum(dm * m) + sum(dg * g) + sum(dw * w)."""
+    li, lf = _t(log_i, True), _t(log_f, True)
+    m0_ = None if m0 is None else _t(m0, True)
+    m, g, w = mlstm_gates_t(li, lf, _done(done), m0_, g_floor)
+    L = (m * _t(dm)).sum() + (g * _t(dg)).sum() + (w * _t(dw)).sum()
+    L.backward()
+    return _np(li.grad), _np(lf.grad), (None if m0 is None else _np(m0_.grad))
+
+
 def elu1_t(x):
     return torch.where(x > 0, x + 1.0, torch.exp(torch.clamp(x, max=0.0)))
 

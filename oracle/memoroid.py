@@ -482,6 +482,26 @@ def mlstm(q, k, v, i_gate, f_gate, done, carry=None, tree=True):
     return nxt, mlstm_read(h, q)
 
 
+def mlstm_gates(log_i, log_f, done, m0=None, g_floor=-60.0):
+    """The stabiliser of mlstm.py:190-206 unrolled over time, resets as memoroid.py:72-85 (the element wins by
+    select): m_t = done_t ? log_i_t : max(m_{t-1} + log_f_t, log_i_t), and with it the log-decay and the key
+    weight of the gated recurrence the stabilised C and n follow: g_t = done_t ? 0 : max(log_f_t + m_{t-1} - m_t,
+    g_floor), w_t = exp(log_i_t - m_t).  log_i, log_f: (B,T,H); m0: (B,H) or None (the cell's initial -1e9).
+    Returns (m, g, w)."""
+    log_i, log_f = np.asarray(log_i, np.float64), np.asarray(log_f, np.float64)
+    B, T, H = log_i.shape
+    done = np.asarray(done) != 0
+    mp = np.full((B, H), -1e9) if m0 is None else np.asarray(m0, np.float64)
+    m, g, w = np.empty((B, T, H)), np.empty((B, T, H)), np.empty((B, T, H))
+    for t in range(T):
+        r = done[:, t][:, None]
+        mt = np.where(r, log_i[:, t], np.maximum(mp + log_f[:, t], log_i[:, t]))
+        g[:, t] = np.where(r, 0.0, np.maximum(log_f[:, t] + mp - mt, g_floor))
+        w[:, t] = np.exp(log_i[:, t] - mt)
+        m[:, t] = mp = mt
+    return m, g, w
+
+
 def mlstm_unstabilised(q, k, v, i_gate, f_gate, done):
     """The recurrence the docstring of mlstm.py:8-11 states, without the stabiliser:
     C~_t = f_t C~_{t-1} + i_t k_t v_t^T, n~_t = f_t n~_{t-1} + i_t k_t (zero carry),

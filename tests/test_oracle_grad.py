@@ -358,3 +358,25 @@ def test_linear_attention_cell_of_the_gradient_oracle():
     c1, y1 = G.linear_attention_cell_t(t(x[:, :s]), t(done[:, :s]), t(Wq), t(Wk), t(Wv), t(ns), t(Wout), t(bout), H)
     c2, y2 = G.linear_attention_cell_t(t(x[:, s:]), t(done[:, s:]), t(Wq), t(Wk), t(Wv), t(ns), t(Wout), t(bout), H, c1)
     assert np.allclose(np.concatenate([y1.numpy(), y2.numpy()], 1), y.numpy(), atol=1e-11)
+
+
+def test_mlstm_gates_grads_fd():
+    """torch autograd through the gates' restatement against central differences on the NumPy forward:
+    a carried m, resets (first step, mid-sequence), one step whose g sits on the floor."""
+    B, T, H = 2, 7, 2
+    li, lf = rnd(B, T, H) * 2, -np.abs(rnd(B, T, H))
+    m0 = rnd(B, H)
+    lf[0, 3] = -100.0                 # g_3 is clamped for batch row 0: no gradient through it
+    d = np.zeros((B, T), bool)
+    d[0, 5] = True
+    d[1, 0] = True
+    dm, dg, dw = rnd(B, T, H), rnd(B, T, H), rnd(B, T, H)
+
+    def L():
+        m, g, w = M.mlstm_gates(li, lf, d, m0)
+        return (m * dm).sum() + (g * dg).sum() + (w * dw).sum()
+    gi, gf, g0 = G.mlstm_gates_grads(li, lf, d, m0, dm, dg, dw)
+    np.testing.assert_allclose(gi, fd(L, li), rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(gf, fd(L, lf), rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(g0, fd(L, m0), rtol=1e-6, atol=1e-7)
+    assert g0[1].tolist() == [0.0, 0.0]   # batch row 1 resets at its first step: the carried m is dropped

@@ -411,3 +411,43 @@ def test_mlstm_stabilised_scan_equals_plain_recurrence():
     nxt, ha = M.mlstm(q[:, :5], k[:, :5], v[:, :5], ig[:, :5], fg[:, :5], done[:, :5])
     _, hb = M.mlstm(q[:, 5:], k[:, 5:], v[:, 5:], ig[:, 5:], fg[:, 5:], done[:, 5:], nxt)
     np.testing.assert_allclose(np.concatenate([ha, hb], 1), h, rtol=1e-9, atol=1e-12)
+
+
+def test_mlstm_gates_are_the_stabilised_scan_unrolled():
+    """oracle.memoroid.mlstm_gates against the cell's own route: m is the m leaf of the stabilised scan
+    (mlstm_operator under the select-reset scan), and a plain gated recurrence driven by its g and w
+    reproduces the scan's C and n leaves step by step -- with a carried state, resets at the first step and
+    in runs, and through a split."""
+    q, k, v, ig, fg, done = _mlstm_inputs(seed=9, p=0.2)
+    done[0, 0] = True
+    done[1, 3:5] = True
+    B, T, H, d = q.shape
+    rng = np.random.default_rng(10)
+    carry = (rng.standard_normal((B, 1, H, d, d)), -np.abs(rng.standard_normal((B, 1, H, 1, 1))),
+             rng.standard_normal((B, 1, H, d, 1)), rng.standard_normal((B, 1, H, 1, 1)))
+    z = M.mlstm_elements(q, k, v, ig, fg)
+    h, nxt = M.scan_fn_sequential(z, carry, done, M.mlstm_operator)
+    log_f = -M.softplus(-fg)
+    m, g, w = M.mlstm_gates(ig, log_f, done, carry[3][:, 0, :, 0, 0], g_floor=-1e30)
+    np.testing.assert_allclose(m, h[3][..., 0, 0], rtol=1e-12, atol=1e-12)
+    assert (g <= 1e-12).all() and (w <= 1 + 1e-12).all()
+    C, n = carry[0][:, 0].copy(), carry[2][:, 0, ..., 0].copy()
+    ks = k / np.sqrt(d)
+    for t in range(T):
+        r = (done[:, t] != 0)[:, None]
+        dec = np.where(r, 0.0, np.exp(g[:, t]))          # a reset drops the state; its g is 0 by convention
+        C = dec[..., None, None] * C + w[:, t][..., None, None] * np.einsum("bhi,bhj->bhij", ks[:, t], v[:, t])
+        n = dec[..., None] * n + w[:, t][..., None] * ks[:, t]
+        np.testing.assert_allclose(C, h[0][:, t], rtol=1e-9, atol=1e-12)
+        np.testing.assert_allclose(n, h[2][:, t, ..., 0], rtol=1e-9, atol=1e-12)
+    # the floor only ever raises a decay that multiplies a state e^60 times smaller than the new term
+    _, g60, _ = M.mlstm_gates(ig, log_f, done, carry[3][:, 0, :, 0, 0])
+    assert (g60 >= -60).all() and np.array_equal(g60[g > -60], g[g > -60])
+    # split through the carried m
+    ma, ga, wa = M.mlstm_gates(ig[:, :5], log_f[:, :5], done[:, :5], carry[3][:, 0, :, 0, 0])
+    mb, gb, wb = M.mlstm_gates(ig[:, 5:], log_f[:, 5:], done[:, 5:], ma[:, -1])
+    for whole, a_, b_ in ((m, ma, mb), (g60, ga, gb), (w, wa, wb)):
+        np.testing.assert_array_equal(np.concatenate([a_, b_], 1), whole)
+    # no carried state = the cell's initial -1e9
+    m_n, _, _ = M.mlstm_gates(ig, log_f, done)
+    np.testing.assert_allclose(m_n, M.mlstm_gates(ig, log_f, done, np.full((B, H), -1e9))[0])
