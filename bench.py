@@ -127,6 +127,7 @@ def main() -> int:
             secondary["torso"].update(bench_torso_full(torch, K))
             secondary["step"] = bench_step(torch, K)
             secondary["rtrl"] = bench_rtrl(torch, K)
+            secondary["mlstm"] = bench_mlstm(torch)
         if not args.no_children:
             secondary["delta_rule_chunk64"] = bench_delta_chunk64()
         torch.cuda.empty_cache()
@@ -599,6 +600,31 @@ def bench_linear_attention(torch, K, np, dev):
     res["normalised_bf16_256x4096x8x64"] = {"ms": ms, "tokens/s": Bn * Tn / ms * 1e3,
                                             "GB/s": (1408 + 136) * Bn * Tn * Hn / ms / 1e6}
     return res
+
+
+def bench_mlstm(torch):
+    """The mLSTM cell's scan through the host mirror (stabiliser kernels, gated chunked kernel, normaliser scan and
+    the read-out's divisions; float32), forward and forward + backward, at a rollout-sized and a larger shape."""
+    from memorax_amd import sequence_models as sm
+    out = {}
+    for (B, T, H, d) in ((64, 128, 4, 64), (256, 512, 4, 64)):
+        cell = sm.mLSTMCell(64, hidden_dim=H * d, num_heads=H).cuda()
+        g = torch.Generator(device="cuda").manual_seed(B)
+        q, k, v = (torch.randn(B, T, H, d, device="cuda", generator=g).requires_grad_() for _ in range(3))
+        li = torch.randn(B, T, H, device="cuda", generator=g).requires_grad_()
+        lf = (-torch.rand(B, T, H, device="cuda", generator=g)).requires_grad_()
+        done = torch.rand(B, T, device="cuda", generator=g) < 0.01
+        carry = cell.initialize_carry(None, (B, 64))
+
+        def fwd():
+            with torch.no_grad():
+                cell.scan((k, v, li, lf, q), carry, done)
+
+        def step():
+            h, c = cell.scan((k, v, li, lf, q), carry, done)
+            (h.sum() + c[0].sum() + c[2].sum()).backward()
+        out[f"scan_{B}x{T}x{H}x{d}"] = {"fwd_ms": _time_ms(torch, fwd, iters=10), "fwd+bwd_ms": _time_ms(torch, step, iters=10)}
+    return out
 
 
 def bench_rtrl(torch, K):
