@@ -29,6 +29,7 @@ import torch.nn.functional as F
 
 from typing import NamedTuple
 
+from .dense import Dense, autocast_dtype, compute_input
 from .functional import (deltanet, gated_linear_attention, linear_attention, linear_scan, mingru_scan, mlstm_gates,
                          normalised_linear_attention)
 
@@ -304,11 +305,12 @@ class MinGRUCell(_DiagonalCell):
         super().__init__()
         self.features, self.fused = features, fused
         in_features = features if in_features is None else in_features
-        self.z = nn.Linear(in_features, features, bias=False)
-        self.h = nn.Linear(in_features, features, bias=False)
+        self.z = Dense(in_features, features, bias=False)
+        self.h = Dense(in_features, features, bias=False)
         self.intermediates = {}
 
     def forward(self, x, **kwargs):
+        x = compute_input(x)
         z, h_tilde = self.z(x), self.h(x)
         self.intermediates["gate"] = z.mean().detach()   # min_gru.py:63 sows the mean gate
         if self.fused:   # the recurrence runs in fp32 whatever the projections' dtype (autocast): the kernels
@@ -351,12 +353,13 @@ class GatedLinearRecurrence(SequenceModel):
         super().__init__()
         hidden = features if hidden is None else hidden
         self.cell = MinGRUCell(hidden, in_features=features)
-        self.gate = nn.Linear(features, hidden, bias=False)
-        self.out = nn.Linear(hidden, features, bias=False)
+        self.gate = Dense(features, hidden, bias=False)
+        self.out = Dense(hidden, features, bias=False)
 
     def forward(self, inputs, done, initial_carry=None, **kwargs):
         if initial_carry is None:
             initial_carry = self.cell.initialize_carry(None, get_input_shape(inputs))
+        inputs = compute_input(inputs)
         h, next_carry = self.cell.scan(self.cell(inputs), initial_carry, done)
         return next_carry, self.out(h[0] * F.silu(self.gate(inputs)))
 
@@ -391,11 +394,11 @@ class LinearAttentionCell(MemoroidCellBase):
         in_features = features if in_features is None else in_features
         self.features, self.head_dim, self.num_heads, self.eps = features, head_dim, num_heads, eps
         hidden = head_dim * num_heads
-        self.key = nn.Linear(in_features, hidden, bias=False)
-        self.value = nn.Linear(in_features, hidden, bias=False)
-        self.query = nn.Linear(in_features, hidden, bias=False)
+        self.key = Dense(in_features, hidden, bias=False)
+        self.value = Dense(in_features, hidden, bias=False)
+        self.query = Dense(in_features, hidden, bias=False)
         self.norm = _RMSNorm(hidden)
-        self.output_projection = nn.Linear(hidden, features)
+        self.output_projection = Dense(hidden, features)
 
     def _heads(self, x):
         return x.view(*x.shape[:2], self.num_heads, self.head_dim)
@@ -404,6 +407,7 @@ class LinearAttentionCell(MemoroidCellBase):
         """Elements in kernel form: (v, k, q), keys and queries before the feature map (phi is applied
         inside the kernel).  The reference's elements are (v phi(k)^T, phi(k)); the query joins them here
         because the kernel contracts the state with it as it goes."""
+        x = compute_input(x)
         return (self._heads(self.value(x)), self._heads(self.key(x)), self._heads(self.query(x)))
 
     def binary_operator(self, a, b):
@@ -454,12 +458,12 @@ class DeltaNetCell(MemoroidCellBase):
         self.features, self.head_dim, self.num_heads, self.dtype = features, head_dim, num_heads, dtype
         self.resets = resets   # None / "passes" / "merged": mrx_reset_path, for rollouts whose episodes end often
         hidden = head_dim * num_heads
-        self.query = nn.Linear(in_features, hidden, bias=False)
-        self.key = nn.Linear(in_features, hidden, bias=False)
-        self.value = nn.Linear(in_features, hidden, bias=False)
-        self.beta = nn.Linear(in_features, num_heads, bias=False)
+        self.query = Dense(in_features, hidden, bias=False)
+        self.key = Dense(in_features, hidden, bias=False)
+        self.value = Dense(in_features, hidden, bias=False)
+        self.beta = Dense(in_features, num_heads, bias=False)
         self.norm = _RMSNorm(hidden)
-        self.output_projection = nn.Linear(hidden, features)
+        self.output_projection = Dense(hidden, features)
 
     def _heads(self, x):
         return x.view(*x.shape[:2], self.num_heads, self.head_dim)
@@ -468,6 +472,7 @@ class DeltaNetCell(MemoroidCellBase):
         """The raw projections (q, k, v, beta logits): the key normalisation and the sigmoid run
         inside the kernels."""
         dt = self.dtype
+        x = compute_input(x)
         return (self._heads(self.query(x)).to(dt), self._heads(self.key(x)).to(dt),
                 self._heads(self.value(x)).to(dt), self.beta(x).to(dt))
 
@@ -512,13 +517,13 @@ class MambaCell(MemoroidCellBase):
         self.D = nn.Parameter(torch.ones(num_heads))
         dt = torch.exp(torch.rand(num_heads) * (math.log(0.1) - math.log(0.001)) + math.log(0.001))
         self.dt_bias = nn.Parameter(dt + torch.log(-torch.expm1(-dt)))
-        self.input_projection = nn.Linear(in_features, hidden * 2, bias=False)
-        self.B = nn.Linear(in_features, sp, bias=False)
-        self.C = nn.Linear(in_features, sp, bias=False)
-        self.dt = nn.Linear(in_features, num_heads, bias=False)
+        self.input_projection = Dense(in_features, hidden * 2, bias=False)
+        self.B = Dense(in_features, sp, bias=False)
+        self.C = Dense(in_features, sp, bias=False)
+        self.dt = Dense(in_features, num_heads, bias=False)
         self.conv = nn.Conv1d(conv_channels, conv_channels, conv_dim, groups=conv_channels)
         self.norm = _RMSNorm(hidden)
-        self.output_projection = nn.Linear(hidden, features)
+        self.output_projection = Dense(hidden, features)
 
     def _project(self, x):
         Bn, T, _ = x.shape
@@ -613,13 +618,13 @@ class mLSTMCell(MemoroidCellBase):
         in_features = features if in_features is None else in_features
         self.features, self.hidden_dim, self.num_heads = features, hidden_dim, num_heads
         self.conv_kernel_size = conv_kernel_size
-        self.up_projection = nn.Linear(in_features, 2 * hidden_dim, bias=False)
+        self.up_projection = Dense(in_features, 2 * hidden_dim, bias=False)
         self.causal_conv = nn.Conv1d(hidden_dim, hidden_dim, conv_kernel_size, groups=hidden_dim)
         self.query = _BlockDiagonalDense(hidden_dim, num_heads)
         self.key = _BlockDiagonalDense(hidden_dim, num_heads)
         self.value = _BlockDiagonalDense(hidden_dim, num_heads)
-        self.i_gate = nn.Linear(3 * hidden_dim, num_heads)
-        self.f_gate = nn.Linear(3 * hidden_dim, num_heads)
+        self.i_gate = Dense(3 * hidden_dim, num_heads)
+        self.f_gate = Dense(3 * hidden_dim, num_heads)
         with torch.no_grad():
             self.i_gate.weight.zero_()
             self.i_gate.bias.normal_(std=0.1)
@@ -627,7 +632,7 @@ class mLSTMCell(MemoroidCellBase):
             self.f_gate.bias.copy_(torch.linspace(3.0, 6.0, num_heads))
         self.learnable_skip = nn.Parameter(torch.ones(hidden_dim))
         self.norm_weight = nn.Parameter(torch.zeros(num_heads, hidden_dim // num_heads))
-        self.output_projection = nn.Linear(hidden_dim, features, bias=False)
+        self.output_projection = Dense(hidden_dim, features, bias=False)
 
     def _project(self, x):
         Bn, T, _ = x.shape
@@ -770,7 +775,7 @@ class GatedResidual(nn.Module):
 
     def __init__(self, module, dim, gate=torch.sigmoid):
         super().__init__()
-        self.module, self.gate, self.gate_fn = module, nn.Linear(dim, dim), gate
+        self.module, self.gate, self.gate_fn = module, Dense(dim, dim), gate
 
     def forward(self, inputs, done=None, initial_carry=None, **kwargs):
         carry, y = self.module(inputs, done, initial_carry, **kwargs)
@@ -792,8 +797,8 @@ class FFN(_Stateless):
 
     def __init__(self, features, expansion_factor=4, activation=F.gelu, dropout_rate=0.0):
         super().__init__()
-        self.up = nn.Linear(features, features * expansion_factor)
-        self.down = nn.Linear(features * expansion_factor, features)
+        self.up = Dense(features, features * expansion_factor)
+        self.down = Dense(features * expansion_factor, features)
         self.activation, self.dropout = activation, nn.Dropout(dropout_rate)
 
     def forward(self, inputs, done=None, initial_carry=None, **kwargs):
@@ -805,7 +810,7 @@ class Projection(_Stateless):
 
     def __init__(self, in_features, features, use_bias=True):
         super().__init__()
-        self.proj = nn.Linear(in_features, features, bias=use_bias)
+        self.proj = Dense(in_features, features, bias=use_bias)
 
     def forward(self, inputs, done=None, initial_carry=None, **kwargs):
         return None, self.proj(inputs)
@@ -818,8 +823,8 @@ class GLU(_Stateless):
     def __init__(self, features, expansion_factor=4, activation=F.gelu, dropout_rate=0.0, use_bias=False):
         super().__init__()
         hidden = features * expansion_factor
-        self.up_proj = nn.Linear(features, 2 * hidden, bias=use_bias)
-        self.down_proj = nn.Linear(hidden, features, bias=use_bias)
+        self.up_proj = Dense(features, 2 * hidden, bias=use_bias)
+        self.down_proj = Dense(hidden, features, bias=use_bias)
         self.activation, self.dropout = activation, nn.Dropout(dropout_rate)
 
     def forward(self, inputs, done=None, initial_carry=None, **kwargs):
