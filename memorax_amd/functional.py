@@ -6,6 +6,7 @@ the role jax.custom_vjp would in a JAX host).
     linear_attention(q, k, v, done, S0=None, feature_map) -> (o, S_last)
     delta_rule(q, k, v, beta, done, S0=None)             -> (o, S_last)
     deltanet(q, k, v, beta_raw, done, S0=None)           -> (o, S_last)   (key L2-norm and sigmoid fused)
+    rms_norm(x, scale, eps, out_dtype)                   -> y
 
 Layouts follow the reference: (B,T,D) / (B,T,H,d), state (B,H,d_v,d_k), done (B,T)
 bool or float where nonzero clears the carry before step t (memoroid.py:60-91).
@@ -451,6 +452,36 @@ def mlstm_gates(log_i, log_f, done, m0=None, g_floor=-60.0):
     g_t = log_f_t + m_{t-1} - m_t (0 at a reset, not below g_floor) and w_t = exp(log_i_t - m_t) -- the log-decay
     and the key weight of the gated linear recurrence that carries the cell's C and n.  m0: (B,H) or None."""
     return _MlstmGates.apply(log_i, log_f, done, m0, g_floor)
+
+
+class _RmsNorm(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, scale, eps, out_dtype):
+        xc = x.contiguous()
+        if xc.dtype not in (torch.float32, torch.bfloat16):
+            xc = xc.float()
+        sc = None if scale is None else scale.contiguous().float()
+        ctx.save_for_backward(xc, *([sc] if sc is not None else []))
+        ctx.eps, ctx.x_dtype = eps, x.dtype
+        return K.rms_norm_fwd(xc, sc, eps, out_dtype)
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, dy):
+        xc, *rest = ctx.saved_tensors
+        sc = rest[0] if rest else None
+        dy = dy.contiguous()
+        if dy.dtype not in (torch.float32, torch.bfloat16):
+            dy = dy.float()
+        dx, dscale = K.rms_norm_bwd(xc, sc, dy, ctx.eps, want_dscale=sc is not None and ctx.needs_input_grad[1])
+        return dx.to(ctx.x_dtype), dscale, None, None
+
+
+def rms_norm(x, scale=None, eps=1e-6, out_dtype=None):
+    """flax.linen.RMSNorm with its defaults over the last axis (linear_attention.py:109-115; the norm of the
+    torso's PreNorm blocks): x * rsqrt(mean(x^2) + eps) * scale, one kernel each way.  x (..., D) float32 or
+    bfloat16 with D a multiple of 4 up to 2048, scale (D) or None; the result in out_dtype (default x's)."""
+    return _RmsNorm.apply(x, scale, eps, out_dtype)
 
 
 def propagate_sensitivities(decay, jacobians, sensitivity, done):

@@ -130,6 +130,52 @@ def mlstm_gates_bwd(log_i, log_f, done, m0, m, dm, dg, dw, g_floor=-60.0, want_d
     return dli, dlf, dm0
 
 
+RMS_NORM_PARTS = 1024   # MRX_RMS_NORM_PARTS: rows of the backward's workspace
+RMS_NORM_MAX_D = 2048
+
+
+def rms_norm_fwd(x, scale, eps=1e-6, out_dtype=None):
+    """y = x * rsqrt(mean(x^2) + eps) * scale over the last axis (mrx_rms_norm_fwd): x (..., D) float32 or
+    bfloat16, scale (D) float32 or None (ones); y in out_dtype (default: x's)."""
+    lib = _lib.load()
+    D = x.shape[-1]
+    out_dtype = x.dtype if out_dtype is None else out_dtype
+    if x.dtype not in (torch.float32, torch.bfloat16) or out_dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("rms_norm takes float32 or bfloat16 arrays")
+    _chk(x, "x")
+    _chk(scale, "scale", torch.float32, (D,))
+    y = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    if x.numel() == 0:
+        return y
+    st = lib.mrx_rms_norm_fwd(_stream(), _ptr(x), _ptr(scale), _ptr(y), x.numel() // D, D, _DT[x.dtype], _DT[out_dtype],
+                              float(eps))
+    _lib.check(st, "mrx_rms_norm_fwd")
+    return y
+
+
+def rms_norm_bwd(x, scale, dy, eps=1e-6, want_dscale=True):
+    """Gradients of rms_norm_fwd: dy (..., D) float32 or bfloat16 in; (dx in x's dtype, dscale (D) float32 or
+    None) out.  The statistics are recomputed from x."""
+    lib = _lib.load()
+    D = x.shape[-1]
+    if x.dtype not in (torch.float32, torch.bfloat16) or dy.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("rms_norm takes float32 or bfloat16 arrays")
+    _chk(x, "x")
+    _chk(dy, "dy", None, x.shape)
+    _chk(scale, "scale", torch.float32, (D,))
+    dx = torch.empty_like(x)
+    dscale = work = None
+    if want_dscale:
+        dscale = torch.zeros((D,), dtype=torch.float32, device=x.device)
+        work = torch.empty((RMS_NORM_PARTS, D), dtype=torch.float32, device=x.device)
+    if x.numel() == 0:
+        return dx, dscale
+    st = lib.mrx_rms_norm_bwd(_stream(), _ptr(x), _ptr(scale), _ptr(dy), _ptr(dx), _ptr(dscale), _ptr(work), x.numel() // D, D,
+                              _DT[x.dtype], _DT[dy.dtype], float(eps))
+    _lib.check(st, "mrx_rms_norm_bwd")
+    return dx, dscale
+
+
 def linear_scan_last(a, b, done, h0=None):
     """Final state of h_t = done ? b_t : a_t h_{t-1} + b_t with one decay per group of channels:
     a: (B,T,D/group), b: (B,T,D), h0: (B,D) or None.  Returns h_last (B,D)."""

@@ -31,7 +31,8 @@ from typing import NamedTuple
 
 from .dense import Dense, autocast_dtype, compute_input
 from .functional import (deltanet, gated_linear_attention, linear_attention, linear_scan, mingru_scan, mlstm_gates,
-                         normalised_linear_attention)
+                         normalised_linear_attention, rms_norm)
+from .kernels import RMS_NORM_MAX_D as _RMS_NORM_MAX_D
 
 
 # ----------------------------------------------------------------------------------
@@ -379,8 +380,14 @@ class _RMSNorm(nn.Module):
         self.eps = eps
 
     def forward(self, x):
-        # one fused kernel each way instead of half a dozen elementwise ones; statistics in fp32
-        return F.rms_norm(x.float(), (x.shape[-1],), self.scale.float(), self.eps).to(x.dtype)
+        """Statistics in float32.  On the device: the library's kernel, one pass each way, with the result in
+        the dtype its readers compute in (under autocast the dense layers behind a norm would each cast it
+        again); rows it does not take (wider than 2048 features, a width that is no multiple of 4) and host
+        arrays go to the array library."""
+        D = x.shape[-1]
+        if x.is_cuda and D % 4 == 0 and D <= _RMS_NORM_MAX_D:
+            return rms_norm(x, self.scale, self.eps, autocast_dtype(x) or x.dtype)
+        return F.rms_norm(x.float(), (D,), self.scale.float(), self.eps).to(x.dtype)
 
 
 class LinearAttentionCell(MemoroidCellBase):

@@ -99,6 +99,17 @@ def mlstm_gates_grads(log_i, log_f, done, m0, dm, dg, dw, g_floor=-60.0):
     return _np(li.grad), _np(lf.grad), (None if m0 is None else _np(m0_.grad))
 
 
+def rms_norm_grads(x, scale, dy, eps=1e-6):
+    """(dx, dscale) of L = sum(dy * rms_norm(x, scale)); scale None: (dx, None)."""
+    x_ = _t(x, True)
+    s_ = None if scale is None else _t(scale, True)
+    y = x_ * torch.rsqrt((x_ * x_).mean(-1, keepdim=True) + eps)
+    if s_ is not None:
+        y = y * s_
+    (y * _t(dy)).sum().backward()
+    return _np(x_.grad), (None if s_ is None else _np(s_.grad))
+
+
 def elu1_t(x):
     return torch.where(x > 0, x + 1.0, torch.exp(torch.clamp(x, max=0.0)))
 

@@ -482,6 +482,15 @@ def mlstm(q, k, v, i_gate, f_gate, done, carry=None, tree=True):
     return nxt, mlstm_read(h, q)
 
 
+def rms_norm(x, scale=None, eps=1e-6):
+    """flax.linen.RMSNorm with its defaults over the last axis (the norm of LinearAttentionCell.read,
+    linear_attention.py:109-115, and of PreNorm blocks built with it, blocks/normalization.py:10-35):
+    x * rsqrt(mean(x^2) + eps) * scale."""
+    x = np.asarray(x, np.float64)
+    y = x / np.sqrt((x * x).mean(-1, keepdims=True) + eps)
+    return y if scale is None else y * np.asarray(scale, np.float64)
+
+
 def mlstm_gates(log_i, log_f, done, m0=None, g_floor=-60.0):
     """The stabiliser of mlstm.py:190-206 unrolled over time, resets as memoroid.py:72-85 (the element wins by
     select): m_t = done_t ? log_i_t : max(m_{t-1} + log_f_t, log_i_t), and with it the log-decay and the key

@@ -1,0 +1,147 @@
+"""The RMS norm kernels (mrx_rms_norm_fwd / _bwd, through the C ABI) against the oracle: y of
+oracle.memoroid.rms_norm and the gradients of oracle.grad.rms_norm_grads (torch-fp64 autograd, pinned by
+closed forms and finite differences in tests/test_oracle_grad.py).  Tolerances: float32 arrays 1e-5 of the
+result's scale; bfloat16 arrays 2e-2 (one rounding of the stored result, 2^-9, and of the inputs read)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import grad as G
+from oracle import memoroid as M
+from gpu_util import dev
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
+
+
+def _close(got, want, tol, what):
+    got = got.float().cpu().numpy().astype(np.float64)
+    scale = np.abs(want).max() + 1e-30
+    err = np.abs(got - want).max() / scale
+    assert err <= tol, f"{what}: {err:.3e} of scale {scale:.3e} (allowed {tol})"
+
+
+def _as(a, dtype):
+    """Array on the device in dtype, and the float64 values the kernel then reads."""
+    t = dev(a.astype(np.float32)).to(dtype)
+    return t, t.float().cpu().numpy().astype(np.float64)
+
+
+@pytest.mark.parametrize("rows,D", [(1, 4), (7, 256), (1000, 260), (33, 512), (5, 1024), (3, 2048), (4099, 64), (16384, 256)])
+@pytest.mark.parametrize("x_dtype,y_dtype", [(torch.float32, torch.float32), (torch.float32, torch.bfloat16),
+                                             (torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32)])
+def test_forward_and_backward(rows, D, x_dtype, y_dtype):
+    from memorax_amd import kernels as K
+    rng = np.random.default_rng(rows + D)
+    print(f"case rms norm rows={rows} D={D} x={x_dtype} y={y_dtype}", flush=True)
+    x, xr = _as(rng.standard_normal((rows, D)) * np.exp(rng.standard_normal((rows, 1))), x_dtype)   # row scales over a decade
+    sc = (1.0 + 0.3 * rng.standard_normal(D)).astype(np.float32)
+    dy, dyr = _as(rng.standard_normal((rows, D)), y_dtype)
+    y = K.rms_norm_fwd(x, dev(sc), 1e-6, y_dtype)
+    assert y.dtype == y_dtype and y.shape == x.shape
+    _close(y, M.rms_norm(xr, sc, 1e-6), TOL[y_dtype], "y")
+    dx, dscale = K.rms_norm_bwd(x, dev(sc), dy, 1e-6)
+    rdx, rds = G.rms_norm_grads(xr, sc.astype(np.float64), dyr, 1e-6)
+    assert dx.dtype == x_dtype and dscale.dtype == torch.float32
+    # dx per row on the row's own scale (rows differ by a decade)
+    got = dx.float().cpu().numpy().astype(np.float64)
+    err = (np.abs(got - rdx).max(-1) / (np.abs(rdx).max(-1) + 1e-30)).max()
+    assert err <= TOL[x_dtype], f"dx: {err:.3e}"
+    _close(dscale, rds, 1e-5 * max(1.0, np.sqrt(rows) / 30), "dscale")   # a float32 sum over the rows
+    # no scale: ones, and no gradient for it
+    y1 = K.rms_norm_fwd(x, None, 1e-6, y_dtype)
+    _close(y1, M.rms_norm(xr, None, 1e-6), TOL[y_dtype], "y without scale")
+    dx1, none = K.rms_norm_bwd(x, None, dy, 1e-6, want_dscale=False)
+    assert none is None
+    rdx1, _ = G.rms_norm_grads(xr, None, dyr, 1e-6)
+    err = (np.abs(dx1.float().cpu().numpy() - rdx1).max(-1) / (np.abs(rdx1).max(-1) + 1e-30)).max()
+    assert err <= TOL[x_dtype], f"dx without scale: {err:.3e}"
+
+
+def test_scale_gradient_does_not_depend_on_the_run():
+    from memorax_amd import kernels as K
+    rng = np.random.default_rng(3)
+    x, dy = dev(rng.standard_normal((50000, 256)).astype(np.float32)), dev(rng.standard_normal((50000, 256)).astype(np.float32))
+    sc = dev(np.ones(256, np.float32))
+    a = K.rms_norm_bwd(x, sc, dy)[1]
+    for _ in range(3):
+        assert torch.equal(K.rms_norm_bwd(x, sc, dy)[1], a)
+
+
+def test_large_eps_and_zero_rows():
+    """A row of zeros normalises to zeros (rsqrt(eps) finite) and passes rsqrt(eps) * scale * dy back."""
+    from memorax_amd import kernels as K
+    x = torch.zeros((3, 8), device="cuda")
+    sc = dev(np.arange(1, 9, dtype=np.float32))
+    dy = dev(np.ones((3, 8), np.float32))
+    assert torch.equal(K.rms_norm_fwd(x, sc, 0.25), torch.zeros_like(x))
+    dx, ds = K.rms_norm_bwd(x, sc, dy, 0.25)
+    np.testing.assert_allclose(dx.cpu().numpy(), 2.0 * np.arange(1, 9)[None] * np.ones((3, 1)), rtol=1e-6)
+    assert torch.equal(ds, torch.zeros_like(ds))
+    xe = torch.empty((0, 8), device="cuda")
+    assert K.rms_norm_fwd(xe, sc).shape == (0, 8)
+    dxe, dse = K.rms_norm_bwd(xe, sc, xe)
+    assert dxe.shape == (0, 8) and torch.equal(dse, torch.zeros_like(dse))
+
+
+def test_autograd_module_and_autocast():
+    from memorax_amd import functional as Fn
+    from memorax_amd import sequence_models as sm
+    rng = np.random.default_rng(9)
+    xn, dyn = rng.standard_normal((4, 9, 256)), rng.standard_normal((4, 9, 256))
+    norm = sm.RMSNorm(256).cuda()
+    with torch.no_grad():
+        norm.scale.copy_(dev((1 + 0.1 * rng.standard_normal(256)).astype(np.float32)))
+    sc = norm.scale.detach().cpu().numpy().astype(np.float64)
+    x = dev(xn.astype(np.float32)).requires_grad_()
+    y = norm(x)
+    assert y.dtype == torch.float32
+    y.backward(dev(dyn.astype(np.float32)))
+    rdx, rds = G.rms_norm_grads(xn.astype(np.float32).astype(np.float64), sc, dyn.astype(np.float32).astype(np.float64))
+    _close(y.detach(), M.rms_norm(xn.astype(np.float32), sc), 1e-5, "module y")
+    _close(x.grad, rdx, 1e-5, "module dx")
+    _close(norm.scale.grad, rds, 1e-5, "module dscale")
+    # under autocast the result comes in the dtype the dense layers behind it compute in
+    x2 = dev(xn.astype(np.float32)).requires_grad_()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y2 = norm(x2)
+    assert y2.dtype == torch.bfloat16
+    y2.float().backward(dev(dyn.astype(np.float32)))
+    _close(y2.detach(), M.rms_norm(xn.astype(np.float32), sc), 2e-2, "autocast y")
+    assert x2.grad.dtype == torch.float32
+    _close(x2.grad, rdx, 2e-2, "autocast dx")
+    # a float64 array is computed in float32 and its gradient comes back as float64; widths the kernel does not take go
+    # to the array library
+    x3 = dev(xn).requires_grad_()
+    y3 = Fn.rms_norm(x3, norm.scale.detach())
+    y3.sum().backward()
+    assert x3.grad.dtype == torch.float64
+    norm6 = sm.RMSNorm(6).cuda()
+    x6 = torch.randn(5, 6, device="cuda")
+    torch.testing.assert_close(norm6(x6), torch.nn.functional.rms_norm(x6, (6,), norm6.scale, 1e-6))
+
+
+def test_refusals():
+    from memorax_amd import _lib
+    lib = _lib.load()
+    x = torch.zeros((4, 256), device="cuda")
+    y = torch.empty_like(x)
+    sc = torch.ones(256, device="cuda")
+    p = lambda t: ctypes.c_void_p(t.data_ptr())   # noqa: E731
+    ok = lambda rows, D, xd=0, yd=0, eps=1e-6, xp=p(x), yp=p(y): lib.mrx_rms_norm_fwd(None, xp, p(sc), yp, rows, D, xd, yd, eps)   # noqa: E731
+    assert ok(4, 256) == 0
+    assert ok(4, 254) == -2          # rows are read four elements at a time
+    assert ok(1, 4096) == -2
+    assert ok(0, 256) == -1
+    assert ok(4, 256, xd=2) == -1     # complex64 is no dtype of this call
+    assert ok(4, 256, eps=-1.0) == -1
+    assert ok(4, 256, xp=None) == -1
+    assert ok(2, 256, xp=ctypes.c_void_p(x.data_ptr() + 4)) == -1
+    dx, ds = torch.empty_like(x), torch.empty(256, device="cuda")
+    bwd = lambda ws, dsp=p(ds): lib.mrx_rms_norm_bwd(None, p(x), p(sc), p(y), p(dx), dsp, ws, 4, 256, 0, 0, 1e-6)   # noqa: E731
+    assert bwd(None) == -1             # the scale's gradient needs the workspace
+    assert bwd(None, None) == 0
+    torch.cuda.synchronize()

@@ -380,3 +380,25 @@ def test_mlstm_gates_grads_fd():
     np.testing.assert_allclose(gf, fd(L, lf), rtol=1e-6, atol=1e-7)
     np.testing.assert_allclose(g0, fd(L, m0), rtol=1e-6, atol=1e-7)
     assert g0[1].tolist() == [0.0, 0.0]   # batch row 1 resets at its first step: the carried m is dropped
+
+
+def test_rms_norm_closed_forms_and_grads_fd():
+    """The norm's restatement against what fixes it: unit mean square and invariance under x -> c x without
+    eps, the closed form of a constant row with it; its gradients against central differences, and dx
+    orthogonal to x (what the invariance implies) with the analytic formula dx = r g - x r^3 (g . x) / D."""
+    x, sc, dy = rnd(3, 5, 8), rnd(8), rnd(3, 5, 8)
+    y = M.rms_norm(x, None, eps=0.0)
+    np.testing.assert_allclose((y * y).mean(-1), 1.0, rtol=1e-12)
+    np.testing.assert_allclose(M.rms_norm(3.7 * x, sc, eps=0.0), M.rms_norm(x, sc, eps=0.0), rtol=1e-12)
+    np.testing.assert_allclose(M.rms_norm(np.full((2, 8), 0.5), sc, eps=0.75), 0.5 * sc[None] * np.ones((2, 1)), rtol=1e-12)
+    for eps in (0.0, 1e-6, 0.3):
+        dx, ds = G.rms_norm_grads(x, sc, dy, eps)
+        np.testing.assert_allclose(dx, fd(lambda: (M.rms_norm(x, sc, eps) * dy).sum(), x), rtol=1e-6, atol=1e-8)
+        np.testing.assert_allclose(ds, fd(lambda: (M.rms_norm(x, sc, eps) * dy).sum(), sc), rtol=1e-6, atol=1e-8)
+        r = 1.0 / np.sqrt((x * x).mean(-1, keepdims=True) + eps)
+        g = dy * sc
+        np.testing.assert_allclose(dx, r * g - x * r ** 3 * (g * x).sum(-1, keepdims=True) / 8, rtol=1e-10, atol=1e-12)
+        np.testing.assert_allclose(ds, (dy * x * r).sum((0, 1)), rtol=1e-10)
+    dx0, none = G.rms_norm_grads(x, None, dy, 0.0)
+    assert none is None
+    np.testing.assert_allclose((dx0 * x).sum(-1), 0.0, atol=1e-12)
