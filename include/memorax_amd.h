@@ -338,14 +338,17 @@ int mrx_linear_scan_last(void *stream, const void *a, const void *b,
  * x, dx: (rows, D) in x_dtype; y in y_dtype, dy in dy_dtype (each MRX_F32 or MRX_BF16; arithmetic in float32);
  * scale (nullable: ones), dscale (nullable: not formed): (D) float32.  D a multiple of 4, at most 2048.
  * The backward recomputes the statistics from x, so the forward leaves nothing behind for it.
+ * dx_add (nullable, like x; not dx itself): added to dx -- the gradient that reaches x along the residual branch
+ * around a pre-norm block (blocks/residual.py:23-26 around normalization.py:30-31), which would otherwise
+ * cost a pass of its own.
  * workspace (required with dscale): MRX_RMS_NORM_PARTS * D floats, overwritten -- per-workgroup partial sums
  * of dscale, added up in a fixed order (the result does not depend on the run). */
 #define MRX_RMS_NORM_PARTS 1024
 int mrx_rms_norm_fwd(void *stream, const void *x, const float *scale, void *y, int64_t rows,
                      int64_t D, int x_dtype, int y_dtype, float eps);
-int mrx_rms_norm_bwd(void *stream, const void *x, const float *scale, const void *dy, void *dx,
-                     float *dscale, float *workspace, int64_t rows, int64_t D, int x_dtype,
-                     int dy_dtype, float eps);
+int mrx_rms_norm_bwd(void *stream, const void *x, const float *scale, const void *dy,
+                     const void *dx_add, void *dx, float *dscale, float *workspace, int64_t rows,
+                     int64_t D, int x_dtype, int dy_dtype, float eps);
 
 /* ---- mLSTM: the stabiliser of the cell's gates ---------------------------------
  * mLSTMCell's elements (C, log_f, n, m) combine by the max-stabilised gated sum of mlstm.py:190-206

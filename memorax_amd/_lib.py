@@ -55,7 +55,7 @@ SIGNATURES = {
     "mrx_mlstm_gates_fwd": (_I, [_P] * 8 + [_L] * 3 + [_I, ctypes.c_float]),
     "mrx_mlstm_gates_bwd": (_I, [_P] * 12 + [_L] * 3 + [_I, ctypes.c_float]),
     "mrx_rms_norm_fwd": (_I, [_P] * 4 + [_L] * 2 + [_I, _I, ctypes.c_float]),
-    "mrx_rms_norm_bwd": (_I, [_P] * 7 + [_L] * 2 + [_I, _I, ctypes.c_float]),
+    "mrx_rms_norm_bwd": (_I, [_P] * 8 + [_L] * 2 + [_I, _I, ctypes.c_float]),
 }
 
 _lib = None

@@ -96,10 +96,13 @@ rms_norm_fwd_kernel(const XT *__restrict__ x, const float *__restrict__ scale, Y
 // With r = rsqrt(mean(x^2) + eps) and g = dy * scale:  dx = r g - x r^3 (g . x) / D,  dscale = sum over rows of
 // dy x r.  The statistics are recomputed from x (it is read for dx anyway): nothing is kept from the forward.
 // parts (gridDim.x, D): this workgroup's share of dscale (null: the scale's gradient is not wanted).
+// dx_add (nullable): a gradient that reaches x by another way -- the residual branch around a pre-norm block --
+// added here instead of by a pass of its own.
 template <typename XT, typename GT, int NV, int RPI>
 __global__ void __launch_bounds__(RN_THREADS)
-rms_norm_bwd_kernel(const XT *__restrict__ x, const float *__restrict__ scale, const GT *__restrict__ dy, XT *__restrict__ dx,
-                    float *__restrict__ parts, int64_t rows, int D, float eps, float inv_D)
+rms_norm_bwd_kernel(const XT *__restrict__ x, const float *__restrict__ scale, const GT *__restrict__ dy,
+                    const XT *__restrict__ dx_add, XT *__restrict__ dx, float *__restrict__ parts, int64_t rows, int D, float eps,
+                    float inv_D)
 {
     __shared__ float red[RN_WAVES][NV * 256];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -112,7 +115,7 @@ rms_norm_bwd_kernel(const XT *__restrict__ x, const float *__restrict__ scale, c
         ds[i] = F4{{0.f, 0.f, 0.f, 0.f}};
     }
     for (int64_t r0 = wave * RPI; r0 < rows; r0 += nwaves * RPI) {
-        F4 xv[RPI][NV], gv[RPI][NV];
+        F4 xv[RPI][NV], gv[RPI][NV], av[RPI][NV];
 #pragma unroll
         for (int j = 0; j < RPI; ++j)
 #pragma unroll
@@ -121,6 +124,7 @@ rms_norm_bwd_kernel(const XT *__restrict__ x, const float *__restrict__ scale, c
                 const bool in = r0 + j < rows && col < D;
                 xv[j][i] = in ? load_quad(x + (r0 + j) * D + col) : F4{{0.f, 0.f, 0.f, 0.f}};
                 gv[j][i] = in ? load_quad(dy + (r0 + j) * D + col) : F4{{0.f, 0.f, 0.f, 0.f}};
+                av[j][i] = (in && dx_add) ? load_quad(dx_add + (r0 + j) * D + col) : F4{{0.f, 0.f, 0.f, 0.f}};
             }
 #pragma unroll
         for (int j = 0; j < RPI; ++j) {
@@ -142,7 +146,7 @@ rms_norm_bwd_kernel(const XT *__restrict__ x, const float *__restrict__ scale, c
                         F4 o;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            o.v[e] = gv[j][i].v[e] * sc[i].v[e] * rstd - xv[j][i].v[e] * c;
+                            o.v[e] = av[j][i].v[e] + (gv[j][i].v[e] * sc[i].v[e] * rstd - xv[j][i].v[e] * c);
                             ds[i].v[e] += gv[j][i].v[e] * xv[j][i].v[e] * rstd;
                         }
                         store_quad(dx + (r0 + j) * D + col, o);
@@ -165,19 +169,30 @@ rms_norm_bwd_kernel(const XT *__restrict__ x, const float *__restrict__ scale, c
     }
 }
 
-// dscale[col] = sum over the nparts rows of parts, in a fixed order: 64 columns per workgroup, four threads per
-// column that each add every fourth row.
-__global__ void __launch_bounds__(RN_THREADS) rms_norm_dscale_kernel(const float *__restrict__ parts, float *__restrict__ dscale,
-                                                                  int nparts, int D)
+// dscale[col] = sum over the nparts rows of parts, in a fixed order: 64 columns per workgroup, sixteen threads per
+// column that each add every sixteenth row, four independent sums in flight per thread.
+constexpr int RD_GROUPS = 16;
+__global__ void __launch_bounds__(64 * RD_GROUPS) rms_norm_dscale_kernel(const float *__restrict__ parts, float *__restrict__ dscale,
+                                                                      int nparts, int D)
 {
-    __shared__ float red[RN_WAVES][64];
+    __shared__ float red[RD_GROUPS][64];
     const int c = threadIdx.x & 63, g = threadIdx.x >> 6, col = blockIdx.x * 64 + c;
-    float s = 0.f;
-    if (col < D)
-        for (int p = g; p < nparts; p += RN_WAVES) s += parts[(int64_t)p * D + col];
-    red[g][c] = s;
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    if (col < D) {
+        int p = g;
+        for (; p + 3 * RD_GROUPS < nparts; p += 4 * RD_GROUPS)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) s[u] += parts[(int64_t)(p + u * RD_GROUPS) * D + col];
+        for (; p < nparts; p += RD_GROUPS) s[0] += parts[(int64_t)p * D + col];
+    }
+    red[g][c] = (s[0] + s[1]) + (s[2] + s[3]);
     __syncthreads();
-    if (g == 0 && col < D) dscale[col] = (red[0][c] + red[1][c]) + (red[2][c] + red[3][c]);
+    if (g == 0 && col < D) {
+        float t = 0.f;
+#pragma unroll
+        for (int j = 0; j < RD_GROUPS; ++j) t += red[j][c];
+        dscale[col] = t;
+    }
 }
 
 int check_rows(const void *x, const void *out, int64_t rows, int64_t D)
@@ -215,22 +230,23 @@ template <typename XT, typename YT> int dispatch_fwd(hipStream_t st, const void 
 }
 
 template <typename XT, typename GT, int NV>
-int launch_bwd(hipStream_t st, const void *x, const float *scale, const void *dy, void *dx, float *parts, unsigned grid, int64_t rows,
-               int D, float eps)
+int launch_bwd(hipStream_t st, const void *x, const float *scale, const void *dy, const void *dx_add, void *dx, float *parts,
+               unsigned grid, int64_t rows, int D, float eps)
 {
     constexpr int RPI = NV <= 2 ? 2 : 1;
     return launch_kernel(rms_norm_bwd_kernel<XT, GT, NV, RPI>, dim3(grid), dim3(RN_THREADS), 0, st, static_cast<const XT *>(x), scale,
-                         static_cast<const GT *>(dy), static_cast<XT *>(dx), parts, rows, D, eps, 1.f / (float)D);
+                         static_cast<const GT *>(dy), static_cast<const XT *>(dx_add), static_cast<XT *>(dx), parts, rows, D, eps,
+                         1.f / (float)D);
 }
 
 template <typename XT, typename GT>
-int dispatch_bwd(hipStream_t st, const void *x, const float *scale, const void *dy, void *dx, float *parts, unsigned grid, int64_t rows,
-                 int D, float eps)
+int dispatch_bwd(hipStream_t st, const void *x, const float *scale, const void *dy, const void *dx_add, void *dx, float *parts,
+                 unsigned grid, int64_t rows, int D, float eps)
 {
-    if (D <= 256) return launch_bwd<XT, GT, 1>(st, x, scale, dy, dx, parts, grid, rows, D, eps);
-    if (D <= 512) return launch_bwd<XT, GT, 2>(st, x, scale, dy, dx, parts, grid, rows, D, eps);
-    if (D <= 1024) return launch_bwd<XT, GT, 4>(st, x, scale, dy, dx, parts, grid, rows, D, eps);
-    return launch_bwd<XT, GT, 8>(st, x, scale, dy, dx, parts, grid, rows, D, eps);
+    if (D <= 256) return launch_bwd<XT, GT, 1>(st, x, scale, dy, dx_add, dx, parts, grid, rows, D, eps);
+    if (D <= 512) return launch_bwd<XT, GT, 2>(st, x, scale, dy, dx_add, dx, parts, grid, rows, D, eps);
+    if (D <= 1024) return launch_bwd<XT, GT, 4>(st, x, scale, dy, dx_add, dx, parts, grid, rows, D, eps);
+    return launch_bwd<XT, GT, 8>(st, x, scale, dy, dx_add, dx, parts, grid, rows, D, eps);
 }
 
 }  // namespace
@@ -253,13 +269,14 @@ extern "C" int mrx_rms_norm_fwd(void *stream, const void *x, const float *scale,
                               : dispatch_fwd<__bf16, __bf16>(st, x, scale, y, rows, d, eps);
 }
 
-extern "C" int mrx_rms_norm_bwd(void *stream, const void *x, const float *scale, const void *dy, void *dx, float *dscale,
-                                float *workspace, int64_t rows, int64_t D, int x_dtype, int dy_dtype, float eps)
+extern "C" int mrx_rms_norm_bwd(void *stream, const void *x, const float *scale, const void *dy, const void *dx_add, void *dx,
+                                float *dscale, float *workspace, int64_t rows, int64_t D, int x_dtype, int dy_dtype, float eps)
 {
     using namespace mrx;
     if (const int rc = check_rows(x, dx, rows, D); rc != MRX_OK) return rc;
     if (!dy || !known(x_dtype) || !known(dy_dtype) || !(eps >= 0.f)) return MRX_ERR_INVALID_ARG;
-    if (!quad_aligned(x, x_dtype) || !quad_aligned(dx, x_dtype) || !quad_aligned(dy, dy_dtype) || (scale && !aligned(scale, 16)))
+    if (!quad_aligned(x, x_dtype) || !quad_aligned(dx, x_dtype) || !quad_aligned(dy, dy_dtype) || (scale && !aligned(scale, 16)) ||
+        (dx_add && !quad_aligned(dx_add, x_dtype)))
         return MRX_ERR_INVALID_ARG;
     if (dscale && !workspace) return MRX_ERR_INVALID_ARG;
     if (const int rc = prepare_device(); rc != MRX_OK) return rc;
@@ -269,12 +286,12 @@ extern "C" int mrx_rms_norm_bwd(void *stream, const void *x, const float *scale,
     float *parts = dscale ? workspace : nullptr;
     int rc;
     if (x_dtype == MRX_F32)
-        rc = dy_dtype == MRX_F32 ? dispatch_bwd<float, float>(st, x, scale, dy, dx, parts, grid, rows, d, eps)
-                                 : dispatch_bwd<float, __bf16>(st, x, scale, dy, dx, parts, grid, rows, d, eps);
+        rc = dy_dtype == MRX_F32 ? dispatch_bwd<float, float>(st, x, scale, dy, dx_add, dx, parts, grid, rows, d, eps)
+                                 : dispatch_bwd<float, __bf16>(st, x, scale, dy, dx_add, dx, parts, grid, rows, d, eps);
     else
-        rc = dy_dtype == MRX_F32 ? dispatch_bwd<__bf16, float>(st, x, scale, dy, dx, parts, grid, rows, d, eps)
-                                 : dispatch_bwd<__bf16, __bf16>(st, x, scale, dy, dx, parts, grid, rows, d, eps);
+        rc = dy_dtype == MRX_F32 ? dispatch_bwd<__bf16, float>(st, x, scale, dy, dx_add, dx, parts, grid, rows, d, eps)
+                                 : dispatch_bwd<__bf16, __bf16>(st, x, scale, dy, dx_add, dx, parts, grid, rows, d, eps);
     if (rc != MRX_OK || !dscale) return rc;
-    return launch_kernel(rms_norm_dscale_kernel, dim3((unsigned)((d + 63) / 64)), dim3(RN_THREADS), 0, st, workspace, dscale,
+    return launch_kernel(rms_norm_dscale_kernel, dim3((unsigned)((d + 63) / 64)), dim3(64 * RD_GROUPS), 0, st, workspace, dscale,
                          (int)grid, d);
 }

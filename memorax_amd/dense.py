@@ -6,8 +6,8 @@ has a hundred thousand rows and a few hundred features, so the weight gradient `
 product with a tiny result and an enormous inner dimension, which the library's GEMM runs on as
 many workgroups as the result has tiles (sixteen for 256 x 256: 330 us where the forward product
 of the same operands takes 32 us).  ``dense`` cuts the rows into slices, multiplies them as one
-batched product with float32 partial results and sums those (41 us), and casts the input once for
-all layers that share it.
+batched product with float32 partial results and sums those (41 us); ``dense_group`` runs the
+layers that share an input on one cast of it and lets their products add up the input gradient.
 """
 from __future__ import annotations
 
@@ -31,13 +31,6 @@ def autocast_dtype(x):
     if x.is_cuda and x.is_floating_point() and torch.is_autocast_enabled("cuda"):
         return torch.get_autocast_dtype("cuda")
     return None
-
-
-def compute_input(x):
-    """``x`` as the dense layers will read it: under autocast one cast serves every layer that
-    takes the same input (each would otherwise make its own copy)."""
-    dt = autocast_dtype(x)
-    return x if dt is None or x.dtype == dt else x.to(dt)
 
 
 def _slices(rows, n_out, n_in):
@@ -88,6 +81,48 @@ class _Dense(torch.autograd.Function):
         if ctx.has_bias and ctx.needs_input_grad[2]:
             db = dy2.sum(0, dtype=_wide(dy2.dtype))
         return dx, dw, db
+
+
+class _DenseGroup(torch.autograd.Function):
+    """Several dense layers on one input.  Their gradients with respect to the input are accumulated by the
+    products themselves (each adds onto the sum so far) instead of by a pass per layer."""
+
+    @staticmethod
+    def forward(ctx, x, n, *params):
+        weights, biases = params[:n], params[n:]
+        dt = autocast_dtype(x)
+        xc = x if dt is None else x.to(dt)
+        wcs = [w if dt is None else w.to(dt) for w in weights]
+        ctx.save_for_backward(xc, *wcs)
+        ctx.set_materialize_grads(False)   # an output nobody used costs no products
+        ctx.x_dtype, ctx.n, ctx.has_bias = x.dtype, n, [b is not None for b in biases]
+        return tuple(F.linear(xc, w, b if b is None or dt is None else b.to(dt)) for w, b in zip(wcs, biases))
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, *dys):
+        xc, *wcs = ctx.saved_tensors
+        n = ctx.n
+        x2 = xc.reshape(-1, xc.shape[-1])
+        dx, dws, dbs = None, [None] * n, [None] * n
+        for i, (dy, w) in enumerate(zip(dys, wcs)):
+            if dy is None:
+                continue
+            dy2 = dy.to(xc.dtype).reshape(-1, dy.shape[-1])
+            if ctx.needs_input_grad[0]:
+                dx = dy2 @ w if dx is None else dx.addmm_(dy2, w)
+            if ctx.needs_input_grad[2 + i]:
+                dws[i] = weight_gradient(dy2, x2)
+            if ctx.has_bias[i] and ctx.needs_input_grad[2 + n + i]:
+                dbs[i] = dy2.sum(0, dtype=_wide(dy2.dtype))
+        if dx is not None:
+            dx = dx.view(xc.shape).to(ctx.x_dtype)
+        return (dx, None, *dws, *dbs)
+
+
+def dense_group(x, layers):
+    """The outputs of several Dense / torch.nn.Linear layers that read the same input, as a tuple."""
+    return _DenseGroup.apply(x, len(layers), *[m.weight for m in layers], *[m.bias for m in layers])
 
 
 def dense(x, weight, bias=None):

@@ -477,6 +477,40 @@ class _RmsNorm(torch.autograd.Function):
         return dx.to(ctx.x_dtype), dscale, None, None
 
 
+class _RmsNormFork(torch.autograd.Function):
+    """(x, rms_norm(x)): the input handed on beside its norm, so that the gradients of both meet in the norm's
+    backward kernel instead of in a pass of their own."""
+
+    @staticmethod
+    def forward(ctx, x, scale, eps, out_dtype):
+        xc = x.contiguous()
+        sc = None if scale is None else scale.contiguous().float()
+        ctx.save_for_backward(xc, *([sc] if sc is not None else []))
+        ctx.eps = eps
+        return xc.view_as(xc), K.rms_norm_fwd(xc, sc, eps, out_dtype)
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, dres, dy):
+        xc, *rest = ctx.saved_tensors
+        sc = rest[0] if rest else None
+        if dy is None:
+            return dres, None, None, None
+        dy = dy.contiguous()
+        if dy.dtype not in (torch.float32, torch.bfloat16):
+            dy = dy.float()
+        add = None if dres is None else dres.contiguous().to(xc.dtype)
+        dx, dscale = K.rms_norm_bwd(xc, sc, dy, ctx.eps, want_dscale=sc is not None and ctx.needs_input_grad[1], dx_add=add)
+        return dx, dscale, None, None
+
+
+def rms_norm_fork(x, scale=None, eps=1e-6, out_dtype=None):
+    """(x, rms_norm(x, scale, eps, out_dtype)) for the residual branch around a pre-norm block
+    (blocks/residual.py:23-26 around normalization.py:30-31): use the first result where x itself would be
+    used.  The backward adds the gradient of that branch inside the norm's kernel.  x float32 or bfloat16."""
+    return _RmsNormFork.apply(x, scale, eps, out_dtype)
+
+
 def rms_norm(x, scale=None, eps=1e-6, out_dtype=None):
     """flax.linen.RMSNorm with its defaults over the last axis (linear_attention.py:109-115; the norm of the
     torso's PreNorm blocks): x * rsqrt(mean(x^2) + eps) * scale, one kernel each way.  x (..., D) float32 or

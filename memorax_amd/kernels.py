@@ -153,25 +153,26 @@ def rms_norm_fwd(x, scale, eps=1e-6, out_dtype=None):
     return y
 
 
-def rms_norm_bwd(x, scale, dy, eps=1e-6, want_dscale=True):
+def rms_norm_bwd(x, scale, dy, eps=1e-6, want_dscale=True, dx_add=None):
     """Gradients of rms_norm_fwd: dy (..., D) float32 or bfloat16 in; (dx in x's dtype, dscale (D) float32 or
-    None) out.  The statistics are recomputed from x."""
+    None) out.  The statistics are recomputed from x.  dx_add (like x, or None): added to dx."""
     lib = _lib.load()
     D = x.shape[-1]
     if x.dtype not in (torch.float32, torch.bfloat16) or dy.dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("rms_norm takes float32 or bfloat16 arrays")
     _chk(x, "x")
     _chk(dy, "dy", None, x.shape)
+    _chk(dx_add, "dx_add", x.dtype, x.shape)
     _chk(scale, "scale", torch.float32, (D,))
     dx = torch.empty_like(x)
     dscale = work = None
     if want_dscale:
-        dscale = torch.zeros((D,), dtype=torch.float32, device=x.device)
+        dscale = torch.empty((D,), dtype=torch.float32, device=x.device)
         work = torch.empty((RMS_NORM_PARTS, D), dtype=torch.float32, device=x.device)
     if x.numel() == 0:
-        return dx, dscale
-    st = lib.mrx_rms_norm_bwd(_stream(), _ptr(x), _ptr(scale), _ptr(dy), _ptr(dx), _ptr(dscale), _ptr(work), x.numel() // D, D,
-                              _DT[x.dtype], _DT[dy.dtype], float(eps))
+        return dx, (None if dscale is None else dscale.zero_())   # dx (and dx_add) are empty
+    st = lib.mrx_rms_norm_bwd(_stream(), _ptr(x), _ptr(scale), _ptr(dy), _ptr(dx_add), _ptr(dx), _ptr(dscale), _ptr(work),
+                              x.numel() // D, D, _DT[x.dtype], _DT[dy.dtype], float(eps))
     _lib.check(st, "mrx_rms_norm_bwd")
     return dx, dscale
 

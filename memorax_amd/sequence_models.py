@@ -29,9 +29,9 @@ import torch.nn.functional as F
 
 from typing import NamedTuple
 
-from .dense import Dense, autocast_dtype, compute_input
+from .dense import Dense, autocast_dtype, dense_group
 from .functional import (deltanet, gated_linear_attention, linear_attention, linear_scan, mingru_scan, mlstm_gates,
-                         normalised_linear_attention, rms_norm)
+                         normalised_linear_attention, rms_norm, rms_norm_fork)
 from .kernels import RMS_NORM_MAX_D as _RMS_NORM_MAX_D
 
 
@@ -286,6 +286,22 @@ class S5Cell(_DiagonalCell):
                 torch.ones(*batch, 1, self.state_size, dtype=torch.complex64, device=dev))
 
 
+class _SownValues(dict):
+    """What the reference records with flax's ``sow`` (min_gru.py:63): the value is formed when it is read,
+    not when it is recorded -- a mean over a (B,T,F) array is a pass over memory that a training step never
+    looks at.  Until then the entry holds on to the array it will be formed from."""
+
+    def sow(self, name, thunk):
+        dict.__setitem__(self, name, thunk)
+
+    def __getitem__(self, name):
+        value = dict.__getitem__(self, name)
+        if callable(value):
+            value = value()
+            dict.__setitem__(self, name, value)
+        return value
+
+
 class MinGRUProjections(NamedTuple):
     """MinGRU's elements before the element map: the step's two projections.  ``MinGRUCell.scan``
     hands them to the kernel that applies the map (a = sigma(-z), b = sigma(z) g(h~)) itself."""
@@ -308,12 +324,14 @@ class MinGRUCell(_DiagonalCell):
         in_features = features if in_features is None else in_features
         self.z = Dense(in_features, features, bias=False)
         self.h = Dense(in_features, features, bias=False)
-        self.intermediates = {}
+        self.intermediates = _SownValues()
 
     def forward(self, x, **kwargs):
-        x = compute_input(x)
-        z, h_tilde = self.z(x), self.h(x)
-        self.intermediates["gate"] = z.mean().detach()   # min_gru.py:63 sows the mean gate
+        return self.elements(*dense_group(x, [self.z, self.h]))
+
+    def elements(self, z, h_tilde):
+        """The cell's elements from its two projections."""
+        self.intermediates.sow("gate", lambda z=z.detach(): z.float().mean())   # min_gru.py:63 sows the mean gate
         if self.fused:   # the recurrence runs in fp32 whatever the projections' dtype (autocast): the kernels
             # read bfloat16 projections as they are (and write bfloat16 states); anything else goes in as float32
             if z.dtype == torch.bfloat16 and h_tilde.dtype == torch.bfloat16:
@@ -360,9 +378,9 @@ class GatedLinearRecurrence(SequenceModel):
     def forward(self, inputs, done, initial_carry=None, **kwargs):
         if initial_carry is None:
             initial_carry = self.cell.initialize_carry(None, get_input_shape(inputs))
-        inputs = compute_input(inputs)
-        h, next_carry = self.cell.scan(self.cell(inputs), initial_carry, done)
-        return next_carry, self.out(h[0] * F.silu(self.gate(inputs)))
+        z, h_tilde, gate = dense_group(inputs, [self.cell.z, self.cell.h, self.gate])
+        h, next_carry = self.cell.scan(self.cell.elements(z, h_tilde), initial_carry, done)
+        return next_carry, self.out(h[0] * F.silu(gate))
 
     def initialize_carry(self, key, input_shape):
         return self.cell.initialize_carry(key, input_shape)
@@ -384,10 +402,19 @@ class _RMSNorm(nn.Module):
         the dtype its readers compute in (under autocast the dense layers behind a norm would each cast it
         again); rows it does not take (wider than 2048 features, a width that is no multiple of 4) and host
         arrays go to the array library."""
-        D = x.shape[-1]
-        if x.is_cuda and D % 4 == 0 and D <= _RMS_NORM_MAX_D:
+        if self._on_kernel(x):
             return rms_norm(x, self.scale, self.eps, autocast_dtype(x) or x.dtype)
-        return F.rms_norm(x.float(), (D,), self.scale.float(), self.eps).to(x.dtype)
+        return F.rms_norm(x.float(), (x.shape[-1],), self.scale.float(), self.eps).to(x.dtype)
+
+    def _on_kernel(self, x):
+        return x.is_cuda and x.shape[-1] % 4 == 0 and x.shape[-1] <= _RMS_NORM_MAX_D
+
+    def fork(self, x):
+        """(x, norm(x)) for a residual branch around this norm: with the first result used in place of x, the
+        gradients of the two branches are added inside the norm's backward kernel."""
+        if self._on_kernel(x) and x.dtype in (torch.float32, torch.bfloat16):
+            return rms_norm_fork(x, self.scale, self.eps, autocast_dtype(x) or x.dtype)
+        return x, self(x)
 
 
 class LinearAttentionCell(MemoroidCellBase):
@@ -414,8 +441,8 @@ class LinearAttentionCell(MemoroidCellBase):
         """Elements in kernel form: (v, k, q), keys and queries before the feature map (phi is applied
         inside the kernel).  The reference's elements are (v phi(k)^T, phi(k)); the query joins them here
         because the kernel contracts the state with it as it goes."""
-        x = compute_input(x)
-        return (self._heads(self.value(x)), self._heads(self.key(x)), self._heads(self.query(x)))
+        v, k, q = dense_group(x, [self.value, self.key, self.query])
+        return (self._heads(v), self._heads(k), self._heads(q))
 
     def binary_operator(self, a, b):
         return tuple(x + y for x, y in zip(a, b))
@@ -479,9 +506,8 @@ class DeltaNetCell(MemoroidCellBase):
         """The raw projections (q, k, v, beta logits): the key normalisation and the sigmoid run
         inside the kernels."""
         dt = self.dtype
-        x = compute_input(x)
-        return (self._heads(self.query(x)).to(dt), self._heads(self.key(x)).to(dt),
-                self._heads(self.value(x)).to(dt), self.beta(x).to(dt))
+        q, k, v, beta = dense_group(x, [self.query, self.key, self.value, self.beta])
+        return (self._heads(q).to(dt), self._heads(k).to(dt), self._heads(v).to(dt), beta.to(dt))
 
     def binary_operator(self, a, b):
         B_i, A_i = a
@@ -535,13 +561,14 @@ class MambaCell(MemoroidCellBase):
     def _project(self, x):
         Bn, T, _ = x.shape
         H, P, N = self.num_heads, self.head_dim, self.state_dim
-        hidden, z = self.input_projection(x).chunk(2, dim=-1)
-        ci = torch.cat([hidden, self.B(x), self.C(x)], dim=-1).transpose(1, 2)      # (B, channels, T)
+        up, B_in, C_in, dt_in = dense_group(x, [self.input_projection, self.B, self.C, self.dt])
+        hidden, z = up.chunk(2, dim=-1)
+        ci = torch.cat([hidden, B_in, C_in], dim=-1).transpose(1, 2)      # (B, channels, T)
         ci = F.silu(self.conv(F.pad(ci, (self.conv_dim - 1, 0)))).transpose(1, 2)   # causal, per call
         hidden = ci[..., :H * P].reshape(Bn, T, H, P)
         B_proj = ci[..., H * P:H * P + H * N].reshape(Bn, T, H, N)
         C_proj = ci[..., H * P + H * N:].reshape(Bn, T, H, N)
-        dt = F.softplus(self.dt(x) + self.dt_bias)
+        dt = F.softplus(dt_in + self.dt_bias)
         return hidden, B_proj, C_proj, z, dt
 
     def forward(self, x, **kwargs):
@@ -654,8 +681,9 @@ class mLSTMCell(MemoroidCellBase):
         Bn, T, _ = x.shape
         q, k, v, _, _ = self._project(x)
         gate_input = torch.cat([q, k, v], dim=-1).reshape(Bn, T, -1)
-        log_i = self.i_gate(gate_input).float()
-        log_f = -F.softplus(-self.f_gate(gate_input).float())
+        i_pre, f_pre = dense_group(gate_input, [self.i_gate, self.f_gate])
+        log_i = i_pre.float()
+        log_f = -F.softplus(-f_pre.float())
         return (k / math.sqrt(k.shape[-1]), v, log_i, log_f, q)
 
     def binary_operator(self, a, b):
@@ -769,7 +797,12 @@ class Residual(nn.Module):
         self.module = module
 
     def forward(self, inputs, done=None, initial_carry=None, **kwargs):
-        carry, y = self.module(inputs, done, initial_carry, **kwargs)
+        inner = self.module
+        if isinstance(inner, PreNorm) and hasattr(inner.norm, "fork"):   # x + f(norm(x)): one kernel takes both gradients of x
+            inputs, normed = inner.norm.fork(inputs)
+            carry, y = inner.module(normed, done, initial_carry, **kwargs)
+        else:
+            carry, y = inner(inputs, done, initial_carry, **kwargs)
         return carry, inputs + y
 
     def initialize_carry(self, key, input_shape):

@@ -51,6 +51,13 @@ def test_forward_and_backward(rows, D, x_dtype, y_dtype):
     err = (np.abs(got - rdx).max(-1) / (np.abs(rdx).max(-1) + 1e-30)).max()
     assert err <= TOL[x_dtype], f"dx: {err:.3e}"
     _close(dscale, rds, 1e-5 * max(1.0, np.sqrt(rows) / 30), "dscale")   # a float32 sum over the rows
+    # a gradient that reaches x by another way is added in the same pass
+    add, addr = _as(rng.standard_normal((rows, D)), x_dtype)
+    dx2, dscale2 = K.rms_norm_bwd(x, dev(sc), dy, 1e-6, dx_add=add)
+    got = dx2.float().cpu().numpy().astype(np.float64)
+    err = (np.abs(got - (rdx + addr)).max(-1) / (np.abs(rdx + addr).max(-1) + 1e-30)).max()
+    assert err <= TOL[x_dtype], f"dx with dx_add: {err:.3e}"
+    assert torch.equal(dscale2, dscale)
     # no scale: ones, and no gradient for it
     y1 = K.rms_norm_fwd(x, None, 1e-6, y_dtype)
     _close(y1, M.rms_norm(xr, None, 1e-6), TOL[y_dtype], "y without scale")
@@ -124,6 +131,39 @@ def test_autograd_module_and_autocast():
     torch.testing.assert_close(norm6(x6), torch.nn.functional.rms_norm(x6, (6,), norm6.scale, 1e-6))
 
 
+def test_residual_around_a_pre_norm_block_adds_both_gradients_in_the_norm_kernel():
+    """Residual(PreNorm(f, RMSNorm)): x + f(norm(x)).  Values and gradients against the same block with the norm and
+    the addition as separate array operations."""
+    from memorax_amd import sequence_models as sm
+    torch.manual_seed(0)
+    inner = sm.Projection(256, 256).cuda()
+    block = sm.Residual(sm.PreNorm(inner, 256, norm=sm.RMSNorm)).cuda()
+    with torch.no_grad():
+        block.module.norm.scale.copy_(1 + 0.1 * torch.randn(256, device="cuda"))
+    x = torch.randn(6, 11, 256, device="cuda", requires_grad=True)
+    x2 = x.detach().clone().requires_grad_()
+    g = torch.randn(6, 11, 256, device="cuda")
+    carry, y = block(x)
+    assert carry is None
+    y.backward(g)
+    sc = block.module.norm.scale.detach().clone().requires_grad_()
+    w, b = inner.proj.weight.detach().double(), inner.proj.bias.detach().double()
+    xd, scd = x2.double(), sc.double()
+    yr = xd + (xd * torch.rsqrt((xd * xd).mean(-1, keepdim=True) + 1e-6) * scd) @ w.T + b
+    yr.backward(g.double())
+    torch.testing.assert_close(y.detach().double(), yr.detach(), rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(x.grad.double(), x2.grad.double(), rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(block.module.norm.scale.grad.double(), sc.grad.double(), rtol=1e-4, atol=1e-4)
+    # an input that needs no gradient, and the norm's branch unused downstream of the fork
+    _, y0 = block(x.detach())
+    torch.testing.assert_close(y0, y.detach())
+    from memorax_amd import functional as Fn
+    x3 = x.detach().clone().requires_grad_()
+    res, _unused = Fn.rms_norm_fork(x3, sc.detach())
+    (res * g).sum().backward()
+    torch.testing.assert_close(x3.grad, g)
+
+
 def test_refusals():
     from memorax_amd import _lib
     lib = _lib.load()
@@ -141,7 +181,7 @@ def test_refusals():
     assert ok(4, 256, xp=None) == -1
     assert ok(2, 256, xp=ctypes.c_void_p(x.data_ptr() + 4)) == -1
     dx, ds = torch.empty_like(x), torch.empty(256, device="cuda")
-    bwd = lambda ws, dsp=p(ds): lib.mrx_rms_norm_bwd(None, p(x), p(sc), p(y), p(dx), dsp, ws, 4, 256, 0, 0, 1e-6)   # noqa: E731
+    bwd = lambda ws, dsp=p(ds): lib.mrx_rms_norm_bwd(None, p(x), p(sc), p(y), None, p(dx), dsp, ws, 4, 256, 0, 0, 1e-6)   # noqa: E731
     assert bwd(None) == -1             # the scale's gradient needs the workspace
     assert bwd(None, None) == 0
     torch.cuda.synchronize()

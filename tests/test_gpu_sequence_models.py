@@ -464,12 +464,15 @@ def test_torso_stack_of_four_blocks_against_the_fp64_restatement(dtype, tol, std
     # terms carrying that slope -- would differ by some 10 %: a property of the function.  The restatement is
     # therefore evaluated on the branches the modules themselves took (their own pre-activations, captured
     # here), and every gradient is held to the one tolerance.
-    sides, hooks = [], []
-    for blk in torso.blocks[1::2]:
-        hooks.append(blk.module.module.cell.h.register_forward_hook(lambda m, i, out: sides.append((out.detach() >= 0).cpu())))
+    sides, cells = [], [blk.module.module.cell for blk in torso.blocks[1::2]]
+    for cell in cells:
+        def recording(z, h_tilde, _elements=cell.elements):
+            sides.append((h_tilde.detach() >= 0).cpu())
+            return _elements(z, h_tilde)
+        cell.elements = recording
     carries, y = torso(x, done)
-    for h_ in hooks:
-        h_.remove()
+    for cell in cells:
+        del cell.elements
     (y * gy).sum().backward()
     xr = _f64(x).requires_grad_()
     rcar, ry, rparams = _torso_reference(G, torso, xr, done.cpu(), None, H, sides)

@@ -90,3 +90,15 @@ def test_prenorm_defaults_to_layer_norm_and_takes_rms_norm():
     yi = inner(x)[1]
     want = (yi - yi.mean(-1, keepdim=True)) / torch.sqrt(yi.var(-1, unbiased=False, keepdim=True) + 1e-6)
     assert torch.allclose(p(x)[1], want * p.norm.weight + p.norm.bias, atol=1e-12)
+
+
+def test_mingru_cell_sows_the_mean_gate_when_it_is_read():
+    """min_gru.py:63 records mean(z) of every call; here the mean is formed on first reading."""
+    cell = sm.MinGRUCell(6, in_features=8)
+    x = _x(seed=4).float()
+    proj = cell(x)
+    assert callable(dict.__getitem__(cell.intermediates, "gate"))     # nothing computed yet
+    want = (x @ cell.z.weight.T).mean()
+    assert torch.allclose(cell.intermediates["gate"], want, atol=1e-6)
+    assert not callable(dict.__getitem__(cell.intermediates, "gate"))  # kept once read
+    assert proj.z.shape == (3, 5, 6) and not cell.intermediates["gate"].requires_grad

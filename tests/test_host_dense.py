@@ -71,3 +71,49 @@ def test_dense_sliced_weight_gradient_on_the_device(n_out, n_in, bias, amp):
     if bias:
         db = ge.reshape(-1, n_out).sum(0)
         assert (den.bias.grad.double() - db).abs().max().item() <= 1e-4 * db.abs().max().item() + 1e-3
+
+
+def test_dense_group_matches_separate_layers_on_cpu():
+    torch.manual_seed(3)
+    layers = [D.Dense(10, 6).double(), D.Dense(10, 3, bias=False).double(), D.Dense(10, 5).double()]
+    x = torch.randn(4, 7, 10, dtype=torch.float64, requires_grad=True)
+    x2 = x.detach().clone().requires_grad_()
+    gs = [torch.randn(4, 7, m.out_features, dtype=torch.float64) for m in layers]
+    ys = D.dense_group(x, layers)
+    # the second output stays unused: its layer gets no gradient, the others are not disturbed
+    (ys[0] * gs[0]).sum().add((ys[2] * gs[2]).sum()).backward()
+    want = [torch.nn.functional.linear(x2, m.weight.detach().clone().requires_grad_(),
+                                       None if m.bias is None else m.bias.detach().clone().requires_grad_()) for m in layers]
+    for y, w in zip(ys, want):
+        assert torch.equal(y, w)
+    (want[0] * gs[0]).sum().add((want[2] * gs[2]).sum()).backward()
+    torch.testing.assert_close(x.grad, x2.grad, rtol=1e-12, atol=1e-12)
+    assert layers[1].weight.grad is None
+    ref0 = gs[0].reshape(-1, 6).t() @ x.detach().reshape(-1, 10)
+    torch.testing.assert_close(layers[0].weight.grad, ref0, rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(layers[2].bias.grad, gs[2].reshape(-1, 5).sum(0), rtol=1e-12, atol=1e-12)
+    params = [m.weight for m in layers] + [layers[0].bias, layers[2].bias]
+    assert torch.autograd.gradcheck(lambda a, *p: D.dense_group(a, layers), (x, *params))
+
+
+@pytest.mark.gpu
+def test_dense_group_on_the_device_under_autocast():
+    torch.manual_seed(4)
+    B, T, n_in = 128, 128, 256
+    layers = [D.Dense(n_in, 256, bias=False).cuda(), D.Dense(n_in, 256, bias=False).cuda(), D.Dense(n_in, 4, bias=True).cuda()]
+    x = torch.randn(B, T, n_in, device="cuda", requires_grad=True)
+    x2 = x.detach().clone().requires_grad_()
+    gs = [torch.randn(B, T, m.out_features, device="cuda") for m in layers]
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        ys = D.dense_group(x, layers)
+        want = [torch.nn.functional.linear(x2, m.weight.detach(), None if m.bias is None else m.bias.detach()) for m in layers]
+    for y, w in zip(ys, want):
+        assert y.dtype == torch.bfloat16 and torch.equal(y, w)
+    sum((y.float() * g).sum() for y, g in zip(ys, gs)).backward()
+    sum((y.float() * g).sum() for y, g in zip(want, gs)).backward()
+    assert x.grad.dtype == torch.float32
+    torch.testing.assert_close(x.grad, x2.grad, rtol=2e-2, atol=2e-2 * x2.grad.abs().max().item())
+    xe = x.detach().bfloat16().double().reshape(-1, n_in)
+    for m, g in zip(layers, gs):
+        dw = g.bfloat16().double().reshape(-1, m.out_features).t() @ xe
+        assert (m.weight.grad.double() - dw).abs().max().item() <= 1e-4 * dw.abs().max().item()
