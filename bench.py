@@ -92,6 +92,9 @@ def main() -> int:
     ap.add_argument("--no-children", action="store_true",
                     help="skip the two measurements that run in child processes (64-step-chunk build, product-phase "
                          "clocks): under a profiler the children would be traced into the same output")
+    ap.add_argument("--torso-only", action="store_true",
+                    help="time configuration 5's whole torso through the host mirror and nothing else (the run a "
+                         "kernel trace of the mirror's array-library side is taken from)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain elementwise kernel of known size (256 MiB read, 256 MiB "
                          "written) so that a rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE run can be scaled")
@@ -116,6 +119,9 @@ def main() -> int:
 
     if args.phase_clocks:
         print(json.dumps(phase_clocks_child(np, torch, K, dev)))
+        return 0
+    if args.torso_only:
+        print(json.dumps(bench_torso_full(torch, K)))
         return 0
     secondary = {}
     if not args.headline_only:
@@ -738,6 +744,7 @@ def bench_torso_full(torch, K):
             torch.nn.init.normal_(p, 0.0, 0.02)
     x = torch.randn(B, T, Fe, device="cuda")
     done = torch.rand(B, T, device="cuda") < 0.01
+    gy = torch.randn(B, T, Fe, device="cuda")
 
     def full(autocast=True):
         for p in torso.parameters():
@@ -746,11 +753,14 @@ def bench_torso_full(torch, K):
         # recurrences in the precision their kernels take (bf16 in / fp32 state; fp32 for the scan)
         with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
             _, y = torso(x, done)
-        y.float().pow(2).mean().backward()
+        y.backward(gy)   # the gradient a policy head would hand back
     ms_full = _time_ms(torch, full, iters=5, warm=2)
     ms_full32 = _time_ms(torch, lambda: full(False), iters=3, warm=1)
+    for blk in torso.blocks[0::2]:   # episodes end every hundred steps here: the caller's choice of merged episodes
+        blk.module.module.cell.resets = "merged"
+    ms_merged = _time_ms(torch, full, iters=5, warm=2)
     return {"full_torso_ms": ms_full, "full_torso_tokens/s": B * T / ms_full * 1e3,
-            "full_torso_ms_fp32_projections": ms_full32}
+            "full_torso_ms_merged_resets": ms_merged, "full_torso_ms_fp32_projections": ms_full32}
 
 
 def cpu_baseline(np, x, do_np):

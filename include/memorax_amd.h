@@ -350,6 +350,15 @@ int mrx_rms_norm_bwd(void *stream, const void *x, const float *scale, const void
                      const void *dx_add, void *dx, float *dscale, float *workspace, int64_t rows,
                      int64_t D, int x_dtype, int dy_dtype, float eps);
 
+/* ---- gating product ----------------------------------------------------------------
+ * y = h * silu(g): activation(gate) * value of the reference's GLU block (blocks/ffn.py:108-121) with silu as
+ * the activation, one read of the operands per direction.  Backward: dh = dy * silu(g),
+ * dg = dy * h * d silu(g).  All arrays n elements of `dtype` (MRX_F32 or MRX_BF16; arithmetic in float32),
+ * 16-byte aligned. */
+int mrx_silu_gate_fwd(void *stream, const void *h, const void *g, void *y, int64_t n, int dtype);
+int mrx_silu_gate_bwd(void *stream, const void *h, const void *g, const void *dy, void *dh, void *dg,
+                      int64_t n, int dtype);
+
 /* ---- mLSTM: the stabiliser of the cell's gates ---------------------------------
  * mLSTMCell's elements (C, log_f, n, m) combine by the max-stabilised gated sum of mlstm.py:190-206
  * (m = max(m_a + log_f_b, m_b), both sides rescaled by exp(. - m)) under Memoroid.scan_fn's select-reset

@@ -14,7 +14,7 @@ cd "$(dirname "$0")"
 HIPCC=${HIPCC:-/opt/rocm/bin/hipcc}
 FLAGS=(--offload-arch=gfx950 -O3 -std=c++17 -fPIC -I../../include
        -Xclang -target-feature -Xclang -packed-fp32-ops -Wall -Wno-unused-function)
-SRCS=(api.hip scan.hip chunk_fwd.hip chunk_bwd.hip step.hip delta_tm.hip la_states.hip mlstm_gates.hip rms_norm.hip)
+SRCS=(api.hip scan.hip chunk_fwd.hip chunk_bwd.hip step.hip delta_tm.hip la_states.hip mlstm_gates.hip rms_norm.hip gate.hip)
 pids=()
 compile() {  # compile <object suffix> <extra flags...>
     local suf=$1; shift

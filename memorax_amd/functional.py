@@ -7,6 +7,7 @@ the role jax.custom_vjp would in a JAX host).
     delta_rule(q, k, v, beta, done, S0=None)             -> (o, S_last)
     deltanet(q, k, v, beta_raw, done, S0=None)           -> (o, S_last)   (key L2-norm and sigmoid fused)
     rms_norm(x, scale, eps, out_dtype)                   -> y
+    silu_gate(h, g)                                      -> h * silu(g)
 
 Layouts follow the reference: (B,T,D) / (B,T,H,d), state (B,H,d_v,d_k), done (B,T)
 bool or float where nonzero clears the carry before step t (memoroid.py:60-91).
@@ -475,6 +476,31 @@ class _RmsNorm(torch.autograd.Function):
             dy = dy.float()
         dx, dscale = K.rms_norm_bwd(xc, sc, dy, ctx.eps, want_dscale=sc is not None and ctx.needs_input_grad[1])
         return dx.to(ctx.x_dtype), dscale, None, None
+
+
+class _SiluGate(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, h, g):
+        dt = torch.promote_types(h.dtype, g.dtype)
+        if dt not in (torch.float32, torch.bfloat16):
+            dt = torch.float32
+        hc, gc = h.to(dt).contiguous(), g.to(dt).contiguous()
+        ctx.save_for_backward(hc, gc)
+        ctx.dtypes = (h.dtype, g.dtype)
+        return K.silu_gate_fwd(hc, gc)
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, dy):
+        hc, gc = ctx.saved_tensors
+        dh, dg = K.silu_gate_bwd(hc, gc, dy.to(hc.dtype).contiguous())
+        return dh.to(ctx.dtypes[0]), dg.to(ctx.dtypes[1])
+
+
+def silu_gate(h, g):
+    """h * silu(g) -- activation(gate) * value of the reference's GLU block (blocks/ffn.py:108-121) with silu --
+    in one kernel each way.  h, g of one shape; float32 or bfloat16 (anything else is computed in float32)."""
+    return _SiluGate.apply(h, g)
 
 
 class _RmsNormFork(torch.autograd.Function):

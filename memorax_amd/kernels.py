@@ -177,6 +177,34 @@ def rms_norm_bwd(x, scale, dy, eps=1e-6, want_dscale=True, dx_add=None):
     return dx, dscale
 
 
+def silu_gate_fwd(h, g):
+    """y = h * silu(g) (mrx_silu_gate_fwd): h, g of one shape and dtype, float32 or bfloat16."""
+    lib = _lib.load()
+    if h.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("silu_gate takes float32 or bfloat16 arrays")
+    _chk(h, "h")
+    _chk(g, "g", h.dtype, h.shape)
+    y = torch.empty_like(h)
+    if h.numel():
+        _lib.check(lib.mrx_silu_gate_fwd(_stream(), _ptr(h), _ptr(g), _ptr(y), h.numel(), _DT[h.dtype]), "mrx_silu_gate_fwd")
+    return y
+
+
+def silu_gate_bwd(h, g, dy):
+    """(dh, dg) of y = h * silu(g) for the gradient dy of y."""
+    lib = _lib.load()
+    if h.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("silu_gate takes float32 or bfloat16 arrays")
+    _chk(h, "h")
+    _chk(g, "g", h.dtype, h.shape)
+    _chk(dy, "dy", h.dtype, h.shape)
+    dh, dg = torch.empty_like(h), torch.empty_like(h)
+    if h.numel():
+        _lib.check(lib.mrx_silu_gate_bwd(_stream(), _ptr(h), _ptr(g), _ptr(dy), _ptr(dh), _ptr(dg), h.numel(), _DT[h.dtype]),
+                   "mrx_silu_gate_bwd")
+    return dh, dg
+
+
 def linear_scan_last(a, b, done, h0=None):
     """Final state of h_t = done ? b_t : a_t h_{t-1} + b_t with one decay per group of channels:
     a: (B,T,D/group), b: (B,T,D), h0: (B,D) or None.  Returns h_last (B,D)."""

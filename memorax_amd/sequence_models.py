@@ -31,7 +31,7 @@ from typing import NamedTuple
 
 from .dense import Dense, autocast_dtype, dense_group
 from .functional import (deltanet, gated_linear_attention, linear_attention, linear_scan, mingru_scan, mlstm_gates,
-                         normalised_linear_attention, rms_norm, rms_norm_fork)
+                         normalised_linear_attention, rms_norm, rms_norm_fork, silu_gate)
 from .kernels import RMS_NORM_MAX_D as _RMS_NORM_MAX_D
 
 
@@ -380,7 +380,8 @@ class GatedLinearRecurrence(SequenceModel):
             initial_carry = self.cell.initialize_carry(None, get_input_shape(inputs))
         z, h_tilde, gate = dense_group(inputs, [self.cell.z, self.cell.h, self.gate])
         h, next_carry = self.cell.scan(self.cell.elements(z, h_tilde), initial_carry, done)
-        return next_carry, self.out(h[0] * F.silu(gate))
+        gated = silu_gate(h[0], gate) if gate.is_cuda else h[0] * F.silu(gate)
+        return next_carry, self.out(gated)
 
     def initialize_carry(self, key, input_shape):
         return self.cell.initialize_carry(key, input_shape)

@@ -99,6 +99,13 @@ def mlstm_gates_grads(log_i, log_f, done, m0, dm, dg, dw, g_floor=-60.0):
     return _np(li.grad), _np(lf.grad), (None if m0 is None else _np(m0_.grad))
 
 
+def silu_gate_grads(h, g, dy):
+    """(dh, dg) of L = sum(dy * h * silu(g))."""
+    h_, g_ = _t(h, True), _t(g, True)
+    (h_ * torch.nn.functional.silu(g_) * _t(dy)).sum().backward()
+    return _np(h_.grad), _np(g_.grad)
+
+
 def rms_norm_grads(x, scale, dy, eps=1e-6):
     """(dx, dscale) of L = sum(dy * rms_norm(x, scale)); scale None: (dx, None)."""
     x_ = _t(x, True)

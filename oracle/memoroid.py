@@ -482,6 +482,12 @@ def mlstm(q, k, v, i_gate, f_gate, done, carry=None, tree=True):
     return nxt, mlstm_read(h, q)
 
 
+def silu_gate(h, g):
+    """activation(gate) * value of the GLU block (blocks/ffn.py:108-121) with silu: h * g * sigmoid(g)."""
+    h, g = np.asarray(h, np.float64), np.asarray(g, np.float64)
+    return h * g / (1.0 + np.exp(-g))
+
+
 def rms_norm(x, scale=None, eps=1e-6):
     """flax.linen.RMSNorm with its defaults over the last axis (the norm of LinearAttentionCell.read,
     linear_attention.py:109-115, and of PreNorm blocks built with it, blocks/normalization.py:10-35):

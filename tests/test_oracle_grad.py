@@ -402,3 +402,18 @@ def test_rms_norm_closed_forms_and_grads_fd():
     dx0, none = G.rms_norm_grads(x, None, dy, 0.0)
     assert none is None
     np.testing.assert_allclose((dx0 * x).sum(-1), 0.0, atol=1e-12)
+
+
+def test_silu_gate_closed_forms_and_grads_fd():
+    """h * silu(g): silu(0) = 0, silu(g) - silu(-g) = g, silu(g) -> g for large g; gradients against central
+    differences and the closed form d silu = s (1 + g (1 - s)), s = sigmoid(g)."""
+    h, g, dy = rnd(4, 6), rnd(4, 6) * 3, rnd(4, 6)
+    one = np.ones_like(g)
+    np.testing.assert_allclose(M.silu_gate(h, np.zeros_like(g)), 0.0)
+    np.testing.assert_allclose(M.silu_gate(one, g) - M.silu_gate(one, -g), g, rtol=1e-12)
+    np.testing.assert_allclose(M.silu_gate(h, np.full_like(g, 50.0)), 50.0 * h, rtol=1e-12)
+    dh, dg = G.silu_gate_grads(h, g, dy)
+    np.testing.assert_allclose(dh, fd(lambda: (M.silu_gate(h, g) * dy).sum(), h), rtol=1e-6, atol=1e-8)
+    np.testing.assert_allclose(dg, fd(lambda: (M.silu_gate(h, g) * dy).sum(), g), rtol=1e-6, atol=1e-8)
+    s = 1 / (1 + np.exp(-g))
+    np.testing.assert_allclose(dg, dy * h * s * (1 + g * (1 - s)), rtol=1e-10)
