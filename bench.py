@@ -93,8 +93,8 @@ def main() -> int:
                     help="skip the two measurements that run in child processes (64-step-chunk build, product-phase "
                          "clocks): under a profiler the children would be traced into the same output")
     ap.add_argument("--torso-only", action="store_true",
-                    help="time configuration 5's whole torso through the host mirror and nothing else (the run a "
-                         "kernel trace of the mirror's array-library side is taken from)")
+                    help="time configuration 5's whole torso through the host mirror under bf16 autocast and nothing "
+                         "else (seven updates: the run a kernel trace of the mirror's array-library side is taken from)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain elementwise kernel of known size (256 MiB read, 256 MiB "
                          "written) so that a rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE run can be scaled")
@@ -121,7 +121,7 @@ def main() -> int:
         print(json.dumps(phase_clocks_child(np, torch, K, dev)))
         return 0
     if args.torso_only:
-        print(json.dumps(bench_torso_full(torch, K)))
+        print(json.dumps(bench_torso_full(torch, K, variants=False)))
         return 0
     secondary = {}
     if not args.headline_only:
@@ -727,10 +727,10 @@ def bench_torso_kernels(torch, K):
                 4 * ((BYTES_FWD + BYTES_BWD) * B * T * H + 18 * B * T * Fe) / ms_h / 1e6 / HBM_PEAK_GBS}
 
 
-def bench_torso_full(torch, K):
+def bench_torso_full(torch, K, variants=True):
     """Configuration 5 through the host mirror, dense projections in torch included: 4 blocks of
     [RMSNorm -> DeltaNet(H=4, d=64) -> +x ; RMSNorm -> gated linear recurrence -> +x], d_model 256,
-    weights N(0, 0.02)."""
+    weights N(0, 0.02).  variants=False: the bf16-autocast update only, seven times (two of them warm-up)."""
     from memorax_amd import sequence_models as sm
     B, T, Fe, H, d = 1024, 128, 256, 4, 64
     torch.manual_seed(5)
@@ -755,6 +755,8 @@ def bench_torso_full(torch, K):
             _, y = torso(x, done)
         y.backward(gy)   # the gradient a policy head would hand back
     ms_full = _time_ms(torch, full, iters=5, warm=2)
+    if not variants:
+        return {"full_torso_ms": ms_full, "full_torso_tokens/s": B * T / ms_full * 1e3}
     ms_full32 = _time_ms(torch, lambda: full(False), iters=3, warm=1)
     for blk in torso.blocks[0::2]:   # episodes end every hundred steps here: the caller's choice of merged episodes
         blk.module.module.cell.resets = "merged"
