@@ -68,6 +68,26 @@ def test_forward_and_backward(rows, D, x_dtype, y_dtype):
     assert err <= TOL[x_dtype], f"dx without scale: {err:.3e}"
 
 
+def test_random_widths_and_row_counts():
+    """Thirty drawn (rows, D): every width class of the kernels (one to eight 256-column groups per lane, widths that
+    leave lanes and whole groups empty), row counts around the waves' strides."""
+    from memorax_amd import kernels as K
+    rng = np.random.default_rng(77)
+    for case in range(30):
+        D = 4 * int(rng.integers(1, 513))
+        rows = int(rng.choice([1, 2, 3, 5, 17, 63, 257, 1025, 4097, 20001]))
+        xd, yd = (torch.float32, torch.bfloat16)[int(rng.integers(2))], (torch.float32, torch.bfloat16)[int(rng.integers(2))]
+        print(f"case rms norm random {case}: rows={rows} D={D} x={xd} y={yd}", flush=True)
+        x, xr = _as(rng.standard_normal((rows, D)) * 2.0, xd)
+        dy, dyr = _as(rng.standard_normal((rows, D)), yd)
+        sc = (1.0 + 0.3 * rng.standard_normal(D)).astype(np.float32)
+        _close(K.rms_norm_fwd(x, dev(sc), 1e-6, yd), M.rms_norm(xr, sc, 1e-6), TOL[yd], "y")
+        dx, ds = K.rms_norm_bwd(x, dev(sc), dy, 1e-6)
+        rdx, rds = G.rms_norm_grads(xr, sc.astype(np.float64), dyr, 1e-6)
+        _close(dx, rdx, TOL[xd], "dx")
+        _close(ds, rds, 1e-5 * max(1.0, np.sqrt(rows) / 30), "dscale")
+
+
 def test_scale_gradient_does_not_depend_on_the_run():
     from memorax_amd import kernels as K
     rng = np.random.default_rng(3)
