@@ -51,7 +51,7 @@ def weight_gradient(dy, x):
     s = _slices(rows, n_out, n_in) if dy.is_cuda else 1
     if s == 1:
         return (dy.t() @ x).to(_wide(dy.dtype))
-    a, b = dy.view(s, rows // s, n_out).transpose(1, 2), x.view(s, rows // s, n_in)
+    a, b = dy.reshape(s, rows // s, n_out).transpose(1, 2), x.reshape(s, rows // s, n_in)
     if dy.dtype in _HALVES:
         return torch.bmm(a, b, out_dtype=torch.float32).sum(0)
     return torch.bmm(a, b).sum(0)
