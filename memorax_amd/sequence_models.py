@@ -302,6 +302,11 @@ class _SownValues(dict):
         return value
 
 
+def _gated(value, gate):
+    """value * silu(gate) (blocks/ffn.py:108-121 with silu): the library's kernel on the device."""
+    return silu_gate(value, gate) if gate.is_cuda else value * F.silu(gate)
+
+
 class MinGRUProjections(NamedTuple):
     """MinGRU's elements before the element map: the step's two projections.  ``MinGRUCell.scan``
     hands them to the kernel that applies the map (a = sigma(-z), b = sigma(z) g(h~)) itself."""
@@ -380,8 +385,7 @@ class GatedLinearRecurrence(SequenceModel):
             initial_carry = self.cell.initialize_carry(None, get_input_shape(inputs))
         z, h_tilde, gate = dense_group(inputs, [self.cell.z, self.cell.h, self.gate])
         h, next_carry = self.cell.scan(self.cell.elements(z, h_tilde), initial_carry, done)
-        gated = silu_gate(h[0], gate) if gate.is_cuda else h[0] * F.silu(gate)
-        return next_carry, self.out(gated)
+        return next_carry, self.out(_gated(h[0], gate))
 
     def initialize_carry(self, key, input_shape):
         return self.cell.initialize_carry(key, input_shape)
@@ -603,7 +607,7 @@ class MambaCell(MemoroidCellBase):
         hidden, _, _, z, _ = self._project(x)
         y = o.float() + self.D[None, None, :, None] * hidden
         y = y.reshape(Bn, T, self.num_heads * self.head_dim)
-        return self.output_projection((self.norm(y) * F.silu(z)).to(x.dtype))
+        return self.output_projection(_gated(self.norm(y), z).to(x.dtype))
 
     def initialize_carry(self, key, input_shape):
         *batch, _ = input_shape
@@ -731,7 +735,7 @@ class mLSTMCell(MemoroidCellBase):
         _, _, _, z, u = self._project(x)
         y = F.layer_norm(h_tilde, (h_tilde.shape[-1],), eps=1e-5) * (1.0 + self.norm_weight)[None, None]
         y = y.reshape(Bn, T, self.hidden_dim) + self.learnable_skip * u
-        return self.output_projection((y * F.silu(z)).to(x.dtype))
+        return self.output_projection(_gated(y, z).to(x.dtype))
 
     def initialize_carry(self, key, input_shape):
         *batch, _ = input_shape
