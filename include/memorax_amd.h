@@ -350,6 +350,16 @@ int mrx_rms_norm_bwd(void *stream, const void *x, const float *scale, const void
                      const void *dx_add, void *dx, float *dscale, float *workspace, int64_t rows,
                      int64_t D, int x_dtype, int dy_dtype, float eps);
 
+/* Layer norm over the last axis: y = (x - mean(x)) * rsqrt(var(x) + eps) * scale + bias -- flax.linen.LayerNorm with
+ * its defaults (eps 1e-6), the default norm of PreNorm / PostNorm (blocks/normalization.py:10-65).  Arguments as
+ * mrx_rms_norm_*; bias, dbias: (D) float32 (bias nullable: zeros); dscale and dbias both or neither; workspace
+ * (required with them): 2 * MRX_RMS_NORM_PARTS * D floats. */
+int mrx_layer_norm_fwd(void *stream, const void *x, const float *scale, const float *bias, void *y,
+                       int64_t rows, int64_t D, int x_dtype, int y_dtype, float eps);
+int mrx_layer_norm_bwd(void *stream, const void *x, const float *scale, const void *dy,
+                       const void *dx_add, void *dx, float *dscale, float *dbias, float *workspace,
+                       int64_t rows, int64_t D, int x_dtype, int dy_dtype, float eps);
+
 /* ---- gating product ----------------------------------------------------------------
  * y = h * silu(g): activation(gate) * value of the reference's GLU block (blocks/ffn.py:108-121) with silu as
  * the activation, one read of the operands per direction.  Backward: dh = dy * silu(g),

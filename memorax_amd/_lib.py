@@ -54,6 +54,8 @@ SIGNATURES = {
     "mrx_gated_linear_attn_step": (_I, [_P] * 9 + [_L] * 4 + [_I] * 3),
     "mrx_mlstm_gates_fwd": (_I, [_P] * 8 + [_L] * 3 + [_I, ctypes.c_float]),
     "mrx_mlstm_gates_bwd": (_I, [_P] * 12 + [_L] * 3 + [_I, ctypes.c_float]),
+    "mrx_layer_norm_fwd": (_I, [_P] * 5 + [_L] * 2 + [_I, _I, ctypes.c_float]),
+    "mrx_layer_norm_bwd": (_I, [_P] * 9 + [_L] * 2 + [_I, _I, ctypes.c_float]),
     "mrx_silu_gate_fwd": (_I, [_P] * 4 + [_L, _I]),
     "mrx_silu_gate_bwd": (_I, [_P] * 6 + [_L, _I]),
     "mrx_rms_norm_fwd": (_I, [_P] * 4 + [_L] * 2 + [_I, _I, ctypes.c_float]),

@@ -6,7 +6,7 @@ the role jax.custom_vjp would in a JAX host).
     linear_attention(q, k, v, done, S0=None, feature_map) -> (o, S_last)
     delta_rule(q, k, v, beta, done, S0=None)             -> (o, S_last)
     deltanet(q, k, v, beta_raw, done, S0=None)           -> (o, S_last)   (key L2-norm and sigmoid fused)
-    rms_norm(x, scale, eps, out_dtype)                   -> y
+    rms_norm(x, scale, eps, out_dtype)                   -> y      (layer_norm likewise, with a bias)
     silu_gate(h, g)                                      -> h * silu(g)
 
 Layouts follow the reference: (B,T,D) / (B,T,H,d), state (B,H,d_v,d_k), done (B,T)
@@ -455,29 +455,6 @@ def mlstm_gates(log_i, log_f, done, m0=None, g_floor=-60.0):
     return _MlstmGates.apply(log_i, log_f, done, m0, g_floor)
 
 
-class _RmsNorm(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, x, scale, eps, out_dtype):
-        xc = x.contiguous()
-        if xc.dtype not in (torch.float32, torch.bfloat16):
-            xc = xc.float()
-        sc = None if scale is None else scale.contiguous().float()
-        ctx.save_for_backward(xc, *([sc] if sc is not None else []))
-        ctx.eps, ctx.x_dtype = eps, x.dtype
-        return K.rms_norm_fwd(xc, sc, eps, out_dtype)
-
-    @staticmethod
-    @torch.autograd.function.once_differentiable
-    def backward(ctx, dy):
-        xc, *rest = ctx.saved_tensors
-        sc = rest[0] if rest else None
-        dy = dy.contiguous()
-        if dy.dtype not in (torch.float32, torch.bfloat16):
-            dy = dy.float()
-        dx, dscale = K.rms_norm_bwd(xc, sc, dy, ctx.eps, want_dscale=sc is not None and ctx.needs_input_grad[1])
-        return dx.to(ctx.x_dtype), dscale, None, None
-
-
 class _SiluGate(torch.autograd.Function):
     @staticmethod
     def forward(ctx, h, g):
@@ -503,45 +480,67 @@ def silu_gate(h, g):
     return _SiluGate.apply(h, g)
 
 
-class _RmsNormFork(torch.autograd.Function):
-    """(x, rms_norm(x)): the input handed on beside its norm, so that the gradients of both meet in the norm's
-    backward kernel instead of in a pass of their own."""
+def _norm_operand(t):
+    t = t.contiguous()
+    return t if t.dtype in (torch.float32, torch.bfloat16) else t.float()
+
+
+class _Norm(torch.autograd.Function):
+    """RMS norm (center False) or layer norm of x; fork: the input is handed on beside its norm -- (x, norm(x)) -- so
+    that the gradients of both meet in the norm's backward kernel instead of in a pass of their own."""
 
     @staticmethod
-    def forward(ctx, x, scale, eps, out_dtype):
-        xc = x.contiguous()
+    def forward(ctx, x, scale, bias, eps, out_dtype, center, fork):
+        xc = _norm_operand(x)
         sc = None if scale is None else scale.contiguous().float()
+        bi = None if bias is None else bias.contiguous().float()
         ctx.save_for_backward(xc, *([sc] if sc is not None else []))
-        ctx.eps = eps
-        return xc.view_as(xc), K.rms_norm_fwd(xc, sc, eps, out_dtype)
+        ctx.eps, ctx.x_dtype, ctx.center, ctx.fork = eps, x.dtype, center, fork
+        ctx.has_scale, ctx.has_bias = sc is not None, bi is not None
+        y = K.layer_norm_fwd(xc, sc, bi, eps, out_dtype, center)
+        if fork:
+            ctx.set_materialize_grads(False)
+            return xc.view_as(xc).to(x.dtype), y
+        return y
 
     @staticmethod
     @torch.autograd.function.once_differentiable
-    def backward(ctx, dres, dy):
+    def backward(ctx, *grads):
         xc, *rest = ctx.saved_tensors
         sc = rest[0] if rest else None
-        if dy is None:
-            return dres, None, None, None
-        dy = dy.contiguous()
-        if dy.dtype not in (torch.float32, torch.bfloat16):
-            dy = dy.float()
+        dres, dy = grads if ctx.fork else (None, grads[0])
+        if dy is None:   # the norm's branch was not used
+            return dres, None, None, None, None, None, None
+        want = (ctx.has_scale and ctx.needs_input_grad[1]) or (ctx.has_bias and ctx.needs_input_grad[2])
         add = None if dres is None else dres.contiguous().to(xc.dtype)
-        dx, dscale = K.rms_norm_bwd(xc, sc, dy, ctx.eps, want_dscale=sc is not None and ctx.needs_input_grad[1], dx_add=add)
-        return dx, dscale, None, None
-
-
-def rms_norm_fork(x, scale=None, eps=1e-6, out_dtype=None):
-    """(x, rms_norm(x, scale, eps, out_dtype)) for the residual branch around a pre-norm block
-    (blocks/residual.py:23-26 around normalization.py:30-31): use the first result where x itself would be
-    used.  The backward adds the gradient of that branch inside the norm's kernel.  x float32 or bfloat16."""
-    return _RmsNormFork.apply(x, scale, eps, out_dtype)
+        dx, dscale, dbias = K.layer_norm_bwd(xc, sc, _norm_operand(dy), ctx.eps, want, add, ctx.center)
+        return (dx.to(ctx.x_dtype), dscale if ctx.has_scale else None, dbias if ctx.has_bias else None, None, None, None, None)
 
 
 def rms_norm(x, scale=None, eps=1e-6, out_dtype=None):
     """flax.linen.RMSNorm with its defaults over the last axis (linear_attention.py:109-115; the norm of the
     torso's PreNorm blocks): x * rsqrt(mean(x^2) + eps) * scale, one kernel each way.  x (..., D) float32 or
     bfloat16 with D a multiple of 4 up to 2048, scale (D) or None; the result in out_dtype (default x's)."""
-    return _RmsNorm.apply(x, scale, eps, out_dtype)
+    return _Norm.apply(x, scale, None, eps, out_dtype, False, False)
+
+
+def rms_norm_fork(x, scale=None, eps=1e-6, out_dtype=None):
+    """(x, rms_norm(x, scale, eps, out_dtype)) for the residual branch around a pre-norm block
+    (blocks/residual.py:23-26 around normalization.py:30-31): use the first result where x itself would be
+    used.  The backward adds the gradient of that branch inside the norm's kernel."""
+    return _Norm.apply(x, scale, None, eps, out_dtype, False, True)
+
+
+def layer_norm(x, scale=None, bias=None, eps=1e-6, out_dtype=None):
+    """flax.linen.LayerNorm with its defaults over the last axis (the default norm of PreNorm / PostNorm,
+    blocks/normalization.py:10-65): (x - mean(x)) * rsqrt(var(x) + eps) * scale + bias, one kernel each way.
+    Shapes and dtypes as rms_norm."""
+    return _Norm.apply(x, scale, bias, eps, out_dtype, True, False)
+
+
+def layer_norm_fork(x, scale=None, bias=None, eps=1e-6, out_dtype=None):
+    """(x, layer_norm(x, ...)): rms_norm_fork for the layer norm."""
+    return _Norm.apply(x, scale, bias, eps, out_dtype, True, True)
 
 
 def propagate_sensitivities(decay, jacobians, sensitivity, done):

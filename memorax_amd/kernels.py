@@ -134,47 +134,75 @@ RMS_NORM_PARTS = 1024   # MRX_RMS_NORM_PARTS: rows of the backward's workspace
 RMS_NORM_MAX_D = 2048
 
 
+def _norm_dtypes(*ts):
+    for t in ts:
+        if t not in (torch.float32, torch.bfloat16):
+            raise ValueError("the norm kernels take float32 or bfloat16 arrays")
+
+
 def rms_norm_fwd(x, scale, eps=1e-6, out_dtype=None):
     """y = x * rsqrt(mean(x^2) + eps) * scale over the last axis (mrx_rms_norm_fwd): x (..., D) float32 or
     bfloat16, scale (D) float32 or None (ones); y in out_dtype (default: x's)."""
-    lib = _lib.load()
-    D = x.shape[-1]
-    out_dtype = x.dtype if out_dtype is None else out_dtype
-    if x.dtype not in (torch.float32, torch.bfloat16) or out_dtype not in (torch.float32, torch.bfloat16):
-        raise ValueError("rms_norm takes float32 or bfloat16 arrays")
-    _chk(x, "x")
-    _chk(scale, "scale", torch.float32, (D,))
-    y = torch.empty(x.shape, dtype=out_dtype, device=x.device)
-    if x.numel() == 0:
-        return y
-    st = lib.mrx_rms_norm_fwd(_stream(), _ptr(x), _ptr(scale), _ptr(y), x.numel() // D, D, _DT[x.dtype], _DT[out_dtype],
-                              float(eps))
-    _lib.check(st, "mrx_rms_norm_fwd")
-    return y
+    return layer_norm_fwd(x, scale, None, eps, out_dtype, center=False)
 
 
 def rms_norm_bwd(x, scale, dy, eps=1e-6, want_dscale=True, dx_add=None):
     """Gradients of rms_norm_fwd: dy (..., D) float32 or bfloat16 in; (dx in x's dtype, dscale (D) float32 or
     None) out.  The statistics are recomputed from x.  dx_add (like x, or None): added to dx."""
+    dx, dscale, _ = layer_norm_bwd(x, scale, dy, eps, want_dscale, dx_add, center=False)
+    return dx, dscale
+
+
+def layer_norm_fwd(x, scale, bias, eps=1e-6, out_dtype=None, center=True):
+    """y = (x - mean(x)) * rsqrt(var(x) + eps) * scale + bias over the last axis (mrx_layer_norm_fwd); center=False:
+    the RMS norm (no mean, no bias).  x (..., D) float32 or bfloat16; scale, bias (D) float32 or None."""
     lib = _lib.load()
     D = x.shape[-1]
-    if x.dtype not in (torch.float32, torch.bfloat16) or dy.dtype not in (torch.float32, torch.bfloat16):
-        raise ValueError("rms_norm takes float32 or bfloat16 arrays")
+    out_dtype = x.dtype if out_dtype is None else out_dtype
+    _norm_dtypes(x.dtype, out_dtype)
+    _chk(x, "x")
+    _chk(scale, "scale", torch.float32, (D,))
+    _chk(bias, "bias", torch.float32, (D,))
+    y = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    if x.numel() == 0:
+        return y
+    rows = x.numel() // D
+    if center:
+        st = lib.mrx_layer_norm_fwd(_stream(), _ptr(x), _ptr(scale), _ptr(bias), _ptr(y), rows, D, _DT[x.dtype], _DT[out_dtype],
+                                    float(eps))
+    else:
+        st = lib.mrx_rms_norm_fwd(_stream(), _ptr(x), _ptr(scale), _ptr(y), rows, D, _DT[x.dtype], _DT[out_dtype], float(eps))
+    _lib.check(st, "mrx_layer_norm_fwd" if center else "mrx_rms_norm_fwd")
+    return y
+
+
+def layer_norm_bwd(x, scale, dy, eps=1e-6, want_dparams=True, dx_add=None, center=True):
+    """Gradients of layer_norm_fwd: (dx in x's dtype, dscale, dbias) -- the parameters' gradients (D) float32, or
+    None when not wanted (dbias also None for the RMS norm).  dx_add (like x, or None): added to dx."""
+    lib = _lib.load()
+    D = x.shape[-1]
+    _norm_dtypes(x.dtype, dy.dtype)
     _chk(x, "x")
     _chk(dy, "dy", None, x.shape)
     _chk(dx_add, "dx_add", x.dtype, x.shape)
     _chk(scale, "scale", torch.float32, (D,))
     dx = torch.empty_like(x)
-    dscale = work = None
-    if want_dscale:
+    dscale = dbias = work = None
+    if want_dparams:
         dscale = torch.empty((D,), dtype=torch.float32, device=x.device)
-        work = torch.empty((RMS_NORM_PARTS, D), dtype=torch.float32, device=x.device)
-    if x.numel() == 0:
-        return dx, (None if dscale is None else dscale.zero_())   # dx (and dx_add) are empty
-    st = lib.mrx_rms_norm_bwd(_stream(), _ptr(x), _ptr(scale), _ptr(dy), _ptr(dx_add), _ptr(dx), _ptr(dscale), _ptr(work),
-                              x.numel() // D, D, _DT[x.dtype], _DT[dy.dtype], float(eps))
-    _lib.check(st, "mrx_rms_norm_bwd")
-    return dx, dscale
+        dbias = torch.empty_like(dscale) if center else None
+        work = torch.empty(((2 if center else 1) * RMS_NORM_PARTS, D), dtype=torch.float32, device=x.device)
+    if x.numel() == 0:   # dx (and dx_add) are empty
+        return dx, (None if dscale is None else dscale.zero_()), (None if dbias is None else dbias.zero_())
+    rows = x.numel() // D
+    if center:
+        st = lib.mrx_layer_norm_bwd(_stream(), _ptr(x), _ptr(scale), _ptr(dy), _ptr(dx_add), _ptr(dx), _ptr(dscale), _ptr(dbias),
+                                    _ptr(work), rows, D, _DT[x.dtype], _DT[dy.dtype], float(eps))
+    else:
+        st = lib.mrx_rms_norm_bwd(_stream(), _ptr(x), _ptr(scale), _ptr(dy), _ptr(dx_add), _ptr(dx), _ptr(dscale), _ptr(work),
+                                  rows, D, _DT[x.dtype], _DT[dy.dtype], float(eps))
+    _lib.check(st, "mrx_layer_norm_bwd" if center else "mrx_rms_norm_bwd")
+    return dx, dscale, dbias
 
 
 def silu_gate_fwd(h, g):

@@ -31,7 +31,7 @@ from typing import NamedTuple
 
 from .dense import Dense, autocast_dtype, dense_group
 from .functional import (deltanet, gated_linear_attention, linear_attention, linear_scan, mingru_scan, mlstm_gates,
-                         normalised_linear_attention, rms_norm, rms_norm_fork, silu_gate)
+                         normalised_linear_attention, layer_norm, layer_norm_fork, rms_norm, rms_norm_fork, silu_gate)
 from .kernels import RMS_NORM_MAX_D as _RMS_NORM_MAX_D
 
 
@@ -394,6 +394,11 @@ class GatedLinearRecurrence(SequenceModel):
 # ----------------------------------------------------------------------------------
 # matrix-state cells
 # ----------------------------------------------------------------------------------
+def _norm_on_kernel(x):
+    """Rows the library's norm kernels take: on the device, a multiple of four features, at most 2048."""
+    return x.is_cuda and x.shape[-1] % 4 == 0 and x.shape[-1] <= _RMS_NORM_MAX_D
+
+
 class _RMSNorm(nn.Module):
     """y = x * rsqrt(mean(x^2) + eps) * scale (flax.linen.RMSNorm defaults, eps = 1e-6)."""
 
@@ -407,17 +412,14 @@ class _RMSNorm(nn.Module):
         the dtype its readers compute in (under autocast the dense layers behind a norm would each cast it
         again); rows it does not take (wider than 2048 features, a width that is no multiple of 4) and host
         arrays go to the array library."""
-        if self._on_kernel(x):
+        if _norm_on_kernel(x):
             return rms_norm(x, self.scale, self.eps, autocast_dtype(x) or x.dtype)
         return F.rms_norm(x.float(), (x.shape[-1],), self.scale.float(), self.eps).to(x.dtype)
-
-    def _on_kernel(self, x):
-        return x.is_cuda and x.shape[-1] % 4 == 0 and x.shape[-1] <= _RMS_NORM_MAX_D
 
     def fork(self, x):
         """(x, norm(x)) for a residual branch around this norm: with the first result used in place of x, the
         gradients of the two branches are added inside the norm's backward kernel."""
-        if self._on_kernel(x) and x.dtype in (torch.float32, torch.bfloat16):
+        if _norm_on_kernel(x) and x.dtype in (torch.float32, torch.bfloat16):
             return rms_norm_fork(x, self.scale, self.eps, autocast_dtype(x) or x.dtype)
         return x, self(x)
 
@@ -755,10 +757,25 @@ class mLSTM(Memoroid):
 # ----------------------------------------------------------------------------------
 # block composition used by the torso configuration (blocks/{stack,residual,normalization,ffn}.py)
 # ----------------------------------------------------------------------------------
+class _LayerNorm(nn.LayerNorm):
+    """torch.nn.LayerNorm (same parameters, same state dict) on the library's kernel where the rows fit it."""
+
+    def forward(self, x):
+        if _norm_on_kernel(x) and self.elementwise_affine:
+            return layer_norm(x, self.weight, self.bias, self.eps, autocast_dtype(x) or x.dtype)
+        return super().forward(x)
+
+    def fork(self, x):
+        """(x, norm(x)) for a residual branch around this norm (see _RMSNorm.fork)."""
+        if _norm_on_kernel(x) and self.elementwise_affine and x.dtype in (torch.float32, torch.bfloat16):
+            return layer_norm_fork(x, self.weight, self.bias, self.eps, autocast_dtype(x) or x.dtype)
+        return x, self(x)
+
+
 def LayerNorm(dim):
     """flax.linen.LayerNorm with its defaults: mean and variance over the last axis, eps = 1e-6,
     learned scale and bias -- the default norm of the reference's PreNorm / PostNorm."""
-    return nn.LayerNorm(dim, eps=1e-6)
+    return _LayerNorm(dim, eps=1e-6)
 
 
 RMSNorm = _RMSNorm

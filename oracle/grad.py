@@ -106,6 +106,15 @@ def silu_gate_grads(h, g, dy):
     return _np(h_.grad), _np(g_.grad)
 
 
+def layer_norm_grads(x, scale, bias, dy, eps=1e-6):
+    """(dx, dscale, dbias) of L = sum(dy * layer_norm(x, scale, bias))."""
+    x_, s_, b_ = _t(x, True), _t(scale, True), _t(bias, True)
+    xc = x_ - x_.mean(-1, keepdim=True)
+    y = xc * torch.rsqrt((xc * xc).mean(-1, keepdim=True) + eps) * s_ + b_
+    (y * _t(dy)).sum().backward()
+    return _np(x_.grad), _np(s_.grad), _np(b_.grad)
+
+
 def rms_norm_grads(x, scale, dy, eps=1e-6):
     """(dx, dscale) of L = sum(dy * rms_norm(x, scale)); scale None: (dx, None)."""
     x_ = _t(x, True)

@@ -497,6 +497,17 @@ def rms_norm(x, scale=None, eps=1e-6):
     return y if scale is None else y * np.asarray(scale, np.float64)
 
 
+def layer_norm(x, scale=None, bias=None, eps=1e-6):
+    """flax.linen.LayerNorm with its defaults over the last axis (the default norm of PreNorm / PostNorm,
+    blocks/normalization.py:10-65): (x - mean) * rsqrt(var + eps) * scale + bias, var the mean squared deviation."""
+    x = np.asarray(x, np.float64)
+    xc = x - x.mean(-1, keepdims=True)
+    y = xc / np.sqrt((xc * xc).mean(-1, keepdims=True) + eps)
+    if scale is not None:
+        y = y * np.asarray(scale, np.float64)
+    return y if bias is None else y + np.asarray(bias, np.float64)
+
+
 def mlstm_gates(log_i, log_f, done, m0=None, g_floor=-60.0):
     """The stabiliser of mlstm.py:190-206 unrolled over time, resets as memoroid.py:72-85 (the element wins by
     select): m_t = done_t ? log_i_t : max(m_{t-1} + log_f_t, log_i_t), and with it the log-decay and the key

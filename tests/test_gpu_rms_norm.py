@@ -1,6 +1,6 @@
-"""The RMS norm kernels (mrx_rms_norm_fwd / _bwd, through the C ABI) against the oracle: y of
-oracle.memoroid.rms_norm and the gradients of oracle.grad.rms_norm_grads (torch-fp64 autograd, pinned by
-closed forms and finite differences in tests/test_oracle_grad.py).  Tolerances: float32 arrays 1e-5 of the
+"""The norm kernels (mrx_rms_norm_fwd / _bwd, mrx_layer_norm_fwd / _bwd, through the C ABI) against the oracle: y of
+oracle.memoroid.rms_norm / layer_norm and the gradients of oracle.grad.rms_norm_grads / layer_norm_grads (torch-fp64
+autograd, pinned by closed forms and finite differences in tests/test_oracle_grad.py).  Tolerances: float32 arrays 1e-5 of the
 result's scale; bfloat16 arrays 2e-2 (one rounding of the stored result, 2^-9, and of the inputs read)."""
 import ctypes
 
@@ -184,6 +184,74 @@ def test_residual_around_a_pre_norm_block_adds_both_gradients_in_the_norm_kernel
     torch.testing.assert_close(x3.grad, g)
 
 
+@pytest.mark.parametrize("rows,D", [(1, 4), (7, 256), (1000, 260), (33, 512), (5, 1024), (3, 2048), (4099, 64), (16384, 256)])
+@pytest.mark.parametrize("x_dtype,y_dtype", [(torch.float32, torch.float32), (torch.float32, torch.bfloat16),
+                                             (torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32)])
+def test_layer_norm_forward_and_backward(rows, D, x_dtype, y_dtype):
+    from memorax_amd import kernels as K
+    rng = np.random.default_rng(7 * rows + D)
+    print(f"case layer norm rows={rows} D={D} x={x_dtype} y={y_dtype}", flush=True)
+    # rows with means of the order of their spread, scales over a decade
+    x, xr = _as((rng.standard_normal((rows, D)) + rng.standard_normal((rows, 1))) * np.exp(rng.standard_normal((rows, 1))), x_dtype)
+    sc = (1.0 + 0.3 * rng.standard_normal(D)).astype(np.float32)
+    bi = (0.2 * rng.standard_normal(D)).astype(np.float32)
+    dy, dyr = _as(rng.standard_normal((rows, D)), y_dtype)
+    add, addr = _as(rng.standard_normal((rows, D)), x_dtype)
+    y = K.layer_norm_fwd(x, dev(sc), dev(bi), 1e-6, y_dtype)
+    assert y.dtype == y_dtype and y.shape == x.shape
+    _close(y, M.layer_norm(xr, sc, bi, 1e-6), TOL[y_dtype], "y")
+    _close(K.layer_norm_fwd(x, None, None, 1e-6, y_dtype), M.layer_norm(xr, None, None, 1e-6), TOL[y_dtype], "y without parameters")
+    dx, dscale, dbias = K.layer_norm_bwd(x, dev(sc), dy, 1e-6, dx_add=add)
+    rdx, rds, rdb = G.layer_norm_grads(xr, sc.astype(np.float64), bi.astype(np.float64), dyr, 1e-6)
+    got = dx.float().cpu().numpy().astype(np.float64)
+    want = rdx + addr
+    err = (np.abs(got - want).max(-1) / (np.abs(want).max(-1) + 1e-30)).max()
+    # a bfloat16 row whose mean is several times its spread loses that factor in the centred values the kernel and the
+    # oracle both start from (the same rounded inputs), so the bound stays the dtype's own
+    assert err <= TOL[x_dtype], f"dx: {err:.3e}"
+    tol_p = 1e-5 * max(1.0, np.sqrt(rows) / 30)
+    _close(dscale, rds, tol_p, "dscale")
+    _close(dbias, rdb, tol_p, "dbias")
+    dx1, n1, n2 = K.layer_norm_bwd(x, dev(sc), dy, 1e-6, want_dparams=False)
+    assert n1 is None and n2 is None
+    err = (np.abs(dx1.float().cpu().numpy() - rdx).max(-1) / (np.abs(rdx).max(-1) + 1e-30)).max()
+    assert err <= TOL[x_dtype], f"dx alone: {err:.3e}"
+
+
+def test_layer_norm_module_pre_norm_residual_and_autocast():
+    """sequence_models.LayerNorm keeps torch.nn.LayerNorm's parameters and values; Residual(PreNorm(f)) with it takes
+    the forked route; values and gradients against torch's own layer norm in float64."""
+    from memorax_amd import sequence_models as sm
+    torch.manual_seed(1)
+    inner = sm.Projection(256, 256).cuda()
+    block = sm.Residual(sm.PreNorm(inner, 256)).cuda()      # the reference's default norm
+    norm = block.module.norm
+    assert isinstance(norm, torch.nn.LayerNorm) and sorted(n for n, _ in norm.named_parameters()) == ["bias", "weight"]
+    with torch.no_grad():
+        norm.weight.copy_(1 + 0.1 * torch.randn(256, device="cuda"))
+        norm.bias.copy_(0.1 * torch.randn(256, device="cuda"))
+    x = (torch.randn(6, 11, 256, device="cuda") + 0.5).requires_grad_()
+    g = torch.randn(6, 11, 256, device="cuda")
+    _, y = block(x)
+    y.backward(g)
+    xd = x.detach().double().requires_grad_()
+    wd, bd = norm.weight.detach().double().requires_grad_(), norm.bias.detach().double().requires_grad_()
+    yr = xd + torch.nn.functional.layer_norm(xd, (256,), wd, bd, 1e-6) @ inner.proj.weight.detach().double().T \
+        + inner.proj.bias.detach().double()
+    yr.backward(g.double())
+    torch.testing.assert_close(y.detach().double(), yr.detach(), rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(x.grad.double(), xd.grad, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(norm.weight.grad.double(), wd.grad, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(norm.bias.grad.double(), bd.grad, rtol=1e-4, atol=1e-4)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        assert norm(x.detach()).dtype == torch.bfloat16
+    # host arrays and widths the kernel does not take: torch's own layer norm
+    n6 = sm.LayerNorm(6)
+    x6 = torch.randn(5, 6)
+    torch.testing.assert_close(n6(x6), torch.nn.functional.layer_norm(x6, (6,), n6.weight, n6.bias, 1e-6))
+    torch.testing.assert_close(n6.cuda()(x6.cuda()).cpu(), n6.cpu()(x6), rtol=1e-5, atol=1e-6)
+
+
 def test_refusals():
     from memorax_amd import _lib
     lib = _lib.load()
@@ -204,4 +272,10 @@ def test_refusals():
     bwd = lambda ws, dsp=p(ds): lib.mrx_rms_norm_bwd(None, p(x), p(sc), p(y), None, p(dx), dsp, ws, 4, 256, 0, 0, 1e-6)   # noqa: E731
     assert bwd(None) == -1             # the scale's gradient needs the workspace
     assert bwd(None, None) == 0
+    db, ws = torch.empty(256, device="cuda"), torch.empty(2 * 1024 * 256, device="cuda")
+    lbwd = lambda dsp, dbp: lib.mrx_layer_norm_bwd(None, p(x), p(sc), p(y), None, p(dx), dsp, dbp, p(ws), 4, 256, 0, 0, 1e-6)   # noqa: E731
+    assert lbwd(p(ds), p(db)) == 0 and lbwd(None, None) == 0
+    assert lbwd(p(ds), None) == -1 and lbwd(None, p(db)) == -1     # the layer norm's parameter gradients come as a pair
+    assert lib.mrx_layer_norm_fwd(None, p(x), p(sc), None, p(y), 4, 256, 0, 0, 1e-6) == 0
+    assert lib.mrx_layer_norm_fwd(None, p(x), p(sc), ctypes.c_void_p(sc.data_ptr() + 4), p(y), 4, 252, 0, 0, 1e-6) == -1
     torch.cuda.synchronize()

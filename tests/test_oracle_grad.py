@@ -417,3 +417,28 @@ def test_silu_gate_closed_forms_and_grads_fd():
     np.testing.assert_allclose(dg, fd(lambda: (M.silu_gate(h, g) * dy).sum(), g), rtol=1e-6, atol=1e-8)
     s = 1 / (1 + np.exp(-g))
     np.testing.assert_allclose(dg, dy * h * s * (1 + g * (1 - s)), rtol=1e-10)
+
+
+def test_layer_norm_closed_forms_and_grads_fd():
+    """The layer norm's restatement: zero mean and unit mean square of every row without eps, invariance under
+    x -> a x + b (a > 0), agreement with the RMS norm on rows of zero mean, scipy's z-score; gradients against
+    central differences, dx orthogonal to the constant row and to x - mean (what the two invariances imply)."""
+    from scipy import stats
+    x, sc, bi, dy = rnd(3, 5, 8), rnd(8), rnd(8), rnd(3, 5, 8)
+    y = M.layer_norm(x, None, None, eps=0.0)
+    np.testing.assert_allclose(y.mean(-1), 0.0, atol=1e-14)
+    np.testing.assert_allclose((y * y).mean(-1), 1.0, rtol=1e-12)
+    np.testing.assert_allclose(y, stats.zscore(x, axis=-1), rtol=1e-12, atol=1e-13)
+    np.testing.assert_allclose(M.layer_norm(2.5 * x - 7.0, sc, bi, eps=0.0), M.layer_norm(x, sc, bi, eps=0.0), rtol=1e-10, atol=1e-12)
+    xz = x - x.mean(-1, keepdims=True)
+    np.testing.assert_allclose(M.layer_norm(xz, sc, None, 1e-6), M.rms_norm(xz, sc, 1e-6), rtol=1e-12, atol=1e-14)
+    for eps in (0.0, 1e-6, 0.3):
+        dx, ds, db = G.layer_norm_grads(x, sc, bi, dy, eps)
+        L = lambda: (M.layer_norm(x, sc, bi, eps) * dy).sum()   # noqa: E731
+        np.testing.assert_allclose(dx, fd(L, x), rtol=1e-6, atol=1e-8)
+        np.testing.assert_allclose(ds, fd(L, sc), rtol=1e-6, atol=1e-8)
+        np.testing.assert_allclose(db, fd(L, bi), rtol=1e-6, atol=1e-8)
+        np.testing.assert_allclose(db, dy.sum((0, 1)), rtol=1e-12)
+        np.testing.assert_allclose(dx.sum(-1), 0.0, atol=1e-12)
+    dx0, _, _ = G.layer_norm_grads(x, sc, bi, dy, 0.0)
+    np.testing.assert_allclose((dx0 * xz).sum(-1), 0.0, atol=1e-12)
