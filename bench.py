@@ -134,6 +134,7 @@ def main() -> int:
             secondary["step"] = bench_step(torch, K)
             secondary["rtrl"] = bench_rtrl(torch, K)
             secondary["mlstm"] = bench_mlstm(torch)
+            secondary["block"] = bench_block_kernels(torch, K)
         if not args.no_children:
             secondary["delta_rule_chunk64"] = bench_delta_chunk64()
         torch.cuda.empty_cache()
@@ -681,6 +682,55 @@ def bench_step(torch, K):
     ms = _time_ms(torch, lambda: K.delta_rule_fwd(q1, k1, v1, b1, d1, S, save_chk=False), iters=50, warm=5)
     res["chunk_kernel_at_T1_for_comparison"] = {"ms": ms}
     return res
+
+
+def bench_block_kernels(torch, K):
+    """The passes of a torso block around its recurrence, at configuration 5's size (131 072 rows of 256 features):
+    the norms as a pre-norm block under bf16 autocast calls them (float32 residual stream in, bfloat16 out; the
+    backward with the residual branch's gradient added), the read-out norm on bfloat16 rows, the gating product, and
+    the array library's own operations for the same work beside them.  Bytes = every operand once."""
+    rows, D = 1024 * 128, 256
+    bf = torch.bfloat16
+    x = torch.randn(rows, D, device="cuda")
+    xb, gb, hb = (torch.randn(rows, D, device="cuda").to(bf) for _ in range(3))
+    add = torch.randn(rows, D, device="cuda")
+    sc, bi = torch.ones(D, device="cuda"), torch.zeros(D, device="cuda")
+    n32, n16 = rows * D * 4, rows * D * 2
+    out = {}
+
+    def put(name, fn, nbytes):
+        ms = _time_ms(torch, fn, iters=20, warm=3)
+        out[name] = {"ms": ms, "GB/s": nbytes / ms / 1e6, "frac_hbm": nbytes / ms / 1e6 / HBM_PEAK_GBS}
+    put("rms_norm_fwd_f32_to_bf16", lambda: K.rms_norm_fwd(x, sc, 1e-6, bf), n32 + n16)
+    put("rms_norm_bwd_f32_with_residual_gradient", lambda: K.rms_norm_bwd(x, sc, gb, 1e-6, dx_add=add), 3 * n32 + n16)
+    put("rms_norm_fwd_bf16", lambda: K.rms_norm_fwd(xb, sc), 2 * n16)
+    put("rms_norm_bwd_bf16", lambda: K.rms_norm_bwd(xb, sc, gb), 3 * n16)
+    put("layer_norm_fwd_f32_to_bf16", lambda: K.layer_norm_fwd(x, sc, bi, 1e-6, bf), n32 + n16)
+    put("layer_norm_bwd_f32_with_residual_gradient", lambda: K.layer_norm_bwd(x, sc, gb, 1e-6, dx_add=add), 3 * n32 + n16)
+    put("silu_gate_fwd_bf16", lambda: K.silu_gate_fwd(hb, gb), 3 * n16)
+    put("silu_gate_bwd_bf16", lambda: K.silu_gate_bwd(hb, gb, xb), 5 * n16)
+    # the array library on the same work: its fused norm kernels plus the cast and the addition around them
+    F = torch.nn.functional
+    xr = x.clone().requires_grad_()
+    scr = sc.clone().requires_grad_()
+
+    def lib_norm():
+        xr.grad = scr.grad = None
+        y = F.rms_norm(xr, (D,), scr, 1e-6).to(bf)
+        y.backward(gb)
+        return xr.grad + add
+    ms = _time_ms(torch, lib_norm, iters=10, warm=2)
+    mine = out["rms_norm_fwd_f32_to_bf16"]["ms"] + out["rms_norm_bwd_f32_with_residual_gradient"]["ms"]
+    out["array_library_rms_norm_cast_backward_add"] = {"ms": ms, "over_the_kernels": ms / mine}
+    hr, gr = hb.clone().requires_grad_(), gb.clone().requires_grad_()
+
+    def lib_gate():
+        hr.grad = gr.grad = None
+        (hr * F.silu(gr)).backward(xb)
+    ms = _time_ms(torch, lib_gate, iters=10, warm=2)
+    mine = out["silu_gate_fwd_bf16"]["ms"] + out["silu_gate_bwd_bf16"]["ms"]
+    out["array_library_gating_forward_backward"] = {"ms": ms, "over_the_kernels": ms / mine}
+    return out
 
 
 def bench_torso_kernels(torch, K):

@@ -277,6 +277,9 @@ template <bool CENTER> int norm_fwd(const FwdCall &a, int x_dtype, int y_dtype)
     return y_dtype == MRX_F32 ? fwd_by_width<__bf16, float, CENTER>(a) : fwd_by_width<__bf16, __bf16, CENTER>(a);
 }
 
+// Rows a wave of the backward kernel has in flight, by the 256-column groups a lane holds.
+constexpr int bwd_rows_in_flight(int nv) { return nv <= 2 ? 2 : 1; }   // four at the narrowest width measured level
+
 struct BwdCall {
     hipStream_t st;
     const void *x;
@@ -292,7 +295,7 @@ struct BwdCall {
 
 template <typename XT, typename GT, int NV, bool CENTER> int launch_bwd(const BwdCall &a)
 {
-    constexpr int RPI = NV <= 2 ? 2 : 1;
+    constexpr int RPI = bwd_rows_in_flight(NV);
     return launch_kernel(norm_bwd_kernel<XT, GT, NV, RPI, CENTER>, dim3(a.grid), dim3(RN_THREADS), 0, a.st, static_cast<const XT *>(a.x),
                          a.scale, static_cast<const GT *>(a.dy), static_cast<const XT *>(a.dx_add), static_cast<XT *>(a.dx),
                          (a.dscale || a.dbias) ? a.workspace : nullptr, a.rows, a.D, a.eps, 1.f / (float)a.D);
@@ -316,7 +319,7 @@ template <bool CENTER> int norm_bwd(BwdCall a, int x_dtype, int dy_dtype)
     if (CENTER && (a.dscale == nullptr) != (a.dbias == nullptr)) return MRX_ERR_INVALID_ARG;
     if ((a.dscale || a.dbias) && !a.workspace) return MRX_ERR_INVALID_ARG;
     if (const int rc = prepare_device(); rc != MRX_OK) return rc;
-    a.grid = grid_for(a.rows, a.D <= 512 ? 2 : 1, MRX_RMS_NORM_PARTS);
+    a.grid = grid_for(a.rows, bwd_rows_in_flight((a.D + 255) / 256), MRX_RMS_NORM_PARTS);
     int rc;
     if (x_dtype == MRX_F32)
         rc = dy_dtype == MRX_F32 ? bwd_by_width<float, float, CENTER>(a) : bwd_by_width<float, __bf16, CENTER>(a);
