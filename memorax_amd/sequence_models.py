@@ -848,6 +848,12 @@ class GatedResidual(nn.Module):
         return self.module.initialize_carry(key, input_shape)
 
 
+def gelu(x):
+    """flax.linen.gelu as the reference's blocks call it (blocks/ffn.py:16,86): the tanh approximation, which is
+    jax.nn.gelu's default -- not the error-function form that is the array library's."""
+    return F.gelu(x, approximate="tanh")
+
+
 class _Stateless(nn.Module):
     """Blocks without a recurrence (blocks/base.py:6-21): the carry is None on the way in and out."""
 
@@ -858,7 +864,7 @@ class _Stateless(nn.Module):
 class FFN(_Stateless):
     """ffn.py:11-50: Dense -> activation -> dropout -> Dense, hidden width features * expansion_factor."""
 
-    def __init__(self, features, expansion_factor=4, activation=F.gelu, dropout_rate=0.0):
+    def __init__(self, features, expansion_factor=4, activation=gelu, dropout_rate=0.0):
         super().__init__()
         self.up = Dense(features, features * expansion_factor)
         self.down = Dense(features * expansion_factor, features)
@@ -883,7 +889,7 @@ class GLU(_Stateless):
     """ffn.py:82-123: up_proj to 2 * hidden, split into (gate, value) in that order,
     activation(gate) * value, dropout, down_proj; no biases by default."""
 
-    def __init__(self, features, expansion_factor=4, activation=F.gelu, dropout_rate=0.0, use_bias=False):
+    def __init__(self, features, expansion_factor=4, activation=gelu, dropout_rate=0.0, use_bias=False):
         super().__init__()
         hidden = features * expansion_factor
         self.up_proj = Dense(features, 2 * hidden, bias=use_bias)

@@ -16,7 +16,9 @@ def test_glu_splits_gate_then_value():
     x = _x()
     carry, y = m(x, done=None, initial_carry=None)
     u = x @ m.up_proj.weight.T
-    want = (F.gelu(u[..., :16]) * u[..., 16:]) @ m.down_proj.weight.T   # ffn.py:108-121
+    g = u[..., :16]
+    tanh_gelu = 0.5 * g * (1 + torch.tanh((2 / torch.pi) ** 0.5 * (g + 0.044715 * g ** 3)))   # jax.nn.gelu's default form
+    want = (tanh_gelu * u[..., 16:]) @ m.down_proj.weight.T   # ffn.py:108-121
     assert carry is None and m.up_proj.bias is None and m.down_proj.bias is None
     assert torch.allclose(y, want, atol=1e-12)
     assert m.initialize_carry(None, (3, 8)) is None
