@@ -17,8 +17,6 @@ import torch.nn.functional as F
 
 _SLICE_ROWS = 2048   # rows per slice of the weight-gradient product
 _MAX_SLICES = 128
-
-
 _HALVES = (torch.bfloat16, torch.float16)
 
 
@@ -127,8 +125,8 @@ def dense_group(x, layers):
 
 def dense(x, weight, bias=None):
     """x W^T + b like torch.nn.functional.linear (autocast included), with the weight gradient as a
-    sliced product (module docstring).  Gradients of weight and bias are formed in float32 when the operands are 16-bit and
-    cast to the parameters' dtype by the array library."""
+    sliced product (module docstring).  Gradients of weight and bias are formed in float32 when the
+    operands are 16-bit and cast to the parameters' dtype by the array library."""
     return _Dense.apply(x, weight, bias)
 
 
