@@ -409,7 +409,9 @@ int mrx_mingru_scan_fwd(void *stream, const void *z, const void *h_tilde, const 
                         const void *h0, const void *P0, void *h, void *h_last, void *P_last,
                         int64_t B, int64_t T, int64_t D, int dtype, int done_dtype);
 
-/* h: the states the forward call wrote.  dz, dh_tilde: gradients with respect to the projections. */
+/* h: the states the forward call wrote (all of them, although a large call -- more than 600 MB through it --
+ * reads only one row in eight and forms the others again from z and h_tilde).  dz, dh_tilde: gradients with
+ * respect to the projections. */
 int mrx_mingru_scan_bwd(void *stream, const void *z, const void *h_tilde, const void *h,
                         const void *done, const void *h0, const void *g, const void *g_last,
                         void *dz, void *dh_tilde, void *dh0, int64_t B, int64_t T, int64_t D,

@@ -733,7 +733,13 @@ diag_scan_last_kernel(const E *__restrict__ a, const E *__restrict__ b, const vo
 }
 
 // MG: a holds z, hx holds x = h~ (a fourth load per step); da receives dz and db receives dx.
-template <typename E, int VEC, int SG, bool MG = false, typename S = E, bool DF = false>
+// RECOMP (with MG): the kernel has what the forward pass had, so it reads only one row of h per group of SG
+// steps -- the state entering the group -- and runs the recurrence forward through the group again for the
+// states between: SG - 1 of SG rows of h not fetched (24 -> 20.5 bytes per element and step in float32) for the
+// map's arithmetic a second time.  That pays where the call is bound by HBM and costs where its arrays fit the
+// last-level cache (float32, 1024 x 128 x 256: 157 -> 138 us; 256 x 128 x 256: 46 -> 49 us; bfloat16 arrays,
+// 1024 x 128 x 256: 80 -> 90 us, 512 x 1024 x 1024: 1.30 -> 1.19 ms): launch_bwd asks for it by the bytes moved.
+template <typename E, int VEC, int SG, bool MG = false, typename S = E, bool DF = false, bool RECOMP = false>
 __global__ void __launch_bounds__(256)
 diag_scan_bwd_stream_kernel(const S *__restrict__ a, const S *__restrict__ hx, const S *__restrict__ hfw,
                             const void *__restrict__ done, int,
@@ -758,7 +764,9 @@ diag_scan_bwd_stream_kernel(const S *__restrict__ a, const S *__restrict__ hx, c
 
     // step r (reversed index), t = T-1-r: needs g_t, a_t (for the carry to t-1), h_{t-1}, done_t
     using R = raw_t<S, VEC>;  // prefetched values stay as stored until they are consumed
-    R xg[SG], xa[SG], xh[SG], ng[SG], na[SG], nh[SG];
+    static_assert(!RECOMP || MG, "the states can be formed again only where the map's inputs are at hand");
+    constexpr int NH = RECOMP ? 1 : SG;  // rows of h per group
+    R xg[SG], xa[SG], xh[NH], ng[SG], na[SG], nh[NH];
     R xx[MG ? SG : 1], nx[MG ? SG : 1];
     uint32_t xd[SG], nd[SG];
     V h0v = vfill<E, VEC>(O::zero());  // h_{-1}: what step 0 multiplies its lam with
@@ -773,14 +781,40 @@ diag_scan_bwd_stream_kernel(const S *__restrict__ a, const S *__restrict__ hx, c
                 pg[s] = ldraw<S, VEC>(g + off);
                 pa[s] = ldraw<S, VEC>(a + (a_ti ? col : off));
                 if constexpr (MG) px[s] = ldraw<S, VEC>(hx + off);
-                if (t > 0) ph[s] = ldraw<S, VEC>(hfw + off - D);
+                if constexpr (!RECOMP) {
+                    if (t > 0) ph[s] = ldraw<S, VEC>(hfw + off - D);
+                }
                 pd[s] = done_raw(done, done_f32, row0 + t);
             }
+        }
+        if constexpr (RECOMP) {  // the state entering the group's earliest step
+            const int t_lo = T - r0 - SG;
+            if (t_lo > 0) ph[0] = ldraw<S, VEC>(hfw + (row0 + t_lo - 1) * D + col);
         }
     };
     load(0, xg, xa, xh, xx, xd);
     for (int r0 = 0; r0 < T; r0 += SG) {
         if (r0 + SG < T) load(r0 + SG, ng, na, nh, nx, nd);
+        V hprev[RECOMP ? SG : 1];  // h_{t-1} of the group's steps, by the recurrence from the state entering the group
+        if constexpr (RECOMP) {
+            V hc = h0v;
+            if (T - r0 - SG > 0) hc = cvtv<S, E, VEC>(xh[0]);
+#pragma unroll
+            for (int s = SG - 1; s >= 0; --s) {  // forward in time
+                const int t = T - 1 - (r0 + s);
+                if (t >= 0) {
+                    hprev[s] = hc;
+                    const bool dn = done_test(xd[s], done_f32);
+                    const V va = cvtv<S, E, VEC>(xa[s]), vx = cvtv<S, E, VEC>(xx[s]);
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) {
+                        float ca = va.v[i], cb = vx.v[i];
+                        MinGru::coeffs(ca, cb);
+                        hc.v[i] = dn ? cb : O::madd(ca, hc.v[i], cb);
+                    }
+                }
+            }
+        }
 #pragma unroll
         for (int s = 0; s < SG; ++s) {
             const int t = T - 1 - (r0 + s);
@@ -789,8 +823,12 @@ diag_scan_bwd_stream_kernel(const S *__restrict__ a, const S *__restrict__ hx, c
                 const int64_t off = (row0 + t) * D + col;
                 const V vg = cvtv<S, E, VEC>(xg[s]), va = cvtv<S, E, VEC>(xa[s]);
                 V vh = h0v, vx;
-                if (t > 0) vh = cvtv<S, E, VEC>(xh[s]);
                 if constexpr (MG) vx = cvtv<S, E, VEC>(xx[s]);
+                if constexpr (RECOMP) {
+                    vh = hprev[s];
+                } else {
+                    if (t > 0) vh = cvtv<S, E, VEC>(xh[s]);
+                }
                 V l, o;
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) {
@@ -819,7 +857,9 @@ diag_scan_bwd_stream_kernel(const S *__restrict__ a, const S *__restrict__ hx, c
             }
         }
 #pragma unroll
-        for (int s = 0; s < SG; ++s) { xg[s] = ng[s]; xa[s] = na[s]; xh[s] = nh[s]; xd[s] = nd[s]; }
+        for (int s = 0; s < SG; ++s) { xg[s] = ng[s]; xa[s] = na[s]; xd[s] = nd[s]; }
+#pragma unroll
+        for (int s = 0; s < NH; ++s) xh[s] = nh[s];
         if constexpr (MG) {
 #pragma unroll
             for (int s = 0; s < SG; ++s) xx[s] = nx[s];
@@ -1057,14 +1097,25 @@ int launch_bwd(hipStream_t st, const void *a, const void *hx, const void *h, con
         const dim3 grid((unsigned)((B * cpr + 255) / 256)), block(256);
         vec_switch<E>(pl.vec, [&](auto vc) {
             constexpr int VEC = decltype(vc)::value;
-            auto go = [&](auto df) {
-                rc = launch_kernel((diag_scan_bwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8), MG, S, decltype(df)::value>),
+            auto go = [&](auto df, auto rcmp) {
+                rc = launch_kernel((diag_scan_bwd_stream_kernel<E, VEC, (VEC * sizeof(E) == 16 ? 4 : 8), MG, S, decltype(df)::value,
+                                                                decltype(rcmp)::value>),
                                    grid, block, 0, st, (const S *)a, (const S *)hx, (const S *)h, done, done_f32,
                                    (const E *)h0, (const S *)g, (const E *)g_last, (S *)da, (S *)db, (E *)dh0, B, (int)T, D,
                                    cpr, a_ti, da_sum);
             };
-            if (done_f32) go(std::true_type{});
-            else go(std::false_type{});
+            // six (B,T,D) arrays pass through the call: more than twice the 256 MB of last-level cache, and the
+            // call is bound by HBM -- then h is better formed again than fetched
+            const bool recompute = MG && 6.0 * (double)B * (double)T * (double)D * sizeof(S) >= 600e6;
+            if constexpr (MG) {
+                if (recompute) {
+                    if (done_f32) go(std::true_type{}, std::true_type{});
+                    else go(std::false_type{}, std::true_type{});
+                    return;
+                }
+            }
+            if (done_f32) go(std::true_type{}, std::false_type{});
+            else go(std::false_type{}, std::false_type{});
         });
     } else {
         const dim3 grid((unsigned)(B * pl.tiles)), block(64 * pl.nw);

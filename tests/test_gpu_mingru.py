@@ -16,6 +16,7 @@ SHAPES = [
     (64, 64, 1024),   # streaming kernels, 16-byte vectors
     (40, 50, 516),    # D a multiple of 4 but not of 64: a partly filled last tile
     (2, 1000, 8),
+    (1536, 131, 128),  # a call that moves over 600 MB: the streaming backward forms h again inside its groups of steps
 ]
 
 
@@ -53,6 +54,9 @@ def test_mingru_scan_fwd_bwd(shape, p):
     rdz = s * (1 - s) * (np.where(x64 >= 0, x64 + 0.5, M.sigmoid(x64)) * lam - da)
     rdx = lam * s * np.where(x64 >= 0, 1.0, M.sigmoid(x64) * (1 - M.sigmoid(x64)))
     assert relerr(dz, rdz) <= TOL and relerr(dx, rdx) <= TOL and relerr(dh0, rdh0) <= TOL
+    if B * T * D > 1 << 24:   # the large call once more with float32 flags: the same kernel on the other flag type
+        dz2, dx2, dh02 = K.mingru_scan_bwd(dev(z), dev(x), h, dev(done.astype(np.float32)), dev(h0), dev(g), dev(gl))
+        assert torch.equal(dz2, dz) and torch.equal(dx2, dx) and torch.equal(dh02, dh0)
 
 
 def test_mingru_autograd_function_against_the_log_space_autograd_oracle():
@@ -135,7 +139,8 @@ def test_mingru_cell_fused_and_unfused_agree_and_match_the_reference_route():
     assert relerr(y, rh) <= TOL and relerr(carry[0], nxt[0]) <= TOL and relerr(carry[1], nxt[1]) <= TOL
 
 
-@pytest.mark.parametrize("shape", [(2, 1, 5), (3, 77, 48), (4, 300, 258), (64, 128, 256), (16, 1000, 130), (512, 128, 64)])
+@pytest.mark.parametrize("shape", [(2, 1, 5), (3, 77, 48), (4, 300, 258), (64, 128, 256), (16, 1000, 130), (512, 128, 64),
+                                   (3072, 131, 128)])   # the last: over 600 MB moved, h formed again in the backward
 @pytest.mark.parametrize("p", [0.0, 0.05])
 def test_bfloat16_arrays_float32_arithmetic(shape, p):
     """z, h~, h, g, dz, dh~ in bfloat16, arithmetic and carries in float32: against the oracle on the rounded
