@@ -119,7 +119,8 @@ class _DenseGroup(torch.autograd.Function):
 
 
 def dense_group(x, layers):
-    """The outputs of several Dense / torch.nn.Linear layers that read the same input, as a tuple."""
+    """The outputs of several Dense / torch.nn.Linear layers that read the same input, as a tuple.
+    The layers lend their parameters; their own ``forward`` (and hooks registered on it) does not run."""
     return _DenseGroup.apply(x, len(layers), *[m.weight for m in layers], *[m.bias for m in layers])
 
 
