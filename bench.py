@@ -682,7 +682,34 @@ def bench_step(torch, K):
         beta[:, None].contiguous(), dn[:, None].contiguous()
     ms = _time_ms(torch, lambda: K.delta_rule_fwd(q1, k1, v1, b1, d1, S, save_chk=False), iters=50, warm=5)
     res["chunk_kernel_at_T1_for_comparison"] = {"ms": ms}
+    res["torso_acting_step_1024_envs"] = bench_acting_step(torch)
     return res
+
+
+def bench_acting_step(torch):
+    """One acting step (T = 1, no gradients, bf16 autocast) of configuration 5's torso through the host mirror for
+    1024 environments: issued kernel by kernel from the host, and replayed as one HIP graph
+    (memorax_amd.rollout.GraphedStep)."""
+    from memorax_amd import sequence_models as sm
+    from memorax_amd.rollout import GraphedStep
+    B, Fe, H, d = 1024, 256, 4, 64
+    torch.manual_seed(5)
+    blocks = []
+    for _ in range(4):
+        blocks += [sm.Residual(sm.PreNorm(sm.Memoroid(sm.DeltaNetCell(Fe, d, H)), Fe, norm=sm.RMSNorm)),
+                   sm.Residual(sm.PreNorm(sm.GatedLinearRecurrence(Fe), Fe, norm=sm.RMSNorm))]
+    torso = sm.Stack(blocks).cuda()
+    x = torch.randn(B, 1, Fe, device="cuda")
+    done = torch.rand(B, 1, device="cuda") < 0.01
+    state = {"carry": torso.initialize_carry(None, (B, Fe))}
+
+    def eager():
+        with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+            state["carry"], _ = torso(x, done, state["carry"])
+    ms_e = _time_ms(torch, eager, iters=30, warm=5)
+    act = GraphedStep(torso, B, Fe, autocast=torch.bfloat16)
+    ms_g = _time_ms(torch, lambda: act(x, done), iters=100, warm=5)
+    return {"ms_issued_from_the_host": ms_e, "ms_as_a_graph": ms_g, "env_steps/s_as_a_graph": B / ms_g * 1e3}
 
 
 def bench_block_kernels(torch, K):
