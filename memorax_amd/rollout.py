@@ -36,7 +36,8 @@ def _leaves(tree, out):
 
 def _map(fn, tree):
     if isinstance(tree, (tuple, list)):
-        return type(tree)(_map(fn, v) for v in tree) if not hasattr(tree, "_fields") else type(tree)(*(_map(fn, v) for v in tree))
+        items = [_map(fn, v) for v in tree]
+        return type(tree)(*items) if hasattr(tree, "_fields") else type(tree)(items)   # named tuples keep their type
     if isinstance(tree, dict):
         return {k: _map(fn, v) for k, v in tree.items()}
     return None if tree is None else fn(tree)
@@ -69,10 +70,12 @@ class GraphedStep:
         self._graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self._graph):
             self._next, self._y = self._run()
-        self._pairs = list(zip(_leaves(self._carry, []), _leaves(self._next, [])))
-        for dst, _ in self._pairs:
-            if not dst.is_cuda:
-                raise ValueError("the model's carry must live on the device")
+        held, made = _leaves(self._carry, []), _leaves(self._next, [])
+        if len(held) != len(made) or any(a.shape != b.shape for a, b in zip(held, made)):
+            raise ValueError("the step's next carry does not have the leaves of the carry it was given")
+        if not all(t.is_cuda for t in held):
+            raise ValueError("the model's carry must live on the device")
+        self._pairs = list(zip(held, made))
         self.reset()
 
     def _run(self):
@@ -96,7 +99,10 @@ class GraphedStep:
         return _map(lambda t: t.clone(), self._carry)
 
     def set_carry(self, carry):
-        for dst, src in zip(_leaves(self._carry, []), _leaves(carry, [])):
+        held, given = _leaves(self._carry, []), _leaves(carry, [])
+        if len(held) != len(given):
+            raise ValueError(f"a carry of {len(given)} leaves for a model whose carry has {len(held)}")
+        for dst, src in zip(held, given):
             dst.copy_(src)
 
     def reset(self):
