@@ -79,7 +79,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--all", action="store_true",
-                    help="also time the whole torso with its dense layers, the single-step kernels and the RTRL scan")
+                    help="also time the single-step kernels and the acting step, the RTRL scan, the mLSTM cell and the "
+                         "block kernels")
     ap.add_argument("--headline-only", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--ramp-ms", type=float, default=CLOCK_RAMP_S * 1e3,
                     help="untimed load before the warm-up steps (0 under a counter-collecting profiler)")
@@ -129,8 +130,8 @@ def main() -> int:
         secondary["scan"] = bench_scan(torch, K)
         secondary["linear_attention"] = bench_linear_attention(torch, K, np, dev)
         secondary["torso"] = bench_torso_kernels(torch, K)
+        secondary["torso"].update(bench_torso_full(torch, K))
         if args.all:
-            secondary["torso"].update(bench_torso_full(torch, K))
             secondary["step"] = bench_step(torch, K)
             secondary["rtrl"] = bench_rtrl(torch, K)
             secondary["mlstm"] = bench_mlstm(torch)
