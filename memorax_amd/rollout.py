@@ -14,6 +14,12 @@ the same results bit for bit, one launch.
 
 Everything the step does must be capturable: no host synchronisation, no data-dependent shapes.  The
 modules of ``sequence_models`` are; the library's kernels take the capturing stream like any other.
+
+Under autocast every dense layer casts its weight on every call -- in a step of 0.7 ms that is a seventh
+of the device's time, for weights that change once per update.  The graph therefore runs on copies of the
+matrices in the autocast dtype, which a call refreshes only for parameters that have been written since
+(``torch.Tensor._version``, which optimisers and ``load_state_dict`` advance; ``sync_weights()`` after
+anything that writes through ``.data``).
 """
 from __future__ import annotations
 
@@ -54,6 +60,14 @@ class GraphedStep:
 
     def __init__(self, model, batch, features, autocast=None, device="cuda", warmup=3):
         self.model, self.autocast = model, autocast
+        # matrices in the dtype the products run in; vectors (norm scales, biases) stay as they are
+        self._shadow, self._seen = {}, {}
+        if autocast is not None:
+            for name, p in model.named_parameters():
+                if p.dim() >= 2 and p.is_floating_point():
+                    self._shadow[name] = p.detach().to(autocast)
+                    self._seen[name] = p._version
+        self._params = dict(model.named_parameters())
         self._x = torch.zeros(batch, 1, features, device=device)
         self._done = torch.zeros(batch, 1, dtype=torch.bool, device=device)
         with torch.no_grad():
@@ -81,11 +95,24 @@ class GraphedStep:
     def _run(self):
         ctx = torch.autocast("cuda", dtype=self.autocast) if self.autocast is not None else contextlib.nullcontext()
         with torch.no_grad(), ctx:
+            if self._shadow:
+                return torch.func.functional_call(self.model, self._shadow, (self._x, self._done, self._carry))
             return self.model(self._x, self._done, self._carry)
+
+    def sync_weights(self, force=True):
+        """Refresh the graph's copies of the weight matrices: all of them, or (force=False) those written since
+        the last refresh."""
+        with torch.no_grad():
+            for name, copy in self._shadow.items():
+                p = self._params[name]
+                if force or p._version != self._seen[name]:
+                    copy.copy_(p)
+                    self._seen[name] = p._version
 
     def __call__(self, inputs, done):
         """inputs (B,1,F), done (B,1) bool or float -> y (B,1,...), a buffer of this object that the next call
         overwrites."""
+        self.sync_weights(force=False)
         self._x.copy_(inputs)
         self._done.copy_(done != 0 if done.dtype != torch.bool else done)
         self._graph.replay()

@@ -62,3 +62,12 @@ def test_graphed_step_equals_the_eager_step(autocast):
     y = act(xs[1], ds[1])
     _, y_ref = eager(xs[1], ds[1], mid)
     assert torch.equal(y, y_ref)
+    # weights written after the capture (an optimiser step) reach the graph's copies with the next call
+    with torch.no_grad():
+        for p in torso.parameters():
+            p.add_(0.01 * torch.randn_like(p))
+    act.set_carry(mid)
+    y = act(xs[1], ds[1])
+    _, y_ref = eager(xs[1], ds[1], mid)
+    assert torch.equal(y, y_ref)
+
