@@ -104,6 +104,9 @@ step_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restric
         f32x4 z4 = (z_in && cin) ? *reinterpret_cast<const f32x4 *>(z_in + bh * dkw + 4 * c4) : zero4;
         if (reset) z4 = zero4;
         z4 += k4;
+        // updated in place, z_out is z_in: every row's lanes must hold the carried z before row 0 overwrites it
+        // (a row that read it afterwards would add k a second time and divide by the wrong normaliser)
+        __syncthreads();
         if (r0 == 0 && cin) *reinterpret_cast<f32x4 *>(z_out + bh * dkw + 4 * c4) = z4;
         den = fmaxf(reduce_row(dot4(z4, q4)), eps);
     }

@@ -14,11 +14,33 @@ bool or float where nonzero clears the carry before step t (memoroid.py:60-91).
 """
 from __future__ import annotations
 
+import contextlib
 import functools
 
 import torch
 
 from . import kernels as K
+
+_step_in_place = False
+
+
+@contextlib.contextmanager
+def step_in_place():
+    """Inside this context the acting paths (one time step, no gradients) update the carried state where it
+    lies instead of writing a new array: the state handed in is overwritten and handed back.  For a caller that
+    owns the carry's buffers (rollout.GraphedStep); elsewhere the carry a caller passes stays untouched."""
+    global _step_in_place
+    before, _step_in_place = _step_in_place, True
+    try:
+        yield
+    finally:
+        _step_in_place = before
+
+
+def _own(given, used):
+    """inplace for a step kernel: only on the caller's own array (a converted copy is a new array already)."""
+    return _step_in_place and given is not None and used is given
+
 
 _FMAP = {None: 0, "none": 0, 0: 0, "elu1": 1, 1: 1}
 _FMAP_NAME = {0: "none", 1: "elu1"}
@@ -248,7 +270,7 @@ class _LinearAttention(torch.autograd.Function):
         need = any(ctx.needs_input_grad)
         if q_.shape[1] == 1 and not need:  # acting: one step, no residuals (memoroid.py:93-109 with T = 1)
             o, S_last, _ = K.linear_attn_step(q_[:, 0], k_[:, 0], v_[:, 0], done[:, 0], S0_,
-                                              feature_map=_FMAP_NAME[fmap])
+                                              feature_map=_FMAP_NAME[fmap], inplace=_own(S0, S0_))
             ctx.done, ctx.fmap, ctx.has_S0 = done, fmap, S0 is not None
             return o[:, None], S_last
         o, S_last, chk = K.linear_attn_fwd(q_, k_, v_, done, S0_, fmap, save_chk=need)
@@ -288,7 +310,8 @@ class _NormalisedLinearAttention(torch.autograd.Function):
         ctx.done, ctx.fmap, ctx.eps, ctx.has_0 = done, fmap, eps, (S0 is not None, z0 is not None)
         if q_.shape[1] == 1 and not need:  # acting: one fused step
             o, S_last, z_last = K.linear_attn_step(q_[:, 0], k_[:, 0], v_[:, 0], done[:, 0], S0_, z0_,
-                                                   feature_map=_FMAP_NAME[fmap], normalise=True, eps=eps)
+                                                   feature_map=_FMAP_NAME[fmap], normalise=True, eps=eps,
+                                                   inplace=_own(S0, S0_) and _own(z0, z0_))
             ss = o.float().square().sum(-1)[..., None] if want_ss else None   # (B,H,1)
             return o[:, None], S_last, z_last, ss
         o, den, S_last, z_last, chk, ss = K.linear_attn_norm_fwd(q_, k_, v_, done, S0_, z0_, fmap, eps, save_chk=need,
@@ -342,7 +365,7 @@ class _GatedLinearAttention(torch.autograd.Function):
         need = any(ctx.needs_input_grad)
         if q_.shape[1] == 1 and not need:  # acting: one step, no residuals (memoroid.py:93-109 with T = 1)
             o, S_last = K.gated_linear_attn_step(q_[:, 0], k_[:, 0], v_[:, 0], g_[:, 0], done[:, 0], S0_,
-                                                 feature_map=_FMAP_NAME[fmap])
+                                                 feature_map=_FMAP_NAME[fmap], inplace=_own(S0, S0_))
             ctx.done, ctx.fmap, ctx.has_S0 = done, fmap, S0 is not None
             return o[:, None], S_last
         o, S_last, S_chk = K.gated_linear_attn_fwd(q_, k_, v_, g_, done, S0_, fmap, save_chk=need)
@@ -386,7 +409,7 @@ class _DeltaRule(torch.autograd.Function):
             if prologue:  # a (B,H,d) array: the prologue as array ops costs nothing here
                 k1 = torch.nn.functional.normalize(k1.float(), dim=-1).to(k_.dtype)
                 b1 = torch.sigmoid(b1.float()).to(b_.dtype)
-            o, S_last = K.delta_rule_step(q_[:, 0], k1, v_[:, 0], b1, done[:, 0], S0_)
+            o, S_last = K.delta_rule_step(q_[:, 0], k1, v_[:, 0], b1, done[:, 0], S0_, inplace=_own(S0, S0_))
             return o[:, None], S_last
         o, S_last, chk = K.delta_rule_fwd(q_, k_, v_, b_, done, S0_, save_chk=need, prologue=prologue, reset_path=resets)
         if need:

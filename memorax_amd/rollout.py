@@ -27,6 +27,8 @@ import contextlib
 
 import torch
 
+from .functional import step_in_place
+
 
 def _leaves(tree, out):
     if isinstance(tree, (tuple, list)):
@@ -55,7 +57,8 @@ class GraphedStep:
     model: a SequenceModel (``(inputs, done, initial_carry) -> (next_carry, y)``, ``initialize_carry``).
     autocast: dtype of a ``torch.autocast`` region around the step, or None.
     The carry lives in buffers of this object: ``reset()`` puts the model's initial carry there, ``set_carry``
-    a given one; after every call the step's next carry is copied over them.
+    a given one; the matrix states are updated in them by the step kernels, every other leaf of the step's next
+    carry is copied over them after the call.
     """
 
     def __init__(self, model, batch, features, autocast=None, device="cuda", warmup=3):
@@ -89,12 +92,15 @@ class GraphedStep:
             raise ValueError("the step's next carry does not have the leaves of the carry it was given")
         if not all(t.is_cuda for t in held):
             raise ValueError("the model's carry must live on the device")
-        self._pairs = list(zip(held, made))
+        # leaves the step has updated in place need no copy back
+        same = lambda a, b: a.data_ptr() == b.data_ptr() and a.stride() == b.stride() and a.dtype == b.dtype   # noqa: E731
+        self._pairs = [(a, b) for a, b in zip(held, made) if not same(a, b)]
         self.reset()
 
     def _run(self):
         ctx = torch.autocast("cuda", dtype=self.autocast) if self.autocast is not None else contextlib.nullcontext()
-        with torch.no_grad(), ctx:
+        # the carry's buffers are this object's own: the single-step kernels update the states where they lie
+        with torch.no_grad(), ctx, step_in_place():
             if self._shadow:
                 return torch.func.functional_call(self.model, self._shadow, (self._x, self._done, self._carry))
             return self.model(self._x, self._done, self._carry)

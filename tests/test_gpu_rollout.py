@@ -46,6 +46,7 @@ def test_graphed_step_equals_the_eager_step(autocast):
         carry, y = eager(x, done, carry)
         want.append((y.clone(), [t.clone() for t in _flat(carry, [])]))
     act = GraphedStep(torso, B, Fe, autocast=autocast)
+    assert len(act._pairs) < len(_flat(carry, []))     # the matrix states are updated where they lie, not copied back
     print(f"case graphed step autocast={autocast}", flush=True)
     for rep in range(2):                     # the second round after reset(): from the initial carry again
         for i, (x, done) in enumerate(zip(xs, ds)):
@@ -70,4 +71,9 @@ def test_graphed_step_equals_the_eager_step(autocast):
     y = act(xs[1], ds[1])
     _, y_ref = eager(xs[1], ds[1], mid)
     assert torch.equal(y, y_ref)
+    # outside a GraphedStep a step leaves the carry it was given untouched
+    before = [t.clone() for t in _flat(mid, [])]
+    eager(xs[2], ds[2], mid)
+    for a, b in zip(_flat(mid, []), before):
+        assert torch.equal(a, b)
 

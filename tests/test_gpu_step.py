@@ -177,6 +177,31 @@ def test_step_inplace_zero_state_and_float_done():
     assert relerr(S4, S_ref.cpu().numpy()) <= 1e-5
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,H,d", [(1024, 4, 64), (5, 3, 32)])
+def test_normalised_and_gated_steps_in_place_equal_the_steps_out_of_place(dtype, B, H, d):
+    """Several steps in a row with the state (and the key sum) updated where they lie, against the same steps
+    writing new arrays: outputs and states bit for bit.  The normaliser z is read by every row of a workgroup and
+    written by one of them; many workgroups, so that rows that lag behind the writing one would show."""
+    from memorax_amd import kernels as K
+    g = torch.Generator(device="cuda").manual_seed(B + d)
+    S, z = torch.randn(B, H, d, d, device="cuda", generator=g), torch.rand(B, H, d, device="cuda", generator=g) + 0.5
+    S_in, z_in = S.clone(), z.clone()          # updated in place
+    Sg, Sg_in = S.clone(), S.clone()
+    print(f"case step in place dtype={dtype} B={B} H={H} d={d}", flush=True)
+    for step in range(4):
+        q, k, v = (torch.randn(B, H, d, device="cuda", generator=g).to(dtype) for _ in range(3))
+        glog = -torch.rand(B, H, device="cuda", generator=g)
+        done = torch.rand(B, device="cuda", generator=g) < 0.2
+        o, S, z = K.linear_attn_step(q, k, v, done, S, z, "elu1", True, 1e-6)
+        o2, S2, z2 = K.linear_attn_step(q, k, v, done, S_in, z_in, "elu1", True, 1e-6, inplace=True)
+        assert S2.data_ptr() == S_in.data_ptr() and z2.data_ptr() == z_in.data_ptr()
+        assert torch.equal(o2, o) and torch.equal(S_in, S) and torch.equal(z_in, z), step
+        og, Sg = K.gated_linear_attn_step(q, k, v, glog, done, Sg, "none")
+        og2, _ = K.gated_linear_attn_step(q, k, v, glog, done, Sg_in, "none", inplace=True)
+        assert torch.equal(og2, og) and torch.equal(Sg_in, Sg), step
+
+
 def test_step_rejects_bad_arguments():
     from memorax_amd import _lib
     lib = _lib.load()
